@@ -1,0 +1,110 @@
+"""Build recipe for the native parts: the gfx950 kernel library (hipcc), the C++ host layer's
+test harness (hipcc, host-only translation units linked against the kernel library) and the
+CPU oracle used by the tests (gcc, through oracle/Makefile).
+
+Everything is built in-tree so that the shared objects travel with the source tree:
+    anygpu_amd/lib/libanygpu_hip.so     kernels + C ABI (include/anygpu_hip.h)
+    anygpu_amd/lib/anygpu_host_tests    reference-style C++ test harness over Tensor<dtype, device>
+    oracle/liboracle.so                 CPU oracle (test infrastructure)
+"""
+from __future__ import annotations
+
+import os
+import shutil
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+from pathlib import Path
+
+PKG_DIR = Path(__file__).resolve().parent
+REPO_DIR = PKG_DIR.parent
+CSRC_DIR = PKG_DIR / "csrc"
+HOST_DIR = PKG_DIR / "host"
+LIB_DIR = PKG_DIR / "lib"
+OBJ_DIR = LIB_DIR / "obj"
+INCLUDE_DIR = REPO_DIR / "include"
+ORACLE_DIR = REPO_DIR / "oracle"
+
+GPU_ARCH = "gfx950"
+KERNEL_SOURCES = ["softmax.hip", "conv1d.hip", "gemm_f16.hip", "gemm_f32.hip", "capi.hip"]
+
+# -packed-fp32-ops is switched off on purpose: packed fp32 VALU forms are not to be generated.
+DEVICE_FLAGS = [
+    f"--offload-arch={GPU_ARCH}", "-O3", "-std=c++20", "-fPIC", "-fvisibility=hidden",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wall", "-Wno-unused-function",
+]
+
+
+def _hipcc() -> str:
+    for cand in (os.environ.get("HIPCC"), "/opt/rocm/bin/hipcc", shutil.which("hipcc")):
+        if cand and Path(cand).exists():
+            return cand
+    raise RuntimeError("hipcc not found (looked at $HIPCC, /opt/rocm/bin/hipcc and PATH)")
+
+
+def _run(cmd: list[str], quiet: bool = True) -> None:
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    out = "\n".join(l for l in proc.stdout.splitlines()
+                    if "'-packed-fp32-ops' is not a recognized feature" not in l)
+    if proc.returncode != 0:
+        raise RuntimeError(f"command failed ({proc.returncode}): {' '.join(cmd)}\n{out}")
+    if out.strip() and not quiet:
+        print(out)
+
+
+def build_kernels(verbose: bool = False) -> Path:
+    """Compile every kernel translation unit for gfx950 and link libanygpu_hip.so."""
+    hipcc = _hipcc()
+    OBJ_DIR.mkdir(parents=True, exist_ok=True)
+    objs = []
+
+    def compile_one(src: str) -> Path:
+        obj = OBJ_DIR / (Path(src).stem + ".o")
+        _run([hipcc, *DEVICE_FLAGS, f"-I{INCLUDE_DIR}", f"-I{CSRC_DIR}", "-c", str(CSRC_DIR / src), "-o", str(obj)],
+             quiet=not verbose)
+        return obj
+
+    with ThreadPoolExecutor(max_workers=min(len(KERNEL_SOURCES), 6)) as pool:
+        objs = list(pool.map(compile_one, KERNEL_SOURCES))
+    out = LIB_DIR / "libanygpu_hip.so"
+    _run([hipcc, f"--offload-arch={GPU_ARCH}", "-shared", "-fPIC", "-o", str(out), *map(str, objs)], quiet=not verbose)
+    return out
+
+
+def build_host_harness(verbose: bool = False) -> Path | None:
+    """Compile the C++ host layer's test harness, if the host layer is present."""
+    main_cpp = HOST_DIR / "harness" / "main.cpp"
+    if not main_cpp.exists():
+        return None
+    hipcc = _hipcc()
+    LIB_DIR.mkdir(parents=True, exist_ok=True)
+    sources = sorted(str(p) for p in (HOST_DIR / "core").glob("*.cpp"))
+    sources += sorted(str(p) for p in (HOST_DIR / "kernels").glob("*.cpp"))
+    sources += sorted(str(p) for p in (HOST_DIR / "harness").glob("*.cpp"))
+    includes = [f"-I{INCLUDE_DIR}"] + [f"-I{HOST_DIR / d}" for d in ("core", "ops", "fused", "kernels", "io", "harness")]
+    out = LIB_DIR / "anygpu_host_tests"
+    _run([hipcc, "-x", "c++", "-std=c++20", "-O2", "-DAC_WITH_ASSERT", "-D__HIP_PLATFORM_AMD__", *includes, *sources,
+          "-o", str(out), f"-L{LIB_DIR}", "-lanygpu_hip", "-L/opt/rocm/lib", "-lamdhip64",
+          f"-Wl,-rpath,$ORIGIN", "-Wl,-rpath,/opt/rocm/lib"], quiet=not verbose)
+    return out
+
+
+def build_oracle(verbose: bool = False) -> Path:
+    """Build the CPU oracle (tests only)."""
+    _run(["make", "-C", str(ORACLE_DIR), "-B"], quiet=not verbose)
+    return ORACLE_DIR / "liboracle.so"
+
+
+def build_all(verbose: bool = False) -> dict[str, str]:
+    built = {"kernels": str(build_kernels(verbose))}
+    harness = build_host_harness(verbose)
+    if harness is not None:
+        built["host_harness"] = str(harness)
+    built["oracle"] = str(build_oracle(verbose))
+    return built
+
+
+if __name__ == "__main__":
+    for name, path in build_all(verbose="-v" in sys.argv).items():
+        print(f"{name}: {path}")

@@ -1,0 +1,154 @@
+// extern "C" layer of libanygpu_hip.so: argument validation, then the kernel launchers.
+// Nothing is launched when an argument is rejected.
+#include "anygpu_hip.h"
+#include "launch.hpp"
+#include "device_utils.hpp"
+
+#include <climits>
+
+namespace {
+
+constexpr int kAbiVersion = 1;
+constexpr int64_t kMaxIndex32 = 0x7FFFFFFFLL;
+
+inline hipStream_t as_stream(void* s) { return static_cast<hipStream_t>(s); }
+
+int check_gemm(const void* A, const void* B, const void* C, int64_t M, int64_t N, int64_t K,
+               int64_t lda, int64_t ldb, int64_t ldc, int b_layout)
+{
+	if (M < 0 || N < 0 || K < 0) return ANYGPU_ERR_BAD_SHAPE;
+	if (b_layout != ANYGPU_B_ROW_MAJOR && b_layout != ANYGPU_B_COL_MAJOR) return ANYGPU_ERR_UNSUPPORTED;
+	if (M == 0 || N == 0) return ANYGPU_OK;
+	if (C == nullptr) return ANYGPU_ERR_NULL_POINTER;
+	if (K > 0 && (A == nullptr || B == nullptr)) return ANYGPU_ERR_NULL_POINTER;
+	if (lda < K || ldc < N) return ANYGPU_ERR_BAD_STRIDE;
+	if (ldb < (b_layout == ANYGPU_B_ROW_MAJOR ? N : K)) return ANYGPU_ERR_BAD_STRIDE;
+	// the grids index 64- or 128-wide tiles with 16-bit y and 31-bit x block numbers
+	if (M > 65535LL * 64 || N > kMaxIndex32 || K > kMaxIndex32) return ANYGPU_ERR_TOO_LARGE;
+	return ANYGPU_OK;
+}
+
+int check_softmax(const void* x, const void* y, int64_t rows, int64_t cols, int64_t xs, int64_t ys, int64_t window)
+{
+	if (rows < 0 || cols < 0 || window < 0) return ANYGPU_ERR_BAD_SHAPE;
+	if (rows == 0 || cols == 0) return ANYGPU_OK;
+	if (x == nullptr || y == nullptr) return ANYGPU_ERR_NULL_POINTER;
+	if (xs < cols || ys < cols) return ANYGPU_ERR_BAD_STRIDE;
+	if (rows > kMaxIndex32 || cols > kMaxIndex32) return ANYGPU_ERR_TOO_LARGE;
+	return ANYGPU_OK;
+}
+
+int check_conv(const void* x, const void* w, const void* b, const void* y,
+               int64_t batch, int64_t chan, int64_t seqlen, int64_t width)
+{
+	if (batch < 0 || chan < 0 || seqlen < 0) return ANYGPU_ERR_BAD_SHAPE;
+	if (width < 1 || width > 4) return ANYGPU_ERR_UNSUPPORTED;
+	if (batch == 0 || chan == 0 || seqlen == 0) return ANYGPU_OK;
+	if (x == nullptr || w == nullptr || b == nullptr || y == nullptr) return ANYGPU_ERR_NULL_POINTER;
+	if (chan > kMaxIndex32 || seqlen > kMaxIndex32) return ANYGPU_ERR_TOO_LARGE;
+	if (batch > kMaxIndex32 / chan) return ANYGPU_ERR_TOO_LARGE;                 // rows fit 31 bits
+	if (batch * chan > (kMaxIndex32 * 256) / seqlen) return ANYGPU_ERR_TOO_LARGE;  // element grid fits 31 bits of blocks
+	return ANYGPU_OK;
+}
+
+template <typename T>
+int softmax_entry(const void* x, void* y, int64_t rows, int64_t cols, int64_t xs, int64_t ys,
+                  int64_t q_len, int64_t diag, float alpha, float softcap, int causal, int64_t window, void* stream)
+{
+	const int rc = check_softmax(x, y, rows, cols, xs, ys, window);
+	if (rc != ANYGPU_OK) return rc;
+	if (q_len > kMaxIndex32) return ANYGPU_ERR_TOO_LARGE;
+	// keep i + diag and i + diag - window + 1 inside 64-bit range whatever the caller passes
+	if (diag > kMaxIndex32 || diag < -kMaxIndex32) return ANYGPU_ERR_TOO_LARGE;
+	return (int)anygpu::launch_softmax_rows<T>(x, y, rows, cols, xs, ys, q_len, diag, alpha, softcap, causal,
+	                                            window, as_stream(stream));
+}
+
+template <typename T>
+int conv_entry(const void* x, const void* w, const void* b, void* y,
+               int64_t batch, int64_t chan, int64_t seqlen, int64_t width, void* stream)
+{
+	const int rc = check_conv(x, w, b, y, batch, chan, seqlen, width);
+	if (rc != ANYGPU_OK) return rc;
+	return (int)anygpu::launch_causal_conv1d_silu<T>(x, w, b, y, batch, chan, seqlen, (int)width, as_stream(stream));
+}
+
+}  // namespace
+
+extern "C" {
+
+#define ANYGPU_EXPORT __attribute__((visibility("default")))
+
+ANYGPU_EXPORT int anygpu_hip_abi_version(void) { return kAbiVersion; }
+
+ANYGPU_EXPORT const char* anygpu_hip_target(void) { return "gfx950"; }
+
+ANYGPU_EXPORT const char* anygpu_hip_error_string(int code)
+{
+	switch (code)
+	{
+	case ANYGPU_OK: return "success";
+	case ANYGPU_ERR_NULL_POINTER: return "a required buffer pointer is NULL";
+	case ANYGPU_ERR_BAD_SHAPE: return "negative or inconsistent sizes";
+	case ANYGPU_ERR_BAD_STRIDE: return "a stride or leading dimension is smaller than the extent it spans";
+	case ANYGPU_ERR_UNSUPPORTED: return "argument value outside what the kernels implement";
+	case ANYGPU_ERR_TOO_LARGE: return "an extent exceeds what the launch geometry can index";
+	default: break;
+	}
+	if (code > 0) return hipGetErrorString(static_cast<hipError_t>(code));
+	return "unknown anygpu error code";
+}
+
+ANYGPU_EXPORT int anygpu_gemm_f16_f32acc(const void* A, const void* B, void* C,
+                                         int64_t M, int64_t N, int64_t K,
+                                         int64_t lda, int64_t ldb, int64_t ldc,
+                                         int b_layout, void* stream)
+{
+	const int rc = check_gemm(A, B, C, M, N, K, lda, ldb, ldc, b_layout);
+	if (rc != ANYGPU_OK) return rc;
+	return (int)anygpu::launch_gemm_f16(A, B, C, M, N, K, lda, ldb, ldc, b_layout, as_stream(stream));
+}
+
+ANYGPU_EXPORT int anygpu_gemm_f32(const float* A, const float* B, const float* bias, float* C,
+                                  int64_t M, int64_t N, int64_t K,
+                                  int64_t lda, int64_t ldb, int64_t ldc,
+                                  int b_layout, void* stream)
+{
+	const int rc = check_gemm(A, B, C, M, N, K, lda, ldb, ldc, b_layout);
+	if (rc != ANYGPU_OK) return rc;
+	return (int)anygpu::launch_gemm_f32(A, B, bias, C, M, N, K, lda, ldb, ldc, b_layout, as_stream(stream));
+}
+
+ANYGPU_EXPORT int anygpu_softmax_rows_f16(const void* x, void* y, int64_t rows, int64_t cols,
+                                          int64_t x_row_stride, int64_t y_row_stride,
+                                          int64_t q_len, int64_t diag,
+                                          float alpha, float softcap, int causal, int64_t window, void* stream)
+{
+	return softmax_entry<anygpu::half_t>(x, y, rows, cols, x_row_stride, y_row_stride, q_len, diag, alpha, softcap,
+	                                     causal, window, stream);
+}
+
+ANYGPU_EXPORT int anygpu_softmax_rows_f32(const float* x, float* y, int64_t rows, int64_t cols,
+                                          int64_t x_row_stride, int64_t y_row_stride,
+                                          int64_t q_len, int64_t diag,
+                                          float alpha, float softcap, int causal, int64_t window, void* stream)
+{
+	return softmax_entry<float>(x, y, rows, cols, x_row_stride, y_row_stride, q_len, diag, alpha, softcap,
+	                            causal, window, stream);
+}
+
+ANYGPU_EXPORT int anygpu_causal_conv1d_silu_f16(const void* x, const void* w, const void* bias, void* y,
+                                                int64_t batch, int64_t chan, int64_t seqlen, int64_t width,
+                                                void* stream)
+{
+	return conv_entry<anygpu::half_t>(x, w, bias, y, batch, chan, seqlen, width, stream);
+}
+
+ANYGPU_EXPORT int anygpu_causal_conv1d_silu_f32(const float* x, const float* w, const float* bias, float* y,
+                                                int64_t batch, int64_t chan, int64_t seqlen, int64_t width,
+                                                void* stream)
+{
+	return conv_entry<float>(x, w, bias, y, batch, chan, seqlen, width, stream);
+}
+
+}  // extern "C"

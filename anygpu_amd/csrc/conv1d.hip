@@ -1,0 +1,202 @@
+// Depthwise causal conv1d + bias + SiLU for gfx950.  Layout [batch, chan, seqlen] with the
+// sequence axis contiguous, so every (batch, chan) pair is one independent row.  HBM-bound:
+// x is read once, y written once, 16 bytes per lane per access.
+//
+// Tiled kernel: a 256-thread block owns a tile of 256 * U consecutive 16-byte vectors of one
+// row.  Each lane needs the width-1 samples in front of its vector; they are the tail of the
+// neighbouring lane's vector, so every lane publishes the tail of its vector in LDS and reads
+// its left neighbour's after one barrier.  The halo in front of the whole tile comes from
+// global memory (zeros at the start of a row).
+// Element kernel: one thread per output sample, for sequence lengths or pointers that do not
+// allow 16-byte row access.
+#include "device_utils.hpp"
+#include "launch.hpp"
+
+namespace anygpu {
+
+constexpr int kMaxWidth = 4;
+constexpr int kHalo = kMaxWidth - 1;
+
+template <typename T> struct ConvVec;
+template <> struct ConvVec<half_t> { using type = half8_t; using tail_type = half4_t; };
+template <> struct ConvVec<float> { using type = float4_t; using tail_type = float4_t; };
+
+__device__ __forceinline__ float silu_f32(float v)
+{
+	// v / (1 + e^{-v})
+	return v * fast_rcp(1.0f + fast_exp2(-v * kLog2e));
+}
+
+// The taps of a channel right-aligned into four slots: slot 3 multiplies the current sample,
+// slot 3 - d the sample d steps back.  Slots below 4 - WIDTH do not exist and are skipped.
+template <int WIDTH>
+__device__ __forceinline__ float conv_point(const float (&wv)[kMaxWidth], float bias, float xm3, float xm2, float xm1, float x0)
+{
+	const float xs[kMaxWidth] = { xm3, xm2, xm1, x0 };
+	float acc = 0.0f;
+#pragma unroll
+	for (int k = kMaxWidth - WIDTH; k < kMaxWidth; ++k) acc += wv[k] * xs[k];
+	acc += bias;
+	return silu_f32(acc);
+}
+
+template <typename T, int WIDTH, int U>
+__global__ __launch_bounds__(256) void causal_conv1d_silu_tile_kernel(
+	const T* __restrict__ x, const T* __restrict__ w, const T* __restrict__ bias, T* __restrict__ y,
+	int chan, int seqlen, int tiles_per_row)
+{
+	constexpr int EPV = 16 / (int)sizeof(T);
+	constexpr int TPV = (int)(sizeof(typename ConvVec<T>::tail_type) / sizeof(T));  // samples in a published tail
+	using Vec = typename ConvVec<T>::type;
+	using Tail = typename ConvVec<T>::tail_type;
+
+	__shared__ Tail tails[U][256];
+
+	const int tid = threadIdx.x;
+	const int row = blockIdx.x / tiles_per_row;           // (batch, chan) pair
+	const int tile = blockIdx.x - row * tiles_per_row;
+	const int ch = row % chan;
+	const int nvec = seqlen / EPV;
+	const int v_base = tile * (256 * U);
+
+	const T* __restrict__ xr = x + (int64_t)row * seqlen;
+	T* __restrict__ yr = y + (int64_t)row * seqlen;
+
+	float wv[kMaxWidth] = { 0.f, 0.f, 0.f, 0.f };
+#pragma unroll
+	for (int k = 0; k < WIDTH; ++k) wv[kMaxWidth - WIDTH + k] = (float)w[(int64_t)ch * WIDTH + k];
+	const float bv = (float)bias[ch];
+
+	Vec xv[U];
+#pragma unroll
+	for (int u = 0; u < U; ++u)
+	{
+		const int v = v_base + u * 256 + tid;
+		Vec val = {};
+		if (v < nvec) val = __builtin_nontemporal_load(reinterpret_cast<const Vec*>(xr) + v);
+		xv[u] = val;
+	}
+	// halo in front of the tile: the TPV samples that end where the tile starts
+	Tail front = {};
+	if (tid == 0 && v_base > 0)
+	{
+		front = *reinterpret_cast<const Tail*>(xr + (int64_t)v_base * EPV - TPV);
+	}
+
+#pragma unroll
+	for (int u = 0; u < U; ++u)
+	{
+		Tail t;
+#pragma unroll
+		for (int e = 0; e < TPV; ++e) t[e] = xv[u][EPV - TPV + e];
+		tails[u][tid] = t;
+	}
+	__syncthreads();
+
+#pragma unroll
+	for (int u = 0; u < U; ++u)
+	{
+		const int v = v_base + u * 256 + tid;
+		if (v >= nvec) continue;
+		Tail prev;
+		if (tid > 0) prev = tails[u][tid - 1];
+		else if (u > 0) prev = tails[u - 1][255];
+		else prev = front;
+
+		float s[kHalo + EPV];
+#pragma unroll
+		for (int e = 0; e < kHalo; ++e) s[e] = (float)prev[TPV - kHalo + e];
+#pragma unroll
+		for (int e = 0; e < EPV; ++e) s[kHalo + e] = (float)xv[u][e];
+
+		Vec out;
+#pragma unroll
+		for (int e = 0; e < EPV; ++e)
+		{
+			out[e] = (T)conv_point<WIDTH>(wv, bv, s[e], s[e + 1], s[e + 2], s[e + 3]);
+		}
+		__builtin_nontemporal_store(out, reinterpret_cast<Vec*>(yr) + v);
+	}
+}
+
+template <typename T, int WIDTH>
+__global__ __launch_bounds__(256) void causal_conv1d_silu_element_kernel(
+	const T* __restrict__ x, const T* __restrict__ w, const T* __restrict__ bias, T* __restrict__ y,
+	int chan, int seqlen, int64_t total)
+{
+	const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+	if (idx >= total) return;
+	const int64_t row = idx / seqlen;
+	const int s = (int)(idx - row * seqlen);
+	const int ch = (int)(row % chan);
+
+	float wv[kMaxWidth] = { 0.f, 0.f, 0.f, 0.f };
+#pragma unroll
+	for (int k = 0; k < WIDTH; ++k) wv[kMaxWidth - WIDTH + k] = (float)w[(int64_t)ch * WIDTH + k];
+	const float bv = (float)bias[ch];
+
+	const T* __restrict__ xr = x + row * seqlen;
+	float xs[kMaxWidth];
+#pragma unroll
+	for (int k = 0; k < kMaxWidth; ++k)
+	{
+		const int pos = s + k - kHalo;
+		xs[k] = (k >= kMaxWidth - WIDTH && pos >= 0) ? (float)xr[pos] : 0.0f;
+	}
+	y[idx] = (T)conv_point<WIDTH>(wv, bv, xs[0], xs[1], xs[2], xs[3]);
+}
+
+template <typename T, int WIDTH>
+static hipError_t launch_width(const void* x, const void* w, const void* bias, void* y,
+                               int64_t batch, int64_t chan, int64_t seqlen, hipStream_t stream)
+{
+	constexpr int EPV = 16 / (int)sizeof(T);
+	constexpr int U = 2;
+	const int64_t rows = batch * chan;
+	const T* xp = static_cast<const T*>(x);
+	const T* wp = static_cast<const T*>(w);
+	const T* bp = static_cast<const T*>(bias);
+	T* yp = static_cast<T*>(y);
+
+	const bool vec_ok = (seqlen % EPV == 0) && (reinterpret_cast<uintptr_t>(x) % 16 == 0) &&
+	                    (reinterpret_cast<uintptr_t>(y) % 16 == 0);
+	if (vec_ok)
+	{
+		const int64_t nvec = seqlen / EPV;
+		const int64_t tiles_per_row = (nvec + 256 * U - 1) / (256 * U);
+		const int64_t blocks = rows * tiles_per_row;
+		if (blocks <= 0x7FFFFFFFLL)
+		{
+			causal_conv1d_silu_tile_kernel<T, WIDTH, U><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(
+				xp, wp, bp, yp, (int)chan, (int)seqlen, (int)tiles_per_row);
+			return hipGetLastError();
+		}
+	}
+	const int64_t total = rows * seqlen;
+	const int64_t blocks = (total + 255) / 256;
+	causal_conv1d_silu_element_kernel<T, WIDTH><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(
+		xp, wp, bp, yp, (int)chan, (int)seqlen, total);
+	return hipGetLastError();
+}
+
+template <typename T>
+hipError_t launch_causal_conv1d_silu(const void* x, const void* w, const void* bias, void* y,
+                                     int64_t batch, int64_t chan, int64_t seqlen, int width,
+                                     hipStream_t stream)
+{
+	if (batch == 0 || chan == 0 || seqlen == 0) return hipSuccess;
+	switch (width)
+	{
+	case 1: return launch_width<T, 1>(x, w, bias, y, batch, chan, seqlen, stream);
+	case 2: return launch_width<T, 2>(x, w, bias, y, batch, chan, seqlen, stream);
+	case 3: return launch_width<T, 3>(x, w, bias, y, batch, chan, seqlen, stream);
+	default: return launch_width<T, 4>(x, w, bias, y, batch, chan, seqlen, stream);
+	}
+}
+
+template hipError_t launch_causal_conv1d_silu<half_t>(const void*, const void*, const void*, void*, int64_t, int64_t,
+                                                       int64_t, int, hipStream_t);
+template hipError_t launch_causal_conv1d_silu<float>(const void*, const void*, const void*, void*, int64_t, int64_t,
+                                                      int64_t, int, hipStream_t);
+
+}  // namespace anygpu

@@ -1,0 +1,65 @@
+// Small device-side helpers shared by the gfx950 kernels: 16-byte vector types, wave64
+// reductions built on DPP, and fp32 transcendental wrappers.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+namespace anygpu {
+
+typedef _Float16 half_t;
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float float2_t __attribute__((ext_vector_type(2)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+
+constexpr int kWaveSize = 64;
+constexpr float kLog2e = 1.4426950408889634f;
+
+// One DPP move: lane l receives `v` from the lane selected by CTRL inside its row of 16
+// lanes; with bound_ctrl set, lanes without a source read 0 (never the case for the
+// permutations and rotations used here).
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v)
+{
+	return __builtin_bit_cast(float,
+		__builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
+
+struct MaxOp { __device__ __forceinline__ float operator()(float a, float b) const { return fmaxf(a, b); } };
+struct SumOp { __device__ __forceinline__ float operator()(float a, float b) const { return a + b; } };
+
+// All-reduce over the 64 lanes of a wave.  Within each row of 16 lanes: two quad
+// permutations (xor 1, xor 2), then row rotations by 4 and 8.  The four row results are
+// then read out as scalars and combined, which leaves the same value in every lane.
+template <typename Op>
+__device__ __forceinline__ float wave_allreduce(float v, Op op)
+{
+	v = op(v, dpp_move<0xB1>(v));    // quad_perm [1,0,3,2]
+	v = op(v, dpp_move<0x4E>(v));    // quad_perm [2,3,0,1]
+	v = op(v, dpp_move<0x124>(v));   // row_ror:4
+	v = op(v, dpp_move<0x128>(v));   // row_ror:8
+	float r0 = __builtin_amdgcn_readlane(v, 0);
+	float r1 = __builtin_amdgcn_readlane(v, 16);
+	float r2 = __builtin_amdgcn_readlane(v, 32);
+	float r3 = __builtin_amdgcn_readlane(v, 48);
+	return op(op(r0, r1), op(r2, r3));
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
+
+// tanh(x) = 1 - 2 / (1 + e^{2x}); saturates cleanly to +-1 for large |x| (e^{2x} -> inf or 0).
+// Near zero that form cancels, so |x| < 1/16 uses the odd Taylor polynomial up to x^7
+// (truncation error below 1e-11 relative at the switch point).
+__device__ __forceinline__ float tanh_f32(float x)
+{
+	float e = fast_exp2(x * (2.0f * kLog2e));
+	float big = 1.0f - 2.0f * fast_rcp(1.0f + e);
+	float x2 = x * x;
+	float small = x * (1.0f + x2 * (-1.0f / 3.0f + x2 * (2.0f / 15.0f + x2 * (-17.0f / 315.0f))));
+	return fabsf(x) < 0.0625f ? small : big;
+}
+
+}  // namespace anygpu

@@ -1,0 +1,133 @@
+"""Thin Python callers of the C ABI on torch device tensors.
+
+torch is used for device memory and the current stream only; every computation happens in
+libanygpu_hip.so.  The function names follow the reference's operator API (tensor_mm,
+tensor_gemm, tensor_softmax, tensor_causal_conv1d; srcs/ops/mm_ops.hpp, srcs/ops/softmax_ops.hpp,
+srcs/fused/causal_conv1d.hpp), with the fused attention prologue and the B layout as the
+additional keyword arguments the C ABI carries.
+"""
+from __future__ import annotations
+
+import torch
+
+from . import capi
+
+
+def _stream_ptr() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _require(cond: bool, msg: str) -> None:
+    if not cond:
+        raise ValueError(msg)
+
+
+def _check_device(*tensors: torch.Tensor) -> None:
+    for t in tensors:
+        _require(t.is_cuda, "anygpu ops take device tensors only (no CPU fallback)")
+
+
+def tensor_mm(lhs: torch.Tensor, rhs: torch.Tensor, out: torch.Tensor | None = None,
+              b_layout: int = capi.B_ROW_MAJOR) -> torch.Tensor:
+    """C = lhs @ B.  lhs is [M, K] row-major (rows may be padded: stride(0) >= K, stride(1) == 1).
+    With b_layout == B_ROW_MAJOR rhs is [K, N]; with B_COL_MAJOR rhs is the [N, K] storage of B.
+    float16 (fp32 accumulate) and float32 are supported."""
+    _check_device(lhs, rhs)
+    _require(lhs.dim() == 2 and rhs.dim() == 2, "matrix multiplication requires compatible matrices")
+    _require(lhs.dtype == rhs.dtype, "operands must share a dtype")
+    _require(lhs.stride(1) == 1 and rhs.stride(1) == 1, "innermost stride must be 1")
+    m, k = lhs.shape
+    if b_layout == capi.B_ROW_MAJOR:
+        _require(rhs.shape[0] == k, "matrix multiplication requires compatible matrices")
+        n = rhs.shape[1]
+    else:
+        _require(rhs.shape[1] == k, "matrix multiplication requires compatible matrices")
+        n = rhs.shape[0]
+    if out is None:
+        out = torch.empty((m, n), dtype=lhs.dtype, device=lhs.device)
+    _require(tuple(out.shape) == (m, n) and out.stride(1) == 1, "result mtx shape is wrong")
+    lib = capi.load()
+    lda = lhs.stride(0) if m > 1 else max(k, 1)
+    ldb = rhs.stride(0) if rhs.shape[0] > 1 else max(rhs.shape[1], 1)
+    ldc = out.stride(0) if m > 1 else max(n, 1)
+    if lhs.dtype == torch.float16:
+        rc = lib.anygpu_gemm_f16_f32acc(lhs.data_ptr(), rhs.data_ptr(), out.data_ptr(), m, n, k,
+                                        lda, ldb, ldc, b_layout, _stream_ptr())
+        capi.check("anygpu_gemm_f16_f32acc", rc)
+    elif lhs.dtype == torch.float32:
+        rc = lib.anygpu_gemm_f32(lhs.data_ptr(), rhs.data_ptr(), None, out.data_ptr(), m, n, k,
+                                 lda, ldb, ldc, b_layout, _stream_ptr())
+        capi.check("anygpu_gemm_f32", rc)
+    else:
+        raise TypeError("Unsupported data type")
+    return out
+
+
+def tensor_gemm(xt: torch.Tensor, wt: torch.Tensor, bt: torch.Tensor,
+                b_layout: int = capi.B_ROW_MAJOR) -> torch.Tensor:
+    """xt @ wt + bt (bias per output column), float32."""
+    _check_device(xt, wt, bt)
+    _require(xt.dim() == 2 and wt.dim() == 2, "matrix multiplication requires compatible matrices")
+    _require(xt.dtype == torch.float32 and wt.dtype == torch.float32 and bt.dtype == torch.float32,
+             "Unsupported data type")
+    _require(xt.is_contiguous() and wt.is_contiguous() and bt.is_contiguous(), "dense operands expected")
+    m, k = xt.shape
+    n = wt.shape[1] if b_layout == capi.B_ROW_MAJOR else wt.shape[0]
+    _require((wt.shape[0] if b_layout == capi.B_ROW_MAJOR else wt.shape[1]) == k,
+             "matrix multiplication requires compatible matrices")
+    _require(bt.numel() == n, "incorrect bias shape")
+    out = torch.empty((m, n), dtype=torch.float32, device=xt.device)
+    rc = capi.load().anygpu_gemm_f32(xt.data_ptr(), wt.data_ptr(), bt.data_ptr(), out.data_ptr(), m, n, k,
+                                     max(k, 1), max(wt.shape[1], 1), max(n, 1), b_layout, _stream_ptr())
+    capi.check("anygpu_gemm_f32", rc)
+    return out
+
+
+def tensor_softmax(x: torch.Tensor, out: torch.Tensor | None = None, *, alpha: float = 1.0, softcap: float = 0.0,
+                   causal: bool = False, window: int = 0, q_len: int = 0, diag: int = 0) -> torch.Tensor:
+    """Row softmax of a 2-D tensor with the fused prologue (scale -> softcap -> masks)."""
+    _check_device(x)
+    _require(x.dim() == 2, "softmax expects 2 dimensional tensors")
+    _require(x.stride(1) == 1 or x.shape[1] <= 1, "rows must be contiguous")
+    rows, cols = x.shape
+    if out is None:
+        out = torch.empty((rows, cols), dtype=x.dtype, device=x.device)
+    _require(tuple(out.shape) == (rows, cols), "result shape is wrong")
+    xs = x.stride(0) if rows > 1 else max(cols, 1)
+    ys = out.stride(0) if rows > 1 else max(cols, 1)
+    lib = capi.load()
+    if x.dtype == torch.float16:
+        fn, name = lib.anygpu_softmax_rows_f16, "anygpu_softmax_rows_f16"
+    elif x.dtype == torch.float32:
+        fn, name = lib.anygpu_softmax_rows_f32, "anygpu_softmax_rows_f32"
+    else:
+        raise TypeError("Unsupported data type")
+    rc = fn(x.data_ptr(), out.data_ptr(), rows, cols, xs, ys, q_len, diag, alpha, softcap, int(causal), window,
+            _stream_ptr())
+    capi.check(name, rc)
+    return out
+
+
+def tensor_causal_conv1d(xt: torch.Tensor, wt: torch.Tensor, bt: torch.Tensor,
+                         out: torch.Tensor | None = None) -> torch.Tensor:
+    """silu(depthwise causal conv1d(xt, wt) + bt); xt [batch, dims, seq_len], wt [dims, width], bt [dims]."""
+    _check_device(xt, wt, bt)
+    _require(xt.dim() == 3, "xt needs to be 3 dimensional")
+    _require(xt.shape[1] == wt.shape[0], "xt and wt need to have the same dims")
+    _require(wt.shape[0] == bt.shape[0], "wt and bt need to have the same dims")
+    _require(wt.shape[1] <= 4, "kernel width needs to be under 4")
+    _require(xt.dtype == wt.dtype == bt.dtype, "operands must share a dtype")
+    _require(xt.is_contiguous() and wt.is_contiguous() and bt.is_contiguous(), "dense operands expected")
+    if out is None:
+        out = torch.empty_like(xt)
+    b, d, s = xt.shape
+    lib = capi.load()
+    if xt.dtype == torch.float16:
+        fn, name = lib.anygpu_causal_conv1d_silu_f16, "anygpu_causal_conv1d_silu_f16"
+    elif xt.dtype == torch.float32:
+        fn, name = lib.anygpu_causal_conv1d_silu_f32, "anygpu_causal_conv1d_silu_f32"
+    else:
+        raise TypeError("Unsupported data types")
+    rc = fn(xt.data_ptr(), wt.data_ptr(), bt.data_ptr(), out.data_ptr(), b, d, s, wt.shape[1], _stream_ptr())
+    capi.check(name, rc)
+    return out

@@ -1,0 +1,121 @@
+/*
+ * C ABI of libanygpu_hip.so: the gfx950 (MI355X) kernels behind anyGPU's matmul, row softmax
+ * and causal conv1d + SiLU entry points.
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer into memory the caller owns; nothing is allocated,
+ *     freed or retained by the library, inputs are only read, outputs only written;
+ *   - sizes, strides and leading dimensions are int64_t counts of ELEMENTS;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream, which is what the
+ *     reference uses for every launch); calls are asynchronous with respect to the host;
+ *   - the return value is 0 on success, a negative ANYGPU_ERR_* code when an argument is
+ *     rejected before anything is launched, or a positive hipError_t value when the runtime
+ *     refuses the launch.  The C++ `cu_*` wrappers turn any non-zero value into the
+ *     reference's convention (log the error, exit(1); srcs/core/core.hpp:445-475).
+ *   - fp16 values are IEEE binary16 stored as 2 bytes (what the reference calls float16,
+ *     srcs/core/core.hpp:37).
+ *
+ * File and line citations name the interface of the reference (adamtiger/anyGPU) that each
+ * entry point stands in for.
+ */
+#ifndef ANYGPU_HIP_H
+#define ANYGPU_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define ANYGPU_OK                 0
+#define ANYGPU_ERR_NULL_POINTER  -1   /* a required buffer pointer is NULL */
+#define ANYGPU_ERR_BAD_SHAPE     -2   /* a size is negative, or sizes are mutually inconsistent */
+#define ANYGPU_ERR_BAD_STRIDE    -3   /* a stride / leading dimension is smaller than the extent it spans */
+#define ANYGPU_ERR_UNSUPPORTED   -4   /* a value outside what the kernels implement (e.g. conv width > 4) */
+#define ANYGPU_ERR_TOO_LARGE     -5   /* an extent exceeds what the launch geometry can index */
+
+/* Layout of the right-hand GEMM operand. */
+#define ANYGPU_B_ROW_MAJOR  0   /* B stored [K, N], element (l, c) at B[l * ldb + c]  (reference layout) */
+#define ANYGPU_B_COL_MAJOR  1   /* B stored [N, K], element (l, c) at B[c * ldb + l]  ("weights as [out, in]") */
+
+/* Library identification: ABI version (bumped on any signature change) and the code object target. */
+int         anygpu_hip_abi_version(void);
+const char* anygpu_hip_target(void);            /* "gfx950" */
+const char* anygpu_hip_error_string(int code);  /* text for ANYGPU_ERR_* and for hipError_t values */
+
+/*
+ * C[M,N] = A[M,K] * B  with fp16 inputs, fp32 accumulation on the MFMA units, fp16 output.
+ * Replaces opt2::cu_tensor_mm_f16 (srcs/kernels/cuda/mm_ops.cuh:60-63, the tensor_mm<float16, CUDA>
+ * path of srcs/ops/mm_ops.hpp:62-65) and the cu_fast_mm_f16_* ladder
+ * (srcs/kernels/cuda/fast_mm.cuh:70-98).  A is row-major with leading dimension lda >= K,
+ * C row-major with ldc >= N, B as selected by b_layout (ldb >= N for row-major, >= K for
+ * column-major).  Any M, N, K >= 0 are accepted; M, N multiples of 256 and K a multiple of 64
+ * with 16-byte aligned rows take the fastest kernel.
+ */
+int anygpu_gemm_f16_f32acc(const void* A, const void* B, void* C,
+                           int64_t M, int64_t N, int64_t K,
+                           int64_t lda, int64_t ldb, int64_t ldc,
+                           int b_layout, void* stream);
+
+/*
+ * C[M,N] = A[M,K] * B (+ bias[N] added to every row when bias != NULL), fp32 throughout, fp32 MFMA.
+ * Replaces cu_tensor_mm_f32_opt0 and cu_tensor_gemm_f32_opt0 (srcs/kernels/cuda/mm_ops.cuh:10-25, the
+ * tensor_mm / tensor_gemm <float32, CUDA> paths of srcs/ops/mm_ops.hpp:58-61,160-163) and the
+ * cu_fast_mm_f32_* ladder (srcs/kernels/cuda/fast_mm.cuh:7-68).  Any shape.
+ */
+int anygpu_gemm_f32(const float* A, const float* B, const float* bias, float* C,
+                    int64_t M, int64_t N, int64_t K,
+                    int64_t lda, int64_t ldb, int64_t ldc,
+                    int b_layout, void* stream);
+
+/*
+ * Row softmax over the last axis of a [rows, cols] matrix, with the steps the attention caller
+ * runs in front of it fused in, applied in this order to each element x[r, j]:
+ *     s = x * alpha                                   (tensor_mul, srcs/ops/binary_ops.hpp:61-76)
+ *     s = softcap * tanh(s / softcap)   if softcap != 0   (srcs/models/gemma2/gemma_linsoftcap.cu:3-9)
+ *     masked if causal != 0 and j >  i + diag         (additive -inf above the diagonal)
+ *     masked if window  > 0 and j <= i + diag - window (srcs/models/gemma2/gemma_slide_mask.cu:21)
+ *     y = softmax over the row, masked elements are exactly 0  (srcs/ops/softmax_ops.hpp:15-82)
+ * where i = r % q_len is the query index of row r (q_len <= 0 means i = r).  With alpha = 1,
+ * softcap = 0, causal = 0, window = 0 this is cu_tensor_softmax_f32
+ * (srcs/kernels/cuda/softmax_ops.cuh:6-8); the fused form replaces the mul -> add -> softmax
+ * launches of srcs/transformers/sdp.hpp:267-269.  Rows are x_row_stride / y_row_stride elements
+ * apart (>= cols), elements of a row are contiguous.  A row whose every element is masked is
+ * written as zeros.  Internals are fp32 for both element types.
+ */
+int anygpu_softmax_rows_f16(const void* x, void* y,
+                            int64_t rows, int64_t cols,
+                            int64_t x_row_stride, int64_t y_row_stride,
+                            int64_t q_len, int64_t diag,
+                            float alpha, float softcap, int causal, int64_t window,
+                            void* stream);
+
+int anygpu_softmax_rows_f32(const float* x, float* y,
+                            int64_t rows, int64_t cols,
+                            int64_t x_row_stride, int64_t y_row_stride,
+                            int64_t q_len, int64_t diag,
+                            float alpha, float softcap, int causal, int64_t window,
+                            void* stream);
+
+/*
+ * Depthwise causal conv1d with bias and fused SiLU:
+ *     y[b, d, s] = silu( bias[d] + sum_{k=0}^{width-1} w[d, k] * x[b, d, s + k - (width - 1)] ),
+ * terms with a negative sequence index dropped (left zero padding of width-1).
+ * x and y are [batch, chan, seqlen] with seqlen contiguous, w is [chan, width], bias [chan], all
+ * densely packed and of the element type of the entry point; fp32 internals.  width must be 1..4,
+ * the bound the reference asserts (srcs/fused/causal_conv1d.hpp:100).
+ * Replaces cu_tensor_causal_conv1d_f32 (srcs/kernels/cuda/causal_conv1d.cuh:6-10).
+ */
+int anygpu_causal_conv1d_silu_f16(const void* x, const void* w, const void* bias, void* y,
+                                  int64_t batch, int64_t chan, int64_t seqlen, int64_t width,
+                                  void* stream);
+
+int anygpu_causal_conv1d_silu_f32(const float* x, const float* w, const float* bias, float* y,
+                                  int64_t batch, int64_t chan, int64_t seqlen, int64_t width,
+                                  void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* ANYGPU_HIP_H */

@@ -1,0 +1,224 @@
+"""numpy-facing wrapper of the CPU oracle (oracle/anygpu_oracle.c -> oracle/liboracle.so).
+
+TEST INFRASTRUCTURE ONLY.  Imported by tests/, by the smoke check and by the CPU-baseline leg
+of the benchmark; the product package (anygpu_amd) never imports it.  Each function forwards
+to the C restatement of the reference's CPU implementation; see the header of
+anygpu_oracle.c for the reference file:line each one follows and how it is pinned.
+"""
+from __future__ import annotations
+
+import ctypes
+import subprocess
+from ctypes import POINTER, c_float, c_int, c_int32, c_int64, c_void_p
+from pathlib import Path
+
+import numpy as np
+
+ORACLE_DIR = Path(__file__).resolve().parent
+LIB_PATH = ORACLE_DIR / "liboracle.so"
+
+_lib = None
+
+
+def build() -> Path:
+    subprocess.run(["make", "-C", str(ORACLE_DIR)], check=True, stdout=subprocess.DEVNULL)
+    return LIB_PATH
+
+
+def lib() -> ctypes.CDLL:
+    global _lib
+    if _lib is None:
+        if not LIB_PATH.exists():
+            build()
+        _lib = ctypes.CDLL(str(LIB_PATH))
+        _lib.oracle_max_threads.restype = c_int
+    return _lib
+
+
+def max_threads() -> int:
+    return int(lib().oracle_max_threads())
+
+
+def _ptr(a: np.ndarray) -> c_void_p:
+    return c_void_p(a.ctypes.data)
+
+
+def _elem_strides(a: np.ndarray) -> tuple[int, ...]:
+    assert all(s % a.itemsize == 0 for s in a.strides)
+    return tuple(s // a.itemsize for s in a.strides)
+
+
+_MM = {np.dtype(np.float32): "oracle_tensor_mm_f32", np.dtype(np.float64): "oracle_tensor_mm_f64",
+       np.dtype(np.int32): "oracle_tensor_mm_i32"}
+
+
+def tensor_mm(lhs: np.ndarray, rhs: np.ndarray, rows: tuple[int, int] | None = None, threads: int = 1) -> np.ndarray:
+    """res = lhs @ rhs the reference's way; strided views are honoured (a transposed view is a
+    column-major operand).  `rows` = (begin, end) computes that row range only (others stay 0)."""
+    assert lhs.ndim == 2 and rhs.ndim == 2 and lhs.shape[1] == rhs.shape[0], \
+        "matrix multiplication requires compatible matrices"
+    assert lhs.dtype == rhs.dtype and lhs.dtype in _MM
+    m, k = lhs.shape
+    n = rhs.shape[1]
+    res = np.zeros((m, n), dtype=lhs.dtype)
+    r0, r1 = rows if rows is not None else (0, m)
+    ls, rs, os_ = _elem_strides(lhs), _elem_strides(rhs), _elem_strides(res)
+    fn = getattr(lib(), _MM[lhs.dtype])
+    fn.restype = None
+    fn(_ptr(lhs), _ptr(rhs), _ptr(res), c_int64(m), c_int64(n), c_int64(k),
+       c_int64(ls[0]), c_int64(ls[1]), c_int64(rs[0]), c_int64(rs[1]), c_int64(os_[0]), c_int64(os_[1]),
+       c_int64(r0), c_int64(r1), c_int(threads))
+    return res
+
+
+def tensor_gemm(xt: np.ndarray, wt: np.ndarray, bt: np.ndarray, threads: int = 1) -> np.ndarray:
+    assert xt.dtype == wt.dtype == bt.dtype == np.float32
+    assert xt.ndim == 2 and wt.ndim == 2 and xt.shape[1] == wt.shape[0] and bt.shape == (wt.shape[1],)
+    m, k = xt.shape
+    n = wt.shape[1]
+    res = np.zeros((m, n), dtype=np.float32)
+    bt = np.ascontiguousarray(bt)
+    xs, ws, os_ = _elem_strides(xt), _elem_strides(wt), _elem_strides(res)
+    fn = lib().oracle_tensor_gemm_f32
+    fn.restype = None
+    fn(_ptr(xt), _ptr(wt), _ptr(bt), _ptr(res), c_int64(m), c_int64(n), c_int64(k),
+       c_int64(xs[0]), c_int64(xs[1]), c_int64(ws[0]), c_int64(ws[1]), c_int64(os_[0]), c_int64(os_[1]),
+       c_int64(0), c_int64(m), c_int(threads))
+    return res
+
+
+def tensor_softmax(x: np.ndarray, threads: int = 1) -> np.ndarray:
+    assert x.ndim == 2, "softmax expects 2 dimensional tensors"
+    assert x.dtype in (np.float32, np.float64)
+    m, n = x.shape
+    y = np.zeros((m, n), dtype=x.dtype)
+    xs, ys = _elem_strides(x), _elem_strides(y)
+    fn = lib().oracle_tensor_softmax_f32 if x.dtype == np.float32 else lib().oracle_tensor_softmax_f64
+    fn.restype = None
+    fn(_ptr(x), _ptr(y), c_int64(m), c_int64(n), c_int64(xs[0]), c_int64(xs[1]), c_int64(ys[0]), c_int64(ys[1]),
+       c_int(threads))
+    return y
+
+
+def tensor_mul_scalar(x: np.ndarray, alpha: float) -> np.ndarray:
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    y = np.empty_like(x)
+    fn = lib().oracle_tensor_mul_scalar_f32
+    fn.restype = None
+    fn(_ptr(x), c_float(alpha), _ptr(y), c_int64(x.size))
+    return y
+
+
+def tensor_add(lhs: np.ndarray, rhs: np.ndarray) -> np.ndarray:
+    lhs = np.ascontiguousarray(lhs, dtype=np.float32)
+    rhs = np.ascontiguousarray(rhs, dtype=np.float32)
+    assert lhs.shape == rhs.shape, "tensors are not elementwise compatible"
+    y = np.empty_like(lhs)
+    fn = lib().oracle_tensor_add_f32
+    fn.restype = None
+    fn(_ptr(lhs), _ptr(rhs), _ptr(y), c_int64(lhs.size))
+    return y
+
+
+def softcap(x: np.ndarray, cap: float) -> np.ndarray:
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    y = np.empty_like(x)
+    fn = lib().oracle_softcap_f32
+    fn.restype = None
+    fn(_ptr(x), c_float(cap), _ptr(y), c_int64(x.size))
+    return y
+
+
+def causal_mask(q_len: int, k_len: int, diag: int = 0) -> np.ndarray:
+    mask = np.empty((q_len, k_len), dtype=np.float32)
+    fn = lib().oracle_causal_mask_f32
+    fn.restype = None
+    fn(_ptr(mask), c_int64(q_len), c_int64(k_len), c_int64(diag))
+    return mask
+
+
+def slide_mask(mask: np.ndarray, window: int) -> np.ndarray:
+    """mask is [batch, 1, seq_len, mask_len] (or [seq_len, mask_len])."""
+    m = np.ascontiguousarray(mask, dtype=np.float32)
+    seq_len, mask_len = m.shape[-2], m.shape[-1]
+    batch = m.size // (seq_len * mask_len)
+    y = np.empty_like(m)
+    fn = lib().oracle_slide_mask_f32
+    fn.restype = None
+    fn(_ptr(m), c_int32(window), c_int64(batch), c_int64(seq_len), c_int64(mask_len), _ptr(y))
+    return y
+
+
+def attention_softmax(x: np.ndarray, *, alpha: float = 1.0, softcap: float = 0.0, causal: bool = False,
+                      window: int = 0, q_len: int = 0, diag: int = 0, row_index: np.ndarray | None = None,
+                      threads: int = 1) -> np.ndarray:
+    """scale -> (softcap) -> mask add -> softmax on the rows of a float32 [rows, cols] matrix,
+    composed from the primitives above in the reference's call order.  With `row_index` only
+    those rows are evaluated and returned, packed in that order."""
+    assert x.ndim == 2 and x.dtype == np.float32 and x.strides[1] == 4
+    rows, cols = x.shape
+    if row_index is not None:
+        idx = np.ascontiguousarray(row_index, dtype=np.int64)
+        count = idx.size
+        idx_ptr = idx.ctypes.data_as(POINTER(c_int64))
+    else:
+        idx, count, idx_ptr = None, rows, None
+    y = np.zeros((count, cols), dtype=np.float32)
+    fn = lib().oracle_attention_softmax_f32
+    fn.restype = None
+    fn(_ptr(x), _ptr(y), c_int64(rows), c_int64(cols), c_int64(x.strides[0] // 4), c_int64(q_len), c_int64(diag),
+       c_float(alpha), c_float(softcap), c_int(int(causal)), c_int64(window), idx_ptr, c_int64(count), c_int(threads))
+    return y
+
+
+def tensor_causal_conv1d(xt: np.ndarray, wt: np.ndarray, bt: np.ndarray, rows: tuple[int, int] | None = None,
+                         threads: int = 1) -> np.ndarray:
+    assert xt.ndim == 3, "xt needs to be 3 dimensional"
+    assert xt.shape[1] == wt.shape[0], "xt and wt need to have the same dims"
+    assert wt.shape[0] == bt.shape[0], "wt and bt need to have the same dims"
+    assert xt.dtype == wt.dtype == bt.dtype and xt.dtype in (np.float32, np.float64)
+    assert xt.strides[2] == xt.itemsize and wt.strides[1] == wt.itemsize
+    b, d, s = xt.shape
+    y = np.zeros((b, d, s), dtype=xt.dtype)
+    bt = np.ascontiguousarray(bt)
+    xs, ys, ws = _elem_strides(xt), _elem_strides(y), _elem_strides(wt)
+    r0, r1 = rows if rows is not None else (0, b * d)
+    fn = lib().oracle_tensor_causal_conv1d_f32 if xt.dtype == np.float32 else lib().oracle_tensor_causal_conv1d_f64
+    fn.restype = None
+    fn(_ptr(xt), _ptr(wt), _ptr(bt), _ptr(y), c_int64(b), c_int64(d), c_int64(s), c_int64(wt.shape[1]),
+       c_int64(xs[0]), c_int64(xs[1]), c_int64(ys[0]), c_int64(ys[1]), c_int64(ws[0]),
+       c_int64(r0), c_int64(r1), c_int(threads))
+    return y
+
+
+def cvt_f16_to_f32(h: np.ndarray) -> np.ndarray:
+    """The reference's half -> float up-cast, from the raw 16-bit patterns."""
+    bits = np.ascontiguousarray(h).view(np.uint16)
+    out = np.empty(bits.shape, dtype=np.float32)
+    fn = lib().oracle_cvt_f16_to_f32
+    fn.restype = None
+    fn(_ptr(bits), _ptr(out), c_int64(bits.size))
+    return out
+
+
+def _compare(name: str, actual: np.ndarray, expected: np.ndarray, tol: float) -> tuple[bool, float]:
+    a = np.ascontiguousarray(actual, dtype=np.float32)
+    e = np.ascontiguousarray(expected, dtype=np.float32)
+    assert a.shape == e.shape
+    worst = c_float(0.0)
+    fn = getattr(lib(), name)
+    fn.restype = c_int
+    ok = fn(_ptr(a), _ptr(e), c_int64(a.size), c_float(tol), ctypes.byref(worst))
+    return bool(ok), float(worst.value)
+
+
+def compare_data_buffers(actual, expected, abs_tol: float = 0.001):
+    return _compare("oracle_compare_abs_f32", actual, expected, abs_tol)
+
+
+def compare_data_buffers_reldiff(actual, expected, rel_tol: float = 0.01):
+    return _compare("oracle_compare_reldiff_f32", actual, expected, rel_tol)
+
+
+def compare_data_buffers_l2(actual, expected, rel_l2: float = 0.01):
+    return _compare("oracle_compare_l2_f32", actual, expected, rel_l2)

@@ -1,0 +1,445 @@
+/*
+ * CPU oracle for the anyGPU hot path: matmul, row softmax (with the scale / softcap /
+ * mask steps the attention caller runs before it) and depthwise causal conv1d + SiLU.
+ *
+ * THIS FILE IS TEST INFRASTRUCTURE, NOT PRODUCT CODE.  It restates, in plain C, the CPU
+ * implementation of the reference (adamtiger/anyGPU, paths relative to its root) with the
+ * same loop order, the same accumulator types and the same stride handling, so that the
+ * HIP kernels can be checked against "what the reference's CPU path would have produced".
+ * Only tests, the smoke check and the CPU-baseline leg of the benchmark may link or load
+ * it; the product library never does.
+ *
+ * How each function is pinned (tests/test_oracle_*.py):
+ *   oracle_tensor_mm_*       integer-valued inputs vs int64 brute force (bit exact), identity /
+ *                            ones / pattern closed forms, strided == explicit transpose,
+ *                            float64 brute force with the K*2^-24*sum|a*b| bound.
+ *   oracle_tensor_gemm_f32   same + bias closed form.
+ *   oracle_tensor_softmax_*  row sums, shift invariance, constant rows (1/n exact for n = 2^p),
+ *                            two-value closed form, one-hot limit, -inf / lowest -> exact 0,
+ *                            long-double brute force.
+ *   oracle_tensor_mul_scalar / oracle_tensor_add   elementwise identities.
+ *   oracle_softcap_f32       odd symmetry, |y| < cap, y(cap*atanh(1/2)) = cap/2, double tanh brute force.
+ *   oracle_slide_mask_f32    brute-force visible set {j : i-W < j <= i}, counts min(i+1, W).
+ *   oracle_causal_mask_f32   tril closed form.
+ *   oracle_tensor_causal_conv1d_*  impulse response, pass-through tap, zero weights, causality
+ *                            under perturbation, linearity of the pre-activation, explicit
+ *                            zero-padded brute force in float64.
+ *   oracle_cvt_f16_to_f32    all 65536 bit patterns vs numpy.float16.
+ *   oracle_compare_*         hand-computed three-element cases.
+ * The reference repository holds no golden vectors for this path (its .dat fixtures are
+ * git-ignored and were drawn from an unseeded generator), so nothing here is pinned against
+ * reference-held data.  PARITY UNPINNED: the composition "scale -> softcap -> mask -> softmax"
+ * (oracle_attention_softmax_f32 with softcap != 0) has no counterpart call site in the
+ * reference; it is the composition of the pinned primitives in the stated order and is
+ * pinned only by the checks listed for those primitives plus a float64 brute force.
+ */
+#include <math.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+#include <float.h>
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+typedef long long i64;
+
+#define ORACLE_API __attribute__((visibility("default")))
+
+static int clamp_threads(int threads)
+{
+#ifdef _OPENMP
+	if (threads < 1) threads = 1;
+	return threads;
+#else
+	(void)threads;
+	return 1;
+#endif
+}
+
+ORACLE_API int oracle_max_threads(void)
+{
+#ifdef _OPENMP
+	return omp_get_max_threads();
+#else
+	return 1;
+#endif
+}
+
+/* ------------------------------------------------------------------------------------------
+ * tensor_mm  --  srcs/ops/mm_ops.hpp:11-45
+ *   res[r,c] = sum_l lhs[r,l] * rhs[l,c]; the product is formed in the element type, the
+ *   running sum `acc` is float32 whatever the element type is (mm_ops.hpp:32), l ascends,
+ *   and every operand is addressed through its own strides (mm_ops.hpp:33-37).
+ *   Rows [row_begin, row_end) only are produced so that large cases can be sampled; outer
+ *   rows may be spread over threads, which leaves each element's arithmetic order untouched.
+ * ---------------------------------------------------------------------------------------- */
+#define DEFINE_MM(NAME, T)                                                                     \
+ORACLE_API void NAME(const T* lhs, const T* rhs, T* res, i64 m, i64 n, i64 k,                  \
+                     i64 ls0, i64 ls1, i64 rs0, i64 rs1, i64 os0, i64 os1,                     \
+                     i64 row_begin, i64 row_end, int threads)                                  \
+{                                                                                              \
+	(void)m;                                                                                   \
+	int nt = clamp_threads(threads);                                                           \
+	(void)nt;                                                                                  \
+	_Pragma("omp parallel for schedule(static) num_threads(nt)")                               \
+	for (i64 r = row_begin; r < row_end; ++r)                                                  \
+	{                                                                                          \
+		for (i64 c = 0; c < n; ++c)                                                            \
+		{                                                                                      \
+			float acc = 0.f;                                                                   \
+			for (i64 l = 0; l < k; ++l)                                                        \
+			{                                                                                  \
+				T prod = lhs[r * ls0 + l * ls1] * rhs[l * rs0 + c * rs1];                      \
+				acc += prod;                                                                   \
+			}                                                                                  \
+			res[r * os0 + c * os1] = (T)acc;                                                   \
+		}                                                                                      \
+	}                                                                                          \
+}
+
+DEFINE_MM(oracle_tensor_mm_f32, float)
+DEFINE_MM(oracle_tensor_mm_f64, double)
+DEFINE_MM(oracle_tensor_mm_i32, int32_t)
+
+/* tensor_gemm  --  srcs/ops/mm_ops.hpp:102-144: same sum, then `acc + bt[c]` (bias indexed by column). */
+ORACLE_API void oracle_tensor_gemm_f32(const float* xt, const float* wt, const float* bt, float* res,
+                                       i64 m, i64 n, i64 k,
+                                       i64 xs0, i64 xs1, i64 ws0, i64 ws1, i64 os0, i64 os1,
+                                       i64 row_begin, i64 row_end, int threads)
+{
+	(void)m;
+	int nt = clamp_threads(threads);
+	(void)nt;
+	#pragma omp parallel for schedule(static) num_threads(nt)
+	for (i64 r = row_begin; r < row_end; ++r)
+	{
+		for (i64 c = 0; c < n; ++c)
+		{
+			float acc = 0.f;
+			for (i64 l = 0; l < k; ++l)
+			{
+				acc += xt[r * xs0 + l * xs1] * wt[l * ws0 + c * ws1];
+			}
+			res[r * os0 + c * os1] = acc + bt[c];
+		}
+	}
+}
+
+/* ------------------------------------------------------------------------------------------
+ * tensor_softmax  --  srcs/ops/softmax_ops.hpp:15-82
+ *   per row: running maximum starting from element 0 (:44-52); e_c = (T)exp((double)(x_c - max))
+ *   written to y (:58-69); the sum is kept in T and grows left to right (:61,68);
+ *   y_c = y_c * ((T)1 / sum) (:72-78).
+ * ---------------------------------------------------------------------------------------- */
+#define DEFINE_SOFTMAX_ROW(NAME, T)                                                            \
+static void NAME(const T* x, T* y, i64 n, i64 xsc, i64 ysc)                                    \
+{                                                                                              \
+	T max_val = x[0];                                                                          \
+	for (i64 c = 1; c < n; ++c)                                                                \
+	{                                                                                          \
+		T v = x[c * xsc];                                                                      \
+		if (v > max_val) max_val = v;                                                          \
+	}                                                                                          \
+	T exponent = x[0] - max_val;                                                               \
+	T exp_val = (T)exp((double)exponent);                                                      \
+	y[0] = exp_val;                                                                            \
+	T reduced = exp_val;                                                                       \
+	for (i64 c = 1; c < n; ++c)                                                                \
+	{                                                                                          \
+		exponent = x[c * xsc] - max_val;                                                       \
+		exp_val = (T)exp((double)exponent);                                                    \
+		y[c * ysc] = exp_val;                                                                  \
+		reduced += exp_val;                                                                    \
+	}                                                                                          \
+	T rec_reduced = (T)1.0 / reduced;                                                          \
+	for (i64 c = 0; c < n; ++c)                                                                \
+	{                                                                                          \
+		y[c * ysc] = y[c * ysc] * rec_reduced;                                                 \
+	}                                                                                          \
+}
+
+DEFINE_SOFTMAX_ROW(softmax_row_f32, float)
+DEFINE_SOFTMAX_ROW(softmax_row_f64, double)
+
+#define DEFINE_SOFTMAX(NAME, ROWFN, T)                                                         \
+ORACLE_API void NAME(const T* x, T* y, i64 m, i64 n, i64 xs0, i64 xs1, i64 ys0, i64 ys1,       \
+                     int threads)                                                              \
+{                                                                                              \
+	int nt = clamp_threads(threads);                                                           \
+	(void)nt;                                                                                  \
+	_Pragma("omp parallel for schedule(static) num_threads(nt)")                               \
+	for (i64 r = 0; r < m; ++r)                                                                \
+	{                                                                                          \
+		ROWFN(x + r * xs0, y + r * ys0, n, xs1, ys1);                                          \
+	}                                                                                          \
+}
+
+DEFINE_SOFTMAX(oracle_tensor_softmax_f32, softmax_row_f32, float)
+DEFINE_SOFTMAX(oracle_tensor_softmax_f64, softmax_row_f64, double)
+
+/* tensor_mul(tensor, scalar)  --  srcs/ops/binary_ops.hpp:61-76 */
+ORACLE_API void oracle_tensor_mul_scalar_f32(const float* x, float alpha, float* y, i64 length)
+{
+	for (i64 ix = 0; ix < length; ++ix) y[ix] = x[ix] * alpha;
+}
+
+/* tensor_add(tensor, tensor)  --  srcs/ops/binary_ops.hpp:11-29 */
+ORACLE_API void oracle_tensor_add_f32(const float* lhs, const float* rhs, float* y, i64 length)
+{
+	for (i64 ix = 0; ix < length; ++ix) y[ix] = lhs[ix] + rhs[ix];
+}
+
+/* softcap(x, cap) = tanhf(x / cap) * cap  --  srcs/models/gemma2/gemma_linsoftcap.cu:3-9 */
+ORACLE_API void oracle_softcap_f32(const float* x, float cap, float* y, i64 length)
+{
+	for (i64 ix = 0; ix < length; ++ix)
+	{
+		float temp = x[ix] / cap;
+		temp = tanhf(temp);
+		y[ix] = temp * cap;
+	}
+}
+
+/* Additive causal mask: 0 on and below the diagonal, -inf above it.
+ * scripts/sdp_test_cases.py:164-168 (tril(diagonal=0), masked_fill(~tril, -inf)).
+ * `diag` shifts the diagonal for a key axis longer than the query axis: key j is visible to
+ * query i iff j <= i + diag. */
+ORACLE_API void oracle_causal_mask_f32(float* mask, i64 q_len, i64 k_len, i64 diag)
+{
+	for (i64 i = 0; i < q_len; ++i)
+		for (i64 j = 0; j < k_len; ++j)
+			mask[i * k_len + j] = (j <= i + diag) ? 0.f : -INFINITY;
+}
+
+/* Sliding-window rule  --  srcs/models/gemma2/gemma_slide_mask.cu:17-29,38:
+ * element (seq_idx, j) is replaced by float lowest iff seq_idx >= W and j <= seq_idx - W,
+ * otherwise the incoming mask value is kept. */
+ORACLE_API void oracle_slide_mask_f32(const float* mask, int32_t window, i64 batch, i64 seq_len, i64 mask_len, float* y)
+{
+	const float f32_min = -FLT_MAX;
+	for (i64 b = 0; b < batch; ++b)
+		for (i64 s = 0; s < seq_len; ++s)
+			for (i64 j = 0; j < mask_len; ++j)
+			{
+				i64 off = b * seq_len * mask_len + s * mask_len + j;
+				if (s >= window && j <= s - window) y[off] = f32_min;
+				else y[off] = mask[off];
+			}
+}
+
+/* ------------------------------------------------------------------------------------------
+ * The chain the attention caller runs on a score matrix before and including softmax:
+ *   nqk = tensor_mul(qk, alpha); nqk_masked = tensor_add(nqk, mask); tensor_softmax(nqk_masked)
+ *   -- srcs/transformers/sdp.hpp:265-269.
+ * With softcap != 0 the capped logits cap*tanh(s/cap) are formed between the scale and the
+ * mask add (the order Gemma2 attention uses; no reference call site, see header).
+ * The mask of row r is built from the rules above for query index (r % q_len): causal -inf
+ * above the diagonal (shifted by diag), then the sliding rule with float lowest when window > 0.
+ * Works row by row so that full-size cases need only O(cols) scratch per thread.
+ * `row_index` (may be NULL) lists which rows of x to process; outputs are packed densely.
+ * ---------------------------------------------------------------------------------------- */
+ORACLE_API void oracle_attention_softmax_f32(const float* x, float* y, i64 rows, i64 cols, i64 x_row_stride,
+                                             i64 q_len, i64 diag, float alpha, float softcap,
+                                             int causal, i64 window,
+                                             const i64* row_index, i64 n_index, int threads)
+{
+	int nt = clamp_threads(threads);
+	(void)nt;
+	i64 count = row_index ? n_index : rows;
+	#pragma omp parallel num_threads(nt)
+	{
+		float* nqk = (float*)malloc(sizeof(float) * (size_t)cols);
+		float* mask = (float*)malloc(sizeof(float) * (size_t)cols);
+		float* tmp = (float*)malloc(sizeof(float) * (size_t)cols);
+		#pragma omp for schedule(dynamic, 8)
+		for (i64 t = 0; t < count; ++t)
+		{
+			i64 r = row_index ? row_index[t] : t;
+			i64 i = (q_len > 0) ? (r % q_len) : r;
+			const float* xr = x + r * x_row_stride;
+			oracle_tensor_mul_scalar_f32(xr, alpha, nqk, cols);
+			if (softcap != 0.f)
+			{
+				oracle_softcap_f32(nqk, softcap, tmp, cols);
+				memcpy(nqk, tmp, sizeof(float) * (size_t)cols);
+			}
+			for (i64 j = 0; j < cols; ++j)
+			{
+				float mv = 0.f;
+				if (causal && j > i + diag) mv = -INFINITY;
+				mask[j] = mv;
+			}
+			if (window > 0)
+			{
+				/* sliding rule on the row of query position i + diag (the absolute position of the query) */
+				i64 s = i + diag;
+				for (i64 j = 0; j < cols; ++j)
+					if (s >= window && j <= s - window) mask[j] = -FLT_MAX;
+			}
+			oracle_tensor_add_f32(nqk, mask, tmp, cols);
+			softmax_row_f32(tmp, y + t * cols, cols, 1, 1);
+		}
+		free(nqk); free(mask); free(tmp);
+	}
+}
+
+/* ------------------------------------------------------------------------------------------
+ * tensor_causal_conv1d  --  srcs/fused/causal_conv1d.hpp:24-87
+ *   x (batch, dims, seq_len), w (dims, width), b (dims) -> y (batch, dims, seq_len)
+ *   out = 0; for k ascending: delta = k + 1 + six - w; if delta >= 0: out += w[d,k] * x[b,d,delta]  (:66-74)
+ *   out += bias (:76); out = out / (1 + exp(-out)) (:79); x and y rows use strides 0 and 1 of
+ *   their tensors and unit step along the sequence, w uses stride 0 (:58-60).
+ *   `exp` on a float argument binds to the float overload of <cmath> in C++; expf here.
+ * ---------------------------------------------------------------------------------------- */
+ORACLE_API void oracle_tensor_causal_conv1d_f32(const float* x, const float* w, const float* bias, float* y,
+                                                i64 b, i64 d, i64 s, i64 width,
+                                                i64 xs0, i64 xs1, i64 ys0, i64 ys1, i64 ws0,
+                                                i64 row_begin, i64 row_end, int threads)
+{
+	int nt = clamp_threads(threads);
+	(void)nt; (void)b;
+	/* a "row" is one (batch, channel) pair, numbered bix * d + dix */
+	#pragma omp parallel for schedule(static) num_threads(nt)
+	for (i64 row = row_begin; row < row_end; ++row)
+	{
+		i64 bix = row / d, dix = row % d;
+		i64 x_offset = bix * xs0 + dix * xs1;
+		i64 y_offset = bix * ys0 + dix * ys1;
+		i64 w_offset = dix * ws0;
+		for (i64 six = 0; six < s; ++six)
+		{
+			float out = 0;
+			for (i64 k = 0; k < width; ++k)
+			{
+				i64 delta = k + 1 + six - width;
+				if (delta >= 0)
+				{
+					out += w[w_offset + k] * x[x_offset + delta];
+				}
+			}
+			out += bias[dix];
+			out = out / (1.0f + expf(-out));
+			y[y_offset + six] = out;
+		}
+	}
+}
+
+ORACLE_API void oracle_tensor_causal_conv1d_f64(const double* x, const double* w, const double* bias, double* y,
+                                                i64 b, i64 d, i64 s, i64 width,
+                                                i64 xs0, i64 xs1, i64 ys0, i64 ys1, i64 ws0,
+                                                i64 row_begin, i64 row_end, int threads)
+{
+	int nt = clamp_threads(threads);
+	(void)nt; (void)b;
+	#pragma omp parallel for schedule(static) num_threads(nt)
+	for (i64 row = row_begin; row < row_end; ++row)
+	{
+		i64 bix = row / d, dix = row % d;
+		i64 x_offset = bix * xs0 + dix * xs1;
+		i64 y_offset = bix * ys0 + dix * ys1;
+		i64 w_offset = dix * ws0;
+		for (i64 six = 0; six < s; ++six)
+		{
+			double out = 0;
+			for (i64 k = 0; k < width; ++k)
+			{
+				i64 delta = k + 1 + six - width;
+				if (delta >= 0)
+				{
+					out += w[w_offset + k] * x[x_offset + delta];
+				}
+			}
+			out += bias[dix];
+			out = out / (1.0 + exp(-out));
+			y[y_offset + six] = out;
+		}
+	}
+}
+
+/* ------------------------------------------------------------------------------------------
+ * fp16 protocol: the reference has no CPU half arithmetic; half tensors are up-cast element by
+ * element to float32 (cvt_tensor_datatype, srcs/core/tensor.hpp:388-410, through __half2float,
+ * srcs/core/core.hpp:263-267) and the float32 CPU op is run (tests/tests.cpp:146-151).
+ * The conversion is exact: IEEE binary16 -> binary32.
+ * ---------------------------------------------------------------------------------------- */
+static float half_bits_to_float(uint16_t h)
+{
+	uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
+	uint32_t exp = (h >> 10) & 0x1Fu;
+	uint32_t man = h & 0x3FFu;
+	uint32_t bits;
+	if (exp == 0)
+	{
+		if (man == 0) bits = sign;
+		else
+		{
+			/* subnormal half: normalise */
+			int e = -1;
+			do { ++e; man <<= 1; } while ((man & 0x400u) == 0);
+			man &= 0x3FFu;
+			bits = sign | ((uint32_t)(127 - 15 - e) << 23) | (man << 13);
+		}
+	}
+	else if (exp == 31) bits = sign | 0x7F800000u | (man << 13);
+	else bits = sign | ((exp + (127 - 15)) << 23) | (man << 13);
+	float f;
+	memcpy(&f, &bits, sizeof(f));
+	return f;
+}
+
+ORACLE_API void oracle_cvt_f16_to_f32(const uint16_t* src, float* dst, i64 n)
+{
+	for (i64 ix = 0; ix < n; ++ix) dst[ix] = half_bits_to_float(src[ix]);
+}
+
+/* ------------------------------------------------------------------------------------------
+ * Comparators  --  tests/test_tools.hpp
+ *   abs:     every |e - a| < abs_tol                                   (:23-43)
+ *   reldiff: every |e - a| / (|e| + 1e-8) < rel_tol                    (:45-66)
+ *   l2:      sqrt( sum (e-a)^2 / sum (e^2 + 1e-8) ) < rel_l2, float32 running sums (:76-103)
+ * Each returns 1 for "equal", 0 otherwise; *worst receives the largest metric seen.
+ * ---------------------------------------------------------------------------------------- */
+ORACLE_API int oracle_compare_abs_f32(const float* actual, const float* expected, i64 length, float abs_tol, float* worst)
+{
+	int eq = 1;
+	float w = 0.f;
+	for (i64 ix = 0; ix < length; ++ix)
+	{
+		float d = fabsf(expected[ix] - actual[ix]);
+		eq = eq && (d < abs_tol);
+		if (!(d <= w)) w = d;
+	}
+	if (worst) *worst = w;
+	return eq;
+}
+
+ORACLE_API int oracle_compare_reldiff_f32(const float* actual, const float* expected, i64 length, float rel_tol, float* worst)
+{
+	int eq = 1;
+	float w = 0.f;
+	for (i64 ix = 0; ix < length; ++ix)
+	{
+		float d = fabsf(expected[ix] - actual[ix]) / (fabsf(expected[ix]) + (float)1e-8);
+		eq = eq && (d < rel_tol);
+		if (!(d <= w)) w = d;
+	}
+	if (worst) *worst = w;
+	return eq;
+}
+
+ORACLE_API int oracle_compare_l2_f32(const float* actual, const float* expected, i64 length, float rel_l2, float* value)
+{
+	float cum_square_diff = 0.f;
+	float cum_square = 0.f;
+	for (i64 ix = 0; ix < length; ++ix)
+	{
+		float temp = expected[ix] - actual[ix];
+		float residual = temp * temp;
+		cum_square_diff += residual;
+		cum_square += expected[ix] * expected[ix] + 1e-8f;
+	}
+	float l2 = sqrtf(cum_square_diff / cum_square);
+	if (value) *value = l2;
+	return l2 < rel_l2;
+}

@@ -1,0 +1,412 @@
+"""GPU parity: the HIP kernels, called through the C ABI, against the CPU oracle on identical
+inputs.  Tolerances (scale-floored relative error, see tests/helpers.py):
+    fp16-in / fp32-accumulate GEMM  <= 1e-2      fp32 ops  <= 1e-4      fp16 softmax / conv1d  <= 2e-3
+Integer-valued cases are bit exact.  Masked softmax outputs must be exactly 0.
+"""
+import ctypes
+import math
+
+import numpy as np
+import pytest
+
+from anygpu_amd import synth
+from helpers import rel_l2, sample_rows, scaled_rel_err
+
+pytestmark = pytest.mark.gpu
+
+TOL_F16_GEMM = 1e-2
+TOL_F32 = 1e-4
+TOL_F16_ROWOPS = 2e-3
+
+
+def dev(a):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def host(t):
+    import torch
+    torch.cuda.synchronize()
+    return t.detach().cpu().numpy()
+
+
+# =============================================================================================
+# softmax
+# =============================================================================================
+
+def test_softmax_f32_reference_case_6x45(ops, oracle):
+    # tests/tests.cpp:187-204: crt_random_tensor (integers 0..10), CPU vs device, abs tol 1e-3
+    x = synth.integers(11, (6, 45), 0, 10)
+    got = host(ops.tensor_softmax(dev(x)))
+    want = oracle.tensor_softmax(x)
+    ok, worst = oracle.compare_data_buffers(got, want)
+    assert ok, worst
+    assert scaled_rel_err(got, want, want.max(axis=1, keepdims=True)) <= TOL_F32
+
+
+@pytest.mark.parametrize("dtype", ["f16", "f32"])
+@pytest.mark.parametrize("rows,cols", [(1, 1), (3, 7), (5, 8), (64, 512), (33, 520), (17, 1024), (9, 2048),
+                                       (6, 4096), (5, 8192), (3, 8200), (2, 16384), (4, 100), (7, 2047)])
+def test_softmax_plain_shapes(ops, oracle, dtype, rows, cols):
+    np_dt = np.float16 if dtype == "f16" else np.float32
+    x = synth.normal(rows * 131 + cols, (rows, cols), std=2.0).astype(np_dt)
+    got = host(ops.tensor_softmax(dev(x))).astype(np.float32)
+    want = oracle.tensor_softmax(oracle.cvt_f16_to_f32(x) if dtype == "f16" else x)
+    tol = TOL_F16_ROWOPS if dtype == "f16" else TOL_F32
+    assert scaled_rel_err(got, want, want.max(axis=1, keepdims=True)) <= tol
+    assert np.all(np.abs(got.sum(axis=1, dtype=np.float64) - 1.0) < (2e-2 if dtype == "f16" else 1e-5))
+
+
+@pytest.mark.parametrize("dtype", ["f16", "f32"])
+def test_softmax_padded_row_strides(ops, oracle, dtype):
+    import torch
+    np_dt = np.float16 if dtype == "f16" else np.float32
+    rows, cols, pitch = 37, 256, 320
+    buf = synth.normal(3, (rows, pitch), std=2.0).astype(np_dt)
+    xb = dev(buf)
+    out = torch.full((rows, pitch + 64), 7.0, dtype=xb.dtype, device="cuda")
+    ops.tensor_softmax(xb[:, :cols], out=out[:, :cols])
+    got = host(out).astype(np.float32)
+    xin = buf[:, :cols]
+    want = oracle.tensor_softmax(np.ascontiguousarray(oracle.cvt_f16_to_f32(xin) if dtype == "f16" else xin))
+    tol = TOL_F16_ROWOPS if dtype == "f16" else TOL_F32
+    assert scaled_rel_err(got[:, :cols], want, want.max(axis=1, keepdims=True)) <= tol
+    assert np.all(got[:, cols:] == 7.0)      # padding is not written
+
+
+FUSED_CASES = [
+    # rows, cols, q_len, diag, alpha, softcap, causal, window
+    (64, 64, 64, 0, 0.125, 0.0, True, 0),
+    (96, 48, 48, 0, 0.125, 0.0, True, 0),           # two heads of 48 queries
+    (64, 64, 64, 0, 0.0625, 50.0, True, 16),
+    (40, 72, 40, 32, 0.125, 0.0, True, 0),          # keys longer than queries: diagonal shifted
+    (40, 72, 40, 32, 0.125, 30.0, True, 24),
+    (33, 100, 33, 0, 1.0, 0.0, False, 10),          # window without causal, scalar kernel
+    (128, 1024, 128, 896, 0.125, 0.0, True, 256),
+    (50, 37, 25, 0, 0.3, 5.0, True, 7),
+    (16, 8192, 16, 8176, 0.0625, 50.0, True, 4096),
+    (8, 64, 8, -3, 0.125, 0.0, True, 0),            # first rows see nothing at all
+]
+
+
+@pytest.mark.parametrize("dtype", ["f16", "f32"])
+@pytest.mark.parametrize("case", FUSED_CASES)
+def test_softmax_fused_prologue(ops, oracle, dtype, case):
+    rows, cols, q_len, diag, alpha, cap, causal, window = case
+    np_dt = np.float16 if dtype == "f16" else np.float32
+    x = synth.normal(rows + cols, (rows, cols), std=1.0 / alpha).astype(np_dt)
+    got = host(ops.tensor_softmax(dev(x), alpha=alpha, softcap=cap, causal=causal, window=window,
+                                  q_len=q_len, diag=diag)).astype(np.float32)
+    x32 = oracle.cvt_f16_to_f32(x) if dtype == "f16" else x
+    i = (np.arange(rows) % q_len)[:, None]
+    j = np.arange(cols)[None, :]
+    vis = np.ones((rows, cols), dtype=bool)
+    if causal:
+        vis &= j <= i + diag
+    if window > 0:
+        vis &= j > i + diag - window
+    live = vis.any(axis=1)
+    want = np.zeros((rows, cols), dtype=np.float32)
+    if live.any():
+        want[live] = oracle.attention_softmax(x32, alpha=alpha, softcap=cap, causal=causal, window=window,
+                                              q_len=q_len, diag=diag, row_index=np.nonzero(live)[0])
+    assert np.all(got[~vis] == 0.0), "masked outputs must be exact zeros"
+    tol = TOL_F16_ROWOPS if dtype == "f16" else TOL_F32
+    floor = np.maximum(want.max(axis=1, keepdims=True), 1e-30)
+    assert scaled_rel_err(got, want, floor) <= tol
+
+
+def test_softmax_first_causal_row_and_neg_inf_inputs(ops):
+    import torch
+    x = torch.randn(4, 64, device="cuda", dtype=torch.float32)
+    x[2, 5:] = float("-inf")
+    x[3, :] = float("-inf")
+    x[3, 9] = 0.5
+    y = host(ops.tensor_softmax(x, causal=True, q_len=64, diag=60))
+    # row 2 (query 2, sees keys 0..62): entries 5.. are -inf inputs -> exact zeros
+    assert np.all(y[2, 5:] == 0.0) and abs(y[2, :5].sum() - 1.0) < 1e-6
+    assert y[3, 9] == 1.0 and y[3].sum() == 1.0
+    y0 = host(ops.tensor_softmax(x[:1], causal=True, q_len=64))
+    assert y0[0, 0] == 1.0 and not y0[0, 1:].any()
+
+
+def test_softmax_empty_and_rejected_arguments(ops):
+    import torch
+    from anygpu_amd import capi
+    lib = capi.load()
+    e = ops.tensor_softmax(torch.empty((0, 16), device="cuda", dtype=torch.float16))
+    assert e.shape == (0, 16)
+    e = ops.tensor_softmax(torch.empty((4, 0), device="cuda", dtype=torch.float32))
+    assert e.shape == (4, 0)
+    x = torch.zeros((4, 16), device="cuda", dtype=torch.float32)
+    y = torch.full((4, 16), 3.0, device="cuda", dtype=torch.float32)
+    assert lib.anygpu_softmax_rows_f32(None, y.data_ptr(), 4, 16, 16, 16, 0, 0, 1.0, 0.0, 0, 0, None) == capi.ANYGPU_ERR_NULL_POINTER
+    assert lib.anygpu_softmax_rows_f32(x.data_ptr(), y.data_ptr(), 4, 16, 8, 16, 0, 0, 1.0, 0.0, 0, 0, None) == capi.ANYGPU_ERR_BAD_STRIDE
+    assert lib.anygpu_softmax_rows_f32(x.data_ptr(), y.data_ptr(), -1, 16, 16, 16, 0, 0, 1.0, 0.0, 0, 0, None) == capi.ANYGPU_ERR_BAD_SHAPE
+    assert lib.anygpu_softmax_rows_f32(x.data_ptr(), y.data_ptr(), 4, 16, 16, 16, 0, 0, 1.0, 0.0, 0, -2, None) == capi.ANYGPU_ERR_BAD_SHAPE
+    torch.cuda.synchronize()
+    assert bool((y == 3.0).all()), "a rejected call must not launch anything"
+
+
+def _full_size_softmax(ops, oracle, heads, q, k, std, alpha, cap, window, n_sample):
+    import torch
+    rows = heads * q
+    g = torch.Generator(device="cuda")
+    g.manual_seed(0)
+    x = (torch.randn((rows, k), device="cuda", dtype=torch.float32, generator=g) * std).to(torch.float16)
+    y = ops.tensor_softmax(x, alpha=alpha, softcap=cap, causal=True, window=window, q_len=q)
+    torch.cuda.synchronize()
+    # size-independent properties over the whole output
+    sums = y.float().sum(dim=1)
+    assert float((sums - 1.0).abs().max()) < 2e-2
+    i = (torch.arange(rows, device="cuda") % q)[:, None]
+    # masked region must be exactly zero: check in row slabs to bound memory
+    for r0 in range(0, rows, 8192):
+        blk = y[r0:r0 + 8192]
+        ii = i[r0:r0 + 8192]
+        j = torch.arange(k, device="cuda")[None, :]
+        masked = j > ii
+        if window > 0:
+            masked |= j <= ii - window
+        assert not bool(blk[masked].any())
+    # sampled rows against the oracle on the very same fp16 inputs
+    idx = sample_rows(rows, n_sample, seed=1)
+    xs = x[torch.from_numpy(idx).cuda()].cpu().numpy()
+    # a sampled row arrives alone, so its query index is handed to the oracle as the diagonal shift
+    want = np.zeros((idx.size, k), dtype=np.float32)
+    x32 = oracle.cvt_f16_to_f32(xs)
+    for t, r in enumerate(idx):
+        want[t] = oracle.attention_softmax(x32[t:t + 1], alpha=alpha, softcap=cap, causal=True, window=window,
+                                           q_len=0, diag=int(r % q))[0]
+    got = y[torch.from_numpy(idx).cuda()].cpu().numpy().astype(np.float32)
+    assert scaled_rel_err(got, want, want.max(axis=1, keepdims=True)) <= TOL_F16_ROWOPS
+
+
+def test_softmax_config_causal_32x2048x2048(ops, oracle):
+    _full_size_softmax(ops, oracle, heads=32, q=2048, k=2048, std=4.0, alpha=1.0 / 8.0, cap=0.0, window=0, n_sample=96)
+
+
+def test_softmax_config_gemma2_8x8192x8192(ops, oracle):
+    _full_size_softmax(ops, oracle, heads=8, q=8192, k=8192, std=16.0, alpha=1.0 / 16.0, cap=50.0, window=4096,
+                       n_sample=48)
+
+
+# =============================================================================================
+# causal conv1d + SiLU
+# =============================================================================================
+
+def _conv_case(ops, oracle, dtype, b, d, s, width, seed, threads=8):
+    np_dt = np.float16 if dtype == "f16" else np.float32
+    x = synth.normal(seed, (b, d, s)).astype(np_dt)
+    w = synth.normal(seed + 1, (d, width), std=0.5).astype(np_dt)
+    bias = synth.normal(seed + 2, (d,), std=0.1).astype(np_dt)
+    got = host(ops.tensor_causal_conv1d(dev(x), dev(w), dev(bias))).astype(np.float32)
+    if dtype == "f16":
+        x, w, bias = (oracle.cvt_f16_to_f32(v) for v in (x, w, bias))
+    want = oracle.tensor_causal_conv1d(x, w, bias, threads=threads)
+    return got, want
+
+
+@pytest.mark.parametrize("dtype", ["f16", "f32"])
+@pytest.mark.parametrize("b,d,s,width", [(1, 1, 1, 1), (2, 3, 5, 4), (2, 5, 64, 4), (1, 7, 520, 3), (3, 4, 4096, 4),
+                                         (2, 3, 8192, 2), (1, 2, 12296, 4), (2, 6, 638, 4), (1, 3, 2048, 1),
+                                         (2, 2, 4104, 4), (1, 5, 33, 2)])
+def test_conv1d_shapes(ops, oracle, dtype, b, d, s, width):
+    got, want = _conv_case(ops, oracle, dtype, b, d, s, width, seed=b * 1000 + d * 100 + s)
+    tol = TOL_F16_ROWOPS if dtype == "f16" else TOL_F32
+    assert scaled_rel_err(got, want, 1.0) <= tol
+
+
+def test_conv1d_f32_reference_generator_shape(ops, oracle):
+    # tests/ext_torch_tests.cpp:745-778 (batch 8, dims 2318, seq 638, width 4), gate: abs tol 1e-3
+    got, want = _conv_case(ops, oracle, "f32", 8, 2318, 638, 4, seed=10)
+    ok, worst = oracle.compare_data_buffers(got, want)
+    assert ok, worst
+    assert scaled_rel_err(got, want, 1.0) <= TOL_F32
+
+
+def test_conv1d_config_zamba2_4x4224x4096_f16(ops, oracle):
+    import torch
+    b, d, s, width = 4, 4224, 4096, 4
+    x = synth.normal(0, (b, d, s)).astype(np.float16)
+    w = synth.normal(1, (d, width), std=0.5).astype(np.float16)
+    bias = synth.normal(2, (d,), std=0.1).astype(np.float16)
+    xd, wd, bd = dev(x), dev(w), dev(bias)
+    yd = ops.tensor_causal_conv1d(xd, wd, bd)
+    got = host(yd).astype(np.float32)
+    want = oracle.tensor_causal_conv1d(oracle.cvt_f16_to_f32(x), oracle.cvt_f16_to_f32(w), oracle.cvt_f16_to_f32(bias),
+                                       threads=16)
+    assert scaled_rel_err(got, want, 1.0) <= TOL_F16_ROWOPS
+    assert rel_l2(got, want) <= 1e-3
+    # causality at full size: perturbing one sample changes that row from there on, 4 samples long
+    xd2 = xd.clone()
+    xd2[2, 1234, 2047] += 1.0
+    yd2 = ops.tensor_causal_conv1d(xd2, wd, bd)
+    diff = (yd2 != yd).nonzero().cpu().numpy()
+    assert len(diff) > 0 and np.all(diff[:, 0] == 2) and np.all(diff[:, 1] == 1234)
+    assert diff[:, 2].min() >= 2047 and diff[:, 2].max() <= 2050
+
+
+def test_conv1d_empty_and_rejected_arguments(ops):
+    import torch
+    from anygpu_amd import capi
+    lib = capi.load()
+    x = torch.zeros((2, 3, 8), device="cuda", dtype=torch.float32)
+    w = torch.zeros((3, 4), device="cuda", dtype=torch.float32)
+    b = torch.zeros((3,), device="cuda", dtype=torch.float32)
+    y = torch.full((2, 3, 8), 3.0, device="cuda", dtype=torch.float32)
+    f = lib.anygpu_causal_conv1d_silu_f32
+    assert f(x.data_ptr(), w.data_ptr(), b.data_ptr(), y.data_ptr(), 2, 3, 8, 5, None) == capi.ANYGPU_ERR_UNSUPPORTED
+    assert f(x.data_ptr(), w.data_ptr(), b.data_ptr(), y.data_ptr(), 2, 3, 8, 0, None) == capi.ANYGPU_ERR_UNSUPPORTED
+    assert f(x.data_ptr(), None, b.data_ptr(), y.data_ptr(), 2, 3, 8, 4, None) == capi.ANYGPU_ERR_NULL_POINTER
+    assert f(x.data_ptr(), w.data_ptr(), b.data_ptr(), y.data_ptr(), 2, -3, 8, 4, None) == capi.ANYGPU_ERR_BAD_SHAPE
+    assert f(x.data_ptr(), w.data_ptr(), b.data_ptr(), y.data_ptr(), 0, 3, 8, 4, None) == capi.ANYGPU_OK
+    torch.cuda.synchronize()
+    assert bool((y == 3.0).all())
+    with pytest.raises(ValueError):
+        ops.tensor_causal_conv1d(x, torch.zeros((3, 5), device="cuda"), b)   # the reference's width assert
+
+
+# =============================================================================================
+# GEMM
+# =============================================================================================
+
+def test_mm_f32_reference_cases_integer_inputs_exact(ops, oracle):
+    # tests/tests.cpp:94-135: crt_random_tensor inputs (integers 0..10): sums are exact in float32
+    for (m, k, n) in [(40, 30, 50), (640, 1280, 320)]:
+        a = synth.integers(11, (m, k), 0, 10)
+        b = synth.integers(18, (k, n), 0, 10)
+        got = host(ops.tensor_mm(dev(a), dev(b)))
+        want = oracle.tensor_mm(a, b, threads=8)
+        assert np.array_equal(got, want)
+        assert np.array_equal(got.astype(np.int64), a.astype(np.int64) @ b.astype(np.int64))
+
+
+@pytest.mark.parametrize("layout", ["row", "col"])
+@pytest.mark.parametrize("m,k,n", [(1, 1, 1), (3, 5, 7), (128, 16, 128), (128, 48, 256), (130, 17, 129),
+                                   (256, 256, 256), (77, 300, 515), (512, 100, 64)])
+def test_mm_f32_shapes_and_layouts(ops, oracle, layout, m, k, n):
+    from anygpu_amd import capi
+    a = synth.uniform(m + k, (m, k))
+    if layout == "row":
+        b = synth.uniform(k + n, (k, n))
+        got = host(ops.tensor_mm(dev(a), dev(b)))
+        want = oracle.tensor_mm(a, b, threads=8)
+    else:
+        bt = synth.uniform(k + n, (n, k))
+        got = host(ops.tensor_mm(dev(a), dev(bt), b_layout=capi.B_COL_MAJOR))
+        want = oracle.tensor_mm(a, bt.T, threads=8)
+    floor = math.sqrt(k) / 3.0          # sigma_a * sigma_b * sqrt(K) for U(-1, 1): sigma^2 = 1/3
+    assert scaled_rel_err(got, want, floor) <= TOL_F32
+
+
+def test_gemm_f32_bias_and_padded_leading_dimensions(ops, oracle):
+    import torch
+    from anygpu_amd import capi
+    x = synth.integers(1, (50, 70), 0, 10)
+    w = synth.integers(2, (70, 90), 0, 10)
+    b = synth.integers(3, (90,), 0, 10)
+    got = host(ops.tensor_gemm(dev(x), dev(w), dev(b)))
+    assert np.array_equal(got, oracle.tensor_gemm(x, w, b))
+    # operands living inside wider buffers
+    abuf, bbuf = synth.uniform(4, (64, 200)), synth.uniform(5, (96, 300))
+    cbuf = torch.full((64, 400), -1.0, device="cuda")
+    ops.tensor_mm(dev(abuf)[:, :96], dev(bbuf)[:, :256], out=cbuf[:, :256])
+    got = host(cbuf)
+    want = oracle.tensor_mm(np.ascontiguousarray(abuf[:, :96]), np.ascontiguousarray(bbuf[:, :256]))
+    assert scaled_rel_err(got[:, :256], want, math.sqrt(96) / 3.0) <= TOL_F32
+    assert np.all(got[:, 256:] == -1.0)
+
+
+def test_mm_f32_config_2048_cubed(ops, oracle):
+    n = 2048
+    a = synth.uniform(0, (n, n))
+    b = synth.uniform(1, (n, n))
+    got = host(ops.tensor_mm(dev(a), dev(b)))
+    idx = sample_rows(n, 24, seed=2)
+    want = np.stack([oracle.tensor_mm(a[r:r + 1], b)[0] for r in idx])
+    assert scaled_rel_err(got[idx], want, math.sqrt(n) / 3.0) <= TOL_F32
+    # every row and column through a checksum: C @ 1 = A @ (B @ 1), 1^T C = (1^T A) B  (float64 on the host)
+    a64, b64 = a.astype(np.float64), b.astype(np.float64)
+    assert np.max(np.abs(got.astype(np.float64).sum(axis=1) - a64 @ b64.sum(axis=1))) < 1e-4 * n
+    assert np.max(np.abs(got.astype(np.float64).sum(axis=0) - a64.sum(axis=0) @ b64)) < 1e-4 * n
+
+
+def test_mm_f16_small_integer_inputs_bit_exact(ops, oracle):
+    # integers in {-2..2} and K <= 256: every partial sum is an integer of magnitude <= 1024, exact in
+    # fp32 and exactly representable in the fp16 output, whatever the tiling or summation order
+    from anygpu_amd import capi
+    for (m, k, n) in [(64, 64, 64), (256, 256, 256), (512, 128, 768), (100, 200, 60), (33, 17, 65)]:
+        a = synth.integers(m, (m, k), -2, 2, dtype=np.float16)
+        bt = synth.integers(n, (n, k), -2, 2, dtype=np.float16)
+        want = oracle.tensor_mm(oracle.cvt_f16_to_f32(a), oracle.cvt_f16_to_f32(bt).T)
+        got_nt = host(ops.tensor_mm(dev(a), dev(bt), b_layout=capi.B_COL_MAJOR)).astype(np.float32)
+        assert np.array_equal(got_nt, want), (m, k, n, "col-major B")
+        got_nn = host(ops.tensor_mm(dev(a), dev(np.ascontiguousarray(bt.T)))).astype(np.float32)
+        assert np.array_equal(got_nn, want), (m, k, n, "row-major B")
+
+
+def test_mm_f16_reference_case_640x1280_1280x320(ops, oracle):
+    # tests/tests.cpp:138-164: N(0,1) fp16 operands, CPU fp32 matmul of the up-cast inputs, rel-L2 <= 0.01
+    a = synth.normal(11, (640, 1280)).astype(np.float16)
+    b = synth.normal(18, (1280, 320)).astype(np.float16)
+    got = host(ops.tensor_mm(dev(a), dev(b))).astype(np.float32)
+    want = oracle.tensor_mm(oracle.cvt_f16_to_f32(a), oracle.cvt_f16_to_f32(b), threads=8)
+    ok, val = oracle.compare_data_buffers_l2(got, want, 0.01)
+    assert ok, val
+    assert scaled_rel_err(got, want, math.sqrt(1280)) <= TOL_F16_GEMM
+
+
+@pytest.mark.parametrize("m,k,n", [(256, 64, 256), (256, 128, 512), (768, 192, 1024), (1024, 1024, 1024)])
+def test_mm_f16_tile_kernel_shapes(ops, oracle, m, k, n):
+    from anygpu_amd import capi
+    a = synth.uniform(m + 1, (m, k)).astype(np.float16)
+    bt = synth.uniform(n + 2, (n, k)).astype(np.float16)
+    got = host(ops.tensor_mm(dev(a), dev(bt), b_layout=capi.B_COL_MAJOR)).astype(np.float32)
+    want = oracle.tensor_mm(oracle.cvt_f16_to_f32(a), oracle.cvt_f16_to_f32(bt).T, threads=8)
+    assert scaled_rel_err(got, want, math.sqrt(k) / 3.0) <= TOL_F16_GEMM
+    assert rel_l2(got, want) <= 1e-2
+
+
+def test_mm_f16_config_4096_cubed_col_major_b(ops, oracle):
+    from anygpu_amd import capi
+    n = 4096
+    a = synth.uniform(0, (n, n)).astype(np.float16)
+    bt = synth.uniform(1, (n, n)).astype(np.float16)      # B stored [N, K]
+    got = host(ops.tensor_mm(dev(a), dev(bt), b_layout=capi.B_COL_MAJOR)).astype(np.float32)
+    a32, bt32 = oracle.cvt_f16_to_f32(a), oracle.cvt_f16_to_f32(bt)
+    idx = sample_rows(n, 24, seed=3)
+    want = np.stack([oracle.tensor_mm(a32[r:r + 1], bt32.T)[0] for r in idx])
+    floor = math.sqrt(n) / 3.0
+    assert scaled_rel_err(got[idx], want, floor) <= TOL_F16_GEMM
+    assert rel_l2(got[idx], want) <= 1e-2
+    # checksums over every row and every column (fp16 output rounding: 2^-11 relative per element)
+    a64, b64 = a32.astype(np.float64), bt32.astype(np.float64)
+    row_sum = a64 @ b64.sum(axis=0)
+    col_sum = a64.sum(axis=0) @ b64.T
+    g64 = got.astype(np.float64)
+    tol = n * floor * 2.0 ** -11 * 4
+    assert np.max(np.abs(g64.sum(axis=1) - row_sum)) < tol
+    assert np.max(np.abs(g64.sum(axis=0) - col_sum)) < tol
+
+
+def test_mm_empty_and_rejected_arguments(ops):
+    import torch
+    from anygpu_amd import capi
+    lib = capi.load()
+    a = torch.zeros((4, 8), device="cuda", dtype=torch.float16)
+    b = torch.zeros((8, 4), device="cuda", dtype=torch.float16)
+    c = torch.full((4, 4), 3.0, device="cuda", dtype=torch.float16)
+    f = lib.anygpu_gemm_f16_f32acc
+    assert f(a.data_ptr(), b.data_ptr(), c.data_ptr(), 4, 4, 8, 4, 4, 4, 0, None) == capi.ANYGPU_ERR_BAD_STRIDE
+    assert f(a.data_ptr(), b.data_ptr(), c.data_ptr(), 4, 4, 8, 8, 4, 4, 7, None) == capi.ANYGPU_ERR_UNSUPPORTED
+    assert f(a.data_ptr(), None, c.data_ptr(), 4, 4, 8, 8, 4, 4, 0, None) == capi.ANYGPU_ERR_NULL_POINTER
+    assert f(a.data_ptr(), b.data_ptr(), c.data_ptr(), 4, -4, 8, 8, 4, 4, 0, None) == capi.ANYGPU_ERR_BAD_SHAPE
+    assert f(a.data_ptr(), b.data_ptr(), c.data_ptr(), 0, 4, 8, 8, 4, 4, 0, None) == capi.ANYGPU_OK
+    torch.cuda.synchronize()
+    assert bool((c == 3.0).all())
+    # K = 0: the product is all zeros
+    z = ops.tensor_mm(torch.zeros((4, 0), device="cuda", dtype=torch.float32), torch.zeros((0, 5), device="cuda"))
+    assert z.shape == (4, 5) and not bool(z.any())
+    with pytest.raises(ValueError):
+        ops.tensor_mm(torch.zeros((4, 8), device="cuda"), torch.zeros((7, 4), device="cuda"))

@@ -1,0 +1,376 @@
+"""Pins the CPU oracle against what the mathematics fixes: closed forms, invariants, special
+cases and independent brute force.  The reference holds no golden vectors for this path (its
+.dat fixtures are not in the repository and came from an unseeded generator), so these checks
+are what ties the oracle down; each is chosen so that a plausible slip (dropped term, wrong
+sign or index, transposed operand, wrong tap order) fails at least one of them.
+"""
+import math
+
+import numpy as np
+import pytest
+
+from anygpu_amd import synth
+
+
+# ---------------------------------------------------------------------------------------------
+# tensor_mm / tensor_gemm
+# ---------------------------------------------------------------------------------------------
+
+def test_mm_integer_inputs_bit_exact_vs_int64(oracle):
+    # values 0..10 and K <= 2304 keep every partial sum below 2^24: float32 sums are exact,
+    # so any correct implementation agrees bit for bit with integer arithmetic
+    for (m, k, n, sa, sb) in [(40, 30, 50, 11, 18), (64, 2304, 33, 1, 2), (7, 1, 5, 3, 4)]:
+        a = synth.integers(sa, (m, k), 0, 10)
+        b = synth.integers(sb, (k, n), 0, 10)
+        want = a.astype(np.int64) @ b.astype(np.int64)
+        got = oracle.tensor_mm(a, b)
+        assert np.array_equal(got.astype(np.int64), want)
+        gi = oracle.tensor_mm(a.astype(np.int32), b.astype(np.int32))
+        assert np.array_equal(gi.astype(np.int64), want)
+
+
+def test_mm_non_square_catches_transposed_operands(oracle):
+    # a product of distinct primes per position: swapping or transposing an operand changes the result
+    a = np.array([[1, 2, 3], [4, 5, 6]], dtype=np.float32)            # 2 x 3
+    b = np.array([[7, 8, 9, 10], [11, 12, 13, 14], [15, 16, 17, 18]], dtype=np.float32)  # 3 x 4
+    want = np.array([[74, 80, 86, 92], [173, 188, 203, 218]], dtype=np.float32)
+    assert np.array_equal(oracle.tensor_mm(a, b), want)
+
+
+def test_mm_identity_ones_pattern(oracle):
+    n = 37
+    eye = np.eye(n, dtype=np.float32)
+    x = synth.normal(5, (n, n))
+    assert np.array_equal(oracle.tensor_mm(eye, x), x)
+    assert np.array_equal(oracle.tensor_mm(x, eye), x)
+    ones = np.ones((9, 123), dtype=np.float32)
+    assert np.array_equal(oracle.tensor_mm(ones, ones.T.copy()), np.full((9, 9), 123, dtype=np.float32))
+    # crt_pattern_tensor: element ix holds ix % 10 (srcs/core/tensor.hpp:514-528)
+    pa = (np.arange(6 * 20) % 10).astype(np.float32).reshape(6, 20)
+    pb = (np.arange(20 * 4) % 10).astype(np.float32).reshape(20, 4)
+    want = np.array([[sum(((r * 20 + l) % 10) * ((l * 4 + c) % 10) for l in range(20)) for c in range(4)]
+                     for r in range(6)], dtype=np.float32)
+    assert np.array_equal(oracle.tensor_mm(pa, pb), want)
+
+
+def test_mm_strided_views_equal_explicit_copies(oracle):
+    a = synth.normal(1, (17, 29))
+    bt = synth.normal(2, (23, 29))          # B stored [N, K]
+    via_view = oracle.tensor_mm(a, bt.T)    # strides (1, K): column-major B
+    via_copy = oracle.tensor_mm(a, np.ascontiguousarray(bt.T))
+    assert np.array_equal(via_view, via_copy)
+    wide = synth.normal(3, (17, 64))
+    assert np.array_equal(oracle.tensor_mm(wide[:, :29], bt.T), oracle.tensor_mm(wide[:, :29].copy(), bt.T))
+
+
+def test_mm_normal_inputs_within_float32_summation_bound(oracle):
+    m, k, n = 33, 512, 41
+    a = synth.normal(0, (m, k))
+    b = synth.normal(1, (k, n))
+    got = oracle.tensor_mm(a, b).astype(np.float64)
+    exact = a.astype(np.float64) @ b.astype(np.float64)
+    bound = k * 2.0 ** -24 * (np.abs(a).astype(np.float64) @ np.abs(b).astype(np.float64))
+    assert np.all(np.abs(got - exact) <= bound)
+    # and it is the sequential float32 sum, not a pairwise or float64 one
+    seq = np.zeros((m, n), dtype=np.float32)
+    for l in range(k):
+        seq += np.outer(a[:, l], b[l, :]).astype(np.float32)
+    assert np.array_equal(oracle.tensor_mm(a, b), seq)
+
+
+def test_mm_float64_elements_use_float32_accumulator(oracle):
+    a = synth.normal(3, (5, 300)).astype(np.float64)
+    b = synth.normal(4, (300, 6)).astype(np.float64)
+    got = oracle.tensor_mm(a, b)
+    acc = np.zeros((5, 6), dtype=np.float32)
+    for l in range(300):
+        acc = (acc.astype(np.float64) + np.outer(a[:, l], b[l, :])).astype(np.float32)
+    assert np.array_equal(got, acc.astype(np.float64))
+
+
+def test_mm_row_range_and_threads_do_not_change_values(oracle):
+    a = synth.normal(6, (64, 100))
+    b = synth.normal(7, (100, 48))
+    full = oracle.tensor_mm(a, b)
+    part = oracle.tensor_mm(a, b, rows=(10, 20))
+    assert np.array_equal(part[10:20], full[10:20]) and not part[:10].any() and not part[20:].any()
+    assert np.array_equal(oracle.tensor_mm(a, b, threads=4), full)
+
+
+def test_gemm_bias_is_added_per_column(oracle):
+    x = synth.integers(1, (6, 9), 0, 10)
+    w = synth.integers(2, (9, 4), 0, 10)
+    b = np.array([1, 20, 300, 4000], dtype=np.float32)
+    want = (x.astype(np.int64) @ w.astype(np.int64) + b.astype(np.int64)[None, :]).astype(np.float32)
+    assert np.array_equal(oracle.tensor_gemm(x, w, b), want)
+
+
+# ---------------------------------------------------------------------------------------------
+# tensor_softmax and the prologue primitives
+# ---------------------------------------------------------------------------------------------
+
+def test_softmax_rows_sum_to_one_and_shift_invariant(oracle):
+    x = synth.normal(0, (13, 257), std=3.0)
+    y = oracle.tensor_softmax(x)
+    assert np.all(np.abs(y.sum(axis=1, dtype=np.float64) - 1.0) <= 257 * 2.0 ** -24)
+    assert np.all(y >= 0)
+    x8 = np.round(x * 8) / 8          # multiples of 1/8: adding 4 is exact in float32
+    assert np.array_equal(oracle.tensor_softmax(x8), oracle.tensor_softmax(x8 + np.float32(4.0)))
+
+
+def test_softmax_constant_rows_are_exactly_one_over_n(oracle):
+    for n in (1, 2, 64, 1024):
+        x = np.full((3, n), 1.75, dtype=np.float32)
+        assert np.array_equal(oracle.tensor_softmax(x), np.full((3, n), 1.0 / n, dtype=np.float32))
+
+
+def test_softmax_two_values_closed_form_and_order(oracle):
+    for delta in (0.5, 1.0, 3.25, 10.0):
+        x = np.array([[0.0, delta], [delta, 0.0]], dtype=np.float32)
+        y = oracle.tensor_softmax(x).astype(np.float64)
+        big = 1.0 / (1.0 + math.exp(-delta))
+        assert abs(y[0, 1] - big) < 2e-7 and abs(y[0, 0] - (1 - big)) < 2e-7
+        assert abs(y[1, 0] - big) < 2e-7 and abs(y[1, 1] - (1 - big)) < 2e-7
+
+
+def test_softmax_one_hot_limit_and_masked_entries_are_exact_zero(oracle):
+    x = np.array([[0.0, 200.0, -5.0], [-np.inf, 2.0, -np.inf], [np.finfo(np.float32).min, 1.0, 1.0]], dtype=np.float32)
+    y = oracle.tensor_softmax(x)
+    assert np.array_equal(y[0], np.array([0, 1, 0], dtype=np.float32))
+    assert np.array_equal(y[1], np.array([0, 1, 0], dtype=np.float32))
+    assert np.array_equal(y[2], np.array([0, 0.5, 0.5], dtype=np.float32))
+
+
+def test_softmax_vs_long_double_brute_force(oracle):
+    x = synth.normal(4, (9, 61), std=2.0)
+    y = oracle.tensor_softmax(x)
+    xl = x.astype(np.longdouble)
+    e = np.exp(xl - xl.max(axis=1, keepdims=True))
+    want = e / e.sum(axis=1, keepdims=True)
+    assert np.max(np.abs(y.astype(np.longdouble) - want)) < 61 * 2.0 ** -23
+    y64 = oracle.tensor_softmax(x.astype(np.float64))
+    assert np.max(np.abs(y64.astype(np.longdouble) - want)) < 1e-15
+
+
+def test_softmax_strided_input(oracle):
+    big = synth.normal(5, (6, 40))
+    assert np.array_equal(oracle.tensor_softmax(big[:, :31]), oracle.tensor_softmax(big[:, :31].copy()))
+    # column step: softmax over every second element
+    assert np.array_equal(oracle.tensor_softmax(big[:, ::2]), oracle.tensor_softmax(big[:, ::2].copy()))
+
+
+def test_mul_and_add_are_elementwise(oracle):
+    x = synth.normal(1, (4, 5))
+    y = synth.normal(2, (4, 5))
+    assert np.array_equal(oracle.tensor_mul_scalar(x, 0.125), x * np.float32(0.125))
+    assert np.array_equal(oracle.tensor_add(x, y), x + y)
+
+
+def test_softcap_properties(oracle):
+    cap = 50.0
+    x = synth.normal(3, (1000,), std=40.0)
+    y = oracle.softcap(x, cap)
+    assert np.array_equal(oracle.softcap(-x, cap), -y)                        # odd
+    assert np.all(np.abs(y) <= cap) and np.all(np.abs(y[np.abs(x) < 100]) < cap)
+    assert np.all(np.sign(y) == np.sign(x))
+    want = cap * np.tanh(x.astype(np.float64) / cap)
+    assert np.max(np.abs(y - want)) < 1e-5 * cap
+    half = np.array([cap * math.atanh(0.5)], dtype=np.float32)
+    assert abs(float(oracle.softcap(half, cap)[0]) - cap / 2) < 1e-5 * cap
+    tiny = np.array([1e-3, -2e-3], dtype=np.float32)
+    assert np.allclose(oracle.softcap(tiny, cap), tiny, rtol=1e-6)              # y -> x as x/cap -> 0
+    # a different cap changes the value: cap is not ignored, and it is not tanh(x) * cap
+    assert abs(float(oracle.softcap(np.array([30.0], dtype=np.float32), 30.0)[0]) - 30 * math.tanh(1.0)) < 1e-4
+
+
+def test_causal_and_slide_mask_rules(oracle):
+    q = k = 9
+    cm = oracle.causal_mask(q, k)
+    for i in range(q):
+        for j in range(k):
+            assert cm[i, j] == (0.0 if j <= i else -np.inf)
+    # sliding window: row i keeps keys {j : i - W < j <= i}; count = min(i + 1, W)
+    window = 4
+    sm = oracle.slide_mask(cm[None, None], window)[0, 0]
+    lowest = np.finfo(np.float32).min
+    for i in range(q):
+        visible = [j for j in range(k) if sm[i, j] == 0.0]
+        assert visible == [j for j in range(k) if i - window < j <= i]
+        assert len(visible) == min(i + 1, window)
+        for j in range(k):
+            if j <= i - window:
+                assert sm[i, j] == lowest
+    # the generator's shape: [5, 1, 121, 41] with W = 34; rule == tril(diagonal=-W)
+    rng_mask = synth.normal(8, (5, 1, 121, 41))
+    out = oracle.slide_mask(rng_mask, 34)
+    tril = np.tril(np.ones((121, 41), dtype=bool), k=-34)
+    want = np.where(tril[None, None], lowest, rng_mask)
+    assert np.array_equal(out, want)
+
+
+def test_attention_softmax_is_the_stated_composition(oracle):
+    rows, cols, q_len = 24, 12, 12
+    x = synth.normal(2, (rows, cols), std=16.0)
+    alpha, cap, window = 1.0 / 16.0, 50.0, 5
+    got = oracle.attention_softmax(x, alpha=alpha, softcap=cap, causal=True, window=window, q_len=q_len)
+    # composed by hand from the separately pinned primitives
+    s = oracle.tensor_mul_scalar(x, alpha)
+    s = oracle.softcap(s, cap).reshape(rows, cols)
+    mask = oracle.slide_mask(oracle.causal_mask(q_len, cols), window)
+    mask = np.tile(mask, (rows // q_len, 1))
+    want = oracle.tensor_softmax(oracle.tensor_add(s, mask))
+    assert np.array_equal(got, want)
+    # float64 brute force of the same formula
+    z = cap * np.tanh(x.astype(np.float64) * alpha / cap)
+    i = (np.arange(rows) % q_len)[:, None]
+    j = np.arange(cols)[None, :]
+    vis = (j <= i) & (j > i - window)
+    z = np.where(vis, z, -np.inf)
+    e = np.exp(z - z.max(axis=1, keepdims=True))
+    brute = e / e.sum(axis=1, keepdims=True)
+    assert np.max(np.abs(got - brute)) < 1e-6
+    assert np.all(got[~vis] == 0.0)
+    assert got[0, 0] == 1.0 and not got[0, 1:].any()       # first causal row is [1, 0, ...]
+    # row subset returns exactly those rows
+    idx = np.array([3, 17, 23])
+    sub = oracle.attention_softmax(x, alpha=alpha, softcap=cap, causal=True, window=window, q_len=q_len, row_index=idx)
+    assert np.array_equal(sub, got[idx])
+    # without softcap / masks it is plain softmax of the scaled input
+    plain = oracle.attention_softmax(x, alpha=0.125)
+    assert np.array_equal(plain, oracle.tensor_softmax(oracle.tensor_mul_scalar(x, 0.125)))
+
+
+# ---------------------------------------------------------------------------------------------
+# tensor_causal_conv1d
+# ---------------------------------------------------------------------------------------------
+
+def _silu64(v):
+    v = np.asarray(v, dtype=np.float64)
+    return v / (1.0 + np.exp(-v))
+
+
+def test_conv1d_impulse_response_reads_taps_backwards(oracle):
+    b, d, s, w = 1, 3, 10, 4
+    x = np.zeros((b, d, s), dtype=np.float32)
+    x[:, :, 0] = 1.0
+    wt = np.array([[1, 2, 3, 4], [-1, 0.5, 0.25, 2], [0.1, 0.2, 0.3, 0.4]], dtype=np.float32)
+    bt = np.array([0.5, -0.25, 0.0], dtype=np.float32)
+    y = oracle.tensor_causal_conv1d(x, wt, bt)
+    for ch in range(d):
+        for t in range(s):
+            pre = (wt[ch, w - 1 - t] if t < w else 0.0) + bt[ch]
+            assert abs(y[0, ch, t] - _silu64(pre)) < 1e-6
+
+
+def test_conv1d_special_weights(oracle):
+    b, d, s = 2, 5, 33
+    x = synth.normal(1, (b, d, s))
+    bt = synth.normal(2, (d,), std=0.1)
+    w_pass = np.zeros((d, 4), dtype=np.float32)
+    w_pass[:, 3] = 1.0                                  # only the current-sample tap
+    y = oracle.tensor_causal_conv1d(x, w_pass, bt)
+    assert np.max(np.abs(y - _silu64(x.astype(np.float64) + bt[None, :, None]))) < 1e-6
+    w_zero = np.zeros((d, 4), dtype=np.float32)
+    y0 = oracle.tensor_causal_conv1d(x, w_zero, bt)
+    assert np.max(np.abs(y0 - _silu64(bt)[None, :, None])) < 1e-6
+    w_delay = np.zeros((d, 4), dtype=np.float32)
+    w_delay[:, 0] = 1.0                                 # tap 0 is the sample three steps back
+    yd = oracle.tensor_causal_conv1d(x, w_delay, np.zeros(d, dtype=np.float32))
+    assert np.max(np.abs(yd[:, :, 3:] - _silu64(x[:, :, :-3]))) < 1e-6
+    assert not yd[:, :, :3].any()                       # silu(0) = 0 in the padded region
+
+
+def test_conv1d_is_causal_and_depthwise(oracle):
+    b, d, s = 2, 4, 40
+    x = synth.normal(3, (b, d, s))
+    wt = synth.normal(4, (d, 4), std=0.5)
+    bt = synth.normal(5, (d,), std=0.1)
+    y = oracle.tensor_causal_conv1d(x, wt, bt)
+    x2 = x.copy()
+    x2[1, 2, 17] += 1.0
+    y2 = oracle.tensor_causal_conv1d(x2, wt, bt)
+    changed = np.argwhere(y != y2)
+    assert set(map(tuple, changed)) == {(1, 2, 17), (1, 2, 18), (1, 2, 19), (1, 2, 20)}
+
+
+def test_conv1d_vs_float64_zero_padded_brute_force(oracle):
+    for width in (1, 2, 3, 4):
+        b, d, s = 2, 7, 29
+        x = synth.normal(6, (b, d, s))
+        wt = synth.normal(7, (d, width), std=0.5)
+        bt = synth.normal(8, (d,), std=0.1)
+        y = oracle.tensor_causal_conv1d(x, wt, bt)
+        xp = np.concatenate([np.zeros((b, d, width - 1)), x.astype(np.float64)], axis=2)
+        pre = np.zeros((b, d, s))
+        for k in range(width):
+            pre += wt[None, :, k, None].astype(np.float64) * xp[:, :, k:k + s]
+        pre += bt[None, :, None]
+        assert np.max(np.abs(y - _silu64(pre))) < 2e-6
+        y64 = oracle.tensor_causal_conv1d(x.astype(np.float64), wt.astype(np.float64), bt.astype(np.float64))
+        assert np.max(np.abs(y64 - _silu64(pre))) < 1e-14
+
+
+def test_conv1d_preactivation_is_linear_in_x(oracle):
+    # with zero bias and small inputs silu is invertible on the image; compare pre-activations
+    b, d, s = 1, 3, 20
+    x1 = synth.integers(1, (b, d, s), -3, 3)
+    x2 = synth.integers(2, (b, d, s), -3, 3)
+    wt = synth.integers(3, (d, 4), -2, 2)
+    zero = np.zeros(d, dtype=np.float32)
+
+    def pre(x):
+        # integer taps and samples: recover the exact integer pre-activation by brute force
+        xp = np.concatenate([np.zeros((b, d, 3)), x], axis=2)
+        return sum(wt[None, :, k, None] * xp[:, :, k:k + s] for k in range(4))
+
+    for x in (x1, x2, x1 + x2):
+        y = oracle.tensor_causal_conv1d(x.astype(np.float32), wt, zero)
+        assert np.max(np.abs(y - _silu64(pre(x)))) < 1e-5
+    assert np.array_equal(pre(x1 + x2), pre(x1) + pre(x2))
+
+
+def test_conv1d_reference_generator_shape_vs_torch_formula(oracle):
+    # scripts/fused_test_cases.py:31-41: batch 8, dims 2318, seq_len 638, width 4 and the one-line torch formula
+    torch = pytest.importorskip("torch")
+    import torch.nn.functional as F
+    b, d, s, width = 8, 2318, 638, 4
+    x = synth.normal(10, (b, d, s))
+    wt = synth.normal(11, (d, width))
+    bt = synth.normal(12, (d,))
+    y = oracle.tensor_causal_conv1d(x, wt, bt, threads=8)
+    tx, tw, tb = (torch.from_numpy(v).double() for v in (x, wt, bt))
+    want = F.silu(F.conv1d(tx, tw.unsqueeze(1), tb, stride=1, padding=width - 1, groups=d))[:, :, :s].numpy()
+    assert np.max(np.abs(y - want)) < 1e-5
+    ok, _ = oracle.compare_data_buffers(y, want.astype(np.float32))      # the reference's own gate: abs 1e-3
+    assert ok
+
+
+# ---------------------------------------------------------------------------------------------
+# fp16 up-cast and comparators
+# ---------------------------------------------------------------------------------------------
+
+def test_f16_upcast_all_bit_patterns(oracle):
+    bits = np.arange(65536, dtype=np.uint16)
+    want = bits.view(np.float16).astype(np.float32)
+    got = oracle.cvt_f16_to_f32(bits.view(np.float16))
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32)) or \
+        np.array_equal(got[~np.isnan(want)], want[~np.isnan(want)])
+    assert np.all(np.isnan(got[np.isnan(want)]))
+
+
+def test_comparators_hand_computed(oracle):
+    e = np.array([1.0, 2.0, 4.0], dtype=np.float32)
+    a = np.array([1.0005, 2.0, 3.9995], dtype=np.float32)
+    ok, worst = oracle.compare_data_buffers(a, e)                 # abs tol 1e-3
+    assert ok and abs(worst - 5e-4) < 1e-6
+    ok, _ = oracle.compare_data_buffers(a, e, abs_tol=4e-4)
+    assert not ok
+    a2 = np.array([1.02, 2.0, 4.0], dtype=np.float32)
+    ok, worst = oracle.compare_data_buffers_reldiff(a2, e)        # 2 % off on the first element
+    assert not ok and abs(worst - 0.02) < 1e-5
+    ok, worst = oracle.compare_data_buffers_reldiff(np.array([1.005, 2.0, 4.0], dtype=np.float32), e)
+    assert ok and abs(worst - 0.005) < 1e-5
+    ok, val = oracle.compare_data_buffers_l2(a2, e)               # sqrt(0.0004 / 21)
+    assert ok and abs(val - math.sqrt(0.0004 / 21.0)) < 1e-6
+    ok, val = oracle.compare_data_buffers_l2(np.array([2.0, 2.0, 4.0], dtype=np.float32), e)
+    assert not ok and abs(val - math.sqrt(1.0 / 21.0)) < 1e-6
