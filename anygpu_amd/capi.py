@@ -60,6 +60,14 @@ def load() -> ctypes.CDLL:
         raise RuntimeError(
             f"{LIB_PATH} is not built; run `python -c 'import __graft_entry__ as g; g.build()'` "
             "(or python anygpu_amd/build.py) first. There is no CPU fallback.")
+    # One HIP runtime per process: PyTorch wheels carry their own libamdhip64 (same soname as the
+    # system one).  If torch is going to be used for device memory it has to be loaded before this
+    # library, so that both resolve to the single runtime already mapped; loaded the other way
+    # round, torch maps a second runtime and streams / device state are no longer shared.
+    try:
+        import torch  # noqa: F401
+    except ImportError:
+        pass
     lib = ctypes.CDLL(str(LIB_PATH))
     for name, (restype, argtypes) in SIGNATURES.items():
         fn = getattr(lib, name)  # AttributeError if the symbol is not exported

@@ -167,6 +167,7 @@ static hipError_t launch_width(const void* x, const void* w, const void* bias, v
 		const int64_t blocks = rows * tiles_per_row;
 		if (blocks <= 0x7FFFFFFFLL)
 		{
+			discard_stale_error();
 			causal_conv1d_silu_tile_kernel<T, WIDTH, U><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(
 				xp, wp, bp, yp, (int)chan, (int)seqlen, (int)tiles_per_row);
 			return hipGetLastError();
@@ -174,6 +175,7 @@ static hipError_t launch_width(const void* x, const void* w, const void* bias, v
 	}
 	const int64_t total = rows * seqlen;
 	const int64_t blocks = (total + 255) / 256;
+	discard_stale_error();
 	causal_conv1d_silu_element_kernel<T, WIDTH><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(
 		xp, wp, bp, yp, (int)chan, (int)seqlen, total);
 	return hipGetLastError();

@@ -27,6 +27,12 @@ __device__ __forceinline__ float dpp_move(float v)
 		__builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
 }
 
+// Value of `v` in lane `lane` as a wave-uniform scalar (the builtin moves 32 raw bits).
+__device__ __forceinline__ float read_lane(float v, int lane)
+{
+	return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
+}
+
 struct MaxOp { __device__ __forceinline__ float operator()(float a, float b) const { return fmaxf(a, b); } };
 struct SumOp { __device__ __forceinline__ float operator()(float a, float b) const { return a + b; } };
 
@@ -40,10 +46,10 @@ __device__ __forceinline__ float wave_allreduce(float v, Op op)
 	v = op(v, dpp_move<0x4E>(v));    // quad_perm [2,3,0,1]
 	v = op(v, dpp_move<0x124>(v));   // row_ror:4
 	v = op(v, dpp_move<0x128>(v));   // row_ror:8
-	float r0 = __builtin_amdgcn_readlane(v, 0);
-	float r1 = __builtin_amdgcn_readlane(v, 16);
-	float r2 = __builtin_amdgcn_readlane(v, 32);
-	float r3 = __builtin_amdgcn_readlane(v, 48);
+	const float r0 = read_lane(v, 0);
+	const float r1 = read_lane(v, 16);
+	const float r2 = read_lane(v, 32);
+	const float r3 = read_lane(v, 48);
 	return op(op(r0, r1), op(r2, r3));
 }
 

@@ -262,6 +262,7 @@ static hipError_t launch_tile(const half_t* A, const half_t* B, half_t* C, int64
 	using Cfg = TileCfg<BM, BN, BK, WM, WN>;
 	auto kernel = gemm_f16_nt_tile_kernel<BM, BN, BK, WM, WN>;
 	static bool configured = false;
+	discard_stale_error();
 	if (!configured)
 	{
 		hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
@@ -292,6 +293,7 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
 	}
 
 	const dim3 grid((unsigned)((N + 63) / 64), (unsigned)((M + 63) / 64));
+	discard_stale_error();
 	if (b_layout == ANYGPU_B_COL_MAJOR)
 		gemm_f16_edge_kernel<ANYGPU_B_COL_MAJOR><<<grid, dim3(256), 0, stream>>>(a, b, c, M, N, K, lda, ldb, ldc);
 	else

@@ -223,6 +223,7 @@ static hipError_t launch_layout(const float* A, const float* B, const float* bia
 	const bool aligned = (reinterpret_cast<uintptr_t>(A) % 16 == 0) && (reinterpret_cast<uintptr_t>(B) % 16 == 0) &&
 	                     (reinterpret_cast<uintptr_t>(C) % 16 == 0) && (lda % 4 == 0) && (ldb % 4 == 0) && (ldc % 4 == 0);
 	const bool full = aligned && (M % kBM == 0) && (N % kBN == 0) && (K % kBK == 0);
+	discard_stale_error();
 	if (full)
 		gemm_f32_kernel<B_LAYOUT, true><<<grid, dim3(256), 0, stream>>>(A, B, bias, C, M, N, K, lda, ldb, ldc);
 	else

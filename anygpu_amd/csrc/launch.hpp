@@ -7,6 +7,11 @@
 
 namespace anygpu {
 
+// The runtime keeps the last error of the calling thread until somebody reads it, whoever
+// caused it.  Launchers call this before their own launch so that the code they return
+// afterwards (hipGetLastError) belongs to that launch and to nothing earlier in the process.
+inline void discard_stale_error() { (void)hipGetLastError(); }
+
 template <typename T>
 hipError_t launch_softmax_rows(const void* x, void* y, int64_t rows, int64_t cols, int64_t xs, int64_t ys,
                                int64_t q_len, int64_t diag, float alpha, float softcap, int causal,

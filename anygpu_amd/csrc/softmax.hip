@@ -209,6 +209,7 @@ template <typename T, int VPL>
 static hipError_t launch_wave(const SoftmaxArgs& a, hipStream_t stream)
 {
 	const unsigned blocks = (unsigned)((a.rows + 3) / 4);
+	discard_stale_error();
 	softmax_rows_wave_kernel<T, VPL><<<dim3(blocks), dim3(256), 0, stream>>>(a);
 	return hipGetLastError();
 }
@@ -242,6 +243,7 @@ hipError_t launch_softmax_rows(const void* x, void* y, int64_t rows, int64_t col
 		if (nvec <= kWaveSize * 16) return launch_wave<T, 16>(a, stream);
 		if constexpr (kMaxVpl >= 32) return launch_wave<T, 32>(a, stream);
 	}
+	discard_stale_error();
 	softmax_rows_block_kernel<T><<<dim3((unsigned)rows), dim3(256), 0, stream>>>(a);
 	return hipGetLastError();
 }
