@@ -25,6 +25,7 @@ OBJ_DIR = LIB_DIR / "obj"
 INCLUDE_DIR = REPO_DIR / "include"
 ORACLE_DIR = REPO_DIR / "oracle"
 
+ROCM_DIR = Path(os.environ.get("ROCM_PATH", "/opt/rocm"))
 GPU_ARCH = "gfx950"
 KERNEL_SOURCES = ["softmax.hip", "conv1d.hip", "gemm_f16.hip", "gemm_f32.hip", "capi.hip"]
 
@@ -82,11 +83,14 @@ def build_host_harness(verbose: bool = False) -> Path | None:
     sources = sorted(str(p) for p in (HOST_DIR / "core").glob("*.cpp"))
     sources += sorted(str(p) for p in (HOST_DIR / "kernels").glob("*.cpp"))
     sources += sorted(str(p) for p in (HOST_DIR / "harness").glob("*.cpp"))
-    includes = [f"-I{INCLUDE_DIR}"] + [f"-I{HOST_DIR / d}" for d in ("core", "ops", "fused", "kernels", "io", "harness")]
+    includes = [f"-I{INCLUDE_DIR}", f"-I{ROCM_DIR / 'include'}"]
+    includes += [f"-I{HOST_DIR / d}" for d in ("core", "ops", "fused", "kernels", "io", "harness")]
     out = LIB_DIR / "anygpu_host_tests"
-    _run([hipcc, "-x", "c++", "-std=c++20", "-O2", "-DAC_WITH_ASSERT", "-D__HIP_PLATFORM_AMD__", *includes, *sources,
-          "-o", str(out), f"-L{LIB_DIR}", "-lanygpu_hip", "-L/opt/rocm/lib", "-lamdhip64",
-          f"-Wl,-rpath,$ORIGIN", "-Wl,-rpath,/opt/rocm/lib"], quiet=not verbose)
+    # host-only C++ (no device code): the ROCm clang, which knows _Float16 on x86-64
+    clangxx = ROCM_DIR / "lib" / "llvm" / "bin" / "clang++"
+    _run([str(clangxx), "-std=c++20", "-O2", "-DAC_WITH_ASSERT", "-D__HIP_PLATFORM_AMD__", "-Wall", "-Wno-unused-function",
+          *includes, *sources, "-o", str(out), f"-L{LIB_DIR}", "-lanygpu_hip", f"-L{ROCM_DIR / 'lib'}", "-lamdhip64",
+          "-Wl,-rpath,$ORIGIN", f"-Wl,-rpath,{ROCM_DIR / 'lib'}"], quiet=not verbose)
     return out
 
 

@@ -18,6 +18,8 @@ ANYGPU_ERR_BAD_STRIDE = -3
 ANYGPU_ERR_UNSUPPORTED = -4
 ANYGPU_ERR_TOO_LARGE = -5
 
+A_ROW_MAJOR = 0
+A_COL_MAJOR = 1
 B_ROW_MAJOR = 0
 B_COL_MAJOR = 1
 
@@ -29,7 +31,7 @@ SIGNATURES = {
     "anygpu_gemm_f16_f32acc": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64,
                                        c_int64, c_int64, c_int64, c_int, c_void_p]),
     "anygpu_gemm_f32": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64,
-                                c_int64, c_int64, c_int64, c_int, c_void_p]),
+                                c_int64, c_int64, c_int64, c_int, c_int, c_void_p]),
     "anygpu_softmax_rows_f16": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,
                                         c_float, c_float, c_int, c_int64, c_void_p]),
     "anygpu_softmax_rows_f32": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,

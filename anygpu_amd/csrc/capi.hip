@@ -14,14 +14,15 @@ constexpr int64_t kMaxIndex32 = 0x7FFFFFFFLL;
 inline hipStream_t as_stream(void* s) { return static_cast<hipStream_t>(s); }
 
 int check_gemm(const void* A, const void* B, const void* C, int64_t M, int64_t N, int64_t K,
-               int64_t lda, int64_t ldb, int64_t ldc, int b_layout)
+               int64_t lda, int64_t ldb, int64_t ldc, int a_layout, int b_layout)
 {
 	if (M < 0 || N < 0 || K < 0) return ANYGPU_ERR_BAD_SHAPE;
+	if (a_layout != ANYGPU_A_ROW_MAJOR && a_layout != ANYGPU_A_COL_MAJOR) return ANYGPU_ERR_UNSUPPORTED;
 	if (b_layout != ANYGPU_B_ROW_MAJOR && b_layout != ANYGPU_B_COL_MAJOR) return ANYGPU_ERR_UNSUPPORTED;
 	if (M == 0 || N == 0) return ANYGPU_OK;
 	if (C == nullptr) return ANYGPU_ERR_NULL_POINTER;
 	if (K > 0 && (A == nullptr || B == nullptr)) return ANYGPU_ERR_NULL_POINTER;
-	if (lda < K || ldc < N) return ANYGPU_ERR_BAD_STRIDE;
+	if (lda < (a_layout == ANYGPU_A_ROW_MAJOR ? K : M) || ldc < N) return ANYGPU_ERR_BAD_STRIDE;
 	if (ldb < (b_layout == ANYGPU_B_ROW_MAJOR ? N : K)) return ANYGPU_ERR_BAD_STRIDE;
 	// the grids index 64- or 128-wide tiles with 16-bit y and 31-bit x block numbers
 	if (M > 65535LL * 64 || N > kMaxIndex32 || K > kMaxIndex32) return ANYGPU_ERR_TOO_LARGE;
@@ -104,7 +105,7 @@ ANYGPU_EXPORT int anygpu_gemm_f16_f32acc(const void* A, const void* B, void* C,
                                          int64_t lda, int64_t ldb, int64_t ldc,
                                          int b_layout, void* stream)
 {
-	const int rc = check_gemm(A, B, C, M, N, K, lda, ldb, ldc, b_layout);
+	const int rc = check_gemm(A, B, C, M, N, K, lda, ldb, ldc, ANYGPU_A_ROW_MAJOR, b_layout);
 	if (rc != ANYGPU_OK) return rc;
 	return (int)anygpu::launch_gemm_f16(A, B, C, M, N, K, lda, ldb, ldc, b_layout, as_stream(stream));
 }
@@ -112,11 +113,12 @@ ANYGPU_EXPORT int anygpu_gemm_f16_f32acc(const void* A, const void* B, void* C,
 ANYGPU_EXPORT int anygpu_gemm_f32(const float* A, const float* B, const float* bias, float* C,
                                   int64_t M, int64_t N, int64_t K,
                                   int64_t lda, int64_t ldb, int64_t ldc,
-                                  int b_layout, void* stream)
+                                  int a_layout, int b_layout, void* stream)
 {
-	const int rc = check_gemm(A, B, C, M, N, K, lda, ldb, ldc, b_layout);
+	const int rc = check_gemm(A, B, C, M, N, K, lda, ldb, ldc, a_layout, b_layout);
 	if (rc != ANYGPU_OK) return rc;
-	return (int)anygpu::launch_gemm_f32(A, B, bias, C, M, N, K, lda, ldb, ldc, b_layout, as_stream(stream));
+	return (int)anygpu::launch_gemm_f32(A, B, bias, C, M, N, K, lda, ldb, ldc, a_layout, b_layout,
+	                                    as_stream(stream));
 }
 
 ANYGPU_EXPORT int anygpu_softmax_rows_f16(const void* x, void* y, int64_t rows, int64_t cols,

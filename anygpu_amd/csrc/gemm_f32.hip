@@ -2,11 +2,13 @@
 // lane supplies one A and one B value per instruction, lanes 0-31 the even and lanes 32-63
 // the odd k of a 2-deep step).  True fp32 products and sums; no reduced-precision tricks.
 //
-// Block tile 128 x 128 x 16, 4 waves, each wave a 64 x 64 patch (2 x 2 MFMA tiles).  A is
-// staged in LDS as [m][16 k] rows, B as [16 k][n] rows for the row-major layout (lanes walk
-// n) or as [n][16 k] rows for the column-major layout.  Inside a slab the lower lane half
-// consumes k = 0..7 and the upper half k = 8..15, one per instruction, so a lane reads its 8
-// A values with two 16-byte LDS loads.
+// Block tile 128 x 128 x 16, 4 waves, each wave a 64 x 64 patch (2 x 2 MFMA tiles).  An
+// operand slab is staged in LDS in the orientation it has in memory: "k-contiguous" operands
+// (row-major A, column-major B) as [row][16 k] rows, "row-contiguous" operands (column-major
+// A, row-major B) as [16 k][row] rows.  Inside a slab the lower lane half consumes k = 0..7
+// and the upper half k = 8..15, one per instruction, so a lane reads its 8 values of a
+// k-contiguous operand with two 16-byte LDS loads and of a row-contiguous operand with eight
+// conflict-free 4-byte loads.
 // The same kernel serves any shape: FULL = true assumes whole tiles and 16-byte aligned
 // rows (vector global loads), FULL = false guards every global access.
 #include "device_utils.hpp"
@@ -17,15 +19,83 @@ namespace anygpu {
 
 constexpr int kBM = 128, kBN = 128, kBK = 16;
 constexpr int kPitchK = kBK + 4;     // floats per [row][k] LDS row: 80 bytes, keeps 16-byte alignment
-constexpr int kPitchN = kBN + 4;     // floats per [k][n] LDS row
+constexpr int kPitchR = 128 + 4;     // floats per [k][row] LDS row
 
-template <int B_LAYOUT, bool FULL>
+// One 128-row x 16-deep operand slab.  KCONTIG: element (row, k) at base[row * ld + k];
+// otherwise at base[k * ld + row].  `rows` / `depth` are the valid extents from the slab origin.
+template <bool KCONTIG, bool FULL>
+struct Slab
+{
+	static constexpr int kLdsFloats = KCONTIG ? 128 * kPitchK : kBK * kPitchR;
+
+	// global -> registers: 512 float4 per slab, 2 per thread
+	__device__ static void load(float4_t (&reg)[2], const float* __restrict__ base, int64_t ld,
+	                            int64_t rows, int64_t depth, int tid)
+	{
+#pragma unroll
+		for (int i = 0; i < 2; ++i)
+		{
+			const int q = tid + 256 * i;
+			const int r = KCONTIG ? (q >> 2) : (q & 31) * 4;       // first row covered
+			const int k = KCONTIG ? (q & 3) * 4 : (q >> 5);        // first k covered
+			if (FULL)
+			{
+				reg[i] = *reinterpret_cast<const float4_t*>(KCONTIG ? base + r * ld + k : base + k * ld + r);
+			}
+			else
+			{
+#pragma unroll
+				for (int e = 0; e < 4; ++e)
+				{
+					const int rr = KCONTIG ? r : r + e;
+					const int kk = KCONTIG ? k + e : k;
+					reg[i][e] = (rr < rows && kk < depth) ? (KCONTIG ? base[rr * ld + kk] : base[kk * ld + rr]) : 0.0f;
+				}
+			}
+		}
+	}
+
+	__device__ static void store(float* lds, const float4_t (&reg)[2], int tid)
+	{
+#pragma unroll
+		for (int i = 0; i < 2; ++i)
+		{
+			const int q = tid + 256 * i;
+			if (KCONTIG)
+				*reinterpret_cast<float4_t*>(&lds[(q >> 2) * kPitchK + (q & 3) * 4]) = reg[i];
+			else
+				*reinterpret_cast<float4_t*>(&lds[(q >> 5) * kPitchR + (q & 31) * 4]) = reg[i];
+		}
+	}
+
+	// the 8 values row `row` contributes for k = kb .. kb + 7
+	__device__ static void fragment(float (&v)[8], const float* lds, int row, int kb)
+	{
+		if (KCONTIG)
+		{
+			const float* src = &lds[row * kPitchK + kb];
+			const float4_t lo = *reinterpret_cast<const float4_t*>(src);
+			const float4_t hi = *reinterpret_cast<const float4_t*>(src + 4);
+#pragma unroll
+			for (int e = 0; e < 4; ++e) { v[e] = lo[e]; v[4 + e] = hi[e]; }
+		}
+		else
+		{
+#pragma unroll
+			for (int e = 0; e < 8; ++e) v[e] = lds[(kb + e) * kPitchR + row];
+		}
+	}
+};
+
+template <int A_LAYOUT, int B_LAYOUT, bool FULL>
 __global__ __launch_bounds__(256) void gemm_f32_kernel(
 	const float* __restrict__ A, const float* __restrict__ B, const float* __restrict__ bias, float* __restrict__ C,
 	int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc)
 {
-	__shared__ __align__(16) float a_lds[2][kBM * kPitchK];
-	__shared__ __align__(16) float b_lds[2][(B_LAYOUT == ANYGPU_B_COL_MAJOR) ? kBN * kPitchK : kBK * kPitchN];
+	using SlabA = Slab<A_LAYOUT == ANYGPU_A_ROW_MAJOR, FULL>;
+	using SlabB = Slab<B_LAYOUT == ANYGPU_B_COL_MAJOR, FULL>;
+	__shared__ __align__(16) float a_lds[2][SlabA::kLdsFloats];
+	__shared__ __align__(16) float b_lds[2][SlabB::kLdsFloats];
 
 	const int tid = threadIdx.x;
 	const int lane = tid & (kWaveSize - 1);
@@ -34,86 +104,12 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(
 	const int64_t m0 = (int64_t)blockIdx.y * kBM;
 	const int64_t n0 = (int64_t)blockIdx.x * kBN;
 
-	// staging registers: A slab 128 x 16 = 512 float4 -> 2 per thread; B slab likewise
-	float4_t ra[2], rb[2];
+	const float* a_base = (A_LAYOUT == ANYGPU_A_ROW_MAJOR) ? A + m0 * lda : A + m0;
+	const float* b_base = (B_LAYOUT == ANYGPU_B_COL_MAJOR) ? B + n0 * ldb : B + n0;
+	auto a_at = [&](int64_t k0) { return (A_LAYOUT == ANYGPU_A_ROW_MAJOR) ? a_base + k0 : a_base + k0 * lda; };
+	auto b_at = [&](int64_t k0) { return (B_LAYOUT == ANYGPU_B_COL_MAJOR) ? b_base + k0 : b_base + k0 * ldb; };
 
-	auto load_a = [&](int64_t k0) {
-#pragma unroll
-		for (int i = 0; i < 2; ++i)
-		{
-			const int q = tid + 256 * i;         // float4 index: row q / 4, k-quad q % 4
-			const int r = q >> 2, c = (q & 3) * 4;
-			const int64_t m = m0 + r;
-			if (FULL)
-			{
-				ra[i] = *reinterpret_cast<const float4_t*>(A + m * lda + k0 + c);
-			}
-			else
-			{
-#pragma unroll
-				for (int e = 0; e < 4; ++e)
-					ra[i][e] = (m < M && k0 + c + e < K) ? A[m * lda + k0 + c + e] : 0.0f;
-			}
-		}
-	};
-	auto load_b = [&](int64_t k0) {
-#pragma unroll
-		for (int i = 0; i < 2; ++i)
-		{
-			const int q = tid + 256 * i;
-			if (B_LAYOUT == ANYGPU_B_COL_MAJOR)
-			{
-				const int r = q >> 2, c = (q & 3) * 4;   // row = n, quad along k
-				const int64_t n = n0 + r;
-				if (FULL)
-				{
-					rb[i] = *reinterpret_cast<const float4_t*>(B + n * ldb + k0 + c);
-				}
-				else
-				{
-#pragma unroll
-					for (int e = 0; e < 4; ++e)
-						rb[i][e] = (n < N && k0 + c + e < K) ? B[n * ldb + k0 + c + e] : 0.0f;
-				}
-			}
-			else
-			{
-				const int r = q >> 5, c = (q & 31) * 4;  // row = k, quad along n
-				const int64_t k = k0 + r;
-				if (FULL)
-				{
-					rb[i] = *reinterpret_cast<const float4_t*>(B + k * ldb + n0 + c);
-				}
-				else
-				{
-#pragma unroll
-					for (int e = 0; e < 4; ++e)
-						rb[i][e] = (k < K && n0 + c + e < N) ? B[k * ldb + n0 + c + e] : 0.0f;
-				}
-			}
-		}
-	};
-	auto store_slab = [&](int buf) {
-#pragma unroll
-		for (int i = 0; i < 2; ++i)
-		{
-			const int q = tid + 256 * i;
-			{
-				const int r = q >> 2, c = (q & 3) * 4;
-				*reinterpret_cast<float4_t*>(&a_lds[buf][r * kPitchK + c]) = ra[i];
-			}
-			if (B_LAYOUT == ANYGPU_B_COL_MAJOR)
-			{
-				const int r = q >> 2, c = (q & 3) * 4;
-				*reinterpret_cast<float4_t*>(&b_lds[buf][r * kPitchK + c]) = rb[i];
-			}
-			else
-			{
-				const int r = q >> 5, c = (q & 31) * 4;
-				*reinterpret_cast<float4_t*>(&b_lds[buf][r * kPitchN + c]) = rb[i];
-			}
-		}
-	};
+	float4_t ra[2], rb[2];
 
 	float16_t acc[2][2];
 #pragma unroll
@@ -129,9 +125,10 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(
 
 	if (ktiles > 0)
 	{
-		load_a(0);
-		load_b(0);
-		store_slab(0);
+		SlabA::load(ra, a_at(0), lda, M - m0, K, tid);
+		SlabB::load(rb, b_at(0), ldb, N - n0, K, tid);
+		SlabA::store(a_lds[0], ra, tid);
+		SlabB::store(b_lds[0], rb, tid);
 	}
 	__syncthreads();
 
@@ -140,38 +137,16 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(
 		const int buf = (int)(kt & 1);
 		if (kt + 1 < ktiles)
 		{
-			load_a((kt + 1) * kBK);
-			load_b((kt + 1) * kBK);
+			const int64_t k1 = (kt + 1) * kBK;
+			SlabA::load(ra, a_at(k1), lda, M - m0, K - k1, tid);
+			SlabB::load(rb, b_at(k1), ldb, N - n0, K - k1, tid);
 		}
 
 		float av[2][8], bv[2][8];
 #pragma unroll
-		for (int i = 0; i < 2; ++i)
-		{
-			const float* src = &a_lds[buf][(wm * 64 + i * 32 + frag_row) * kPitchK + kb];
-			const float4_t lo = *reinterpret_cast<const float4_t*>(src);
-			const float4_t hi = *reinterpret_cast<const float4_t*>(src + 4);
+		for (int i = 0; i < 2; ++i) SlabA::fragment(av[i], a_lds[buf], wm * 64 + i * 32 + frag_row, kb);
 #pragma unroll
-			for (int e = 0; e < 4; ++e) { av[i][e] = lo[e]; av[i][4 + e] = hi[e]; }
-		}
-#pragma unroll
-		for (int j = 0; j < 2; ++j)
-		{
-			const int n = wn * 64 + j * 32 + frag_row;
-			if (B_LAYOUT == ANYGPU_B_COL_MAJOR)
-			{
-				const float* src = &b_lds[buf][n * kPitchK + kb];
-				const float4_t lo = *reinterpret_cast<const float4_t*>(src);
-				const float4_t hi = *reinterpret_cast<const float4_t*>(src + 4);
-#pragma unroll
-				for (int e = 0; e < 4; ++e) { bv[j][e] = lo[e]; bv[j][4 + e] = hi[e]; }
-			}
-			else
-			{
-#pragma unroll
-				for (int e = 0; e < 8; ++e) bv[j][e] = b_lds[buf][(kb + e) * kPitchN + n];
-			}
-		}
+		for (int j = 0; j < 2; ++j) SlabB::fragment(bv[j], b_lds[buf], wn * 64 + j * 32 + frag_row, kb);
 #pragma unroll
 		for (int e = 0; e < 8; ++e)
 #pragma unroll
@@ -180,7 +155,11 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(
 				for (int j = 0; j < 2; ++j)
 					acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(bv[j][e], av[i][e], acc[i][j], 0, 0, 0);
 
-		if (kt + 1 < ktiles) store_slab(buf ^ 1);
+		if (kt + 1 < ktiles)
+		{
+			SlabA::store(a_lds[buf ^ 1], ra, tid);
+			SlabB::store(b_lds[buf ^ 1], rb, tid);
+		}
 		__syncthreads();
 	}
 
@@ -214,7 +193,7 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(
 	}
 }
 
-template <int B_LAYOUT>
+template <int A_LAYOUT, int B_LAYOUT>
 static hipError_t launch_layout(const float* A, const float* B, const float* bias, float* C,
                                 int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc,
                                 hipStream_t stream)
@@ -225,20 +204,26 @@ static hipError_t launch_layout(const float* A, const float* B, const float* bia
 	const bool full = aligned && (M % kBM == 0) && (N % kBN == 0) && (K % kBK == 0);
 	discard_stale_error();
 	if (full)
-		gemm_f32_kernel<B_LAYOUT, true><<<grid, dim3(256), 0, stream>>>(A, B, bias, C, M, N, K, lda, ldb, ldc);
+		gemm_f32_kernel<A_LAYOUT, B_LAYOUT, true><<<grid, dim3(256), 0, stream>>>(A, B, bias, C, M, N, K, lda, ldb, ldc);
 	else
-		gemm_f32_kernel<B_LAYOUT, false><<<grid, dim3(256), 0, stream>>>(A, B, bias, C, M, N, K, lda, ldb, ldc);
+		gemm_f32_kernel<A_LAYOUT, B_LAYOUT, false><<<grid, dim3(256), 0, stream>>>(A, B, bias, C, M, N, K, lda, ldb, ldc);
 	return hipGetLastError();
 }
 
 hipError_t launch_gemm_f32(const float* A, const float* B, const float* bias, float* C,
                            int64_t M, int64_t N, int64_t K,
-                           int64_t lda, int64_t ldb, int64_t ldc, int b_layout, hipStream_t stream)
+                           int64_t lda, int64_t ldb, int64_t ldc, int a_layout, int b_layout, hipStream_t stream)
 {
 	if (M == 0 || N == 0) return hipSuccess;
+	if (a_layout == ANYGPU_A_ROW_MAJOR)
+	{
+		if (b_layout == ANYGPU_B_COL_MAJOR)
+			return launch_layout<ANYGPU_A_ROW_MAJOR, ANYGPU_B_COL_MAJOR>(A, B, bias, C, M, N, K, lda, ldb, ldc, stream);
+		return launch_layout<ANYGPU_A_ROW_MAJOR, ANYGPU_B_ROW_MAJOR>(A, B, bias, C, M, N, K, lda, ldb, ldc, stream);
+	}
 	if (b_layout == ANYGPU_B_COL_MAJOR)
-		return launch_layout<ANYGPU_B_COL_MAJOR>(A, B, bias, C, M, N, K, lda, ldb, ldc, stream);
-	return launch_layout<ANYGPU_B_ROW_MAJOR>(A, B, bias, C, M, N, K, lda, ldb, ldc, stream);
+		return launch_layout<ANYGPU_A_COL_MAJOR, ANYGPU_B_COL_MAJOR>(A, B, bias, C, M, N, K, lda, ldb, ldc, stream);
+	return launch_layout<ANYGPU_A_COL_MAJOR, ANYGPU_B_ROW_MAJOR>(A, B, bias, C, M, N, K, lda, ldb, ldc, stream);
 }
 
 }  // namespace anygpu

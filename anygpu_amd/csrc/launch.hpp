@@ -27,6 +27,6 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
 
 hipError_t launch_gemm_f32(const float* A, const float* B, const float* bias, float* C,
                            int64_t M, int64_t N, int64_t K,
-                           int64_t lda, int64_t ldb, int64_t ldc, int b_layout, hipStream_t stream);
+                           int64_t lda, int64_t ldb, int64_t ldc, int a_layout, int b_layout, hipStream_t stream);
 
 }  // namespace anygpu

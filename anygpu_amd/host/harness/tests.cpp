@@ -1,0 +1,464 @@
+// Test cases of the host layer, in the style of the reference harness (tests/tests.cpp,
+// tests/ext_torch_tests.cpp): build inputs with a seeded factory, run the GPU overload, copy back,
+// run the CPU overload on the same data, compare with the harness comparators, print
+// "TestCase [name]: PASSED|FAILED".  Unlike the reference, every case also returns its verdict so
+// that the process exit code reflects failures.
+#include "harness.hpp"
+
+#include "ops.hpp"
+#include "fast_mm.cuh"
+#include "dat_file.hpp"
+#include "test_tools.hpp"
+
+#include <cstdio>
+#include <limits>
+
+namespace {
+
+// Column-major view of a dense [N, K] host tensor as the [K, N] matrix it stores.
+template<typename T>
+Tensor<T, CPU> as_transposed_view(const Tensor<T, CPU>& t_nk)
+{
+	Tensor<T, CPU> v = t_nk;
+	v.shape = { t_nk.shape[1], t_nk.shape[0] };
+	v.stride = { t_nk.stride[1], t_nk.stride[0] };
+	return v;
+}
+
+template<typename T>
+Tensor<T, CPU> transposed_copy(const Tensor<T, CPU>& x)
+{
+	Tensor<T, CPU> y(std::vector<int64>({ x.shape[1], x.shape[0] }));
+	for (int64 r = 0; r < x.shape[0]; ++r)
+		for (int64 c = 0; c < x.shape[1]; ++c)
+			y.buffer()[c * y.stride[0] + r] = x.buffer()[r * x.stride[0] + c];
+	return y;
+}
+
+// Additive mask of an attention block on the host: -inf above the (shifted) diagonal, float
+// lowest for keys that fell out of the sliding window.
+Tensor<float32, CPU> build_mask(int64 q_len, int64 k_len, bool causal, int64 window, int64 diag)
+{
+	Tensor<float32, CPU> mask(std::vector<int64>({ q_len, k_len }));
+	for (int64 i = 0; i < q_len; ++i)
+		for (int64 j = 0; j < k_len; ++j)
+		{
+			float32 v = 0.f;
+			if (causal && j > i + diag) v = -std::numeric_limits<float32>::infinity();
+			if (window > 0 && (i + diag) >= window && j <= i + diag - window) v = std::numeric_limits<float32>::lowest();
+			mask.buffer()[i * k_len + j] = v;
+		}
+	return mask;
+}
+
+// softcap(x, cap) = tanhf(x / cap) * cap, elementwise on the host
+Tensor<float32, CPU> host_softcap(const Tensor<float32, CPU>& x, float32 cap)
+{
+	Tensor<float32, CPU> y(x.dim, x.shape, x.stride);
+	for (int64 ix = 0; ix < x.size(); ++ix) y.buffer()[ix] = tanhf(x.buffer()[ix] / cap) * cap;
+	return y;
+}
+
+}  // namespace
+
+/* ------------------------------------------------------------------ host-only cases ---- */
+
+TEST_CASE(test_cpu_mm_f32_256x512_512x1024, HOST)
+{
+	// fp32 matmul on the CPU path with N(0,1) operands, seed 0, checked elementwise against a
+	// float64 product with the bound K * 2^-24 * sum |a| |b|
+	auto a = crt_random_normal_tensor<float32, CPU>({ 256, 512 }, 0);
+	auto b = crt_random_normal_tensor<float32, CPU>({ 512, 1024 }, 0);
+	auto c = tensor_mm(a, b);
+	bool ok = c.shape[0] == 256 && c.shape[1] == 1024;
+	for (int64 r = 0; r < 256 && ok; ++r)
+		for (int64 col = 0; col < 1024; ++col)
+		{
+			double exact = 0.0, mag = 0.0;
+			for (int64 l = 0; l < 512; ++l)
+			{
+				const double p = (double)a.buffer()[r * 512 + l] * (double)b.buffer()[l * 1024 + col];
+				exact += p;
+				mag += std::abs(p);
+			}
+			if (std::abs((double)c.buffer()[r * 1024 + col] - exact) > 512 * std::ldexp(1.0, -24) * mag) { ok = false; break; }
+		}
+	return ok;
+}
+
+TEST_CASE(test_cpu_mm_pattern_and_strides, HOST)
+{
+	auto a = crt_pattern_tensor<float32, CPU>({ 6, 20 });
+	auto b = crt_pattern_tensor<float32, CPU>({ 20, 4 });
+	auto c = tensor_mm(a, b);
+	bool ok = true;
+	for (int64 r = 0; r < 6; ++r)
+		for (int64 col = 0; col < 4; ++col)
+		{
+			int64 want = 0;
+			for (int64 l = 0; l < 20; ++l) want += ((r * 20 + l) % 10) * ((l * 4 + col) % 10);
+			ok = ok && c.buffer()[r * 4 + col] == (float32)want;
+		}
+	// a transposed view multiplies like the explicit transpose
+	auto bt = transposed_copy(b);                       // [4, 20]
+	auto c2 = tensor_mm(a, as_transposed_view(bt));
+	ok = ok && compare_data_buffers(c2, c, 1e-6f);
+	// int32 matrices go through the same loops
+	auto ai = crt_random_tensor<int32, CPU>({ 5, 7 }, 3);
+	auto bi = crt_random_tensor<int32, CPU>({ 7, 3 }, 4);
+	auto ci = tensor_mm(ai, bi);
+	for (int64 r = 0; r < 5; ++r)
+		for (int64 col = 0; col < 3; ++col)
+		{
+			int32 want = 0;
+			for (int64 l = 0; l < 7; ++l) want += ai.buffer()[r * 7 + l] * bi.buffer()[l * 3 + col];
+			ok = ok && ci.buffer()[r * 3 + col] == want;
+		}
+	return ok;
+}
+
+TEST_CASE(test_cpu_softmax_properties, HOST)
+{
+	auto x = crt_random_normal_tensor<float32, CPU>({ 13, 257 }, 4);
+	auto y = tensor_softmax(x);
+	bool ok = true;
+	for (int64 r = 0; r < 13; ++r)
+	{
+		double s = 0.0;
+		for (int64 c = 0; c < 257; ++c) s += y.buffer()[r * 257 + c];
+		ok = ok && std::abs(s - 1.0) < 1e-5;
+	}
+	auto ones = crt_ones_tensor<float32, CPU>({ 3, 64 });
+	auto u = tensor_softmax(ones);
+	for (int64 ix = 0; ix < 3 * 64; ++ix) ok = ok && u.buffer()[ix] == 1.0f / 64;
+	return ok;
+}
+
+TEST_CASE(test_cpu_causal_conv1d_impulse, HOST)
+{
+	Tensor<float32, CPU> x(std::vector<int64>({ 1, 2, 8 }));
+	x.buffer()[0] = 1.f;
+	x.buffer()[8] = 1.f;
+	Tensor<float32, CPU> w({ 2, 4 }, std::vector<float32>({ 1, 2, 3, 4, -1, 0.5f, 0.25f, 2 }));
+	Tensor<float32, CPU> b({ 2 }, std::vector<float32>({ 0.5f, -0.25f }));
+	auto y = tensor_causal_conv1d(x, w, b);
+	bool ok = true;
+	for (int64 d = 0; d < 2; ++d)
+		for (int64 t = 0; t < 8; ++t)
+		{
+			const float32 pre = (t < 4 ? w.buffer()[d * 4 + 3 - t] : 0.f) + b.buffer()[d];
+			const float32 want = pre / (1.f + std::exp(-pre));
+			ok = ok && std::abs(y.buffer()[d * 8 + t] - want) < 1e-6f;
+		}
+	return ok;
+}
+
+TEST_CASE(test_tensor_views_and_linear_cpu, HOST)
+{
+	auto x = crt_pattern_tensor<float32, CPU>({ 2, 3, 4 });
+	auto v = tensor_view(x, { 6, 4 });
+	bool ok = v.buffer() == x.buffer() && v.buffer_id() == x.buffer_id() && v.dim == 2 && v.stride[0] == 4;
+	auto parts = tensor_split(tensor_view(x, { 2, 3, 4 }), 2);
+	ok = ok && parts.size() == 2 && parts[1].buffer() == x.buffer() + 12 && parts[1].shape[0] == 1;
+	auto w = crt_random_tensor<float32, CPU>({ 4, 5 }, 1);
+	auto bias = crt_random_tensor<float32, CPU>({ 5 }, 2);
+	auto y = tensor_linear(x, w, bias);                 // (2, 3, 4) x (4, 5) + (5) -> (2, 3, 5)
+	ok = ok && y.dim == 3 && y.shape[0] == 2 && y.shape[1] == 3 && y.shape[2] == 5;
+	auto y2 = tensor_gemm(v, w, bias);
+	ok = ok && compare_data_buffers(tensor_view(y, { 6, 5 }), y2, 1e-6f);
+	auto y3 = tensor_linear(x, w);
+	ok = ok && compare_data_buffers(tensor_view(y3, { 6, 5 }), tensor_mm(v, w), 1e-6f);
+	return ok;
+}
+
+TEST_CASE(test_small_float_types, HOST)
+{
+	bool ok = true;
+	// every finite code of both fp8 formats survives a decode / encode round trip
+	for (int code = 0; code < 256; ++code)
+	{
+		fp8e4m3 a; a.bits = (uint8_t)code;
+		fp8e5m2 b; b.bits = (uint8_t)code;
+		const float fa = (float)a, fb = (float)b;
+		if (!std::isnan(fa)) ok = ok && fp8e4m3(fa).bits == a.bits;
+		if (!std::isnan(fb)) ok = ok && fp8e5m2(fb).bits == b.bits;
+	}
+	ok = ok && (float)fp8e4m3(448.f) == 448.f && (float)fp8e4m3(1000.f) == 448.f;      // E4M3 saturates at 448
+	ok = ok && (float)fp8e5m2(57344.f) == 57344.f && std::isinf((float)fp8e5m2(1e6f));
+	ok = ok && (float)fp8e4m3(0.3f) == 0.3125f && (float)fp8e5m2(0.3f) == 0.3125f;
+	ok = ok && (float)bfloat16(1.0f) == 1.0f && (float)bfloat16(3.140625f) == 3.140625f;
+	ok = ok && (float)bfloat16(1.00390625f) == 1.0f;                                    // tie rounds to even
+	ok = ok && cvt_any_to_float32((float16)0.5f) == 0.5f;
+	ok = ok && get_datatype_enum<float16>() == DataType::FLOAT16 && represent_datatype<bfloat16>() == "BFLOAT16";
+	ok = ok && sizeof(float16) == 2 && sizeof(bfloat16) == 2 && sizeof(fp8e4m3) == 1;
+	return ok;
+}
+
+TEST_CASE(test_comparators, HOST)
+{
+	Tensor<float32, CPU> e({ 3 }, std::vector<float32>({ 1.f, 2.f, 4.f }));
+	Tensor<float32, CPU> a({ 3 }, std::vector<float32>({ 1.0005f, 2.f, 3.9995f }));
+	Tensor<float32, CPU> a2({ 3 }, std::vector<float32>({ 1.02f, 2.f, 4.f }));
+	bool ok = compare_data_buffers(a, e);
+	std::cout << "(the next mismatch lines are expected)\n";
+	ok = ok && !compare_data_buffers(a, e, 4e-4f);
+	ok = ok && !compare_data_buffers_reldiff(a2, e) && compare_data_buffers_reldiff(a, e);
+	ok = ok && compare_data_buffers_l2(a2, e) && !compare_data_buffers_l2(a2, e, 0.004f);
+	Tensor<int32, CPU> ie({ 3 }, std::vector<int32>({ 1, 2, 3 }));
+	Tensor<int32, CPU> ia({ 3 }, std::vector<int32>({ 1, 2, 4 }));
+	ok = ok && compare_data_buffers(ie, ie) && !compare_data_buffers(ia, ie);
+	return ok;
+}
+
+TEST_CASE(test_dat_file_roundtrip, HOST)
+{
+	const std::string path = (std::filesystem::temp_directory_path() / "anygpu_roundtrip.dat").string();
+	auto x = crt_random_normal_tensor<float32, CPU>({ 3, 5, 7 }, 9);
+	save_tensor(x, path);
+	auto y = load_tensor<float32>(path);
+	bool ok = elementwise_compatible(x, y) && std::memcmp(x.buffer(), y.buffer(), sizeof(float32) * x.numel()) == 0;
+	// byte layout: dim, shape..., dtype code 5, data
+	std::ifstream f(path, std::ios::binary);
+	int32 head[5];
+	f.read(reinterpret_cast<char*>(head), sizeof(head));
+	ok = ok && head[0] == 3 && head[1] == 3 && head[2] == 5 && head[3] == 7 && head[4] == 5;
+	auto h = cvt_tensor_from_float32<float16>(x);
+	save_tensor(h, path);
+	auto h2 = load_tensor<float16>(path);
+	ok = ok && std::memcmp(h.buffer(), h2.buffer(), 2 * h.numel()) == 0;
+	std::remove(path.c_str());
+	return ok;
+}
+
+/* Cases that must stop the process with exit code 1 (run one at a time by name). */
+
+TEST_CASE(death_mm_shape_mismatch, DEATH)
+{
+	auto a = crt_ones_tensor<float32, CPU>({ 4, 5 });
+	auto b = crt_ones_tensor<float32, CPU>({ 6, 3 });
+	auto c = tensor_mm(a, b);
+	return c.dim == 2;
+}
+
+TEST_CASE(death_softmax_not_2d, DEATH)
+{
+	auto x = crt_ones_tensor<float32, CPU>({ 2, 3, 4 });
+	auto y = tensor_softmax(x);
+	return y.dim == 2;
+}
+
+TEST_CASE(death_conv1d_channel_mismatch, DEATH)
+{
+	auto x = crt_ones_tensor<float32, CPU>({ 2, 3, 8 });
+	auto w = crt_ones_tensor<float32, CPU>({ 4, 4 });
+	auto b = crt_ones_tensor<float32, CPU>({ 4 });
+	auto y = tensor_causal_conv1d(x, w, b);
+	return y.dim == 3;
+}
+
+TEST_CASE(death_missing_dat_file, DEATH)
+{
+	auto x = load_tensor<float32>("/nonexistent/anygpu/tensor.dat");
+	return x.dim > 0;
+}
+
+/* ------------------------------------------------------------------ GPU cases ---- */
+
+TEST_CASE(test_mm_f32, GPU)
+{
+	auto dta = crt_random_tensor<float32, CUDA>({ 40, 30 }, 11);
+	auto dtb = crt_random_tensor<float32, CUDA>({ 30, 50 }, 18);
+	auto dtc = tensor_mm(dta, dtb);
+
+	auto hta = dta.copy_to_host();
+	auto htb = dtb.copy_to_host();
+	auto htc = tensor_mm(hta, htb);
+
+	auto htc_from_cuda = dtc.copy_to_host();
+	return elementwise_compatible(htc_from_cuda, htc) && compare_data_buffers(htc_from_cuda, htc);
+}
+
+TEST_CASE(test_mm_f32_640x1280_1280x320, GPU)
+{
+	auto dta = crt_random_tensor<float32, CUDA>({ 640, 1280 }, 11);
+	auto dtb = crt_random_tensor<float32, CUDA>({ 1280, 320 }, 18);
+	auto dtc = tensor_mm(dta, dtb);
+
+	auto htc = tensor_mm(dta.copy_to_host(), dtb.copy_to_host());
+	auto htc_from_cuda = dtc.copy_to_host();
+	return elementwise_compatible(htc_from_cuda, htc) && compare_data_buffers(htc_from_cuda, htc);
+}
+
+TEST_CASE(test_mm_f16_640x1280_1280x320, GPU)
+{
+	auto dta = crt_random_normal_tensor<float16, CUDA>({ 640, 1280 }, 11);
+	auto dtb = crt_random_normal_tensor<float16, CUDA>({ 1280, 320 }, 18);
+	auto dtc = tensor_mm(dta, dtb);
+
+	// no half arithmetic on the host: up-cast the same half inputs and multiply in float32
+	auto hta = cvt_tensor_datatype<float32, float16>(dta.copy_to_host());
+	auto htb = cvt_tensor_datatype<float32, float16>(dtb.copy_to_host());
+	auto htc = tensor_mm(hta, htb);
+
+	auto htc_from_cuda = cvt_tensor_datatype<float32, float16>(dtc.copy_to_host());
+	return elementwise_compatible(htc_from_cuda, htc) && compare_data_buffers_l2(htc_from_cuda, htc, 0.01f);
+}
+
+TEST_CASE(test_mm_nt_f16_512x256_768, GPU)
+{
+	// B handed over as its [N, K] storage; the tile kernel path (multiples of 256 / 64)
+	auto dta = crt_random_normal_tensor<float16, CUDA>({ 512, 256 }, 5);
+	auto dtb_nk = crt_random_normal_tensor<float16, CUDA>({ 768, 256 }, 6);
+	auto dtc = tensor_mm_nt(dta, dtb_nk);
+
+	auto hta = cvt_tensor_datatype<float32, float16>(dta.copy_to_host());
+	auto htb_nk = cvt_tensor_datatype<float32, float16>(dtb_nk.copy_to_host());
+	auto htc = tensor_mm(hta, as_transposed_view(htb_nk));
+
+	auto htc_from_cuda = cvt_tensor_datatype<float32, float16>(dtc.copy_to_host());
+	return elementwise_compatible(htc_from_cuda, htc) && compare_data_buffers_l2(htc_from_cuda, htc, 0.01f);
+}
+
+TEST_CASE(test_gemm_and_linear_f32, GPU)
+{
+	auto dx = crt_random_tensor<float32, CUDA>({ 4, 9, 70 }, 1);
+	auto dw = crt_random_tensor<float32, CUDA>({ 70, 90 }, 2);
+	auto db = crt_random_tensor<float32, CUDA>({ 90 }, 3);
+	auto dy = tensor_linear(dx, dw, db);
+	auto dy_nobias = tensor_linear(dx, dw);
+
+	auto hx = dx.copy_to_host();
+	auto hw = dw.copy_to_host();
+	auto hb = db.copy_to_host();
+	auto hy = tensor_linear(hx, hw, hb);
+	auto hy_nobias = tensor_linear(hx, hw);
+
+	auto got = dy.copy_to_host();
+	auto got_nobias = dy_nobias.copy_to_host();
+	bool ok = got.dim == 3 && got.shape[2] == 90;
+	ok = ok && elementwise_compatible(got, hy) && compare_data_buffers(got, hy);
+	ok = ok && elementwise_compatible(got_nobias, hy_nobias) && compare_data_buffers(got_nobias, hy_nobias);
+	return ok;
+}
+
+TEST_CASE(test_fast_mm_entry_points, GPU)
+{
+	// the rung the reference's float32 golden test drives takes the left operand transposed;
+	// the one its float16 test drives is checked with rel-L2 4 %
+	auto hx = crt_random_normal_tensor<float32, CPU>({ 256, 384 }, 21);
+	auto hw = crt_random_normal_tensor<float32, CPU>({ 384, 128 }, 22);
+	auto hy = tensor_mm(hx, hw);
+	auto dx = hx.copy_to_cuda();
+	auto dw = hw.copy_to_cuda();
+	bool ok = true;
+
+	Tensor<float32, CUDA> dy(hy.dim, hy.shape);
+	cu_fast_mm_f32_v4_1(dx, dw, dy);
+	ok = ok && compare_data_buffers(dy.copy_to_host(), hy);
+
+	auto dx_tr = transposed_copy(hx).copy_to_cuda();    // [K, M]
+	Tensor<float32, CUDA> dy2(hy.dim, hy.shape);
+	cu_fast_mm_f32_v4_2(dx_tr, dw, dy2);
+	ok = ok && compare_data_buffers(dy2.copy_to_host(), hy);
+
+	auto hx16 = cvt_tensor_from_float32<float16>(hx);
+	auto hw16 = cvt_tensor_from_float32<float16>(hw);
+	auto hy16_ref = tensor_mm(cvt_tensor_datatype<float32, float16>(hx16), cvt_tensor_datatype<float32, float16>(hw16));
+	Tensor<float16, CUDA> dy16(hy.dim, hy.shape);
+	cu_fast_mm_f16_v3_2(hx16.copy_to_cuda(), hw16.copy_to_cuda(), dy16);
+	ok = ok && compare_data_buffers_l2(cvt_tensor_datatype<float32, float16>(dy16.copy_to_host()), hy16_ref, 0.04f);
+	return ok;
+}
+
+TEST_CASE(test_softmax_f32, GPU)
+{
+	auto dta = crt_random_tensor<float32, CUDA>({ 6, 45 }, 11);
+	auto dtc = tensor_softmax(dta);
+
+	auto htc = tensor_softmax(dta.copy_to_host());
+	auto htc_from_cuda = dtc.copy_to_host();
+	return elementwise_compatible(htc_from_cuda, htc) && compare_data_buffers(htc_from_cuda, htc);
+}
+
+TEST_CASE(test_softmax_f16_64x2048, GPU)
+{
+	auto dx = crt_random_normal_tensor<float16, CUDA>({ 64, 2048 }, 7);
+	auto dy = tensor_softmax(dx);
+	auto hy = tensor_softmax(cvt_tensor_datatype<float32, float16>(dx.copy_to_host()));
+	auto got = cvt_tensor_datatype<float32, float16>(dy.copy_to_host());
+	return elementwise_compatible(got, hy) && compare_data_buffers(got, hy, 1e-3f) && compare_data_buffers_l2(got, hy, 2e-3f);
+}
+
+TEST_CASE(test_softmax_fused_vs_mul_add_softmax, GPU)
+{
+	// the attention chain on the host: scale, (softcap), add mask, softmax -- against the fused kernel
+	const int64 heads = 3, q = 96, k = 160, diag = k - q, window = 48;
+	auto hx = crt_random_normal_tensor<float32, CPU>({ heads * q, k }, 31);
+	for (int64 ix = 0; ix < hx.size(); ++ix) hx.buffer()[ix] *= 16.f;
+	auto dx = hx.copy_to_cuda();
+	auto mask = build_mask(q, k, true, window, diag);
+	bool ok = true;
+	for (float32 cap : { 0.f, 50.f })
+	{
+		SoftmaxPrologue p;
+		p.alpha = 0.0625f; p.softcap = cap; p.causal = true; p.window = window; p.q_len = q; p.diag = diag;
+		auto got = tensor_softmax(dx, p).copy_to_host();
+
+		auto heads_x = tensor_split(tensor_view(hx, { heads, q, k }), heads);
+		auto heads_got = tensor_split(tensor_view(got, { heads, q, k }), heads);
+		for (int64 h = 0; h < heads; ++h)
+		{
+			auto scores = tensor_mul(tensor_view(heads_x[h], { q, k }), p.alpha);
+			if (cap != 0.f) scores = host_softcap(scores, cap);
+			auto want = tensor_softmax(tensor_add(scores, mask));
+			auto have = tensor_view(heads_got[h], { q, k });
+			ok = ok && compare_data_buffers(have, want, 1e-5f);
+			for (int64 ix = 0; ix < q * k; ++ix)
+				if (mask.buffer()[ix] != 0.f) ok = ok && have.buffer()[ix] == 0.f;   // masked keys: exact zeros
+		}
+	}
+	return ok;
+}
+
+TEST_CASE(test_causal_conv1d_f32_8x2318x638, GPU)
+{
+	// shape of the reference's golden case (batch 8, dims 2318, seq_len 638, width 4)
+	auto hx = crt_random_normal_tensor<float32, CPU>({ 8, 2318, 638 }, 1);
+	auto hw = crt_random_normal_tensor<float32, CPU>({ 2318, 4 }, 2);
+	auto hb = crt_random_normal_tensor<float32, CPU>({ 2318 }, 3);
+	auto exp_hy = tensor_causal_conv1d(hx, hw, hb);
+	auto act_hy = tensor_causal_conv1d(hx.copy_to_cuda(), hw.copy_to_cuda(), hb.copy_to_cuda()).copy_to_host();
+	return elementwise_compatible(exp_hy, act_hy) && compare_data_buffers(act_hy, exp_hy);
+}
+
+TEST_CASE(test_causal_conv1d_f16_2x96x4096, GPU)
+{
+	auto dx = crt_random_normal_tensor<float16, CUDA>({ 2, 96, 4096 }, 4);
+	auto dw = crt_random_normal_tensor<float16, CUDA>({ 96, 4 }, 5);
+	auto db = crt_random_normal_tensor<float16, CUDA>({ 96 }, 6);
+	auto dy = tensor_causal_conv1d(dx, dw, db);
+	auto hy = tensor_causal_conv1d(cvt_tensor_datatype<float32, float16>(dx.copy_to_host()),
+	                               cvt_tensor_datatype<float32, float16>(dw.copy_to_host()),
+	                               cvt_tensor_datatype<float32, float16>(db.copy_to_host()));
+	auto got = cvt_tensor_datatype<float32, float16>(dy.copy_to_host());
+	return elementwise_compatible(got, hy) && compare_data_buffers_l2(got, hy, 2e-3f) && compare_data_buffers(got, hy, 2e-2f);
+}
+
+TEST_CASE(test_device_tensor_plumbing, GPU)
+{
+	// new device buffers are zero-filled; copies keep view metadata; views share the device buffer
+	Tensor<float32, CUDA> z(std::vector<int64>({ 5, 7 }));
+	auto hz = z.copy_to_host();
+	bool ok = true;
+	for (int64 ix = 0; ix < 35; ++ix) ok = ok && hz.buffer()[ix] == 0.f;
+	auto hp = crt_pattern_tensor<float32, CPU>({ 4, 6 });
+	auto dp = hp.copy_to_cuda();
+	auto dv = tensor_view(dp, { 2, 12 });
+	ok = ok && dv.buffer_id() == dp.buffer_id() && dv.buffer() == dp.buffer();
+	auto back = dv.copy_to_host();
+	ok = ok && back.dim == 2 && back.shape[1] == 12 && std::memcmp(back.buffer(), hp.buffer(), 24 * sizeof(float32)) == 0;
+	auto dd = dp.copy_to_cuda();                         // device to device
+	ok = ok && dd.buffer_id() != dp.buffer_id() && compare_data_buffers(dd.copy_to_host(), hp, 1e-9f);
+	std::cout << print_cuda_device_props();
+	return ok;
+}

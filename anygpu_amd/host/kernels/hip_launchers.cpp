@@ -1,0 +1,154 @@
+// Host-layer launchers -> C ABI of libanygpu_hip.so.  This is the only translation unit of
+// the host layer that knows the ABI; it turns every non-zero return code into the fail-stop
+// convention of the layer (message with the code and its text, exit(1)).
+#include "mm_ops.cuh"
+#include "fast_mm.cuh"
+#include "softmax_ops.cuh"
+#include "causal_conv1d.cuh"
+
+#include "anygpu_hip.h"
+
+namespace {
+
+void* const kNullStream = nullptr;
+
+void check_abi(int code, const char* what, const char* file, int line)
+{
+	if (code == ANYGPU_OK) return;
+	std::string msg = std::string(what) + ": " + anygpu_hip_error_string(code);
+	fail_runtime(code, msg.c_str(), file, line);
+}
+
+#define ABI_CHECK(call) check_abi((call), #call, __FILE__, __LINE__)
+
+// out[M, N] = lhs * rhs with rhs either [K, N] (row-major) or [N, K] (column-major storage of B)
+template <typename T>
+void mm_dispatch(const Tensor<T, CUDA>& lhs, const Tensor<T, CUDA>& rhs, const Tensor<T, CUDA>& out,
+                 int a_layout, int b_layout, const float32* bias)
+{
+	const int64 m = (a_layout == ANYGPU_A_ROW_MAJOR) ? lhs.shape[0] : lhs.shape[1];
+	const int64 k = (a_layout == ANYGPU_A_ROW_MAJOR) ? lhs.shape[1] : lhs.shape[0];
+	const int64 n = (b_layout == ANYGPU_B_ROW_MAJOR) ? rhs.shape[1] : rhs.shape[0];
+	// dense operands: the leading dimension is the extent of the innermost axis
+	const int64 lda = std::max<int64>(lhs.shape[1], 1);
+	const int64 ldb = std::max<int64>(rhs.shape[1], 1);
+	const int64 ldc = std::max<int64>(n, 1);
+	if constexpr (std::is_same_v<T, float32>)
+	{
+		ABI_CHECK(anygpu_gemm_f32(lhs.buffer(), rhs.buffer(), bias, out.buffer(), m, n, k, lda, ldb, ldc,
+		                          a_layout, b_layout, kNullStream));
+	}
+	else
+	{
+		static_assert(std::is_same_v<T, float16>, "Unsupported data type");
+		ABI_CHECK(anygpu_gemm_f16_f32acc(lhs.buffer(), rhs.buffer(), out.buffer(), m, n, k, lda, ldb, ldc,
+		                                 b_layout, kNullStream));
+	}
+}
+
+template <typename T>
+void softmax_dispatch(const Tensor<T, CUDA>& x, const SoftmaxPrologue& p, Tensor<T, CUDA>& y)
+{
+	const int64 rows = x.shape[0], cols = x.shape[1];
+	const int64 pitch = std::max<int64>(cols, 1);
+	if constexpr (std::is_same_v<T, float32>)
+	{
+		ABI_CHECK(anygpu_softmax_rows_f32(x.buffer(), y.buffer(), rows, cols, pitch, pitch, p.q_len, p.diag,
+		                                  p.alpha, p.softcap, p.causal ? 1 : 0, p.window, kNullStream));
+	}
+	else
+	{
+		static_assert(std::is_same_v<T, float16>, "Unsupported data type");
+		ABI_CHECK(anygpu_softmax_rows_f16(x.buffer(), y.buffer(), rows, cols, pitch, pitch, p.q_len, p.diag,
+		                                  p.alpha, p.softcap, p.causal ? 1 : 0, p.window, kNullStream));
+	}
+}
+
+}  // namespace
+
+void cu_tensor_mm_f32_opt0(const Tensor<float32, CUDA>& lhs, const Tensor<float32, CUDA>& rhs, const Tensor<float32, CUDA>& out)
+{
+	mm_dispatch(lhs, rhs, out, ANYGPU_A_ROW_MAJOR, ANYGPU_B_ROW_MAJOR, nullptr);
+}
+
+void cu_tensor_gemm_f32_opt0(const Tensor<float32, CUDA>& xt, const Tensor<float32, CUDA>& wt,
+                             const Tensor<float32, CUDA>& bt, const Tensor<float32, CUDA>& out)
+{
+	mm_dispatch(xt, wt, out, ANYGPU_A_ROW_MAJOR, ANYGPU_B_ROW_MAJOR, bt.buffer());
+}
+
+void opt1::cu_tensor_mm_f32(const Tensor<float32, CUDA>& lhs, const Tensor<float32, CUDA>& rhs, const Tensor<float32, CUDA>& out)
+{
+	mm_dispatch(lhs, rhs, out, ANYGPU_A_ROW_MAJOR, ANYGPU_B_ROW_MAJOR, nullptr);
+}
+
+void opt2::cu_tensor_mm_f16(const Tensor<float16, CUDA>& lhs, const Tensor<float16, CUDA>& rhs, const Tensor<float16, CUDA>& out)
+{
+	mm_dispatch(lhs, rhs, out, ANYGPU_A_ROW_MAJOR, ANYGPU_B_ROW_MAJOR, nullptr);
+}
+
+void hip_tensor_mm_nt_f16(const Tensor<float16, CUDA>& lhs, const Tensor<float16, CUDA>& rhs_nk, const Tensor<float16, CUDA>& out)
+{
+	mm_dispatch(lhs, rhs_nk, out, ANYGPU_A_ROW_MAJOR, ANYGPU_B_COL_MAJOR, nullptr);
+}
+
+void hip_tensor_mm_nt_f32(const Tensor<float32, CUDA>& lhs, const Tensor<float32, CUDA>& rhs_nk, const Tensor<float32, CUDA>& out)
+{
+	mm_dispatch(lhs, rhs_nk, out, ANYGPU_A_ROW_MAJOR, ANYGPU_B_COL_MAJOR, nullptr);
+}
+
+#define ANYGPU_DEFINE_FAST_MM(NAME, T, A_LAYOUT)                                              \
+	void NAME(const Tensor<T, CUDA>& xt, const Tensor<T, CUDA>& wt, Tensor<T, CUDA>& yt)      \
+	{                                                                                         \
+		mm_dispatch(xt, wt, yt, A_LAYOUT, ANYGPU_B_ROW_MAJOR, nullptr);                       \
+	}
+
+ANYGPU_DEFINE_FAST_MM(cu_fast_mm_f32_cb, float32, ANYGPU_A_ROW_MAJOR)
+ANYGPU_DEFINE_FAST_MM(cu_fast_mm_f32_v1, float32, ANYGPU_A_ROW_MAJOR)
+ANYGPU_DEFINE_FAST_MM(cu_fast_mm_f32_v2, float32, ANYGPU_A_ROW_MAJOR)
+ANYGPU_DEFINE_FAST_MM(cu_fast_mm_f32_v2_1, float32, ANYGPU_A_ROW_MAJOR)
+ANYGPU_DEFINE_FAST_MM(cu_fast_mm_f32_v3, float32, ANYGPU_A_ROW_MAJOR)
+ANYGPU_DEFINE_FAST_MM(cu_fast_mm_f32_v4, float32, ANYGPU_A_ROW_MAJOR)
+ANYGPU_DEFINE_FAST_MM(cu_fast_mm_f32_v4_1, float32, ANYGPU_A_ROW_MAJOR)
+ANYGPU_DEFINE_FAST_MM(cu_fast_mm_f32_v4_2, float32, ANYGPU_A_COL_MAJOR)
+ANYGPU_DEFINE_FAST_MM(cu_fast_mm_f16_v1, float16, ANYGPU_A_ROW_MAJOR)
+ANYGPU_DEFINE_FAST_MM(cu_fast_mm_f16_v2, float16, ANYGPU_A_ROW_MAJOR)
+ANYGPU_DEFINE_FAST_MM(cu_fast_mm_f16_v3, float16, ANYGPU_A_ROW_MAJOR)
+ANYGPU_DEFINE_FAST_MM(cu_fast_mm_f16_v3_1, float16, ANYGPU_A_ROW_MAJOR)
+ANYGPU_DEFINE_FAST_MM(cu_fast_mm_f16_v3_2, float16, ANYGPU_A_ROW_MAJOR)
+
+#undef ANYGPU_DEFINE_FAST_MM
+
+void cu_tensor_softmax_f32(const Tensor<float32, CUDA>& x, Tensor<float32, CUDA>& y)
+{
+	softmax_dispatch(x, SoftmaxPrologue{}, y);
+}
+
+void hip_tensor_softmax_f16(const Tensor<float16, CUDA>& x, Tensor<float16, CUDA>& y)
+{
+	softmax_dispatch(x, SoftmaxPrologue{}, y);
+}
+
+void hip_tensor_softmax_fused_f32(const Tensor<float32, CUDA>& x, const SoftmaxPrologue& prologue, Tensor<float32, CUDA>& y)
+{
+	softmax_dispatch(x, prologue, y);
+}
+
+void hip_tensor_softmax_fused_f16(const Tensor<float16, CUDA>& x, const SoftmaxPrologue& prologue, Tensor<float16, CUDA>& y)
+{
+	softmax_dispatch(x, prologue, y);
+}
+
+void cu_tensor_causal_conv1d_f32(const Tensor<float32, CUDA>& xt, const Tensor<float32, CUDA>& wt,
+                                 const Tensor<float32, CUDA>& bt, Tensor<float32, CUDA>& yt)
+{
+	ABI_CHECK(anygpu_causal_conv1d_silu_f32(xt.buffer(), wt.buffer(), bt.buffer(), yt.buffer(),
+	                                        xt.shape[0], xt.shape[1], xt.shape[2], wt.shape[1], kNullStream));
+}
+
+void hip_tensor_causal_conv1d_f16(const Tensor<float16, CUDA>& xt, const Tensor<float16, CUDA>& wt,
+                                  const Tensor<float16, CUDA>& bt, Tensor<float16, CUDA>& yt)
+{
+	ABI_CHECK(anygpu_causal_conv1d_silu_f16(xt.buffer(), wt.buffer(), bt.buffer(), yt.buffer(),
+	                                        xt.shape[0], xt.shape[1], xt.shape[2], wt.shape[1], kNullStream));
+}

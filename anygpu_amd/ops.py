@@ -28,15 +28,16 @@ def _check_device(*tensors: torch.Tensor) -> None:
 
 
 def tensor_mm(lhs: torch.Tensor, rhs: torch.Tensor, out: torch.Tensor | None = None,
-              b_layout: int = capi.B_ROW_MAJOR) -> torch.Tensor:
-    """C = lhs @ B.  lhs is [M, K] row-major (rows may be padded: stride(0) >= K, stride(1) == 1).
+              b_layout: int = capi.B_ROW_MAJOR, a_layout: int = capi.A_ROW_MAJOR) -> torch.Tensor:
+    """C = A @ B.  With a_layout == A_ROW_MAJOR lhs is [M, K] (rows may be padded: stride(0) >= K,
+    stride(1) == 1); with A_COL_MAJOR (float32 only) lhs is the [K, M] storage of A.
     With b_layout == B_ROW_MAJOR rhs is [K, N]; with B_COL_MAJOR rhs is the [N, K] storage of B.
     float16 (fp32 accumulate) and float32 are supported."""
     _check_device(lhs, rhs)
     _require(lhs.dim() == 2 and rhs.dim() == 2, "matrix multiplication requires compatible matrices")
     _require(lhs.dtype == rhs.dtype, "operands must share a dtype")
     _require(lhs.stride(1) == 1 and rhs.stride(1) == 1, "innermost stride must be 1")
-    m, k = lhs.shape
+    m, k = lhs.shape if a_layout == capi.A_ROW_MAJOR else (lhs.shape[1], lhs.shape[0])
     if b_layout == capi.B_ROW_MAJOR:
         _require(rhs.shape[0] == k, "matrix multiplication requires compatible matrices")
         n = rhs.shape[1]
@@ -47,16 +48,17 @@ def tensor_mm(lhs: torch.Tensor, rhs: torch.Tensor, out: torch.Tensor | None = N
         out = torch.empty((m, n), dtype=lhs.dtype, device=lhs.device)
     _require(tuple(out.shape) == (m, n) and out.stride(1) == 1, "result mtx shape is wrong")
     lib = capi.load()
-    lda = lhs.stride(0) if m > 1 else max(k, 1)
+    lda = lhs.stride(0) if lhs.shape[0] > 1 else max(lhs.shape[1], 1)
     ldb = rhs.stride(0) if rhs.shape[0] > 1 else max(rhs.shape[1], 1)
     ldc = out.stride(0) if m > 1 else max(n, 1)
     if lhs.dtype == torch.float16:
+        _require(a_layout == capi.A_ROW_MAJOR, "the fp16 GEMM takes a row-major left operand")
         rc = lib.anygpu_gemm_f16_f32acc(lhs.data_ptr(), rhs.data_ptr(), out.data_ptr(), m, n, k,
                                         lda, ldb, ldc, b_layout, _stream_ptr())
         capi.check("anygpu_gemm_f16_f32acc", rc)
     elif lhs.dtype == torch.float32:
         rc = lib.anygpu_gemm_f32(lhs.data_ptr(), rhs.data_ptr(), None, out.data_ptr(), m, n, k,
-                                 lda, ldb, ldc, b_layout, _stream_ptr())
+                                 lda, ldb, ldc, a_layout, b_layout, _stream_ptr())
         capi.check("anygpu_gemm_f32", rc)
     else:
         raise TypeError("Unsupported data type")
@@ -78,7 +80,8 @@ def tensor_gemm(xt: torch.Tensor, wt: torch.Tensor, bt: torch.Tensor,
     _require(bt.numel() == n, "incorrect bias shape")
     out = torch.empty((m, n), dtype=torch.float32, device=xt.device)
     rc = capi.load().anygpu_gemm_f32(xt.data_ptr(), wt.data_ptr(), bt.data_ptr(), out.data_ptr(), m, n, k,
-                                     max(k, 1), max(wt.shape[1], 1), max(n, 1), b_layout, _stream_ptr())
+                                     max(k, 1), max(wt.shape[1], 1), max(n, 1), capi.A_ROW_MAJOR, b_layout,
+                                     _stream_ptr())
     capi.check("anygpu_gemm_f32", rc)
     return out
 

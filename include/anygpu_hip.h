@@ -34,6 +34,10 @@ extern "C" {
 #define ANYGPU_ERR_UNSUPPORTED   -4   /* a value outside what the kernels implement (e.g. conv width > 4) */
 #define ANYGPU_ERR_TOO_LARGE     -5   /* an extent exceeds what the launch geometry can index */
 
+/* Layout of the left-hand GEMM operand (fp32 entry point only). */
+#define ANYGPU_A_ROW_MAJOR  0   /* A stored [M, K], element (r, l) at A[r * lda + l]  (reference layout) */
+#define ANYGPU_A_COL_MAJOR  1   /* A stored [K, M], element (r, l) at A[l * lda + r]  (pre-transposed input) */
+
 /* Layout of the right-hand GEMM operand. */
 #define ANYGPU_B_ROW_MAJOR  0   /* B stored [K, N], element (l, c) at B[l * ldb + c]  (reference layout) */
 #define ANYGPU_B_COL_MAJOR  1   /* B stored [N, K], element (l, c) at B[c * ldb + l]  ("weights as [out, in]") */
@@ -61,12 +65,14 @@ int anygpu_gemm_f16_f32acc(const void* A, const void* B, void* C,
  * C[M,N] = A[M,K] * B (+ bias[N] added to every row when bias != NULL), fp32 throughout, fp32 MFMA.
  * Replaces cu_tensor_mm_f32_opt0 and cu_tensor_gemm_f32_opt0 (srcs/kernels/cuda/mm_ops.cuh:10-25, the
  * tensor_mm / tensor_gemm <float32, CUDA> paths of srcs/ops/mm_ops.hpp:58-61,160-163) and the
- * cu_fast_mm_f32_* ladder (srcs/kernels/cuda/fast_mm.cuh:7-68).  Any shape.
+ * cu_fast_mm_f32_* ladder (srcs/kernels/cuda/fast_mm.cuh:7-68), whose last rung takes the left operand
+ * pre-transposed ([K, M], srcs/kernels/cuda/fast_mm_f32_v4.2.cu:190-199): a_layout selects that storage
+ * (lda >= K for row-major A, >= M for column-major A).  Any shape.
  */
 int anygpu_gemm_f32(const float* A, const float* B, const float* bias, float* C,
                     int64_t M, int64_t N, int64_t K,
                     int64_t lda, int64_t ldb, int64_t ldc,
-                    int b_layout, void* stream);
+                    int a_layout, int b_layout, void* stream);
 
 /*
  * Row softmax over the last axis of a [rows, cols] matrix, with the steps the attention caller

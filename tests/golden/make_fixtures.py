@@ -1,0 +1,75 @@
+#!/usr/bin/env python3
+"""Writes the small .dat fixtures under tests/golden/ from seeded synthetic inputs and the CPU
+oracle.  Folder and file names follow the reference's golden-test layout (one folder per case
+with x.dat / w.dat / b.dat / y.dat ..., tests/ext_torch_tests.cpp:587-644,745-778), at sizes of
+a few KB so that they can be committed.  Re-run from the repository root:
+    python tests/golden/make_fixtures.py
+The reference's own fixtures are not available (not in its repository, unseeded generator), so
+expected outputs come from the oracle, which tests/test_oracle_pins.py ties down independently.
+"""
+from __future__ import annotations
+
+import sys
+from pathlib import Path
+
+import numpy as np
+
+HERE = Path(__file__).resolve().parent
+REPO = HERE.parent.parent
+sys.path.insert(0, str(REPO))
+sys.path.insert(0, str(HERE))
+
+import oracle  # noqa: E402
+from anygpu_amd import synth  # noqa: E402
+from dat_codec import save_tensor  # noqa: E402
+
+
+def case_dir(name: str) -> Path:
+    d = HERE / name
+    d.mkdir(exist_ok=True)
+    return d
+
+
+def main() -> None:
+    # causal conv1d + SiLU, float32: the reference case's layout at a committed size
+    d = case_dir("test_causal_conv1d_fwd_f32")
+    x = synth.normal(100, (2, 6, 40))
+    w = synth.normal(101, (6, 4))
+    b = synth.normal(102, (6,))
+    save_tensor(x, d / "x.dat"); save_tensor(w, d / "w.dat"); save_tensor(b, d / "b.dat")
+    save_tensor(oracle.tensor_causal_conv1d(x, w, b), d / "y.dat")
+
+    # float32 matmul (positive inputs like the reference's torch.rand case: elementwise rel 1 % gate)
+    d = case_dir("test_mm_m24_n16_k40_f32")
+    x = synth.uniform(110, (24, 40), 0.0, 1.0)
+    w = synth.uniform(111, (40, 16), 0.0, 1.0)
+    save_tensor(x, d / "x.dat"); save_tensor(w, d / "w.dat")
+    save_tensor(oracle.tensor_mm(x, w), d / "y.dat")
+
+    # float16 matmul: half inputs, expected output = float32 oracle on the up-cast inputs, rounded to half
+    d = case_dir("test_mm_m64_n64_k128_f16")
+    x = synth.uniform(120, (64, 128), 0.0, 1.0).astype(np.float16)
+    w = synth.uniform(121, (128, 64), 0.0, 1.0).astype(np.float16)
+    y = oracle.tensor_mm(oracle.cvt_f16_to_f32(x), oracle.cvt_f16_to_f32(w))
+    save_tensor(x, d / "x.dat"); save_tensor(w, d / "w.dat"); save_tensor(y.astype(np.float16), d / "y.dat")
+
+    # masked, scaled attention scores -> probabilities: [heads * q, k] scores, causal -inf mask, scale 0.125
+    d = case_dir("test_softmax_masked_scaled_f32")
+    heads, q, k = 2, 16, 16
+    s = synth.normal(130, (heads * q, k), std=8.0)
+    mask = oracle.causal_mask(q, k)
+    save_tensor(s, d / "scores.dat"); save_tensor(mask, d / "mask.dat")
+    save_tensor(oracle.attention_softmax(s, alpha=0.125, causal=True, q_len=q), d / "y.dat")
+
+    # Gemma2-style: scale 1/16, softcap 50, causal + sliding window 6
+    d = case_dir("test_softmax_softcap_window_f32")
+    s = synth.normal(140, (heads * q, k), std=16.0)
+    mask = oracle.slide_mask(oracle.causal_mask(q, k), 6)
+    save_tensor(s, d / "scores.dat"); save_tensor(mask, d / "mask.dat")
+    save_tensor(oracle.attention_softmax(s, alpha=0.0625, softcap=50.0, causal=True, window=6, q_len=q), d / "y.dat")
+
+    print("fixtures written under", HERE)
+
+
+if __name__ == "__main__":
+    main()

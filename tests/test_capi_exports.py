@@ -1,0 +1,78 @@
+"""The C ABI library loads and exports exactly what include/anygpu_hip.h declares (no compute
+calls here; argument validation that needs no GPU is exercised as well)."""
+import ctypes
+import re
+import subprocess
+from pathlib import Path
+
+import pytest
+
+REPO = Path(__file__).resolve().parent.parent
+HEADER = REPO / "include" / "anygpu_hip.h"
+
+
+def declared_functions():
+    text = re.sub(r"/\*.*?\*/", "", HEADER.read_text(), flags=re.S)
+    return sorted(set(re.findall(r"\b(anygpu_\w+)\s*\(", text)))
+
+
+def test_header_and_binding_table_agree():
+    from anygpu_amd import capi
+    assert declared_functions() == sorted(capi.SIGNATURES)
+
+
+def test_library_exports_every_declared_symbol():
+    from anygpu_amd import capi
+    lib = capi.load()
+    for name in declared_functions():
+        assert getattr(lib, name) is not None
+    out = subprocess.run(["nm", "-D", "--defined-only", str(capi.LIB_PATH)], capture_output=True, text=True, check=True)
+    exported = set(re.findall(r"\bT (anygpu_\w+)", out.stdout))
+    assert exported == set(declared_functions()), "exported symbols and header declarations differ"
+    assert lib.anygpu_hip_abi_version() == 1
+    assert lib.anygpu_hip_target() == b"gfx950"
+
+
+def test_error_strings():
+    from anygpu_amd import capi
+    assert capi.error_string(0) == "success"
+    for code in (-1, -2, -3, -4, -5):
+        assert capi.error_string(code) not in ("", "success", "unknown anygpu error code")
+    assert capi.error_string(-99) == "unknown anygpu error code"
+
+
+def test_argument_validation_needs_no_gpu():
+    # rejected before any runtime call: shapes, strides, NULL pointers, unsupported values
+    from anygpu_amd import capi
+    lib = capi.load()
+    fake = ctypes.c_void_p(0x1000)      # never dereferenced: every call below is rejected first
+    assert lib.anygpu_gemm_f32(fake, fake, None, fake, 4, 4, 8, 4, 4, 4, 0, 0, None) == capi.ANYGPU_ERR_BAD_STRIDE
+    assert lib.anygpu_gemm_f32(fake, fake, None, fake, 4, 4, 8, 8, 4, 4, 2, 0, None) == capi.ANYGPU_ERR_UNSUPPORTED
+    assert lib.anygpu_gemm_f16_f32acc(fake, fake, None, 4, 4, 8, 8, 4, 4, 0, None) == capi.ANYGPU_ERR_NULL_POINTER
+    assert lib.anygpu_gemm_f16_f32acc(fake, fake, fake, -1, 4, 8, 8, 4, 4, 0, None) == capi.ANYGPU_ERR_BAD_SHAPE
+    assert lib.anygpu_gemm_f16_f32acc(fake, fake, fake, 1 << 40, 4, 8, 8, 4, 4, 0, None) == capi.ANYGPU_ERR_TOO_LARGE
+    assert lib.anygpu_softmax_rows_f16(fake, fake, 4, 16, 8, 16, 0, 0, 1.0, 0.0, 0, 0, None) == capi.ANYGPU_ERR_BAD_STRIDE
+    assert lib.anygpu_softmax_rows_f16(fake, None, 4, 16, 16, 16, 0, 0, 1.0, 0.0, 0, 0, None) == capi.ANYGPU_ERR_NULL_POINTER
+    assert lib.anygpu_causal_conv1d_silu_f16(fake, fake, fake, fake, 2, 3, 8, 5, None) == capi.ANYGPU_ERR_UNSUPPORTED
+    assert lib.anygpu_causal_conv1d_silu_f32(fake, fake, fake, fake, 2, 3, -8, 4, None) == capi.ANYGPU_ERR_BAD_SHAPE
+    # empty problems succeed without touching the device
+    assert lib.anygpu_gemm_f32(None, None, None, None, 0, 4, 8, 8, 4, 4, 0, 0, None) == capi.ANYGPU_OK
+    assert lib.anygpu_softmax_rows_f32(None, None, 0, 16, 16, 16, 0, 0, 1.0, 0.0, 0, 0, None) == capi.ANYGPU_OK
+    assert lib.anygpu_causal_conv1d_silu_f32(None, None, None, None, 0, 3, 8, 4, None) == capi.ANYGPU_OK
+
+
+def test_ops_refuse_cpu_tensors():
+    torch = pytest.importorskip("torch")
+    from anygpu_amd import ops
+    with pytest.raises(ValueError):
+        ops.tensor_softmax(torch.zeros(2, 4))
+    with pytest.raises(ValueError):
+        ops.tensor_mm(torch.zeros(2, 4), torch.zeros(4, 2))
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    from anygpu_amd import capi
+    monkeypatch.setattr(capi, "_lib", None)
+    monkeypatch.setattr(capi, "LIB_PATH", tmp_path / "libanygpu_hip.so")
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        capi.load()

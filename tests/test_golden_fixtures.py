@@ -1,0 +1,50 @@
+"""The committed .dat fixtures are what tests/golden/make_fixtures.py produces (so the generator
+and the data cannot drift apart) and the oracle reproduces every expected output."""
+import sys
+from pathlib import Path
+
+import numpy as np
+
+GOLDEN = Path(__file__).resolve().parent / "golden"
+sys.path.insert(0, str(GOLDEN))
+
+from dat_codec import load_tensor, save_tensor  # noqa: E402
+
+
+def test_codec_roundtrip_and_byte_layout(tmp_path):
+    x = np.arange(24, dtype=np.float32).reshape(2, 3, 4)
+    save_tensor(x, tmp_path / "t.dat")
+    raw = (tmp_path / "t.dat").read_bytes()
+    assert np.frombuffer(raw[:20], dtype="<i4").tolist() == [3, 2, 3, 4, 5]      # dim, shape, code FLOAT32
+    assert len(raw) == 20 + 24 * 4
+    assert np.array_equal(load_tensor(tmp_path / "t.dat"), x)
+    h = x.astype(np.float16)
+    save_tensor(h, tmp_path / "h.dat")
+    assert np.frombuffer((tmp_path / "h.dat").read_bytes()[16:20], dtype="<i4")[0] == 4
+    assert np.array_equal(load_tensor(tmp_path / "h.dat"), h)
+
+
+def test_fixtures_match_the_oracle(oracle):
+    d = GOLDEN / "test_causal_conv1d_fwd_f32"
+    y = oracle.tensor_causal_conv1d(load_tensor(d / "x.dat"), load_tensor(d / "w.dat"), load_tensor(d / "b.dat"))
+    assert np.array_equal(y, load_tensor(d / "y.dat"))
+    d = GOLDEN / "test_mm_m24_n16_k40_f32"
+    assert np.array_equal(oracle.tensor_mm(load_tensor(d / "x.dat"), load_tensor(d / "w.dat")), load_tensor(d / "y.dat"))
+    d = GOLDEN / "test_mm_m64_n64_k128_f16"
+    y = oracle.tensor_mm(oracle.cvt_f16_to_f32(load_tensor(d / "x.dat")), oracle.cvt_f16_to_f32(load_tensor(d / "w.dat")))
+    assert np.array_equal(y.astype(np.float16), load_tensor(d / "y.dat"))
+    for name, kw in [("test_softmax_masked_scaled_f32", dict(alpha=0.125, causal=True, q_len=16)),
+                     ("test_softmax_softcap_window_f32", dict(alpha=0.0625, softcap=50.0, causal=True, window=6, q_len=16))]:
+        d = GOLDEN / name
+        y = oracle.attention_softmax(load_tensor(d / "scores.dat"), **kw)
+        assert np.array_equal(y, load_tensor(d / "y.dat"))
+        # the stored additive mask is the one the kernel parameters describe
+        mask = load_tensor(d / "mask.dat")
+        assert np.all(y[np.tile(mask, (2, 1)) != 0] == 0)
+        # torch's library formula on the same data: softmax(scale * s [capped] + mask)
+        import torch
+        s = torch.from_numpy(load_tensor(d / "scores.dat")).double() * kw["alpha"]
+        if kw.get("softcap"):
+            s = kw["softcap"] * torch.tanh(s / kw["softcap"])
+        ref = torch.softmax(s + torch.from_numpy(np.tile(mask, (2, 1))).double(), dim=-1).numpy()
+        assert np.max(np.abs(y - ref)) < 1e-6

@@ -300,6 +300,21 @@ def test_mm_f32_shapes_and_layouts(ops, oracle, layout, m, k, n):
     assert scaled_rel_err(got, want, floor) <= TOL_F32
 
 
+def test_mm_f32_transposed_left_operand(ops, oracle):
+    # the layout of the reference's last fp32 rung: A handed over as [K, M]
+    from anygpu_amd import capi
+    for (m, k, n) in [(128, 64, 128), (100, 37, 61), (256, 272, 384)]:
+        a = synth.uniform(m * 7 + k, (m, k))
+        b = synth.uniform(k * 5 + n, (k, n))
+        at = np.ascontiguousarray(a.T)
+        got = host(ops.tensor_mm(dev(at), dev(b), a_layout=capi.A_COL_MAJOR))
+        want = oracle.tensor_mm(a, b, threads=8)
+        assert scaled_rel_err(got, want, math.sqrt(k) / 3.0) <= TOL_F32
+        bt = np.ascontiguousarray(b.T)
+        got2 = host(ops.tensor_mm(dev(at), dev(bt), a_layout=capi.A_COL_MAJOR, b_layout=capi.B_COL_MAJOR))
+        assert scaled_rel_err(got2, want, math.sqrt(k) / 3.0) <= TOL_F32
+
+
 def test_gemm_f32_bias_and_padded_leading_dimensions(ops, oracle):
     import torch
     from anygpu_amd import capi
@@ -410,3 +425,41 @@ def test_mm_empty_and_rejected_arguments(ops):
     assert z.shape == (4, 5) and not bool(z.any())
     with pytest.raises(ValueError):
         ops.tensor_mm(torch.zeros((4, 8), device="cuda"), torch.zeros((7, 4), device="cuda"))
+
+
+# =============================================================================================
+# committed golden fixtures (tests/golden/*.dat)
+# =============================================================================================
+
+def test_golden_fixtures_through_c_abi(ops):
+    import sys
+    from pathlib import Path
+    golden = Path(__file__).resolve().parent / "golden"
+    sys.path.insert(0, str(golden))
+    from dat_codec import load_tensor
+
+    d = golden / "test_causal_conv1d_fwd_f32"
+    got = host(ops.tensor_causal_conv1d(dev(load_tensor(d / "x.dat")), dev(load_tensor(d / "w.dat")),
+                                        dev(load_tensor(d / "b.dat"))))
+    assert scaled_rel_err(got, load_tensor(d / "y.dat"), 1.0) <= TOL_F32
+
+    d = golden / "test_mm_m24_n16_k40_f32"
+    got = host(ops.tensor_mm(dev(load_tensor(d / "x.dat")), dev(load_tensor(d / "w.dat"))))
+    assert scaled_rel_err(got, load_tensor(d / "y.dat"), math.sqrt(40) / 3.0) <= TOL_F32
+
+    d = golden / "test_mm_m64_n64_k128_f16"
+    got = host(ops.tensor_mm(dev(load_tensor(d / "x.dat")), dev(load_tensor(d / "w.dat")))).astype(np.float32)
+    assert scaled_rel_err(got, load_tensor(d / "y.dat").astype(np.float32), math.sqrt(128) / 3.0) <= TOL_F16_GEMM
+
+    d = golden / "test_softmax_masked_scaled_f32"
+    want = load_tensor(d / "y.dat")
+    got = host(ops.tensor_softmax(dev(load_tensor(d / "scores.dat")), alpha=0.125, causal=True, q_len=16))
+    assert scaled_rel_err(got, want, want.max(axis=1, keepdims=True)) <= TOL_F32
+    assert np.all(got[np.tile(load_tensor(d / "mask.dat"), (2, 1)) != 0] == 0.0)
+
+    d = golden / "test_softmax_softcap_window_f32"
+    want = load_tensor(d / "y.dat")
+    got = host(ops.tensor_softmax(dev(load_tensor(d / "scores.dat")), alpha=0.0625, softcap=50.0, causal=True,
+                                  window=6, q_len=16))
+    assert scaled_rel_err(got, want, want.max(axis=1, keepdims=True)) <= TOL_F32
+    assert np.all(got[np.tile(load_tensor(d / "mask.dat"), (2, 1)) != 0] == 0.0)
