@@ -1,0 +1,372 @@
+// Tile kernel of the fp16 GEMM ("NT": A [M,K] and B [N,K], both K-contiguous) for gfx950.
+//
+// A block owns a BM x BN tile of C.  Per 64-deep step it stages a BM x 64 slab of A and a
+// BN x 64 slab of B in LDS (two stages, so the loads of slab t+1 are in flight while slab t
+// is multiplied) and each wave accumulates a (BM/WM) x (BN/WN) patch on the matrix cores with
+// fp32 accumulators, either with v_mfma_f32_32x32x16_f16 or with v_mfma_f32_16x16x32_f16
+// (both take 8 halves per lane per operand and have the same peak rate).
+//
+// Global -> LDS goes through global_load_lds_dwordx4: every lane fetches 16 bytes and the
+// hardware writes the 64 lanes of a wave to 1 KB of consecutive LDS, bypassing the VGPRs.
+// An LDS slab row is 64 halves = 128 bytes = eight 16-byte chunks; chunk c of row r is stored
+// at chunk position c ^ swz(r), so that the lanes which read the same logical chunk of
+// consecutive rows for an MFMA operand (ds_read_b128) spread over all banks.  Because the
+// LDS side of the direct load is fixed (lane i -> base + 16 i), the swizzle is applied on the
+// global side: lane i of a load instruction fetches the chunk that belongs at position i.
+//
+// The products are formed transposed (the B slab is the first MFMA operand), which leaves
+// every lane with 4 consecutive columns of one row of C; the epilogue parks row bands of the
+// wave's patch in LDS and writes whole rows back, 16 bytes per lane.
+//
+// Under this kernel the MI355X is power-limited, not issue-limited: measured with
+// s_memtime / s_memrealtime inside the main loop, the shader clock sits near 1.6 GHz (not 2.4)
+// and schedules with fewer MFMA stalls simply run at a lower clock for the same wall time.
+#pragma once
+
+#include "device_utils.hpp"
+
+namespace anygpu {
+
+constexpr int kNumXcd = 8;
+
+// Tile -> block mapping.  Workgroups are dealt round-robin to the 8 XCDs (each with its own
+// L2), so block b runs on XCD b % 8.  Blocks of one XCD get a contiguous range of tile
+// numbers, and tile numbers walk the tile grid in column strips of kGroupM rows, so an XCD
+// works on a compact patch of C and re-uses A and B slabs out of its own L2.
+template <int kGroupM>
+__device__ __forceinline__ void tile_of_block(int bid, int tiles_m, int tiles_n, int& tm, int& tn)
+{
+	const int total = tiles_m * tiles_n;
+	int id = bid;
+	if (total % kNumXcd == 0)
+	{
+		id = (bid % kNumXcd) * (total / kNumXcd) + bid / kNumXcd;
+	}
+	const int per_group = kGroupM * tiles_n;
+	const int g = id / per_group;
+	const int first_m = g * kGroupM;
+	const int rows = min(kGroupM, tiles_m - first_m);
+	const int in_group = id - g * per_group;
+	tm = first_m + in_group % rows;
+	tn = in_group / rows;
+}
+
+// SWZ selects which row bits permute the chunk position: 0 -> row & 7 (conflict free for 8
+// lanes per LDS pass over 32 banks), 1 -> (row >> 1) & 7 (conflict free for 16 lanes per pass
+// over 64 banks; measured conflict free on gfx950 with SQ_LDS_BANK_CONFLICT).
+template <int SWZ>
+__device__ __forceinline__ int swizzle_of_row(int row)
+{
+	return SWZ == 0 ? (row & 7) : ((row >> 1) & 7);
+}
+
+// The two MFMA shapes.  MI x MI output tile; a lane supplies row (lane % MI) of each operand
+// and k group (lane / MI), 8 consecutive halves; one instruction is 512 / MI deep.
+template <int MI> struct MfmaShape;
+
+template <> struct MfmaShape<32>
+{
+	using Acc = float16_t;
+	static constexpr int kAccRegs = 16;
+	__device__ static __forceinline__ Acc mma(half8_t first, half8_t second, Acc c)
+	{
+		return __builtin_amdgcn_mfma_f32_32x32x16_f16(first, second, c, 0, 0, 0);
+	}
+	// register group g (4 registers) of lane l: row l % 32 of the second operand, 4 consecutive
+	// rows of the first operand starting at:
+	__device__ static __forceinline__ int first_row_of_group(int g, int lane) { return 8 * g + 4 * (lane >> 5); }
+};
+
+template <> struct MfmaShape<16>
+{
+	using Acc = float4_t;
+	static constexpr int kAccRegs = 4;
+	__device__ static __forceinline__ Acc mma(half8_t first, half8_t second, Acc c)
+	{
+		return __builtin_amdgcn_mfma_f32_16x16x32_f16(first, second, c, 0, 0, 0);
+	}
+	__device__ static __forceinline__ int first_row_of_group(int g, int lane) { (void)g; return 4 * (lane >> 4); }
+};
+
+template <int BM_, int BN_, int WM_, int WN_, int SWZ_, int ILV_ = 0, int GROUP_M_ = 4, int MI_ = 32>
+struct GemmTileCfg
+{
+	static constexpr int BM = BM_, BN = BN_, BK = 64, WM = WM_, WN = WN_, SWZ = SWZ_;
+	static constexpr int ILV = ILV_;          // how LDS reads are spread between the MFMAs of one step
+	static constexpr int GROUP_M = GROUP_M_;  // rows of tiles per column strip of the tile walk
+	static constexpr int MI = MI_;            // MFMA tile edge: 32 (x16 deep) or 16 (x32 deep)
+	static constexpr int kKGroups = kWaveSize / MI;       // k groups of 8 halves per instruction
+	static constexpr int kSteps = 8 / kKGroups;           // MFMA steps per 64-deep slab
+	static constexpr int kWaves = WM * WN;
+	static constexpr int kThreads = kWaves * kWaveSize;
+	static constexpr int kWaveM = BM / WM;
+	static constexpr int kWaveN = BN / WN;
+	static constexpr int kTilesM = kWaveM / MI;
+	static constexpr int kTilesN = kWaveN / MI;
+	static constexpr int kSlabABytes = BM * BK * 2;
+	static constexpr int kSlabBBytes = BN * BK * 2;
+	static constexpr int kStageBytes = kSlabABytes + kSlabBBytes;
+	static constexpr int kLdsBytes = 2 * kStageBytes;
+	// one direct load instruction of a wave moves 1 KB = 8 slab rows
+	static constexpr int kLoadsA = BM / 8 / kWaves;
+	static constexpr int kLoadsB = BN / 8 / kWaves;
+	static_assert(MI == 32 || MI == 16, "unknown MFMA shape");
+	static_assert(BM % (8 * kWaves) == 0 && BN % (8 * kWaves) == 0, "slab rows must divide over the waves");
+	static_assert(kWaveM % MI == 0 && kWaveN % MI == 0, "wave patch must be whole MFMA tiles");
+};
+
+// vmcnt(0) with the other counters left alone (gfx9 encoding: vmcnt in [3:0] and [15:14],
+// expcnt [6:4], lgkmcnt [11:8])
+__device__ __forceinline__ void wait_vmem_all()
+{
+	__builtin_amdgcn_s_waitcnt(0x0F70);
+}
+
+// Epilogue through LDS.  With the B slab as the first MFMA operand, a group of 4 accumulator
+// registers of a lane holds 4 consecutive columns of ONE row of C (row = lane % MI of the tile),
+// so a direct store instruction would touch MI different rows with 8 bytes each.  Instead each
+// wave parks one MI-row band of its patch (MI x kWaveN halves) in its own LDS scratch and reads
+// it back row by row, 16 bytes per lane, so that the global stores cover whole rows of the band.
+// The scratch row pitch is 16 bytes more than the row, which spreads the 8-byte writes of the
+// rows over the banks.  The caller guarantees that nobody still reads or fills LDS.
+template <typename Cfg>
+__device__ __forceinline__ void store_patch_via_lds(
+	const typename MfmaShape<Cfg::MI>::Acc (&acc)[Cfg::kTilesM][Cfg::kTilesN], char* lds,
+	half_t* __restrict__ C, int64_t ldc, int64_t m_base, int64_t n_base, int wave, int lane)
+{
+	using Shape = MfmaShape<Cfg::MI>;
+	constexpr int MI = Cfg::MI, TM = Cfg::kTilesM, TN = Cfg::kTilesN;
+	constexpr int kRowBytes = Cfg::kWaveN * 2;
+	constexpr int kPitch = kRowBytes + 16;
+	constexpr int kLanesPerRow = kRowBytes / 16;
+	constexpr int kRowsPerPass = kWaveSize / kLanesPerRow;
+	static_assert(Cfg::kWaves * MI * kPitch <= Cfg::kLdsBytes, "epilogue scratch must fit in the staging LDS");
+	char* scratch = lds + wave * (MI * kPitch);
+	const int frag_row = lane % MI;
+#pragma unroll
+	for (int i = 0; i < TM; ++i)
+	{
+#pragma unroll
+		for (int j = 0; j < TN; ++j)
+#pragma unroll
+			for (int g = 0; g < Shape::kAccRegs / 4; ++g)
+			{
+				half4_t out;
+#pragma unroll
+				for (int e = 0; e < 4; ++e) out[e] = (half_t)acc[i][j][4 * g + e];
+				*reinterpret_cast<half4_t*>(scratch + frag_row * kPitch +
+				                            (j * MI + Shape::first_row_of_group(g, lane)) * 2) = out;
+			}
+		constexpr int kPasses = (MI + kRowsPerPass - 1) / kRowsPerPass;
+#pragma unroll
+		for (int pass = 0; pass < kPasses; ++pass)
+		{
+			const int row = pass * kRowsPerPass + lane / kLanesPerRow;
+			const int col16 = lane % kLanesPerRow;
+			if (kRowsPerPass <= MI || row < MI)
+			{
+				const half8_t v = *reinterpret_cast<const half8_t*>(scratch + row * kPitch + col16 * 16);
+				*reinterpret_cast<half8_t*>(C + (m_base + i * MI + row) * ldc + n_base + col16 * 8) = v;
+			}
+		}
+	}
+}
+
+// Scheduling-group masks of __builtin_amdgcn_sched_group_barrier
+constexpr int kSchedMfma = 0x008;
+constexpr int kSchedVmemRead = 0x020;
+constexpr int kSchedDsRead = 0x100;
+
+// The tile kernel, software pipelined.  Operand fragments are double-buffered in registers:
+// while the MFMAs of one step run, the ds_read_b128 of the next step are issued in between
+// them.  The barrier of a 64-deep slab sits in front of its LAST step, whose fragments are in
+// registers by then: behind it the loads of slab t+2 go out (the stage they overwrite is no
+// longer read by anybody) and the first fragments of slab t+1 are fetched, all under the
+// shadow of the MFMAs of the last step of slab t.
+template <typename Cfg>
+__global__ __launch_bounds__(Cfg::kThreads) void gemm_f16_nt_tile_kernel(
+	const half_t* __restrict__ A, const half_t* __restrict__ B, half_t* __restrict__ C,
+	int K, int64_t lda, int64_t ldb, int64_t ldc, int tiles_m, int tiles_n)
+{
+	using Shape = MfmaShape<Cfg::MI>;
+	using Acc = typename Shape::Acc;
+	constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK, MI = Cfg::MI;
+	constexpr int TM = Cfg::kTilesM, TN = Cfg::kTilesN;
+	extern __shared__ __align__(1024) char lds[];
+	typedef __attribute__((address_space(3))) void lds_void;
+	typedef const __attribute__((address_space(1))) void global_void;
+
+	const int tid = threadIdx.x;
+	const int lane = tid & (kWaveSize - 1);
+	const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // scalar: LDS targets of direct loads stay in SGPRs
+	const int wm = wave / Cfg::WN;
+	const int wn = wave % Cfg::WN;
+
+	int tile_m, tile_n;
+	tile_of_block<Cfg::GROUP_M>(blockIdx.x, tiles_m, tiles_n, tile_m, tile_n);
+	const int64_t m0 = (int64_t)tile_m * BM;
+	const int64_t n0 = (int64_t)tile_n * BN;
+
+	// Direct loads.  Load instruction i of this wave fills slab rows [8 * (wave * kLoads + i), +8):
+	// lane -> row offset lane / 8, chunk position lane % 8, i.e. logical chunk (lane % 8) ^ swz(row).
+	const int ld_row = lane >> 3;
+	const int ld_pos = lane & 7;
+	const half_t* a_src[Cfg::kLoadsA];
+	const half_t* b_src[Cfg::kLoadsB];
+#pragma unroll
+	for (int i = 0; i < Cfg::kLoadsA; ++i)
+	{
+		const int row = 8 * (wave * Cfg::kLoadsA + i) + ld_row;
+		a_src[i] = A + (m0 + row) * lda + ((ld_pos ^ swizzle_of_row<Cfg::SWZ>(row)) << 3);
+	}
+#pragma unroll
+	for (int i = 0; i < Cfg::kLoadsB; ++i)
+	{
+		const int row = 8 * (wave * Cfg::kLoadsB + i) + ld_row;
+		b_src[i] = B + (n0 + row) * ldb + ((ld_pos ^ swizzle_of_row<Cfg::SWZ>(row)) << 3);
+	}
+
+	auto issue_loads = [&](int kt, int stage) {
+		char* a_lds = lds + stage * Cfg::kStageBytes;
+		char* b_lds = a_lds + Cfg::kSlabABytes;
+		const int64_t koff = (int64_t)kt * BK;
+#pragma unroll
+		for (int i = 0; i < Cfg::kLoadsA; ++i)
+			__builtin_amdgcn_global_load_lds((global_void*)(a_src[i] + koff),
+			                                 (lds_void*)(a_lds + 1024 * (wave * Cfg::kLoadsA + i)), 16, 0, 0);
+#pragma unroll
+		for (int i = 0; i < Cfg::kLoadsB; ++i)
+			__builtin_amdgcn_global_load_lds((global_void*)(b_src[i] + koff),
+			                                 (lds_void*)(b_lds + 1024 * (wave * Cfg::kLoadsB + i)), 16, 0, 0);
+	};
+
+	Acc acc[TM][TN];
+#pragma unroll
+	for (int i = 0; i < TM; ++i)
+#pragma unroll
+		for (int j = 0; j < TN; ++j)
+#pragma unroll
+			for (int r = 0; r < Shape::kAccRegs; ++r) acc[i][j][r] = 0.0f;
+
+	// operand fragments: lane -> slab row (lane % MI) of its MFMA tile, k group (lane / MI)
+	const int frag_row = lane % MI;
+	const int frag_kgroup = lane / MI;
+	int a_off[TM], a_swz[TM], b_off[TN], b_swz[TN];
+#pragma unroll
+	for (int i = 0; i < TM; ++i)
+	{
+		const int row = wm * Cfg::kWaveM + i * MI + frag_row;
+		a_off[i] = row * 128;
+		a_swz[i] = swizzle_of_row<Cfg::SWZ>(row);
+	}
+#pragma unroll
+	for (int j = 0; j < TN; ++j)
+	{
+		const int row = wn * Cfg::kWaveN + j * MI + frag_row;
+		b_off[j] = Cfg::kSlabABytes + row * 128;
+		b_swz[j] = swizzle_of_row<Cfg::SWZ>(row);
+	}
+
+	half8_t af[2][TM], bf[2][TN];
+	auto read_frags = [&](int buf, int stage, int step) {
+		const char* base = lds + stage * Cfg::kStageBytes;
+		const int chunk = step * Cfg::kKGroups + frag_kgroup;
+#pragma unroll
+		for (int i = 0; i < TM; ++i)
+			af[buf][i] = *reinterpret_cast<const half8_t*>(base + a_off[i] + ((chunk ^ a_swz[i]) << 4));
+#pragma unroll
+		for (int j = 0; j < TN; ++j)
+			bf[buf][j] = *reinterpret_cast<const half8_t*>(base + b_off[j] + ((chunk ^ b_swz[j]) << 4));
+	};
+	auto multiply = [&](int buf) {
+#pragma unroll
+		for (int i = 0; i < TM; ++i)
+#pragma unroll
+			for (int j = 0; j < TN; ++j)
+				acc[i][j] = Shape::mma(bf[buf][j], af[buf][i], acc[i][j]);
+	};
+	// where the TM + TN LDS reads of the next step go between the TM * TN MFMAs of this one
+	auto interleave_reads = [&]() {
+		if constexpr (Cfg::ILV == 0)
+		{
+#pragma unroll
+			for (int i = 0; i < TM + TN; ++i)
+			{
+				__builtin_amdgcn_sched_group_barrier(kSchedMfma, 1, 0);
+				__builtin_amdgcn_sched_group_barrier(kSchedDsRead, 1, 0);
+			}
+			__builtin_amdgcn_sched_group_barrier(kSchedMfma, TM * TN - (TM + TN), 0);
+		}
+		else if constexpr (Cfg::ILV == 1)
+		{
+#pragma unroll
+			for (int i = 0; i < (TM + TN) / 2; ++i)
+			{
+				__builtin_amdgcn_sched_group_barrier(kSchedMfma, 1, 0);
+				__builtin_amdgcn_sched_group_barrier(kSchedDsRead, 2, 0);
+			}
+			__builtin_amdgcn_sched_group_barrier(kSchedMfma, TM * TN - (TM + TN) / 2, 0);
+		}
+		// any other value: leave the placement to the compiler
+	};
+
+	const int ktiles = K / BK;
+
+	// Loads past the last slab are clamped to the last slab: they land in a stage nobody reads
+	// any more, which keeps the loop body free of branches.
+	const int last = ktiles - 1;
+	issue_loads(0, 0);
+	wait_vmem_all();
+	__syncthreads();
+	issue_loads(min(1, last), 1);
+	read_frags(0, 0, 0);
+
+	for (int kt = 0; kt < ktiles; ++kt)
+	{
+		const int stage = kt & 1;
+
+#pragma unroll
+		for (int step = 0; step < Cfg::kSteps - 1; ++step)
+		{
+			read_frags((step + 1) & 1, stage, step + 1);
+			multiply(step & 1);
+			interleave_reads();
+		}
+
+		// slab t+1 has landed (own loads) and, behind the barrier, everybody's; stage `stage` is free
+		wait_vmem_all();
+		__syncthreads();
+		issue_loads(min(kt + 2, last), stage);
+		read_frags(0, stage ^ 1, 0);
+		multiply((Cfg::kSteps - 1) & 1);
+		__builtin_amdgcn_sched_group_barrier(kSchedMfma, 1, 0);
+		__builtin_amdgcn_sched_group_barrier(kSchedVmemRead, Cfg::kLoadsA + Cfg::kLoadsB, 0);
+		interleave_reads();
+	}
+	// no direct load may still be writing LDS when the scratch is reused or the block retires
+	wait_vmem_all();
+	__syncthreads();
+	store_patch_via_lds<Cfg>(acc, lds, C, ldc, m0 + wm * Cfg::kWaveM, n0 + wn * Cfg::kWaveN, wave, lane);
+}
+
+template <typename Cfg>
+hipError_t launch_gemm_f16_tile(const half_t* A, const half_t* B, half_t* C, int64_t M, int64_t N, int64_t K,
+                                int64_t lda, int64_t ldb, int64_t ldc, hipStream_t stream)
+{
+	auto kernel = gemm_f16_nt_tile_kernel<Cfg>;
+	static bool configured = false;
+	(void)hipGetLastError();
+	if (!configured)
+	{
+		hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+		                                   hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::kLdsBytes);
+		if (e != hipSuccess) return e;
+		configured = true;
+	}
+	const int tiles_m = (int)(M / Cfg::BM), tiles_n = (int)(N / Cfg::BN);
+	kernel<<<dim3((unsigned)(tiles_m * tiles_n)), dim3(Cfg::kThreads), Cfg::kLdsBytes, stream>>>(
+		A, B, C, (int)K, lda, ldb, ldc, tiles_m, tiles_n);
+	return hipGetLastError();
+}
+
+}  // namespace anygpu

@@ -12,6 +12,8 @@
 #include "device_utils.hpp"
 #include "launch.hpp"
 
+#include <algorithm>
+
 namespace anygpu {
 
 struct SoftmaxArgs
@@ -162,6 +164,145 @@ __global__ __launch_bounds__(256) void softmax_rows_wave_kernel(const SoftmaxArg
 	}
 }
 
+// ---------------------------------------------------------------------------------------------
+// fp16 fast kernel.  One wave per row, the VISIBLE part of the row in registers: lane l owns the
+// 16-byte vectors v_lo + l + 64 t (t < VPL), where v_lo is the first vector that holds a visible
+// key, so a sliding window of W keys needs W / 512 + 1 vectors per lane however long the row is.
+// Vectors without a visible key are never loaded; they are stored as zeros.
+//
+// One pass over the registers runs the online max/sum recurrence per vector and leaves
+// e = exp2(z - m_t) (m_t = running maximum after vector t) in the registers as halves, in place
+// of the input; the sum is accumulated in fp32 from the unrounded values.  After the DPP
+// reductions a second pass over the registers multiplies by exp2(m_t - M) / S in fp32 and rounds
+// to the fp16 output.  The logit transform (scale, softcap) therefore runs once per element.
+// ---------------------------------------------------------------------------------------------
+template <bool SOFTCAP>
+__device__ __forceinline__ float logit2_fast(float x, float k_in, float k_cap)
+{
+	// without softcap: k_in = alpha * log2(e)
+	// with softcap:    cap * log2(e) * tanh(alpha x / cap) = k_cap - 2 k_cap / (1 + exp2(x * k_in)),
+	//                  k_in = 2 log2(e) alpha / cap, k_cap = cap * log2(e); saturates to +-k_cap
+	if constexpr (SOFTCAP)
+	{
+		const float t = fast_exp2(x * k_in);
+		return fmaf(fast_rcp(1.0f + t), -2.0f * k_cap, k_cap);
+	}
+	return x * k_in;
+}
+
+template <int VPL, bool SOFTCAP>
+__global__ __launch_bounds__(256) void softmax_rows_f16_window_kernel(const SoftmaxArgs a)
+{
+	constexpr int EPV = 8;
+	const int lane = threadIdx.x & (kWaveSize - 1);
+	const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+	if (row >= a.rows) return;  // uniform over the wave
+
+	const RowSpan span = row_span(a, row);
+	const half8_t* __restrict__ xr = reinterpret_cast<const half8_t*>(static_cast<const half_t*>(a.x) + row * a.xs);
+	half8_t* __restrict__ yr = reinterpret_cast<half8_t*>(static_cast<half_t*>(a.y) + row * a.ys);
+	const int nvec = (int)(a.cols / EPV);
+	const int lo = (int)span.lo, hi = (int)span.hi;
+	const half8_t zeros = {};
+
+	if (hi < lo)
+	{
+		for (int v = lane; v < nvec; v += kWaveSize) __builtin_nontemporal_store(zeros, yr + v);
+		return;
+	}
+	const int v_lo = lo / EPV, v_hi = hi / EPV;
+
+	half8_t reg[VPL];
+#pragma unroll
+	for (int t = 0; t < VPL; ++t)
+	{
+		const int v = v_lo + lane + kWaveSize * t;
+		half8_t val = {};
+		if (v <= v_hi) val = __builtin_nontemporal_load(xr + v);
+		reg[t] = val;
+	}
+
+	// keys outside the visible interval: exact zeros
+	for (int v = lane; v < v_lo; v += kWaveSize) __builtin_nontemporal_store(zeros, yr + v);
+	for (int v = v_hi + 1 + lane; v < nvec; v += kWaveSize) __builtin_nontemporal_store(zeros, yr + v);
+
+	const float k_in = SOFTCAP ? 2.0f * kLog2e * a.alpha * a.inv_cap : a.alpha_log2e;
+	const float k_cap = a.cap_log2e;
+
+	OnlineState st;
+	float m_at[VPL];
+#pragma unroll
+	for (int t = 0; t < VPL; ++t)
+	{
+		const int v = v_lo + lane + kWaveSize * t;
+		m_at[t] = -INFINITY;
+		if (v <= v_hi)
+		{
+			float z[EPV];
+#pragma unroll
+			for (int e = 0; e < EPV; ++e) z[e] = logit2_fast<SOFTCAP>((float)reg[t][e], k_in, k_cap);
+			if (v == v_lo || v == v_hi)
+			{
+				// only the two end vectors can hold keys outside [lo, hi]
+#pragma unroll
+				for (int e = 0; e < EPV; ++e)
+				{
+					const int j = v * EPV + e;
+					if (j < lo || j > hi) z[e] = -INFINITY;
+				}
+			}
+			float vmax = z[0];
+#pragma unroll
+			for (int e = 1; e < EPV; ++e) vmax = fmaxf(vmax, z[e]);
+			const float mn = fmaxf(st.m, vmax);
+			const float shift = (mn == -INFINITY) ? 0.0f : mn;
+			float acc = st.s * fast_exp2(st.m - shift);
+			half8_t ev;
+#pragma unroll
+			for (int e = 0; e < EPV; ++e)
+			{
+				const float p = fast_exp2(z[e] - shift);
+				acc += p;
+				ev[e] = (half_t)p;
+			}
+			reg[t] = ev;
+			m_at[t] = mn;
+			st.s = acc;
+			st.m = mn;
+		}
+	}
+
+	const float M = wave_allreduce(st.m, MaxOp());
+	const float S = wave_allreduce(st.s * exp2_shift(st.m, M), SumOp());
+	const float inv = S > 0.0f ? 1.0f / S : 0.0f;
+
+#pragma unroll
+	for (int t = 0; t < VPL; ++t)
+	{
+		const int v = v_lo + lane + kWaveSize * t;
+		if (v <= v_hi)
+		{
+			const float scale = exp2_shift(m_at[t], M) * inv;
+			half8_t out;
+#pragma unroll
+			for (int e = 0; e < EPV; ++e) out[e] = (half_t)((float)reg[t][e] * scale);
+			__builtin_nontemporal_store(out, yr + v);
+		}
+	}
+}
+
+template <int VPL>
+static hipError_t launch_f16_window(const SoftmaxArgs& a, hipStream_t stream)
+{
+	const unsigned blocks = (unsigned)((a.rows + 3) / 4);
+	discard_stale_error();
+	if (a.inv_cap != 0.0f)
+		softmax_rows_f16_window_kernel<VPL, true><<<dim3(blocks), dim3(256), 0, stream>>>(a);
+	else
+		softmax_rows_f16_window_kernel<VPL, false><<<dim3(blocks), dim3(256), 0, stream>>>(a);
+	return hipGetLastError();
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void softmax_rows_block_kernel(const SoftmaxArgs a)
 {
@@ -233,6 +374,23 @@ hipError_t launch_softmax_rows(const void* x, void* y, int64_t rows, int64_t col
 	const bool vec_ok = (cols % EPV == 0) && (xs % EPV == 0) && (ys % EPV == 0) &&
 	                    (reinterpret_cast<uintptr_t>(x) % 16 == 0) && (reinterpret_cast<uintptr_t>(y) % 16 == 0);
 	const int64_t nvec = cols / EPV;
+	if constexpr (sizeof(T) == 2)
+	{
+		// vectors a row can touch: its visible keys (the window when causal + window, else the
+		// whole row) plus one for an interval that starts inside a vector
+		const int64_t span = (causal && window > 0) ? std::min<int64_t>(cols, window) : cols;
+		const int64_t span_vecs = std::min<int64_t>(nvec, (span + EPV - 1) / EPV + 1);
+		if (vec_ok)
+		{
+			if (span_vecs <= kWaveSize * 1) return launch_f16_window<1>(a, stream);
+			if (span_vecs <= kWaveSize * 2) return launch_f16_window<2>(a, stream);
+			if (span_vecs <= kWaveSize * 4) return launch_f16_window<4>(a, stream);
+			if (span_vecs <= kWaveSize * 6) return launch_f16_window<6>(a, stream);
+			if (span_vecs <= kWaveSize * 9) return launch_f16_window<9>(a, stream);
+			if (span_vecs <= kWaveSize * 12) return launch_f16_window<12>(a, stream);
+			if (span_vecs <= kWaveSize * 16) return launch_f16_window<16>(a, stream);
+		}
+	}
 	constexpr int kMaxVpl = sizeof(T) == 2 ? 16 : 32;
 	if (vec_ok && nvec <= (int64_t)kWaveSize * kMaxVpl)
 	{

@@ -372,7 +372,8 @@ def test_mm_f16_reference_case_640x1280_1280x320(ops, oracle):
     assert scaled_rel_err(got, want, math.sqrt(1280)) <= TOL_F16_GEMM
 
 
-@pytest.mark.parametrize("m,k,n", [(256, 64, 256), (256, 128, 512), (768, 192, 1024), (1024, 1024, 1024)])
+@pytest.mark.parametrize("m,k,n", [(256, 64, 256), (256, 128, 512), (768, 192, 1024), (1024, 1024, 1024),
+                                   (128, 64, 128), (384, 320, 640), (128, 128, 1152), (2304, 192, 256)])
 def test_mm_f16_tile_kernel_shapes(ops, oracle, m, k, n):
     from anygpu_amd import capi
     a = synth.uniform(m + 1, (m, k)).astype(np.float16)
