@@ -32,9 +32,11 @@ PEAK_FP16_TFLOPS = 2516.6      # dense fp16 MFMA, 256 CU x 4096 flop/clk/CU x 2.
 PEAK_FP32_TFLOPS = 157.3       # fp32 matrix path
 PEAK_HBM_GBS = 8000.0          # HBM3E
 
-# HBM bytes per launch of the headline kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# (see profiles/); None until measured for the current kernel.
-MEASURED_TRAFFIC_BYTES = {"gemm_f16": None, "conv1d": None, "softmax_causal": None, "softmax_gemma2": None}
+# Bytes per launch moved behind the L2s, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE (KiB per
+# dispatch), scaled by what the same counters read for a plain 256 MiB device copy (fetch x 2.000,
+# write x 1.000); the summaries are under profiles/.
+MEASURED_TRAFFIC_BYTES = {"gemm_f16": 234962687, "gemm_f32": 167970906, "conv1d": 277226336,
+                          "softmax_causal": 410887952, "softmax_gemma2": 1514268488}
 
 
 def parse_args():
@@ -51,8 +53,21 @@ def parse_args():
     return ap.parse_args()
 
 
+SETTLE_SECONDS = 0.3
+
+
 def timed_region(torch, fn, steps, warmup):
-    """(host seconds, event seconds) for `steps` calls of fn after `warmup` untimed calls."""
+    """(host seconds, event seconds) for `steps` calls of fn after `warmup` untimed calls.
+
+    Before the warm-up the kernel runs untimed for SETTLE_SECONDS: after an idle period the
+    power management of the GPU over- and undershoots for some tens of milliseconds (a 4096^3
+    GEMM takes 124 us, then up to 160 us, then settles near 100 us after about 150 launches), and
+    the number that matters for a long-running job is the settled one."""
+    t_end = time.perf_counter() + SETTLE_SECONDS
+    while time.perf_counter() < t_end:
+        for _ in range(20):
+            fn()
+        torch.cuda.synchronize()
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
@@ -94,7 +109,7 @@ def bench_gemm_f32(torch, ops, synth, steps, warmup):
         "name": "gemm_f32", "workload": "fp32 GEMM M=N=K=2048, row-major operands, U(-1,1)",
         "us_per_launch": t * 1e6, "value": flops / t / 1e12, "unit": "TFLOP/s", "dtype": "f32",
         "roofline": {"bound": "mfma", "achieved": flops / t / 1e12, "peak": PEAK_FP32_TFLOPS, "unit": "TFLOP/s",
-                     "frac": flops / t / 1e12 / PEAK_FP32_TFLOPS, "traffic": None},
+                     "frac": flops / t / 1e12 / PEAK_FP32_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES["gemm_f32"]},
     }
 
 
@@ -239,7 +254,7 @@ def main():
         "metric": "fp16 GEMM TFLOP/s; conv1d & softmax HBM GB/s (% roofline) on 1 MI355X",
         "value": None, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": None, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f16", "data": "synthetic",
+        "dtype": "f16", "data": "synthetic", "settle_s": SETTLE_SECONDS,
         "config": {"workload": "fp16 GEMM M=N=K=4096, A row-major, B column-major ([N,K] storage), U(-1,1) inputs, "
                                "fp32 accumulate on MFMA, fp16 output (BASELINE.json configs[1])"},
         "device": {"name": props.name, "compute_units": props.multi_processor_count,
