@@ -1,7 +1,8 @@
 // fp16 x fp16 -> fp32-accumulate -> fp16 GEMM for gfx950 on the MFMA units.
 //
-// Tile kernel (gemm_f16_tile.hpp; "NT": A [M,K] and B [N,K], both K-contiguous): 256 x 256 or
-// 128 x 128 tiles of C, direct global -> LDS loads, double-buffered LDS, software-pipelined MFMAs.
+// Tile kernel (gemm_f16_tile.hpp): 256 x 256 or 128 x 128 tiles of C, direct global -> LDS loads,
+// double-buffered LDS, software-pipelined MFMAs; B either [N, K] (k-contiguous like A) or [K, N]
+// (the reference layout, transposed on the way out of LDS).
 //
 // Edge kernel: 64 x 64 tiles, guarded scalar loads and stores, either B layout, any
 // shape, stride and alignment.
@@ -108,6 +109,23 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
 			return launch_gemm_f16_tile<Big>(a, b, c, M, N, K, lda, ldb, ldc, stream);
 		if (M % 128 == 0 && N % 128 == 0 && (M / 128) * (N / 128) <= 0x7FFFFFFFLL)
 			return launch_gemm_f16_tile<Small>(a, b, c, M, N, K, lda, ldb, ldc, stream);
+		// 4 waves, 32 x 32 patch per wave: the granularity the reference's own fp16 kernels require
+		using Tiny = GemmTileCfg<64, 64, 2, 2, 1, 0, 4, 16>;
+		if (M % 64 == 0 && N % 64 == 0 && (M / 64) * (N / 64) <= 0x7FFFFFFFLL)
+			return launch_gemm_f16_tile<Tiny>(a, b, c, M, N, K, lda, ldb, ldc, stream);
+	}
+	if (b_layout == ANYGPU_B_ROW_MAJOR && aligned && K > 0 && K % 64 == 0)
+	{
+		// the reference layout, B stored [K, N]: same tiling, B operand through transposing LDS reads
+		using BigKN = GemmTileCfg<256, 256, 2, 4, 1, 0, 4, 16, true>;
+		using SmallKN = GemmTileCfg<128, 128, 2, 2, 1, 0, 4, 16, true>;
+		if (M % 256 == 0 && N % 256 == 0 && (M / 256) * (N / 256) <= 0x7FFFFFFFLL)
+			return launch_gemm_f16_tile<BigKN>(a, b, c, M, N, K, lda, ldb, ldc, stream);
+		if (M % 128 == 0 && N % 128 == 0 && (M / 128) * (N / 128) <= 0x7FFFFFFFLL)
+			return launch_gemm_f16_tile<SmallKN>(a, b, c, M, N, K, lda, ldb, ldc, stream);
+		using TinyKN = GemmTileCfg<64, 64, 2, 2, 1, 0, 4, 16, true>;
+		if (M % 64 == 0 && N % 64 == 0 && (M / 64) * (N / 64) <= 0x7FFFFFFFLL)
+			return launch_gemm_f16_tile<TinyKN>(a, b, c, M, N, K, lda, ldb, ldc, stream);
 	}
 
 	const dim3 grid((unsigned)((N + 63) / 64), (unsigned)((M + 63) / 64));

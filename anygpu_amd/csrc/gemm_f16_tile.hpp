@@ -88,9 +88,14 @@ template <> struct MfmaShape<16>
 	__device__ static __forceinline__ int first_row_of_group(int g, int lane) { (void)g; return 4 * (lane >> 4); }
 };
 
-template <int BM_, int BN_, int WM_, int WN_, int SWZ_, int ILV_ = 0, int GROUP_M_ = 4, int MI_ = 32>
+template <int BM_, int BN_, int WM_, int WN_, int SWZ_, int ILV_ = 0, int GROUP_M_ = 4, int MI_ = 32, bool B_KN_ = false>
 struct GemmTileCfg
 {
+	// B_KN = false: B stored [N, K] (k-contiguous, like A).  true: B stored [K, N] (the reference
+	// layout): its slab is staged as [64 k][BN n] rows and the k-contiguous MFMA operand is formed by
+	// the transposing LDS read ds_read_b64_tr_b16.
+	static constexpr bool B_KN = B_KN_;
+	static_assert(!B_KN_ || MI_ == 16, "the transposed-B path is written for the 16 x 16 x 32 MFMA");
 	static constexpr int BM = BM_, BN = BN_, BK = 64, WM = WM_, WN = WN_, SWZ = SWZ_;
 	static constexpr int ILV = ILV_;          // how LDS reads are spread between the MFMAs of one step
 	static constexpr int GROUP_M = GROUP_M_;  // rows of tiles per column strip of the tile walk
@@ -120,6 +125,28 @@ struct GemmTileCfg
 __device__ __forceinline__ void wait_vmem_all()
 {
 	__builtin_amdgcn_s_waitcnt(0x0F70);
+}
+
+// Swizzle of a [k][n] slab row (B stored [K, N]): 16-byte chunks move in pairs (a transposing read
+// takes 32 contiguous bytes of a row), pair index ^ s(k).  The 16 lanes of a transposing read cover
+// 4 consecutive k, the four lane groups of a wave sit 8 k apart: s(k) = (k & 3) | ((k >> 3) & 1) << 2
+// gives the 8 rows that 32 lanes read together 8 different 32-byte bank slots.
+__device__ __forceinline__ int kn_row_swizzle(int k)
+{
+	return 2 * ((k & 3) | (((k >> 3) & 1) << 2));
+}
+
+typedef short short4_t __attribute__((ext_vector_type(4)));
+
+// ds_read_b64_tr_b16: within each group of 16 lanes, lane i receives element (i % 4) of the
+// 4-element rows addressed by lanes i / 4, i / 4 + 4, i / 4 + 8, i / 4 + 12 of the group
+// (lane mapping measured on gfx950).  With lane r of a group pointing at B[k0 + r / 4][n0 + 4 (r % 4) ...],
+// lane i ends up with B[k0 .. k0 + 3][n0 + i]: four consecutive k of one column.
+__device__ __forceinline__ half4_t lds_read_transposed_b64(const char* lds_addr)
+{
+	const short4_t v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+		(__attribute__((address_space(3))) short4_t*)(lds_addr));
+	return __builtin_bit_cast(half4_t, v);
 }
 
 // Epilogue through LDS.  With the B slab as the first MFMA operand, a group of 4 accumulator
@@ -219,24 +246,38 @@ __global__ __launch_bounds__(Cfg::kThreads) void gemm_f16_nt_tile_kernel(
 		const int row = 8 * (wave * Cfg::kLoadsA + i) + ld_row;
 		a_src[i] = A + (m0 + row) * lda + ((ld_pos ^ swizzle_of_row<Cfg::SWZ>(row)) << 3);
 	}
+	constexpr int kRowBytesKN = BN * 2;                 // [k][n] slab row
+	constexpr int kRowsPerLoadKN = 1024 / kRowBytesKN;  // k rows one direct load instruction fills
+	constexpr int kChunkMaskKN = BN / 8 - 1;            // narrow slabs have fewer chunk pairs to permute
 #pragma unroll
 	for (int i = 0; i < Cfg::kLoadsB; ++i)
 	{
-		const int row = 8 * (wave * Cfg::kLoadsB + i) + ld_row;
-		b_src[i] = B + (n0 + row) * ldb + ((ld_pos ^ swizzle_of_row<Cfg::SWZ>(row)) << 3);
+		if constexpr (Cfg::B_KN)
+		{
+			const int lanes_per_row = kWaveSize / kRowsPerLoadKN;
+			const int k = kRowsPerLoadKN * (wave * Cfg::kLoadsB + i) + lane / lanes_per_row;
+			const int pos = lane % lanes_per_row;
+			b_src[i] = B + (int64_t)k * ldb + n0 + ((pos ^ (kn_row_swizzle(k) & kChunkMaskKN)) << 3);
+		}
+		else
+		{
+			const int row = 8 * (wave * Cfg::kLoadsB + i) + ld_row;
+			b_src[i] = B + (n0 + row) * ldb + ((ld_pos ^ swizzle_of_row<Cfg::SWZ>(row)) << 3);
+		}
 	}
 
 	auto issue_loads = [&](int kt, int stage) {
 		char* a_lds = lds + stage * Cfg::kStageBytes;
 		char* b_lds = a_lds + Cfg::kSlabABytes;
 		const int64_t koff = (int64_t)kt * BK;
+		const int64_t koff_b = Cfg::B_KN ? koff * ldb : koff;
 #pragma unroll
 		for (int i = 0; i < Cfg::kLoadsA; ++i)
 			__builtin_amdgcn_global_load_lds((global_void*)(a_src[i] + koff),
 			                                 (lds_void*)(a_lds + 1024 * (wave * Cfg::kLoadsA + i)), 16, 0, 0);
 #pragma unroll
 		for (int i = 0; i < Cfg::kLoadsB; ++i)
-			__builtin_amdgcn_global_load_lds((global_void*)(b_src[i] + koff),
+			__builtin_amdgcn_global_load_lds((global_void*)(b_src[i] + koff_b),
 			                                 (lds_void*)(b_lds + 1024 * (wave * Cfg::kLoadsB + i)), 16, 0, 0);
 	};
 
@@ -259,12 +300,25 @@ __global__ __launch_bounds__(Cfg::kThreads) void gemm_f16_nt_tile_kernel(
 		a_off[i] = row * 128;
 		a_swz[i] = swizzle_of_row<Cfg::SWZ>(row);
 	}
+	int b_off_kn[TN][2];   // transposed-B path: byte offsets of the two 4-deep transposing reads of a fragment
 #pragma unroll
 	for (int j = 0; j < TN; ++j)
 	{
 		const int row = wn * Cfg::kWaveN + j * MI + frag_row;
 		b_off[j] = Cfg::kSlabABytes + row * 128;
 		b_swz[j] = swizzle_of_row<Cfg::SWZ>(row);
+		if constexpr (Cfg::B_KN)
+		{
+			// lane r of a 16-lane group addresses row k = 8 g + 4 h + r / 4, columns n .. n + 3
+			const int n = wn * Cfg::kWaveN + j * MI + 4 * (frag_row & 3);
+#pragma unroll
+			for (int h = 0; h < 2; ++h)
+			{
+				const int k = 8 * frag_kgroup + 4 * h + (frag_row >> 2);
+				b_off_kn[j][h] = Cfg::kSlabABytes + k * kRowBytesKN +
+				                 (((n >> 3) ^ (kn_row_swizzle(k) & kChunkMaskKN)) << 4) + (n & 7) * 2;
+			}
+		}
 	}
 
 	half8_t af[2][TM], bf[2][TN];
@@ -276,7 +330,20 @@ __global__ __launch_bounds__(Cfg::kThreads) void gemm_f16_nt_tile_kernel(
 			af[buf][i] = *reinterpret_cast<const half8_t*>(base + a_off[i] + ((chunk ^ a_swz[i]) << 4));
 #pragma unroll
 		for (int j = 0; j < TN; ++j)
-			bf[buf][j] = *reinterpret_cast<const half8_t*>(base + b_off[j] + ((chunk ^ b_swz[j]) << 4));
+		{
+			if constexpr (Cfg::B_KN)
+			{
+				// a step is 32 k deep; + 32 k rows leaves the row swizzle (bits 0, 1, 3 of k) unchanged
+				const char* src = base + step * (32 * kRowBytesKN);
+				const half4_t lo = lds_read_transposed_b64(src + b_off_kn[j][0]);
+				const half4_t hi = lds_read_transposed_b64(src + b_off_kn[j][1]);
+				bf[buf][j] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+			}
+			else
+			{
+				bf[buf][j] = *reinterpret_cast<const half8_t*>(base + b_off[j] + ((chunk ^ b_swz[j]) << 4));
+			}
+		}
 	};
 	auto multiply = [&](int buf) {
 #pragma unroll
@@ -285,27 +352,28 @@ __global__ __launch_bounds__(Cfg::kThreads) void gemm_f16_nt_tile_kernel(
 			for (int j = 0; j < TN; ++j)
 				acc[i][j] = Shape::mma(bf[buf][j], af[buf][i], acc[i][j]);
 	};
-	// where the TM + TN LDS reads of the next step go between the TM * TN MFMAs of this one
+	// where the LDS reads of the next step go between the TM * TN MFMAs of this one
+	constexpr int kReads = TM + (Cfg::B_KN ? 2 * TN : TN);
 	auto interleave_reads = [&]() {
 		if constexpr (Cfg::ILV == 0)
 		{
 #pragma unroll
-			for (int i = 0; i < TM + TN; ++i)
+			for (int i = 0; i < kReads; ++i)
 			{
 				__builtin_amdgcn_sched_group_barrier(kSchedMfma, 1, 0);
 				__builtin_amdgcn_sched_group_barrier(kSchedDsRead, 1, 0);
 			}
-			__builtin_amdgcn_sched_group_barrier(kSchedMfma, TM * TN - (TM + TN), 0);
+			__builtin_amdgcn_sched_group_barrier(kSchedMfma, TM * TN - kReads, 0);
 		}
 		else if constexpr (Cfg::ILV == 1)
 		{
 #pragma unroll
-			for (int i = 0; i < (TM + TN) / 2; ++i)
+			for (int i = 0; i < kReads / 2; ++i)
 			{
 				__builtin_amdgcn_sched_group_barrier(kSchedMfma, 1, 0);
 				__builtin_amdgcn_sched_group_barrier(kSchedDsRead, 2, 0);
 			}
-			__builtin_amdgcn_sched_group_barrier(kSchedMfma, TM * TN - (TM + TN) / 2, 0);
+			__builtin_amdgcn_sched_group_barrier(kSchedMfma, TM * TN - kReads / 2, 0);
 		}
 		// any other value: leave the placement to the compiler
 	};

@@ -373,15 +373,21 @@ def test_mm_f16_reference_case_640x1280_1280x320(ops, oracle):
 
 
 @pytest.mark.parametrize("m,k,n", [(256, 64, 256), (256, 128, 512), (768, 192, 1024), (1024, 1024, 1024),
-                                   (128, 64, 128), (384, 320, 640), (128, 128, 1152), (2304, 192, 256)])
+                                   (128, 64, 128), (384, 320, 640), (128, 128, 1152), (2304, 192, 256),
+                                   (64, 64, 64), (640, 1280, 320), (192, 448, 64), (320, 64, 1088)])
 def test_mm_f16_tile_kernel_shapes(ops, oracle, m, k, n):
     from anygpu_amd import capi
     a = synth.uniform(m + 1, (m, k)).astype(np.float16)
     bt = synth.uniform(n + 2, (n, k)).astype(np.float16)
-    got = host(ops.tensor_mm(dev(a), dev(bt), b_layout=capi.B_COL_MAJOR)).astype(np.float32)
     want = oracle.tensor_mm(oracle.cvt_f16_to_f32(a), oracle.cvt_f16_to_f32(bt).T, threads=8)
+    got = host(ops.tensor_mm(dev(a), dev(bt), b_layout=capi.B_COL_MAJOR)).astype(np.float32)
     assert scaled_rel_err(got, want, math.sqrt(k) / 3.0) <= TOL_F16_GEMM
     assert rel_l2(got, want) <= 1e-2
+    # the same product with B in the reference layout [K, N] (transposing LDS reads)
+    got_kn = host(ops.tensor_mm(dev(a), dev(np.ascontiguousarray(bt.T)))).astype(np.float32)
+    assert scaled_rel_err(got_kn, want, math.sqrt(k) / 3.0) <= TOL_F16_GEMM
+    # both layouts feed the same MFMA sequence: identical results
+    assert np.array_equal(got_kn, got)
 
 
 def test_mm_f16_config_4096_cubed_col_major_b(ops, oracle):
