@@ -32,6 +32,16 @@ SIGNATURES = {
                                        c_int64, c_int64, c_int64, c_int, c_void_p]),
     "anygpu_gemm_f32": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64,
                                 c_int64, c_int64, c_int64, c_int, c_int, c_void_p]),
+    "anygpu_gemm_f16_f32acc_batched": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64,
+                                               c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,
+                                               c_int, c_void_p]),
+    "anygpu_gemm_f32_batched": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64,
+                                        c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,
+                                        c_int, c_int, c_void_p]),
+    "anygpu_softmax_rows_masked_f16": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64,
+                                               c_int64, c_float, c_float, c_void_p]),
+    "anygpu_softmax_rows_masked_f32": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64,
+                                               c_int64, c_float, c_float, c_void_p]),
     "anygpu_softmax_rows_f16": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,
                                         c_float, c_float, c_int, c_int64, c_void_p]),
     "anygpu_softmax_rows_f32": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,

@@ -62,7 +62,30 @@ int softmax_entry(const void* x, void* y, int64_t rows, int64_t cols, int64_t xs
 	// keep i + diag and i + diag - window + 1 inside 64-bit range whatever the caller passes
 	if (diag > kMaxIndex32 || diag < -kMaxIndex32) return ANYGPU_ERR_TOO_LARGE;
 	return (int)anygpu::launch_softmax_rows<T>(x, y, rows, cols, xs, ys, q_len, diag, alpha, softcap, causal,
-	                                            window, as_stream(stream));
+	                                            window, nullptr, 0, as_stream(stream));
+}
+
+template <typename T>
+int softmax_masked_entry(const void* x, const void* mask, void* y, int64_t rows, int64_t cols,
+                         int64_t xs, int64_t ms, int64_t ys, int64_t q_len, float alpha, float softcap, void* stream)
+{
+	const int rc = check_softmax(x, y, rows, cols, xs, ys, 0);
+	if (rc != ANYGPU_OK) return rc;
+	if (rows == 0 || cols == 0) return ANYGPU_OK;
+	if (mask == nullptr) return ANYGPU_ERR_NULL_POINTER;
+	if (ms < cols) return ANYGPU_ERR_BAD_STRIDE;
+	if (q_len > kMaxIndex32) return ANYGPU_ERR_TOO_LARGE;
+	return (int)anygpu::launch_softmax_rows<T>(x, y, rows, cols, xs, ys, q_len, 0, alpha, softcap, 0, 0,
+	                                            mask, ms, as_stream(stream));
+}
+
+int check_batch(int64_t batch, int64_t stride_a, int64_t stride_b, int64_t stride_c, int64_t M, int64_t N, int64_t ldc)
+{
+	if (batch < 0 || stride_a < 0 || stride_b < 0 || stride_c < 0) return ANYGPU_ERR_BAD_SHAPE;
+	if (batch > 65535) return ANYGPU_ERR_TOO_LARGE;
+	// results of different products must not overlap
+	if (batch > 1 && M > 0 && N > 0 && stride_c < (M - 1) * ldc + N) return ANYGPU_ERR_BAD_STRIDE;
+	return ANYGPU_OK;
 }
 
 template <typename T>
@@ -107,7 +130,20 @@ ANYGPU_EXPORT int anygpu_gemm_f16_f32acc(const void* A, const void* B, void* C,
 {
 	const int rc = check_gemm(A, B, C, M, N, K, lda, ldb, ldc, ANYGPU_A_ROW_MAJOR, b_layout);
 	if (rc != ANYGPU_OK) return rc;
-	return (int)anygpu::launch_gemm_f16(A, B, C, M, N, K, lda, ldb, ldc, b_layout, as_stream(stream));
+	return (int)anygpu::launch_gemm_f16(A, B, C, M, N, K, lda, ldb, ldc, 0, 0, 0, 1, b_layout, as_stream(stream));
+}
+
+ANYGPU_EXPORT int anygpu_gemm_f16_f32acc_batched(const void* A, const void* B, void* C,
+                                                 int64_t M, int64_t N, int64_t K,
+                                                 int64_t lda, int64_t ldb, int64_t ldc,
+                                                 int64_t stride_a, int64_t stride_b, int64_t stride_c, int64_t batch,
+                                                 int b_layout, void* stream)
+{
+	int rc = check_gemm(A, B, C, M, N, K, lda, ldb, ldc, ANYGPU_A_ROW_MAJOR, b_layout);
+	if (rc == ANYGPU_OK) rc = check_batch(batch, stride_a, stride_b, stride_c, M, N, ldc);
+	if (rc != ANYGPU_OK) return rc;
+	return (int)anygpu::launch_gemm_f16(A, B, C, M, N, K, lda, ldb, ldc, stride_a, stride_b, stride_c, batch,
+	                                    b_layout, as_stream(stream));
 }
 
 ANYGPU_EXPORT int anygpu_gemm_f32(const float* A, const float* B, const float* bias, float* C,
@@ -117,8 +153,21 @@ ANYGPU_EXPORT int anygpu_gemm_f32(const float* A, const float* B, const float* b
 {
 	const int rc = check_gemm(A, B, C, M, N, K, lda, ldb, ldc, a_layout, b_layout);
 	if (rc != ANYGPU_OK) return rc;
-	return (int)anygpu::launch_gemm_f32(A, B, bias, C, M, N, K, lda, ldb, ldc, a_layout, b_layout,
+	return (int)anygpu::launch_gemm_f32(A, B, bias, C, M, N, K, lda, ldb, ldc, 0, 0, 0, 1, a_layout, b_layout,
 	                                    as_stream(stream));
+}
+
+ANYGPU_EXPORT int anygpu_gemm_f32_batched(const float* A, const float* B, float* C,
+                                          int64_t M, int64_t N, int64_t K,
+                                          int64_t lda, int64_t ldb, int64_t ldc,
+                                          int64_t stride_a, int64_t stride_b, int64_t stride_c, int64_t batch,
+                                          int a_layout, int b_layout, void* stream)
+{
+	int rc = check_gemm(A, B, C, M, N, K, lda, ldb, ldc, a_layout, b_layout);
+	if (rc == ANYGPU_OK) rc = check_batch(batch, stride_a, stride_b, stride_c, M, N, ldc);
+	if (rc != ANYGPU_OK) return rc;
+	return (int)anygpu::launch_gemm_f32(A, B, nullptr, C, M, N, K, lda, ldb, ldc, stride_a, stride_b, stride_c, batch,
+	                                    a_layout, b_layout, as_stream(stream));
 }
 
 ANYGPU_EXPORT int anygpu_softmax_rows_f16(const void* x, void* y, int64_t rows, int64_t cols,
@@ -137,6 +186,22 @@ ANYGPU_EXPORT int anygpu_softmax_rows_f32(const float* x, float* y, int64_t rows
 {
 	return softmax_entry<float>(x, y, rows, cols, x_row_stride, y_row_stride, q_len, diag, alpha, softcap,
 	                            causal, window, stream);
+}
+
+ANYGPU_EXPORT int anygpu_softmax_rows_masked_f16(const void* x, const void* mask, void* y, int64_t rows, int64_t cols,
+                                                 int64_t x_row_stride, int64_t mask_row_stride, int64_t y_row_stride,
+                                                 int64_t q_len, float alpha, float softcap, void* stream)
+{
+	return softmax_masked_entry<anygpu::half_t>(x, mask, y, rows, cols, x_row_stride, mask_row_stride, y_row_stride,
+	                                            q_len, alpha, softcap, stream);
+}
+
+ANYGPU_EXPORT int anygpu_softmax_rows_masked_f32(const float* x, const float* mask, float* y, int64_t rows, int64_t cols,
+                                                 int64_t x_row_stride, int64_t mask_row_stride, int64_t y_row_stride,
+                                                 int64_t q_len, float alpha, float softcap, void* stream)
+{
+	return softmax_masked_entry<float>(x, mask, y, rows, cols, x_row_stride, mask_row_stride, y_row_stride,
+	                                   q_len, alpha, softcap, stream);
 }
 
 ANYGPU_EXPORT int anygpu_causal_conv1d_silu_f16(const void* x, const void* w, const void* bias, void* y,

@@ -20,9 +20,13 @@ namespace anygpu {
 template <int B_LAYOUT>
 __global__ __launch_bounds__(256) void gemm_f16_edge_kernel(
 	const half_t* __restrict__ A, const half_t* __restrict__ B, half_t* __restrict__ C,
-	int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc)
+	int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc,
+	int64_t stride_a, int64_t stride_b, int64_t stride_c)
 {
 	__shared__ half_t a_lds[64][16 + 8];
+	A += (int64_t)blockIdx.z * stride_a;
+	B += (int64_t)blockIdx.z * stride_b;
+	C += (int64_t)blockIdx.z * stride_c;
 	__shared__ half_t b_lds[64][16 + 8];
 
 	const int tid = threadIdx.x;
@@ -87,15 +91,18 @@ __global__ __launch_bounds__(256) void gemm_f16_edge_kernel(
 }
 
 hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K,
-                           int64_t lda, int64_t ldb, int64_t ldc, int b_layout, hipStream_t stream)
+                           int64_t lda, int64_t ldb, int64_t ldc,
+                           int64_t stride_a, int64_t stride_b, int64_t stride_c, int64_t batch,
+                           int b_layout, hipStream_t stream)
 {
-	if (M == 0 || N == 0) return hipSuccess;
+	if (M == 0 || N == 0 || batch == 0) return hipSuccess;
 	const half_t* a = static_cast<const half_t*>(A);
 	const half_t* b = static_cast<const half_t*>(B);
 	half_t* c = static_cast<half_t*>(C);
 
 	const bool aligned = (reinterpret_cast<uintptr_t>(A) % 16 == 0) && (reinterpret_cast<uintptr_t>(B) % 16 == 0) &&
-	                     (reinterpret_cast<uintptr_t>(C) % 16 == 0) && (lda % 8 == 0) && (ldb % 8 == 0) && (ldc % 8 == 0);
+	                     (reinterpret_cast<uintptr_t>(C) % 16 == 0) && (lda % 8 == 0) && (ldb % 8 == 0) && (ldc % 8 == 0) &&
+	                     (stride_a % 8 == 0) && (stride_b % 8 == 0) && (stride_c % 8 == 0);
 	if (b_layout == ANYGPU_B_COL_MAJOR && aligned && K > 0 && K % 64 == 0)
 	{
 		// 8 waves, 128 x 64 patch per wave, 64-bank swizzle, one LDS read behind each of the first
@@ -106,13 +113,13 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
 		// 4 waves, 64 x 64 patch per wave: two blocks fit a CU; for shapes that are not multiples of 256
 		using Small = GemmTileCfg<128, 128, 2, 2, 1, 0, 4, 16>;
 		if (M % 256 == 0 && N % 256 == 0 && (M / 256) * (N / 256) <= 0x7FFFFFFFLL)
-			return launch_gemm_f16_tile<Big>(a, b, c, M, N, K, lda, ldb, ldc, stream);
+			return launch_gemm_f16_tile<Big>(a, b, c, M, N, K, lda, ldb, ldc, stride_a, stride_b, stride_c, batch, stream);
 		if (M % 128 == 0 && N % 128 == 0 && (M / 128) * (N / 128) <= 0x7FFFFFFFLL)
-			return launch_gemm_f16_tile<Small>(a, b, c, M, N, K, lda, ldb, ldc, stream);
+			return launch_gemm_f16_tile<Small>(a, b, c, M, N, K, lda, ldb, ldc, stride_a, stride_b, stride_c, batch, stream);
 		// 4 waves, 32 x 32 patch per wave: the granularity the reference's own fp16 kernels require
 		using Tiny = GemmTileCfg<64, 64, 2, 2, 1, 0, 4, 16>;
 		if (M % 64 == 0 && N % 64 == 0 && (M / 64) * (N / 64) <= 0x7FFFFFFFLL)
-			return launch_gemm_f16_tile<Tiny>(a, b, c, M, N, K, lda, ldb, ldc, stream);
+			return launch_gemm_f16_tile<Tiny>(a, b, c, M, N, K, lda, ldb, ldc, stride_a, stride_b, stride_c, batch, stream);
 	}
 	if (b_layout == ANYGPU_B_ROW_MAJOR && aligned && K > 0 && K % 64 == 0)
 	{
@@ -120,20 +127,22 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
 		using BigKN = GemmTileCfg<256, 256, 2, 4, 1, 0, 4, 16, true>;
 		using SmallKN = GemmTileCfg<128, 128, 2, 2, 1, 0, 4, 16, true>;
 		if (M % 256 == 0 && N % 256 == 0 && (M / 256) * (N / 256) <= 0x7FFFFFFFLL)
-			return launch_gemm_f16_tile<BigKN>(a, b, c, M, N, K, lda, ldb, ldc, stream);
+			return launch_gemm_f16_tile<BigKN>(a, b, c, M, N, K, lda, ldb, ldc, stride_a, stride_b, stride_c, batch, stream);
 		if (M % 128 == 0 && N % 128 == 0 && (M / 128) * (N / 128) <= 0x7FFFFFFFLL)
-			return launch_gemm_f16_tile<SmallKN>(a, b, c, M, N, K, lda, ldb, ldc, stream);
+			return launch_gemm_f16_tile<SmallKN>(a, b, c, M, N, K, lda, ldb, ldc, stride_a, stride_b, stride_c, batch, stream);
 		using TinyKN = GemmTileCfg<64, 64, 2, 2, 1, 0, 4, 16, true>;
 		if (M % 64 == 0 && N % 64 == 0 && (M / 64) * (N / 64) <= 0x7FFFFFFFLL)
-			return launch_gemm_f16_tile<TinyKN>(a, b, c, M, N, K, lda, ldb, ldc, stream);
+			return launch_gemm_f16_tile<TinyKN>(a, b, c, M, N, K, lda, ldb, ldc, stride_a, stride_b, stride_c, batch, stream);
 	}
 
-	const dim3 grid((unsigned)((N + 63) / 64), (unsigned)((M + 63) / 64));
+	const dim3 grid((unsigned)((N + 63) / 64), (unsigned)((M + 63) / 64), (unsigned)batch);
 	discard_stale_error();
 	if (b_layout == ANYGPU_B_COL_MAJOR)
-		gemm_f16_edge_kernel<ANYGPU_B_COL_MAJOR><<<grid, dim3(256), 0, stream>>>(a, b, c, M, N, K, lda, ldb, ldc);
+		gemm_f16_edge_kernel<ANYGPU_B_COL_MAJOR><<<grid, dim3(256), 0, stream>>>(a, b, c, M, N, K, lda, ldb, ldc,
+		                                                                 stride_a, stride_b, stride_c);
 	else
-		gemm_f16_edge_kernel<ANYGPU_B_ROW_MAJOR><<<grid, dim3(256), 0, stream>>>(a, b, c, M, N, K, lda, ldb, ldc);
+		gemm_f16_edge_kernel<ANYGPU_B_ROW_MAJOR><<<grid, dim3(256), 0, stream>>>(a, b, c, M, N, K, lda, ldb, ldc,
+		                                                                 stride_a, stride_b, stride_c);
 	return hipGetLastError();
 }
 

@@ -213,9 +213,14 @@ constexpr int kSchedDsRead = 0x100;
 template <typename Cfg>
 __global__ __launch_bounds__(Cfg::kThreads) void gemm_f16_nt_tile_kernel(
 	const half_t* __restrict__ A, const half_t* __restrict__ B, half_t* __restrict__ C,
-	int K, int64_t lda, int64_t ldb, int64_t ldc, int tiles_m, int tiles_n)
+	int K, int64_t lda, int64_t ldb, int64_t ldc, int tiles_m, int tiles_n,
+	int64_t stride_a, int64_t stride_b, int64_t stride_c)
 {
 	using Shape = MfmaShape<Cfg::MI>;
+	// blockIdx.y walks a batch of independent products that share the shape
+	A += (int64_t)blockIdx.y * stride_a;
+	B += (int64_t)blockIdx.y * stride_b;
+	C += (int64_t)blockIdx.y * stride_c;
 	using Acc = typename Shape::Acc;
 	constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK, MI = Cfg::MI;
 	constexpr int TM = Cfg::kTilesM, TN = Cfg::kTilesN;
@@ -419,7 +424,8 @@ __global__ __launch_bounds__(Cfg::kThreads) void gemm_f16_nt_tile_kernel(
 
 template <typename Cfg>
 hipError_t launch_gemm_f16_tile(const half_t* A, const half_t* B, half_t* C, int64_t M, int64_t N, int64_t K,
-                                int64_t lda, int64_t ldb, int64_t ldc, hipStream_t stream)
+                                int64_t lda, int64_t ldb, int64_t ldc,
+                                int64_t stride_a, int64_t stride_b, int64_t stride_c, int64_t batch, hipStream_t stream)
 {
 	auto kernel = gemm_f16_nt_tile_kernel<Cfg>;
 	static bool configured = false;
@@ -432,8 +438,8 @@ hipError_t launch_gemm_f16_tile(const half_t* A, const half_t* B, half_t* C, int
 		configured = true;
 	}
 	const int tiles_m = (int)(M / Cfg::BM), tiles_n = (int)(N / Cfg::BN);
-	kernel<<<dim3((unsigned)(tiles_m * tiles_n)), dim3(Cfg::kThreads), Cfg::kLdsBytes, stream>>>(
-		A, B, C, (int)K, lda, ldb, ldc, tiles_m, tiles_n);
+	kernel<<<dim3((unsigned)(tiles_m * tiles_n), (unsigned)batch), dim3(Cfg::kThreads), Cfg::kLdsBytes, stream>>>(
+		A, B, C, (int)K, lda, ldb, ldc, tiles_m, tiles_n, stride_a, stride_b, stride_c);
 	return hipGetLastError();
 }
 

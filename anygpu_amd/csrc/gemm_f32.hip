@@ -90,8 +90,12 @@ struct Slab
 template <int A_LAYOUT, int B_LAYOUT, bool FULL>
 __global__ __launch_bounds__(256) void gemm_f32_kernel(
 	const float* __restrict__ A, const float* __restrict__ B, const float* __restrict__ bias, float* __restrict__ C,
-	int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc)
+	int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc,
+	int64_t stride_a, int64_t stride_b, int64_t stride_c)
 {
+	A += (int64_t)blockIdx.z * stride_a;
+	B += (int64_t)blockIdx.z * stride_b;
+	C += (int64_t)blockIdx.z * stride_c;
 	using SlabA = Slab<A_LAYOUT == ANYGPU_A_ROW_MAJOR, FULL>;
 	using SlabB = Slab<B_LAYOUT == ANYGPU_B_COL_MAJOR, FULL>;
 	__shared__ __align__(16) float a_lds[2][SlabA::kLdsFloats];
@@ -196,34 +200,44 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(
 template <int A_LAYOUT, int B_LAYOUT>
 static hipError_t launch_layout(const float* A, const float* B, const float* bias, float* C,
                                 int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc,
+                                int64_t stride_a, int64_t stride_b, int64_t stride_c, int64_t batch,
                                 hipStream_t stream)
 {
-	const dim3 grid((unsigned)((N + kBN - 1) / kBN), (unsigned)((M + kBM - 1) / kBM));
+	const dim3 grid((unsigned)((N + kBN - 1) / kBN), (unsigned)((M + kBM - 1) / kBM), (unsigned)batch);
 	const bool aligned = (reinterpret_cast<uintptr_t>(A) % 16 == 0) && (reinterpret_cast<uintptr_t>(B) % 16 == 0) &&
-	                     (reinterpret_cast<uintptr_t>(C) % 16 == 0) && (lda % 4 == 0) && (ldb % 4 == 0) && (ldc % 4 == 0);
+	                     (reinterpret_cast<uintptr_t>(C) % 16 == 0) && (lda % 4 == 0) && (ldb % 4 == 0) && (ldc % 4 == 0) &&
+	                     (stride_a % 4 == 0) && (stride_b % 4 == 0) && (stride_c % 4 == 0);
 	const bool full = aligned && (M % kBM == 0) && (N % kBN == 0) && (K % kBK == 0);
 	discard_stale_error();
 	if (full)
-		gemm_f32_kernel<A_LAYOUT, B_LAYOUT, true><<<grid, dim3(256), 0, stream>>>(A, B, bias, C, M, N, K, lda, ldb, ldc);
+		gemm_f32_kernel<A_LAYOUT, B_LAYOUT, true><<<grid, dim3(256), 0, stream>>>(A, B, bias, C, M, N, K, lda, ldb, ldc,
+		                                                                            stride_a, stride_b, stride_c);
 	else
-		gemm_f32_kernel<A_LAYOUT, B_LAYOUT, false><<<grid, dim3(256), 0, stream>>>(A, B, bias, C, M, N, K, lda, ldb, ldc);
+		gemm_f32_kernel<A_LAYOUT, B_LAYOUT, false><<<grid, dim3(256), 0, stream>>>(A, B, bias, C, M, N, K, lda, ldb, ldc,
+		                                                                            stride_a, stride_b, stride_c);
 	return hipGetLastError();
 }
 
 hipError_t launch_gemm_f32(const float* A, const float* B, const float* bias, float* C,
                            int64_t M, int64_t N, int64_t K,
-                           int64_t lda, int64_t ldb, int64_t ldc, int a_layout, int b_layout, hipStream_t stream)
+                           int64_t lda, int64_t ldb, int64_t ldc,
+                           int64_t stride_a, int64_t stride_b, int64_t stride_c, int64_t batch,
+                           int a_layout, int b_layout, hipStream_t stream)
 {
-	if (M == 0 || N == 0) return hipSuccess;
+	if (M == 0 || N == 0 || batch == 0) return hipSuccess;
 	if (a_layout == ANYGPU_A_ROW_MAJOR)
 	{
 		if (b_layout == ANYGPU_B_COL_MAJOR)
-			return launch_layout<ANYGPU_A_ROW_MAJOR, ANYGPU_B_COL_MAJOR>(A, B, bias, C, M, N, K, lda, ldb, ldc, stream);
-		return launch_layout<ANYGPU_A_ROW_MAJOR, ANYGPU_B_ROW_MAJOR>(A, B, bias, C, M, N, K, lda, ldb, ldc, stream);
+			return launch_layout<ANYGPU_A_ROW_MAJOR, ANYGPU_B_COL_MAJOR>(A, B, bias, C, M, N, K, lda, ldb, ldc,
+		                                                             stride_a, stride_b, stride_c, batch, stream);
+		return launch_layout<ANYGPU_A_ROW_MAJOR, ANYGPU_B_ROW_MAJOR>(A, B, bias, C, M, N, K, lda, ldb, ldc,
+		                                                             stride_a, stride_b, stride_c, batch, stream);
 	}
 	if (b_layout == ANYGPU_B_COL_MAJOR)
-		return launch_layout<ANYGPU_A_COL_MAJOR, ANYGPU_B_COL_MAJOR>(A, B, bias, C, M, N, K, lda, ldb, ldc, stream);
-	return launch_layout<ANYGPU_A_COL_MAJOR, ANYGPU_B_ROW_MAJOR>(A, B, bias, C, M, N, K, lda, ldb, ldc, stream);
+		return launch_layout<ANYGPU_A_COL_MAJOR, ANYGPU_B_COL_MAJOR>(A, B, bias, C, M, N, K, lda, ldb, ldc,
+		                                                             stride_a, stride_b, stride_c, batch, stream);
+	return launch_layout<ANYGPU_A_COL_MAJOR, ANYGPU_B_ROW_MAJOR>(A, B, bias, C, M, N, K, lda, ldb, ldc,
+		                                                             stride_a, stride_b, stride_c, batch, stream);
 }
 
 }  // namespace anygpu

@@ -12,21 +12,27 @@ namespace anygpu {
 // afterwards (hipGetLastError) belongs to that launch and to nothing earlier in the process.
 inline void discard_stale_error() { (void)hipGetLastError(); }
 
+// mask (may be NULL): additive [q_len, cols] matrix of the element type, rows mask_stride apart
 template <typename T>
 hipError_t launch_softmax_rows(const void* x, void* y, int64_t rows, int64_t cols, int64_t xs, int64_t ys,
                                int64_t q_len, int64_t diag, float alpha, float softcap, int causal,
-                               int64_t window, hipStream_t stream);
+                               int64_t window, const void* mask, int64_t mask_stride, hipStream_t stream);
 
 template <typename T>
 hipError_t launch_causal_conv1d_silu(const void* x, const void* w, const void* bias, void* y,
                                      int64_t batch, int64_t chan, int64_t seqlen, int width,
                                      hipStream_t stream);
 
+// `batch` independent products of one shape, operand b of product i at base + i * stride_b (elements)
 hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K,
-                           int64_t lda, int64_t ldb, int64_t ldc, int b_layout, hipStream_t stream);
+                           int64_t lda, int64_t ldb, int64_t ldc,
+                           int64_t stride_a, int64_t stride_b, int64_t stride_c, int64_t batch,
+                           int b_layout, hipStream_t stream);
 
 hipError_t launch_gemm_f32(const float* A, const float* B, const float* bias, float* C,
                            int64_t M, int64_t N, int64_t K,
-                           int64_t lda, int64_t ldb, int64_t ldc, int a_layout, int b_layout, hipStream_t stream);
+                           int64_t lda, int64_t ldb, int64_t ldc,
+                           int64_t stride_a, int64_t stride_b, int64_t stride_c, int64_t batch,
+                           int a_layout, int b_layout, hipStream_t stream);
 
 }  // namespace anygpu

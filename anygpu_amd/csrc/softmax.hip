@@ -29,23 +29,26 @@ struct SoftmaxArgs
 	float alpha_log2e;     // alpha * log2(e), used when the softcap is off
 	int causal;
 	int64_t window;
+	const void* mask;      // optional additive mask [q_len, cols] of the element type (NULL: none)
+	int64_t mask_stride;   // elements between mask rows
 };
 
 template <typename T> struct Vec16;
 template <> struct Vec16<half_t> { using type = half8_t; };
 template <> struct Vec16<float> { using type = float4_t; };
 
+// Query index of a row: which mask row / causal diagonal it belongs to.
+__device__ __forceinline__ int64_t query_of_row(const SoftmaxArgs& a, int64_t row)
+{
+	return a.q_len > 0 ? (int64_t)((uint32_t)row % (uint32_t)a.q_len) : row;
+}
+
 // Visible key interval of a row, inclusive on both ends; empty when hi < lo.
 struct RowSpan { int64_t lo, hi; };
 
 __device__ __forceinline__ RowSpan row_span(const SoftmaxArgs& a, int64_t row)
 {
-	int64_t i = row;
-	if (a.q_len > 0)
-	{
-		// rows and q_len are validated to fit 32 bits by the host entry point
-		i = (int64_t)((uint32_t)row % (uint32_t)a.q_len);
-	}
+	const int64_t i = query_of_row(a, row);   // rows and q_len fit 32 bits (checked by the entry point)
 	RowSpan s;
 	s.hi = a.cols - 1;
 	s.lo = 0;
@@ -95,6 +98,20 @@ __global__ __launch_bounds__(256) void softmax_rows_wave_kernel(const SoftmaxArg
 	T* __restrict__ yr = static_cast<T*>(a.y) + row * a.ys;
 	const int nvec = (int)(a.cols / EPV);
 	const int lo = (int)span.lo, hi = (int)span.hi;
+	// additive mask row of this query (shared by all heads, so it is served from L2); it is
+	// fetched again in each register pass instead of being held in registers
+	const Vec* __restrict__ mrow = a.mask
+		? reinterpret_cast<const Vec*>(static_cast<const T*>(a.mask) + query_of_row(a, row) * a.mask_stride) : nullptr;
+	auto mask_of = [&](int v, float (&mk)[EPV]) {
+#pragma unroll
+		for (int e = 0; e < EPV; ++e) mk[e] = 0.0f;
+		if (mrow != nullptr)
+		{
+			const Vec mv = mrow[v];
+#pragma unroll
+			for (int e = 0; e < EPV; ++e) mk[e] = (float)mv[e] * kLog2e;   // -inf and float lowest both end at -inf
+		}
+	};
 
 	Vec raw[VPL];
 #pragma unroll
@@ -117,13 +134,14 @@ __global__ __launch_bounds__(256) void softmax_rows_wave_kernel(const SoftmaxArg
 		const bool need = (v < nvec) && (e0 <= hi) && (e0 + EPV - 1 >= lo);
 		if (need)
 		{
-			float z[EPV];
+			float z[EPV], mk[EPV];
+			mask_of(v, mk);
 			float vmax = -INFINITY;
 #pragma unroll
 			for (int e = 0; e < EPV; ++e)
 			{
 				const int j = e0 + e;
-				const float zz = logit2(a, (float)raw[t][e]);
+				const float zz = logit2(a, (float)raw[t][e]) + mk[e];
 				z[e] = (j >= lo && j <= hi) ? zz : -INFINITY;
 				vmax = fmaxf(vmax, z[e]);
 			}
@@ -151,11 +169,13 @@ __global__ __launch_bounds__(256) void softmax_rows_wave_kernel(const SoftmaxArg
 			const bool need = (e0 <= hi) && (e0 + EPV - 1 >= lo);
 			if (need)
 			{
+				float mk[EPV];
+				mask_of(v, mk);
 #pragma unroll
 				for (int e = 0; e < EPV; ++e)
 				{
 					const int j = e0 + e;
-					const float p = exp2_shift(logit2(a, (float)raw[t][e]), M) * inv;
+					const float p = exp2_shift(logit2(a, (float)raw[t][e]) + mk[e], M) * inv;
 					out[e] = (T)((j >= lo && j <= hi) ? p : 0.0f);
 				}
 			}
@@ -313,11 +333,13 @@ __global__ __launch_bounds__(256) void softmax_rows_block_kernel(const SoftmaxAr
 	const RowSpan span = row_span(a, row);
 	const T* __restrict__ xr = static_cast<const T*>(a.x) + row * a.xs;
 	T* __restrict__ yr = static_cast<T*>(a.y) + row * a.ys;
+	const T* __restrict__ mrow = a.mask ? static_cast<const T*>(a.mask) + query_of_row(a, row) * a.mask_stride : nullptr;
+	auto mask_at = [&](int64_t j) { return mrow ? (float)mrow[j] * kLog2e : 0.0f; };
 
 	OnlineState st;
 	for (int64_t j = span.lo + threadIdx.x; j <= span.hi; j += blockDim.x)
 	{
-		const float z = logit2(a, (float)xr[j]);
+		const float z = logit2(a, (float)xr[j]) + mask_at(j);
 		const float mn = fmaxf(st.m, z);
 		st.s = st.s * exp2_shift(st.m, mn) + exp2_shift(z, mn);
 		st.m = mn;
@@ -341,7 +363,7 @@ __global__ __launch_bounds__(256) void softmax_rows_block_kernel(const SoftmaxAr
 	for (int64_t j = threadIdx.x; j < a.cols; j += blockDim.x)
 	{
 		float p = 0.0f;
-		if (j >= span.lo && j <= span.hi) p = exp2_shift(logit2(a, (float)xr[j]), M) * inv;
+		if (j >= span.lo && j <= span.hi) p = exp2_shift(logit2(a, (float)xr[j]) + mask_at(j), M) * inv;
 		yr[j] = (T)p;
 	}
 }
@@ -358,7 +380,7 @@ static hipError_t launch_wave(const SoftmaxArgs& a, hipStream_t stream)
 template <typename T>
 hipError_t launch_softmax_rows(const void* x, void* y, int64_t rows, int64_t cols, int64_t xs, int64_t ys,
                                int64_t q_len, int64_t diag, float alpha, float softcap, int causal,
-                               int64_t window, hipStream_t stream)
+                               int64_t window, const void* mask, int64_t mask_stride, hipStream_t stream)
 {
 	if (rows == 0 || cols == 0) return hipSuccess;
 
@@ -369,10 +391,12 @@ hipError_t launch_softmax_rows(const void* x, void* y, int64_t rows, int64_t col
 	a.cap_log2e = softcap * kLog2e;
 	a.alpha_log2e = alpha * kLog2e;
 	a.causal = causal; a.window = window;
+	a.mask = mask; a.mask_stride = mask_stride;
 
 	constexpr int EPV = 16 / (int)sizeof(T);
 	const bool vec_ok = (cols % EPV == 0) && (xs % EPV == 0) && (ys % EPV == 0) &&
-	                    (reinterpret_cast<uintptr_t>(x) % 16 == 0) && (reinterpret_cast<uintptr_t>(y) % 16 == 0);
+	                    (reinterpret_cast<uintptr_t>(x) % 16 == 0) && (reinterpret_cast<uintptr_t>(y) % 16 == 0) &&
+	                    (mask == nullptr || (mask_stride % EPV == 0 && reinterpret_cast<uintptr_t>(mask) % 16 == 0));
 	const int64_t nvec = cols / EPV;
 	if constexpr (sizeof(T) == 2)
 	{
@@ -380,7 +404,7 @@ hipError_t launch_softmax_rows(const void* x, void* y, int64_t rows, int64_t col
 		// whole row) plus one for an interval that starts inside a vector
 		const int64_t span = (causal && window > 0) ? std::min<int64_t>(cols, window) : cols;
 		const int64_t span_vecs = std::min<int64_t>(nvec, (span + EPV - 1) / EPV + 1);
-		if (vec_ok)
+		if (vec_ok && mask == nullptr)
 		{
 			if (span_vecs <= kWaveSize * 1) return launch_f16_window<1>(a, stream);
 			if (span_vecs <= kWaveSize * 2) return launch_f16_window<2>(a, stream);
@@ -407,8 +431,8 @@ hipError_t launch_softmax_rows(const void* x, void* y, int64_t rows, int64_t col
 }
 
 template hipError_t launch_softmax_rows<half_t>(const void*, void*, int64_t, int64_t, int64_t, int64_t, int64_t,
-                                                 int64_t, float, float, int, int64_t, hipStream_t);
+                                                 int64_t, float, float, int, int64_t, const void*, int64_t, hipStream_t);
 template hipError_t launch_softmax_rows<float>(const void*, void*, int64_t, int64_t, int64_t, int64_t, int64_t,
-                                                int64_t, float, float, int, int64_t, hipStream_t);
+                                                int64_t, float, float, int, int64_t, const void*, int64_t, hipStream_t);
 
 }  // namespace anygpu

@@ -5,6 +5,7 @@
 #include "harness.hpp"
 
 #include "ops.hpp"
+#include "sdp.hpp"
 #include "fast_mm.cuh"
 #include "dat_file.hpp"
 #include "test_tools.hpp"
@@ -149,4 +150,32 @@ TEST_CASE(external_test_softmax_softcap_window_f32, GPU)
 	p.alpha = 0.0625f; p.softcap = 50.f; p.causal = true; p.window = 6; p.q_len = f.q_len;
 	auto act = tensor_softmax(f.scores.copy_to_cuda(), p).copy_to_host();
 	return same_shape_and(f.expected, act, [](auto& a, auto& e) { return compare_data_buffers(a, e, 1e-5f); });
+}
+
+TEST_CASE(external_test_sdp_masked_scaled_fwd_f32_cpu, HOST)
+{
+	const auto path = golden_dir() / "test_sdp_fwd_masked_scaled_f32_16_32";
+	auto hq = load_tensor((path / "q.dat").string());
+	auto hk = load_tensor((path / "k.dat").string());
+	auto hv = load_tensor((path / "v.dat").string());
+	auto hmask = load_tensor((path / "mask.dat").string());
+	auto hy = load_tensor((path / "y.dat").string());
+	auto act = sdp_attention_masked_scaled_fwd(hq, hk, hv, hmask, 0.125f);
+	// same chain, same order as the generator of the fixture: identical to the last bit
+	return elementwise_compatible(act, hy) && std::memcmp(act.buffer(), hy.buffer(), sizeof(float32) * hy.numel()) == 0;
+}
+
+TEST_CASE(external_test_sdp_masked_scaled_fwd_f32, GPU)
+{
+	const auto path = golden_dir() / "test_sdp_fwd_masked_scaled_f32_16_32";
+	auto hq = load_tensor((path / "q.dat").string());
+	auto hk = load_tensor((path / "k.dat").string());
+	auto hv = load_tensor((path / "v.dat").string());
+	auto hmask = load_tensor((path / "mask.dat").string());
+	auto hy = load_tensor((path / "y.dat").string());
+
+	auto dy = sdp_attention_masked_scaled_fwd(hq.copy_to_cuda(), hk.copy_to_cuda(), hv.copy_to_cuda(),
+	                                          hmask.copy_to_cuda(), 0.125f);
+	auto hy_from_cuda = dy.copy_to_host();
+	return elementwise_compatible(hy_from_cuda, hy) && compare_data_buffers(hy_from_cuda, hy);
 }

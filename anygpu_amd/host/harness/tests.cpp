@@ -6,6 +6,7 @@
 #include "harness.hpp"
 
 #include "ops.hpp"
+#include "sdp.hpp"
 #include "fast_mm.cuh"
 #include "dat_file.hpp"
 #include "test_tools.hpp"
@@ -417,6 +418,45 @@ TEST_CASE(test_softmax_fused_vs_mul_add_softmax, GPU)
 				if (mask.buffer()[ix] != 0.f) ok = ok && have.buffer()[ix] == 0.f;   // masked keys: exact zeros
 		}
 	}
+	return ok;
+}
+
+TEST_CASE(test_sdp_fwd_f32, GPU)
+{
+	// tests/tests.cpp:229-250 of the reference: 14 x 64 integer-valued q, k, v, CPU against GPU
+	auto dqw = crt_random_tensor<float32, CUDA>({ 14, 64 }, 11);
+	auto dkw = crt_random_tensor<float32, CUDA>({ 14, 64 }, 18);
+	auto dvw = crt_random_tensor<float32, CUDA>({ 14, 64 }, 15);
+	auto dy = single_head_attention_fwd(dqw, dkw, dvw);
+	auto hy = single_head_attention_fwd(dqw.copy_to_host(), dkw.copy_to_host(), dvw.copy_to_host());
+	auto hy_from_cuda = dy.copy_to_host();
+	return elementwise_compatible(hy_from_cuda, hy) && compare_data_buffers(hy_from_cuda, hy);
+}
+
+TEST_CASE(test_sdp_masked_scaled_fwd_f32_and_f16, GPU)
+{
+	// [2, 6, 96, 64] queries against 160 keys, causal mask shifted by the key surplus plus a sliding window
+	const int64 b = 2, h = 6, n_q = 96, n_k = 160, d = 64;
+	auto hq = crt_random_normal_tensor<float32, CPU>({ b, h, n_q, d }, 41);
+	auto hk = crt_random_normal_tensor<float32, CPU>({ b, h, n_k, d }, 42);
+	auto hv = crt_random_normal_tensor<float32, CPU>({ b, h, n_k, d }, 43);
+	auto mask2d = build_mask(n_q, n_k, true, 80, n_k - n_q);
+	auto hmask = tensor_view(mask2d, { 1, 1, n_q, n_k });
+	auto hy = sdp_attention_masked_scaled_fwd(hq, hk, hv, hmask, 0.125f);
+
+	auto dy = sdp_attention_masked_scaled_fwd(hq.copy_to_cuda(), hk.copy_to_cuda(), hv.copy_to_cuda(), hmask.copy_to_cuda(), 0.125f);
+	auto got = dy.copy_to_host();
+	bool ok = elementwise_compatible(got, hy) && compare_data_buffers(got, hy, 1e-4f);
+
+	// half precision on the GPU against the float32 host chain on the same (half-rounded) inputs
+	auto hq16 = cvt_tensor_from_float32<float16>(hq), hk16 = cvt_tensor_from_float32<float16>(hk);
+	auto hv16 = cvt_tensor_from_float32<float16>(hv), hm16 = cvt_tensor_from_float32<float16>(hmask);
+	auto hy16_ref = sdp_attention_masked_scaled_fwd(cvt_tensor_datatype<float32, float16>(hq16), cvt_tensor_datatype<float32, float16>(hk16),
+	                                                cvt_tensor_datatype<float32, float16>(hv16), hmask, 0.125f);
+	auto dy16 = sdp_attention_masked_scaled_fwd(hq16.copy_to_cuda(), hk16.copy_to_cuda(), hv16.copy_to_cuda(), hm16.copy_to_cuda(),
+	                                            static_cast<float16>(0.125f));
+	auto got16 = cvt_tensor_datatype<float32, float16>(dy16.copy_to_host());
+	ok = ok && elementwise_compatible(got16, hy16_ref) && compare_data_buffers_l2(got16, hy16_ref, 0.01f);
 	return ok;
 }
 

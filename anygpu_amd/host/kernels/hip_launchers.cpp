@@ -139,6 +139,54 @@ void hip_tensor_softmax_fused_f16(const Tensor<float16, CUDA>& x, const SoftmaxP
 	softmax_dispatch(x, prologue, y);
 }
 
+template<typename dtype>
+void hip_tensor_mm_batched(const Tensor<dtype, CUDA>& lhs, const Tensor<dtype, CUDA>& rhs, const Tensor<dtype, CUDA>& out,
+                           const int64 batch, const int64 m, const int64 n, const int64 k, const bool rhs_is_nk)
+{
+	const int b_layout = rhs_is_nk ? ANYGPU_B_COL_MAJOR : ANYGPU_B_ROW_MAJOR;
+	const int64 lda = std::max<int64>(k, 1), ldb = std::max<int64>(rhs_is_nk ? k : n, 1), ldc = std::max<int64>(n, 1);
+	if constexpr (std::is_same_v<dtype, float32>)
+	{
+		ABI_CHECK(anygpu_gemm_f32_batched(lhs.buffer(), rhs.buffer(), out.buffer(), m, n, k, lda, ldb, ldc,
+		                                  m * k, n * k, m * n, batch, ANYGPU_A_ROW_MAJOR, b_layout, kNullStream));
+	}
+	else
+	{
+		static_assert(std::is_same_v<dtype, float16>, "Unsupported data type");
+		ABI_CHECK(anygpu_gemm_f16_f32acc_batched(lhs.buffer(), rhs.buffer(), out.buffer(), m, n, k, lda, ldb, ldc,
+		                                         m * k, n * k, m * n, batch, b_layout, kNullStream));
+	}
+}
+
+template void hip_tensor_mm_batched<float32>(const Tensor<float32, CUDA>&, const Tensor<float32, CUDA>&,
+                                             const Tensor<float32, CUDA>&, int64, int64, int64, int64, bool);
+template void hip_tensor_mm_batched<float16>(const Tensor<float16, CUDA>&, const Tensor<float16, CUDA>&,
+                                             const Tensor<float16, CUDA>&, int64, int64, int64, int64, bool);
+
+template<typename dtype>
+void hip_tensor_softmax_masked(const Tensor<dtype, CUDA>& x, const Tensor<dtype, CUDA>& mask, const float32 alpha,
+                               const int64 q_len, Tensor<dtype, CUDA>& y)
+{
+	const int64 rows = x.shape[0], cols = x.shape[1];
+	const int64 pitch = std::max<int64>(cols, 1);
+	if constexpr (std::is_same_v<dtype, float32>)
+	{
+		ABI_CHECK(anygpu_softmax_rows_masked_f32(x.buffer(), mask.buffer(), y.buffer(), rows, cols, pitch, pitch, pitch,
+		                                         q_len, alpha, 0.f, kNullStream));
+	}
+	else
+	{
+		static_assert(std::is_same_v<dtype, float16>, "Unsupported data type");
+		ABI_CHECK(anygpu_softmax_rows_masked_f16(x.buffer(), mask.buffer(), y.buffer(), rows, cols, pitch, pitch, pitch,
+		                                         q_len, alpha, 0.f, kNullStream));
+	}
+}
+
+template void hip_tensor_softmax_masked<float32>(const Tensor<float32, CUDA>&, const Tensor<float32, CUDA>&, float32,
+                                                 int64, Tensor<float32, CUDA>&);
+template void hip_tensor_softmax_masked<float16>(const Tensor<float16, CUDA>&, const Tensor<float16, CUDA>&, float32,
+                                                 int64, Tensor<float16, CUDA>&);
+
 void cu_tensor_causal_conv1d_f32(const Tensor<float32, CUDA>& xt, const Tensor<float32, CUDA>& wt,
                                  const Tensor<float32, CUDA>& bt, Tensor<float32, CUDA>& yt)
 {

@@ -53,4 +53,17 @@ void hip_tensor_mm_nt_f32(
 	const Tensor<float32, CUDA>& rhs_nk,
 	const Tensor<float32, CUDA>& out);
 
+/*
+  `batch` products of one shape in one launch over densely packed operands:
+  out[i] (m x n) = lhs[i] (m x k) * rhs[i], rhs[i] stored [k, n] or, with rhs_is_nk, [n, k].
+  The tensors may have any number of leading axes; only their buffers are used.
+*/
+template<typename dtype>
+void hip_tensor_mm_batched(
+	const Tensor<dtype, CUDA>& lhs,
+	const Tensor<dtype, CUDA>& rhs,
+	const Tensor<dtype, CUDA>& out,
+	const int64 batch, const int64 m, const int64 n, const int64 k,
+	const bool rhs_is_nk);
+
 #endif  // __MM_OPS_CUH__

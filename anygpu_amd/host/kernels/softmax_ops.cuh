@@ -40,4 +40,16 @@ void hip_tensor_softmax_fused_f16(
 	const SoftmaxPrologue& prologue,
 	Tensor<float16, CUDA>& y);
 
+/*
+  y[r, :] = softmax(alpha * x[r, :] + mask[r % q_len, :]); mask is a dense [q_len, cols] additive
+  matrix (any leading axes of extent 1), x and y dense [rows, cols].
+*/
+template<typename dtype>
+void hip_tensor_softmax_masked(
+	const Tensor<dtype, CUDA>& x,
+	const Tensor<dtype, CUDA>& mask,
+	const float32 alpha,
+	const int64 q_len,
+	Tensor<dtype, CUDA>& y);
+
 #endif  // __SOFTMAX_OPS_CUH__

@@ -134,3 +134,68 @@ def tensor_causal_conv1d(xt: torch.Tensor, wt: torch.Tensor, bt: torch.Tensor,
     rc = fn(xt.data_ptr(), wt.data_ptr(), bt.data_ptr(), out.data_ptr(), b, d, s, wt.shape[1], _stream_ptr())
     capi.check(name, rc)
     return out
+
+
+def tensor_mm_batched(lhs: torch.Tensor, rhs: torch.Tensor, b_layout: int = capi.B_ROW_MAJOR) -> torch.Tensor:
+    """out[i] = lhs[i] @ B[i] for dense 3-D operands [batch, M, K] and [batch, K, N] (or [batch, N, K] with
+    B_COL_MAJOR) in one launch: the per-head loop of the reference's attention collapsed."""
+    _check_device(lhs, rhs)
+    _require(lhs.dim() == 3 and rhs.dim() == 3 and lhs.shape[0] == rhs.shape[0], "batched operands must be 3-D")
+    _require(lhs.dtype == rhs.dtype and lhs.is_contiguous() and rhs.is_contiguous(), "dense operands of one dtype expected")
+    batch, m, k = lhs.shape
+    n = rhs.shape[2] if b_layout == capi.B_ROW_MAJOR else rhs.shape[1]
+    _require((rhs.shape[1] if b_layout == capi.B_ROW_MAJOR else rhs.shape[2]) == k,
+             "matrix multiplication requires compatible matrices")
+    out = torch.empty((batch, m, n), dtype=lhs.dtype, device=lhs.device)
+    lib = capi.load()
+    lda, ldb, ldc = max(k, 1), max(rhs.shape[2], 1), max(n, 1)
+    if lhs.dtype == torch.float16:
+        rc = lib.anygpu_gemm_f16_f32acc_batched(lhs.data_ptr(), rhs.data_ptr(), out.data_ptr(), m, n, k, lda, ldb, ldc,
+                                                m * k, n * k, m * n, batch, b_layout, _stream_ptr())
+        capi.check("anygpu_gemm_f16_f32acc_batched", rc)
+    elif lhs.dtype == torch.float32:
+        rc = lib.anygpu_gemm_f32_batched(lhs.data_ptr(), rhs.data_ptr(), out.data_ptr(), m, n, k, lda, ldb, ldc,
+                                         m * k, n * k, m * n, batch, capi.A_ROW_MAJOR, b_layout, _stream_ptr())
+        capi.check("anygpu_gemm_f32_batched", rc)
+    else:
+        raise TypeError("Unsupported data type")
+    return out
+
+
+def tensor_softmax_masked(x: torch.Tensor, mask: torch.Tensor, *, alpha: float = 1.0, softcap: float = 0.0,
+                          q_len: int = 0) -> torch.Tensor:
+    """softmax(softcap(alpha * x) + mask[r % q_len]) over the rows of a dense 2-D tensor; mask is a dense
+    additive [q_len, cols] matrix of the same dtype."""
+    _check_device(x, mask)
+    _require(x.dim() == 2 and mask.dim() == 2 and mask.shape[1] == x.shape[1], "mask shape does not fit the scores")
+    _require(x.dtype == mask.dtype and x.is_contiguous() and mask.is_contiguous(), "dense operands of one dtype expected")
+    rows, cols = x.shape
+    out = torch.empty_like(x)
+    lib = capi.load()
+    if x.dtype == torch.float16:
+        fn, name = lib.anygpu_softmax_rows_masked_f16, "anygpu_softmax_rows_masked_f16"
+    elif x.dtype == torch.float32:
+        fn, name = lib.anygpu_softmax_rows_masked_f32, "anygpu_softmax_rows_masked_f32"
+    else:
+        raise TypeError("Unsupported data type")
+    pitch = max(cols, 1)
+    rc = fn(x.data_ptr(), mask.data_ptr(), out.data_ptr(), rows, cols, pitch, pitch, pitch, q_len, alpha, softcap,
+            _stream_ptr())
+    capi.check(name, rc)
+    return out
+
+
+def sdp_attention_masked_scaled_fwd(qw: torch.Tensor, kw: torch.Tensor, vw: torch.Tensor, mask: torch.Tensor,
+                                    alpha: float) -> torch.Tensor:
+    """softmax(alpha q k^T + mask) v over [..., n, d] tensors (reference: srcs/transformers/sdp.hpp:207-274):
+    one batched GEMM for q k^T (k in its own storage), one fused softmax, one batched GEMM for p v."""
+    _require(qw.dim() == kw.dim() == vw.dim() == mask.dim() and qw.dim() >= 2, "dimension missmatch")
+    n_q, d = qw.shape[-2:]
+    n_k, d_v = kw.shape[-2], vw.shape[-1]
+    lead = qw.shape[:-2]
+    _require(all(s == 1 for s in mask.shape[:-2]), "mask needs to have 1s in the first dims except the last two")
+    q3, k3, v3 = qw.reshape(-1, n_q, d), kw.reshape(-1, n_k, d), vw.reshape(-1, n_k, d_v)
+    scores = tensor_mm_batched(q3.contiguous(), k3.contiguous(), b_layout=capi.B_COL_MAJOR)
+    probs = tensor_softmax_masked(scores.reshape(-1, n_k), mask.reshape(n_q, n_k).contiguous(), alpha=alpha, q_len=n_q)
+    out = tensor_mm_batched(probs.reshape(-1, n_q, n_k), v3.contiguous())
+    return out.reshape(*lead, n_q, d_v)

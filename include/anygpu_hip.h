@@ -62,6 +62,18 @@ int anygpu_gemm_f16_f32acc(const void* A, const void* B, void* C,
                            int b_layout, void* stream);
 
 /*
+ * `batch` products of one shape in one launch: product i reads A + i * stride_a, B + i * stride_b and
+ * writes C + i * stride_c (strides in elements, 0 shares an operand).  This is what the per-head host
+ * loop of srcs/transformers/sdp.hpp:258-271 (one tensor_mm launch per head for Q K^T and again for P V)
+ * collapses into.  batch <= 65535.
+ */
+int anygpu_gemm_f16_f32acc_batched(const void* A, const void* B, void* C,
+                                   int64_t M, int64_t N, int64_t K,
+                                   int64_t lda, int64_t ldb, int64_t ldc,
+                                   int64_t stride_a, int64_t stride_b, int64_t stride_c, int64_t batch,
+                                   int b_layout, void* stream);
+
+/*
  * C[M,N] = A[M,K] * B (+ bias[N] added to every row when bias != NULL), fp32 throughout, fp32 MFMA.
  * Replaces cu_tensor_mm_f32_opt0 and cu_tensor_gemm_f32_opt0 (srcs/kernels/cuda/mm_ops.cuh:10-25, the
  * tensor_mm / tensor_gemm <float32, CUDA> paths of srcs/ops/mm_ops.hpp:58-61,160-163) and the
@@ -73,6 +85,13 @@ int anygpu_gemm_f32(const float* A, const float* B, const float* bias, float* C,
                     int64_t M, int64_t N, int64_t K,
                     int64_t lda, int64_t ldb, int64_t ldc,
                     int a_layout, int b_layout, void* stream);
+
+/* Batched form of anygpu_gemm_f32 (no bias); see anygpu_gemm_f16_f32acc_batched. */
+int anygpu_gemm_f32_batched(const float* A, const float* B, float* C,
+                            int64_t M, int64_t N, int64_t K,
+                            int64_t lda, int64_t ldb, int64_t ldc,
+                            int64_t stride_a, int64_t stride_b, int64_t stride_c, int64_t batch,
+                            int a_layout, int b_layout, void* stream);
 
 /*
  * Row softmax over the last axis of a [rows, cols] matrix, with the steps the attention caller
@@ -102,6 +121,23 @@ int anygpu_softmax_rows_f32(const float* x, float* y,
                             int64_t q_len, int64_t diag,
                             float alpha, float softcap, int causal, int64_t window,
                             void* stream);
+
+/*
+ * The same with the mask handed over as data, the way srcs/transformers/sdp.hpp:207-274 receives it:
+ *     y[r, :] = softmax( softcap( x[r, :] * alpha ) + mask[r % q_len, :] )
+ * mask is an additive [q_len, cols] matrix of the element type (0 = visible, -inf or the lowest finite
+ * value = masked; masked outputs are exact zeros), rows mask_row_stride elements apart, shared by all
+ * heads (q_len <= 0: one mask row per matrix row).  Every element of x and of the mask is read.
+ */
+int anygpu_softmax_rows_masked_f16(const void* x, const void* mask, void* y,
+                                   int64_t rows, int64_t cols,
+                                   int64_t x_row_stride, int64_t mask_row_stride, int64_t y_row_stride,
+                                   int64_t q_len, float alpha, float softcap, void* stream);
+
+int anygpu_softmax_rows_masked_f32(const float* x, const float* mask, float* y,
+                                   int64_t rows, int64_t cols,
+                                   int64_t x_row_stride, int64_t mask_row_stride, int64_t y_row_stride,
+                                   int64_t q_len, float alpha, float softcap, void* stream);
 
 /*
  * Depthwise causal conv1d with bias and fused SiLU:

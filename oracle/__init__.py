@@ -171,6 +171,23 @@ def attention_softmax(x: np.ndarray, *, alpha: float = 1.0, softcap: float = 0.0
     return y
 
 
+def sdp_attention_masked_scaled_fwd(q: np.ndarray, k: np.ndarray, v: np.ndarray, mask: np.ndarray, alpha: float,
+                                    threads: int = 1) -> np.ndarray:
+    """q [..., n_q, d], k and v [..., n_k, d] (same leading axes), mask [..., n_q, n_k] with leading 1s."""
+    q, k, v = (np.ascontiguousarray(t, dtype=np.float32) for t in (q, k, v))
+    n_q, d = q.shape[-2:]
+    n_k = k.shape[-2]
+    assert k.shape[-1] == d and v.shape[-2:] == (n_k, d) and q.shape[:-2] == k.shape[:-2] == v.shape[:-2]
+    m2 = np.ascontiguousarray(mask, dtype=np.float32).reshape(n_q, n_k)
+    num = int(np.prod(q.shape[:-2], dtype=np.int64)) if q.ndim > 2 else 1
+    y = np.zeros(q.shape, dtype=np.float32)
+    fn = lib().oracle_sdp_attention_masked_scaled_fwd_f32
+    fn.restype = None
+    fn(_ptr(q), _ptr(k), _ptr(v), _ptr(m2), c_float(alpha), _ptr(y), c_int64(num), c_int64(n_q), c_int64(n_k),
+       c_int64(d), c_int(threads))
+    return y
+
+
 def tensor_causal_conv1d(xt: np.ndarray, wt: np.ndarray, bt: np.ndarray, rows: tuple[int, int] | None = None,
                          threads: int = 1) -> np.ndarray:
     assert xt.ndim == 3, "xt needs to be 3 dimensional"

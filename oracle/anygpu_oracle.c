@@ -18,6 +18,9 @@
  *                            two-value closed form, one-hot limit, -inf / lowest -> exact 0,
  *                            long-double brute force.
  *   oracle_tensor_mul_scalar / oracle_tensor_add   elementwise identities.
+ *   oracle_sdp_attention_masked_scaled_fwd_f32   float64 softmax(alpha q k^T + mask) v brute force (the
+ *                            library formula of the reference generator, scripts/sdp_test_cases.py:171),
+ *                            first causal row equals v[0], equality with the chain of the primitives above.
  *   oracle_softcap_f32       odd symmetry, |y| < cap, y(cap*atanh(1/2)) = cap/2, double tanh brute force.
  *   oracle_slide_mask_f32    brute-force visible set {j : i-W < j <= i}, counts min(i+1, W).
  *   oracle_causal_mask_f32   tril closed form.
@@ -281,6 +284,40 @@ ORACLE_API void oracle_attention_softmax_f32(const float* x, float* y, i64 rows,
 			softmax_row_f32(tmp, y + t * cols, cols, 1, 1);
 		}
 		free(nqk); free(mask); free(tmp);
+	}
+}
+
+/* ------------------------------------------------------------------------------------------
+ * sdp_attention_masked_scaled_fwd  --  srcs/transformers/sdp.hpp:207-274
+ *   q, k, v are [num_mtcs, n, d] (the leading axes folded), mask is [n_q, n_k] shared by all
+ *   matrices; per matrix (sdp.hpp:258-271):
+ *     kw_tr = tensor_transp(kw); qk = tensor_mm(qw, kw_tr); nqk = tensor_mul(qk, alpha);
+ *     nqk_masked = tensor_add(nqk, mask); score = tensor_softmax(nqk_masked); y = tensor_mm(score, vw)
+ *   The transpose is taken as a strided view: tensor_mm walks its operands through their strides,
+ *   so the sums are formed in the same order as over the transposed copy.
+ * ---------------------------------------------------------------------------------------- */
+ORACLE_API void oracle_sdp_attention_masked_scaled_fwd_f32(const float* q, const float* k, const float* v,
+                                                           const float* mask, float alpha, float* y,
+                                                           i64 num_mtcs, i64 n_q, i64 n_k, i64 d, int threads)
+{
+	int nt = clamp_threads(threads);
+	(void)nt;
+	#pragma omp parallel for schedule(static) num_threads(nt)
+	for (i64 ix = 0; ix < num_mtcs; ++ix)
+	{
+		const float* qm = q + ix * n_q * d;
+		const float* km = k + ix * n_k * d;
+		const float* vm = v + ix * n_k * d;
+		float* ym = y + ix * n_q * d;
+		float* qk = (float*)malloc(sizeof(float) * (size_t)(n_q * n_k));
+		float* tmp = (float*)malloc(sizeof(float) * (size_t)(n_q * n_k));
+		/* qk = q [n_q, d] x k^T: k^T as the [d, n_k] view with strides (1, d) */
+		oracle_tensor_mm_f32(qm, km, qk, n_q, n_k, d, d, 1, 1, d, n_k, 1, 0, n_q, 1);
+		oracle_tensor_mul_scalar_f32(qk, alpha, tmp, n_q * n_k);
+		oracle_tensor_add_f32(tmp, mask, qk, n_q * n_k);
+		oracle_tensor_softmax_f32(qk, tmp, n_q, n_k, n_k, 1, n_k, 1, 1);
+		oracle_tensor_mm_f32(tmp, vm, ym, n_q, d, n_k, n_k, 1, d, 1, d, 1, 0, n_q, 1);
+		free(qk); free(tmp);
 	}
 }
 

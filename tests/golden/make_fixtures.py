@@ -68,6 +68,16 @@ def main() -> None:
     save_tensor(s, d / "scores.dat"); save_tensor(mask, d / "mask.dat")
     save_tensor(oracle.attention_softmax(s, alpha=0.0625, softcap=50.0, causal=True, window=6, q_len=q), d / "y.dat")
 
+    # masked, scaled dot-product attention in the layout of the reference's golden case
+    # (tests/ext_torch_tests.cpp:84-109: [1, heads, N, d], tril -inf mask, scale 0.125), small
+    d = case_dir("test_sdp_fwd_masked_scaled_f32_16_32")
+    heads, n, dh = 4, 16, 32
+    q = synth.normal(150, (1, heads, n, dh)); k = synth.normal(151, (1, heads, n, dh)); v = synth.normal(152, (1, heads, n, dh))
+    mask = oracle.causal_mask(n, n).reshape(1, 1, n, n)
+    for name, t in (("q", q), ("k", k), ("v", v), ("mask", mask)):
+        save_tensor(t, d / f"{name}.dat")
+    save_tensor(oracle.sdp_attention_masked_scaled_fwd(q, k, v, mask, 0.125), d / "y.dat")
+
     print("fixtures written under", HERE)
 
 

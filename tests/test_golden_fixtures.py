@@ -33,6 +33,9 @@ def test_fixtures_match_the_oracle(oracle):
     d = GOLDEN / "test_mm_m64_n64_k128_f16"
     y = oracle.tensor_mm(oracle.cvt_f16_to_f32(load_tensor(d / "x.dat")), oracle.cvt_f16_to_f32(load_tensor(d / "w.dat")))
     assert np.array_equal(y.astype(np.float16), load_tensor(d / "y.dat"))
+    d = GOLDEN / "test_sdp_fwd_masked_scaled_f32_16_32"
+    q, k, v, mask = (load_tensor(d / f"{n}.dat") for n in ("q", "k", "v", "mask"))
+    assert np.array_equal(oracle.sdp_attention_masked_scaled_fwd(q, k, v, mask, 0.125), load_tensor(d / "y.dat"))
     for name, kw in [("test_softmax_masked_scaled_f32", dict(alpha=0.125, causal=True, q_len=16)),
                      ("test_softmax_softcap_window_f32", dict(alpha=0.0625, softcap=50.0, causal=True, window=6, q_len=16))]:
         d = GOLDEN / name

@@ -435,6 +435,74 @@ def test_mm_empty_and_rejected_arguments(ops):
 
 
 # =============================================================================================
+# the caller of the path: masked, scaled dot-product attention
+# =============================================================================================
+
+@pytest.mark.parametrize("dtype", ["f16", "f32"])
+@pytest.mark.parametrize("batch,m,k,n", [(1, 64, 64, 64), (5, 16, 128, 16), (32, 256, 64, 256), (3, 100, 37, 60), (8, 128, 256, 64)])
+def test_mm_batched(ops, oracle, dtype, batch, m, k, n):
+    from anygpu_amd import capi
+    np_dt = np.float16 if dtype == "f16" else np.float32
+    a = synth.uniform(batch + m, (batch, m, k)).astype(np_dt)
+    bt = synth.uniform(batch + n, (batch, n, k)).astype(np_dt)
+    a32 = oracle.cvt_f16_to_f32(a) if dtype == "f16" else a
+    b32 = oracle.cvt_f16_to_f32(bt) if dtype == "f16" else bt
+    want = np.stack([oracle.tensor_mm(a32[i], b32[i].T) for i in range(batch)])
+    tol = TOL_F16_GEMM if dtype == "f16" else TOL_F32
+    got_nt = host(ops.tensor_mm_batched(dev(a), dev(bt), b_layout=capi.B_COL_MAJOR)).astype(np.float32)
+    assert scaled_rel_err(got_nt, want, math.sqrt(k) / 3.0) <= tol
+    got_nn = host(ops.tensor_mm_batched(dev(a), dev(np.ascontiguousarray(bt.transpose(0, 2, 1))))).astype(np.float32)
+    assert scaled_rel_err(got_nn, want, math.sqrt(k) / 3.0) <= tol
+
+
+@pytest.mark.parametrize("dtype", ["f16", "f32"])
+@pytest.mark.parametrize("rows,cols,q_len,cap", [(64, 64, 64, 0.0), (96, 48, 48, 0.0), (40, 72, 40, 30.0), (33, 100, 33, 0.0),
+                                                 (256, 2048, 128, 0.0), (12, 8192, 4, 50.0)])
+def test_softmax_with_mask_tensor(ops, oracle, dtype, rows, cols, q_len, cap):
+    # the mask arrives as data (the reference's attention interface); it must agree with the index-rule form
+    np_dt = np.float16 if dtype == "f16" else np.float32
+    alpha = 0.125
+    x = synth.normal(rows + cols, (rows, cols), std=8.0).astype(np_dt)
+    diag = cols - q_len
+    mask = oracle.slide_mask(oracle.causal_mask(q_len, cols, diag=diag), max(cols // 3, 1)) if rows != 33 \
+        else oracle.causal_mask(q_len, cols, diag=diag)
+    with np.errstate(over="ignore"):
+        mask_dev = mask.astype(np_dt)       # float lowest becomes -inf in half precision: masked all the same
+    got = host(ops.tensor_softmax_masked(dev(x), dev(mask_dev), alpha=alpha, softcap=cap, q_len=q_len)).astype(np.float32)
+    x32 = oracle.cvt_f16_to_f32(x) if dtype == "f16" else x
+    s = oracle.tensor_mul_scalar(x32, alpha).reshape(rows, cols)
+    if cap:
+        s = oracle.softcap(s, cap).reshape(rows, cols)
+    m32 = np.tile(mask.astype(np.float32), (rows // q_len, 1))
+    want = oracle.tensor_softmax(oracle.tensor_add(s, m32))
+    tol = TOL_F16_ROWOPS if dtype == "f16" else TOL_F32
+    assert np.all(got[m32 != 0] == 0.0)
+    assert scaled_rel_err(got, want, want.max(axis=1, keepdims=True)) <= tol
+
+
+def test_sdp_attention_masked_scaled_fwd(ops, oracle):
+    import torch
+    # the reference's golden shape [1, 32, 16, 128] with a tril -inf mask and scale 0.125, float32
+    q, k, v = (synth.normal(s, (1, 32, 16, 128)) for s in (1, 2, 3))
+    mask = oracle.causal_mask(16, 16).reshape(1, 1, 16, 16)
+    want = oracle.sdp_attention_masked_scaled_fwd(q, k, v, mask, 0.125, threads=8)
+    got = host(ops.sdp_attention_masked_scaled_fwd(dev(q), dev(k), dev(v), dev(mask), 0.125))
+    ok, worst = oracle.compare_data_buffers(got, want)            # the reference's gate: abs 1e-3
+    assert ok, worst
+    assert scaled_rel_err(got, want, 1.0) <= TOL_F32
+    # a Gemma2-like block in half precision: 8 heads, 512 queries and keys, d = 256, causal + window 128
+    h, n, d = 8, 512, 256
+    q, k, v = (synth.normal(s, (1, h, n, d)).astype(np.float16) for s in (4, 5, 6))
+    mask = oracle.slide_mask(oracle.causal_mask(n, n), 128).reshape(1, 1, n, n)
+    want = oracle.sdp_attention_masked_scaled_fwd(*(oracle.cvt_f16_to_f32(t) for t in (q, k, v)), mask, 0.0625, threads=8)
+    with np.errstate(over="ignore"):
+        mask16 = mask.astype(np.float16)
+    got = host(ops.sdp_attention_masked_scaled_fwd(dev(q), dev(k), dev(v), dev(mask16), 0.0625)).astype(np.float32)
+    assert rel_l2(got, want) <= 1e-2
+    assert scaled_rel_err(got, want, 1.0) <= TOL_F16_GEMM
+
+
+# =============================================================================================
 # committed golden fixtures (tests/golden/*.dat)
 # =============================================================================================
 

@@ -240,6 +240,38 @@ def test_attention_softmax_is_the_stated_composition(oracle):
     assert np.array_equal(plain, oracle.tensor_softmax(oracle.tensor_mul_scalar(x, 0.125)))
 
 
+def test_sdp_attention_masked_scaled_vs_float64_formula(oracle):
+    # the reference generator's case: [1, 32, N, d] with a tril -inf mask and scale 0.125
+    # (scripts/sdp_test_cases.py:150-171, N = 16, d = 128 in tests/ext_torch_tests.cpp:86)
+    heads, n, d = 32, 16, 128
+    q = synth.normal(1, (1, heads, n, d))
+    k = synth.normal(2, (1, heads, n, d))
+    v = synth.normal(3, (1, heads, n, d))
+    mask = oracle.causal_mask(n, n).reshape(1, 1, n, n)
+    y = oracle.sdp_attention_masked_scaled_fwd(q, k, v, mask, 0.125, threads=4)
+    q64, k64, v64 = (t.astype(np.float64) for t in (q, k, v))
+    s = 0.125 * np.einsum("bhqd,bhkd->bhqk", q64, k64) + mask.astype(np.float64)
+    e = np.exp(s - s.max(axis=-1, keepdims=True))
+    want = np.einsum("bhqk,bhkd->bhqd", e / e.sum(axis=-1, keepdims=True), v64)
+    assert np.max(np.abs(y - want)) < 2e-5
+    assert np.array_equal(y[:, :, 0, :], v[:, :, 0, :])       # the first causal row attends to key 0 only
+    # the chain of primitives, one head
+    h = 5
+    qk = oracle.tensor_mm(q[0, h], k[0, h].T)
+    chain = oracle.tensor_mm(oracle.tensor_softmax(oracle.tensor_add(oracle.tensor_mul_scalar(qk, 0.125), mask[0, 0])),
+                             v[0, h])
+    assert np.array_equal(y[0, h], chain)
+    # rectangular: more keys than queries, window-style finite mask values
+    q2, k2, v2 = synth.normal(4, (3, 5, 8)), synth.normal(5, (3, 9, 8)), synth.normal(6, (3, 9, 8))
+    m2 = oracle.slide_mask(oracle.causal_mask(5, 9, diag=4), 3)
+    y2 = oracle.sdp_attention_masked_scaled_fwd(q2, k2, v2, m2, 0.3)
+    s2 = 0.3 * np.einsum("hqd,hkd->hqk", q2.astype(np.float64), k2.astype(np.float64))
+    s2 = np.where(m2[None] == 0, s2, -np.inf)
+    e2 = np.exp(s2 - s2.max(axis=-1, keepdims=True))
+    want2 = np.einsum("hqk,hkd->hqd", e2 / e2.sum(axis=-1, keepdims=True), v2.astype(np.float64))
+    assert np.max(np.abs(y2 - want2)) < 1e-5
+
+
 # ---------------------------------------------------------------------------------------------
 # tensor_causal_conv1d
 # ---------------------------------------------------------------------------------------------
