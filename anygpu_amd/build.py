@@ -84,7 +84,7 @@ def build_host_harness(verbose: bool = False) -> Path | None:
     sources += sorted(str(p) for p in (HOST_DIR / "kernels").glob("*.cpp"))
     sources += sorted(str(p) for p in (HOST_DIR / "harness").glob("*.cpp"))
     includes = [f"-I{INCLUDE_DIR}", f"-I{ROCM_DIR / 'include'}"]
-    includes += [f"-I{HOST_DIR / d}" for d in ("core", "ops", "fused", "kernels", "io", "transformers", "harness")]
+    includes += [f"-I{HOST_DIR / d}" for d in ("core", "ops", "fused", "kernels", "io", "transformers", "models/gemma2", "harness")]
     out = LIB_DIR / "anygpu_host_tests"
     # host-only C++ (no device code): the ROCm clang, which knows _Float16 on x86-64
     clangxx = ROCM_DIR / "lib" / "llvm" / "bin" / "clang++"

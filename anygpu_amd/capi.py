@@ -32,6 +32,10 @@ SIGNATURES = {
                                        c_int64, c_int64, c_int64, c_int, c_void_p]),
     "anygpu_gemm_f32": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64,
                                 c_int64, c_int64, c_int64, c_int, c_int, c_void_p]),
+    "anygpu_gemm_f32_softcap": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64,
+                                        c_int64, c_int64, c_int64, c_int, c_float, c_void_p]),
+    "anygpu_gemm_f32_gelu_mul": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64,
+                                         c_int64, c_int64, c_int64, c_int, c_void_p]),
     "anygpu_gemm_f16_f32acc_batched": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64,
                                                c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,
                                                c_int, c_void_p]),

@@ -5,6 +5,7 @@
 #include "device_utils.hpp"
 
 #include <climits>
+#include <cmath>
 
 namespace {
 
@@ -168,6 +169,28 @@ ANYGPU_EXPORT int anygpu_gemm_f32_batched(const float* A, const float* B, float*
 	if (rc != ANYGPU_OK) return rc;
 	return (int)anygpu::launch_gemm_f32(A, B, nullptr, C, M, N, K, lda, ldb, ldc, stride_a, stride_b, stride_c, batch,
 	                                    a_layout, b_layout, as_stream(stream));
+}
+
+ANYGPU_EXPORT int anygpu_gemm_f32_softcap(const float* A, const float* B, float* C,
+                                          int64_t M, int64_t N, int64_t K,
+                                          int64_t lda, int64_t ldb, int64_t ldc,
+                                          int b_layout, float softcap, void* stream)
+{
+	const int rc = check_gemm(A, B, C, M, N, K, lda, ldb, ldc, ANYGPU_A_ROW_MAJOR, b_layout);
+	if (rc != ANYGPU_OK) return rc;
+	if (!(softcap > 0.0f) || !std::isfinite(softcap)) return ANYGPU_ERR_UNSUPPORTED;
+	return (int)anygpu::launch_gemm_f32_softcap(A, B, C, M, N, K, lda, ldb, ldc, b_layout, softcap, as_stream(stream));
+}
+
+ANYGPU_EXPORT int anygpu_gemm_f32_gelu_mul(const float* A, const float* B_gate, const float* B_up, float* C,
+                                           int64_t M, int64_t N, int64_t K,
+                                           int64_t lda, int64_t ldb, int64_t ldc,
+                                           int b_layout, void* stream)
+{
+	const int rc = check_gemm(A, B_gate, C, M, N, K, lda, ldb, ldc, ANYGPU_A_ROW_MAJOR, b_layout);
+	if (rc != ANYGPU_OK) return rc;
+	if (B_up == nullptr && M > 0 && N > 0 && K > 0) return ANYGPU_ERR_NULL_POINTER;
+	return (int)anygpu::launch_gemm_f32_gelu_mul(A, B_gate, B_up, C, M, N, K, lda, ldb, ldc, b_layout, as_stream(stream));
 }
 
 ANYGPU_EXPORT int anygpu_softmax_rows_f16(const void* x, void* y, int64_t rows, int64_t cols,

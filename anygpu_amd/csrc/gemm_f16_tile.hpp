@@ -25,6 +25,8 @@
 
 #include "device_utils.hpp"
 
+#include <atomic>
+
 namespace anygpu {
 
 constexpr int kNumXcd = 8;
@@ -428,14 +430,19 @@ hipError_t launch_gemm_f16_tile(const half_t* A, const half_t* B, half_t* C, int
                                 int64_t stride_a, int64_t stride_b, int64_t stride_c, int64_t batch, hipStream_t stream)
 {
 	auto kernel = gemm_f16_nt_tile_kernel<Cfg>;
-	static bool configured = false;
+	// More than 64 KB of dynamic LDS has to be granted per function and per device, once.
+	static std::atomic<uint64_t> configured_devices{0};
 	(void)hipGetLastError();
-	if (!configured)
+	int device = 0;
+	hipError_t e = hipGetDevice(&device);
+	if (e != hipSuccess) return e;
+	const uint64_t bit = 1ull << (device & 63);
+	if ((configured_devices.load(std::memory_order_relaxed) & bit) == 0)
 	{
-		hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-		                                   hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::kLdsBytes);
+		e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+		                        hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::kLdsBytes);
 		if (e != hipSuccess) return e;
-		configured = true;
+		configured_devices.fetch_or(bit, std::memory_order_relaxed);
 	}
 	const int tiles_m = (int)(M / Cfg::BM), tiles_n = (int)(N / Cfg::BN);
 	kernel<<<dim3((unsigned)(tiles_m * tiles_n), (unsigned)batch), dim3(Cfg::kThreads), Cfg::kLdsBytes, stream>>>(

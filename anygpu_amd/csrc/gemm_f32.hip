@@ -91,12 +91,29 @@ struct Slab
 	}
 };
 
-template <int A_LAYOUT, int B_LAYOUT, bool FULL, int BM, int BN>
-__global__ __launch_bounds__(256) void gemm_f32_kernel(
-	const float* __restrict__ A, const float* __restrict__ B, const float* __restrict__ bias, float* __restrict__ C,
-	int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc,
-	int64_t stride_a, int64_t stride_b, int64_t stride_c)
+// What happens to the finished sums before they are stored.
+enum Epilogue
 {
+	kEpiBias = 0,      // + bias[n] when bias != NULL, else nothing
+	kEpiSoftcap = 1,   // cap * tanh(sum / cap)
+	kEpiGeluMul = 2    // gelu_tanh(A * B) * (A * B2): two products that share A, combined elementwise
+};
+
+// gelu(z) with the tanh approximation: z / 2 * (1 + tanh(sqrt(2 / pi) * (z + 0.044715 z^3)))
+__device__ __forceinline__ float gelu_tanh_f32(float z)
+{
+	const float inner = 0.7978845608028654f * (z + 0.044715f * z * z * z);
+	return z * 0.5f * (1.0f + tanh_f32(inner));
+}
+
+template <int A_LAYOUT, int B_LAYOUT, bool FULL, int BM, int BN, int EPI>
+__global__ __launch_bounds__(256) void gemm_f32_kernel(
+	const float* __restrict__ A, const float* __restrict__ B, const float* __restrict__ B2,
+	const float* __restrict__ bias, float* __restrict__ C,
+	int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc,
+	int64_t stride_a, int64_t stride_b, int64_t stride_c, float ep_param)
+{
+	constexpr bool DUAL = (EPI == kEpiGeluMul);
 	A += (int64_t)blockIdx.z * stride_a;
 	B += (int64_t)blockIdx.z * stride_b;
 	C += (int64_t)blockIdx.z * stride_c;
@@ -106,6 +123,7 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(
 	constexpr int TM = WTM / 32, TN = WTN / 32;     // MFMA tiles per wave
 	__shared__ __align__(16) float a_lds[2][SlabA::kLdsFloats];
 	__shared__ __align__(16) float b_lds[2][SlabB::kLdsFloats];
+	__shared__ __align__(16) float b2_lds[DUAL ? 2 : 1][DUAL ? SlabB::kLdsFloats : 4];
 
 	const int tid = threadIdx.x;
 	const int lane = tid & (kWaveSize - 1);
@@ -118,16 +136,21 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(
 	const float* b_base = (B_LAYOUT == ANYGPU_B_COL_MAJOR) ? B + n0 * ldb : B + n0;
 	auto a_at = [&](int64_t k0) { return (A_LAYOUT == ANYGPU_A_ROW_MAJOR) ? a_base + k0 : a_base + k0 * lda; };
 	auto b_at = [&](int64_t k0) { return (B_LAYOUT == ANYGPU_B_COL_MAJOR) ? b_base + k0 : b_base + k0 * ldb; };
+	const int64_t b2_shift = DUAL ? (B2 - B) : 0;   // the second right operand has the layout and pitch of the first
 
-	float4_t ra[SlabA::kVecs], rb[SlabB::kVecs];
+	float4_t ra[SlabA::kVecs], rb[SlabB::kVecs], rb2[DUAL ? SlabB::kVecs : 1];
 
-	float16_t acc[TM][TN];
+	float16_t acc[TM][TN], acc2[DUAL ? TM : 1][DUAL ? TN : 1];
 #pragma unroll
 	for (int i = 0; i < TM; ++i)
 #pragma unroll
 		for (int j = 0; j < TN; ++j)
 #pragma unroll
-			for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+			for (int r = 0; r < 16; ++r)
+			{
+				acc[i][j][r] = 0.0f;
+				if constexpr (DUAL) acc2[i][j][r] = 0.0f;
+			}
 
 	const int frag_row = lane & 31;
 	const int kb = (lane >> 5) * 8;          // this lane half's k range inside the slab
@@ -139,6 +162,11 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(
 		SlabB::load(rb, b_at(0), ldb, N - n0, K, tid);
 		SlabA::store(a_lds[0], ra, tid);
 		SlabB::store(b_lds[0], rb, tid);
+		if constexpr (DUAL)
+		{
+			SlabB::load(rb2, b_at(0) + b2_shift, ldb, N - n0, K, tid);
+			SlabB::store(b2_lds[0], rb2, tid);
+		}
 	}
 	__syncthreads();
 
@@ -150,6 +178,7 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(
 			const int64_t k1 = (kt + 1) * kBK;
 			SlabA::load(ra, a_at(k1), lda, M - m0, K - k1, tid);
 			SlabB::load(rb, b_at(k1), ldb, N - n0, K - k1, tid);
+			if constexpr (DUAL) SlabB::load(rb2, b_at(k1) + b2_shift, ldb, N - n0, K - k1, tid);
 		}
 
 		float av[TM][8], bv[TN][8];
@@ -164,11 +193,25 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(
 #pragma unroll
 				for (int j = 0; j < TN; ++j)
 					acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(bv[j][e], av[i][e], acc[i][j], 0, 0, 0);
+		if constexpr (DUAL)
+		{
+			float bv2[TN][8];
+#pragma unroll
+			for (int j = 0; j < TN; ++j) SlabB::fragment(bv2[j], b2_lds[buf], wn * WTN + j * 32 + frag_row, kb);
+#pragma unroll
+			for (int e = 0; e < 8; ++e)
+#pragma unroll
+				for (int i = 0; i < TM; ++i)
+#pragma unroll
+					for (int j = 0; j < TN; ++j)
+						acc2[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(bv2[j][e], av[i][e], acc2[i][j], 0, 0, 0);
+		}
 
 		if (kt + 1 < ktiles)
 		{
 			SlabA::store(a_lds[buf ^ 1], ra, tid);
 			SlabB::store(b_lds[buf ^ 1], rb, tid);
+			if constexpr (DUAL) SlabB::store(b2_lds[buf ^ 1], rb2, tid);
 		}
 		__syncthreads();
 	}
@@ -185,59 +228,66 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(
 			for (int g = 0; g < 4; ++g)
 			{
 				const int64_t n = n0 + wn * WTN + j * 32 + 8 * g + 4 * (lane >> 5);
+				auto finish = [&](int e) {
+					const float sum = acc[i][j][4 * g + e];
+					if constexpr (EPI == kEpiSoftcap) return ep_param * tanh_f32(sum / ep_param);
+					else if constexpr (EPI == kEpiGeluMul) return gelu_tanh_f32(sum) * acc2[i][j][4 * g + e];
+					else return sum + (bias ? bias[n + e] : 0.0f);
+				};
 				if (FULL)
 				{
 					float4_t out;
 #pragma unroll
-					for (int e = 0; e < 4; ++e) out[e] = acc[i][j][4 * g + e] + (bias ? bias[n + e] : 0.0f);
+					for (int e = 0; e < 4; ++e) out[e] = finish(e);
 					*reinterpret_cast<float4_t*>(C + m * ldc + n) = out;
 				}
 				else if (m < M)
 				{
 #pragma unroll
 					for (int e = 0; e < 4; ++e)
-						if (n + e < N) C[m * ldc + n + e] = acc[i][j][4 * g + e] + (bias ? bias[n + e] : 0.0f);
+						if (n + e < N) C[m * ldc + n + e] = finish(e);
 				}
 			}
 		}
 	}
 }
 
-template <int A_LAYOUT, int B_LAYOUT, int BM, int BN>
-static hipError_t launch_tiles(const float* A, const float* B, const float* bias, float* C,
+template <int A_LAYOUT, int B_LAYOUT, int BM, int BN, int EPI>
+static hipError_t launch_tiles(const float* A, const float* B, const float* B2, const float* bias, float* C,
                                 int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc,
                                 int64_t stride_a, int64_t stride_b, int64_t stride_c, int64_t batch,
-                                hipStream_t stream)
+                                float ep_param, hipStream_t stream)
 {
 	const dim3 grid((unsigned)((N + BN - 1) / BN), (unsigned)((M + BM - 1) / BM), (unsigned)batch);
 	const bool aligned = (reinterpret_cast<uintptr_t>(A) % 16 == 0) && (reinterpret_cast<uintptr_t>(B) % 16 == 0) &&
+	                     (reinterpret_cast<uintptr_t>(B2) % 16 == 0) &&
 	                     (reinterpret_cast<uintptr_t>(C) % 16 == 0) && (lda % 4 == 0) && (ldb % 4 == 0) && (ldc % 4 == 0) &&
 	                     (stride_a % 4 == 0) && (stride_b % 4 == 0) && (stride_c % 4 == 0);
 	const bool full = aligned && (M % BM == 0) && (N % BN == 0) && (K % kBK == 0);
 	discard_stale_error();
 	if (full)
-		gemm_f32_kernel<A_LAYOUT, B_LAYOUT, true, BM, BN><<<grid, dim3(256), 0, stream>>>(A, B, bias, C, M, N, K, lda, ldb, ldc,
-		                                                                            stride_a, stride_b, stride_c);
+		gemm_f32_kernel<A_LAYOUT, B_LAYOUT, true, BM, BN, EPI><<<grid, dim3(256), 0, stream>>>(
+			A, B, B2, bias, C, M, N, K, lda, ldb, ldc, stride_a, stride_b, stride_c, ep_param);
 	else
-		gemm_f32_kernel<A_LAYOUT, B_LAYOUT, false, BM, BN><<<grid, dim3(256), 0, stream>>>(A, B, bias, C, M, N, K, lda, ldb, ldc,
-		                                                                            stride_a, stride_b, stride_c);
+		gemm_f32_kernel<A_LAYOUT, B_LAYOUT, false, BM, BN, EPI><<<grid, dim3(256), 0, stream>>>(
+			A, B, B2, bias, C, M, N, K, lda, ldb, ldc, stride_a, stride_b, stride_c, ep_param);
 	return hipGetLastError();
 }
 
 // Tile choice: 128 x 128 tiles have the best operand reuse (2048^3: 153 us against 183 us with
 // 64 x 64 tiles); problems too small to give every CU one of them take 64 x 64 tiles to spread out.
-template <int A_LAYOUT, int B_LAYOUT>
-static hipError_t launch_layout(const float* A, const float* B, const float* bias, float* C,
+template <int A_LAYOUT, int B_LAYOUT, int EPI>
+static hipError_t launch_layout(const float* A, const float* B, const float* B2, const float* bias, float* C,
                                 int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc,
                                 int64_t stride_a, int64_t stride_b, int64_t stride_c, int64_t batch,
-                                hipStream_t stream)
+                                float ep_param, hipStream_t stream)
 {
 	const int64_t big_tiles = ((M + 127) / 128) * ((N + 127) / 128) * batch;
 	if (big_tiles >= kBigTileThreshold)
-		return launch_tiles<A_LAYOUT, B_LAYOUT, 128, 128>(A, B, bias, C, M, N, K, lda, ldb, ldc,
-		                                                  stride_a, stride_b, stride_c, batch, stream);
-	return launch_tiles<A_LAYOUT, B_LAYOUT, 64, 64>(A, B, bias, C, M, N, K, lda, ldb, ldc,
-	                                                stride_a, stride_b, stride_c, batch, stream);
+		return launch_tiles<A_LAYOUT, B_LAYOUT, 128, 128, EPI>(A, B, B2, bias, C, M, N, K, lda, ldb, ldc,
+		                                                       stride_a, stride_b, stride_c, batch, ep_param, stream);
+	return launch_tiles<A_LAYOUT, B_LAYOUT, 64, 64, EPI>(A, B, B2, bias, C, M, N, K, lda, ldb, ldc,
+	                                                     stride_a, stride_b, stride_c, batch, ep_param, stream);
 }
 
 hipError_t launch_gemm_f32(const float* A, const float* B, const float* bias, float* C,
@@ -247,19 +297,39 @@ hipError_t launch_gemm_f32(const float* A, const float* B, const float* bias, fl
                            int a_layout, int b_layout, hipStream_t stream)
 {
 	if (M == 0 || N == 0 || batch == 0) return hipSuccess;
+#define ANYGPU_F32_LAYOUT(AL, BL) \
+	return launch_layout<AL, BL, kEpiBias>(A, B, nullptr, bias, C, M, N, K, lda, ldb, ldc, stride_a, stride_b, stride_c, batch, 0.0f, stream)
 	if (a_layout == ANYGPU_A_ROW_MAJOR)
 	{
-		if (b_layout == ANYGPU_B_COL_MAJOR)
-			return launch_layout<ANYGPU_A_ROW_MAJOR, ANYGPU_B_COL_MAJOR>(A, B, bias, C, M, N, K, lda, ldb, ldc,
-		                                                             stride_a, stride_b, stride_c, batch, stream);
-		return launch_layout<ANYGPU_A_ROW_MAJOR, ANYGPU_B_ROW_MAJOR>(A, B, bias, C, M, N, K, lda, ldb, ldc,
-		                                                             stride_a, stride_b, stride_c, batch, stream);
+		if (b_layout == ANYGPU_B_COL_MAJOR) ANYGPU_F32_LAYOUT(ANYGPU_A_ROW_MAJOR, ANYGPU_B_COL_MAJOR);
+		ANYGPU_F32_LAYOUT(ANYGPU_A_ROW_MAJOR, ANYGPU_B_ROW_MAJOR);
 	}
+	if (b_layout == ANYGPU_B_COL_MAJOR) ANYGPU_F32_LAYOUT(ANYGPU_A_COL_MAJOR, ANYGPU_B_COL_MAJOR);
+	ANYGPU_F32_LAYOUT(ANYGPU_A_COL_MAJOR, ANYGPU_B_ROW_MAJOR);
+#undef ANYGPU_F32_LAYOUT
+}
+
+hipError_t launch_gemm_f32_softcap(const float* A, const float* B, float* C, int64_t M, int64_t N, int64_t K,
+                                   int64_t lda, int64_t ldb, int64_t ldc, int b_layout, float softcap, hipStream_t stream)
+{
+	if (M == 0 || N == 0) return hipSuccess;
 	if (b_layout == ANYGPU_B_COL_MAJOR)
-		return launch_layout<ANYGPU_A_COL_MAJOR, ANYGPU_B_COL_MAJOR>(A, B, bias, C, M, N, K, lda, ldb, ldc,
-		                                                             stride_a, stride_b, stride_c, batch, stream);
-	return launch_layout<ANYGPU_A_COL_MAJOR, ANYGPU_B_ROW_MAJOR>(A, B, bias, C, M, N, K, lda, ldb, ldc,
-		                                                             stride_a, stride_b, stride_c, batch, stream);
+		return launch_layout<ANYGPU_A_ROW_MAJOR, ANYGPU_B_COL_MAJOR, kEpiSoftcap>(A, B, nullptr, nullptr, C, M, N, K, lda, ldb, ldc,
+		                                                                         0, 0, 0, 1, softcap, stream);
+	return launch_layout<ANYGPU_A_ROW_MAJOR, ANYGPU_B_ROW_MAJOR, kEpiSoftcap>(A, B, nullptr, nullptr, C, M, N, K, lda, ldb, ldc,
+	                                                                         0, 0, 0, 1, softcap, stream);
+}
+
+hipError_t launch_gemm_f32_gelu_mul(const float* A, const float* B_gate, const float* B_up, float* C,
+                                    int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc,
+                                    int b_layout, hipStream_t stream)
+{
+	if (M == 0 || N == 0) return hipSuccess;
+	if (b_layout == ANYGPU_B_COL_MAJOR)
+		return launch_layout<ANYGPU_A_ROW_MAJOR, ANYGPU_B_COL_MAJOR, kEpiGeluMul>(A, B_gate, B_up, nullptr, C, M, N, K, lda, ldb, ldc,
+		                                                                         0, 0, 0, 1, 0.0f, stream);
+	return launch_layout<ANYGPU_A_ROW_MAJOR, ANYGPU_B_ROW_MAJOR, kEpiGeluMul>(A, B_gate, B_up, nullptr, C, M, N, K, lda, ldb, ldc,
+	                                                                         0, 0, 0, 1, 0.0f, stream);
 }
 
 }  // namespace anygpu

@@ -35,4 +35,13 @@ hipError_t launch_gemm_f32(const float* A, const float* B, const float* bias, fl
                            int64_t stride_a, int64_t stride_b, int64_t stride_c, int64_t batch,
                            int a_layout, int b_layout, hipStream_t stream);
 
+// C = softcap * tanh((A * B) / softcap)
+hipError_t launch_gemm_f32_softcap(const float* A, const float* B, float* C, int64_t M, int64_t N, int64_t K,
+                                   int64_t lda, int64_t ldb, int64_t ldc, int b_layout, float softcap, hipStream_t stream);
+
+// C = gelu_tanh(A * B_gate) * (A * B_up), elementwise; both right operands share layout and leading dimension
+hipError_t launch_gemm_f32_gelu_mul(const float* A, const float* B_gate, const float* B_up, float* C,
+                                    int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc,
+                                    int b_layout, hipStream_t stream);
+
 }  // namespace anygpu

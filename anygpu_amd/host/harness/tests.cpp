@@ -7,6 +7,8 @@
 
 #include "ops.hpp"
 #include "sdp.hpp"
+#include "gemma_linsoftcap.hpp"
+#include "gemma_mlp.hpp"
 #include "fast_mm.cuh"
 #include "dat_file.hpp"
 #include "test_tools.hpp"
@@ -482,6 +484,53 @@ TEST_CASE(test_causal_conv1d_f16_2x96x4096, GPU)
 	                               cvt_tensor_datatype<float32, float16>(db.copy_to_host()));
 	auto got = cvt_tensor_datatype<float32, float16>(dy.copy_to_host());
 	return elementwise_compatible(got, hy) && compare_data_buffers_l2(got, hy, 2e-3f) && compare_data_buffers(got, hy, 2e-2f);
+}
+
+TEST_CASE(test_cpu_gelu_known_values, HOST)
+{
+	Tensor<float32, CPU> x(std::vector<int64>({ 5 }), std::vector<float32>({ 0.f, 1.f, -1.f, 10.f, -10.f }));
+	auto exact = tensor_gelu(x);
+	auto approx = tensor_gelu(x, true);
+	bool ok = exact.buffer()[0] == 0.f && approx.buffer()[0] == 0.f;
+	ok = ok && std::fabs(exact.buffer()[1] - 0.8413447f) < 1e-6f && std::fabs(approx.buffer()[1] - 0.8411920f) < 1e-6f;
+	ok = ok && std::fabs(exact.buffer()[1] - exact.buffer()[2] - 1.f) < 1e-6f;      // gelu(x) - gelu(-x) = x
+	ok = ok && std::fabs(approx.buffer()[1] - approx.buffer()[2] - 1.f) < 1e-6f;
+	ok = ok && approx.buffer()[3] == 10.f && approx.buffer()[4] == 0.f;
+	return ok;
+}
+
+TEST_CASE(test_gemma2_lmhead_softcap_2x9x300_v1000, GPU)
+{
+	// logits well beyond the cap of 30 so that the tanh bends them
+	auto hx = crt_random_normal_tensor<float32, CPU>({ 2, 9, 300 }, 1);
+	auto hw = tensor_mul(crt_random_normal_tensor<float32, CPU>({ 1000, 300 }, 2), 2.f);
+	auto dy = tensor_gemma_linear_softcap(hx.copy_to_cuda(), hw.copy_to_cuda(), 30.f);
+	auto act = dy.copy_to_host();
+	auto logits = tensor_mm(tensor_view(hx, { 18, 300 }), as_transposed_view(hw));
+	Tensor<float32, CPU> exp_hy(std::vector<int64>({ 2, 9, 1000 }));
+	float32 largest = 0.f;
+	for (int64 ix = 0; ix < logits.size(); ++ix)
+	{
+		exp_hy.buffer()[ix] = std::tanh(logits.buffer()[ix] / 30.f) * 30.f;
+		largest = std::max(largest, std::fabs(logits.buffer()[ix]));
+	}
+	return largest > 60.f && elementwise_compatible(exp_hy, act) && compare_data_buffers(act, exp_hy);
+}
+
+TEST_CASE(test_gemma2_mlp_fused_upproj_1x37x288_i1152, GPU)
+{
+	GemmaMLPweights<float32, CPU> hw;
+	hw.gate_proj_weight = tensor_mul(crt_random_normal_tensor<float32, CPU>({ 288, 1152 }, 3), 0.06f);
+	hw.up_proj_weight = tensor_mul(crt_random_normal_tensor<float32, CPU>({ 288, 1152 }, 4), 0.06f);
+	auto hx = crt_random_normal_tensor<float32, CPU>({ 1, 37, 288 }, 5);
+	auto exp_hy = tensor_gemma_mlp_fused_uprpoj<float32, CPU, 0>(hw, hx);
+	GemmaMLPweights<float32, CUDA> dw;
+	dw.gate_proj_weight = hw.gate_proj_weight.copy_to_cuda();
+	dw.up_proj_weight = hw.up_proj_weight.copy_to_cuda();
+	auto dx = hx.copy_to_cuda();
+	auto act1 = tensor_gemma_mlp_fused_uprpoj<float32, CUDA, 1>(dw, dx).copy_to_host();
+	auto act2 = tensor_gemma_mlp_fused_uprpoj<float32, CUDA, 2>(dw, dx).copy_to_host();
+	return elementwise_compatible(exp_hy, act1) && compare_data_buffers(act1, exp_hy) && compare_data_buffers(act2, exp_hy);
 }
 
 TEST_CASE(test_device_tensor_plumbing, GPU)

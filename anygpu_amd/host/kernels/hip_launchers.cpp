@@ -5,6 +5,8 @@
 #include "fast_mm.cuh"
 #include "softmax_ops.cuh"
 #include "causal_conv1d.cuh"
+#include "mlp_gemma2_fused_upproj.cuh"
+#include "gemma_linsoftcap.cuh"
 
 #include "anygpu_hip.h"
 
@@ -199,4 +201,42 @@ void hip_tensor_causal_conv1d_f16(const Tensor<float16, CUDA>& xt, const Tensor<
 {
 	ABI_CHECK(anygpu_causal_conv1d_silu_f16(xt.buffer(), wt.buffer(), bt.buffer(), yt.buffer(),
 	                                        xt.shape[0], xt.shape[1], xt.shape[2], wt.shape[1], kNullStream));
+}
+
+/* ---- GEMM epilogues of the Gemma2 callers ---- */
+
+void cu_tensor_gemma_linear_softcap_f32(const Tensor<float32, CUDA>& xt, const Tensor<float32, CUDA>& wt,
+                                        const float32 final_softcapping, Tensor<float32, CUDA>& yt)
+{
+	const int64 n = xt.shape[0] * xt.shape[1];   // batch * seq_len rows
+	const int64 hsize = wt.shape[1], vsize = wt.shape[0];
+	ABI_CHECK(anygpu_gemm_f32_softcap(xt.buffer(), wt.buffer(), yt.buffer(), n, vsize, hsize,
+	                                  std::max<int64>(hsize, 1), std::max<int64>(hsize, 1), std::max<int64>(vsize, 1),
+	                                  ANYGPU_B_COL_MAJOR, final_softcapping, kNullStream));
+}
+
+namespace {
+
+void fused_upproj(const Tensor<float32, CUDA>& xt, const Tensor<float32, CUDA>& wt_gp,
+                  const Tensor<float32, CUDA>& wt_up, Tensor<float32, CUDA>& yt)
+{
+	const int64 sl = xt.shape[0] * xt.shape[1];
+	const int64 hsize = wt_gp.shape[0], isize = wt_gp.shape[1];
+	ABI_CHECK(anygpu_gemm_f32_gelu_mul(xt.buffer(), wt_gp.buffer(), wt_up.buffer(), yt.buffer(), sl, isize, hsize,
+	                                   std::max<int64>(hsize, 1), std::max<int64>(isize, 1), std::max<int64>(isize, 1),
+	                                   ANYGPU_B_ROW_MAJOR, kNullStream));
+}
+
+}  // namespace
+
+void cu_mlp_gemma2_fused_upproj_f32_v1(const Tensor<float32, CUDA>& xt, const Tensor<float32, CUDA>& wt_gp,
+                                       const Tensor<float32, CUDA>& wt_up, Tensor<float32, CUDA>& yt)
+{
+	fused_upproj(xt, wt_gp, wt_up, yt);
+}
+
+void cu_mlp_gemma2_fused_upproj_f32_v2(const Tensor<float32, CUDA>& xt, const Tensor<float32, CUDA>& wt_gp,
+                                       const Tensor<float32, CUDA>& wt_up, Tensor<float32, CUDA>& yt)
+{
+	fused_upproj(xt, wt_gp, wt_up, yt);
 }

@@ -1,0 +1,53 @@
+// Gemma2 MLP, first half: act(x Wgate) (*) (x Wup) with the tanh form of GELU.
+// Reference interface: srcs/models/gemma2/gemma_mlp.hpp:51-95 (tensor_gemma_mlp_fused_uprpoj).
+#ifndef __GEMMA_MLP__
+#define __GEMMA_MLP__
+
+#include "mlp_gemma2_fused_upproj.cuh"
+
+#include "tensor.hpp"
+#include "core_concepts.hpp"
+#include "ops.hpp"
+
+template<FloatingPointType dtype, Device device>
+struct GemmaMLPweights
+{
+	Tensor<dtype, device> gate_proj_weight;  // (hidden, intermediate)
+	Tensor<dtype, device> up_proj_weight;    // (hidden, intermediate)
+};
+
+/*
+  variant 0: three operator calls (the path a host tensor takes): linear, gelu, linear, mul.
+  variant 1, 2: the fused kernel (GPU tensors only); the two numbers are the reference's names for two
+  generations of its fused kernel and select the same kernel here.
+*/
+template<FloatingPointType dtype, Device device, int variant>
+inline Tensor<dtype, device> tensor_gemma_mlp_fused_uprpoj(
+	const GemmaMLPweights<dtype, device>& mlp_weights,
+	const Tensor<dtype, device>& x)
+{
+	if constexpr (device == CUDA)
+	{
+		static_assert(std::is_same_v<dtype, float32>, "Unsupported data types");
+		static_assert(variant == 1 || variant == 2, "a GPU tensor takes the fused kernel");
+		ACASSERT(x.dim == 3, "x should be 3 dim");
+		ACASSERT(elementwise_compatible(mlp_weights.gate_proj_weight, mlp_weights.up_proj_weight),
+		         "gate and up weights must have one shape");
+		ACASSERT(x.shape[2] == mlp_weights.gate_proj_weight.shape[0], "hidden size should match for x and the weights");
+		Tensor<dtype, device> out(std::vector<int64>{ x.shape[0], x.shape[1], mlp_weights.gate_proj_weight.shape[1] });
+		if constexpr (variant == 1)
+			cu_mlp_gemma2_fused_upproj_f32_v1(x, mlp_weights.gate_proj_weight, mlp_weights.up_proj_weight, out);
+		else
+			cu_mlp_gemma2_fused_upproj_f32_v2(x, mlp_weights.gate_proj_weight, mlp_weights.up_proj_weight, out);
+		return out;
+	}
+	else
+	{
+		auto gated_x = tensor_linear(x, mlp_weights.gate_proj_weight);
+		auto act_gated_x = tensor_gelu(gated_x, true);
+		auto up_x = tensor_linear(x, mlp_weights.up_proj_weight);
+		return tensor_mul(act_gated_x, up_x);
+	}
+}
+
+#endif  // __GEMMA_MLP__

@@ -3,6 +3,7 @@
 #define __OPS__
 
 #include "binary_ops.hpp"
+#include "math_ops.hpp"
 #include "mm_ops.hpp"
 #include "shape_ops.hpp"
 #include "softmax_ops.hpp"

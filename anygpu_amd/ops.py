@@ -86,6 +86,45 @@ def tensor_gemm(xt: torch.Tensor, wt: torch.Tensor, bt: torch.Tensor,
     return out
 
 
+def tensor_gemma_linear_softcap(xt: torch.Tensor, wt: torch.Tensor, final_softcapping: float) -> torch.Tensor:
+    """softcap(xt @ wt^T): xt [b, s, hidden], wt [vocab, hidden] -> [b, s, vocab], float32.
+
+    Same contract as tensor_gemma_linear_softcap of the reference (srcs/models/gemma2/gemma_linsoftcap.hpp:12-41).
+    """
+    _check_device(xt, wt)
+    _require(xt.dim() == 3, "xt should be 3 dim")
+    _require(wt.dim() == 2 and xt.shape[2] == wt.shape[1], "hidden size should match for xt and wt")
+    _require(xt.dtype == torch.float32 and wt.dtype == torch.float32, "Unsupported data types")
+    _require(xt.is_contiguous() and wt.is_contiguous(), "dense operands expected")
+    m, k, n = xt.shape[0] * xt.shape[1], xt.shape[2], wt.shape[0]
+    out = torch.empty((xt.shape[0], xt.shape[1], n), dtype=torch.float32, device=xt.device)
+    rc = capi.load().anygpu_gemm_f32_softcap(xt.data_ptr(), wt.data_ptr(), out.data_ptr(), m, n, k,
+                                             max(k, 1), max(k, 1), max(n, 1), capi.B_COL_MAJOR,
+                                             float(final_softcapping), _stream_ptr())
+    capi.check("anygpu_gemm_f32_softcap", rc)
+    return out
+
+
+def mlp_gemma2_fused_upproj(xt: torch.Tensor, wt_gp: torch.Tensor, wt_up: torch.Tensor) -> torch.Tensor:
+    """gelu_tanh(xt @ wt_gp) * (xt @ wt_up): xt [..., hidden], weights [hidden, intermediate], float32.
+
+    Same contract as cu_mlp_gemma2_fused_upproj_f32_v1 / _v2 (srcs/kernels/cuda/mlp_gemma2_fused_upproj.cuh:6-16).
+    """
+    _check_device(xt, wt_gp, wt_up)
+    _require(wt_gp.dim() == 2 and tuple(wt_gp.shape) == tuple(wt_up.shape), "gate and up weights must agree")
+    _require(xt.dim() >= 1 and xt.shape[-1] == wt_gp.shape[0], "hidden size should match for xt and the weights")
+    _require(all(t.dtype == torch.float32 for t in (xt, wt_gp, wt_up)), "Unsupported data types")
+    _require(xt.is_contiguous() and wt_gp.is_contiguous() and wt_up.is_contiguous(), "dense operands expected")
+    k, n = wt_gp.shape
+    m = xt.numel() // k if k else 0
+    out = torch.empty(tuple(xt.shape[:-1]) + (n,), dtype=torch.float32, device=xt.device)
+    rc = capi.load().anygpu_gemm_f32_gelu_mul(xt.data_ptr(), wt_gp.data_ptr(), wt_up.data_ptr(), out.data_ptr(),
+                                              m, n, k, max(k, 1), max(n, 1), max(n, 1), capi.B_ROW_MAJOR,
+                                              _stream_ptr())
+    capi.check("anygpu_gemm_f32_gelu_mul", rc)
+    return out
+
+
 def tensor_softmax(x: torch.Tensor, out: torch.Tensor | None = None, *, alpha: float = 1.0, softcap: float = 0.0,
                    causal: bool = False, window: int = 0, q_len: int = 0, diag: int = 0) -> torch.Tensor:
     """Row softmax of a 2-D tensor with the fused prologue (scale -> softcap -> masks)."""

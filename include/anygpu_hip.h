@@ -94,6 +94,31 @@ int anygpu_gemm_f32_batched(const float* A, const float* B, float* C,
                             int a_layout, int b_layout, void* stream);
 
 /*
+ * C[M,N] = softcap * tanh((A[M,K] * B) / softcap), fp32.  The Gemma2 output head with its final logit
+ * soft-capping in the GEMM's epilogue: replaces cu_tensor_gemma_linear_softcap_f32
+ * (srcs/models/gemma2/gemma_linsoftcap.cu:3-60; the weight there is [vocab, hidden], i.e.
+ * ANYGPU_B_COL_MAJOR with ldb = hidden, and M = batch * seq).  softcap must be > 0.  Any shape.
+ */
+int anygpu_gemm_f32_softcap(const float* A, const float* B, float* C,
+                            int64_t M, int64_t N, int64_t K,
+                            int64_t lda, int64_t ldb, int64_t ldc,
+                            int b_layout, float softcap, void* stream);
+
+/*
+ * C[M,N] = gelu_tanh(A[M,K] * B_gate) (*) (A * B_up), (*) elementwise, fp32; gelu_tanh(z) =
+ * z / 2 * (1 + tanh(sqrt(2 / pi) * (z + 0.044715 z^3))).  The Gemma2 MLP's gate and up projections with
+ * the activation and the product in the epilogue of one kernel that reads A once: replaces
+ * cu_mlp_gemma2_fused_upproj_f32_v1 / _v2 (srcs/kernels/cuda/mlp_gemma2_fused_upproj.cuh:6-16, weights
+ * there are [hidden, intermediate] = ANYGPU_B_ROW_MAJOR) and the three-launch default path
+ * tensor_gelu(tensor_linear(x, gate), true) * tensor_linear(x, up) of srcs/models/gemma2/gemma_mlp.hpp:85-90.
+ * B_gate and B_up share b_layout and ldb.  Any shape.
+ */
+int anygpu_gemm_f32_gelu_mul(const float* A, const float* B_gate, const float* B_up, float* C,
+                             int64_t M, int64_t N, int64_t K,
+                             int64_t lda, int64_t ldb, int64_t ldc,
+                             int b_layout, void* stream);
+
+/*
  * Row softmax over the last axis of a [rows, cols] matrix, with the steps the attention caller
  * runs in front of it fused in, applied in this order to each element x[r, j]:
  *     s = x * alpha                                   (tensor_mul, srcs/ops/binary_ops.hpp:61-76)

@@ -129,6 +129,55 @@ def softcap(x: np.ndarray, cap: float) -> np.ndarray:
     return y
 
 
+def gemma_linear_softcap(x: np.ndarray, w: np.ndarray, cap: float, threads: int = 1) -> np.ndarray:
+    """x [..., hsize], w [vsize, hsize] -> softcap(x w^T, cap) of shape [..., vsize]."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    w = np.ascontiguousarray(w, dtype=np.float32)
+    hsize = x.shape[-1]
+    assert w.ndim == 2 and w.shape[1] == hsize, "hidden size should match for xt and wt"
+    n = x.size // hsize if hsize else 0
+    y = np.empty(x.shape[:-1] + (w.shape[0],), dtype=np.float32)
+    fn = lib().oracle_gemma_linear_softcap_f32
+    fn.restype = None
+    fn(_ptr(x), _ptr(w), c_float(cap), _ptr(y), c_int64(n), c_int64(hsize), c_int64(w.shape[0]), c_int(threads))
+    return y
+
+
+def tensor_gelu_tanh(x: np.ndarray) -> np.ndarray:
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    y = np.empty_like(x)
+    fn = lib().oracle_tensor_gelu_tanh_f32
+    fn.restype = None
+    fn(_ptr(x), _ptr(y), c_int64(x.size))
+    return y
+
+
+def tensor_mul(lhs: np.ndarray, rhs: np.ndarray) -> np.ndarray:
+    lhs = np.ascontiguousarray(lhs, dtype=np.float32)
+    rhs = np.ascontiguousarray(rhs, dtype=np.float32)
+    assert lhs.shape == rhs.shape, "tensors are not elementwise compatible"
+    y = np.empty_like(lhs)
+    fn = lib().oracle_tensor_mul_f32
+    fn.restype = None
+    fn(_ptr(lhs), _ptr(rhs), _ptr(y), c_int64(lhs.size))
+    return y
+
+
+def gemma_mlp_upproj(x: np.ndarray, w_gate: np.ndarray, w_up: np.ndarray, threads: int = 1) -> np.ndarray:
+    """x [..., hsize], w_gate / w_up [hsize, isize] -> gelu_tanh(x w_gate) * (x w_up) of shape [..., isize]."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    w_gate = np.ascontiguousarray(w_gate, dtype=np.float32)
+    w_up = np.ascontiguousarray(w_up, dtype=np.float32)
+    hsize = x.shape[-1]
+    assert w_gate.shape == w_up.shape and w_gate.shape[0] == hsize
+    n = x.size // hsize if hsize else 0
+    y = np.empty(x.shape[:-1] + (w_gate.shape[1],), dtype=np.float32)
+    fn = lib().oracle_gemma_mlp_upproj_f32
+    fn.restype = None
+    fn(_ptr(x), _ptr(w_gate), _ptr(w_up), _ptr(y), c_int64(n), c_int64(hsize), c_int64(w_gate.shape[1]), c_int(threads))
+    return y
+
+
 def causal_mask(q_len: int, k_len: int, diag: int = 0) -> np.ndarray:
     mask = np.empty((q_len, k_len), dtype=np.float32)
     fn = lib().oracle_causal_mask_f32

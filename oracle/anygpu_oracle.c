@@ -27,6 +27,14 @@
  *   oracle_tensor_causal_conv1d_*  impulse response, pass-through tap, zero weights, causality
  *                            under perturbation, linearity of the pre-activation, explicit
  *                            zero-padded brute force in float64.
+ *   oracle_gemma_linear_softcap_f32   one-hot rows select a weight entry (y = softcap(w[v,h0])), float64
+ *                            x w^T then tanh brute force, equality with oracle_tensor_mm over the
+ *                            transposed view followed by oracle_softcap.
+ *   oracle_tensor_gelu_tanh_f32   gelu(0) = 0, gelu(x) - gelu(-x) = x, limits x and -0 at |x| = 10,
+ *                            float64 formula, closeness to the erf form x Phi(x) (the approximation's
+ *                            error stays below 1e-3).
+ *   oracle_gemma_mlp_upproj_f32   equality with the chain tensor_mm, gelu, tensor_mm, tensor_mul of the
+ *                            functions above (bit exact), float64 brute force.
  *   oracle_cvt_f16_to_f32    all 65536 bit patterns vs numpy.float16.
  *   oracle_compare_*         hand-computed three-element cases.
  * The reference repository holds no golden vectors for this path (its .dat fixtures are
@@ -390,6 +398,76 @@ ORACLE_API void oracle_tensor_causal_conv1d_f64(const double* x, const double* w
 			out += bias[dix];
 			out = out / (1.0 + exp(-out));
 			y[y_offset + six] = out;
+		}
+	}
+}
+
+/* ------------------------------------------------------------------------------------------
+ * Gemma2 output head with final logit soft-capping  --  srcs/models/gemma2/gemma_linsoftcap.cu:3-33
+ *   x [n, hsize], w [vsize, hsize] (the tied embedding table, one row per token id):
+ *   acc = 0; for h ascending: acc += x[s,h] * w[v,h]; y[s,v] = softcap(acc, cap) with
+ *   softcap(t, cap) = tanhf(t / cap) * cap (:3-9).  The reference has this op on the GPU only;
+ *   the loop is its kernel's per-element program, which is sequential in h.
+ * ---------------------------------------------------------------------------------------- */
+ORACLE_API void oracle_gemma_linear_softcap_f32(const float* x, const float* w, float cap, float* y,
+                                                i64 n, i64 hsize, i64 vsize, int threads)
+{
+	threads = clamp_threads(threads);
+#pragma omp parallel for num_threads(threads) schedule(static)
+	for (i64 s = 0; s < n; ++s)
+	{
+		for (i64 v = 0; v < vsize; ++v)
+		{
+			float acc = 0.f;
+			for (i64 h = 0; h < hsize; ++h) acc += x[s * hsize + h] * w[v * hsize + h];
+			float temp = acc / cap;
+			temp = tanhf(temp);
+			y[s * vsize + v] = temp * cap;
+		}
+	}
+}
+
+/* tensor_gelu(x, approx = true)  --  srcs/ops/math_ops.hpp:83-89
+ *   y = x * 0.5 * (1 + tanh((T)sqrt(2.0 / pi) * (x + 0.044715 * x * x * x))), every constant cast to T and
+ *   the tanh taken in T (the float overload for float32). */
+ORACLE_API void oracle_tensor_gelu_tanh_f32(const float* x, float* y, i64 length)
+{
+	const float c = (float)sqrt(2.0 / 3.14159265358979323846);
+	for (i64 k = 0; k < length; ++k)
+	{
+		float t = x[k];
+		y[k] = t * 0.5f * (1.0f + tanhf(c * (t + 0.044715f * t * t * t)));
+	}
+}
+
+/* tensor_mul(tensor, tensor)  --  srcs/ops/binary_ops.hpp:103-121 */
+ORACLE_API void oracle_tensor_mul_f32(const float* lhs, const float* rhs, float* y, i64 length)
+{
+	for (i64 ix = 0; ix < length; ++ix) y[ix] = lhs[ix] * rhs[ix];
+}
+
+/* ------------------------------------------------------------------------------------------
+ * Gemma2 MLP, gate and up projections  --  srcs/models/gemma2/gemma_mlp.hpp:85-90 (the path every
+ * device takes by default; cu_mlp_gemma2_fused_upproj_f32_v1/_v2 compute the same value in one kernel)
+ *   gated = tensor_linear(x, w_gate) = tensor_mm(x, w_gate) (srcs/ops/mm_ops.hpp:205-232);
+ *   act = tensor_gelu(gated, true); up = tensor_linear(x, w_up); y = tensor_mul(act, up)
+ *   x [n, hsize], w_gate and w_up [hsize, isize] row-major, y [n, isize].
+ * ---------------------------------------------------------------------------------------- */
+ORACLE_API void oracle_gemma_mlp_upproj_f32(const float* x, const float* w_gate, const float* w_up, float* y,
+                                            i64 n, i64 hsize, i64 isize, int threads)
+{
+	threads = clamp_threads(threads);
+#pragma omp parallel for num_threads(threads) schedule(static)
+	for (i64 r = 0; r < n; ++r)
+	{
+		for (i64 c = 0; c < isize; ++c)
+		{
+			float gate = 0.f, up = 0.f;
+			for (i64 l = 0; l < hsize; ++l) gate += x[r * hsize + l] * w_gate[l * isize + c];
+			for (i64 l = 0; l < hsize; ++l) up += x[r * hsize + l] * w_up[l * isize + c];
+			float act;
+			oracle_tensor_gelu_tanh_f32(&gate, &act, 1);
+			y[r * isize + c] = act * up;
 		}
 	}
 }

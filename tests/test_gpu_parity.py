@@ -435,6 +435,94 @@ def test_mm_empty_and_rejected_arguments(ops):
 
 
 # =============================================================================================
+# GEMM epilogues: Gemma2 output head (soft-capped logits), MLP gate / up projections
+# =============================================================================================
+
+@pytest.mark.parametrize("b,s,hsize,vsize", [(1, 1, 1, 1), (2, 9, 300, 1000), (1, 5, 64, 37), (1, 128, 256, 512),
+                                             (3, 100, 130, 259), (1, 512, 512, 2048)])
+def test_gemma_linear_softcap_shapes(ops, oracle, b, s, hsize, vsize):
+    cap = 30.0
+    x = synth.normal(b * s + hsize, (b, s, hsize))
+    w = synth.normal(vsize + hsize, (vsize, hsize)) * np.float32(4.0)      # logits reach well past the cap
+    got = host(ops.tensor_gemma_linear_softcap(dev(x), dev(w), cap))
+    want = oracle.gemma_linear_softcap(x, w, cap, threads=8)
+    assert got.shape == (b, s, vsize)
+    # |d softcap / d logit| <= 1: the GEMM's tolerance carries over, floored by the logit scale (at most the cap)
+    assert scaled_rel_err(got, want, min(cap, 4.0 * math.sqrt(hsize))) <= TOL_F32
+    assert np.all(np.abs(got) <= cap)
+
+
+def test_gemma_linear_softcap_gemma2_hidden_2304_vocab_slice(ops, oracle):
+    # srcs/models/gemma2/gemma_causallm.hpp:60-64: hidden 2304, cap 30; 32000 rows of the 256000-row table
+    b, s, hsize, vsize, cap = 1, 96, 2304, 32000, 30.0
+    x = synth.normal(1, (b, s, hsize))
+    w = synth.normal(2, (vsize, hsize)) * np.float32(0.3)
+    got = host(ops.tensor_gemma_linear_softcap(dev(x), dev(w), cap))
+    idx = sample_rows(s, 12, seed=3)
+    want = oracle.gemma_linear_softcap(x[:, idx], w, cap, threads=8)
+    assert scaled_rel_err(got[:, idx], want, 0.3 * math.sqrt(hsize)) <= TOL_F32
+    # all rows: tanh is odd and monotone, so atanh(y / cap) * cap recovers the logits; check their row sums
+    logits = np.arctanh(np.clip(got.astype(np.float64) / cap, -1 + 1e-12, 1 - 1e-12)) * cap
+    row_sum = x.astype(np.float64).reshape(s, hsize) @ w.astype(np.float64).sum(axis=0)
+    assert np.max(np.abs(logits.reshape(s, vsize).sum(axis=1) - row_sum)) < 2e-3 * vsize
+
+
+@pytest.mark.parametrize("b,s,hsize,isize", [(1, 1, 1, 1), (1, 37, 288, 1152), (2, 5, 64, 37), (1, 128, 256, 512),
+                                             (3, 50, 130, 259), (1, 256, 512, 2048)])
+def test_gemma_mlp_fused_upproj_shapes(ops, oracle, b, s, hsize, isize):
+    x = synth.normal(b * s + hsize, (b, s, hsize))
+    wg = synth.normal(isize + 1, (hsize, isize)) * np.float32(1.5 / math.sqrt(hsize))
+    wu = synth.normal(isize + 2, (hsize, isize)) * np.float32(1.5 / math.sqrt(hsize))
+    got = host(ops.mlp_gemma2_fused_upproj(dev(x), dev(wg), dev(wu)))
+    want = oracle.gemma_mlp_upproj(x, wg, wu, threads=8)
+    assert got.shape == (b, s, isize)
+    # gate and up are O(1.5) each; |gelu'| <= 1.13, so the product's error scale is that of the two sums
+    assert scaled_rel_err(got, want, 1.5 * 1.5) <= TOL_F32
+    # the two weights are not interchangeable
+    if isize > 1:
+        swapped = host(ops.mlp_gemma2_fused_upproj(dev(x), dev(wu), dev(wg)))
+        assert not np.allclose(swapped, got, atol=1e-3)
+
+
+def test_gemma_mlp_fused_upproj_gemma2_2304_9216(ops, oracle):
+    # srcs/kernels/cuda/mlp_gemma2_fused_upproj.cuh:6-16: hidden 2304, intermediate 9216
+    b, s, hsize, isize = 1, 256, 2304, 9216
+    x = synth.normal(1, (b, s, hsize))
+    wg = synth.normal(2, (hsize, isize)) * np.float32(1.0 / math.sqrt(hsize))
+    wu = synth.normal(3, (hsize, isize)) * np.float32(1.0 / math.sqrt(hsize))
+    got = host(ops.mlp_gemma2_fused_upproj(dev(x), dev(wg), dev(wu)))
+    idx = sample_rows(s, 10, seed=4)
+    want = oracle.gemma_mlp_upproj(x[:, idx], wg, wu, threads=8)
+    assert scaled_rel_err(got[:, idx], want, 1.0) <= TOL_F32
+    # against the three-kernel chain on the device: same sums, so only the activation's rounding differs
+    import torch
+    g = ops.tensor_mm(dev(x.reshape(s, hsize)), dev(wg))
+    u = ops.tensor_mm(dev(x.reshape(s, hsize)), dev(wu))
+    chain = host(torch.nn.functional.gelu(g, approximate="tanh") * u)
+    assert scaled_rel_err(got.reshape(s, isize), chain, 1.0) <= TOL_F32
+
+
+def test_gemm_epilogues_rejected_arguments(ops):
+    import torch
+    from anygpu_amd import capi
+    lib = capi.load()
+    a = torch.zeros((4, 8), device="cuda")
+    w = torch.zeros((8, 4), device="cuda")
+    c = torch.full((4, 4), 3.0, device="cuda")
+    f = lib.anygpu_gemm_f32_softcap
+    assert f(a.data_ptr(), w.data_ptr(), c.data_ptr(), 4, 4, 8, 8, 4, 4, capi.B_ROW_MAJOR, 0.0, None) == capi.ANYGPU_ERR_UNSUPPORTED
+    assert f(a.data_ptr(), w.data_ptr(), c.data_ptr(), 4, 4, 8, 8, 4, 4, capi.B_ROW_MAJOR, float("nan"), None) == capi.ANYGPU_ERR_UNSUPPORTED
+    assert f(a.data_ptr(), w.data_ptr(), c.data_ptr(), 4, 4, 8, 8, 2, 4, capi.B_ROW_MAJOR, 30.0, None) == capi.ANYGPU_ERR_BAD_STRIDE
+    g = lib.anygpu_gemm_f32_gelu_mul
+    assert g(a.data_ptr(), w.data_ptr(), None, c.data_ptr(), 4, 4, 8, 8, 4, 4, capi.B_ROW_MAJOR, None) == capi.ANYGPU_ERR_NULL_POINTER
+    assert g(a.data_ptr(), w.data_ptr(), w.data_ptr(), c.data_ptr(), 4, 0, 8, 8, 4, 4, capi.B_ROW_MAJOR, None) == capi.ANYGPU_OK
+    torch.cuda.synchronize()
+    assert bool((c == 3.0).all())
+    with pytest.raises(ValueError):
+        ops.tensor_gemma_linear_softcap(torch.zeros((1, 4, 8), device="cuda"), torch.zeros((5, 7), device="cuda"), 30.0)
+
+
+# =============================================================================================
 # the caller of the path: masked, scaled dot-product attention
 # =============================================================================================
 

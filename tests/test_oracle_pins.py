@@ -378,6 +378,76 @@ def test_conv1d_reference_generator_shape_vs_torch_formula(oracle):
 
 
 # ---------------------------------------------------------------------------------------------
+# GEMM epilogues: Gemma2 output head with logit soft-capping, MLP gate / up projections
+# ---------------------------------------------------------------------------------------------
+
+def test_linear_softcap_one_hot_rows_select_weight_entries(oracle):
+    # x = e_h0 for every row: acc is a single product 1 * w[v, h0], so y[s, v] = softcap(w[v, h0]) exactly
+    n, hsize, vsize, cap = 3, 11, 7, 30.0
+    w = synth.normal(1, (vsize, hsize)) * np.float32(40.0)
+    for h0 in (0, 5, 10):
+        x = np.zeros((1, n, hsize), dtype=np.float32)
+        x[..., h0] = 1.0
+        y = oracle.gemma_linear_softcap(x, w, cap)
+        assert y.shape == (1, n, vsize)
+        want = oracle.softcap(w[:, h0], cap)
+        assert np.array_equal(y, np.broadcast_to(want, (1, n, vsize)))
+    # a transposed weight index (w[h, v]) or a row/column swap of y would fail the shapes above (7 != 11)
+
+
+def test_linear_softcap_vs_float64_and_vs_mm_chain(oracle):
+    n, hsize, vsize, cap = 9, 130, 37, 30.0
+    x = synth.normal(2, (2, n, hsize))
+    w = synth.normal(3, (vsize, hsize)) * np.float32(3.0)
+    y = oracle.gemma_linear_softcap(x, w, cap, threads=4)
+    logits = x.astype(np.float64).reshape(-1, hsize) @ w.astype(np.float64).T
+    want = cap * np.tanh(logits / cap)
+    assert np.abs(logits).max() > cap                      # the cap bites somewhere
+    assert np.max(np.abs(y.reshape(-1, vsize) - want)) < 2e-5 * cap
+    assert np.all(np.abs(y) < cap)
+    # same sums as tensor_mm over the [hsize, vsize] strided view of w, then the scalar softcap
+    chain = oracle.softcap(oracle.tensor_mm(x.reshape(-1, hsize), w.T), cap)
+    assert np.array_equal(y.reshape(-1, vsize), chain)
+
+
+def test_gelu_tanh_closed_forms(oracle):
+    x = np.array([0.0, 1.0, -1.0, 10.0, -10.0, 0.5, -3.0], dtype=np.float32)
+    y = oracle.tensor_gelu_tanh(x)
+    assert y[0] == 0.0
+    assert y[3] == 10.0 and abs(y[4]) == 0.0                # tanh saturates to +-1 in float32
+    # gelu(x) - gelu(-x) = x / 2 * (tanh(u) - tanh(-u)) + x = x for the tanh form: tanh is odd
+    grid = np.linspace(-6, 6, 4001).astype(np.float32)
+    g = oracle.tensor_gelu_tanh(grid).astype(np.float64)
+    gm = oracle.tensor_gelu_tanh(-grid).astype(np.float64)
+    assert np.max(np.abs(g - gm - grid)) < 1e-6
+    g64 = grid.astype(np.float64)
+    want = 0.5 * g64 * (1 + np.tanh(math.sqrt(2 / math.pi) * (g64 + 0.044715 * g64 ** 3)))
+    assert np.max(np.abs(g - want)) < 1e-6
+    from scipy.special import erf
+    exact = 0.5 * g64 * (1 + erf(g64 / math.sqrt(2)))
+    assert np.max(np.abs(g - exact)) < 1e-3
+    assert abs(y[1] - 0.841192) < 1e-5                      # published value of the tanh form at 1
+
+
+def test_mlp_upproj_equals_primitive_chain_and_float64(oracle):
+    n, hsize, isize = 7, 96, 50
+    x = synth.normal(4, (1, n, hsize))
+    wg = synth.normal(5, (hsize, isize)) * np.float32(0.2)
+    wu = synth.normal(6, (hsize, isize)) * np.float32(0.2)
+    y = oracle.gemma_mlp_upproj(x, wg, wu, threads=4)
+    assert y.shape == (1, n, isize)
+    x2 = x.reshape(n, hsize)
+    chain = oracle.tensor_mul(oracle.tensor_gelu_tanh(oracle.tensor_mm(x2, wg)), oracle.tensor_mm(x2, wu))
+    assert np.array_equal(y.reshape(n, isize), chain)
+    g = x2.astype(np.float64) @ wg.astype(np.float64)
+    u = x2.astype(np.float64) @ wu.astype(np.float64)
+    want = 0.5 * g * (1 + np.tanh(math.sqrt(2 / math.pi) * (g + 0.044715 * g ** 3))) * u
+    assert np.max(np.abs(y.reshape(n, isize) - want)) < 1e-4 * max(1.0, np.abs(want).max())
+    # gate and up are not interchangeable: swapping them changes the result
+    assert not np.allclose(oracle.gemma_mlp_upproj(x, wu, wg), y, atol=1e-3)
+
+
+# ---------------------------------------------------------------------------------------------
 # fp16 up-cast and comparators
 # ---------------------------------------------------------------------------------------------
 
