@@ -15,11 +15,19 @@
 #include "launch.hpp"
 #include "anygpu_hip.h"
 
+#include <type_traits>
+
 namespace anygpu {
 
 constexpr int kBK = 16;
 constexpr int64_t kBigTileThreshold = 256;    // 128 x 128 tiles once they give every one of the 256 CUs a block
 constexpr int kPitchK = kBK + 4;     // floats per [row][k] LDS row: 80 bytes, keeps 16-byte alignment
+
+// Scheduling-group masks of __builtin_amdgcn_sched_group_barrier
+constexpr int kSchedMfma = 0x008;
+constexpr int kSchedVmemRead = 0x020;
+constexpr int kSchedDsRead = 0x100;
+constexpr int kSchedDsWrite = 0x200;
 
 // One ROWS-row x 16-deep operand slab (ROWS = 64 or 128).  KCONTIG: element (row, k) at
 // base[row * ld + k]; otherwise at base[k * ld + row].  `rows` / `depth` are the valid extents
@@ -27,6 +35,7 @@ constexpr int kPitchK = kBK + 4;     // floats per [row][k] LDS row: 80 bytes, k
 template <bool KCONTIG, bool FULL, int ROWS>
 struct Slab
 {
+	static constexpr bool kKContig = KCONTIG;
 	static constexpr int kPitchR = ROWS + 4;                 // floats per [k][row] LDS row
 	static constexpr int kLdsFloats = KCONTIG ? ROWS * kPitchK : kBK * kPitchR;
 	static constexpr int kVecs = ROWS * kBK / 4 / 256;       // float4 per thread per slab
@@ -138,7 +147,7 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(
 	auto b_at = [&](int64_t k0) { return (B_LAYOUT == ANYGPU_B_COL_MAJOR) ? b_base + k0 : b_base + k0 * ldb; };
 	const int64_t b2_shift = DUAL ? (B2 - B) : 0;   // the second right operand has the layout and pitch of the first
 
-	float4_t ra[SlabA::kVecs], rb[SlabB::kVecs], rb2[DUAL ? SlabB::kVecs : 1];
+	float4_t ra[2][SlabA::kVecs], rb[2][SlabB::kVecs], rb2[2][DUAL ? SlabB::kVecs : 1];   // two staging sets
 
 	float16_t acc[TM][TN], acc2[DUAL ? TM : 1][DUAL ? TN : 1];
 #pragma unroll
@@ -156,64 +165,119 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(
 	const int kb = (lane >> 5) * 8;          // this lane half's k range inside the slab
 	const int64_t ktiles = (K + kBK - 1) / kBK;
 
-	if (ktiles > 0)
-	{
-		SlabA::load(ra, a_at(0), lda, M - m0, K, tid);
-		SlabB::load(rb, b_at(0), ldb, N - n0, K, tid);
-		SlabA::store(a_lds[0], ra, tid);
-		SlabB::store(b_lds[0], rb, tid);
+	// Five tiles are in flight: tile t is multiplied out of one fragment register set while the
+	// fragments of tile t + 1 are read from LDS into the other set, tile t + 2 moves from a
+	// staging register set into the LDS buffer tile t has left, tile t + 3 is on its way from
+	// memory into the other staging set and the global loads of tile t + 4 are issued (two tile
+	// times cover the memory latency).  One barrier per tile separates a buffer's last read from
+	// its next write.  Tile indices past the end are clamped to the last tile: its data is
+	// fetched and staged again into a buffer nobody multiplies from, which keeps the loop body
+	// free of branches.
+	float av[2][TM][8], bv[2][TN][8], bv2[2][DUAL ? TN : 1][8];
+	const int64_t last = ktiles - 1;
+
+	auto fetch = [&](auto set, int64_t kt) {
+		constexpr int S = decltype(set)::value;
+		const int64_t k0 = (kt < last ? kt : last) * kBK;
+		SlabA::load(ra[S], a_at(k0), lda, M - m0, K - k0, tid);
+		SlabB::load(rb[S], b_at(k0), ldb, N - n0, K - k0, tid);
+		if constexpr (DUAL) SlabB::load(rb2[S], b_at(k0) + b2_shift, ldb, N - n0, K - k0, tid);
+	};
+	auto stage = [&](auto set) {               // staging set S -> LDS buffer S
+		constexpr int S = decltype(set)::value;
+		SlabA::store(a_lds[S], ra[S], tid);
+		SlabB::store(b_lds[S], rb[S], tid);
+		if constexpr (DUAL) SlabB::store(b2_lds[S], rb2[S], tid);
+	};
+	auto read_frags = [&](auto set) {          // LDS buffer S -> fragment set S
+		constexpr int S = decltype(set)::value;
+#pragma unroll
+		for (int i = 0; i < TM; ++i) SlabA::fragment(av[S][i], a_lds[S], wm * WTM + i * 32 + frag_row, kb);
+#pragma unroll
+		for (int j = 0; j < TN; ++j) SlabB::fragment(bv[S][j], b_lds[S], wn * WTN + j * 32 + frag_row, kb);
 		if constexpr (DUAL)
 		{
-			SlabB::load(rb2, b_at(0) + b2_shift, ldb, N - n0, K, tid);
-			SlabB::store(b2_lds[0], rb2, tid);
-		}
-	}
-	__syncthreads();
-
-	for (int64_t kt = 0; kt < ktiles; ++kt)
-	{
-		const int buf = (int)(kt & 1);
-		if (kt + 1 < ktiles)
-		{
-			const int64_t k1 = (kt + 1) * kBK;
-			SlabA::load(ra, a_at(k1), lda, M - m0, K - k1, tid);
-			SlabB::load(rb, b_at(k1), ldb, N - n0, K - k1, tid);
-			if constexpr (DUAL) SlabB::load(rb2, b_at(k1) + b2_shift, ldb, N - n0, K - k1, tid);
-		}
-
-		float av[TM][8], bv[TN][8];
 #pragma unroll
-		for (int i = 0; i < TM; ++i) SlabA::fragment(av[i], a_lds[buf], wm * WTM + i * 32 + frag_row, kb);
-#pragma unroll
-		for (int j = 0; j < TN; ++j) SlabB::fragment(bv[j], b_lds[buf], wn * WTN + j * 32 + frag_row, kb);
+			for (int j = 0; j < TN; ++j) SlabB::fragment(bv2[S][j], b2_lds[S], wn * WTN + j * 32 + frag_row, kb);
+		}
+	};
+	auto multiply = [&](auto set) {
+		constexpr int S = decltype(set)::value;
 #pragma unroll
 		for (int e = 0; e < 8; ++e)
 #pragma unroll
 			for (int i = 0; i < TM; ++i)
 #pragma unroll
 				for (int j = 0; j < TN; ++j)
-					acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(bv[j][e], av[i][e], acc[i][j], 0, 0, 0);
-		if constexpr (DUAL)
-		{
-			float bv2[TN][8];
-#pragma unroll
-			for (int j = 0; j < TN; ++j) SlabB::fragment(bv2[j], b2_lds[buf], wn * WTN + j * 32 + frag_row, kb);
-#pragma unroll
-			for (int e = 0; e < 8; ++e)
-#pragma unroll
-				for (int i = 0; i < TM; ++i)
-#pragma unroll
-					for (int j = 0; j < TN; ++j)
-						acc2[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(bv2[j][e], av[i][e], acc2[i][j], 0, 0, 0);
-		}
+				{
+					acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(bv[S][j][e], av[S][i][e], acc[i][j], 0, 0, 0);
+					if constexpr (DUAL)
+						acc2[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(bv2[S][j][e], av[S][i][e], acc2[i][j], 0, 0, 0);
+				}
+	};
+	using Set0 = std::integral_constant<int, 0>;
+	using Set1 = std::integral_constant<int, 1>;
 
-		if (kt + 1 < ktiles)
+	// even tiles live in set / buffer 0, odd tiles in set / buffer 1
+	auto step = [&](int64_t kt, auto set) {
+		using Other = std::integral_constant<int, decltype(set)::value ^ 1>;
+		read_frags(Other{});                       // tile kt + 1
+		multiply(set);                             // tile kt
+		stage(set);                                // tile kt + 2
+		fetch(set, kt + 4);
+		if constexpr (FULL)
 		{
-			SlabA::store(a_lds[buf ^ 1], ra, tid);
-			SlabB::store(b_lds[buf ^ 1], rb, tid);
-			if constexpr (DUAL) SlabB::store(b2_lds[buf ^ 1], rb2, tid);
+			// Issue order inside the step: the LDS reads ride on the first half of the MFMAs, the
+			// LDS writes and then the global loads (which reuse the registers just written out) on
+			// the second half, and the last MFMAs run into the barrier.
+			constexpr int kMfma = 8 * TM * TN * (DUAL ? 2 : 1);
+			constexpr int kReads = TM * (SlabA::kKContig ? 2 : 4) + (DUAL ? 2 : 1) * TN * (SlabB::kKContig ? 2 : 4);
+			constexpr int kMoves = SlabA::kVecs + (DUAL ? 2 : 1) * SlabB::kVecs;
+			constexpr int kHalf = kMfma / 2;
+			constexpr int kReadsPer = (kReads + kHalf - 1) / kHalf;
+			constexpr int kQuarter = kMfma / 4;
+			constexpr int kMovesPer = (kMoves + kQuarter - 1) / kQuarter;
+#pragma unroll
+			for (int i = 0; i < kHalf; ++i)
+			{
+				__builtin_amdgcn_sched_group_barrier(kSchedMfma, 1, 0);
+				__builtin_amdgcn_sched_group_barrier(kSchedDsRead, kReadsPer, 0);
+			}
+#pragma unroll
+			for (int i = 0; i < kQuarter; ++i)
+			{
+				__builtin_amdgcn_sched_group_barrier(kSchedMfma, 1, 0);
+				__builtin_amdgcn_sched_group_barrier(kSchedDsWrite, kMovesPer, 0);
+			}
+#pragma unroll
+			for (int i = 0; i < kQuarter; ++i)
+			{
+				__builtin_amdgcn_sched_group_barrier(kSchedMfma, 1, 0);
+				__builtin_amdgcn_sched_group_barrier(kSchedVmemRead, kMovesPer, 0);
+			}
 		}
 		__syncthreads();
+	};
+
+	if (ktiles > 0)
+	{
+		fetch(Set0{}, 0);
+		fetch(Set1{}, 1);
+		stage(Set0{});
+		fetch(Set0{}, 2);
+		stage(Set1{});
+		fetch(Set1{}, 3);
+		__syncthreads();
+		read_frags(Set0{});
+		__syncthreads();                           // buffer 0 is overwritten by the first step
+
+		int64_t kt = 0;
+		for (; kt + 1 < ktiles; kt += 2)
+		{
+			step(kt, Set0{});
+			step(kt + 1, Set1{});
+		}
+		if (kt < ktiles) multiply(Set0{});
 	}
 
 	// register r of lane l: C[m = l % 32][n = 8 * (r / 4) + 4 * (l / 32) + r % 4] of a 32 x 32 tile
