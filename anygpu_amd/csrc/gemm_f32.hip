@@ -12,6 +12,7 @@
 // The same kernel serves any shape: FULL = true assumes whole tiles and 16-byte aligned
 // rows (vector global loads), FULL = false guards every global access.
 #include "device_utils.hpp"
+#include "gemm_epilogue.hpp"
 #include "launch.hpp"
 #include "anygpu_hip.h"
 
@@ -99,21 +100,6 @@ struct Slab
 		}
 	}
 };
-
-// What happens to the finished sums before they are stored.
-enum Epilogue
-{
-	kEpiBias = 0,      // + bias[n] when bias != NULL, else nothing
-	kEpiSoftcap = 1,   // cap * tanh(sum / cap)
-	kEpiGeluMul = 2    // gelu_tanh(A * B) * (A * B2): two products that share A, combined elementwise
-};
-
-// gelu(z) with the tanh approximation: z / 2 * (1 + tanh(sqrt(2 / pi) * (z + 0.044715 z^3)))
-__device__ __forceinline__ float gelu_tanh_f32(float z)
-{
-	const float inner = 0.7978845608028654f * (z + 0.044715f * z * z * z);
-	return z * 0.5f * (1.0f + tanh_f32(inner));
-}
 
 template <int A_LAYOUT, int B_LAYOUT, bool FULL, int BM, int BN, int EPI>
 __global__ __launch_bounds__(256) void gemm_f32_kernel(
@@ -293,10 +279,9 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(
 			{
 				const int64_t n = n0 + wn * WTN + j * 32 + 8 * g + 4 * (lane >> 5);
 				auto finish = [&](int e) {
-					const float sum = acc[i][j][4 * g + e];
-					if constexpr (EPI == kEpiSoftcap) return ep_param * tanh_f32(sum / ep_param);
-					else if constexpr (EPI == kEpiGeluMul) return gelu_tanh_f32(sum) * acc2[i][j][4 * g + e];
-					else return sum + (bias ? bias[n + e] : 0.0f);
+					const float sum2 = DUAL ? acc2[DUAL ? i : 0][DUAL ? j : 0][4 * g + e] : 0.0f;
+					const float bias_n = (EPI == kEpiBias && bias) ? bias[n + e] : 0.0f;
+					return finish_sum<EPI>(acc[i][j][4 * g + e], sum2, bias_n, ep_param);
 				};
 				if (FULL)
 				{
@@ -361,6 +346,8 @@ hipError_t launch_gemm_f32(const float* A, const float* B, const float* bias, fl
                            int a_layout, int b_layout, hipStream_t stream)
 {
 	if (M == 0 || N == 0 || batch == 0) return hipSuccess;
+	if (batch == 1 && a_layout == ANYGPU_A_ROW_MAJOR && gemm_skinny_applies<float>(A, B, nullptr, M, N, K, lda, ldb, b_layout))
+		return launch_gemm_skinny<float>(A, B, nullptr, bias, C, M, N, K, lda, ldb, ldc, b_layout, kEpiBias, 0.0f, stream);
 #define ANYGPU_F32_LAYOUT(AL, BL) \
 	return launch_layout<AL, BL, kEpiBias>(A, B, nullptr, bias, C, M, N, K, lda, ldb, ldc, stride_a, stride_b, stride_c, batch, 0.0f, stream)
 	if (a_layout == ANYGPU_A_ROW_MAJOR)
@@ -377,6 +364,8 @@ hipError_t launch_gemm_f32_softcap(const float* A, const float* B, float* C, int
                                    int64_t lda, int64_t ldb, int64_t ldc, int b_layout, float softcap, hipStream_t stream)
 {
 	if (M == 0 || N == 0) return hipSuccess;
+	if (gemm_skinny_applies<float>(A, B, nullptr, M, N, K, lda, ldb, b_layout))
+		return launch_gemm_skinny<float>(A, B, nullptr, nullptr, C, M, N, K, lda, ldb, ldc, b_layout, kEpiSoftcap, softcap, stream);
 	if (b_layout == ANYGPU_B_COL_MAJOR)
 		return launch_layout<ANYGPU_A_ROW_MAJOR, ANYGPU_B_COL_MAJOR, kEpiSoftcap>(A, B, nullptr, nullptr, C, M, N, K, lda, ldb, ldc,
 		                                                                         0, 0, 0, 1, softcap, stream);
@@ -389,6 +378,8 @@ hipError_t launch_gemm_f32_gelu_mul(const float* A, const float* B_gate, const f
                                     int b_layout, hipStream_t stream)
 {
 	if (M == 0 || N == 0) return hipSuccess;
+	if (gemm_skinny_applies<float>(A, B_gate, B_up, M, N, K, lda, ldb, b_layout))
+		return launch_gemm_skinny<float>(A, B_gate, B_up, nullptr, C, M, N, K, lda, ldb, ldc, b_layout, kEpiGeluMul, 0.0f, stream);
 	if (b_layout == ANYGPU_B_COL_MAJOR)
 		return launch_layout<ANYGPU_A_ROW_MAJOR, ANYGPU_B_COL_MAJOR, kEpiGeluMul>(A, B_gate, B_up, nullptr, C, M, N, K, lda, ldb, ldc,
 		                                                                         0, 0, 0, 1, 0.0f, stream);

@@ -44,4 +44,19 @@ hipError_t launch_gemm_f32_gelu_mul(const float* A, const float* B_gate, const f
                                     int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc,
                                     int b_layout, hipStream_t stream);
 
+// Few-row products (M <= kSkinnyMaxRows, one product, row-major A): bandwidth-shaped kernels that
+// stream B once.  `epilogue` is an Epilogue value; B2 only for kEpiGeluMul, bias only for kEpiBias
+// (either may be NULL).  T is float or _Float16.  gemm_skinny_applies says whether shape, leading
+// dimensions and alignment allow them; the launchers of the tile kernels ask it first.
+constexpr int64_t kSkinnyMaxRows = 8;
+
+template <typename T>
+bool gemm_skinny_applies(const T* A, const T* B, const T* B2, int64_t M, int64_t N, int64_t K,
+                         int64_t lda, int64_t ldb, int b_layout);
+
+template <typename T>
+hipError_t launch_gemm_skinny(const T* A, const T* B, const T* B2, const float* bias, T* C,
+                              int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc,
+                              int b_layout, int epilogue, float ep_param, hipStream_t stream);
+
 }  // namespace anygpu

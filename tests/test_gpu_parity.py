@@ -412,6 +412,64 @@ def test_mm_f16_config_4096_cubed_col_major_b(ops, oracle):
     assert np.max(np.abs(g64.sum(axis=0) - col_sum)) < tol
 
 
+@pytest.mark.parametrize("dtype", ["f16", "f32"])
+@pytest.mark.parametrize("layout", ["row", "col"])
+@pytest.mark.parametrize("m,k,n", [(1, 2304, 9216), (1, 64, 8), (2, 512, 1000), (3, 2304, 2050), (4, 1000, 512),
+                                   (5, 72, 70), (8, 4096, 1024), (7, 8, 3), (1, 9216, 2304), (8, 33, 64)])
+def test_mm_few_rows(ops, oracle, dtype, layout, m, k, n):
+    # the decode-step shapes (M <= 8) take the bandwidth-shaped kernels when alignment allows, the tile kernels otherwise
+    from anygpu_amd import capi
+    np_dt = np.float16 if dtype == "f16" else np.float32
+    a = synth.uniform(m * 3 + k, (m, k)).astype(np_dt)
+    b = synth.uniform(k * 5 + n, (k, n)).astype(np_dt)
+    a32 = oracle.cvt_f16_to_f32(a) if dtype == "f16" else a
+    b32 = oracle.cvt_f16_to_f32(b) if dtype == "f16" else b
+    want = oracle.tensor_mm(a32, b32, threads=8)
+    if layout == "row":
+        got = host(ops.tensor_mm(dev(a), dev(b)))
+    else:
+        got = host(ops.tensor_mm(dev(a), dev(np.ascontiguousarray(b.T)), b_layout=capi.B_COL_MAJOR))
+    tol = TOL_F16_GEMM if dtype == "f16" else TOL_F32
+    assert got.shape == (m, n)
+    assert scaled_rel_err(got.astype(np.float32), want, math.sqrt(k) / 3.0) <= tol
+
+
+def test_mm_few_rows_integer_inputs_exact_and_padded_buffers(ops, oracle):
+    import torch
+    from anygpu_amd import capi
+    for (m, k, n) in [(1, 256, 96), (6, 128, 260)]:
+        a = synth.integers(1, (m, k), -4, 4)
+        b = synth.integers(2, (k, n), -4, 4)
+        want = oracle.tensor_mm(a, b)
+        assert np.array_equal(host(ops.tensor_mm(dev(a), dev(b))), want)
+        assert np.array_equal(host(ops.tensor_mm(dev(a), dev(np.ascontiguousarray(b.T)), b_layout=capi.B_COL_MAJOR)), want)
+        bias = synth.integers(3, (n,), -9, 9)
+        assert np.array_equal(host(ops.tensor_gemm(dev(a), dev(b), dev(bias))), oracle.tensor_gemm(a, b, bias))
+    # operands and result inside wider buffers
+    abuf, bbuf = synth.uniform(4, (4, 200)), synth.uniform(5, (96, 300))
+    cbuf = torch.full((4, 400), -1.0, device="cuda")
+    ops.tensor_mm(dev(abuf)[:, :96], dev(bbuf)[:, :256], out=cbuf[:, :256])
+    got = host(cbuf)
+    want = oracle.tensor_mm(np.ascontiguousarray(abuf[:, :96]), np.ascontiguousarray(bbuf[:, :256]))
+    assert scaled_rel_err(got[:, :256], want, math.sqrt(96) / 3.0) <= TOL_F32
+    assert np.all(got[:, 256:] == -1.0)
+
+
+@pytest.mark.parametrize("s", [1, 3, 8])
+def test_gemm_epilogues_decode_step(ops, oracle, s):
+    cap, hsize, vsize, isize = 30.0, 2304, 4000, 9216
+    x = synth.normal(s, (1, s, hsize))
+    w = synth.normal(2, (vsize, hsize)) * np.float32(0.3)
+    got = host(ops.tensor_gemma_linear_softcap(dev(x), dev(w), cap))
+    want = oracle.gemma_linear_softcap(x, w, cap, threads=8)
+    assert scaled_rel_err(got, want, 0.3 * math.sqrt(hsize)) <= TOL_F32
+    wg = synth.normal(3, (hsize, isize)) * np.float32(1.0 / math.sqrt(hsize))
+    wu = synth.normal(4, (hsize, isize)) * np.float32(1.0 / math.sqrt(hsize))
+    got = host(ops.mlp_gemma2_fused_upproj(dev(x), dev(wg), dev(wu)))
+    want = oracle.gemma_mlp_upproj(x, wg, wu, threads=8)
+    assert scaled_rel_err(got, want, 1.0) <= TOL_F32
+
+
 def test_mm_empty_and_rejected_arguments(ops):
     import torch
     from anygpu_amd import capi
