@@ -27,7 +27,7 @@ ORACLE_DIR = REPO_DIR / "oracle"
 
 ROCM_DIR = Path(os.environ.get("ROCM_PATH", "/opt/rocm"))
 GPU_ARCH = "gfx950"
-KERNEL_SOURCES = ["softmax.hip", "conv1d.hip", "gemm_f16.hip", "gemm_f32.hip", "gemm_skinny.hip", "capi.hip"]
+KERNEL_SOURCES = ["softmax.hip", "conv1d.hip", "gemm_f16.hip", "gemm_f32.hip", "gemm_skinny.hip", "rmsnorm.hip", "capi.hip"]
 
 # -packed-fp32-ops is switched off on purpose: packed fp32 VALU forms are not to be generated.
 DEVICE_FLAGS = [
@@ -84,7 +84,7 @@ def build_host_harness(verbose: bool = False) -> Path | None:
     sources += sorted(str(p) for p in (HOST_DIR / "kernels").glob("*.cpp"))
     sources += sorted(str(p) for p in (HOST_DIR / "harness").glob("*.cpp"))
     includes = [f"-I{INCLUDE_DIR}", f"-I{ROCM_DIR / 'include'}"]
-    includes += [f"-I{HOST_DIR / d}" for d in ("core", "ops", "fused", "kernels", "io", "transformers", "models/gemma2", "harness")]
+    includes += [f"-I{HOST_DIR / d}" for d in ("core", "ops", "fused", "kernels", "io", "transformers", "models/gemma2", "models/zamba2", "harness")]
     out = LIB_DIR / "anygpu_host_tests"
     # host-only C++ (no device code): the ROCm clang, which knows _Float16 on x86-64
     clangxx = ROCM_DIR / "lib" / "llvm" / "bin" / "clang++"

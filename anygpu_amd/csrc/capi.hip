@@ -90,6 +90,31 @@ int check_batch(int64_t batch, int64_t stride_a, int64_t stride_b, int64_t strid
 }
 
 template <typename T>
+int conv_update_entry(const void* x, void* state, const void* w, const void* b, void* y,
+                      int64_t batch, int64_t chan, int64_t width, void* stream)
+{
+	if (batch < 0 || chan < 0) return ANYGPU_ERR_BAD_SHAPE;
+	if (width < 1 || width > 4) return ANYGPU_ERR_UNSUPPORTED;
+	if (batch == 0 || chan == 0) return ANYGPU_OK;
+	if (x == nullptr || w == nullptr || b == nullptr || y == nullptr) return ANYGPU_ERR_NULL_POINTER;
+	if (state == nullptr && width > 1) return ANYGPU_ERR_NULL_POINTER;
+	if (chan > kMaxIndex32 || batch > (kMaxIndex32 * 256) / chan) return ANYGPU_ERR_TOO_LARGE;   // grid of rows / 256 blocks
+	return (int)anygpu::launch_causal_conv1d_silu_update<T>(x, state, w, b, y, batch, chan, (int)width, as_stream(stream));
+}
+
+template <typename T>
+int gated_rmsnorm_entry(const void* x, const void* z, const void* w, void* y, int64_t rows, int64_t cols,
+                        float eps, int zero_centered, void* stream)
+{
+	if (rows < 0 || cols < 0) return ANYGPU_ERR_BAD_SHAPE;
+	if (rows == 0 || cols == 0) return ANYGPU_OK;
+	if (x == nullptr || w == nullptr || y == nullptr) return ANYGPU_ERR_NULL_POINTER;
+	if (!(eps >= 0.0f)) return ANYGPU_ERR_UNSUPPORTED;
+	if (rows > kMaxIndex32 || cols > kMaxIndex32) return ANYGPU_ERR_TOO_LARGE;                 // one block per row
+	return (int)anygpu::launch_gated_rmsnorm<T>(x, z, w, y, rows, cols, eps, zero_centered, as_stream(stream));
+}
+
+template <typename T>
 int conv_entry(const void* x, const void* w, const void* b, void* y,
                int64_t batch, int64_t chan, int64_t seqlen, int64_t width, void* stream)
 {
@@ -239,6 +264,31 @@ ANYGPU_EXPORT int anygpu_causal_conv1d_silu_f32(const float* x, const float* w, 
                                                 void* stream)
 {
 	return conv_entry<float>(x, w, bias, y, batch, chan, seqlen, width, stream);
+}
+
+
+ANYGPU_EXPORT int anygpu_causal_conv1d_silu_update_f16(const void* x, void* state, const void* w, const void* bias, void* y,
+                                                       int64_t batch, int64_t chan, int64_t width, void* stream)
+{
+	return conv_update_entry<anygpu::half_t>(x, state, w, bias, y, batch, chan, width, stream);
+}
+
+ANYGPU_EXPORT int anygpu_causal_conv1d_silu_update_f32(const float* x, float* state, const float* w, const float* bias, float* y,
+                                                       int64_t batch, int64_t chan, int64_t width, void* stream)
+{
+	return conv_update_entry<float>(x, state, w, bias, y, batch, chan, width, stream);
+}
+
+ANYGPU_EXPORT int anygpu_gated_rmsnorm_f16(const void* x, const void* z, const void* w, void* y,
+                                           int64_t rows, int64_t cols, float eps, int zero_centered, void* stream)
+{
+	return gated_rmsnorm_entry<anygpu::half_t>(x, z, w, y, rows, cols, eps, zero_centered, stream);
+}
+
+ANYGPU_EXPORT int anygpu_gated_rmsnorm_f32(const float* x, const float* z, const float* w, float* y,
+                                           int64_t rows, int64_t cols, float eps, int zero_centered, void* stream)
+{
+	return gated_rmsnorm_entry<float>(x, z, w, y, rows, cols, eps, zero_centered, stream);
 }
 
 }  // extern "C"

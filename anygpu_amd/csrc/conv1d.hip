@@ -196,6 +196,59 @@ hipError_t launch_causal_conv1d_silu(const void* x, const void* w, const void* b
 	}
 }
 
+// Decode step: one new sample per (batch, chan) row.  `state` keeps the width - 1 samples in
+// front of it, oldest first, [batch, chan, width - 1]; it is shifted by one and takes the new
+// sample.  One thread per row: the row's state, taps, bias and sample are a few bytes each.
+template <typename T, int WIDTH>
+__global__ __launch_bounds__(256) void causal_conv1d_silu_update_kernel(
+	const T* __restrict__ x, T* __restrict__ state, const T* __restrict__ w, const T* __restrict__ bias,
+	T* __restrict__ y, int chan, int64_t rows)
+{
+	const int64_t row = (int64_t)blockIdx.x * 256 + threadIdx.x;
+	if (row >= rows) return;
+	const int ch = (int)(row % chan);
+	T* st = state + row * (WIDTH - 1);
+	T hist[WIDTH];
+#pragma unroll
+	for (int k = 0; k < WIDTH - 1; ++k) hist[k] = st[k];
+	hist[WIDTH - 1] = x[row];
+	float acc = 0.0f;
+#pragma unroll
+	for (int k = 0; k < WIDTH; ++k) acc += (float)w[(int64_t)ch * WIDTH + k] * (float)hist[k];
+	acc += (float)bias[ch];
+	y[row] = (T)silu_f32(acc);
+#pragma unroll
+	for (int k = 0; k < WIDTH - 1; ++k) st[k] = hist[k + 1];
+}
+
+template <typename T>
+hipError_t launch_causal_conv1d_silu_update(const void* x, void* state, const void* w, const void* bias, void* y,
+                                            int64_t batch, int64_t chan, int width, hipStream_t stream)
+{
+	const int64_t rows = batch * chan;
+	if (rows == 0) return hipSuccess;
+	const dim3 grid((unsigned)((rows + 255) / 256));
+	const T* xp = static_cast<const T*>(x);
+	T* sp = static_cast<T*>(state);
+	const T* wp = static_cast<const T*>(w);
+	const T* bp = static_cast<const T*>(bias);
+	T* yp = static_cast<T*>(y);
+	discard_stale_error();
+	switch (width)
+	{
+	case 1: causal_conv1d_silu_update_kernel<T, 1><<<grid, dim3(256), 0, stream>>>(xp, sp, wp, bp, yp, (int)chan, rows); break;
+	case 2: causal_conv1d_silu_update_kernel<T, 2><<<grid, dim3(256), 0, stream>>>(xp, sp, wp, bp, yp, (int)chan, rows); break;
+	case 3: causal_conv1d_silu_update_kernel<T, 3><<<grid, dim3(256), 0, stream>>>(xp, sp, wp, bp, yp, (int)chan, rows); break;
+	default: causal_conv1d_silu_update_kernel<T, 4><<<grid, dim3(256), 0, stream>>>(xp, sp, wp, bp, yp, (int)chan, rows); break;
+	}
+	return hipGetLastError();
+}
+
+template hipError_t launch_causal_conv1d_silu_update<half_t>(const void*, void*, const void*, const void*, void*, int64_t, int64_t,
+                                                              int, hipStream_t);
+template hipError_t launch_causal_conv1d_silu_update<float>(const void*, void*, const void*, const void*, void*, int64_t, int64_t,
+                                                             int, hipStream_t);
+
 template hipError_t launch_causal_conv1d_silu<half_t>(const void*, const void*, const void*, void*, int64_t, int64_t,
                                                        int64_t, int, hipStream_t);
 template hipError_t launch_causal_conv1d_silu<float>(const void*, const void*, const void*, void*, int64_t, int64_t,

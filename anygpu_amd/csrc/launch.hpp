@@ -23,6 +23,16 @@ hipError_t launch_causal_conv1d_silu(const void* x, const void* w, const void* b
                                      int64_t batch, int64_t chan, int64_t seqlen, int width,
                                      hipStream_t stream);
 
+// one new sample per (batch, chan) row; state [batch, chan, width - 1] is shifted in place
+template <typename T>
+hipError_t launch_causal_conv1d_silu_update(const void* x, void* state, const void* w, const void* bias, void* y,
+                                            int64_t batch, int64_t chan, int width, hipStream_t stream);
+
+// y = rms_norm(x * silu(z)) * (w + zero_centered) over rows of `cols`; z == NULL: no gate
+template <typename T>
+hipError_t launch_gated_rmsnorm(const void* x, const void* z, const void* w, void* y, int64_t rows, int64_t cols,
+                                float eps, int zero_centered, hipStream_t stream);
+
 // `batch` independent products of one shape, operand b of product i at base + i * stride_b (elements)
 hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K,
                            int64_t lda, int64_t ldb, int64_t ldc,

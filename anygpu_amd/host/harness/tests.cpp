@@ -9,6 +9,7 @@
 #include "sdp.hpp"
 #include "gemma_linsoftcap.hpp"
 #include "gemma_mlp.hpp"
+#include "zamba_gated_rmsnorm.hpp"
 #include "fast_mm.cuh"
 #include "dat_file.hpp"
 #include "test_tools.hpp"
@@ -531,6 +532,82 @@ TEST_CASE(test_gemma2_mlp_fused_upproj_1x37x288_i1152, GPU)
 	auto act1 = tensor_gemma_mlp_fused_uprpoj<float32, CUDA, 1>(dw, dx).copy_to_host();
 	auto act2 = tensor_gemma_mlp_fused_uprpoj<float32, CUDA, 2>(dw, dx).copy_to_host();
 	return elementwise_compatible(exp_hy, act1) && compare_data_buffers(act1, exp_hy) && compare_data_buffers(act2, exp_hy);
+}
+
+TEST_CASE(test_cpu_causal_conv1d_update_steps, HOST)
+{
+	// seq_len decode steps from a zero state give the columns of the whole-sequence op, bit for bit
+	auto x = crt_random_normal_tensor<float32, CPU>({ 2, 3, 11 }, 1);
+	auto w = crt_random_normal_tensor<float32, CPU>({ 3, 4 }, 2);
+	auto b = crt_random_normal_tensor<float32, CPU>({ 3 }, 3);
+	auto full = tensor_causal_conv1d(x, w, b);
+	Tensor<float32, CPU> state(std::vector<int64>({ 2, 3, 3 }));
+	for (int64 ix = 0; ix < state.size(); ++ix) state.buffer()[ix] = 0.f;
+	bool ok = true;
+	for (int64 t = 0; t < 11; ++t)
+	{
+		Tensor<float32, CPU> xt(std::vector<int64>({ 2, 3 }));
+		for (int64 r = 0; r < 6; ++r) xt.buffer()[r] = x.buffer()[r * 11 + t];
+		auto y = tensor_causal_conv1d_update(xt, state, w, b);
+		for (int64 r = 0; r < 6; ++r) ok = ok && y.buffer()[r] == full.buffer()[r * 11 + t];
+	}
+	for (int64 r = 0; r < 6; ++r)
+		for (int64 k = 0; k < 3; ++k) ok = ok && state.buffer()[r * 3 + k] == x.buffer()[r * 11 + 8 + k];
+	return ok;
+}
+
+TEST_CASE(test_cpu_rms_norm_constant_rows, HOST)
+{
+	// constant rows: y = w c / sqrt(c^2 + eps)
+	Tensor<float32, CPU> x(std::vector<int64>({ 2, 8 }));
+	for (int64 ix = 0; ix < 16; ++ix) x.buffer()[ix] = ix < 8 ? 2.f : -0.5f;
+	auto w = crt_pattern_tensor<float32, CPU>({ 8 });
+	auto y = tensor_rms_norm(x, -1, w, 1e-5f);
+	auto y1 = tensor_rms_norm(x, -1, w, 1e-5f, true);
+	bool ok = true;
+	for (int64 ix = 0; ix < 16; ++ix)
+	{
+		const float32 c = ix < 8 ? 2.f : -0.5f;
+		const float32 unit = c / std::sqrt(c * c + 1e-5f);
+		ok = ok && std::fabs(y.buffer()[ix] - unit * w.buffer()[ix % 8]) < 1e-6f;
+		ok = ok && std::fabs(y1.buffer()[ix] - unit * (w.buffer()[ix % 8] + 1.f)) < 1e-6f;
+	}
+	return ok;
+}
+
+TEST_CASE(test_mamba2_layer_gated_rmsnorm_1x70x4096, GPU)
+{
+	// the reference's external case: eps 1e-5, group size 4096 = the row
+	auto hx = crt_random_normal_tensor<float32, CPU>({ 1, 70, 4096 }, 1);
+	auto hz = crt_random_normal_tensor<float32, CPU>({ 1, 70, 4096 }, 2);
+	auto hw = crt_random_uniform_tensor<float32, CPU>({ 4096 }, 3, 0.5f, 1.5f);
+	auto exp_hy = tensor_zamba_gated_rmsnorm(hx, hz, hw, 4096, 1e-5f);
+	auto act_hy = tensor_zamba_gated_rmsnorm(hx.copy_to_cuda(), hz.copy_to_cuda(), hw.copy_to_cuda(), 4096, 1e-5f).copy_to_host();
+	bool ok = elementwise_compatible(exp_hy, act_hy) && compare_data_buffers(act_hy, exp_hy);
+	auto plain = tensor_rms_norm(hx.copy_to_cuda(), -1, hw.copy_to_cuda(), 1e-5f, true).copy_to_host();
+	return ok && compare_data_buffers(plain, tensor_rms_norm(hx, -1, hw, 1e-5f, true));
+}
+
+TEST_CASE(test_causal_conv1d_update_f32_4x4224, GPU)
+{
+	auto hw = crt_random_normal_tensor<float32, CPU>({ 4224, 4 }, 2);
+	auto hb = crt_random_normal_tensor<float32, CPU>({ 4224 }, 3);
+	Tensor<float32, CPU> hstate(std::vector<int64>({ 4, 4224, 3 }));
+	for (int64 ix = 0; ix < hstate.size(); ++ix) hstate.buffer()[ix] = 0.f;
+	auto dstate = hstate.copy_to_cuda();
+	auto dw = hw.copy_to_cuda();
+	auto db = hb.copy_to_cuda();
+	bool ok = true;
+	for (int64 t = 0; t < 6; ++t)
+	{
+		auto hx = crt_random_normal_tensor<float32, CPU>({ 4, 4224 }, 10 + t);
+		auto exp_hy = tensor_causal_conv1d_update(hx, hstate, hw, hb);
+		auto act_hy = tensor_causal_conv1d_update(hx.copy_to_cuda(), dstate, dw, db).copy_to_host();
+		ok = ok && elementwise_compatible(exp_hy, act_hy) && compare_data_buffers(act_hy, exp_hy);
+		auto got_state = dstate.copy_to_host();
+		ok = ok && std::memcmp(got_state.buffer(), hstate.buffer(), hstate.size() * sizeof(float32)) == 0;
+	}
+	return ok;
 }
 
 TEST_CASE(test_device_tensor_plumbing, GPU)

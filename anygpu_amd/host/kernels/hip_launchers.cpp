@@ -5,6 +5,7 @@
 #include "fast_mm.cuh"
 #include "softmax_ops.cuh"
 #include "causal_conv1d.cuh"
+#include "norm_ops.cuh"
 #include "mlp_gemma2_fused_upproj.cuh"
 #include "gemma_linsoftcap.cuh"
 
@@ -239,4 +240,64 @@ void cu_mlp_gemma2_fused_upproj_f32_v2(const Tensor<float32, CUDA>& xt, const Te
                                        const Tensor<float32, CUDA>& wt_up, Tensor<float32, CUDA>& yt)
 {
 	fused_upproj(xt, wt_gp, wt_up, yt);
+}
+
+/* ---- Mamba2 neighbours of the convolution ---- */
+
+void hip_tensor_causal_conv1d_update_f32(const Tensor<float32, CUDA>& xt, Tensor<float32, CUDA>& state,
+                                         const Tensor<float32, CUDA>& wt, const Tensor<float32, CUDA>& bt,
+                                         Tensor<float32, CUDA>& yt)
+{
+	ABI_CHECK(anygpu_causal_conv1d_silu_update_f32(xt.buffer(), wt.shape[1] > 1 ? state.buffer() : nullptr, wt.buffer(),
+	                                               bt.buffer(), yt.buffer(), xt.shape[0], xt.shape[1], wt.shape[1], kNullStream));
+}
+
+void hip_tensor_causal_conv1d_update_f16(const Tensor<float16, CUDA>& xt, Tensor<float16, CUDA>& state,
+                                         const Tensor<float16, CUDA>& wt, const Tensor<float16, CUDA>& bt,
+                                         Tensor<float16, CUDA>& yt)
+{
+	ABI_CHECK(anygpu_causal_conv1d_silu_update_f16(xt.buffer(), wt.shape[1] > 1 ? state.buffer() : nullptr, wt.buffer(),
+	                                               bt.buffer(), yt.buffer(), xt.shape[0], xt.shape[1], wt.shape[1], kNullStream));
+}
+
+namespace {
+
+// rows of wt.numel() contiguous elements; a default-constructed zt (no axes, no buffer) means "no gate"
+template <typename T>
+void rms_norm_dispatch(const Tensor<T, CUDA>& xt, const Tensor<T, CUDA>& zt, const Tensor<T, CUDA>& wt,
+                       float32 eps, bool zero_centered, Tensor<T, CUDA>& yt)
+{
+	const int64 cols = wt.numel();
+	const int64 rows = cols > 0 ? xt.numel() / cols : 0;
+	const T* gate = zt.dim > 0 ? zt.buffer() : nullptr;
+	if constexpr (std::is_same_v<T, float32>)
+		ABI_CHECK(anygpu_gated_rmsnorm_f32(xt.buffer(), gate, wt.buffer(), yt.buffer(), rows, cols, eps, zero_centered ? 1 : 0, kNullStream));
+	else
+		ABI_CHECK(anygpu_gated_rmsnorm_f16(xt.buffer(), gate, wt.buffer(), yt.buffer(), rows, cols, eps, zero_centered ? 1 : 0, kNullStream));
+}
+
+}  // namespace
+
+void cu_tensor_rms_norm_f32(const Tensor<float32, CUDA>& xt, const Tensor<float32, CUDA> wt, const float32 eps,
+                            const bool zero_centered, Tensor<float32, CUDA>& yt)
+{
+	rms_norm_dispatch(xt, Tensor<float32, CUDA>(), wt, eps, zero_centered, yt);
+}
+
+void cu_tensor_rms_norm_f32_v1(const Tensor<float32, CUDA>& xt, const Tensor<float32, CUDA> wt, const float32 eps,
+                               const bool zero_centered, Tensor<float32, CUDA>& yt)
+{
+	rms_norm_dispatch(xt, Tensor<float32, CUDA>(), wt, eps, zero_centered, yt);
+}
+
+void hip_tensor_gated_rms_norm_f32(const Tensor<float32, CUDA>& xt, const Tensor<float32, CUDA>& zt, const Tensor<float32, CUDA>& wt,
+                                   const float32 eps, const bool zero_centered, Tensor<float32, CUDA>& yt)
+{
+	rms_norm_dispatch(xt, zt, wt, eps, zero_centered, yt);
+}
+
+void hip_tensor_gated_rms_norm_f16(const Tensor<float16, CUDA>& xt, const Tensor<float16, CUDA>& zt, const Tensor<float16, CUDA>& wt,
+                                   const float32 eps, const bool zero_centered, Tensor<float16, CUDA>& yt)
+{
+	rms_norm_dispatch(xt, zt, wt, eps, zero_centered, yt);
 }

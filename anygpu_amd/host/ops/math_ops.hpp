@@ -1,6 +1,6 @@
 // Elementwise activation on host tensors.  On the GPU the one caller on this path (the Gemma2 MLP)
 // has the activation folded into the epilogue of its projection kernel, so only the host form
-// exists here.  Reference: srcs/ops/math_ops.hpp:55-93 (tensor_gelu, exact and tanh form).
+// exists here.  Reference: srcs/ops/math_ops.hpp:16-35 (tensor_silu), :55-93 (tensor_gelu, exact and tanh form).
 #ifndef __MATH_OPS__
 #define __MATH_OPS__
 
@@ -8,6 +8,18 @@
 #include "core_concepts.hpp"
 
 #include <cmath>
+
+/* silu(x) = x / (1 + exp(-x)), evaluated in dtype. */
+template<PreciseFloatType dtype>
+inline Tensor<dtype, CPU> tensor_silu(const Tensor<dtype, CPU>& xt)
+{
+	Tensor<dtype, CPU> yt(xt.dim, xt.shape);
+	const dtype* x_data = xt.buffer();
+	dtype* y_data = yt.buffer();
+	const int64 length = xt.size();
+	for (int64 k = 0; k < length; ++k) y_data[k] = x_data[k] / (static_cast<dtype>(1.0) + std::exp(-x_data[k]));
+	return yt;
+}
 
 /*
   gelu(x) = x / 2 * (1 + erf(x / sqrt(2)));  with approx: x / 2 * (1 + tanh(sqrt(2 / pi) * (x + 0.044715 x^3))).

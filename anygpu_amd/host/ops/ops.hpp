@@ -5,6 +5,7 @@
 #include "binary_ops.hpp"
 #include "math_ops.hpp"
 #include "mm_ops.hpp"
+#include "norm_ops.hpp"
 #include "shape_ops.hpp"
 #include "softmax_ops.hpp"
 #include "causal_conv1d.hpp"

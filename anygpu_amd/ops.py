@@ -175,6 +175,61 @@ def tensor_causal_conv1d(xt: torch.Tensor, wt: torch.Tensor, bt: torch.Tensor,
     return out
 
 
+def tensor_causal_conv1d_update(xt: torch.Tensor, state: torch.Tensor, wt: torch.Tensor, bt: torch.Tensor) -> torch.Tensor:
+    """One decode step of tensor_causal_conv1d: xt [batch, dims] is the new sample of every row, state
+    [batch, dims, width - 1] holds the samples in front of it (oldest first) and is updated in place."""
+    _check_device(xt, state, wt, bt)
+    _require(xt.dim() == 2 and state.dim() == 3, "xt needs to be 2 and state 3 dimensional")
+    _require(xt.shape[1] == wt.shape[0], "xt and wt need to have the same dims")
+    _require(wt.shape[0] == bt.shape[0], "wt and bt need to have the same dims")
+    _require(wt.shape[1] <= 4, "kernel width needs to be under 4")
+    _require(tuple(state.shape) == (xt.shape[0], xt.shape[1], wt.shape[1] - 1), "state needs to be (batch, dims, width - 1)")
+    _require(xt.dtype == wt.dtype == bt.dtype == state.dtype, "operands must share a dtype")
+    _require(all(t.is_contiguous() for t in (xt, state, wt, bt)), "dense operands expected")
+    out = torch.empty_like(xt)
+    lib = capi.load()
+    if xt.dtype == torch.float16:
+        fn, name = lib.anygpu_causal_conv1d_silu_update_f16, "anygpu_causal_conv1d_silu_update_f16"
+    elif xt.dtype == torch.float32:
+        fn, name = lib.anygpu_causal_conv1d_silu_update_f32, "anygpu_causal_conv1d_silu_update_f32"
+    else:
+        raise TypeError("Unsupported data types")
+    rc = fn(xt.data_ptr(), state.data_ptr() if state.numel() else None, wt.data_ptr(), bt.data_ptr(), out.data_ptr(),
+            xt.shape[0], xt.shape[1], wt.shape[1], _stream_ptr())
+    capi.check(name, rc)
+    return out
+
+
+def tensor_rms_norm(xt: torch.Tensor, wt: torch.Tensor, eps: float, zero_centered: bool = False,
+                    gate: torch.Tensor | None = None) -> torch.Tensor:
+    """rms_norm(xt * silu(gate)) * (wt + zero_centered) over the last axis; gate None: plain RMS norm."""
+    _check_device(xt, wt) if gate is None else _check_device(xt, wt, gate)
+    _require(wt.dim() == 1 and xt.dim() >= 1 and xt.shape[-1] == wt.shape[0], "wt shape is incorrect")
+    _require(gate is None or tuple(gate.shape) == tuple(xt.shape), "tensors are not elementwise compatible")
+    _require(xt.dtype == wt.dtype and (gate is None or gate.dtype == xt.dtype), "operands must share a dtype")
+    _require(xt.is_contiguous() and wt.is_contiguous() and (gate is None or gate.is_contiguous()), "dense operands expected")
+    cols = wt.shape[0]
+    rows = xt.numel() // cols if cols else 0
+    out = torch.empty_like(xt)
+    lib = capi.load()
+    if xt.dtype == torch.float16:
+        fn, name = lib.anygpu_gated_rmsnorm_f16, "anygpu_gated_rmsnorm_f16"
+    elif xt.dtype == torch.float32:
+        fn, name = lib.anygpu_gated_rmsnorm_f32, "anygpu_gated_rmsnorm_f32"
+    else:
+        raise TypeError("Unsupported data types")
+    rc = fn(xt.data_ptr(), None if gate is None else gate.data_ptr(), wt.data_ptr(), out.data_ptr(), rows, cols,
+            float(eps), int(zero_centered), _stream_ptr())
+    capi.check(name, rc)
+    return out
+
+
+def tensor_zamba_gated_rmsnorm(xt: torch.Tensor, zt: torch.Tensor, wt: torch.Tensor, gsize: int, eps: float) -> torch.Tensor:
+    """Same contract as tensor_zamba_gated_rmsnorm of the reference (srcs/models/zamba2/zamba_gated_rmsnorm.hpp:9-23):
+    one group spans the row, gsize is accepted and, as there, not used."""
+    return tensor_rms_norm(xt, wt, eps, False, gate=zt)
+
+
 def tensor_mm_batched(lhs: torch.Tensor, rhs: torch.Tensor, b_layout: int = capi.B_ROW_MAJOR) -> torch.Tensor:
     """out[i] = lhs[i] @ B[i] for dense 3-D operands [batch, M, K] and [batch, K, N] (or [batch, N, K] with
     B_COL_MAJOR) in one launch: the per-head loop of the reference's attention collapsed."""

@@ -181,6 +181,35 @@ int anygpu_causal_conv1d_silu_f32(const float* x, const float* w, const float* b
                                   int64_t batch, int64_t chan, int64_t seqlen, int64_t width,
                                   void* stream);
 
+/*
+ * One decode step of the same convolution: x is [batch, chan] (the new sample of every row), state is
+ * [batch, chan, width - 1], the samples in front of it, oldest first, and is updated in place
+ * (shifted by one, x appended); y[b, d] = silu(bias[d] + sum_{k < width-1} w[d, k] * state[b, d, k]
+ * + w[d, width-1] * x[b, d]).  Starting from a zero state, seqlen calls reproduce
+ * anygpu_causal_conv1d_silu_* column by column.  The reference has no decode path for its Mamba2
+ * convolution (srcs/fused/causal_conv1d.hpp:24-117 is the whole-sequence form this step continues).
+ * state may be NULL when width == 1.
+ */
+int anygpu_causal_conv1d_silu_update_f16(const void* x, void* state, const void* w, const void* bias, void* y,
+                                         int64_t batch, int64_t chan, int64_t width, void* stream);
+
+int anygpu_causal_conv1d_silu_update_f32(const float* x, float* state, const float* w, const float* bias, float* y,
+                                         int64_t batch, int64_t chan, int64_t width, void* stream);
+
+/*
+ * Gated RMS normalisation over rows of `cols` contiguous elements:
+ *     g = x * silu(z) (g = x when z == NULL);  y = g / sqrt(mean(g^2) + eps) * (w + (zero_centered ? 1 : 0))
+ * x, z, y are [rows, cols], w is [cols]; fp32 internals.  One kernel for tensor_zamba_gated_rmsnorm
+ * (srcs/models/zamba2/zamba_gated_rmsnorm.hpp:9-23: tensor_silu, tensor_mul, tensor_rms_norm, three
+ * kernels there) and, with z == NULL, for cu_tensor_rms_norm_f32 / _v1 (srcs/kernels/cuda/norm_ops.cuh:14-37)
+ * normalising over the last axis.
+ */
+int anygpu_gated_rmsnorm_f16(const void* x, const void* z, const void* w, void* y,
+                             int64_t rows, int64_t cols, float eps, int zero_centered, void* stream);
+
+int anygpu_gated_rmsnorm_f32(const float* x, const float* z, const float* w, float* y,
+                             int64_t rows, int64_t cols, float eps, int zero_centered, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

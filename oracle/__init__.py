@@ -178,6 +178,57 @@ def gemma_mlp_upproj(x: np.ndarray, w_gate: np.ndarray, w_up: np.ndarray, thread
     return y
 
 
+def tensor_silu(x: np.ndarray) -> np.ndarray:
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    y = np.empty_like(x)
+    fn = lib().oracle_tensor_silu_f32
+    fn.restype = None
+    fn(_ptr(x), _ptr(y), c_int64(x.size))
+    return y
+
+
+def tensor_rms_norm(x: np.ndarray, w: np.ndarray, eps: float, zero_centered: bool = False) -> np.ndarray:
+    """RMS normalisation over the trailing axes that w spans."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    w = np.ascontiguousarray(w, dtype=np.float32)
+    assert tuple(x.shape[x.ndim - w.ndim:]) == tuple(w.shape), "wt shape is incorrect"
+    size = w.size
+    y = np.empty_like(x)
+    fn = lib().oracle_tensor_rms_norm_f32
+    fn.restype = None
+    fn(_ptr(x), _ptr(w), c_float(eps), c_int(int(zero_centered)), _ptr(y), c_int64(x.size // size if size else 0), c_int64(size))
+    return y
+
+
+def zamba_gated_rmsnorm(x: np.ndarray, z: np.ndarray, w: np.ndarray, eps: float) -> np.ndarray:
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    z = np.ascontiguousarray(z, dtype=np.float32)
+    w = np.ascontiguousarray(w, dtype=np.float32)
+    assert x.shape == z.shape and w.ndim == 1 and x.shape[-1] == w.shape[0]
+    cols = w.shape[0]
+    y = np.empty_like(x)
+    fn = lib().oracle_zamba_gated_rmsnorm_f32
+    fn.restype = None
+    fn(_ptr(x), _ptr(z), _ptr(w), c_float(eps), _ptr(y), c_int64(x.size // cols if cols else 0), c_int64(cols))
+    return y
+
+
+def causal_conv1d_update(x: np.ndarray, state: np.ndarray, w: np.ndarray, b: np.ndarray):
+    """One decode step.  x [batch, dims], state [batch, dims, width - 1] -> (y [batch, dims], new state)."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    w = np.ascontiguousarray(w, dtype=np.float32)
+    b = np.ascontiguousarray(b, dtype=np.float32)
+    batch, dims = x.shape
+    width = w.shape[1]
+    assert w.shape[0] == dims and b.shape == (dims,) and state.shape == (batch, dims, width - 1)
+    new_state = np.array(state, dtype=np.float32, order="C", copy=True)
+    y = np.empty_like(x)
+    fn = lib().oracle_causal_conv1d_update_f32
+    fn.restype = None
+    fn(_ptr(x), _ptr(new_state), _ptr(w), _ptr(b), _ptr(y), c_int64(batch), c_int64(dims), c_int64(width))
+    return y, new_state
+
+
 def causal_mask(q_len: int, k_len: int, diag: int = 0) -> np.ndarray:
     mask = np.empty((q_len, k_len), dtype=np.float32)
     fn = lib().oracle_causal_mask_f32

@@ -35,6 +35,14 @@
  *                            error stays below 1e-3).
  *   oracle_gemma_mlp_upproj_f32   equality with the chain tensor_mm, gelu, tensor_mm, tensor_mul of the
  *                            functions above (bit exact), float64 brute force.
+ *   oracle_tensor_silu_f32   silu(0) = 0, silu(x) - silu(-x) = x, float64 formula.
+ *   oracle_tensor_rms_norm_f32   constant rows (y = w c / sqrt(c^2 + eps)), sum (y / w)^2 = n at eps = 0, scale
+ *                            invariance at eps = 0, zero-centred weights = weights + 1, float64 brute force.
+ *   oracle_zamba_gated_rmsnorm_f32   equality with the chain silu, mul, rms_norm (bit exact), z = 0 gives y = 0
+ *                            up to the eps floor, float64 brute force.
+ *   oracle_causal_conv1d_update_f32   seq_len successive steps from a zero state equal the whole-sequence
+ *                            oracle_tensor_causal_conv1d_f32 bit for bit (up to the sign of zero); the state after
+ *                            the steps holds the last width-1 samples.
  *   oracle_cvt_f16_to_f32    all 65536 bit patterns vs numpy.float16.
  *   oracle_compare_*         hand-computed three-element cases.
  * The reference repository holds no golden vectors for this path (its .dat fixtures are
@@ -469,6 +477,73 @@ ORACLE_API void oracle_gemma_mlp_upproj_f32(const float* x, const float* w_gate,
 			oracle_tensor_gelu_tanh_f32(&gate, &act, 1);
 			y[r * isize + c] = act * up;
 		}
+	}
+}
+
+/* tensor_silu  --  srcs/ops/math_ops.hpp:16-35: y = x / (1 + exp(-x)); the float overload of exp for float32 */
+ORACLE_API void oracle_tensor_silu_f32(const float* x, float* y, i64 length)
+{
+	for (i64 k = 0; k < length; ++k) y[k] = x[k] / (1.0f + expf(-x[k]));
+}
+
+/* ------------------------------------------------------------------------------------------
+ * tensor_rms_norm  --  srcs/ops/norm_ops.hpp:129-190
+ *   per region of `size` contiguous elements: accum = sum x^2 left to right in T (:170-176);
+ *   mean = accum / size (:178); y = (x / sqrt(mean + eps)) * (w + delta), delta = 1 for zero-centred
+ *   weights else 0 (:148,181-187).
+ * ---------------------------------------------------------------------------------------- */
+ORACLE_API void oracle_tensor_rms_norm_f32(const float* x, const float* w, float eps, int zero_centered, float* y,
+                                           i64 regions, i64 size)
+{
+	const float delta = zero_centered ? 1.0f : 0.0f;
+	for (i64 r = 0; r < regions; ++r)
+	{
+		const float* xr = x + r * size;
+		float* yr = y + r * size;
+		float accum = 0.f;
+		for (i64 ix = 0; ix < size; ++ix) accum += xr[ix] * xr[ix];
+		const float mean = accum / (float)size;
+		for (i64 ix = 0; ix < size; ++ix) yr[ix] = (xr[ix] / sqrtf(mean + eps)) * (w[ix] + delta);
+	}
+}
+
+/* tensor_zamba_gated_rmsnorm  --  srcs/models/zamba2/zamba_gated_rmsnorm.hpp:9-23
+ *   silu_z = tensor_silu(z); gated = tensor_mul(x, silu_z); y = tensor_rms_norm(gated, -1, w, eps)
+ *   (the group size argument is unused there: one group spans the row). */
+ORACLE_API void oracle_zamba_gated_rmsnorm_f32(const float* x, const float* z, const float* w, float eps, float* y,
+                                               i64 rows, i64 cols)
+{
+	float* gated = (float*)malloc((size_t)(cols > 0 ? cols : 1) * sizeof(float));
+	for (i64 r = 0; r < rows; ++r)
+	{
+		oracle_tensor_silu_f32(z + r * cols, gated, cols);
+		for (i64 c = 0; c < cols; ++c) gated[c] = x[r * cols + c] * gated[c];
+		oracle_tensor_rms_norm_f32(gated, w, eps, 0, y + r * cols, 1, cols);
+	}
+	free(gated);
+}
+
+/* ------------------------------------------------------------------------------------------
+ * Decode step of tensor_causal_conv1d.  The reference has only the whole-sequence form
+ * (srcs/fused/causal_conv1d.hpp:24-87); this is its loop body for one position s with the samples
+ * x[s - (width-1) .. s - 1] handed over in `state` (oldest first) instead of being read from the row:
+ *   out = 0; for k ascending: out += w[d,k] * (k < width-1 ? state[k] : x); out += bias; out = out / (1 + exp(-out))
+ * then the state is shifted by one and takes x.  From a zero state the terms the whole-sequence loop
+ * skips (negative positions) are added here as w * 0, which changes no sum.
+ * ---------------------------------------------------------------------------------------- */
+ORACLE_API void oracle_causal_conv1d_update_f32(const float* x, float* state, const float* w, const float* b, float* y,
+                                                i64 batch, i64 dims, i64 width)
+{
+	for (i64 row = 0; row < batch * dims; ++row)
+	{
+		const i64 d = row % dims;
+		float* st = state + row * (width - 1);
+		float out = 0.f;
+		for (i64 k = 0; k < width; ++k) out += w[d * width + k] * (k < width - 1 ? st[k] : x[row]);
+		out += b[d];
+		y[row] = out / (1.0f + expf(-out));
+		for (i64 k = 0; k + 1 < width - 1; ++k) st[k] = st[k + 1];
+		if (width > 1) st[width - 2] = x[row];
 	}
 }
 

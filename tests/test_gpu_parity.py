@@ -268,6 +268,89 @@ def test_conv1d_empty_and_rejected_arguments(ops):
 
 
 # =============================================================================================
+# Mamba2 neighbours of the convolution: decode step, gated RMS norm
+# =============================================================================================
+
+@pytest.mark.parametrize("dtype", ["f16", "f32"])
+@pytest.mark.parametrize("b,d,width", [(1, 1, 1), (2, 5, 4), (3, 300, 3), (4, 4224, 4), (1, 257, 2)])
+def test_conv1d_update_steps_match_whole_sequence(ops, oracle, dtype, b, d, width):
+    import torch
+    np_dt = np.float16 if dtype == "f16" else np.float32
+    s = 9
+    x = synth.normal(b + d, (b, d, s)).astype(np_dt)
+    w = (synth.normal(1, (d, width)) * np.float32(0.5)).astype(np_dt)
+    bias = (synth.normal(2, (d,)) * np.float32(0.1)).astype(np_dt)
+    up = (lambda a: oracle.cvt_f16_to_f32(a)) if dtype == "f16" else (lambda a: a)
+    tol = TOL_F16_ROWOPS if dtype == "f16" else TOL_F32
+    state = torch.zeros((b, d, width - 1), dtype=torch.float16 if dtype == "f16" else torch.float32, device="cuda")
+    ref_state = np.zeros((b, d, width - 1), dtype=np.float32)
+    dw, db = dev(w), dev(bias)
+    for t in range(s):
+        got = host(ops.tensor_causal_conv1d_update(dev(x[:, :, t]), state, dw, db)).astype(np.float32)
+        want, ref_state = oracle.causal_conv1d_update(up(x[:, :, t]), ref_state, up(w), up(bias))
+        assert scaled_rel_err(got, want, 1.0) <= tol, t
+        assert np.array_equal(host(state).astype(np.float32), ref_state)         # the state is a copy of samples: exact
+    # and the steps together are the whole-sequence kernel
+    whole = host(ops.tensor_causal_conv1d(dev(x), dw, db)).astype(np.float32)
+    want_last = oracle.tensor_causal_conv1d(up(x), up(w), up(bias))[:, :, -1]
+    assert scaled_rel_err(whole[:, :, -1], want_last, 1.0) <= tol
+    assert scaled_rel_err(got, whole[:, :, -1], 1.0) <= tol
+
+
+@pytest.mark.parametrize("dtype", ["f16", "f32"])
+@pytest.mark.parametrize("rows,cols", [(1, 1), (3, 7), (5, 64), (4, 1000), (6, 1024), (3, 2048), (2, 4096), (2, 8192),
+                                       (2, 8200), (1, 16384), (2, 20000), (9, 4104)])
+def test_gated_rmsnorm_shapes(ops, oracle, dtype, rows, cols):
+    np_dt = np.float16 if dtype == "f16" else np.float32
+    eps = 1e-5
+    x = synth.normal(rows + cols, (rows, cols)).astype(np_dt)
+    z = (synth.normal(cols, (rows, cols)) * np.float32(2.0)).astype(np_dt)
+    w = synth.uniform(3, (cols,), 0.5, 1.5).astype(np_dt)
+    up = (lambda a: oracle.cvt_f16_to_f32(a)) if dtype == "f16" else (lambda a: a)
+    tol = TOL_F16_ROWOPS if dtype == "f16" else TOL_F32
+    got = host(ops.tensor_zamba_gated_rmsnorm(dev(x), dev(z), dev(w), cols, eps)).astype(np.float32)
+    want = oracle.zamba_gated_rmsnorm(up(x), up(z), up(w), eps)
+    assert scaled_rel_err(got, want, 1.0) <= tol                      # outputs have unit mean square times w ~ 1
+    plain = host(ops.tensor_rms_norm(dev(x), dev(w), eps, zero_centered=True)).astype(np.float32)
+    assert scaled_rel_err(plain, oracle.tensor_rms_norm(up(x), up(w), eps, zero_centered=True), 1.0) <= tol
+
+
+def test_gated_rmsnorm_reference_case_group_4096(ops, oracle):
+    # tests/zamba2_tests.cpp:458-476: eps 1e-5, group size 4096 = the row; rows of a [1, 70, 4096] activation
+    x, z = synth.normal(1, (1, 70, 4096)), synth.normal(2, (1, 70, 4096))
+    w = synth.uniform(3, (4096,), 0.5, 1.5)
+    got = host(ops.tensor_zamba_gated_rmsnorm(dev(x), dev(z), dev(w), 4096, 1e-5))
+    want = oracle.zamba_gated_rmsnorm(x, z, w, 1e-5)
+    ok, worst = oracle.compare_data_buffers(got, want)                # the reference's own gate: abs 1e-3
+    assert ok, worst
+    assert scaled_rel_err(got, want, 1.0) <= TOL_F32
+    # closed gate: silu(0) = 0, every output is exactly 0
+    assert not host(ops.tensor_zamba_gated_rmsnorm(dev(x), dev(np.zeros_like(z)), dev(w), 4096, 1e-5)).any()
+
+
+def test_mamba2_neighbours_rejected_arguments(ops):
+    import torch
+    from anygpu_amd import capi
+    lib = capi.load()
+    x = torch.zeros((2, 8), device="cuda")
+    y = torch.full((2, 8), 3.0, device="cuda")
+    w = torch.ones((8,), device="cuda")
+    f = lib.anygpu_gated_rmsnorm_f32
+    assert f(x.data_ptr(), None, None, y.data_ptr(), 2, 8, 1e-5, 0, None) == capi.ANYGPU_ERR_NULL_POINTER
+    assert f(x.data_ptr(), None, w.data_ptr(), y.data_ptr(), 2, -8, 1e-5, 0, None) == capi.ANYGPU_ERR_BAD_SHAPE
+    assert f(x.data_ptr(), None, w.data_ptr(), y.data_ptr(), 2, 8, -1.0, 0, None) == capi.ANYGPU_ERR_UNSUPPORTED
+    assert f(x.data_ptr(), None, w.data_ptr(), y.data_ptr(), 0, 8, 1e-5, 0, None) == capi.ANYGPU_OK
+    g = lib.anygpu_causal_conv1d_silu_update_f32
+    wt = torch.ones((8, 4), device="cuda")
+    assert g(x.data_ptr(), None, wt.data_ptr(), w.data_ptr(), y.data_ptr(), 2, 8, 4, None) == capi.ANYGPU_ERR_NULL_POINTER
+    assert g(x.data_ptr(), x.data_ptr(), wt.data_ptr(), w.data_ptr(), y.data_ptr(), 2, 8, 5, None) == capi.ANYGPU_ERR_UNSUPPORTED
+    torch.cuda.synchronize()
+    assert bool((y == 3.0).all())
+    with pytest.raises(ValueError):
+        ops.tensor_causal_conv1d_update(x, torch.zeros((2, 8, 2), device="cuda"), wt, w)
+
+
+# =============================================================================================
 # GEMM
 # =============================================================================================
 

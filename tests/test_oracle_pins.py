@@ -448,6 +448,72 @@ def test_mlp_upproj_equals_primitive_chain_and_float64(oracle):
 
 
 # ---------------------------------------------------------------------------------------------
+# Mamba2 neighbours of the convolution: gated RMS norm, decode step of the convolution
+# ---------------------------------------------------------------------------------------------
+
+def test_silu_closed_forms(oracle):
+    grid = np.linspace(-20, 20, 4001).astype(np.float32)
+    s = oracle.tensor_silu(grid).astype(np.float64)
+    sm = oracle.tensor_silu(-grid).astype(np.float64)
+    assert oracle.tensor_silu(np.zeros(1, dtype=np.float32))[0] == 0.0
+    assert np.max(np.abs(s - sm - grid)) < 2e-6                     # x s(x) - (-x) s(-x) = x (s(x) + s(-x)) = x
+    g64 = grid.astype(np.float64)
+    assert np.max(np.abs(s - g64 / (1 + np.exp(-g64)))) < 2e-6
+
+
+def test_rms_norm_closed_forms(oracle):
+    n = 64
+    w = synth.uniform(1, (n,), 0.5, 1.5)
+    # constant rows: mean x^2 = c^2 exactly, y = w c / sqrt(c^2 + eps)
+    for c, eps in ((2.0, 1e-5), (-0.5, 0.0), (3.0, 1.0)):
+        y = oracle.tensor_rms_norm(np.full((3, n), c, dtype=np.float32), w, eps)
+        want = w.astype(np.float64) * c / math.sqrt(c * c + eps)
+        assert np.max(np.abs(y - want)) < 1e-6
+    x = synth.normal(2, (5, n))
+    y0 = oracle.tensor_rms_norm(x, w, 0.0)
+    assert np.max(np.abs(((y0 / w).astype(np.float64) ** 2).sum(axis=1) - n)) < 1e-3      # unit mean square
+    assert np.max(np.abs(oracle.tensor_rms_norm(x * np.float32(4.0), w, 0.0) - y0)) < 1e-5  # scale invariance (x4 is exact)
+    assert np.array_equal(oracle.tensor_rms_norm(x, w, 1e-5, zero_centered=True),
+                          oracle.tensor_rms_norm(x, w + np.float32(1.0), 1e-5))
+    x64 = x.astype(np.float64)
+    want = x64 / np.sqrt((x64 ** 2).mean(axis=1, keepdims=True) + 1e-5) * w
+    assert np.max(np.abs(oracle.tensor_rms_norm(x, w, 1e-5) - want)) < 1e-5
+    # a norm taken over the wrong axis or with the weight indexed by row would fail the shapes: w spans the last axis
+    with pytest.raises(AssertionError):
+        oracle.tensor_rms_norm(x.T.copy(), w, 1e-5)
+
+
+def test_gated_rmsnorm_equals_chain_and_float64(oracle):
+    rows, n, eps = 6, 96, 1e-5
+    x, z = synth.normal(1, (rows, n)), synth.normal(2, (rows, n)) * np.float32(2.0)
+    w = synth.uniform(3, (n,), 0.5, 1.5)
+    y = oracle.zamba_gated_rmsnorm(x, z, w, eps)
+    chain = oracle.tensor_rms_norm(oracle.tensor_mul(x, oracle.tensor_silu(z)), w, eps)
+    assert np.array_equal(y, chain)
+    x64, z64 = x.astype(np.float64), z.astype(np.float64)
+    g = x64 * z64 / (1 + np.exp(-z64))
+    want = g / np.sqrt((g ** 2).mean(axis=1, keepdims=True) + eps) * w
+    assert np.max(np.abs(y - want)) < 1e-5
+    assert not np.any(oracle.zamba_gated_rmsnorm(x, np.zeros_like(z), w, eps))            # silu(0) = 0 closes the gate
+    # the gate is on z, not on x: swapping the two changes the result
+    assert not np.allclose(oracle.zamba_gated_rmsnorm(z, x, w, eps), y, atol=1e-3)
+
+
+def test_conv1d_update_steps_reproduce_whole_sequence(oracle):
+    for width in (1, 2, 3, 4):
+        b, d, s = 2, 5, 19
+        x = synth.normal(width, (b, d, s))
+        wt = synth.normal(10 + width, (d, width))
+        bt = synth.normal(20 + width, (d,))
+        full = oracle.tensor_causal_conv1d(x, wt, bt)
+        state = np.zeros((b, d, width - 1), dtype=np.float32)
+        for t in range(s):
+            y, state = oracle.causal_conv1d_update(x[:, :, t], state, wt, bt)
+            assert np.array_equal(y, full[:, :, t]), (width, t)
+        assert np.array_equal(state, x[:, :, s - (width - 1):] if width > 1 else state)
+
+
+# ---------------------------------------------------------------------------------------------
 # fp16 up-cast and comparators
 # ---------------------------------------------------------------------------------------------
 
