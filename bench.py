@@ -35,7 +35,7 @@ PEAK_HBM_GBS = 8000.0          # HBM3E
 # Bytes per launch moved behind the L2s, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE (KiB per
 # dispatch), scaled by what the same counters read for a plain 256 MiB device copy (fetch x 2.000,
 # write x 1.000); the summaries are under profiles/.
-MEASURED_TRAFFIC_BYTES = {"gemm_f16": 234962687, "gemm_f32": 167970906, "conv1d": 277226336,
+MEASURED_TRAFFIC_BYTES = {"gemm_f16": 234962687, "gemm_f32": 167994164, "conv1d": 277226336,
                           "softmax_causal": 410887952, "softmax_gemma2": 1514268488}
 
 
