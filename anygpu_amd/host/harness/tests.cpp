@@ -10,6 +10,7 @@
 #include "gemma_linsoftcap.hpp"
 #include "gemma_mlp.hpp"
 #include "zamba_gated_rmsnorm.hpp"
+#include "sdpa_gemma2_linear.cuh"
 #include "fast_mm.cuh"
 #include "dat_file.hpp"
 #include "test_tools.hpp"
@@ -532,6 +533,32 @@ TEST_CASE(test_gemma2_mlp_fused_upproj_1x37x288_i1152, GPU)
 	auto act1 = tensor_gemma_mlp_fused_uprpoj<float32, CUDA, 1>(dw, dx).copy_to_host();
 	auto act2 = tensor_gemma_mlp_fused_uprpoj<float32, CUDA, 2>(dw, dx).copy_to_host();
 	return elementwise_compatible(exp_hy, act1) && compare_data_buffers(act1, exp_hy) && compare_data_buffers(act2, exp_hy);
+}
+
+TEST_CASE(test_gemma2_decoder_mlp_1x21x256_i1024, GPU)
+{
+	// the whole block (gate / up, activation, product, down) against the operator chain on the host
+	GemmaMLPweights<float32, CPU> hw;
+	hw.gate_proj_weight = tensor_mul(crt_random_normal_tensor<float32, CPU>({ 256, 1024 }, 3), 0.06f);
+	hw.up_proj_weight = tensor_mul(crt_random_normal_tensor<float32, CPU>({ 256, 1024 }, 4), 0.06f);
+	hw.down_proj_weight = tensor_mul(crt_random_normal_tensor<float32, CPU>({ 1024, 256 }, 5), 0.03f);
+	auto hx = crt_random_normal_tensor<float32, CPU>({ 1, 21, 256 }, 6);
+	auto exp_hy = tensor_gemma_mlp(hw, hx);
+	GemmaMLPweights<float32, CUDA> dw;
+	dw.gate_proj_weight = hw.gate_proj_weight.copy_to_cuda();
+	dw.up_proj_weight = hw.up_proj_weight.copy_to_cuda();
+	dw.down_proj_weight = hw.down_proj_weight.copy_to_cuda();
+	auto dx = hx.copy_to_cuda();
+	auto act_hy = tensor_gemma_mlp(dw, dx).copy_to_host();
+	bool ok = elementwise_compatible(exp_hy, act_hy) && compare_data_buffers(act_hy, exp_hy);
+	// single token: the decode step takes the few-row kernels
+	auto hx1 = crt_random_normal_tensor<float32, CPU>({ 1, 1, 256 }, 7);
+	auto act1 = tensor_gemma_mlp(dw, hx1.copy_to_cuda()).copy_to_host();
+	ok = ok && compare_data_buffers(act1, tensor_gemma_mlp(hw, hx1));
+	// the attention block's projection launcher
+	Tensor<float32, CUDA> proj(std::vector<int64>{ 1, 21, 1024 });
+	cu_sdpa_gemma2_linear_f32_v1(dx, dw.gate_proj_weight, proj);
+	return ok && compare_data_buffers(proj.copy_to_host(), tensor_linear(hx, hw.gate_proj_weight));
 }
 
 TEST_CASE(test_cpu_causal_conv1d_update_steps, HOST)

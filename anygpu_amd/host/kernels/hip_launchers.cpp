@@ -7,6 +7,8 @@
 #include "causal_conv1d.cuh"
 #include "norm_ops.cuh"
 #include "mlp_gemma2_fused_upproj.cuh"
+#include "mlp_gemma2_dp_linear.cuh"
+#include "sdpa_gemma2_linear.cuh"
 #include "gemma_linsoftcap.cuh"
 
 #include "anygpu_hip.h"
@@ -240,6 +242,35 @@ void cu_mlp_gemma2_fused_upproj_f32_v2(const Tensor<float32, CUDA>& xt, const Te
                                        const Tensor<float32, CUDA>& wt_up, Tensor<float32, CUDA>& yt)
 {
 	fused_upproj(xt, wt_gp, wt_up, yt);
+}
+
+namespace {
+
+// y (batch, seq_len, out) = x (batch, seq_len, in) * w (in, out): the leading axes fold into rows
+void linear_over_tokens(const Tensor<float32, CUDA>& xt, const Tensor<float32, CUDA>& wt, Tensor<float32, CUDA>& yt)
+{
+	const int64 sl = xt.shape[0] * xt.shape[1];
+	const int64 in_features = wt.shape[0], out_features = wt.shape[1];
+	ABI_CHECK(anygpu_gemm_f32(xt.buffer(), wt.buffer(), nullptr, yt.buffer(), sl, out_features, in_features,
+	                          std::max<int64>(in_features, 1), std::max<int64>(out_features, 1), std::max<int64>(out_features, 1),
+	                          ANYGPU_A_ROW_MAJOR, ANYGPU_B_ROW_MAJOR, kNullStream));
+}
+
+}  // namespace
+
+void cu_mlp_gemma2_dp_linear_f32_v1(const Tensor<float32, CUDA>& xt, const Tensor<float32, CUDA>& wt_dp, Tensor<float32, CUDA>& yt)
+{
+	linear_over_tokens(xt, wt_dp, yt);
+}
+
+void cu_mlp_gemma2_dp_linear_f32_v4(const Tensor<float32, CUDA>& xt, const Tensor<float32, CUDA>& wt_dp, Tensor<float32, CUDA>& yt)
+{
+	linear_over_tokens(xt, wt_dp, yt);
+}
+
+void cu_sdpa_gemma2_linear_f32_v1(const Tensor<float32, CUDA>& xt, const Tensor<float32, CUDA>& wt, Tensor<float32, CUDA>& yt)
+{
+	linear_over_tokens(xt, wt, yt);
 }
 
 /* ---- Mamba2 neighbours of the convolution ---- */

@@ -1,9 +1,11 @@
-// Gemma2 MLP, first half: act(x Wgate) (*) (x Wup) with the tanh form of GELU.
-// Reference interface: srcs/models/gemma2/gemma_mlp.hpp:51-95 (tensor_gemma_mlp_fused_uprpoj).
+// Gemma2 MLP: down(act(x Wgate) (*) (x Wup)) with the tanh form of GELU.
+// Reference interface: srcs/models/gemma2/gemma_mlp.hpp:12-141 (weights, tensor_gemma_mlp_fused_uprpoj,
+// tensor_gemma_mlp_dp_linear, tensor_gemma_mlp).
 #ifndef __GEMMA_MLP__
 #define __GEMMA_MLP__
 
 #include "mlp_gemma2_fused_upproj.cuh"
+#include "mlp_gemma2_dp_linear.cuh"
 
 #include "tensor.hpp"
 #include "core_concepts.hpp"
@@ -14,6 +16,7 @@ struct GemmaMLPweights
 {
 	Tensor<dtype, device> gate_proj_weight;  // (hidden, intermediate)
 	Tensor<dtype, device> up_proj_weight;    // (hidden, intermediate)
+	Tensor<dtype, device> down_proj_weight;  // (intermediate, hidden)
 };
 
 /*
@@ -47,6 +50,51 @@ inline Tensor<dtype, device> tensor_gemma_mlp_fused_uprpoj(
 		auto act_gated_x = tensor_gelu(gated_x, true);
 		auto up_x = tensor_linear(x, mlp_weights.up_proj_weight);
 		return tensor_mul(act_gated_x, up_x);
+	}
+}
+
+/*
+  Down projection.  variant 0: tensor_linear (any device); variant 1, 4: the reference's names for two
+  generations of its specialised kernel, the fp32 MFMA GEMM here (GPU tensors only).
+*/
+template<FloatingPointType dtype, Device device, int variant>
+inline Tensor<dtype, device> tensor_gemma_mlp_dp_linear(
+	const GemmaMLPweights<dtype, device>& mlp_weights,
+	const Tensor<dtype, device>& x)
+{
+	if constexpr (device == CUDA && (variant == 1 || variant == 4))
+	{
+		static_assert(std::is_same_v<dtype, float32>, "Unsupported data types");
+		ACASSERT(x.dim == 3, "x should be 3 dim");
+		ACASSERT(x.shape[2] == mlp_weights.down_proj_weight.shape[0], "intermediate size should match for x and the weight");
+		Tensor<dtype, device> out(std::vector<int64>{ x.shape[0], x.shape[1], mlp_weights.down_proj_weight.shape[1] });
+		if constexpr (variant == 1)
+			cu_mlp_gemma2_dp_linear_f32_v1(x, mlp_weights.down_proj_weight, out);
+		else
+			cu_mlp_gemma2_dp_linear_f32_v4(x, mlp_weights.down_proj_weight, out);
+		return out;
+	}
+	else
+	{
+		return tensor_linear(x, mlp_weights.down_proj_weight);
+	}
+}
+
+/* The whole block: fused gate / up projection and down projection on the GPU, operator calls on the host. */
+template<FloatingPointType dtype, Device device>
+inline Tensor<dtype, device> tensor_gemma_mlp(
+	const GemmaMLPweights<dtype, device>& mlp_weights,
+	const Tensor<dtype, device>& x)
+{
+	if constexpr (device == CUDA)
+	{
+		auto mid = tensor_gemma_mlp_fused_uprpoj<dtype, device, 2>(mlp_weights, x);
+		return tensor_gemma_mlp_dp_linear<dtype, device, 4>(mlp_weights, mid);
+	}
+	else
+	{
+		auto mid = tensor_gemma_mlp_fused_uprpoj<dtype, device, 0>(mlp_weights, x);
+		return tensor_gemma_mlp_dp_linear<dtype, device, 0>(mlp_weights, mid);
 	}
 }
 
