@@ -58,6 +58,8 @@ SIGNATURES = {
                                                      c_int64, c_int64, c_int64, c_void_p]),
     "anygpu_causal_conv1d_silu_update_f32": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                                      c_int64, c_int64, c_int64, c_void_p]),
+    "anygpu_sdp_attention_fwd_f16": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64,
+                                             c_float, c_float, c_int, c_int64, c_void_p]),
     "anygpu_gated_rmsnorm_f16": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_float, c_int, c_void_p]),
     "anygpu_gated_rmsnorm_f32": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_float, c_int, c_void_p]),
 }

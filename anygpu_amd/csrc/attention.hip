@@ -1,0 +1,351 @@
+// Fused scaled-dot-product attention, forward, fp16 in / fp16 out, for gfx950:
+//     y = softmax(mask(softcap(alpha * q k^T))) v        per (batch, head)
+// in ONE kernel.  The score matrix never reaches HBM: for 8 heads x 8192 x 8192 keys the
+// three-launch form (q k^T, row softmax, p v) writes and reads 1 GiB of scores twice; this kernel
+// reads q, k, v and writes y.
+//
+// A block of 4 waves owns 128 consecutive queries of one head, a wave 32 of them (two blocks of
+// 16).  It walks the visible key range in tiles of 64 keys.  Per tile:
+//   * K and V rows go global -> registers -> LDS (the loads of the next tile are in flight
+//     while this one is being used);
+//   * S^T = K Q^T with v_mfma_f32_16x16x32_f16: the K fragment is the first operand, the Q
+//     fragment (kept in registers for the whole kernel) the second, so a lane ends up holding,
+//     for ONE query (lane % 16), the scores of keys 4 (lane / 16) + r of each 16-key block.
+//     Row maxima and sums are therefore in-lane loops plus two cross-lane steps (xor 16, xor 32);
+//   * scale / softcap / mask in fp32, online max / sum in the log2 domain, p = exp2(z - m)
+//     rounded to fp16;
+//   * O^T += V^T P^T: first operand V^T, read out of the row-major V tile with transposing LDS
+//     loads (ds_read_b64_tr_b16: four consecutive keys of one column per lane), second operand the
+//     p values exactly as they sit in the lane.  The result again has the query in lane % 16, so the
+//     running rescale exp2(m_old - m_new) is an in-lane multiply.
+// The summation index of the second product is "key slot" (lane group, j): both operands use
+// slot j <-> key 16 * (2 t + j / 4) + 4 * (lane / 16) + j % 4 of the tile, so no shuffle is needed
+// between the two products.
+//
+// Masks are index rules (causal with the diagonal at n_k - n_q, sliding window); tiles without a
+// visible key are skipped.  A query without any visible key gets zeros.
+#include "device_utils.hpp"
+#include "launch.hpp"
+
+#include <atomic>
+
+namespace anygpu {
+
+namespace {
+
+constexpr int kAttnQueriesPerBlock = 128;
+constexpr int kAttnKeysPerTile = 64;
+
+typedef short short4_t __attribute__((ext_vector_type(4)));
+
+// ds_read_b64_tr_b16: within each group of 16 lanes, lane i receives element (i % 4) of the
+// 4-element rows addressed by lanes i / 4, i / 4 + 4, i / 4 + 8, i / 4 + 12 of the group.  With lane
+// r of a group pointing at V[k0 + r / 4][d0 + 4 (r % 4) ...], lane i ends up with V[k0 .. k0 + 3][d0 + i].
+__device__ __forceinline__ half4_t lds_read_tr_b64(const char* lds_addr)
+{
+	const short4_t v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4_t*)(lds_addr));
+	return __builtin_bit_cast(half4_t, v);
+}
+
+struct AttnArgs
+{
+	const half_t* q;
+	const half_t* k;
+	const half_t* v;
+	half_t* y;
+	int n_q, n_k;
+	int q_per_kv;          // query heads that share one k / v head
+	int diag;              // key j is causally visible to query i iff j <= i + diag
+	int causal;
+	int window;            // 0: off; else key j is visible iff j > i + diag - window
+	float k_in, k_cap;     // logit transform constants (see logit2)
+};
+
+// log2(e) * softcap(alpha * s); without softcap k_in = alpha log2(e); with it
+// cap log2(e) tanh(alpha s / cap) = k_cap - 2 k_cap / (1 + exp2(s k_in)), k_in = 2 log2(e) alpha / cap
+template <bool SOFTCAP>
+__device__ __forceinline__ float logit2(float s, float k_in, float k_cap)
+{
+	if constexpr (SOFTCAP)
+	{
+		const float t = fast_exp2(s * k_in);
+		return fmaf(fast_rcp(1.0f + t), -2.0f * k_cap, k_cap);
+	}
+	return s * k_in;
+}
+
+template <int D>
+struct AttnLds
+{
+	static constexpr int kPitchK = 2 * D + 16;      // bytes; 16-byte reads of 16 rows hit 64 different banks
+	static constexpr int kPitchV = 2 * D + 32;      // bytes; the 8 rows of a half wave's transposing read do
+	static constexpr int kBytes = kAttnKeysPerTile * (kPitchK + kPitchV);
+};
+
+template <int D, bool SOFTCAP>
+__global__ __launch_bounds__(256) void sdp_attention_fwd_f16_kernel(const AttnArgs a)
+{
+	extern __shared__ __align__(16) char lds[];
+	using L = AttnLds<D>;
+	char* k_lds = lds;
+	char* v_lds = lds + kAttnKeysPerTile * L::kPitchK;
+	constexpr int KS = D / 32;                      // MFMA steps along the head dimension (q k^T)
+	constexpr int DC = D / 16;                      // 16-wide column blocks of the output
+	constexpr int VPT = kAttnKeysPerTile * D / 8 / 256;   // 16-byte vectors per thread per tile and matrix
+	constexpr int VPR = D / 8;                      // vectors per row
+
+	const int tid = threadIdx.x;
+	const int lane = tid & (kWaveSize - 1);
+	const int wave = tid >> 6;
+	const int n = lane & 15;                        // query inside a 16-block (second MFMA operand index)
+	const int g = lane >> 4;                        // lane group: k slots 8 g .. 8 g + 7 of an MFMA
+	const int bh = blockIdx.y;
+	const int q0 = blockIdx.x * kAttnQueriesPerBlock;
+	const half_t* qp = a.q + (int64_t)bh * a.n_q * D;
+	const half_t* kp = a.k + (int64_t)(bh / a.q_per_kv) * a.n_k * D;
+	const half_t* vp = a.v + (int64_t)(bh / a.q_per_kv) * a.n_k * D;
+	half_t* yp = a.y + (int64_t)bh * a.n_q * D;
+
+	// visible key range of the whole block: from the first key of its first query to the last of its last
+	const int q_last = (q0 + kAttnQueriesPerBlock - 1 < a.n_q ? q0 + kAttnQueriesPerBlock - 1 : a.n_q - 1);
+	int key_hi = a.n_k - 1;
+	if (a.causal && q_last + a.diag < key_hi) key_hi = q_last + a.diag;
+	int key_lo = 0;
+	if (a.window > 0 && q0 + a.diag - a.window + 1 > 0) key_lo = q0 + a.diag - a.window + 1;
+	const int t_first = key_lo / kAttnKeysPerTile;
+	const int t_last = key_hi >= 0 ? key_hi / kAttnKeysPerTile : -1;
+
+	// this wave's queries as second operands: lane (n, g) holds q[row][32 s + 8 g .. + 7]
+	int q_row[2];
+	half8_t qf[2][KS];
+#pragma unroll
+	for (int b = 0; b < 2; ++b)
+	{
+		q_row[b] = q0 + 32 * wave + 16 * b + n;
+#pragma unroll
+		for (int s = 0; s < KS; ++s)
+		{
+			half8_t val = {};
+			if (q_row[b] < a.n_q) val = *reinterpret_cast<const half8_t*>(qp + (int64_t)q_row[b] * D + 32 * s + 8 * g);
+			qf[b][s] = val;
+		}
+	}
+	// visible keys of each of the two queries this lane serves: lo <= key <= hi
+	int vis_lo[2], vis_hi[2];
+#pragma unroll
+	for (int b = 0; b < 2; ++b)
+	{
+		vis_hi[b] = a.causal ? q_row[b] + a.diag : a.n_k - 1;
+		if (vis_hi[b] > a.n_k - 1) vis_hi[b] = a.n_k - 1;
+		vis_lo[b] = a.window > 0 ? q_row[b] + a.diag - a.window + 1 : 0;
+	}
+
+	float m_run[2] = { -INFINITY, -INFINITY };
+	float l_run[2] = { 0.0f, 0.0f };               // this lane's share of the row sum
+	float4_t o[2][DC];
+#pragma unroll
+	for (int b = 0; b < 2; ++b)
+#pragma unroll
+		for (int c = 0; c < DC; ++c) o[b][c] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+
+	float4_t kr[VPT], vr[VPT];
+	auto tile_load = [&](int t) {
+#pragma unroll
+		for (int i = 0; i < VPT; ++i)
+		{
+			const int idx = tid + 256 * i;
+			const int row = idx / VPR, col = idx % VPR;
+			const int key = t * kAttnKeysPerTile + row;
+			float4_t kv = {}, vv = {};
+			if (key < a.n_k)
+			{
+				kv = *reinterpret_cast<const float4_t*>(kp + (int64_t)key * D + col * 8);
+				vv = *reinterpret_cast<const float4_t*>(vp + (int64_t)key * D + col * 8);
+			}
+			kr[i] = kv;
+			vr[i] = vv;
+		}
+	};
+	auto tile_store = [&]() {
+#pragma unroll
+		for (int i = 0; i < VPT; ++i)
+		{
+			const int idx = tid + 256 * i;
+			const int row = idx / VPR, col = idx % VPR;
+			*reinterpret_cast<float4_t*>(k_lds + row * L::kPitchK + col * 16) = kr[i];
+			*reinterpret_cast<float4_t*>(v_lds + row * L::kPitchV + col * 16) = vr[i];
+		}
+	};
+
+	if (t_first <= t_last) tile_load(t_first);
+	for (int t = t_first; t <= t_last; ++t)
+	{
+		__syncthreads();                           // the previous tile has been read by everybody
+		tile_store();
+		__syncthreads();
+		if (t < t_last) tile_load(t + 1);          // in flight while this tile is used
+
+		// ---- S^T = K Q^T: s[b][kb] = scores of query block b against key block kb ----
+		float4_t s[2][4];
+#pragma unroll
+		for (int b = 0; b < 2; ++b)
+#pragma unroll
+			for (int kb = 0; kb < 4; ++kb) s[b][kb] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+		for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+			for (int st = 0; st < KS; ++st)
+			{
+				const half8_t kf = *reinterpret_cast<const half8_t*>(k_lds + (16 * kb + n) * L::kPitchK + (32 * st + 8 * g) * 2);
+#pragma unroll
+				for (int b = 0; b < 2; ++b)
+					s[b][kb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf, qf[b][st], s[b][kb], 0, 0, 0);
+			}
+
+		// ---- online softmax; p as the second operand of the next product ----
+		half8_t pf[2][2];
+#pragma unroll
+		for (int b = 0; b < 2; ++b)
+		{
+			float z[4][4];
+			float mt = -INFINITY;
+#pragma unroll
+			for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+				for (int r = 0; r < 4; ++r)
+				{
+					const int key = t * kAttnKeysPerTile + 16 * kb + 4 * g + r;
+					const float zz = logit2<SOFTCAP>(s[b][kb][r], a.k_in, a.k_cap);
+					z[kb][r] = (key >= vis_lo[b] && key <= vis_hi[b]) ? zz : -INFINITY;
+					mt = fmaxf(mt, z[kb][r]);
+				}
+			mt = fmaxf(mt, __shfl_xor(mt, 16));
+			mt = fmaxf(mt, __shfl_xor(mt, 32));
+			const float m_new = fmaxf(m_run[b], mt);
+			const float m_safe = (m_new == -INFINITY) ? 0.0f : m_new;   // nothing visible so far: every term is exp2(-inf) = 0
+			const float corr = fast_exp2(m_run[b] - m_safe);
+			float psum = 0.0f;
+			float p[4][4];
+#pragma unroll
+			for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+				for (int r = 0; r < 4; ++r)
+				{
+					p[kb][r] = fast_exp2(z[kb][r] - m_safe);
+					psum += p[kb][r];
+				}
+			l_run[b] = l_run[b] * corr + psum;
+			m_run[b] = m_new;
+#pragma unroll
+			for (int c = 0; c < DC; ++c) o[b][c] *= corr;
+#pragma unroll
+			for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+				for (int j = 0; j < 8; ++j) pf[b][tt][j] = (half_t)p[2 * tt + j / 4][j % 4];
+		}
+
+		// ---- O^T += V^T P^T ----
+#pragma unroll
+		for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+			for (int c = 0; c < DC; ++c)
+			{
+				const char* src = v_lds + (32 * tt + 4 * g + (n >> 2)) * L::kPitchV + (16 * c + 4 * (n & 3)) * 2;
+				const half4_t lo = lds_read_tr_b64(src);
+				const half4_t hi = lds_read_tr_b64(src + 16 * L::kPitchV);
+				const half8_t vf = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+#pragma unroll
+				for (int b = 0; b < 2; ++b)
+					o[b][c] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf, pf[b][tt], o[b][c], 0, 0, 0);
+			}
+	}
+
+	// ---- normalise and store: lane (n, g) holds y[row][16 c + 4 g .. + 3] ----
+#pragma unroll
+	for (int b = 0; b < 2; ++b)
+	{
+		float l = l_run[b];
+		l += __shfl_xor(l, 16);
+		l += __shfl_xor(l, 32);
+		const float inv = l > 0.0f ? 1.0f / l : 0.0f;
+		if (q_row[b] < a.n_q)
+		{
+#pragma unroll
+			for (int c = 0; c < DC; ++c)
+			{
+				half4_t out;
+#pragma unroll
+				for (int r = 0; r < 4; ++r) out[r] = (half_t)(o[b][c][r] * inv);
+				*reinterpret_cast<half4_t*>(yp + (int64_t)q_row[b] * D + 16 * c + 4 * g) = out;
+			}
+		}
+	}
+}
+
+template <int D, bool SOFTCAP>
+hipError_t launch_variant(const AttnArgs& args, int64_t batch_heads, hipStream_t stream)
+{
+	auto kernel = sdp_attention_fwd_f16_kernel<D, SOFTCAP>;
+	constexpr int kLdsBytes = AttnLds<D>::kBytes;
+	(void)hipGetLastError();
+	if (kLdsBytes > 64 * 1024)
+	{
+		// more than 64 KB of dynamic LDS has to be granted per function and per device, once
+		static std::atomic<uint64_t> configured_devices{0};
+		int device = 0;
+		hipError_t e = hipGetDevice(&device);
+		if (e != hipSuccess) return e;
+		const uint64_t bit = 1ull << (device & 63);
+		if ((configured_devices.load(std::memory_order_relaxed) & bit) == 0)
+		{
+			e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+			if (e != hipSuccess) return e;
+			configured_devices.fetch_or(bit, std::memory_order_relaxed);
+		}
+	}
+	const dim3 grid((unsigned)((args.n_q + kAttnQueriesPerBlock - 1) / kAttnQueriesPerBlock), (unsigned)batch_heads);
+	kernel<<<grid, dim3(256), kLdsBytes, stream>>>(args);
+	return hipGetLastError();
+}
+
+template <int D>
+hipError_t launch_dim(const AttnArgs& args, bool softcap, int64_t batch_heads, hipStream_t stream)
+{
+	return softcap ? launch_variant<D, true>(args, batch_heads, stream) : launch_variant<D, false>(args, batch_heads, stream);
+}
+
+}  // namespace
+
+bool sdp_attention_fwd_f16_supports(int64_t head_dim)
+{
+	return head_dim == 64 || head_dim == 128 || head_dim == 256;
+}
+
+hipError_t launch_sdp_attention_fwd_f16(const void* q, const void* k, const void* v, void* y,
+                                        int64_t batch_heads, int64_t q_per_kv, int64_t n_q, int64_t n_k, int64_t head_dim,
+                                        float alpha, float softcap, int causal, int64_t window, hipStream_t stream)
+{
+	if (batch_heads == 0 || n_q == 0) return hipSuccess;
+	AttnArgs args;
+	args.q = static_cast<const half_t*>(q);
+	args.k = static_cast<const half_t*>(k);
+	args.v = static_cast<const half_t*>(v);
+	args.y = static_cast<half_t*>(y);
+	args.n_q = (int)n_q;
+	args.n_k = (int)n_k;
+	args.q_per_kv = (int)q_per_kv;
+	args.diag = (int)(n_k - n_q);
+	args.causal = causal ? 1 : 0;
+	args.window = (int)window;
+	const bool capped = softcap != 0.0f;
+	args.k_in = capped ? 2.0f * kLog2e * alpha / softcap : alpha * kLog2e;
+	args.k_cap = capped ? softcap * kLog2e : 0.0f;
+	switch (head_dim)
+	{
+	case 64: return launch_dim<64>(args, capped, batch_heads, stream);
+	case 128: return launch_dim<128>(args, capped, batch_heads, stream);
+	default: return launch_dim<256>(args, capped, batch_heads, stream);
+	}
+}
+
+}  // namespace anygpu

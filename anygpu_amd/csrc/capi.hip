@@ -252,6 +252,27 @@ ANYGPU_EXPORT int anygpu_softmax_rows_masked_f32(const float* x, const float* ma
 	                                   q_len, alpha, softcap, stream);
 }
 
+ANYGPU_EXPORT int anygpu_sdp_attention_fwd_f16(const void* q, const void* k, const void* v, void* y,
+                                               int64_t batch_heads, int64_t q_per_kv, int64_t n_q, int64_t n_k, int64_t head_dim,
+                                               float alpha, float softcap, int causal, int64_t window, void* stream)
+{
+	if (batch_heads < 0 || n_q < 0 || n_k < 0 || head_dim < 0 || window < 0) return ANYGPU_ERR_BAD_SHAPE;
+	if (q_per_kv < 1 || batch_heads % q_per_kv != 0) return ANYGPU_ERR_BAD_SHAPE;
+	if (!anygpu::sdp_attention_fwd_f16_supports(head_dim)) return ANYGPU_ERR_UNSUPPORTED;
+	if (!(softcap >= 0.0f) || !std::isfinite(softcap) || !std::isfinite(alpha)) return ANYGPU_ERR_UNSUPPORTED;
+	if (batch_heads == 0 || n_q == 0) return ANYGPU_OK;
+	if (q == nullptr || y == nullptr) return ANYGPU_ERR_NULL_POINTER;
+	if (n_k > 0 && (k == nullptr || v == nullptr)) return ANYGPU_ERR_NULL_POINTER;
+	if (batch_heads > 65535) return ANYGPU_ERR_TOO_LARGE;                        // one grid row per head
+	// query and key indices, their sums and differences with the window stay inside 32 bits
+	if (n_q > kMaxIndex32 / 4 || n_k > kMaxIndex32 / 4 || window > kMaxIndex32 / 4) return ANYGPU_ERR_TOO_LARGE;
+	const uintptr_t bits = reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) | reinterpret_cast<uintptr_t>(v) |
+	                       reinterpret_cast<uintptr_t>(y);
+	if (bits % 16 != 0) return ANYGPU_ERR_UNSUPPORTED;
+	return (int)anygpu::launch_sdp_attention_fwd_f16(q, k, v, y, batch_heads, q_per_kv, n_q, n_k, head_dim, alpha, softcap,
+	                                                 causal, window, as_stream(stream));
+}
+
 ANYGPU_EXPORT int anygpu_causal_conv1d_silu_f16(const void* x, const void* w, const void* bias, void* y,
                                                 int64_t batch, int64_t chan, int64_t seqlen, int64_t width,
                                                 void* stream)

@@ -54,6 +54,13 @@ hipError_t launch_gemm_f32_gelu_mul(const float* A, const float* B_gate, const f
                                     int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc,
                                     int b_layout, hipStream_t stream);
 
+// Fused attention forward, fp16: q [batch_heads, n_q, head_dim], k and v [batch_heads / q_per_kv, n_k, head_dim],
+// y like q; mask rules as in launch_softmax_rows with the diagonal at n_k - n_q.
+bool sdp_attention_fwd_f16_supports(int64_t head_dim);
+hipError_t launch_sdp_attention_fwd_f16(const void* q, const void* k, const void* v, void* y,
+                                        int64_t batch_heads, int64_t q_per_kv, int64_t n_q, int64_t n_k, int64_t head_dim,
+                                        float alpha, float softcap, int causal, int64_t window, hipStream_t stream);
+
 // Few-row products (M <= kSkinnyMaxRows, one product, row-major A): bandwidth-shaped kernels that
 // stream B once.  `epilogue` is an Epilogue value; B2 only for kEpiGeluMul, bias only for kEpiBias
 // (either may be NULL).  T is float or _Float16.  gemm_skinny_applies says whether shape, leading

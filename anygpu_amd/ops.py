@@ -293,3 +293,25 @@ def sdp_attention_masked_scaled_fwd(qw: torch.Tensor, kw: torch.Tensor, vw: torc
     probs = tensor_softmax_masked(scores.reshape(-1, n_k), mask.reshape(n_q, n_k).contiguous(), alpha=alpha, q_len=n_q)
     out = tensor_mm_batched(probs.reshape(-1, n_q, n_k), v3.contiguous())
     return out.reshape(*lead, n_q, d_v)
+
+
+def sdp_attention_fwd(qw: torch.Tensor, kw: torch.Tensor, vw: torch.Tensor, alpha: float, *, softcap: float = 0.0,
+                      causal: bool = False, window: int = 0) -> torch.Tensor:
+    """softmax(mask(softcap(alpha q k^T))) v in one kernel; q [..., heads, n_q, d], k and v [..., kv_heads, n_k, d]
+    with heads a multiple of kv_heads, float16; masks are index rules with the causal diagonal at n_k - n_q."""
+    _check_device(qw, kw, vw)
+    _require(qw.dim() == kw.dim() == vw.dim() and qw.dim() >= 3, "dimension missmatch")
+    _require(qw.dtype == kw.dtype == vw.dtype == torch.float16, "Unsupported data types")
+    _require(tuple(kw.shape) == tuple(vw.shape) and kw.shape[-1] == qw.shape[-1], "q, k and v need one head dimension")
+    _require(qw.shape[:-3] == kw.shape[:-3] and kw.shape[-3] > 0 and qw.shape[-3] % kw.shape[-3] == 0,
+             "query heads need to be a multiple of key / value heads")
+    _require(qw.is_contiguous() and kw.is_contiguous() and vw.is_contiguous(), "dense operands expected")
+    heads, n_q, d = qw.shape[-3:]
+    kv_heads, n_k = kw.shape[-3], kw.shape[-2]
+    batch_heads = qw.numel() // (n_q * d) if n_q * d else 0
+    out = torch.empty_like(qw)
+    rc = capi.load().anygpu_sdp_attention_fwd_f16(qw.data_ptr(), kw.data_ptr(), vw.data_ptr(), out.data_ptr(),
+                                                  batch_heads, heads // kv_heads, n_q, n_k, d, float(alpha),
+                                                  float(softcap), int(causal), int(window), _stream_ptr())
+    capi.check("anygpu_sdp_attention_fwd_f16", rc)
+    return out

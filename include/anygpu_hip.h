@@ -165,6 +165,24 @@ int anygpu_softmax_rows_masked_f32(const float* x, const float* mask, float* y,
                                    int64_t q_len, float alpha, float softcap, void* stream);
 
 /*
+ * Scaled-dot-product attention, forward, in one kernel (the score matrix stays on chip):
+ *     y[h] = softmax( mask( softcap( alpha * q[h] k[h / q_per_kv]^T ) ) ) v[h / q_per_kv]
+ * q and y are [batch_heads, n_q, head_dim], k and v [batch_heads / q_per_kv, n_k, head_dim] (q_per_kv query
+ * heads share one key / value head; 1 for ordinary multi-head attention), all fp16 and densely packed;
+ * fp32 scores, sums and output accumulators.  The prologue steps and their order are those of
+ * anygpu_softmax_rows_f16 with q_len = n_q and diag = n_k - n_q (the last query sees the last key):
+ * causal != 0 hides key j from query i when j > i + diag, window > 0 also when j <= i + diag - window.
+ * A query without a visible key gets zeros.  head_dim must be 64, 128 or 256, pointers 16-byte aligned.
+ * Replaces the per-head loop of sdp_attention_masked_scaled_fwd (srcs/transformers/sdp.hpp:258-271: transpose,
+ * tensor_mm, tensor_mul, tensor_add, tensor_softmax, tensor_mm per head) for masks that are index rules, and
+ * is the half-precision counterpart of cu_flash_sdpa_fwd_d256_v1 (srcs/kernels/cuda/flash_sdpa_fwd.cuh:6-15,
+ * fp32, head_dim 256, no mask).
+ */
+int anygpu_sdp_attention_fwd_f16(const void* q, const void* k, const void* v, void* y,
+                                 int64_t batch_heads, int64_t q_per_kv, int64_t n_q, int64_t n_k, int64_t head_dim,
+                                 float alpha, float softcap, int causal, int64_t window, void* stream);
+
+/*
  * Depthwise causal conv1d with bias and fused SiLU:
  *     y[b, d, s] = silu( bias[d] + sum_{k=0}^{width-1} w[d, k] * x[b, d, s + k - (width - 1)] ),
  * terms with a negative sequence index dropped (left zero padding of width-1).

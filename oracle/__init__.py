@@ -288,6 +288,31 @@ def sdp_attention_masked_scaled_fwd(q: np.ndarray, k: np.ndarray, v: np.ndarray,
     return y
 
 
+def sdp_attention_rules(q: np.ndarray, k: np.ndarray, v: np.ndarray, *, alpha: float, softcap: float = 0.0,
+                        causal: bool = False, window: int = 0, q_per_kv: int = 1,
+                        query_index: np.ndarray | None = None, threads: int = 1) -> np.ndarray:
+    """softmax(mask(softcap(alpha q k^T))) v with masks given as index rules, composed per head from tensor_mm,
+    attention_softmax and tensor_mm in the call order of srcs/transformers/sdp.hpp:258-271.  q [heads, n_q, d],
+    k and v [heads / q_per_kv, n_k, d]; the causal diagonal sits at n_k - n_q.  With `query_index` only those
+    queries of every head are evaluated (result [heads, len(query_index), d])."""
+    q, k, v = (np.ascontiguousarray(t, dtype=np.float32) for t in (q, k, v))
+    heads, n_q, d = q.shape
+    n_k = k.shape[1]
+    assert k.shape == v.shape and k.shape[0] * q_per_kv == heads and k.shape[2] == d
+    idx = np.arange(n_q, dtype=np.int64) if query_index is None else np.ascontiguousarray(query_index, dtype=np.int64)
+    out = np.zeros((heads, idx.size, d), dtype=np.float32)
+    for h in range(heads):
+        kh, vh = k[h // q_per_kv], v[h // q_per_kv]
+        qk = tensor_mm(q[h][idx], kh.T, threads=threads)
+        # row r of qk is query idx[r]: hand the softmax one-row matrices' worth of indices through q_len / diag
+        p = np.empty_like(qk)
+        for r, i in enumerate(idx):
+            p[r] = attention_softmax(qk[r:r + 1], alpha=alpha, softcap=softcap, causal=causal, window=window,
+                                     q_len=0, diag=int(i) + (n_k - n_q))[0]
+        out[h] = tensor_mm(p, vh, threads=threads)
+    return out
+
+
 def tensor_causal_conv1d(xt: np.ndarray, wt: np.ndarray, bt: np.ndarray, rows: tuple[int, int] | None = None,
                          threads: int = 1) -> np.ndarray:
     assert xt.ndim == 3, "xt needs to be 3 dimensional"

@@ -731,6 +731,89 @@ def test_sdp_attention_masked_scaled_fwd(ops, oracle):
     assert scaled_rel_err(got, want, 1.0) <= TOL_F16_GEMM
 
 
+ATTN_CASES = [
+    # heads, kv_heads, n_q, n_k, d, alpha, softcap, causal, window
+    (2, 2, 16, 16, 64, 0.125, 0.0, False, 0),
+    (3, 3, 100, 100, 64, 0.125, 0.0, True, 0),
+    (4, 2, 130, 130, 128, 0.0884, 0.0, True, 0),
+    (2, 1, 257, 257, 256, 0.0625, 50.0, True, 96),
+    (2, 2, 64, 200, 128, 0.0884, 0.0, True, 0),          # queries are the last 64 positions of a 200-key cache
+    (2, 2, 1, 300, 128, 0.0884, 30.0, True, 128),        # decode step
+    (1, 1, 200, 77, 64, 0.125, 0.0, False, 0),
+    (2, 2, 192, 192, 64, 0.125, 0.0, False, 40),         # window without the causal rule
+]
+
+
+@pytest.mark.parametrize("case", ATTN_CASES)
+def test_sdp_attention_fused_kernel(ops, oracle, case):
+    heads, kv_heads, n_q, n_k, d, alpha, cap, causal, window = case
+    q = synth.normal(1 + n_q, (1, heads, n_q, d)).astype(np.float16)
+    k = synth.normal(2 + n_k, (1, kv_heads, n_k, d)).astype(np.float16)
+    v = synth.normal(3 + d, (1, kv_heads, n_k, d)).astype(np.float16)
+    got = host(ops.sdp_attention_fwd(dev(q), dev(k), dev(v), alpha, softcap=cap, causal=causal, window=window)).astype(np.float32)
+    want = oracle.sdp_attention_rules(*(oracle.cvt_f16_to_f32(t)[0] for t in (q, k, v)), alpha=alpha, softcap=cap,
+                                      causal=causal, window=window, q_per_kv=heads // kv_heads, threads=8)
+    assert got.shape == (1, heads, n_q, d)
+    # outputs are convex combinations of N(0, 1) values: scale floor 1
+    assert scaled_rel_err(got[0], want, 1.0) <= TOL_F16_ROWOPS * 2          # p is rounded to fp16 before the second product
+    assert rel_l2(got[0], want) <= 2e-3
+
+
+def test_sdp_attention_fused_kernel_structure(ops, oracle):
+    import torch
+    # first causal row attends to key 0 only: y[0] = v[0] exactly; a changed future key changes nothing before it
+    heads, n, d = 2, 160, 128
+    q, k, v = (synth.normal(s, (heads, n, d)).astype(np.float16) for s in (1, 2, 3))
+    y = host(ops.sdp_attention_fwd(dev(q), dev(k), dev(v), 0.0884, causal=True))
+    assert np.array_equal(y[:, 0, :], v[:, 0, :])
+    k2, v2 = k.copy(), v.copy()
+    k2[:, 100:, :] += np.float16(1.0)
+    v2[:, 100:, :] -= np.float16(2.0)
+    y2 = host(ops.sdp_attention_fwd(dev(q), dev(k2), dev(v2), 0.0884, causal=True))
+    assert np.array_equal(y[:, :100, :], y2[:, :100, :])
+    assert not np.array_equal(y[:, 100:, :], y2[:, 100:, :])
+    # constant v: every output equals that constant whatever the scores are
+    vc = np.full_like(v, 0.5)
+    yc = host(ops.sdp_attention_fwd(dev(q), dev(k), dev(vc), 0.0884, softcap=20.0, causal=True, window=33))
+    assert np.max(np.abs(yc.astype(np.float32) - 0.5)) <= 1e-3
+    # more queries than keys with the causal rule: the first n_q - n_k queries see nothing and get zeros
+    ys = host(ops.sdp_attention_fwd(dev(q), dev(k[:, :60]), dev(v[:, :60]), 0.0884, causal=True))
+    assert not ys[:, :100, :].any() and ys[:, 100:, :].any()
+    # against the three-launch form with the mask as data
+    mask = oracle.slide_mask(oracle.causal_mask(n, n), 48).reshape(1, n, n)
+    with np.errstate(over="ignore"):
+        mask16 = mask.astype(np.float16)
+    three = host(ops.sdp_attention_masked_scaled_fwd(dev(q), dev(k), dev(v), dev(mask16), 0.0884)).astype(np.float32)
+    fused = host(ops.sdp_attention_fwd(dev(q), dev(k), dev(v), 0.0884, causal=True, window=48)).astype(np.float32)
+    assert scaled_rel_err(fused, three, 1.0) <= TOL_F16_ROWOPS * 2
+    # rejected arguments launch nothing
+    from anygpu_amd import capi
+    lib = capi.load()
+    t = torch.zeros((2, 16, 96), device="cuda", dtype=torch.float16)
+    out = torch.full_like(t, 3.0)
+    f = lib.anygpu_sdp_attention_fwd_f16
+    assert f(t.data_ptr(), t.data_ptr(), t.data_ptr(), out.data_ptr(), 2, 1, 16, 16, 96, 0.1, 0.0, 1, 0, None) == capi.ANYGPU_ERR_UNSUPPORTED
+    assert f(t.data_ptr(), t.data_ptr(), t.data_ptr(), out.data_ptr(), 3, 2, 16, 16, 64, 0.1, 0.0, 1, 0, None) == capi.ANYGPU_ERR_BAD_SHAPE
+    assert f(t.data_ptr(), None, t.data_ptr(), out.data_ptr(), 2, 1, 16, 16, 64, 0.1, 0.0, 1, 0, None) == capi.ANYGPU_ERR_NULL_POINTER
+    torch.cuda.synchronize()
+    assert bool((out == 3.0).all())
+
+
+def test_sdp_attention_fused_kernel_gemma2_block(ops, oracle):
+    # Gemma2 attention at the softmax configuration of the headline set: 8 query heads over 4 key / value heads,
+    # head_dim 256, scale 1 / 16, softcap 50, causal + window 4096; 6144 positions so that the window cuts
+    h, hkv, n, d = 8, 4, 6144, 256
+    q = synth.normal(1, (h, n, d)).astype(np.float16)
+    k = synth.normal(2, (hkv, n, d)).astype(np.float16)
+    v = synth.normal(3, (hkv, n, d)).astype(np.float16)
+    got = host(ops.sdp_attention_fwd(dev(q), dev(k), dev(v), 0.0625, softcap=50.0, causal=True, window=4096)).astype(np.float32)
+    idx = np.array([0, 1, 63, 64, 127, 128, 1000, 4095, 4096, 4097, 5000, 6143], dtype=np.int64)
+    want = oracle.sdp_attention_rules(*(oracle.cvt_f16_to_f32(t) for t in (q, k, v)), alpha=0.0625, softcap=50.0,
+                                      causal=True, window=4096, q_per_kv=2, query_index=idx, threads=8)
+    assert scaled_rel_err(got[:, idx, :], want, 1.0) <= TOL_F16_ROWOPS * 2
+    assert np.isfinite(got).all()
+
+
 # =============================================================================================
 # committed golden fixtures (tests/golden/*.dat)
 # =============================================================================================
