@@ -4,8 +4,9 @@
 // three-launch form (q k^T, row softmax, p v) writes and reads 1 GiB of scores twice; this kernel
 // reads q, k, v and writes y.
 //
-// A block of 4 waves owns 128 consecutive queries of one head, a wave 32 of them (two blocks of
-// 16).  It walks the visible key range in tiles of 64 keys.  Per tile:
+// A block owns 128 consecutive queries of one head: 8 waves with 16 queries each (or 4 waves with
+// 32), so that two waves share a SIMD and one wave's MFMAs run under the other's softmax
+// arithmetic.  It walks the visible key range in tiles of 64 keys.  Per tile:
 //   * K and V rows go global -> registers -> LDS (the loads of the next tile are in flight
 //     while this one is being used);
 //   * S^T = K Q^T with v_mfma_f32_16x16x32_f16: the K fragment is the first operand, the Q
@@ -82,16 +83,19 @@ struct AttnLds
 	static constexpr int kBytes = kAttnKeysPerTile * (kPitchK + kPitchV);
 };
 
-template <int D, bool SOFTCAP>
-__global__ __launch_bounds__(256) void sdp_attention_fwd_f16_kernel(const AttnArgs a)
+// QB: 16-query blocks per wave, WAVES: waves per block; QB * WAVES = 8.
+template <int D, bool SOFTCAP, int QB, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f16_kernel(const AttnArgs a)
 {
+	static_assert(16 * QB * WAVES == kAttnQueriesPerBlock, "a block owns 128 queries");
+	constexpr int THREADS = 64 * WAVES;
 	extern __shared__ __align__(16) char lds[];
 	using L = AttnLds<D>;
 	char* k_lds = lds;
 	char* v_lds = lds + kAttnKeysPerTile * L::kPitchK;
 	constexpr int KS = D / 32;                      // MFMA steps along the head dimension (q k^T)
 	constexpr int DC = D / 16;                      // 16-wide column blocks of the output
-	constexpr int VPT = kAttnKeysPerTile * D / 8 / 256;   // 16-byte vectors per thread per tile and matrix
+	constexpr int VPT = kAttnKeysPerTile * D / 8 / THREADS;   // 16-byte vectors per thread per tile and matrix
 	constexpr int VPR = D / 8;                      // vectors per row
 
 	const int tid = threadIdx.x;
@@ -100,7 +104,8 @@ __global__ __launch_bounds__(256) void sdp_attention_fwd_f16_kernel(const AttnAr
 	const int n = lane & 15;                        // query inside a 16-block (second MFMA operand index)
 	const int g = lane >> 4;                        // lane group: k slots 8 g .. 8 g + 7 of an MFMA
 	const int bh = blockIdx.y;
-	const int q0 = blockIdx.x * kAttnQueriesPerBlock;
+	// under the causal rule the last query blocks have the most keys to walk: they are dispatched first
+	const int q0 = (int)(gridDim.x - 1 - blockIdx.x) * kAttnQueriesPerBlock;
 	const half_t* qp = a.q + (int64_t)bh * a.n_q * D;
 	const half_t* kp = a.k + (int64_t)(bh / a.q_per_kv) * a.n_k * D;
 	const half_t* vp = a.v + (int64_t)(bh / a.q_per_kv) * a.n_k * D;
@@ -116,12 +121,12 @@ __global__ __launch_bounds__(256) void sdp_attention_fwd_f16_kernel(const AttnAr
 	const int t_last = key_hi >= 0 ? key_hi / kAttnKeysPerTile : -1;
 
 	// this wave's queries as second operands: lane (n, g) holds q[row][32 s + 8 g .. + 7]
-	int q_row[2];
-	half8_t qf[2][KS];
+	int q_row[QB];
+	half8_t qf[QB][KS];
 #pragma unroll
-	for (int b = 0; b < 2; ++b)
+	for (int b = 0; b < QB; ++b)
 	{
-		q_row[b] = q0 + 32 * wave + 16 * b + n;
+		q_row[b] = q0 + 16 * QB * wave + 16 * b + n;
 #pragma unroll
 		for (int s = 0; s < KS; ++s)
 		{
@@ -131,29 +136,36 @@ __global__ __launch_bounds__(256) void sdp_attention_fwd_f16_kernel(const AttnAr
 		}
 	}
 	// visible keys of each of the two queries this lane serves: lo <= key <= hi
-	int vis_lo[2], vis_hi[2];
+	int vis_lo[QB], vis_hi[QB];
 #pragma unroll
-	for (int b = 0; b < 2; ++b)
+	for (int b = 0; b < QB; ++b)
 	{
 		vis_hi[b] = a.causal ? q_row[b] + a.diag : a.n_k - 1;
 		if (vis_hi[b] > a.n_k - 1) vis_hi[b] = a.n_k - 1;
 		vis_lo[b] = a.window > 0 ? q_row[b] + a.diag - a.window + 1 : 0;
 	}
 
-	float m_run[2] = { -INFINITY, -INFINITY };
-	float l_run[2] = { 0.0f, 0.0f };               // this lane's share of the row sum
-	float4_t o[2][DC];
+	float m_run[QB], l_run[QB];                    // l_run: this lane's share of the row sum
+	float4_t o[QB][DC];
 #pragma unroll
-	for (int b = 0; b < 2; ++b)
+	for (int b = 0; b < QB; ++b)
+	{
+		m_run[b] = -INFINITY;
+		l_run[b] = 0.0f;
 #pragma unroll
 		for (int c = 0; c < DC; ++c) o[b][c] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+	}
+	// keys visible to every query of this wave need no per-element test: [all_lo, all_hi]
+	const int wq0 = q0 + 16 * QB * wave, wq1 = wq0 + 16 * QB - 1;
+	const int all_hi = a.causal ? (wq0 + a.diag < a.n_k - 1 ? wq0 + a.diag : a.n_k - 1) : a.n_k - 1;
+	const int all_lo = a.window > 0 ? wq1 + a.diag - a.window + 1 : 0;
 
 	float4_t kr[VPT], vr[VPT];
 	auto tile_load = [&](int t) {
 #pragma unroll
 		for (int i = 0; i < VPT; ++i)
 		{
-			const int idx = tid + 256 * i;
+			const int idx = tid + THREADS * i;
 			const int row = idx / VPR, col = idx % VPR;
 			const int key = t * kAttnKeysPerTile + row;
 			float4_t kv = {}, vv = {};
@@ -170,7 +182,7 @@ __global__ __launch_bounds__(256) void sdp_attention_fwd_f16_kernel(const AttnAr
 #pragma unroll
 		for (int i = 0; i < VPT; ++i)
 		{
-			const int idx = tid + 256 * i;
+			const int idx = tid + THREADS * i;
 			const int row = idx / VPR, col = idx % VPR;
 			*reinterpret_cast<float4_t*>(k_lds + row * L::kPitchK + col * 16) = kr[i];
 			*reinterpret_cast<float4_t*>(v_lds + row * L::kPitchV + col * 16) = vr[i];
@@ -186,9 +198,9 @@ __global__ __launch_bounds__(256) void sdp_attention_fwd_f16_kernel(const AttnAr
 		if (t < t_last) tile_load(t + 1);          // in flight while this tile is used
 
 		// ---- S^T = K Q^T: s[b][kb] = scores of query block b against key block kb ----
-		float4_t s[2][4];
+		float4_t s[QB][4];
 #pragma unroll
-		for (int b = 0; b < 2; ++b)
+		for (int b = 0; b < QB; ++b)
 #pragma unroll
 			for (int kb = 0; kb < 4; ++kb) s[b][kb] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
@@ -198,32 +210,47 @@ __global__ __launch_bounds__(256) void sdp_attention_fwd_f16_kernel(const AttnAr
 			{
 				const half8_t kf = *reinterpret_cast<const half8_t*>(k_lds + (16 * kb + n) * L::kPitchK + (32 * st + 8 * g) * 2);
 #pragma unroll
-				for (int b = 0; b < 2; ++b)
+				for (int b = 0; b < QB; ++b)
 					s[b][kb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf, qf[b][st], s[b][kb], 0, 0, 0);
 			}
 
 		// ---- online softmax; p as the second operand of the next product ----
-		half8_t pf[2][2];
+		half8_t pf[QB][2];
+		const int tile_key0 = t * kAttnKeysPerTile;
+		const bool interior = tile_key0 >= all_lo && tile_key0 + kAttnKeysPerTile - 1 <= all_hi;   // wave-uniform
 #pragma unroll
-		for (int b = 0; b < 2; ++b)
+		for (int b = 0; b < QB; ++b)
 		{
 			float z[4][4];
 			float mt = -INFINITY;
+			if (interior)
+			{
 #pragma unroll
-			for (int kb = 0; kb < 4; ++kb)
+				for (int kb = 0; kb < 4; ++kb)
 #pragma unroll
-				for (int r = 0; r < 4; ++r)
-				{
-					const int key = t * kAttnKeysPerTile + 16 * kb + 4 * g + r;
-					const float zz = logit2<SOFTCAP>(s[b][kb][r], a.k_in, a.k_cap);
-					z[kb][r] = (key >= vis_lo[b] && key <= vis_hi[b]) ? zz : -INFINITY;
-					mt = fmaxf(mt, z[kb][r]);
-				}
+					for (int r = 0; r < 4; ++r)
+					{
+						z[kb][r] = logit2<SOFTCAP>(s[b][kb][r], a.k_in, a.k_cap);
+						mt = fmaxf(mt, z[kb][r]);
+					}
+			}
+			else
+			{
+#pragma unroll
+				for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+					for (int r = 0; r < 4; ++r)
+					{
+						const int key = tile_key0 + 16 * kb + 4 * g + r;
+						const float zz = logit2<SOFTCAP>(s[b][kb][r], a.k_in, a.k_cap);
+						z[kb][r] = (key >= vis_lo[b] && key <= vis_hi[b]) ? zz : -INFINITY;
+						mt = fmaxf(mt, z[kb][r]);
+					}
+			}
 			mt = fmaxf(mt, __shfl_xor(mt, 16));
 			mt = fmaxf(mt, __shfl_xor(mt, 32));
 			const float m_new = fmaxf(m_run[b], mt);
 			const float m_safe = (m_new == -INFINITY) ? 0.0f : m_new;   // nothing visible so far: every term is exp2(-inf) = 0
-			const float corr = fast_exp2(m_run[b] - m_safe);
 			float psum = 0.0f;
 			float p[4][4];
 #pragma unroll
@@ -234,10 +261,17 @@ __global__ __launch_bounds__(256) void sdp_attention_fwd_f16_kernel(const AttnAr
 					p[kb][r] = fast_exp2(z[kb][r] - m_safe);
 					psum += p[kb][r];
 				}
-			l_run[b] = l_run[b] * corr + psum;
-			m_run[b] = m_new;
+			// the running maximum settles after a few tiles; when no query of the wave raised it, the
+			// rescale factor is 1 everywhere and the pass over the accumulators is skipped
+			if (__builtin_amdgcn_ballot_w64(m_new > m_run[b]) != 0)
+			{
+				const float corr = fast_exp2(m_run[b] - m_safe);
+				l_run[b] *= corr;
 #pragma unroll
-			for (int c = 0; c < DC; ++c) o[b][c] *= corr;
+				for (int c = 0; c < DC; ++c) o[b][c] *= corr;
+			}
+			l_run[b] += psum;
+			m_run[b] = m_new;
 #pragma unroll
 			for (int tt = 0; tt < 2; ++tt)
 #pragma unroll
@@ -255,14 +289,14 @@ __global__ __launch_bounds__(256) void sdp_attention_fwd_f16_kernel(const AttnAr
 				const half4_t hi = lds_read_tr_b64(src + 16 * L::kPitchV);
 				const half8_t vf = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
 #pragma unroll
-				for (int b = 0; b < 2; ++b)
+				for (int b = 0; b < QB; ++b)
 					o[b][c] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf, pf[b][tt], o[b][c], 0, 0, 0);
 			}
 	}
 
 	// ---- normalise and store: lane (n, g) holds y[row][16 c + 4 g .. + 3] ----
 #pragma unroll
-	for (int b = 0; b < 2; ++b)
+	for (int b = 0; b < QB; ++b)
 	{
 		float l = l_run[b];
 		l += __shfl_xor(l, 16);
@@ -285,7 +319,10 @@ __global__ __launch_bounds__(256) void sdp_attention_fwd_f16_kernel(const AttnAr
 template <int D, bool SOFTCAP>
 hipError_t launch_variant(const AttnArgs& args, int64_t batch_heads, hipStream_t stream)
 {
-	auto kernel = sdp_attention_fwd_f16_kernel<D, SOFTCAP>;
+	// 8 waves x 16 queries measured 1.1 - 1.5 x faster than 4 waves x 32 queries (16 x 4096 x 128 causal: 173 us
+	// against 266 us): the smaller register footprint lets two blocks share a CU
+	constexpr int QB = 1, WAVES = 8 / QB;
+	auto kernel = sdp_attention_fwd_f16_kernel<D, SOFTCAP, QB, WAVES>;
 	constexpr int kLdsBytes = AttnLds<D>::kBytes;
 	(void)hipGetLastError();
 	if (kLdsBytes > 64 * 1024)
@@ -304,7 +341,7 @@ hipError_t launch_variant(const AttnArgs& args, int64_t batch_heads, hipStream_t
 		}
 	}
 	const dim3 grid((unsigned)((args.n_q + kAttnQueriesPerBlock - 1) / kAttnQueriesPerBlock), (unsigned)batch_heads);
-	kernel<<<grid, dim3(256), kLdsBytes, stream>>>(args);
+	kernel<<<grid, dim3(64 * WAVES), kLdsBytes, stream>>>(args);
 	return hipGetLastError();
 }
 
