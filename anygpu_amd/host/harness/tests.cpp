@@ -40,20 +40,10 @@ Tensor<T, CPU> transposed_copy(const Tensor<T, CPU>& x)
 	return y;
 }
 
-// Additive mask of an attention block on the host: -inf above the (shifted) diagonal, float
-// lowest for keys that fell out of the sliding window.
+// Additive mask of an attention block on the host (the shared helper of the attention callers).
 Tensor<float32, CPU> build_mask(int64 q_len, int64 k_len, bool causal, int64 window, int64 diag)
 {
-	Tensor<float32, CPU> mask(std::vector<int64>({ q_len, k_len }));
-	for (int64 i = 0; i < q_len; ++i)
-		for (int64 j = 0; j < k_len; ++j)
-		{
-			float32 v = 0.f;
-			if (causal && j > i + diag) v = -std::numeric_limits<float32>::infinity();
-			if (window > 0 && (i + diag) >= window && j <= i + diag - window) v = std::numeric_limits<float32>::lowest();
-			mask.buffer()[i * k_len + j] = v;
-		}
-	return mask;
+	return crt_rule_mask<float32>(q_len, k_len, causal, window, diag);
 }
 
 // softcap(x, cap) = tanhf(x / cap) * cap, elementwise on the host
@@ -533,6 +523,46 @@ TEST_CASE(test_gemma2_mlp_fused_upproj_1x37x288_i1152, GPU)
 	auto act1 = tensor_gemma_mlp_fused_uprpoj<float32, CUDA, 1>(dw, dx).copy_to_host();
 	auto act2 = tensor_gemma_mlp_fused_uprpoj<float32, CUDA, 2>(dw, dx).copy_to_host();
 	return elementwise_compatible(exp_hy, act1) && compare_data_buffers(act1, exp_hy) && compare_data_buffers(act2, exp_hy);
+}
+
+TEST_CASE(test_sdp_attention_rules_fused_f16, GPU)
+{
+	// Gemma2-like block: 4 query heads over 2 key / value heads, d = 256, causal + window, 200 queries at the end of
+	// 260 keys; the fused kernel against the operator chain on the host (k and v repeated per query head there)
+	const int64 h = 4, hkv = 2, n_q = 200, n_k = 260, d = 256;
+	auto hq16 = cvt_tensor_from_float32<float16>(crt_random_normal_tensor<float32, CPU>({ 1, h, n_q, d }, 1));
+	auto hk16 = cvt_tensor_from_float32<float16>(crt_random_normal_tensor<float32, CPU>({ 1, hkv, n_k, d }, 2));
+	auto hv16 = cvt_tensor_from_float32<float16>(crt_random_normal_tensor<float32, CPU>({ 1, hkv, n_k, d }, 3));
+	SoftmaxPrologue rules;
+	rules.alpha = 0.0625f;
+	rules.causal = true;
+	rules.window = 96;
+	auto got = cvt_tensor_datatype<float32, float16>(
+		sdp_attention_rules_fwd(hq16.copy_to_cuda(), hk16.copy_to_cuda(), hv16.copy_to_cuda(), rules).copy_to_host());
+	auto hq = cvt_tensor_datatype<float32, float16>(hq16);
+	auto hk = cvt_tensor_datatype<float32, float16>(hk16);
+	auto hv = cvt_tensor_datatype<float32, float16>(hv16);
+	Tensor<float32, CPU> hk_rep(std::vector<int64>({ 1, h, n_k, d })), hv_rep(std::vector<int64>({ 1, h, n_k, d }));
+	for (int64 head = 0; head < h; ++head)
+	{
+		std::memcpy(hk_rep.buffer() + head * n_k * d, hk.buffer() + (head / 2) * n_k * d, n_k * d * sizeof(float32));
+		std::memcpy(hv_rep.buffer() + head * n_k * d, hv.buffer() + (head / 2) * n_k * d, n_k * d * sizeof(float32));
+	}
+	auto want = sdp_attention_rules_fwd(hq, hk_rep, hv_rep, rules);
+	bool ok = elementwise_compatible(got, want) && compare_data_buffers_l2(got, want, 4e-3f) && compare_data_buffers(got, want, 2e-2f);
+	// one matrix through the flash entry point, half precision and float32
+	auto q2 = crt_random_normal_tensor<float32, CPU>({ 96, 128 }, 4);
+	auto k2 = crt_random_normal_tensor<float32, CPU>({ 96, 128 }, 5);
+	auto v2 = crt_random_normal_tensor<float32, CPU>({ 96, 128 }, 6);
+	auto want2 = single_head_attention_fwd(q2, k2, v2);
+	auto got32 = sdp_attention_fwd_cuda_flash(q2.copy_to_cuda(), k2.copy_to_cuda(), v2.copy_to_cuda()).copy_to_host();
+	ok = ok && compare_data_buffers(got32, want2);
+	auto q16 = cvt_tensor_from_float32<float16>(q2), k16 = cvt_tensor_from_float32<float16>(k2), v16 = cvt_tensor_from_float32<float16>(v2);
+	auto want16 = single_head_attention_fwd(cvt_tensor_datatype<float32, float16>(q16), cvt_tensor_datatype<float32, float16>(k16),
+	                                        cvt_tensor_datatype<float32, float16>(v16));
+	auto got16 = cvt_tensor_datatype<float32, float16>(
+		sdp_attention_fwd_cuda_flash(q16.copy_to_cuda(), k16.copy_to_cuda(), v16.copy_to_cuda()).copy_to_host());
+	return ok && compare_data_buffers_l2(got16, want16, 4e-3f);
 }
 
 TEST_CASE(test_gemma2_decoder_mlp_1x21x256_i1024, GPU)

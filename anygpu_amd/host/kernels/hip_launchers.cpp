@@ -6,6 +6,7 @@
 #include "softmax_ops.cuh"
 #include "causal_conv1d.cuh"
 #include "norm_ops.cuh"
+#include "flash_sdpa_fwd.cuh"
 #include "mlp_gemma2_fused_upproj.cuh"
 #include "mlp_gemma2_dp_linear.cuh"
 #include "sdpa_gemma2_linear.cuh"
@@ -331,4 +332,18 @@ void hip_tensor_gated_rms_norm_f16(const Tensor<float16, CUDA>& xt, const Tensor
                                    const float32 eps, const bool zero_centered, Tensor<float16, CUDA>& yt)
 {
 	rms_norm_dispatch(xt, zt, wt, eps, zero_centered, yt);
+}
+
+/* ---- fused attention ---- */
+
+void hip_flash_sdpa_fwd_f16(const SoftmaxPrologue& prologue, const Tensor<float16, CUDA>& qt, const Tensor<float16, CUDA>& kt,
+                            const Tensor<float16, CUDA>& vt, Tensor<float16, CUDA>& yt)
+{
+	const int64 dim = qt.dim;
+	const int64 n_q = qt.shape[dim - 2], d = qt.shape[dim - 1], n_k = kt.shape[dim - 2];
+	const int64 heads = dim >= 3 ? qt.shape[dim - 3] : 1, kv_heads = dim >= 3 ? kt.shape[dim - 3] : 1;
+	const int64 batch_heads = (n_q * d) > 0 ? qt.numel() / (n_q * d) : 0;
+	ABI_CHECK(anygpu_sdp_attention_fwd_f16(qt.buffer(), kt.buffer(), vt.buffer(), yt.buffer(), batch_heads,
+	                                       kv_heads > 0 ? heads / kv_heads : 1, n_q, n_k, d, prologue.alpha, prologue.softcap,
+	                                       prologue.causal ? 1 : 0, prologue.window, kNullStream));
 }

@@ -11,6 +11,7 @@
 
 #include "ops.hpp"
 #include "attention_tools.hpp"
+#include "flash_sdpa_fwd.cuh"
 
 namespace sdp_detail {
 
@@ -120,6 +121,77 @@ inline Tensor<dtype, device> single_head_attention_fwd(
 		SoftmaxPrologue p;
 		p.alpha = static_cast<float32>(alpha);
 		return tensor_mm(tensor_softmax(qk, p), vw);
+	}
+}
+
+/*
+  Single-matrix attention through the fused path (reference: sdp_attention_fwd_cuda_flash, sdp.hpp:48-73, float32,
+  d = 256 only).  Half precision runs the one-kernel form; float32 runs q k^T, softmax with the scale folded in and
+  p v, which is what the reference's float32 kernel computes, for any d.
+*/
+template<FloatingPointType dtype>
+inline Tensor<dtype, CUDA> sdp_attention_fwd_cuda_flash(
+	const Tensor<dtype, CUDA>& qw,
+	const Tensor<dtype, CUDA>& kw,
+	const Tensor<dtype, CUDA>& vw)
+{
+	const int64 N = qw.shape[0], d = qw.shape[1];   // (N, d)
+	ACASSERT(kw.shape[0] == N, "qw and kw differs in sequence length");
+	ACASSERT(vw.shape[0] == N, "qw and vw differs in sequence length");
+	ACASSERT(kw.shape[1] == d && vw.shape[1] == d, "hidden dimensions differ");
+	if constexpr (std::is_same_v<dtype, float16>)
+	{
+		ACASSERT(d == 64 || d == 128 || d == 256, "hidden dimension must be 64, 128 or 256");
+		Tensor<dtype, CUDA> y(qw.dim, qw.shape);
+		SoftmaxPrologue p;
+		p.alpha = static_cast<float32>(calculate_alpha<float32>(static_cast<int>(d)));
+		hip_flash_sdpa_fwd_f16(p, qw, kw, vw, y);
+		return y;
+	}
+	else
+	{
+		return single_head_attention_fwd(qw, kw, vw);
+	}
+}
+
+/*
+  Attention over (..., heads, n, d) tensors with the mask given by rules instead of a tensor: scale, optional
+  softcap, causal rule with the diagonal at n_k - n_q, optional sliding window (the fields of SoftmaxPrologue).
+  Half precision GPU tensors take the fused kernel (k and v may have fewer heads than q); host tensors and float32
+  take sdp_attention_masked_scaled_fwd with the mask the rules describe.
+*/
+template<FloatingPointType dtype, Device device>
+inline Tensor<dtype, device> sdp_attention_rules_fwd(
+	const Tensor<dtype, device>& qw,
+	const Tensor<dtype, device>& kw,
+	const Tensor<dtype, device>& vw,
+	const SoftmaxPrologue& rules)
+{
+	const int64 dim = qw.dim;
+	ACASSERT(dim >= 2 && kw.dim == dim && vw.dim == dim, "dimension missmatch");
+	const int64 n_q = qw.shape[dim - 2], n_k = kw.shape[dim - 2], d = qw.shape[dim - 1];
+	ACASSERT(kw.shape[dim - 1] == d && vw.shape[dim - 1] == d && vw.shape[dim - 2] == n_k, "q, k and v need one head dimension");
+	if constexpr (device == CUDA && std::is_same_v<dtype, float16>)
+	{
+		ACASSERT(d == 64 || d == 128 || d == 256, "hidden dimension must be 64, 128 or 256");
+		ACASSERT(rules.softcap >= 0.f && rules.window >= 0, "softcap and window must not be negative");
+		Tensor<dtype, CUDA> y(qw.dim, qw.shape);
+		hip_flash_sdpa_fwd_f16(rules, qw, kw, vw, y);
+		return y;
+	}
+	else
+	{
+		ACASSERT(rules.softcap == 0.f, "the softcap needs the fused kernel");
+		auto hmask = crt_rule_mask<float32>(n_q, n_k, rules.causal, rules.window, n_k - n_q);
+		Tensor<dtype, CPU> hm = cvt_tensor_from_float32<dtype>(hmask);
+		std::vector<int64> mshape(static_cast<size_t>(dim), 1);
+		mshape[dim - 2] = n_q;
+		mshape[dim - 1] = n_k;
+		auto mview = tensor_view(hm, mshape);
+		if constexpr (device == CUDA)
+			return sdp_attention_masked_scaled_fwd(qw, kw, vw, mview.copy_to_cuda(), static_cast<dtype>(rules.alpha));
+		else
+			return sdp_attention_masked_scaled_fwd(qw, kw, vw, mview, static_cast<dtype>(rules.alpha));
 	}
 }
 
