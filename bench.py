@@ -46,7 +46,7 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--cpu-seconds", type=float, default=12.0,
                     help="target wall time of the CPU-oracle sample (0 disables the CPU baseline)")
-    ap.add_argument("--only", default="", help="comma list of: gemm,gemm32,conv,softmax (default: all)")
+    ap.add_argument("--only", default="", help="comma list of: gemm,gemm32,conv,softmax,attn,norm (default: all)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain device copy of 256 MiB (read 256 MiB + write 256 MiB) a few times, "
                          "as the known-size reference for scaling FETCH_SIZE / WRITE_SIZE counter readings")
@@ -171,6 +171,56 @@ def bench_softmax(torch, ops, steps, warmup, *, name, heads, q, k, std, alpha, c
     }
 
 
+def bench_attention(torch, ops, steps, warmup):
+    # Gemma2 attention block at the shape of the softmax headline configuration: 8 query heads over 4 key / value
+    # heads, 8192 positions, head_dim 256, scale 1 / 16, softcap 50, causal + window 4096, one fused kernel
+    h, hkv, n, d, win = 8, 4, 8192, 256, 4096
+    g = torch.Generator(device="cuda")
+    g.manual_seed(0)
+    q = torch.randn((1, h, n, d), device="cuda", generator=g).half()
+    k = torch.randn((1, hkv, n, d), device="cuda", generator=g).half()
+    v = torch.randn((1, hkv, n, d), device="cuda", generator=g).half()
+    host_s, ev_s = timed_region(torch, lambda: ops.sdp_attention_fwd(q, k, v, 1.0 / 16.0, softcap=50.0, causal=True, window=win),
+                                steps, warmup)
+    pairs = win * (win + 1) // 2 + (n - win) * win          # visible (query, key) pairs per head
+    flops = 4.0 * d * pairs * h                             # q k^T and p v, 2 flop per multiply-add
+    t = ev_s / steps
+    return {
+        "name": "sdp_attention_fwd_f16",
+        "workload": "fused attention fp16 q [1, 8, 8192, 256], k / v [1, 4, 8192, 256], x 1/16, softcap 50, causal + window 4096",
+        "us_per_launch": t * 1e6, "value": flops / t / 1e12, "unit": "TFLOP/s", "dtype": "f16",
+        "roofline": {"bound": "mfma", "achieved": flops / t / 1e12, "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": flops / t / 1e12 / PEAK_FP16_TFLOPS, "traffic": None,
+                     "algorithmic_flops": flops, "visible_pairs_per_head": pairs},
+    }
+
+
+def bench_gated_rmsnorm(torch, ops, steps, warmup):
+    # Zamba2-7B Mamba2 mixer: batch 4 x 4096 positions, d_inner 8192
+    rows, cols, nbuf = 4 * 4096, 8192, 3                    # 3 x 805 MB of x + z + y: past the Infinity Cache
+    g = torch.Generator(device="cuda")
+    g.manual_seed(0)
+    xs = [torch.randn((rows, cols), device="cuda", generator=g).half() for _ in range(nbuf)]
+    zs = [torch.randn((rows, cols), device="cuda", generator=g).half() for _ in range(nbuf)]
+    w = (torch.rand((cols,), device="cuda", generator=g) + 0.5).half()
+    it = [0]
+
+    def step():
+        i = it[0] % nbuf
+        it[0] += 1
+        ops.tensor_zamba_gated_rmsnorm(xs[i], zs[i], w, cols, 1e-5)
+
+    host_s, ev_s = timed_region(torch, step, steps, warmup)
+    nbytes = 3 * rows * cols * 2 + cols * 2
+    t = ev_s / steps
+    return {
+        "name": "gated_rmsnorm_f16", "workload": "gated RMS norm fp16 x, z [16384, 8192], w [8192], eps 1e-5",
+        "us_per_launch": t * 1e6, "value": nbytes / t / 1e9, "unit": "GB/s", "dtype": "f16",
+        "roofline": {"bound": "hbm", "achieved": nbytes / t / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": nbytes / t / 1e9 / PEAK_HBM_GBS, "traffic": None, "algorithmic_bytes": nbytes},
+    }
+
+
 def cpu_baseline_gemm(a_dev, bt_dev, target_seconds):
     """The oracle's tensor_mm (1 thread, the reference's loop order) on the first R rows of the
     same 4096^3 problem; R is sized from a short probe so that the sample takes about
@@ -249,6 +299,11 @@ def main():
             torch, ops, max(args.steps // 4, 1), max(args.warmup // 4, 1), name="softmax_gemma2_f16",
             key="softmax_gemma2", heads=8, q=8192, k=8192, std=16.0, alpha=1.0 / 16.0, cap=50.0, window=4096, nbuf=2,
             workload="Gemma2 softmax fp16 [1, 8, 8192, 8192], N(0,16) x 1/16, softcap 50, causal + window 4096"))
+
+    if want("attn"):
+        kernels.append(bench_attention(torch, ops, max(args.steps // 8, 1), max(args.warmup // 4, 1)))
+    if want("norm"):
+        kernels.append(bench_gated_rmsnorm(torch, ops, max(args.steps // 4, 1), max(args.warmup // 4, 1)))
 
     line = {
         "metric": "fp16 GEMM TFLOP/s; conv1d & softmax HBM GB/s (% roofline) on 1 MI355X",
