@@ -6,6 +6,9 @@
 
 #include "ops.hpp"
 #include "sdp.hpp"
+#include "gemma_linsoftcap.hpp"
+#include "gemma_mlp.hpp"
+#include "zamba_gated_rmsnorm.hpp"
 #include "fast_mm.cuh"
 #include "dat_file.hpp"
 #include "test_tools.hpp"
@@ -178,4 +181,102 @@ TEST_CASE(external_test_sdp_masked_scaled_fwd_f32, GPU)
 	                                          hmask.copy_to_cuda(), 0.125f);
 	auto hy_from_cuda = dy.copy_to_host();
 	return elementwise_compatible(hy_from_cuda, hy) && compare_data_buffers(hy_from_cuda, hy);
+}
+
+/* ---- cases of the Gemma2 / Zamba2 callers, bodies after tests/gemma2_tests.cpp and tests/zamba2_tests.cpp ---- */
+
+TEST_CASE(external_test_gemma2_lmhead_softcap, GPU)
+{
+	auto path = golden_dir() / "test_gemma2_lmhead_softcap";
+	// hw is tied to the embedding weights
+	auto hx = load_tensor((path / "in_0.dat").string());
+	auto hw = load_tensor((path / "gemma2_causal_lm.gemma2forcausallm.model.embed_tokens.weight.dat").string());
+	auto exp_hy = load_tensor((path / "out_0.dat").string());
+
+	auto dx = hx.copy_to_cuda();
+	auto dw = hw.copy_to_cuda();
+	auto act_dy_cuda = tensor_gemma_linear_softcap(dx, dw, 30.f);
+	auto act_hy_cuda = act_dy_cuda.copy_to_host();
+	return same_shape_and(exp_hy, act_hy_cuda, [](auto& a, auto& e) { return compare_data_buffers(a, e); });
+}
+
+TEST_CASE(external_test_gemma2_decoder_mlp_cpu, HOST)
+{
+	auto path = golden_dir() / "test_gemma2decoder_mlp";
+	auto hx = load_tensor((path / "in_0.dat").string());
+	auto exp_hy = load_tensor((path / "out_0.dat").string());
+	GemmaMLPweights<float32, CPU> mlp_weights;
+	mlp_weights.load_weights(
+		(path / "gemma2decoder_mlp.gemma2mlp.gate_proj.weight.dat").string(),
+		(path / "gemma2decoder_mlp.gemma2mlp.up_proj.weight.dat").string(),
+		(path / "gemma2decoder_mlp.gemma2mlp.down_proj.weight.dat").string());
+	auto act_hy = tensor_gemma_mlp(mlp_weights, hx);
+	return same_shape_and(exp_hy, act_hy, [](auto& a, auto& e) { return compare_data_buffers(a, e, 1e-5f); });
+}
+
+TEST_CASE(external_test_gemma2_decoder_mlp, GPU)
+{
+	auto path = golden_dir() / "test_gemma2decoder_mlp";
+	auto hx = load_tensor((path / "in_0.dat").string());
+	auto exp_hy = load_tensor((path / "out_0.dat").string());
+
+	GemmaMLPweights<float32, CUDA> mlp_weights;
+	mlp_weights.load_weights(
+		(path / "gemma2decoder_mlp.gemma2mlp.gate_proj.weight.dat").string(),
+		(path / "gemma2decoder_mlp.gemma2mlp.up_proj.weight.dat").string(),
+		(path / "gemma2decoder_mlp.gemma2mlp.down_proj.weight.dat").string());
+
+	auto dx = hx.copy_to_cuda();
+	auto act_dy_cuda = tensor_gemma_mlp(mlp_weights, dx);
+	auto act_hy_cuda = act_dy_cuda.copy_to_host();
+	return same_shape_and(exp_hy, act_hy_cuda, [](auto& a, auto& e) { return compare_data_buffers(a, e); });
+}
+
+TEST_CASE(external_test_mamba2_layer_gated_rmsnorm_cpu, HOST)
+{
+	auto path = golden_dir() / "test_mamba2layer_gated_rmsnorm";
+	auto hx = load_tensor((path / "in_0.dat").string());
+	auto hz = load_tensor((path / "in_1.dat").string());
+	auto hw = load_tensor((path / "mamba2layer_rmsnorm.rmsnorm.weight.dat").string());
+	auto exp_hy = load_tensor((path / "out_0.dat").string());
+	auto act_hy = tensor_zamba_gated_rmsnorm(hx, hz, hw, 64, 1e-5f);
+	return same_shape_and(exp_hy, act_hy, [](auto& a, auto& e) { return compare_data_buffers(a, e, 1e-6f); });
+}
+
+TEST_CASE(external_test_mamba2_layer_gated_rmsnorm, GPU)
+{
+	auto path = golden_dir() / "test_mamba2layer_gated_rmsnorm";
+
+	// constant params
+	const float32 eps = 1e-5f;
+	const int32 gsize = 64;  // group size: the row
+
+	auto hx = load_tensor((path / "in_0.dat").string());
+	auto hz = load_tensor((path / "in_1.dat").string());
+	auto hw = load_tensor((path / "mamba2layer_rmsnorm.rmsnorm.weight.dat").string());
+	auto exp_hy = load_tensor((path / "out_0.dat").string());
+
+	auto dx = hx.copy_to_cuda();
+	auto dz = hz.copy_to_cuda();
+	auto dw = hw.copy_to_cuda();
+	auto act_dy_cuda = tensor_zamba_gated_rmsnorm(dx, dz, dw, gsize, eps);
+	auto act_hy_cuda = act_dy_cuda.copy_to_host();
+	return same_shape_and(exp_hy, act_hy_cuda, [](auto& a, auto& e) { return compare_data_buffers(a, e); });
+}
+
+TEST_CASE(external_test_sdp_rules_f16_gqa, GPU)
+{
+	auto path = golden_dir() / "test_sdp_rules_f16_gqa";
+	auto hq = load_tensor<float16>((path / "q.dat").string());
+	auto hk = load_tensor<float16>((path / "k.dat").string());
+	auto hv = load_tensor<float16>((path / "v.dat").string());
+	auto exp_hy = load_tensor((path / "y.dat").string());
+	SoftmaxPrologue rules;
+	rules.alpha = 0.125f;
+	rules.softcap = 20.f;
+	rules.causal = true;
+	rules.window = 12;
+	auto act = cvt_tensor_datatype<float32, float16>(
+		sdp_attention_rules_fwd(hq.copy_to_cuda(), hk.copy_to_cuda(), hv.copy_to_cuda(), rules).copy_to_host());
+	return same_shape_and(exp_hy, act, [](auto& a, auto& e) { return compare_data_buffers_l2(a, e, 4e-3f) && compare_data_buffers(a, e, 2e-2f); });
 }

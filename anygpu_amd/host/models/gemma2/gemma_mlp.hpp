@@ -10,6 +10,7 @@
 #include "tensor.hpp"
 #include "core_concepts.hpp"
 #include "ops.hpp"
+#include "dat_file.hpp"
 
 template<FloatingPointType dtype, Device device>
 struct GemmaMLPweights
@@ -17,6 +18,23 @@ struct GemmaMLPweights
 	Tensor<dtype, device> gate_proj_weight;  // (hidden, intermediate)
 	Tensor<dtype, device> up_proj_weight;    // (hidden, intermediate)
 	Tensor<dtype, device> down_proj_weight;  // (intermediate, hidden)
+
+	/* Reads the three matrices from .dat files.  Checkpoints keep them as (out_features, in_features);
+	   with transpose they are turned into the (in_features, out_features) form the products take. */
+	void load_weights(
+		const std::string& path_gate_proj_weight,
+		const std::string& path_up_proj_weight,
+		const std::string& path_down_proj_weight,
+		const bool transpose = true)
+	{
+		auto fetch = [&](const std::string& path) {
+			auto t = load_tensor<dtype>(path);
+			return copy_to_device<dtype, CPU, device>(transpose ? tensor_transp(t) : t);
+		};
+		gate_proj_weight = fetch(path_gate_proj_weight);
+		up_proj_weight = fetch(path_up_proj_weight);
+		down_proj_weight = fetch(path_down_proj_weight);
+	}
 };
 
 /*

@@ -8,6 +8,7 @@
 #include "norm_ops.hpp"
 #include "shape_ops.hpp"
 #include "softmax_ops.hpp"
+#include "transp_ops.hpp"
 #include "causal_conv1d.hpp"
 
 #endif  // __OPS__

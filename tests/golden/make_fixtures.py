@@ -78,6 +78,54 @@ def main() -> None:
         save_tensor(t, d / f"{name}.dat")
     save_tensor(oracle.sdp_attention_masked_scaled_fwd(q, k, v, mask, 0.125), d / "y.dat")
 
+    # Gemma2 output head with logit soft-capping, file names of tests/gemma2_tests.cpp:312-335
+    d = case_dir("test_gemma2_lmhead_softcap")
+    x = synth.normal(160, (1, 5, 48))
+    w = synth.normal(161, (70, 48)) * np.float32(4.0)                     # [vocab, hidden]; logits reach past the cap of 30
+    save_tensor(x, d / "in_0.dat"); save_tensor(w, d / "gemma2_causal_lm.gemma2forcausallm.model.embed_tokens.weight.dat")
+    save_tensor(oracle.gemma_linear_softcap(x, w, 30.0), d / "out_0.dat")
+
+    # Gemma2 MLP, gate / up / down weights stored [out, in] as in the reference's checkpoints (gemma_mlp.hpp:20-38
+    # transposes them at load), tests/gemma2_tests.cpp:22-52
+    d = case_dir("test_gemma2decoder_mlp")
+    hidden, inter = 32, 96
+    x = synth.normal(170, (1, 7, hidden))
+    wg = synth.normal(171, (inter, hidden)) * np.float32(0.3)
+    wu = synth.normal(172, (inter, hidden)) * np.float32(0.3)
+    wd = synth.normal(173, (hidden, inter)) * np.float32(0.2)
+    mid = oracle.gemma_mlp_upproj(x, np.ascontiguousarray(wg.T), np.ascontiguousarray(wu.T))
+    y = oracle.tensor_mm(mid.reshape(7, inter), np.ascontiguousarray(wd.T)).reshape(1, 7, hidden)
+    save_tensor(x, d / "in_0.dat")
+    for name, t in (("gate_proj", wg), ("up_proj", wu), ("down_proj", wd)):
+        save_tensor(t, d / f"gemma2decoder_mlp.gemma2mlp.{name}.weight.dat")
+    save_tensor(y, d / "out_0.dat")
+
+    # gated RMS norm of the Mamba2 mixer, tests/zamba2_tests.cpp:458-489 (eps 1e-5, one group = the row)
+    d = case_dir("test_mamba2layer_gated_rmsnorm")
+    x = synth.normal(180, (1, 6, 64)); z = synth.normal(181, (1, 6, 64)) * np.float32(2.0)
+    w = synth.uniform(182, (64,), 0.5, 1.5)
+    save_tensor(x, d / "in_0.dat"); save_tensor(z, d / "in_1.dat"); save_tensor(w, d / "mamba2layer_rmsnorm.rmsnorm.weight.dat")
+    save_tensor(oracle.zamba_gated_rmsnorm(x, z, w, 1e-5), d / "out_0.dat")
+
+    # decode steps of the causal convolution: the columns of x one at a time, state carried along
+    d = case_dir("test_causal_conv1d_update_f32")
+    x = synth.normal(190, (2, 6, 9)); w = synth.normal(191, (6, 4)); b = synth.normal(192, (6,))
+    save_tensor(x, d / "x.dat"); save_tensor(w, d / "w.dat"); save_tensor(b, d / "b.dat")
+    save_tensor(oracle.tensor_causal_conv1d(x, w, b), d / "y.dat")     # column t is the output of step t
+    save_tensor(np.ascontiguousarray(x[:, :, -3:]), d / "state.dat")   # the state after the last step
+
+    # attention with rule masks, half precision inputs: 4 query heads over 2 key / value heads, 24 queries at the end
+    # of 40 keys, d = 64, scale 0.125, softcap 20, causal + window 12
+    d = case_dir("test_sdp_rules_f16_gqa")
+    q = synth.normal(200, (1, 4, 24, 64)).astype(np.float16)
+    k = synth.normal(201, (1, 2, 40, 64)).astype(np.float16)
+    v = synth.normal(202, (1, 2, 40, 64)).astype(np.float16)
+    y = oracle.sdp_attention_rules(*(oracle.cvt_f16_to_f32(t)[0] for t in (q, k, v)), alpha=0.125, softcap=20.0,
+                                   causal=True, window=12, q_per_kv=2)
+    for name, t in (("q", q), ("k", k), ("v", v)):
+        save_tensor(t, d / f"{name}.dat")
+    save_tensor(y.reshape(1, 4, 24, 64), d / "y.dat")
+
     print("fixtures written under", HERE)
 
 

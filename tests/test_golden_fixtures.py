@@ -36,6 +36,40 @@ def test_fixtures_match_the_oracle(oracle):
     d = GOLDEN / "test_sdp_fwd_masked_scaled_f32_16_32"
     q, k, v, mask = (load_tensor(d / f"{n}.dat") for n in ("q", "k", "v", "mask"))
     assert np.array_equal(oracle.sdp_attention_masked_scaled_fwd(q, k, v, mask, 0.125), load_tensor(d / "y.dat"))
+    d = GOLDEN / "test_gemma2_lmhead_softcap"
+    w = load_tensor(d / "gemma2_causal_lm.gemma2forcausallm.model.embed_tokens.weight.dat")
+    assert np.array_equal(oracle.gemma_linear_softcap(load_tensor(d / "in_0.dat"), w, 30.0), load_tensor(d / "out_0.dat"))
+    d = GOLDEN / "test_gemma2decoder_mlp"
+    wg, wu, wd = (load_tensor(d / f"gemma2decoder_mlp.gemma2mlp.{n}_proj.weight.dat") for n in ("gate", "up", "down"))
+    x = load_tensor(d / "in_0.dat")
+    mid = oracle.gemma_mlp_upproj(x, np.ascontiguousarray(wg.T), np.ascontiguousarray(wu.T))
+    y = oracle.tensor_mm(mid.reshape(-1, wd.shape[1]), np.ascontiguousarray(wd.T)).reshape(x.shape)
+    assert np.array_equal(y, load_tensor(d / "out_0.dat"))
+    # torch's library formula for the block: down(gelu_tanh(gate(x)) * up(x)) with [out, in] weights
+    import torch
+    import torch.nn.functional as F
+    tx, tg, tu, td = (torch.from_numpy(t).double() for t in (x, wg, wu, wd))
+    ref = F.linear(F.gelu(F.linear(tx, tg), approximate="tanh") * F.linear(tx, tu), td).numpy()
+    assert np.max(np.abs(y - ref)) < 1e-5
+    d = GOLDEN / "test_mamba2layer_gated_rmsnorm"
+    x, z, w = load_tensor(d / "in_0.dat"), load_tensor(d / "in_1.dat"), load_tensor(d / "mamba2layer_rmsnorm.rmsnorm.weight.dat")
+    y = oracle.zamba_gated_rmsnorm(x, z, w, 1e-5)
+    assert np.array_equal(y, load_tensor(d / "out_0.dat"))
+    g = torch.from_numpy(x).double() * F.silu(torch.from_numpy(z).double())
+    ref = (g * torch.rsqrt(g.pow(2).mean(-1, keepdim=True) + 1e-5) * torch.from_numpy(w).double()).numpy()
+    assert np.max(np.abs(y - ref)) < 1e-5
+    d = GOLDEN / "test_causal_conv1d_update_f32"
+    x, w, b = load_tensor(d / "x.dat"), load_tensor(d / "w.dat"), load_tensor(d / "b.dat")
+    state = np.zeros((x.shape[0], x.shape[1], w.shape[1] - 1), dtype=np.float32)
+    want = load_tensor(d / "y.dat")
+    for t in range(x.shape[2]):
+        yt, state = oracle.causal_conv1d_update(x[:, :, t], state, w, b)
+        assert np.array_equal(yt, want[:, :, t])
+    assert np.array_equal(state, load_tensor(d / "state.dat"))
+    d = GOLDEN / "test_sdp_rules_f16_gqa"
+    q, k, v = (oracle.cvt_f16_to_f32(load_tensor(d / f"{n}.dat"))[0] for n in ("q", "k", "v"))
+    y = oracle.sdp_attention_rules(q, k, v, alpha=0.125, softcap=20.0, causal=True, window=12, q_per_kv=2)
+    assert np.array_equal(y.reshape(1, 4, 24, 64), load_tensor(d / "y.dat"))
     for name, kw in [("test_softmax_masked_scaled_f32", dict(alpha=0.125, causal=True, q_len=16)),
                      ("test_softmax_softcap_window_f32", dict(alpha=0.0625, softcap=50.0, causal=True, window=6, q_len=16))]:
         d = GOLDEN / name

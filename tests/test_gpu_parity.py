@@ -850,3 +850,36 @@ def test_golden_fixtures_through_c_abi(ops):
                                   window=6, q_len=16))
     assert scaled_rel_err(got, want, want.max(axis=1, keepdims=True)) <= TOL_F32
     assert np.all(got[np.tile(load_tensor(d / "mask.dat"), (2, 1)) != 0] == 0.0)
+
+    d = golden / "test_gemma2_lmhead_softcap"
+    w = load_tensor(d / "gemma2_causal_lm.gemma2forcausallm.model.embed_tokens.weight.dat")
+    got = host(ops.tensor_gemma_linear_softcap(dev(load_tensor(d / "in_0.dat")), dev(w), 30.0))
+    assert scaled_rel_err(got, load_tensor(d / "out_0.dat"), 30.0) <= TOL_F32
+
+    d = golden / "test_gemma2decoder_mlp"
+    wg, wu, wd = (load_tensor(d / f"gemma2decoder_mlp.gemma2mlp.{n}_proj.weight.dat") for n in ("gate", "up", "down"))
+    x = load_tensor(d / "in_0.dat")
+    mid = ops.mlp_gemma2_fused_upproj(dev(x), dev(np.ascontiguousarray(wg.T)), dev(np.ascontiguousarray(wu.T)))
+    from anygpu_amd import capi
+    got = host(ops.tensor_mm(mid.reshape(-1, wd.shape[1]), dev(wd), b_layout=capi.B_COL_MAJOR)).reshape(x.shape)
+    assert scaled_rel_err(got, load_tensor(d / "out_0.dat"), 1.0) <= TOL_F32
+
+    d = golden / "test_mamba2layer_gated_rmsnorm"
+    got = host(ops.tensor_zamba_gated_rmsnorm(dev(load_tensor(d / "in_0.dat")), dev(load_tensor(d / "in_1.dat")),
+                                              dev(load_tensor(d / "mamba2layer_rmsnorm.rmsnorm.weight.dat")), 64, 1e-5))
+    assert scaled_rel_err(got, load_tensor(d / "out_0.dat"), 1.0) <= TOL_F32
+
+    d = golden / "test_causal_conv1d_update_f32"
+    x, w, b = load_tensor(d / "x.dat"), load_tensor(d / "w.dat"), load_tensor(d / "b.dat")
+    want = load_tensor(d / "y.dat")
+    import torch
+    state = torch.zeros((x.shape[0], x.shape[1], w.shape[1] - 1), device="cuda")
+    for t in range(x.shape[2]):
+        got = host(ops.tensor_causal_conv1d_update(dev(x[:, :, t]), state, dev(w), dev(b)))
+        assert scaled_rel_err(got, want[:, :, t], 1.0) <= TOL_F32
+    assert np.array_equal(host(state), load_tensor(d / "state.dat"))
+
+    d = golden / "test_sdp_rules_f16_gqa"
+    got = host(ops.sdp_attention_fwd(*(dev(load_tensor(d / f"{n}.dat")) for n in ("q", "k", "v")), 0.125, softcap=20.0,
+                                     causal=True, window=12)).astype(np.float32)
+    assert scaled_rel_err(got, load_tensor(d / "y.dat"), 1.0) <= TOL_F16_ROWOPS * 2
