@@ -4,9 +4,9 @@
 // three-launch form (q k^T, row softmax, p v) writes and reads 1 GiB of scores twice; this kernel
 // reads q, k, v and writes y.
 //
-// A block owns 128 consecutive queries of one head: 8 waves with 16 queries each (or 4 waves with
-// 32), so that two waves share a SIMD and one wave's MFMAs run under the other's softmax
-// arithmetic.  It walks the visible key range in tiles of 64 keys.  Per tile:
+// A block of 8 waves owns 128 consecutive queries of one head, 16 per wave (256 and 32 at head
+// dimension 128), so that at least two waves share a SIMD and one wave's MFMAs run under the
+// other's softmax arithmetic.  It walks the visible key range in tiles of 64 keys.  Per tile:
 //   * K and V rows go global -> registers -> LDS (the loads of the next tile are in flight
 //     while this one is being used);
 //   * S^T = K Q^T with v_mfma_f32_16x16x32_f16: the K fragment is the first operand, the Q
@@ -34,7 +34,6 @@ namespace anygpu {
 
 namespace {
 
-constexpr int kAttnQueriesPerBlock = 128;
 constexpr int kAttnKeysPerTile = 64;
 
 typedef short short4_t __attribute__((ext_vector_type(4)));
@@ -78,16 +77,18 @@ __device__ __forceinline__ float logit2(float s, float k_in, float k_cap)
 template <int D>
 struct AttnLds
 {
-	static constexpr int kPitchK = 2 * D + 16;      // bytes; 16-byte reads of 16 rows hit 64 different banks
-	static constexpr int kPitchV = 2 * D + 32;      // bytes; the 8 rows of a half wave's transposing read do
+	// Row pitches in bytes.  Measured over pads of 16 / 32 / 48 bytes for K and 16 / 32 / 64 for V: 32 and 32 is
+	// the fastest pair at every head dimension (8 - 10 % over 16 and 32).
+	static constexpr int kPitchK = 2 * D + 32;
+	static constexpr int kPitchV = 2 * D + 32;
 	static constexpr int kBytes = kAttnKeysPerTile * (kPitchK + kPitchV);
 };
 
-// QB: 16-query blocks per wave, WAVES: waves per block; QB * WAVES = 8.
+// QB: 16-query blocks per wave, WAVES: waves per block; a block owns 16 * QB * WAVES consecutive queries.
 template <int D, bool SOFTCAP, int QB, int WAVES>
 __global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f16_kernel(const AttnArgs a)
 {
-	static_assert(16 * QB * WAVES == kAttnQueriesPerBlock, "a block owns 128 queries");
+	constexpr int kAttnQueriesPerBlock = 16 * QB * WAVES;
 	constexpr int THREADS = 64 * WAVES;
 	extern __shared__ __align__(16) char lds[];
 	using L = AttnLds<D>;
@@ -316,14 +317,13 @@ __global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f16_kernel(const
 	}
 }
 
-template <int D, bool SOFTCAP>
+template <int D, bool SOFTCAP, int QB>
 hipError_t launch_variant(const AttnArgs& args, int64_t batch_heads, hipStream_t stream)
 {
-	// 8 waves x 16 queries measured 1.1 - 1.5 x faster than 4 waves x 32 queries (16 x 4096 x 128 causal: 173 us
-	// against 266 us): the smaller register footprint lets two blocks share a CU
-	constexpr int QB = 1, WAVES = 8 / QB;
+	constexpr int WAVES = 8;
 	auto kernel = sdp_attention_fwd_f16_kernel<D, SOFTCAP, QB, WAVES>;
 	constexpr int kLdsBytes = AttnLds<D>::kBytes;
+	constexpr int kQueriesPerBlock = 16 * QB * WAVES;
 	(void)hipGetLastError();
 	if (kLdsBytes > 64 * 1024)
 	{
@@ -340,15 +340,24 @@ hipError_t launch_variant(const AttnArgs& args, int64_t batch_heads, hipStream_t
 			configured_devices.fetch_or(bit, std::memory_order_relaxed);
 		}
 	}
-	const dim3 grid((unsigned)((args.n_q + kAttnQueriesPerBlock - 1) / kAttnQueriesPerBlock), (unsigned)batch_heads);
+	const dim3 grid((unsigned)((args.n_q + kQueriesPerBlock - 1) / kQueriesPerBlock), (unsigned)batch_heads);
 	kernel<<<grid, dim3(64 * WAVES), kLdsBytes, stream>>>(args);
 	return hipGetLastError();
 }
 
+// Queries per wave: 16 everywhere (8 waves x 16 queries measured 1.1 - 1.5 x faster than 4 waves x 32: the smaller
+// register footprint lets more waves share a SIMD), except head_dim 128 with enough query blocks to fill the chip,
+// where 8 waves x 32 queries halve the LDS reads per flop and fit the register file (16 x 4096 x 128 causal: 148 us
+// against 172 us).  At head_dim 256 the 32-query form does not fit the registers.
 template <int D>
 hipError_t launch_dim(const AttnArgs& args, bool softcap, int64_t batch_heads, hipStream_t stream)
 {
-	return softcap ? launch_variant<D, true>(args, batch_heads, stream) : launch_variant<D, false>(args, batch_heads, stream);
+	if constexpr (D == 128)
+	{
+		if (batch_heads * ((args.n_q + 255) / 256) >= 256)
+			return softcap ? launch_variant<D, true, 2>(args, batch_heads, stream) : launch_variant<D, false, 2>(args, batch_heads, stream);
+	}
+	return softcap ? launch_variant<D, true, 1>(args, batch_heads, stream) : launch_variant<D, false, 1>(args, batch_heads, stream);
 }
 
 }  // namespace

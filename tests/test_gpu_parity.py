@@ -799,6 +799,25 @@ def test_sdp_attention_fused_kernel_structure(ops, oracle):
     assert bool((out == 3.0).all())
 
 
+def test_sdp_attention_fused_kernel_many_heads_d128(ops, oracle):
+    # enough query blocks at head_dim 128 for the 32-queries-per-wave form: 64 heads over 16 key / value heads,
+    # 1000 queries at the end of 1100 keys, softcap + causal + window
+    h, hkv, n_q, n_k, d = 64, 16, 1000, 1100, 128
+    q = synth.normal(1, (h, n_q, d)).astype(np.float16)
+    k = synth.normal(2, (hkv, n_k, d)).astype(np.float16)
+    v = synth.normal(3, (hkv, n_k, d)).astype(np.float16)
+    got = host(ops.sdp_attention_fwd(dev(q), dev(k), dev(v), 0.0884, softcap=30.0, causal=True, window=300)).astype(np.float32)
+    idx = np.array([0, 1, 15, 16, 31, 32, 255, 256, 257, 511, 700, 998, 999], dtype=np.int64)
+    want = oracle.sdp_attention_rules(*(oracle.cvt_f16_to_f32(t) for t in (q, k, v)), alpha=0.0884, softcap=30.0,
+                                      causal=True, window=300, q_per_kv=4, query_index=idx, threads=8)
+    assert scaled_rel_err(got[:, idx, :], want, 1.0) <= TOL_F16_ROWOPS * 2
+    # every query against the same kernel's 16-queries-per-wave form (fewer heads per launch take it)
+    parts = [host(ops.sdp_attention_fwd(dev(q[i:i + 4]), dev(k[i // 4:i // 4 + 1]), dev(v[i // 4:i // 4 + 1]), 0.0884,
+                                        softcap=30.0, causal=True, window=300)) for i in (0, 28, 60)]
+    for i, part in zip((0, 28, 60), parts):
+        assert scaled_rel_err(got[i:i + 4], part.astype(np.float32), 1.0) <= 2e-3
+
+
 def test_sdp_attention_fused_kernel_gemma2_block(ops, oracle):
     # Gemma2 attention at the softmax configuration of the headline set: 8 query heads over 4 key / value heads,
     # head_dim 256, scale 1 / 16, softcap 50, causal + window 4096; 6144 positions so that the window cuts
