@@ -360,6 +360,258 @@ hipError_t launch_dim(const AttnArgs& args, bool softcap, int64_t batch_heads, h
 	return softcap ? launch_variant<D, true, 1>(args, batch_heads, stream) : launch_variant<D, false, 1>(args, batch_heads, stream);
 }
 
+// ---------------------------------------------------------------------------------------------
+// Decode form: very few queries per head (a generation step), long key range.  The fused kernel
+// above would give every head one block walking all keys in sequence; here the KEYS are split.
+//
+// The q_per_kv query heads that share a key / value head, times the n_q queries of each, are the
+// (at most 16) "rows" of one 16-query MFMA block, so K and V of a head are read once for all of
+// them.  Pass 1: one wave per (key / value head, split of the visible key range).  K fragments
+// go straight from global memory into the MFMA operand layout (16 bytes per lane, no LDS); V
+// passes through a wave-private LDS tile for the transposing reads.  The wave leaves its
+// running maximum, sum and unnormalised accumulators in the workspace.  Pass 2 merges the
+// splits of a row: M = max m_i, y = sum o_i 2^(m_i - M) / sum l_i 2^(m_i - M).
+// Workspace per (head, split, row): head_dim accumulators + maximum + sum, fp32.
+// ---------------------------------------------------------------------------------------------
+constexpr int kDecodeMaxRows = 16;
+constexpr int kDecodeMaxSplits = 64;
+constexpr int kDecodeTargetWaves = 1024;          // about 4 waves per CU
+
+struct DecodeArgs
+{
+	AttnArgs a;
+	float* ws;              // [kv_heads][splits][rows][D + 2]
+	int rows;               // q_per_kv * n_q
+	int splits;
+	int tiles_per_split;
+	int t_first, t_last;    // visible key tiles of the group
+};
+
+template <int D, bool SOFTCAP>
+__global__ __launch_bounds__(64) void sdp_decode_partial_kernel(const DecodeArgs da)
+{
+	extern __shared__ __align__(16) char lds[];           // the V tile: 64 keys x (2 D + 32) bytes
+	const AttnArgs& a = da.a;
+	constexpr int kPitchV = AttnLds<D>::kPitchV;
+	constexpr int KS = D / 32, DC = D / 16, VPR = D / 8;
+	constexpr int VPT = kAttnKeysPerTile * D / 8 / 64;    // V vectors per lane per tile
+
+	const int lane = threadIdx.x;
+	const int n = lane & 15, g = lane >> 4;
+	const int split = blockIdx.x;
+	const int kvh = blockIdx.y;
+	const half_t* qp = a.q + (int64_t)kvh * da.rows * D;  // the rows of a group are contiguous: [q_per_kv][n_q][D]
+	const half_t* kp = a.k + (int64_t)kvh * a.n_k * D;
+	const half_t* vp = a.v + (int64_t)kvh * a.n_k * D;
+
+	const bool row_ok = n < da.rows;
+	const int q_idx = row_ok ? n % a.n_q : 0;             // position of this lane's row among the n_q queries
+	half8_t qf[KS];
+#pragma unroll
+	for (int s = 0; s < KS; ++s)
+	{
+		half8_t val = {};
+		if (row_ok) val = *reinterpret_cast<const half8_t*>(qp + (int64_t)n * D + 32 * s + 8 * g);
+		qf[s] = val;
+	}
+	int vis_hi = a.causal ? q_idx + a.diag : a.n_k - 1;
+	if (vis_hi > a.n_k - 1) vis_hi = a.n_k - 1;
+	if (!row_ok) vis_hi = -1;                              // padding rows see nothing
+	const int vis_lo = a.window > 0 ? q_idx + a.diag - a.window + 1 : 0;
+
+	float m_run = -INFINITY, l_run = 0.0f;
+	float4_t o[DC];
+#pragma unroll
+	for (int c = 0; c < DC; ++c) o[c] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+
+	const int t0 = da.t_first + split * da.tiles_per_split;
+	int t1 = t0 + da.tiles_per_split - 1;
+	if (t1 > da.t_last) t1 = da.t_last;
+	for (int t = t0; t <= t1; ++t)
+	{
+		const int key0 = t * kAttnKeysPerTile;
+		// K fragments and the V tile: all loads of the tile are issued before the first use
+		half8_t kf[4][KS];
+#pragma unroll
+		for (int kb = 0; kb < 4; ++kb)
+		{
+			const int key = key0 + 16 * kb + n;
+#pragma unroll
+			for (int st = 0; st < KS; ++st)
+			{
+				half8_t val = {};
+				if (key < a.n_k) val = __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(kp + (int64_t)key * D + 32 * st + 8 * g));
+				kf[kb][st] = val;
+			}
+		}
+		float4_t vr[VPT];
+#pragma unroll
+		for (int i = 0; i < VPT; ++i)
+		{
+			const int idx = lane + 64 * i;
+			const int key = key0 + idx / VPR;
+			float4_t val = {};
+			if (key < a.n_k) val = __builtin_nontemporal_load(reinterpret_cast<const float4_t*>(vp + (int64_t)key * D + (idx % VPR) * 8));
+			vr[i] = val;
+		}
+#pragma unroll
+		for (int i = 0; i < VPT; ++i)
+		{
+			const int idx = lane + 64 * i;
+			*reinterpret_cast<float4_t*>(lds + (idx / VPR) * kPitchV + (idx % VPR) * 16) = vr[i];
+		}
+
+		float4_t s[4];
+#pragma unroll
+		for (int kb = 0; kb < 4; ++kb)
+		{
+			s[kb] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+			for (int st = 0; st < KS; ++st) s[kb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf[kb][st], qf[st], s[kb], 0, 0, 0);
+		}
+
+		float z[4][4];
+		float mt = -INFINITY;
+#pragma unroll
+		for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+			for (int r = 0; r < 4; ++r)
+			{
+				const int key = key0 + 16 * kb + 4 * g + r;
+				const float zz = logit2<SOFTCAP>(s[kb][r], a.k_in, a.k_cap);
+				z[kb][r] = (key >= vis_lo && key <= vis_hi) ? zz : -INFINITY;
+				mt = fmaxf(mt, z[kb][r]);
+			}
+		mt = fmaxf(mt, __shfl_xor(mt, 16));
+		mt = fmaxf(mt, __shfl_xor(mt, 32));
+		const float m_new = fmaxf(m_run, mt);
+		const float m_safe = (m_new == -INFINITY) ? 0.0f : m_new;
+		const float corr = fast_exp2(m_run - m_safe);
+		float psum = 0.0f;
+		half8_t pf[2];
+#pragma unroll
+		for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+			for (int r = 0; r < 4; ++r)
+			{
+				const float p = fast_exp2(z[kb][r] - m_safe);
+				psum += p;
+				pf[kb >> 1][4 * (kb & 1) + r] = (half_t)p;
+			}
+		l_run = l_run * corr + psum;
+		m_run = m_new;
+#pragma unroll
+		for (int c = 0; c < DC; ++c) o[c] *= corr;
+
+		// the V tile was written by this wave alone: its LDS writes are complete once the wave's counter says so
+		__builtin_amdgcn_s_waitcnt(0xC07F);               // lgkmcnt(0)
+		__builtin_amdgcn_wave_barrier();
+#pragma unroll
+		for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+			for (int c = 0; c < DC; ++c)
+			{
+				const char* src = lds + (32 * tt + 4 * g + (n >> 2)) * kPitchV + (16 * c + 4 * (n & 3)) * 2;
+				const half4_t lo = lds_read_tr_b64(src);
+				const half4_t hi = lds_read_tr_b64(src + 16 * kPitchV);
+				const half8_t vf = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+				o[c] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf, pf[tt], o[c], 0, 0, 0);
+			}
+		__builtin_amdgcn_s_waitcnt(0xC07F);               // the tile has been read before the next one overwrites it
+		__builtin_amdgcn_wave_barrier();
+	}
+
+	// partial result of this split: lane (n, g) holds o[row n][16 c + 4 g .. + 3]
+	float l = l_run;
+	l += __shfl_xor(l, 16);
+	l += __shfl_xor(l, 32);
+	if (row_ok)
+	{
+		float* dst = da.ws + (((int64_t)kvh * da.splits + split) * da.rows + n) * (D + 2);
+#pragma unroll
+		for (int c = 0; c < DC; ++c) *reinterpret_cast<float4_t*>(dst + 16 * c + 4 * g) = o[c];
+		if (g == 0)
+		{
+			dst[D] = m_run;
+			dst[D + 1] = l;
+		}
+	}
+}
+
+// One block per (key / value head, row), one thread per output column.  The first threads fetch the maxima and
+// sums of the splits in parallel and leave the weights 2^(m_i - M) in LDS; the column sums then run over
+// independent loads.
+template <int D>
+__global__ __launch_bounds__(D) void sdp_decode_merge_kernel(const float* __restrict__ ws, half_t* __restrict__ y, int rows, int splits)
+{
+	__shared__ float weight[kDecodeMaxSplits];
+	__shared__ float total;
+	const int row = blockIdx.x, kvh = blockIdx.y, d = threadIdx.x;
+	const float* base = ws + (((int64_t)kvh * splits) * rows + row) * (D + 2);
+	const int64_t step = (int64_t)rows * (D + 2);
+	if (d < kWaveSize)
+	{
+		// splits <= 64: one split per lane of the first wave
+		const float m = d < splits ? base[d * step + D] : -INFINITY;
+		const float l = d < splits ? base[d * step + D + 1] : 0.0f;
+		const float big = wave_allreduce(m, MaxOp());
+		const float w = fast_exp2(m - (big == -INFINITY ? 0.0f : big));
+		const float sum = wave_allreduce(l * w, SumOp());
+		if (d < splits) weight[d] = w;
+		if (d == 0) total = sum;
+	}
+	__syncthreads();
+	float acc = 0.0f;
+#pragma unroll 8
+	for (int i = 0; i < splits; ++i) acc += base[i * step + d] * weight[i];
+	const float sum = total;
+	y[((int64_t)kvh * rows + row) * D + d] = (half_t)(sum > 0.0f ? acc / sum : 0.0f);
+}
+
+struct DecodePlan
+{
+	int t_first, t_last, splits, tiles_per_split;
+};
+
+DecodePlan plan_decode(int64_t kv_heads, int64_t n_q, int64_t n_k, int causal, int64_t window)
+{
+	// visible key tiles of a group: its first query decides the low end, its last the high end
+	const int64_t diag = n_k - n_q;
+	int64_t key_hi = n_k - 1;
+	if (causal && (n_q - 1) + diag < key_hi) key_hi = (n_q - 1) + diag;
+	int64_t key_lo = 0;
+	if (window > 0 && diag - window + 1 > 0) key_lo = diag - window + 1;
+	DecodePlan p;
+	p.t_first = (int)(key_lo / kAttnKeysPerTile);
+	p.t_last = key_hi >= 0 ? (int)(key_hi / kAttnKeysPerTile) : p.t_first - 1;
+	const int64_t tiles = p.t_last - p.t_first + 1;
+	if (tiles <= 0)
+	{
+		p.splits = 1;
+		p.tiles_per_split = 0;
+		return p;
+	}
+	int64_t want = (kDecodeTargetWaves + kv_heads - 1) / kv_heads;
+	if (want > kDecodeMaxSplits) want = kDecodeMaxSplits;
+	if (want > tiles) want = tiles;
+	if (want < 1) want = 1;
+	p.tiles_per_split = (int)((tiles + want - 1) / want);
+	p.splits = (int)((tiles + p.tiles_per_split - 1) / p.tiles_per_split);
+	return p;
+}
+
+template <int D, bool SOFTCAP>
+hipError_t launch_decode_variant(const DecodeArgs& da, int64_t kv_heads, hipStream_t stream)
+{
+	constexpr int kLdsBytes = kAttnKeysPerTile * AttnLds<D>::kPitchV;
+	(void)hipGetLastError();
+	sdp_decode_partial_kernel<D, SOFTCAP><<<dim3((unsigned)da.splits, (unsigned)kv_heads), dim3(64), kLdsBytes, stream>>>(da);
+	hipError_t e = hipGetLastError();
+	if (e != hipSuccess) return e;
+	sdp_decode_merge_kernel<D><<<dim3((unsigned)da.rows, (unsigned)kv_heads), dim3(D), 0, stream>>>(da.ws, da.a.y, da.rows, da.splits);
+	return hipGetLastError();
+}
+
 }  // namespace
 
 bool sdp_attention_fwd_f16_supports(int64_t head_dim)
@@ -392,6 +644,58 @@ hipError_t launch_sdp_attention_fwd_f16(const void* q, const void* k, const void
 	case 128: return launch_dim<128>(args, capped, batch_heads, stream);
 	default: return launch_dim<256>(args, capped, batch_heads, stream);
 	}
+}
+
+bool sdp_attention_decode_f16_supports(int64_t q_per_kv, int64_t n_q, int64_t head_dim)
+{
+	return sdp_attention_fwd_f16_supports(head_dim) && q_per_kv >= 1 && n_q >= 1 && q_per_kv * n_q <= kDecodeMaxRows;
+}
+
+int64_t sdp_attention_decode_workspace_bytes(int64_t batch_heads, int64_t q_per_kv, int64_t n_q, int64_t n_k, int64_t head_dim,
+                                             int causal, int64_t window)
+{
+	if (batch_heads == 0 || n_q == 0) return 0;
+	const int64_t kv_heads = batch_heads / q_per_kv;
+	const DecodePlan p = plan_decode(kv_heads, n_q, n_k, causal, window);
+	return kv_heads * p.splits * (q_per_kv * n_q) * (head_dim + 2) * (int64_t)sizeof(float);
+}
+
+hipError_t launch_sdp_attention_decode_f16(const void* q, const void* k, const void* v, void* y, void* workspace,
+                                           int64_t batch_heads, int64_t q_per_kv, int64_t n_q, int64_t n_k, int64_t head_dim,
+                                           float alpha, float softcap, int causal, int64_t window, hipStream_t stream)
+{
+	if (batch_heads == 0 || n_q == 0) return hipSuccess;
+	const int64_t kv_heads = batch_heads / q_per_kv;
+	const DecodePlan p = plan_decode(kv_heads, n_q, n_k, causal, window);
+	DecodeArgs da;
+	da.a.q = static_cast<const half_t*>(q);
+	da.a.k = static_cast<const half_t*>(k);
+	da.a.v = static_cast<const half_t*>(v);
+	da.a.y = static_cast<half_t*>(y);
+	da.a.n_q = (int)n_q;
+	da.a.n_k = (int)n_k;
+	da.a.q_per_kv = (int)q_per_kv;
+	da.a.diag = (int)(n_k - n_q);
+	da.a.causal = causal ? 1 : 0;
+	da.a.window = (int)window;
+	const bool capped = softcap != 0.0f;
+	da.a.k_in = capped ? 2.0f * kLog2e * alpha / softcap : alpha * kLog2e;
+	da.a.k_cap = capped ? softcap * kLog2e : 0.0f;
+	da.ws = static_cast<float*>(workspace);
+	da.rows = (int)(q_per_kv * n_q);
+	da.splits = p.splits;
+	da.tiles_per_split = p.tiles_per_split;
+	da.t_first = p.t_first;
+	da.t_last = p.t_last;
+#define ANYGPU_DECODE_DIM(DIM) \
+	return capped ? launch_decode_variant<DIM, true>(da, kv_heads, stream) : launch_decode_variant<DIM, false>(da, kv_heads, stream)
+	switch (head_dim)
+	{
+	case 64: ANYGPU_DECODE_DIM(64);
+	case 128: ANYGPU_DECODE_DIM(128);
+	default: ANYGPU_DECODE_DIM(256);
+	}
+#undef ANYGPU_DECODE_DIM
 }
 
 }  // namespace anygpu

@@ -89,6 +89,32 @@ int check_batch(int64_t batch, int64_t stride_a, int64_t stride_b, int64_t strid
 	return ANYGPU_OK;
 }
 
+int check_attention_shape(int64_t batch_heads, int64_t q_per_kv, int64_t n_q, int64_t n_k, int64_t head_dim, int64_t window)
+{
+	if (batch_heads < 0 || n_q < 0 || n_k < 0 || head_dim < 0 || window < 0) return ANYGPU_ERR_BAD_SHAPE;
+	if (q_per_kv < 1 || batch_heads % q_per_kv != 0) return ANYGPU_ERR_BAD_SHAPE;
+	if (!anygpu::sdp_attention_fwd_f16_supports(head_dim)) return ANYGPU_ERR_UNSUPPORTED;
+	if (batch_heads > 65535) return ANYGPU_ERR_TOO_LARGE;                        // one grid row per head
+	// query and key indices, their sums and differences with the window stay inside 32 bits
+	if (n_q > kMaxIndex32 / 4 || n_k > kMaxIndex32 / 4 || window > kMaxIndex32 / 4) return ANYGPU_ERR_TOO_LARGE;
+	return ANYGPU_OK;
+}
+
+int check_attention(const void* q, const void* k, const void* v, const void* y, int64_t batch_heads, int64_t q_per_kv,
+                    int64_t n_q, int64_t n_k, int64_t head_dim, float alpha, float softcap, int64_t window)
+{
+	const int rc = check_attention_shape(batch_heads, q_per_kv, n_q, n_k, head_dim, window);
+	if (rc != ANYGPU_OK) return rc;
+	if (!(softcap >= 0.0f) || !std::isfinite(softcap) || !std::isfinite(alpha)) return ANYGPU_ERR_UNSUPPORTED;
+	if (batch_heads == 0 || n_q == 0) return ANYGPU_OK;
+	if (q == nullptr || y == nullptr) return ANYGPU_ERR_NULL_POINTER;
+	if (n_k > 0 && (k == nullptr || v == nullptr)) return ANYGPU_ERR_NULL_POINTER;
+	const uintptr_t bits = reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) | reinterpret_cast<uintptr_t>(v) |
+	                       reinterpret_cast<uintptr_t>(y);
+	if (bits % 16 != 0) return ANYGPU_ERR_UNSUPPORTED;
+	return ANYGPU_OK;
+}
+
 template <typename T>
 int conv_update_entry(const void* x, void* state, const void* w, const void* b, void* y,
                       int64_t batch, int64_t chan, int64_t width, void* stream)
@@ -256,21 +282,38 @@ ANYGPU_EXPORT int anygpu_sdp_attention_fwd_f16(const void* q, const void* k, con
                                                int64_t batch_heads, int64_t q_per_kv, int64_t n_q, int64_t n_k, int64_t head_dim,
                                                float alpha, float softcap, int causal, int64_t window, void* stream)
 {
-	if (batch_heads < 0 || n_q < 0 || n_k < 0 || head_dim < 0 || window < 0) return ANYGPU_ERR_BAD_SHAPE;
-	if (q_per_kv < 1 || batch_heads % q_per_kv != 0) return ANYGPU_ERR_BAD_SHAPE;
-	if (!anygpu::sdp_attention_fwd_f16_supports(head_dim)) return ANYGPU_ERR_UNSUPPORTED;
-	if (!(softcap >= 0.0f) || !std::isfinite(softcap) || !std::isfinite(alpha)) return ANYGPU_ERR_UNSUPPORTED;
+	const int rc = check_attention(q, k, v, y, batch_heads, q_per_kv, n_q, n_k, head_dim, alpha, softcap, window);
+	if (rc != ANYGPU_OK) return rc;
 	if (batch_heads == 0 || n_q == 0) return ANYGPU_OK;
-	if (q == nullptr || y == nullptr) return ANYGPU_ERR_NULL_POINTER;
-	if (n_k > 0 && (k == nullptr || v == nullptr)) return ANYGPU_ERR_NULL_POINTER;
-	if (batch_heads > 65535) return ANYGPU_ERR_TOO_LARGE;                        // one grid row per head
-	// query and key indices, their sums and differences with the window stay inside 32 bits
-	if (n_q > kMaxIndex32 / 4 || n_k > kMaxIndex32 / 4 || window > kMaxIndex32 / 4) return ANYGPU_ERR_TOO_LARGE;
-	const uintptr_t bits = reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) | reinterpret_cast<uintptr_t>(v) |
-	                       reinterpret_cast<uintptr_t>(y);
-	if (bits % 16 != 0) return ANYGPU_ERR_UNSUPPORTED;
 	return (int)anygpu::launch_sdp_attention_fwd_f16(q, k, v, y, batch_heads, q_per_kv, n_q, n_k, head_dim, alpha, softcap,
 	                                                 causal, window, as_stream(stream));
+}
+
+ANYGPU_EXPORT int64_t anygpu_sdp_attention_decode_workspace_bytes(int64_t batch_heads, int64_t q_per_kv, int64_t n_q, int64_t n_k,
+                                                                  int64_t head_dim, int causal, int64_t window)
+{
+	const int rc = check_attention_shape(batch_heads, q_per_kv, n_q, n_k, head_dim, window);
+	if (rc != ANYGPU_OK) return rc;
+	if (batch_heads == 0 || n_q == 0) return 0;
+	if (!anygpu::sdp_attention_decode_f16_supports(q_per_kv, n_q, head_dim)) return ANYGPU_ERR_UNSUPPORTED;
+	return anygpu::sdp_attention_decode_workspace_bytes(batch_heads, q_per_kv, n_q, n_k, head_dim, causal, window);
+}
+
+ANYGPU_EXPORT int anygpu_sdp_attention_decode_f16(const void* q, const void* k, const void* v, void* y,
+                                                  void* workspace, int64_t workspace_bytes,
+                                                  int64_t batch_heads, int64_t q_per_kv, int64_t n_q, int64_t n_k, int64_t head_dim,
+                                                  float alpha, float softcap, int causal, int64_t window, void* stream)
+{
+	const int rc = check_attention(q, k, v, y, batch_heads, q_per_kv, n_q, n_k, head_dim, alpha, softcap, window);
+	if (rc != ANYGPU_OK) return rc;
+	if (batch_heads == 0 || n_q == 0) return ANYGPU_OK;
+	if (!anygpu::sdp_attention_decode_f16_supports(q_per_kv, n_q, head_dim)) return ANYGPU_ERR_UNSUPPORTED;
+	const int64_t need = anygpu::sdp_attention_decode_workspace_bytes(batch_heads, q_per_kv, n_q, n_k, head_dim, causal, window);
+	if (workspace == nullptr) return ANYGPU_ERR_NULL_POINTER;
+	if (workspace_bytes < need) return ANYGPU_ERR_BAD_SHAPE;
+	if (reinterpret_cast<uintptr_t>(workspace) % 16 != 0) return ANYGPU_ERR_UNSUPPORTED;
+	return (int)anygpu::launch_sdp_attention_decode_f16(q, k, v, y, workspace, batch_heads, q_per_kv, n_q, n_k, head_dim, alpha,
+	                                                    softcap, causal, window, as_stream(stream));
 }
 
 ANYGPU_EXPORT int anygpu_causal_conv1d_silu_f16(const void* x, const void* w, const void* bias, void* y,

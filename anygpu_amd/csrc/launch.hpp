@@ -61,6 +61,15 @@ hipError_t launch_sdp_attention_fwd_f16(const void* q, const void* k, const void
                                         int64_t batch_heads, int64_t q_per_kv, int64_t n_q, int64_t n_k, int64_t head_dim,
                                         float alpha, float softcap, int causal, int64_t window, hipStream_t stream);
 
+// Decode form of the fused attention (q_per_kv * n_q <= 16 rows per key / value head): the key range is split over
+// waves, partial results go through `workspace` (sdp_attention_decode_workspace_bytes of fp32 scratch, 16-byte aligned).
+bool sdp_attention_decode_f16_supports(int64_t q_per_kv, int64_t n_q, int64_t head_dim);
+int64_t sdp_attention_decode_workspace_bytes(int64_t batch_heads, int64_t q_per_kv, int64_t n_q, int64_t n_k, int64_t head_dim,
+                                             int causal, int64_t window);
+hipError_t launch_sdp_attention_decode_f16(const void* q, const void* k, const void* v, void* y, void* workspace,
+                                           int64_t batch_heads, int64_t q_per_kv, int64_t n_q, int64_t n_k, int64_t head_dim,
+                                           float alpha, float softcap, int causal, int64_t window, hipStream_t stream);
+
 // Few-row products (M <= kSkinnyMaxRows, one product, row-major A): bandwidth-shaped kernels that
 // stream B once.  `epilogue` is an Epilogue value; B2 only for kEpiGeluMul, bias only for kEpiBias
 // (either may be NULL).  T is float or _Float16.  gemm_skinny_applies says whether shape, leading

@@ -183,6 +183,25 @@ int anygpu_sdp_attention_fwd_f16(const void* q, const void* k, const void* v, vo
                                  float alpha, float softcap, int causal, int64_t window, void* stream);
 
 /*
+ * Decode form of anygpu_sdp_attention_fwd_f16 for generation steps: few queries per head, long key range.  Same
+ * arguments, meaning and result; additionally q_per_kv * n_q <= 16 (the queries of the heads that share a key /
+ * value head are processed together, so k and v are read once per key / value head) and a workspace: the visible
+ * key range is split over up to 64 waves per key / value head, whose partial results (running maximum, sum and
+ * unnormalised accumulators, fp32) pass through `workspace` and are merged by a second kernel on the same stream.
+ * anygpu_sdp_attention_decode_workspace_bytes returns the bytes needed for a shape (a negative error code for
+ * arguments the decode form rejects); workspace must be 16-byte aligned device memory of at least that size and
+ * may be reused by the next call on the same stream.  The reference has no decode kernel: its generation step
+ * runs the per-head loop of srcs/transformers/sdp.hpp:258-271 against the cached keys.
+ */
+int64_t anygpu_sdp_attention_decode_workspace_bytes(int64_t batch_heads, int64_t q_per_kv, int64_t n_q, int64_t n_k,
+                                                    int64_t head_dim, int causal, int64_t window);
+
+int anygpu_sdp_attention_decode_f16(const void* q, const void* k, const void* v, void* y,
+                                    void* workspace, int64_t workspace_bytes,
+                                    int64_t batch_heads, int64_t q_per_kv, int64_t n_q, int64_t n_k, int64_t head_dim,
+                                    float alpha, float softcap, int causal, int64_t window, void* stream);
+
+/*
  * Depthwise causal conv1d with bias and fused SiLU:
  *     y[b, d, s] = silu( bias[d] + sum_{k=0}^{width-1} w[d, k] * x[b, d, s + k - (width - 1)] ),
  * terms with a negative sequence index dropped (left zero padding of width-1).

@@ -818,6 +818,77 @@ def test_sdp_attention_fused_kernel_many_heads_d128(ops, oracle):
         assert scaled_rel_err(got[i:i + 4], part.astype(np.float32), 1.0) <= 2e-3
 
 
+DECODE_CASES = [
+    # heads, kv_heads, n_q, n_k, d, alpha, softcap, causal, window
+    (8, 4, 1, 4500, 256, 0.0625, 50.0, True, 4096),       # Gemma2 generation step: window cuts the cache
+    (32, 8, 1, 1000, 128, 0.0884, 0.0, True, 0),
+    (16, 16, 1, 300, 64, 0.125, 0.0, False, 0),
+    (8, 2, 4, 2049, 128, 0.0884, 0.0, True, 0),           # 4 query heads x 4 queries = 16 rows per key / value head
+    (4, 4, 3, 777, 64, 0.125, 30.0, True, 100),
+    (2, 1, 1, 63, 128, 0.0884, 0.0, True, 0),             # less than one tile of keys
+    (4, 2, 5, 3, 64, 0.125, 0.0, True, 0),                # more queries than keys: the first two see nothing
+]
+
+
+@pytest.mark.parametrize("case", DECODE_CASES)
+def test_sdp_attention_decode_form(ops, oracle, case):
+    heads, kv_heads, n_q, n_k, d, alpha, cap, causal, window = case
+    q = synth.normal(1 + n_q, (1, heads, n_q, d)).astype(np.float16)
+    k = synth.normal(2 + n_k, (1, kv_heads, n_k, d)).astype(np.float16)
+    v = synth.normal(3 + d, (1, kv_heads, n_k, d)).astype(np.float16)
+    got = host(ops.sdp_attention_fwd(dev(q), dev(k), dev(v), alpha, softcap=cap, causal=causal, window=window,
+                                     decode=True)).astype(np.float32)
+    want = oracle.sdp_attention_rules(*(oracle.cvt_f16_to_f32(t)[0] for t in (q, k, v)), alpha=alpha, softcap=cap,
+                                      causal=causal, window=window, q_per_kv=heads // kv_heads, threads=8)
+    # a query that sees no key: the operator chain divides 0 by 0 (NaN), the kernels give zeros
+    blind = np.isnan(want).all(axis=(0, 2))
+    assert blind.sum() == (max(n_q - n_k, 0) if causal else 0)
+    assert not got[0][:, blind, :].any()
+    assert scaled_rel_err(got[0][:, ~blind, :], want[:, ~blind, :], 1.0) <= TOL_F16_ROWOPS * 2
+    # and against the fused form of the same arguments
+    fused = host(ops.sdp_attention_fwd(dev(q), dev(k), dev(v), alpha, softcap=cap, causal=causal, window=window,
+                                       decode=False)).astype(np.float32)
+    assert scaled_rel_err(got, fused, 1.0) <= 2e-3
+
+
+def test_sdp_attention_decode_workspace_and_rejected_arguments(ops):
+    import torch
+    from anygpu_amd import capi
+    lib = capi.load()
+    ws_bytes = lib.anygpu_sdp_attention_decode_workspace_bytes
+    # 4 key / value heads, 2 rows each, 4096 visible keys = 64 tiles -> 64 splits: 4 * 64 * 2 * (256 + 2) floats
+    assert ws_bytes(8, 2, 1, 8192, 256, 1, 4096) == 4 * 64 * 2 * 258 * 4
+    assert ws_bytes(8, 2, 1, 100, 256, 1, 0) == 4 * 2 * 2 * 258 * 4          # 2 tiles -> 2 splits
+    assert ws_bytes(0, 1, 1, 100, 64, 1, 0) == 0
+    assert ws_bytes(8, 2, 9, 100, 64, 1, 0) == capi.ANYGPU_ERR_UNSUPPORTED   # 18 rows per key / value head
+    assert ws_bytes(8, 3, 1, 100, 64, 1, 0) == capi.ANYGPU_ERR_BAD_SHAPE
+    q = torch.zeros((4, 1, 64), device="cuda", dtype=torch.float16)
+    kv = torch.zeros((2, 500, 64), device="cuda", dtype=torch.float16)
+    y = torch.full_like(q, 3.0)
+    need = ws_bytes(4, 2, 1, 500, 64, 1, 0)
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    f = lib.anygpu_sdp_attention_decode_f16
+    args = (4, 2, 1, 500, 64, 0.125, 0.0, 1, 0, None)
+    assert f(q.data_ptr(), kv.data_ptr(), kv.data_ptr(), y.data_ptr(), None, need, *args) == capi.ANYGPU_ERR_NULL_POINTER
+    assert f(q.data_ptr(), kv.data_ptr(), kv.data_ptr(), y.data_ptr(), ws.data_ptr(), need - 1, *args) == capi.ANYGPU_ERR_BAD_SHAPE
+    assert f(q.data_ptr(), kv.data_ptr(), kv.data_ptr(), y.data_ptr(), ws.data_ptr() + 4, need, *args) == capi.ANYGPU_ERR_UNSUPPORTED
+    torch.cuda.synchronize()
+    assert bool((y == 3.0).all())
+    # a workspace larger than needed and reused by a second, smaller call
+    big = torch.empty(need + 4096, dtype=torch.uint8, device="cuda")
+    qr = torch.randn((4, 1, 64), device="cuda", dtype=torch.float16)
+    kr = torch.randn((2, 500, 64), device="cuda", dtype=torch.float16)
+    vr = torch.randn((2, 500, 64), device="cuda", dtype=torch.float16)
+    for n_k in (500, 130):
+        out = torch.empty_like(qr)
+        kk, vv = kr[:, :n_k].contiguous(), vr[:, :n_k].contiguous()
+        assert f(qr.data_ptr(), kk.data_ptr(), vv.data_ptr(), out.data_ptr(), big.data_ptr(), big.numel(),
+                 4, 2, 1, n_k, 64, 0.125, 0.0, 1, 0, None) == capi.ANYGPU_OK
+        ref = ops.sdp_attention_fwd(qr, kk, vv, 0.125, causal=True, decode=False)
+        torch.cuda.synchronize()
+        assert float((out.float() - ref.float()).abs().max()) <= 2e-3
+
+
 def test_sdp_attention_fused_kernel_gemma2_block(ops, oracle):
     # Gemma2 attention at the softmax configuration of the headline set: 8 query heads over 4 key / value heads,
     # head_dim 256, scale 1 / 16, softcap 50, causal + window 4096; 6144 positions so that the window cuts
