@@ -565,6 +565,33 @@ TEST_CASE(test_sdp_attention_rules_fused_f16, GPU)
 	return ok && compare_data_buffers_l2(got16, want16, 4e-3f);
 }
 
+TEST_CASE(test_sdp_attention_rules_decode_step_f16, GPU)
+{
+	// generation step over a cache of 700 keys: 8 query heads on 4 key / value heads, d = 128, causal + window;
+	// the split-key form (picked by the shape) against the operator chain on the host
+	const int64 h = 8, hkv = 4, n_k = 700, d = 128;
+	auto hq16 = cvt_tensor_from_float32<float16>(crt_random_normal_tensor<float32, CPU>({ 1, h, 1, d }, 1));
+	auto hk16 = cvt_tensor_from_float32<float16>(crt_random_normal_tensor<float32, CPU>({ 1, hkv, n_k, d }, 2));
+	auto hv16 = cvt_tensor_from_float32<float16>(crt_random_normal_tensor<float32, CPU>({ 1, hkv, n_k, d }, 3));
+	SoftmaxPrologue rules;
+	rules.alpha = 0.0884f;
+	rules.causal = true;
+	rules.window = 512;
+	auto dq = hq16.copy_to_cuda(), dk = hk16.copy_to_cuda(), dv = hv16.copy_to_cuda();
+	bool ok = hip_flash_sdpa_decode_applies(dq, dk);
+	auto got = cvt_tensor_datatype<float32, float16>(sdp_attention_rules_fwd(dq, dk, dv, rules).copy_to_host());
+	auto hk = cvt_tensor_datatype<float32, float16>(hk16);
+	auto hv = cvt_tensor_datatype<float32, float16>(hv16);
+	Tensor<float32, CPU> hk_rep(std::vector<int64>({ 1, h, n_k, d })), hv_rep(std::vector<int64>({ 1, h, n_k, d }));
+	for (int64 head = 0; head < h; ++head)
+	{
+		std::memcpy(hk_rep.buffer() + head * n_k * d, hk.buffer() + (head / 2) * n_k * d, n_k * d * sizeof(float32));
+		std::memcpy(hv_rep.buffer() + head * n_k * d, hv.buffer() + (head / 2) * n_k * d, n_k * d * sizeof(float32));
+	}
+	auto want = sdp_attention_rules_fwd(cvt_tensor_datatype<float32, float16>(hq16), hk_rep, hv_rep, rules);
+	return ok && elementwise_compatible(got, want) && compare_data_buffers_l2(got, want, 4e-3f) && compare_data_buffers(got, want, 2e-2f);
+}
+
 TEST_CASE(test_gemma2_decoder_mlp_1x21x256_i1024, GPU)
 {
 	// the whole block (gate / up, activation, product, down) against the operator chain on the host

@@ -20,4 +20,26 @@ void hip_flash_sdpa_fwd_f16(
 	const Tensor<float16, CUDA>& vt,
 	Tensor<float16, CUDA>& yt);
 
+/*
+  Decode form for generation steps: (query heads per key / value head) x n_q <= 16.  The key range is split over
+  many waves; their partial results pass through `workspace`, a float32 tensor with at least
+  hip_flash_sdpa_decode_workspace_floats(...) elements, which the caller owns and may reuse.
+*/
+bool hip_flash_sdpa_decode_applies(
+	const Tensor<float16, CUDA>& qt,
+	const Tensor<float16, CUDA>& kt);
+
+int64 hip_flash_sdpa_decode_workspace_floats(
+	const SoftmaxPrologue& prologue,
+	const Tensor<float16, CUDA>& qt,
+	const Tensor<float16, CUDA>& kt);
+
+void hip_flash_sdpa_decode_f16(
+	const SoftmaxPrologue& prologue,
+	const Tensor<float16, CUDA>& qt,
+	const Tensor<float16, CUDA>& kt,
+	const Tensor<float16, CUDA>& vt,
+	Tensor<float32, CUDA>& workspace,
+	Tensor<float16, CUDA>& yt);
+
 #endif  // __FLASH_SDPA_FWD_CUH__

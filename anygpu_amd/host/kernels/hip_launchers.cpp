@@ -347,3 +347,52 @@ void hip_flash_sdpa_fwd_f16(const SoftmaxPrologue& prologue, const Tensor<float1
 	                                       kv_heads > 0 ? heads / kv_heads : 1, n_q, n_k, d, prologue.alpha, prologue.softcap,
 	                                       prologue.causal ? 1 : 0, prologue.window, kNullStream));
 }
+
+namespace {
+
+struct AttentionShape
+{
+	int64 batch_heads, q_per_kv, n_q, n_k, d;
+};
+
+AttentionShape attention_shape(const Tensor<float16, CUDA>& qt, const Tensor<float16, CUDA>& kt)
+{
+	const int64 dim = qt.dim;
+	AttentionShape s;
+	s.n_q = qt.shape[dim - 2];
+	s.d = qt.shape[dim - 1];
+	s.n_k = kt.shape[dim - 2];
+	const int64 heads = dim >= 3 ? qt.shape[dim - 3] : 1, kv_heads = dim >= 3 ? kt.shape[dim - 3] : 1;
+	s.q_per_kv = kv_heads > 0 ? heads / kv_heads : 1;
+	s.batch_heads = (s.n_q * s.d) > 0 ? qt.numel() / (s.n_q * s.d) : 0;
+	return s;
+}
+
+}  // namespace
+
+bool hip_flash_sdpa_decode_applies(const Tensor<float16, CUDA>& qt, const Tensor<float16, CUDA>& kt)
+{
+	const AttentionShape s = attention_shape(qt, kt);
+	// few rows per key / value head and enough keys for the split to pay
+	return s.q_per_kv * s.n_q >= 1 && s.q_per_kv * s.n_q <= 16 && s.n_k >= 256;
+}
+
+int64 hip_flash_sdpa_decode_workspace_floats(const SoftmaxPrologue& prologue, const Tensor<float16, CUDA>& qt,
+                                             const Tensor<float16, CUDA>& kt)
+{
+	const AttentionShape s = attention_shape(qt, kt);
+	const int64 bytes = anygpu_sdp_attention_decode_workspace_bytes(s.batch_heads, s.q_per_kv, s.n_q, s.n_k, s.d,
+	                                                                prologue.causal ? 1 : 0, prologue.window);
+	if (bytes < 0) check_abi(static_cast<int>(bytes), "anygpu_sdp_attention_decode_workspace_bytes", __FILE__, __LINE__);
+	return (bytes + 3) / 4;
+}
+
+void hip_flash_sdpa_decode_f16(const SoftmaxPrologue& prologue, const Tensor<float16, CUDA>& qt, const Tensor<float16, CUDA>& kt,
+                               const Tensor<float16, CUDA>& vt, Tensor<float32, CUDA>& workspace, Tensor<float16, CUDA>& yt)
+{
+	const AttentionShape s = attention_shape(qt, kt);
+	ABI_CHECK(anygpu_sdp_attention_decode_f16(qt.buffer(), kt.buffer(), vt.buffer(), yt.buffer(), workspace.buffer(),
+	                                          workspace.numel() * static_cast<int64>(sizeof(float32)), s.batch_heads, s.q_per_kv,
+	                                          s.n_q, s.n_k, s.d, prologue.alpha, prologue.softcap, prologue.causal ? 1 : 0,
+	                                          prologue.window, kNullStream));
+}

@@ -176,7 +176,16 @@ inline Tensor<dtype, device> sdp_attention_rules_fwd(
 		ACASSERT(d == 64 || d == 128 || d == 256, "hidden dimension must be 64, 128 or 256");
 		ACASSERT(rules.softcap >= 0.f && rules.window >= 0, "softcap and window must not be negative");
 		Tensor<dtype, CUDA> y(qw.dim, qw.shape);
-		hip_flash_sdpa_fwd_f16(rules, qw, kw, vw, y);
+		if (hip_flash_sdpa_decode_applies(qw, kw))
+		{
+			// generation step: the split-key form; its scratch lives for this call only
+			Tensor<float32, CUDA> workspace(std::vector<int64>{ std::max<int64>(hip_flash_sdpa_decode_workspace_floats(rules, qw, kw), 4) });
+			hip_flash_sdpa_decode_f16(rules, qw, kw, vw, workspace, y);
+		}
+		else
+		{
+			hip_flash_sdpa_fwd_f16(rules, qw, kw, vw, y);
+		}
 		return y;
 	}
 	else
