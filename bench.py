@@ -36,7 +36,8 @@ PEAK_HBM_GBS = 8000.0          # HBM3E
 # dispatch), scaled by what the same counters read for a plain 256 MiB device copy (fetch x 2.000,
 # write x 1.000); the summaries are under profiles/.
 MEASURED_TRAFFIC_BYTES = {"gemm_f16": 234962687, "gemm_f32": 167994164, "conv1d": 277226336,
-                          "softmax_causal": 410887952, "softmax_gemma2": 1514268488}
+                          "softmax_causal": 410887952, "softmax_gemma2": 1514268488,
+                          "attention_gemma2": 689788928, "gated_rmsnorm": 805489664}
 
 
 def parse_args():
@@ -190,7 +191,7 @@ def bench_attention(torch, ops, steps, warmup):
         "workload": "fused attention fp16 q [1, 8, 8192, 256], k / v [1, 4, 8192, 256], x 1/16, softcap 50, causal + window 4096",
         "us_per_launch": t * 1e6, "value": flops / t / 1e12, "unit": "TFLOP/s", "dtype": "f16",
         "roofline": {"bound": "mfma", "achieved": flops / t / 1e12, "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": flops / t / 1e12 / PEAK_FP16_TFLOPS, "traffic": None,
+                     "frac": flops / t / 1e12 / PEAK_FP16_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES["attention_gemma2"],
                      "algorithmic_flops": flops, "visible_pairs_per_head": pairs},
     }
 
@@ -217,7 +218,8 @@ def bench_gated_rmsnorm(torch, ops, steps, warmup):
         "name": "gated_rmsnorm_f16", "workload": "gated RMS norm fp16 x, z [16384, 8192], w [8192], eps 1e-5",
         "us_per_launch": t * 1e6, "value": nbytes / t / 1e9, "unit": "GB/s", "dtype": "f16",
         "roofline": {"bound": "hbm", "achieved": nbytes / t / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                     "frac": nbytes / t / 1e9 / PEAK_HBM_GBS, "traffic": None, "algorithmic_bytes": nbytes},
+                     "frac": nbytes / t / 1e9 / PEAK_HBM_GBS, "traffic": MEASURED_TRAFFIC_BYTES["gated_rmsnorm"],
+                     "algorithmic_bytes": nbytes},
     }
 
 
