@@ -106,36 +106,39 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
 	const bool aligned = (reinterpret_cast<uintptr_t>(A) % 16 == 0) && (reinterpret_cast<uintptr_t>(B) % 16 == 0) &&
 	                     (reinterpret_cast<uintptr_t>(C) % 16 == 0) && (lda % 8 == 0) && (ldb % 8 == 0) && (ldc % 8 == 0) &&
 	                     (stride_a % 8 == 0) && (stride_b % 8 == 0) && (stride_c % 8 == 0);
-	if (b_layout == ANYGPU_B_COL_MAJOR && aligned && K > 0 && K % 64 == 0)
+	if (aligned && K >= 64 && K % 8 == 0 && N % 8 == 0)
 	{
-		// 8 waves, 128 x 64 patch per wave, 64-bank swizzle, one LDS read behind each of the first
-		// MFMAs, 16 x 16 x 32 MFMA.  Both MFMA shapes have the same peak rate, but under this kernel
-		// the chip is power-limited and the 16 x 16 x 32 form measured 13 % faster at 4096^3
-		// (99 us against 114 us for 32 x 32 x 16 with the same tiling).
-		using Big = GemmTileCfg<256, 256, 2, 4, 1, 0, 4, 16>;
-		// 4 waves, 64 x 64 patch per wave: two blocks fit a CU; for shapes that are not multiples of 256
-		using Small = GemmTileCfg<128, 128, 2, 2, 1, 0, 4, 16>;
-		if (M % 256 == 0 && N % 256 == 0 && (M / 256) * (N / 256) <= 0x7FFFFFFFLL)
-			return launch_gemm_f16_tile<Big>(a, b, c, M, N, K, lda, ldb, ldc, stride_a, stride_b, stride_c, batch, stream);
-		if (M % 128 == 0 && N % 128 == 0 && (M / 128) * (N / 128) <= 0x7FFFFFFFLL)
-			return launch_gemm_f16_tile<Small>(a, b, c, M, N, K, lda, ldb, ldc, stride_a, stride_b, stride_c, batch, stream);
-		// 4 waves, 32 x 32 patch per wave: the granularity the reference's own fp16 kernels require
-		using Tiny = GemmTileCfg<64, 64, 2, 2, 1, 0, 4, 16>;
-		if (M % 64 == 0 && N % 64 == 0 && (M / 64) * (N / 64) <= 0x7FFFFFFFLL)
-			return launch_gemm_f16_tile<Tiny>(a, b, c, M, N, K, lda, ldb, ldc, stride_a, stride_b, stride_c, batch, stream);
-	}
-	if (b_layout == ANYGPU_B_ROW_MAJOR && aligned && K > 0 && K % 64 == 0)
-	{
-		// the reference layout, B stored [K, N]: same tiling, B operand through transposing LDS reads
-		using BigKN = GemmTileCfg<256, 256, 2, 4, 1, 0, 4, 16, true>;
-		using SmallKN = GemmTileCfg<128, 128, 2, 2, 1, 0, 4, 16, true>;
-		if (M % 256 == 0 && N % 256 == 0 && (M / 256) * (N / 256) <= 0x7FFFFFFFLL)
-			return launch_gemm_f16_tile<BigKN>(a, b, c, M, N, K, lda, ldb, ldc, stride_a, stride_b, stride_c, batch, stream);
-		if (M % 128 == 0 && N % 128 == 0 && (M / 128) * (N / 128) <= 0x7FFFFFFFLL)
-			return launch_gemm_f16_tile<SmallKN>(a, b, c, M, N, K, lda, ldb, ldc, stride_a, stride_b, stride_c, batch, stream);
-		using TinyKN = GemmTileCfg<64, 64, 2, 2, 1, 0, 4, 16, true>;
-		if (M % 64 == 0 && N % 64 == 0 && (M / 64) * (N / 64) <= 0x7FFFFFFFLL)
-			return launch_gemm_f16_tile<TinyKN>(a, b, c, M, N, K, lda, ldb, ldc, stride_a, stride_b, stride_c, batch, stream);
+		// Tile kernels.  Big: 8 waves, 128 x 64 patch per wave, 64-bank swizzle, one LDS read behind each of the
+		// first MFMAs, 16 x 16 x 32 MFMA (both MFMA shapes have the same peak rate, but under this kernel the chip
+		// is power-limited and the 16 x 16 x 32 form measured 13 % faster at 4096^3: 99 us against 114 us for
+		// 32 x 32 x 16 with the same tiling).  Small: 4 waves, 64 x 64 patch per wave, two blocks fit a CU.
+		// Tiny: 4 waves, 32 x 32 patch per wave, the granularity the reference's own fp16 kernels require.
+		// The KN forms take the reference layout, B stored [K, N], through transposing LDS reads.
+		// The largest tile that still gives the chip enough blocks is taken; shapes that are not multiples of
+		// it run the same kernels with clamped operand rows and guarded stores; a K that is not a multiple of the
+		// 64-deep slab adds a tail multiplied from registers.
+		const auto blocks = [&](int64_t tile) { return ((M + tile - 1) / tile) * ((N + tile - 1) / tile) * batch; };
+		constexpr int64_t kEnoughBlocks = 192;
+		const int64_t tile = blocks(256) >= kEnoughBlocks ? 256 : blocks(128) >= kEnoughBlocks ? 128 : 64;
+		// one "general" instantiation serves ragged M / N and a K tail alike
+		const bool ragged = (M % tile != 0) || (N % tile != 0) || (K % 64 != 0);
+		const bool fits = ((M + tile - 1) / tile) * ((N + tile - 1) / tile) <= 0x7FFFFFFFLL;
+#define ANYGPU_F16_TILE(BT, WM, WN, KN) \
+		return ragged ? launch_gemm_f16_tile<GemmTileCfg<BT, BT, WM, WN, 1, 0, 4, 16, KN>, true, true>(a, b, c, M, N, K, lda, ldb, ldc, stride_a, stride_b, stride_c, batch, stream) \
+		              : launch_gemm_f16_tile<GemmTileCfg<BT, BT, WM, WN, 1, 0, 4, 16, KN>, false, false>(a, b, c, M, N, K, lda, ldb, ldc, stride_a, stride_b, stride_c, batch, stream)
+		if (fits && b_layout == ANYGPU_B_COL_MAJOR)
+		{
+			if (tile == 256) ANYGPU_F16_TILE(256, 2, 4, false);
+			if (tile == 128) ANYGPU_F16_TILE(128, 2, 2, false);
+			ANYGPU_F16_TILE(64, 2, 2, false);
+		}
+		if (fits && b_layout == ANYGPU_B_ROW_MAJOR)
+		{
+			if (tile == 256) ANYGPU_F16_TILE(256, 2, 4, true);
+			if (tile == 128) ANYGPU_F16_TILE(128, 2, 2, true);
+			ANYGPU_F16_TILE(64, 2, 2, true);
+		}
+#undef ANYGPU_F16_TILE
 	}
 
 	const dim3 grid((unsigned)((N + 63) / 64), (unsigned)((M + 63) / 64), (unsigned)batch);

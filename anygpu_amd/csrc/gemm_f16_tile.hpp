@@ -158,10 +158,11 @@ __device__ __forceinline__ half4_t lds_read_transposed_b64(const char* lds_addr)
 // it back row by row, 16 bytes per lane, so that the global stores cover whole rows of the band.
 // The scratch row pitch is 16 bytes more than the row, which spreads the 8-byte writes of the
 // rows over the banks.  The caller guarantees that nobody still reads or fills LDS.
-template <typename Cfg>
+// RAGGED: rows at or beyond M and 8-column chunks at or beyond N (N a multiple of 8) are not stored.
+template <typename Cfg, bool RAGGED>
 __device__ __forceinline__ void store_patch_via_lds(
 	const typename MfmaShape<Cfg::MI>::Acc (&acc)[Cfg::kTilesM][Cfg::kTilesN], char* lds,
-	half_t* __restrict__ C, int64_t ldc, int64_t m_base, int64_t n_base, int wave, int lane)
+	half_t* __restrict__ C, int64_t ldc, int64_t m_base, int64_t n_base, int wave, int lane, int64_t M, int64_t N)
 {
 	using Shape = MfmaShape<Cfg::MI>;
 	constexpr int MI = Cfg::MI, TM = Cfg::kTilesM, TN = Cfg::kTilesN;
@@ -192,7 +193,8 @@ __device__ __forceinline__ void store_patch_via_lds(
 		{
 			const int row = pass * kRowsPerPass + lane / kLanesPerRow;
 			const int col16 = lane % kLanesPerRow;
-			if (kRowsPerPass <= MI || row < MI)
+			const bool inside = !RAGGED || (m_base + i * MI + row < M && n_base + col16 * 8 < N);
+			if ((kRowsPerPass <= MI || row < MI) && inside)
 			{
 				const half8_t v = *reinterpret_cast<const half8_t*>(scratch + row * kPitch + col16 * 16);
 				*reinterpret_cast<half8_t*>(C + (m_base + i * MI + row) * ldc + n_base + col16 * 8) = v;
@@ -212,11 +214,16 @@ constexpr int kSchedDsRead = 0x100;
 // registers by then: behind it the loads of slab t+2 go out (the stage they overwrite is no
 // longer read by anybody) and the first fragments of slab t+1 are fetched, all under the
 // shadow of the MFMAs of the last step of slab t.
-template <typename Cfg>
+// RAGGED: M and N need not be multiples of the tile (N a multiple of 8).  Operand rows past the
+// end are read from the last valid row instead (they only feed results that are not stored).
+// KTAIL: K need not be a multiple of the 64-deep slab (K >= 64, a multiple of 8).  The slabs cover
+// the multiple; the remaining K % 64 columns are multiplied after the loop from fragments that
+// every lane loads straight from global memory in the MFMA operand layout, zeros past K.
+template <typename Cfg, bool RAGGED = false, bool KTAIL = false>
 __global__ __launch_bounds__(Cfg::kThreads) void gemm_f16_nt_tile_kernel(
 	const half_t* __restrict__ A, const half_t* __restrict__ B, half_t* __restrict__ C,
 	int K, int64_t lda, int64_t ldb, int64_t ldc, int tiles_m, int tiles_n,
-	int64_t stride_a, int64_t stride_b, int64_t stride_c)
+	int64_t stride_a, int64_t stride_b, int64_t stride_c, int64_t M, int64_t N)
 {
 	using Shape = MfmaShape<Cfg::MI>;
 	// blockIdx.y walks a batch of independent products that share the shape
@@ -251,7 +258,9 @@ __global__ __launch_bounds__(Cfg::kThreads) void gemm_f16_nt_tile_kernel(
 	for (int i = 0; i < Cfg::kLoadsA; ++i)
 	{
 		const int row = 8 * (wave * Cfg::kLoadsA + i) + ld_row;
-		a_src[i] = A + (m0 + row) * lda + ((ld_pos ^ swizzle_of_row<Cfg::SWZ>(row)) << 3);
+		int64_t grow = m0 + row;
+		if (RAGGED && grow > M - 1) grow = M - 1;
+		a_src[i] = A + grow * lda + ((ld_pos ^ swizzle_of_row<Cfg::SWZ>(row)) << 3);
 	}
 	constexpr int kRowBytesKN = BN * 2;                 // [k][n] slab row
 	constexpr int kRowsPerLoadKN = 1024 / kRowBytesKN;  // k rows one direct load instruction fills
@@ -264,12 +273,16 @@ __global__ __launch_bounds__(Cfg::kThreads) void gemm_f16_nt_tile_kernel(
 			const int lanes_per_row = kWaveSize / kRowsPerLoadKN;
 			const int k = kRowsPerLoadKN * (wave * Cfg::kLoadsB + i) + lane / lanes_per_row;
 			const int pos = lane % lanes_per_row;
-			b_src[i] = B + (int64_t)k * ldb + n0 + ((pos ^ (kn_row_swizzle(k) & kChunkMaskKN)) << 3);
+			int64_t gcol = n0 + ((pos ^ (kn_row_swizzle(k) & kChunkMaskKN)) << 3);
+			if (RAGGED && gcol > N - 8) gcol = N - 8;
+			b_src[i] = B + (int64_t)k * ldb + gcol;
 		}
 		else
 		{
 			const int row = 8 * (wave * Cfg::kLoadsB + i) + ld_row;
-			b_src[i] = B + (n0 + row) * ldb + ((ld_pos ^ swizzle_of_row<Cfg::SWZ>(row)) << 3);
+			int64_t grow = n0 + row;
+			if (RAGGED && grow > N - 1) grow = N - 1;
+			b_src[i] = B + grow * ldb + ((ld_pos ^ swizzle_of_row<Cfg::SWZ>(row)) << 3);
 		}
 	}
 
@@ -418,18 +431,60 @@ __global__ __launch_bounds__(Cfg::kThreads) void gemm_f16_nt_tile_kernel(
 		__builtin_amdgcn_sched_group_barrier(kSchedVmemRead, Cfg::kLoadsA + Cfg::kLoadsB, 0);
 		interleave_reads();
 	}
+	if constexpr (KTAIL)
+	{
+		constexpr int kStepDepth = 512 / MI;                 // k covered by one MFMA
+		for (int k0 = ktiles * BK; k0 < K; k0 += kStepDepth)
+		{
+			const int kk = k0 + 8 * frag_kgroup;             // this lane's 8 consecutive k
+			half8_t at[TM], bt[TN];
+#pragma unroll
+			for (int i = 0; i < TM; ++i)
+			{
+				int64_t grow = m0 + wm * Cfg::kWaveM + i * MI + frag_row;
+				if (RAGGED && grow > M - 1) grow = M - 1;
+				half8_t v = {};
+				if (kk < K) v = *reinterpret_cast<const half8_t*>(A + grow * lda + kk);
+				at[i] = v;
+			}
+#pragma unroll
+			for (int j = 0; j < TN; ++j)
+			{
+				int64_t gcol = n0 + wn * Cfg::kWaveN + j * MI + frag_row;
+				if (RAGGED && gcol > N - 1) gcol = N - 1;
+				half8_t v = {};
+				if (kk < K)
+				{
+					if constexpr (Cfg::B_KN)
+					{
+#pragma unroll
+						for (int e = 0; e < 8; ++e) v[e] = B[(int64_t)(kk + e) * ldb + gcol];
+					}
+					else
+					{
+						v = *reinterpret_cast<const half8_t*>(B + gcol * ldb + kk);
+					}
+				}
+				bt[j] = v;
+			}
+#pragma unroll
+			for (int i = 0; i < TM; ++i)
+#pragma unroll
+				for (int j = 0; j < TN; ++j) acc[i][j] = Shape::mma(bt[j], at[i], acc[i][j]);
+		}
+	}
 	// no direct load may still be writing LDS when the scratch is reused or the block retires
 	wait_vmem_all();
 	__syncthreads();
-	store_patch_via_lds<Cfg>(acc, lds, C, ldc, m0 + wm * Cfg::kWaveM, n0 + wn * Cfg::kWaveN, wave, lane);
+	store_patch_via_lds<Cfg, RAGGED>(acc, lds, C, ldc, m0 + wm * Cfg::kWaveM, n0 + wn * Cfg::kWaveN, wave, lane, M, N);
 }
 
-template <typename Cfg>
+template <typename Cfg, bool RAGGED = false, bool KTAIL = false>
 hipError_t launch_gemm_f16_tile(const half_t* A, const half_t* B, half_t* C, int64_t M, int64_t N, int64_t K,
                                 int64_t lda, int64_t ldb, int64_t ldc,
                                 int64_t stride_a, int64_t stride_b, int64_t stride_c, int64_t batch, hipStream_t stream)
 {
-	auto kernel = gemm_f16_nt_tile_kernel<Cfg>;
+	auto kernel = gemm_f16_nt_tile_kernel<Cfg, RAGGED, KTAIL>;
 	// More than 64 KB of dynamic LDS has to be granted per function and per device, once.
 	static std::atomic<uint64_t> configured_devices{0};
 	(void)hipGetLastError();
@@ -444,9 +499,9 @@ hipError_t launch_gemm_f16_tile(const half_t* A, const half_t* B, half_t* C, int
 		if (e != hipSuccess) return e;
 		configured_devices.fetch_or(bit, std::memory_order_relaxed);
 	}
-	const int tiles_m = (int)(M / Cfg::BM), tiles_n = (int)(N / Cfg::BN);
+	const int tiles_m = (int)((M + Cfg::BM - 1) / Cfg::BM), tiles_n = (int)((N + Cfg::BN - 1) / Cfg::BN);
 	kernel<<<dim3((unsigned)(tiles_m * tiles_n), (unsigned)batch), dim3(Cfg::kThreads), Cfg::kLdsBytes, stream>>>(
-		A, B, C, (int)K, lda, ldb, ldc, tiles_m, tiles_n, stride_a, stride_b, stride_c);
+		A, B, C, (int)K, lda, ldb, ldc, tiles_m, tiles_n, stride_a, stride_b, stride_c, M, N);
 	return hipGetLastError();
 }
 

@@ -473,6 +473,45 @@ def test_mm_f16_tile_kernel_shapes(ops, oracle, m, k, n):
     assert np.array_equal(got_kn, got)
 
 
+@pytest.mark.parametrize("layout", ["row", "col"])
+@pytest.mark.parametrize("m,k,n", [(100, 64, 72), (130, 128, 264), (257, 192, 1000), (1000, 256, 520), (300, 64, 8),
+                                   (65, 64, 136), (9, 128, 4096), (2047, 64, 2056), (520, 320, 248),
+                                   (128, 72, 128), (256, 200, 256), (100, 136, 72), (1024, 1000, 1024), (300, 88, 520)])
+def test_mm_f16_ragged_shapes_through_tile_kernels(ops, oracle, layout, m, k, n):
+    # K >= 64 and K, N multiples of 8: the MFMA tile kernels with clamped operand rows, guarded stores and,
+    # when K is not a multiple of 64, a tail multiplied from registers
+    import torch
+    from anygpu_amd import capi
+    a = synth.uniform(m + k, (m, k)).astype(np.float16)
+    b = synth.uniform(k + n, (k, n)).astype(np.float16)
+    want = oracle.tensor_mm(oracle.cvt_f16_to_f32(a), oracle.cvt_f16_to_f32(b), threads=8)
+    # the result sits inside a larger buffer: nothing outside [m, n] may be touched
+    cbuf = torch.full((m + 3, n + 16), -7.0, device="cuda", dtype=torch.float16)
+    if layout == "row":
+        ops.tensor_mm(dev(a), dev(b), out=cbuf[:m, :n])
+    else:
+        ops.tensor_mm(dev(a), dev(np.ascontiguousarray(b.T)), out=cbuf[:m, :n], b_layout=capi.B_COL_MAJOR)
+    got = host(cbuf).astype(np.float32)
+    assert scaled_rel_err(got[:m, :n], want, math.sqrt(k) / 3.0) <= TOL_F16_GEMM
+    assert np.all(got[m:, :] == -7.0) and np.all(got[:, n:] == -7.0)
+
+
+def test_mm_f16_ragged_integer_inputs_bit_exact_and_batched(ops, oracle):
+    from anygpu_amd import capi
+    a = synth.integers(1, (200, 128), -4, 4).astype(np.float16)
+    b = synth.integers(2, (128, 328), -4, 4).astype(np.float16)
+    want = oracle.tensor_mm(a.astype(np.float32), b.astype(np.float32))
+    assert np.array_equal(host(ops.tensor_mm(dev(a), dev(b))).astype(np.float32), want)
+    assert np.array_equal(host(ops.tensor_mm(dev(a), dev(np.ascontiguousarray(b.T)), b_layout=capi.B_COL_MAJOR)).astype(np.float32), want)
+    # a batch of ragged products (attention shapes: 100 queries x 72 keys, d = 64)
+    q = synth.normal(3, (6, 100, 64)).astype(np.float16)
+    kk = synth.normal(4, (6, 72, 64)).astype(np.float16)
+    got = host(ops.tensor_mm_batched(dev(q), dev(kk), b_layout=capi.B_COL_MAJOR)).astype(np.float32)
+    for i in range(6):
+        w = oracle.tensor_mm(oracle.cvt_f16_to_f32(q[i]), oracle.cvt_f16_to_f32(kk[i]).T)
+        assert scaled_rel_err(got[i], w, math.sqrt(64)) <= TOL_F16_GEMM
+
+
 def test_mm_f16_config_4096_cubed_col_major_b(ops, oracle):
     from anygpu_amd import capi
     n = 4096
