@@ -9,8 +9,10 @@
 // and the upper half k = 8..15, one per instruction, so a lane reads its 8 values of a
 // k-contiguous operand with two 16-byte LDS loads and of a row-contiguous operand with eight
 // conflict-free 4-byte loads.
-// The same kernel serves any shape: FULL = true assumes whole tiles and 16-byte aligned
-// rows (vector global loads), FULL = false guards every global access.
+// The same kernel serves any shape through its access mode: whole tiles and 16-byte aligned rows
+// (vector loads, no tests), aligned rows but ragged extents (vector loads from clamped rows, the
+// last vectors of a row or column guarded, vector stores where they fit), or anything (every
+// global access guarded).
 #include "device_utils.hpp"
 #include "gemm_epilogue.hpp"
 #include "launch.hpp"
@@ -19,6 +21,11 @@
 #include <type_traits>
 
 namespace anygpu {
+
+// how the kernel may touch global memory
+constexpr int kAccessFull = 0;      // whole tiles, aligned: no tests
+constexpr int kAccessAligned = 1;   // 16-byte aligned rows and leading dimensions, ragged M / N / K
+constexpr int kAccessAny = 2;       // nothing assumed
 
 constexpr int kBK = 16;
 constexpr int64_t kBigTileThreshold = 256;    // 128 x 128 tiles once they give every one of the 256 CUs a block
@@ -33,9 +40,10 @@ constexpr int kSchedDsWrite = 0x200;
 // One ROWS-row x 16-deep operand slab (ROWS = 64 or 128).  KCONTIG: element (row, k) at
 // base[row * ld + k]; otherwise at base[k * ld + row].  `rows` / `depth` are the valid extents
 // from the slab origin.
-template <bool KCONTIG, bool FULL, int ROWS>
+template <bool KCONTIG, int ACCESS, int ROWS>
 struct Slab
 {
+	static constexpr bool FULL = (ACCESS == kAccessFull);
 	static constexpr bool kKContig = KCONTIG;
 	static constexpr int kPitchR = ROWS + 4;                 // floats per [k][row] LDS row
 	static constexpr int kLdsFloats = KCONTIG ? ROWS * kPitchK : kBK * kPitchR;
@@ -55,6 +63,13 @@ struct Slab
 			if (FULL)
 			{
 				reg[i] = *reinterpret_cast<const float4_t*>(KCONTIG ? base + r * ld + k : base + k * ld + r);
+			}
+			else if (ACCESS == kAccessAligned && (KCONTIG ? (k + 4 <= depth) : (k < depth && r + 4 <= rows)))
+			{
+				// the vector lies inside the operand along its own axis; across it, rows past the end are
+				// replaced by the last row (they only feed results that are not stored)
+				const int64_t rc = KCONTIG ? (r < rows ? r : rows - 1) : r;
+				reg[i] = *reinterpret_cast<const float4_t*>(KCONTIG ? base + rc * ld + k : base + k * ld + r);
 			}
 			else
 			{
@@ -101,7 +116,7 @@ struct Slab
 	}
 };
 
-template <int A_LAYOUT, int B_LAYOUT, bool FULL, int BM, int BN, int EPI>
+template <int A_LAYOUT, int B_LAYOUT, int ACCESS, int BM, int BN, int EPI>
 __global__ __launch_bounds__(256) void gemm_f32_kernel(
 	const float* __restrict__ A, const float* __restrict__ B, const float* __restrict__ B2,
 	const float* __restrict__ bias, float* __restrict__ C,
@@ -109,11 +124,12 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(
 	int64_t stride_a, int64_t stride_b, int64_t stride_c, float ep_param)
 {
 	constexpr bool DUAL = (EPI == kEpiGeluMul);
+	constexpr bool FULL = (ACCESS == kAccessFull);
 	A += (int64_t)blockIdx.z * stride_a;
 	B += (int64_t)blockIdx.z * stride_b;
 	C += (int64_t)blockIdx.z * stride_c;
-	using SlabA = Slab<A_LAYOUT == ANYGPU_A_ROW_MAJOR, FULL, BM>;
-	using SlabB = Slab<B_LAYOUT == ANYGPU_B_COL_MAJOR, FULL, BN>;
+	using SlabA = Slab<A_LAYOUT == ANYGPU_A_ROW_MAJOR, ACCESS, BM>;
+	using SlabB = Slab<B_LAYOUT == ANYGPU_B_COL_MAJOR, ACCESS, BN>;
 	constexpr int WTM = BM / 2, WTN = BN / 2;       // wave patch (2 x 2 waves)
 	constexpr int TM = WTM / 32, TN = WTN / 32;     // MFMA tiles per wave
 	__shared__ __align__(16) float a_lds[2][SlabA::kLdsFloats];
@@ -283,7 +299,7 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(
 					const float bias_n = (EPI == kEpiBias && bias) ? bias[n + e] : 0.0f;
 					return finish_sum<EPI>(acc[i][j][4 * g + e], sum2, bias_n, ep_param);
 				};
-				if (FULL)
+				if (FULL || (ACCESS == kAccessAligned && m < M && n + 4 <= N))
 				{
 					float4_t out;
 #pragma unroll
@@ -315,10 +331,13 @@ static hipError_t launch_tiles(const float* A, const float* B, const float* B2, 
 	const bool full = aligned && (M % BM == 0) && (N % BN == 0) && (K % kBK == 0);
 	discard_stale_error();
 	if (full)
-		gemm_f32_kernel<A_LAYOUT, B_LAYOUT, true, BM, BN, EPI><<<grid, dim3(256), 0, stream>>>(
+		gemm_f32_kernel<A_LAYOUT, B_LAYOUT, kAccessFull, BM, BN, EPI><<<grid, dim3(256), 0, stream>>>(
+			A, B, B2, bias, C, M, N, K, lda, ldb, ldc, stride_a, stride_b, stride_c, ep_param);
+	else if (aligned)
+		gemm_f32_kernel<A_LAYOUT, B_LAYOUT, kAccessAligned, BM, BN, EPI><<<grid, dim3(256), 0, stream>>>(
 			A, B, B2, bias, C, M, N, K, lda, ldb, ldc, stride_a, stride_b, stride_c, ep_param);
 	else
-		gemm_f32_kernel<A_LAYOUT, B_LAYOUT, false, BM, BN, EPI><<<grid, dim3(256), 0, stream>>>(
+		gemm_f32_kernel<A_LAYOUT, B_LAYOUT, kAccessAny, BM, BN, EPI><<<grid, dim3(256), 0, stream>>>(
 			A, B, B2, bias, C, M, N, K, lda, ldb, ldc, stride_a, stride_b, stride_c, ep_param);
 	return hipGetLastError();
 }

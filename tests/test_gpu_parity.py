@@ -367,7 +367,9 @@ def test_mm_f32_reference_cases_integer_inputs_exact(ops, oracle):
 
 @pytest.mark.parametrize("layout", ["row", "col"])
 @pytest.mark.parametrize("m,k,n", [(1, 1, 1), (3, 5, 7), (128, 16, 128), (128, 48, 256), (130, 17, 129),
-                                   (256, 256, 256), (77, 300, 515), (512, 100, 64)])
+                                   (256, 256, 256), (77, 300, 515), (512, 100, 64),
+                                   # 16-byte aligned rows, ragged extents: vector accesses with clamped rows and guarded ends
+                                   (100, 36, 72), (130, 20, 260), (257, 100, 516), (1000, 304, 520), (60, 4, 4)])
 def test_mm_f32_shapes_and_layouts(ops, oracle, layout, m, k, n):
     from anygpu_amd import capi
     a = synth.uniform(m + k, (m, k))
@@ -386,7 +388,7 @@ def test_mm_f32_shapes_and_layouts(ops, oracle, layout, m, k, n):
 def test_mm_f32_transposed_left_operand(ops, oracle):
     # the layout of the reference's last fp32 rung: A handed over as [K, M]
     from anygpu_amd import capi
-    for (m, k, n) in [(128, 64, 128), (100, 37, 61), (256, 272, 384)]:
+    for (m, k, n) in [(128, 64, 128), (100, 37, 61), (256, 272, 384), (100, 36, 72), (260, 300, 132)]:
         a = synth.uniform(m * 7 + k, (m, k))
         b = synth.uniform(k * 5 + n, (k, n))
         at = np.ascontiguousarray(a.T)
@@ -619,7 +621,7 @@ def test_mm_empty_and_rejected_arguments(ops):
 # =============================================================================================
 
 @pytest.mark.parametrize("b,s,hsize,vsize", [(1, 1, 1, 1), (2, 9, 300, 1000), (1, 5, 64, 37), (1, 128, 256, 512),
-                                             (3, 100, 130, 259), (1, 512, 512, 2048)])
+                                             (3, 100, 130, 259), (1, 512, 512, 2048), (3, 100, 132, 260)])
 def test_gemma_linear_softcap_shapes(ops, oracle, b, s, hsize, vsize):
     cap = 30.0
     x = synth.normal(b * s + hsize, (b, s, hsize))
@@ -648,7 +650,7 @@ def test_gemma_linear_softcap_gemma2_hidden_2304_vocab_slice(ops, oracle):
 
 
 @pytest.mark.parametrize("b,s,hsize,isize", [(1, 1, 1, 1), (1, 37, 288, 1152), (2, 5, 64, 37), (1, 128, 256, 512),
-                                             (3, 50, 130, 259), (1, 256, 512, 2048)])
+                                             (3, 50, 130, 259), (1, 256, 512, 2048), (3, 50, 132, 260)])
 def test_gemma_mlp_fused_upproj_shapes(ops, oracle, b, s, hsize, isize):
     x = synth.normal(b * s + hsize, (b, s, hsize))
     wg = synth.normal(isize + 1, (hsize, isize)) * np.float32(1.5 / math.sqrt(hsize))
