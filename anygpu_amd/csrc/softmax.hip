@@ -83,31 +83,63 @@ __device__ __forceinline__ float exp2_shift(float a, float b)
 	return fast_exp2(a - (b == -INFINITY ? 0.0f : b));
 }
 
-template <typename T, int VPL>
+// LOOSE: rows may start at any element (not only at 16-byte boundaries) and cols need not be a multiple of
+// the vector length.  Vector accesses then go out at element alignment (global memory takes them; the
+// compiler is told through the type) and the last, partial vector of a row is moved element by element.
+// GROUP: threads that share a row: 64 (a wave per row, four rows per block) or 256 (the block per row, for rows
+// longer than a wave's registers hold).
+template <typename T, int VPL, bool LOOSE, int GROUP>
 __global__ __launch_bounds__(256) void softmax_rows_wave_kernel(const SoftmaxArgs a)
 {
+	static_assert(GROUP == 64 || GROUP == 256, "a wave or the block per row");
 	constexpr int EPV = 16 / (int)sizeof(T);
 	using Vec = typename Vec16<T>::type;
+	typedef Vec LooseVec __attribute__((aligned(sizeof(T))));
+	constexpr int kWaveSize = GROUP;               // from here on "lane" counts inside the group and strides are the group's
+	__shared__ float red_m[4], red_s[4];
 
-	const int lane = threadIdx.x & (kWaveSize - 1);
-	const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-	if (row >= a.rows) return;  // uniform over the wave
+	const int lane = threadIdx.x & (GROUP - 1);
+	const int64_t row = GROUP == 64 ? (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6) : (int64_t)blockIdx.x;
+	if (row >= a.rows) return;  // uniform over the group
 
 	const RowSpan span = row_span(a, row);
 	const T* __restrict__ xr = static_cast<const T*>(a.x) + row * a.xs;
 	T* __restrict__ yr = static_cast<T*>(a.y) + row * a.ys;
-	const int nvec = (int)(a.cols / EPV);
+	const int tail = LOOSE ? (int)(a.cols % EPV) : 0;             // elements of a partial last vector
+	const int nvec = (int)(a.cols / EPV) + (tail ? 1 : 0);
 	const int lo = (int)span.lo, hi = (int)span.hi;
+	// vector v of a row: whole vectors in one access, the partial last one element by element (zeros behind it)
+	auto fetch = [&](const T* base, int v) {
+		Vec val = {};
+		if (LOOSE && tail && v == nvec - 1)
+		{
+#pragma unroll
+			for (int e = 0; e < EPV; ++e)
+				if (e < tail) val[e] = base[(int64_t)v * EPV + e];
+		}
+		else if (LOOSE) val = __builtin_nontemporal_load(reinterpret_cast<const LooseVec*>(base) + v);
+		else val = __builtin_nontemporal_load(reinterpret_cast<const Vec*>(base) + v);
+		return val;
+	};
+	auto put = [&](T* base, int v, Vec val) {
+		if (LOOSE && tail && v == nvec - 1)
+		{
+#pragma unroll
+			for (int e = 0; e < EPV; ++e)
+				if (e < tail) base[(int64_t)v * EPV + e] = val[e];
+		}
+		else if (LOOSE) __builtin_nontemporal_store(val, reinterpret_cast<LooseVec*>(base) + v);
+		else __builtin_nontemporal_store(val, reinterpret_cast<Vec*>(base) + v);
+	};
 	// additive mask row of this query (shared by all heads, so it is served from L2); it is
 	// fetched again in each register pass instead of being held in registers
-	const Vec* __restrict__ mrow = a.mask
-		? reinterpret_cast<const Vec*>(static_cast<const T*>(a.mask) + query_of_row(a, row) * a.mask_stride) : nullptr;
+	const T* __restrict__ mrow = a.mask ? static_cast<const T*>(a.mask) + query_of_row(a, row) * a.mask_stride : nullptr;
 	auto mask_of = [&](int v, float (&mk)[EPV]) {
 #pragma unroll
 		for (int e = 0; e < EPV; ++e) mk[e] = 0.0f;
 		if (mrow != nullptr)
 		{
-			const Vec mv = mrow[v];
+			const Vec mv = fetch(mrow, v);
 #pragma unroll
 			for (int e = 0; e < EPV; ++e) mk[e] = (float)mv[e] * kLog2e;   // -inf and float lowest both end at -inf
 		}
@@ -121,7 +153,7 @@ __global__ __launch_bounds__(256) void softmax_rows_wave_kernel(const SoftmaxArg
 		const int e0 = v * EPV;
 		const bool need = (v < nvec) && (e0 <= hi) && (e0 + EPV - 1 >= lo);
 		Vec val = {};
-		if (need) val = __builtin_nontemporal_load(reinterpret_cast<const Vec*>(xr) + v);
+		if (need) val = fetch(xr, v);
 		raw[t] = val;
 	}
 
@@ -154,8 +186,22 @@ __global__ __launch_bounds__(256) void softmax_rows_wave_kernel(const SoftmaxArg
 		}
 	}
 
-	const float M = wave_allreduce(st.m, MaxOp());
-	const float S = wave_allreduce(st.s * exp2_shift(st.m, M), SumOp());
+	float M = wave_allreduce(st.m, MaxOp());
+	float S = wave_allreduce(st.s * exp2_shift(st.m, M), SumOp());
+	if constexpr (GROUP == 256)
+	{
+		const int wave = threadIdx.x >> 6;
+		if ((threadIdx.x & 63) == 0)
+		{
+			red_m[wave] = M;
+			red_s[wave] = S;
+		}
+		__syncthreads();
+		M = fmaxf(fmaxf(red_m[0], red_m[1]), fmaxf(red_m[2], red_m[3]));
+		S = 0.0f;
+#pragma unroll
+		for (int w = 0; w < 4; ++w) S += red_s[w] * exp2_shift(red_m[w], M);
+	}
 	const float inv = S > 0.0f ? 1.0f / S : 0.0f;
 
 #pragma unroll
@@ -179,7 +225,7 @@ __global__ __launch_bounds__(256) void softmax_rows_wave_kernel(const SoftmaxArg
 					out[e] = (T)((j >= lo && j <= hi) ? p : 0.0f);
 				}
 			}
-			__builtin_nontemporal_store(out, reinterpret_cast<Vec*>(yr) + v);
+			put(yr, v, out);
 		}
 	}
 }
@@ -368,13 +414,24 @@ __global__ __launch_bounds__(256) void softmax_rows_block_kernel(const SoftmaxAr
 	}
 }
 
-template <typename T, int VPL>
+template <typename T, int VPL, bool LOOSE = false, int GROUP = 64>
 static hipError_t launch_wave(const SoftmaxArgs& a, hipStream_t stream)
 {
-	const unsigned blocks = (unsigned)((a.rows + 3) / 4);
+	const unsigned blocks = GROUP == 64 ? (unsigned)((a.rows + 3) / 4) : (unsigned)a.rows;
 	discard_stale_error();
-	softmax_rows_wave_kernel<T, VPL><<<dim3(blocks), dim3(256), 0, stream>>>(a);
+	softmax_rows_wave_kernel<T, VPL, LOOSE, GROUP><<<dim3(blocks), dim3(256), 0, stream>>>(a);
 	return hipGetLastError();
+}
+
+// rows longer than a wave holds: the block per row, 256 * VPL vectors in registers
+template <typename T, bool LOOSE>
+static hipError_t launch_long_rows(const SoftmaxArgs& a, int64_t nvec, hipStream_t stream)
+{
+	constexpr int kMaxVpl = sizeof(T) == 2 ? 16 : 32;
+	if (nvec <= 256 * 8) return launch_wave<T, 8, LOOSE, 256>(a, stream);
+	if (nvec <= 256 * 16) return launch_wave<T, 16, LOOSE, 256>(a, stream);
+	if constexpr (kMaxVpl >= 32) return launch_wave<T, 32, LOOSE, 256>(a, stream);
+	return hipErrorInvalidValue;       // not reached: the caller checks the capacity
 }
 
 template <typename T>
@@ -425,6 +482,19 @@ hipError_t launch_softmax_rows(const void* x, void* y, int64_t rows, int64_t col
 		if (nvec <= kWaveSize * 16) return launch_wave<T, 16>(a, stream);
 		if constexpr (kMaxVpl >= 32) return launch_wave<T, 32>(a, stream);
 	}
+	if (vec_ok && nvec <= (int64_t)256 * kMaxVpl) return launch_long_rows<T, false>(a, nvec, stream);
+	// rows at element alignment, any width: the same wave kernel with element-aligned vector accesses
+	const int64_t nvec_loose = (cols + EPV - 1) / EPV;
+	if (!vec_ok && nvec_loose <= (int64_t)kWaveSize * kMaxVpl)
+	{
+		if (nvec_loose <= kWaveSize * 1) return launch_wave<T, 1, true>(a, stream);
+		if (nvec_loose <= kWaveSize * 2) return launch_wave<T, 2, true>(a, stream);
+		if (nvec_loose <= kWaveSize * 4) return launch_wave<T, 4, true>(a, stream);
+		if (nvec_loose <= kWaveSize * 8) return launch_wave<T, 8, true>(a, stream);
+		if (nvec_loose <= kWaveSize * 16) return launch_wave<T, 16, true>(a, stream);
+		if constexpr (kMaxVpl >= 32) return launch_wave<T, 32, true>(a, stream);
+	}
+	if (!vec_ok && nvec_loose <= (int64_t)256 * kMaxVpl) return launch_long_rows<T, true>(a, nvec_loose, stream);
 	discard_stale_error();
 	softmax_rows_block_kernel<T><<<dim3((unsigned)rows), dim3(256), 0, stream>>>(a);
 	return hipGetLastError();
