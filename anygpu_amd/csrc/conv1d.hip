@@ -40,7 +40,9 @@ __device__ __forceinline__ float conv_point(const float (&wv)[kMaxWidth], float 
 	return silu_f32(acc);
 }
 
-template <typename T, int WIDTH, int U>
+// LOOSE: rows may start at any element and seqlen need not be a multiple of the vector length: vector
+// accesses go out at element alignment, the partial last vector of a row is moved element by element.
+template <typename T, int WIDTH, int U, bool LOOSE>
 __global__ __launch_bounds__(256) void causal_conv1d_silu_tile_kernel(
 	const T* __restrict__ x, const T* __restrict__ w, const T* __restrict__ bias, T* __restrict__ y,
 	int chan, int seqlen, int tiles_per_row)
@@ -49,6 +51,8 @@ __global__ __launch_bounds__(256) void causal_conv1d_silu_tile_kernel(
 	constexpr int TPV = (int)(sizeof(typename ConvVec<T>::tail_type) / sizeof(T));  // samples in a published tail
 	using Vec = typename ConvVec<T>::type;
 	using Tail = typename ConvVec<T>::tail_type;
+	typedef Vec LooseVec __attribute__((aligned(sizeof(T))));
+	typedef Tail LooseTail __attribute__((aligned(sizeof(T))));
 
 	__shared__ Tail tails[U][256];
 
@@ -56,7 +60,8 @@ __global__ __launch_bounds__(256) void causal_conv1d_silu_tile_kernel(
 	const int row = blockIdx.x / tiles_per_row;           // (batch, chan) pair
 	const int tile = blockIdx.x - row * tiles_per_row;
 	const int ch = row % chan;
-	const int nvec = seqlen / EPV;
+	const int rest = LOOSE ? seqlen % EPV : 0;               // samples of a partial last vector
+	const int nvec = seqlen / EPV + (rest ? 1 : 0);
 	const int v_base = tile * (256 * U);
 
 	const T* __restrict__ xr = x + (int64_t)row * seqlen;
@@ -73,14 +78,25 @@ __global__ __launch_bounds__(256) void causal_conv1d_silu_tile_kernel(
 	{
 		const int v = v_base + u * 256 + tid;
 		Vec val = {};
-		if (v < nvec) val = __builtin_nontemporal_load(reinterpret_cast<const Vec*>(xr) + v);
+		if (v < nvec)
+		{
+			if (LOOSE && rest && v == nvec - 1)
+			{
+#pragma unroll
+				for (int e = 0; e < EPV; ++e)
+					if (e < rest) val[e] = xr[(int64_t)v * EPV + e];
+			}
+			else if (LOOSE) val = __builtin_nontemporal_load(reinterpret_cast<const LooseVec*>(xr) + v);
+			else val = __builtin_nontemporal_load(reinterpret_cast<const Vec*>(xr) + v);
+		}
 		xv[u] = val;
 	}
 	// halo in front of the tile: the TPV samples that end where the tile starts
 	Tail front = {};
 	if (tid == 0 && v_base > 0)
 	{
-		front = *reinterpret_cast<const Tail*>(xr + (int64_t)v_base * EPV - TPV);
+		if (LOOSE) front = *reinterpret_cast<const LooseTail*>(xr + (int64_t)v_base * EPV - TPV);
+		else front = *reinterpret_cast<const Tail*>(xr + (int64_t)v_base * EPV - TPV);
 	}
 
 #pragma unroll
@@ -115,8 +131,94 @@ __global__ __launch_bounds__(256) void causal_conv1d_silu_tile_kernel(
 		{
 			out[e] = (T)conv_point<WIDTH>(wv, bv, s[e], s[e + 1], s[e + 2], s[e + 3]);
 		}
-		__builtin_nontemporal_store(out, reinterpret_cast<Vec*>(yr) + v);
+		if (LOOSE && rest && v == nvec - 1)
+		{
+#pragma unroll
+			for (int e = 0; e < EPV; ++e)
+				if (e < rest) yr[(int64_t)v * EPV + e] = out[e];
+		}
+		else if (LOOSE) __builtin_nontemporal_store(out, reinterpret_cast<LooseVec*>(yr) + v);
+		else __builtin_nontemporal_store(out, reinterpret_cast<Vec*>(yr) + v);
 	}
+}
+
+// Short rows: a row has fewer vectors than a tile of the kernel above has slots, so the tile would be mostly idle.
+// Here the (row, vector) pairs of the whole tensor are numbered consecutively and a block takes 256 of them,
+// whichever rows they belong to; a thread finds its halo in its left neighbour's tail unless its vector is
+// the first of a row (zeros) or the first of the block (global memory).  Taps and bias are loaded per thread.
+template <typename T, int WIDTH, bool LOOSE>
+__global__ __launch_bounds__(256) void causal_conv1d_silu_short_rows_kernel(
+	const T* __restrict__ x, const T* __restrict__ w, const T* __restrict__ bias, T* __restrict__ y,
+	int chan, int seqlen, int nvec, int64_t total_vecs)
+{
+	constexpr int EPV = 16 / (int)sizeof(T);
+	constexpr int TPV = (int)(sizeof(typename ConvVec<T>::tail_type) / sizeof(T));
+	using Vec = typename ConvVec<T>::type;
+	using Tail = typename ConvVec<T>::tail_type;
+	typedef Vec LooseVec __attribute__((aligned(sizeof(T))));
+	typedef Tail LooseTail __attribute__((aligned(sizeof(T))));
+	__shared__ Tail tails[256];
+
+	const int tid = threadIdx.x;
+	const int64_t g = (int64_t)blockIdx.x * 256 + tid;
+	const bool live = g < total_vecs;
+	const int64_t row = live ? g / nvec : 0;
+	const int v = live ? (int)(g - row * nvec) : 0;
+	const int rest = LOOSE ? seqlen % EPV : 0;
+	const bool partial = LOOSE && rest && v == nvec - 1;
+	const T* __restrict__ xr = x + row * seqlen;
+	T* __restrict__ yr = y + row * seqlen;
+
+	Vec xv = {};
+	if (live)
+	{
+		if (partial)
+		{
+#pragma unroll
+			for (int e = 0; e < EPV; ++e)
+				if (e < rest) xv[e] = xr[(int64_t)v * EPV + e];
+		}
+		else if (LOOSE) xv = __builtin_nontemporal_load(reinterpret_cast<const LooseVec*>(xr) + v);
+		else xv = __builtin_nontemporal_load(reinterpret_cast<const Vec*>(xr) + v);
+	}
+	Tail front = {};
+	if (tid == 0 && live && v > 0)
+	{
+		if (LOOSE) front = *reinterpret_cast<const LooseTail*>(xr + (int64_t)v * EPV - TPV);
+		else front = *reinterpret_cast<const Tail*>(xr + (int64_t)v * EPV - TPV);
+	}
+	Tail mine;
+#pragma unroll
+	for (int e = 0; e < TPV; ++e) mine[e] = xv[EPV - TPV + e];
+	tails[tid] = mine;
+	__syncthreads();
+	if (!live) return;
+
+	Tail prev = {};
+	if (v > 0) prev = tid > 0 ? tails[tid - 1] : front;
+
+	const int ch = (int)(row % chan);
+	float wv[kMaxWidth] = { 0.f, 0.f, 0.f, 0.f };
+#pragma unroll
+	for (int k = 0; k < WIDTH; ++k) wv[kMaxWidth - WIDTH + k] = (float)w[(int64_t)ch * WIDTH + k];
+	const float bv = (float)bias[ch];
+
+	float s[kHalo + EPV];
+#pragma unroll
+	for (int e = 0; e < kHalo; ++e) s[e] = (float)prev[TPV - kHalo + e];
+#pragma unroll
+	for (int e = 0; e < EPV; ++e) s[kHalo + e] = (float)xv[e];
+	Vec out;
+#pragma unroll
+	for (int e = 0; e < EPV; ++e) out[e] = (T)conv_point<WIDTH>(wv, bv, s[e], s[e + 1], s[e + 2], s[e + 3]);
+	if (partial)
+	{
+#pragma unroll
+		for (int e = 0; e < EPV; ++e)
+			if (e < rest) yr[(int64_t)v * EPV + e] = out[e];
+	}
+	else if (LOOSE) __builtin_nontemporal_store(out, reinterpret_cast<LooseVec*>(yr) + v);
+	else __builtin_nontemporal_store(out, reinterpret_cast<Vec*>(yr) + v);
 }
 
 template <typename T, int WIDTH>
@@ -160,16 +262,34 @@ static hipError_t launch_width(const void* x, const void* w, const void* bias, v
 
 	const bool vec_ok = (seqlen % EPV == 0) && (reinterpret_cast<uintptr_t>(x) % 16 == 0) &&
 	                    (reinterpret_cast<uintptr_t>(y) % 16 == 0);
-	if (vec_ok)
 	{
-		const int64_t nvec = seqlen / EPV;
+		// vectors per row, a partial last one included; rows shorter than the halo take the element kernel
+		const int64_t nvec = (seqlen + EPV - 1) / EPV;
 		const int64_t tiles_per_row = (nvec + 256 * U - 1) / (256 * U);
 		const int64_t blocks = rows * tiles_per_row;
-		if (blocks <= 0x7FFFFFFFLL)
+		if (nvec < 256 * U && seqlen >= EPV && (rows * nvec + 255) / 256 <= 0x7FFFFFFFLL)
+		{
+			// short rows: blocks over the consecutive (row, vector) pairs
+			const int64_t total_vecs = rows * nvec;
+			const dim3 grid((unsigned)((total_vecs + 255) / 256));
+			discard_stale_error();
+			if (vec_ok)
+				causal_conv1d_silu_short_rows_kernel<T, WIDTH, false><<<grid, dim3(256), 0, stream>>>(
+					xp, wp, bp, yp, (int)chan, (int)seqlen, (int)nvec, total_vecs);
+			else
+				causal_conv1d_silu_short_rows_kernel<T, WIDTH, true><<<grid, dim3(256), 0, stream>>>(
+					xp, wp, bp, yp, (int)chan, (int)seqlen, (int)nvec, total_vecs);
+			return hipGetLastError();
+		}
+		if (blocks <= 0x7FFFFFFFLL && seqlen >= EPV)
 		{
 			discard_stale_error();
-			causal_conv1d_silu_tile_kernel<T, WIDTH, U><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(
-				xp, wp, bp, yp, (int)chan, (int)seqlen, (int)tiles_per_row);
+			if (vec_ok)
+				causal_conv1d_silu_tile_kernel<T, WIDTH, U, false><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(
+					xp, wp, bp, yp, (int)chan, (int)seqlen, (int)tiles_per_row);
+			else
+				causal_conv1d_silu_tile_kernel<T, WIDTH, U, true><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(
+					xp, wp, bp, yp, (int)chan, (int)seqlen, (int)tiles_per_row);
 			return hipGetLastError();
 		}
 	}

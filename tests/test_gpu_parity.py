@@ -249,6 +249,34 @@ def test_conv1d_shapes(ops, oracle, dtype, b, d, s, width):
     assert scaled_rel_err(got, want, 1.0) <= tol
 
 
+@pytest.mark.parametrize("dtype", ["f16", "f32"])
+@pytest.mark.parametrize("b,d,s,width", [(2, 5, 638, 4), (1, 3, 4095, 4), (3, 4, 9, 3), (2, 7, 17, 2), (1, 2, 1031, 4)])
+def test_conv1d_rows_at_element_alignment(ops, oracle, dtype, b, d, s, width):
+    # sequence lengths that are no multiple of the 16-byte vector; tensors in the middle of a flat buffer whose
+    # surroundings must stay untouched
+    import torch
+    np_dt = np.float16 if dtype == "f16" else np.float32
+    t_dt = torch.float16 if dtype == "f16" else torch.float32
+    x = synth.normal(b * d + s, (b, d, s)).astype(np_dt)
+    w = (synth.normal(1, (d, width)) * np.float32(0.5)).astype(np_dt)
+    bias = (synth.normal(2, (d,)) * np.float32(0.1)).astype(np_dt)
+    up = (lambda a: oracle.cvt_f16_to_f32(a)) if dtype == "f16" else (lambda a: a)
+    want = oracle.tensor_causal_conv1d(up(x), up(w), up(bias))
+    n = b * d * s
+    flat_x = torch.full((n + 64,), 9.0, device="cuda", dtype=t_dt)
+    flat_y = torch.full_like(flat_x, -5.0)
+    for front in (0, 1, 6):
+        xv = flat_x[front:front + n].view(b, d, s)
+        yv = flat_y[front:front + n].view(b, d, s)
+        xv.copy_(dev(x))
+        flat_y.fill_(-5.0)
+        ops.tensor_causal_conv1d(xv, dev(w), dev(bias), out=yv)
+        got_flat = host(flat_y).astype(np.float32)
+        got = got_flat[front:front + n].reshape(b, d, s)
+        assert scaled_rel_err(got, want, 1.0) <= (TOL_F16_ROWOPS if dtype == "f16" else TOL_F32)
+        assert np.all(got_flat[:front] == -5.0) and np.all(got_flat[front + n:] == -5.0)
+
+
 def test_conv1d_f32_reference_generator_shape(ops, oracle):
     # tests/ext_torch_tests.cpp:745-778 (batch 8, dims 2318, seq 638, width 4), gate: abs tol 1e-3
     got, want = _conv_case(ops, oracle, "f32", 8, 2318, 638, 4, seed=10)
