@@ -11,8 +11,8 @@
 // conflict-free 4-byte loads.
 // The same kernel serves any shape through its access mode: whole tiles and 16-byte aligned rows
 // (vector loads, no tests), aligned rows but ragged extents (vector loads from clamped rows, the
-// last vectors of a row or column guarded, vector stores where they fit), or anything (every
-// global access guarded).
+// last vectors of a row or column guarded, vector stores where they fit), or anything (the same
+// with the vectors at element alignment).
 #include "device_utils.hpp"
 #include "gemm_epilogue.hpp"
 #include "launch.hpp"
@@ -25,7 +25,7 @@ namespace anygpu {
 // how the kernel may touch global memory
 constexpr int kAccessFull = 0;      // whole tiles, aligned: no tests
 constexpr int kAccessAligned = 1;   // 16-byte aligned rows and leading dimensions, ragged M / N / K
-constexpr int kAccessAny = 2;       // nothing assumed
+constexpr int kAccessAny = 2;       // nothing assumed: vectors at element alignment, guarded ends
 
 constexpr int kBK = 16;
 constexpr int64_t kBigTileThreshold = 256;    // 128 x 128 tiles once they give every one of the 256 CUs a block
@@ -64,12 +64,16 @@ struct Slab
 			{
 				reg[i] = *reinterpret_cast<const float4_t*>(KCONTIG ? base + r * ld + k : base + k * ld + r);
 			}
-			else if (ACCESS == kAccessAligned && (KCONTIG ? (k + 4 <= depth) : (k < depth && r + 4 <= rows)))
+			else if (KCONTIG ? (k + 4 <= depth) : (k < depth && r + 4 <= rows))
 			{
 				// the vector lies inside the operand along its own axis; across it, rows past the end are
-				// replaced by the last row (they only feed results that are not stored)
+				// replaced by the last row (they only feed results that are not stored).  Without the
+				// alignment guarantee the same 16 bytes are fetched at element alignment.
+				typedef float4_t LooseVec __attribute__((aligned(4)));
 				const int64_t rc = KCONTIG ? (r < rows ? r : rows - 1) : r;
-				reg[i] = *reinterpret_cast<const float4_t*>(KCONTIG ? base + rc * ld + k : base + k * ld + r);
+				const float* src = KCONTIG ? base + rc * ld + k : base + k * ld + r;
+				if (ACCESS == kAccessAligned) reg[i] = *reinterpret_cast<const float4_t*>(src);
+				else reg[i] = *reinterpret_cast<const LooseVec*>(src);
 			}
 			else
 			{
@@ -299,12 +303,14 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(
 					const float bias_n = (EPI == kEpiBias && bias) ? bias[n + e] : 0.0f;
 					return finish_sum<EPI>(acc[i][j][4 * g + e], sum2, bias_n, ep_param);
 				};
-				if (FULL || (ACCESS == kAccessAligned && m < M && n + 4 <= N))
+				if (FULL || (m < M && n + 4 <= N))
 				{
+					typedef float4_t LooseVec __attribute__((aligned(4)));
 					float4_t out;
 #pragma unroll
 					for (int e = 0; e < 4; ++e) out[e] = finish(e);
-					*reinterpret_cast<float4_t*>(C + m * ldc + n) = out;
+					if (ACCESS == kAccessAny) *reinterpret_cast<LooseVec*>(C + m * ldc + n) = out;
+					else *reinterpret_cast<float4_t*>(C + m * ldc + n) = out;
 				}
 				else if (m < M)
 				{
