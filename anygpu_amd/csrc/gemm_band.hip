@@ -1,0 +1,484 @@
+// Products with a band of few left-operand rows (M <= 64: a short prompt, a small decode batch) against
+// k-contiguous weights (column-major B, [N, K]).  The weight matrix dominates the traffic and has to be
+// streamed from HBM once at full rate; a square MFMA tile of 64 or 128 rows would spend most of its matrix
+// cycles on padding and leave the loads waiting behind them.
+//
+// Here the band of A rows is one MFMA operand of 16 or 32 rows (two of 32 for 33 .. 64 rows, which share every
+// weight register) and the weights never pass through LDS:
+// every lane loads 16-byte vectors of "its" weight row straight into the MFMA operand registers.  The
+// k index inside an MFMA is a dummy index, so the lanes are free to take any k they like as long as both
+// operands agree: with G lane groups (4 in the 16-row form, 2 in the 32-row form) load i of lane group g
+// takes the 16 bytes (i * G + g) * 16 .. of each k step, so that one load instruction reads 64 or 32
+// contiguous bytes of every weight row, four of them a contiguous run of 256 or 128 bytes, and the matching
+// A values are read from an LDS copy of the band with the same addressing.  A block of 4 waves covers 128 output columns
+// (32 per wave) and shares the band chunk in LDS; the loads of the next k step are in flight while the
+// current one is multiplied.
+//
+// Weight matrices with few rows do not have 128-column tiles for every CU, so K is split over blockIdx.y:
+// each split writes its partial sums (in register layout) to a workspace and a second small kernel adds
+// them in split order, applies the epilogue and stores.  (Finishing in the last block to arrive, behind a
+// ticket counter, needs a device-scope fence per block; with one L2 per XCD that fence writes the L2 back
+// and cost more than the whole product: 60 - 90 us against 20.)  The workspace belongs to the
+// (device, stream) pair, is allocated on first use and kept for the life of the process, like the
+// workspace of a BLAS handle; a stream that is being captured and has none yet runs without the split.
+#include "device_utils.hpp"
+#include "gemm_epilogue.hpp"
+#include "launch.hpp"
+#include "anygpu_hip.h"
+
+#include <map>
+#include <mutex>
+#include <type_traits>
+#include <utility>
+
+namespace anygpu {
+
+namespace {
+
+constexpr int kBandThreads = 256;
+constexpr int kBandCols = 128;                    // output columns per block, 32 per wave
+constexpr int kBandMaxSplits = 32;
+constexpr int64_t kBandEnoughBlocks = 256;        // tiles from which K is not split
+constexpr int64_t kBandWantedBlocks = 512;
+constexpr size_t kBandPartialBytes = (size_t)16 << 20;
+
+typedef float4_t Vec;      // 16 raw bytes of either element type
+
+template <typename T, int MR> struct BandMma;
+
+template <> struct BandMma<float, 16>
+{
+	typedef float4_t Acc;
+	static constexpr int kRegs = 4;
+	__device__ static void mma(const Vec& w, const Vec& a, Acc& acc)
+	{
+#pragma unroll
+		for (int e = 0; e < 4; ++e) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(w[e], a[e], acc, 0, 0, 0);
+	}
+};
+
+template <> struct BandMma<float, 32>
+{
+	typedef float16_t Acc;
+	static constexpr int kRegs = 16;
+	__device__ static void mma(const Vec& w, const Vec& a, Acc& acc)
+	{
+#pragma unroll
+		for (int e = 0; e < 4; ++e) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(w[e], a[e], acc, 0, 0, 0);
+	}
+};
+
+template <> struct BandMma<half_t, 16>
+{
+	typedef float4_t Acc;
+	static constexpr int kRegs = 4;
+	__device__ static void mma(const Vec& w, const Vec& a, Acc& acc)
+	{
+		acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, w), __builtin_bit_cast(half8_t, a), acc, 0, 0, 0);
+	}
+};
+
+template <> struct BandMma<half_t, 32>
+{
+	typedef float16_t Acc;
+	static constexpr int kRegs = 16;
+	__device__ static void mma(const Vec& w, const Vec& a, Acc& acc)
+	{
+		acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, w), __builtin_bit_cast(half8_t, a), acc, 0, 0, 0);
+	}
+};
+
+template <typename T, int MR, int MB>
+struct BandShape
+{
+	static constexpr int kEV = 16 / (int)sizeof(T);      // elements per vector
+	static constexpr int kGroups = kWaveSize / MR;        // lane groups along k
+	static constexpr int kStepVecs = 4 * kGroups;         // vectors of one row per k step
+	static constexpr int kStep = kStepVecs * kEV;         // elements per k step
+	static constexpr int kRows = MR * MB;                 // band rows: MB MFMA row blocks of MR
+	static constexpr int kStepsPerChunk = 4 / MB;         // an LDS chunk of the band is always 1024 vectors
+	static constexpr int kChunkVecs = kStepsPerChunk * kStepVecs;
+	static constexpr int kChunk = kChunkVecs * kEV;       // elements of K per LDS chunk of the band
+	static constexpr int kPitchVecs = kChunkVecs + 1;     // LDS row pitch: 16 bytes of padding
+	static constexpr int kNG = 32 / MR;                   // MFMA column groups per wave
+};
+
+__device__ __forceinline__ void store4(float* dst, const float4_t& v) { *reinterpret_cast<float4_t*>(dst) = v; }
+__device__ __forceinline__ void store4(half_t* dst, const float4_t& v)
+{
+	*reinterpret_cast<half4_t*>(dst) = half4_t{(half_t)v[0], (half_t)v[1], (half_t)v[2], (half_t)v[3]};
+}
+
+// Epilogue and store of one thread's sums.  Register 4 q + e of a lane: column 4 * grp + e (16-row form) or
+// 8 q + 4 * grp + e (32-row form) of the MFMA column group, band row idx.
+template <typename T, int MR, int MB, int EPI, typename Acc>
+__device__ __forceinline__ void band_store(const Acc (*acc)[MB], const float* __restrict__ bias, T* __restrict__ C,
+                                           int M, int64_t N, int64_t ldc, int64_t n0, int idx, int grp, float ep_param)
+{
+	using S = BandShape<T, MR, MB>;
+	constexpr bool DUAL = (EPI == kEpiGeluMul);
+	constexpr int kRegs = BandMma<T, MR>::kRegs;
+#pragma unroll
+	for (int b = 0; b < MB; ++b)
+	{
+		const int m = b * MR + idx;
+		if (m >= M) continue;
+#pragma unroll
+		for (int j = 0; j < S::kNG; ++j)
+#pragma unroll
+			for (int q = 0; q < kRegs / 4; ++q)
+			{
+				const int64_t n = n0 + j * MR + (MR == 16 ? 4 * grp : 8 * q + 4 * grp);
+				float4_t out;
+#pragma unroll
+				for (int e = 0; e < 4; ++e)
+				{
+					const float sum2 = DUAL ? acc[DUAL ? S::kNG + j : 0][b][4 * q + e] : 0.0f;
+					const float bias_n = (EPI == kEpiBias && bias && n + e < N) ? bias[n + e] : 0.0f;
+					out[e] = finish_sum<EPI>(acc[j][b][4 * q + e], sum2, bias_n, ep_param);
+				}
+				T* dst = C + (int64_t)m * ldc + n;
+				if (n + 4 <= N) store4(dst, out);
+				else
+				{
+#pragma unroll
+					for (int e = 0; e < 4; ++e)
+						if (n + e < N) dst[e] = (T)out[e];
+				}
+			}
+	}
+}
+
+// C[m, n] = finish(sum_k A[m, k] * B[n, k]), M <= MR * MB.  grid (tiles of 128 columns, splits of K);
+// `chunks_per_split` LDS chunks of K per split.  With gridDim.y > 1 the sums of split y go to
+// partial[tile][y][thread][register] and gemm_band_merge_kernel finishes.
+template <typename T, int MR, int MB, int EPI>
+__global__ __launch_bounds__(kBandThreads) void gemm_band_kernel(
+	const T* __restrict__ A, const T* __restrict__ B, const T* __restrict__ B2, const float* __restrict__ bias,
+	T* __restrict__ C, float* __restrict__ partial,
+	int M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc, int chunks_per_split, float ep_param)
+{
+	using S = BandShape<T, MR, MB>;
+	using Mma = BandMma<T, MR>;
+	using Acc = typename Mma::Acc;
+	constexpr bool DUAL = (EPI == kEpiGeluMul);
+	constexpr int kW = S::kNG * (DUAL ? 2 : 1);          // weight rows per lane
+
+	__shared__ Vec band[2][S::kRows * S::kPitchVecs];
+
+	const int tid = threadIdx.x;
+	const int lane = tid & (kWaveSize - 1);
+	const int wave = tid >> 6;
+	const int idx = lane % MR;                            // weight row (as W operand) / band row (as A operand)
+	const int grp = lane / MR;
+	const int64_t n0 = (int64_t)blockIdx.x * kBandCols + wave * 32;
+
+	const int64_t kb = (int64_t)blockIdx.y * chunks_per_split * S::kChunk;
+	const int64_t ke_want = kb + (int64_t)chunks_per_split * S::kChunk;
+	const int64_t ke = ke_want < K ? ke_want : K;
+
+	// weight row pointers of this lane; rows past the end are replaced by the last one (never stored)
+	const T* wrow[kW];
+#pragma unroll
+	for (int j = 0; j < S::kNG; ++j)
+	{
+		int64_t n = n0 + j * MR + idx;
+		n = n < N ? n : N - 1;
+		wrow[j] = B + n * ldb;
+		if constexpr (DUAL) wrow[S::kNG + j] = B2 + n * ldb;
+	}
+
+	// Weight vectors of one k step.  GUARDED: vectors at or past the end of the k range are fetched from the
+	// start of the range instead (a valid address) and zeroed by mask_w before they are multiplied; the selects
+	// sit at the use so that the loads stay in flight over the previous step.
+	Vec wr[2][kW][4];
+	const Vec zero = {0.0f, 0.0f, 0.0f, 0.0f};
+	auto issue_w = [&](Vec (&dst)[kW][4], int64_t step, auto guarded) {
+		const int64_t k0 = kb + step * S::kStep + grp * S::kEV;
+#pragma unroll
+		for (int i = 0; i < 4; ++i)
+		{
+			const int64_t k = k0 + i * S::kGroups * S::kEV;
+			const int64_t kk = (decltype(guarded)::value && k >= ke) ? kb : k;
+#pragma unroll
+			for (int j = 0; j < kW; ++j) dst[j][i] = *reinterpret_cast<const Vec*>(wrow[j] + kk);
+		}
+	};
+	auto mask_w = [&](Vec (&w)[kW][4], int64_t step) {
+		const int64_t k0 = kb + step * S::kStep + grp * S::kEV;
+#pragma unroll
+		for (int i = 0; i < 4; ++i)
+		{
+			const bool valid = k0 + i * S::kGroups * S::kEV < ke;
+#pragma unroll
+			for (int j = 0; j < kW; ++j) w[j][i] = valid ? w[j][i] : zero;
+		}
+	};
+
+	// the band chunk: kRows rows x kChunkVecs vectors = 1024 vectors, 4 per thread; rows past M and k past the
+	// range are fetched from valid addresses and zeroed on their way into LDS
+	Vec ar[4];
+	auto issue_band = [&](int chunk) {
+		const int64_t kc = kb + (int64_t)chunk * S::kChunk;
+#pragma unroll
+		for (int i = 0; i < 4; ++i)
+		{
+			const int q = tid + kBandThreads * i;
+			const int row = q / S::kChunkVecs;
+			const int64_t k = kc + (q % S::kChunkVecs) * S::kEV;
+			ar[i] = *reinterpret_cast<const Vec*>(A + (int64_t)(row < M ? row : M - 1) * lda + (k < ke ? k : kb));
+		}
+	};
+	auto stage_band = [&](int chunk) {
+		const int64_t kc = kb + (int64_t)chunk * S::kChunk;
+#pragma unroll
+		for (int i = 0; i < 4; ++i)
+		{
+			const int q = tid + kBandThreads * i;
+			const int row = q / S::kChunkVecs;
+			const bool valid = row < M && kc + (q % S::kChunkVecs) * S::kEV < ke;
+			band[chunk & 1][row * S::kPitchVecs + (q % S::kChunkVecs)] = valid ? ar[i] : zero;
+		}
+	};
+
+	Acc acc[kW][MB];
+#pragma unroll
+	for (int j = 0; j < kW; ++j)
+#pragma unroll
+		for (int b = 0; b < MB; ++b)
+#pragma unroll
+			for (int r = 0; r < Mma::kRegs; ++r) acc[j][b][r] = 0.0f;
+
+	auto multiply = [&](const Vec (&w)[kW][4], int buf, int s) {
+		Vec a[MB][4];
+#pragma unroll
+		for (int b = 0; b < MB; ++b)
+		{
+			const Vec* src = &band[buf][(b * MR + idx) * S::kPitchVecs + s * S::kStepVecs + grp];
+#pragma unroll
+			for (int i = 0; i < 4; ++i) a[b][i] = src[i * S::kGroups];
+		}
+#pragma unroll
+		for (int i = 0; i < 4; ++i)
+#pragma unroll
+			for (int j = 0; j < kW; ++j)
+#pragma unroll
+				for (int b = 0; b < MB; ++b) Mma::mma(w[j][i], a[b][i], acc[j][b]);
+	};
+
+	using Plain = std::false_type;
+	using Guarded = std::true_type;
+	const int full_chunks = (int)((ke - kb) / S::kChunk);          // chunks whose every vector lies inside the range
+	const bool tail = (ke - kb) % S::kChunk != 0;
+	const int64_t last_full_step = (int64_t)full_chunks * S::kStepsPerChunk - 1;
+
+	issue_band(0);
+	if (full_chunks > 0) issue_w(wr[0], 0, Plain{});
+	stage_band(0);
+	__syncthreads();
+	for (int c = 0; c < full_chunks; ++c)
+	{
+		issue_band(c + 1);                       // past the end: zeros, staged into a buffer nobody reads
+#pragma unroll
+		for (int s = 0; s < S::kStepsPerChunk; ++s)
+		{
+			// the loads of the next step are issued before this step's MFMAs; after the last full step the same
+			// step is fetched again and dropped
+			const int64_t next = (int64_t)c * S::kStepsPerChunk + s + 1;
+			issue_w(wr[(s + 1) & 1], next < last_full_step ? next : last_full_step, Plain{});
+			__builtin_amdgcn_sched_barrier(0);
+			multiply(wr[s & 1], c & 1, s);
+		}
+		stage_band(c + 1);
+		__syncthreads();
+	}
+	if (tail)
+	{
+		const int c = full_chunks;
+		issue_w(wr[0], (int64_t)c * S::kStepsPerChunk, Guarded{});
+#pragma unroll
+		for (int s = 0; s < S::kStepsPerChunk; ++s)
+		{
+			const int64_t step = (int64_t)c * S::kStepsPerChunk + s;
+			issue_w(wr[(s + 1) & 1], step + 1, Guarded{});
+			__builtin_amdgcn_sched_barrier(0);
+			mask_w(wr[s & 1], step);
+			multiply(wr[s & 1], c & 1, s);
+		}
+	}
+
+	if (gridDim.y > 1)
+	{
+		constexpr int kAccFloats = kW * MB * Mma::kRegs;
+		float* mine = partial + (((int64_t)blockIdx.x * gridDim.y + blockIdx.y) * kBandThreads + tid) * kAccFloats;
+#pragma unroll
+		for (int j = 0; j < kW; ++j)
+#pragma unroll
+			for (int b = 0; b < MB; ++b)
+#pragma unroll
+				for (int r = 0; r < Mma::kRegs; r += 4)
+					*reinterpret_cast<float4_t*>(mine + (j * MB + b) * Mma::kRegs + r) =
+						float4_t{acc[j][b][r], acc[j][b][r + 1], acc[j][b][r + 2], acc[j][b][r + 3]};
+		return;
+	}
+	band_store<T, MR, MB, EPI>(acc, bias, C, M, N, ldc, n0, idx, grp, ep_param);
+}
+
+// Adds the partial sums of the `splits` K ranges of one tile in split order and finishes; one block per tile, the
+// thread layout of gemm_band_kernel.
+template <typename T, int MR, int MB, int EPI>
+__global__ __launch_bounds__(kBandThreads) void gemm_band_merge_kernel(
+	const float* __restrict__ partial, const float* __restrict__ bias, T* __restrict__ C,
+	int M, int64_t N, int64_t ldc, int splits, float ep_param)
+{
+	using S = BandShape<T, MR, MB>;
+	using Mma = BandMma<T, MR>;
+	constexpr int kW = S::kNG * (EPI == kEpiGeluMul ? 2 : 1);
+	constexpr int kAccFloats = kW * MB * Mma::kRegs;
+	const int tid = threadIdx.x;
+	const int lane = tid & (kWaveSize - 1);
+	typename Mma::Acc acc[kW][MB];
+#pragma unroll
+	for (int j = 0; j < kW; ++j)
+#pragma unroll
+		for (int b = 0; b < MB; ++b)
+#pragma unroll
+			for (int r = 0; r < Mma::kRegs; ++r) acc[j][b][r] = 0.0f;
+	const float* theirs = partial + ((int64_t)blockIdx.x * splits * kBandThreads + tid) * kAccFloats;
+	for (int sp = 0; sp < splits; ++sp, theirs += kBandThreads * kAccFloats)
+	{
+#pragma unroll
+		for (int j = 0; j < kW; ++j)
+#pragma unroll
+			for (int b = 0; b < MB; ++b)
+#pragma unroll
+				for (int r = 0; r < Mma::kRegs; r += 4)
+				{
+					const float4_t v = *reinterpret_cast<const float4_t*>(theirs + (j * MB + b) * Mma::kRegs + r);
+#pragma unroll
+					for (int e = 0; e < 4; ++e) acc[j][b][r + e] += v[e];
+				}
+	}
+	const int64_t n0 = (int64_t)blockIdx.x * kBandCols + (tid >> 6) * 32;
+	band_store<T, MR, MB, EPI>(acc, bias, C, M, N, ldc, n0, lane % MR, lane / MR, ep_param);
+}
+
+// Partial-sum workspace of one (device, stream) pair; NULL when there is none and none can be made now.
+float* band_workspace(hipStream_t stream)
+{
+	static std::mutex lock;
+	static std::map<std::pair<int, hipStream_t>, float*> cache;
+	int device = 0;
+	if (hipGetDevice(&device) != hipSuccess) return nullptr;
+	std::lock_guard<std::mutex> guard(lock);
+	const auto key = std::make_pair(device, stream);
+	const auto found = cache.find(key);
+	if (found != cache.end()) return found->second;
+	hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+	if (hipStreamIsCapturing(stream, &capture) != hipSuccess || capture != hipStreamCaptureStatusNone)
+	{
+		(void)hipGetLastError();
+		return nullptr;                       // no allocation under capture: the caller runs unsplit
+	}
+	void* base = nullptr;
+	if (hipMalloc(&base, kBandPartialBytes) != hipSuccess)
+	{
+		(void)hipGetLastError();
+		return nullptr;
+	}
+	cache.emplace(key, static_cast<float*>(base));
+	return static_cast<float*>(base);
+}
+
+template <typename T, int MR, int MB, int EPI>
+hipError_t launch_band(const T* A, const T* B, const T* B2, const float* bias, T* C, int M, int64_t N, int64_t K,
+                       int64_t lda, int64_t ldb, int64_t ldc, float ep_param, hipStream_t stream)
+{
+	using S = BandShape<T, MR, MB>;
+	constexpr int kAccFloats = S::kNG * (EPI == kEpiGeluMul ? 2 : 1) * MB * BandMma<T, MR>::kRegs;
+	const int64_t tiles = (N + kBandCols - 1) / kBandCols;
+	const int64_t kchunks = (K + S::kChunk - 1) / S::kChunk;
+	int64_t splits = 1;
+	if (tiles < kBandEnoughBlocks)
+	{
+		splits = (kBandWantedBlocks + tiles - 1) / tiles;
+		if (splits > kBandMaxSplits) splits = kBandMaxSplits;
+		// a split writes and reads back 8 bytes per sum where it streams depth * sizeof(T) bytes of weights per
+		// column: splits stay deep enough for the partial sums to be at most a quarter of the traffic
+		const int64_t min_depth = 32 * S::kRows / (int64_t)sizeof(T);
+		const int64_t min_chunks = (min_depth + S::kChunk - 1) / S::kChunk;
+		if (splits > kchunks / min_chunks) splits = kchunks / min_chunks;
+		const int64_t room = (int64_t)(kBandPartialBytes / (tiles * kBandThreads * kAccFloats * sizeof(float)));
+		if (splits > room) splits = room;
+		if (splits < 1) splits = 1;
+	}
+	int64_t chunks_per_split = (kchunks + splits - 1) / splits;
+	splits = (kchunks + chunks_per_split - 1) / chunks_per_split;
+	float* partial = nullptr;
+	if (splits > 1)
+	{
+		partial = band_workspace(stream);
+		if (!partial)
+		{
+			splits = 1;
+			chunks_per_split = kchunks;
+		}
+	}
+	discard_stale_error();
+	gemm_band_kernel<T, MR, MB, EPI><<<dim3((unsigned)tiles, (unsigned)splits), dim3(kBandThreads), 0, stream>>>(
+		A, B, B2, bias, C, partial, M, N, K, lda, ldb, ldc, (int)chunks_per_split, ep_param);
+	if (splits > 1)
+		gemm_band_merge_kernel<T, MR, MB, EPI><<<dim3((unsigned)tiles), dim3(kBandThreads), 0, stream>>>(
+			partial, bias, C, M, N, ldc, (int)splits, ep_param);
+	return hipGetLastError();
+}
+
+inline bool aligned16(const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; }
+
+}  // namespace
+
+template <typename T>
+bool gemm_band_applies(const T* A, const T* B, const T* B2, const T* C, int64_t M, int64_t N, int64_t K,
+                       int64_t lda, int64_t ldb, int64_t ldc, int b_layout)
+{
+	constexpr int EV = 16 / (int)sizeof(T);
+	if (b_layout != ANYGPU_B_COL_MAJOR) return false;
+	if (M < kBandMinRows || M > kBandMaxRows || N < 1 || K < 1) return false;
+	if ((N + kBandCols - 1) / kBandCols > 0x7FFFFFFFLL) return false;
+	// 33 .. 64 rows: two row blocks per weight register.  Worth it where the weights dominate and the columns or a
+	// deep K give the chip enough blocks (256000 x 2304 fp32, 64 rows: 711 us against 1238 us through the tiles;
+	// 2304 x 9216: 63 against 160); small weight matrices are quicker through the tile kernels.
+	if (M > 32 && N < kBandEnoughBlocks * kBandCols && K < 4096) return false;
+	// 16-byte loads along K from every row of A and B, 4-element stores along N
+	return K % EV == 0 && lda % EV == 0 && ldb % EV == 0 && ldc % 4 == 0 && aligned16(A) && aligned16(B) && aligned16(B2) &&
+	       reinterpret_cast<uintptr_t>(C) % (4 * sizeof(T)) == 0;
+}
+
+template <typename T>
+hipError_t launch_gemm_band(const T* A, const T* B, const T* B2, const float* bias, T* C,
+                            int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc,
+                            int epilogue, float ep_param, hipStream_t stream)
+{
+#define ANYGPU_BAND_ROWS(MR, MB) \
+	switch (epilogue) \
+	{ \
+	case kEpiSoftcap: return launch_band<T, MR, MB, kEpiSoftcap>(A, B, B2, bias, C, (int)M, N, K, lda, ldb, ldc, ep_param, stream); \
+	case kEpiGeluMul: return launch_band<T, MR, MB, kEpiGeluMul>(A, B, B2, bias, C, (int)M, N, K, lda, ldb, ldc, ep_param, stream); \
+	default: return launch_band<T, MR, MB, kEpiBias>(A, B, B2, bias, C, (int)M, N, K, lda, ldb, ldc, ep_param, stream); \
+	}
+	if (M <= 16) { ANYGPU_BAND_ROWS(16, 1) }
+	if (M <= 32) { ANYGPU_BAND_ROWS(32, 1) }
+	ANYGPU_BAND_ROWS(32, 2)
+#undef ANYGPU_BAND_ROWS
+}
+
+template bool gemm_band_applies<float>(const float*, const float*, const float*, const float*, int64_t, int64_t, int64_t,
+                                       int64_t, int64_t, int64_t, int);
+template bool gemm_band_applies<half_t>(const half_t*, const half_t*, const half_t*, const half_t*, int64_t, int64_t, int64_t,
+                                        int64_t, int64_t, int64_t, int);
+template hipError_t launch_gemm_band<float>(const float*, const float*, const float*, const float*, float*, int64_t, int64_t, int64_t,
+                                            int64_t, int64_t, int64_t, int, float, hipStream_t);
+template hipError_t launch_gemm_band<half_t>(const half_t*, const half_t*, const half_t*, const float*, half_t*, int64_t, int64_t, int64_t,
+                                             int64_t, int64_t, int64_t, int, float, hipStream_t);
+
+}  // namespace anygpu

@@ -100,6 +100,8 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
 	const half_t* b = static_cast<const half_t*>(B);
 	half_t* c = static_cast<half_t*>(C);
 
+	if (batch == 1 && gemm_band_applies<half_t>(a, b, nullptr, c, M, N, K, lda, ldb, ldc, b_layout))
+		return launch_gemm_band<half_t>(a, b, nullptr, nullptr, c, M, N, K, lda, ldb, ldc, 0, 0.0f, stream);
 	if (batch == 1 && gemm_skinny_applies<half_t>(a, b, nullptr, M, N, K, lda, ldb, b_layout))
 		return launch_gemm_skinny<half_t>(a, b, nullptr, nullptr, c, M, N, K, lda, ldb, ldc, b_layout, 0, 0.0f, stream);
 

@@ -371,6 +371,8 @@ hipError_t launch_gemm_f32(const float* A, const float* B, const float* bias, fl
                            int a_layout, int b_layout, hipStream_t stream)
 {
 	if (M == 0 || N == 0 || batch == 0) return hipSuccess;
+	if (batch == 1 && a_layout == ANYGPU_A_ROW_MAJOR && gemm_band_applies<float>(A, B, nullptr, C, M, N, K, lda, ldb, ldc, b_layout))
+		return launch_gemm_band<float>(A, B, nullptr, bias, C, M, N, K, lda, ldb, ldc, kEpiBias, 0.0f, stream);
 	if (batch == 1 && a_layout == ANYGPU_A_ROW_MAJOR && gemm_skinny_applies<float>(A, B, nullptr, M, N, K, lda, ldb, b_layout))
 		return launch_gemm_skinny<float>(A, B, nullptr, bias, C, M, N, K, lda, ldb, ldc, b_layout, kEpiBias, 0.0f, stream);
 #define ANYGPU_F32_LAYOUT(AL, BL) \
@@ -389,6 +391,8 @@ hipError_t launch_gemm_f32_softcap(const float* A, const float* B, float* C, int
                                    int64_t lda, int64_t ldb, int64_t ldc, int b_layout, float softcap, hipStream_t stream)
 {
 	if (M == 0 || N == 0) return hipSuccess;
+	if (gemm_band_applies<float>(A, B, nullptr, C, M, N, K, lda, ldb, ldc, b_layout))
+		return launch_gemm_band<float>(A, B, nullptr, nullptr, C, M, N, K, lda, ldb, ldc, kEpiSoftcap, softcap, stream);
 	if (gemm_skinny_applies<float>(A, B, nullptr, M, N, K, lda, ldb, b_layout))
 		return launch_gemm_skinny<float>(A, B, nullptr, nullptr, C, M, N, K, lda, ldb, ldc, b_layout, kEpiSoftcap, softcap, stream);
 	if (b_layout == ANYGPU_B_COL_MAJOR)
@@ -403,6 +407,8 @@ hipError_t launch_gemm_f32_gelu_mul(const float* A, const float* B_gate, const f
                                     int b_layout, hipStream_t stream)
 {
 	if (M == 0 || N == 0) return hipSuccess;
+	if (gemm_band_applies<float>(A, B_gate, B_up, C, M, N, K, lda, ldb, ldc, b_layout))
+		return launch_gemm_band<float>(A, B_gate, B_up, nullptr, C, M, N, K, lda, ldb, ldc, kEpiGeluMul, 0.0f, stream);
 	if (gemm_skinny_applies<float>(A, B_gate, B_up, M, N, K, lda, ldb, b_layout))
 		return launch_gemm_skinny<float>(A, B_gate, B_up, nullptr, C, M, N, K, lda, ldb, ldc, b_layout, kEpiGeluMul, 0.0f, stream);
 	if (b_layout == ANYGPU_B_COL_MAJOR)

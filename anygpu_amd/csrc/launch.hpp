@@ -85,4 +85,21 @@ hipError_t launch_gemm_skinny(const T* A, const T* B, const T* B2, const float* 
                               int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc,
                               int b_layout, int epilogue, float ep_param, hipStream_t stream);
 
+// Bands of few rows (kBandMinRows <= M <= kBandMaxRows, one product, row-major A, k-contiguous B): the
+// weights stream through the MFMA operand registers once, K is split over blocks when the columns alone do
+// not fill the chip.  Same arguments as the skinny launchers, which the launchers ask after these: from 5
+// rows on the FMA loops of the skinny kernels fall behind (256000 x 2304 fp32 weights, 8 rows: 511 us
+// against 398 us).
+constexpr int64_t kBandMinRows = 5;
+constexpr int64_t kBandMaxRows = 64;
+
+template <typename T>
+bool gemm_band_applies(const T* A, const T* B, const T* B2, const T* C, int64_t M, int64_t N, int64_t K,
+                       int64_t lda, int64_t ldb, int64_t ldc, int b_layout);
+
+template <typename T>
+hipError_t launch_gemm_band(const T* A, const T* B, const T* B2, const float* bias, T* C,
+                            int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc,
+                            int epilogue, float ep_param, hipStream_t stream);
+
 }  // namespace anygpu

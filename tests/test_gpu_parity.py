@@ -639,7 +639,62 @@ def test_mm_few_rows_integer_inputs_exact_and_padded_buffers(ops, oracle):
     assert np.all(got[:, 256:] == -1.0)
 
 
-@pytest.mark.parametrize("s", [1, 3, 8])
+@pytest.mark.parametrize("dtype", ["f16", "f32"])
+@pytest.mark.parametrize("m,k,n", [(9, 2304, 9216), (16, 9216, 2304), (17, 512, 1000), (32, 2304, 2052), (12, 72, 68),
+                                   (31, 264, 132), (24, 4096, 128), (10, 8, 4), (20, 1000, 130), (13, 16, 3000),
+                                   (33, 2304, 2052), (64, 9216, 2304), (48, 200, 1000), (5, 2304, 4100), (57, 72, 36),
+                                   (40, 520, 33000), (37, 4104, 260)])
+def test_mm_row_bands(ops, oracle, dtype, m, k, n):
+    # 5 <= M <= 64 against k-contiguous weights: the streaming kernels, with K split over blocks where N alone gives
+    # too few tiles (the split is invisible in the result: every launch adds the partial sums in the same order)
+    from anygpu_amd import capi
+    np_dt = np.float16 if dtype == "f16" else np.float32
+    a = synth.uniform(m * 3 + k, (m, k)).astype(np_dt)
+    bt = synth.uniform(k * 5 + n, (n, k)).astype(np_dt)
+    a32 = oracle.cvt_f16_to_f32(a) if dtype == "f16" else a
+    b32 = np.ascontiguousarray((oracle.cvt_f16_to_f32(bt) if dtype == "f16" else bt).T)
+    want = oracle.tensor_mm(a32, b32, threads=8)
+    da, db = dev(a), dev(bt)
+    got = host(ops.tensor_mm(da, db, b_layout=capi.B_COL_MAJOR))
+    tol = TOL_F16_GEMM if dtype == "f16" else TOL_F32
+    assert got.shape == (m, n)
+    assert scaled_rel_err(got.astype(np.float32), want, math.sqrt(k) / 3.0) <= tol
+    again = host(ops.tensor_mm(da, db, b_layout=capi.B_COL_MAJOR))
+    assert np.array_equal(got, again)
+
+
+def test_mm_row_bands_integer_inputs_exact_streams_and_padded_buffers(ops, oracle):
+    import torch
+    from anygpu_amd import capi
+    side = torch.cuda.Stream()
+    for (m, k, n) in [(9, 256, 96), (16, 2048, 260), (32, 1024, 1000), (27, 4096, 36), (64, 4096, 132), (40, 512, 5000)]:
+        a = synth.integers(1, (m, k), -4, 4)
+        b = synth.integers(2, (k, n), -4, 4)
+        bt = dev(np.ascontiguousarray(b.T))
+        want = oracle.tensor_mm(a, b)
+        assert np.array_equal(host(ops.tensor_mm(dev(a), bt, b_layout=capi.B_COL_MAJOR)), want)
+        bias = synth.integers(3, (n,), -9, 9)
+        assert np.array_equal(host(ops.tensor_gemm(dev(a), bt, dev(bias), b_layout=capi.B_COL_MAJOR)), oracle.tensor_gemm(a, b, bias))
+        a16, b16 = a.astype(np.float16), np.ascontiguousarray(b.T).astype(np.float16)
+        assert np.array_equal(host(ops.tensor_mm(dev(a16), dev(b16), b_layout=capi.B_COL_MAJOR)).astype(np.float32), want)
+        # a second stream has a workspace of its own
+        da = dev(a)
+        torch.cuda.synchronize()
+        with torch.cuda.stream(side):
+            got = ops.tensor_mm(da, bt, b_layout=capi.B_COL_MAJOR)
+        side.synchronize()
+        assert np.array_equal(host(got), want)
+    # operands and result inside wider buffers
+    abuf, bbuf = synth.uniform(4, (20, 200)), synth.uniform(5, (256, 300))
+    cbuf = torch.full((20, 400), -1.0, device="cuda")
+    ops.tensor_mm(dev(abuf)[:, :96], dev(bbuf)[:, :96], out=cbuf[:, :256], b_layout=capi.B_COL_MAJOR)
+    got = host(cbuf)
+    want = oracle.tensor_mm(np.ascontiguousarray(abuf[:, :96]), np.ascontiguousarray(bbuf[:, :96].T))
+    assert scaled_rel_err(got[:, :256], want, math.sqrt(96) / 3.0) <= TOL_F32
+    assert np.all(got[:, 256:] == -1.0)
+
+
+@pytest.mark.parametrize("s", [1, 3, 8, 9, 16, 29, 50])
 def test_gemm_epilogues_decode_step(ops, oracle, s):
     cap, hsize, vsize, isize = 30.0, 2304, 4000, 9216
     x = synth.normal(s, (1, s, hsize))
@@ -681,7 +736,7 @@ def test_mm_empty_and_rejected_arguments(ops):
 # =============================================================================================
 
 @pytest.mark.parametrize("b,s,hsize,vsize", [(1, 1, 1, 1), (2, 9, 300, 1000), (1, 5, 64, 37), (1, 128, 256, 512),
-                                             (3, 100, 130, 259), (1, 512, 512, 2048), (3, 100, 132, 260)])
+                                             (3, 100, 130, 259), (1, 512, 512, 2048), (3, 100, 132, 260), (1, 50, 4100, 300)])
 def test_gemma_linear_softcap_shapes(ops, oracle, b, s, hsize, vsize):
     cap = 30.0
     x = synth.normal(b * s + hsize, (b, s, hsize))
@@ -742,6 +797,23 @@ def test_gemma_mlp_fused_upproj_gemma2_2304_9216(ops, oracle):
     u = ops.tensor_mm(dev(x.reshape(s, hsize)), dev(wu))
     chain = host(torch.nn.functional.gelu(g, approximate="tanh") * u)
     assert scaled_rel_err(got.reshape(s, isize), chain, 1.0) <= TOL_F32
+
+
+@pytest.mark.parametrize("m,hsize,isize", [(3, 288, 1152), (12, 288, 1152), (32, 2304, 516), (17, 64, 40), (64, 4608, 300), (37, 2304, 9216)])
+def test_gemm_gelu_mul_k_contiguous_weights(ops, oracle, m, hsize, isize):
+    # the fused up-projection with the weights stored [intermediate, hidden], through the C entry point
+    import torch
+    from anygpu_amd import capi
+    x = synth.normal(m, (m, hsize))
+    wg = synth.normal(3, (hsize, isize)) * np.float32(1.0 / math.sqrt(hsize))
+    wu = synth.normal(4, (hsize, isize)) * np.float32(1.0 / math.sqrt(hsize))
+    want = oracle.gemma_mlp_upproj(x, wg, wu, threads=8)
+    dx, dg, du = dev(x), dev(np.ascontiguousarray(wg.T)), dev(np.ascontiguousarray(wu.T))
+    out = torch.empty((m, isize), device="cuda")
+    rc = capi.load().anygpu_gemm_f32_gelu_mul(dx.data_ptr(), dg.data_ptr(), du.data_ptr(), out.data_ptr(), m, isize, hsize,
+                                              hsize, hsize, isize, capi.B_COL_MAJOR, None)
+    assert rc == capi.ANYGPU_OK
+    assert scaled_rel_err(host(out), want, 1.0) <= TOL_F32
 
 
 def test_gemm_epilogues_rejected_arguments(ops):
