@@ -21,9 +21,7 @@
 // and cost more than the whole product: 60 - 90 us against 20.)  The workspace belongs to the
 // (device, stream) pair, is allocated on first use and kept for the life of the process, like the
 // workspace of a BLAS handle; a stream that is being captured and has none yet runs without the split.
-#include "device_utils.hpp"
-#include "gemm_epilogue.hpp"
-#include "launch.hpp"
+#include "gemm_band.hpp"
 #include "anygpu_hip.h"
 
 #include <map>
@@ -33,60 +31,11 @@
 
 namespace anygpu {
 
+using namespace band;
+
 namespace {
 
-constexpr int kBandThreads = 256;
 constexpr int kBandCols = 128;                    // output columns per block, 32 per wave
-constexpr int kBandMaxSplits = 32;
-constexpr int64_t kBandEnoughBlocks = 256;        // tiles from which K is not split
-constexpr int64_t kBandWantedBlocks = 512;
-constexpr size_t kBandPartialBytes = (size_t)16 << 20;
-
-typedef float4_t Vec;      // 16 raw bytes of either element type
-
-template <typename T, int MR> struct BandMma;
-
-template <> struct BandMma<float, 16>
-{
-	typedef float4_t Acc;
-	static constexpr int kRegs = 4;
-	__device__ static void mma(const Vec& w, const Vec& a, Acc& acc)
-	{
-#pragma unroll
-		for (int e = 0; e < 4; ++e) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(w[e], a[e], acc, 0, 0, 0);
-	}
-};
-
-template <> struct BandMma<float, 32>
-{
-	typedef float16_t Acc;
-	static constexpr int kRegs = 16;
-	__device__ static void mma(const Vec& w, const Vec& a, Acc& acc)
-	{
-#pragma unroll
-		for (int e = 0; e < 4; ++e) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(w[e], a[e], acc, 0, 0, 0);
-	}
-};
-
-template <> struct BandMma<half_t, 16>
-{
-	typedef float4_t Acc;
-	static constexpr int kRegs = 4;
-	__device__ static void mma(const Vec& w, const Vec& a, Acc& acc)
-	{
-		acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, w), __builtin_bit_cast(half8_t, a), acc, 0, 0, 0);
-	}
-};
-
-template <> struct BandMma<half_t, 32>
-{
-	typedef float16_t Acc;
-	static constexpr int kRegs = 16;
-	__device__ static void mma(const Vec& w, const Vec& a, Acc& acc)
-	{
-		acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, w), __builtin_bit_cast(half8_t, a), acc, 0, 0, 0);
-	}
-};
 
 template <typename T, int MR, int MB>
 struct BandShape
@@ -324,47 +273,99 @@ __global__ __launch_bounds__(kBandThreads) void gemm_band_kernel(
 	band_store<T, MR, MB, EPI>(acc, bias, C, M, N, ldc, n0, idx, grp, ep_param);
 }
 
-// Adds the partial sums of the `splits` K ranges of one tile in split order and finishes; one block per tile, the
-// thread layout of gemm_band_kernel.
+// Adds the partial sums of the `splits` K ranges in split order and finishes.  One thread per output vector of four
+// columns (tile, thread of gemm_band_kernel, column group, row block, register quad), so that the short,
+// latency-bound job is spread over many waves; the loads of four splits are in flight together and added in order.
 template <typename T, int MR, int MB, int EPI>
 __global__ __launch_bounds__(kBandThreads) void gemm_band_merge_kernel(
 	const float* __restrict__ partial, const float* __restrict__ bias, T* __restrict__ C,
-	int M, int64_t N, int64_t ldc, int splits, float ep_param)
+	int M, int64_t N, int64_t ldc, int splits, int64_t tiles, float ep_param)
 {
 	using S = BandShape<T, MR, MB>;
 	using Mma = BandMma<T, MR>;
-	constexpr int kW = S::kNG * (EPI == kEpiGeluMul ? 2 : 1);
-	constexpr int kAccFloats = kW * MB * Mma::kRegs;
-	const int tid = threadIdx.x;
+	constexpr bool DUAL = (EPI == kEpiGeluMul);
+	constexpr int kMats = DUAL ? 2 : 1;
+	constexpr int kQuads = Mma::kRegs / 4;
+	constexpr int kItems = S::kNG * MB * kQuads;            // output vectors per thread of the product kernel
+	constexpr int kAccFloats = kMats * kItems * 4;
+	const int64_t item = (int64_t)blockIdx.x * kBandThreads + threadIdx.x;
+	const int q = (int)(item % kItems);
+	const int tid = (int)((item / kItems) % kBandThreads);
+	const int64_t tile = item / (kItems * kBandThreads);
+	if (tile >= tiles) return;
+	const int j = q / (MB * kQuads), b = (q / kQuads) % MB, quad = q % kQuads;
 	const int lane = tid & (kWaveSize - 1);
-	typename Mma::Acc acc[kW][MB];
+	const int m = b * MR + lane % MR;
+	const int grp = lane / MR;
+	const int64_t n = tile * kBandCols + (tid >> 6) * 32 + j * MR + (MR == 16 ? 4 * grp : 8 * quad + 4 * grp);
+	if (m >= M || n >= N) return;
+
+	const int64_t stride = (int64_t)kBandThreads * kAccFloats;
+	const float* src = partial + (tile * splits * kBandThreads + tid) * kAccFloats + q * 4;
+	float4_t sum[kMats];
 #pragma unroll
-	for (int j = 0; j < kW; ++j)
+	for (int w = 0; w < kMats; ++w) sum[w] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+	int sp = 0;
+	for (; sp + 4 <= splits; sp += 4)
+	{
+		float4_t v[4][kMats];
 #pragma unroll
-		for (int b = 0; b < MB; ++b)
+		for (int i = 0; i < 4; ++i)
 #pragma unroll
-			for (int r = 0; r < Mma::kRegs; ++r) acc[j][b][r] = 0.0f;
-	const float* theirs = partial + ((int64_t)blockIdx.x * splits * kBandThreads + tid) * kAccFloats;
-	for (int sp = 0; sp < splits; ++sp, theirs += kBandThreads * kAccFloats)
+			for (int w = 0; w < kMats; ++w)
+				v[i][w] = *reinterpret_cast<const float4_t*>(src + (sp + i) * stride + w * kItems * 4);
+#pragma unroll
+		for (int i = 0; i < 4; ++i)
+#pragma unroll
+			for (int w = 0; w < kMats; ++w) sum[w] += v[i][w];
+	}
+	for (; sp < splits; ++sp)
+#pragma unroll
+		for (int w = 0; w < kMats; ++w) sum[w] += *reinterpret_cast<const float4_t*>(src + sp * stride + w * kItems * 4);
+
+	float4_t out;
+#pragma unroll
+	for (int e = 0; e < 4; ++e)
+	{
+		const float bias_n = (EPI == kEpiBias && bias && n + e < N) ? bias[n + e] : 0.0f;
+		out[e] = finish_sum<EPI>(sum[0][e], sum[kMats - 1][e], bias_n, ep_param);
+	}
+	T* dst = C + (int64_t)m * ldc + n;
+	if (n + 4 <= N) store4(dst, out);
+	else
 	{
 #pragma unroll
-		for (int j = 0; j < kW; ++j)
-#pragma unroll
-			for (int b = 0; b < MB; ++b)
-#pragma unroll
-				for (int r = 0; r < Mma::kRegs; r += 4)
-				{
-					const float4_t v = *reinterpret_cast<const float4_t*>(theirs + (j * MB + b) * Mma::kRegs + r);
-#pragma unroll
-					for (int e = 0; e < 4; ++e) acc[j][b][r + e] += v[e];
-				}
+		for (int e = 0; e < 4; ++e)
+			if (n + e < N) dst[e] = (T)out[e];
 	}
-	const int64_t n0 = (int64_t)blockIdx.x * kBandCols + (tid >> 6) * 32;
-	band_store<T, MR, MB, EPI>(acc, bias, C, M, N, ldc, n0, lane % MR, lane / MR, ep_param);
 }
 
+template <typename T, int MR, int MB, int EPI>
+hipError_t launch_band(const T* A, const T* B, const T* B2, const float* bias, T* C, int M, int64_t N, int64_t K,
+                       int64_t lda, int64_t ldb, int64_t ldc, float ep_param, hipStream_t stream)
+{
+	using S = BandShape<T, MR, MB>;
+	constexpr int kAccFloats = S::kNG * (EPI == kEpiGeluMul ? 2 : 1) * MB * BandMma<T, MR>::kRegs;
+	const int64_t tiles = (N + kBandCols - 1) / kBandCols;
+	const SplitPlan plan = plan_band_splits(tiles, K, S::kChunk, S::kRows, (int)sizeof(T), kAccFloats, stream);
+	const int64_t splits = plan.splits, chunks_per_split = plan.chunks_per_split;
+	float* partial = plan.partial;
+	discard_stale_error();
+	gemm_band_kernel<T, MR, MB, EPI><<<dim3((unsigned)tiles, (unsigned)splits), dim3(kBandThreads), 0, stream>>>(
+		A, B, B2, bias, C, partial, M, N, K, lda, ldb, ldc, (int)chunks_per_split, ep_param);
+	if (splits > 1)
+	{
+		const int64_t items = tiles * kBandThreads * (kAccFloats / (EPI == kEpiGeluMul ? 8 : 4));
+		gemm_band_merge_kernel<T, MR, MB, EPI><<<dim3((unsigned)((items + kBandThreads - 1) / kBandThreads)), dim3(kBandThreads), 0, stream>>>(
+			partial, bias, C, M, N, ldc, (int)splits, tiles, ep_param);
+	}
+	return hipGetLastError();
+}
+
+}  // namespace
+
 // Partial-sum workspace of one (device, stream) pair; NULL when there is none and none can be made now.
-float* band_workspace(hipStream_t stream)
+float* band::band_workspace(hipStream_t stream)
 {
 	static std::mutex lock;
 	static std::map<std::pair<int, hipStream_t>, float*> cache;
@@ -390,53 +391,6 @@ float* band_workspace(hipStream_t stream)
 	return static_cast<float*>(base);
 }
 
-template <typename T, int MR, int MB, int EPI>
-hipError_t launch_band(const T* A, const T* B, const T* B2, const float* bias, T* C, int M, int64_t N, int64_t K,
-                       int64_t lda, int64_t ldb, int64_t ldc, float ep_param, hipStream_t stream)
-{
-	using S = BandShape<T, MR, MB>;
-	constexpr int kAccFloats = S::kNG * (EPI == kEpiGeluMul ? 2 : 1) * MB * BandMma<T, MR>::kRegs;
-	const int64_t tiles = (N + kBandCols - 1) / kBandCols;
-	const int64_t kchunks = (K + S::kChunk - 1) / S::kChunk;
-	int64_t splits = 1;
-	if (tiles < kBandEnoughBlocks)
-	{
-		splits = (kBandWantedBlocks + tiles - 1) / tiles;
-		if (splits > kBandMaxSplits) splits = kBandMaxSplits;
-		// a split writes and reads back 8 bytes per sum where it streams depth * sizeof(T) bytes of weights per
-		// column: splits stay deep enough for the partial sums to be at most a quarter of the traffic
-		const int64_t min_depth = 32 * S::kRows / (int64_t)sizeof(T);
-		const int64_t min_chunks = (min_depth + S::kChunk - 1) / S::kChunk;
-		if (splits > kchunks / min_chunks) splits = kchunks / min_chunks;
-		const int64_t room = (int64_t)(kBandPartialBytes / (tiles * kBandThreads * kAccFloats * sizeof(float)));
-		if (splits > room) splits = room;
-		if (splits < 1) splits = 1;
-	}
-	int64_t chunks_per_split = (kchunks + splits - 1) / splits;
-	splits = (kchunks + chunks_per_split - 1) / chunks_per_split;
-	float* partial = nullptr;
-	if (splits > 1)
-	{
-		partial = band_workspace(stream);
-		if (!partial)
-		{
-			splits = 1;
-			chunks_per_split = kchunks;
-		}
-	}
-	discard_stale_error();
-	gemm_band_kernel<T, MR, MB, EPI><<<dim3((unsigned)tiles, (unsigned)splits), dim3(kBandThreads), 0, stream>>>(
-		A, B, B2, bias, C, partial, M, N, K, lda, ldb, ldc, (int)chunks_per_split, ep_param);
-	if (splits > 1)
-		gemm_band_merge_kernel<T, MR, MB, EPI><<<dim3((unsigned)tiles), dim3(kBandThreads), 0, stream>>>(
-			partial, bias, C, M, N, ldc, (int)splits, ep_param);
-	return hipGetLastError();
-}
-
-inline bool aligned16(const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; }
-
-}  // namespace
-
 template <typename T>
 bool gemm_band_applies(const T* A, const T* B, const T* B2, const T* C, int64_t M, int64_t N, int64_t K,
                        int64_t lda, int64_t ldb, int64_t ldc, int b_layout)
@@ -450,7 +404,7 @@ bool gemm_band_applies(const T* A, const T* B, const T* B2, const T* C, int64_t 
 	// 2304 x 9216: 63 against 160); small weight matrices are quicker through the tile kernels.
 	if (M > 32 && N < kBandEnoughBlocks * kBandCols && K < 4096) return false;
 	// 16-byte loads along K from every row of A and B, 4-element stores along N
-	return K % EV == 0 && lda % EV == 0 && ldb % EV == 0 && ldc % 4 == 0 && aligned16(A) && aligned16(B) && aligned16(B2) &&
+	return K % EV == 0 && lda % EV == 0 && ldb % EV == 0 && ldc % 4 == 0 && band::aligned16(A) && band::aligned16(B) && band::aligned16(B2) &&
 	       reinterpret_cast<uintptr_t>(C) % (4 * sizeof(T)) == 0;
 }
 

@@ -373,6 +373,9 @@ hipError_t launch_gemm_f32(const float* A, const float* B, const float* bias, fl
 	if (M == 0 || N == 0 || batch == 0) return hipSuccess;
 	if (batch == 1 && a_layout == ANYGPU_A_ROW_MAJOR && gemm_band_applies<float>(A, B, nullptr, C, M, N, K, lda, ldb, ldc, b_layout))
 		return launch_gemm_band<float>(A, B, nullptr, bias, C, M, N, K, lda, ldb, ldc, kEpiBias, 0.0f, stream);
+	if (batch == 1 && a_layout == ANYGPU_A_ROW_MAJOR && b_layout == ANYGPU_B_ROW_MAJOR &&
+	    gemm_band_ncontig_applies(A, B, nullptr, C, M, N, K, lda, ldb, ldc, false))
+		return launch_gemm_band_ncontig(A, B, nullptr, bias, C, M, N, K, lda, ldb, ldc, kEpiBias, 0.0f, stream);
 	if (batch == 1 && a_layout == ANYGPU_A_ROW_MAJOR && gemm_skinny_applies<float>(A, B, nullptr, M, N, K, lda, ldb, b_layout))
 		return launch_gemm_skinny<float>(A, B, nullptr, bias, C, M, N, K, lda, ldb, ldc, b_layout, kEpiBias, 0.0f, stream);
 #define ANYGPU_F32_LAYOUT(AL, BL) \
@@ -393,6 +396,8 @@ hipError_t launch_gemm_f32_softcap(const float* A, const float* B, float* C, int
 	if (M == 0 || N == 0) return hipSuccess;
 	if (gemm_band_applies<float>(A, B, nullptr, C, M, N, K, lda, ldb, ldc, b_layout))
 		return launch_gemm_band<float>(A, B, nullptr, nullptr, C, M, N, K, lda, ldb, ldc, kEpiSoftcap, softcap, stream);
+	if (b_layout == ANYGPU_B_ROW_MAJOR && gemm_band_ncontig_applies(A, B, nullptr, C, M, N, K, lda, ldb, ldc, false))
+		return launch_gemm_band_ncontig(A, B, nullptr, nullptr, C, M, N, K, lda, ldb, ldc, kEpiSoftcap, softcap, stream);
 	if (gemm_skinny_applies<float>(A, B, nullptr, M, N, K, lda, ldb, b_layout))
 		return launch_gemm_skinny<float>(A, B, nullptr, nullptr, C, M, N, K, lda, ldb, ldc, b_layout, kEpiSoftcap, softcap, stream);
 	if (b_layout == ANYGPU_B_COL_MAJOR)
@@ -409,6 +414,8 @@ hipError_t launch_gemm_f32_gelu_mul(const float* A, const float* B_gate, const f
 	if (M == 0 || N == 0) return hipSuccess;
 	if (gemm_band_applies<float>(A, B_gate, B_up, C, M, N, K, lda, ldb, ldc, b_layout))
 		return launch_gemm_band<float>(A, B_gate, B_up, nullptr, C, M, N, K, lda, ldb, ldc, kEpiGeluMul, 0.0f, stream);
+	if (b_layout == ANYGPU_B_ROW_MAJOR && gemm_band_ncontig_applies(A, B_gate, B_up, C, M, N, K, lda, ldb, ldc, true))
+		return launch_gemm_band_ncontig(A, B_gate, B_up, nullptr, C, M, N, K, lda, ldb, ldc, kEpiGeluMul, 0.0f, stream);
 	if (gemm_skinny_applies<float>(A, B_gate, B_up, M, N, K, lda, ldb, b_layout))
 		return launch_gemm_skinny<float>(A, B_gate, B_up, nullptr, C, M, N, K, lda, ldb, ldc, b_layout, kEpiGeluMul, 0.0f, stream);
 	if (b_layout == ANYGPU_B_COL_MAJOR)

@@ -663,6 +663,35 @@ def test_mm_row_bands(ops, oracle, dtype, m, k, n):
     assert np.array_equal(got, again)
 
 
+@pytest.mark.parametrize("m,k,n", [(9, 2304, 9216), (16, 9216, 2304), (17, 512, 1000), (32, 2304, 2052), (12, 72, 68),
+                                   (31, 264, 132), (24, 4096, 128), (10, 8, 4), (20, 1000, 132), (13, 16, 3000),
+                                   (64, 9216, 2304), (48, 200, 1000), (5, 2304, 4100), (57, 72, 36), (40, 520, 132000),
+                                   (37, 4104, 260), (8, 1028, 516)])
+def test_mm_f32_row_bands_n_contiguous_weights(ops, oracle, m, k, n):
+    # the same bands against weights stored [K, N], the layout of the reference's linear layers
+    import torch
+    a = synth.uniform(m * 3 + k, (m, k))
+    b = synth.uniform(k * 5 + n, (k, n))
+    want = oracle.tensor_mm(a, b, threads=8)
+    da, db = dev(a), dev(b)
+    got = host(ops.tensor_mm(da, db))
+    assert scaled_rel_err(got, want, math.sqrt(k) / 3.0) <= TOL_F32
+    assert np.array_equal(got, host(ops.tensor_mm(da, db)))
+    bias = synth.uniform(7, (n,))
+    got = host(ops.tensor_gemm(da, db, dev(bias)))
+    assert scaled_rel_err(got, want + bias, math.sqrt(k) / 3.0) <= TOL_F32
+    if m <= 40 and n <= 9216:
+        ai, bi = synth.integers(1, (m, k), -4, 4), synth.integers(2, (k, n), -4, 4)
+        assert np.array_equal(host(ops.tensor_mm(dev(ai), dev(bi))), oracle.tensor_mm(ai, bi, threads=8))
+        # operands and result inside wider buffers
+        abuf, bbuf = torch.zeros((m, k + 8), device="cuda"), torch.zeros((k, n + 12), device="cuda")
+        abuf[:, :k], bbuf[:, :n] = da, db
+        cbuf = torch.full((m, n + 4), -1.0, device="cuda")
+        ops.tensor_mm(abuf[:, :k], bbuf[:, :n], out=cbuf[:, :n])
+        assert np.array_equal(host(cbuf[:, :n]), host(ops.tensor_mm(da, db)))
+        assert bool((cbuf[:, n:] == -1.0).all())
+
+
 def test_mm_row_bands_integer_inputs_exact_streams_and_padded_buffers(ops, oracle):
     import torch
     from anygpu_amd import capi
@@ -764,7 +793,7 @@ def test_gemma_linear_softcap_gemma2_hidden_2304_vocab_slice(ops, oracle):
     assert np.max(np.abs(logits.reshape(s, vsize).sum(axis=1) - row_sum)) < 2e-3 * vsize
 
 
-@pytest.mark.parametrize("b,s,hsize,isize", [(1, 1, 1, 1), (1, 37, 288, 1152), (2, 5, 64, 37), (1, 128, 256, 512),
+@pytest.mark.parametrize("b,s,hsize,isize", [(1, 1, 1, 1), (1, 37, 288, 1152), (1, 9, 2304, 1156), (2, 16, 520, 9216), (2, 5, 64, 37), (1, 128, 256, 512),
                                              (3, 50, 130, 259), (1, 256, 512, 2048), (3, 50, 132, 260)])
 def test_gemma_mlp_fused_upproj_shapes(ops, oracle, b, s, hsize, isize):
     x = synth.normal(b * s + hsize, (b, s, hsize))
