@@ -16,6 +16,7 @@
 #include "device_utils.hpp"
 #include "gemm_epilogue.hpp"
 #include "launch.hpp"
+#include "gemm_band.hpp"
 #include "anygpu_hip.h"
 
 #include <type_traits>
@@ -28,7 +29,6 @@ constexpr int kAccessAligned = 1;   // 16-byte aligned rows and leading dimensio
 constexpr int kAccessAny = 2;       // nothing assumed: vectors at element alignment, guarded ends
 
 constexpr int kBK = 16;
-constexpr int64_t kBigTileThreshold = 256;    // 128 x 128 tiles once they give every one of the 256 CUs a block
 constexpr int kPitchK = kBK + 4;     // floats per [row][k] LDS row: 80 bytes, keeps 16-byte alignment
 
 // Scheduling-group masks of __builtin_amdgcn_sched_group_barrier
@@ -125,10 +125,16 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(
 	const float* __restrict__ A, const float* __restrict__ B, const float* __restrict__ B2,
 	const float* __restrict__ bias, float* __restrict__ C,
 	int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc,
-	int64_t stride_a, int64_t stride_b, int64_t stride_c, float ep_param)
+	int64_t stride_a, int64_t stride_b, int64_t stride_c, float ep_param, int64_t k_split)
 {
 	constexpr bool DUAL = (EPI == kEpiGeluMul);
 	constexpr bool FULL = (ACCESS == kAccessFull);
+	if (k_split > 0)
+	{
+		// blockIdx.z counts ranges of K of one product instead of products: the strides step along K
+		const int64_t left = K - (int64_t)blockIdx.z * k_split;
+		K = left < k_split ? left : k_split;
+	}
 	A += (int64_t)blockIdx.z * stride_a;
 	B += (int64_t)blockIdx.z * stride_b;
 	C += (int64_t)blockIdx.z * stride_c;
@@ -323,45 +329,172 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(
 	}
 }
 
+// One launch of the tile kernel.  k_split > 0: `batch` ranges of K (k_split deep) of a single product, see the kernel.
 template <int A_LAYOUT, int B_LAYOUT, int BM, int BN, int EPI>
-static hipError_t launch_tiles(const float* A, const float* B, const float* B2, const float* bias, float* C,
-                                int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc,
-                                int64_t stride_a, int64_t stride_b, int64_t stride_c, int64_t batch,
-                                float ep_param, hipStream_t stream)
+static hipError_t launch_tiles_once(const float* A, const float* B, const float* B2, const float* bias, float* C,
+                                    int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc,
+                                    int64_t stride_a, int64_t stride_b, int64_t stride_c, int64_t batch,
+                                    float ep_param, int64_t k_split, hipStream_t stream)
 {
 	const dim3 grid((unsigned)((N + BN - 1) / BN), (unsigned)((M + BM - 1) / BM), (unsigned)batch);
 	const bool aligned = (reinterpret_cast<uintptr_t>(A) % 16 == 0) && (reinterpret_cast<uintptr_t>(B) % 16 == 0) &&
 	                     (reinterpret_cast<uintptr_t>(B2) % 16 == 0) &&
 	                     (reinterpret_cast<uintptr_t>(C) % 16 == 0) && (lda % 4 == 0) && (ldb % 4 == 0) && (ldc % 4 == 0) &&
 	                     (stride_a % 4 == 0) && (stride_b % 4 == 0) && (stride_c % 4 == 0);
-	const bool full = aligned && (M % BM == 0) && (N % BN == 0) && (K % kBK == 0);
+	const bool full = aligned && (M % BM == 0) && (N % BN == 0) && (K % kBK == 0) && (k_split % kBK == 0);
 	discard_stale_error();
 	if (full)
 		gemm_f32_kernel<A_LAYOUT, B_LAYOUT, kAccessFull, BM, BN, EPI><<<grid, dim3(256), 0, stream>>>(
-			A, B, B2, bias, C, M, N, K, lda, ldb, ldc, stride_a, stride_b, stride_c, ep_param);
+			A, B, B2, bias, C, M, N, K, lda, ldb, ldc, stride_a, stride_b, stride_c, ep_param, k_split);
 	else if (aligned)
 		gemm_f32_kernel<A_LAYOUT, B_LAYOUT, kAccessAligned, BM, BN, EPI><<<grid, dim3(256), 0, stream>>>(
-			A, B, B2, bias, C, M, N, K, lda, ldb, ldc, stride_a, stride_b, stride_c, ep_param);
+			A, B, B2, bias, C, M, N, K, lda, ldb, ldc, stride_a, stride_b, stride_c, ep_param, k_split);
 	else
 		gemm_f32_kernel<A_LAYOUT, B_LAYOUT, kAccessAny, BM, BN, EPI><<<grid, dim3(256), 0, stream>>>(
-			A, B, B2, bias, C, M, N, K, lda, ldb, ldc, stride_a, stride_b, stride_c, ep_param);
+			A, B, B2, bias, C, M, N, K, lda, ldb, ldc, stride_a, stride_b, stride_c, ep_param, k_split);
 	return hipGetLastError();
 }
 
-// Tile choice: 128 x 128 tiles have the best operand reuse (2048^3: 153 us against 183 us with
-// 64 x 64 tiles); problems too small to give every CU one of them take 64 x 64 tiles to spread out.
+// C[m, n] = finish(sum over splits of partial[split][m][n]), one thread per four columns, splits added in order
+template <int EPI, bool VEC>
+__global__ __launch_bounds__(256) void gemm_f32_split_merge_kernel(
+	const float* __restrict__ partial, const float* __restrict__ bias, float* __restrict__ C,
+	int64_t M, int64_t N, int64_t ldc, int splits, float ep_param)
+{
+	const int64_t quads = (N + 3) / 4;
+	const int64_t item = (int64_t)blockIdx.x * 256 + threadIdx.x;
+	const int64_t m = item / quads;
+	const int64_t n = (item % quads) * 4;
+	if (m >= M) return;
+	const int64_t plane = M * N;
+	const float* src = partial + m * N + n;
+	float4_t sum = {0.0f, 0.0f, 0.0f, 0.0f};
+	if (VEC)
+	{
+		int sp = 0;
+		for (; sp + 4 <= splits; sp += 4)
+		{
+			float4_t v[4];
+#pragma unroll
+			for (int i = 0; i < 4; ++i) v[i] = *reinterpret_cast<const float4_t*>(src + (sp + i) * plane);
+#pragma unroll
+			for (int i = 0; i < 4; ++i) sum += v[i];
+		}
+		for (; sp < splits; ++sp) sum += *reinterpret_cast<const float4_t*>(src + sp * plane);
+	}
+	else
+	{
+		for (int sp = 0; sp < splits; ++sp)
+#pragma unroll
+			for (int e = 0; e < 4; ++e)
+				if (n + e < N) sum[e] += src[sp * plane + e];
+	}
+#pragma unroll
+	for (int e = 0; e < 4; ++e)
+	{
+		const float bias_n = (EPI == kEpiBias && bias && n + e < N) ? bias[n + e] : 0.0f;
+		sum[e] = finish_sum<EPI>(sum[e], 0.0f, bias_n, ep_param);
+	}
+	if (VEC) *reinterpret_cast<float4_t*>(C + m * ldc + n) = sum;
+	else
+	{
+#pragma unroll
+		for (int e = 0; e < 4; ++e)
+			if (n + e < N) C[m * ldc + n + e] = sum[e];
+	}
+}
+
+// Tiling plan.  A CU works on the blocks it was given side by side, so a launch of 288 tiles takes as long as one
+// of 512: some CUs have two blocks.  Two remedies, both priced by a small model of the launch: the smaller tile,
+// and for a single product a cut along K.  The model counts "rounds" (blocks per CU) times the 16-deep slabs times
+// the time per slab and round, 1.0 us for a 128 x 128 tile and 0.36 us for a 64 x 64 one (2048^3 at 131 us and
+// 183 us).  Rounds are whole numbers for the big tile; the small one, of which a CU holds several at once, was
+// measured to follow the average beyond two per CU (per slab: 64 tiles 0.32 us, 288 0.64, 576 0.83, 1024 1.43).  Every range of K is then a launch "batch" that writes raw sums to its own [M, N]
+// plane of the stream's workspace and a merge kernel adds the planes in order and applies the epilogue; the model
+// charges it the merge launch and the traffic of the planes.
+struct TilePlan
+{
+	int tile;          // 128 or 64
+	int64_t splits;    // ranges of K, 1 = no cut
+	double cost;       // modelled time in us
+};
+
+constexpr int64_t kSplitMinDepth = 256;
+constexpr int64_t kSplitMax = 16;
+constexpr int64_t kChipCus = 256;
+
+static TilePlan plan_tiles(int tile, int64_t M, int64_t N, int64_t K, int64_t batch, bool may_split)
+{
+	const double slab_us = tile == 128 ? 1.0 : 0.36;
+	const int64_t tiles = ((M + tile - 1) / tile) * ((N + tile - 1) / tile) * batch;
+	const int64_t slabs = (K + kBK - 1) / kBK;
+	const auto rounds_of = [tile](int64_t blocks) {
+		if (tile == 64 && blocks > 2 * kChipCus) return (double)blocks / (double)kChipCus;
+		return (double)((blocks + kChipCus - 1) / kChipCus);
+	};
+	TilePlan best{tile, 1, rounds_of(tiles) * (double)slabs * slab_us};
+	if (!may_split || batch != 1) return best;
+	const int64_t room = (int64_t)(band::kBandPartialBytes / ((size_t)M * N * sizeof(float)));
+	for (int64_t s = 2; s <= kSplitMax && s <= K / kSplitMinDepth && s <= room; ++s)
+	{
+		const double rounds = rounds_of(tiles * s);
+		const double planes_us = 8.0 * (double)s * (double)M * (double)N / 3.0e6;    // written and read back at ~3 TB/s
+		const double cost = rounds * ((double)slabs / (double)s + 5.0) * slab_us + 3.0 + planes_us;
+		if (cost < best.cost * 0.9) best = TilePlan{tile, s, cost};
+	}
+	return best;
+}
+
+template <int A_LAYOUT, int B_LAYOUT, int BM, int BN, int EPI>
+static hipError_t launch_tiles(const float* A, const float* B, const float* B2, const float* bias, float* C,
+                                int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc,
+                                int64_t stride_a, int64_t stride_b, int64_t stride_c, int64_t batch,
+                                float ep_param, int64_t splits, hipStream_t stream)
+{
+	if constexpr (EPI != kEpiGeluMul)
+	{
+		if (splits > 1)
+		{
+			int64_t k_split = (K + splits - 1) / splits;
+			k_split = (k_split + kBK - 1) / kBK * kBK;
+			splits = (K + k_split - 1) / k_split;
+			float* partial = splits > 1 ? band::band_workspace(stream) : nullptr;
+			if (partial)
+			{
+				const int64_t step_a = (A_LAYOUT == ANYGPU_A_ROW_MAJOR) ? k_split : k_split * lda;
+				const int64_t step_b = (B_LAYOUT == ANYGPU_B_COL_MAJOR) ? k_split : k_split * ldb;
+				const hipError_t err = launch_tiles_once<A_LAYOUT, B_LAYOUT, BM, BN, kEpiBias>(
+					A, B, nullptr, nullptr, partial, M, N, K, lda, ldb, N, step_a, step_b, M * N, splits, 0.0f, k_split, stream);
+				if (err != hipSuccess) return err;
+				const int64_t items = M * ((N + 3) / 4);
+				const dim3 grid((unsigned)((items + 255) / 256));
+				const bool vec = (N % 4 == 0) && (ldc % 4 == 0) && (reinterpret_cast<uintptr_t>(C) % 16 == 0);
+				if (vec)
+					gemm_f32_split_merge_kernel<EPI, true><<<grid, dim3(256), 0, stream>>>(partial, bias, C, M, N, ldc, (int)splits, ep_param);
+				else
+					gemm_f32_split_merge_kernel<EPI, false><<<grid, dim3(256), 0, stream>>>(partial, bias, C, M, N, ldc, (int)splits, ep_param);
+				return hipGetLastError();
+			}
+		}
+	}
+	return launch_tiles_once<A_LAYOUT, B_LAYOUT, BM, BN, EPI>(A, B, B2, bias, C, M, N, K, lda, ldb, ldc,
+	                                                          stride_a, stride_b, stride_c, batch, ep_param, 0, stream);
+}
+
 template <int A_LAYOUT, int B_LAYOUT, int EPI>
 static hipError_t launch_layout(const float* A, const float* B, const float* B2, const float* bias, float* C,
                                 int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc,
                                 int64_t stride_a, int64_t stride_b, int64_t stride_c, int64_t batch,
                                 float ep_param, hipStream_t stream)
 {
-	const int64_t big_tiles = ((M + 127) / 128) * ((N + 127) / 128) * batch;
-	if (big_tiles >= kBigTileThreshold)
+	const bool may_split = (EPI != kEpiGeluMul);
+	const TilePlan big = plan_tiles(128, M, N, K, batch, may_split);
+	const TilePlan small = plan_tiles(64, M, N, K, batch, may_split);
+	if (big.cost <= small.cost)
 		return launch_tiles<A_LAYOUT, B_LAYOUT, 128, 128, EPI>(A, B, B2, bias, C, M, N, K, lda, ldb, ldc,
-		                                                       stride_a, stride_b, stride_c, batch, ep_param, stream);
+		                                                       stride_a, stride_b, stride_c, batch, ep_param, big.splits, stream);
 	return launch_tiles<A_LAYOUT, B_LAYOUT, 64, 64, EPI>(A, B, B2, bias, C, M, N, K, lda, ldb, ldc,
-	                                                     stride_a, stride_b, stride_c, batch, ep_param, stream);
+	                                                     stride_a, stride_b, stride_c, batch, ep_param, small.splits, stream);
 }
 
 hipError_t launch_gemm_f32(const float* A, const float* B, const float* bias, float* C,

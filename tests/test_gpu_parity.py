@@ -445,6 +445,32 @@ def test_mm_f32_shapes_and_layouts(ops, oracle, layout, m, k, n):
     assert scaled_rel_err(got, want, floor) <= TOL_F32
 
 
+@pytest.mark.parametrize("layout", ["row", "col"])
+@pytest.mark.parametrize("m,k,n", [(128, 2304, 2048), (65, 1000, 130), (100, 4096, 72), (200, 1024, 516), (70, 515, 33),
+                                   (512, 9216, 256)])
+def test_mm_f32_few_tiles_split_along_k(ops, oracle, layout, m, k, n):
+    # products whose tiles would not fill the chip are cut along K and merged; the cut is invisible in the result
+    from anygpu_amd import capi
+    a = synth.uniform(m + k, (m, k))
+    b = synth.uniform(k + n, (k, n))
+    want = oracle.tensor_mm(a, b, threads=8)
+    da = dev(a)
+    db = dev(b) if layout == "row" else dev(np.ascontiguousarray(b.T))
+    lay = capi.B_ROW_MAJOR if layout == "row" else capi.B_COL_MAJOR
+    got = host(ops.tensor_mm(da, db, b_layout=lay))
+    assert scaled_rel_err(got, want, math.sqrt(k) / 3.0) <= TOL_F32
+    assert np.array_equal(got, host(ops.tensor_mm(da, db, b_layout=lay)))
+    bias = synth.uniform(9, (n,))
+    got = host(ops.tensor_gemm(da, db, dev(bias), b_layout=lay))
+    assert scaled_rel_err(got, want + bias, math.sqrt(k) / 3.0) <= TOL_F32
+    ai, bi = synth.integers(1, (m, k), -4, 4), synth.integers(2, (k, n), -4, 4)
+    dbi = dev(bi) if layout == "row" else dev(np.ascontiguousarray(bi.T))
+    assert np.array_equal(host(ops.tensor_mm(dev(ai), dbi, b_layout=lay)), oracle.tensor_mm(ai, bi, threads=8))
+    if layout == "row":
+        got = host(ops.tensor_mm(dev(np.ascontiguousarray(a.T)), db, a_layout=capi.A_COL_MAJOR))
+        assert scaled_rel_err(got, want, math.sqrt(k) / 3.0) <= TOL_F32
+
+
 def test_mm_f32_transposed_left_operand(ops, oracle):
     # the layout of the reference's last fp32 rung: A handed over as [K, M]
     from anygpu_amd import capi
