@@ -9,6 +9,7 @@
 #include "device_utils.hpp"
 #include "gemm_f16_tile.hpp"
 #include "launch.hpp"
+#include "gemm_band.hpp"
 #include "anygpu_hip.h"
 
 namespace anygpu {
@@ -90,6 +91,51 @@ __global__ __launch_bounds__(256) void gemm_f16_edge_kernel(
 	}
 }
 
+// C[m, n] = half(sum over splits of planes[split][m][n]), one thread per eight columns (N a multiple of 8), the
+// planes added in order
+__global__ __launch_bounds__(256) void gemm_f16_split_merge_kernel(
+	const float* __restrict__ planes, half_t* __restrict__ C, int64_t M, int64_t N, int64_t ldc, int splits)
+{
+	const int64_t chunks = N / 8;
+	const int64_t item = (int64_t)blockIdx.x * 256 + threadIdx.x;
+	const int64_t m = item / chunks;
+	const int64_t n = (item % chunks) * 8;
+	if (m >= M) return;
+	const int64_t plane = M * N;
+	const float* src = planes + m * N + n;
+	float4_t lo = {0.0f, 0.0f, 0.0f, 0.0f}, hi = {0.0f, 0.0f, 0.0f, 0.0f};
+	int sp = 0;
+	for (; sp + 4 <= splits; sp += 4)
+	{
+		float4_t v[4][2];
+#pragma unroll
+		for (int i = 0; i < 4; ++i)
+		{
+			v[i][0] = *reinterpret_cast<const float4_t*>(src + (sp + i) * plane);
+			v[i][1] = *reinterpret_cast<const float4_t*>(src + (sp + i) * plane + 4);
+		}
+#pragma unroll
+		for (int i = 0; i < 4; ++i)
+		{
+			lo += v[i][0];
+			hi += v[i][1];
+		}
+	}
+	for (; sp < splits; ++sp)
+	{
+		lo += *reinterpret_cast<const float4_t*>(src + sp * plane);
+		hi += *reinterpret_cast<const float4_t*>(src + sp * plane + 4);
+	}
+	half8_t out;
+#pragma unroll
+	for (int e = 0; e < 4; ++e)
+	{
+		out[e] = (half_t)lo[e];
+		out[4 + e] = (half_t)hi[e];
+	}
+	*reinterpret_cast<half8_t*>(C + m * ldc + n) = out;
+}
+
 hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K,
                            int64_t lda, int64_t ldb, int64_t ldc,
                            int64_t stride_a, int64_t stride_b, int64_t stride_c, int64_t batch,
@@ -120,11 +166,77 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
 		// it run the same kernels with clamped operand rows and guarded stores; a K that is not a multiple of the
 		// 64-deep slab adds a tail multiplied from registers.
 		const auto blocks = [&](int64_t tile) { return ((M + tile - 1) / tile) * ((N + tile - 1) / tile) * batch; };
-		constexpr int64_t kEnoughBlocks = 192;
-		const int64_t tile = blocks(256) >= kEnoughBlocks ? 256 : blocks(128) >= kEnoughBlocks ? 128 : 64;
+		// Time per 64-deep slab of `nblocks` blocks spread over 256 CUs, in us, from measurements: a 256 x 256 tile takes
+		// 1.56 per round of blocks (4096^3: 256 blocks, 64 slabs, 100 us); the smaller tiles, of which a CU holds several,
+		// follow the average number of blocks per CU with a floor where a lone block waits on latency: 0.75 per block
+		// and CU for 128 x 128 (144 blocks 0.75 - 1.0, 288 1.0, 576 1.7 - 2.0), 0.27 for 64 x 64 with a floor of 0.43.
+		// The cheapest launch is taken, the bigger tile on a tie.
+		const auto slab_us = [](int64_t t, int64_t nblocks) {
+			const double rounds = (double)((nblocks + 255) / 256);
+			const double share = nblocks > 256 ? (double)nblocks / 256.0 : 1.0;
+			if (t == 256) return 1.56 * rounds;
+			if (t == 128) return 0.75 * share;
+			return 0.27 * share > 0.43 ? 0.27 * share : 0.43;
+		};
+		const double cost256 = slab_us(256, blocks(256)), cost128 = slab_us(128, blocks(128)), cost64 = slab_us(64, blocks(64));
+		const int64_t tile = (cost256 <= cost128 && cost256 <= cost64) ? 256 : cost128 <= cost64 ? 128 : 64;
 		// one "general" instantiation serves ragged M / N and a K tail alike
 		const bool ragged = (M % tile != 0) || (N % tile != 0) || (K % 64 != 0);
 		const bool fits = ((M + tile - 1) / tile) * ((N + tile - 1) / tile) <= 0x7FFFFFFFLL;
+
+		// A single product with fewer blocks than CUs and a deep K is cut along K: every range is a launch "batch"
+		// writing raw fp32 sums to its own [M, N] plane of the stream's workspace, and a merge kernel adds the planes
+		// in order and rounds once.  Priced with the same slab times plus the merge launch and the traffic of the planes.
+		if (fits && batch == 1 && blocks(tile) < 256 && K >= 1024)
+		{
+			const double slabs = (double)(K / 64);
+			double best = slabs * slab_us(tile, blocks(tile));
+			int64_t splits = 1;
+			const int64_t room = (int64_t)(band::kBandPartialBytes / ((size_t)M * N * sizeof(float)));
+			for (int64_t s = 2; s <= 16 && s <= K / 512 && s <= room; ++s)
+			{
+				const double cost = (slabs / (double)s + 3.0) * slab_us(tile, blocks(tile) * s) + 3.0 + 8.0 * (double)s * (double)M * (double)N / 3.0e6;
+				if (cost < 0.85 * best)
+				{
+					best = cost;
+					splits = s;
+				}
+			}
+			int64_t k_split = 0;
+			while (splits > 1)
+			{
+				k_split = ((K + splits - 1) / splits + 63) / 64 * 64;
+				const int64_t ranges = (K + k_split - 1) / k_split;
+				if (ranges == splits && K - (splits - 1) * k_split >= 64) break;     // every range holds at least a slab
+				splits = ranges == splits ? splits - 1 : ranges;
+			}
+			float* planes = splits > 1 ? band::band_workspace(stream) : nullptr;
+			if (planes)
+			{
+				const int64_t step_b = (b_layout == ANYGPU_B_COL_MAJOR) ? k_split : k_split * ldb;
+				hipError_t err;
+#define ANYGPU_F16_SPLIT(BT, WM, WN, KN) \
+				err = launch_gemm_f16_tile<GemmTileCfg<BT, BT, WM, WN, 1, 0, 4, 16, KN>, true, true, true>( \
+					a, b, c, M, N, K, lda, ldb, ldc, k_split, step_b, 0, splits, stream, planes, k_split)
+				if (b_layout == ANYGPU_B_COL_MAJOR)
+				{
+					if (tile == 256) ANYGPU_F16_SPLIT(256, 2, 4, false);
+					else if (tile == 128) ANYGPU_F16_SPLIT(128, 2, 2, false);
+					else ANYGPU_F16_SPLIT(64, 2, 2, false);
+				}
+				else
+				{
+					if (tile == 256) ANYGPU_F16_SPLIT(256, 2, 4, true);
+					else if (tile == 128) ANYGPU_F16_SPLIT(128, 2, 2, true);
+					else ANYGPU_F16_SPLIT(64, 2, 2, true);
+				}
+#undef ANYGPU_F16_SPLIT
+				if (err != hipSuccess) return err;
+				const int64_t items = M * (N / 8);
+				gemm_f16_split_merge_kernel<<<dim3((unsigned)((items + 255) / 256)), dim3(256), 0, stream>>>(planes, c, M, N, ldc, (int)splits);
+				return hipGetLastError();
+			}
+		}
 #define ANYGPU_F16_TILE(BT, WM, WN, KN) \
 		return ragged ? launch_gemm_f16_tile<GemmTileCfg<BT, BT, WM, WN, 1, 0, 4, 16, KN>, true, true>(a, b, c, M, N, K, lda, ldb, ldc, stride_a, stride_b, stride_c, batch, stream) \
 		              : launch_gemm_f16_tile<GemmTileCfg<BT, BT, WM, WN, 1, 0, 4, 16, KN>, false, false>(a, b, c, M, N, K, lda, ldb, ldc, stride_a, stride_b, stride_c, batch, stream)

@@ -203,6 +203,32 @@ __device__ __forceinline__ void store_patch_via_lds(
 	}
 }
 
+// The patch as raw fp32 sums into an [M, N] plane (ld = N, a multiple of 8): every lane stores its groups of four
+// consecutive columns directly.  Rows at or beyond M and columns at or beyond N are not stored.
+template <typename Cfg>
+__device__ __forceinline__ void store_patch_f32(
+	const typename MfmaShape<Cfg::MI>::Acc (&acc)[Cfg::kTilesM][Cfg::kTilesN],
+	float* __restrict__ plane, int64_t m_base, int64_t n_base, int lane, int64_t M, int64_t N)
+{
+	using Shape = MfmaShape<Cfg::MI>;
+	constexpr int MI = Cfg::MI;
+#pragma unroll
+	for (int i = 0; i < Cfg::kTilesM; ++i)
+	{
+		const int64_t m = m_base + i * MI + lane % MI;
+#pragma unroll
+		for (int j = 0; j < Cfg::kTilesN; ++j)
+#pragma unroll
+			for (int g = 0; g < Shape::kAccRegs / 4; ++g)
+			{
+				const int64_t n = n_base + j * MI + Shape::first_row_of_group(g, lane);
+				if (m < M && n < N)
+					*reinterpret_cast<float4_t*>(plane + m * N + n) =
+						float4_t{acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
+			}
+	}
+}
+
 // Scheduling-group masks of __builtin_amdgcn_sched_group_barrier
 constexpr int kSchedMfma = 0x008;
 constexpr int kSchedVmemRead = 0x020;
@@ -219,13 +245,21 @@ constexpr int kSchedDsRead = 0x100;
 // KTAIL: K need not be a multiple of the 64-deep slab (K >= 64, a multiple of 8).  The slabs cover
 // the multiple; the remaining K % 64 columns are multiplied after the loop from fragments that
 // every lane loads straight from global memory in the MFMA operand layout, zeros past K.
-template <typename Cfg, bool RAGGED = false, bool KTAIL = false>
+// SPLIT: blockIdx.y walks ranges of K (k_split deep, the strides step along K) of one product instead of a batch,
+// and the raw fp32 sums of range y go to planes[y][M][N]; C is not touched.
+template <typename Cfg, bool RAGGED = false, bool KTAIL = false, bool SPLIT = false>
 __global__ __launch_bounds__(Cfg::kThreads) void gemm_f16_nt_tile_kernel(
 	const half_t* __restrict__ A, const half_t* __restrict__ B, half_t* __restrict__ C,
 	int K, int64_t lda, int64_t ldb, int64_t ldc, int tiles_m, int tiles_n,
-	int64_t stride_a, int64_t stride_b, int64_t stride_c, int64_t M, int64_t N)
+	int64_t stride_a, int64_t stride_b, int64_t stride_c, int64_t M, int64_t N,
+	float* __restrict__ planes, int k_split)
 {
 	using Shape = MfmaShape<Cfg::MI>;
+	if constexpr (SPLIT)
+	{
+		const int left = K - (int)blockIdx.y * k_split;
+		K = left < k_split ? left : k_split;
+	}
 	// blockIdx.y walks a batch of independent products that share the shape
 	A += (int64_t)blockIdx.y * stride_a;
 	B += (int64_t)blockIdx.y * stride_b;
@@ -476,15 +510,20 @@ __global__ __launch_bounds__(Cfg::kThreads) void gemm_f16_nt_tile_kernel(
 	// no direct load may still be writing LDS when the scratch is reused or the block retires
 	wait_vmem_all();
 	__syncthreads();
-	store_patch_via_lds<Cfg, RAGGED>(acc, lds, C, ldc, m0 + wm * Cfg::kWaveM, n0 + wn * Cfg::kWaveN, wave, lane, M, N);
+	if constexpr (SPLIT)
+		store_patch_f32<Cfg>(acc, planes + (int64_t)blockIdx.y * M * N, m0 + wm * Cfg::kWaveM, n0 + wn * Cfg::kWaveN, lane, M, N);
+	else
+		store_patch_via_lds<Cfg, RAGGED>(acc, lds, C, ldc, m0 + wm * Cfg::kWaveM, n0 + wn * Cfg::kWaveN, wave, lane, M, N);
 }
 
-template <typename Cfg, bool RAGGED = false, bool KTAIL = false>
+// planes != NULL (SPLIT): `batch` is the number of K ranges, k_split their depth.
+template <typename Cfg, bool RAGGED = false, bool KTAIL = false, bool SPLIT = false>
 hipError_t launch_gemm_f16_tile(const half_t* A, const half_t* B, half_t* C, int64_t M, int64_t N, int64_t K,
                                 int64_t lda, int64_t ldb, int64_t ldc,
-                                int64_t stride_a, int64_t stride_b, int64_t stride_c, int64_t batch, hipStream_t stream)
+                                int64_t stride_a, int64_t stride_b, int64_t stride_c, int64_t batch, hipStream_t stream,
+                                float* planes = nullptr, int64_t k_split = 0)
 {
-	auto kernel = gemm_f16_nt_tile_kernel<Cfg, RAGGED, KTAIL>;
+	auto kernel = gemm_f16_nt_tile_kernel<Cfg, RAGGED, KTAIL, SPLIT>;
 	// More than 64 KB of dynamic LDS has to be granted per function and per device, once.
 	static std::atomic<uint64_t> configured_devices{0};
 	(void)hipGetLastError();
@@ -501,7 +540,7 @@ hipError_t launch_gemm_f16_tile(const half_t* A, const half_t* B, half_t* C, int
 	}
 	const int tiles_m = (int)((M + Cfg::BM - 1) / Cfg::BM), tiles_n = (int)((N + Cfg::BN - 1) / Cfg::BN);
 	kernel<<<dim3((unsigned)(tiles_m * tiles_n), (unsigned)batch), dim3(Cfg::kThreads), Cfg::kLdsBytes, stream>>>(
-		A, B, C, (int)K, lda, ldb, ldc, tiles_m, tiles_n, stride_a, stride_b, stride_c, M, N);
+		A, B, C, (int)K, lda, ldb, ldc, tiles_m, tiles_n, stride_a, stride_b, stride_c, M, N, planes, (int)k_split);
 	return hipGetLastError();
 }
 

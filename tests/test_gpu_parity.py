@@ -584,6 +584,27 @@ def test_mm_f16_ragged_shapes_through_tile_kernels(ops, oracle, layout, m, k, n)
     assert np.all(got[m:, :] == -7.0) and np.all(got[:, n:] == -7.0)
 
 
+@pytest.mark.parametrize("layout", ["row", "col"])
+@pytest.mark.parametrize("m,k,n", [(128, 9216, 2304), (100, 1032, 72), (256, 4104, 520), (65, 2304, 2048), (300, 1024, 64),
+                                   (512, 8200, 256)])
+def test_mm_f16_few_tiles_split_along_k(ops, oracle, layout, m, k, n):
+    # fewer blocks than CUs and a deep K: ranges of K write fp32 planes that a merge kernel adds and rounds once
+    from anygpu_amd import capi
+    a = synth.uniform(m + k, (m, k)).astype(np.float16)
+    b = synth.uniform(k + n, (k, n)).astype(np.float16)
+    want = oracle.tensor_mm(oracle.cvt_f16_to_f32(a), oracle.cvt_f16_to_f32(b), threads=8)
+    da = dev(a)
+    db = dev(b) if layout == "row" else dev(np.ascontiguousarray(b.T))
+    lay = capi.B_ROW_MAJOR if layout == "row" else capi.B_COL_MAJOR
+    got = host(ops.tensor_mm(da, db, b_layout=lay))
+    assert scaled_rel_err(got.astype(np.float32), want, math.sqrt(k) / 3.0) <= TOL_F16_GEMM
+    assert np.array_equal(got, host(ops.tensor_mm(da, db, b_layout=lay)))
+    ai, bi = synth.integers(1, (m, k), -2, 2).astype(np.float16), synth.integers(2, (k, n), -2, 2).astype(np.float16)
+    dbi = dev(bi) if layout == "row" else dev(np.ascontiguousarray(bi.T))
+    want_i = oracle.tensor_mm(ai.astype(np.float32), bi.astype(np.float32), threads=8)
+    assert np.array_equal(host(ops.tensor_mm(dev(ai), dbi, b_layout=lay)).astype(np.float32), want_i.astype(np.float16).astype(np.float32))
+
+
 def test_mm_f16_ragged_integer_inputs_bit_exact_and_batched(ops, oracle):
     from anygpu_amd import capi
     a = synth.integers(1, (200, 128), -4, 4).astype(np.float16)
