@@ -1,0 +1,425 @@
+// Fused scaled-dot-product attention, forward, float32 throughout, for gfx950:
+//     y = softmax(mask(softcap(alpha * q k^T))) v        per (batch, head)
+// in one kernel, with the true fp32 matrix instruction v_mfma_f32_16x16x4_f32.  The score matrix never
+// reaches HBM (8 heads x 8192 x 8192 keys: 2 GiB of fp32 scores written and read twice by the three-launch form).
+//
+// The structure is the one of the half precision kernel: a wave owns 16 queries, the query of a lane is
+// lane % 16 in every product, so row maxima and sums are in-lane loops plus two cross-lane steps, and the
+// rescale of the running output is an in-lane multiply.  Per tile of 32 keys:
+//   * S^T = K Q^T: first operand K, second operand Q (in registers for the whole kernel).  The summation index
+//     of an MFMA is a dummy index: lane group g takes head-dimension elements 16 s + 4 g + e in step (s, e), so
+//     that a lane reads its four K values of four consecutive MFMAs with one 16-byte LDS load and holds its Q
+//     values as the matching vectors.  A lane ends up with the scores of keys 16 kb + 4 g + r of its query.
+//   * scale / softcap / mask, online max / sum in the log2 domain, p = exp2(z - m), all fp32;
+//   * O^T += V^T P^T: second operand the p values exactly as they sit in the lane (key slot (kb, r) of lane
+//     group g <-> key 16 kb + 4 g + r), first operand V^T: lane (i, g) loads the four columns 64 c + 4 i .. + 3
+//     of that key's V row with one 16-byte LDS load, and element e of the vector feeds its own MFMA and
+//     accumulator, which therefore holds head-dimension elements 64 c + 4 i' + e: permuted between lanes and
+//     accumulators, and un-permuted for free at the store, where the four accumulators of a lane hold four
+//     consecutive elements.
+// At 32 cycles per MFMA the matrix pipe is the bound by a wide margin (the softmax arithmetic of a tile is
+// about 2 % of its MFMA time); the K and V tiles of the next step are in flight meanwhile.
+//
+// Masks are index rules (causal with the diagonal at n_k - n_q, sliding window); tiles without a visible key
+// are skipped.  A query without any visible key gets zeros.
+#include "device_utils.hpp"
+#include "launch.hpp"
+
+#include <atomic>
+
+namespace anygpu {
+
+namespace {
+
+
+struct AttnArgsF32
+{
+	const float* q;
+	const float* k;
+	const float* v;
+	float* y;
+	int n_q, n_k;
+	int q_per_kv;          // query heads that share one k / v head
+	int diag;              // key j is causally visible to query i iff j <= i + diag
+	int causal;
+	int window;            // 0: off; else key j is visible iff j > i + diag - window
+	float k_in, k_cap;     // logit transform constants (see logit2)
+};
+
+// log2(e) * softcap(alpha * s); without softcap k_in = alpha log2(e); with it
+// cap log2(e) tanh(alpha s / cap) = k_cap - 2 k_cap / (1 + exp2(s k_in)), k_in = 2 log2(e) alpha / cap
+template <bool SOFTCAP>
+__device__ __forceinline__ float logit2(float s, float k_in, float k_cap)
+{
+	if constexpr (SOFTCAP)
+	{
+		const float t = fast_exp2(s * k_in);
+		return fmaf(fast_rcp(1.0f + t), -2.0f * k_cap, k_cap);
+	}
+	return s * k_in;
+}
+
+template <int D, int KT>
+struct AttnLdsF32
+{
+	static constexpr int kPitch = D + 4;                      // floats per tile row: 16 bytes of padding
+	static constexpr int kStageFloats = 2 * KT * kPitch;      // a K tile and a V tile of KT keys
+};
+
+// Scheduling-group masks of __builtin_amdgcn_sched_group_barrier
+constexpr int kSchedMfma = 0x008;
+constexpr int kSchedDsRead = 0x100;
+
+// vmcnt(0) with the other counters left alone (gfx9 encoding: vmcnt in [3:0] and [15:14], expcnt [6:4], lgkmcnt [11:8])
+__device__ __forceinline__ void wait_vmem_all()
+{
+	__builtin_amdgcn_s_waitcnt(0x0F70);
+}
+
+// WAVES waves per block, 16 queries per wave, tiles of KT keys.
+// DIRECT (head dimension 256, where a tile row is exactly the 1024 bytes one wave-wide load instruction moves): the
+// tiles go from memory straight into LDS, into one of two stages, so no staging registers are held and a block of
+// 8 waves (two per SIMD: one multiplies while the other does its softmax arithmetic) fits the register file.
+// Otherwise the tiles pass through registers into a single stage.
+template <int D, bool SOFTCAP, int WAVES, int KT, bool DIRECT>
+__global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f32_kernel(const AttnArgsF32 a)
+{
+	constexpr int kKeysPerTile = KT;
+	static_assert(!DIRECT || D == 256, "one load instruction per tile row");
+	constexpr int kQueriesPerBlock = 16 * WAVES;
+	constexpr int THREADS = 64 * WAVES;
+	extern __shared__ __align__(16) char lds_raw[];
+	using L = AttnLdsF32<D, KT>;
+	float* const lds_base = reinterpret_cast<float*>(lds_raw);
+	typedef __attribute__((address_space(3))) void lds_void;
+	typedef const __attribute__((address_space(1))) void global_void;
+	constexpr int KS = D / 16;                      // 16-element groups of the head dimension (q k^T: 4 MFMAs each)
+	constexpr int DC = D / 64;                      // 64-wide column groups of the output (4 accumulators each)
+	constexpr int KB = kKeysPerTile / 16;           // 16-key blocks per tile
+	constexpr int VPR = D / 4;                      // 16-byte vectors per row
+	constexpr int VPT = kKeysPerTile * VPR / THREADS;   // vectors per thread per tile and matrix
+	static_assert(kKeysPerTile * VPR % THREADS == 0, "the tile divides over the threads");
+
+	const int tid = threadIdx.x;
+	const int lane = tid & (kWaveSize - 1);
+	const int wave = tid >> 6;
+	const int n = lane & 15;                        // query inside the wave's block (second MFMA operand index)
+	const int g = lane >> 4;                        // lane group: summation slot g of an MFMA
+	const int bh = blockIdx.y;
+	// under the causal rule the last query blocks have the most keys to walk: they are dispatched first
+	const int q0 = (int)(gridDim.x - 1 - blockIdx.x) * kQueriesPerBlock;
+	const float* qp = a.q + (int64_t)bh * a.n_q * D;
+	const float* kp = a.k + (int64_t)(bh / a.q_per_kv) * a.n_k * D;
+	const float* vp = a.v + (int64_t)(bh / a.q_per_kv) * a.n_k * D;
+	float* yp = a.y + (int64_t)bh * a.n_q * D;
+
+	// visible key range of the whole block: from the first key of its first query to the last of its last
+	const int q_last = (q0 + kQueriesPerBlock - 1 < a.n_q ? q0 + kQueriesPerBlock - 1 : a.n_q - 1);
+	int key_hi = a.n_k - 1;
+	if (a.causal && q_last + a.diag < key_hi) key_hi = q_last + a.diag;
+	int key_lo = 0;
+	if (a.window > 0 && q0 + a.diag - a.window + 1 > 0) key_lo = q0 + a.diag - a.window + 1;
+	const int t_first = key_lo / kKeysPerTile;
+	const int t_last = key_hi >= 0 ? key_hi / kKeysPerTile : -1;
+
+	// this lane's query as second operand: q[row][16 s + 4 g .. + 3]
+	const int q_row = q0 + 16 * wave + n;
+	float4_t qf[KS];
+#pragma unroll
+	for (int s = 0; s < KS; ++s)
+	{
+		float4_t val = {0.0f, 0.0f, 0.0f, 0.0f};
+		if (q_row < a.n_q) val = *reinterpret_cast<const float4_t*>(qp + (int64_t)q_row * D + 16 * s + 4 * g);
+		qf[s] = val;
+	}
+	int vis_hi = a.causal ? q_row + a.diag : a.n_k - 1;
+	if (vis_hi > a.n_k - 1) vis_hi = a.n_k - 1;
+	const int vis_lo = a.window > 0 ? q_row + a.diag - a.window + 1 : 0;
+
+	float m_run = -INFINITY, l_run = 0.0f;         // l_run: this lane's share of the row sum
+	float4_t o[DC][4];
+#pragma unroll
+	for (int c = 0; c < DC; ++c)
+#pragma unroll
+		for (int e = 0; e < 4; ++e) o[c][e] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+	// keys visible to every query of this wave need no per-element test: [all_lo, all_hi]
+	const int wq0 = q0 + 16 * wave, wq1 = wq0 + 15;
+	const int all_hi = a.causal ? (wq0 + a.diag < a.n_k - 1 ? wq0 + a.diag : a.n_k - 1) : a.n_k - 1;
+	const int all_lo = a.window > 0 ? wq1 + a.diag - a.window + 1 : 0;
+
+	// DIRECT: wave w moves rows w, w + WAVES, ... of the K tile and of the V tile; rows past the last key are
+	// replaced by the last one (their scores are masked, their p is 0)
+	auto tile_direct = [&](int t, int stage) {
+		float* k_dst = lds_base + stage * L::kStageFloats;
+		float* v_dst = k_dst + kKeysPerTile * L::kPitch;
+		const int w = __builtin_amdgcn_readfirstlane(wave);
+#pragma unroll
+		for (int i = 0; i < kKeysPerTile / WAVES; ++i)
+		{
+			const int row = w + WAVES * i;
+			int key = t * kKeysPerTile + row;
+			key = key < a.n_k ? key : a.n_k - 1;
+			__builtin_amdgcn_global_load_lds((global_void*)(kp + (int64_t)key * D + 4 * lane), (lds_void*)(k_dst + row * L::kPitch), 16, 0, 0);
+			__builtin_amdgcn_global_load_lds((global_void*)(vp + (int64_t)key * D + 4 * lane), (lds_void*)(v_dst + row * L::kPitch), 16, 0, 0);
+		}
+	};
+
+	float4_t kr[DIRECT ? 1 : VPT], vr[DIRECT ? 1 : VPT];
+	auto tile_load = [&](int t) {
+#pragma unroll
+		for (int i = 0; i < (DIRECT ? 0 : VPT); ++i)
+		{
+			const int idx = tid + THREADS * i;
+			const int row = idx / VPR, col = idx % VPR;
+			const int key = t * kKeysPerTile + row;
+			float4_t kv = {0.0f, 0.0f, 0.0f, 0.0f}, vv = {0.0f, 0.0f, 0.0f, 0.0f};
+			if (key < a.n_k)
+			{
+				kv = *reinterpret_cast<const float4_t*>(kp + (int64_t)key * D + col * 4);
+				vv = *reinterpret_cast<const float4_t*>(vp + (int64_t)key * D + col * 4);
+			}
+			kr[i] = kv;
+			vr[i] = vv;
+		}
+	};
+	auto tile_store = [&]() {
+		float* k_dst = lds_base;
+		float* v_dst = k_dst + kKeysPerTile * L::kPitch;
+#pragma unroll
+		for (int i = 0; i < (DIRECT ? 0 : VPT); ++i)
+		{
+			const int idx = tid + THREADS * i;
+			const int row = idx / VPR, col = idx % VPR;
+			*reinterpret_cast<float4_t*>(k_dst + row * L::kPitch + col * 4) = kr[i];
+			*reinterpret_cast<float4_t*>(v_dst + row * L::kPitch + col * 4) = vr[i];
+		}
+	};
+
+	if (t_first <= t_last)
+	{
+		if constexpr (DIRECT) tile_direct(t_first, 0);
+		else tile_load(t_first);
+	}
+	for (int t = t_first; t <= t_last; ++t)
+	{
+		const float* k_lds = lds_base;
+		if constexpr (DIRECT)
+		{
+			// own loads of tile t have landed; behind the barrier everybody's have, and everybody is done with the
+			// stage of tile t - 1, which the loads of tile t + 1 overwrite
+			wait_vmem_all();
+			__syncthreads();
+			if (t < t_last) tile_direct(t + 1, (t - t_first + 1) & 1);
+			k_lds = lds_base + ((t - t_first) & 1) * L::kStageFloats;
+		}
+		else
+		{
+			__syncthreads();                       // the previous tile has been read by everybody
+			tile_store();
+			__syncthreads();
+			if (t < t_last) tile_load(t + 1);      // in flight while this tile is used
+		}
+		const float* v_lds = k_lds + kKeysPerTile * L::kPitch;
+
+		// ---- S^T = K Q^T: s[kb][r] = score of key 16 kb + 4 g + r against this lane's query ----
+		// The K vectors of step st + 1 are read from LDS before the MFMAs of step st are issued (the scheduling
+		// groups pin that order: left alone the compiler puts every read right in front of its first use and the
+		// matrix pipe drains while the wave waits for LDS).
+		float4_t s[KB];
+#pragma unroll
+		for (int kb = 0; kb < KB; ++kb) s[kb] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+		float4_t kf[2][KB];
+		auto read_k = [&](float4_t (&dst)[KB], int st) {
+#pragma unroll
+			for (int kb = 0; kb < KB; ++kb)
+				dst[kb] = *reinterpret_cast<const float4_t*>(k_lds + (16 * kb + n) * L::kPitch + 16 * st + 4 * g);
+		};
+		read_k(kf[0], 0);
+		__builtin_amdgcn_sched_group_barrier(kSchedDsRead, KB, 0);
+#pragma unroll
+		for (int st = 0; st < KS; ++st)
+		{
+			if (st + 1 < KS) read_k(kf[(st + 1) & 1], st + 1);
+#pragma unroll
+			for (int e = 0; e < 4; ++e)
+#pragma unroll
+				for (int kb = 0; kb < KB; ++kb)
+					s[kb] = __builtin_amdgcn_mfma_f32_16x16x4f32(kf[st & 1][kb][e], qf[st][e], s[kb], 0, 0, 0);
+			// the reads go out behind the step's first MFMA: the wait in front of that MFMA then covers exactly the
+			// vectors it needs, not the ones just requested
+			__builtin_amdgcn_sched_group_barrier(kSchedMfma, 1, 0);
+			if (st + 1 < KS) __builtin_amdgcn_sched_group_barrier(kSchedDsRead, KB, 0);
+			__builtin_amdgcn_sched_group_barrier(kSchedMfma, 4 * KB - 1, 0);
+		}
+
+		// ---- online softmax ----
+		const int tile_key0 = t * kKeysPerTile;
+		const bool interior = tile_key0 >= all_lo && tile_key0 + kKeysPerTile - 1 <= all_hi;   // wave-uniform
+		float z[KB][4];
+		float mt = -INFINITY;
+		if (interior)
+		{
+#pragma unroll
+			for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+				for (int r = 0; r < 4; ++r)
+				{
+					z[kb][r] = logit2<SOFTCAP>(s[kb][r], a.k_in, a.k_cap);
+					mt = fmaxf(mt, z[kb][r]);
+				}
+		}
+		else
+		{
+#pragma unroll
+			for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+				for (int r = 0; r < 4; ++r)
+				{
+					const int key = tile_key0 + 16 * kb + 4 * g + r;
+					const float zz = logit2<SOFTCAP>(s[kb][r], a.k_in, a.k_cap);
+					z[kb][r] = (key >= vis_lo && key <= vis_hi) ? zz : -INFINITY;
+					mt = fmaxf(mt, z[kb][r]);
+				}
+		}
+		mt = fmaxf(mt, __shfl_xor(mt, 16));
+		mt = fmaxf(mt, __shfl_xor(mt, 32));
+		const float m_new = fmaxf(m_run, mt);
+		const float m_safe = (m_new == -INFINITY) ? 0.0f : m_new;   // nothing visible so far: every term is exp2(-inf) = 0
+		float psum = 0.0f;
+		float p[KB][4];
+#pragma unroll
+		for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+			for (int r = 0; r < 4; ++r)
+			{
+				p[kb][r] = fast_exp2(z[kb][r] - m_safe);
+				psum += p[kb][r];
+			}
+		// the running maximum settles after a few tiles; when no query of the wave raised it, the rescale
+		// factor is 1 everywhere and the pass over the accumulators is skipped
+		if (__builtin_amdgcn_ballot_w64(m_new > m_run) != 0)
+		{
+			const float corr = fast_exp2(m_run - m_safe);
+			l_run *= corr;
+#pragma unroll
+			for (int c = 0; c < DC; ++c)
+#pragma unroll
+				for (int e = 0; e < 4; ++e) o[c][e] *= corr;
+		}
+		l_run += psum;
+		m_run = m_new;
+
+		// ---- O^T += V^T P^T, the V vectors of key slot i + 1 read before the MFMAs of slot i ----
+		float4_t vf[2][DC];
+		auto read_v = [&](float4_t (&dst)[DC], int slot) {
+			const int kb = slot >> 2, r = slot & 3;
+#pragma unroll
+			for (int c = 0; c < DC; ++c)
+				dst[c] = *reinterpret_cast<const float4_t*>(v_lds + (16 * kb + 4 * g + r) * L::kPitch + 64 * c + 4 * n);
+		};
+		read_v(vf[0], 0);
+		__builtin_amdgcn_sched_group_barrier(kSchedDsRead, DC, 0);
+#pragma unroll
+		for (int slot = 0; slot < 4 * KB; ++slot)
+		{
+			if (slot + 1 < 4 * KB) read_v(vf[(slot + 1) & 1], slot + 1);
+#pragma unroll
+			for (int c = 0; c < DC; ++c)
+#pragma unroll
+				for (int e = 0; e < 4; ++e)
+					o[c][e] = __builtin_amdgcn_mfma_f32_16x16x4f32(vf[slot & 1][c][e], p[slot >> 2][slot & 3], o[c][e], 0, 0, 0);
+			__builtin_amdgcn_sched_group_barrier(kSchedMfma, 1, 0);
+			if (slot + 1 < 4 * KB) __builtin_amdgcn_sched_group_barrier(kSchedDsRead, DC, 0);
+			__builtin_amdgcn_sched_group_barrier(kSchedMfma, 4 * DC - 1, 0);
+		}
+	}
+
+	// ---- normalise and store: register r of accumulator (c, e) is y[row][64 c + 4 (4 g + r) + e] ----
+	float l = l_run;
+	l += __shfl_xor(l, 16);
+	l += __shfl_xor(l, 32);
+	const float inv = l > 0.0f ? 1.0f / l : 0.0f;
+	if (q_row < a.n_q)
+	{
+#pragma unroll
+		for (int c = 0; c < DC; ++c)
+#pragma unroll
+			for (int r = 0; r < 4; ++r)
+			{
+				const float4_t out = {o[c][0][r] * inv, o[c][1][r] * inv, o[c][2][r] * inv, o[c][3][r] * inv};
+				*reinterpret_cast<float4_t*>(yp + (int64_t)q_row * D + 64 * c + 16 * g + 4 * r) = out;
+			}
+	}
+}
+
+template <int D, bool SOFTCAP>
+hipError_t launch_variant_f32(const AttnArgsF32& args, int64_t batch_heads, hipStream_t stream)
+{
+	// head dimension 256: 8 waves (two per SIMD) on tiles of 32 keys in two stages, 130 KB, one block per CU.  Two
+	// alternatives with two blocks of 4 waves per CU, for a better balance of long and short blocks under the causal
+	// rule, measured 5 - 12 % slower: tiles of 16 keys, and one K and one V buffer refilled in turn.
+	constexpr bool DIRECT = (D == 256);
+	constexpr int WAVES = DIRECT ? 8 : 4;
+	constexpr int KT = 32;
+	auto kernel = sdp_attention_fwd_f32_kernel<D, SOFTCAP, WAVES, KT, DIRECT>;
+	constexpr int kLdsBytes = AttnLdsF32<D, KT>::kStageFloats * 4 * (DIRECT ? 2 : 1);
+	constexpr int kQueriesPerBlock = 16 * WAVES;
+	(void)hipGetLastError();
+	if (kLdsBytes > 64 * 1024)
+	{
+		// more than 64 KB of dynamic LDS has to be granted per function and per device, once
+		static std::atomic<uint64_t> configured_devices{0};
+		int device = 0;
+		hipError_t e = hipGetDevice(&device);
+		if (e != hipSuccess) return e;
+		const uint64_t bit = 1ull << (device & 63);
+		if ((configured_devices.load(std::memory_order_relaxed) & bit) == 0)
+		{
+			e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+			if (e != hipSuccess) return e;
+			configured_devices.fetch_or(bit, std::memory_order_relaxed);
+		}
+	}
+	const dim3 grid((unsigned)((args.n_q + kQueriesPerBlock - 1) / kQueriesPerBlock), (unsigned)batch_heads);
+	kernel<<<grid, dim3(64 * WAVES), kLdsBytes, stream>>>(args);
+	return hipGetLastError();
+}
+
+}  // namespace
+
+bool sdp_attention_fwd_f32_supports(int64_t head_dim)
+{
+	return head_dim == 64 || head_dim == 128 || head_dim == 256;
+}
+
+hipError_t launch_sdp_attention_fwd_f32(const float* q, const float* k, const float* v, float* y,
+                                        int64_t batch_heads, int64_t q_per_kv, int64_t n_q, int64_t n_k, int64_t head_dim,
+                                        float alpha, float softcap, int causal, int64_t window, hipStream_t stream)
+{
+	if (batch_heads == 0 || n_q == 0) return hipSuccess;
+	AttnArgsF32 args;
+	args.q = q;
+	args.k = k;
+	args.v = v;
+	args.y = y;
+	args.n_q = (int)n_q;
+	args.n_k = (int)n_k;
+	args.q_per_kv = (int)q_per_kv;
+	args.diag = (int)(n_k - n_q);
+	args.causal = causal ? 1 : 0;
+	args.window = (int)window;
+	const bool capped = softcap != 0.0f;
+	args.k_in = capped ? 2.0f * kLog2e * alpha / softcap : alpha * kLog2e;
+	args.k_cap = capped ? softcap * kLog2e : 0.0f;
+#define ANYGPU_ATTN_F32_DIM(DIM) \
+	return capped ? launch_variant_f32<DIM, true>(args, batch_heads, stream) : launch_variant_f32<DIM, false>(args, batch_heads, stream)
+	switch (head_dim)
+	{
+	case 64: ANYGPU_ATTN_F32_DIM(64);
+	case 128: ANYGPU_ATTN_F32_DIM(128);
+	default: ANYGPU_ATTN_F32_DIM(256);
+	}
+#undef ANYGPU_ATTN_F32_DIM
+}
+
+}  // namespace anygpu

@@ -289,6 +289,17 @@ ANYGPU_EXPORT int anygpu_sdp_attention_fwd_f16(const void* q, const void* k, con
 	                                                 causal, window, as_stream(stream));
 }
 
+ANYGPU_EXPORT int anygpu_sdp_attention_fwd_f32(const float* q, const float* k, const float* v, float* y,
+                                               int64_t batch_heads, int64_t q_per_kv, int64_t n_q, int64_t n_k, int64_t head_dim,
+                                               float alpha, float softcap, int causal, int64_t window, void* stream)
+{
+	const int rc = check_attention(q, k, v, y, batch_heads, q_per_kv, n_q, n_k, head_dim, alpha, softcap, window);
+	if (rc != ANYGPU_OK) return rc;
+	if (batch_heads == 0 || n_q == 0) return ANYGPU_OK;
+	return (int)anygpu::launch_sdp_attention_fwd_f32(q, k, v, y, batch_heads, q_per_kv, n_q, n_k, head_dim, alpha, softcap,
+	                                                 causal, window, as_stream(stream));
+}
+
 ANYGPU_EXPORT int64_t anygpu_sdp_attention_decode_workspace_bytes(int64_t batch_heads, int64_t q_per_kv, int64_t n_q, int64_t n_k,
                                                                   int64_t head_dim, int causal, int64_t window)
 {

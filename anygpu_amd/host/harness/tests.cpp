@@ -565,6 +565,35 @@ TEST_CASE(test_sdp_attention_rules_fused_f16, GPU)
 	return ok && compare_data_buffers_l2(got16, want16, 4e-3f);
 }
 
+TEST_CASE(test_sdp_attention_rules_fused_f32, GPU)
+{
+	// the same block in float32: the fp32 fused kernel against the operator chain on the host, and the reference's
+	// flash entry (one matrix, d = 256, no mask) under its own name
+	const int64 h = 4, hkv = 2, n_q = 200, n_k = 260, d = 256;
+	auto hq = crt_random_normal_tensor<float32, CPU>({ 1, h, n_q, d }, 1);
+	auto hk = crt_random_normal_tensor<float32, CPU>({ 1, hkv, n_k, d }, 2);
+	auto hv = crt_random_normal_tensor<float32, CPU>({ 1, hkv, n_k, d }, 3);
+	SoftmaxPrologue rules;
+	rules.alpha = 0.0625f;
+	rules.causal = true;
+	rules.window = 96;
+	auto got = sdp_attention_rules_fwd(hq.copy_to_cuda(), hk.copy_to_cuda(), hv.copy_to_cuda(), rules).copy_to_host();
+	Tensor<float32, CPU> hk_rep(std::vector<int64>({ 1, h, n_k, d })), hv_rep(std::vector<int64>({ 1, h, n_k, d }));
+	for (int64 head = 0; head < h; ++head)
+	{
+		std::memcpy(hk_rep.buffer() + head * n_k * d, hk.buffer() + (head / 2) * n_k * d, n_k * d * sizeof(float32));
+		std::memcpy(hv_rep.buffer() + head * n_k * d, hv.buffer() + (head / 2) * n_k * d, n_k * d * sizeof(float32));
+	}
+	auto want = sdp_attention_rules_fwd(hq, hk_rep, hv_rep, rules);
+	bool ok = elementwise_compatible(got, want) && compare_data_buffers(got, want);
+	auto q2 = crt_random_normal_tensor<float32, CPU>({ 132, 256 }, 4);
+	auto k2 = crt_random_normal_tensor<float32, CPU>({ 132, 256 }, 5);
+	auto v2 = crt_random_normal_tensor<float32, CPU>({ 132, 256 }, 6);
+	auto want2 = single_head_attention_fwd(q2, k2, v2);
+	auto got2 = sdp_attention_fwd_cuda_flash(q2.copy_to_cuda(), k2.copy_to_cuda(), v2.copy_to_cuda()).copy_to_host();
+	return ok && elementwise_compatible(got2, want2) && compare_data_buffers(got2, want2);
+}
+
 TEST_CASE(test_sdp_attention_rules_decode_step_f16, GPU)
 {
 	// generation step over a cache of 700 keys: 8 query heads on 4 key / value heads, d = 128, causal + window;

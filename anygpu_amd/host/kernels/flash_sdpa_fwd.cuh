@@ -10,8 +10,7 @@
   qt, yt (..., heads, n_q, d), kt, vt (..., kv_heads, n_k, d) with heads a multiple of kv_heads and
   d 64, 128 or 256.  Of the prologue, alpha, softcap, causal and window are used; the causal diagonal sits
   at n_k - n_q (q_len and diag of the prologue are implied by the shapes).
-  The reference's fused kernel (cu_flash_sdpa_fwd_d256_v1) is float32, one matrix, d = 256, no mask; its
-  float32 interface is served by sdp_attention_fwd_cuda_flash in sdp.hpp.
+  The reference's fused kernel (cu_flash_sdpa_fwd_d256_v1) is float32, one matrix, d = 256, no mask: below.
 */
 void hip_flash_sdpa_fwd_f16(
 	const SoftmaxPrologue& prologue,
@@ -19,6 +18,27 @@ void hip_flash_sdpa_fwd_f16(
 	const Tensor<float16, CUDA>& kt,
 	const Tensor<float16, CUDA>& vt,
 	Tensor<float16, CUDA>& yt);
+
+/*
+  The same in float32 (the fp32 matrix instruction; results agree with the unfused float32 path to fp32 rounding).
+*/
+void hip_flash_sdpa_fwd_f32(
+	const SoftmaxPrologue& prologue,
+	const Tensor<float32, CUDA>& qt,
+	const Tensor<float32, CUDA>& kt,
+	const Tensor<float32, CUDA>& vt,
+	Tensor<float32, CUDA>& yt);
+
+/*
+  The reference's fused kernel by its own name and contract (srcs/kernels/cuda/flash_sdpa_fwd.cuh:6-15): one
+  matrix, hidden dim 256, no mask; any sequence length here.
+*/
+void cu_flash_sdpa_fwd_d256_v1(
+	const float32 alpha,
+	const Tensor<float32, CUDA>& qt,
+	const Tensor<float32, CUDA>& kt,
+	const Tensor<float32, CUDA>& vt,
+	Tensor<float32, CUDA>& yt);
 
 /*
   Decode form for generation steps: (query heads per key / value head) x n_q <= 16.  The key range is split over

@@ -125,9 +125,9 @@ inline Tensor<dtype, device> single_head_attention_fwd(
 }
 
 /*
-  Single-matrix attention through the fused path (reference: sdp_attention_fwd_cuda_flash, sdp.hpp:48-73, float32,
-  d = 256 only).  Half precision runs the one-kernel form; float32 runs q k^T, softmax with the scale folded in and
-  p v, which is what the reference's float32 kernel computes, for any d.
+  Single-matrix attention through the fused kernels (reference: sdp_attention_fwd_cuda_flash, sdp.hpp:48-73, float32,
+  d = 256 only).  Both precisions run the one-kernel form for d = 64, 128 or 256; float32 with another d runs
+  q k^T, softmax with the scale folded in and p v.
 */
 template<FloatingPointType dtype>
 inline Tensor<dtype, CUDA> sdp_attention_fwd_cuda_flash(
@@ -150,15 +150,28 @@ inline Tensor<dtype, CUDA> sdp_attention_fwd_cuda_flash(
 	}
 	else
 	{
-		return single_head_attention_fwd(qw, kw, vw);
+		if (d != 64 && d != 128 && d != 256) return single_head_attention_fwd(qw, kw, vw);
+		Tensor<dtype, CUDA> y(qw.dim, qw.shape);
+		const float32 alpha = static_cast<float32>(calculate_alpha<float32>(static_cast<int>(d)));
+		if (d == 256)
+		{
+			cu_flash_sdpa_fwd_d256_v1(alpha, qw, kw, vw, y);
+		}
+		else
+		{
+			SoftmaxPrologue p;
+			p.alpha = alpha;
+			hip_flash_sdpa_fwd_f32(p, qw, kw, vw, y);
+		}
+		return y;
 	}
 }
 
 /*
   Attention over (..., heads, n, d) tensors with the mask given by rules instead of a tensor: scale, optional
   softcap, causal rule with the diagonal at n_k - n_q, optional sliding window (the fields of SoftmaxPrologue).
-  Half precision GPU tensors take the fused kernel (k and v may have fewer heads than q); host tensors and float32
-  take sdp_attention_masked_scaled_fwd with the mask the rules describe.
+  GPU tensors with d = 64, 128 or 256 take the fused kernels (k and v may have fewer heads than q); host tensors and
+  float32 with another d take sdp_attention_masked_scaled_fwd with the mask the rules describe.
 */
 template<FloatingPointType dtype, Device device>
 inline Tensor<dtype, device> sdp_attention_rules_fwd(
@@ -187,6 +200,23 @@ inline Tensor<dtype, device> sdp_attention_rules_fwd(
 			hip_flash_sdpa_fwd_f16(rules, qw, kw, vw, y);
 		}
 		return y;
+	}
+	else if constexpr (device == CUDA && std::is_same_v<dtype, float32>)
+	{
+		if (d == 64 || d == 128 || d == 256)
+		{
+			ACASSERT(rules.softcap >= 0.f && rules.window >= 0, "softcap and window must not be negative");
+			Tensor<dtype, CUDA> y(qw.dim, qw.shape);
+			hip_flash_sdpa_fwd_f32(rules, qw, kw, vw, y);
+			return y;
+		}
+		ACASSERT(rules.softcap == 0.f, "the softcap needs the fused kernel");
+		auto hmask = crt_rule_mask<float32>(n_q, n_k, rules.causal, rules.window, n_k - n_q);
+		std::vector<int64> mshape(static_cast<size_t>(dim), 1);
+		mshape[dim - 2] = n_q;
+		mshape[dim - 1] = n_k;
+		auto mview = tensor_view(hmask, mshape);
+		return sdp_attention_masked_scaled_fwd(qw, kw, vw, mview.copy_to_cuda(), static_cast<dtype>(rules.alpha));
 	}
 	else
 	{

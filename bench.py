@@ -47,7 +47,7 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--cpu-seconds", type=float, default=12.0,
                     help="target wall time of the CPU-oracle sample (0 disables the CPU baseline)")
-    ap.add_argument("--only", default="", help="comma list of: gemm,gemm32,conv,softmax,attn,norm (default: all)")
+    ap.add_argument("--only", default="", help="comma list of: gemm,gemm32,conv,softmax,attn,attn32,norm (default: all)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain device copy of 256 MiB (read 256 MiB + write 256 MiB) a few times, "
                          "as the known-size reference for scaling FETCH_SIZE / WRITE_SIZE counter readings")
@@ -196,6 +196,29 @@ def bench_attention(torch, ops, steps, warmup):
     }
 
 
+def bench_attention_f32(torch, ops, steps, warmup):
+    # the same block in float32 (the precision the reference runs Gemma2 in): fp32 operands, fp32 MFMA
+    h, hkv, n, d, win = 8, 4, 8192, 256, 4096
+    g = torch.Generator(device="cuda")
+    g.manual_seed(0)
+    q = torch.randn((1, h, n, d), device="cuda", generator=g)
+    k = torch.randn((1, hkv, n, d), device="cuda", generator=g)
+    v = torch.randn((1, hkv, n, d), device="cuda", generator=g)
+    host_s, ev_s = timed_region(torch, lambda: ops.sdp_attention_fwd(q, k, v, 1.0 / 16.0, softcap=50.0, causal=True, window=win),
+                                steps, warmup)
+    pairs = win * (win + 1) // 2 + (n - win) * win
+    flops = 4.0 * d * pairs * h
+    t = ev_s / steps
+    return {
+        "name": "sdp_attention_fwd_f32",
+        "workload": "fused attention fp32 q [1, 8, 8192, 256], k / v [1, 4, 8192, 256], x 1/16, softcap 50, causal + window 4096",
+        "us_per_launch": t * 1e6, "value": flops / t / 1e12, "unit": "TFLOP/s", "dtype": "f32",
+        "roofline": {"bound": "mfma", "achieved": flops / t / 1e12, "peak": PEAK_FP32_TFLOPS, "unit": "TFLOP/s",
+                     "frac": flops / t / 1e12 / PEAK_FP32_TFLOPS, "traffic": None,
+                     "algorithmic_flops": flops, "visible_pairs_per_head": pairs},
+    }
+
+
 def bench_gated_rmsnorm(torch, ops, steps, warmup):
     # Zamba2-7B Mamba2 mixer: batch 4 x 4096 positions, d_inner 8192
     rows, cols, nbuf = 4 * 4096, 8192, 3                    # 3 x 805 MB of x + z + y: past the Infinity Cache
@@ -304,6 +327,8 @@ def main():
 
     if want("attn"):
         kernels.append(bench_attention(torch, ops, max(args.steps // 8, 1), max(args.warmup // 4, 1)))
+    if want("attn32"):
+        kernels.append(bench_attention_f32(torch, ops, max(args.steps // 16, 1), max(args.warmup // 8, 1)))
     if want("norm"):
         kernels.append(bench_gated_rmsnorm(torch, ops, max(args.steps // 4, 1), max(args.warmup // 4, 1)))
 

@@ -183,6 +183,17 @@ int anygpu_sdp_attention_fwd_f16(const void* q, const void* k, const void* v, vo
                                  float alpha, float softcap, int causal, int64_t window, void* stream);
 
 /*
+ * anygpu_sdp_attention_fwd_f16 in float32: operands, scores, sums and output are fp32 and both products run on the
+ * fp32 matrix instruction, so results agree with the unfused float32 path to fp32 rounding.  Same arguments and
+ * rules.  Replaces cu_flash_sdpa_fwd_d256_v1 (srcs/kernels/cuda/flash_sdpa_fwd.cuh:6-15: one head, head_dim 256,
+ * no mask; here any number of heads, head_dim 64 / 128 / 256, the index-rule masks) and, for masks that are
+ * index rules, the per-head loop of sdp_attention_masked_scaled_fwd (srcs/transformers/sdp.hpp:258-271).
+ */
+int anygpu_sdp_attention_fwd_f32(const float* q, const float* k, const float* v, float* y,
+                                 int64_t batch_heads, int64_t q_per_kv, int64_t n_q, int64_t n_k, int64_t head_dim,
+                                 float alpha, float softcap, int causal, int64_t window, void* stream);
+
+/*
  * Decode form of anygpu_sdp_attention_fwd_f16 for generation steps: few queries per head, long key range.  Same
  * arguments, meaning and result; additionally q_per_kv * n_q <= 16 (the queries of the heads that share a key /
  * value head are processed together, so k and v are read once per key / value head) and a workspace: the visible

@@ -1008,6 +1008,46 @@ def test_sdp_attention_fused_kernel(ops, oracle, case):
     assert rel_l2(got[0], want) <= 2e-3
 
 
+@pytest.mark.parametrize("case", ATTN_CASES)
+def test_sdp_attention_fused_kernel_f32(ops, oracle, case):
+    # the float32 form of the same kernel: fp32 operands and the fp32 matrix instruction, fp32 tolerance
+    heads, kv_heads, n_q, n_k, d, alpha, cap, causal, window = case
+    q = synth.normal(1 + n_q, (1, heads, n_q, d))
+    k = synth.normal(2 + n_k, (1, kv_heads, n_k, d))
+    v = synth.normal(3 + d, (1, kv_heads, n_k, d))
+    got = host(ops.sdp_attention_fwd(dev(q), dev(k), dev(v), alpha, softcap=cap, causal=causal, window=window))
+    want = oracle.sdp_attention_rules(q[0], k[0], v[0], alpha=alpha, softcap=cap, causal=causal, window=window,
+                                      q_per_kv=heads // kv_heads, threads=8)
+    assert got.shape == (1, heads, n_q, d) and got.dtype == np.float32
+    blind = ~np.isfinite(want).all(axis=-1)                      # queries without a visible key: zeros
+    assert not got[0][blind].any()
+    assert scaled_rel_err(got[0][~blind], want[~blind], 1.0) <= TOL_F32
+
+
+def test_sdp_attention_fused_kernel_f32_structure(ops, oracle):
+    heads, n, d = 2, 160, 128
+    q, k, v = (synth.normal(s, (heads, n, d)) for s in (1, 2, 3))
+    y = host(ops.sdp_attention_fwd(dev(q), dev(k), dev(v), 0.0884, causal=True))
+    assert np.array_equal(y[:, 0, :], v[:, 0, :])               # first causal row attends to key 0 only
+    k2, v2 = k.copy(), v.copy()
+    k2[:, 100:, :] += 1.0
+    v2[:, 100:, :] -= 2.0
+    y2 = host(ops.sdp_attention_fwd(dev(q), dev(k2), dev(v2), 0.0884, causal=True))
+    assert np.array_equal(y[:, :100, :], y2[:, :100, :])         # causality, bit for bit
+    assert not np.array_equal(y[:, 100:, :], y2[:, 100:, :])
+    ys = host(ops.sdp_attention_fwd(dev(q), dev(k[:, :60]), dev(v[:, :60]), 0.0884, causal=True))
+    assert not ys[:, :100, :].any() and ys[:, 100:, :].any()
+    # against the three-launch form with the mask as data
+    mask = oracle.slide_mask(oracle.causal_mask(n, n), 48).reshape(1, n, n)
+    three = host(ops.sdp_attention_masked_scaled_fwd(dev(q), dev(k), dev(v), dev(mask), 0.0884))
+    fused = host(ops.sdp_attention_fwd(dev(q), dev(k), dev(v), 0.0884, causal=True, window=48))
+    assert scaled_rel_err(fused, three, 1.0) <= TOL_F32
+    # integer-valued v and a single visible key per query (window 1): the output is that row of v exactly
+    vi = synth.integers(5, (heads, n, d), -8, 8)
+    yi = host(ops.sdp_attention_fwd(dev(q), dev(k), dev(vi), 0.0884, causal=True, window=1))
+    assert np.array_equal(yi, vi)
+
+
 def test_sdp_attention_fused_kernel_structure(ops, oracle):
     import torch
     # first causal row attends to key 0 only: y[0] = v[0] exactly; a changed future key changes nothing before it
