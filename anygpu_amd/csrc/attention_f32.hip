@@ -360,7 +360,7 @@ hipError_t launch_variant_f32(const AttnArgsF32& args, int64_t batch_heads, hipS
 	// rule, measured 5 - 12 % slower: tiles of 16 keys, and one K and one V buffer refilled in turn.
 	constexpr bool DIRECT = (D == 256);
 	constexpr int WAVES = DIRECT ? 8 : 4;
-	constexpr int KT = 32;
+	constexpr int KT = DIRECT ? 32 : 64;
 	auto kernel = sdp_attention_fwd_f32_kernel<D, SOFTCAP, WAVES, KT, DIRECT>;
 	constexpr int kLdsBytes = AttnLdsF32<D, KT>::kStageFloats * 4 * (DIRECT ? 2 : 1);
 	constexpr int kQueriesPerBlock = 16 * WAVES;
