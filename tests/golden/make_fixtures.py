@@ -126,6 +126,17 @@ def main() -> None:
         save_tensor(t, d / f"{name}.dat")
     save_tensor(y.reshape(1, 4, 24, 64), d / "y.dat")
 
+    # the same rules in float32 at head dimension 256 (the reference's fused kernel is float32, d = 256): 2 query heads
+    # over 1 key / value head, 20 queries at the end of 36 keys, scale 1/16, softcap 50, causal + window 10
+    d = case_dir("test_sdp_rules_f32_d256")
+    q = synth.normal(210, (1, 2, 20, 256))
+    k = synth.normal(211, (1, 1, 36, 256))
+    v = synth.normal(212, (1, 1, 36, 256))
+    y = oracle.sdp_attention_rules(q[0], k[0], v[0], alpha=0.0625, softcap=50.0, causal=True, window=10, q_per_kv=2)
+    for name, t in (("q", q), ("k", k), ("v", v)):
+        save_tensor(t, d / f"{name}.dat")
+    save_tensor(y.reshape(1, 2, 20, 256), d / "y.dat")
+
     print("fixtures written under", HERE)
 
 

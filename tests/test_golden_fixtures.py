@@ -70,6 +70,10 @@ def test_fixtures_match_the_oracle(oracle):
     q, k, v = (oracle.cvt_f16_to_f32(load_tensor(d / f"{n}.dat"))[0] for n in ("q", "k", "v"))
     y = oracle.sdp_attention_rules(q, k, v, alpha=0.125, softcap=20.0, causal=True, window=12, q_per_kv=2)
     assert np.array_equal(y.reshape(1, 4, 24, 64), load_tensor(d / "y.dat"))
+    d = GOLDEN / "test_sdp_rules_f32_d256"
+    q, k, v = (load_tensor(d / f"{n}.dat")[0] for n in ("q", "k", "v"))
+    y = oracle.sdp_attention_rules(q, k, v, alpha=0.0625, softcap=50.0, causal=True, window=10, q_per_kv=2)
+    assert np.array_equal(y.reshape(1, 2, 20, 256), load_tensor(d / "y.dat"))
     for name, kw in [("test_softmax_masked_scaled_f32", dict(alpha=0.125, causal=True, q_len=16)),
                      ("test_softmax_softcap_window_f32", dict(alpha=0.0625, softcap=50.0, causal=True, window=6, q_len=16))]:
         d = GOLDEN / name

@@ -1262,3 +1262,8 @@ def test_golden_fixtures_through_c_abi(ops):
     got = host(ops.sdp_attention_fwd(*(dev(load_tensor(d / f"{n}.dat")) for n in ("q", "k", "v")), 0.125, softcap=20.0,
                                      causal=True, window=12)).astype(np.float32)
     assert scaled_rel_err(got, load_tensor(d / "y.dat"), 1.0) <= TOL_F16_ROWOPS * 2
+
+    d = golden / "test_sdp_rules_f32_d256"
+    got = host(ops.sdp_attention_fwd(*(dev(load_tensor(d / f"{n}.dat")) for n in ("q", "k", "v")), 0.0625, softcap=50.0,
+                                     causal=True, window=10))
+    assert scaled_rel_err(got, load_tensor(d / "y.dat"), 1.0) <= TOL_F32
