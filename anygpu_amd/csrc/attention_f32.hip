@@ -385,6 +385,230 @@ hipError_t launch_variant_f32(const AttnArgsF32& args, int64_t batch_heads, hipS
 	return hipGetLastError();
 }
 
+// ---------------------------------------------------------------------------------------------
+// Decode form: very few queries per head (a generation step), long key range: the KEYS are split.
+//
+// The q_per_kv query heads that share a key / value head, times the n_q queries of each, are the (at most 16)
+// rows of one 16-query MFMA block, so K and V of a head are read once for all of them.  Pass 1: one wave per
+// (key / value head, split of the visible key range) walks its keys in tiles of 16.  Both operands come straight
+// from global memory in MFMA operand layout, no LDS: the K vectors as in the fused kernel, and the V vectors with
+// the permuted accumulators described at the top (a lane loads four consecutive columns of a V row).  The wave
+// leaves its running maximum, sum and unnormalised accumulators in the workspace.  Pass 2 merges the splits of a
+// row: M = max m_i, y = sum o_i 2^(m_i - M) / sum l_i 2^(m_i - M).
+// Workspace per (head, split, row): head_dim accumulators + maximum + sum, fp32.
+// ---------------------------------------------------------------------------------------------
+constexpr int kDecodeKeysPerTile = 16;
+constexpr int kDecodeMaxRows = 16;
+constexpr int kDecodeMaxSplits = 64;
+constexpr int kDecodeTargetWaves = 1024;          // about 4 waves per CU
+
+struct DecodeArgsF32
+{
+	AttnArgsF32 a;
+	float* ws;              // [kv_heads][splits][rows][D + 2]
+	int rows;               // q_per_kv * n_q
+	int splits;
+	int tiles_per_split;
+	int t_first, t_last;    // visible key tiles of the group
+};
+
+template <int D, bool SOFTCAP>
+__global__ __launch_bounds__(64) void sdp_decode_partial_f32_kernel(const DecodeArgsF32 da)
+{
+	const AttnArgsF32& a = da.a;
+	constexpr int KS = D / 16, DC = D / 64;
+	const int lane = threadIdx.x;
+	const int n = lane & 15, g = lane >> 4;
+	const int split = blockIdx.x;
+	const int kvh = blockIdx.y;
+	const float* qp = a.q + (int64_t)kvh * da.rows * D;   // the rows of a group are contiguous: [q_per_kv][n_q][D]
+	const float* kp = a.k + (int64_t)kvh * a.n_k * D;
+	const float* vp = a.v + (int64_t)kvh * a.n_k * D;
+
+	const bool row_ok = n < da.rows;
+	const int q_idx = row_ok ? n % a.n_q : 0;             // position of this lane's row among the n_q queries
+	float4_t qf[KS];
+#pragma unroll
+	for (int s = 0; s < KS; ++s)
+	{
+		float4_t val = {0.0f, 0.0f, 0.0f, 0.0f};
+		if (row_ok) val = *reinterpret_cast<const float4_t*>(qp + (int64_t)n * D + 16 * s + 4 * g);
+		qf[s] = val;
+	}
+	int vis_hi = a.causal ? q_idx + a.diag : a.n_k - 1;
+	if (vis_hi > a.n_k - 1) vis_hi = a.n_k - 1;
+	if (!row_ok) vis_hi = -1;                              // padding rows see nothing
+	const int vis_lo = a.window > 0 ? q_idx + a.diag - a.window + 1 : 0;
+
+	float m_run = -INFINITY, l_run = 0.0f;
+	float4_t o[DC][4];
+#pragma unroll
+	for (int c = 0; c < DC; ++c)
+#pragma unroll
+		for (int e = 0; e < 4; ++e) o[c][e] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+
+	const int t0 = da.t_first + split * da.tiles_per_split;
+	int t1 = t0 + da.tiles_per_split - 1;
+	if (t1 > da.t_last) t1 = da.t_last;
+	for (int t = t0; t <= t1; ++t)
+	{
+		const int key0 = t * kDecodeKeysPerTile;
+		// all loads of the tile are issued before the first use; keys past the end are replaced by the last one
+		// (their scores are masked)
+		float4_t kf[KS], vf[4][DC];
+		{
+			int key = key0 + n;
+			key = key < a.n_k ? key : a.n_k - 1;
+#pragma unroll
+			for (int st = 0; st < KS; ++st)
+				kf[st] = __builtin_nontemporal_load(reinterpret_cast<const float4_t*>(kp + (int64_t)key * D + 16 * st + 4 * g));
+		}
+#pragma unroll
+		for (int r = 0; r < 4; ++r)
+		{
+			int key = key0 + 4 * g + r;
+			key = key < a.n_k ? key : a.n_k - 1;
+#pragma unroll
+			for (int c = 0; c < DC; ++c)
+				vf[r][c] = __builtin_nontemporal_load(reinterpret_cast<const float4_t*>(vp + (int64_t)key * D + 64 * c + 4 * n));
+		}
+
+		float4_t s = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+		for (int st = 0; st < KS; ++st)
+#pragma unroll
+			for (int e = 0; e < 4; ++e) s = __builtin_amdgcn_mfma_f32_16x16x4f32(kf[st][e], qf[st][e], s, 0, 0, 0);
+
+		float z[4];
+		float mt = -INFINITY;
+#pragma unroll
+		for (int r = 0; r < 4; ++r)
+		{
+			const int key = key0 + 4 * g + r;
+			const float zz = logit2<SOFTCAP>(s[r], a.k_in, a.k_cap);
+			z[r] = (key >= vis_lo && key <= vis_hi) ? zz : -INFINITY;
+			mt = fmaxf(mt, z[r]);
+		}
+		mt = fmaxf(mt, __shfl_xor(mt, 16));
+		mt = fmaxf(mt, __shfl_xor(mt, 32));
+		const float m_new = fmaxf(m_run, mt);
+		const float m_safe = (m_new == -INFINITY) ? 0.0f : m_new;
+		const float corr = fast_exp2(m_run - m_safe);
+		float psum = 0.0f;
+		float p[4];
+#pragma unroll
+		for (int r = 0; r < 4; ++r)
+		{
+			p[r] = fast_exp2(z[r] - m_safe);
+			psum += p[r];
+		}
+		l_run = l_run * corr + psum;
+		m_run = m_new;
+#pragma unroll
+		for (int c = 0; c < DC; ++c)
+#pragma unroll
+			for (int e = 0; e < 4; ++e) o[c][e] *= corr;
+#pragma unroll
+		for (int r = 0; r < 4; ++r)
+#pragma unroll
+			for (int c = 0; c < DC; ++c)
+#pragma unroll
+				for (int e = 0; e < 4; ++e) o[c][e] = __builtin_amdgcn_mfma_f32_16x16x4f32(vf[r][c][e], p[r], o[c][e], 0, 0, 0);
+	}
+
+	// partial result of this split: register r of accumulator (c, e) is o[row n][64 c + 16 g + 4 r + e]
+	float l = l_run;
+	l += __shfl_xor(l, 16);
+	l += __shfl_xor(l, 32);
+	if (row_ok)
+	{
+		float* dst = da.ws + (((int64_t)kvh * da.splits + split) * da.rows + n) * (D + 2);
+#pragma unroll
+		for (int c = 0; c < DC; ++c)
+#pragma unroll
+			for (int r = 0; r < 4; ++r)
+				*reinterpret_cast<float4_t*>(dst + 64 * c + 16 * g + 4 * r) = float4_t{o[c][0][r], o[c][1][r], o[c][2][r], o[c][3][r]};
+		if (g == 0)
+		{
+			dst[D] = m_run;
+			dst[D + 1] = l;
+		}
+	}
+}
+
+// One block per (key / value head, row), one thread per output column.  The first threads fetch the maxima and
+// sums of the splits in parallel and leave the weights 2^(m_i - M) in LDS; the column sums then run over
+// independent loads.
+template <int D>
+__global__ __launch_bounds__(D) void sdp_decode_merge_f32_kernel(const float* __restrict__ ws, float* __restrict__ y, int rows, int splits)
+{
+	__shared__ float weight[kDecodeMaxSplits];
+	__shared__ float total;
+	const int row = blockIdx.x, kvh = blockIdx.y, d = threadIdx.x;
+	const float* base = ws + (((int64_t)kvh * splits) * rows + row) * (D + 2);
+	const int64_t step = (int64_t)rows * (D + 2);
+	if (d < kWaveSize)
+	{
+		// splits <= 64: one split per lane of the first wave
+		const float m = d < splits ? base[d * step + D] : -INFINITY;
+		const float l = d < splits ? base[d * step + D + 1] : 0.0f;
+		const float big = wave_allreduce(m, MaxOp());
+		const float w = fast_exp2(m - (big == -INFINITY ? 0.0f : big));
+		const float sum = wave_allreduce(l * w, SumOp());
+		if (d < splits) weight[d] = w;
+		if (d == 0) total = sum;
+	}
+	__syncthreads();
+	float acc = 0.0f;
+#pragma unroll 8
+	for (int i = 0; i < splits; ++i) acc += base[i * step + d] * weight[i];
+	const float sum = total;
+	y[((int64_t)kvh * rows + row) * D + d] = sum > 0.0f ? acc / sum : 0.0f;
+}
+
+struct DecodePlanF32
+{
+	int t_first, t_last, splits, tiles_per_split;
+};
+
+DecodePlanF32 plan_decode_f32(int64_t kv_heads, int64_t n_q, int64_t n_k, int causal, int64_t window)
+{
+	// visible key tiles of a group: its first query decides the low end, its last the high end
+	const int64_t diag = n_k - n_q;
+	int64_t key_hi = n_k - 1;
+	if (causal && (n_q - 1) + diag < key_hi) key_hi = (n_q - 1) + diag;
+	int64_t key_lo = 0;
+	if (window > 0 && diag - window + 1 > 0) key_lo = diag - window + 1;
+	DecodePlanF32 p;
+	p.t_first = (int)(key_lo / kDecodeKeysPerTile);
+	p.t_last = key_hi >= 0 ? (int)(key_hi / kDecodeKeysPerTile) : p.t_first - 1;
+	const int64_t tiles = p.t_last - p.t_first + 1;
+	if (tiles <= 0)
+	{
+		p.splits = 1;
+		p.tiles_per_split = 0;
+		return p;
+	}
+	int64_t want = (kDecodeTargetWaves + kv_heads - 1) / kv_heads;
+	if (want > kDecodeMaxSplits) want = kDecodeMaxSplits;
+	if (want > tiles) want = tiles;
+	if (want < 1) want = 1;
+	p.tiles_per_split = (int)((tiles + want - 1) / want);
+	p.splits = (int)((tiles + p.tiles_per_split - 1) / p.tiles_per_split);
+	return p;
+}
+
+template <int D, bool SOFTCAP>
+hipError_t launch_decode_variant_f32(const DecodeArgsF32& da, int64_t kv_heads, hipStream_t stream)
+{
+	(void)hipGetLastError();
+	sdp_decode_partial_f32_kernel<D, SOFTCAP><<<dim3((unsigned)da.splits, (unsigned)kv_heads), dim3(64), 0, stream>>>(da);
+	hipError_t e = hipGetLastError();
+	if (e != hipSuccess) return e;
+	sdp_decode_merge_f32_kernel<D><<<dim3((unsigned)da.rows, (unsigned)kv_heads), dim3(D), 0, stream>>>(da.ws, da.a.y, da.rows, da.splits);
+	return hipGetLastError();
+}
+
 }  // namespace
 
 bool sdp_attention_fwd_f32_supports(int64_t head_dim)
@@ -420,6 +644,58 @@ hipError_t launch_sdp_attention_fwd_f32(const float* q, const float* k, const fl
 	default: ANYGPU_ATTN_F32_DIM(256);
 	}
 #undef ANYGPU_ATTN_F32_DIM
+}
+
+bool sdp_attention_decode_f32_supports(int64_t q_per_kv, int64_t n_q, int64_t head_dim)
+{
+	return sdp_attention_fwd_f32_supports(head_dim) && q_per_kv >= 1 && n_q >= 1 && q_per_kv * n_q <= kDecodeMaxRows;
+}
+
+int64_t sdp_attention_decode_f32_workspace_bytes(int64_t batch_heads, int64_t q_per_kv, int64_t n_q, int64_t n_k, int64_t head_dim,
+                                                 int causal, int64_t window)
+{
+	if (batch_heads == 0 || n_q == 0) return 0;
+	const int64_t kv_heads = batch_heads / q_per_kv;
+	const DecodePlanF32 p = plan_decode_f32(kv_heads, n_q, n_k, causal, window);
+	return kv_heads * p.splits * (q_per_kv * n_q) * (head_dim + 2) * (int64_t)sizeof(float);
+}
+
+hipError_t launch_sdp_attention_decode_f32(const float* q, const float* k, const float* v, float* y, void* workspace,
+                                           int64_t batch_heads, int64_t q_per_kv, int64_t n_q, int64_t n_k, int64_t head_dim,
+                                           float alpha, float softcap, int causal, int64_t window, hipStream_t stream)
+{
+	if (batch_heads == 0 || n_q == 0) return hipSuccess;
+	const int64_t kv_heads = batch_heads / q_per_kv;
+	const DecodePlanF32 p = plan_decode_f32(kv_heads, n_q, n_k, causal, window);
+	DecodeArgsF32 da;
+	da.a.q = q;
+	da.a.k = k;
+	da.a.v = v;
+	da.a.y = y;
+	da.a.n_q = (int)n_q;
+	da.a.n_k = (int)n_k;
+	da.a.q_per_kv = (int)q_per_kv;
+	da.a.diag = (int)(n_k - n_q);
+	da.a.causal = causal ? 1 : 0;
+	da.a.window = (int)window;
+	const bool capped = softcap != 0.0f;
+	da.a.k_in = capped ? 2.0f * kLog2e * alpha / softcap : alpha * kLog2e;
+	da.a.k_cap = capped ? softcap * kLog2e : 0.0f;
+	da.ws = static_cast<float*>(workspace);
+	da.rows = (int)(q_per_kv * n_q);
+	da.splits = p.splits;
+	da.tiles_per_split = p.tiles_per_split;
+	da.t_first = p.t_first;
+	da.t_last = p.t_last;
+#define ANYGPU_DECODE_F32_DIM(DIM) \
+	return capped ? launch_decode_variant_f32<DIM, true>(da, kv_heads, stream) : launch_decode_variant_f32<DIM, false>(da, kv_heads, stream)
+	switch (head_dim)
+	{
+	case 64: ANYGPU_DECODE_F32_DIM(64);
+	case 128: ANYGPU_DECODE_F32_DIM(128);
+	default: ANYGPU_DECODE_F32_DIM(256);
+	}
+#undef ANYGPU_DECODE_F32_DIM
 }
 
 }  // namespace anygpu

@@ -327,6 +327,33 @@ ANYGPU_EXPORT int anygpu_sdp_attention_decode_f16(const void* q, const void* k, 
 	                                                    softcap, causal, window, as_stream(stream));
 }
 
+ANYGPU_EXPORT int64_t anygpu_sdp_attention_decode_f32_workspace_bytes(int64_t batch_heads, int64_t q_per_kv, int64_t n_q, int64_t n_k,
+                                                                      int64_t head_dim, int causal, int64_t window)
+{
+	const int rc = check_attention_shape(batch_heads, q_per_kv, n_q, n_k, head_dim, window);
+	if (rc != ANYGPU_OK) return rc;
+	if (batch_heads == 0 || n_q == 0) return 0;
+	if (!anygpu::sdp_attention_decode_f32_supports(q_per_kv, n_q, head_dim)) return ANYGPU_ERR_UNSUPPORTED;
+	return anygpu::sdp_attention_decode_f32_workspace_bytes(batch_heads, q_per_kv, n_q, n_k, head_dim, causal, window);
+}
+
+ANYGPU_EXPORT int anygpu_sdp_attention_decode_f32(const float* q, const float* k, const float* v, float* y,
+                                                  void* workspace, int64_t workspace_bytes,
+                                                  int64_t batch_heads, int64_t q_per_kv, int64_t n_q, int64_t n_k, int64_t head_dim,
+                                                  float alpha, float softcap, int causal, int64_t window, void* stream)
+{
+	const int rc = check_attention(q, k, v, y, batch_heads, q_per_kv, n_q, n_k, head_dim, alpha, softcap, window);
+	if (rc != ANYGPU_OK) return rc;
+	if (batch_heads == 0 || n_q == 0) return ANYGPU_OK;
+	if (!anygpu::sdp_attention_decode_f32_supports(q_per_kv, n_q, head_dim)) return ANYGPU_ERR_UNSUPPORTED;
+	const int64_t need = anygpu::sdp_attention_decode_f32_workspace_bytes(batch_heads, q_per_kv, n_q, n_k, head_dim, causal, window);
+	if (workspace == nullptr) return ANYGPU_ERR_NULL_POINTER;
+	if (workspace_bytes < need) return ANYGPU_ERR_BAD_SHAPE;
+	if (reinterpret_cast<uintptr_t>(workspace) % 16 != 0) return ANYGPU_ERR_UNSUPPORTED;
+	return (int)anygpu::launch_sdp_attention_decode_f32(q, k, v, y, workspace, batch_heads, q_per_kv, n_q, n_k, head_dim, alpha,
+	                                                    softcap, causal, window, as_stream(stream));
+}
+
 ANYGPU_EXPORT int anygpu_causal_conv1d_silu_f16(const void* x, const void* w, const void* bias, void* y,
                                                 int64_t batch, int64_t chan, int64_t seqlen, int64_t width,
                                                 void* stream)

@@ -76,6 +76,14 @@ hipError_t launch_sdp_attention_decode_f16(const void* q, const void* k, const v
                                            int64_t batch_heads, int64_t q_per_kv, int64_t n_q, int64_t n_k, int64_t head_dim,
                                            float alpha, float softcap, int causal, int64_t window, hipStream_t stream);
 
+// Decode form in float32: keys in tiles of 16, both operands straight from global memory.
+bool sdp_attention_decode_f32_supports(int64_t q_per_kv, int64_t n_q, int64_t head_dim);
+int64_t sdp_attention_decode_f32_workspace_bytes(int64_t batch_heads, int64_t q_per_kv, int64_t n_q, int64_t n_k, int64_t head_dim,
+                                                 int causal, int64_t window);
+hipError_t launch_sdp_attention_decode_f32(const float* q, const float* k, const float* v, float* y, void* workspace,
+                                           int64_t batch_heads, int64_t q_per_kv, int64_t n_q, int64_t n_k, int64_t head_dim,
+                                           float alpha, float softcap, int causal, int64_t window, hipStream_t stream);
+
 // Few-row products (M <= kSkinnyMaxRows, one product, row-major A): bandwidth-shaped kernels that
 // stream B once.  `epilogue` is an Epilogue value; B2 only for kEpiGeluMul, bias only for kEpiBias
 // (either may be NULL).  T is float or _Float16.  gemm_skinny_applies says whether shape, leading

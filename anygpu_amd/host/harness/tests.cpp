@@ -594,6 +594,29 @@ TEST_CASE(test_sdp_attention_rules_fused_f32, GPU)
 	return ok && elementwise_compatible(got2, want2) && compare_data_buffers(got2, want2);
 }
 
+TEST_CASE(test_sdp_attention_rules_decode_step_f32, GPU)
+{
+	// generation step in float32 over a cache of 700 keys: 8 query heads on 4 key / value heads, d = 256, softcap,
+	// causal + window; the split-key form (picked by the shape) against the operator chain on the host
+	const int64 h = 8, hkv = 4, n_k = 700, d = 256;
+	auto hq = crt_random_normal_tensor<float32, CPU>({ 1, h, 1, d }, 1);
+	auto hk = crt_random_normal_tensor<float32, CPU>({ 1, hkv, n_k, d }, 2);
+	auto hv = crt_random_normal_tensor<float32, CPU>({ 1, hkv, n_k, d }, 3);
+	SoftmaxPrologue rules;
+	rules.alpha = 0.0625f;
+	rules.causal = true;
+	rules.window = 512;
+	auto got = sdp_attention_rules_fwd(hq.copy_to_cuda(), hk.copy_to_cuda(), hv.copy_to_cuda(), rules).copy_to_host();
+	Tensor<float32, CPU> hk_rep(std::vector<int64>({ 1, h, n_k, d })), hv_rep(std::vector<int64>({ 1, h, n_k, d }));
+	for (int64 head = 0; head < h; ++head)
+	{
+		std::memcpy(hk_rep.buffer() + head * n_k * d, hk.buffer() + (head / 2) * n_k * d, n_k * d * sizeof(float32));
+		std::memcpy(hv_rep.buffer() + head * n_k * d, hv.buffer() + (head / 2) * n_k * d, n_k * d * sizeof(float32));
+	}
+	auto want = sdp_attention_rules_fwd(hq, hk_rep, hv_rep, rules);
+	return elementwise_compatible(got, want) && compare_data_buffers(got, want);
+}
+
 TEST_CASE(test_sdp_attention_rules_decode_step_f16, GPU)
 {
 	// generation step over a cache of 700 keys: 8 query heads on 4 key / value heads, d = 128, causal + window;

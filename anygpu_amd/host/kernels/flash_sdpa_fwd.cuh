@@ -62,4 +62,24 @@ void hip_flash_sdpa_decode_f16(
 	Tensor<float32, CUDA>& workspace,
 	Tensor<float16, CUDA>& yt);
 
+/*
+  The decode form in float32 (same roles of the arguments).
+*/
+bool hip_flash_sdpa_decode_applies(
+	const Tensor<float32, CUDA>& qt,
+	const Tensor<float32, CUDA>& kt);
+
+int64 hip_flash_sdpa_decode_workspace_floats(
+	const SoftmaxPrologue& prologue,
+	const Tensor<float32, CUDA>& qt,
+	const Tensor<float32, CUDA>& kt);
+
+void hip_flash_sdpa_decode_f32(
+	const SoftmaxPrologue& prologue,
+	const Tensor<float32, CUDA>& qt,
+	const Tensor<float32, CUDA>& kt,
+	const Tensor<float32, CUDA>& vt,
+	Tensor<float32, CUDA>& workspace,
+	Tensor<float32, CUDA>& yt);
+
 #endif  // __FLASH_SDPA_FWD_CUH__

@@ -375,7 +375,8 @@ struct AttentionShape
 	int64 batch_heads, q_per_kv, n_q, n_k, d;
 };
 
-AttentionShape attention_shape(const Tensor<float16, CUDA>& qt, const Tensor<float16, CUDA>& kt)
+template <typename T>
+AttentionShape attention_shape(const Tensor<T, CUDA>& qt, const Tensor<T, CUDA>& kt)
 {
 	const int64 dim = qt.dim;
 	AttentionShape s;
@@ -412,6 +413,32 @@ void hip_flash_sdpa_decode_f16(const SoftmaxPrologue& prologue, const Tensor<flo
 {
 	const AttentionShape s = attention_shape(qt, kt);
 	ABI_CHECK(anygpu_sdp_attention_decode_f16(qt.buffer(), kt.buffer(), vt.buffer(), yt.buffer(), workspace.buffer(),
+	                                          workspace.numel() * static_cast<int64>(sizeof(float32)), s.batch_heads, s.q_per_kv,
+	                                          s.n_q, s.n_k, s.d, prologue.alpha, prologue.softcap, prologue.causal ? 1 : 0,
+	                                          prologue.window, kNullStream));
+}
+
+bool hip_flash_sdpa_decode_applies(const Tensor<float32, CUDA>& qt, const Tensor<float32, CUDA>& kt)
+{
+	const AttentionShape s = attention_shape(qt, kt);
+	return s.q_per_kv * s.n_q >= 1 && s.q_per_kv * s.n_q <= 16 && s.n_k >= 256;
+}
+
+int64 hip_flash_sdpa_decode_workspace_floats(const SoftmaxPrologue& prologue, const Tensor<float32, CUDA>& qt,
+                                             const Tensor<float32, CUDA>& kt)
+{
+	const AttentionShape s = attention_shape(qt, kt);
+	const int64 bytes = anygpu_sdp_attention_decode_f32_workspace_bytes(s.batch_heads, s.q_per_kv, s.n_q, s.n_k, s.d,
+	                                                                    prologue.causal ? 1 : 0, prologue.window);
+	if (bytes < 0) check_abi(static_cast<int>(bytes), "anygpu_sdp_attention_decode_f32_workspace_bytes", __FILE__, __LINE__);
+	return (bytes + 3) / 4;
+}
+
+void hip_flash_sdpa_decode_f32(const SoftmaxPrologue& prologue, const Tensor<float32, CUDA>& qt, const Tensor<float32, CUDA>& kt,
+                               const Tensor<float32, CUDA>& vt, Tensor<float32, CUDA>& workspace, Tensor<float32, CUDA>& yt)
+{
+	const AttentionShape s = attention_shape(qt, kt);
+	ABI_CHECK(anygpu_sdp_attention_decode_f32(qt.buffer(), kt.buffer(), vt.buffer(), yt.buffer(), workspace.buffer(),
 	                                          workspace.numel() * static_cast<int64>(sizeof(float32)), s.batch_heads, s.q_per_kv,
 	                                          s.n_q, s.n_k, s.d, prologue.alpha, prologue.softcap, prologue.causal ? 1 : 0,
 	                                          prologue.window, kNullStream));

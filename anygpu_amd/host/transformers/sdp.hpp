@@ -207,7 +207,15 @@ inline Tensor<dtype, device> sdp_attention_rules_fwd(
 		{
 			ACASSERT(rules.softcap >= 0.f && rules.window >= 0, "softcap and window must not be negative");
 			Tensor<dtype, CUDA> y(qw.dim, qw.shape);
-			hip_flash_sdpa_fwd_f32(rules, qw, kw, vw, y);
+			if (hip_flash_sdpa_decode_applies(qw, kw))
+			{
+				Tensor<float32, CUDA> workspace(std::vector<int64>{ std::max<int64>(hip_flash_sdpa_decode_workspace_floats(rules, qw, kw), 4) });
+				hip_flash_sdpa_decode_f32(rules, qw, kw, vw, workspace, y);
+			}
+			else
+			{
+				hip_flash_sdpa_fwd_f32(rules, qw, kw, vw, y);
+			}
 			return y;
 		}
 		ACASSERT(rules.softcap == 0.f, "the softcap needs the fused kernel");

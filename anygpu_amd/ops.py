@@ -299,8 +299,7 @@ def sdp_attention_fwd(qw: torch.Tensor, kw: torch.Tensor, vw: torch.Tensor, alph
                       causal: bool = False, window: int = 0, decode: bool | None = None) -> torch.Tensor:
     """softmax(mask(softcap(alpha q k^T))) v in one kernel; q [..., heads, n_q, d], k and v [..., kv_heads, n_k, d]
     with heads a multiple of kv_heads, float16 or float32; masks are index rules with the causal diagonal at
-    n_k - n_q.  decode (float16 only): True / False forces the split-key decode form or the fused form, None picks
-    by shape."""
+    n_k - n_q.  decode: True / False forces the split-key decode form or the fused form, None picks by shape."""
     _check_device(qw, kw, vw)
     _require(qw.dim() == kw.dim() == vw.dim() and qw.dim() >= 3, "dimension missmatch")
     _require(qw.dtype == kw.dtype == vw.dtype and qw.dtype in (torch.float16, torch.float32), "Unsupported data types")
@@ -314,16 +313,24 @@ def sdp_attention_fwd(qw: torch.Tensor, kw: torch.Tensor, vw: torch.Tensor, alph
     q_per_kv = heads // kv_heads
     out = torch.empty_like(qw)
     lib = capi.load()
+    if decode is None:
+        # generation steps: few rows per key / value head and enough keys for the split to pay
+        decode = 0 < q_per_kv * n_q <= 16 and n_k >= 256 and d in (64, 128, 256)
     if qw.dtype == torch.float32:
-        _require(not decode, "the decode form is float16 only")
+        if decode:
+            need = lib.anygpu_sdp_attention_decode_f32_workspace_bytes(batch_heads, q_per_kv, n_q, n_k, d, int(causal), int(window))
+            capi.check("anygpu_sdp_attention_decode_f32_workspace_bytes", min(int(need), 0))
+            workspace = torch.empty(max(int(need), 16), dtype=torch.uint8, device=qw.device)
+            rc = lib.anygpu_sdp_attention_decode_f32(qw.data_ptr(), kw.data_ptr(), vw.data_ptr(), out.data_ptr(),
+                                                     workspace.data_ptr(), workspace.numel(), batch_heads, q_per_kv, n_q, n_k, d,
+                                                     float(alpha), float(softcap), int(causal), int(window), _stream_ptr())
+            capi.check("anygpu_sdp_attention_decode_f32", rc)
+            return out
         rc = lib.anygpu_sdp_attention_fwd_f32(qw.data_ptr(), kw.data_ptr(), vw.data_ptr(), out.data_ptr(),
                                               batch_heads, q_per_kv, n_q, n_k, d, float(alpha),
                                               float(softcap), int(causal), int(window), _stream_ptr())
         capi.check("anygpu_sdp_attention_fwd_f32", rc)
         return out
-    if decode is None:
-        # generation steps: few rows per key / value head and enough keys for the split to pay
-        decode = 0 < q_per_kv * n_q <= 16 and n_k >= 256 and d in (64, 128, 256)
     if decode:
         need = lib.anygpu_sdp_attention_decode_workspace_bytes(batch_heads, q_per_kv, n_q, n_k, d, int(causal), int(window))
         capi.check("anygpu_sdp_attention_decode_workspace_bytes", min(int(need), 0))

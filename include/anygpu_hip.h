@@ -213,6 +213,21 @@ int anygpu_sdp_attention_decode_f16(const void* q, const void* k, const void* v,
                                     float alpha, float softcap, int causal, int64_t window, void* stream);
 
 /*
+ * The decode form in float32: anygpu_sdp_attention_decode_f16 with fp32 operands and the fp32 matrix instruction
+ * (keys in tiles of 16, K and V straight from global memory into the MFMA operands).  Its workspace size comes
+ * from anygpu_sdp_attention_decode_f32_workspace_bytes.  The reference has no counterpart: its generation loop
+ * runs the per-head operator chain of sdp_attention_masked_scaled_fwd (srcs/transformers/sdp.hpp:258-271)
+ * against the key / value cache (srcs/models/gemma2/gemma_kv_cache.hpp).
+ */
+int64_t anygpu_sdp_attention_decode_f32_workspace_bytes(int64_t batch_heads, int64_t q_per_kv, int64_t n_q, int64_t n_k,
+                                                        int64_t head_dim, int causal, int64_t window);
+
+int anygpu_sdp_attention_decode_f32(const float* q, const float* k, const float* v, float* y,
+                                    void* workspace, int64_t workspace_bytes,
+                                    int64_t batch_heads, int64_t q_per_kv, int64_t n_q, int64_t n_k, int64_t head_dim,
+                                    float alpha, float softcap, int causal, int64_t window, void* stream);
+
+/*
  * Depthwise causal conv1d with bias and fused SiLU:
  *     y[b, d, s] = silu( bias[d] + sum_{k=0}^{width-1} w[d, k] * x[b, d, s + k - (width - 1)] ),
  * terms with a negative sequence index dropped (left zero padding of width-1).

@@ -1140,6 +1140,46 @@ def test_sdp_attention_decode_form(ops, oracle, case):
     assert scaled_rel_err(got, fused, 1.0) <= 2e-3
 
 
+@pytest.mark.parametrize("case", DECODE_CASES)
+def test_sdp_attention_decode_form_f32(ops, oracle, case):
+    heads, kv_heads, n_q, n_k, d, alpha, cap, causal, window = case
+    q = synth.normal(1 + n_q, (1, heads, n_q, d))
+    k = synth.normal(2 + n_k, (1, kv_heads, n_k, d))
+    v = synth.normal(3 + d, (1, kv_heads, n_k, d))
+    got = host(ops.sdp_attention_fwd(dev(q), dev(k), dev(v), alpha, softcap=cap, causal=causal, window=window, decode=True))
+    want = oracle.sdp_attention_rules(q[0], k[0], v[0], alpha=alpha, softcap=cap, causal=causal, window=window,
+                                      q_per_kv=heads // kv_heads, threads=8)
+    blind = np.isnan(want).all(axis=(0, 2))
+    assert blind.sum() == (max(n_q - n_k, 0) if causal else 0)
+    assert got.dtype == np.float32 and not got[0][:, blind, :].any()
+    assert scaled_rel_err(got[0][:, ~blind, :], want[:, ~blind, :], 1.0) <= TOL_F32
+    fused = host(ops.sdp_attention_fwd(dev(q), dev(k), dev(v), alpha, softcap=cap, causal=causal, window=window, decode=False))
+    assert scaled_rel_err(got, fused, 1.0) <= TOL_F32
+
+
+def test_sdp_attention_decode_f32_workspace_and_rejected_arguments(ops):
+    import torch
+    from anygpu_amd import capi
+    lib = capi.load()
+    ws_bytes = lib.anygpu_sdp_attention_decode_f32_workspace_bytes
+    # 4 key / value heads, 2 rows each, 4096 visible keys = 256 tiles of 16 -> 64 splits: 4 * 64 * 2 * (256 + 2) floats
+    assert ws_bytes(8, 2, 1, 8192, 256, 1, 4096) == 4 * 64 * 2 * 258 * 4
+    assert ws_bytes(8, 2, 1, 40, 256, 1, 0) == 4 * 3 * 2 * 258 * 4           # 3 tiles -> 3 splits
+    assert ws_bytes(0, 1, 1, 100, 64, 1, 0) == 0
+    assert ws_bytes(8, 2, 9, 100, 64, 1, 0) == capi.ANYGPU_ERR_UNSUPPORTED   # 18 rows per key / value head
+    q = torch.zeros((4, 1, 64), device="cuda")
+    kv = torch.zeros((2, 500, 64), device="cuda")
+    y = torch.full_like(q, 3.0)
+    need = ws_bytes(4, 2, 1, 500, 64, 1, 0)
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    f = lib.anygpu_sdp_attention_decode_f32
+    args = (4, 2, 1, 500, 64, 0.125, 0.0, 1, 0, None)
+    assert f(q.data_ptr(), kv.data_ptr(), kv.data_ptr(), y.data_ptr(), None, need, *args) == capi.ANYGPU_ERR_NULL_POINTER
+    assert f(q.data_ptr(), kv.data_ptr(), kv.data_ptr(), y.data_ptr(), ws.data_ptr(), need - 1, *args) == capi.ANYGPU_ERR_BAD_SHAPE
+    torch.cuda.synchronize()
+    assert bool((y == 3.0).all())
+
+
 def test_sdp_attention_decode_workspace_and_rejected_arguments(ops):
     import torch
     from anygpu_amd import capi
