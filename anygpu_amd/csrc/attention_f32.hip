@@ -62,7 +62,7 @@ __device__ __forceinline__ float logit2(float s, float k_in, float k_cap)
 template <int D, int KT>
 struct AttnLdsF32
 {
-	static constexpr int kPitch = D + 4;                      // floats per tile row: 16 bytes of padding
+	static constexpr int kPitch = D + 8;                      // floats per tile row: 32 bytes of padding
 	static constexpr int kStageFloats = 2 * KT * kPitch;      // a K tile and a V tile of KT keys
 };
 

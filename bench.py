@@ -37,7 +37,7 @@ PEAK_HBM_GBS = 8000.0          # HBM3E
 # write x 1.000); the summaries are under profiles/.
 MEASURED_TRAFFIC_BYTES = {"gemm_f16": 234962687, "gemm_f32": 167994164, "conv1d": 277226336,
                           "softmax_causal": 410887952, "softmax_gemma2": 1514268488,
-                          "attention_gemma2": 689788928, "gated_rmsnorm": 805513216}
+                          "attention_gemma2": 689788928, "attention_gemma2_f32": 1426475418, "gated_rmsnorm": 805513216}
 
 
 def parse_args():
@@ -214,7 +214,7 @@ def bench_attention_f32(torch, ops, steps, warmup):
         "workload": "fused attention fp32 q [1, 8, 8192, 256], k / v [1, 4, 8192, 256], x 1/16, softcap 50, causal + window 4096",
         "us_per_launch": t * 1e6, "value": flops / t / 1e12, "unit": "TFLOP/s", "dtype": "f32",
         "roofline": {"bound": "mfma", "achieved": flops / t / 1e12, "peak": PEAK_FP32_TFLOPS, "unit": "TFLOP/s",
-                     "frac": flops / t / 1e12 / PEAK_FP32_TFLOPS, "traffic": None,
+                     "frac": flops / t / 1e12 / PEAK_FP32_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES["attention_gemma2_f32"],
                      "algorithmic_flops": flops, "visible_pairs_per_head": pairs},
     }
 
