@@ -1234,6 +1234,82 @@ def test_sdp_attention_fused_kernel_gemma2_block(ops, oracle):
 
 
 # =============================================================================================
+# launches recorded into a HIP graph
+# =============================================================================================
+
+def test_launches_replayed_from_a_graph(ops, oracle):
+    # a stream is warmed up eagerly (which gives it the K-split workspace), then the same calls are captured on it and
+    # replayed three times with new input values and eager work in between; every replay must equal the eager result
+    import torch
+    from anygpu_amd import capi
+    side = torch.cuda.Stream()
+    a32 = torch.empty((24, 4096), device="cuda")
+    w32 = dev(synth.uniform(1, (4096, 260)))                        # [K, N] fp32: band kernel, K split
+    a16 = torch.empty((128, 2304), device="cuda", dtype=torch.float16)
+    w16 = dev(synth.uniform(2, (2048, 2304)).astype(np.float16))    # [N, K] fp16: tile kernel, K split
+    sc = torch.empty((64, 512), device="cuda", dtype=torch.float16)
+    cx = torch.empty((2, 16, 300), device="cuda", dtype=torch.float16)
+    cw, cb = dev(synth.normal(3, (16, 4)).astype(np.float16)), dev(synth.normal(4, (16,)).astype(np.float16))
+    q = torch.empty((1, 4, 100, 128), device="cuda")
+    kv = dev(synth.normal(5, (1, 2, 100, 128)))
+
+    def fill(seed):
+        a32.copy_(dev(synth.uniform(seed, tuple(a32.shape))))
+        a16.copy_(dev(synth.uniform(seed + 1, tuple(a16.shape)).astype(np.float16)))
+        sc.copy_(dev((synth.normal(seed + 2, tuple(sc.shape)) * np.float32(4.0)).astype(np.float16)))
+        cx.copy_(dev(synth.normal(seed + 3, tuple(cx.shape)).astype(np.float16)))
+        q.copy_(dev(synth.normal(seed + 4, tuple(q.shape))))
+
+    def work():
+        return (ops.tensor_mm(a32, w32),
+                ops.tensor_mm(a16, w16, b_layout=capi.B_COL_MAJOR),
+                ops.tensor_softmax(sc, alpha=0.125, causal=True, q_len=64),
+                ops.tensor_causal_conv1d(cx, cw, cb),
+                ops.sdp_attention_fwd(q, kv, kv, 0.0884, softcap=30.0, causal=True, window=40))
+
+    fill(10)
+    with torch.cuda.stream(side):
+        work()
+    side.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        outs = work()
+    for rep in range(3):
+        fill(20 + 10 * rep)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [host(t).copy() for t in outs]
+        want = [host(t) for t in work()]                             # eager, on the default stream
+        torch.cuda.synchronize()
+        for g, w in zip(got, want):
+            assert np.array_equal(g, w)
+
+
+def test_k_split_products_on_concurrent_streams(ops, oracle):
+    # every stream owns its partial-sum workspace: products that are cut along K may overlap on different streams
+    import torch
+    from anygpu_amd import capi
+    streams = [torch.cuda.Stream() for _ in range(3)]
+    problems = []
+    for i, (m, k, n) in enumerate([(24, 8192, 260), (128, 4608, 512), (16, 9216, 2304)]):
+        a = dev(synth.uniform(10 + i, (m, k)))
+        w = dev(synth.uniform(20 + i, (n, k)))
+        problems.append((a, w, host(ops.tensor_mm(a, w, b_layout=capi.B_COL_MAJOR))))
+    torch.cuda.synchronize()
+    results = [[] for _ in streams]
+    for rep in range(8):
+        for si, st in enumerate(streams):
+            a, w, _ = problems[(si + rep) % 3]
+            with torch.cuda.stream(st):
+                results[si].append(((si + rep) % 3, ops.tensor_mm(a, w, b_layout=capi.B_COL_MAJOR)))
+    torch.cuda.synchronize()
+    for per_stream in results:
+        for which, out in per_stream:
+            assert np.array_equal(host(out), problems[which][2])
+
+
+# =============================================================================================
 # committed golden fixtures (tests/golden/*.dat)
 # =============================================================================================
 
