@@ -3,8 +3,14 @@
  * and causal conv1d + SiLU entry points.
  *
  * Conventions
- *   - every pointer is a DEVICE pointer into memory the caller owns; nothing is allocated,
- *     freed or retained by the library, inputs are only read, outputs only written;
+ *   - every pointer is a DEVICE pointer into memory the caller owns; inputs are only read,
+ *     outputs only written.  The library frees nothing and keeps one thing, like a BLAS handle:
+ *     the GEMM entry points cut some products along K (few tiles and a deep K, few rows against
+ *     a weight matrix) and put the partial sums of such a launch into a 16 MiB device buffer
+ *     that is allocated the first time a (device, stream) pair needs it and kept until the
+ *     process ends.  Launches on one stream share it in stream order, other streams have their
+ *     own.  No allocation is made while the stream is being captured into a graph: a pair
+ *     without a buffer then runs uncut.  Nothing else allocates;
  *   - sizes, strides and leading dimensions are int64_t counts of ELEMENTS;
  *   - `stream` is a hipStream_t passed as void* (NULL = the null stream, which is what the
  *     reference uses for every launch); calls are asynchronous with respect to the host;
