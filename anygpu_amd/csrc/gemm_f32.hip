@@ -490,6 +490,37 @@ static hipError_t launch_layout(const float* A, const float* B, const float* B2,
 	const bool may_split = (EPI != kEpiGeluMul);
 	const TilePlan big = plan_tiles(128, M, N, K, batch, may_split);
 	const TilePlan small = plan_tiles(64, M, N, K, batch, may_split);
+	if constexpr (EPI != kEpiGeluMul)
+	{
+		// A product of big tiles that fills whole rounds and a bit, e.g. 576 tiles = 2.25 rounds, pays three rounds.  It
+		// is divided by columns into the whole rounds, launched as they are, and the rest, which as a product of its
+		// own is cut along K by the plan above (1024 x 2304 x 9216: 411 us as one launch).
+		const int64_t tiles_m = (M + 127) / 128, tiles_n = (N + 127) / 128;
+		const int64_t whole = tiles_m * tiles_n / kChipCus * kChipCus;
+		const int64_t head_cols = whole / tiles_m;                      // tile columns of the first part
+		if (batch == 1 && whole > 0 && head_cols > 0 && head_cols < tiles_n)
+		{
+			const int64_t n_head = head_cols * 128, n_tail = N - n_head;
+			const TilePlan head = plan_tiles(128, M, n_head, K, 1, false);
+			const TilePlan tail_big = plan_tiles(128, M, n_tail, K, 1, true);
+			const TilePlan tail_small = plan_tiles(64, M, n_tail, K, 1, true);
+			const TilePlan& tail = tail_big.cost <= tail_small.cost ? tail_big : tail_small;
+			const double best_whole = big.cost <= small.cost ? big.cost : small.cost;
+			if (head.cost + tail.cost + 3.0 < 0.96 * best_whole)
+			{
+				const hipError_t err = launch_tiles<A_LAYOUT, B_LAYOUT, 128, 128, EPI>(
+					A, B, B2, bias, C, M, n_head, K, lda, ldb, ldc, 0, 0, 0, 1, ep_param, 1, stream);
+				if (err != hipSuccess) return err;
+				const float* b_tail = (B_LAYOUT == ANYGPU_B_COL_MAJOR) ? B + n_head * ldb : B + n_head;
+				const float* bias_tail = bias ? bias + n_head : nullptr;
+				if (tail.tile == 128)
+					return launch_tiles<A_LAYOUT, B_LAYOUT, 128, 128, EPI>(A, b_tail, nullptr, bias_tail, C + n_head, M, n_tail, K,
+					                                                       lda, ldb, ldc, 0, 0, 0, 1, ep_param, tail.splits, stream);
+				return launch_tiles<A_LAYOUT, B_LAYOUT, 64, 64, EPI>(A, b_tail, nullptr, bias_tail, C + n_head, M, n_tail, K,
+				                                                     lda, ldb, ldc, 0, 0, 0, 1, ep_param, tail.splits, stream);
+			}
+		}
+	}
 	if (big.cost <= small.cost)
 		return launch_tiles<A_LAYOUT, B_LAYOUT, 128, 128, EPI>(A, B, B2, bias, C, M, N, K, lda, ldb, ldc,
 		                                                       stride_a, stride_b, stride_c, batch, ep_param, big.splits, stream);
