@@ -471,6 +471,29 @@ def test_mm_f32_few_tiles_split_along_k(ops, oracle, layout, m, k, n):
         assert scaled_rel_err(got, want, math.sqrt(k) / 3.0) <= TOL_F32
 
 
+@pytest.mark.parametrize("layout", ["row", "col"])
+@pytest.mark.parametrize("m,k,n", [(520, 512, 9300), (1024, 640, 4608 + 128), (300, 1024, 11000)])
+def test_mm_f32_whole_rounds_and_a_rest(ops, oracle, layout, m, k, n):
+    # more big tiles than one round of blocks but not a whole number of rounds: the columns of the whole rounds and
+    # the rest (cut along K where that pays) are separate launches; bias and softcap reach both parts
+    from anygpu_amd import capi
+    a = synth.uniform(m + k, (m, k))
+    b = synth.uniform(k + n, (k, n))
+    bias = synth.uniform(5, (n,))
+    want = oracle.tensor_mm(a, b, threads=8)
+    da = dev(a)
+    db = dev(b) if layout == "row" else dev(np.ascontiguousarray(b.T))
+    lay = capi.B_ROW_MAJOR if layout == "row" else capi.B_COL_MAJOR
+    got = host(ops.tensor_mm(da, db, b_layout=lay))
+    assert scaled_rel_err(got, want, math.sqrt(k) / 3.0) <= TOL_F32
+    got = host(ops.tensor_gemm(da, db, dev(bias), b_layout=lay))
+    assert scaled_rel_err(got, want + bias, math.sqrt(k) / 3.0) <= TOL_F32
+    if layout == "col":
+        got = host(ops.tensor_gemma_linear_softcap(da.reshape(1, m, k), db, 30.0))[0]
+        ref = oracle.gemma_linear_softcap(a.reshape(1, m, k), np.ascontiguousarray(b.T), 30.0, threads=8)[0]
+        assert scaled_rel_err(got, ref, math.sqrt(k) / 3.0) <= TOL_F32
+
+
 def test_mm_f32_transposed_left_operand(ops, oracle):
     # the layout of the reference's last fp32 rung: A handed over as [K, M]
     from anygpu_amd import capi
