@@ -184,6 +184,31 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
 		};
 		const double cost256 = slab_us(256, blocks(256)), cost128 = slab_us(128, blocks(128)), cost64 = slab_us(64, blocks(64));
 		const int64_t tile = (cost256 <= cost128 && cost256 <= cost64) ? 256 : cost128 <= cost64 ? 128 : 64;
+		// A product of 256 x 256 tiles that fills whole rounds of blocks and a bit (320 tiles pay two rounds) is divided
+		// by columns into the whole rounds and the rest, which is launched as a product of its own with its own tile.
+		if (tile == 256 && batch == 1)
+		{
+			const int64_t tiles_m = (M + 255) / 256, tiles_n = (N + 255) / 256;
+			const int64_t whole = tiles_m * tiles_n / 256 * 256;
+			const int64_t head_cols = whole / tiles_m;
+			if (whole > 0 && head_cols > 0 && head_cols < tiles_n)
+			{
+				const int64_t n_head = head_cols * 256, n_tail = N - n_head;
+				const auto tail_blocks = [&](int64_t t) { return ((M + t - 1) / t) * ((n_tail + t - 1) / t); };
+				double tail_cost = slab_us(256, tail_blocks(256));
+				if (slab_us(128, tail_blocks(128)) < tail_cost) tail_cost = slab_us(128, tail_blocks(128));
+				if (slab_us(64, tail_blocks(64)) < tail_cost) tail_cost = slab_us(64, tail_blocks(64));
+				const double slabs = (double)((K + 63) / 64);
+				const double divided = (slab_us(256, head_cols * tiles_m) + tail_cost) * slabs + 3.0;
+				if (divided < 0.93 * cost256 * slabs)
+				{
+					const hipError_t err = launch_gemm_f16(A, B, C, M, n_head, K, lda, ldb, ldc, 0, 0, 0, 1, b_layout, stream);
+					if (err != hipSuccess) return err;
+					const half_t* b_tail = (b_layout == ANYGPU_B_COL_MAJOR) ? b + n_head * ldb : b + n_head;
+					return launch_gemm_f16(A, b_tail, c + n_head, M, n_tail, K, lda, ldb, ldc, 0, 0, 0, 1, b_layout, stream);
+				}
+			}
+		}
 		// one "general" instantiation serves ragged M / N and a K tail alike
 		const bool ragged = (M % tile != 0) || (N % tile != 0) || (K % 64 != 0);
 		const bool fits = ((M + tile - 1) / tile) * ((N + tile - 1) / tile) <= 0x7FFFFFFFLL;

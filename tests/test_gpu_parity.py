@@ -628,6 +628,20 @@ def test_mm_f16_few_tiles_split_along_k(ops, oracle, layout, m, k, n):
     assert np.array_equal(host(ops.tensor_mm(dev(ai), dbi, b_layout=lay)).astype(np.float32), want_i.astype(np.float16).astype(np.float32))
 
 
+@pytest.mark.parametrize("layout", ["row", "col"])
+@pytest.mark.parametrize("m,k,n", [(4096, 128, 5120), (2100, 64, 8000), (4352, 64, 4352)])
+def test_mm_f16_whole_rounds_and_a_rest(ops, oracle, layout, m, k, n):
+    # more 256 x 256 tiles than one round of blocks but not a whole number of rounds: two launches, divided by columns
+    from anygpu_amd import capi
+    a = synth.integers(m + k, (m, k), -2, 2).astype(np.float16)
+    b = synth.integers(k + n, (k, n), -2, 2).astype(np.float16)
+    want = oracle.tensor_mm(a.astype(np.float32), b.astype(np.float32), threads=8)
+    db = dev(b) if layout == "row" else dev(np.ascontiguousarray(b.T))
+    lay = capi.B_ROW_MAJOR if layout == "row" else capi.B_COL_MAJOR
+    got = host(ops.tensor_mm(dev(a), db, b_layout=lay)).astype(np.float32)
+    assert np.array_equal(got, want)
+
+
 def test_mm_f16_ragged_integer_inputs_bit_exact_and_batched(ops, oracle):
     from anygpu_amd import capi
     a = synth.integers(1, (200, 128), -4, 4).astype(np.float16)
