@@ -822,6 +822,45 @@ def test_gemm_epilogues_decode_step(ops, oracle, s):
     assert scaled_rel_err(got, want, 1.0) <= TOL_F32
 
 
+def _random_mm_shapes(seed, count, k_max):
+    rng = np.random.default_rng(seed)
+    shapes = []
+    while len(shapes) < count:
+        regime = len(shapes) % 5
+        if regime == 0:      # few rows, wide weights
+            m, k, n = int(rng.integers(1, 70)), int(rng.integers(1, k_max)), int(rng.integers(1, 9000))
+        elif regime == 1:    # few rows, deep K
+            m, k, n = int(rng.integers(1, 70)), int(rng.integers(k_max // 2, k_max)), int(rng.integers(1, 700))
+        elif regime == 2:    # a few tiles
+            m, k, n = int(rng.integers(60, 600)), int(rng.integers(1, k_max)), int(rng.integers(60, 700))
+        elif regime == 3:    # more than one round of big tiles
+            m, k, n = int(rng.integers(1000, 2600)), int(rng.integers(1, 80)), int(rng.integers(3000, 6000))
+        else:                # aligned versions of the above
+            m, k, n = int(rng.integers(1, 40)) * 8, int(rng.integers(1, max(k_max // 64, 2))) * 64, int(rng.integers(1, 40)) * 128
+        if m * k * n <= 400_000_000:
+            shapes.append((m, k, n))
+    return shapes
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f16"])
+def test_mm_random_shapes_integer_inputs_exact(ops, oracle, dtype):
+    # small integers make every sum exact whatever the order, so every kernel family, every cut along K and every
+    # division of a launch has to reproduce the oracle bit for bit; 40 shapes over the dispatch regimes, both layouts
+    from anygpu_amd import capi
+    k_max = 4000 if dtype == "f32" else 500          # |sum| < 2^24 in fp32; <= 2048, an fp16 integer, in half precision
+    lo, hi = (-4, 4) if dtype == "f32" else (-2, 2)
+    np_dt = np.float32 if dtype == "f32" else np.float16
+    for i, (m, k, n) in enumerate(_random_mm_shapes(7 if dtype == "f32" else 8, 40, k_max)):
+        a = synth.integers(100 + i, (m, k), lo, hi)
+        b = synth.integers(200 + i, (k, n), lo, hi)
+        want = oracle.tensor_mm(a, b, threads=8)
+        da = dev(a.astype(np_dt))
+        got_row = host(ops.tensor_mm(da, dev(b.astype(np_dt)))).astype(np.float32)
+        got_col = host(ops.tensor_mm(da, dev(np.ascontiguousarray(b.T).astype(np_dt)), b_layout=capi.B_COL_MAJOR)).astype(np.float32)
+        assert np.array_equal(got_row, want), ("row", m, k, n)
+        assert np.array_equal(got_col, want), ("col", m, k, n)
+
+
 def test_mm_empty_and_rejected_arguments(ops):
     import torch
     from anygpu_amd import capi
