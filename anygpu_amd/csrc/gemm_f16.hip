@@ -15,79 +15,151 @@
 namespace anygpu {
 
 // ---------------------------------------------------------------------------------------------
-// Edge kernel: 64 x 64 tile, 4 waves, one 32 x 32 MFMA tile per wave, 16-deep steps.
-// Every global access is guarded and scalar; K tails are zero-filled in LDS.
+// Edge kernel for operands the tile kernels cannot take (N or K no multiple of 8, rows or pointers that are not
+// 16-byte aligned): 128 x 128 tile, 4 waves with a 64 x 64 patch each (2 x 2 MFMA tiles of 32 x 32 x 16), 32-deep
+// slabs through registers into LDS.  A vector of 8 halves that lies inside its row is fetched with one 16-byte
+// load at element alignment, the ends of rows element by element, everything outside the operand is zero in LDS.
+// [K, N] weights are transposed on their way into LDS (the MFMA operand is k-contiguous).
 // ---------------------------------------------------------------------------------------------
+constexpr int kEdgeTile = 128;
+constexpr int kEdgeDepth = 32;
+constexpr int kEdgePitch = kEdgeDepth + 8;      // halves per LDS row: 80 bytes, keeps 16-byte alignment
+
+typedef half8_t LooseHalf8 __attribute__((aligned(2)));
+typedef half4_t LooseHalf4 __attribute__((aligned(2)));
+
+// 8 consecutive elements of a row of `len` valid elements starting at `pos`; zeros past the end
+__device__ __forceinline__ half8_t edge_fetch(const half_t* row, int64_t pos, int64_t len, bool row_ok)
+{
+	half8_t v = {};
+	if (!row_ok || pos >= len) return v;
+	if (pos + 8 <= len) return *reinterpret_cast<const LooseHalf8*>(row + pos);
+#pragma unroll
+	for (int e = 0; e < 8; ++e)
+		if (pos + e < len) v[e] = row[pos + e];
+	return v;
+}
+
 template <int B_LAYOUT>
 __global__ __launch_bounds__(256) void gemm_f16_edge_kernel(
 	const half_t* __restrict__ A, const half_t* __restrict__ B, half_t* __restrict__ C,
 	int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc,
 	int64_t stride_a, int64_t stride_b, int64_t stride_c)
 {
-	__shared__ half_t a_lds[64][16 + 8];
+	__shared__ __align__(16) half_t a_lds[kEdgeTile * kEdgePitch];
+	__shared__ __align__(16) half_t b_lds[kEdgeTile * kEdgePitch];
 	A += (int64_t)blockIdx.z * stride_a;
 	B += (int64_t)blockIdx.z * stride_b;
 	C += (int64_t)blockIdx.z * stride_c;
-	__shared__ half_t b_lds[64][16 + 8];
 
 	const int tid = threadIdx.x;
 	const int lane = tid & (kWaveSize - 1);
 	const int wave = tid >> 6;
-	const int64_t m0 = (int64_t)blockIdx.y * 64;
-	const int64_t n0 = (int64_t)blockIdx.x * 64;
+	const int64_t m0 = (int64_t)blockIdx.y * kEdgeTile;
+	const int64_t n0 = (int64_t)blockIdx.x * kEdgeTile;
 	const int wm = wave >> 1, wn = wave & 1;
 
-	float16_t acc;
+	float16_t acc[2][2];
 #pragma unroll
-	for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
+	for (int i = 0; i < 2; ++i)
+#pragma unroll
+		for (int j = 0; j < 2; ++j)
+#pragma unroll
+			for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
-	for (int64_t k0 = 0; k0 < K; k0 += 16)
-	{
+	// a slab is 128 rows x 4 vectors (k-contiguous operands) or 32 k rows x 16 vectors ([K, N] weights): 2 per thread
+	half8_t ar[2], br[2];
+	auto fetch = [&](int64_t k0) {
 #pragma unroll
-		for (int i = 0; i < 4; ++i)
+		for (int i = 0; i < 2; ++i)
 		{
-			const int q = tid + 256 * i;      // 0..1023
+			const int q = tid + 256 * i;
 			{
-				const int r = q / 16, c = q % 16;
-				const int64_t m = m0 + r, k = k0 + c;
-				a_lds[r][c] = (m < M && k < K) ? A[m * lda + k] : (half_t)0.0f;
+				const int r = q >> 2, c = (q & 3) * 8;
+				ar[i] = edge_fetch(A + (m0 + r) * lda, k0 + c, K, m0 + r < M);
 			}
 			if (B_LAYOUT == ANYGPU_B_COL_MAJOR)
 			{
-				const int r = q / 16, c = q % 16;
-				const int64_t n = n0 + r, k = k0 + c;
-				b_lds[r][c] = (n < N && k < K) ? B[n * ldb + k] : (half_t)0.0f;
+				const int r = q >> 2, c = (q & 3) * 8;
+				br[i] = edge_fetch(B + (n0 + r) * ldb, k0 + c, K, n0 + r < N);
 			}
 			else
 			{
-				const int c = q / 64, r = q % 64;  // consecutive threads walk n
-				const int64_t n = n0 + r, k = k0 + c;
-				b_lds[r][c] = (n < N && k < K) ? B[k * ldb + n] : (half_t)0.0f;
+				const int kr = q & 31, c = (q >> 5) * 8;    // a wave's lanes on consecutive k: conflict-free LDS rows below
+				br[i] = edge_fetch(B + (k0 + kr) * ldb, n0 + c, N, k0 + kr < K);
 			}
 		}
-		__syncthreads();
-
-		half8_t af, bf;
-		const int kb = (lane >> 5) * 8;
+	};
+	auto stage = [&]() {
 #pragma unroll
-		for (int e = 0; e < 8; ++e)
+		for (int i = 0; i < 2; ++i)
 		{
-			af[e] = a_lds[wm * 32 + (lane & 31)][kb + e];
-			bf[e] = b_lds[wn * 32 + (lane & 31)][kb + e];
+			const int q = tid + 256 * i;
+			*reinterpret_cast<half8_t*>(&a_lds[(q >> 2) * kEdgePitch + (q & 3) * 8]) = ar[i];
+			if (B_LAYOUT == ANYGPU_B_COL_MAJOR)
+			{
+				*reinterpret_cast<half8_t*>(&b_lds[(q >> 2) * kEdgePitch + (q & 3) * 8]) = br[i];
+			}
+			else
+			{
+				const int kr = q & 31, c = (q >> 5) * 8;
+#pragma unroll
+				for (int e = 0; e < 8; ++e) b_lds[(c + e) * kEdgePitch + kr] = br[i][e];
+			}
 		}
-		acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf, af, acc, 0, 0, 0);
+	};
+
+	const int frag_row = lane & 31;
+	const int kb = (lane >> 5) * 8;
+	fetch(0);
+	for (int64_t k0 = 0; k0 < K; k0 += kEdgeDepth)
+	{
+		__syncthreads();                        // the previous slab has been read
+		stage();
 		__syncthreads();
+		if (k0 + kEdgeDepth < K) fetch(k0 + kEdgeDepth);
+#pragma unroll
+		for (int st = 0; st < kEdgeDepth / 16; ++st)
+		{
+			half8_t af[2], bf[2];
+#pragma unroll
+			for (int i = 0; i < 2; ++i)
+			{
+				af[i] = *reinterpret_cast<const half8_t*>(&a_lds[(wm * 64 + i * 32 + frag_row) * kEdgePitch + 16 * st + kb]);
+				bf[i] = *reinterpret_cast<const half8_t*>(&b_lds[(wn * 64 + i * 32 + frag_row) * kEdgePitch + 16 * st + kb]);
+			}
+#pragma unroll
+			for (int i = 0; i < 2; ++i)
+#pragma unroll
+				for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[j], af[i], acc[i][j], 0, 0, 0);
+		}
 	}
 
-	const int64_t m = m0 + wm * 32 + (lane & 31);
-	if (m < M)
-	{
+	// register 4 g + e of a lane: row lane % 32 of the A tile, column 8 g + 4 (lane / 32) + e of the B tile
 #pragma unroll
-		for (int r = 0; r < 16; ++r)
-		{
-			const int64_t n = n0 + wn * 32 + 8 * (r / 4) + 4 * (lane >> 5) + (r % 4);
-			if (n < N) C[m * ldc + n] = (half_t)acc[r];
-		}
+	for (int i = 0; i < 2; ++i)
+	{
+		const int64_t m = m0 + wm * 64 + i * 32 + frag_row;
+		if (m >= M) continue;
+#pragma unroll
+		for (int j = 0; j < 2; ++j)
+#pragma unroll
+			for (int g = 0; g < 4; ++g)
+			{
+				const int64_t n = n0 + wn * 64 + j * 32 + 8 * g + 4 * (lane >> 5);
+				half_t* dst = C + m * ldc + n;
+				if (n + 4 <= N)
+				{
+					*reinterpret_cast<LooseHalf4*>(dst) = half4_t{(half_t)acc[i][j][4 * g], (half_t)acc[i][j][4 * g + 1],
+					                                              (half_t)acc[i][j][4 * g + 2], (half_t)acc[i][j][4 * g + 3]};
+				}
+				else
+				{
+#pragma unroll
+					for (int e = 0; e < 4; ++e)
+						if (n + e < N) dst[e] = (half_t)acc[i][j][4 * g + e];
+				}
+			}
 	}
 }
 
@@ -284,7 +356,7 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
 #undef ANYGPU_F16_TILE
 	}
 
-	const dim3 grid((unsigned)((N + 63) / 64), (unsigned)((M + 63) / 64), (unsigned)batch);
+	const dim3 grid((unsigned)((N + kEdgeTile - 1) / kEdgeTile), (unsigned)((M + kEdgeTile - 1) / kEdgeTile), (unsigned)batch);
 	discard_stale_error();
 	if (b_layout == ANYGPU_B_COL_MAJOR)
 		gemm_f16_edge_kernel<ANYGPU_B_COL_MAJOR><<<grid, dim3(256), 0, stream>>>(a, b, c, M, N, K, lda, ldb, ldc,
