@@ -12,7 +12,7 @@
 //   * S^T = K Q^T with v_mfma_f32_16x16x32_f16: the K fragment is the first operand, the Q
 //     fragment (kept in registers for the whole kernel) the second, so a lane ends up holding,
 //     for ONE query (lane % 16), the scores of keys 4 (lane / 16) + r of each 16-key block.
-//     Row maxima and sums are therefore in-lane loops plus two cross-lane steps (xor 16, xor 32);
+//     Row maxima and sums are therefore in-lane loops plus two cross-row steps (row swaps in the VALU);
 //   * scale / softcap / mask in fp32, online max / sum in the log2 domain, p = exp2(z - m)
 //     rounded to fp16;
 //   * O^T += V^T P^T: first operand V^T, read out of the row-major V tile with transposing LDS
@@ -248,8 +248,7 @@ __global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f16_kernel(const
 						mt = fmaxf(mt, z[kb][r]);
 					}
 			}
-			mt = fmaxf(mt, __shfl_xor(mt, 16));
-			mt = fmaxf(mt, __shfl_xor(mt, 32));
+			mt = max_over_lane_rows(mt);
 			const float m_new = fmaxf(m_run[b], mt);
 			const float m_safe = (m_new == -INFINITY) ? 0.0f : m_new;   // nothing visible so far: every term is exp2(-inf) = 0
 			float psum = 0.0f;
@@ -482,8 +481,7 @@ __global__ __launch_bounds__(64) void sdp_decode_partial_kernel(const DecodeArgs
 				z[kb][r] = (key >= vis_lo && key <= vis_hi) ? zz : -INFINITY;
 				mt = fmaxf(mt, z[kb][r]);
 			}
-		mt = fmaxf(mt, __shfl_xor(mt, 16));
-		mt = fmaxf(mt, __shfl_xor(mt, 32));
+		mt = max_over_lane_rows(mt);
 		const float m_new = fmaxf(m_run, mt);
 		const float m_safe = (m_new == -INFINITY) ? 0.0f : m_new;
 		const float corr = fast_exp2(m_run - m_safe);

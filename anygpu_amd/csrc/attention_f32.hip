@@ -281,8 +281,7 @@ __global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f32_kernel(const
 					mt = fmaxf(mt, z[kb][r]);
 				}
 		}
-		mt = fmaxf(mt, __shfl_xor(mt, 16));
-		mt = fmaxf(mt, __shfl_xor(mt, 32));
+		mt = max_over_lane_rows(mt);
 		const float m_new = fmaxf(m_run, mt);
 		const float m_safe = (m_new == -INFINITY) ? 0.0f : m_new;   // nothing visible so far: every term is exp2(-inf) = 0
 		float psum = 0.0f;
@@ -489,8 +488,7 @@ __global__ __launch_bounds__(64) void sdp_decode_partial_f32_kernel(const Decode
 			z[r] = (key >= vis_lo && key <= vis_hi) ? zz : -INFINITY;
 			mt = fmaxf(mt, z[r]);
 		}
-		mt = fmaxf(mt, __shfl_xor(mt, 16));
-		mt = fmaxf(mt, __shfl_xor(mt, 32));
+		mt = max_over_lane_rows(mt);
 		const float m_new = fmaxf(m_run, mt);
 		const float m_safe = (m_new == -INFINITY) ? 0.0f : m_new;
 		const float corr = fast_exp2(m_run - m_safe);

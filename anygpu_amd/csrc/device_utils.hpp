@@ -56,6 +56,23 @@ __device__ __forceinline__ float wave_allreduce(float v, Op op)
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
 
+// Maximum over the four 16-lane rows of a wave, for every lane % 16, left in all four rows.  gfx950's row swaps do in
+// the VALU what two cross-lane shuffles (each a trip through the LDS crossbar) do: v_permlane16_swap exchanges the
+// odd rows of its first operand with the even rows of its second, v_permlane32_swap the upper half of the first with
+// the lower half of the second; fed two copies of x they return {row 0, 0, 2, 2} and {1, 1, 3, 3}, then {lower, lower}
+// and {upper, upper}.  (Written as assembly: the builtins of this compiler release fold the pair of results of a swap
+// of two equal operands into one value.)
+__device__ __forceinline__ float max_over_lane_rows(float x)
+{
+	float a = x, b = x;
+	asm("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+	const float m = fmaxf(a, b);
+	a = m;
+	b = m;
+	asm("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+	return fmaxf(a, b);
+}
+
 // tanh(x) = 1 - 2 / (1 + e^{2x}); saturates cleanly to +-1 for large |x| (e^{2x} -> inf or 0).
 // Near zero that form cancels, so |x| < 1/16 uses the odd Taylor polynomial up to x^7
 // (truncation error below 1e-11 relative at the switch point).
