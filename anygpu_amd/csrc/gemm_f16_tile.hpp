@@ -124,6 +124,13 @@ struct GemmTileCfg
 
 // vmcnt(0) with the other counters left alone (gfx9 encoding: vmcnt in [3:0] and [15:14],
 // expcnt [6:4], lgkmcnt [11:8])
+// global_load_lds_dwordx4 with the LDS base of the wave-wide 1 KB destination in M0 (wave-uniform)
+__device__ __forceinline__ void direct_load_asm(const void* src, const char* lds_dst)
+{
+	const unsigned m0 = __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)(const __attribute__((address_space(3))) char*)lds_dst);
+	asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src), "s"(m0) : "m0");
+}
+
 __device__ __forceinline__ void wait_vmem_all()
 {
 	__builtin_amdgcn_s_waitcnt(0x0F70);
@@ -325,14 +332,30 @@ __global__ __launch_bounds__(Cfg::kThreads) void gemm_f16_nt_tile_kernel(
 		char* b_lds = a_lds + Cfg::kSlabABytes;
 		const int64_t koff = (int64_t)kt * BK;
 		const int64_t koff_b = Cfg::B_KN ? koff * ldb : koff;
+		if constexpr (Cfg::B_KN)
+		{
+			// Written as assembly for this layout: in front of a transposing LDS read the compiler waits for ALL of the
+			// wave's outstanding direct loads (it cannot tell that they fill the other stage), which would put the
+			// whole memory latency of the slab just requested in front of the first fragment read behind the barrier.
+			// The waits these loads need are the explicit vmcnt(0) in front of every slab barrier.
 #pragma unroll
-		for (int i = 0; i < Cfg::kLoadsA; ++i)
-			__builtin_amdgcn_global_load_lds((global_void*)(a_src[i] + koff),
-			                                 (lds_void*)(a_lds + 1024 * (wave * Cfg::kLoadsA + i)), 16, 0, 0);
+			for (int i = 0; i < Cfg::kLoadsA; ++i)
+				direct_load_asm(a_src[i] + koff, a_lds + 1024 * (wave * Cfg::kLoadsA + i));
 #pragma unroll
-		for (int i = 0; i < Cfg::kLoadsB; ++i)
-			__builtin_amdgcn_global_load_lds((global_void*)(b_src[i] + koff_b),
-			                                 (lds_void*)(b_lds + 1024 * (wave * Cfg::kLoadsB + i)), 16, 0, 0);
+			for (int i = 0; i < Cfg::kLoadsB; ++i)
+				direct_load_asm(b_src[i] + koff_b, b_lds + 1024 * (wave * Cfg::kLoadsB + i));
+		}
+		else
+		{
+#pragma unroll
+			for (int i = 0; i < Cfg::kLoadsA; ++i)
+				__builtin_amdgcn_global_load_lds((global_void*)(a_src[i] + koff),
+				                                 (lds_void*)(a_lds + 1024 * (wave * Cfg::kLoadsA + i)), 16, 0, 0);
+#pragma unroll
+			for (int i = 0; i < Cfg::kLoadsB; ++i)
+				__builtin_amdgcn_global_load_lds((global_void*)(b_src[i] + koff_b),
+				                                 (lds_void*)(b_lds + 1024 * (wave * Cfg::kLoadsB + i)), 16, 0, 0);
+		}
 	};
 
 	Acc acc[TM][TN];
