@@ -137,7 +137,7 @@ __global__ __launch_bounds__(kBandThreads) void gemm_band_ncontig_kernel(
 			const int64_t k = k0 + t;
 			const int64_t kk = (decltype(guarded)::value && k >= ke) ? kb : k;
 #pragma unroll
-			for (int w = 0; w < S::kMats; ++w) dst[w][t] = *reinterpret_cast<const Vec*>(wcol[w] + kk * ldb);
+			for (int w = 0; w < S::kMats; ++w) dst[w][t] = __builtin_nontemporal_load(reinterpret_cast<const Vec*>(wcol[w] + kk * ldb));
 		}
 	};
 	auto mask_w = [&](Vec (&v)[S::kMats][4], int64_t wstep) {
