@@ -162,9 +162,10 @@ __global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f16_kernel(const
 	const int all_lo = a.window > 0 ? wq1 + a.diag - a.window + 1 : 0;
 
 	float4_t kr[VPT], vr[VPT];
-	auto tile_load = [&](int t) {
+	// vectors [i0, i1) of this thread's share of tile t
+	auto tile_load_part = [&](int t, int i0, int i1) {
 #pragma unroll
-		for (int i = 0; i < VPT; ++i)
+		for (int i = i0; i < i1; ++i)
 		{
 			const int idx = tid + THREADS * i;
 			const int row = idx / VPR, col = idx % VPR;
@@ -179,6 +180,7 @@ __global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f16_kernel(const
 			vr[i] = vv;
 		}
 	};
+	auto tile_load = [&](int t) { tile_load_part(t, 0, VPT); };
 	auto tile_store = [&]() {
 #pragma unroll
 		for (int i = 0; i < VPT; ++i)
@@ -196,7 +198,13 @@ __global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f16_kernel(const
 		__syncthreads();                           // the previous tile has been read by everybody
 		tile_store();
 		__syncthreads();
-		if (t < t_last) tile_load(t + 1);          // in flight while this tile is used
+		// At head dimension 256 the next tile's loads are issued two at a time behind the key blocks of the first
+		// product: a wave that issues its eight in one burst is held until the CU's vector memory path (64 bytes per
+		// clock) has taken them, and all eight waves are then held at once.  (With one or two vectors per thread and
+		// matrix the burst is as fast; spreading the V loads over the second product as well was slower.)
+		const bool more = t < t_last;
+		constexpr int kLoadParts = VPT >= 4 ? 4 : 0;
+		if (kLoadParts == 0 && more) tile_load(t + 1);
 
 		// ---- S^T = K Q^T: s[b][kb] = scores of query block b against key block kb ----
 		float4_t s[QB][4];
@@ -213,6 +221,10 @@ __global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f16_kernel(const
 #pragma unroll
 				for (int b = 0; b < QB; ++b)
 					s[b][kb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf, qf[b][st], s[b][kb], 0, 0, 0);
+				if constexpr (kLoadParts > 0)
+				{
+					if (st == KS - 1 && more) tile_load_part(t + 1, kb * (VPT / kLoadParts), (kb + 1) * (VPT / kLoadParts));
+				}
 			}
 
 		// ---- online softmax; p as the second operand of the next product ----
