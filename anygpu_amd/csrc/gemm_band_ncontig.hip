@@ -49,6 +49,9 @@ struct RowBandShape
 	static_assert(!KW || kWaveSize * kAccFloats * 4 <= 2 * kRows * kPitchVecs * 16, "the sums of a wave fit the band buffers");
 };
 
+// 16 bytes at element alignment: weight rows and rows of C need not be multiples of four elements long
+typedef float4_t LooseVec __attribute__((aligned(4)));
+
 template <int MR>
 __device__ __forceinline__ void mma1(float w, float a, typename BandMma<float, MR>::Acc& acc)
 {
@@ -72,8 +75,9 @@ __device__ __forceinline__ void row_band_store(const Acc (*acc)[4][MB], const fl
 		for (int r = 0; r < S::kRegs; ++r)
 		{
 			const int slot = (MR == 16) ? 4 * grp + r : 8 * (r / 4) + 4 * grp + r % 4;
-			const int64_t n = n0 + 4 * slot;
-			if (n >= N) continue;                 // N is a multiple of 4: a vector is inside or outside as a whole
+			int64_t n = n0 + 4 * slot;
+			if (n >= N) continue;
+			if (n + 4 > N) n = N - 4;             // the lane that loaded this slot took the last four columns instead
 			float4_t out;
 #pragma unroll
 			for (int e = 0; e < 4; ++e)
@@ -82,12 +86,12 @@ __device__ __forceinline__ void row_band_store(const Acc (*acc)[4][MB], const fl
 				const float bias_n = (EPI == kEpiBias && bias) ? bias[n + e] : 0.0f;
 				out[e] = finish_sum<EPI>(acc[0][e][b][r], sum2, bias_n, ep_param);
 			}
-			*reinterpret_cast<float4_t*>(C + (int64_t)m * ldc + n) = out;
+			*reinterpret_cast<LooseVec*>(C + (int64_t)m * ldc + n) = out;
 		}
 	}
 }
 
-// C[m, n] = finish(sum_k A[m, k] * B[k, n]), M <= MR * MB, N a multiple of 4.  grid (column tiles, splits of K).
+// C[m, n] = finish(sum_k A[m, k] * B[k, n]), M <= MR * MB, N >= 4.  grid (column tiles, splits of K).
 // KW: the waves of a block share their columns and divide K.  With gridDim.y > 1 the sums go to
 // partial[wave tile][split][lane][register].
 template <int MR, int MB, int EPI, bool KW>
@@ -114,7 +118,8 @@ __global__ __launch_bounds__(kBandThreads) void gemm_band_ncontig_kernel(
 	const int64_t ke_want = kb + (int64_t)chunks_per_split * S::kChunk;
 	const int64_t ke = ke_want < K ? ke_want : K;
 
-	// the four columns of this lane; past the end the last four stand in (never stored)
+	// the four columns of this lane; a vector that would cross or lie past the end of a row is moved back to the last
+	// four columns (crossing: stored there, with the same values as its neighbour's; past: never stored)
 	int64_t n_lane = n0 + 4 * idx;
 	n_lane = n_lane + 4 <= N ? n_lane : N - 4;
 	const float* wcol[S::kMats];
@@ -137,7 +142,7 @@ __global__ __launch_bounds__(kBandThreads) void gemm_band_ncontig_kernel(
 			const int64_t k = k0 + t;
 			const int64_t kk = (decltype(guarded)::value && k >= ke) ? kb : k;
 #pragma unroll
-			for (int w = 0; w < S::kMats; ++w) dst[w][t] = __builtin_nontemporal_load(reinterpret_cast<const Vec*>(wcol[w] + kk * ldb));
+			for (int w = 0; w < S::kMats; ++w) dst[w][t] = __builtin_nontemporal_load(reinterpret_cast<const LooseVec*>(wcol[w] + kk * ldb));
 		}
 	};
 	auto mask_w = [&](Vec (&v)[S::kMats][4], int64_t wstep) {
@@ -321,8 +326,9 @@ __global__ __launch_bounds__(kBandThreads) void gemm_band_ncontig_merge_kernel(
 	const int m = b * MR + lane % MR;
 	const int grp = lane / MR;
 	const int slot = (MR == 16) ? 4 * grp + r : 8 * (r / 4) + 4 * grp + r % 4;
-	const int64_t n = wave_tile * S::kWaveCols + 4 * slot;
+	int64_t n = wave_tile * S::kWaveCols + 4 * slot;
 	if (m >= M || n >= N) return;
+	if (n + 4 > N) n = N - 4;                     // as in row_band_store
 
 	const int64_t stride = (int64_t)kWaveSize * S::kAccFloats;
 	const float* src = partial + (wave_tile * splits * kWaveSize + lane) * S::kAccFloats + q * 4;
@@ -354,7 +360,7 @@ __global__ __launch_bounds__(kBandThreads) void gemm_band_ncontig_merge_kernel(
 		const float bias_n = (EPI == kEpiBias && bias) ? bias[n + e] : 0.0f;
 		out[e] = finish_sum<EPI>(sum[0][e], sum[S::kMats - 1][e], bias_n, ep_param);
 	}
-	*reinterpret_cast<float4_t*>(C + (int64_t)m * ldc + n) = out;
+	*reinterpret_cast<LooseVec*>(C + (int64_t)m * ldc + n) = out;
 }
 
 template <int MR, int MB, int EPI, bool KW>
@@ -396,9 +402,14 @@ bool gemm_band_ncontig_applies(const float* A, const float* B, const float* B2, 
 	if (M < 1 || M > kBandMaxRows || N < 4 || K < 1) return false;
 	if (N / 64 > 0x7FFFFFFFLL) return false;
 	if (M > 32 && (dual || (N < kBandEnoughBlocks * 512 && K < 4096))) return false;
-	// 16-byte loads along K from A, along N from B, 16-byte stores along N
-	return K % 4 == 0 && N % 4 == 0 && lda % 4 == 0 && ldb % 4 == 0 && ldc % 4 == 0 && aligned16(A) && aligned16(B) &&
-	       aligned16(B2) && aligned16(C);
+	// 16-byte loads along K from A; the loads along N from B and the stores to C are 16 bytes at element alignment, and
+	// with N no multiple of four the vector that would cross the end of a row is moved back to end with it
+	(void)B;
+	(void)B2;
+	(void)C;
+	(void)ldb;
+	(void)ldc;
+	return K % 4 == 0 && lda % 4 == 0 && aligned16(A);
 }
 
 hipError_t launch_gemm_band_ncontig(const float* A, const float* B, const float* B2, const float* bias, float* C,

@@ -776,6 +776,36 @@ def test_mm_f32_row_bands_n_contiguous_weights(ops, oracle, m, k, n):
         assert bool((cbuf[:, n:] == -1.0).all())
 
 
+@pytest.mark.parametrize("m,k,n", [(1, 2304, 32003), (8, 2304, 32001), (16, 512, 1001), (32, 1028, 518), (5, 64, 7), (9, 72, 5),
+                                   (24, 4096, 131), (40, 520, 132002), (64, 9216, 2305), (3, 16, 4), (12, 200, 258), (33, 512, 1003)])
+def test_mm_row_bands_rows_of_any_length(ops, oracle, m, k, n):
+    # N no multiple of four: weight rows ([K, N]) and result rows start at any element; small integers, so exact
+    import torch
+    from anygpu_amd import capi
+    a = synth.integers(m + 1, (m, k), -4, 4)
+    b = synth.integers(n + 2, (k, n), -4, 4)
+    want = oracle.tensor_mm(a, b, threads=8)
+    da, db = dev(a), dev(b)
+    assert np.array_equal(host(ops.tensor_mm(da, db)), want)
+    bias = synth.integers(3, (n,), -9, 9)
+    assert np.array_equal(host(ops.tensor_gemm(da, db, dev(bias))), want + bias)
+    # the same weights stored [N, K]: only the rows of the result are unaligned
+    dbt = dev(np.ascontiguousarray(b.T))
+    assert np.array_equal(host(ops.tensor_mm(da, dbt, b_layout=capi.B_COL_MAJOR)), want)
+    if k % 8 == 0 and np.abs(want).max() <= 2048:      # (integers up to 2048 are exact in fp16)
+        a16, bt16 = a.astype(np.float16), np.ascontiguousarray(b.T).astype(np.float16)
+        assert np.array_equal(host(ops.tensor_mm(dev(a16), dev(bt16), b_layout=capi.B_COL_MAJOR)).astype(np.float32), want)
+    # result inside a wider buffer with an odd row length: nothing beyond column n is touched
+    cbuf = torch.full((m, n + 3), -1.0, device="cuda")
+    ops.tensor_mm(da, db, out=cbuf[:, :n])
+    assert np.array_equal(host(cbuf[:, :n]), want)
+    assert bool((cbuf[:, n:] == -1.0).all())
+    cbuf.fill_(-1.0)
+    ops.tensor_mm(da, dbt, out=cbuf[:, :n], b_layout=capi.B_COL_MAJOR)
+    assert np.array_equal(host(cbuf[:, :n]), want)
+    assert bool((cbuf[:, n:] == -1.0).all())
+
+
 def test_mm_row_bands_integer_inputs_exact_streams_and_padded_buffers(ops, oracle):
     import torch
     from anygpu_amd import capi
