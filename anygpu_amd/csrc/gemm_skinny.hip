@@ -152,7 +152,10 @@ __global__ __launch_bounds__(1024) void gemm_skinny_ncontig_kernel(
 	const int col_lane = lane & 31;
 	const int slice = wave * 2 + (lane >> 5);
 	const int64_t col = (int64_t)blockIdx.x * COLS + col_lane * VECN;
-	const int64_t col_load = col < N ? col : N - VECN;      // N is a multiple of VECN
+	// a vector that would cross or lie past the end of a row is moved back to the last VECN columns (crossing: stored
+	// there, with the same values as its neighbour's; past: never stored); loads are made at element alignment
+	typedef vec_t loose_t __attribute__((aligned(sizeof(T))));
+	const int64_t col_load = col + VECN <= N ? col : N - VECN;
 	const T* b_col = B + col_load;
 	const int64_t b2_shift = DUAL ? (B2 - B) : 0;
 
@@ -185,8 +188,8 @@ __global__ __launch_bounds__(1024) void gemm_skinny_ncontig_kernel(
 			{
 				int64_t row = k0 + kk + d * kSkinnySlices;
 				row = row < K ? row : K - 1;                 // the A values of such a row are zero
-				w[d] = __builtin_nontemporal_load(reinterpret_cast<const vec_t*>(b_col + row * ldb));
-				if constexpr (DUAL) w2[d] = __builtin_nontemporal_load(reinterpret_cast<const vec_t*>(b_col + b2_shift + row * ldb));
+				w[d] = __builtin_nontemporal_load(reinterpret_cast<const loose_t*>(b_col + row * ldb));
+				if constexpr (DUAL) w2[d] = __builtin_nontemporal_load(reinterpret_cast<const loose_t*>(b_col + b2_shift + row * ldb));
 			}
 #pragma unroll
 			for (int d = 0; d < kSkinnyDepth; ++d)
@@ -236,7 +239,9 @@ __global__ __launch_bounds__(1024) void gemm_skinny_ncontig_kernel(
 			sum += red(w, 0, m, v, cl);
 			if constexpr (DUAL) sum2 += red(w, NSUM - 1, m, v, cl);
 		}
-		const int64_t n = (int64_t)blockIdx.x * COLS + cl * VECN + v;
+		int64_t n_vec = (int64_t)blockIdx.x * COLS + cl * VECN;
+		if (n_vec < N && n_vec + VECN > N) n_vec = N - VECN;        // as col_load of that lane
+		const int64_t n = n_vec + v;
 		if (m < M && n < N)
 		{
 			const float bias_n = (EPI == kEpiBias && bias) ? bias[n] : 0.0f;
@@ -283,9 +288,9 @@ bool gemm_skinny_applies(const T* A, const T* B, const T* B2, int64_t M, int64_t
 		if (N > (int64_t)0x7FFFFFFF * 4) return false;       // grid of at most N / 4 blocks
 		return K % VEC == 0 && lda % VEC == 0 && ldb % VEC == 0 && aligned_to(A, 16) && aligned_to(B, 16) && aligned_to(B2, 16);
 	}
-	// 4-byte loads along N
+	// 4-byte loads along N at element alignment
 	constexpr int VECN = Vec4B<T>::kLen;
-	return N % VECN == 0 && ldb % VECN == 0 && aligned_to(B, 4) && aligned_to(B2, 4);
+	return N >= VECN;
 }
 
 template <typename T>

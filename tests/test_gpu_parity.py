@@ -777,7 +777,8 @@ def test_mm_f32_row_bands_n_contiguous_weights(ops, oracle, m, k, n):
 
 
 @pytest.mark.parametrize("m,k,n", [(1, 2304, 32003), (8, 2304, 32001), (16, 512, 1001), (32, 1028, 518), (5, 64, 7), (9, 72, 5),
-                                   (24, 4096, 131), (40, 520, 132002), (64, 9216, 2305), (3, 16, 4), (12, 200, 258), (33, 512, 1003)])
+                                   (24, 4096, 131), (40, 520, 132002), (64, 9216, 2305), (3, 16, 4), (12, 200, 258), (33, 512, 1003),
+                                   (2, 256, 1001), (4, 64, 3), (1, 1024, 50257), (3, 72, 2)])
 def test_mm_row_bands_rows_of_any_length(ops, oracle, m, k, n):
     # N no multiple of four: weight rows ([K, N]) and result rows start at any element; small integers, so exact
     import torch
@@ -795,6 +796,7 @@ def test_mm_row_bands_rows_of_any_length(ops, oracle, m, k, n):
     if k % 8 == 0 and np.abs(want).max() <= 2048:      # (integers up to 2048 are exact in fp16)
         a16, bt16 = a.astype(np.float16), np.ascontiguousarray(b.T).astype(np.float16)
         assert np.array_equal(host(ops.tensor_mm(dev(a16), dev(bt16), b_layout=capi.B_COL_MAJOR)).astype(np.float32), want)
+        assert np.array_equal(host(ops.tensor_mm(dev(a16), dev(b.astype(np.float16)))).astype(np.float32), want)
     # result inside a wider buffer with an odd row length: nothing beyond column n is touched
     cbuf = torch.full((m, n + 3), -1.0, device="cuda")
     ops.tensor_mm(da, db, out=cbuf[:, :n])
