@@ -205,7 +205,7 @@ __global__ __launch_bounds__(256) void gemm_f16_split_merge_kernel(
 		out[e] = (half_t)lo[e];
 		out[4 + e] = (half_t)hi[e];
 	}
-	*reinterpret_cast<half8_t*>(C + m * ldc + n) = out;
+	*reinterpret_cast<LooseHalf8*>(C + m * ldc + n) = out;      // rows of C may start at any element
 }
 
 hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K,
@@ -220,10 +220,13 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
 
 	if (batch == 1 && gemm_band_applies<half_t>(a, b, nullptr, c, M, N, K, lda, ldb, ldc, b_layout))
 		return launch_gemm_band<half_t>(a, b, nullptr, nullptr, c, M, N, K, lda, ldb, ldc, 0, 0.0f, stream);
+	// The tile kernels fetch 16-byte chunks of the operands along K (along N for [K, N] weights), which have to be
+	// aligned; C is stored at element alignment, so with k-contiguous weights N, ldc and the start of C are free.
 	const bool aligned = (reinterpret_cast<uintptr_t>(A) % 16 == 0) && (reinterpret_cast<uintptr_t>(B) % 16 == 0) &&
-	                     (reinterpret_cast<uintptr_t>(C) % 16 == 0) && (lda % 8 == 0) && (ldb % 8 == 0) && (ldc % 8 == 0) &&
-	                     (stride_a % 8 == 0) && (stride_b % 8 == 0) && (stride_c % 8 == 0);
-	const bool tiles_ok = aligned && K >= 64 && K % 8 == 0 && N % 8 == 0;
+	                     (lda % 8 == 0) && (ldb % 8 == 0) && (stride_a % 8 == 0) && (stride_b % 8 == 0);
+	const bool tiles_ok = aligned && K >= 64 && K % 8 == 0 && (b_layout == ANYGPU_B_COL_MAJOR || N % 8 == 0);
+	// (the cut along K writes fp32 planes with rows of N: 16-byte stores there)
+	const bool planes_ok = N % 8 == 0;
 	// The skinny kernels: k-contiguous weights with up to 4 rows (from 5 on the band kernels above), and n-contiguous
 	// weights only where the tile kernels cannot go: cut along K those stream [K, N] weights faster at every row
 	// count (9216 x 2304 weights, 4 rows: 17 us against 51 us; 2304 x 256000: 214 us against 247 us).
@@ -288,7 +291,7 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
 		// A single product with fewer blocks than CUs and a deep K is cut along K: every range is a launch "batch"
 		// writing raw fp32 sums to its own [M, N] plane of the stream's workspace, and a merge kernel adds the planes
 		// in order and rounds once.  Priced with the same slab times plus the merge launch and the traffic of the planes.
-		if (fits && batch == 1 && blocks(tile) < 256 && K >= 1024)
+		if (fits && batch == 1 && planes_ok && blocks(tile) < 256 && K >= 1024)
 		{
 			const double slabs = (double)(K / 64);
 			double best = slabs * slab_us(tile, blocks(tile));

@@ -165,7 +165,10 @@ __device__ __forceinline__ half4_t lds_read_transposed_b64(const char* lds_addr)
 // it back row by row, 16 bytes per lane, so that the global stores cover whole rows of the band.
 // The scratch row pitch is 16 bytes more than the row, which spreads the 8-byte writes of the
 // rows over the banks.  The caller guarantees that nobody still reads or fills LDS.
-// RAGGED: rows at or beyond M and 8-column chunks at or beyond N (N a multiple of 8) are not stored.
+// RAGGED: rows at or beyond M and columns at or beyond N are not stored (the 8-column chunk that crosses N goes out
+// element by element).  Stores are made at element alignment: rows of C may start anywhere.
+typedef half8_t LooseHalf8Store __attribute__((aligned(2)));
+
 template <typename Cfg, bool RAGGED>
 __device__ __forceinline__ void store_patch_via_lds(
 	const typename MfmaShape<Cfg::MI>::Acc (&acc)[Cfg::kTilesM][Cfg::kTilesN], char* lds,
@@ -204,7 +207,14 @@ __device__ __forceinline__ void store_patch_via_lds(
 			if ((kRowsPerPass <= MI || row < MI) && inside)
 			{
 				const half8_t v = *reinterpret_cast<const half8_t*>(scratch + row * kPitch + col16 * 16);
-				*reinterpret_cast<half8_t*>(C + (m_base + i * MI + row) * ldc + n_base + col16 * 8) = v;
+				half_t* dst = C + (m_base + i * MI + row) * ldc + n_base + col16 * 8;
+				if (!RAGGED || n_base + col16 * 8 + 8 <= N) *reinterpret_cast<LooseHalf8Store*>(dst) = v;
+				else
+				{
+#pragma unroll
+					for (int e = 0; e < 8; ++e)
+						if (n_base + col16 * 8 + e < N) dst[e] = v[e];
+				}
 			}
 		}
 	}

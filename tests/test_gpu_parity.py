@@ -808,6 +808,24 @@ def test_mm_row_bands_rows_of_any_length(ops, oracle, m, k, n):
     assert bool((cbuf[:, n:] == -1.0).all())
 
 
+@pytest.mark.parametrize("m,k,n", [(512, 256, 1003), (300, 512, 259), (128, 64, 65), (1000, 128, 4097), (65, 192, 7), (257, 320, 511)])
+def test_mm_f16_k_contiguous_weights_result_rows_of_any_length(ops, oracle, m, k, n):
+    # the tile kernels with [N, K] weights: N, the row length of C and its first element are free; integers, exact
+    import torch
+    from anygpu_amd import capi
+    a = synth.integers(m + 5, (m, k), -2, 2)
+    b = synth.integers(n + 6, (k, n), -2, 2)
+    want = oracle.tensor_mm(a, b, threads=8)
+    assert np.abs(want).max() <= 2048
+    da, dbt = dev(a.astype(np.float16)), dev(np.ascontiguousarray(b.T).astype(np.float16))
+    assert np.array_equal(host(ops.tensor_mm(da, dbt, b_layout=capi.B_COL_MAJOR)).astype(np.float32), want)
+    # C inside a wider buffer, starting one element in: nothing around it is touched
+    cbuf = torch.full((m, n + 5), -1.0, device="cuda", dtype=torch.float16)
+    ops.tensor_mm(da, dbt, out=cbuf[:, 1:n + 1], b_layout=capi.B_COL_MAJOR)
+    assert np.array_equal(host(cbuf[:, 1:n + 1]).astype(np.float32), want)
+    assert bool((cbuf[:, :1] == -1.0).all()) and bool((cbuf[:, n + 1:] == -1.0).all())
+
+
 def test_mm_row_bands_integer_inputs_exact_streams_and_padded_buffers(ops, oracle):
     import torch
     from anygpu_amd import capi
