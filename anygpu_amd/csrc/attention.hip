@@ -26,6 +26,7 @@
 // Masks are index rules (causal with the diagonal at n_k - n_q, sliding window); tiles without a
 // visible key are skipped.  A query without any visible key gets zeros.
 #include "device_utils.hpp"
+#include "attention_walk.hpp"
 #include "launch.hpp"
 
 #include <atomic>
@@ -86,7 +87,7 @@ struct AttnLds
 
 // QB: 16-query blocks per wave, WAVES: waves per block; a block owns 16 * QB * WAVES consecutive queries.
 template <int D, bool SOFTCAP, int QB, int WAVES>
-__global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f16_kernel(const AttnArgs a)
+__global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f16_kernel(const AttnArgs a, const AttnWalk walk)
 {
 	constexpr int kAttnQueriesPerBlock = 16 * QB * WAVES;
 	constexpr int THREADS = 64 * WAVES;
@@ -104,9 +105,9 @@ __global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f16_kernel(const
 	const int wave = tid >> 6;
 	const int n = lane & 15;                        // query inside a 16-block (second MFMA operand index)
 	const int g = lane >> 4;                        // lane group: k slots 8 g .. 8 g + 7 of an MFMA
-	const int bh = blockIdx.y;
-	// under the causal rule the last query blocks have the most keys to walk: they are dispatched first
-	const int q0 = (int)(gridDim.x - 1 - blockIdx.x) * kAttnQueriesPerBlock;
+	int bh, q_block;
+	if (!attn_walk_locate(walk, blockIdx.x, bh, q_block)) return;       // the whole block
+	const int q0 = q_block * kAttnQueriesPerBlock;
 	const half_t* qp = a.q + (int64_t)bh * a.n_q * D;
 	const half_t* kp = a.k + (int64_t)(bh / a.q_per_kv) * a.n_k * D;
 	const half_t* vp = a.v + (int64_t)(bh / a.q_per_kv) * a.n_k * D;
@@ -351,8 +352,8 @@ hipError_t launch_variant(const AttnArgs& args, int64_t batch_heads, hipStream_t
 			configured_devices.fetch_or(bit, std::memory_order_relaxed);
 		}
 	}
-	const dim3 grid((unsigned)((args.n_q + kQueriesPerBlock - 1) / kQueriesPerBlock), (unsigned)batch_heads);
-	kernel<<<grid, dim3(64 * WAVES), kLdsBytes, stream>>>(args);
+	const AttnWalk walk = make_attn_walk((args.n_q + kQueriesPerBlock - 1) / kQueriesPerBlock, batch_heads, args.q_per_kv);
+	kernel<<<dim3((unsigned)attn_walk_blocks(walk)), dim3(64 * WAVES), kLdsBytes, stream>>>(args, walk);
 	return hipGetLastError();
 }
 

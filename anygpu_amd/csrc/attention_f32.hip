@@ -23,6 +23,7 @@
 // Masks are index rules (causal with the diagonal at n_k - n_q, sliding window); tiles without a visible key
 // are skipped.  A query without any visible key gets zeros.
 #include "device_utils.hpp"
+#include "attention_walk.hpp"
 #include "launch.hpp"
 
 #include <atomic>
@@ -82,7 +83,7 @@ __device__ __forceinline__ void wait_vmem_all()
 // 8 waves (two per SIMD: one multiplies while the other does its softmax arithmetic) fits the register file.
 // Otherwise the tiles pass through registers into a single stage.
 template <int D, bool SOFTCAP, int WAVES, int KT, bool DIRECT>
-__global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f32_kernel(const AttnArgsF32 a)
+__global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f32_kernel(const AttnArgsF32 a, const AttnWalk walk)
 {
 	constexpr int kKeysPerTile = KT;
 	static_assert(!DIRECT || D == 256, "one load instruction per tile row");
@@ -105,9 +106,9 @@ __global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f32_kernel(const
 	const int wave = tid >> 6;
 	const int n = lane & 15;                        // query inside the wave's block (second MFMA operand index)
 	const int g = lane >> 4;                        // lane group: summation slot g of an MFMA
-	const int bh = blockIdx.y;
-	// under the causal rule the last query blocks have the most keys to walk: they are dispatched first
-	const int q0 = (int)(gridDim.x - 1 - blockIdx.x) * kQueriesPerBlock;
+	int bh, q_block;
+	if (!attn_walk_locate(walk, blockIdx.x, bh, q_block)) return;       // the whole block
+	const int q0 = q_block * kQueriesPerBlock;
 	const float* qp = a.q + (int64_t)bh * a.n_q * D;
 	const float* kp = a.k + (int64_t)(bh / a.q_per_kv) * a.n_k * D;
 	const float* vp = a.v + (int64_t)(bh / a.q_per_kv) * a.n_k * D;
@@ -379,8 +380,8 @@ hipError_t launch_variant_f32(const AttnArgsF32& args, int64_t batch_heads, hipS
 			configured_devices.fetch_or(bit, std::memory_order_relaxed);
 		}
 	}
-	const dim3 grid((unsigned)((args.n_q + kQueriesPerBlock - 1) / kQueriesPerBlock), (unsigned)batch_heads);
-	kernel<<<grid, dim3(64 * WAVES), kLdsBytes, stream>>>(args);
+	const AttnWalk walk = make_attn_walk((args.n_q + kQueriesPerBlock - 1) / kQueriesPerBlock, batch_heads, args.q_per_kv);
+	kernel<<<dim3((unsigned)attn_walk_blocks(walk)), dim3(64 * WAVES), kLdsBytes, stream>>>(args, walk);
 	return hipGetLastError();
 }
 

@@ -94,7 +94,9 @@ int check_attention_shape(int64_t batch_heads, int64_t q_per_kv, int64_t n_q, in
 	if (batch_heads < 0 || n_q < 0 || n_k < 0 || head_dim < 0 || window < 0) return ANYGPU_ERR_BAD_SHAPE;
 	if (q_per_kv < 1 || batch_heads % q_per_kv != 0) return ANYGPU_ERR_BAD_SHAPE;
 	if (!anygpu::sdp_attention_fwd_f16_supports(head_dim)) return ANYGPU_ERR_UNSUPPORTED;
-	if (batch_heads > 65535) return ANYGPU_ERR_TOO_LARGE;                        // one grid row per head
+	if (batch_heads > 65535) return ANYGPU_ERR_TOO_LARGE;                        // (the decode form: one grid row per head)
+	// the fused form's grid: one block per (head, block of 64 queries at least), plus padding of its block walk
+	if (batch_heads * (n_q / 64 + 32) > kMaxIndex32 / 2) return ANYGPU_ERR_TOO_LARGE;
 	// query and key indices, their sums and differences with the window stay inside 32 bits
 	if (n_q > kMaxIndex32 / 4 || n_k > kMaxIndex32 / 4 || window > kMaxIndex32 / 4) return ANYGPU_ERR_TOO_LARGE;
 	return ANYGPU_OK;
