@@ -37,7 +37,7 @@ PEAK_HBM_GBS = 8000.0          # HBM3E
 # write x 1.000); the summaries are under profiles/.
 MEASURED_TRAFFIC_BYTES = {"gemm_f16": 234962687, "gemm_f32": 167994164, "conv1d": 277226336,
                           "softmax_causal": 410887952, "softmax_gemma2": 1514268488,
-                          "attention_gemma2": 689788928, "attention_gemma2_f32": 1426475418, "gated_rmsnorm": 805513216}
+                          "attention_gemma2": 188478908, "attention_gemma2_f32": 887738788, "gated_rmsnorm": 805513216}
 
 
 def parse_args():
