@@ -7,8 +7,8 @@
 // A block of 8 waves owns 128 consecutive queries of one head, 16 per wave (256 and 32 at head
 // dimension 128), so that at least two waves share a SIMD and one wave's MFMAs run under the
 // other's softmax arithmetic.  It walks the visible key range in tiles of 64 keys.  Per tile:
-//   * K and V rows go global -> registers -> LDS (the loads of the next tile are in flight
-//     while this one is being used);
+//   * K and V rows go global -> LDS directly into two stages (head dimension 256 with softcap: global -> registers
+//     -> LDS, one stage); the loads of the next tile are in flight while this one is being used;
 //   * S^T = K Q^T with v_mfma_f32_16x16x32_f16: the K fragment is the first operand, the Q
 //     fragment (kept in registers for the whole kernel) the second, so a lane ends up holding,
 //     for ONE query (lane % 16), the scores of keys 4 (lane / 16) + r of each 16-key block.
@@ -86,15 +86,16 @@ struct AttnLds
 };
 
 // QB: 16-query blocks per wave, WAVES: waves per block; a block owns 16 * QB * WAVES consecutive queries.
-template <int D, bool SOFTCAP, int QB, int WAVES>
+template <int D, bool SOFTCAP, int QB, int WAVES, bool DIRECT>
 __global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f16_kernel(const AttnArgs a, const AttnWalk walk)
 {
 	constexpr int kAttnQueriesPerBlock = 16 * QB * WAVES;
 	constexpr int THREADS = 64 * WAVES;
 	extern __shared__ __align__(16) char lds[];
 	using L = AttnLds<D>;
-	char* k_lds = lds;
-	char* v_lds = lds + kAttnKeysPerTile * L::kPitchK;
+	// (without DIRECT: the one stage; with it these follow the stage of the tile in use)
+	const char* k_lds = lds;
+	const char* v_lds = lds + kAttnKeysPerTile * L::kPitchK;
 	constexpr int KS = D / 32;                      // MFMA steps along the head dimension (q k^T)
 	constexpr int DC = D / 16;                      // 16-wide column blocks of the output
 	constexpr int VPT = kAttnKeysPerTile * D / 8 / THREADS;   // 16-byte vectors per thread per tile and matrix
@@ -188,24 +189,89 @@ __global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f16_kernel(const
 		{
 			const int idx = tid + THREADS * i;
 			const int row = idx / VPR, col = idx % VPR;
-			*reinterpret_cast<float4_t*>(k_lds + row * L::kPitchK + col * 16) = kr[i];
-			*reinterpret_cast<float4_t*>(v_lds + row * L::kPitchV + col * 16) = vr[i];
+			*reinterpret_cast<float4_t*>(lds + row * L::kPitchK + col * 16) = kr[i];
+			*reinterpret_cast<float4_t*>(lds + kAttnKeysPerTile * L::kPitchK + row * L::kPitchV + col * 16) = vr[i];
 		}
 	};
 
-	if (t_first <= t_last) tile_load(t_first);
+	// DIRECT: tiles go global -> LDS without staging registers, into two stages.  A load instruction fills 1 KB of
+	// consecutive LDS; with padded tile rows a few of its lanes land in the padding and fetch a valid chunk nobody
+	// reads.  Load i = wave + WAVES j of a tile: this lane's 16 bytes are the chunk at byte slot_src[j] from the
+	// tile's first key.  Rows past the last key are replaced by the last one (their scores are masked, their p is
+	// 0).  Written as assembly: the compiler would make every transposing LDS read wait for all outstanding
+	// direct loads of the wave; the waits they need are the explicit ones in front of the tile barrier.
+	constexpr int kStageBytes = L::kBytes;
+	constexpr int kLoadsPerTile = kAttnKeysPerTile * L::kPitchK / 1024;
+	constexpr int kSlots = (kLoadsPerTile + WAVES - 1) / WAVES;
+	static_assert(!DIRECT || (L::kPitchK == L::kPitchV && kAttnKeysPerTile * L::kPitchK % 1024 == 0), "whole load instructions");
+	int slot_src[DIRECT ? kSlots : 1];
+	const int wave_s = __builtin_amdgcn_readfirstlane(wave);
+	if constexpr (DIRECT)
+	{
+#pragma unroll
+		for (int j = 0; j < kSlots; ++j)
+		{
+			const int byte = (wave_s + WAVES * j) * 1024 + lane * 16;
+			const int row = (byte / L::kPitchK) % kAttnKeysPerTile;      // (an instruction past the tile is never issued)
+			const int off = byte % L::kPitchK;
+			slot_src[j] = row * (2 * D) + (off < 2 * D ? off : 0);
+		}
+	}
+	const unsigned lds_base = (unsigned)(uintptr_t)(__attribute__((address_space(3))) char*)lds;
+	auto issue_slot = [&](int t, int stage, int j) {
+		const int i = wave_s + WAVES * j;
+		if (WAVES * j + WAVES - 1 < kLoadsPerTile || i < kLoadsPerTile)
+		{
+			int rel = slot_src[DIRECT ? j : 0];
+			if ((t + 1) * kAttnKeysPerTile > a.n_k)                       // block-uniform: the ragged last tile
+			{
+				const int row = rel / (2 * D);
+				const int last = a.n_k - 1 - t * kAttnKeysPerTile;
+				if (row > last) rel -= (row - last) * (2 * D);
+			}
+			const int64_t tile_off = (int64_t)t * (kAttnKeysPerTile * 2 * D);
+			const char* ksrc = (const char*)kp + tile_off;
+			const char* vsrc = (const char*)vp + tile_off;
+			const unsigned m0k = lds_base + stage * kStageBytes + i * 1024;
+			const unsigned m0v = m0k + kAttnKeysPerTile * L::kPitchK;
+			asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(rel), "s"(ksrc), "s"(m0k) : "memory", "m0");
+			asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(rel), "s"(vsrc), "s"(m0v) : "memory", "m0");
+		}
+	};
+
+	if constexpr (DIRECT)
+	{
+		if (t_first <= t_last)
+		{
+#pragma unroll
+			for (int j = 0; j < kSlots; ++j) issue_slot(t_first, 0, j);
+		}
+	}
+	else if (t_first <= t_last) tile_load(t_first);
 	for (int t = t_first; t <= t_last; ++t)
 	{
-		__syncthreads();                           // the previous tile has been read by everybody
-		tile_store();
-		__syncthreads();
+		if constexpr (DIRECT)
+		{
+			// own loads of tile t have landed; behind the barrier everybody's have, and everybody is done with the
+			// stage of tile t - 1, which the loads of tile t + 1 overwrite
+			__builtin_amdgcn_s_waitcnt(0x0F70);        // vmcnt(0)
+			__syncthreads();
+			k_lds = lds + ((t - t_first) & 1) * kStageBytes;
+			v_lds = k_lds + kAttnKeysPerTile * L::kPitchK;
+		}
+		else
+		{
+			__syncthreads();                           // the previous tile has been read by everybody
+			tile_store();
+			__syncthreads();
+		}
 		// At head dimension 256 the next tile's loads are issued two at a time behind the key blocks of the first
 		// product: a wave that issues its eight in one burst is held until the CU's vector memory path (64 bytes per
 		// clock) has taken them, and all eight waves are then held at once.  (With one or two vectors per thread and
 		// matrix the burst is as fast; spreading the V loads over the second product as well was slower.)
 		const bool more = t < t_last;
-		constexpr int kLoadParts = VPT >= 4 ? 4 : 0;
-		if (kLoadParts == 0 && more) tile_load(t + 1);
+		constexpr int kLoadParts = DIRECT ? 0 : VPT >= 4 ? 4 : 0;
+		if (!DIRECT && kLoadParts == 0 && more) tile_load(t + 1);
 
 		// ---- S^T = K Q^T: s[b][kb] = scores of query block b against key block kb ----
 		float4_t s[QB][4];
@@ -225,6 +291,15 @@ __global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f16_kernel(const
 				if constexpr (kLoadParts > 0)
 				{
 					if (st == KS - 1 && more) tile_load_part(t + 1, kb * (VPT / kLoadParts), (kb + 1) * (VPT / kLoadParts));
+				}
+				if constexpr (DIRECT)
+				{
+					// the next tile's loads, spread behind the key blocks of this product
+					if (st == KS - 1 && more)
+					{
+#pragma unroll
+						for (int j = kb; j < kSlots; j += 4) issue_slot(t + 1, (t + 1 - t_first) & 1, j);
+					}
 				}
 			}
 
@@ -329,12 +404,12 @@ __global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f16_kernel(const
 	}
 }
 
-template <int D, bool SOFTCAP, int QB>
+template <int D, bool SOFTCAP, int QB, bool DIRECT = false>
 hipError_t launch_variant(const AttnArgs& args, int64_t batch_heads, hipStream_t stream)
 {
 	constexpr int WAVES = 8;
-	auto kernel = sdp_attention_fwd_f16_kernel<D, SOFTCAP, QB, WAVES>;
-	constexpr int kLdsBytes = AttnLds<D>::kBytes;
+	auto kernel = sdp_attention_fwd_f16_kernel<D, SOFTCAP, QB, WAVES, DIRECT>;
+	constexpr int kLdsBytes = AttnLds<D>::kBytes * (DIRECT ? 2 : 1);
 	constexpr int kQueriesPerBlock = 16 * QB * WAVES;
 	(void)hipGetLastError();
 	if (kLdsBytes > 64 * 1024)
@@ -364,12 +439,24 @@ hipError_t launch_variant(const AttnArgs& args, int64_t batch_heads, hipStream_t
 template <int D>
 hipError_t launch_dim(const AttnArgs& args, bool softcap, int64_t batch_heads, hipStream_t stream)
 {
+	// Tiles go global -> LDS directly (two stages, no staging registers, one barrier per tile) at head_dim 64 and 128
+	// (16 x 4096 x 128 causal: 157 -> 141 us, with softcap 198 -> 182 us; 32 x 2048 x 64: 43 -> 41 us) and, at head_dim
+	// 256, without softcap (8 x 8192 x 256 causal: 384 -> 350 us); with it, where the softmax arithmetic weighs
+	// more, the same form measured 2 % slower than staging through registers.
 	if constexpr (D == 128)
 	{
 		if (batch_heads * ((args.n_q + 255) / 256) >= 256)
-			return softcap ? launch_variant<D, true, 2>(args, batch_heads, stream) : launch_variant<D, false, 2>(args, batch_heads, stream);
+			return softcap ? launch_variant<D, true, 2, true>(args, batch_heads, stream) : launch_variant<D, false, 2, true>(args, batch_heads, stream);
 	}
-	return softcap ? launch_variant<D, true, 1>(args, batch_heads, stream) : launch_variant<D, false, 1>(args, batch_heads, stream);
+	if constexpr (D != 256)
+	{
+		return softcap ? launch_variant<D, true, 1, true>(args, batch_heads, stream) : launch_variant<D, false, 1, true>(args, batch_heads, stream);
+	}
+	else
+	{
+		if (!softcap) return launch_variant<D, false, 1, true>(args, batch_heads, stream);
+		return launch_variant<D, true, 1>(args, batch_heads, stream);
+	}
 }
 
 // ---------------------------------------------------------------------------------------------
