@@ -288,10 +288,6 @@ __global__ __launch_bounds__(256) void softmax_rows_f16_window_kernel(const Soft
 		reg[t] = val;
 	}
 
-	// keys outside the visible interval: exact zeros
-	for (int v = lane; v < v_lo; v += kWaveSize) __builtin_nontemporal_store(zeros, yr + v);
-	for (int v = v_hi + 1 + lane; v < nvec; v += kWaveSize) __builtin_nontemporal_store(zeros, yr + v);
-
 	const float k_in = SOFTCAP ? 2.0f * kLog2e * a.alpha * a.inv_cap : a.alpha_log2e;
 	const float k_cap = a.cap_log2e;
 
@@ -342,6 +338,8 @@ __global__ __launch_bounds__(256) void softmax_rows_f16_window_kernel(const Soft
 	const float S = wave_allreduce(st.s * exp2_shift(st.m, M), SumOp());
 	const float inv = S > 0.0f ? 1.0f / S : 0.0f;
 
+	// the whole row goes out in address order: zeros in front of the visible interval, the values, zeros behind
+	for (int v = lane; v < v_lo; v += kWaveSize) __builtin_nontemporal_store(zeros, yr + v);
 #pragma unroll
 	for (int t = 0; t < VPL; ++t)
 	{
@@ -355,6 +353,7 @@ __global__ __launch_bounds__(256) void softmax_rows_f16_window_kernel(const Soft
 			__builtin_nontemporal_store(out, yr + v);
 		}
 	}
+	for (int v = v_hi + 1 + lane; v < nvec; v += kWaveSize) __builtin_nontemporal_store(zeros, yr + v);
 }
 
 template <int VPL>
