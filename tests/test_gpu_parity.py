@@ -1134,6 +1134,41 @@ def test_sdp_attention_fused_kernel(ops, oracle, case):
     assert rel_l2(got[0], want) <= 2e-3
 
 
+def _random_attention_cases(count, seed):
+    import random
+    rnd = random.Random(seed)
+    cases = []
+    for _ in range(count):
+        d = rnd.choice([64, 128, 256])
+        kv_heads = rnd.choice([1, 2, 3])
+        group = rnd.choice([1, 2, 4, 8])
+        n_q = rnd.choice([1, 17, 64, 100, 129, 300, 512, 777])
+        n_k = n_q + rnd.choice([0, 0, 5, 64, 200])
+        causal = rnd.choice([True, True, False])
+        window = rnd.choice([0, 0, 33, 128, 500]) if causal else 0
+        cap = rnd.choice([0.0, 0.0, 30.0])
+        alpha = rnd.choice([d ** -0.5, 0.0625, -0.05])
+        cases.append((kv_heads * group, kv_heads, n_q, n_k, d, alpha, cap, causal, window))
+    return cases
+
+
+@pytest.mark.parametrize("dtype", ["f16", "f32"])
+def test_sdp_attention_fused_kernel_random_shapes(ops, oracle, dtype):
+    # many (heads, groups, lengths, masks) at random: every (head, query block) of the one-dimensional grid's block
+    # walk has to turn up exactly once, on both tile paths of the fp16 kernel (softcap or not at head dimension 256)
+    for case in _random_attention_cases(24, 7 if dtype == "f16" else 8):
+        heads, kv_heads, n_q, n_k, d, alpha, cap, causal, window = case
+        np_t = np.float16 if dtype == "f16" else np.float32
+        q = synth.normal(1 + n_q, (1, heads, n_q, d)).astype(np_t)
+        k = synth.normal(2 + n_k, (1, kv_heads, n_k, d)).astype(np_t)
+        v = synth.normal(3 + d, (1, kv_heads, n_k, d)).astype(np_t)
+        got = host(ops.sdp_attention_fwd(dev(q), dev(k), dev(v), alpha, softcap=cap, causal=causal, window=window)).astype(np.float32)
+        want = oracle.sdp_attention_rules(*(t.astype(np.float32)[0] for t in (q, k, v)), alpha=alpha, softcap=cap,
+                                          causal=causal, window=window, q_per_kv=heads // kv_heads, threads=8)
+        tol = TOL_F16_ROWOPS * 2 if dtype == "f16" else TOL_F32 * 2
+        assert scaled_rel_err(got[0], want, 1.0) <= tol, case
+
+
 @pytest.mark.parametrize("case", ATTN_CASES)
 def test_sdp_attention_fused_kernel_f32(ops, oracle, case):
     # the float32 form of the same kernel: fp32 operands and the fp32 matrix instruction, fp32 tolerance
