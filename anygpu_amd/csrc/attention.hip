@@ -27,6 +27,7 @@
 // visible key are skipped.  A query without any visible key gets zeros.
 #include "device_utils.hpp"
 #include "attention_walk.hpp"
+#include "attention_split.hpp"
 #include "launch.hpp"
 
 #include <atomic>
@@ -472,9 +473,6 @@ hipError_t launch_dim(const AttnArgs& args, bool softcap, int64_t batch_heads, h
 // splits of a row: M = max m_i, y = sum o_i 2^(m_i - M) / sum l_i 2^(m_i - M).
 // Workspace per (head, split, row): head_dim accumulators + maximum + sum, fp32.
 // ---------------------------------------------------------------------------------------------
-constexpr int kDecodeMaxRows = 16;
-constexpr int kDecodeMaxSplits = 64;
-constexpr int kDecodeTargetWaves = 1024;          // about 4 waves per CU
 
 struct DecodeArgs
 {
@@ -526,53 +524,55 @@ __global__ __launch_bounds__(64) void sdp_decode_partial_kernel(const DecodeArgs
 	const int t0 = da.t_first + split * da.tiles_per_split;
 	int t1 = t0 + da.tiles_per_split - 1;
 	if (t1 > da.t_last) t1 = da.t_last;
-	for (int t = t0; t <= t1; ++t)
-	{
-		const int key0 = t * kAttnKeysPerTile;
-		// K fragments and the V tile: all loads of the tile are issued before the first use
-		half8_t kf[4][KS];
+	// The keys are walked in sub-tiles of 32 (one MFMA step of the second product).  The loads of sub-tile u + 1 (K
+	// fragments straight into operand layout, V vectors for the wave's LDS tile) are in flight while sub-tile u is
+	// multiplied: a wave that loaded, waited and multiplied in turn left the memory system idle half of the time.
+	constexpr int kSub = 32;
+	constexpr int VPS = kSub * D / 8 / 64;                // V vectors per lane per sub-tile
+	half8_t kf[2][2][KS];
+	float4_t vr[2][VPS];
+	auto fetch = [&](half8_t (&kd)[2][KS], float4_t (&vd)[VPS], int key0) {
 #pragma unroll
-		for (int kb = 0; kb < 4; ++kb)
+		for (int kb = 0; kb < 2; ++kb)
 		{
 			const int key = key0 + 16 * kb + n;
 #pragma unroll
 			for (int st = 0; st < KS; ++st)
 			{
 				half8_t val = {};
-				if (key < a.n_k) val = __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(kp + (int64_t)key * D + 32 * st + 8 * g));
-				kf[kb][st] = val;
+				if (key < a.n_k) val = *reinterpret_cast<const half8_t*>(kp + (int64_t)key * D + 32 * st + 8 * g);
+				kd[kb][st] = val;
 			}
 		}
-		float4_t vr[VPT];
 #pragma unroll
-		for (int i = 0; i < VPT; ++i)
+		for (int i = 0; i < VPS; ++i)
 		{
 			const int idx = lane + 64 * i;
 			const int key = key0 + idx / VPR;
 			float4_t val = {};
 			if (key < a.n_k) val = __builtin_nontemporal_load(reinterpret_cast<const float4_t*>(vp + (int64_t)key * D + (idx % VPR) * 8));
-			vr[i] = val;
+			vd[i] = val;
 		}
+	};
+	auto consume = [&](const half8_t (&kd)[2][KS], const float4_t (&vd)[VPS], int key0) {
 #pragma unroll
-		for (int i = 0; i < VPT; ++i)
+		for (int i = 0; i < VPS; ++i)
 		{
 			const int idx = lane + 64 * i;
-			*reinterpret_cast<float4_t*>(lds + (idx / VPR) * kPitchV + (idx % VPR) * 16) = vr[i];
+			*reinterpret_cast<float4_t*>(lds + (idx / VPR) * kPitchV + (idx % VPR) * 16) = vd[i];
 		}
-
-		float4_t s[4];
+		float4_t s[2];
 #pragma unroll
-		for (int kb = 0; kb < 4; ++kb)
+		for (int kb = 0; kb < 2; ++kb)
 		{
 			s[kb] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-			for (int st = 0; st < KS; ++st) s[kb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf[kb][st], qf[st], s[kb], 0, 0, 0);
+			for (int st = 0; st < KS; ++st) s[kb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kd[kb][st], qf[st], s[kb], 0, 0, 0);
 		}
-
-		float z[4][4];
+		float z[2][4];
 		float mt = -INFINITY;
 #pragma unroll
-		for (int kb = 0; kb < 4; ++kb)
+		for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
 			for (int r = 0; r < 4; ++r)
 			{
@@ -586,15 +586,15 @@ __global__ __launch_bounds__(64) void sdp_decode_partial_kernel(const DecodeArgs
 		const float m_safe = (m_new == -INFINITY) ? 0.0f : m_new;
 		const float corr = fast_exp2(m_run - m_safe);
 		float psum = 0.0f;
-		half8_t pf[2];
+		half8_t pf;
 #pragma unroll
-		for (int kb = 0; kb < 4; ++kb)
+		for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
 			for (int r = 0; r < 4; ++r)
 			{
 				const float p = fast_exp2(z[kb][r] - m_safe);
 				psum += p;
-				pf[kb >> 1][4 * (kb & 1) + r] = (half_t)p;
+				pf[4 * kb + r] = (half_t)p;
 			}
 		l_run = l_run * corr + psum;
 		m_run = m_new;
@@ -605,18 +605,31 @@ __global__ __launch_bounds__(64) void sdp_decode_partial_kernel(const DecodeArgs
 		__builtin_amdgcn_s_waitcnt(0xC07F);               // lgkmcnt(0)
 		__builtin_amdgcn_wave_barrier();
 #pragma unroll
-		for (int tt = 0; tt < 2; ++tt)
-#pragma unroll
-			for (int c = 0; c < DC; ++c)
-			{
-				const char* src = lds + (32 * tt + 4 * g + (n >> 2)) * kPitchV + (16 * c + 4 * (n & 3)) * 2;
-				const half4_t lo = lds_read_tr_b64(src);
-				const half4_t hi = lds_read_tr_b64(src + 16 * kPitchV);
-				const half8_t vf = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-				o[c] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf, pf[tt], o[c], 0, 0, 0);
-			}
+		for (int c = 0; c < DC; ++c)
+		{
+			const char* src = lds + (4 * g + (n >> 2)) * kPitchV + (16 * c + 4 * (n & 3)) * 2;
+			const half4_t lo = lds_read_tr_b64(src);
+			const half4_t hi = lds_read_tr_b64(src + 16 * kPitchV);
+			const half8_t vf = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+			o[c] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf, pf, o[c], 0, 0, 0);
+		}
 		__builtin_amdgcn_s_waitcnt(0xC07F);               // the tile has been read before the next one overwrites it
 		__builtin_amdgcn_wave_barrier();
+	};
+	// sub-tiles u0 .. u1, two per step so that the buffer of a sub-tile is a compile-time constant
+	const int u0 = 2 * t0, u1 = 2 * t1 + 1;
+	if (u0 <= u1) fetch(kf[0], vr[0], u0 * kSub);
+	for (int u = u0; u <= u1; u += 2)
+	{
+		if (u + 1 <= u1) fetch(kf[1], vr[1], (u + 1) * kSub);
+		__builtin_amdgcn_sched_barrier(0);
+		consume(kf[0], vr[0], u * kSub);
+		if (u + 1 <= u1)
+		{
+			if (u + 2 <= u1) fetch(kf[0], vr[0], (u + 2) * kSub);
+			__builtin_amdgcn_sched_barrier(0);
+			consume(kf[1], vr[1], (u + 1) * kSub);
+		}
 	}
 
 	// partial result of this split: lane (n, g) holds o[row n][16 c + 4 g .. + 3]
@@ -627,75 +640,13 @@ __global__ __launch_bounds__(64) void sdp_decode_partial_kernel(const DecodeArgs
 	{
 		float* dst = da.ws + (((int64_t)kvh * da.splits + split) * da.rows + n) * (D + 2);
 #pragma unroll
-		for (int c = 0; c < DC; ++c) *reinterpret_cast<float4_t*>(dst + 16 * c + 4 * g) = o[c];
+		for (int c = 0; c < DC; ++c) *reinterpret_cast<WsFloat4*>(dst + 16 * c + 4 * g) = o[c];
 		if (g == 0)
 		{
 			dst[D] = m_run;
 			dst[D + 1] = l;
 		}
 	}
-}
-
-// One block per (key / value head, row), one thread per output column.  The first threads fetch the maxima and
-// sums of the splits in parallel and leave the weights 2^(m_i - M) in LDS; the column sums then run over
-// independent loads.
-template <int D>
-__global__ __launch_bounds__(D) void sdp_decode_merge_kernel(const float* __restrict__ ws, half_t* __restrict__ y, int rows, int splits)
-{
-	__shared__ float weight[kDecodeMaxSplits];
-	__shared__ float total;
-	const int row = blockIdx.x, kvh = blockIdx.y, d = threadIdx.x;
-	const float* base = ws + (((int64_t)kvh * splits) * rows + row) * (D + 2);
-	const int64_t step = (int64_t)rows * (D + 2);
-	if (d < kWaveSize)
-	{
-		// splits <= 64: one split per lane of the first wave
-		const float m = d < splits ? base[d * step + D] : -INFINITY;
-		const float l = d < splits ? base[d * step + D + 1] : 0.0f;
-		const float big = wave_allreduce(m, MaxOp());
-		const float w = fast_exp2(m - (big == -INFINITY ? 0.0f : big));
-		const float sum = wave_allreduce(l * w, SumOp());
-		if (d < splits) weight[d] = w;
-		if (d == 0) total = sum;
-	}
-	__syncthreads();
-	float acc = 0.0f;
-#pragma unroll 8
-	for (int i = 0; i < splits; ++i) acc += base[i * step + d] * weight[i];
-	const float sum = total;
-	y[((int64_t)kvh * rows + row) * D + d] = (half_t)(sum > 0.0f ? acc / sum : 0.0f);
-}
-
-struct DecodePlan
-{
-	int t_first, t_last, splits, tiles_per_split;
-};
-
-DecodePlan plan_decode(int64_t kv_heads, int64_t n_q, int64_t n_k, int causal, int64_t window)
-{
-	// visible key tiles of a group: its first query decides the low end, its last the high end
-	const int64_t diag = n_k - n_q;
-	int64_t key_hi = n_k - 1;
-	if (causal && (n_q - 1) + diag < key_hi) key_hi = (n_q - 1) + diag;
-	int64_t key_lo = 0;
-	if (window > 0 && diag - window + 1 > 0) key_lo = diag - window + 1;
-	DecodePlan p;
-	p.t_first = (int)(key_lo / kAttnKeysPerTile);
-	p.t_last = key_hi >= 0 ? (int)(key_hi / kAttnKeysPerTile) : p.t_first - 1;
-	const int64_t tiles = p.t_last - p.t_first + 1;
-	if (tiles <= 0)
-	{
-		p.splits = 1;
-		p.tiles_per_split = 0;
-		return p;
-	}
-	int64_t want = (kDecodeTargetWaves + kv_heads - 1) / kv_heads;
-	if (want > kDecodeMaxSplits) want = kDecodeMaxSplits;
-	if (want > tiles) want = tiles;
-	if (want < 1) want = 1;
-	p.tiles_per_split = (int)((tiles + want - 1) / want);
-	p.splits = (int)((tiles + p.tiles_per_split - 1) / p.tiles_per_split);
-	return p;
 }
 
 template <int D, bool SOFTCAP>
@@ -706,7 +657,7 @@ hipError_t launch_decode_variant(const DecodeArgs& da, int64_t kv_heads, hipStre
 	sdp_decode_partial_kernel<D, SOFTCAP><<<dim3((unsigned)da.splits, (unsigned)kv_heads), dim3(64), kLdsBytes, stream>>>(da);
 	hipError_t e = hipGetLastError();
 	if (e != hipSuccess) return e;
-	sdp_decode_merge_kernel<D><<<dim3((unsigned)da.rows, (unsigned)kv_heads), dim3(D), 0, stream>>>(da.ws, da.a.y, da.rows, da.splits);
+	sdp_decode_merge_kernel<D, half_t><<<dim3((unsigned)da.rows, (unsigned)kv_heads), dim3(256), 0, stream>>>(da.ws, da.a.y, da.rows, da.splits);
 	return hipGetLastError();
 }
 
@@ -754,7 +705,7 @@ int64_t sdp_attention_decode_workspace_bytes(int64_t batch_heads, int64_t q_per_
 {
 	if (batch_heads == 0 || n_q == 0) return 0;
 	const int64_t kv_heads = batch_heads / q_per_kv;
-	const DecodePlan p = plan_decode(kv_heads, n_q, n_k, causal, window);
+	const DecodePlan p = plan_decode(kv_heads, n_q, n_k, causal, window, kAttnKeysPerTile);
 	return kv_heads * p.splits * (q_per_kv * n_q) * (head_dim + 2) * (int64_t)sizeof(float);
 }
 
@@ -764,7 +715,7 @@ hipError_t launch_sdp_attention_decode_f16(const void* q, const void* k, const v
 {
 	if (batch_heads == 0 || n_q == 0) return hipSuccess;
 	const int64_t kv_heads = batch_heads / q_per_kv;
-	const DecodePlan p = plan_decode(kv_heads, n_q, n_k, causal, window);
+	const DecodePlan p = plan_decode(kv_heads, n_q, n_k, causal, window, kAttnKeysPerTile);
 	DecodeArgs da;
 	da.a.q = static_cast<const half_t*>(q);
 	da.a.k = static_cast<const half_t*>(k);

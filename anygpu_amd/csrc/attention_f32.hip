@@ -24,6 +24,7 @@
 // are skipped.  A query without any visible key gets zeros.
 #include "device_utils.hpp"
 #include "attention_walk.hpp"
+#include "attention_split.hpp"
 #include "launch.hpp"
 
 #include <atomic>
@@ -398,9 +399,6 @@ hipError_t launch_variant_f32(const AttnArgsF32& args, int64_t batch_heads, hipS
 // Workspace per (head, split, row): head_dim accumulators + maximum + sum, fp32.
 // ---------------------------------------------------------------------------------------------
 constexpr int kDecodeKeysPerTile = 16;
-constexpr int kDecodeMaxRows = 16;
-constexpr int kDecodeMaxSplits = 64;
-constexpr int kDecodeTargetWaves = 1024;          // about 4 waves per CU
 
 struct DecodeArgsF32
 {
@@ -526,75 +524,13 @@ __global__ __launch_bounds__(64) void sdp_decode_partial_f32_kernel(const Decode
 		for (int c = 0; c < DC; ++c)
 #pragma unroll
 			for (int r = 0; r < 4; ++r)
-				*reinterpret_cast<float4_t*>(dst + 64 * c + 16 * g + 4 * r) = float4_t{o[c][0][r], o[c][1][r], o[c][2][r], o[c][3][r]};
+				*reinterpret_cast<WsFloat4*>(dst + 64 * c + 16 * g + 4 * r) = float4_t{o[c][0][r], o[c][1][r], o[c][2][r], o[c][3][r]};
 		if (g == 0)
 		{
 			dst[D] = m_run;
 			dst[D + 1] = l;
 		}
 	}
-}
-
-// One block per (key / value head, row), one thread per output column.  The first threads fetch the maxima and
-// sums of the splits in parallel and leave the weights 2^(m_i - M) in LDS; the column sums then run over
-// independent loads.
-template <int D>
-__global__ __launch_bounds__(D) void sdp_decode_merge_f32_kernel(const float* __restrict__ ws, float* __restrict__ y, int rows, int splits)
-{
-	__shared__ float weight[kDecodeMaxSplits];
-	__shared__ float total;
-	const int row = blockIdx.x, kvh = blockIdx.y, d = threadIdx.x;
-	const float* base = ws + (((int64_t)kvh * splits) * rows + row) * (D + 2);
-	const int64_t step = (int64_t)rows * (D + 2);
-	if (d < kWaveSize)
-	{
-		// splits <= 64: one split per lane of the first wave
-		const float m = d < splits ? base[d * step + D] : -INFINITY;
-		const float l = d < splits ? base[d * step + D + 1] : 0.0f;
-		const float big = wave_allreduce(m, MaxOp());
-		const float w = fast_exp2(m - (big == -INFINITY ? 0.0f : big));
-		const float sum = wave_allreduce(l * w, SumOp());
-		if (d < splits) weight[d] = w;
-		if (d == 0) total = sum;
-	}
-	__syncthreads();
-	float acc = 0.0f;
-#pragma unroll 8
-	for (int i = 0; i < splits; ++i) acc += base[i * step + d] * weight[i];
-	const float sum = total;
-	y[((int64_t)kvh * rows + row) * D + d] = sum > 0.0f ? acc / sum : 0.0f;
-}
-
-struct DecodePlanF32
-{
-	int t_first, t_last, splits, tiles_per_split;
-};
-
-DecodePlanF32 plan_decode_f32(int64_t kv_heads, int64_t n_q, int64_t n_k, int causal, int64_t window)
-{
-	// visible key tiles of a group: its first query decides the low end, its last the high end
-	const int64_t diag = n_k - n_q;
-	int64_t key_hi = n_k - 1;
-	if (causal && (n_q - 1) + diag < key_hi) key_hi = (n_q - 1) + diag;
-	int64_t key_lo = 0;
-	if (window > 0 && diag - window + 1 > 0) key_lo = diag - window + 1;
-	DecodePlanF32 p;
-	p.t_first = (int)(key_lo / kDecodeKeysPerTile);
-	p.t_last = key_hi >= 0 ? (int)(key_hi / kDecodeKeysPerTile) : p.t_first - 1;
-	const int64_t tiles = p.t_last - p.t_first + 1;
-	if (tiles <= 0)
-	{
-		p.splits = 1;
-		p.tiles_per_split = 0;
-		return p;
-	}
-	int64_t want = (kDecodeTargetWaves + kv_heads - 1) / kv_heads;
-	if (want > kDecodeMaxSplits) want = kDecodeMaxSplits;
-	if (want > tiles) want = tiles;
-	if (want < 1) want = 1;
-	p.tiles_per_split = (int)((tiles + want - 1) / want);
-	p.splits = (int)((tiles + p.tiles_per_split - 1) / p.tiles_per_split);
-	return p;
 }
 
 template <int D, bool SOFTCAP>
@@ -604,7 +540,7 @@ hipError_t launch_decode_variant_f32(const DecodeArgsF32& da, int64_t kv_heads, 
 	sdp_decode_partial_f32_kernel<D, SOFTCAP><<<dim3((unsigned)da.splits, (unsigned)kv_heads), dim3(64), 0, stream>>>(da);
 	hipError_t e = hipGetLastError();
 	if (e != hipSuccess) return e;
-	sdp_decode_merge_f32_kernel<D><<<dim3((unsigned)da.rows, (unsigned)kv_heads), dim3(D), 0, stream>>>(da.ws, da.a.y, da.rows, da.splits);
+	sdp_decode_merge_kernel<D, float><<<dim3((unsigned)da.rows, (unsigned)kv_heads), dim3(256), 0, stream>>>(da.ws, da.a.y, da.rows, da.splits);
 	return hipGetLastError();
 }
 
@@ -655,7 +591,7 @@ int64_t sdp_attention_decode_f32_workspace_bytes(int64_t batch_heads, int64_t q_
 {
 	if (batch_heads == 0 || n_q == 0) return 0;
 	const int64_t kv_heads = batch_heads / q_per_kv;
-	const DecodePlanF32 p = plan_decode_f32(kv_heads, n_q, n_k, causal, window);
+	const DecodePlan p = plan_decode(kv_heads, n_q, n_k, causal, window, kDecodeKeysPerTile);
 	return kv_heads * p.splits * (q_per_kv * n_q) * (head_dim + 2) * (int64_t)sizeof(float);
 }
 
@@ -665,7 +601,7 @@ hipError_t launch_sdp_attention_decode_f32(const float* q, const float* k, const
 {
 	if (batch_heads == 0 || n_q == 0) return hipSuccess;
 	const int64_t kv_heads = batch_heads / q_per_kv;
-	const DecodePlanF32 p = plan_decode_f32(kv_heads, n_q, n_k, causal, window);
+	const DecodePlan p = plan_decode(kv_heads, n_q, n_k, causal, window, kDecodeKeysPerTile);
 	DecodeArgsF32 da;
 	da.a.q = q;
 	da.a.k = k;

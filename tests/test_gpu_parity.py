@@ -1278,6 +1278,7 @@ DECODE_CASES = [
     (4, 4, 3, 777, 64, 0.125, 30.0, True, 100),
     (2, 1, 1, 63, 128, 0.0884, 0.0, True, 0),             # less than one tile of keys
     (4, 2, 5, 3, 64, 0.125, 0.0, True, 0),                # more queries than keys: the first two see nothing
+    (4, 2, 1, 12000, 64, 0.125, 0.0, True, 0),            # 188 key tiles of 64: more splits than one wave of the merge holds
 ]
 
 
@@ -1324,8 +1325,8 @@ def test_sdp_attention_decode_f32_workspace_and_rejected_arguments(ops):
     from anygpu_amd import capi
     lib = capi.load()
     ws_bytes = lib.anygpu_sdp_attention_decode_f32_workspace_bytes
-    # 4 key / value heads, 2 rows each, 4096 visible keys = 256 tiles of 16 -> 64 splits: 4 * 64 * 2 * (256 + 2) floats
-    assert ws_bytes(8, 2, 1, 8192, 256, 1, 4096) == 4 * 64 * 2 * 258 * 4
+    # 4 key / value heads, 2 rows each, 4096 visible keys = 256 tiles of 16 -> 256 splits: 4 * 256 * 2 * (256 + 2) floats
+    assert ws_bytes(8, 2, 1, 8192, 256, 1, 4096) == 4 * 256 * 2 * 258 * 4
     assert ws_bytes(8, 2, 1, 40, 256, 1, 0) == 4 * 3 * 2 * 258 * 4           # 3 tiles -> 3 splits
     assert ws_bytes(0, 1, 1, 100, 64, 1, 0) == 0
     assert ws_bytes(8, 2, 9, 100, 64, 1, 0) == capi.ANYGPU_ERR_UNSUPPORTED   # 18 rows per key / value head
