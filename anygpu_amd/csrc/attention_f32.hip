@@ -448,18 +448,15 @@ __global__ __launch_bounds__(64) void sdp_decode_partial_f32_kernel(const Decode
 	const int t0 = da.t_first + split * da.tiles_per_split;
 	int t1 = t0 + da.tiles_per_split - 1;
 	if (t1 > da.t_last) t1 = da.t_last;
-	for (int t = t0; t <= t1; ++t)
-	{
-		const int key0 = t * kDecodeKeysPerTile;
-		// all loads of the tile are issued before the first use; keys past the end are replaced by the last one
-		// (their scores are masked)
-		float4_t kf[KS], vf[4][DC];
+	// All loads of a tile are issued before the first use; keys past the end are replaced by the last one (their
+	// scores are masked).  A K load instruction covers half of each 128-byte line it touches, so it stays a plain
+	// load (the other half is the next instruction's); a V load covers whole lines and is non-temporal.
+	auto fetch = [&](float4_t (&kd)[KS], float4_t (&vd)[4][DC], int key0) {
 		{
 			int key = key0 + n;
 			key = key < a.n_k ? key : a.n_k - 1;
 #pragma unroll
-			for (int st = 0; st < KS; ++st)
-				kf[st] = __builtin_nontemporal_load(reinterpret_cast<const float4_t*>(kp + (int64_t)key * D + 16 * st + 4 * g));
+			for (int st = 0; st < KS; ++st) kd[st] = *reinterpret_cast<const float4_t*>(kp + (int64_t)key * D + 16 * st + 4 * g);
 		}
 #pragma unroll
 		for (int r = 0; r < 4; ++r)
@@ -468,14 +465,15 @@ __global__ __launch_bounds__(64) void sdp_decode_partial_f32_kernel(const Decode
 			key = key < a.n_k ? key : a.n_k - 1;
 #pragma unroll
 			for (int c = 0; c < DC; ++c)
-				vf[r][c] = __builtin_nontemporal_load(reinterpret_cast<const float4_t*>(vp + (int64_t)key * D + 64 * c + 4 * n));
+				vd[r][c] = __builtin_nontemporal_load(reinterpret_cast<const float4_t*>(vp + (int64_t)key * D + 64 * c + 4 * n));
 		}
-
+	};
+	auto consume = [&](const float4_t (&kd)[KS], const float4_t (&vd)[4][DC], int key0) {
 		float4_t s = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
 		for (int st = 0; st < KS; ++st)
 #pragma unroll
-			for (int e = 0; e < 4; ++e) s = __builtin_amdgcn_mfma_f32_16x16x4f32(kf[st][e], qf[st][e], s, 0, 0, 0);
+			for (int e = 0; e < 4; ++e) s = __builtin_amdgcn_mfma_f32_16x16x4f32(kd[st][e], qf[st][e], s, 0, 0, 0);
 
 		float z[4];
 		float mt = -INFINITY;
@@ -510,7 +508,35 @@ __global__ __launch_bounds__(64) void sdp_decode_partial_f32_kernel(const Decode
 #pragma unroll
 			for (int c = 0; c < DC; ++c)
 #pragma unroll
-				for (int e = 0; e < 4; ++e) o[c][e] = __builtin_amdgcn_mfma_f32_16x16x4f32(vf[r][c][e], p[r], o[c][e], 0, 0, 0);
+				for (int e = 0; e < 4; ++e) o[c][e] = __builtin_amdgcn_mfma_f32_16x16x4f32(vd[r][c][e], p[r], o[c][e], 0, 0, 0);
+	};
+	if constexpr (D <= 128)
+	{
+		// two register buffers: the loads of tile t + 1 are in flight while tile t is multiplied (at head_dim 256 a
+		// second buffer does not fit beside the accumulators)
+		float4_t kf[2][KS], vf[2][4][DC];
+		if (t0 <= t1) fetch(kf[0], vf[0], t0 * kDecodeKeysPerTile);
+		for (int t = t0; t <= t1; t += 2)
+		{
+			if (t + 1 <= t1) fetch(kf[1], vf[1], (t + 1) * kDecodeKeysPerTile);
+			__builtin_amdgcn_sched_barrier(0);
+			consume(kf[0], vf[0], t * kDecodeKeysPerTile);
+			if (t + 1 <= t1)
+			{
+				if (t + 2 <= t1) fetch(kf[0], vf[0], (t + 2) * kDecodeKeysPerTile);
+				__builtin_amdgcn_sched_barrier(0);
+				consume(kf[1], vf[1], (t + 1) * kDecodeKeysPerTile);
+			}
+		}
+	}
+	else
+	{
+		for (int t = t0; t <= t1; ++t)
+		{
+			float4_t kf[KS], vf[4][DC];
+			fetch(kf, vf, t * kDecodeKeysPerTile);
+			consume(kf, vf, t * kDecodeKeysPerTile);
+		}
 	}
 
 	// partial result of this split: register r of accumulator (c, e) is o[row n][64 c + 16 g + 4 r + e]
