@@ -61,7 +61,7 @@ hipError_t launch_sdp_attention_fwd_f16(const void* q, const void* k, const void
                                         int64_t batch_heads, int64_t q_per_kv, int64_t n_q, int64_t n_k, int64_t head_dim,
                                         float alpha, float softcap, int causal, int64_t window, hipStream_t stream);
 
-// The same in float32 with the fp32 matrix instruction (no decode form).
+// The same in float32 with the fp32 matrix instruction.
 bool sdp_attention_fwd_f32_supports(int64_t head_dim);
 hipError_t launch_sdp_attention_fwd_f32(const float* q, const float* k, const float* v, float* y,
                                         int64_t batch_heads, int64_t q_per_kv, int64_t n_q, int64_t n_k, int64_t head_dim,
@@ -117,7 +117,7 @@ hipError_t launch_gemm_band(const T* A, const T* B, const T* B2, const float* bi
                             int epilogue, float ep_param, hipStream_t stream);
 
 // The same for n-contiguous fp32 weights (row-major B) from one row on: there the band kernel is ahead of the
-// skinny one at every row count (9216 x 2304 weights, 4 rows: 21 us against 50 us).  N must be a multiple of 4.
+// skinny one at every row count (9216 x 2304 weights, 4 rows: 21 us against 50 us).  Any N from 4 on (the last vector of a row is moved back to end at N).
 // `dual`: two weight matrices (kEpiGeluMul), which are limited to 32 rows.
 bool gemm_band_ncontig_applies(const float* A, const float* B, const float* B2, const float* C, int64_t M, int64_t N, int64_t K,
                                int64_t lda, int64_t ldb, int64_t ldc, bool dual);
