@@ -37,7 +37,8 @@ PEAK_HBM_GBS = 8000.0          # HBM3E
 # write x 1.000); the summaries are under profiles/.
 MEASURED_TRAFFIC_BYTES = {"gemm_f16": 234962687, "gemm_f32": 167994164, "conv1d": 277226336,
                           "softmax_causal": 410887952, "softmax_gemma2": 1514268488,
-                          "attention_gemma2": 188478908, "attention_gemma2_f32": 887738788, "gated_rmsnorm": 805513216}
+                          "attention_gemma2": 188478908, "attention_gemma2_f32": 887738788, "gated_rmsnorm": 805513216,
+                          "attention_decode": 144061440}
 
 
 def parse_args():
@@ -47,7 +48,7 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--cpu-seconds", type=float, default=12.0,
                     help="target wall time of the CPU-oracle sample (0 disables the CPU baseline)")
-    ap.add_argument("--only", default="", help="comma list of: gemm,gemm32,conv,softmax,attn,attn32,norm (default: all)")
+    ap.add_argument("--only", default="", help="comma list of: gemm,gemm32,conv,softmax,attn,attn32,decode,norm (default: all)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain device copy of 256 MiB (read 256 MiB + write 256 MiB) a few times, "
                          "as the known-size reference for scaling FETCH_SIZE / WRITE_SIZE counter readings")
@@ -219,6 +220,41 @@ def bench_attention_f32(torch, ops, steps, warmup):
     }
 
 
+def bench_attention_decode(torch, capi, steps, warmup):
+    # One generation step against a long cache: 64 query heads over 8 key / value heads, 32768 cached positions,
+    # head_dim 128, causal.  The split-key decode form through the C ABI with the caller's workspace: two launches
+    # (partial results per split, merge), timed together; the bytes are the K and V caches, read once.
+    h, hkv, n_k, d = 64, 8, 32768, 128
+    lib = capi.load()
+    g = torch.Generator(device="cuda")
+    g.manual_seed(0)
+    q = torch.randn((1, h, 1, d), device="cuda", generator=g).half()
+    k = torch.randn((1, hkv, n_k, d), device="cuda", generator=g).half()
+    v = torch.randn((1, hkv, n_k, d), device="cuda", generator=g).half()
+    y = torch.empty_like(q)
+    need = int(lib.anygpu_sdp_attention_decode_workspace_bytes(h, h // hkv, 1, n_k, d, 1, 0))
+    capi.check("anygpu_sdp_attention_decode_workspace_bytes", min(need, 0))
+    ws = torch.empty(max(need, 16), dtype=torch.uint8, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+    call = (q.data_ptr(), k.data_ptr(), v.data_ptr(), y.data_ptr(), ws.data_ptr(), ws.numel(), h, h // hkv, 1, n_k, d,
+            1.0 / math.sqrt(d), 0.0, 1, 0, stream)
+
+    def step():
+        capi.check("anygpu_sdp_attention_decode_f16", lib.anygpu_sdp_attention_decode_f16(*call))
+
+    host_s, ev_s = timed_region(torch, step, steps, warmup)
+    nbytes = 2 * hkv * n_k * d * 2 + 2 * h * d * 2
+    t = ev_s / steps
+    return {
+        "name": "sdp_attention_decode_f16",
+        "workload": "decode attention fp16 q [1, 64, 1, 128], k / v [1, 8, 32768, 128], x 1/sqrt(128), causal; partial + merge launches",
+        "us_per_launch": t * 1e6, "value": nbytes / t / 1e9, "unit": "GB/s", "dtype": "f16",
+        "roofline": {"bound": "hbm", "achieved": nbytes / t / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": nbytes / t / 1e9 / PEAK_HBM_GBS, "traffic": MEASURED_TRAFFIC_BYTES.get("attention_decode"),
+                     "algorithmic_bytes": nbytes, "workspace_bytes": need},
+    }
+
+
 def bench_gated_rmsnorm(torch, ops, steps, warmup):
     # Zamba2-7B Mamba2 mixer: batch 4 x 4096 positions, d_inner 8192
     rows, cols, nbuf = 4 * 4096, 8192, 3                    # 3 x 805 MB of x + z + y: past the Infinity Cache
@@ -329,6 +365,8 @@ def main():
         kernels.append(bench_attention(torch, ops, max(args.steps // 8, 1), max(args.warmup // 4, 1)))
     if want("attn32"):
         kernels.append(bench_attention_f32(torch, ops, max(args.steps // 16, 1), max(args.warmup // 8, 1)))
+    if want("decode"):
+        kernels.append(bench_attention_decode(torch, capi, args.steps, args.warmup))
     if want("norm"):
         kernels.append(bench_gated_rmsnorm(torch, ops, max(args.steps // 4, 1), max(args.warmup // 4, 1)))
 
