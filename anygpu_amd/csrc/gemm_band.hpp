@@ -13,7 +13,12 @@ constexpr int kBandThreads = 256;
 constexpr int kBandMaxSplits = 32;
 constexpr int64_t kBandEnoughBlocks = 256;        // tiles from which K is not split
 constexpr int64_t kBandWantedBlocks = 512;
-constexpr size_t kBandPartialBytes = (size_t)16 << 20;
+// Workspace of a (device, stream) pair.  The cut along K of the tile kernels prices the traffic of its fp32 planes and
+// uses all of it (2048 x 14336 . 14336 x 4096 fp16: two planes of 32 MB, 244 -> 184 us); the band kernels keep their
+// partial sums within the first kBandPlanBytes: their plan does not price that traffic, and more splits than fit
+// there lost (64 x 4096 . 4096 x 14336 fp32: 83 us with 2 splits, 95 us with 5).
+constexpr size_t kBandPartialBytes = (size_t)64 << 20;
+constexpr size_t kBandPlanBytes = (size_t)16 << 20;
 
 typedef float4_t Vec;      // 16 raw bytes of either element type
 
@@ -91,7 +96,7 @@ inline SplitPlan plan_band_splits(int64_t tiles, int64_t K, int64_t chunk, int64
 		const int64_t min_depth = 32 * rows / elem_bytes;
 		const int64_t min_chunks = (min_depth + chunk - 1) / chunk;
 		if (splits > kchunks / min_chunks) splits = kchunks / min_chunks;
-		const int64_t room = (int64_t)(kBandPartialBytes / ((size_t)tiles * kBandThreads * acc_floats * sizeof(float)));
+		const int64_t room = (int64_t)(kBandPlanBytes / ((size_t)tiles * kBandThreads * acc_floats * sizeof(float)));
 		if (splits > room) splits = room;
 		if (splits < 1) splits = 1;
 	}

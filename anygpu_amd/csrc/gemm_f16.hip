@@ -258,7 +258,7 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
 			return 0.27 * share > 0.43 ? 0.27 * share : 0.43;
 		};
 		const double cost256 = slab_us(256, blocks(256)), cost128 = slab_us(128, blocks(128)), cost64 = slab_us(64, blocks(64));
-		const int64_t tile = (cost256 <= cost128 && cost256 <= cost64) ? 256 : cost128 <= cost64 ? 128 : 64;
+		int64_t tile = (cost256 <= cost128 && cost256 <= cost64) ? 256 : cost128 <= cost64 ? 128 : 64;
 		// A product of 256 x 256 tiles that fills whole rounds of blocks and a bit (320 tiles pay two rounds) is divided
 		// by columns into the whole rounds and the rest, which is launched as a product of its own with its own tile.
 		if (tile == 256 && batch == 1)
@@ -284,28 +284,37 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
 				}
 			}
 		}
-		// one "general" instantiation serves ragged M / N and a K tail alike
-		const bool ragged = (M % tile != 0) || (N % tile != 0) || (K % 64 != 0);
-		const bool fits = ((M + tile - 1) / tile) * ((N + tile - 1) / tile) <= 0x7FFFFFFFLL;
-
 		// A single product with fewer blocks than CUs and a deep K is cut along K: every range is a launch "batch"
 		// writing raw fp32 sums to its own [M, N] plane of the stream's workspace, and a merge kernel adds the planes
-		// in order and rounds once.  Priced with the same slab times plus the merge launch and the traffic of the planes.
-		if (fits && batch == 1 && planes_ok && blocks(tile) < 256 && K >= 1024)
+		// in order and rounds once.  Priced with the same slab times plus the merge launch (4.5 us) and the traffic of
+		// the planes (written under the product, read back by the merge: 8 bytes per sum at 5 TB/s), for every tile
+		// size that leaves CUs idle: a bigger tile cut along K often beats the smaller tile that fills the chip
+		// unsplit (256 x 14336 . 14336 x 4096: 128 x 128 tiles in 4 ranges, 98 -> 50 us, vendor 53;
+		// 1024 x 9216 . 9216 x 2304: 73 -> 60 us, vendor 58 - 64).
+		int64_t splits = 1;
+		const int64_t tile_unsplit = tile;
+		if (batch == 1 && planes_ok && K >= 1024)
 		{
 			const double slabs = (double)(K / 64);
 			double best = slabs * slab_us(tile, blocks(tile));
-			int64_t splits = 1;
 			const int64_t room = (int64_t)(band::kBandPartialBytes / ((size_t)M * N * sizeof(float)));
-			for (int64_t s = 2; s <= 16 && s <= K / 512 && s <= room; ++s)
+			for (const int64_t t : {(int64_t)256, (int64_t)128, (int64_t)64})
 			{
-				const double cost = (slabs / (double)s + 3.0) * slab_us(tile, blocks(tile) * s) + 3.0 + 8.0 * (double)s * (double)M * (double)N / 3.0e6;
-				if (cost < 0.85 * best)
+				if (blocks(t) >= 256) continue;
+				for (int64_t sp = 2; sp <= 16 && sp <= K / 512 && sp <= room; ++sp)
 				{
-					best = cost;
-					splits = s;
+					const double cost = (slabs / (double)sp + 3.0) * slab_us(t, blocks(t) * sp) + 4.5 + 8.0 * (double)sp * (double)M * (double)N / 5.0e6;
+					if (cost < 0.85 * best)
+					{
+						best = cost;
+						splits = sp;
+						tile = t;
+					}
 				}
 			}
+		}
+		if (splits > 1)
+		{
 			int64_t k_split = 0;
 			while (splits > 1)
 			{
@@ -341,6 +350,11 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
 				return hipGetLastError();
 			}
 		}
+		// unsplit (also when the workspace cannot be had, as under stream capture): the tile priced for that.
+		// One "general" instantiation serves ragged M / N and a K tail alike.
+		tile = tile_unsplit;
+		const bool ragged = (M % tile != 0) || (N % tile != 0) || (K % 64 != 0);
+		const bool fits = ((M + tile - 1) / tile) * ((N + tile - 1) / tile) <= 0x7FFFFFFFLL;
 #define ANYGPU_F16_TILE(BT, WM, WN, KN) \
 		return ragged ? launch_gemm_f16_tile<GemmTileCfg<BT, BT, WM, WN, 1, 0, 4, 16, KN>, true, true>(a, b, c, M, N, K, lda, ldb, ldc, stride_a, stride_b, stride_c, batch, stream) \
 		              : launch_gemm_f16_tile<GemmTileCfg<BT, BT, WM, WN, 1, 0, 4, 16, KN>, false, false>(a, b, c, M, N, K, lda, ldb, ldc, stride_a, stride_b, stride_c, batch, stream)
