@@ -21,6 +21,11 @@ namespace anygpu {
 // load at element alignment, the ends of rows element by element, everything outside the operand is zero in LDS.
 // [K, N] weights are transposed on their way into LDS (the MFMA operand is k-contiguous).
 // ---------------------------------------------------------------------------------------------
+// Launches of at most this many 64 x 64 tiles (two per CU) run the form with four LDS stages: alone on its CU a
+// block multiplies a slab in a tenth of the memory latency, and with two stages it advanced one slab per latency
+// (256 x 4096 . 4096 x 4096: 29.9 -> 16.0 us, vendor 19.1).  Denser launches keep two stages: 16 KB per stage, five
+// blocks per CU cover the latency with occupancy (1024 x 2048 . 2048 x 2304: 19.3 us against 21.9 with four stages).
+constexpr int64_t kDeepStageBlocks = 512;
 constexpr int kEdgeTile = 128;
 constexpr int kEdgeDepth = 32;
 constexpr int kEdgePitch = kEdgeDepth + 8;      // halves per LDS row: 80 bytes, keeps 16-byte alignment
@@ -248,14 +253,17 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
 		// Time per 64-deep slab of `nblocks` blocks spread over 256 CUs, in us, from measurements: a 256 x 256 tile takes
 		// 1.56 per round of blocks (4096^3: 256 blocks, 64 slabs, 100 us); the smaller tiles, of which a CU holds several,
 		// follow the average number of blocks per CU with a floor where a lone block waits on latency: 0.75 per block
-		// and CU for 128 x 128 (144 blocks 0.75 - 1.0, 288 1.0, 576 1.7 - 2.0), 0.27 for 64 x 64 with a floor of 0.43.
+		// and CU for 128 x 128 (144 blocks 0.75 - 1.0, 288 1.0, 576 1.7 - 2.0), 0.27 for 64 x 64 in dense launches.
 		// The cheapest launch is taken, the bigger tile on a tie.
 		const auto slab_us = [](int64_t t, int64_t nblocks) {
 			const double rounds = (double)((nblocks + 255) / 256);
 			const double share = nblocks > 256 ? (double)nblocks / 256.0 : 1.0;
 			if (t == 256) return 1.56 * rounds;
 			if (t == 128) return 0.75 * share;
-			return 0.27 * share > 0.43 ? 0.27 * share : 0.43;
+			// four stages (see kDeepStageBlocks): 0.22 where every block has a CU of its own, twice 0.21 where some
+			// CUs hold two (they decide when the launch ends)
+			if (nblocks <= kDeepStageBlocks) return nblocks <= 256 ? 0.22 : 0.42;
+			return 0.27 * share;
 		};
 		const double cost256 = slab_us(256, blocks(256)), cost128 = slab_us(128, blocks(128)), cost64 = slab_us(64, blocks(64));
 		int64_t tile = (cost256 <= cost128 && cost256 <= cost64) ? 256 : cost128 <= cost64 ? 128 : 64;
@@ -327,21 +335,24 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
 			if (planes)
 			{
 				const int64_t step_b = (b_layout == ANYGPU_B_COL_MAJOR) ? k_split : k_split * ldb;
+				const bool deep_stages = blocks(64) * splits <= kDeepStageBlocks;
 				hipError_t err;
-#define ANYGPU_F16_SPLIT(BT, WM, WN, KN) \
-				err = launch_gemm_f16_tile<GemmTileCfg<BT, BT, WM, WN, 1, 0, 4, 16, KN>, true, true, true>( \
+#define ANYGPU_F16_SPLIT(BT, WM, WN, KN, STG) \
+				err = launch_gemm_f16_tile<GemmTileCfg<BT, BT, WM, WN, 1, 0, 4, 16, KN, STG>, true, true, true>( \
 					a, b, c, M, N, K, lda, ldb, ldc, k_split, step_b, 0, splits, stream, planes, k_split)
 				if (b_layout == ANYGPU_B_COL_MAJOR)
 				{
-					if (tile == 256) ANYGPU_F16_SPLIT(256, 2, 4, false);
-					else if (tile == 128) ANYGPU_F16_SPLIT(128, 2, 2, false);
-					else ANYGPU_F16_SPLIT(64, 2, 2, false);
+					if (tile == 256) ANYGPU_F16_SPLIT(256, 2, 4, false, 2);
+					else if (tile == 128) ANYGPU_F16_SPLIT(128, 2, 2, false, 2);
+					else if (deep_stages) ANYGPU_F16_SPLIT(64, 2, 2, false, 4);
+					else ANYGPU_F16_SPLIT(64, 2, 2, false, 2);
 				}
 				else
 				{
-					if (tile == 256) ANYGPU_F16_SPLIT(256, 2, 4, true);
-					else if (tile == 128) ANYGPU_F16_SPLIT(128, 2, 2, true);
-					else ANYGPU_F16_SPLIT(64, 2, 2, true);
+					if (tile == 256) ANYGPU_F16_SPLIT(256, 2, 4, true, 2);
+					else if (tile == 128) ANYGPU_F16_SPLIT(128, 2, 2, true, 2);
+					else if (deep_stages) ANYGPU_F16_SPLIT(64, 2, 2, true, 4);
+					else ANYGPU_F16_SPLIT(64, 2, 2, true, 2);
 				}
 #undef ANYGPU_F16_SPLIT
 				if (err != hipSuccess) return err;
@@ -355,20 +366,23 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
 		tile = tile_unsplit;
 		const bool ragged = (M % tile != 0) || (N % tile != 0) || (K % 64 != 0);
 		const bool fits = ((M + tile - 1) / tile) * ((N + tile - 1) / tile) <= 0x7FFFFFFFLL;
-#define ANYGPU_F16_TILE(BT, WM, WN, KN) \
-		return ragged ? launch_gemm_f16_tile<GemmTileCfg<BT, BT, WM, WN, 1, 0, 4, 16, KN>, true, true>(a, b, c, M, N, K, lda, ldb, ldc, stride_a, stride_b, stride_c, batch, stream) \
-		              : launch_gemm_f16_tile<GemmTileCfg<BT, BT, WM, WN, 1, 0, 4, 16, KN>, false, false>(a, b, c, M, N, K, lda, ldb, ldc, stride_a, stride_b, stride_c, batch, stream)
+		const bool deep_stages = blocks(64) <= kDeepStageBlocks;
+#define ANYGPU_F16_TILE(BT, WM, WN, KN, STG) \
+		return ragged ? launch_gemm_f16_tile<GemmTileCfg<BT, BT, WM, WN, 1, 0, 4, 16, KN, STG>, true, true>(a, b, c, M, N, K, lda, ldb, ldc, stride_a, stride_b, stride_c, batch, stream) \
+		              : launch_gemm_f16_tile<GemmTileCfg<BT, BT, WM, WN, 1, 0, 4, 16, KN, STG>, false, false>(a, b, c, M, N, K, lda, ldb, ldc, stride_a, stride_b, stride_c, batch, stream)
 		if (fits && b_layout == ANYGPU_B_COL_MAJOR)
 		{
-			if (tile == 256) ANYGPU_F16_TILE(256, 2, 4, false);
-			if (tile == 128) ANYGPU_F16_TILE(128, 2, 2, false);
-			ANYGPU_F16_TILE(64, 2, 2, false);
+			if (tile == 256) ANYGPU_F16_TILE(256, 2, 4, false, 2);
+			if (tile == 128) ANYGPU_F16_TILE(128, 2, 2, false, 2);
+			if (deep_stages) ANYGPU_F16_TILE(64, 2, 2, false, 4);
+			ANYGPU_F16_TILE(64, 2, 2, false, 2);
 		}
 		if (fits && b_layout == ANYGPU_B_ROW_MAJOR)
 		{
-			if (tile == 256) ANYGPU_F16_TILE(256, 2, 4, true);
-			if (tile == 128) ANYGPU_F16_TILE(128, 2, 2, true);
-			ANYGPU_F16_TILE(64, 2, 2, true);
+			if (tile == 256) ANYGPU_F16_TILE(256, 2, 4, true, 2);
+			if (tile == 128) ANYGPU_F16_TILE(128, 2, 2, true, 2);
+			if (deep_stages) ANYGPU_F16_TILE(64, 2, 2, true, 4);
+			ANYGPU_F16_TILE(64, 2, 2, true, 2);
 		}
 #undef ANYGPU_F16_TILE
 	}

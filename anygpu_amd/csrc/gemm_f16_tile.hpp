@@ -90,7 +90,7 @@ template <> struct MfmaShape<16>
 	__device__ static __forceinline__ int first_row_of_group(int g, int lane) { (void)g; return 4 * (lane >> 4); }
 };
 
-template <int BM_, int BN_, int WM_, int WN_, int SWZ_, int ILV_ = 0, int GROUP_M_ = 4, int MI_ = 32, bool B_KN_ = false>
+template <int BM_, int BN_, int WM_, int WN_, int SWZ_, int ILV_ = 0, int GROUP_M_ = 4, int MI_ = 32, bool B_KN_ = false, int STAGES_ = 2>
 struct GemmTileCfg
 {
 	// B_KN = false: B stored [N, K] (k-contiguous, like A).  true: B stored [K, N] (the reference
@@ -113,7 +113,12 @@ struct GemmTileCfg
 	static constexpr int kSlabABytes = BM * BK * 2;
 	static constexpr int kSlabBBytes = BN * BK * 2;
 	static constexpr int kStageBytes = kSlabABytes + kSlabBBytes;
-	static constexpr int kLdsBytes = 2 * kStageBytes;
+	// LDS stages: slab t + STAGES - 1 is requested when slab t has been multiplied.  Two are enough where a slab takes
+	// longer to multiply than to fetch (the big tiles); a 64 x 64 tile multiplies a slab in a tenth of the memory
+	// latency and, alone on its CU, advanced one slab per latency with two stages.
+	static constexpr int kStages = STAGES_;
+	static_assert(STAGES_ >= 2, "double buffering at least");
+	static constexpr int kLdsBytes = kStages * kStageBytes;
 	// one direct load instruction of a wave moves 1 KB = 8 slab rows
 	static constexpr int kLoadsA = BM / 8 / kWaves;
 	static constexpr int kLoadsB = BN / 8 / kWaves;
@@ -134,6 +139,14 @@ __device__ __forceinline__ void direct_load_asm(const void* src, const char* lds
 __device__ __forceinline__ void wait_vmem_all()
 {
 	__builtin_amdgcn_s_waitcnt(0x0F70);
+}
+
+// vmcnt(N): all but the N most recent vector memory operations of the wave have completed
+template <int N>
+__device__ __forceinline__ void wait_vmem_but()
+{
+	static_assert(N >= 0 && N < 64, "vmcnt has 6 bits");
+	__builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));
 }
 
 // Swizzle of a [k][n] slab row (B stored [K, N]): 16-byte chunks move in pairs (a transposing read
@@ -342,12 +355,14 @@ __global__ __launch_bounds__(Cfg::kThreads) void gemm_f16_nt_tile_kernel(
 		char* b_lds = a_lds + Cfg::kSlabABytes;
 		const int64_t koff = (int64_t)kt * BK;
 		const int64_t koff_b = Cfg::B_KN ? koff * ldb : koff;
-		if constexpr (Cfg::B_KN)
+		if constexpr (Cfg::B_KN || Cfg::kStages > 2)
 		{
 			// Written as assembly for this layout: in front of a transposing LDS read the compiler waits for ALL of the
 			// wave's outstanding direct loads (it cannot tell that they fill the other stage), which would put the
 			// whole memory latency of the slab just requested in front of the first fragment read behind the barrier.
-			// The waits these loads need are the explicit vmcnt(0) in front of every slab barrier.
+			// The waits these loads need are the explicit vmcnt in front of every slab barrier.  With more than two
+			// stages the same holds for every layout: the compiler turns the vmcnt(n) that leaves the younger slabs in
+			// flight into vmcnt(0) when it knows of direct loads.
 #pragma unroll
 			for (int i = 0; i < Cfg::kLoadsA; ++i)
 				direct_load_asm(a_src[i] + koff, a_lds + 1024 * (wave * Cfg::kLoadsA + i));
@@ -470,15 +485,20 @@ __global__ __launch_bounds__(Cfg::kThreads) void gemm_f16_nt_tile_kernel(
 	// Loads past the last slab are clamped to the last slab: they land in a stage nobody reads
 	// any more, which keeps the loop body free of branches.
 	const int last = ktiles - 1;
-	issue_loads(0, 0);
-	wait_vmem_all();
+	constexpr int S = Cfg::kStages;
+	// loads of the S - 2 slabs that may stay in flight over a slab barrier
+	constexpr int kInFlight = (S - 2) * (Cfg::kLoadsA + Cfg::kLoadsB);
+#pragma unroll
+	for (int i = 0; i < S - 1; ++i) issue_loads(min(i, last), i);
+	wait_vmem_but<kInFlight>();
 	__syncthreads();
-	issue_loads(min(1, last), 1);
+	issue_loads(min(S - 1, last), S - 1);
 	read_frags(0, 0, 0);
 
+	int stage = 0;
 	for (int kt = 0; kt < ktiles; ++kt)
 	{
-		const int stage = kt & 1;
+		const int next_stage = stage + 1 == S ? 0 : stage + 1;
 
 #pragma unroll
 		for (int step = 0; step < Cfg::kSteps - 1; ++step)
@@ -489,14 +509,15 @@ __global__ __launch_bounds__(Cfg::kThreads) void gemm_f16_nt_tile_kernel(
 		}
 
 		// slab t+1 has landed (own loads) and, behind the barrier, everybody's; stage `stage` is free
-		wait_vmem_all();
+		wait_vmem_but<kInFlight>();
 		__syncthreads();
-		issue_loads(min(kt + 2, last), stage);
-		read_frags(0, stage ^ 1, 0);
+		issue_loads(min(kt + S, last), stage);
+		read_frags(0, next_stage, 0);
 		multiply((Cfg::kSteps - 1) & 1);
 		__builtin_amdgcn_sched_group_barrier(kSchedMfma, 1, 0);
 		__builtin_amdgcn_sched_group_barrier(kSchedVmemRead, Cfg::kLoadsA + Cfg::kLoadsB, 0);
 		interleave_reads();
+		stage = next_stage;
 	}
 	if constexpr (KTAIL)
 	{
