@@ -223,8 +223,6 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
 	const half_t* b = static_cast<const half_t*>(B);
 	half_t* c = static_cast<half_t*>(C);
 
-	if (batch == 1 && gemm_band_applies<half_t>(a, b, nullptr, c, M, N, K, lda, ldb, ldc, b_layout))
-		return launch_gemm_band<half_t>(a, b, nullptr, nullptr, c, M, N, K, lda, ldb, ldc, 0, 0.0f, stream);
 	// The tile kernels fetch 16-byte chunks of the operands along K (along N for [K, N] weights), which have to be
 	// aligned; C is stored at element alignment, so with k-contiguous weights N, ldc and the start of C are free.
 	const bool aligned = (reinterpret_cast<uintptr_t>(A) % 16 == 0) && (reinterpret_cast<uintptr_t>(B) % 16 == 0) &&
@@ -232,10 +230,18 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
 	const bool tiles_ok = aligned && K >= 64 && K % 8 == 0 && (b_layout == ANYGPU_B_COL_MAJOR || N % 8 == 0);
 	// (the cut along K writes fp32 planes with rows of N: 16-byte stores there)
 	const bool planes_ok = N % 8 == 0;
-	// The skinny kernels: k-contiguous weights with up to 4 rows (from 5 on the band kernels above), and n-contiguous
-	// weights only where the tile kernels cannot go: cut along K those stream [K, N] weights faster at every row
-	// count (9216 x 2304 weights, 4 rows: 17 us against 51 us; 2304 x 256000: 214 us against 247 us).
-	if (batch == 1 && !(tiles_ok && b_layout == ANYGPU_B_ROW_MAJOR) && gemm_skinny_applies<half_t>(a, b, nullptr, M, N, K, lda, ldb, b_layout))
+	// Few rows.  With four LDS stages and the cut along K the 64 x 64 tiles stream weights as fast as the kernels
+	// written for few rows or faster, although most of their MFMA rows are padding: k-contiguous weights from three
+	// rows on (4 x 14336 . 14336 x 4096: skinny 45 us, tiles 21 us; 8 rows of the same: band 25 us, tiles 21 us;
+	// 32 x 2304 . 2304 x 32003: band 32 us, tiles 23 us; 64 x 4096 . 4096 x 14336: band 30 us, tiles 20 us), and
+	// n-contiguous weights at every row count (9216 x 2304 weights, 4 rows: 17 us against 51 us; 2304 x 256000: 214 us
+	// against 247 us).  One and two rows of k-contiguous weights stay with the skinny kernels (1 x 2304 . 2304 x 256000:
+	// 166 us against 198 us; small weights 9 us against 13 us), and whatever the tile kernels cannot take goes to the
+	// band kernels (5 .. 64 rows) or the skinny ones.
+	const bool tiles_first = tiles_ok && (b_layout == ANYGPU_B_ROW_MAJOR || M >= 3);
+	if (batch == 1 && !tiles_first && gemm_band_applies<half_t>(a, b, nullptr, c, M, N, K, lda, ldb, ldc, b_layout))
+		return launch_gemm_band<half_t>(a, b, nullptr, nullptr, c, M, N, K, lda, ldb, ldc, 0, 0.0f, stream);
+	if (batch == 1 && !tiles_first && gemm_skinny_applies<half_t>(a, b, nullptr, M, N, K, lda, ldb, b_layout))
 		return launch_gemm_skinny<half_t>(a, b, nullptr, nullptr, c, M, N, K, lda, ldb, ldc, b_layout, 0, 0.0f, stream);
 
 	if (tiles_ok)
