@@ -826,6 +826,22 @@ def test_mm_f16_k_contiguous_weights_result_rows_of_any_length(ops, oracle, m, k
     assert bool((cbuf[:, :1] == -1.0).all()) and bool((cbuf[:, n + 1:] == -1.0).all())
 
 
+@pytest.mark.parametrize("m,k,n", [(3, 64, 64), (4, 128, 72), (17, 136, 128), (64, 256, 64), (100, 320, 200), (5, 192, 1000),
+                                   (3, 14336, 4096), (64, 4096, 1024), (256, 2048, 1024), (130, 8200, 512)])
+def test_mm_f16_sparse_launches_of_small_tiles(ops, oracle, m, k, n):
+    # few 64 x 64 tiles: the form with four LDS stages, from one slab (fewer slabs than stages) to hundreds, with a K
+    # tail, and cut along K where the tiles alone leave CUs idle; both weight layouts; integers, so exact
+    from anygpu_amd import capi
+    a = synth.integers(m + 11, (m, k), -1, 1)
+    b = synth.integers(n + 12, (k, n), -1, 1)
+    want = oracle.tensor_mm(a, b, threads=8)
+    assert np.abs(want).max() <= 2048
+    da = dev(a.astype(np.float16))
+    dbt = dev(np.ascontiguousarray(b.T).astype(np.float16))
+    assert np.array_equal(host(ops.tensor_mm(da, dbt, b_layout=capi.B_COL_MAJOR)).astype(np.float32), want)
+    assert np.array_equal(host(ops.tensor_mm(da, dev(b.astype(np.float16)))).astype(np.float32), want)
+
+
 def test_mm_row_bands_integer_inputs_exact_streams_and_padded_buffers(ops, oracle):
     import torch
     from anygpu_amd import capi
