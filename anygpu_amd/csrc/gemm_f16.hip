@@ -318,7 +318,7 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
 				for (int64_t sp = 2; sp <= 16 && sp <= K / 512 && sp <= room; ++sp)
 				{
 					const double cost = (slabs / (double)sp + 3.0) * slab_us(t, blocks(t) * sp) + 4.5 + 8.0 * (double)sp * (double)M * (double)N / 5.0e6;
-					if (cost < 0.85 * best)
+					if (cost < 0.9 * best)
 					{
 						best = cost;
 						splits = sp;
