@@ -498,7 +498,9 @@ __global__ __launch_bounds__(Cfg::kThreads) void gemm_f16_nt_tile_kernel(
 	int stage = 0;
 	for (int kt = 0; kt < ktiles; ++kt)
 	{
-		const int next_stage = stage + 1 == S ? 0 : stage + 1;
+		if constexpr (S == 2) stage = kt & 1;               // (spelled this way the loop of the big tile is two scalar
+		                                                     // instructions and a wait state shorter)
+		const int next_stage = S == 2 ? (stage ^ 1) : (stage + 1 == S ? 0 : stage + 1);
 
 #pragma unroll
 		for (int step = 0; step < Cfg::kSteps - 1; ++step)
@@ -517,7 +519,7 @@ __global__ __launch_bounds__(Cfg::kThreads) void gemm_f16_nt_tile_kernel(
 		__builtin_amdgcn_sched_group_barrier(kSchedMfma, 1, 0);
 		__builtin_amdgcn_sched_group_barrier(kSchedVmemRead, Cfg::kLoadsA + Cfg::kLoadsB, 0);
 		interleave_reads();
-		stage = next_stage;
+		if constexpr (S != 2) stage = next_stage;
 	}
 	if constexpr (KTAIL)
 	{
