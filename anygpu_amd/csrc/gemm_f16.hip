@@ -26,6 +26,7 @@ namespace anygpu {
 // (256 x 4096 . 4096 x 4096: 29.9 -> 16.0 us, vendor 19.1).  Denser launches keep two stages: 16 KB per stage, five
 // blocks per CU cover the latency with occupancy (1024 x 2048 . 2048 x 2304: 19.3 us against 21.9 with four stages).
 constexpr int64_t kDeepStageBlocks = 512;
+constexpr double kRectSlabUs = 0.93;           // 256 x 128 tile in two k groups: us per 64-deep slab and round of blocks
 constexpr int kEdgeTile = 128;
 constexpr int kEdgeDepth = 32;
 constexpr int kEdgePitch = kEdgeDepth + 8;      // halves per LDS row: 80 bytes, keeps 16-byte alignment
@@ -273,6 +274,7 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
 		};
 		const double cost256 = slab_us(256, blocks(256)), cost128 = slab_us(128, blocks(128)), cost64 = slab_us(64, blocks(64));
 		int64_t tile = (cost256 <= cost128 && cost256 <= cost64) ? 256 : cost128 <= cost64 ? 128 : 64;
+
 		// A product of 256 x 256 tiles that fills whole rounds of blocks and a bit (320 tiles pay two rounds) is divided
 		// by columns into the whole rounds and the rest, which is launched as a product of its own with its own tile.
 		if (tile == 256 && batch == 1)
@@ -298,6 +300,16 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
 				}
 			}
 		}
+		// 256 x 128 tiles: eight waves in two groups that split every slab between them (one block per CU).  Per flop
+		// they cost a fifth more than the 256 x 256 tiles and a third less than the 128 x 128 ones, and they are taken
+		// where their number suits the 256 CUs better (2048 x 4096 . 4096 x 4096: 76 -> 62 us, vendor 62;
+		// 1024 x 4096 . 4096 x 6144: 70 -> 55 us, vendor 51).
+		const int64_t blocks_rect = ((M + 255) / 256) * ((N + 127) / 128) * batch;
+		const double cost_rect = kRectSlabUs * (double)((blocks_rect + 255) / 256);
+		const double cost_square = tile == 256 ? cost256 : tile == 128 ? cost128 : cost64;
+		// (against several rounds of 256 x 256 tiles the margin is wider: their later rounds run faster than priced,
+		// 4096 x 4096 . 4096 x 6144, 384 tiles: 176 us where two full rounds would take 200)
+		const bool rect = K >= 512 && cost_rect < (tile == 256 ? 0.85 : 0.95) * cost_square;
 		// A single product with fewer blocks than CUs and a deep K is cut along K: every range is a launch "batch"
 		// writing raw fp32 sums to its own [M, N] plane of the stream's workspace, and a merge kernel adds the planes
 		// in order and rounds once.  Priced with the same slab times plus the merge launch (4.5 us) and the traffic of
@@ -310,7 +322,7 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
 		if (batch == 1 && planes_ok && K >= 1024)
 		{
 			const double slabs = (double)(K / 64);
-			double best = slabs * slab_us(tile, blocks(tile));
+			double best = slabs * (rect ? cost_rect : cost_square);
 			const int64_t room = (int64_t)(band::kBandPartialBytes / ((size_t)M * N * sizeof(float)));
 			for (const int64_t t : {(int64_t)256, (int64_t)128, (int64_t)64})
 			{
@@ -370,6 +382,16 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
 		// unsplit (also when the workspace cannot be had, as under stream capture): the tile priced for that.
 		// One "general" instantiation serves ragged M / N and a K tail alike.
 		tile = tile_unsplit;
+		if (rect && blocks_rect / batch <= 0x7FFFFFFFLL)
+		{
+			const bool ragged_rect = (M % 256 != 0) || (N % 128 != 0) || (K % 64 != 0);
+#define ANYGPU_F16_RECT(KN) \
+			return ragged_rect ? launch_gemm_f16_tile<GemmTileCfg<256, 128, 2, 2, 1, 0, 4, 16, KN, 2, 2>, true, true>(a, b, c, M, N, K, lda, ldb, ldc, stride_a, stride_b, stride_c, batch, stream) \
+			                   : launch_gemm_f16_tile<GemmTileCfg<256, 128, 2, 2, 1, 0, 4, 16, KN, 2, 2>, false, false>(a, b, c, M, N, K, lda, ldb, ldc, stride_a, stride_b, stride_c, batch, stream)
+			if (b_layout == ANYGPU_B_COL_MAJOR) ANYGPU_F16_RECT(false);
+			ANYGPU_F16_RECT(true);
+#undef ANYGPU_F16_RECT
+		}
 		const bool ragged = (M % tile != 0) || (N % tile != 0) || (K % 64 != 0);
 		const bool fits = ((M + tile - 1) / tile) * ((N + tile - 1) / tile) <= 0x7FFFFFFFLL;
 		const bool deep_stages = blocks(64) <= kDeepStageBlocks;

@@ -26,6 +26,7 @@
 #include "device_utils.hpp"
 
 #include <atomic>
+#include <type_traits>
 
 namespace anygpu {
 
@@ -90,7 +91,7 @@ template <> struct MfmaShape<16>
 	__device__ static __forceinline__ int first_row_of_group(int g, int lane) { (void)g; return 4 * (lane >> 4); }
 };
 
-template <int BM_, int BN_, int WM_, int WN_, int SWZ_, int ILV_ = 0, int GROUP_M_ = 4, int MI_ = 32, bool B_KN_ = false, int STAGES_ = 2>
+template <int BM_, int BN_, int WM_, int WN_, int SWZ_, int ILV_ = 0, int GROUP_M_ = 4, int MI_ = 32, bool B_KN_ = false, int STAGES_ = 2, int KGROUPS_ = 1>
 struct GemmTileCfg
 {
 	// B_KN = false: B stored [N, K] (k-contiguous, like A).  true: B stored [K, N] (the reference
@@ -104,7 +105,12 @@ struct GemmTileCfg
 	static constexpr int MI = MI_;            // MFMA tile edge: 32 (x16 deep) or 16 (x32 deep)
 	static constexpr int kKGroups = kWaveSize / MI;       // k groups of 8 halves per instruction
 	static constexpr int kSteps = 8 / kKGroups;           // MFMA steps per 64-deep slab
-	static constexpr int kWaves = WM * WN;
+	// KGROUPS = 2: two groups of WM x WN waves share the tile; group g multiplies step g of the two 32-deep steps of
+	// every slab and the groups' accumulators are added through LDS at the end.  Half the tile area of the plain form
+	// with the same number of waves, the same wave patch and the same LDS bytes per MFMA.
+	static constexpr int kKGroupsOfWaves = KGROUPS_;
+	static_assert(KGROUPS_ == 1 || (KGROUPS_ == 2 && MI_ == 16 && STAGES_ == 2), "two k groups: one step of 32 each");
+	static constexpr int kWaves = WM * WN * KGROUPS_;
 	static constexpr int kThreads = kWaves * kWaveSize;
 	static constexpr int kWaveM = BM / WM;
 	static constexpr int kWaveN = BN / WN;
@@ -304,8 +310,10 @@ __global__ __launch_bounds__(Cfg::kThreads) void gemm_f16_nt_tile_kernel(
 	const int tid = threadIdx.x;
 	const int lane = tid & (kWaveSize - 1);
 	const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // scalar: LDS targets of direct loads stay in SGPRs
-	const int wm = wave / Cfg::WN;
-	const int wn = wave % Cfg::WN;
+	const int wk = wave / (Cfg::WM * Cfg::WN);                   // k group (0 unless the tile has two)
+	const int wave_in_group = wave % (Cfg::WM * Cfg::WN);
+	const int wm = wave_in_group / Cfg::WN;
+	const int wn = wave_in_group % Cfg::WN;
 
 	int tile_m, tile_n;
 	tile_of_block<Cfg::GROUP_M>(blockIdx.x, tiles_m, tiles_n, tile_m, tile_n);
@@ -493,38 +501,63 @@ __global__ __launch_bounds__(Cfg::kThreads) void gemm_f16_nt_tile_kernel(
 	wait_vmem_but<kInFlight>();
 	__syncthreads();
 	issue_loads(min(S - 1, last), S - 1);
-	read_frags(0, 0, 0);
+	read_frags(0, 0, Cfg::kKGroupsOfWaves == 2 ? wk : 0);
 
-	int stage = 0;
-	for (int kt = 0; kt < ktiles; ++kt)
+	if constexpr (Cfg::kKGroupsOfWaves == 2)
 	{
-		if constexpr (S == 2) stage = kt & 1;               // (spelled this way the loop of the big tile is two scalar
-		                                                     // instructions and a wait state shorter)
-		const int next_stage = S == 2 ? (stage ^ 1) : (stage + 1 == S ? 0 : stage + 1);
-
-#pragma unroll
-		for (int step = 0; step < Cfg::kSteps - 1; ++step)
-		{
-			read_frags((step + 1) & 1, stage, step + 1);
-			multiply(step & 1);
+		// one step per wave and slab: the fragments of the next slab are read under the MFMAs of this one; two slabs
+		// per trip so that the fragment buffers are compile-time
+		auto slab = [&](int kt, auto buf) {
+			constexpr int kBuf = decltype(buf)::value;
+			const int stage_now = kt & 1;
+			wait_vmem_but<kInFlight>();
+			__syncthreads();
+			issue_loads(min(kt + S, last), stage_now);
+			read_frags(kBuf ^ 1, stage_now ^ 1, wk);
+			multiply(kBuf);
+			__builtin_amdgcn_sched_group_barrier(kSchedMfma, 1, 0);
+			__builtin_amdgcn_sched_group_barrier(kSchedVmemRead, Cfg::kLoadsA + Cfg::kLoadsB, 0);
 			interleave_reads();
+		};
+		for (int kt = 0; kt < ktiles; kt += 2)
+		{
+			slab(kt, std::integral_constant<int, 0>());
+			if (kt + 1 < ktiles) slab(kt + 1, std::integral_constant<int, 1>());
 		}
+	}
+	else
+	{
+		int stage = 0;
+		for (int kt = 0; kt < ktiles; ++kt)
+		{
+			if constexpr (S == 2) stage = kt & 1;               // (spelled this way the loop of the big tile is two scalar
+			                                                     // instructions and a wait state shorter)
+			const int next_stage = S == 2 ? (stage ^ 1) : (stage + 1 == S ? 0 : stage + 1);
 
-		// slab t+1 has landed (own loads) and, behind the barrier, everybody's; stage `stage` is free
-		wait_vmem_but<kInFlight>();
-		__syncthreads();
-		issue_loads(min(kt + S, last), stage);
-		read_frags(0, next_stage, 0);
-		multiply((Cfg::kSteps - 1) & 1);
-		__builtin_amdgcn_sched_group_barrier(kSchedMfma, 1, 0);
-		__builtin_amdgcn_sched_group_barrier(kSchedVmemRead, Cfg::kLoadsA + Cfg::kLoadsB, 0);
-		interleave_reads();
-		if constexpr (S != 2) stage = next_stage;
+	#pragma unroll
+			for (int step = 0; step < Cfg::kSteps - 1; ++step)
+			{
+				read_frags((step + 1) & 1, stage, step + 1);
+				multiply(step & 1);
+				interleave_reads();
+			}
+
+			// slab t+1 has landed (own loads) and, behind the barrier, everybody's; stage `stage` is free
+			wait_vmem_but<kInFlight>();
+			__syncthreads();
+			issue_loads(min(kt + S, last), stage);
+			read_frags(0, next_stage, 0);
+			multiply((Cfg::kSteps - 1) & 1);
+			__builtin_amdgcn_sched_group_barrier(kSchedMfma, 1, 0);
+			__builtin_amdgcn_sched_group_barrier(kSchedVmemRead, Cfg::kLoadsA + Cfg::kLoadsB, 0);
+			interleave_reads();
+			if constexpr (S != 2) stage = next_stage;
+		}
 	}
 	if constexpr (KTAIL)
 	{
 		constexpr int kStepDepth = 512 / MI;                 // k covered by one MFMA
-		for (int k0 = ktiles * BK; k0 < K; k0 += kStepDepth)
+		for (int k0 = ktiles * BK; k0 < K && wk == 0; k0 += kStepDepth)
 		{
 			const int kk = k0 + 8 * frag_kgroup;             // this lane's 8 consecutive k
 			half8_t at[TM], bt[TN];
@@ -566,10 +599,40 @@ __global__ __launch_bounds__(Cfg::kThreads) void gemm_f16_nt_tile_kernel(
 	// no direct load may still be writing LDS when the scratch is reused or the block retires
 	wait_vmem_all();
 	__syncthreads();
+	if constexpr (Cfg::kKGroupsOfWaves == 2)
+	{
+		// the second group's accumulators reach the first through LDS, half of them at a time (a wave's half is
+		// 16 KB: [register][lane] floats), and only the first group stores
+		static_assert(Cfg::WM * Cfg::WN * (TM * TN / 2) * Shape::kAccRegs * kWaveSize * 4 <= Cfg::kLdsBytes, "half the accumulators fit in LDS");
+		float* red = reinterpret_cast<float*>(lds) + wave_in_group * ((TM * TN / 2) * Shape::kAccRegs * kWaveSize) + lane;
+#pragma unroll
+		for (int half = 0; half < 2; ++half)
+		{
+			if (wk == 1)
+			{
+#pragma unroll
+				for (int t = 0; t < TM * TN / 2; ++t)
+#pragma unroll
+					for (int r = 0; r < Shape::kAccRegs; ++r)
+						red[(t * Shape::kAccRegs + r) * kWaveSize] = acc[(half * (TM * TN / 2) + t) / TN][(half * (TM * TN / 2) + t) % TN][r];
+			}
+			__syncthreads();
+			if (wk == 0)
+			{
+#pragma unroll
+				for (int t = 0; t < TM * TN / 2; ++t)
+#pragma unroll
+					for (int r = 0; r < Shape::kAccRegs; ++r)
+						acc[(half * (TM * TN / 2) + t) / TN][(half * (TM * TN / 2) + t) % TN][r] += red[(t * Shape::kAccRegs + r) * kWaveSize];
+			}
+			__syncthreads();
+		}
+		if (wk == 1) return;
+	}
 	if constexpr (SPLIT)
 		store_patch_f32<Cfg>(acc, planes + (int64_t)blockIdx.y * M * N, m0 + wm * Cfg::kWaveM, n0 + wn * Cfg::kWaveN, lane, M, N);
 	else
-		store_patch_via_lds<Cfg, RAGGED>(acc, lds, C, ldc, m0 + wm * Cfg::kWaveM, n0 + wn * Cfg::kWaveN, wave, lane, M, N);
+		store_patch_via_lds<Cfg, RAGGED>(acc, lds, C, ldc, m0 + wm * Cfg::kWaveM, n0 + wn * Cfg::kWaveN, wave_in_group, lane, M, N);
 }
 
 // planes != NULL (SPLIT): `batch` is the number of K ranges, k_split their depth.

@@ -842,6 +842,22 @@ def test_mm_f16_sparse_launches_of_small_tiles(ops, oracle, m, k, n):
     assert np.array_equal(host(ops.tensor_mm(da, dev(b.astype(np.float16)))).astype(np.float32), want)
 
 
+@pytest.mark.parametrize("m,k,n", [(2048, 512, 4096), (2000, 576, 4000), (1024, 1032, 6100), (1024, 1032, 6144)])
+def test_mm_f16_tiles_of_two_k_groups(ops, oracle, m, k, n):
+    # shapes that take the 256 x 128 tile whose two wave groups split every slab and add up through LDS: whole and
+    # ragged tiles, an odd number of slabs, a K tail; both weight layouts; integers, so exact
+    from anygpu_amd import capi
+    a = synth.integers(m + 21, (m, k), -1, 1)
+    b = synth.integers(n + 22, (k, n), -1, 1)
+    want = oracle.tensor_mm(a, b, threads=8)
+    assert np.abs(want).max() <= 2048
+    da = dev(a.astype(np.float16))
+    dbt = dev(np.ascontiguousarray(b.T).astype(np.float16))
+    assert np.array_equal(host(ops.tensor_mm(da, dbt, b_layout=capi.B_COL_MAJOR)).astype(np.float32), want)
+    if n % 8 == 0:
+        assert np.array_equal(host(ops.tensor_mm(da, dev(b.astype(np.float16)))).astype(np.float32), want)
+
+
 def test_mm_row_bands_integer_inputs_exact_streams_and_padded_buffers(ops, oracle):
     import torch
     from anygpu_amd import capi
