@@ -355,22 +355,22 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
 				const int64_t step_b = (b_layout == ANYGPU_B_COL_MAJOR) ? k_split : k_split * ldb;
 				const bool deep_stages = blocks(64) * splits <= kDeepStageBlocks;
 				hipError_t err;
-#define ANYGPU_F16_SPLIT(BT, WM, WN, KN, STG) \
-				err = launch_gemm_f16_tile<GemmTileCfg<BT, BT, WM, WN, 1, 0, 4, 16, KN, STG>, true, true, true>( \
+#define ANYGPU_F16_SPLIT(BT, WM, WN, KN, STG, KG) \
+				err = launch_gemm_f16_tile<GemmTileCfg<BT, BT, WM, WN, 1, 0, 4, 16, KN, STG, KG>, true, true, true>( \
 					a, b, c, M, N, K, lda, ldb, ldc, k_split, step_b, 0, splits, stream, planes, k_split)
 				if (b_layout == ANYGPU_B_COL_MAJOR)
 				{
-					if (tile == 256) ANYGPU_F16_SPLIT(256, 2, 4, false, 2);
-					else if (tile == 128) ANYGPU_F16_SPLIT(128, 2, 2, false, 2);
-					else if (deep_stages) ANYGPU_F16_SPLIT(64, 2, 2, false, 4);
-					else ANYGPU_F16_SPLIT(64, 2, 2, false, 2);
+					if (tile == 256) ANYGPU_F16_SPLIT(256, 2, 4, false, 2, 1);
+					else if (tile == 128) ANYGPU_F16_SPLIT(128, 2, 2, false, 2, 1);
+					else if (deep_stages) ANYGPU_F16_SPLIT(64, 2, 2, false, 4, 1);
+					else ANYGPU_F16_SPLIT(64, 2, 2, false, 2, 1);
 				}
 				else
 				{
-					if (tile == 256) ANYGPU_F16_SPLIT(256, 2, 4, true, 2);
-					else if (tile == 128) ANYGPU_F16_SPLIT(128, 2, 2, true, 2);
-					else if (deep_stages) ANYGPU_F16_SPLIT(64, 2, 2, true, 4);
-					else ANYGPU_F16_SPLIT(64, 2, 2, true, 2);
+					if (tile == 256) ANYGPU_F16_SPLIT(256, 2, 4, true, 2, 1);
+					else if (tile == 128) ANYGPU_F16_SPLIT(128, 2, 2, true, 2, 1);
+					else if (deep_stages) ANYGPU_F16_SPLIT(64, 2, 2, true, 4, 1);
+					else ANYGPU_F16_SPLIT(64, 2, 2, true, 2, 1);
 				}
 #undef ANYGPU_F16_SPLIT
 				if (err != hipSuccess) return err;
@@ -395,22 +395,22 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
 		const bool ragged = (M % tile != 0) || (N % tile != 0) || (K % 64 != 0);
 		const bool fits = ((M + tile - 1) / tile) * ((N + tile - 1) / tile) <= 0x7FFFFFFFLL;
 		const bool deep_stages = blocks(64) <= kDeepStageBlocks;
-#define ANYGPU_F16_TILE(BT, WM, WN, KN, STG) \
-		return ragged ? launch_gemm_f16_tile<GemmTileCfg<BT, BT, WM, WN, 1, 0, 4, 16, KN, STG>, true, true>(a, b, c, M, N, K, lda, ldb, ldc, stride_a, stride_b, stride_c, batch, stream) \
-		              : launch_gemm_f16_tile<GemmTileCfg<BT, BT, WM, WN, 1, 0, 4, 16, KN, STG>, false, false>(a, b, c, M, N, K, lda, ldb, ldc, stride_a, stride_b, stride_c, batch, stream)
+#define ANYGPU_F16_TILE(BT, WM, WN, KN, STG, KG) \
+		return ragged ? launch_gemm_f16_tile<GemmTileCfg<BT, BT, WM, WN, 1, 0, 4, 16, KN, STG, KG>, true, true>(a, b, c, M, N, K, lda, ldb, ldc, stride_a, stride_b, stride_c, batch, stream) \
+		              : launch_gemm_f16_tile<GemmTileCfg<BT, BT, WM, WN, 1, 0, 4, 16, KN, STG, KG>, false, false>(a, b, c, M, N, K, lda, ldb, ldc, stride_a, stride_b, stride_c, batch, stream)
 		if (fits && b_layout == ANYGPU_B_COL_MAJOR)
 		{
-			if (tile == 256) ANYGPU_F16_TILE(256, 2, 4, false, 2);
-			if (tile == 128) ANYGPU_F16_TILE(128, 2, 2, false, 2);
-			if (deep_stages) ANYGPU_F16_TILE(64, 2, 2, false, 4);
-			ANYGPU_F16_TILE(64, 2, 2, false, 2);
+			if (tile == 256) ANYGPU_F16_TILE(256, 2, 4, false, 2, 1);
+			if (tile == 128) ANYGPU_F16_TILE(128, 2, 2, false, 2, 1);
+			if (deep_stages) ANYGPU_F16_TILE(64, 2, 2, false, 4, 1);
+			ANYGPU_F16_TILE(64, 2, 2, false, 2, 1);
 		}
 		if (fits && b_layout == ANYGPU_B_ROW_MAJOR)
 		{
-			if (tile == 256) ANYGPU_F16_TILE(256, 2, 4, true, 2);
-			if (tile == 128) ANYGPU_F16_TILE(128, 2, 2, true, 2);
-			if (deep_stages) ANYGPU_F16_TILE(64, 2, 2, true, 4);
-			ANYGPU_F16_TILE(64, 2, 2, true, 2);
+			if (tile == 256) ANYGPU_F16_TILE(256, 2, 4, true, 2, 1);
+			if (tile == 128) ANYGPU_F16_TILE(128, 2, 2, true, 2, 1);
+			if (deep_stages) ANYGPU_F16_TILE(64, 2, 2, true, 4, 1);
+			ANYGPU_F16_TILE(64, 2, 2, true, 2, 1);
 		}
 #undef ANYGPU_F16_TILE
 	}
