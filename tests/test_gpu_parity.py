@@ -1076,7 +1076,8 @@ def test_gemm_epilogues_rejected_arguments(ops):
 
 @pytest.mark.parametrize("dtype", ["f16", "f32"])
 @pytest.mark.parametrize("batch,m,k,n", [(1, 64, 64, 64), (5, 16, 128, 16), (32, 256, 64, 256), (3, 100, 37, 60), (8, 128, 256, 64),
-                                         (2, 129, 100, 131), (3, 128, 4096, 128), (2, 300, 1001, 257)])
+                                         (2, 129, 100, 131), (3, 128, 4096, 128), (2, 300, 1001, 257),
+                                         (2, 1000, 520, 4096)])     # (the last: fp16 takes the 256 x 128 tile in two k groups)
 def test_mm_batched(ops, oracle, dtype, batch, m, k, n):
     from anygpu_amd import capi
     np_dt = np.float16 if dtype == "f16" else np.float32
