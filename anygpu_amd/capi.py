@@ -17,6 +17,8 @@ ANYGPU_ERR_BAD_SHAPE = -2
 ANYGPU_ERR_BAD_STRIDE = -3
 ANYGPU_ERR_UNSUPPORTED = -4
 ANYGPU_ERR_TOO_LARGE = -5
+ANYGPU_ERR_SCRATCH_TOO_SMALL = -6
+DECODE_STATIC_SCRATCH_BYTES = 8 * 1024 * 1024
 
 A_ROW_MAJOR = 0
 A_COL_MAJOR = 1
@@ -67,6 +69,9 @@ SIGNATURES = {
     "anygpu_sdp_attention_decode_f16": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64,
                                                 c_int64, c_int64, c_int64, c_int64, c_int64,
                                                 c_float, c_float, c_int, c_int64, c_void_p]),
+    "anygpu_sdp_attention_decode_f16_static": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p,
+                                                       c_int64, c_int64, c_int64, c_int64, c_int64,
+                                                       c_float, c_float, c_int, c_int64, c_void_p]),
     "anygpu_sdp_attention_decode_f32": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64,
                                                 c_int64, c_int64, c_int64, c_int64, c_int64,
                                                 c_float, c_float, c_int, c_int64, c_void_p]),

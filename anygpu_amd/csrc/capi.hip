@@ -4,8 +4,14 @@
 #include "launch.hpp"
 #include "device_utils.hpp"
 
+#include <atomic>
 #include <climits>
 #include <cmath>
+
+// Scratch of anygpu_sdp_attention_decode_f16_static: the per-split partial results of the decode attention, for
+// callers that can hand in no workspace.  Every GPU holds its own copy of the array from the moment the code
+// object is loaded until the process ends.  In host code the name is only a handle for hipGetSymbolAddress.
+static __device__ __align__(256) unsigned char scratch[ANYGPU_DECODE_STATIC_SCRATCH_BYTES];
 
 namespace {
 
@@ -117,6 +123,28 @@ int check_attention(const void* q, const void* k, const void* v, const void* y, 
 	return ANYGPU_OK;
 }
 
+// Device address of `scratch` on the current device, looked up once per device.
+constexpr int kMaxDevices = 64;
+std::atomic<void*> scratch_ptr[kMaxDevices];
+
+hipError_t scratch_of_current_device(void** ptr)
+{
+	int device = 0;
+	hipError_t e = hipGetDevice(&device);
+	if (e != hipSuccess) return e;
+	if (device < 0 || device >= kMaxDevices) return hipErrorInvalidDevice;
+	void* p = scratch_ptr[device].load(std::memory_order_acquire);
+	if (p == nullptr)
+	{
+		e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+		if (e != hipSuccess) return e;
+		if (p == nullptr) return hipErrorInvalidSymbol;
+		scratch_ptr[device].store(p, std::memory_order_release);     // (two threads racing here store the same address)
+	}
+	*ptr = p;
+	return hipSuccess;
+}
+
 template <typename T>
 int conv_update_entry(const void* x, void* state, const void* w, const void* b, void* y,
                       int64_t batch, int64_t chan, int64_t width, void* stream)
@@ -171,6 +199,7 @@ ANYGPU_EXPORT const char* anygpu_hip_error_string(int code)
 	case ANYGPU_ERR_BAD_STRIDE: return "a stride or leading dimension is smaller than the extent it spans";
 	case ANYGPU_ERR_UNSUPPORTED: return "argument value outside what the kernels implement";
 	case ANYGPU_ERR_TOO_LARGE: return "an extent exceeds what the launch geometry can index";
+	case ANYGPU_ERR_SCRATCH_TOO_SMALL: return "the shape needs more scratch than the library's fixed device array holds";
 	default: break;
 	}
 	if (code > 0) return hipGetErrorString(static_cast<hipError_t>(code));
@@ -326,6 +355,24 @@ ANYGPU_EXPORT int anygpu_sdp_attention_decode_f16(const void* q, const void* k, 
 	if (workspace_bytes < need) return ANYGPU_ERR_BAD_SHAPE;
 	if (reinterpret_cast<uintptr_t>(workspace) % 16 != 0) return ANYGPU_ERR_UNSUPPORTED;
 	return (int)anygpu::launch_sdp_attention_decode_f16(q, k, v, y, workspace, batch_heads, q_per_kv, n_q, n_k, head_dim, alpha,
+	                                                    softcap, causal, window, as_stream(stream));
+}
+
+ANYGPU_EXPORT int anygpu_sdp_attention_decode_f16_static(const void* q, const void* k, const void* v, void* y,
+                                                         int64_t batch_heads, int64_t q_per_kv, int64_t n_q, int64_t n_k, int64_t head_dim,
+                                                         float alpha, float softcap, int causal, int64_t window, void* stream)
+{
+	const int rc = check_attention(q, k, v, y, batch_heads, q_per_kv, n_q, n_k, head_dim, alpha, softcap, window);
+	if (rc != ANYGPU_OK) return rc;
+	// (looked up before the early return for empty problems, so that an empty call can serve as the set-up call)
+	void* ws = nullptr;
+	const hipError_t e = scratch_of_current_device(&ws);
+	if (e != hipSuccess) return (int)e;
+	if (batch_heads == 0 || n_q == 0) return ANYGPU_OK;
+	if (!anygpu::sdp_attention_decode_f16_supports(q_per_kv, n_q, head_dim)) return ANYGPU_ERR_UNSUPPORTED;
+	const int64_t need = anygpu::sdp_attention_decode_workspace_bytes(batch_heads, q_per_kv, n_q, n_k, head_dim, causal, window);
+	if (need > (int64_t)ANYGPU_DECODE_STATIC_SCRATCH_BYTES) return ANYGPU_ERR_SCRATCH_TOO_SMALL;
+	return (int)anygpu::launch_sdp_attention_decode_f16(q, k, v, y, ws, batch_heads, q_per_kv, n_q, n_k, head_dim, alpha,
 	                                                    softcap, causal, window, as_stream(stream));
 }
 

@@ -39,6 +39,7 @@ extern "C" {
 #define ANYGPU_ERR_BAD_STRIDE    -3   /* a stride / leading dimension is smaller than the extent it spans */
 #define ANYGPU_ERR_UNSUPPORTED   -4   /* a value outside what the kernels implement (e.g. conv width > 4) */
 #define ANYGPU_ERR_TOO_LARGE     -5   /* an extent exceeds what the launch geometry can index */
+#define ANYGPU_ERR_SCRATCH_TOO_SMALL -6 /* the shape needs more scratch than the library's fixed device array holds */
 
 /* Layout of the left-hand GEMM operand (fp32 entry point only). */
 #define ANYGPU_A_ROW_MAJOR  0   /* A stored [M, K], element (r, l) at A[r * lda + l]  (reference layout) */
@@ -217,6 +218,25 @@ int anygpu_sdp_attention_decode_f16(const void* q, const void* k, const void* v,
                                     void* workspace, int64_t workspace_bytes,
                                     int64_t batch_heads, int64_t q_per_kv, int64_t n_q, int64_t n_k, int64_t head_dim,
                                     float alpha, float softcap, int causal, int64_t window, void* stream);
+
+/*
+ * anygpu_sdp_attention_decode_f16 without the workspace arguments, for callers that cannot allocate device memory
+ * and have no workspace to hand in: code under HIP graph capture, tight serving loops, harnesses that forbid
+ * allocation.  It has no counterpart in the reference.  The partial results pass through a fixed array of
+ * ANYGPU_DECODE_STATIC_SCRATCH_BYTES of device memory that is part of the library's code object (every GPU the
+ * library runs on holds its copy until the process ends); the call allocates and frees nothing.  Same kernels,
+ * same split plan and bit-identical results to anygpu_sdp_attention_decode_f16.  A shape for which
+ * anygpu_sdp_attention_decode_workspace_bytes exceeds the array is rejected with ANYGPU_ERR_SCRATCH_TOO_SMALL and
+ * nothing is launched.  All calls on one GPU share the array: calls on one stream are ordered by the stream, calls
+ * that overlap on different streams of one GPU race.  The first call on a device looks up the array's address
+ * (hipGetSymbolAddress, which may load the code object): make it outside graph capture; a call with
+ * batch_heads = 0 does that and nothing else.
+ */
+#define ANYGPU_DECODE_STATIC_SCRATCH_BYTES (8 * 1024 * 1024)
+
+int anygpu_sdp_attention_decode_f16_static(const void* q, const void* k, const void* v, void* y,
+                                           int64_t batch_heads, int64_t q_per_kv, int64_t n_q, int64_t n_k, int64_t head_dim,
+                                           float alpha, float softcap, int causal, int64_t window, void* stream);
 
 /*
  * The decode form in float32: anygpu_sdp_attention_decode_f16 with fp32 operands and the fp32 matrix instruction
