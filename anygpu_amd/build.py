@@ -33,7 +33,7 @@ KERNEL_SOURCES = ["softmax.hip", "conv1d.hip", "gemm_f16.hip", "gemm_f32.hip", "
 DEVICE_FLAGS = [
     f"--offload-arch={GPU_ARCH}", "-O3", "-std=c++20", "-fPIC", "-fvisibility=hidden",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-    "-Wall", "-Wno-unused-function",
+    "-Wall", "-Wno-unused-function", "-Wno-inline-asm",
 ]
 
 
@@ -59,6 +59,8 @@ def build_kernels(verbose: bool = False) -> Path:
     hipcc = _hipcc()
     OBJ_DIR.mkdir(parents=True, exist_ok=True)
     objs = []
+    # the main loop of the four-wave fp16 GEMM tile is generated text (an inline-assembly block with fixed registers)
+    _run([sys.executable, str(CSRC_DIR / "gen_gemm_f16_ring_loop.py"), str(CSRC_DIR / "gemm_f16_ring_loop.inc")], quiet=not verbose)
 
     def compile_one(src: str) -> Path:
         obj = OBJ_DIR / (Path(src).stem + ".o")

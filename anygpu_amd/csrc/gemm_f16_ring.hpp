@@ -1,0 +1,146 @@
+// 256 x 256 tile of the fp16 GEMM ("NT": A [M, K] and B [N, K], both K-contiguous) for whole tiles: four waves, one per
+// SIMD, each with a 128 x 128 patch of C in 256 accumulator registers, v_mfma_f32_16x16x32_f16.
+//
+// Against the eight-wave tile kernel (128 x 64 patches) a patch of 128 x 128 needs a third fewer LDS bytes per MFMA, and
+// under this product the MI355X is power-limited: the bytes saved come back as clock.  One wave per SIMD has nobody to
+// hide its stalls, so the main loop is one block of assembly with fixed registers (gemm_f16_ring_loop.inc, written by
+// gen_gemm_f16_ring_loop.py, which also describes the register plan, the five-unit LDS ring and the schedule).  Measured
+// in that loop at 4096^3: the matrix cores busy 94 - 95 % of the cycles at the 1.6 GHz the part sustains under it.
+#pragma once
+
+#include "gemm_f16_tile.hpp"
+
+namespace anygpu {
+
+typedef float float32x_t __attribute__((ext_vector_type(32)));
+
+struct GemmRingCfg
+{
+	static constexpr int BM = 256, BN = 256, BK = 64, MI = 16;
+	static constexpr int kThreads = 256, kWaves = 4;
+	static constexpr int kUnitBytes = 256 * 128;          // one operand, one 64-deep slab
+	static constexpr int kUnits = 5;
+	static constexpr int kLdsBytes = kUnits * kUnitBytes;
+	static constexpr int kWaveM = 128, kWaveN = 128, kTilesM = 8, kTilesN = 8;
+	static constexpr int WM = 2, WN = 2;
+};
+
+// blockIdx.y walks a batch of independent products that share the shape.  M and N multiples of 256, K of 64.
+__global__ __launch_bounds__(256) void gemm_f16_nt_ring_kernel(
+	const half_t* __restrict__ A, const half_t* __restrict__ B, half_t* __restrict__ C,
+	int K, int64_t lda, int64_t ldb, int64_t ldc, int tiles_m, int tiles_n,
+	int64_t stride_a, int64_t stride_b, int64_t stride_c)
+{
+	using Cfg = GemmRingCfg;
+	extern __shared__ __align__(1024) char lds[];
+
+	A += (int64_t)blockIdx.y * stride_a;
+	B += (int64_t)blockIdx.y * stride_b;
+	C += (int64_t)blockIdx.y * stride_c;
+	const int tid = threadIdx.x;
+	const int lane = tid & 63;
+	const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+	const int wm = wave >> 1, wn = wave & 1;
+
+	int tile_m, tile_n;
+	tile_of_block<4>(blockIdx.x, tiles_m, tiles_n, tile_m, tile_n);
+	const int64_t m0 = (int64_t)tile_m * 256;
+	const int64_t n0 = (int64_t)tile_n * 256;
+
+	// Direct loads.  A unit row is 64 halves = 128 bytes = eight 16-byte chunks; chunk c of row r sits at position
+	// c ^ ((r >> 1) & 7).  One instruction fills 8 rows: lane -> row lane / 8, position lane % 8.  Instruction q of this
+	// wave covers rows 64 wave + 8 q .. + 7 of the operand's 256; the swizzle of those rows is 4 (q & 1) + lane / 16,
+	// so the even and the odd instructions have one offset each and instruction q + 2 lies 16 rows further on.
+	const unsigned ld_row = lane >> 3, ld_pos = lane & 7, ld_hi = lane >> 4;
+	const unsigned a_voff_e = (unsigned)(ld_row * lda + (ld_pos ^ ld_hi) * 8) * 2;
+	const unsigned a_voff_o = (unsigned)((8 + ld_row) * lda + (ld_pos ^ (4 + ld_hi)) * 8) * 2;
+	const unsigned b_voff_e = (unsigned)(ld_row * ldb + (ld_pos ^ ld_hi) * 8) * 2;
+	const unsigned b_voff_o = (unsigned)((8 + ld_row) * ldb + (ld_pos ^ (4 + ld_hi)) * 8) * 2;
+	const uintptr_t a_wave = reinterpret_cast<uintptr_t>(A + (m0 + 64 * wave) * lda);
+	const uintptr_t b_wave = reinterpret_cast<uintptr_t>(B + (n0 + 64 * wave) * ldb);
+	const unsigned lds0 = (unsigned)(uintptr_t)(const __attribute__((address_space(3))) char*)lds;
+	const unsigned wave_share = wave * 8192;               // the wave's 64 rows inside a unit
+	const unsigned lds_wave = lds0 + wave_share;
+	const int slabs = K / 64;
+
+	// Fragments: lane -> row lane % 16 of its MFMA tile, k group lane / 16 (8 halves) of the 32-deep step.  Relative to
+	// the unit offsets the loop keeps, which include the wave's share.
+	const unsigned frag_row = lane & 15;
+	const unsigned frag_chunk = (lane >> 4) ^ ((frag_row >> 1) & 7);
+	const unsigned a_addr = (wm * 128 + frag_row) * 128 + frag_chunk * 16 - wave_share;
+	const unsigned b_addr = (wn * 128 + frag_row) * 128 + frag_chunk * 16 - wave_share;
+
+	// The accumulators leave the block as eight vectors of 32 registers pinned to a[0:255]: row i of the patch's MFMA
+	// tiles in vector i.
+	float32x_t r0, r1, r2, r3, r4, r5, r6, r7;
+	asm volatile(
+#include "gemm_f16_ring_loop.inc"
+		: "={a[0:31]}"(r0), "={a[32:63]}"(r1), "={a[64:95]}"(r2), "={a[96:127]}"(r3),
+		  "={a[128:159]}"(r4), "={a[160:191]}"(r5), "={a[192:223]}"(r6), "={a[224:255]}"(r7)
+		: [avoffe] "v"(a_voff_e), [avoffo] "v"(a_voff_o), [bvoffe] "v"(b_voff_e), [bvoffo] "v"(b_voff_o),
+		  [aaddr] "v"(a_addr), [baddr] "v"(b_addr),
+		  [arow16] "s"((unsigned)(32 * lda)), [brow16] "s"((unsigned)(32 * ldb)),
+		  [abaselo] "s"((unsigned)a_wave), [abasehi] "s"((unsigned)(a_wave >> 32)),
+		  [bbaselo] "s"((unsigned)b_wave), [bbasehi] "s"((unsigned)(b_wave >> 32)),
+		  [ldsw] "s"(lds_wave), [slabs] "s"(slabs)
+		:
+		  "v96", "v97", "v98", "v99", "v100", "v101", "v102", "v103", "v104", "v105", "v106", "v107", "v108", "v109",
+		  "v110", "v111", "v112", "v113", "v114", "v115", "v116", "v117", "v118", "v119", "v120", "v121", "v122", "v123",
+		  "v124", "v125", "v126", "v127", "v128", "v129", "v130", "v131", "v132", "v133", "v134", "v135", "v136", "v137",
+		  "v138", "v139", "v140", "v141", "v142", "v143", "v144", "v145", "v146", "v147", "v148", "v149", "v150", "v151",
+		  "v152", "v153", "v154", "v155", "v156", "v157", "v158", "v159", "v160", "v161", "v162", "v163", "v164", "v165",
+		  "v166", "v167", "v168", "v169", "v170", "v171", "v172", "v173", "v174", "v175", "v176", "v177", "v178", "v179",
+		  "v180", "v181", "v182", "v183", "v184", "v185", "v186", "v187", "v188", "v189", "v190", "v191", "v192", "v193",
+		  "v194", "v195", "v196", "v197", "v198", "v199", "v200", "v201", "v202", "v203", "v204", "v205", "v206", "v207",
+		  "v208", "v209", "v210", "v211", "v212", "v213", "v214", "v215", "v216", "v217", "v218", "v219", "v220", "v221",
+		  "v222", "v223", "v224", "v225", "v226", "v227", "v228", "v229", "v230", "v231", "v232", "v233", "v234", "v235",
+		  "v236", "v237", "v238", "v239", "v240", "v241", "v242", "v243", "v244", "v245", "v246", "v247", "v248", "v249",
+		  "v250", "v251", "v252", "v253", "v254", "v255", "s60", "s61", "s62", "s63", "s64", "s65", "s66", "s67", "s68",
+		  "s69", "s70", "s71", "s72", "scc", "m0", "memory");
+
+	float4_t acc[8][8];
+	const float32x_t* rows[8] = {&r0, &r1, &r2, &r3, &r4, &r5, &r6, &r7};
+#pragma unroll
+	for (int i = 0; i < 8; ++i)
+#pragma unroll
+		for (int j = 0; j < 8; ++j)
+			acc[i][j] = float4_t{(*rows[i])[4 * j], (*rows[i])[4 * j + 1], (*rows[i])[4 * j + 2], (*rows[i])[4 * j + 3]};
+	store_patch_via_lds<Cfg, false>(acc, lds, C, ldc, m0 + wm * 128, n0 + wn * 128, wave, lane, 0, 0);
+}
+
+// What the kernel assumes, checked on the host before every launch: whole tiles, whole slabs, 16-byte aligned operand
+// rows, and operands small enough for the 32-bit lane offsets (a wave's 64 rows) and the 32-bit row steps.
+inline bool gemm_f16_ring_applies(const half_t* A, const half_t* B, int64_t M, int64_t N, int64_t K,
+                                  int64_t lda, int64_t ldb, int64_t stride_a, int64_t stride_b, int64_t batch)
+{
+	const bool aligned = reinterpret_cast<uintptr_t>(A) % 16 == 0 && reinterpret_cast<uintptr_t>(B) % 16 == 0 &&
+	                     lda % 8 == 0 && ldb % 8 == 0 && stride_a % 8 == 0 && stride_b % 8 == 0;
+	return aligned && M > 0 && N > 0 && M % 256 == 0 && N % 256 == 0 && K >= 64 && K % 64 == 0 &&
+	       lda < (1 << 24) && ldb < (1 << 24) && (M / 256) * (N / 256) <= 0x7FFFFFFFLL && batch >= 1 && batch <= 65535;
+}
+
+inline hipError_t launch_gemm_f16_ring(const half_t* A, const half_t* B, half_t* C, int64_t M, int64_t N, int64_t K,
+                                       int64_t lda, int64_t ldb, int64_t ldc,
+                                       int64_t stride_a, int64_t stride_b, int64_t stride_c, int64_t batch, hipStream_t stream)
+{
+	auto kernel = gemm_f16_nt_ring_kernel;
+	// More than 64 KB of dynamic LDS has to be granted per function and per device, once.
+	static std::atomic<uint64_t> configured_devices{0};
+	(void)hipGetLastError();
+	int device = 0;
+	hipError_t e = hipGetDevice(&device);
+	if (e != hipSuccess) return e;
+	const uint64_t bit = 1ull << (device & 63);
+	if ((configured_devices.load(std::memory_order_relaxed) & bit) == 0)
+	{
+		e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, GemmRingCfg::kLdsBytes);
+		if (e != hipSuccess) return e;
+		configured_devices.fetch_or(bit, std::memory_order_relaxed);
+	}
+	const int tiles_m = (int)(M / 256), tiles_n = (int)(N / 256);
+	kernel<<<dim3((unsigned)(tiles_m * tiles_n), (unsigned)batch), dim3(256), GemmRingCfg::kLdsBytes, stream>>>(
+		A, B, C, (int)K, lda, ldb, ldc, tiles_m, tiles_n, stride_a, stride_b, stride_c);
+	return hipGetLastError();
+}
+
+}  // namespace anygpu

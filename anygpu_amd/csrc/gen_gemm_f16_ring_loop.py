@@ -1,0 +1,184 @@
+#!/usr/bin/env python3
+"""Writes gemm_f16_ring_loop.inc: the main loop of the 256 x 256 fp16 GEMM tile kernel of gemm_f16_ring.hpp (four waves, a
+128 x 128 patch per wave) as the text of one inline-assembly block, every instruction in issue order.
+
+Why assembly: with one wave per SIMD nothing hides a stall, and the 256 accumulator registers of a lane fill the AGPR file
+exactly, which leaves the compiler's register allocator no room (it answered with copies between the two register files
+or with spills).  Here every register is fixed:
+
+  a[0:255]                 accumulators, MFMA tile (i, j) of the wave's 8 x 8 patch in a[4 (8 i + j) : + 3]
+  v[128:159] / v[160:191]  B / A fragments of a 32-deep step, buffer 0;  v[192:223] / v[224:255]  buffer 1
+  v[96:103]                byte offsets of this lane in the wave's eight A loads of a slab, v[104:111] the same for B
+  v112, v113               LDS addresses the fragment reads of the current step start from (A, B)
+  v114, v115               fragment addresses of the second step of a slab (chunk + 4: address bit 6 flipped)
+  s[60:64]                 LDS offsets of the units holding A(t), B(t), A(t+1), B(t+1) and of the free unit
+  s65 slab counter, s66 last slab, s67 temporary, s[68:69] / s[70:71] global address of the A / B slab being requested,
+  s72 unit that takes the B loads of the step
+
+LDS holds five operand units of 32 KB: a unit is the 256 rows x 64 k (128-byte rows, 16-byte chunks swizzled by the row) of
+A or of B for one 64-deep slab.  Operand slab n of the sequence A(0), B(0), A(1), B(1), ... lives in unit n mod 5.  While
+slab t is multiplied, A(t), B(t), A(t+1), B(t+1) are resident and the fifth unit takes A(t+2) during the first 32-deep
+step; at mid-slab, the one barrier of a slab, everybody has read A(t) and B(t), and B(t+2) goes where A(t) was during the
+second step.  So a wave issues one direct load (1 KB: 8 rows x 128 bytes, whole cache lines) per eight MFMAs, all the
+time, and every load has at least a step (64 MFMAs) to land.  Loads past the last slab fetch the last slab again into a
+unit nobody reads, which keeps the loop free of branches and the counters uniform.
+
+Under the 64 MFMAs of a step a wave issues the 16 fragment reads of the next step (one behind every second MFMA of the
+first half), its 8 loads with their M0 writes, and the address arithmetic of the next step, never more than three
+instructions behind one MFMA: with one wave per SIMD an MFMA covers 16 cycles, four instructions' worth of issue.
+
+Operands of the block (named): avoffe / avoffo, bvoffe / bvoffo (VGPR: the lane's byte offset in the even / odd loads),
+aaddr, baddr (VGPR: LDS byte address of the lane's fragment chunk inside a unit, minus the wave's share), arow16, brow16
+(SGPR: bytes between rows 16 apart), abaselo / abasehi, bbaselo / bbasehi (SGPR: global address of the wave's first row),
+ldsw (SGPR: LDS address of the wave's 8 KB share of unit 0), slabs (SGPR: K / 64).
+
+Usage: gen_gemm_f16_ring_loop.py OUTPUT
+"""
+import sys
+
+UNIT = 32768
+LOADS_AT = 5        # the load of a group of eight MFMAs goes behind this one, its M0 write behind the one before
+EXTRA_FROM = 33     # address arithmetic starts behind this MFMA (the reads of the step have been issued by then)
+
+lines = []
+
+
+def emit(s, comment=None):
+    if isinstance(s, tuple):
+        for x in s:
+            emit(x)
+        return
+    lines.append((s, comment))
+
+
+def acc(i, j):
+    r = 4 * (8 * i + j)
+    return f"a[{r}:{r + 3}]"
+
+
+def bfrag(buf, j):
+    r = 128 + 64 * buf + 4 * j
+    return f"v[{r}:{r + 3}]"
+
+
+def afrag(buf, i):
+    r = 160 + 64 * buf + 4 * i
+    return f"v[{r}:{r + 3}]"
+
+
+O = ["s60", "s61", "s62", "s63", "s64"]
+S_T, S_LAST, S_TMP, S_LD = "s65", "s66", "s67", "s72"
+A_CUR, B_CUR = "s[68:69]", "s[70:71]"
+V_RA, V_RB, V_A1, V_B1 = "v112", "v113", "v114", "v115"
+
+
+def base_ops(cur, name, add):
+    """global address of slab min(t + add, last) of one operand: 128 bytes per slab.  The add / add-with-carry pair is
+    one entry: nothing that writes SCC may come between the two."""
+    lo, hi = cur[2:-1].split(":")
+    return [f"s_add_u32 {S_TMP}, {S_T}, {add}", f"s_min_u32 {S_TMP}, {S_TMP}, {S_LAST}", f"s_lshl_b32 {S_TMP}, {S_TMP}, 7",
+            (f"s_add_u32 s{lo}, %[{name}lo], {S_TMP}", f"s_addc_u32 s{hi}, %[{name}hi], 0")]
+
+
+def loads(operand, unit_reg):
+    """the wave's eight loads of one operand slab as (M0 write, load) pairs"""
+    out = []
+    for q in range(8):
+        v = 96 + q + (8 if operand == "b" else 0)
+        out.append((f"s_add_u32 m0, {unit_reg}, {q * 1024}",
+                    f"global_load_lds_dwordx4 v{v}, {A_CUR if operand == 'a' else B_CUR}"))
+    return out
+
+
+def reads(buf, va, vb):
+    """the 16 fragment reads of a step: MFMA tile i of the patch lies 16 rows = 2048 bytes further on"""
+    out = [f"ds_read_b128 {bfrag(buf, q)}, {vb} offset:{q * 2048}" for q in range(8)]
+    out += [f"ds_read_b128 {afrag(buf, q)}, {va} offset:{q * 2048}" for q in range(8)]
+    return out
+
+
+# ---- prologue: A(0), B(0), A(1), B(1) into units 0 .. 3, fragments of the first step
+emit(f"s_mov_b32 {S_T}, 0", "prologue")
+emit(f"s_sub_u32 {S_LAST}, %[slabs], 1")
+for x in range(5):
+    emit(f"s_add_u32 {O[x]}, %[ldsw], {x * UNIT}")
+for q in range(8):
+    src = "%[avoffe]" if q % 2 == 0 else "%[avoffo]"
+    emit(f"v_mov_b32 v{96 + q}, {src}" if q < 2 else f"v_add_u32 v{96 + q}, %[arow16], v{96 + q - 2}")
+for q in range(8):
+    src = "%[bvoffe]" if q % 2 == 0 else "%[bvoffo]"
+    emit(f"v_mov_b32 v{104 + q}, {src}" if q < 2 else f"v_add_u32 v{104 + q}, %[brow16], v{104 + q - 2}")
+emit(f"v_xor_b32 {V_A1}, 64, %[aaddr]")
+emit(f"v_xor_b32 {V_B1}, 64, %[baddr]")
+for n, (operand, slab) in enumerate([("a", 0), ("b", 0), ("a", 1), ("b", 1)]):
+    for ins in base_ops(A_CUR if operand == "a" else B_CUR, operand + "base", slab):
+        emit(ins)
+    for m0w, ld in loads(operand, O[n]):
+        emit(m0w)
+        emit("s_nop 0")
+        emit(ld)
+for r in range(256):
+    emit(f"v_accvgpr_write_b32 a{r}, 0")
+emit("s_waitcnt vmcnt(16)", "A(0), B(0) have landed")
+emit("s_barrier")
+emit(f"v_add_u32 {V_RA}, {O[0]}, %[aaddr]")
+emit(f"v_add_u32 {V_RB}, {O[1]}, %[baddr]")
+for ins in reads(0, V_RA, V_RB):
+    emit(ins)
+emit(f"v_add_u32 {V_RA}, {O[0]}, {V_A1}", "addresses of the first step's reads (second half of slab 0), address of A(2)")
+emit(f"v_add_u32 {V_RB}, {O[1]}, {V_B1}")
+for ins in base_ops(A_CUR, "abase", 2):
+    emit(ins)
+emit("s_waitcnt lgkmcnt(0)")
+
+# ---- main loop: one slab per trip
+emit("1:", "main loop: one 64-deep slab per trip")
+for step in range(2):
+    gaps = [[] for _ in range(64)]          # gaps[m]: what is issued behind MFMA m of the step
+    buf = step
+    # fragments of the next step: step 0 reads the second half of slab t, step 1 the first half of slab t + 1
+    for q, ins in enumerate(reads(buf ^ 1, V_RA, V_RB)):
+        gaps[2 * q].append(ins)
+    # step 0: A(t + 2) into the free unit; step 1: B(t + 2) into the unit A(t) has left
+    if step == 1:
+        gaps[0].append(f"s_mov_b32 {S_LD}, {O[0]}")
+    for q, (m0w, ld) in enumerate(loads("a", O[4]) if step == 0 else loads("b", S_LD)):
+        gaps[8 * q + LOADS_AT - 1].append(m0w)
+        gaps[8 * q + LOADS_AT].append(ld)
+    if step == 0:
+        # read addresses of step 1 (first half of slab t + 1); address of B(t + 2)
+        extra = [f"v_add_u32 {V_RA}, {O[2]}, %[aaddr]", f"v_add_u32 {V_RB}, {O[3]}, %[baddr]"] + base_ops(B_CUR, "bbase", 2)
+    else:
+        # the units move on by two operand slabs, t advances; read addresses of the next slab's first step; address of A(t + 3)
+        extra = [f"s_mov_b32 {S_TMP}, {O[0]}", f"s_mov_b32 {O[0]}, {O[2]}", f"s_mov_b32 {O[2]}, {O[4]}", f"s_mov_b32 {O[4]}, {O[1]}",
+                 f"s_mov_b32 {O[1]}, {O[3]}", f"s_mov_b32 {O[3]}, {S_TMP}", f"s_add_u32 {S_T}, {S_T}, 1",
+                 f"v_add_u32 {V_RA}, {O[0]}, {V_A1}", f"v_add_u32 {V_RB}, {O[1]}, {V_B1}"] + base_ops(A_CUR, "abase", 2)
+    for k, ins in enumerate(extra):
+        gaps[EXTRA_FROM + k].append(ins)
+    if step == 1:
+        emit("s_waitcnt vmcnt(8)", "mid-slab: A(t+1), B(t+1) have landed (the loads of A(t+2) may be in flight)")
+        emit("s_barrier")
+    for m in range(64):
+        # row by row through the patch, every other row backwards, so that one operand stays when the row changes
+        i, j = m // 8, m % 8
+        if i % 2 == 1:
+            j = 7 - j
+        emit(f"v_mfma_f32_16x16x32_f16 {acc(i, j)}, {bfrag(buf, j)}, {afrag(buf, i)}, {acc(i, j)}",
+             f"step {step}" if m == 0 else None)
+        for ins in gaps[m]:
+            emit(ins)
+    emit("s_waitcnt lgkmcnt(0)")
+emit(f"s_cmp_lt_u32 {S_T}, %[slabs]")
+emit("s_cbranch_scc1 1b")
+emit("s_waitcnt vmcnt(0)", "nothing may still be writing LDS; the last MFMAs leave the pipeline before the accumulators are read")
+emit("s_barrier")
+emit("s_nop 15")
+emit("s_nop 15")
+
+if __name__ == "__main__":
+    with open(sys.argv[1], "w") as f:
+        f.write("// Written by gen_gemm_f16_ring_loop.py (the register plan and the schedule are explained there): do not edit.\n")
+        for s, c in lines:
+            if c:
+                f.write(f"// {c}\n")
+            f.write(f'"{s}\\n\\t"\n')

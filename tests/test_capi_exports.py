@@ -76,3 +76,12 @@ def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     monkeypatch.setattr(capi, "LIB_PATH", tmp_path / "libanygpu_hip.so")
     with pytest.raises(RuntimeError, match="no CPU fallback"):
         capi.load()
+
+
+def test_generated_gemm_loop_is_current(tmp_path):
+    # gemm_f16_ring_loop.inc is generated text that is committed: it has to be what the generator beside it writes
+    import sys
+    csrc = REPO / "anygpu_amd" / "csrc"
+    out = tmp_path / "loop.inc"
+    subprocess.run([sys.executable, str(csrc / "gen_gemm_f16_ring_loop.py"), str(out)], check=True)
+    assert out.read_text() == (csrc / "gemm_f16_ring_loop.inc").read_text()

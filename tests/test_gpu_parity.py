@@ -680,6 +680,43 @@ def test_mm_f16_config_4096_cubed_col_major_b(ops, oracle):
     assert np.max(np.abs(g64.sum(axis=0) - col_sum)) < tol
 
 
+@pytest.mark.parametrize("m,n,k,pad", [(4096, 4096, 64, 0), (4096, 4096, 128, 0), (4096, 4096, 192, 8), (2048, 8192, 320, 0),
+                                       (8192, 2048, 256, 72), (3840, 4352, 64, 0)])
+def test_mm_f16_whole_256_tiles_integer_inputs_exact(ops, m, n, k, pad):
+    # Shapes of whole 256 x 256 tiles with k-contiguous weights take the four-wave kernel whose main loop is an assembly
+    # block: one slab (K = 64), two, an odd number, padded leading dimensions, a tile count that is no multiple of the
+    # 8 XCDs.  Integers in -2 .. 2 with K <= 320: every sum is an integer below 2^11, exact in fp32 and in the fp16
+    # result, whatever the order of summation.
+    import torch
+    from anygpu_amd import capi
+    a = synth.integers(m + k, (m, k), -2, 2).astype(np.float16)
+    bt = synth.integers(n + k + 1, (n, k), -2, 2).astype(np.float16)
+    a_dev = torch.zeros((m, k + pad), dtype=torch.float16, device="cuda")
+    b_dev = torch.full((n, k + pad), 7.0, dtype=torch.float16, device="cuda")      # the padding must not be read as data
+    a_dev[:, :k] = dev(a)
+    b_dev[:, :k] = dev(bt)
+    got = host(ops.tensor_mm(a_dev[:, :k], b_dev[:, :k], b_layout=capi.B_COL_MAJOR)).astype(np.int64)
+    want = a.astype(np.int64) @ bt.astype(np.int64).T
+    assert np.array_equal(got, want)
+
+
+def test_mm_f16_whole_256_tiles_batched(ops, oracle):
+    # four products of 2048 x 2048 x 128 in one launch: 256 tiles of 256 x 256, the four-wave kernel over blockIdx.y
+    from anygpu_amd import capi
+    batch, n, k = 4, 2048, 128
+    a = synth.uniform(5, (batch, n, k)).astype(np.float16)
+    bt = synth.uniform(6, (batch, n, k)).astype(np.float16)
+    got = host(ops.tensor_mm_batched(dev(a), dev(bt), b_layout=capi.B_COL_MAJOR)).astype(np.float32)
+    a32, bt32 = oracle.cvt_f16_to_f32(a), oracle.cvt_f16_to_f32(bt)
+    floor = math.sqrt(k) / 3.0
+    for i in range(batch):
+        idx = sample_rows(n, 16, seed=i)
+        want = np.stack([oracle.tensor_mm(a32[i, r:r + 1], bt32[i].T)[0] for r in idx])
+        assert scaled_rel_err(got[i][idx], want, floor) <= TOL_F16_GEMM
+        ref64 = a32[i].astype(np.float64) @ bt32[i].astype(np.float64).T
+        assert np.max(np.abs(got[i] - ref64)) <= floor * 2e-2
+
+
 @pytest.mark.parametrize("dtype", ["f16", "f32"])
 @pytest.mark.parametrize("layout", ["row", "col"])
 @pytest.mark.parametrize("m,k,n", [(1, 2304, 9216), (1, 64, 8), (2, 512, 1000), (3, 2304, 2050), (4, 1000, 512),
