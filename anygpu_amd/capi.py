@@ -19,6 +19,7 @@ ANYGPU_ERR_UNSUPPORTED = -4
 ANYGPU_ERR_TOO_LARGE = -5
 ANYGPU_ERR_SCRATCH_TOO_SMALL = -6
 DECODE_STATIC_SCRATCH_BYTES = 8 * 1024 * 1024
+WORKSPACE_BYTES = 64 * 1024 * 1024
 
 A_ROW_MAJOR = 0
 A_COL_MAJOR = 1
@@ -30,6 +31,8 @@ SIGNATURES = {
     "anygpu_hip_abi_version": (c_int, []),
     "anygpu_hip_target": (c_char_p, []),
     "anygpu_hip_error_string": (c_char_p, [c_int]),
+    "anygpu_set_workspace": (c_int, [c_void_p, c_void_p, c_int64]),
+    "anygpu_release_workspaces": (c_int, []),
     "anygpu_gemm_f16_f32acc": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64,
                                        c_int64, c_int64, c_int64, c_int, c_void_p]),
     "anygpu_gemm_f32": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64,

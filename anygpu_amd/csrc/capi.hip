@@ -2,6 +2,7 @@
 // Nothing is launched when an argument is rejected.
 #include "anygpu_hip.h"
 #include "launch.hpp"
+#include "gemm_band.hpp"
 #include "device_utils.hpp"
 
 #include <atomic>
@@ -204,6 +205,19 @@ ANYGPU_EXPORT const char* anygpu_hip_error_string(int code)
 	}
 	if (code > 0) return hipGetErrorString(static_cast<hipError_t>(code));
 	return "unknown anygpu error code";
+}
+
+ANYGPU_EXPORT int anygpu_set_workspace(void* stream, void* workspace, int64_t bytes)
+{
+	if (bytes < 0) return ANYGPU_ERR_BAD_SHAPE;
+	if (workspace == nullptr && bytes > 0) return ANYGPU_ERR_NULL_POINTER;
+	if (reinterpret_cast<uintptr_t>(workspace) % 256 != 0) return ANYGPU_ERR_UNSUPPORTED;
+	return anygpu::band::workspace_set(as_stream(stream), workspace, (size_t)bytes);
+}
+
+ANYGPU_EXPORT int anygpu_release_workspaces(void)
+{
+	return (int)anygpu::band::workspace_release_all();
 }
 
 ANYGPU_EXPORT int anygpu_gemm_f16_f32acc(const void* A, const void* B, void* C,

@@ -350,7 +350,9 @@ hipError_t launch_band(const T* A, const T* B, const T* B2, const float* bias, T
 	using S = BandShape<T, MR, MB>;
 	constexpr int kAccFloats = S::kNG * (EPI == kEpiGeluMul ? 2 : 1) * MB * BandMma<T, MR>::kRegs;
 	const int64_t tiles = (N + kBandCols - 1) / kBandCols;
-	const SplitPlan plan = plan_band_splits(tiles, K, S::kChunk, S::kRows, (int)sizeof(T), kAccFloats, stream);
+	SplitPlan plan;
+	const hipError_t plan_err = plan_band_splits(tiles, K, S::kChunk, S::kRows, (int)sizeof(T), kAccFloats, stream, &plan);
+	if (plan_err != hipSuccess) return plan_err;
 	const int64_t splits = plan.splits, chunks_per_split = plan.chunks_per_split;
 	float* partial = plan.partial;
 	discard_stale_error();
@@ -367,31 +369,117 @@ hipError_t launch_band(const T* A, const T* B, const T* B2, const float* bias, T
 
 }  // namespace
 
-// Partial-sum workspace of one (device, stream) pair; NULL when there is none and none can be made now.
-float* band::band_workspace(hipStream_t stream)
+// ---------------------------------------------------------------------------------------------
+// Partial-sum workspaces, one per (device, stream) pair that has cut a product or been given one.
+// ---------------------------------------------------------------------------------------------
+namespace {
+
+struct WorkspaceEntry
 {
-	static std::mutex lock;
-	static std::map<std::pair<int, hipStream_t>, float*> cache;
-	int device = 0;
-	if (hipGetDevice(&device) != hipSuccess) return nullptr;
-	std::lock_guard<std::mutex> guard(lock);
-	const auto key = std::make_pair(device, stream);
-	const auto found = cache.find(key);
-	if (found != cache.end()) return found->second;
+	float* base;
+	size_t bytes;
+	bool from_caller;
+};
+
+std::mutex workspace_lock;
+std::map<std::pair<int, hipStream_t>, WorkspaceEntry> workspaces;
+
+bool stream_is_capturing(hipStream_t stream)
+{
 	hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
-	if (hipStreamIsCapturing(stream, &capture) != hipSuccess || capture != hipStreamCaptureStatusNone)
+	if (hipStreamIsCapturing(stream, &capture) != hipSuccess)
 	{
 		(void)hipGetLastError();
-		return nullptr;                       // no allocation under capture: the caller runs unsplit
+		return true;                          // (a stream whose state cannot be read is treated like one under capture)
 	}
-	void* base = nullptr;
-	if (hipMalloc(&base, kBandPartialBytes) != hipSuccess)
+	return capture != hipStreamCaptureStatusNone;
+}
+
+}  // namespace
+
+size_t band::workspace_capacity(hipStream_t stream)
+{
+	int device = 0;
+	if (hipGetDevice(&device) != hipSuccess) return 0;
+	{
+		std::lock_guard<std::mutex> guard(workspace_lock);
+		const auto found = workspaces.find(std::make_pair(device, stream));
+		if (found != workspaces.end() && found->second.from_caller) return found->second.bytes;
+	}
+	// the library's own buffer: eager launches only
+	return stream_is_capturing(stream) ? 0 : kBandPartialBytes;
+}
+
+hipError_t band::workspace_acquire(hipStream_t stream, float** base)
+{
+	*base = nullptr;
+	int device = 0;
+	hipError_t err = hipGetDevice(&device);
+	if (err != hipSuccess) return err;
+	std::lock_guard<std::mutex> guard(workspace_lock);
+	const auto key = std::make_pair(device, stream);
+	const auto found = workspaces.find(key);
+	if (found != workspaces.end())
+	{
+		*base = found->second.base;
+		return hipSuccess;
+	}
+	// First cut on this stream.  Another thread may be capturing some other stream in the global mode, in which an
+	// allocation made anywhere invalidates its capture: this thread allocates in the relaxed mode.
+	hipStreamCaptureMode mode = hipStreamCaptureModeRelaxed;
+	(void)hipThreadExchangeStreamCaptureMode(&mode);
+	void* mem = nullptr;
+	err = hipMalloc(&mem, kBandPartialBytes);
+	(void)hipThreadExchangeStreamCaptureMode(&mode);
+	if (err != hipSuccess)
 	{
 		(void)hipGetLastError();
-		return nullptr;
+		return err;
 	}
-	cache.emplace(key, static_cast<float*>(base));
-	return static_cast<float*>(base);
+	workspaces.emplace(key, WorkspaceEntry{static_cast<float*>(mem), kBandPartialBytes, false});
+	*base = static_cast<float*>(mem);
+	return hipSuccess;
+}
+
+int band::workspace_set(hipStream_t stream, void* base, size_t bytes)
+{
+	int device = 0;
+	const hipError_t err = hipGetDevice(&device);
+	if (err != hipSuccess) return (int)err;
+	std::lock_guard<std::mutex> guard(workspace_lock);
+	const auto key = std::make_pair(device, stream);
+	const auto found = workspaces.find(key);
+	if (found != workspaces.end())
+	{
+		// the library's own buffer of this stream makes way (the caller has made sure that nothing on the stream
+		// still uses it)
+		if (!found->second.from_caller)
+		{
+			const hipError_t freed = hipFree(found->second.base);
+			if (freed != hipSuccess) return (int)freed;
+		}
+		workspaces.erase(found);
+	}
+	if (base != nullptr && bytes > 0) workspaces.emplace(key, WorkspaceEntry{static_cast<float*>(base), bytes, true});
+	return ANYGPU_OK;
+}
+
+hipError_t band::workspace_release_all()
+{
+	std::lock_guard<std::mutex> guard(workspace_lock);
+	hipError_t result = hipSuccess;
+	for (auto& entry : workspaces)
+	{
+		if (entry.second.from_caller) continue;
+		int current = 0;
+		(void)hipGetDevice(&current);
+		if (current != entry.first.first) (void)hipSetDevice(entry.first.first);
+		const hipError_t freed = hipFree(entry.second.base);
+		if (freed != hipSuccess) result = freed;
+		if (current != entry.first.first) (void)hipSetDevice(current);
+	}
+	workspaces.clear();
+	return result;
 }
 
 template <typename T>

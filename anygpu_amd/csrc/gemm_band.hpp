@@ -66,9 +66,20 @@ template <> struct BandMma<half_t, 32>
 	}
 };
 
-// Partial-sum workspace of one (device, stream) pair: kBandPartialBytes, allocated on first use and kept
-// for the life of the process; NULL when there is none and none can be made now (stream under capture).
-float* band_workspace(hipStream_t stream);
+// Partial-sum workspace of a (device, stream) pair.  Either the caller has handed one in for the stream
+// (anygpu_set_workspace: any size, the library then allocates nothing for that stream), or the library owns one of
+// kBandPartialBytes, allocated the first time an eager launch on the stream cuts a product and kept until
+// anygpu_release_workspaces or the end of the process.  A stream that is being captured into a graph uses a caller's
+// workspace or none: a graph never records the library's own buffer, and what a captured launch computes does not depend
+// on what ran on the stream before.
+// workspace_capacity: bytes a launch on `stream` may plan partial sums for right now (0: run uncut), without allocating.
+// workspace_acquire: the buffer of at least that size; allocates the library's own on first use and returns the error if
+// that fails.
+size_t workspace_capacity(hipStream_t stream);
+hipError_t workspace_acquire(hipStream_t stream, float** base);
+// the C ABI's anygpu_set_workspace / anygpu_release_workspaces
+int workspace_set(hipStream_t stream, void* base, size_t bytes);
+hipError_t workspace_release_all();
 
 inline bool aligned16(const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; }
 
@@ -82,12 +93,13 @@ struct SplitPlan
 
 // `chunk`: K elements per LDS chunk of the band (splits are whole chunks), `rows`: band rows (padded),
 // `elem_bytes`: weight element size, `acc_floats`: partial sums per thread and split.
-inline SplitPlan plan_band_splits(int64_t tiles, int64_t K, int64_t chunk, int64_t rows, int elem_bytes, int acc_floats,
-                                  hipStream_t stream)
+inline hipError_t plan_band_splits(int64_t tiles, int64_t K, int64_t chunk, int64_t rows, int elem_bytes, int acc_floats,
+                                   hipStream_t stream, SplitPlan* out)
 {
 	const int64_t kchunks = (K + chunk - 1) / chunk;
 	int64_t splits = 1;
-	if (tiles < kBandEnoughBlocks)
+	const size_t capacity = tiles < kBandEnoughBlocks ? workspace_capacity(stream) : 0;
+	if (tiles < kBandEnoughBlocks && capacity > 0)
 	{
 		splits = (kBandWantedBlocks + tiles - 1) / tiles;
 		if (splits > kBandMaxSplits) splits = kBandMaxSplits;
@@ -96,7 +108,8 @@ inline SplitPlan plan_band_splits(int64_t tiles, int64_t K, int64_t chunk, int64
 		const int64_t min_depth = 32 * rows / elem_bytes;
 		const int64_t min_chunks = (min_depth + chunk - 1) / chunk;
 		if (splits > kchunks / min_chunks) splits = kchunks / min_chunks;
-		const int64_t room = (int64_t)(kBandPlanBytes / ((size_t)tiles * kBandThreads * acc_floats * sizeof(float)));
+		const size_t plan_bytes = capacity < kBandPlanBytes ? capacity : kBandPlanBytes;
+		const int64_t room = (int64_t)(plan_bytes / ((size_t)tiles * kBandThreads * acc_floats * sizeof(float)));
 		if (splits > room) splits = room;
 		if (splits < 1) splits = 1;
 	}
@@ -106,14 +119,11 @@ inline SplitPlan plan_band_splits(int64_t tiles, int64_t K, int64_t chunk, int64
 	plan.partial = nullptr;
 	if (plan.splits > 1)
 	{
-		plan.partial = band_workspace(stream);
-		if (!plan.partial)
-		{
-			plan.splits = 1;
-			plan.chunks_per_split = kchunks;
-		}
+		const hipError_t err = workspace_acquire(stream, &plan.partial);
+		if (err != hipSuccess) return err;
 	}
-	return plan;
+	*out = plan;
+	return hipSuccess;
 }
 
 }  // namespace band

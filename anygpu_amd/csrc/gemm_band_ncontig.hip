@@ -371,7 +371,9 @@ hipError_t launch_row_band_waves(const float* A, const float* B, const float* B2
 	const int64_t tiles = (N + S::kBlockCols - 1) / S::kBlockCols;
 	const int64_t wave_tiles = (N + S::kWaveCols - 1) / S::kWaveCols;
 	// one wave's worth of sums per wave tile and split: a quarter of a 256-thread block's
-	const SplitPlan plan = plan_band_splits(tiles, K, S::kChunk, S::kRows, (int)sizeof(float), S::kAccFloats / (KW ? 4 : 1), stream);
+	SplitPlan plan;
+	const hipError_t plan_err = plan_band_splits(tiles, K, S::kChunk, S::kRows, (int)sizeof(float), S::kAccFloats / (KW ? 4 : 1), stream, &plan);
+	if (plan_err != hipSuccess) return plan_err;
 	discard_stale_error();
 	gemm_band_ncontig_kernel<MR, MB, EPI, KW><<<dim3((unsigned)tiles, (unsigned)plan.splits), dim3(kBandThreads), 0, stream>>>(
 		A, B, B2, bias, C, plan.partial, M, N, K, lda, ldb, ldc, (int)plan.chunks_per_split, ep_param);

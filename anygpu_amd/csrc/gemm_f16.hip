@@ -324,7 +324,9 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
 		{
 			const double slabs = (double)(K / 64);
 			double best = slabs * (rect ? cost_rect : cost_square);
-			const int64_t room = (int64_t)(band::kBandPartialBytes / ((size_t)M * N * sizeof(float)));
+			// (as many planes as the stream's workspace holds: the caller's, or the library's own for eager launches; a
+			// stream under capture without a caller's workspace has none and runs uncut)
+			const int64_t room = (int64_t)(band::workspace_capacity(stream) / ((size_t)M * N * sizeof(float)));
 			for (const int64_t t : {(int64_t)256, (int64_t)128, (int64_t)64})
 			{
 				if (blocks(t) >= 256) continue;
@@ -350,9 +352,11 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
 				if (ranges == splits && K - (splits - 1) * k_split >= 64) break;     // every range holds at least a slab
 				splits = ranges == splits ? splits - 1 : ranges;
 			}
-			float* planes = splits > 1 ? band::band_workspace(stream) : nullptr;
-			if (planes)
+			if (splits > 1)
 			{
+				float* planes = nullptr;
+				const hipError_t ws_err = band::workspace_acquire(stream, &planes);
+				if (ws_err != hipSuccess) return ws_err;
 				const int64_t step_b = (b_layout == ANYGPU_B_COL_MAJOR) ? k_split : k_split * ldb;
 				const bool deep_stages = blocks(64) * splits <= kDeepStageBlocks;
 				hipError_t err;
@@ -380,7 +384,7 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
 				return hipGetLastError();
 			}
 		}
-		// unsplit (also when the workspace cannot be had, as under stream capture): the tile priced for that.
+		// unsplit (also where the stream has no workspace to cut into, as under capture): the tile priced for that.
 		// One "general" instantiation serves ragged M / N and a K tail alike.
 		tile = tile_unsplit;
 		if (rect && blocks_rect / batch <= 0x7FFFFFFFLL)
@@ -403,7 +407,8 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
 		{
 			// whole 256 x 256 tiles of k-contiguous operands: the four-wave kernel with 128 x 128 patches (4096^3: 93 us
 			// against 99 us for the eight-wave tile on the same box, vendor library 93 us)
-			if (tile == 256 && !ragged && gemm_f16_ring_applies(a, b, M, N, K, lda, ldb, stride_a, stride_b, batch))
+			const bool c_aligned = reinterpret_cast<uintptr_t>(C) % 16 == 0 && ldc % 8 == 0 && stride_c % 8 == 0;
+			if (tile == 256 && !ragged && c_aligned && gemm_f16_ring_applies(a, b, M, N, K, lda, ldb, stride_a, stride_b, batch))
 				return launch_gemm_f16_ring(a, b, c, M, N, K, lda, ldb, ldc, stride_a, stride_b, stride_c, batch, stream);
 			if (tile == 256) ANYGPU_F16_TILE(256, 2, 4, false, 2, 1);
 			if (tile == 128) ANYGPU_F16_TILE(128, 2, 2, false, 2, 1);

@@ -105,7 +105,7 @@ __global__ __launch_bounds__(256) void gemm_f16_nt_ring_kernel(
 #pragma unroll
 		for (int j = 0; j < 8; ++j)
 			acc[i][j] = float4_t{(*rows[i])[4 * j], (*rows[i])[4 * j + 1], (*rows[i])[4 * j + 2], (*rows[i])[4 * j + 3]};
-	store_patch_via_lds<Cfg, false>(acc, lds, C, ldc, m0 + wm * 128, n0 + wn * 128, wave, lane, 0, 0);
+	store_patch_via_lds<Cfg, false, true>(acc, lds, C, ldc, m0 + wm * 128, n0 + wn * 128, wave, lane, 0, 0);
 }
 
 // What the kernel assumes, checked on the host before every launch: whole tiles, whole slabs, 16-byte aligned operand
@@ -115,6 +115,7 @@ inline bool gemm_f16_ring_applies(const half_t* A, const half_t* B, int64_t M, i
 {
 	const bool aligned = reinterpret_cast<uintptr_t>(A) % 16 == 0 && reinterpret_cast<uintptr_t>(B) % 16 == 0 &&
 	                     lda % 8 == 0 && ldb % 8 == 0 && stride_a % 8 == 0 && stride_b % 8 == 0;
+	// (the epilogue streams whole 16-byte vectors: C has to be aligned like the operands, which the caller checks)
 	return aligned && M > 0 && N > 0 && M % 256 == 0 && N % 256 == 0 && K >= 64 && K % 64 == 0 &&
 	       lda < (1 << 24) && ldb < (1 << 24) && (M / 256) * (N / 256) <= 0x7FFFFFFFLL && batch >= 1 && batch <= 65535;
 }

@@ -186,9 +186,13 @@ __device__ __forceinline__ half4_t lds_read_transposed_b64(const char* lds_addr)
 // rows over the banks.  The caller guarantees that nobody still reads or fills LDS.
 // RAGGED: rows at or beyond M and columns at or beyond N are not stored (the 8-column chunk that crosses N goes out
 // element by element).  Stores are made at element alignment: rows of C may start anywhere.
+// STREAM: the whole vectors are stored with the non-temporal hint (C is 16-byte aligned then).  A launch that writes tens
+// of megabytes otherwise ends with all of C dirty in the L2s and pays for the write-back when the kernel retires
+// (4096^3: 93.5 -> 92.4 us); the same bytes written without the LDS pass, 64 contiguous bytes per row and instruction
+// after a v_permlane16_swap between neighbouring tiles, were 1.5 us slower than whole rows through LDS.
 typedef half8_t LooseHalf8Store __attribute__((aligned(2)));
 
-template <typename Cfg, bool RAGGED>
+template <typename Cfg, bool RAGGED, bool STREAM = false>
 __device__ __forceinline__ void store_patch_via_lds(
 	const typename MfmaShape<Cfg::MI>::Acc (&acc)[Cfg::kTilesM][Cfg::kTilesN], char* lds,
 	half_t* __restrict__ C, int64_t ldc, int64_t m_base, int64_t n_base, int wave, int lane, int64_t M, int64_t N)
@@ -227,7 +231,8 @@ __device__ __forceinline__ void store_patch_via_lds(
 			{
 				const half8_t v = *reinterpret_cast<const half8_t*>(scratch + row * kPitch + col16 * 16);
 				half_t* dst = C + (m_base + i * MI + row) * ldc + n_base + col16 * 8;
-				if (!RAGGED || n_base + col16 * 8 + 8 <= N) *reinterpret_cast<LooseHalf8Store*>(dst) = v;
+				if constexpr (STREAM && !RAGGED) __builtin_nontemporal_store(v, reinterpret_cast<half8_t*>(dst));
+				else if (!RAGGED || n_base + col16 * 8 + 8 <= N) *reinterpret_cast<LooseHalf8Store*>(dst) = v;
 				else
 				{
 #pragma unroll

@@ -423,7 +423,7 @@ constexpr int64_t kSplitMinDepth = 256;
 constexpr int64_t kSplitMax = 16;
 constexpr int64_t kChipCus = 256;
 
-static TilePlan plan_tiles(int tile, int64_t M, int64_t N, int64_t K, int64_t batch, bool may_split)
+static TilePlan plan_tiles(int tile, int64_t M, int64_t N, int64_t K, int64_t batch, bool may_split, size_t workspace_bytes)
 {
 	const double slab_us = tile == 128 ? 1.0 : 0.36;
 	const int64_t tiles = ((M + tile - 1) / tile) * ((N + tile - 1) / tile) * batch;
@@ -434,7 +434,7 @@ static TilePlan plan_tiles(int tile, int64_t M, int64_t N, int64_t K, int64_t ba
 	};
 	TilePlan best{tile, 1, rounds_of(tiles) * (double)slabs * slab_us};
 	if (!may_split || batch != 1) return best;
-	const int64_t room = (int64_t)(band::kBandPartialBytes / ((size_t)M * N * sizeof(float)));
+	const int64_t room = (int64_t)(workspace_bytes / ((size_t)M * N * sizeof(float)));
 	for (int64_t s = 2; s <= kSplitMax && s <= K / kSplitMinDepth && s <= room; ++s)
 	{
 		const double rounds = rounds_of(tiles * s);
@@ -458,9 +458,11 @@ static hipError_t launch_tiles(const float* A, const float* B, const float* B2, 
 			int64_t k_split = (K + splits - 1) / splits;
 			k_split = (k_split + kBK - 1) / kBK * kBK;
 			splits = (K + k_split - 1) / k_split;
-			float* partial = splits > 1 ? band::band_workspace(stream) : nullptr;
-			if (partial)
+			if (splits > 1)
 			{
+				float* partial = nullptr;
+				const hipError_t ws_err = band::workspace_acquire(stream, &partial);
+				if (ws_err != hipSuccess) return ws_err;
 				const int64_t step_a = (A_LAYOUT == ANYGPU_A_ROW_MAJOR) ? k_split : k_split * lda;
 				const int64_t step_b = (B_LAYOUT == ANYGPU_B_COL_MAJOR) ? k_split : k_split * ldb;
 				const hipError_t err = launch_tiles_once<A_LAYOUT, B_LAYOUT, BM, BN, kEpiBias>(
@@ -488,8 +490,11 @@ static hipError_t launch_layout(const float* A, const float* B, const float* B2,
                                 float ep_param, hipStream_t stream)
 {
 	const bool may_split = (EPI != kEpiGeluMul);
-	const TilePlan big = plan_tiles(128, M, N, K, batch, may_split);
-	const TilePlan small = plan_tiles(64, M, N, K, batch, may_split);
+	// (what the stream's workspace holds bounds the cuts along K: the caller's, or the library's own for eager launches;
+	// a stream under capture without a caller's workspace has none and runs uncut)
+	const size_t ws_bytes = (may_split && batch == 1) ? band::workspace_capacity(stream) : 0;
+	const TilePlan big = plan_tiles(128, M, N, K, batch, may_split, ws_bytes);
+	const TilePlan small = plan_tiles(64, M, N, K, batch, may_split, ws_bytes);
 	if constexpr (EPI != kEpiGeluMul)
 	{
 		// A product of big tiles that fills whole rounds and a bit, e.g. 576 tiles = 2.25 rounds, pays three rounds.  It
@@ -501,9 +506,9 @@ static hipError_t launch_layout(const float* A, const float* B, const float* B2,
 		if (batch == 1 && whole > 0 && head_cols > 0 && head_cols < tiles_n)
 		{
 			const int64_t n_head = head_cols * 128, n_tail = N - n_head;
-			const TilePlan head = plan_tiles(128, M, n_head, K, 1, false);
-			const TilePlan tail_big = plan_tiles(128, M, n_tail, K, 1, true);
-			const TilePlan tail_small = plan_tiles(64, M, n_tail, K, 1, true);
+			const TilePlan head = plan_tiles(128, M, n_head, K, 1, false, 0);
+			const TilePlan tail_big = plan_tiles(128, M, n_tail, K, 1, true, ws_bytes);
+			const TilePlan tail_small = plan_tiles(64, M, n_tail, K, 1, true, ws_bytes);
 			const TilePlan& tail = tail_big.cost <= tail_small.cost ? tail_big : tail_small;
 			const double best_whole = big.cost <= small.cost ? big.cost : small.cost;
 			if (head.cost + tail.cost + 3.0 < 0.96 * best_whole)

@@ -27,6 +27,24 @@ def _check_device(*tensors: torch.Tensor) -> None:
         _require(t.is_cuda, "anygpu ops take device tensors only (no CPU fallback)")
 
 
+def set_workspace(workspace: torch.Tensor | None, stream: torch.cuda.Stream | None = None) -> None:
+    """Hand the GEMM entry points a caller-owned K-split workspace for `stream` (default: the current stream), or take
+    it back with None.  The tensor must stay alive while launches or graphs that used it can still run."""
+    lib = capi.load()
+    handle = (stream or torch.cuda.current_stream()).cuda_stream
+    if workspace is None:
+        capi.check("anygpu_set_workspace", lib.anygpu_set_workspace(handle, None, 0))
+        return
+    _check_device(workspace)
+    _require(workspace.is_contiguous(), "the workspace must be dense")
+    capi.check("anygpu_set_workspace", lib.anygpu_set_workspace(handle, workspace.data_ptr(), workspace.numel() * workspace.element_size()))
+
+
+def release_workspaces() -> None:
+    """Free every K-split workspace the library allocated itself and forget all registrations."""
+    capi.check("anygpu_release_workspaces", capi.load().anygpu_release_workspaces())
+
+
 def tensor_mm(lhs: torch.Tensor, rhs: torch.Tensor, out: torch.Tensor | None = None,
               b_layout: int = capi.B_ROW_MAJOR, a_layout: int = capi.A_ROW_MAJOR) -> torch.Tensor:
     """C = A @ B.  With a_layout == A_ROW_MAJOR lhs is [M, K] (rows may be padded: stride(0) >= K,

@@ -4,13 +4,16 @@
  *
  * Conventions
  *   - every pointer is a DEVICE pointer into memory the caller owns; inputs are only read,
- *     outputs only written.  The library frees nothing and keeps one thing, like a BLAS handle:
- *     the GEMM entry points cut some products along K (few tiles and a deep K, few rows against
- *     a weight matrix) and put the partial sums of such a launch into a 16 MiB device buffer
- *     that is allocated the first time a (device, stream) pair needs it and kept until the
- *     process ends.  Launches on one stream share it in stream order, other streams have their
- *     own.  No allocation is made while the stream is being captured into a graph: a pair
- *     without a buffer then runs uncut.  Nothing else allocates;
+ *     outputs only written.  One kind of scratch exists: the GEMM entry points cut some products
+ *     along K (few tiles and a deep K, few rows against a weight matrix) and pass the partial
+ *     sums of such a launch through a workspace that belongs to the (device, stream) pair of the
+ *     call.  Who owns it is the caller's choice, see anygpu_set_workspace: by default the library
+ *     allocates ANYGPU_WORKSPACE_BYTES (64 MiB) the first time an eager launch on a stream cuts a
+ *     product and keeps them until anygpu_release_workspaces or the end of the process; a caller
+ *     that hands in its own workspace for a stream makes the library allocate nothing there.
+ *     While a stream is being captured into a graph only a caller's workspace is used, never the
+ *     library's: without one every captured product runs uncut (a valid result, summed in
+ *     another order than the cut one).  Nothing else allocates;
  *   - sizes, strides and leading dimensions are int64_t counts of ELEMENTS;
  *   - `stream` is a hipStream_t passed as void* (NULL = the null stream, which is what the
  *     reference uses for every launch); calls are asynchronous with respect to the host;
@@ -53,6 +56,29 @@ extern "C" {
 int         anygpu_hip_abi_version(void);
 const char* anygpu_hip_target(void);            /* "gfx950" */
 const char* anygpu_hip_error_string(int code);  /* text for ANYGPU_ERR_* and for hipError_t values */
+
+/*
+ * The K-split workspace of the GEMM entry points (all of anygpu_gemm_*), per (current device, stream).
+ *
+ * anygpu_set_workspace(stream, workspace, bytes) hands in `bytes` of device memory, 256-byte aligned, for the launches
+ * made on `stream` from now on: the library then allocates nothing for that stream, plans its cuts along K within
+ * `bytes` (too small for a shape: that shape runs uncut) and makes the same plan whether the stream is being captured
+ * or not, so a captured product equals the eager one bit for bit.  The memory stays the caller's: it must outlive every
+ * launch and every graph that used it, launches on the stream share it in stream order, and a graph that recorded
+ * cut products owns it while it replays (no other work that uses the same workspace may overlap the replay, on
+ * whatever stream).  workspace = NULL (bytes = 0) takes the registration back; a buffer the library had allocated for
+ * the stream is freed by either call, so nothing on the stream may still be running.  The reference has no such
+ * scratch: its ops layer allocates every buffer and its kernels none (srcs/core/tensor.hpp:56-57).
+ *
+ * anygpu_release_workspaces() frees every buffer the library itself allocated (on all devices) and forgets all
+ * registrations; call it when no GEMM of this library is in flight.  Every (device, stream) pair that cuts a product
+ * without a caller's workspace holds ANYGPU_WORKSPACE_BYTES until then; the library does not notice a stream being
+ * destroyed.
+ */
+#define ANYGPU_WORKSPACE_BYTES (64 * 1024 * 1024)
+
+int anygpu_set_workspace(void* stream, void* workspace, int64_t bytes);
+int anygpu_release_workspaces(void);
 
 /*
  * C[M,N] = A[M,K] * B  with fp16 inputs, fp32 accumulation on the MFMA units, fp16 output.

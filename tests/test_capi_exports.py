@@ -55,6 +55,10 @@ def test_argument_validation_needs_no_gpu():
     assert lib.anygpu_softmax_rows_f16(fake, None, 4, 16, 16, 16, 0, 0, 1.0, 0.0, 0, 0, None) == capi.ANYGPU_ERR_NULL_POINTER
     assert lib.anygpu_causal_conv1d_silu_f16(fake, fake, fake, fake, 2, 3, 8, 5, None) == capi.ANYGPU_ERR_UNSUPPORTED
     assert lib.anygpu_causal_conv1d_silu_f32(fake, fake, fake, fake, 2, 3, -8, 4, None) == capi.ANYGPU_ERR_BAD_SHAPE
+    # the K-split workspace: rejected before the runtime is asked for the device
+    assert lib.anygpu_set_workspace(None, fake, -1) == capi.ANYGPU_ERR_BAD_SHAPE
+    assert lib.anygpu_set_workspace(None, None, 4096) == capi.ANYGPU_ERR_NULL_POINTER
+    assert lib.anygpu_set_workspace(None, ctypes.c_void_p(0x1010), 4096) == capi.ANYGPU_ERR_UNSUPPORTED
     # empty problems succeed without touching the device
     assert lib.anygpu_gemm_f32(None, None, None, None, 0, 4, 8, 8, 4, 4, 0, 0, None) == capi.ANYGPU_OK
     assert lib.anygpu_softmax_rows_f32(None, None, 0, 16, 16, 16, 0, 0, 1.0, 0.0, 0, 0, None) == capi.ANYGPU_OK

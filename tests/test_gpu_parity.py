@@ -1470,12 +1470,9 @@ def test_sdp_attention_fused_kernel_gemma2_block(ops, oracle):
 # launches recorded into a HIP graph
 # =============================================================================================
 
-def test_launches_replayed_from_a_graph(ops, oracle):
-    # a stream is warmed up eagerly (which gives it the K-split workspace), then the same calls are captured on it and
-    # replayed three times with new input values and eager work in between; every replay must equal the eager result
+def _graph_problem(ops):
     import torch
     from anygpu_amd import capi
-    side = torch.cuda.Stream()
     a32 = torch.empty((24, 4096), device="cuda")
     w32 = dev(synth.uniform(1, (4096, 260)))                        # [K, N] fp32: band kernel, K split
     a16 = torch.empty((128, 2304), device="cuda", dtype=torch.float16)
@@ -1500,23 +1497,106 @@ def test_launches_replayed_from_a_graph(ops, oracle):
                 ops.tensor_causal_conv1d(cx, cw, cb),
                 ops.sdp_attention_fwd(q, kv, kv, 0.0884, softcap=30.0, causal=True, window=40))
 
+    return fill, work
+
+
+def test_launches_replayed_from_a_graph_with_a_caller_workspace(ops, oracle):
+    # A stream that has never run anything gets a caller's K-split workspace, the calls are captured on it and replayed
+    # three times with new input values and eager work in between.  The library allocates nothing (free device memory
+    # does not move), the workspace is written by the replays, and every replay equals the eager result of the default
+    # stream bit for bit, because with a workspace of the same size both make the same cuts.
+    import torch
+    from anygpu_amd import capi
+    fill, work = _graph_problem(ops)
+    side = torch.cuda.Stream()
+    ws_side = torch.full((capi.WORKSPACE_BYTES // 4,), float("nan"), device="cuda")
+    ws_main = torch.empty((capi.WORKSPACE_BYTES // 4,), device="cuda")
+    fill(10)
+    torch.cuda.synchronize()
+    ops.set_workspace(ws_side, side)
+    ops.set_workspace(ws_main)
+    try:
+        free_before = torch.cuda.mem_get_info()[0]
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            outs = work()
+        for rep in range(3):
+            fill(20 + 10 * rep)
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            got = [host(t).copy() for t in outs]
+            want = [host(t) for t in work()]                         # eager, on the default stream
+            torch.cuda.synchronize()
+            for g, w in zip(got, want):
+                assert np.array_equal(g, w)
+        assert not bool(torch.isnan(ws_side[:1024]).all()), "the replays did not use the workspace handed in"
+        # (torch's own pool may have grown by the small result tensors of work(): far less than a 64 MiB workspace)
+        assert free_before - torch.cuda.mem_get_info()[0] < capi.WORKSPACE_BYTES // 2
+    finally:
+        torch.cuda.synchronize()
+        ops.set_workspace(None, side)
+        ops.set_workspace(None)
+
+
+def test_captured_launches_without_a_workspace_run_uncut(ops, oracle):
+    # Under capture the library's own workspace is never used, warmed up or not: every product runs uncut, which is what
+    # an eager launch does whose workspace is too small for a single plane.  Both agree bit for bit, and with the cut
+    # result of an ordinary eager launch to the rounding of another order of summation.
+    import torch
+    fill, work = _graph_problem(ops)
+    side = torch.cuda.Stream()
     fill(10)
     with torch.cuda.stream(side):
-        work()
+        cut = [host(t).copy() for t in work()]                      # eager: allocates the stream's own workspace and cuts
     side.synchronize()
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph, stream=side):
         outs = work()
-    for rep in range(3):
-        fill(20 + 10 * rep)
+    tiny = torch.empty((64,), device="cuda")
+    ops.set_workspace(tiny)
+    try:
+        for rep in range(2):
+            fill(10 if rep == 0 else 40)
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            got = [host(t).copy() for t in outs]
+            want = [host(t) for t in work()]                         # eager and uncut: the workspace holds no plane
+            torch.cuda.synchronize()
+            for g, w in zip(got, want):
+                assert np.array_equal(g, w)
+            if rep == 0:
+                assert scaled_rel_err(got[0], cut[0], math.sqrt(4096) / 3.0) <= TOL_F32
+                assert scaled_rel_err(got[1].astype(np.float32), cut[1].astype(np.float32), math.sqrt(2304) / 3.0) <= TOL_F16_GEMM
+                assert not np.array_equal(got[0], cut[0]) or not np.array_equal(got[1], cut[1])
+    finally:
         torch.cuda.synchronize()
-        graph.replay()
-        torch.cuda.synchronize()
-        got = [host(t).copy() for t in outs]
-        want = [host(t) for t in work()]                             # eager, on the default stream
-        torch.cuda.synchronize()
-        for g, w in zip(got, want):
-            assert np.array_equal(g, w)
+        ops.set_workspace(None)
+        ops.set_workspace(None, side)
+
+
+def test_release_workspaces_returns_the_memory(ops):
+    import torch
+    from anygpu_amd import capi
+    ops.release_workspaces()
+    stream = torch.cuda.Stream()
+    a = dev(synth.uniform(1, (24, 8192)))
+    w = dev(synth.uniform(2, (260, 8192)))
+    torch.cuda.synchronize()
+    free0 = torch.cuda.mem_get_info()[0]
+    with torch.cuda.stream(stream):
+        ops.tensor_mm(a, w, b_layout=capi.B_COL_MAJOR)              # few rows, deep K: cut, into the library's own buffer
+    torch.cuda.synchronize()
+    free1 = torch.cuda.mem_get_info()[0]
+    assert free0 - free1 >= capi.WORKSPACE_BYTES
+    ops.release_workspaces()
+    assert torch.cuda.mem_get_info()[0] - free1 >= capi.WORKSPACE_BYTES
+    # and the stream simply gets a new one the next time
+    with torch.cuda.stream(stream):
+        again = ops.tensor_mm(a, w, b_layout=capi.B_COL_MAJOR)
+    assert np.isfinite(host(again)).all()
+    ops.release_workspaces()
 
 
 def test_k_split_products_on_concurrent_streams(ops, oracle):
