@@ -230,6 +230,18 @@ ANYGPU_EXPORT int anygpu_gemm_f16_f32acc(const void* A, const void* B, void* C,
 	return (int)anygpu::launch_gemm_f16(A, B, C, M, N, K, lda, ldb, ldc, 0, 0, 0, 1, b_layout, as_stream(stream));
 }
 
+ANYGPU_EXPORT int anygpu_gemm_f16_f32acc_probe(const void* A, const void* B, void* C,
+                                               int64_t M, int64_t N, int64_t K,
+                                               int64_t lda, int64_t ldb, int64_t ldc,
+                                               int b_layout, uint64_t* probe, void* stream)
+{
+	const int rc = check_gemm(A, B, C, M, N, K, lda, ldb, ldc, ANYGPU_A_ROW_MAJOR, b_layout);
+	if (rc != ANYGPU_OK) return rc;
+	if (probe == nullptr) return ANYGPU_ERR_NULL_POINTER;
+	if (!anygpu::gemm_f16_probe_applies(A, B, C, M, N, K, lda, ldb, ldc, b_layout)) return ANYGPU_ERR_UNSUPPORTED;
+	return (int)anygpu::launch_gemm_f16_probe(A, B, C, M, N, K, lda, ldb, ldc, reinterpret_cast<unsigned long long*>(probe), as_stream(stream));
+}
+
 ANYGPU_EXPORT int anygpu_gemm_f16_f32acc_batched(const void* A, const void* B, void* C,
                                                  int64_t M, int64_t N, int64_t K,
                                                  int64_t lda, int64_t ldb, int64_t ldc,

@@ -215,6 +215,20 @@ __global__ __launch_bounds__(256) void gemm_f16_split_merge_kernel(
 	*reinterpret_cast<LooseHalf8*>(C + m * ldc + n) = out;      // rows of C may start at any element
 }
 
+bool gemm_f16_probe_applies(const void* A, const void* B, const void* C, int64_t M, int64_t N, int64_t K,
+                            int64_t lda, int64_t ldb, int64_t ldc, int b_layout)
+{
+	return b_layout == ANYGPU_B_COL_MAJOR && reinterpret_cast<uintptr_t>(C) % 16 == 0 && ldc % 8 == 0 &&
+	       gemm_f16_ring_applies(static_cast<const half_t*>(A), static_cast<const half_t*>(B), M, N, K, lda, ldb, 0, 0, 1);
+}
+
+hipError_t launch_gemm_f16_probe(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K,
+                                 int64_t lda, int64_t ldb, int64_t ldc, unsigned long long* probe, hipStream_t stream)
+{
+	return launch_gemm_f16_ring(static_cast<const half_t*>(A), static_cast<const half_t*>(B), static_cast<half_t*>(C), M, N, K,
+	                            lda, ldb, ldc, 0, 0, 0, 1, stream, probe);
+}
+
 hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K,
                            int64_t lda, int64_t ldb, int64_t ldc,
                            int64_t stride_a, int64_t stride_b, int64_t stride_c, int64_t batch,

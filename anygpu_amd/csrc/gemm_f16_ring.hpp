@@ -26,10 +26,13 @@ struct GemmRingCfg
 };
 
 // blockIdx.y walks a batch of independent products that share the shape.  M and N multiples of 256, K of 64.
+// probe (may be NULL; first product of a batch only): lane 0 of every block leaves the shader clock count (s_memtime) and
+// the constant 100 MHz count (s_memrealtime) at entry and exit of its main loop in probe[4 block .. + 3], from which a
+// caller gets the clock the part sustained under this kernel and the share of those cycles the matrix cores were busy.
 __global__ __launch_bounds__(256) void gemm_f16_nt_ring_kernel(
 	const half_t* __restrict__ A, const half_t* __restrict__ B, half_t* __restrict__ C,
 	int K, int64_t lda, int64_t ldb, int64_t ldc, int tiles_m, int tiles_n,
-	int64_t stride_a, int64_t stride_b, int64_t stride_c)
+	int64_t stride_a, int64_t stride_b, int64_t stride_c, unsigned long long* __restrict__ probe)
 {
 	using Cfg = GemmRingCfg;
 	extern __shared__ __align__(1024) char lds[];
@@ -72,6 +75,12 @@ __global__ __launch_bounds__(256) void gemm_f16_nt_ring_kernel(
 
 	// The accumulators leave the block as eight vectors of 32 registers pinned to a[0:255]: row i of the patch's MFMA
 	// tiles in vector i.
+	unsigned long long clock_in = 0, ticks_in = 0;
+	if (probe != nullptr)
+	{
+		clock_in = __builtin_amdgcn_s_memtime();
+		ticks_in = __builtin_amdgcn_s_memrealtime();
+	}
 	float32x_t r0, r1, r2, r3, r4, r5, r6, r7;
 	asm volatile(
 #include "gemm_f16_ring_loop.inc"
@@ -98,6 +107,18 @@ __global__ __launch_bounds__(256) void gemm_f16_nt_ring_kernel(
 		  "v250", "v251", "v252", "v253", "v254", "v255", "s60", "s61", "s62", "s63", "s64", "s65", "s66", "s67", "s68",
 		  "s69", "s70", "s71", "s72", "scc", "m0", "memory");
 
+	if (probe != nullptr)
+	{
+		const unsigned long long clock_out = __builtin_amdgcn_s_memtime(), ticks_out = __builtin_amdgcn_s_memrealtime();
+		if (tid == 0 && blockIdx.y == 0)
+		{
+			unsigned long long* slot = probe + 4 * (size_t)blockIdx.x;
+			slot[0] = clock_in;
+			slot[1] = clock_out;
+			slot[2] = ticks_in;
+			slot[3] = ticks_out;
+		}
+	}
 	float4_t acc[8][8];
 	const float32x_t* rows[8] = {&r0, &r1, &r2, &r3, &r4, &r5, &r6, &r7};
 #pragma unroll
@@ -122,7 +143,8 @@ inline bool gemm_f16_ring_applies(const half_t* A, const half_t* B, int64_t M, i
 
 inline hipError_t launch_gemm_f16_ring(const half_t* A, const half_t* B, half_t* C, int64_t M, int64_t N, int64_t K,
                                        int64_t lda, int64_t ldb, int64_t ldc,
-                                       int64_t stride_a, int64_t stride_b, int64_t stride_c, int64_t batch, hipStream_t stream)
+                                       int64_t stride_a, int64_t stride_b, int64_t stride_c, int64_t batch, hipStream_t stream,
+                                       unsigned long long* probe = nullptr)
 {
 	auto kernel = gemm_f16_nt_ring_kernel;
 	// More than 64 KB of dynamic LDS has to be granted per function and per device, once.
@@ -140,7 +162,7 @@ inline hipError_t launch_gemm_f16_ring(const half_t* A, const half_t* B, half_t*
 	}
 	const int tiles_m = (int)(M / 256), tiles_n = (int)(N / 256);
 	kernel<<<dim3((unsigned)(tiles_m * tiles_n), (unsigned)batch), dim3(256), GemmRingCfg::kLdsBytes, stream>>>(
-		A, B, C, (int)K, lda, ldb, ldc, tiles_m, tiles_n, stride_a, stride_b, stride_c);
+		A, B, C, (int)K, lda, ldb, ldc, tiles_m, tiles_n, stride_a, stride_b, stride_c, probe);
 	return hipGetLastError();
 }
 

@@ -39,6 +39,13 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
                            int64_t stride_a, int64_t stride_b, int64_t stride_c, int64_t batch,
                            int b_layout, hipStream_t stream);
 
+// The fp16 product through the four-wave 256 x 256 tile kernel with its clock probe (see gemm_f16_ring.hpp); false /
+// nothing launched when the product does not meet that kernel's conditions.
+bool gemm_f16_probe_applies(const void* A, const void* B, const void* C, int64_t M, int64_t N, int64_t K,
+                            int64_t lda, int64_t ldb, int64_t ldc, int b_layout);
+hipError_t launch_gemm_f16_probe(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K,
+                                 int64_t lda, int64_t ldb, int64_t ldc, unsigned long long* probe, hipStream_t stream);
+
 hipError_t launch_gemm_f32(const float* A, const float* B, const float* bias, float* C,
                            int64_t M, int64_t N, int64_t K,
                            int64_t lda, int64_t ldb, int64_t ldc,

@@ -30,3 +30,16 @@ def uniform(seed: int, shape, lo: float = -1.0, hi: float = 1.0, dtype=np.float3
 def integers(seed: int, shape, lo: int, hi: int, dtype=np.float32) -> np.ndarray:
     """Integer values in [lo, hi] stored in a floating type (exact sums, order independent)."""
     return _gen(seed).integers(lo, hi + 1, size=shape).astype(dtype)
+
+
+def normal_matrix_f16(seed: int, rows: int, cols: int, std: float = 1.0, slab_rows: int = 8192) -> np.ndarray:
+    """N(0, std) as float16 [rows, cols], drawn in float32 in slabs of rows from one stream and rounded once: the large
+    score matrices of the softmax configurations without a float32 copy of the whole."""
+    out = np.empty((rows, cols), dtype=np.float16)
+    gen = _gen(seed)
+    for r0 in range(0, rows, slab_rows):
+        blk = gen.standard_normal(size=(min(slab_rows, rows - r0), cols), dtype=np.float32)
+        if std != 1.0:
+            blk *= np.float32(std)
+        out[r0:r0 + blk.shape[0]] = blk
+    return out

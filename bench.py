@@ -3,16 +3,23 @@
 
 Headline (one JSON line on stdout): fp16 GEMM M = N = K = 4096, A row-major, B column-major,
 fp32 accumulate, fp16 output -- TFLOP/s, with the roofline of that kernel and the CPU oracle
-timed next to it.  The memory-bound kernels of the same path (Zamba2-shaped causal conv1d +
+timed next to it.  The other kernels of the path (fp32 GEMM 2048^3, Zamba2-shaped causal conv1d +
 SiLU, causal softmax 32 x 2048 x 2048, Gemma2 softmax 8 x 8192 x 8192 with softcap and sliding
-window) are measured in the same run and reported under "kernels", each with its own roofline
-object (dense algorithmic bytes / average launch time against 8 TB/s).
+window, and the callers either side: fused attention, decode attention, gated RMS norm) are
+measured in the same run and reported under "kernels", each with its own roofline object and,
+for the configurations the metric names, the CPU oracle timed on a bounded sample.
 
 A step is one launch of the kernel over one batch of synthetic input that is already resident
-in HBM.  Timing: W untimed warm-up steps, then exactly K steps between two device
-synchronisations (host clock -> `value`) and between two HIP events recorded on the launch
-stream (-> `roofline.achieved`).  The memory-bound kernels rotate over several buffer sets so
-that the working set exceeds the 256 MB Infinity Cache.
+in HBM.  Inputs are drawn on the host by anygpu_amd.synth with the stated seeds (the generator of
+the parity tests).  Timing of every kernel:
+  * W untimed warm-up steps, then exactly K steps between two device synchronisations (host
+    clock -> `value` of the headline) and between two HIP events recorded on the launch stream
+    (-> `us_per_launch`, `roofline.achieved`); for the kernels under "kernels", whose K is a
+    fraction of --steps, K is never below 20;
+  * then the same number of launches (at least 20, at most 200) with an event pair around every
+    single launch -> `median_us`, `min_us` (these leave out the gap between two launches).
+The memory-bound kernels rotate over several buffer sets so that the working set exceeds the
+256 MB Infinity Cache.
 """
 from __future__ import annotations
 
@@ -20,6 +27,7 @@ import argparse
 import json
 import math
 import os
+import statistics
 import sys
 import time
 from pathlib import Path
@@ -28,17 +36,32 @@ REPO = Path(__file__).resolve().parent
 if str(REPO) not in sys.path:
     sys.path.insert(0, str(REPO))
 
+PEAK_CLOCK_GHZ = 2.4
+FP16_FLOP_PER_CLK_PER_CU = 4096
 PEAK_FP16_TFLOPS = 2516.6      # dense fp16 MFMA, 256 CU x 4096 flop/clk/CU x 2.4 GHz
 PEAK_FP32_TFLOPS = 157.3       # fp32 matrix path
 PEAK_HBM_GBS = 8000.0          # HBM3E
+MIN_TIMED_LAUNCHES = 20
 
-# Bytes per launch moved behind the L2s, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE (KiB per
-# dispatch), scaled by what the same counters read for a plain 256 MiB device copy (fetch x 2.000,
-# write x 1.000); the summaries are under profiles/.
-MEASURED_TRAFFIC_BYTES = {"gemm_f16": 234962687, "gemm_f32": 167994164, "conv1d": 277226336,
-                          "softmax_causal": 410887952, "softmax_gemma2": 1514268488,
-                          "attention_gemma2": 188478908, "attention_gemma2_f32": 887738788, "gated_rmsnorm": 805513216,
-                          "attention_decode": 144061440}
+# Bytes per launch moved behind the L2s: NOT measured by this run.  They come from two rocprofv3 --pmc runs of this
+# command (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), scaled by what the same counters read for a plain 256 MiB
+# device copy (fetch x 2.000, write x 1.000); the summary each figure is copied from is named beside it.
+MEASURED_TRAFFIC = {
+    "gemm_f16": (234397696, "profiles/gemm_f16_4096_ring_kernel.md"),
+    "gemm_f32": (167994164, "profiles/gemm_f32_2048_kernel.md"),
+    "conv1d": (277226336, "profiles/causal_conv1d_silu_zamba2_tile_kernel.md"),
+    "softmax_causal": (410887952, "profiles/softmax_causal_32x2048x2048_window_kernel.md"),
+    "softmax_gemma2": (1514268488, "profiles/softmax_gemma2_8x8192x8192_window_kernel.md"),
+    "attention_gemma2": (188478908, "profiles/sdp_attention_fwd_f16_gemma2_kernel.md"),
+    "attention_gemma2_f32": (887738788, "profiles/sdp_attention_fwd_f32_gemma2_kernel.md"),
+    "gated_rmsnorm": (805513216, "profiles/gated_rmsnorm_f16_row_kernel.md"),
+    "attention_decode": (144061440, "profiles/sdp_attention_decode_f16_partial_and_merge_kernels.md"),
+}
+
+
+def traffic_fields(key):
+    nbytes, source = MEASURED_TRAFFIC[key]
+    return {"traffic": nbytes, "traffic_source": f"{source} (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this command; copied, not measured in this run)"}
 
 
 def parse_args():
@@ -47,7 +70,8 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--cpu-seconds", type=float, default=12.0,
-                    help="target wall time of the CPU-oracle sample (0 disables the CPU baseline)")
+                    help="target wall time of the CPU-oracle sample of the headline (0 disables every CPU baseline); "
+                         "the other configurations get a quarter of it each")
     ap.add_argument("--only", default="", help="comma list of: gemm,gemm32,conv,softmax,attn,attn32,decode,norm (default: all)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain device copy of 256 MiB (read 256 MiB + write 256 MiB) a few times, "
@@ -58,13 +82,15 @@ def parse_args():
 SETTLE_SECONDS = 0.3
 
 
-def timed_region(torch, fn, steps, warmup):
-    """(host seconds, event seconds) for `steps` calls of fn after `warmup` untimed calls.
+def timed_region(torch, fn, steps, warmup, floor=MIN_TIMED_LAUNCHES):
+    """Timing of `fn`: a dict with the host and event time of `steps` back-to-back calls (after the settle period and
+    `warmup` untimed calls) and the median / minimum of per-launch event pairs.
 
     Before the warm-up the kernel runs untimed for SETTLE_SECONDS: after an idle period the
     power management of the GPU over- and undershoots for some tens of milliseconds (a 4096^3
-    GEMM takes 124 us, then up to 160 us, then settles near 100 us after about 150 launches), and
+    GEMM takes 124 us, then up to 160 us, then settles near 95 us after about 150 launches), and
     the number that matters for a long-running job is the settled one."""
+    steps = max(int(steps), floor)
     t_end = time.perf_counter() + SETTLE_SECONDS
     while time.perf_counter() < t_end:
         for _ in range(20):
@@ -81,49 +107,143 @@ def timed_region(torch, fn, steps, warmup):
     stop.record()
     torch.cuda.synchronize()
     t1 = time.perf_counter()
-    return t1 - t0, start.elapsed_time(stop) * 1e-3
+    singles = min(max(steps, MIN_TIMED_LAUNCHES), 200)
+    pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(singles)]
+    for a, b in pairs:
+        a.record()
+        fn()
+        b.record()
+    torch.cuda.synchronize()
+    each = sorted(a.elapsed_time(b) * 1e3 for a, b in pairs)
+    return {"steps": steps, "host_s": t1 - t0, "event_s": start.elapsed_time(stop) * 1e-3,
+            "us_per_launch": start.elapsed_time(stop) * 1e3 / steps,
+            "median_us": statistics.median(each), "min_us": each[0], "single_launches": singles}
 
+
+def timing_fields(t):
+    return {"us_per_launch": t["us_per_launch"], "median_us": t["median_us"], "min_us": t["min_us"],
+            "timed_launches": t["steps"], "single_launches": t["single_launches"]}
+
+
+def sized_sample(run, unit_cost_probe, total_units, target_seconds):
+    """Run `run(units)` on as many units as fit `target_seconds`, sized from a short probe; (units, seconds)."""
+    probe_units = max(1, unit_cost_probe)
+    t0 = time.perf_counter()
+    run(probe_units)
+    per_unit = (time.perf_counter() - t0) / probe_units
+    units = int(max(probe_units, min(total_units, target_seconds / max(per_unit, 1e-9))))
+    t0 = time.perf_counter()
+    run(units)
+    return units, time.perf_counter() - t0
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# GEMM
+# ---------------------------------------------------------------------------------------------------------------
 
 def bench_gemm_f16(torch, ops, capi, synth, steps, warmup):
     n = 4096
     a = torch.from_numpy(synth.uniform(0, (n, n)).astype("float16")).cuda()
     bt = torch.from_numpy(synth.uniform(1, (n, n)).astype("float16")).cuda()   # B stored [N, K]
     c = torch.empty((n, n), dtype=torch.float16, device="cuda")
-    host_s, ev_s = timed_region(torch, lambda: ops.tensor_mm(a, bt, out=c, b_layout=capi.B_COL_MAJOR), steps, warmup)
+    # (the headline times exactly --steps launches; only the kernels below are floored)
+    t = timed_region(torch, lambda: ops.tensor_mm(a, bt, out=c, b_layout=capi.B_COL_MAJOR), steps, warmup, floor=1)
     flops = 2.0 * n ** 3
+    # the clock the part sustains under this kernel and the matrix cores' share of those cycles, from the kernel's own
+    # counters (anygpu_gemm_f16_f32acc_probe): launched for another settle period, the last launch read
+    lib = capi.load()
+    tiles = (n // 256) ** 2
+    probe = torch.zeros((tiles, 4), dtype=torch.int64, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+    t_end = time.perf_counter() + SETTLE_SECONDS
+    while time.perf_counter() < t_end:
+        for _ in range(20):
+            capi.check("anygpu_gemm_f16_f32acc_probe",
+                       lib.anygpu_gemm_f16_f32acc_probe(a.data_ptr(), bt.data_ptr(), c.data_ptr(), n, n, n, n, n, n,
+                                                        capi.B_COL_MAJOR, probe.data_ptr(), stream))
+        torch.cuda.synchronize()
+    p = probe.cpu().double()
+    cycles, ns = p[:, 1] - p[:, 0], (p[:, 3] - p[:, 2]) * 10.0
+    clock_ghz = float((cycles / ns).mean())
+    busy = float(((n // 32) * 64 * 16 / cycles).mean())
     return {
-        "host_s": host_s, "event_s": ev_s, "flops": flops,
-        "tflops_host": flops * steps / host_s / 1e12,
-        "tflops_event": flops * steps / ev_s / 1e12,
+        "timing": t, "flops": flops,
+        "tflops_host": flops * t["steps"] / t["host_s"] / 1e12,
+        "tflops_event": flops * t["steps"] / t["event_s"] / 1e12,
         "operands": (a, bt),
+        "clock": {"sustained_clock_ghz": clock_ghz, "mfma_busy_in_main_loop": busy,
+                  "main_loop_us_mean": float(ns.mean() / 1e3), "main_loop_us_max": float(ns.max() / 1e3),
+                  "main_loop_us_min": float(ns.min() / 1e3),
+                  "source": "s_memtime / s_memrealtime around the main loop of every tile (anygpu_gemm_f16_f32acc_probe), "
+                            "last launch of a settle period of back-to-back launches after the timed region"},
     }
 
 
-def bench_gemm_f32(torch, ops, synth, steps, warmup):
-    n = 2048
-    a = torch.from_numpy(synth.uniform(0, (n, n))).cuda()
-    b = torch.from_numpy(synth.uniform(1, (n, n))).cuda()
-    c = torch.empty((n, n), dtype=torch.float32, device="cuda")
-    host_s, ev_s = timed_region(torch, lambda: ops.tensor_mm(a, b, out=c), steps, warmup)
-    flops = 2.0 * n ** 3
-    t = ev_s / steps
+def cpu_baseline_gemm(oracle, a32, b_view, target_seconds, what):
+    """The oracle's tensor_mm (1 thread, the reference's loop order) on the first R rows of the problem; R is sized from a
+    short probe so that the sample takes about `target_seconds`.  Also times rows spread over all host cores."""
+    m, k = a32.shape
+    n = b_view.shape[1]
+
+    def run(rows, threads=1):
+        oracle.tensor_mm(a32[:rows], b_view, threads=threads)
+
+    rows, t1 = sized_sample(run, 2, m, target_seconds)
+    flops = 2.0 * rows * n * k
+    cores = min(oracle.max_threads(), int(os.environ.get("OMP_NUM_THREADS", "16") or 16), 16)
+    rows_mt = min(m, rows * cores)
+    t0 = time.perf_counter()
+    run(rows_mt, cores)
+    tn = time.perf_counter() - t0
     return {
-        "name": "gemm_f32", "workload": "fp32 GEMM M=N=K=2048, row-major operands, U(-1,1)",
-        "us_per_launch": t * 1e6, "value": flops / t / 1e12, "unit": "TFLOP/s", "dtype": "f32",
-        "roofline": {"bound": "mfma", "achieved": flops / t / 1e12, "peak": PEAK_FP32_TFLOPS, "unit": "TFLOP/s",
-                     "frac": flops / t / 1e12 / PEAK_FP32_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES["gemm_f32"]},
+        "value": flops / t1 / 1e12, "unit": "TFLOP/s", "cores": 1, "kind": "port",
+        "sample": f"rows 0..{rows - 1} of C ({rows} x {n} x {k} MACs) of {what}, reference loop order, float32 accumulator, "
+                  f"{t1:.1f} s" + ("" if rows == m else "; a row sample, the whole product extrapolates linearly"),
+        "all_cores": {"value": 2.0 * rows_mt * n * k / tn / 1e12, "unit": "TFLOP/s", "cores": cores,
+                      "sample": f"rows 0..{rows_mt - 1}, outer rows split over {cores} threads, {tn:.1f} s"},
     }
 
 
-def bench_conv1d(torch, ops, steps, warmup):
+def bench_gemm_f32(torch, ops, synth, steps, warmup, cpu_seconds):
+    n = 2048
+    a_host, b_host = synth.uniform(0, (n, n)), synth.uniform(1, (n, n))
+    a, b = torch.from_numpy(a_host).cuda(), torch.from_numpy(b_host).cuda()
+    c = torch.empty((n, n), dtype=torch.float32, device="cuda")
+    t = timed_region(torch, lambda: ops.tensor_mm(a, b, out=c), steps, warmup)
+    flops = 2.0 * n ** 3
+    sec = t["us_per_launch"] * 1e-6
+    out = {
+        "name": "gemm_f32", "workload": "fp32 GEMM M=N=K=2048, row-major operands, U(-1,1), seeds 0 / 1 (BASELINE.json configs[1], fp32 variant)",
+        **timing_fields(t), "value": flops / sec / 1e12, "unit": "TFLOP/s", "dtype": "f32",
+        "roofline": {"bound": "mfma", "achieved": flops / sec / 1e12, "peak": PEAK_FP32_TFLOPS, "unit": "TFLOP/s",
+                     "frac": flops / sec / 1e12 / PEAK_FP32_TFLOPS, **traffic_fields("gemm_f32"), "algorithmic_flops": flops},
+    }
+    if cpu_seconds > 0:
+        import oracle
+        out["cpu_baseline"] = cpu_baseline_gemm(oracle, a_host, b_host, cpu_seconds, "the same 2048^3 inputs")
+    return out
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# conv1d, softmax
+# ---------------------------------------------------------------------------------------------------------------
+
+def rotation(torch, first, nbuf):
+    """`nbuf` buffer sets for a memory-bound kernel: the seeded tensor and copies of it rolled by whole rows (same
+    values at other addresses), so that consecutive launches do not find their input in the Infinity Cache."""
+    return [first] + [torch.roll(first, shifts=i, dims=0) for i in range(1, nbuf)]
+
+
+def bench_conv1d(torch, ops, synth, steps, warmup, cpu_seconds):
+    import numpy as np
     b, d, s, width = 4, 4224, 4096, 4
     nbuf = 4                                     # 4 x 277 MB of x + y: well past the Infinity Cache
-    g = torch.Generator(device="cuda")
-    g.manual_seed(0)
-    xs = [torch.randn((b, d, s), device="cuda", generator=g).half() for _ in range(nbuf)]
+    x_host = synth.normal(0, (b, d, s)).astype(np.float16)
+    w_host = synth.normal(1, (d, width), std=0.5).astype(np.float16)
+    b_host = synth.normal(2, (d,), std=0.1).astype(np.float16)
+    xs = rotation(torch, torch.from_numpy(x_host).cuda(), nbuf)
     ys = [torch.empty_like(x) for x in xs]
-    w = (torch.randn((d, width), device="cuda", generator=g) * 0.5).half()
-    bias = (torch.randn((d,), device="cuda", generator=g) * 0.1).half()
+    w, bias = torch.from_numpy(w_host).cuda(), torch.from_numpy(b_host).cuda()
     it = [0]
 
     def step():
@@ -131,24 +251,40 @@ def bench_conv1d(torch, ops, steps, warmup):
         it[0] += 1
         ops.tensor_causal_conv1d(xs[i], w, bias, out=ys[i])
 
-    host_s, ev_s = timed_region(torch, step, steps, warmup)
+    t = timed_region(torch, step, steps, warmup)
     nbytes = 2 * b * d * s * 2 + d * width * 2 + d * 2
-    t = ev_s / steps
-    return {
+    sec = t["us_per_launch"] * 1e-6
+    out = {
         "name": "causal_conv1d_silu_f16",
-        "workload": "Zamba2-1.2B conv1d + SiLU: x fp16 [4, 4224, 4096], w [4224, 4], bias [4224], left pad 3",
-        "us_per_launch": t * 1e6, "value": nbytes / t / 1e9, "unit": "GB/s", "dtype": "f16",
-        "roofline": {"bound": "hbm", "achieved": nbytes / t / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                     "frac": nbytes / t / 1e9 / PEAK_HBM_GBS, "traffic": MEASURED_TRAFFIC_BYTES["conv1d"],
-                     "algorithmic_bytes": nbytes},
+        "workload": "Zamba2-1.2B conv1d + SiLU: x fp16 [4, 4224, 4096] N(0,1) seed 0, w [4224, 4] N(0,0.5) seed 1, bias [4224] "
+                    "N(0,0.1) seed 2, left pad 3 (BASELINE.json configs[2]); 4 rotating buffer sets",
+        **timing_fields(t), "value": nbytes / sec / 1e9, "unit": "GB/s", "dtype": "f16",
+        "roofline": {"bound": "hbm", "achieved": nbytes / sec / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": nbytes / sec / 1e9 / PEAK_HBM_GBS, **traffic_fields("conv1d"), "algorithmic_bytes": nbytes},
     }
+    if cpu_seconds > 0:
+        import oracle
+        x32 = oracle.cvt_f16_to_f32(x_host[0])[None]          # batch 0: [1, d, s]
+        w32, b32 = oracle.cvt_f16_to_f32(w_host), oracle.cvt_f16_to_f32(b_host)
+
+        def run(chans):
+            oracle.tensor_causal_conv1d(x32[:, :chans], w32[:chans], b32[:chans])
+
+        chans, sec_cpu = sized_sample(run, 8, d, cpu_seconds)
+        sample_bytes = 2 * chans * s * 2 + chans * width * 2 + chans * 2
+        out["cpu_baseline"] = {
+            "value": sample_bytes / sec_cpu / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": f"channels 0..{chans - 1} of batch 0 ({chans} rows of 4096 samples; fp16 inputs up-cast to float32 as the "
+                      f"reference's tests do) of the same inputs, {sec_cpu:.1f} s; algorithmic fp16 bytes of those rows over the "
+                      f"time, the whole tensor ({b * d} rows) extrapolates linearly"}
+    return out
 
 
-def bench_softmax(torch, ops, steps, warmup, *, name, heads, q, k, std, alpha, cap, window, nbuf, workload, key):
-    g = torch.Generator(device="cuda")
-    g.manual_seed(0)
+def bench_softmax(torch, ops, synth, steps, warmup, cpu_seconds, *, name, heads, q, k, std, alpha, cap, window, nbuf, workload, key):
+    import numpy as np
     rows = heads * q
-    xs = [(torch.randn((rows, k), device="cuda", generator=g) * std).half() for _ in range(nbuf)]
+    x_host = synth.normal_matrix_f16(0, rows, k, std)
+    xs = rotation(torch, torch.from_numpy(x_host).cuda(), nbuf)
     ys = [torch.empty_like(x) for x in xs]
     it = [0]
 
@@ -157,80 +293,82 @@ def bench_softmax(torch, ops, steps, warmup, *, name, heads, q, k, std, alpha, c
         it[0] += 1
         ops.tensor_softmax(xs[i], out=ys[i], alpha=alpha, softcap=cap, causal=True, window=window, q_len=q)
 
-    host_s, ev_s = timed_region(torch, step, steps, warmup)
+    t = timed_region(torch, step, steps, warmup)
     dense = 2 * rows * k * 2                        # read every score once, write every probability once
     i = torch.arange(q, dtype=torch.int64)
     visible = torch.minimum(i + 1, torch.tensor(window if window > 0 else q)).sum().item() * heads
     mask_aware = visible * 2 + rows * k * 2         # reads of visible keys only + full write
-    t = ev_s / steps
-    return {
+    sec = t["us_per_launch"] * 1e-6
+    out = {
         "name": name, "workload": workload,
-        "us_per_launch": t * 1e6, "value": dense / t / 1e9, "unit": "GB/s", "dtype": "f16",
-        "roofline": {"bound": "hbm", "achieved": dense / t / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                     "frac": dense / t / 1e9 / PEAK_HBM_GBS, "traffic": MEASURED_TRAFFIC_BYTES[key],
+        **timing_fields(t), "value": dense / sec / 1e9, "unit": "GB/s", "dtype": "f16",
+        "roofline": {"bound": "hbm", "achieved": dense / sec / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": dense / sec / 1e9 / PEAK_HBM_GBS, **traffic_fields(key),
                      "algorithmic_bytes": dense, "mask_aware_bytes": mask_aware,
-                     "mask_aware_gbs": mask_aware / t / 1e9},
+                     "mask_aware_gbs": mask_aware / sec / 1e9, "physical_gbs": MEASURED_TRAFFIC[key][0] / sec / 1e9},
     }
+    if cpu_seconds > 0:
+        import oracle
+        # every (rows / n)-th row, so that short and long visible ranges are sampled alike; a row travels alone, with
+        # its query index as the diagonal shift
+        def run(n):
+            idx = np.linspace(0, rows - 1, n).astype(np.int64)
+            x32 = oracle.cvt_f16_to_f32(x_host[idx])
+            for tt, r in enumerate(idx):
+                oracle.attention_softmax(x32[tt:tt + 1], alpha=alpha, softcap=cap, causal=True, window=window, q_len=0, diag=int(r % q))
+
+        n, sec_cpu = sized_sample(run, 16, rows, cpu_seconds)
+        out["cpu_baseline"] = {
+            "value": n * 2 * k * 2 / sec_cpu / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": f"{n} rows spread evenly over the {rows} of the same inputs (fp16 up-cast to float32; scale, softcap, mask and "
+                      f"softmax in the reference's arithmetic: exp in double, sum in float32), {sec_cpu:.1f} s; dense fp16 bytes "
+                      f"of those rows over the time, the whole matrix extrapolates linearly"}
+    return out
 
 
-def bench_attention(torch, ops, steps, warmup):
+# ---------------------------------------------------------------------------------------------------------------
+# the callers either side of the path
+# ---------------------------------------------------------------------------------------------------------------
+
+def attention_inputs(torch, synth, h, hkv, n, d, dtype):
+    q = torch.from_numpy(synth.normal(1, (1, h, n, d)).astype(dtype)).cuda()
+    k = torch.from_numpy(synth.normal(2, (1, hkv, n, d)).astype(dtype)).cuda()
+    v = torch.from_numpy(synth.normal(3, (1, hkv, n, d)).astype(dtype)).cuda()
+    return q, k, v
+
+
+def bench_attention(torch, ops, synth, steps, warmup, dtype):
     # Gemma2 attention block at the shape of the softmax headline configuration: 8 query heads over 4 key / value
-    # heads, 8192 positions, head_dim 256, scale 1 / 16, softcap 50, causal + window 4096, one fused kernel
+    # heads, 8192 positions, head_dim 256, scale 1 / 16, softcap 50, causal + window 4096, one fused kernel.  fp16, and
+    # float32 (the precision the reference runs Gemma2 in: fp32 operands, fp32 MFMA).
     h, hkv, n, d, win = 8, 4, 8192, 256, 4096
-    g = torch.Generator(device="cuda")
-    g.manual_seed(0)
-    q = torch.randn((1, h, n, d), device="cuda", generator=g).half()
-    k = torch.randn((1, hkv, n, d), device="cuda", generator=g).half()
-    v = torch.randn((1, hkv, n, d), device="cuda", generator=g).half()
-    host_s, ev_s = timed_region(torch, lambda: ops.sdp_attention_fwd(q, k, v, 1.0 / 16.0, softcap=50.0, causal=True, window=win),
-                                steps, warmup)
+    q, k, v = attention_inputs(torch, synth, h, hkv, n, d, "float16" if dtype == "f16" else "float32")
+    t = timed_region(torch, lambda: ops.sdp_attention_fwd(q, k, v, 1.0 / 16.0, softcap=50.0, causal=True, window=win), steps, warmup)
     pairs = win * (win + 1) // 2 + (n - win) * win          # visible (query, key) pairs per head
     flops = 4.0 * d * pairs * h                             # q k^T and p v, 2 flop per multiply-add
-    t = ev_s / steps
+    sec = t["us_per_launch"] * 1e-6
+    peak = PEAK_FP16_TFLOPS if dtype == "f16" else PEAK_FP32_TFLOPS
     return {
-        "name": "sdp_attention_fwd_f16",
-        "workload": "fused attention fp16 q [1, 8, 8192, 256], k / v [1, 4, 8192, 256], x 1/16, softcap 50, causal + window 4096",
-        "us_per_launch": t * 1e6, "value": flops / t / 1e12, "unit": "TFLOP/s", "dtype": "f16",
-        "roofline": {"bound": "mfma", "achieved": flops / t / 1e12, "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": flops / t / 1e12 / PEAK_FP16_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES["attention_gemma2"],
+        "name": f"sdp_attention_fwd_{dtype}",
+        "workload": f"fused attention {'fp16' if dtype == 'f16' else 'fp32'} q [1, 8, 8192, 256], k / v [1, 4, 8192, 256] N(0,1) seeds 1 / 2 / 3, "
+                    "x 1/16, softcap 50, causal + window 4096",
+        **timing_fields(t), "value": flops / sec / 1e12, "unit": "TFLOP/s", "dtype": dtype,
+        "roofline": {"bound": "mfma", "achieved": flops / sec / 1e12, "peak": peak, "unit": "TFLOP/s",
+                     "frac": flops / sec / 1e12 / peak,
+                     **traffic_fields("attention_gemma2" if dtype == "f16" else "attention_gemma2_f32"),
                      "algorithmic_flops": flops, "visible_pairs_per_head": pairs},
     }
 
 
-def bench_attention_f32(torch, ops, steps, warmup):
-    # the same block in float32 (the precision the reference runs Gemma2 in): fp32 operands, fp32 MFMA
-    h, hkv, n, d, win = 8, 4, 8192, 256, 4096
-    g = torch.Generator(device="cuda")
-    g.manual_seed(0)
-    q = torch.randn((1, h, n, d), device="cuda", generator=g)
-    k = torch.randn((1, hkv, n, d), device="cuda", generator=g)
-    v = torch.randn((1, hkv, n, d), device="cuda", generator=g)
-    host_s, ev_s = timed_region(torch, lambda: ops.sdp_attention_fwd(q, k, v, 1.0 / 16.0, softcap=50.0, causal=True, window=win),
-                                steps, warmup)
-    pairs = win * (win + 1) // 2 + (n - win) * win
-    flops = 4.0 * d * pairs * h
-    t = ev_s / steps
-    return {
-        "name": "sdp_attention_fwd_f32",
-        "workload": "fused attention fp32 q [1, 8, 8192, 256], k / v [1, 4, 8192, 256], x 1/16, softcap 50, causal + window 4096",
-        "us_per_launch": t * 1e6, "value": flops / t / 1e12, "unit": "TFLOP/s", "dtype": "f32",
-        "roofline": {"bound": "mfma", "achieved": flops / t / 1e12, "peak": PEAK_FP32_TFLOPS, "unit": "TFLOP/s",
-                     "frac": flops / t / 1e12 / PEAK_FP32_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES["attention_gemma2_f32"],
-                     "algorithmic_flops": flops, "visible_pairs_per_head": pairs},
-    }
-
-
-def bench_attention_decode(torch, capi, steps, warmup):
+def bench_attention_decode(torch, capi, synth, steps, warmup):
     # One generation step against a long cache: 64 query heads over 8 key / value heads, 32768 cached positions,
     # head_dim 128, causal.  The split-key decode form through the C ABI with the caller's workspace: two launches
     # (partial results per split, merge), timed together; the bytes are the K and V caches, read once.
     h, hkv, n_k, d = 64, 8, 32768, 128
     lib = capi.load()
-    g = torch.Generator(device="cuda")
-    g.manual_seed(0)
-    q = torch.randn((1, h, 1, d), device="cuda", generator=g).half()
-    k = torch.randn((1, hkv, n_k, d), device="cuda", generator=g).half()
-    v = torch.randn((1, hkv, n_k, d), device="cuda", generator=g).half()
+    q = torch.from_numpy(synth.normal(1, (1, h, 1, d)).astype("float16")).cuda()
+    k = torch.from_numpy(synth.normal(2, (1, hkv, n_k, d)).astype("float16")).cuda()
+    v = torch.from_numpy(synth.normal(3, (1, hkv, n_k, d)).astype("float16")).cuda()
     y = torch.empty_like(q)
     need = int(lib.anygpu_sdp_attention_decode_workspace_bytes(h, h // hkv, 1, n_k, d, 1, 0))
     capi.check("anygpu_sdp_attention_decode_workspace_bytes", min(need, 0))
@@ -242,27 +380,25 @@ def bench_attention_decode(torch, capi, steps, warmup):
     def step():
         capi.check("anygpu_sdp_attention_decode_f16", lib.anygpu_sdp_attention_decode_f16(*call))
 
-    host_s, ev_s = timed_region(torch, step, steps, warmup)
+    t = timed_region(torch, step, steps, warmup)
     nbytes = 2 * hkv * n_k * d * 2 + 2 * h * d * 2
-    t = ev_s / steps
+    sec = t["us_per_launch"] * 1e-6
     return {
         "name": "sdp_attention_decode_f16",
         "workload": "decode attention fp16 q [1, 64, 1, 128], k / v [1, 8, 32768, 128], x 1/sqrt(128), causal; partial + merge launches",
-        "us_per_launch": t * 1e6, "value": nbytes / t / 1e9, "unit": "GB/s", "dtype": "f16",
-        "roofline": {"bound": "hbm", "achieved": nbytes / t / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                     "frac": nbytes / t / 1e9 / PEAK_HBM_GBS, "traffic": MEASURED_TRAFFIC_BYTES.get("attention_decode"),
+        **timing_fields(t), "value": nbytes / sec / 1e9, "unit": "GB/s", "dtype": "f16",
+        "roofline": {"bound": "hbm", "achieved": nbytes / sec / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": nbytes / sec / 1e9 / PEAK_HBM_GBS, **traffic_fields("attention_decode"),
                      "algorithmic_bytes": nbytes, "workspace_bytes": need},
     }
 
 
-def bench_gated_rmsnorm(torch, ops, steps, warmup):
+def bench_gated_rmsnorm(torch, ops, synth, steps, warmup):
     # Zamba2-7B Mamba2 mixer: batch 4 x 4096 positions, d_inner 8192
     rows, cols, nbuf = 4 * 4096, 8192, 3                    # 3 x 805 MB of x + z + y: past the Infinity Cache
-    g = torch.Generator(device="cuda")
-    g.manual_seed(0)
-    xs = [torch.randn((rows, cols), device="cuda", generator=g).half() for _ in range(nbuf)]
-    zs = [torch.randn((rows, cols), device="cuda", generator=g).half() for _ in range(nbuf)]
-    w = (torch.rand((cols,), device="cuda", generator=g) + 0.5).half()
+    xs = rotation(torch, torch.from_numpy(synth.normal(0, (rows, cols)).astype("float16")).cuda(), nbuf)
+    zs = rotation(torch, torch.from_numpy(synth.normal(1, (rows, cols)).astype("float16")).cuda(), nbuf)
+    w = torch.from_numpy(synth.uniform(2, (cols,), 0.5, 1.5).astype("float16")).cuda()
     it = [0]
 
     def step():
@@ -270,50 +406,14 @@ def bench_gated_rmsnorm(torch, ops, steps, warmup):
         it[0] += 1
         ops.tensor_zamba_gated_rmsnorm(xs[i], zs[i], w, cols, 1e-5)
 
-    host_s, ev_s = timed_region(torch, step, steps, warmup)
+    t = timed_region(torch, step, steps, warmup)
     nbytes = 3 * rows * cols * 2 + cols * 2
-    t = ev_s / steps
+    sec = t["us_per_launch"] * 1e-6
     return {
-        "name": "gated_rmsnorm_f16", "workload": "gated RMS norm fp16 x, z [16384, 8192], w [8192], eps 1e-5",
-        "us_per_launch": t * 1e6, "value": nbytes / t / 1e9, "unit": "GB/s", "dtype": "f16",
-        "roofline": {"bound": "hbm", "achieved": nbytes / t / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                     "frac": nbytes / t / 1e9 / PEAK_HBM_GBS, "traffic": MEASURED_TRAFFIC_BYTES["gated_rmsnorm"],
-                     "algorithmic_bytes": nbytes},
-    }
-
-
-def cpu_baseline_gemm(a_dev, bt_dev, target_seconds):
-    """The oracle's tensor_mm (1 thread, the reference's loop order) on the first R rows of the
-    same 4096^3 problem; R is sized from a short probe so that the sample takes about
-    `target_seconds`.  Also times the same rows spread over all host cores."""
-    import numpy as np
-    import oracle
-
-    a = oracle.cvt_f16_to_f32(a_dev.cpu().numpy())
-    bt = oracle.cvt_f16_to_f32(bt_dev.cpu().numpy())
-    n = a.shape[0]
-    b_view = bt.T                                    # column-major B as a strided view
-
-    def run(rows, threads):
-        t0 = time.perf_counter()
-        oracle.tensor_mm(a[:rows], b_view, threads=threads)
-        return time.perf_counter() - t0
-
-    probe_rows = 2
-    probe_s = run(probe_rows, 1)
-    per_row = probe_s / probe_rows
-    rows = int(max(probe_rows, min(n, target_seconds / max(per_row, 1e-9))))
-    t1 = run(rows, 1)
-    flops = 2.0 * rows * n * n
-    cores = min(oracle.max_threads(), int(os.environ.get("OMP_NUM_THREADS", "16") or 16), 16)
-    rows_mt = min(n, rows * cores)
-    tn = run(rows_mt, cores)
-    return {
-        "value": flops / t1 / 1e12, "unit": "TFLOP/s", "cores": 1, "kind": "port",
-        "sample": f"rows 0..{rows - 1} of C ({rows} x {n} x {n} MACs) of the same 4096^3 inputs, "
-                  f"reference loop order, float32 accumulator, {t1:.1f} s",
-        "all_cores": {"value": 2.0 * rows_mt * n * n / tn / 1e12, "unit": "TFLOP/s", "cores": cores,
-                      "sample": f"rows 0..{rows_mt - 1}, outer rows split over {cores} threads, {tn:.1f} s"},
+        "name": "gated_rmsnorm_f16", "workload": "gated RMS norm fp16 x, z [16384, 8192] N(0,1) seeds 0 / 1, w [8192] U(0.5,1.5) seed 2, eps 1e-5",
+        **timing_fields(t), "value": nbytes / sec / 1e9, "unit": "GB/s", "dtype": "f16",
+        "roofline": {"bound": "hbm", "achieved": nbytes / sec / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": nbytes / sec / 1e9 / PEAK_HBM_GBS, **traffic_fields("gated_rmsnorm"), "algorithmic_bytes": nbytes},
     }
 
 
@@ -335,6 +435,7 @@ def main():
     only = set(filter(None, args.only.split(",")))
     want = lambda name: not only or name in only
     props = torch.cuda.get_device_properties(0)
+    cpu_side = args.cpu_seconds / 4.0
 
     kernels = []
     gemm = None
@@ -348,48 +449,56 @@ def main():
     if want("gemm"):
         gemm = bench_gemm_f16(torch, ops, capi, synth, args.steps, args.warmup)
     if want("gemm32"):
-        kernels.append(bench_gemm_f32(torch, ops, synth, max(args.steps // 2, 1), args.warmup))
+        kernels.append(bench_gemm_f32(torch, ops, synth, args.steps // 2, args.warmup, cpu_side))
     if want("conv"):
-        kernels.append(bench_conv1d(torch, ops, args.steps, args.warmup))
+        kernels.append(bench_conv1d(torch, ops, synth, args.steps, args.warmup, cpu_side))
     if want("softmax"):
         kernels.append(bench_softmax(
-            torch, ops, args.steps, args.warmup, name="softmax_causal_f16", key="softmax_causal",
+            torch, ops, synth, args.steps, args.warmup, cpu_side, name="softmax_causal_f16", key="softmax_causal",
             heads=32, q=2048, k=2048, std=4.0, alpha=1.0 / 8.0, cap=0.0, window=0, nbuf=3,
-            workload="causal softmax fp16 [1, 32, 2048, 2048], scores N(0,4) scaled by 1/8 in-kernel"))
+            workload="causal softmax fp16 [1, 32, 2048, 2048], scores N(0,4) seed 0, scaled by 1/8 in-kernel "
+                     "(BASELINE.json configs[3]); 3 rotating buffer sets"))
         kernels.append(bench_softmax(
-            torch, ops, max(args.steps // 4, 1), max(args.warmup // 4, 1), name="softmax_gemma2_f16",
+            torch, ops, synth, args.steps // 4, max(args.warmup // 4, 1), cpu_side, name="softmax_gemma2_f16",
             key="softmax_gemma2", heads=8, q=8192, k=8192, std=16.0, alpha=1.0 / 16.0, cap=50.0, window=4096, nbuf=2,
-            workload="Gemma2 softmax fp16 [1, 8, 8192, 8192], N(0,16) x 1/16, softcap 50, causal + window 4096"))
-
+            workload="Gemma2 softmax fp16 [1, 8, 8192, 8192], N(0,16) seed 0, x 1/16, softcap 50, causal + window 4096 "
+                     "(BASELINE.json configs[4]); 2 rotating buffer sets"))
     if want("attn"):
-        kernels.append(bench_attention(torch, ops, max(args.steps // 8, 1), max(args.warmup // 4, 1)))
+        kernels.append(bench_attention(torch, ops, synth, args.steps // 8, max(args.warmup // 4, 1), "f16"))
     if want("attn32"):
-        kernels.append(bench_attention_f32(torch, ops, max(args.steps // 16, 1), max(args.warmup // 8, 1)))
+        kernels.append(bench_attention(torch, ops, synth, args.steps // 16, max(args.warmup // 8, 1), "f32"))
     if want("decode"):
-        kernels.append(bench_attention_decode(torch, capi, args.steps, args.warmup))
+        kernels.append(bench_attention_decode(torch, capi, synth, args.steps, args.warmup))
     if want("norm"):
-        kernels.append(bench_gated_rmsnorm(torch, ops, max(args.steps // 4, 1), max(args.warmup // 4, 1)))
+        kernels.append(bench_gated_rmsnorm(torch, ops, synth, args.steps // 4, max(args.warmup // 4, 1)))
 
     line = {
         "metric": "fp16 GEMM TFLOP/s; conv1d & softmax HBM GB/s (% roofline) on 1 MI355X",
         "value": None, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": None, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16", "data": "synthetic", "settle_s": SETTLE_SECONDS,
-        "config": {"workload": "fp16 GEMM M=N=K=4096, A row-major, B column-major ([N,K] storage), U(-1,1) inputs, "
+        "config": {"workload": "fp16 GEMM M=N=K=4096, A row-major, B column-major ([N,K] storage), U(-1,1) inputs (seeds 0 / 1), "
                                "fp32 accumulate on MFMA, fp16 output (BASELINE.json configs[1])"},
-        "device": {"name": props.name, "compute_units": props.multi_processor_count,
-                   "clock_mhz": getattr(props, "clock_rate", 0) / 1e3 if hasattr(props, "clock_rate") else None},
+        "device": {"name": props.name, "compute_units": props.multi_processor_count, "peak_clock_ghz": PEAK_CLOCK_GHZ},
     }
     if gemm is not None:
-        t_ev = gemm["event_s"] / args.steps
+        t = gemm["timing"]
         line["value"] = gemm["tflops_host"]
-        line["ms_per_step"] = gemm["host_s"] / args.steps * 1e3
+        line["ms_per_step"] = t["host_s"] / t["steps"] * 1e3
+        clock = gemm["clock"]
+        peak_at_clock = props.multi_processor_count * FP16_FLOP_PER_CLK_PER_CU * clock["sustained_clock_ghz"] * 1e9 / 1e12
         line["roofline"] = {"bound": "mfma", "achieved": gemm["tflops_event"], "peak": PEAK_FP16_TFLOPS,
                             "unit": "TFLOP/s", "frac": gemm["tflops_event"] / PEAK_FP16_TFLOPS,
-                            "traffic": MEASURED_TRAFFIC_BYTES["gemm_f16"], "us_per_launch": t_ev * 1e6,
-                            "algorithmic_flops": gemm["flops"], "min_bytes": 3 * 4096 * 4096 * 2}
+                            **traffic_fields("gemm_f16"), **timing_fields(t),
+                            "algorithmic_flops": gemm["flops"], "min_bytes": 3 * 4096 * 4096 * 2,
+                            **clock, "peak_at_sustained_clock": peak_at_clock,
+                            "frac_at_sustained_clock": gemm["tflops_event"] / peak_at_clock}
         if args.cpu_seconds > 0:
-            line["cpu_baseline"] = cpu_baseline_gemm(*gemm["operands"], args.cpu_seconds)
+            import oracle
+            a_dev, bt_dev = gemm["operands"]
+            a32 = oracle.cvt_f16_to_f32(a_dev.cpu().numpy())
+            bt32 = oracle.cvt_f16_to_f32(bt_dev.cpu().numpy())
+            line["cpu_baseline"] = cpu_baseline_gemm(oracle, a32, bt32.T, args.cpu_seconds, "the same 4096^3 inputs")
     line["kernels"] = kernels
     print(json.dumps(line))
     return 0

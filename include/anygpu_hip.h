@@ -95,6 +95,21 @@ int anygpu_gemm_f16_f32acc(const void* A, const void* B, void* C,
                            int b_layout, void* stream);
 
 /*
+ * Measurement hook: anygpu_gemm_f16_f32acc through the kernel of the whole-tile case (M and N multiples of 256, K a
+ * multiple of 64, B column-major, 16-byte aligned rows; anything else returns ANYGPU_ERR_UNSUPPORTED and launches
+ * nothing), which additionally leaves four 64-bit counts per 256 x 256 tile in probe[4 * tile .. + 3] (device memory,
+ * 4 * (M / 256) * (N / 256) values): the shader clock count at entry and at exit of that tile's main loop, then the
+ * count of the constant 100 MHz clock at the same two points.  (exit - entry) of the first pair over 10 ns times
+ * (exit - entry) of the second is the clock the part sustained under the kernel; K / 32 * 64 matrix instructions of 16
+ * cycles over the first difference is the share of cycles its matrix cores were busy.  The result in C is that of
+ * anygpu_gemm_f16_f32acc.  No counterpart in the reference.
+ */
+int anygpu_gemm_f16_f32acc_probe(const void* A, const void* B, void* C,
+                                 int64_t M, int64_t N, int64_t K,
+                                 int64_t lda, int64_t ldb, int64_t ldc,
+                                 int b_layout, uint64_t* probe, void* stream);
+
+/*
  * `batch` products of one shape in one launch: product i reads A + i * stride_a, B + i * stride_b and
  * writes C + i * stride_c (strides in elements, 0 shares an operand).  This is what the per-head host
  * loop of srcs/transformers/sdp.hpp:258-271 (one tensor_mm launch per head for Q K^T and again for P V)

@@ -183,9 +183,7 @@ def test_softmax_empty_and_rejected_arguments(ops):
 def _full_size_softmax(ops, oracle, heads, q, k, std, alpha, cap, window, n_sample):
     import torch
     rows = heads * q
-    g = torch.Generator(device="cuda")
-    g.manual_seed(0)
-    x = (torch.randn((rows, k), device="cuda", dtype=torch.float32, generator=g) * std).to(torch.float16)
+    x = dev(synth.normal_matrix_f16(0, rows, k, std))          # the scores the benchmark times: seed 0, drawn on the host
     y = ops.tensor_softmax(x, alpha=alpha, softcap=cap, causal=True, window=window, q_len=q)
     torch.cuda.synchronize()
     # size-independent properties over the whole output
