@@ -35,6 +35,12 @@ SIGNATURES = {
     "anygpu_release_workspaces": (c_int, []),
     "anygpu_gemm_f16_f32acc": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64,
                                        c_int64, c_int64, c_int64, c_int, c_void_p]),
+    "anygpu_gemm_f16_f32acc_bias": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64,
+                                            c_int64, c_int64, c_int64, c_int, c_void_p]),
+    "anygpu_gemm_f16_f32acc_softcap": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64,
+                                               c_int64, c_int64, c_int64, c_int, c_float, c_void_p]),
+    "anygpu_gemm_f16_f32acc_gelu_mul": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64,
+                                                c_int64, c_int64, c_int64, c_int, c_void_p]),
     "anygpu_gemm_f16_f32acc_probe": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64,
                                              c_int64, c_int64, c_int64, c_int, c_void_p, c_void_p]),
     "anygpu_gemm_f32": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64,

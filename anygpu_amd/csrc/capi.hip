@@ -3,6 +3,7 @@
 #include "anygpu_hip.h"
 #include "launch.hpp"
 #include "gemm_band.hpp"
+#include "gemm_epilogue.hpp"
 #include "device_utils.hpp"
 
 #include <atomic>
@@ -228,6 +229,49 @@ ANYGPU_EXPORT int anygpu_gemm_f16_f32acc(const void* A, const void* B, void* C,
 	const int rc = check_gemm(A, B, C, M, N, K, lda, ldb, ldc, ANYGPU_A_ROW_MAJOR, b_layout);
 	if (rc != ANYGPU_OK) return rc;
 	return (int)anygpu::launch_gemm_f16(A, B, C, M, N, K, lda, ldb, ldc, 0, 0, 0, 1, b_layout, as_stream(stream));
+}
+
+namespace {
+
+int gemm_f16_epilogue_entry(const void* A, const void* B, const void* B2, const void* bias, void* C,
+                            int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc,
+                            int b_layout, int epilogue, float ep_param, void* stream)
+{
+	const int rc = check_gemm(A, B, C, M, N, K, lda, ldb, ldc, ANYGPU_A_ROW_MAJOR, b_layout);
+	if (rc != ANYGPU_OK) return rc;
+	if (M == 0 || N == 0) return ANYGPU_OK;
+	if (K == 0) return ANYGPU_ERR_UNSUPPORTED;            // (an empty sum with an epilogue: not a case any caller has)
+	bool supported = true;
+	const hipError_t err = anygpu::launch_gemm_f16_epilogue(A, B, B2, bias, C, M, N, K, lda, ldb, ldc, b_layout, epilogue, ep_param,
+	                                                        as_stream(stream), &supported);
+	if (!supported) return ANYGPU_ERR_UNSUPPORTED;
+	return (int)err;
+}
+
+}  // namespace
+
+ANYGPU_EXPORT int anygpu_gemm_f16_f32acc_bias(const void* A, const void* B, const void* bias, void* C,
+                                              int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc,
+                                              int b_layout, void* stream)
+{
+	if (bias == nullptr && M > 0 && N > 0) return ANYGPU_ERR_NULL_POINTER;
+	return gemm_f16_epilogue_entry(A, B, nullptr, bias, C, M, N, K, lda, ldb, ldc, b_layout, anygpu::kEpiBias, 0.0f, stream);
+}
+
+ANYGPU_EXPORT int anygpu_gemm_f16_f32acc_softcap(const void* A, const void* B, void* C,
+                                                 int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc,
+                                                 int b_layout, float softcap, void* stream)
+{
+	if (!(softcap > 0.0f) || !std::isfinite(softcap)) return ANYGPU_ERR_UNSUPPORTED;
+	return gemm_f16_epilogue_entry(A, B, nullptr, nullptr, C, M, N, K, lda, ldb, ldc, b_layout, anygpu::kEpiSoftcap, softcap, stream);
+}
+
+ANYGPU_EXPORT int anygpu_gemm_f16_f32acc_gelu_mul(const void* A, const void* B_gate, const void* B_up, void* C,
+                                                  int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc,
+                                                  int b_layout, void* stream)
+{
+	if (B_up == nullptr && M > 0 && N > 0 && K > 0) return ANYGPU_ERR_NULL_POINTER;
+	return gemm_f16_epilogue_entry(A, B_gate, B_up, nullptr, C, M, N, K, lda, ldb, ldc, b_layout, anygpu::kEpiGeluMul, 0.0f, stream);
 }
 
 ANYGPU_EXPORT int anygpu_gemm_f16_f32acc_probe(const void* A, const void* B, void* C,

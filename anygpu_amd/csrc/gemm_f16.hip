@@ -170,6 +170,23 @@ __global__ __launch_bounds__(256) void gemm_f16_edge_kernel(
 	}
 }
 
+// Time per 64-deep slab of `nblocks` blocks spread over 256 CUs, in us, from measurements: a 256 x 256 tile takes
+// 1.56 per round of blocks (4096^3: 256 blocks, 64 slabs, 100 us); the smaller tiles, of which a CU holds several,
+// follow the average number of blocks per CU with a floor where a lone block waits on latency: 0.75 per block
+// and CU for 128 x 128 (144 blocks 0.75 - 1.0, 288 1.0, 576 1.7 - 2.0), 0.27 for 64 x 64 in dense launches.
+// The cheapest launch is taken, the bigger tile on a tie.
+static double slab_us(int64_t t, int64_t nblocks)
+{
+	const double rounds = (double)((nblocks + 255) / 256);
+	const double share = nblocks > 256 ? (double)nblocks / 256.0 : 1.0;
+	if (t == 256) return 1.56 * rounds;
+	if (t == 128) return 0.75 * share;
+	// four stages (see kDeepStageBlocks): 0.22 where every block has a CU of its own, twice 0.21 where some
+	// CUs hold two (they decide when the launch ends)
+	if (nblocks <= kDeepStageBlocks) return nblocks <= 256 ? 0.22 : 0.42;
+	return 0.27 * share;
+}
+
 // C[m, n] = half(sum over splits of planes[split][m][n]), one thread per eight columns (N a multiple of 8), the
 // planes added in order
 __global__ __launch_bounds__(256) void gemm_f16_split_merge_kernel(
@@ -272,21 +289,6 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
 		// it run the same kernels with clamped operand rows and guarded stores; a K that is not a multiple of the
 		// 64-deep slab adds a tail multiplied from registers.
 		const auto blocks = [&](int64_t tile) { return ((M + tile - 1) / tile) * ((N + tile - 1) / tile) * batch; };
-		// Time per 64-deep slab of `nblocks` blocks spread over 256 CUs, in us, from measurements: a 256 x 256 tile takes
-		// 1.56 per round of blocks (4096^3: 256 blocks, 64 slabs, 100 us); the smaller tiles, of which a CU holds several,
-		// follow the average number of blocks per CU with a floor where a lone block waits on latency: 0.75 per block
-		// and CU for 128 x 128 (144 blocks 0.75 - 1.0, 288 1.0, 576 1.7 - 2.0), 0.27 for 64 x 64 in dense launches.
-		// The cheapest launch is taken, the bigger tile on a tie.
-		const auto slab_us = [](int64_t t, int64_t nblocks) {
-			const double rounds = (double)((nblocks + 255) / 256);
-			const double share = nblocks > 256 ? (double)nblocks / 256.0 : 1.0;
-			if (t == 256) return 1.56 * rounds;
-			if (t == 128) return 0.75 * share;
-			// four stages (see kDeepStageBlocks): 0.22 where every block has a CU of its own, twice 0.21 where some
-			// CUs hold two (they decide when the launch ends)
-			if (nblocks <= kDeepStageBlocks) return nblocks <= 256 ? 0.22 : 0.42;
-			return 0.27 * share;
-		};
 		const double cost256 = slab_us(256, blocks(256)), cost128 = slab_us(128, blocks(128)), cost64 = slab_us(64, blocks(64));
 		int64_t tile = (cost256 <= cost128 && cost256 <= cost64) ? 256 : cost128 <= cost64 ? 128 : 64;
 
@@ -448,6 +450,84 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
 		gemm_f16_edge_kernel<ANYGPU_B_ROW_MAJOR><<<grid, dim3(256), 0, stream>>>(a, b, c, M, N, K, lda, ldb, ldc,
 		                                                                 stride_a, stride_b, stride_c);
 	return hipGetLastError();
+}
+
+// bias / softcap applied in place to a finished product (the shapes only the edge kernel takes)
+template <int EPI>
+__global__ __launch_bounds__(256) void gemm_f16_finish_kernel(half_t* __restrict__ C, const half_t* __restrict__ bias,
+                                                              int64_t M, int64_t N, int64_t ldc, float ep_param)
+{
+	const int64_t item = (int64_t)blockIdx.x * 256 + threadIdx.x;
+	if (item >= M * N) return;
+	const int64_t m = item / N, n = item % N;
+	half_t* p = C + m * ldc + n;
+	*p = (half_t)finish_sum<EPI>((float)*p, 0.0f, EPI == kEpiBias ? (float)bias[n] : 0.0f, ep_param);
+}
+
+// The fp16 product with an epilogue: kEpiBias (+ bias[n], fp16), kEpiSoftcap (cap * tanh(sum / cap)) or kEpiGeluMul
+// (gelu_tanh(A B) * (A B2)), applied to the fp32 sums before the one rounding to fp16.  Few rows against k-contiguous
+// weights take the band kernels; everything else the plain tile kernels (256 / 128 / 64, priced like the unfused
+// product, uncut), whose epilogue does the work.
+hipError_t launch_gemm_f16_epilogue(const void* A, const void* B, const void* B2, const void* bias, void* C,
+                                    int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc,
+                                    int b_layout, int epilogue, float ep_param, hipStream_t stream, bool* supported)
+{
+	*supported = true;
+	if (M == 0 || N == 0) return hipSuccess;
+	const half_t* a = static_cast<const half_t*>(A);
+	const half_t* b = static_cast<const half_t*>(B);
+	const half_t* b2 = static_cast<const half_t*>(B2);
+	const half_t* bs = static_cast<const half_t*>(bias);
+	half_t* c = static_cast<half_t*>(C);
+	const bool dual = epilogue == kEpiGeluMul;
+	const bool aligned = (reinterpret_cast<uintptr_t>(A) % 16 == 0) && (reinterpret_cast<uintptr_t>(B) % 16 == 0) &&
+	                     (!dual || reinterpret_cast<uintptr_t>(B2) % 16 == 0) && (lda % 8 == 0) && (ldb % 8 == 0);
+	const bool tiles_ok = aligned && K >= 64 && K % 8 == 0 && (b_layout == ANYGPU_B_COL_MAJOR || N % 8 == 0);
+	if (epilogue != kEpiBias && gemm_band_applies<half_t>(a, b, b2, c, M, N, K, lda, ldb, ldc, b_layout))
+		return launch_gemm_band<half_t>(a, b, b2, nullptr, c, M, N, K, lda, ldb, ldc, epilogue, ep_param, stream);
+	if (!tiles_ok)
+	{
+		if (dual)
+		{
+			*supported = false;
+			return hipSuccess;
+		}
+		const hipError_t err = launch_gemm_f16(A, B, C, M, N, K, lda, ldb, ldc, 0, 0, 0, 1, b_layout, stream);
+		if (err != hipSuccess) return err;
+		const dim3 grid((unsigned)((M * N + 255) / 256));
+		if (epilogue == kEpiBias) gemm_f16_finish_kernel<kEpiBias><<<grid, dim3(256), 0, stream>>>(c, bs, M, N, ldc, ep_param);
+		else gemm_f16_finish_kernel<kEpiSoftcap><<<grid, dim3(256), 0, stream>>>(c, bs, M, N, ldc, ep_param);
+		return hipGetLastError();
+	}
+	// a tile of edge t covers t (t / 2 with two products) output columns
+	const auto blocks = [&](int64_t t) { return ((M + t - 1) / t) * ((N + (dual ? t / 2 : t) - 1) / (dual ? t / 2 : t)); };
+	const double cost256 = slab_us(256, blocks(256)), cost128 = slab_us(128, blocks(128)), cost64 = slab_us(64, blocks(64));
+	const int64_t tile = (cost256 <= cost128 && cost256 <= cost64) ? 256 : cost128 <= cost64 ? 128 : 64;
+	if (blocks(tile) > 0x7FFFFFFFLL)
+	{
+		*supported = false;
+		return hipSuccess;
+	}
+#define ANYGPU_F16_EPI_TILE(BT, WM, WN, KN, EPI) \
+	return launch_gemm_f16_tile<GemmTileCfg<BT, BT, WM, WN, 1, 0, 4, 16, KN, 2, 1>, true, true, false, EPI>( \
+		a, b, c, M, N, K, lda, ldb, ldc, 0, 0, 0, 1, stream, nullptr, 0, b2, bs, ep_param)
+#define ANYGPU_F16_EPI_LAYOUT(KN, EPI) \
+	do { \
+		if (tile == 256) ANYGPU_F16_EPI_TILE(256, 2, 4, KN, EPI); \
+		if (tile == 128) ANYGPU_F16_EPI_TILE(128, 2, 2, KN, EPI); \
+		ANYGPU_F16_EPI_TILE(64, 2, 2, KN, EPI); \
+	} while (0)
+#define ANYGPU_F16_EPI(EPI) \
+	do { \
+		if (b_layout == ANYGPU_B_COL_MAJOR) ANYGPU_F16_EPI_LAYOUT(false, EPI); \
+		ANYGPU_F16_EPI_LAYOUT(true, EPI); \
+	} while (0)
+	if (epilogue == kEpiSoftcap) ANYGPU_F16_EPI(kEpiSoftcap);
+	if (epilogue == kEpiGeluMul) ANYGPU_F16_EPI(kEpiGeluMul);
+	ANYGPU_F16_EPI(kEpiBias);
+#undef ANYGPU_F16_EPI
+#undef ANYGPU_F16_EPI_LAYOUT
+#undef ANYGPU_F16_EPI_TILE
 }
 
 }  // namespace anygpu

@@ -24,6 +24,7 @@
 #pragma once
 
 #include "device_utils.hpp"
+#include "gemm_epilogue.hpp"
 
 #include <atomic>
 #include <type_traits>
@@ -192,20 +193,44 @@ __device__ __forceinline__ half4_t lds_read_transposed_b64(const char* lds_addr)
 // after a v_permlane16_swap between neighbouring tiles, were 1.5 us slower than whole rows through LDS.
 typedef half8_t LooseHalf8Store __attribute__((aligned(2)));
 
-template <typename Cfg, bool RAGGED, bool STREAM = false>
+// EPI: what happens to a sum on its way out (gemm_epilogue.hpp).  kEpiBias adds bias[n] (fp16), kEpiSoftcap
+// caps, and with kEpiGeluMul the patch holds two products side by side: MFMA column tiles 0 .. TN / 2 - 1 are A x B_gate
+// and TN / 2 .. TN - 1 are A x B_up for the same kWaveN / 2 output columns (the kernel staged the B slab that way), and
+// gelu_tanh(gate) * up goes out; n_base and N then count output columns.
+constexpr int kEpiNone = -1;      // the sums go out as they are
+
+template <typename Cfg, bool RAGGED, bool STREAM = false, int EPI = kEpiNone>
 __device__ __forceinline__ void store_patch_via_lds(
 	const typename MfmaShape<Cfg::MI>::Acc (&acc)[Cfg::kTilesM][Cfg::kTilesN], char* lds,
-	half_t* __restrict__ C, int64_t ldc, int64_t m_base, int64_t n_base, int wave, int lane, int64_t M, int64_t N)
+	half_t* __restrict__ C, int64_t ldc, int64_t m_base, int64_t n_base, int wave, int lane, int64_t M, int64_t N,
+	const half_t* __restrict__ bias = nullptr, float ep_param = 0.0f)
 {
 	using Shape = MfmaShape<Cfg::MI>;
-	constexpr int MI = Cfg::MI, TM = Cfg::kTilesM, TN = Cfg::kTilesN;
-	constexpr int kRowBytes = Cfg::kWaveN * 2;
+	constexpr int MI = Cfg::MI, TM = Cfg::kTilesM;
+	constexpr int TN = EPI == kEpiGeluMul ? Cfg::kTilesN / 2 : Cfg::kTilesN;        // column tiles that are stored
+	constexpr int kRowBytes = (EPI == kEpiGeluMul ? Cfg::kWaveN / 2 : Cfg::kWaveN) * 2;
+	static_assert(EPI != kEpiGeluMul || Cfg::kTilesN % 2 == 0, "gate and up halves of the patch");
 	constexpr int kPitch = kRowBytes + 16;
 	constexpr int kLanesPerRow = kRowBytes / 16;
 	constexpr int kRowsPerPass = kWaveSize / kLanesPerRow;
 	static_assert(Cfg::kWaves * MI * kPitch <= Cfg::kLdsBytes, "epilogue scratch must fit in the staging LDS");
 	char* scratch = lds + wave * (MI * kPitch);
 	const int frag_row = lane % MI;
+	// the bias of this lane's columns (the same for every row band)
+	[[maybe_unused]] float bias_of[TN][Shape::kAccRegs / 4][4] = {};
+	if constexpr (EPI == kEpiBias)
+	{
+#pragma unroll
+		for (int j = 0; j < TN; ++j)
+#pragma unroll
+			for (int g = 0; g < Shape::kAccRegs / 4; ++g)
+#pragma unroll
+				for (int e = 0; e < 4; ++e)
+				{
+					const int64_t n = n_base + j * MI + Shape::first_row_of_group(g, lane) + e;
+					bias_of[j][g][e] = (!RAGGED || n < N) ? (float)bias[n] : 0.0f;
+				}
+	}
 #pragma unroll
 	for (int i = 0; i < TM; ++i)
 	{
@@ -216,7 +241,17 @@ __device__ __forceinline__ void store_patch_via_lds(
 			{
 				half4_t out;
 #pragma unroll
-				for (int e = 0; e < 4; ++e) out[e] = (half_t)acc[i][j][4 * g + e];
+				for (int e = 0; e < 4; ++e)
+				{
+					if constexpr (EPI == kEpiGeluMul)
+						out[e] = (half_t)finish_sum<EPI>(acc[i][j][4 * g + e], acc[i][j + TN][4 * g + e], 0.0f, ep_param);
+					else if constexpr (EPI == kEpiSoftcap)
+						out[e] = (half_t)finish_sum<EPI>(acc[i][j][4 * g + e], 0.0f, 0.0f, ep_param);
+					else if constexpr (EPI == kEpiBias)
+						out[e] = (half_t)(acc[i][j][4 * g + e] + bias_of[j][g][e]);
+					else
+						out[e] = (half_t)acc[i][j][4 * g + e];
+				}
 				*reinterpret_cast<half4_t*>(scratch + frag_row * kPitch +
 				                            (j * MI + Shape::first_row_of_group(g, lane)) * 2) = out;
 			}
@@ -288,14 +323,29 @@ constexpr int kSchedDsRead = 0x100;
 // every lane loads straight from global memory in the MFMA operand layout, zeros past K.
 // SPLIT: blockIdx.y walks ranges of K (k_split deep, the strides step along K) of one product instead of a batch,
 // and the raw fp32 sums of range y go to planes[y][M][N]; C is not touched.
-template <typename Cfg, bool RAGGED = false, bool KTAIL = false, bool SPLIT = false>
+// EPI: the epilogue (see store_patch_via_lds).  With kEpiGeluMul the tile is BN / 2 output columns wide (N and tiles_n
+// count those) and its B slab is put together from two matrices: of every wave's kWaveN slab rows the first half comes
+// from B (the gate weights) and the second half from B2 (the up weights), both for the same kWaveN / 2 output columns,
+// so gate and up sums of an output element meet in one lane and A is read once for both products.
+template <typename Cfg, bool RAGGED = false, bool KTAIL = false, bool SPLIT = false, int EPI = kEpiNone>
 __global__ __launch_bounds__(Cfg::kThreads) void gemm_f16_nt_tile_kernel(
 	const half_t* __restrict__ A, const half_t* __restrict__ B, half_t* __restrict__ C,
 	int K, int64_t lda, int64_t ldb, int64_t ldc, int tiles_m, int tiles_n,
 	int64_t stride_a, int64_t stride_b, int64_t stride_c, int64_t M, int64_t N,
-	float* __restrict__ planes, int k_split)
+	float* __restrict__ planes, int k_split,
+	const half_t* __restrict__ B2 = nullptr, const half_t* __restrict__ bias = nullptr, float ep_param = 0.0f)
 {
 	using Shape = MfmaShape<Cfg::MI>;
+	constexpr bool DUAL = EPI == kEpiGeluMul;
+	static_assert(EPI == kEpiNone || (!SPLIT && Cfg::kKGroupsOfWaves == 1), "epilogues: the plain tile, uncut");
+	constexpr int kOutN = DUAL ? Cfg::BN / 2 : Cfg::BN;           // output columns of a tile
+	constexpr int kHalfWaveN = Cfg::kWaveN / 2;
+	// DUAL: slab row (or column, for [K, N] weights) c of the tile -> which matrix, which output column of the tile
+	const auto dual_col = [](int c, bool& second) {
+		const int group = c / kHalfWaveN;
+		second = (group & 1) != 0;
+		return (group >> 1) * kHalfWaveN + c % kHalfWaveN;
+	};
 	if constexpr (SPLIT)
 	{
 		const int left = K - (int)blockIdx.y * k_split;
@@ -323,7 +373,7 @@ __global__ __launch_bounds__(Cfg::kThreads) void gemm_f16_nt_tile_kernel(
 	int tile_m, tile_n;
 	tile_of_block<Cfg::GROUP_M>(blockIdx.x, tiles_m, tiles_n, tile_m, tile_n);
 	const int64_t m0 = (int64_t)tile_m * BM;
-	const int64_t n0 = (int64_t)tile_n * BN;
+	const int64_t n0 = (int64_t)tile_n * kOutN;
 
 	// Direct loads.  Load instruction i of this wave fills slab rows [8 * (wave * kLoads + i), +8):
 	// lane -> row offset lane / 8, chunk position lane % 8, i.e. logical chunk (lane % 8) ^ swz(row).
@@ -350,16 +400,20 @@ __global__ __launch_bounds__(Cfg::kThreads) void gemm_f16_nt_tile_kernel(
 			const int lanes_per_row = kWaveSize / kRowsPerLoadKN;
 			const int k = kRowsPerLoadKN * (wave * Cfg::kLoadsB + i) + lane / lanes_per_row;
 			const int pos = lane % lanes_per_row;
-			int64_t gcol = n0 + ((pos ^ (kn_row_swizzle(k) & kChunkMaskKN)) << 3);
+			int col = (pos ^ (kn_row_swizzle(k) & kChunkMaskKN)) << 3;
+			bool second = false;
+			if constexpr (DUAL) col = dual_col(col, second);
+			int64_t gcol = n0 + col;
 			if (RAGGED && gcol > N - 8) gcol = N - 8;
-			b_src[i] = B + (int64_t)k * ldb + gcol;
+			b_src[i] = (second ? B2 : B) + (int64_t)k * ldb + gcol;
 		}
 		else
 		{
 			const int row = 8 * (wave * Cfg::kLoadsB + i) + ld_row;
-			int64_t grow = n0 + row;
+			bool second = false;
+			int64_t grow = n0 + (DUAL ? dual_col(row, second) : row);
 			if (RAGGED && grow > N - 1) grow = N - 1;
-			b_src[i] = B + grow * ldb + ((ld_pos ^ swizzle_of_row<Cfg::SWZ>(row)) << 3);
+			b_src[i] = (second ? B2 : B) + grow * ldb + ((ld_pos ^ swizzle_of_row<Cfg::SWZ>(row)) << 3);
 		}
 	}
 
@@ -578,19 +632,22 @@ __global__ __launch_bounds__(Cfg::kThreads) void gemm_f16_nt_tile_kernel(
 #pragma unroll
 			for (int j = 0; j < TN; ++j)
 			{
-				int64_t gcol = n0 + wn * Cfg::kWaveN + j * MI + frag_row;
+				const int col = wn * Cfg::kWaveN + j * MI + frag_row;
+				bool second = false;
+				int64_t gcol = n0 + (DUAL ? dual_col(col, second) : col);
 				if (RAGGED && gcol > N - 1) gcol = N - 1;
+				const half_t* Bt = second ? B2 : B;
 				half8_t v = {};
 				if (kk < K)
 				{
 					if constexpr (Cfg::B_KN)
 					{
 #pragma unroll
-						for (int e = 0; e < 8; ++e) v[e] = B[(int64_t)(kk + e) * ldb + gcol];
+						for (int e = 0; e < 8; ++e) v[e] = Bt[(int64_t)(kk + e) * ldb + gcol];
 					}
 					else
 					{
-						v = *reinterpret_cast<const half8_t*>(B + gcol * ldb + kk);
+						v = *reinterpret_cast<const half8_t*>(Bt + gcol * ldb + kk);
 					}
 				}
 				bt[j] = v;
@@ -637,17 +694,20 @@ __global__ __launch_bounds__(Cfg::kThreads) void gemm_f16_nt_tile_kernel(
 	if constexpr (SPLIT)
 		store_patch_f32<Cfg>(acc, planes + (int64_t)blockIdx.y * M * N, m0 + wm * Cfg::kWaveM, n0 + wn * Cfg::kWaveN, lane, M, N);
 	else
-		store_patch_via_lds<Cfg, RAGGED>(acc, lds, C, ldc, m0 + wm * Cfg::kWaveM, n0 + wn * Cfg::kWaveN, wave_in_group, lane, M, N);
+		store_patch_via_lds<Cfg, RAGGED, false, EPI>(acc, lds, C, ldc, m0 + wm * Cfg::kWaveM, n0 + wn * (DUAL ? kHalfWaveN : Cfg::kWaveN),
+		                                             wave_in_group, lane, M, N, bias, ep_param);
 }
 
 // planes != NULL (SPLIT): `batch` is the number of K ranges, k_split their depth.
-template <typename Cfg, bool RAGGED = false, bool KTAIL = false, bool SPLIT = false>
+template <typename Cfg, bool RAGGED = false, bool KTAIL = false, bool SPLIT = false, int EPI = kEpiNone>
 hipError_t launch_gemm_f16_tile(const half_t* A, const half_t* B, half_t* C, int64_t M, int64_t N, int64_t K,
                                 int64_t lda, int64_t ldb, int64_t ldc,
                                 int64_t stride_a, int64_t stride_b, int64_t stride_c, int64_t batch, hipStream_t stream,
-                                float* planes = nullptr, int64_t k_split = 0)
+                                float* planes = nullptr, int64_t k_split = 0,
+                                const half_t* B2 = nullptr, const half_t* bias = nullptr, float ep_param = 0.0f)
 {
-	auto kernel = gemm_f16_nt_tile_kernel<Cfg, RAGGED, KTAIL, SPLIT>;
+	auto kernel = gemm_f16_nt_tile_kernel<Cfg, RAGGED, KTAIL, SPLIT, EPI>;
+	constexpr int kOutN = EPI == kEpiGeluMul ? Cfg::BN / 2 : Cfg::BN;
 	// More than 64 KB of dynamic LDS has to be granted per function and per device, once.
 	static std::atomic<uint64_t> configured_devices{0};
 	(void)hipGetLastError();
@@ -662,9 +722,10 @@ hipError_t launch_gemm_f16_tile(const half_t* A, const half_t* B, half_t* C, int
 		if (e != hipSuccess) return e;
 		configured_devices.fetch_or(bit, std::memory_order_relaxed);
 	}
-	const int tiles_m = (int)((M + Cfg::BM - 1) / Cfg::BM), tiles_n = (int)((N + Cfg::BN - 1) / Cfg::BN);
+	const int tiles_m = (int)((M + Cfg::BM - 1) / Cfg::BM), tiles_n = (int)((N + kOutN - 1) / kOutN);
 	kernel<<<dim3((unsigned)(tiles_m * tiles_n), (unsigned)batch), dim3(Cfg::kThreads), Cfg::kLdsBytes, stream>>>(
-		A, B, C, (int)K, lda, ldb, ldc, tiles_m, tiles_n, stride_a, stride_b, stride_c, M, N, planes, (int)k_split);
+		A, B, C, (int)K, lda, ldb, ldc, tiles_m, tiles_n, stride_a, stride_b, stride_c, M, N, planes, (int)k_split,
+		B2, bias, ep_param);
 	return hipGetLastError();
 }
 

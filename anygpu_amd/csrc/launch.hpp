@@ -39,6 +39,12 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
                            int64_t stride_a, int64_t stride_b, int64_t stride_c, int64_t batch,
                            int b_layout, hipStream_t stream);
 
+// The fp16 product with an epilogue (gemm_epilogue.hpp: kEpiBias with an fp16 bias, kEpiSoftcap, kEpiGeluMul with B2);
+// *supported = false and nothing launched for the few shapes no kernel with that epilogue takes.
+hipError_t launch_gemm_f16_epilogue(const void* A, const void* B, const void* B2, const void* bias, void* C,
+                                    int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc,
+                                    int b_layout, int epilogue, float ep_param, hipStream_t stream, bool* supported);
+
 // The fp16 product through the four-wave 256 x 256 tile kernel with its clock probe (see gemm_f16_ring.hpp); false /
 // nothing launched when the product does not meet that kernel's conditions.
 bool gemm_f16_probe_applies(const void* A, const void* B, const void* C, int64_t M, int64_t N, int64_t K,

@@ -85,10 +85,10 @@ def tensor_mm(lhs: torch.Tensor, rhs: torch.Tensor, out: torch.Tensor | None = N
 
 def tensor_gemm(xt: torch.Tensor, wt: torch.Tensor, bt: torch.Tensor,
                 b_layout: int = capi.B_ROW_MAJOR) -> torch.Tensor:
-    """xt @ wt + bt (bias per output column), float32."""
+    """xt @ wt + bt (bias per output column), float32 or float16 (fp32 sums, bias added before the rounding)."""
     _check_device(xt, wt, bt)
     _require(xt.dim() == 2 and wt.dim() == 2, "matrix multiplication requires compatible matrices")
-    _require(xt.dtype == torch.float32 and wt.dtype == torch.float32 and bt.dtype == torch.float32,
+    _require(xt.dtype in (torch.float32, torch.float16) and wt.dtype == xt.dtype and bt.dtype == xt.dtype,
              "Unsupported data type")
     _require(xt.is_contiguous() and wt.is_contiguous() and bt.is_contiguous(), "dense operands expected")
     m, k = xt.shape
@@ -96,7 +96,12 @@ def tensor_gemm(xt: torch.Tensor, wt: torch.Tensor, bt: torch.Tensor,
     _require((wt.shape[0] if b_layout == capi.B_ROW_MAJOR else wt.shape[1]) == k,
              "matrix multiplication requires compatible matrices")
     _require(bt.numel() == n, "incorrect bias shape")
-    out = torch.empty((m, n), dtype=torch.float32, device=xt.device)
+    out = torch.empty((m, n), dtype=xt.dtype, device=xt.device)
+    if xt.dtype == torch.float16:
+        rc = capi.load().anygpu_gemm_f16_f32acc_bias(xt.data_ptr(), wt.data_ptr(), bt.data_ptr(), out.data_ptr(), m, n, k,
+                                                     max(k, 1), max(wt.shape[1], 1), max(n, 1), b_layout, _stream_ptr())
+        capi.check("anygpu_gemm_f16_f32acc_bias", rc)
+        return out
     rc = capi.load().anygpu_gemm_f32(xt.data_ptr(), wt.data_ptr(), bt.data_ptr(), out.data_ptr(), m, n, k,
                                      max(k, 1), max(wt.shape[1], 1), max(n, 1), capi.A_ROW_MAJOR, b_layout,
                                      _stream_ptr())
@@ -105,17 +110,23 @@ def tensor_gemm(xt: torch.Tensor, wt: torch.Tensor, bt: torch.Tensor,
 
 
 def tensor_gemma_linear_softcap(xt: torch.Tensor, wt: torch.Tensor, final_softcapping: float) -> torch.Tensor:
-    """softcap(xt @ wt^T): xt [b, s, hidden], wt [vocab, hidden] -> [b, s, vocab], float32.
+    """softcap(xt @ wt^T): xt [b, s, hidden], wt [vocab, hidden] -> [b, s, vocab], float32 or float16.
 
     Same contract as tensor_gemma_linear_softcap of the reference (srcs/models/gemma2/gemma_linsoftcap.hpp:12-41).
     """
     _check_device(xt, wt)
     _require(xt.dim() == 3, "xt should be 3 dim")
     _require(wt.dim() == 2 and xt.shape[2] == wt.shape[1], "hidden size should match for xt and wt")
-    _require(xt.dtype == torch.float32 and wt.dtype == torch.float32, "Unsupported data types")
+    _require(xt.dtype in (torch.float32, torch.float16) and wt.dtype == xt.dtype, "Unsupported data types")
     _require(xt.is_contiguous() and wt.is_contiguous(), "dense operands expected")
     m, k, n = xt.shape[0] * xt.shape[1], xt.shape[2], wt.shape[0]
-    out = torch.empty((xt.shape[0], xt.shape[1], n), dtype=torch.float32, device=xt.device)
+    out = torch.empty((xt.shape[0], xt.shape[1], n), dtype=xt.dtype, device=xt.device)
+    if xt.dtype == torch.float16:
+        rc = capi.load().anygpu_gemm_f16_f32acc_softcap(xt.data_ptr(), wt.data_ptr(), out.data_ptr(), m, n, k,
+                                                        max(k, 1), max(k, 1), max(n, 1), capi.B_COL_MAJOR,
+                                                        float(final_softcapping), _stream_ptr())
+        capi.check("anygpu_gemm_f16_f32acc_softcap", rc)
+        return out
     rc = capi.load().anygpu_gemm_f32_softcap(xt.data_ptr(), wt.data_ptr(), out.data_ptr(), m, n, k,
                                              max(k, 1), max(k, 1), max(n, 1), capi.B_COL_MAJOR,
                                              float(final_softcapping), _stream_ptr())
@@ -123,23 +134,25 @@ def tensor_gemma_linear_softcap(xt: torch.Tensor, wt: torch.Tensor, final_softca
     return out
 
 
-def mlp_gemma2_fused_upproj(xt: torch.Tensor, wt_gp: torch.Tensor, wt_up: torch.Tensor) -> torch.Tensor:
-    """gelu_tanh(xt @ wt_gp) * (xt @ wt_up): xt [..., hidden], weights [hidden, intermediate], float32.
+def mlp_gemma2_fused_upproj(xt: torch.Tensor, wt_gp: torch.Tensor, wt_up: torch.Tensor,
+                            b_layout: int = capi.B_ROW_MAJOR) -> torch.Tensor:
+    """gelu_tanh(xt @ wt_gp) * (xt @ wt_up): xt [..., hidden], weights [hidden, intermediate] (or [intermediate, hidden]
+    with B_COL_MAJOR), float32 or float16.
 
     Same contract as cu_mlp_gemma2_fused_upproj_f32_v1 / _v2 (srcs/kernels/cuda/mlp_gemma2_fused_upproj.cuh:6-16).
     """
     _check_device(xt, wt_gp, wt_up)
     _require(wt_gp.dim() == 2 and tuple(wt_gp.shape) == tuple(wt_up.shape), "gate and up weights must agree")
-    _require(xt.dim() >= 1 and xt.shape[-1] == wt_gp.shape[0], "hidden size should match for xt and the weights")
-    _require(all(t.dtype == torch.float32 for t in (xt, wt_gp, wt_up)), "Unsupported data types")
+    k, n = wt_gp.shape if b_layout == capi.B_ROW_MAJOR else (wt_gp.shape[1], wt_gp.shape[0])
+    _require(xt.dim() >= 1 and xt.shape[-1] == k, "hidden size should match for xt and the weights")
+    _require(xt.dtype in (torch.float32, torch.float16) and all(t.dtype == xt.dtype for t in (wt_gp, wt_up)), "Unsupported data types")
     _require(xt.is_contiguous() and wt_gp.is_contiguous() and wt_up.is_contiguous(), "dense operands expected")
-    k, n = wt_gp.shape
     m = xt.numel() // k if k else 0
-    out = torch.empty(tuple(xt.shape[:-1]) + (n,), dtype=torch.float32, device=xt.device)
-    rc = capi.load().anygpu_gemm_f32_gelu_mul(xt.data_ptr(), wt_gp.data_ptr(), wt_up.data_ptr(), out.data_ptr(),
-                                              m, n, k, max(k, 1), max(n, 1), max(n, 1), capi.B_ROW_MAJOR,
-                                              _stream_ptr())
-    capi.check("anygpu_gemm_f32_gelu_mul", rc)
+    out = torch.empty(tuple(xt.shape[:-1]) + (n,), dtype=xt.dtype, device=xt.device)
+    fn_name = "anygpu_gemm_f16_f32acc_gelu_mul" if xt.dtype == torch.float16 else "anygpu_gemm_f32_gelu_mul"
+    rc = getattr(capi.load(), fn_name)(xt.data_ptr(), wt_gp.data_ptr(), wt_up.data_ptr(), out.data_ptr(),
+                                       m, n, k, max(k, 1), max(wt_gp.shape[1], 1), max(n, 1), b_layout, _stream_ptr())
+    capi.check(fn_name, rc)
     return out
 
 

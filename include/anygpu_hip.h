@@ -95,6 +95,32 @@ int anygpu_gemm_f16_f32acc(const void* A, const void* B, void* C,
                            int b_layout, void* stream);
 
 /*
+ * anygpu_gemm_f16_f32acc with the epilogues the models hang on their linear layers, applied to the fp32 sums before the
+ * one rounding to fp16 (operands, layouts and leading dimensions as above):
+ *   _bias      C = A * B + bias[N] (bias fp16)          tensor_gemm / tensor_linear with a bias (srcs/ops/mm_ops.hpp:102-171)
+ *   _softcap   C = softcap * tanh((A * B) / softcap)    the Gemma2 output head, cu_tensor_gemma_linear_softcap_f32
+ *                                                       (srcs/models/gemma2/gemma_linsoftcap.cu:11-33; weights [vocab, hidden]
+ *                                                       = ANYGPU_B_COL_MAJOR), softcap > 0
+ *   _gelu_mul  C = gelu_tanh(A * B_gate) (*) (A * B_up) the Gemma2 MLP up-projection (srcs/models/gemma2/gemma_mlp.hpp:85-90,
+ *                                                       cu_mlp_gemma2_fused_upproj_f32_v1 / _v2); A is read once, B_gate and
+ *                                                       B_up share b_layout and ldb
+ * The reference runs these layers in float32 (anygpu_gemm_f32 and its _softcap / _gelu_mul forms); these are the same
+ * operators for a model held in fp16.  K >= 1.  _gelu_mul needs 16-byte aligned operand rows, K >= 64 and K a multiple
+ * of 8 (with row-major B also N a multiple of 8) unless M <= 64; other shapes return ANYGPU_ERR_UNSUPPORTED.
+ */
+int anygpu_gemm_f16_f32acc_bias(const void* A, const void* B, const void* bias, void* C,
+                                int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc,
+                                int b_layout, void* stream);
+
+int anygpu_gemm_f16_f32acc_softcap(const void* A, const void* B, void* C,
+                                   int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc,
+                                   int b_layout, float softcap, void* stream);
+
+int anygpu_gemm_f16_f32acc_gelu_mul(const void* A, const void* B_gate, const void* B_up, void* C,
+                                    int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc,
+                                    int b_layout, void* stream);
+
+/*
  * Measurement hook: anygpu_gemm_f16_f32acc through the kernel of the whole-tile case (M and N multiples of 256, K a
  * multiple of 64, B column-major, 16-byte aligned rows; anything else returns ANYGPU_ERR_UNSUPPORTED and launches
  * nothing), which additionally leaves four 64-bit counts per 256 x 256 tile in probe[4 * tile .. + 3] (device memory,

@@ -939,6 +939,90 @@ def test_gemm_epilogues_decode_step(ops, oracle, s):
     assert scaled_rel_err(got, want, 1.0) <= TOL_F32
 
 
+# fp16 products with the epilogues: the oracle's float32 operators on the fp16-rounded inputs, tolerance of the fp16 GEMM
+F16_EPILOGUE_SHAPES = [
+    # m, k, n: few rows (band kernels), one tile, ragged tiles of every size, a K tail, whole 256 tiles, several rounds
+    (1, 2304, 1000), (16, 512, 520), (64, 256, 264), (100, 320, 200), (130, 64, 72), (300, 1000, 392), (513, 2304, 1160),
+    (1024, 512, 2048), (2048, 192, 4096), (2304, 136, 4104),
+]
+
+
+@pytest.mark.parametrize("layout", ["row", "col"])
+@pytest.mark.parametrize("m,k,n", F16_EPILOGUE_SHAPES)
+def test_gemm_f16_bias(ops, oracle, layout, m, k, n):
+    from anygpu_amd import capi
+    a = synth.uniform(m + k, (m, k)).astype(np.float16)
+    b = synth.uniform(k + n, (k, n)).astype(np.float16)
+    bias = (synth.normal(n, (n,)) * np.float32(3.0)).astype(np.float16)
+    want = oracle.tensor_gemm(oracle.cvt_f16_to_f32(a), oracle.cvt_f16_to_f32(b), oracle.cvt_f16_to_f32(bias), threads=8)
+    if layout == "row":
+        got = host(ops.tensor_gemm(dev(a), dev(b), dev(bias)))
+    else:
+        got = host(ops.tensor_gemm(dev(a), dev(np.ascontiguousarray(b.T)), dev(bias), b_layout=capi.B_COL_MAJOR))
+    assert got.dtype == np.float16 and got.shape == (m, n)
+    assert scaled_rel_err(got.astype(np.float32), want, math.sqrt(k) / 3.0 + 3.0) <= TOL_F16_GEMM
+    # the bias is part of the result: without it the columns are off by it
+    assert rel_l2(got.astype(np.float32) - oracle.cvt_f16_to_f32(bias)[None, :], oracle.tensor_mm(oracle.cvt_f16_to_f32(a), oracle.cvt_f16_to_f32(b), threads=8)) <= 2e-2
+
+
+@pytest.mark.parametrize("m,k,n", F16_EPILOGUE_SHAPES)
+def test_gemm_f16_softcap(ops, oracle, m, k, n):
+    # the Gemma2 output head in fp16: weights [vocab, hidden], cap 30, logits well past the cap
+    cap = 30.0
+    x = synth.normal(m + k, (1, m, k)).astype(np.float16)
+    w = (synth.normal(k + n, (n, k)) * np.float32(2.0)).astype(np.float16)
+    got = host(ops.tensor_gemma_linear_softcap(dev(x), dev(w), cap)).astype(np.float32)
+    want = oracle.gemma_linear_softcap(oracle.cvt_f16_to_f32(x), oracle.cvt_f16_to_f32(w), cap, threads=8)
+    assert got.shape == (1, m, n)
+    assert scaled_rel_err(got, want, min(cap, 2.0 * math.sqrt(k))) <= TOL_F16_GEMM
+    assert np.all(np.abs(got) <= cap)
+
+
+@pytest.mark.parametrize("layout", ["row", "col"])
+@pytest.mark.parametrize("m,k,n", F16_EPILOGUE_SHAPES)
+def test_gemm_f16_gelu_mul(ops, oracle, layout, m, k, n):
+    # the Gemma2 MLP up-projection in fp16: gate and up weights side by side in one tile, A read once
+    from anygpu_amd import capi
+    x = synth.normal(m + k, (1, m, k)).astype(np.float16)
+    wg = (synth.normal(n + 1, (k, n)) * np.float32(1.5 / math.sqrt(k))).astype(np.float16)
+    wu = (synth.normal(n + 2, (k, n)) * np.float32(1.5 / math.sqrt(k))).astype(np.float16)
+    want = oracle.gemma_mlp_upproj(oracle.cvt_f16_to_f32(x), oracle.cvt_f16_to_f32(wg), oracle.cvt_f16_to_f32(wu), threads=8)
+    if layout == "row":
+        got = host(ops.mlp_gemma2_fused_upproj(dev(x), dev(wg), dev(wu))).astype(np.float32)
+        swapped = host(ops.mlp_gemma2_fused_upproj(dev(x), dev(wu), dev(wg))).astype(np.float32)
+    else:
+        wgt, wut = dev(np.ascontiguousarray(wg.T)), dev(np.ascontiguousarray(wu.T))
+        got = host(ops.mlp_gemma2_fused_upproj(dev(x), wgt, wut, b_layout=capi.B_COL_MAJOR)).astype(np.float32)
+        swapped = host(ops.mlp_gemma2_fused_upproj(dev(x), wut, wgt, b_layout=capi.B_COL_MAJOR)).astype(np.float32)
+    assert got.shape == (1, m, n)
+    assert scaled_rel_err(got, want, 1.5 * 1.5) <= TOL_F16_GEMM
+    if n > 1:
+        assert not np.allclose(swapped, got, atol=1e-2)       # the two weights are not interchangeable
+
+
+def test_gemm_f16_epilogues_rejected_and_odd_shapes(ops, oracle):
+    import torch
+    from anygpu_amd import capi
+    lib = capi.load()
+    # K and N no multiples of 8: bias and softcap fall back to the plain product and a pass over it, the fused
+    # up-projection has no kernel for such operands
+    m, k, n = 70, 100, 51
+    a = synth.uniform(1, (m, k)).astype(np.float16)
+    b = synth.uniform(2, (k, n)).astype(np.float16)
+    bias = synth.normal(3, (n,)).astype(np.float16)
+    got = host(ops.tensor_gemm(dev(a), dev(b), dev(bias))).astype(np.float32)
+    want = oracle.tensor_gemm(oracle.cvt_f16_to_f32(a), oracle.cvt_f16_to_f32(b), oracle.cvt_f16_to_f32(bias))
+    assert scaled_rel_err(got, want, math.sqrt(k) / 3.0 + 1.0) <= TOL_F16_GEMM
+    ad, bd = dev(a), dev(b)
+    y = torch.full((m, n), 3.0, dtype=torch.float16, device="cuda")
+    rc = lib.anygpu_gemm_f16_f32acc_gelu_mul(ad.data_ptr(), bd.data_ptr(), bd.data_ptr(), y.data_ptr(), m, n, k, k, n, n, capi.B_ROW_MAJOR, None)
+    assert rc == capi.ANYGPU_ERR_UNSUPPORTED
+    assert lib.anygpu_gemm_f16_f32acc_softcap(ad.data_ptr(), bd.data_ptr(), y.data_ptr(), m, n, k, k, n, n, capi.B_ROW_MAJOR, 0.0, None) == capi.ANYGPU_ERR_UNSUPPORTED
+    assert lib.anygpu_gemm_f16_f32acc_bias(ad.data_ptr(), bd.data_ptr(), None, y.data_ptr(), m, n, k, k, n, n, capi.B_ROW_MAJOR, None) == capi.ANYGPU_ERR_NULL_POINTER
+    torch.cuda.synchronize()
+    assert bool((y == 3.0).all())
+
+
 def _random_mm_shapes(seed, count, k_max):
     rng = np.random.default_rng(seed)
     shapes = []
