@@ -23,21 +23,33 @@ constexpr int kAttnXcds = 8;
 // 56 us); the heads of a group always stay together.
 constexpr int kAttnUnitBlocks = 4;
 
+// Key splits.  Under a sliding window many query blocks walk the same, maximal number of key tiles, and when that number
+// is a large share of what one CU gets of the whole launch, whole blocks cannot be packed evenly onto the CUs (8 heads x
+// 8192 queries, window 4096: 256 blocks of 66 tiles and 256 of 2 .. 64 on 256 CUs last 66 + 64 tile times where the
+// work averages 99).  The `n_split` latest query blocks of every head are therefore dispatched as two blocks, one per
+// half of the key range, that leave unnormalised partial results for a merge kernel.  Dispatch order, heaviest first:
+// the `n_big` unsplit blocks below the split range that still walk more tiles than a half, then the halves, then the rest.
 struct AttnWalk
 {
-	int q_blocks;        // query blocks per head
+	int q_blocks;        // dispatched ("virtual") query blocks per head: the real ones + n_split
 	int groups;          // key / value groups (batch x kv heads)
 	int q_per_kv;        // query heads per group
 	int chunk;           // adjacent query blocks per unit
 	int chunks;          // units per group
 	int units;           // chunks * groups
 	int units_per_xcd;
+	int real_q_blocks;   // query blocks per head
+	int n_split;         // the latest n_split query blocks of a head are dispatched in two halves of their key range
+	int n_big;           // unsplit blocks dispatched before the halves
 };
 
-inline AttnWalk make_attn_walk(int64_t q_blocks, int64_t batch_heads, int64_t q_per_kv)
+inline AttnWalk make_attn_walk(int64_t q_blocks, int64_t batch_heads, int64_t q_per_kv, int64_t n_split = 0, int64_t n_big = 0)
 {
 	AttnWalk w;
-	w.q_blocks = (int)q_blocks;
+	w.real_q_blocks = (int)q_blocks;
+	w.n_split = (int)n_split;
+	w.n_big = (int)n_big;
+	w.q_blocks = (int)(q_blocks + n_split);
 	w.q_per_kv = (int)q_per_kv;
 	w.groups = (int)(batch_heads / q_per_kv);
 	w.chunk = q_per_kv >= kAttnUnitBlocks ? 1 : (int)(kAttnUnitBlocks / q_per_kv);
@@ -53,8 +65,19 @@ inline int64_t attn_walk_blocks(const AttnWalk& w)
 	return (int64_t)kAttnXcds * w.units_per_xcd * w.chunk * w.q_per_kv;
 }
 
-// false: a padding block (the last round of units or the last chunk of a head is not full)
+// false: a padding block (the last round of units or the last chunk of a head is not full).  part / parts: which half
+// of the key range the block walks (parts = 1: all of it); split_slot numbers the split blocks of a head from the last.
+__device__ __forceinline__ bool attn_walk_locate_part(const AttnWalk& w, unsigned block, int& head, int& q_block,
+                                                      int& part, int& parts, int& split_slot);
+
 __device__ __forceinline__ bool attn_walk_locate(const AttnWalk& w, unsigned block, int& head, int& q_block)
+{
+	int part, parts, slot;
+	return attn_walk_locate_part(w, block, head, q_block, part, parts, slot);
+}
+
+__device__ __forceinline__ bool attn_walk_locate_part(const AttnWalk& w, unsigned block, int& head, int& q_block,
+                                                      int& part, int& parts, int& split_slot)
 {
 	const int xcd = (int)(block % kAttnXcds);
 	const int slot = (int)(block / kAttnXcds);
@@ -64,9 +87,28 @@ __device__ __forceinline__ bool attn_walk_locate(const AttnWalk& w, unsigned blo
 	if (unit >= w.units) return false;
 	const int chunk_index = w.chunks - 1 - unit / w.groups;       // late query blocks walk the most keys: first
 	const int group = unit % w.groups;
-	q_block = chunk_index * w.chunk + (w.chunk - 1 - member / w.q_per_kv);
+	const int v_block = chunk_index * w.chunk + (w.chunk - 1 - member / w.q_per_kv);
 	head = group * w.q_per_kv + member % w.q_per_kv;
-	return q_block < w.q_blocks;
+	part = 0;
+	parts = 1;
+	split_slot = 0;
+	q_block = v_block;
+	if (v_block >= w.q_blocks) return false;
+	if (w.n_split > 0)
+	{
+		const int rank = w.q_blocks - 1 - v_block;               // 0: dispatched first
+		const int first_split = w.real_q_blocks - w.n_split;     // first split query block
+		if (rank < w.n_big) q_block = first_split - 1 - rank;
+		else if (rank < w.n_big + 2 * w.n_split)
+		{
+			split_slot = (rank - w.n_big) >> 1;
+			part = (rank - w.n_big) & 1;
+			parts = 2;
+			q_block = w.real_q_blocks - 1 - split_slot;
+		}
+		else q_block = first_split - w.n_big - 1 - (rank - w.n_big - 2 * w.n_split);
+	}
+	return true;
 }
 
 }  // namespace anygpu

@@ -12,6 +12,21 @@ namespace anygpu {
 // afterwards (hipGetLastError) belongs to that launch and to nothing earlier in the process.
 inline void discard_stale_error() { (void)hipGetLastError(); }
 
+// Compute units of the current device (256 on an MI355X), asked once per device; 256 if the runtime cannot tell.
+inline int device_cu_count()
+{
+	static int cached[64] = {};
+	int device = 0;
+	if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64) return 256;
+	if (cached[device] == 0)
+	{
+		int cus = 0;
+		if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || cus <= 0) cus = 256;
+		cached[device] = cus;
+	}
+	return cached[device];
+}
+
 // mask (may be NULL): additive [q_len, cols] matrix of the element type, rows mask_stride apart
 template <typename T>
 hipError_t launch_softmax_rows(const void* x, void* y, int64_t rows, int64_t cols, int64_t xs, int64_t ys,

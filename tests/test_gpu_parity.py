@@ -1548,6 +1548,35 @@ def test_sdp_attention_fused_kernel_gemma2_block(ops, oracle):
     assert np.isfinite(got).all()
 
 
+def test_sdp_attention_key_split_blocks_agree_with_whole_blocks(ops, oracle):
+    # A windowed launch with at least a block per CU whose longest blocks are a large share of a CU's work is dispatched
+    # with those blocks in two key halves plus a merge (partial results in the stream's K-split workspace).  With a
+    # workspace too small for a single partial the same call runs whole blocks.  Both against the oracle, and against
+    # each other to the rounding of the fp16 result; a ragged last query block and a head_dim of 128 included.
+    import torch
+    for h, hkv, n, d, win, cap in [(8, 4, 6144 - 40, 256, 2048, 50.0), (16, 8, 4096, 128, 1024, 0.0)]:
+        q = synth.normal(1, (h, n, d)).astype(np.float16)
+        k = synth.normal(2, (hkv, n, d)).astype(np.float16)
+        v = synth.normal(3, (hkv, n, d)).astype(np.float16)
+        alpha = 1.0 / math.sqrt(d)
+        split = host(ops.sdp_attention_fwd(dev(q), dev(k), dev(v), alpha, softcap=cap, causal=True, window=win)).astype(np.float32)
+        tiny = torch.empty((64,), device="cuda")
+        ops.set_workspace(tiny)
+        try:
+            whole = host(ops.sdp_attention_fwd(dev(q), dev(k), dev(v), alpha, softcap=cap, causal=True, window=win)).astype(np.float32)
+        finally:
+            torch.cuda.synchronize()
+            ops.set_workspace(None)
+        assert np.isfinite(split).all()
+        assert scaled_rel_err(split, whole, 1.0) <= 2e-3
+        assert not np.array_equal(split, whole), "the launch was expected to take the key-split path"
+        idx = np.array([0, 127, 128, 1000, n - 2049, n - 2048, n - 1000, n - 129, n - 128, n - 1], dtype=np.int64)
+        want = oracle.sdp_attention_rules(*(oracle.cvt_f16_to_f32(t) for t in (q, k, v)), alpha=alpha, softcap=cap,
+                                          causal=True, window=win, q_per_kv=h // hkv, query_index=idx, threads=8)
+        assert scaled_rel_err(split[:, idx, :], want, 1.0) <= TOL_F16_ROWOPS * 2
+        assert scaled_rel_err(whole[:, idx, :], want, 1.0) <= TOL_F16_ROWOPS * 2
+
+
 # =============================================================================================
 # launches recorded into a HIP graph
 # =============================================================================================
