@@ -25,6 +25,7 @@
 #include "device_utils.hpp"
 #include "attention_walk.hpp"
 #include "attention_split.hpp"
+#include "gemm_band.hpp"
 #include "launch.hpp"
 
 #include <atomic>
@@ -46,6 +47,7 @@ struct AttnArgsF32
 	int causal;
 	int window;            // 0: off; else key j is visible iff j > i + diag - window
 	float k_in, k_cap;     // logit transform constants (see logit2)
+	float* partials;       // key-split blocks leave their partial results here: [head][split slot][part][query][D + 2]
 };
 
 // log2(e) * softcap(alpha * s); without softcap k_in = alpha log2(e); with it
@@ -107,8 +109,8 @@ __global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f32_kernel(const
 	const int wave = tid >> 6;
 	const int n = lane & 15;                        // query inside the wave's block (second MFMA operand index)
 	const int g = lane >> 4;                        // lane group: summation slot g of an MFMA
-	int bh, q_block;
-	if (!attn_walk_locate(walk, blockIdx.x, bh, q_block)) return;       // the whole block
+	int bh, q_block, part, parts, split_slot;
+	if (!attn_walk_locate_part(walk, blockIdx.x, bh, q_block, part, parts, split_slot)) return;       // the whole block
 	const int q0 = q_block * kQueriesPerBlock;
 	const float* qp = a.q + (int64_t)bh * a.n_q * D;
 	const float* kp = a.k + (int64_t)(bh / a.q_per_kv) * a.n_k * D;
@@ -121,8 +123,15 @@ __global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f32_kernel(const
 	if (a.causal && q_last + a.diag < key_hi) key_hi = q_last + a.diag;
 	int key_lo = 0;
 	if (a.window > 0 && q0 + a.diag - a.window + 1 > 0) key_lo = q0 + a.diag - a.window + 1;
-	const int t_first = key_lo / kKeysPerTile;
-	const int t_last = key_hi >= 0 ? key_hi / kKeysPerTile : -1;
+	int t_first = key_lo / kKeysPerTile;
+	int t_last = key_hi >= 0 ? key_hi / kKeysPerTile : -1;
+	if (parts == 2)
+	{
+		// one half of the block's key tiles; the other half is another block's, a merge kernel combines the two
+		const int mid = t_first + (t_last - t_first + 2) / 2;
+		if (part == 0) t_last = mid - 1;
+		else t_first = mid;
+	}
 
 	// this lane's query as second operand: q[row][16 s + 4 g .. + 3]
 	const int q_row = q0 + 16 * wave + n;
@@ -339,6 +348,25 @@ __global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f32_kernel(const
 	float l = l_run;
 	l += __shfl_xor(l, 16);
 	l += __shfl_xor(l, 32);
+	if (parts == 2)
+	{
+		// unnormalised accumulators, running maximum and sum of this half of the keys
+		if (q_row < a.n_q)
+		{
+			float* dst = a.partials + ((((int64_t)bh * walk.n_split + split_slot) * 2 + part) * kQueriesPerBlock + (q_row - q0)) * (D + 2);
+#pragma unroll
+			for (int c = 0; c < DC; ++c)
+#pragma unroll
+				for (int r = 0; r < 4; ++r)
+					*reinterpret_cast<WsFloat4*>(dst + 64 * c + 16 * g + 4 * r) = float4_t{o[c][0][r], o[c][1][r], o[c][2][r], o[c][3][r]};
+			if (g == 0)
+			{
+				dst[D] = m_run;
+				dst[D + 1] = l;
+			}
+		}
+		return;
+	}
 	const float inv = l > 0.0f ? 1.0f / l : 0.0f;
 	if (q_row < a.n_q)
 	{
@@ -354,7 +382,7 @@ __global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f32_kernel(const
 }
 
 template <int D, bool SOFTCAP>
-hipError_t launch_variant_f32(const AttnArgsF32& args, int64_t batch_heads, hipStream_t stream)
+hipError_t launch_variant_f32(const AttnArgsF32& args_in, int64_t batch_heads, hipStream_t stream)
 {
 	// head dimension 256: 8 waves (two per SIMD) on tiles of 32 keys in two stages, 130 KB, one block per CU.  Two
 	// alternatives with two blocks of 4 waves per CU, for a better balance of long and short blocks under the causal
@@ -381,8 +409,24 @@ hipError_t launch_variant_f32(const AttnArgsF32& args, int64_t batch_heads, hipS
 			configured_devices.fetch_or(bit, std::memory_order_relaxed);
 		}
 	}
-	const AttnWalk walk = make_attn_walk((args.n_q + kQueriesPerBlock - 1) / kQueriesPerBlock, batch_heads, args.q_per_kv);
+	AttnArgsF32 args = args_in;
+	const int64_t q_blocks = (args.n_q + kQueriesPerBlock - 1) / kQueriesPerBlock;
+	const AttnSplitPlan plan = plan_attention_split(args.n_q, args.n_k, args.causal, args.diag, args.window, batch_heads,
+	                                                kQueriesPerBlock, KT, D, band::workspace_capacity(stream));
+	args.partials = nullptr;
+	if (plan.n_split > 0)
+	{
+		const hipError_t ws_err = band::workspace_acquire(stream, &args.partials);
+		if (ws_err != hipSuccess) return ws_err;
+	}
+	const AttnWalk walk = make_attn_walk(q_blocks, batch_heads, args.q_per_kv, plan.n_split, plan.n_big);
+	if (attn_walk_blocks(walk) > 0x7FFFFFFFLL) return hipErrorInvalidValue;
 	kernel<<<dim3((unsigned)attn_walk_blocks(walk)), dim3(64 * WAVES), kLdsBytes, stream>>>(args, walk);
+	const hipError_t err = hipGetLastError();
+	if (err != hipSuccess || plan.n_split == 0) return err;
+	const int64_t items = batch_heads * plan.n_split * kQueriesPerBlock * (D / 4);
+	sdp_attention_merge_halves_kernel<D, float><<<dim3((unsigned)((items + 255) / 256)), dim3(256), 0, stream>>>(
+		args.partials, args.y, args.n_q, (int)q_blocks, (int)plan.n_split, kQueriesPerBlock);
 	return hipGetLastError();
 }
 
@@ -596,6 +640,7 @@ hipError_t launch_sdp_attention_fwd_f32(const float* q, const float* k, const fl
 	const bool capped = softcap != 0.0f;
 	args.k_in = capped ? 2.0f * kLog2e * alpha / softcap : alpha * kLog2e;
 	args.k_cap = capped ? softcap * kLog2e : 0.0f;
+	args.partials = nullptr;
 #define ANYGPU_ATTN_F32_DIM(DIM) \
 	return capped ? launch_variant_f32<DIM, true>(args, batch_heads, stream) : launch_variant_f32<DIM, false>(args, batch_heads, stream)
 	switch (head_dim)
@@ -642,6 +687,7 @@ hipError_t launch_sdp_attention_decode_f32(const float* q, const float* k, const
 	const bool capped = softcap != 0.0f;
 	da.a.k_in = capped ? 2.0f * kLog2e * alpha / softcap : alpha * kLog2e;
 	da.a.k_cap = capped ? softcap * kLog2e : 0.0f;
+	da.a.partials = nullptr;
 	da.ws = static_cast<float*>(workspace);
 	da.rows = (int)(q_per_kv * n_q);
 	da.splits = p.splits;

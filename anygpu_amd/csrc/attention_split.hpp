@@ -7,11 +7,13 @@
 // M = max m_i,  y = sum o_i 2^(m_i - M) / sum l_i 2^(m_i - M).
 #pragma once
 
+#include <algorithm>
 #include <cstdint>
 
 #include <hip/hip_runtime.h>
 
 #include "device_utils.hpp"
+#include "launch.hpp"
 
 namespace anygpu {
 
@@ -113,6 +115,81 @@ __global__ __launch_bounds__(256) void sdp_decode_merge_kernel(const float* __re
 		const float4_t zero = {0.0f, 0.0f, 0.0f, 0.0f};
 		store_merged(y + ((int64_t)kvh * rows + row) * D + 4 * t, sum > 0.0f ? acc / sum : zero);
 	}
+}
+
+// ---------------------------------------------------------------------------------------------
+// Key-split query blocks of the fused kernels (see AttnWalk): two blocks walk one half each of a query block's key tiles
+// and leave [query][head_dim accumulators, maximum, sum] in the workspace, [head][split slot][half][query][head_dim + 2].
+// ---------------------------------------------------------------------------------------------
+
+// y rows of the key-split blocks from the two partial results of each: one thread per four columns of a row.
+template <int D, typename OutT>
+__global__ __launch_bounds__(256) void sdp_attention_merge_halves_kernel(const float* __restrict__ partials, OutT* __restrict__ y,
+                                                                         int n_q, int q_blocks, int n_split, int queries_per_block)
+{
+	constexpr int kQuads = D / 4;
+	const int64_t item = (int64_t)blockIdx.x * 256 + threadIdx.x;
+	const int quad = (int)(item % kQuads);
+	const int64_t row_item = item / kQuads;
+	const int r = (int)(row_item % queries_per_block);
+	const int64_t slot_item = row_item / queries_per_block;            // head * n_split + split slot
+	const int split_slot = (int)(slot_item % n_split);
+	const int64_t bh = slot_item / n_split;
+	const int q_row = (q_blocks - 1 - split_slot) * queries_per_block + r;
+	if (q_row >= n_q) return;
+	const float* p0 = partials + ((slot_item * 2) * queries_per_block + r) * (D + 2);
+	const float* p1 = p0 + (int64_t)queries_per_block * (D + 2);
+	const float m0 = p0[D], l0 = p0[D + 1], m1 = p1[D], l1 = p1[D + 1];
+	const float big = fmaxf(m0, m1);
+	const float safe = big == -INFINITY ? 0.0f : big;
+	const float w0 = fast_exp2(m0 - safe), w1 = fast_exp2(m1 - safe);
+	const float sum = l0 * w0 + l1 * w1;
+	const float inv = sum > 0.0f ? 1.0f / sum : 0.0f;
+	const float4_t a0 = *reinterpret_cast<const WsFloat4*>(p0 + 4 * quad), a1 = *reinterpret_cast<const WsFloat4*>(p1 + 4 * quad);
+	store_merged(y + (bh * n_q + q_row) * D + 4 * quad, (a0 * w0 + a1 * w1) * inv);
+}
+
+// How many of a head's latest query blocks to dispatch in two key halves (and how many unsplit ones go out before the
+// halves).  Worth it when whole blocks cannot be packed evenly: at least a block per CU, and the longest block a large
+// share of what a CU gets of the whole launch.  Bounded by the workspace of the stream (the K-split workspace of the
+// GEMMs: a caller's, or the library's own for eager launches; none under capture without a caller's: then no split).
+struct AttnSplitPlan { int64_t n_split, n_big; };
+
+inline AttnSplitPlan plan_attention_split(int n_q, int n_k, int causal, int diag, int window, int64_t batch_heads,
+                                          int queries_per_block, int keys_per_tile, int head_dim, size_t capacity)
+{
+	AttnSplitPlan plan{0, 0};
+	const int64_t q_blocks = (n_q + queries_per_block - 1) / queries_per_block;
+	const int cus = device_cu_count();
+	if (q_blocks * batch_heads < cus || q_blocks > 65536 || capacity == 0) return plan;
+	const auto tiles_of = [&](int64_t b) {
+		const int64_t q0 = b * queries_per_block;
+		const int64_t q_last = std::min<int64_t>(q0 + queries_per_block - 1, n_q - 1);
+		int64_t key_hi = n_k - 1;
+		if (causal && q_last + diag < key_hi) key_hi = q_last + diag;
+		int64_t key_lo = 0;
+		if (window > 0 && q0 + diag - window + 1 > 0) key_lo = q0 + diag - window + 1;
+		return key_hi >= 0 && key_hi >= key_lo ? key_hi / keys_per_tile - key_lo / keys_per_tile + 1 : (int64_t)0;
+	};
+	int64_t total = 0, longest = 0;
+	for (int64_t b = 0; b < q_blocks; ++b)
+	{
+		total += tiles_of(b);
+		longest = std::max(longest, tiles_of(b));
+	}
+	const double per_cu = (double)total * (double)batch_heads / (double)cus;
+	if (longest < 16 || (double)longest <= 0.6 * per_cu) return plan;
+	const int64_t split_min = std::max<int64_t>(16, (int64_t)(0.6 * per_cu));
+	// the latest blocks that are long enough, as far as the workspace holds their partial results
+	const int64_t room = (int64_t)(capacity / ((size_t)batch_heads * 2 * queries_per_block * (head_dim + 2) * sizeof(float)));
+	int64_t n_split = 0;
+	while (n_split < q_blocks && n_split < room && tiles_of(q_blocks - 1 - n_split) >= split_min) ++n_split;
+	if (n_split == 0) return plan;
+	int64_t n_big = 0;
+	while (n_split + n_big < q_blocks && 2 * tiles_of(q_blocks - 1 - n_split - n_big) > longest) ++n_big;
+	plan.n_split = n_split;
+	plan.n_big = n_big;
+	return plan;
 }
 
 }  // namespace anygpu

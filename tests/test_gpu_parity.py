@@ -1575,6 +1575,17 @@ def test_sdp_attention_key_split_blocks_agree_with_whole_blocks(ops, oracle):
                                           causal=True, window=win, q_per_kv=h // hkv, query_index=idx, threads=8)
         assert scaled_rel_err(split[:, idx, :], want, 1.0) <= TOL_F16_ROWOPS * 2
         assert scaled_rel_err(whole[:, idx, :], want, 1.0) <= TOL_F16_ROWOPS * 2
+        # the float32 kernel takes the same path
+        q32, k32, v32 = (oracle.cvt_f16_to_f32(t) for t in (q, k, v))
+        split32 = host(ops.sdp_attention_fwd(dev(q32), dev(k32), dev(v32), alpha, softcap=cap, causal=True, window=win))
+        ops.set_workspace(tiny)
+        try:
+            whole32 = host(ops.sdp_attention_fwd(dev(q32), dev(k32), dev(v32), alpha, softcap=cap, causal=True, window=win))
+        finally:
+            torch.cuda.synchronize()
+            ops.set_workspace(None)
+        assert scaled_rel_err(split32, whole32, 1.0) <= TOL_F32
+        assert scaled_rel_err(split32[:, idx, :], want, 1.0) <= TOL_F32
 
 
 # =============================================================================================
