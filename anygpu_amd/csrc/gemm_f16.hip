@@ -22,12 +22,10 @@ namespace anygpu {
 // load at element alignment, the ends of rows element by element, everything outside the operand is zero in LDS.
 // [K, N] weights are transposed on their way into LDS (the MFMA operand is k-contiguous).
 // ---------------------------------------------------------------------------------------------
-// Launches of at most this many 64 x 64 tiles (two per CU) run the form with four LDS stages: alone on its CU a
+// Launches of at most two 64 x 64 tiles per CU run the form with four LDS stages: alone on its CU a
 // block multiplies a slab in a tenth of the memory latency, and with two stages it advanced one slab per latency
 // (256 x 4096 . 4096 x 4096: 29.9 -> 16.0 us, vendor 19.1).  Denser launches keep two stages: 16 KB per stage, five
 // blocks per CU cover the latency with occupancy (1024 x 2048 . 2048 x 2304: 19.3 us against 21.9 with four stages).
-constexpr int64_t kDeepStageBlocks = 512;
-constexpr double kRectSlabUs = 0.93;           // 256 x 128 tile in two k groups: us per 64-deep slab and round of blocks
 constexpr int kEdgeTile = 128;
 constexpr int kEdgeDepth = 32;
 constexpr int kEdgePitch = kEdgeDepth + 8;      // halves per LDS row: 80 bytes, keeps 16-byte alignment
@@ -170,21 +168,34 @@ __global__ __launch_bounds__(256) void gemm_f16_edge_kernel(
 	}
 }
 
-// Time per 64-deep slab of `nblocks` blocks spread over 256 CUs, in us, from measurements: a 256 x 256 tile takes
-// 1.56 per round of blocks (4096^3: 256 blocks, 64 slabs, 100 us); the smaller tiles, of which a CU holds several,
-// follow the average number of blocks per CU with a floor where a lone block waits on latency: 0.75 per block
-// and CU for 128 x 128 (144 blocks 0.75 - 1.0, 288 1.0, 576 1.7 - 2.0), 0.27 for 64 x 64 in dense launches.
-// The cheapest launch is taken, the bigger tile on a tie.
-static double slab_us(int64_t t, int64_t nblocks)
+// What the launcher knows about the cost of its kernels: microseconds per 64-deep slab, measured on one MI355X.  It
+// only ever compares sums of these with each other (and with the two absolute terms of a cut along K), so what decides
+// is their ratios; the boxes of the pool differ by up to 7 % in the clock they sustain, which moves all of them alike.
+// The number of CUs is the device's, not a constant.
+struct TilePrices
 {
-	const double rounds = (double)((nblocks + 255) / 256);
-	const double share = nblocks > 256 ? (double)nblocks / 256.0 : 1.0;
-	if (t == 256) return 1.56 * rounds;
-	if (t == 128) return 0.75 * share;
-	// four stages (see kDeepStageBlocks): 0.22 where every block has a CU of its own, twice 0.21 where some
-	// CUs hold two (they decide when the launch ends)
-	if (nblocks <= kDeepStageBlocks) return nblocks <= 256 ? 0.22 : 0.42;
-	return 0.27 * share;
+	static constexpr double kBig = 1.56;          // 256 x 256, eight waves: per round of blocks (4096^3: 256 blocks, 64 slabs, 100 us)
+	static constexpr double kBigWhole = 1.45;     // 256 x 256, four waves (whole tiles of k-contiguous operands): 4096^3 93 us
+	static constexpr double kRect = 0.93;         // 256 x 128 in two k groups: per round of blocks
+	static constexpr double kMid = 0.75;          // 128 x 128: per block and CU (144 blocks 0.75 - 1.0, 288 1.0, 576 1.7 - 2.0)
+	static constexpr double kSmallAlone = 0.22;   // 64 x 64 with four stages, a CU per block
+	static constexpr double kSmallPair = 0.42;    //   ... where some CUs hold two (they decide when the launch ends)
+	static constexpr double kSmallDense = 0.27;   // 64 x 64 with two stages in dense launches: per block and CU
+	static constexpr double kMergeLaunchUs = 4.5; // the merge launch of a cut along K
+	static constexpr double kPlaneBytesPerUs = 5.0e6;   // its planes, written and read back at 5 TB/s
+	static constexpr double kSplitSetupSlabs = 3.0;     // prologue and epilogue of a block, in slabs
+};
+
+// Time per 64-deep slab of `nblocks` blocks of tile edge t spread over `cus` CUs.  The smaller tiles, of which a CU holds
+// several, follow the average number of blocks per CU with a floor where a lone block waits on latency.
+static double slab_us(int64_t t, int64_t nblocks, int64_t cus, bool whole_tiles = false)
+{
+	const double rounds = (double)((nblocks + cus - 1) / cus);
+	const double share = nblocks > cus ? (double)nblocks / (double)cus : 1.0;
+	if (t == 256) return (whole_tiles ? TilePrices::kBigWhole : TilePrices::kBig) * rounds;
+	if (t == 128) return TilePrices::kMid * share;
+	if (nblocks <= 2 * cus) return nblocks <= cus ? TilePrices::kSmallAlone : TilePrices::kSmallPair;
+	return TilePrices::kSmallDense * share;
 }
 
 // C[m, n] = half(sum over splits of planes[split][m][n]), one thread per eight columns (N a multiple of 8), the
@@ -289,6 +300,11 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
 		// it run the same kernels with clamped operand rows and guarded stores; a K that is not a multiple of the
 		// 64-deep slab adds a tail multiplied from registers.
 		const auto blocks = [&](int64_t tile) { return ((M + tile - 1) / tile) * ((N + tile - 1) / tile) * batch; };
+		const int64_t cus = device_cu_count();
+		// whole 256 x 256 tiles of k-contiguous operands take the four-wave kernel, which is cheaper per slab
+		const bool whole_tiles = b_layout == ANYGPU_B_COL_MAJOR && reinterpret_cast<uintptr_t>(C) % 16 == 0 && ldc % 8 == 0 && stride_c % 8 == 0 &&
+		                         gemm_f16_ring_applies(a, b, M, N, K, lda, ldb, stride_a, stride_b, batch);
+		const auto slab_us = [cus, whole_tiles](int64_t t, int64_t nblocks) { return anygpu::slab_us(t, nblocks, cus, whole_tiles); };
 		const double cost256 = slab_us(256, blocks(256)), cost128 = slab_us(128, blocks(128)), cost64 = slab_us(64, blocks(64));
 		int64_t tile = (cost256 <= cost128 && cost256 <= cost64) ? 256 : cost128 <= cost64 ? 128 : 64;
 
@@ -297,7 +313,7 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
 		if (tile == 256 && batch == 1)
 		{
 			const int64_t tiles_m = (M + 255) / 256, tiles_n = (N + 255) / 256;
-			const int64_t whole = tiles_m * tiles_n / 256 * 256;
+			const int64_t whole = tiles_m * tiles_n / cus * cus;
 			const int64_t head_cols = whole / tiles_m;
 			if (whole > 0 && head_cols > 0 && head_cols < tiles_n)
 			{
@@ -307,7 +323,7 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
 				if (slab_us(128, tail_blocks(128)) < tail_cost) tail_cost = slab_us(128, tail_blocks(128));
 				if (slab_us(64, tail_blocks(64)) < tail_cost) tail_cost = slab_us(64, tail_blocks(64));
 				const double slabs = (double)((K + 63) / 64);
-				const double divided = (slab_us(256, head_cols * tiles_m) + tail_cost) * slabs + 3.0;
+				const double divided = (slab_us(256, head_cols * tiles_m) + tail_cost) * slabs + TilePrices::kSplitSetupSlabs;
 				if (divided < 0.93 * cost256 * slabs)
 				{
 					const hipError_t err = launch_gemm_f16(A, B, C, M, n_head, K, lda, ldb, ldc, 0, 0, 0, 1, b_layout, stream);
@@ -322,7 +338,7 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
 		// where their number suits the 256 CUs better (2048 x 4096 . 4096 x 4096: 76 -> 62 us, vendor 62;
 		// 1024 x 4096 . 4096 x 6144: 70 -> 55 us, vendor 51).
 		const int64_t blocks_rect = ((M + 255) / 256) * ((N + 127) / 128) * batch;
-		const double cost_rect = kRectSlabUs * (double)((blocks_rect + 255) / 256);
+		const double cost_rect = TilePrices::kRect * (double)((blocks_rect + cus - 1) / cus);
 		const double cost_square = tile == 256 ? cost256 : tile == 128 ? cost128 : cost64;
 		// (against several rounds of 256 x 256 tiles the margin is wider: their later rounds run faster than priced,
 		// 4096 x 4096 . 4096 x 6144, 384 tiles: 176 us where two full rounds would take 200)
@@ -345,10 +361,11 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
 			const int64_t room = (int64_t)(band::workspace_capacity(stream) / ((size_t)M * N * sizeof(float)));
 			for (const int64_t t : {(int64_t)256, (int64_t)128, (int64_t)64})
 			{
-				if (blocks(t) >= 256) continue;
+				if (blocks(t) >= cus) continue;
 				for (int64_t sp = 2; sp <= 16 && sp <= K / 512 && sp <= room; ++sp)
 				{
-					const double cost = (slabs / (double)sp + 3.0) * slab_us(t, blocks(t) * sp) + 4.5 + 8.0 * (double)sp * (double)M * (double)N / 5.0e6;
+					const double cost = (slabs / (double)sp + TilePrices::kSplitSetupSlabs) * anygpu::slab_us(t, blocks(t) * sp, cus) + TilePrices::kMergeLaunchUs +
+					                    8.0 * (double)sp * (double)M * (double)N / TilePrices::kPlaneBytesPerUs;
 					if (cost < 0.9 * best)
 					{
 						best = cost;
@@ -374,7 +391,7 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
 				const hipError_t ws_err = band::workspace_acquire(stream, &planes);
 				if (ws_err != hipSuccess) return ws_err;
 				const int64_t step_b = (b_layout == ANYGPU_B_COL_MAJOR) ? k_split : k_split * ldb;
-				const bool deep_stages = blocks(64) * splits <= kDeepStageBlocks;
+				const bool deep_stages = blocks(64) * splits <= 2 * cus;
 				hipError_t err;
 #define ANYGPU_F16_SPLIT(BT, WM, WN, KN, STG, KG) \
 				err = launch_gemm_f16_tile<GemmTileCfg<BT, BT, WM, WN, 1, 0, 4, 16, KN, STG, KG>, true, true, true>( \
@@ -415,7 +432,7 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
 		}
 		const bool ragged = (M % tile != 0) || (N % tile != 0) || (K % 64 != 0);
 		const bool fits = ((M + tile - 1) / tile) * ((N + tile - 1) / tile) <= 0x7FFFFFFFLL;
-		const bool deep_stages = blocks(64) <= kDeepStageBlocks;
+		const bool deep_stages = blocks(64) <= 2 * cus;
 #define ANYGPU_F16_TILE(BT, WM, WN, KN, STG, KG) \
 		return ragged ? launch_gemm_f16_tile<GemmTileCfg<BT, BT, WM, WN, 1, 0, 4, 16, KN, STG, KG>, true, true>(a, b, c, M, N, K, lda, ldb, ldc, stride_a, stride_b, stride_c, batch, stream) \
 		              : launch_gemm_f16_tile<GemmTileCfg<BT, BT, WM, WN, 1, 0, 4, 16, KN, STG, KG>, false, false>(a, b, c, M, N, K, lda, ldb, ldc, stride_a, stride_b, stride_c, batch, stream)
@@ -423,8 +440,7 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
 		{
 			// whole 256 x 256 tiles of k-contiguous operands: the four-wave kernel with 128 x 128 patches (4096^3: 93 us
 			// against 99 us for the eight-wave tile on the same box, vendor library 93 us)
-			const bool c_aligned = reinterpret_cast<uintptr_t>(C) % 16 == 0 && ldc % 8 == 0 && stride_c % 8 == 0;
-			if (tile == 256 && !ragged && c_aligned && gemm_f16_ring_applies(a, b, M, N, K, lda, ldb, stride_a, stride_b, batch))
+			if (tile == 256 && whole_tiles)
 				return launch_gemm_f16_ring(a, b, c, M, N, K, lda, ldb, ldc, stride_a, stride_b, stride_c, batch, stream);
 			if (tile == 256) ANYGPU_F16_TILE(256, 2, 4, false, 2, 1);
 			if (tile == 128) ANYGPU_F16_TILE(128, 2, 2, false, 2, 1);
@@ -501,7 +517,8 @@ hipError_t launch_gemm_f16_epilogue(const void* A, const void* B, const void* B2
 	}
 	// a tile of edge t covers t (t / 2 with two products) output columns
 	const auto blocks = [&](int64_t t) { return ((M + t - 1) / t) * ((N + (dual ? t / 2 : t) - 1) / (dual ? t / 2 : t)); };
-	const double cost256 = slab_us(256, blocks(256)), cost128 = slab_us(128, blocks(128)), cost64 = slab_us(64, blocks(64));
+	const int64_t cus = device_cu_count();
+	const double cost256 = slab_us(256, blocks(256), cus), cost128 = slab_us(128, blocks(128), cus), cost64 = slab_us(64, blocks(64), cus);
 	const int64_t tile = (cost256 <= cost128 && cost256 <= cost64) ? 256 : cost128 <= cost64 ? 128 : 64;
 	if (blocks(tile) > 0x7FFFFFFFLL)
 	{

@@ -421,7 +421,8 @@ struct TilePlan
 
 constexpr int64_t kSplitMinDepth = 256;
 constexpr int64_t kSplitMax = 16;
-constexpr int64_t kChipCus = 256;
+// the number of CUs is the device's (256 on an MI355X)
+static inline int64_t chip_cus() { return device_cu_count(); }
 
 static TilePlan plan_tiles(int tile, int64_t M, int64_t N, int64_t K, int64_t batch, bool may_split, size_t workspace_bytes)
 {
@@ -429,8 +430,8 @@ static TilePlan plan_tiles(int tile, int64_t M, int64_t N, int64_t K, int64_t ba
 	const int64_t tiles = ((M + tile - 1) / tile) * ((N + tile - 1) / tile) * batch;
 	const int64_t slabs = (K + kBK - 1) / kBK;
 	const auto rounds_of = [tile](int64_t blocks) {
-		if (tile == 64 && blocks > 2 * kChipCus) return (double)blocks / (double)kChipCus;
-		return (double)((blocks + kChipCus - 1) / kChipCus);
+		if (tile == 64 && blocks > 2 * chip_cus()) return (double)blocks / (double)chip_cus();
+		return (double)((blocks + chip_cus() - 1) / chip_cus());
 	};
 	TilePlan best{tile, 1, rounds_of(tiles) * (double)slabs * slab_us};
 	if (!may_split || batch != 1) return best;
@@ -501,7 +502,7 @@ static hipError_t launch_layout(const float* A, const float* B, const float* B2,
 		// is divided by columns into the whole rounds, launched as they are, and the rest, which as a product of its
 		// own is cut along K by the plan above (1024 x 2304 x 9216: 411 us as one launch).
 		const int64_t tiles_m = (M + 127) / 128, tiles_n = (N + 127) / 128;
-		const int64_t whole = tiles_m * tiles_n / kChipCus * kChipCus;
+		const int64_t whole = tiles_m * tiles_n / chip_cus() * chip_cus();
 		const int64_t head_cols = whole / tiles_m;                      // tile columns of the first part
 		if (batch == 1 && whole > 0 && head_cols > 0 && head_cols < tiles_n)
 		{
