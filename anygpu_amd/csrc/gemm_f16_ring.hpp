@@ -25,14 +25,17 @@ struct GemmRingCfg
 	static constexpr int WM = 2, WN = 2;
 };
 
-// blockIdx.y walks a batch of independent products that share the shape.  M and N multiples of 256, K of 64.
+// blockIdx.y walks a batch of independent products that share the shape.  K a multiple of 64.
+// RAGGED: M and N need not be multiples of 256.  Operand rows past the end are read from the last valid row instead (they
+// only feed results that are not stored) and the stores are guarded.
 // probe (may be NULL; first product of a batch only): lane 0 of every block leaves the shader clock count (s_memtime) and
 // the constant 100 MHz count (s_memrealtime) at entry and exit of its main loop in probe[4 block .. + 3], from which a
 // caller gets the clock the part sustained under this kernel and the share of those cycles the matrix cores were busy.
+template <bool RAGGED>
 __global__ __launch_bounds__(256) void gemm_f16_nt_ring_kernel(
 	const half_t* __restrict__ A, const half_t* __restrict__ B, half_t* __restrict__ C,
 	int K, int64_t lda, int64_t ldb, int64_t ldc, int tiles_m, int tiles_n,
-	int64_t stride_a, int64_t stride_b, int64_t stride_c, unsigned long long* __restrict__ probe)
+	int64_t stride_a, int64_t stride_b, int64_t stride_c, unsigned long long* __restrict__ probe, int64_t M, int64_t N)
 {
 	using Cfg = GemmRingCfg;
 	extern __shared__ __align__(1024) char lds[];
@@ -52,16 +55,36 @@ __global__ __launch_bounds__(256) void gemm_f16_nt_ring_kernel(
 
 	// Direct loads.  A unit row is 64 halves = 128 bytes = eight 16-byte chunks; chunk c of row r sits at position
 	// c ^ ((r >> 1) & 7).  One instruction fills 8 rows: lane -> row lane / 8, position lane % 8.  Instruction q of this
-	// wave covers rows 64 wave + 8 q .. + 7 of the operand's 256; the swizzle of those rows is 4 (q & 1) + lane / 16,
-	// so the even and the odd instructions have one offset each and instruction q + 2 lies 16 rows further on.
-	const unsigned ld_row = lane >> 3, ld_pos = lane & 7, ld_hi = lane >> 4;
-	const unsigned a_voff_e = (unsigned)(ld_row * lda + (ld_pos ^ ld_hi) * 8) * 2;
-	const unsigned a_voff_o = (unsigned)((8 + ld_row) * lda + (ld_pos ^ (4 + ld_hi)) * 8) * 2;
-	const unsigned b_voff_e = (unsigned)(ld_row * ldb + (ld_pos ^ ld_hi) * 8) * 2;
-	const unsigned b_voff_o = (unsigned)((8 + ld_row) * ldb + (ld_pos ^ (4 + ld_hi)) * 8) * 2;
-	const uintptr_t a_wave = reinterpret_cast<uintptr_t>(A + (m0 + 64 * wave) * lda);
-	const uintptr_t b_wave = reinterpret_cast<uintptr_t>(B + (n0 + 64 * wave) * ldb);
+	// wave covers rows 64 wave + 8 q .. + 7 of the operand's 256.  The lane's byte offset from the tile's first row for
+	// each of its 16 loads of a slab goes to the assembly block through a table in LDS (the fifth unit, which the loop
+	// fills last): table[q][lane] for this wave, q < 8 for A, the rest for B.
 	const unsigned lds0 = (unsigned)(uintptr_t)(const __attribute__((address_space(3))) char*)lds;
+	const int ld_row = lane >> 3, ld_pos = lane & 7;
+	unsigned* const table = reinterpret_cast<unsigned*>(lds + 4 * Cfg::kUnitBytes) + wave * (16 * 64) + lane;
+	// (offsets count from the first row of the wave's 64, which keeps them below 2^32 for the row pitches admitted)
+	int64_t a_first = m0 + 64 * wave, b_first = n0 + 64 * wave;
+	if constexpr (RAGGED)
+	{
+		a_first = a_first < M - 1 ? a_first : M - 1;
+		b_first = b_first < N - 1 ? b_first : N - 1;
+	}
+#pragma unroll
+	for (int q = 0; q < 8; ++q)
+	{
+		const int row = 64 * wave + 8 * q + ld_row;
+		const unsigned chunk = ld_pos ^ ((row >> 1) & 7);
+		int64_t a_row = m0 + row, b_row = n0 + row;
+		if constexpr (RAGGED)
+		{
+			a_row = a_row < M - 1 ? a_row : M - 1;
+			b_row = b_row < N - 1 ? b_row : N - 1;
+		}
+		table[64 * q] = (unsigned)(((a_row - a_first) * lda + chunk * 8) * 2);
+		table[64 * (8 + q)] = (unsigned)(((b_row - b_first) * ldb + chunk * 8) * 2);
+	}
+	const unsigned table_addr = lds0 + 4 * Cfg::kUnitBytes + (wave * (16 * 64) + lane) * 4;
+	const uintptr_t a_wave = reinterpret_cast<uintptr_t>(A + a_first * lda);
+	const uintptr_t b_wave = reinterpret_cast<uintptr_t>(B + b_first * ldb);
 	const unsigned wave_share = wave * 8192;               // the wave's 64 rows inside a unit
 	const unsigned lds_wave = lds0 + wave_share;
 	const int slabs = K / 64;
@@ -86,9 +109,7 @@ __global__ __launch_bounds__(256) void gemm_f16_nt_ring_kernel(
 #include "gemm_f16_ring_loop.inc"
 		: "={a[0:31]}"(r0), "={a[32:63]}"(r1), "={a[64:95]}"(r2), "={a[96:127]}"(r3),
 		  "={a[128:159]}"(r4), "={a[160:191]}"(r5), "={a[192:223]}"(r6), "={a[224:255]}"(r7)
-		: [avoffe] "v"(a_voff_e), [avoffo] "v"(a_voff_o), [bvoffe] "v"(b_voff_e), [bvoffo] "v"(b_voff_o),
-		  [aaddr] "v"(a_addr), [baddr] "v"(b_addr),
-		  [arow16] "s"((unsigned)(32 * lda)), [brow16] "s"((unsigned)(32 * ldb)),
+		: [vtab] "v"(table_addr), [aaddr] "v"(a_addr), [baddr] "v"(b_addr),
 		  [abaselo] "s"((unsigned)a_wave), [abasehi] "s"((unsigned)(a_wave >> 32)),
 		  [bbaselo] "s"((unsigned)b_wave), [bbasehi] "s"((unsigned)(b_wave >> 32)),
 		  [ldsw] "s"(lds_wave), [slabs] "s"(slabs)
@@ -126,19 +147,19 @@ __global__ __launch_bounds__(256) void gemm_f16_nt_ring_kernel(
 #pragma unroll
 		for (int j = 0; j < 8; ++j)
 			acc[i][j] = float4_t{(*rows[i])[4 * j], (*rows[i])[4 * j + 1], (*rows[i])[4 * j + 2], (*rows[i])[4 * j + 3]};
-	store_patch_via_lds<Cfg, false, true>(acc, lds, C, ldc, m0 + wm * 128, n0 + wn * 128, wave, lane, 0, 0);
+	store_patch_via_lds<Cfg, RAGGED, !RAGGED>(acc, lds, C, ldc, m0 + wm * 128, n0 + wn * 128, wave, lane, M, N);
 }
 
-// What the kernel assumes, checked on the host before every launch: whole tiles, whole slabs, 16-byte aligned operand
-// rows, and operands small enough for the 32-bit lane offsets (a wave's 64 rows) and the 32-bit row steps.
+// What the kernel assumes, checked on the host before every launch: whole slabs, 16-byte aligned operand rows, and
+// operands small enough for the 32-bit lane offsets (a wave's 64 rows).
 inline bool gemm_f16_ring_applies(const half_t* A, const half_t* B, int64_t M, int64_t N, int64_t K,
                                   int64_t lda, int64_t ldb, int64_t stride_a, int64_t stride_b, int64_t batch)
 {
 	const bool aligned = reinterpret_cast<uintptr_t>(A) % 16 == 0 && reinterpret_cast<uintptr_t>(B) % 16 == 0 &&
 	                     lda % 8 == 0 && ldb % 8 == 0 && stride_a % 8 == 0 && stride_b % 8 == 0;
 	// (the epilogue streams whole 16-byte vectors: C has to be aligned like the operands, which the caller checks)
-	return aligned && M > 0 && N > 0 && M % 256 == 0 && N % 256 == 0 && K >= 64 && K % 64 == 0 &&
-	       lda < (1 << 24) && ldb < (1 << 24) && (M / 256) * (N / 256) <= 0x7FFFFFFFLL && batch >= 1 && batch <= 65535;
+	return aligned && M > 0 && N > 0 && K >= 64 && K % 64 == 0 && lda < (1 << 24) && ldb < (1 << 24) &&
+	       ((M + 255) / 256) * ((N + 255) / 256) <= 0x7FFFFFFFLL && batch >= 1 && batch <= 65535;
 }
 
 inline hipError_t launch_gemm_f16_ring(const half_t* A, const half_t* B, half_t* C, int64_t M, int64_t N, int64_t K,
@@ -146,23 +167,24 @@ inline hipError_t launch_gemm_f16_ring(const half_t* A, const half_t* B, half_t*
                                        int64_t stride_a, int64_t stride_b, int64_t stride_c, int64_t batch, hipStream_t stream,
                                        unsigned long long* probe = nullptr)
 {
-	auto kernel = gemm_f16_nt_ring_kernel;
+	const bool ragged = M % 256 != 0 || N % 256 != 0;
+	auto kernel = ragged ? gemm_f16_nt_ring_kernel<true> : gemm_f16_nt_ring_kernel<false>;
 	// More than 64 KB of dynamic LDS has to be granted per function and per device, once.
-	static std::atomic<uint64_t> configured_devices{0};
+	static std::atomic<uint64_t> configured_devices[2];
 	(void)hipGetLastError();
 	int device = 0;
 	hipError_t e = hipGetDevice(&device);
 	if (e != hipSuccess) return e;
 	const uint64_t bit = 1ull << (device & 63);
-	if ((configured_devices.load(std::memory_order_relaxed) & bit) == 0)
+	if ((configured_devices[ragged].load(std::memory_order_relaxed) & bit) == 0)
 	{
 		e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, GemmRingCfg::kLdsBytes);
 		if (e != hipSuccess) return e;
-		configured_devices.fetch_or(bit, std::memory_order_relaxed);
+		configured_devices[ragged].fetch_or(bit, std::memory_order_relaxed);
 	}
-	const int tiles_m = (int)(M / 256), tiles_n = (int)(N / 256);
+	const int tiles_m = (int)((M + 255) / 256), tiles_n = (int)((N + 255) / 256);
 	kernel<<<dim3((unsigned)(tiles_m * tiles_n), (unsigned)batch), dim3(256), GemmRingCfg::kLdsBytes, stream>>>(
-		A, B, C, (int)K, lda, ldb, ldc, tiles_m, tiles_n, stride_a, stride_b, stride_c, probe);
+		A, B, C, (int)K, lda, ldb, ldc, tiles_m, tiles_n, stride_a, stride_b, stride_c, probe, M, N);
 	return hipGetLastError();
 }
 

@@ -9,6 +9,8 @@ or with spills).  Here every register is fixed:
   a[0:255]                 accumulators, MFMA tile (i, j) of the wave's 8 x 8 patch in a[4 (8 i + j) : + 3]
   v[128:159] / v[160:191]  B / A fragments of a 32-deep step, buffer 0;  v[192:223] / v[224:255]  buffer 1
   v[96:103]                byte offsets of this lane in the wave's eight A loads of a slab, v[104:111] the same for B
+                           (computed by the kernel's C++ part, rows past the end of an operand clamped to its last row,
+                           and handed over through a table in the fifth LDS unit, which the loop fills last)
   v112, v113               LDS addresses the fragment reads of the current step start from (A, B)
   v114, v115               fragment addresses of the second step of a slab (chunk + 4: address bit 6 flipped)
   s[60:64]                 LDS offsets of the units holding A(t), B(t), A(t+1), B(t+1) and of the free unit
@@ -27,10 +29,10 @@ Under the 64 MFMAs of a step a wave issues the 16 fragment reads of the next ste
 first half), its 8 loads with their M0 writes, and the address arithmetic of the next step, never more than three
 instructions behind one MFMA: with one wave per SIMD an MFMA covers 16 cycles, four instructions' worth of issue.
 
-Operands of the block (named): avoffe / avoffo, bvoffe / bvoffo (VGPR: the lane's byte offset in the even / odd loads),
-aaddr, baddr (VGPR: LDS byte address of the lane's fragment chunk inside a unit, minus the wave's share), arow16, brow16
-(SGPR: bytes between rows 16 apart), abaselo / abasehi, bbaselo / bbasehi (SGPR: global address of the wave's first row),
-ldsw (SGPR: LDS address of the wave's 8 KB share of unit 0), slabs (SGPR: K / 64).
+Operands of the block (named): vtab (VGPR: LDS address of the lane's table of 16 load offsets, 256 bytes apart), aaddr,
+baddr (VGPR: LDS byte address of the lane's fragment chunk inside a unit, minus the wave's share), abaselo / abasehi,
+bbaselo / bbasehi (SGPR: global address of the wave's first row), ldsw (SGPR: LDS address of the wave's 8 KB share of
+unit 0), slabs (SGPR: K / 64).
 
 Usage: gen_gemm_f16_ring_loop.py OUTPUT
 """
@@ -102,12 +104,9 @@ emit(f"s_mov_b32 {S_T}, 0", "prologue")
 emit(f"s_sub_u32 {S_LAST}, %[slabs], 1")
 for x in range(5):
     emit(f"s_add_u32 {O[x]}, %[ldsw], {x * UNIT}")
-for q in range(8):
-    src = "%[avoffe]" if q % 2 == 0 else "%[avoffo]"
-    emit(f"v_mov_b32 v{96 + q}, {src}" if q < 2 else f"v_add_u32 v{96 + q}, %[arow16], v{96 + q - 2}")
-for q in range(8):
-    src = "%[bvoffe]" if q % 2 == 0 else "%[bvoffo]"
-    emit(f"v_mov_b32 v{104 + q}, {src}" if q < 2 else f"v_add_u32 v{104 + q}, %[brow16], v{104 + q - 2}")
+for q in range(16):
+    emit(f"ds_read_b32 v{96 + q}, %[vtab] offset:{256 * q}")
+emit("s_waitcnt lgkmcnt(0)")
 emit(f"v_xor_b32 {V_A1}, 64, %[aaddr]")
 emit(f"v_xor_b32 {V_B1}, 64, %[baddr]")
 for n, (operand, slab) in enumerate([("a", 0), ("b", 0), ("a", 1), ("b", 1)]):

@@ -679,11 +679,12 @@ def test_mm_f16_config_4096_cubed_col_major_b(ops, oracle):
 
 
 @pytest.mark.parametrize("m,n,k,pad", [(4096, 4096, 64, 0), (4096, 4096, 128, 0), (4096, 4096, 192, 8), (2048, 8192, 320, 0),
-                                       (8192, 2048, 256, 72), (3840, 4352, 64, 0)])
+                                       (8192, 2048, 256, 72), (3840, 4352, 64, 0), (4000, 3896, 128, 0), (3841, 4104, 64, 8),
+                                       (4095, 4088, 192, 0), (3969, 3848, 64, 0)])
 def test_mm_f16_whole_256_tiles_integer_inputs_exact(ops, m, n, k, pad):
-    # Shapes of whole 256 x 256 tiles with k-contiguous weights take the four-wave kernel whose main loop is an assembly
+    # Shapes of 256 x 256 tiles with k-contiguous weights take the four-wave kernel whose main loop is an assembly
     # block: one slab (K = 64), two, an odd number, padded leading dimensions, a tile count that is no multiple of the
-    # 8 XCDs.  Integers in -2 .. 2 with K <= 320: every sum is an integer below 2^11, exact in fp32 and in the fp16
+    # 8 XCDs, ragged M and N (a last tile of 1 row, of 8 columns: whole waves of it read clamped rows).  Integers in -2 .. 2 with K <= 320: every sum is an integer below 2^11, exact in fp32 and in the fp16
     # result, whatever the order of summation.
     import torch
     from anygpu_amd import capi
