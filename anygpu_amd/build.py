@@ -61,6 +61,7 @@ def build_kernels(verbose: bool = False) -> Path:
     objs = []
     # the main loop of the four-wave fp16 GEMM tile is generated text (an inline-assembly block with fixed registers)
     _run([sys.executable, str(CSRC_DIR / "gen_gemm_f16_ring_loop.py"), str(CSRC_DIR / "gemm_f16_ring_loop.inc")], quiet=not verbose)
+    _run([sys.executable, str(CSRC_DIR / "gen_gemm_f16_ring_loop.py"), str(CSRC_DIR / "gemm_f16_ring_loop_kn.inc"), "kn"], quiet=not verbose)
 
     def compile_one(src: str) -> Path:
         obj = OBJ_DIR / (Path(src).stem + ".o")

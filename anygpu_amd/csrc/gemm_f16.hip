@@ -301,9 +301,9 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
 		// 64-deep slab adds a tail multiplied from registers.
 		const auto blocks = [&](int64_t tile) { return ((M + tile - 1) / tile) * ((N + tile - 1) / tile) * batch; };
 		const int64_t cus = device_cu_count();
-		// whole 256 x 256 tiles of k-contiguous operands take the four-wave kernel, which is cheaper per slab
-		const bool whole_tiles = b_layout == ANYGPU_B_COL_MAJOR && reinterpret_cast<uintptr_t>(C) % 16 == 0 && ldc % 8 == 0 && stride_c % 8 == 0 &&
-		                         gemm_f16_ring_applies(a, b, M, N, K, lda, ldb, stride_a, stride_b, batch);
+		// 256 x 256 tiles of whole 64-deep slabs take the four-wave kernel, which is cheaper per slab
+		const bool whole_tiles = reinterpret_cast<uintptr_t>(C) % 16 == 0 && ldc % 8 == 0 && stride_c % 8 == 0 &&
+		                         gemm_f16_ring_applies(a, b, M, N, K, lda, ldb, stride_a, stride_b, batch, b_layout);
 		const auto slab_us = [cus, whole_tiles](int64_t t, int64_t nblocks) { return anygpu::slab_us(t, nblocks, cus, whole_tiles); };
 		const double cost256 = slab_us(256, blocks(256)), cost128 = slab_us(128, blocks(128)), cost64 = slab_us(64, blocks(64));
 		int64_t tile = (cost256 <= cost128 && cost256 <= cost64) ? 256 : cost128 <= cost64 ? 128 : 64;
@@ -449,6 +449,8 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
 		}
 		if (fits && b_layout == ANYGPU_B_ROW_MAJOR)
 		{
+			if (tile == 256 && whole_tiles)
+				return launch_gemm_f16_ring(a, b, c, M, N, K, lda, ldb, ldc, stride_a, stride_b, stride_c, batch, stream, nullptr, b_layout);
 			if (tile == 256) ANYGPU_F16_TILE(256, 2, 4, true, 2, 1);
 			if (tile == 128) ANYGPU_F16_TILE(128, 2, 2, true, 2, 1);
 			if (deep_stages) ANYGPU_F16_TILE(64, 2, 2, true, 4, 1);

@@ -1,5 +1,5 @@
-// 256 x 256 tile of the fp16 GEMM ("NT": A [M, K] and B [N, K], both K-contiguous) for whole tiles: four waves, one per
-// SIMD, each with a 128 x 128 patch of C in 256 accumulator registers, v_mfma_f32_16x16x32_f16.
+// 256 x 256 tile of the fp16 GEMM (A [M, K]; B [N, K], k-contiguous like A, or [K, N]) for whole 64-deep slabs: four
+// waves, one per SIMD, each with a 128 x 128 patch of C in 256 accumulator registers, v_mfma_f32_16x16x32_f16.
 //
 // Against the eight-wave tile kernel (128 x 64 patches) a patch of 128 x 128 needs a third fewer LDS bytes per MFMA, and
 // under this product the MI355X is power-limited: the bytes saved come back as clock.  One wave per SIMD has nobody to
@@ -8,6 +8,7 @@
 // in that loop at 4096^3: the matrix cores busy 94 - 95 % of the cycles at the 1.6 GHz the part sustains under it.
 #pragma once
 
+#include "anygpu_hip.h"
 #include "gemm_f16_tile.hpp"
 
 namespace anygpu {
@@ -31,7 +32,9 @@ struct GemmRingCfg
 // probe (may be NULL; first product of a batch only): lane 0 of every block leaves the shader clock count (s_memtime) and
 // the constant 100 MHz count (s_memrealtime) at entry and exit of its main loop in probe[4 block .. + 3], from which a
 // caller gets the clock the part sustained under this kernel and the share of those cycles the matrix cores were busy.
-template <bool RAGGED>
+// B_KN: B stored [K, N] (row k holds the n), staged as a [64 k][256 n] unit and read through transposing LDS reads; N is a
+// multiple of 8 then, and column chunks past N are read from the last whole chunk of the row.
+template <bool RAGGED, bool B_KN>
 __global__ __launch_bounds__(256) void gemm_f16_nt_ring_kernel(
 	const half_t* __restrict__ A, const half_t* __restrict__ B, half_t* __restrict__ C,
 	int K, int64_t lda, int64_t ldb, int64_t ldc, int tiles_m, int tiles_n,
@@ -62,6 +65,9 @@ __global__ __launch_bounds__(256) void gemm_f16_nt_ring_kernel(
 	const int ld_row = lane >> 3, ld_pos = lane & 7;
 	unsigned* const table = reinterpret_cast<unsigned*>(lds + 4 * Cfg::kUnitBytes) + wave * (16 * 64) + lane;
 	// (offsets count from the first row of the wave's 64, which keeps them below 2^32 for the row pitches admitted)
+	// A [K, N] unit of B has rows of 256 n = 512 bytes = 32 chunks; one instruction fills 2 k rows: lane -> row lane / 32,
+	// position lane % 32, and the chunk at position p of row k is chunk p ^ kn_row_swizzle(k).  Instruction q of this wave
+	// covers rows 16 wave + 2 q, + 1 of the slab's 64.
 	int64_t a_first = m0 + 64 * wave, b_first = n0 + 64 * wave;
 	if constexpr (RAGGED)
 	{
@@ -80,11 +86,20 @@ __global__ __launch_bounds__(256) void gemm_f16_nt_ring_kernel(
 			b_row = b_row < N - 1 ? b_row : N - 1;
 		}
 		table[64 * q] = (unsigned)(((a_row - a_first) * lda + chunk * 8) * 2);
-		table[64 * (8 + q)] = (unsigned)(((b_row - b_first) * ldb + chunk * 8) * 2);
+		if constexpr (B_KN)
+		{
+			const int k_wave = 2 * q + (lane >> 5);                // the k row, counted from the wave's first
+			int64_t col = (int64_t)(((lane & 31) ^ kn_row_swizzle(16 * wave + k_wave)) << 3);
+			if constexpr (RAGGED)
+				if (n0 + col + 8 > N) col = N - 8 - n0;
+			table[64 * (8 + q)] = (unsigned)((k_wave * ldb + col) * 2);
+		}
+		else
+			table[64 * (8 + q)] = (unsigned)(((b_row - b_first) * ldb + chunk * 8) * 2);
 	}
 	const unsigned table_addr = lds0 + 4 * Cfg::kUnitBytes + (wave * (16 * 64) + lane) * 4;
 	const uintptr_t a_wave = reinterpret_cast<uintptr_t>(A + a_first * lda);
-	const uintptr_t b_wave = reinterpret_cast<uintptr_t>(B + b_first * ldb);
+	const uintptr_t b_wave = reinterpret_cast<uintptr_t>(B_KN ? B + (int64_t)(16 * wave) * ldb + n0 : B + b_first * ldb);
 	const unsigned wave_share = wave * 8192;               // the wave's 64 rows inside a unit
 	const unsigned lds_wave = lds0 + wave_share;
 	const int slabs = K / 64;
@@ -94,7 +109,14 @@ __global__ __launch_bounds__(256) void gemm_f16_nt_ring_kernel(
 	const unsigned frag_row = lane & 15;
 	const unsigned frag_chunk = (lane >> 4) ^ ((frag_row >> 1) & 7);
 	const unsigned a_addr = (wm * 128 + frag_row) * 128 + frag_chunk * 16 - wave_share;
-	const unsigned b_addr = (wn * 128 + frag_row) * 128 + frag_chunk * 16 - wave_share;
+	// B stored [K, N]: lane r of a 16-lane group points a transposing read at k row 8 g + r / 4 (g: the lane's k group),
+	// columns 4 (r % 4) .. + 3 of the MFMA tile; tile j of the patch lies at chunk pair j ^ (row swizzle / 2), a term the
+	// assembly block adds per tile from `b_swizzle`.
+	const unsigned kn_k = 8 * (lane >> 4) + (frag_row >> 2);
+	const unsigned b_addr = B_KN ? kn_k * 512 + (wn * 16 + ((frag_row & 3) >> 1)) * 16 + 8 * (frag_row & 1) - wave_share
+	                             : (wn * 128 + frag_row) * 128 + frag_chunk * 16 - wave_share;
+	[[maybe_unused]] const unsigned b_swizzle = (unsigned)(kn_row_swizzle((int)kn_k) >> 1) << 5;
+	[[maybe_unused]] const unsigned b_step = (unsigned)(128 * ldb);      // bytes from one [K, N] slab to the next
 
 	// The accumulators leave the block as eight vectors of 32 registers pinned to a[0:255]: row i of the patch's MFMA
 	// tiles in vector i.
@@ -105,28 +127,44 @@ __global__ __launch_bounds__(256) void gemm_f16_nt_ring_kernel(
 		ticks_in = __builtin_amdgcn_s_memrealtime();
 	}
 	float32x_t r0, r1, r2, r3, r4, r5, r6, r7;
-	asm volatile(
+#define ANYGPU_RING_OUTPUTS \
+	"={a[0:31]}"(r0), "={a[32:63]}"(r1), "={a[64:95]}"(r2), "={a[96:127]}"(r3), \
+	"={a[128:159]}"(r4), "={a[160:191]}"(r5), "={a[192:223]}"(r6), "={a[224:255]}"(r7)
+#define ANYGPU_RING_INPUTS \
+	[vtab] "v"(table_addr), [aaddr] "v"(a_addr), [baddr] "v"(b_addr), \
+	[abaselo] "s"((unsigned)a_wave), [abasehi] "s"((unsigned)(a_wave >> 32)), \
+	[bbaselo] "s"((unsigned)b_wave), [bbasehi] "s"((unsigned)(b_wave >> 32)), \
+	[ldsw] "s"(lds_wave), [slabs] "s"(slabs)
+#define ANYGPU_RING_CLOBBERS \
+	"v80", "v81", "v82", "v83", "v84", "v85", "v86", "v87", "v88", "v89", "v90", "v91", "v92", "v93", "v94", "v95", \
+	"v96", "v97", "v98", "v99", "v100", "v101", "v102", "v103", "v104", "v105", "v106", "v107", "v108", "v109", \
+	"v110", "v111", "v112", "v113", "v114", "v115", "v116", "v117", "v118", "v119", "v120", "v121", "v122", "v123", \
+	"v124", "v125", "v126", "v127", "v128", "v129", "v130", "v131", "v132", "v133", "v134", "v135", "v136", "v137", \
+	"v138", "v139", "v140", "v141", "v142", "v143", "v144", "v145", "v146", "v147", "v148", "v149", "v150", "v151", \
+	"v152", "v153", "v154", "v155", "v156", "v157", "v158", "v159", "v160", "v161", "v162", "v163", "v164", "v165", \
+	"v166", "v167", "v168", "v169", "v170", "v171", "v172", "v173", "v174", "v175", "v176", "v177", "v178", "v179", \
+	"v180", "v181", "v182", "v183", "v184", "v185", "v186", "v187", "v188", "v189", "v190", "v191", "v192", "v193", \
+	"v194", "v195", "v196", "v197", "v198", "v199", "v200", "v201", "v202", "v203", "v204", "v205", "v206", "v207", \
+	"v208", "v209", "v210", "v211", "v212", "v213", "v214", "v215", "v216", "v217", "v218", "v219", "v220", "v221", \
+	"v222", "v223", "v224", "v225", "v226", "v227", "v228", "v229", "v230", "v231", "v232", "v233", "v234", "v235", \
+	"v236", "v237", "v238", "v239", "v240", "v241", "v242", "v243", "v244", "v245", "v246", "v247", "v248", "v249", \
+	"v250", "v251", "v252", "v253", "v254", "v255", "s60", "s61", "s62", "s63", "s64", "s65", "s66", "s67", "s68", \
+	"s69", "s70", "s71", "s72", "s73", "scc", "m0", "memory"
+	if constexpr (B_KN)
+		asm volatile(
+#include "gemm_f16_ring_loop_kn.inc"
+			: ANYGPU_RING_OUTPUTS
+			: ANYGPU_RING_INPUTS, [bsx] "v"(b_swizzle), [bstep] "s"(b_step)
+			: ANYGPU_RING_CLOBBERS);
+	else
+		asm volatile(
 #include "gemm_f16_ring_loop.inc"
-		: "={a[0:31]}"(r0), "={a[32:63]}"(r1), "={a[64:95]}"(r2), "={a[96:127]}"(r3),
-		  "={a[128:159]}"(r4), "={a[160:191]}"(r5), "={a[192:223]}"(r6), "={a[224:255]}"(r7)
-		: [vtab] "v"(table_addr), [aaddr] "v"(a_addr), [baddr] "v"(b_addr),
-		  [abaselo] "s"((unsigned)a_wave), [abasehi] "s"((unsigned)(a_wave >> 32)),
-		  [bbaselo] "s"((unsigned)b_wave), [bbasehi] "s"((unsigned)(b_wave >> 32)),
-		  [ldsw] "s"(lds_wave), [slabs] "s"(slabs)
-		:
-		  "v96", "v97", "v98", "v99", "v100", "v101", "v102", "v103", "v104", "v105", "v106", "v107", "v108", "v109",
-		  "v110", "v111", "v112", "v113", "v114", "v115", "v116", "v117", "v118", "v119", "v120", "v121", "v122", "v123",
-		  "v124", "v125", "v126", "v127", "v128", "v129", "v130", "v131", "v132", "v133", "v134", "v135", "v136", "v137",
-		  "v138", "v139", "v140", "v141", "v142", "v143", "v144", "v145", "v146", "v147", "v148", "v149", "v150", "v151",
-		  "v152", "v153", "v154", "v155", "v156", "v157", "v158", "v159", "v160", "v161", "v162", "v163", "v164", "v165",
-		  "v166", "v167", "v168", "v169", "v170", "v171", "v172", "v173", "v174", "v175", "v176", "v177", "v178", "v179",
-		  "v180", "v181", "v182", "v183", "v184", "v185", "v186", "v187", "v188", "v189", "v190", "v191", "v192", "v193",
-		  "v194", "v195", "v196", "v197", "v198", "v199", "v200", "v201", "v202", "v203", "v204", "v205", "v206", "v207",
-		  "v208", "v209", "v210", "v211", "v212", "v213", "v214", "v215", "v216", "v217", "v218", "v219", "v220", "v221",
-		  "v222", "v223", "v224", "v225", "v226", "v227", "v228", "v229", "v230", "v231", "v232", "v233", "v234", "v235",
-		  "v236", "v237", "v238", "v239", "v240", "v241", "v242", "v243", "v244", "v245", "v246", "v247", "v248", "v249",
-		  "v250", "v251", "v252", "v253", "v254", "v255", "s60", "s61", "s62", "s63", "s64", "s65", "s66", "s67", "s68",
-		  "s69", "s70", "s71", "s72", "scc", "m0", "memory");
+			: ANYGPU_RING_OUTPUTS
+			: ANYGPU_RING_INPUTS
+			: ANYGPU_RING_CLOBBERS);
+#undef ANYGPU_RING_OUTPUTS
+#undef ANYGPU_RING_INPUTS
+#undef ANYGPU_RING_CLOBBERS
 
 	if (probe != nullptr)
 	{
@@ -153,8 +191,10 @@ __global__ __launch_bounds__(256) void gemm_f16_nt_ring_kernel(
 // What the kernel assumes, checked on the host before every launch: whole slabs, 16-byte aligned operand rows, and
 // operands small enough for the 32-bit lane offsets (a wave's 64 rows).
 inline bool gemm_f16_ring_applies(const half_t* A, const half_t* B, int64_t M, int64_t N, int64_t K,
-                                  int64_t lda, int64_t ldb, int64_t stride_a, int64_t stride_b, int64_t batch)
+                                  int64_t lda, int64_t ldb, int64_t stride_a, int64_t stride_b, int64_t batch,
+                                  int b_layout = ANYGPU_B_COL_MAJOR)
 {
+	if (b_layout == ANYGPU_B_ROW_MAJOR && N % 8 != 0) return false;
 	const bool aligned = reinterpret_cast<uintptr_t>(A) % 16 == 0 && reinterpret_cast<uintptr_t>(B) % 16 == 0 &&
 	                     lda % 8 == 0 && ldb % 8 == 0 && stride_a % 8 == 0 && stride_b % 8 == 0;
 	// (the epilogue streams whole 16-byte vectors: C has to be aligned like the operands, which the caller checks)
@@ -165,12 +205,14 @@ inline bool gemm_f16_ring_applies(const half_t* A, const half_t* B, int64_t M, i
 inline hipError_t launch_gemm_f16_ring(const half_t* A, const half_t* B, half_t* C, int64_t M, int64_t N, int64_t K,
                                        int64_t lda, int64_t ldb, int64_t ldc,
                                        int64_t stride_a, int64_t stride_b, int64_t stride_c, int64_t batch, hipStream_t stream,
-                                       unsigned long long* probe = nullptr)
+                                       unsigned long long* probe = nullptr, int b_layout = ANYGPU_B_COL_MAJOR)
 {
-	const bool ragged = M % 256 != 0 || N % 256 != 0;
-	auto kernel = ragged ? gemm_f16_nt_ring_kernel<true> : gemm_f16_nt_ring_kernel<false>;
+	const bool kn = b_layout == ANYGPU_B_ROW_MAJOR;
+	const int ragged = (M % 256 != 0 || N % 256 != 0) + 2 * kn;       // which instantiation
+	auto kernel = ragged == 0 ? gemm_f16_nt_ring_kernel<false, false> : ragged == 1 ? gemm_f16_nt_ring_kernel<true, false>
+	            : ragged == 2 ? gemm_f16_nt_ring_kernel<false, true> : gemm_f16_nt_ring_kernel<true, true>;
 	// More than 64 KB of dynamic LDS has to be granted per function and per device, once.
-	static std::atomic<uint64_t> configured_devices[2];
+	static std::atomic<uint64_t> configured_devices[4];
 	(void)hipGetLastError();
 	int device = 0;
 	hipError_t e = hipGetDevice(&device);

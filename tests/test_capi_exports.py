@@ -83,9 +83,10 @@ def test_missing_library_fails_loudly(monkeypatch, tmp_path):
 
 
 def test_generated_gemm_loop_is_current(tmp_path):
-    # gemm_f16_ring_loop.inc is generated text that is committed: it has to be what the generator beside it writes
+    # gemm_f16_ring_loop*.inc are generated texts that are committed: they have to be what the generator beside them writes
     import sys
     csrc = REPO / "anygpu_amd" / "csrc"
-    out = tmp_path / "loop.inc"
-    subprocess.run([sys.executable, str(csrc / "gen_gemm_f16_ring_loop.py"), str(out)], check=True)
-    assert out.read_text() == (csrc / "gemm_f16_ring_loop.inc").read_text()
+    for name, form in (("gemm_f16_ring_loop.inc", []), ("gemm_f16_ring_loop_kn.inc", ["kn"])):
+        out = tmp_path / name
+        subprocess.run([sys.executable, str(csrc / "gen_gemm_f16_ring_loop.py"), str(out), *form], check=True)
+        assert out.read_text() == (csrc / name).read_text()

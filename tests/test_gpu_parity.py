@@ -699,6 +699,22 @@ def test_mm_f16_whole_256_tiles_integer_inputs_exact(ops, m, n, k, pad):
     assert np.array_equal(got, want)
 
 
+@pytest.mark.parametrize("m,n,k,pad", [(4096, 4096, 64, 0), (4096, 4096, 128, 8), (2048, 8192, 320, 0), (3840, 4352, 192, 264),
+                                       (4000, 3896, 128, 0), (3841, 4104, 64, 8), (4095, 4088, 192, 0), (3969, 3848, 64, 0)])
+def test_mm_f16_256_tiles_reference_layout_integer_inputs_exact(ops, m, n, k, pad):
+    # the same kernel with B stored [K, N] as the reference stores it: units of 64 k rows, transposing LDS reads, a row
+    # pitch that is not the row length, a last tile of 8 columns whose other chunks are read from inside the row
+    import torch
+    from anygpu_amd import capi
+    a = synth.integers(m + k + 2, (m, k), -2, 2).astype(np.float16)
+    b = synth.integers(n + k + 3, (k, n), -2, 2).astype(np.float16)
+    b_dev = torch.full((k, n + pad), 7.0, dtype=torch.float16, device="cuda")
+    b_dev[:, :n] = dev(b)
+    got = host(ops.tensor_mm(dev(a), b_dev[:, :n], b_layout=capi.B_ROW_MAJOR)).astype(np.int64)
+    want = a.astype(np.int64) @ b.astype(np.int64)
+    assert np.array_equal(got, want)
+
+
 def test_mm_f16_whole_256_tiles_batched(ops, oracle):
     # four products of 2048 x 2048 x 128 in one launch: 256 tiles of 256 x 256, the four-wave kernel over blockIdx.y
     from anygpu_amd import capi
