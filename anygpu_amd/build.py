@@ -62,6 +62,8 @@ def build_kernels(verbose: bool = False) -> Path:
     # the main loop of the four-wave fp16 GEMM tile is generated text (an inline-assembly block with fixed registers)
     _run([sys.executable, str(CSRC_DIR / "gen_gemm_f16_ring_loop.py"), str(CSRC_DIR / "gemm_f16_ring_loop.inc")], quiet=not verbose)
     _run([sys.executable, str(CSRC_DIR / "gen_gemm_f16_ring_loop.py"), str(CSRC_DIR / "gemm_f16_ring_loop_kn.inc"), "kn"], quiet=not verbose)
+    _run([sys.executable, str(CSRC_DIR / "gen_gemm_f16_ring_loop.py"), str(CSRC_DIR / "gemm_f16_ring_loop_8x4.inc"), "8x4"], quiet=not verbose)
+    _run([sys.executable, str(CSRC_DIR / "gen_gemm_f16_ring_loop.py"), str(CSRC_DIR / "gemm_f16_ring_loop_4x4.inc"), "4x4"], quiet=not verbose)
 
     def compile_one(src: str) -> Path:
         obj = OBJ_DIR / (Path(src).stem + ".o")

@@ -6,9 +6,12 @@
 //
 // Edge kernel: 64 x 64 tiles, guarded scalar loads and stores, either B layout, any
 // shape, stride and alignment.
+#include <algorithm>
+
 #include "device_utils.hpp"
 #include "gemm_f16_tile.hpp"
 #include "gemm_f16_ring.hpp"
+#include "gemm_f16_ring3.hpp"
 #include "launch.hpp"
 #include "gemm_band.hpp"
 #include "anygpu_hip.h"
@@ -198,6 +201,59 @@ static double slab_us(int64_t t, int64_t nblocks, int64_t cus, bool whole_tiles 
 	return TilePrices::kSmallDense * share;
 }
 
+// The four-wave kernels (one block per CU; k-contiguous operands, whole 64-deep slabs): 256 x 256, 256 x 128 and
+// 128 x 128 tiles, the two smaller ones also cut along K into planes.  Microseconds per slab and round of blocks with the
+// chip full and half full (fewer blocks share the L2s and the power budget), and per launch, from sweeps over K with
+// uniform random operands (operands of small integers run up to a fifth faster: the clock follows the power drawn).
+// 256 x 256: 4096 x 4096 x K 53.7 / 189.3 us at K = 2048 / 8192, 2048 x 4096 x K (half full) 43.8 / 139.2;
+// 256 x 128: 2048 x 4096 x K 30.0 / 103.5, 2048 x 2048 x K 24.7 / 79.8;  128 x 128: 2048 x 2048 x K 17.8 / 62.6,
+// 1024 x 2048 x K 14.5 / 49.6 (the vendor library on 2048 x 2048 x K: 24 / 73).
+struct FourWavePrices
+{
+	static constexpr double kSlabFull[3] = {1.41, 0.77, 0.465};
+	static constexpr double kSlabHalf[3] = {1.0, 0.575, 0.36};
+	static constexpr double kLaunch[3] = {8.5, 5.5, 3.0};
+};
+
+struct FourWavePlan
+{
+	int kind = -1;         // 0: 256 x 256, 1: 256 x 128, 2: 128 x 128
+	int64_t splits = 1;
+	double us = 1e30;
+};
+
+static FourWavePlan plan_four_wave(int64_t M, int64_t N, int64_t K, int64_t batch, int64_t cus, int64_t plane_room)
+{
+	FourWavePlan best;
+	const int64_t slabs = K / 64;
+	for (int kind = 0; kind < 3; ++kind)
+	{
+		const int64_t bm = kind == 2 ? 128 : 256, bn = kind == 0 ? 256 : 128;
+		const int64_t blocks = ((M + bm - 1) / bm) * ((N + bn - 1) / bn) * batch;
+		if (blocks / batch > 0x7FFFFFFFLL) continue;
+		const int64_t max_splits = (kind == 0 || batch != 1) ? 1 : std::min<int64_t>({16, K / 512, plane_room});
+		for (int64_t sp = 1; sp <= std::max<int64_t>(1, max_splits); ++sp)
+		{
+			const int64_t nb = blocks * sp;
+			if (sp > 1 && nb > 2 * cus) break;
+			const int64_t rounds = (nb + cus - 1) / cus;
+			const double fill = nb >= cus ? 1.0 : (double)nb / (double)cus;
+			const double t = fill <= 0.5 ? 0.0 : (fill - 0.5) / 0.5;
+			const double per_slab = FourWavePrices::kSlabHalf[kind] + t * (FourWavePrices::kSlabFull[kind] - FourWavePrices::kSlabHalf[kind]);
+			const int64_t depth = (slabs + sp - 1) / sp;
+			double us = (double)rounds * (double)depth * per_slab + FourWavePrices::kLaunch[kind];
+			if (sp > 1) us += TilePrices::kMergeLaunchUs + 8.0 * (double)sp * (double)M * (double)N / TilePrices::kPlaneBytesPerUs;
+			if (us < best.us)
+			{
+				best.kind = kind;
+				best.splits = sp;
+				best.us = us;
+			}
+		}
+	}
+	return best;
+}
+
 // C[m, n] = half(sum over splits of planes[split][m][n]), one thread per eight columns (N a multiple of 8), the
 // planes added in order
 __global__ __launch_bounds__(256) void gemm_f16_split_merge_kernel(
@@ -352,6 +408,9 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
 		// 1024 x 9216 . 9216 x 2304: 73 -> 60 us, vendor 58 - 64).
 		int64_t splits = 1;
 		const int64_t tile_unsplit = tile;
+		const double kLaunchUs = 6.0;             // prologue, epilogue and the gap between launches, for comparing plans
+		double plan_us = (double)((K + 63) / 64) * (rect ? cost_rect : cost_square) + kLaunchUs;
+		int64_t plane_room = 0;
 		if (batch == 1 && planes_ok && K >= 1024)
 		{
 			const double slabs = (double)(K / 64);
@@ -359,6 +418,7 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
 			// (as many planes as the stream's workspace holds: the caller's, or the library's own for eager launches; a
 			// stream under capture without a caller's workspace has none and runs uncut)
 			const int64_t room = (int64_t)(band::workspace_capacity(stream) / ((size_t)M * N * sizeof(float)));
+			plane_room = room;
 			for (const int64_t t : {(int64_t)256, (int64_t)128, (int64_t)64})
 			{
 				if (blocks(t) >= cus) continue;
@@ -373,6 +433,40 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
 						tile = t;
 					}
 				}
+			}
+			if (splits > 1) plan_us = best + kLaunchUs;
+		}
+		// The four-wave kernels where they apply and come out cheaper than the plan so far: their smaller tiles cost
+		// about half per slab of what the eight-wave tiles of the same size do (2048^3: 26 -> 16 us, vendor 22;
+		// 2048 x 4096 x 4096: 60 -> 44 us, vendor 55 - 60; 512 x 6144 x 4096: 43 -> 24 us, vendor 29 - 32).
+		if (whole_tiles && b_layout == ANYGPU_B_COL_MAJOR)
+		{
+			const FourWavePlan four = plan_four_wave(M, N, K, batch, cus, planes_ok ? plane_room : 0);
+			if (four.kind >= 0 && four.us < plan_us)
+			{
+				if (four.kind == 0)
+					return launch_gemm_f16_ring(a, b, c, M, N, K, lda, ldb, ldc, stride_a, stride_b, stride_c, batch, stream);
+				float* planes = nullptr;
+				int64_t ranges = four.splits, k_split = 0;
+				if (ranges > 1)
+				{
+					k_split = ((K / 64 + ranges - 1) / ranges) * 64;
+					ranges = (K + k_split - 1) / k_split;
+				}
+				if (ranges > 1)
+				{
+					const hipError_t ws_err = band::workspace_acquire(stream, &planes);
+					if (ws_err != hipSuccess) return ws_err;
+				}
+				const int64_t sa = ranges > 1 ? k_split : stride_a, sb = ranges > 1 ? k_split : stride_b;
+				const int64_t count = ranges > 1 ? ranges : batch;
+				const hipError_t err = four.kind == 1
+					? launch_gemm_f16_ring3<8, 4>(a, b, c, M, N, K, lda, ldb, ldc, sa, sb, stride_c, count, stream, planes, k_split)
+					: launch_gemm_f16_ring3<4, 4>(a, b, c, M, N, K, lda, ldb, ldc, sa, sb, stride_c, count, stream, planes, k_split);
+				if (err != hipSuccess || ranges <= 1) return err;
+				const int64_t items = M * (N / 8);
+				gemm_f16_split_merge_kernel<<<dim3((unsigned)((items + 255) / 256)), dim3(256), 0, stream>>>(planes, c, M, N, ldc, (int)ranges);
+				return hipGetLastError();
 			}
 		}
 		if (splits > 1)

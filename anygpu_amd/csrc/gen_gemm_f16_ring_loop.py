@@ -41,7 +41,16 @@ bbaselo / bbasehi (SGPR: global address of the wave's first row), ldsw (SGPR: LD
 unit 0), slabs (SGPR: K / 64); kn form also bsx (VGPR: the lane's swizzle, (k row bits) << 5) and bstep (SGPR: bytes
 from one B slab to the next).
 
-Usage: gen_gemm_f16_ring_loop.py OUTPUT [kn]
+Smaller tiles ("8x4": 256 x 128, a 128 x 64 patch per wave; "4x4": 128 x 128, 64 x 64 patches) leave LDS room for three
+whole stages of an A unit and a B unit, which is simpler: stage s mod 3 holds slab s, the mid-slab barrier of slab t frees
+the stage of slab t (its last fragments were read during the first step), and the loads of slab t + 3 go there, half of
+them during the second step of slab t and half during the first step of slab t + 1.  Registers as above except: s60 .. s62
+LDS addresses of the stages of slabs t, t + 1, t + 2; s72 / s73 where the wave's A / B loads of the current step go;
+v112 / v113 and v114 / v115 the fragment addresses of the first and of the second step, v116 / v117 the lane's fragment
+addresses inside a stage with bit 6 flipped.  Operands: vtab, aaddr, baddr (inside a stage), abaselo .. bbasehi, slabs as
+above, lds0 (SGPR: LDS address of stage 0), ldsa / ldsb (SGPR: offset of the wave's share of the A / B unit in a stage).
+
+Usage: gen_gemm_f16_ring_loop.py OUTPUT [kn | 8x4 | 4x4]
 """
 import sys
 
@@ -214,11 +223,147 @@ def generate(kn):
     return lines
 
 
+def generate_three_stages(tm, tn):
+    """the block for a patch of tm x tn MFMA tiles per wave (tile 32 tm x 32 tn), three LDS stages"""
+    lines = []
+    bm, bn = 32 * tm, 32 * tn
+    stage = (bm + bn) * 128
+    la, lb = bm // 32, bn // 32                 # loads per wave and slab
+    half = (la + lb) // 2
+    load_list = [("a", q) for q in range(la)] + [("b", q) for q in range(lb)]
+    S = ["s60", "s61", "s62"]
+    S_ROT, S_LDA, S_LDB = "s63", "s72", "s73"
+    V_RA0, V_RB0, V_RA1, V_RB1, V_A64, V_B64 = "v112", "v113", "v114", "v115", "v116", "v117"
+    mfmas = tm * tn
+
+    def emit(s, comment=None):
+        if isinstance(s, tuple):
+            for x in s:
+                emit(x)
+            return
+        lines.append((s, comment))
+
+    def tile_acc(i, j):
+        r = 4 * (tn * i + j)
+        return f"a[{r}:{r + 3}]"
+
+    def load_set(stage_reg, add):
+        """where the loads of slab min(t + add, last) go and come from: entries of one or two instructions"""
+        return [f"s_add_u32 {S_LDA}, {stage_reg}, %[ldsa]", f"s_add_u32 {S_LDB}, {stage_reg}, %[ldsb]",
+                f"s_add_u32 {S_TMP}, {S_T}, {add}", f"s_min_u32 {S_TMP}, {S_TMP}, {S_LAST}", f"s_lshl_b32 {S_TMP}, {S_TMP}, 7",
+                ("s_add_u32 s68, %[abaselo], " + S_TMP, "s_addc_u32 s69, %[abasehi], 0"),
+                ("s_add_u32 s70, %[bbaselo], " + S_TMP, "s_addc_u32 s71, %[bbasehi], 0")]
+
+    def loads(which):
+        out = []
+        for operand, q in load_list[:half] if which == 0 else load_list[half:]:
+            v = 96 + q + (8 if operand == "b" else 0)
+            out.append((f"s_add_u32 m0, {S_LDA if operand == 'a' else S_LDB}, {q * 1024}",
+                        f"global_load_lds_dwordx4 v{v}, {A_CUR if operand == 'a' else B_CUR}"))
+        return out
+
+    def reads(buf, va, vb):
+        out = [f"ds_read_b128 {bfrag(buf, q)}, {vb} offset:{q * 2048}" for q in range(tn)]
+        out += [f"ds_read_b128 {afrag(buf, q)}, {va} offset:{q * 2048}" for q in range(tm)]
+        return out
+
+    # ---- prologue: slabs 0 and 1 and the first half of the loads of slab 2, fragments of the first step
+    emit(f"s_mov_b32 {S_T}, 0", "prologue")
+    emit(f"s_sub_u32 {S_LAST}, %[slabs], 1")
+    for x in range(3):
+        emit(f"s_add_u32 {S[x]}, %[lds0], {x * stage}")
+    for q in range(la):
+        emit(f"ds_read_b32 v{96 + q}, %[vtab] offset:{256 * q}")
+    for q in range(lb):
+        emit(f"ds_read_b32 v{104 + q}, %[vtab] offset:{256 * (8 + q)}")
+    emit("s_waitcnt lgkmcnt(0)")
+    emit(f"v_xor_b32 {V_A64}, 64, %[aaddr]")
+    emit(f"v_xor_b32 {V_B64}, 64, %[baddr]")
+    for slab in range(3):
+        for ins in load_set(S[slab], slab):
+            emit(ins)
+        for m0w, ld in (loads(0) + loads(1)) if slab < 2 else loads(0):
+            emit(m0w)
+            emit("s_nop 0")
+            emit(ld)
+    for r in range(4 * mfmas):
+        emit(f"v_accvgpr_write_b32 a{r}, 0")
+    emit(f"s_waitcnt vmcnt({la + lb + half})", "slab 0 has landed")
+    emit("s_barrier")
+    emit(f"v_add_u32 {V_RA1}, {S[0]}, %[aaddr]")
+    emit(f"v_add_u32 {V_RB1}, {S[0]}, %[baddr]")
+    for ins in reads(0, V_RA1, V_RB1):
+        emit(ins)
+    emit(f"v_add_u32 {V_RA0}, {S[0]}, {V_A64}")
+    emit(f"v_add_u32 {V_RB0}, {S[0]}, {V_B64}")
+    emit("s_waitcnt lgkmcnt(0)")
+
+    # ---- main loop: one slab per trip
+    emit("1:", "main loop: one 64-deep slab per trip")
+    for step in range(2):
+        gaps = [[] for _ in range(mfmas)]
+
+        def place(entry, earliest):
+            """behind the first MFMA from `earliest` on that has fewer than two instructions behind it (three if none has)"""
+            n = len(entry) if isinstance(entry, tuple) else 1
+            for cap in (2, 3):
+                for g in range(earliest, mfmas):
+                    if sum(len(x) if isinstance(x, tuple) else 1 for x in gaps[g]) + n <= cap:
+                        gaps[g].append(entry)
+                        return g
+            raise RuntimeError("the step has no room left")
+
+        buf = step
+        # fragments of the next step: step 0 reads the second half of slab t, step 1 the first half of slab t + 1
+        for q, ins in enumerate(reads(buf ^ 1, V_RA0 if step == 0 else V_RA1, V_RB0 if step == 0 else V_RB1)):
+            gaps[2 * q].append(ins)
+        # step 0: the second half of the loads of slab t + 2; step 1: the first half of the loads of slab t + 3
+        every = max(2, (mfmas - 10) // half)
+        last_load = 0
+        for q, (m0w, ld) in enumerate(loads(1) if step == 0 else loads(0)):
+            gaps[every * q].append(m0w)
+            gaps[every * q + 1].append(ld)
+            last_load = every * q + 1
+        if step == 0:
+            # fragment addresses of step 1; once this step's loads are out, where the loads of slab t + 3 go (the stage of
+            # slab t) and come from
+            g = place(f"v_add_u32 {V_RA1}, {S[1]}, %[aaddr]", 1)
+            g = place(f"v_add_u32 {V_RB1}, {S[1]}, %[baddr]", g)
+            g = last_load + 1
+            for ins in load_set(S[0], 3):
+                g = place(ins, g)
+        else:
+            # the stages move on by one slab, t advances; fragment addresses of the next trip's first step
+            g = 1
+            for ins in [f"s_mov_b32 {S_ROT}, {S[0]}", f"s_mov_b32 {S[0]}, {S[1]}", f"s_mov_b32 {S[1]}, {S[2]}", f"s_mov_b32 {S[2]}, {S_ROT}",
+                        f"s_add_u32 {S_T}, {S_T}, 1", f"v_add_u32 {V_RA0}, {S[0]}, {V_A64}", f"v_add_u32 {V_RB0}, {S[0]}, {V_B64}"]:
+                g = place(ins, g + 1)
+        if step == 1:
+            emit(f"s_waitcnt vmcnt({la + lb})", "mid-slab: slab t + 1 has landed (the loads of slab t + 2 may be in flight)")
+            emit("s_barrier")
+        for m in range(mfmas):
+            i, j = m // tn, m % tn
+            if i % 2 == 1:
+                j = tn - 1 - j
+            emit(f"v_mfma_f32_16x16x32_f16 {tile_acc(i, j)}, {bfrag(buf, j)}, {afrag(buf, i)}, {tile_acc(i, j)}",
+                 f"step {step}" if m == 0 else None)
+            for ins in gaps[m]:
+                emit(ins)
+        emit("s_waitcnt lgkmcnt(0)")
+    emit(f"s_cmp_lt_u32 {S_T}, %[slabs]")
+    emit("s_cbranch_scc1 1b")
+    emit("s_waitcnt vmcnt(0)", "nothing may still be writing LDS; the last MFMAs leave the pipeline before the accumulators are read")
+    emit("s_barrier")
+    emit("s_nop 15")
+    emit("s_nop 15")
+    return lines
+
+
 if __name__ == "__main__":
-    kn = len(sys.argv) > 2 and sys.argv[2] == "kn"
+    form = sys.argv[2] if len(sys.argv) > 2 else ""
     with open(sys.argv[1], "w") as f:
         f.write("// Written by gen_gemm_f16_ring_loop.py (the register plan and the schedule are explained there): do not edit.\n")
-        for s, c in generate(kn):
+        for s, c in (generate_three_stages(*(int(x) for x in form.split("x"))) if "x" in form else generate(form == "kn")):
             if c:
                 f.write(f"// {c}\n")
             f.write(f'"{s}\\n\\t"\n')

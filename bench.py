@@ -20,6 +20,10 @@ the parity tests).  Timing of every kernel:
     single launch -> `median_us`, `min_us` (these leave out the gap between two launches).
 The memory-bound kernels rotate over several buffer sets so that the working set exceeds the
 256 MB Infinity Cache.
+
+`--gemm-shapes` prints, instead of the JSON line, a table of the fp16 GEMM over the projection shapes of the models
+the path serves (8 row counts x 14 weight shapes, weights k-contiguous) next to torch.matmul, i.e. the vendor library,
+on the same operands.
 """
 from __future__ import annotations
 
@@ -73,6 +77,8 @@ def parse_args():
                     help="target wall time of the CPU-oracle sample of the headline (0 disables every CPU baseline); "
                          "the other configurations get a quarter of it each")
     ap.add_argument("--only", default="", help="comma list of: gemm,gemm32,conv,softmax,attn,attn32,decode,norm (default: all)")
+    ap.add_argument("--gemm-shapes", action="store_true",
+                    help="print the table of fp16 GEMM layer shapes against torch.matmul and exit")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain device copy of 256 MiB (read 256 MiB + write 256 MiB) a few times, "
                          "as the known-size reference for scaling FETCH_SIZE / WRITE_SIZE counter readings")
@@ -417,6 +423,46 @@ def bench_gated_rmsnorm(torch, ops, synth, steps, warmup):
     }
 
 
+LAYER_WEIGHTS = [(9216, 2304), (18432, 2304), (2304, 9216), (2048, 2304), (1024, 2304), (4096, 2304), (2304, 2048),
+                 (2048, 2048), (8192, 2048), (2048, 8192), (4096, 4096), (14336, 4096), (4096, 14336), (6144, 4096)]
+LAYER_ROWS = (16, 64, 128, 256, 512, 1024, 2048, 4096)
+
+
+def sweep_gemm_shapes(torch, ops, capi):
+    """[rows, K] x [N, K]^T for the (N, K) of Gemma2-2B / Zamba2 / Llama-8B-sized projections: microseconds of this
+    library and of torch.matmul (hipBLASLt) on the same uniform random operands, each the better of two runs of 40
+    back-to-back launches taken alternately."""
+    def timed(fn, iters=40, warm=8):
+        for _ in range(warm):
+            fn()
+        torch.cuda.synchronize()
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(iters):
+            fn()
+        stop.record()
+        torch.cuda.synchronize()
+        return start.elapsed_time(stop) / iters * 1e3
+
+    print("| rows | K | N | this library us | torch.matmul us | ratio |")
+    print("|---:|---:|---:|---:|---:|---:|")
+    ratios = []
+    for n, k in LAYER_WEIGHTS:
+        weight = (torch.rand(n, k, device="cuda") * 2 - 1).half()
+        for rows in LAYER_ROWS:
+            a = (torch.rand(rows, k, device="cuda") * 2 - 1).half()
+            c = torch.empty(rows, n, device="cuda", dtype=torch.half)
+            mine = lambda: ops.tensor_mm(a, weight, out=c, b_layout=capi.B_COL_MAJOR)
+            theirs = lambda: torch.matmul(a, weight.t(), out=c)
+            t_mine, t_theirs = timed(mine), timed(theirs)
+            t_mine, t_theirs = min(t_mine, timed(mine)), min(t_theirs, timed(theirs))
+            ratios.append(t_mine / t_theirs)
+            print(f"| {rows} | {k} | {n} | {t_mine:.1f} | {t_theirs:.1f} | {t_mine / t_theirs:.2f} |", flush=True)
+    ratios.sort()
+    print(f"\n{len(ratios)} shapes: median ratio {statistics.median(ratios):.2f}, worst {ratios[-1]:.2f}, "
+          f"{sum(r > 1.05 for r in ratios)} above 1.05, {sum(r < 0.95 for r in ratios)} below 0.95")
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -432,6 +478,9 @@ def main():
         return 1
     capi.load()
     torch.cuda.set_device(0)
+    if args.gemm_shapes:
+        sweep_gemm_shapes(torch, ops, capi)
+        return 0
     only = set(filter(None, args.only.split(",")))
     want = lambda name: not only or name in only
     props = torch.cuda.get_device_properties(0)

@@ -715,6 +715,27 @@ def test_mm_f16_256_tiles_reference_layout_integer_inputs_exact(ops, m, n, k, pa
     assert np.array_equal(got, want)
 
 
+@pytest.mark.parametrize("m,n,k,pad,span", [(2048, 2048, 192, 0, 2), (1000, 2000, 128, 8, 2), (2048, 4096, 64, 0, 2), (1100, 4000, 320, 0, 2),
+                                            (520, 6152, 256, 0, 2), (128, 128, 64, 0, 2), (512, 2304, 9216, 0, 1), (300, 1000, 4096, 72, 1),
+                                            (2048, 1024, 2048, 0, 1)])
+def test_mm_f16_smaller_four_wave_tiles_integer_inputs_exact(ops, m, n, k, pad, span):
+    # products that do not fill the chip with 256 x 256 tiles: the four-wave kernels with 256 x 128 and 128 x 128 tiles,
+    # whole and ragged, one slab and several, and cut along K into fp32 planes (the deep ones).  Integer operands whose
+    # sums stay below 2^11 in magnitude are exact in fp32 and in the fp16 result in any order of summation.
+    import torch
+    from anygpu_amd import capi
+    a = synth.integers(m + k + 4, (m, k), -span, span).astype(np.float16)
+    bt = synth.integers(n + k + 5, (n, k), -span, span).astype(np.float16)
+    a_dev = torch.full((m, k + pad), 7.0, dtype=torch.float16, device="cuda")
+    b_dev = torch.full((n, k + pad), 7.0, dtype=torch.float16, device="cuda")
+    a_dev[:, :k] = dev(a)
+    b_dev[:, :k] = dev(bt)
+    got = host(ops.tensor_mm(a_dev[:, :k], b_dev[:, :k], b_layout=capi.B_COL_MAJOR)).astype(np.int64)
+    want = a.astype(np.int64) @ bt.astype(np.int64).T
+    assert np.abs(want).max() < 2048
+    assert np.array_equal(got, want)
+
+
 def test_mm_f16_whole_256_tiles_batched(ops, oracle):
     # four products of 2048 x 2048 x 128 in one launch: 256 tiles of 256 x 256, the four-wave kernel over blockIdx.y
     from anygpu_amd import capi
