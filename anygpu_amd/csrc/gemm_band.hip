@@ -397,17 +397,38 @@ bool stream_is_capturing(hipStream_t stream)
 
 }  // namespace
 
+namespace {
+thread_local size_t reserved_front = 0;      // bytes at the front of every workspace this thread's launches leave alone
+}
+
+band::WorkspaceReserve::WorkspaceReserve(size_t bytes) : previous_(reserved_front)
+{
+	reserved_front += (bytes + 255) / 256 * 256;
+}
+
+band::WorkspaceReserve::~WorkspaceReserve()
+{
+	reserved_front = previous_;
+}
+
 size_t band::workspace_capacity(hipStream_t stream)
 {
 	int device = 0;
 	if (hipGetDevice(&device) != hipSuccess) return 0;
+	size_t bytes = 0;
+	bool from_caller = false;
 	{
 		std::lock_guard<std::mutex> guard(workspace_lock);
 		const auto found = workspaces.find(std::make_pair(device, stream));
-		if (found != workspaces.end() && found->second.from_caller) return found->second.bytes;
+		if (found != workspaces.end() && found->second.from_caller)
+		{
+			bytes = found->second.bytes;
+			from_caller = true;
+		}
 	}
 	// the library's own buffer: eager launches only
-	return stream_is_capturing(stream) ? 0 : kBandPartialBytes;
+	if (!from_caller) bytes = stream_is_capturing(stream) ? 0 : kBandPartialBytes;
+	return bytes > reserved_front ? bytes - reserved_front : 0;
 }
 
 hipError_t band::workspace_acquire(hipStream_t stream, float** base)
@@ -421,7 +442,7 @@ hipError_t band::workspace_acquire(hipStream_t stream, float** base)
 	const auto found = workspaces.find(key);
 	if (found != workspaces.end())
 	{
-		*base = found->second.base;
+		*base = reinterpret_cast<float*>(reinterpret_cast<char*>(found->second.base) + reserved_front);
 		return hipSuccess;
 	}
 	// First cut on this stream.  Another thread may be capturing some other stream in the global mode, in which an
@@ -437,7 +458,7 @@ hipError_t band::workspace_acquire(hipStream_t stream, float** base)
 		return err;
 	}
 	workspaces.emplace(key, WorkspaceEntry{static_cast<float*>(mem), kBandPartialBytes, false});
-	*base = static_cast<float*>(mem);
+	*base = reinterpret_cast<float*>(static_cast<char*>(mem) + reserved_front);
 	return hipSuccess;
 }
 

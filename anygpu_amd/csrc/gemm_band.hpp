@@ -77,6 +77,20 @@ template <> struct BandMma<half_t, 32>
 // that fails.
 size_t workspace_capacity(hipStream_t stream);
 hipError_t workspace_acquire(hipStream_t stream, float** base);
+// While one of these lives, the calling thread's view of every workspace starts `bytes` (rounded up to 256) further on:
+// a launcher that has parked operand copies at the front of the stream's workspace calls the ordinary launchers
+// underneath it, whose partial sums then go behind the copies.
+class WorkspaceReserve
+{
+public:
+	explicit WorkspaceReserve(size_t bytes);
+	~WorkspaceReserve();
+	WorkspaceReserve(const WorkspaceReserve&) = delete;
+	WorkspaceReserve& operator=(const WorkspaceReserve&) = delete;
+
+private:
+	size_t previous_;
+};
 // the C ABI's anygpu_set_workspace / anygpu_release_workspaces
 int workspace_set(hipStream_t stream, void* base, size_t bytes);
 hipError_t workspace_release_all();

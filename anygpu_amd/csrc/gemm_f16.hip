@@ -339,6 +339,55 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
 	// 166 us against 198 us; small weights 9 us against 13 us), and whatever the tile kernels cannot take goes to the
 	// band kernels (5 .. 64 rows) or the skinny ones.
 	const bool tiles_first = tiles_ok && (b_layout == ANYGPU_B_ROW_MAJOR || M >= 3);
+	// Operands the tile kernels cannot fetch (an odd start or row pitch, K no multiple of 8, [K, N] weights with such an
+	// N) are copied into the stream's workspace as aligned k-contiguous rows, zeros up to the next multiple of 64 behind
+	// K, and the product runs on the copies: 4096 x 4100 . [4096, 4100] weights 270 -> 117 us (vendor 105 - 110).  From
+	// 16 rows on (below that the weights are streamed once anyway and a copy would triple that), for products worth
+	// two more launches, where the workspace holds the copies; otherwise the element-wise kernel at the bottom.
+	if (!tiles_ok && batch == 1 && M >= 16 && (double)M * (double)N * (double)K >= (double)(1 << 27))
+	{
+		const bool k_odd = K % 8 != 0;
+		const bool copy_a = k_odd || reinterpret_cast<uintptr_t>(A) % 16 != 0 || lda % 8 != 0;
+		const bool copy_b = k_odd || reinterpret_cast<uintptr_t>(B) % 16 != 0 || ldb % 8 != 0 || (b_layout == ANYGPU_B_ROW_MAJOR && N % 8 != 0);
+		const int64_t k_pad = (K + 63) / 64 * 64;
+		const size_t bytes_b = copy_b ? ((size_t)N * k_pad * 2 + 255) / 256 * 256 : 0;
+		const size_t room = band::workspace_capacity(stream);
+		// (a copy of A that does not fit beside the one of B is made and used in bands of rows, one after the other)
+		int64_t band_rows = M;
+		if (copy_a && bytes_b < room && (size_t)M * k_pad * 2 > room - bytes_b)
+			band_rows = (int64_t)((room - bytes_b) / ((size_t)k_pad * 2)) / 256 * 256;
+		const size_t bytes_a = copy_a ? ((size_t)band_rows * k_pad * 2 + 255) / 256 * 256 : 0;
+		if ((copy_a || copy_b) && (band_rows == M || band_rows >= 256) && bytes_a + bytes_b <= room)
+		{
+			float* front = nullptr;
+			hipError_t err = band::workspace_acquire(stream, &front);
+			if (err != hipSuccess) return err;
+			half_t* b_copy = reinterpret_cast<half_t*>(front);
+			half_t* a_copy = reinterpret_cast<half_t*>(reinterpret_cast<char*>(front) + bytes_b);
+			if (copy_b)
+			{
+				err = b_layout == ANYGPU_B_COL_MAJOR ? launch_repack_rows(b, ldb, N, K, b_copy, k_pad, 2, stream)
+				                                     : launch_repack_transposed(b, ldb, K, N, b_copy, k_pad, 2, stream);
+				if (err != hipSuccess) return err;
+			}
+			// (both copied: the zeros behind K make whole slabs of it; one copied: K stays, the copy just has its own pitch)
+			const int64_t k_used = copy_a && copy_b ? k_pad : K;
+			const band::WorkspaceReserve keep(bytes_a + bytes_b);
+			for (int64_t m0 = 0; m0 < M; m0 += band_rows)
+			{
+				const int64_t rows = std::min(band_rows, M - m0);
+				if (copy_a)
+				{
+					err = launch_repack_rows(a + m0 * lda, lda, rows, K, a_copy, k_pad, 2, stream);
+					if (err != hipSuccess) return err;
+				}
+				err = launch_gemm_f16(copy_a ? a_copy : a + m0 * lda, copy_b ? b_copy : b, c + m0 * ldc, rows, N, k_used,
+				                      copy_a ? k_pad : lda, copy_b ? k_pad : ldb, ldc, 0, 0, 0, 1, copy_b ? ANYGPU_B_COL_MAJOR : b_layout, stream);
+				if (err != hipSuccess) return err;
+			}
+			return hipSuccess;
+		}
+	}
 	if (batch == 1 && !tiles_first && gemm_band_applies<half_t>(a, b, nullptr, c, M, N, K, lda, ldb, ldc, b_layout))
 		return launch_gemm_band<half_t>(a, b, nullptr, nullptr, c, M, N, K, lda, ldb, ldc, 0, 0.0f, stream);
 	if (batch == 1 && !tiles_first && gemm_skinny_applies<half_t>(a, b, nullptr, M, N, K, lda, ldb, b_layout))
@@ -358,8 +407,7 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
 		const auto blocks = [&](int64_t tile) { return ((M + tile - 1) / tile) * ((N + tile - 1) / tile) * batch; };
 		const int64_t cus = device_cu_count();
 		// 256 x 256 tiles of whole 64-deep slabs take the four-wave kernel, which is cheaper per slab
-		const bool whole_tiles = reinterpret_cast<uintptr_t>(C) % 16 == 0 && ldc % 8 == 0 && stride_c % 8 == 0 &&
-		                         gemm_f16_ring_applies(a, b, M, N, K, lda, ldb, stride_a, stride_b, batch, b_layout);
+		const bool whole_tiles = gemm_f16_ring_applies(a, b, M, N, K, lda, ldb, stride_a, stride_b, batch, b_layout);
 		const auto slab_us = [cus, whole_tiles](int64_t t, int64_t nblocks) { return anygpu::slab_us(t, nblocks, cus, whole_tiles); };
 		const double cost256 = slab_us(256, blocks(256)), cost128 = slab_us(128, blocks(128)), cost64 = slab_us(64, blocks(64));
 		int64_t tile = (cost256 <= cost128 && cost256 <= cost64) ? 256 : cost128 <= cost64 ? 128 : 64;

@@ -27,8 +27,8 @@ struct GemmRingCfg
 };
 
 // blockIdx.y walks a batch of independent products that share the shape.  K a multiple of 64.
-// RAGGED: M and N need not be multiples of 256.  Operand rows past the end are read from the last valid row instead (they
-// only feed results that are not stored) and the stores are guarded.
+// RAGGED: M and N need not be multiples of 256 and C may start and step at any element.  Operand rows past the end are
+// read from the last valid row instead (they only feed results that are not stored) and the stores are guarded.
 // probe (may be NULL; first product of a batch only): lane 0 of every block leaves the shader clock count (s_memtime) and
 // the constant 100 MHz count (s_memrealtime) at entry and exit of its main loop in probe[4 block .. + 3], from which a
 // caller gets the clock the part sustained under this kernel and the share of those cycles the matrix cores were busy.
@@ -197,7 +197,6 @@ inline bool gemm_f16_ring_applies(const half_t* A, const half_t* B, int64_t M, i
 	if (b_layout == ANYGPU_B_ROW_MAJOR && N % 8 != 0) return false;
 	const bool aligned = reinterpret_cast<uintptr_t>(A) % 16 == 0 && reinterpret_cast<uintptr_t>(B) % 16 == 0 &&
 	                     lda % 8 == 0 && ldb % 8 == 0 && stride_a % 8 == 0 && stride_b % 8 == 0;
-	// (the epilogue streams whole 16-byte vectors: C has to be aligned like the operands, which the caller checks)
 	return aligned && M > 0 && N > 0 && K >= 64 && K % 64 == 0 && lda < (1 << 24) && ldb < (1 << 24) &&
 	       ((M + 255) / 256) * ((N + 255) / 256) <= 0x7FFFFFFFLL && batch >= 1 && batch <= 65535;
 }
@@ -208,7 +207,9 @@ inline hipError_t launch_gemm_f16_ring(const half_t* A, const half_t* B, half_t*
                                        unsigned long long* probe = nullptr, int b_layout = ANYGPU_B_COL_MAJOR)
 {
 	const bool kn = b_layout == ANYGPU_B_ROW_MAJOR;
-	const int ragged = (M % 256 != 0 || N % 256 != 0) + 2 * kn;       // which instantiation
+	// (whole tiles of an aligned C are streamed out in 16-byte vectors; anything else takes the guarded stores)
+	const bool c_aligned = reinterpret_cast<uintptr_t>(C) % 16 == 0 && ldc % 8 == 0 && stride_c % 8 == 0;
+	const int ragged = (M % 256 != 0 || N % 256 != 0 || !c_aligned) + 2 * kn;       // which instantiation
 	auto kernel = ragged == 0 ? gemm_f16_nt_ring_kernel<false, false> : ragged == 1 ? gemm_f16_nt_ring_kernel<true, false>
 	            : ragged == 2 ? gemm_f16_nt_ring_kernel<false, true> : gemm_f16_nt_ring_kernel<true, true>;
 	// More than 64 KB of dynamic LDS has to be granted per function and per device, once.

@@ -26,7 +26,8 @@ struct GemmRing3Cfg
 };
 
 // blockIdx.y walks a batch of independent products that share the shape.  K a multiple of 64.  RAGGED: M and N need not
-// be multiples of the tile; operand rows past the end are read from the last valid row and the stores are guarded.
+// be multiples of the tile and C may start and step at any element; operand rows past the end are read from the last
+// valid row and the stores are guarded.
 // SPLIT: blockIdx.y walks ranges of K (k_split deep, a multiple of 64; the strides step along K) of one product instead
 // of a batch, and the raw fp32 sums of range y go to planes[y][M][N]; C is not touched.
 template <int TM, int TN, bool RAGGED, bool SPLIT>
@@ -175,7 +176,8 @@ inline hipError_t launch_gemm_f16_ring3(const half_t* A, const half_t* B, half_t
                                         float* planes = nullptr, int64_t k_split = 0)
 {
 	using Cfg = GemmRing3Cfg<TM, TN>;
-	const bool ragged = M % Cfg::BM != 0 || N % Cfg::BN != 0;
+	const bool c_aligned = reinterpret_cast<uintptr_t>(C) % 16 == 0 && ldc % 8 == 0 && stride_c % 8 == 0;
+	const bool ragged = M % Cfg::BM != 0 || N % Cfg::BN != 0 || !c_aligned;
 	const int which = planes != nullptr ? 2 : ragged ? 1 : 0;
 	auto kernel = which == 2 ? gemm_f16_nt_ring3_kernel<TM, TN, true, true>
 	            : which == 1 ? gemm_f16_nt_ring3_kernel<TM, TN, true, false> : gemm_f16_nt_ring3_kernel<TM, TN, false, false>;

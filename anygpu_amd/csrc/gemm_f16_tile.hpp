@@ -192,6 +192,26 @@ __device__ __forceinline__ half4_t lds_read_transposed_b64(const char* lds_addr)
 // (4096^3: 93.5 -> 92.4 us); the same bytes written without the LDS pass, 64 contiguous bytes per row and instruction
 // after a v_permlane16_swap between neighbouring tiles, were 1.5 us slower than whole rows through LDS.
 typedef half8_t LooseHalf8Store __attribute__((aligned(2)));
+typedef half4_t LooseHalf4Store __attribute__((aligned(8)));
+typedef half2_t LooseHalf2Store __attribute__((aligned(4)));
+
+// Eight halves to an address that is a multiple of 16 bytes plus `misalign` (the same for every store of a launch: rows
+// of C start where its base and its pitch put them): in the widest pieces that alignment allows.
+__device__ __forceinline__ void store_half8_at_alignment(half_t* dst, const half8_t& v, unsigned misalign)
+{
+	if (misalign == 0) *reinterpret_cast<half8_t*>(dst) = v;
+	else if ((misalign & 7) == 0)
+	{
+		reinterpret_cast<LooseHalf4Store*>(dst)[0] = half4_t{v[0], v[1], v[2], v[3]};
+		reinterpret_cast<LooseHalf4Store*>(dst)[1] = half4_t{v[4], v[5], v[6], v[7]};
+	}
+	else if ((misalign & 3) == 0)
+	{
+#pragma unroll
+		for (int e = 0; e < 4; ++e) reinterpret_cast<LooseHalf2Store*>(dst)[e] = half2_t{v[2 * e], v[2 * e + 1]};
+	}
+	else *reinterpret_cast<LooseHalf8Store*>(dst) = v;
+}
 
 // EPI: what happens to a sum on its way out (gemm_epilogue.hpp).  kEpiBias adds bias[n] (fp16), kEpiSoftcap
 // caps, and with kEpiGeluMul the patch holds two products side by side: MFMA column tiles 0 .. TN / 2 - 1 are A x B_gate
@@ -216,6 +236,8 @@ __device__ __forceinline__ void store_patch_via_lds(
 	static_assert(Cfg::kWaves * MI * kPitch <= Cfg::kLdsBytes, "epilogue scratch must fit in the staging LDS");
 	char* scratch = lds + wave * (MI * kPitch);
 	const int frag_row = lane % MI;
+	// (n_base and the 8-column chunks are multiples of 16 bytes: a store is as aligned as C and its row pitch are)
+	[[maybe_unused]] const unsigned misalign = (unsigned)((reinterpret_cast<uintptr_t>(C) | (uintptr_t)(ldc * 2)) & 15);
 	// the bias of this lane's columns (the same for every row band)
 	[[maybe_unused]] float bias_of[TN][Shape::kAccRegs / 4][4] = {};
 	if constexpr (EPI == kEpiBias)
@@ -267,7 +289,7 @@ __device__ __forceinline__ void store_patch_via_lds(
 				const half8_t v = *reinterpret_cast<const half8_t*>(scratch + row * kPitch + col16 * 16);
 				half_t* dst = C + (m_base + i * MI + row) * ldc + n_base + col16 * 8;
 				if constexpr (STREAM && !RAGGED) __builtin_nontemporal_store(v, reinterpret_cast<half8_t*>(dst));
-				else if (!RAGGED || n_base + col16 * 8 + 8 <= N) *reinterpret_cast<LooseHalf8Store*>(dst) = v;
+				else if (!RAGGED || n_base + col16 * 8 + 8 <= N) store_half8_at_alignment(dst, v, misalign);
 				else
 				{
 #pragma unroll

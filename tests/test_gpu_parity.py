@@ -736,6 +736,41 @@ def test_mm_f16_smaller_four_wave_tiles_integer_inputs_exact(ops, m, n, k, pad, 
     assert np.array_equal(got, want)
 
 
+@pytest.mark.parametrize("layout,m,n,k,a_off,b_off,pad", [
+    ("row", 1024, 1028, 512, 0, 0, 0),       # [K, N] weights with N no multiple of 8
+    ("row", 512, 1000, 1027, 0, 0, 0),       # K no multiple of 8: both operands
+    ("col", 600, 1000, 1027, 0, 0, 0),
+    ("col", 512, 1024, 512, 1, 0, 0),        # A starts at an odd element
+    ("col", 512, 1024, 512, 0, 3, 0),        # B starts at an odd element
+    ("col", 512, 1024, 512, 0, 0, 3),        # row pitches no multiple of 8
+    ("row", 700, 1096, 520, 5, 1, 1),        # everything at once
+    ("col", 2048, 2052, 1000, 1, 1, 0),
+])
+def test_mm_f16_operands_the_tile_kernels_cannot_fetch_are_copied(ops, layout, m, n, k, a_off, b_off, pad):
+    # operands at odd addresses, with odd row pitches, a K or (weights stored [K, N]) an N that is no multiple of 8, in
+    # products big enough to pay for it: aligned zero-padded copies in the stream's workspace, then the ordinary
+    # kernels.  Integer operands: exact whatever the summation order.  Guard values around every buffer: the copies must
+    # not read them as data, the product must not write outside the result.
+    import torch
+    from anygpu_amd import capi
+    a = synth.integers(m + k + 6, (m, k), -1, 1).astype(np.float16)
+    b = synth.integers(n + k + 7, (k, n), -1, 1).astype(np.float16)
+    a_flat = torch.full((a_off + m * (k + pad) + 8,), 9.0, dtype=torch.float16, device="cuda")
+    a_view = a_flat[a_off:a_off + m * (k + pad)].view(m, k + pad)[:, :k]
+    a_view.copy_(dev(a))
+    rows, cols = (k, n) if layout == "row" else (n, k)
+    b_flat = torch.full((b_off + rows * (cols + pad) + 8,), 9.0, dtype=torch.float16, device="cuda")
+    b_view = b_flat[b_off:b_off + rows * (cols + pad)].view(rows, cols + pad)[:, :cols]
+    b_view.copy_(dev(b if layout == "row" else np.ascontiguousarray(b.T)))
+    cbuf = torch.full((m + 2, n + 9), -7.0, device="cuda", dtype=torch.float16)
+    ops.tensor_mm(a_view, b_view, out=cbuf[:m, :n], b_layout=capi.B_ROW_MAJOR if layout == "row" else capi.B_COL_MAJOR)
+    got = host(cbuf).astype(np.int64)
+    want = a.astype(np.int64) @ b.astype(np.int64)
+    assert np.abs(want).max() < 2048
+    assert np.array_equal(got[:m, :n], want)
+    assert np.all(got[m:, :] == -7) and np.all(got[:, n:] == -7)
+
+
 def test_mm_f16_whole_256_tiles_batched(ops, oracle):
     # four products of 2048 x 2048 x 128 in one launch: 256 tiles of 256 x 256, the four-wave kernel over blockIdx.y
     from anygpu_amd import capi
