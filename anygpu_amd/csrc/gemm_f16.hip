@@ -342,9 +342,9 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
 	// Operands the tile kernels cannot fetch (an odd start or row pitch, K no multiple of 8, [K, N] weights with such an
 	// N) are copied into the stream's workspace as aligned k-contiguous rows, zeros up to the next multiple of 64 behind
 	// K, and the product runs on the copies: 4096 x 4100 . [4096, 4100] weights 270 -> 117 us (vendor 105 - 110).  From
-	// 16 rows on (below that the weights are streamed once anyway and a copy would triple that), for products worth
+	// 64 rows on (below that the weights are streamed once anyway and a copy would triple that), for products worth
 	// two more launches, where the workspace holds the copies; otherwise the element-wise kernel at the bottom.
-	if (!tiles_ok && batch == 1 && M >= 16 && (double)M * (double)N * (double)K >= (double)(1 << 27))
+	if (!tiles_ok && batch == 1 && M >= 64 && (double)M * (double)N * (double)K >= (double)(1 << 27))
 	{
 		const bool k_odd = K % 8 != 0;
 		const bool copy_a = k_odd || reinterpret_cast<uintptr_t>(A) % 16 != 0 || lda % 8 != 0;

@@ -27,6 +27,7 @@ namespace anygpu {
 constexpr int kAccessFull = 0;      // whole tiles, aligned: no tests
 constexpr int kAccessAligned = 1;   // 16-byte aligned rows and leading dimensions, ragged M / N / K
 constexpr int kAccessAny = 2;       // nothing assumed: vectors at element alignment, guarded ends
+constexpr int kAccessPadded = 3;    // operands as in kAccessFull (aligned copies padded with zeros to whole tiles), C as in kAccessAny
 
 constexpr int kBK = 16;
 constexpr int kPitchK = kBK + 4;     // floats per [row][k] LDS row: 80 bytes, keeps 16-byte alignment
@@ -43,7 +44,7 @@ constexpr int kSchedDsWrite = 0x200;
 template <bool KCONTIG, int ACCESS, int ROWS>
 struct Slab
 {
-	static constexpr bool FULL = (ACCESS == kAccessFull);
+	static constexpr bool FULL = (ACCESS == kAccessFull || ACCESS == kAccessPadded);
 	static constexpr bool kKContig = KCONTIG;
 	static constexpr int kPitchR = ROWS + 4;                 // floats per [k][row] LDS row
 	static constexpr int kLdsFloats = KCONTIG ? ROWS * kPitchK : kBK * kPitchR;
@@ -128,7 +129,8 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(
 	int64_t stride_a, int64_t stride_b, int64_t stride_c, float ep_param, int64_t k_split)
 {
 	constexpr bool DUAL = (EPI == kEpiGeluMul);
-	constexpr bool FULL = (ACCESS == kAccessFull);
+	constexpr bool FULL = (ACCESS == kAccessFull);                                  // no test anywhere
+	constexpr bool FULL_IN = FULL || ACCESS == kAccessPadded;                       // none on the operand side
 	if (k_split > 0)
 	{
 		// blockIdx.z counts ranges of K of one product instead of products: the strides step along K
@@ -237,7 +239,7 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(
 		multiply(set);                             // tile kt
 		stage(set);                                // tile kt + 2
 		fetch(set, kt + 4);
-		if constexpr (FULL)
+		if constexpr (FULL_IN)
 		{
 			// Issue order inside the step: the LDS reads ride on the first half of the MFMAs, the
 			// LDS writes and then the global loads (which reuse the registers just written out) on
@@ -315,7 +317,7 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(
 					float4_t out;
 #pragma unroll
 					for (int e = 0; e < 4; ++e) out[e] = finish(e);
-					if (ACCESS == kAccessAny) *reinterpret_cast<LooseVec*>(C + m * ldc + n) = out;
+					if (ACCESS == kAccessAny || ACCESS == kAccessPadded) *reinterpret_cast<LooseVec*>(C + m * ldc + n) = out;
 					else *reinterpret_cast<float4_t*>(C + m * ldc + n) = out;
 				}
 				else if (m < M)
@@ -334,17 +336,22 @@ template <int A_LAYOUT, int B_LAYOUT, int BM, int BN, int EPI>
 static hipError_t launch_tiles_once(const float* A, const float* B, const float* B2, const float* bias, float* C,
                                     int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc,
                                     int64_t stride_a, int64_t stride_b, int64_t stride_c, int64_t batch,
-                                    float ep_param, int64_t k_split, hipStream_t stream)
+                                    float ep_param, int64_t k_split, hipStream_t stream, bool padded = false)
 {
 	const dim3 grid((unsigned)((N + BN - 1) / BN), (unsigned)((M + BM - 1) / BM), (unsigned)batch);
-	const bool aligned = (reinterpret_cast<uintptr_t>(A) % 16 == 0) && (reinterpret_cast<uintptr_t>(B) % 16 == 0) &&
-	                     (reinterpret_cast<uintptr_t>(B2) % 16 == 0) &&
-	                     (reinterpret_cast<uintptr_t>(C) % 16 == 0) && (lda % 4 == 0) && (ldb % 4 == 0) && (ldc % 4 == 0) &&
-	                     (stride_a % 4 == 0) && (stride_b % 4 == 0) && (stride_c % 4 == 0);
+	const bool aligned_in = (reinterpret_cast<uintptr_t>(A) % 16 == 0) && (reinterpret_cast<uintptr_t>(B) % 16 == 0) &&
+	                        (reinterpret_cast<uintptr_t>(B2) % 16 == 0) && (lda % 4 == 0) && (ldb % 4 == 0) &&
+	                        (stride_a % 4 == 0) && (stride_b % 4 == 0);
+	const bool aligned = aligned_in && (reinterpret_cast<uintptr_t>(C) % 16 == 0) && (ldc % 4 == 0) && (stride_c % 4 == 0);
 	const bool full = aligned && (M % BM == 0) && (N % BN == 0) && (K % kBK == 0) && (k_split % kBK == 0);
+	// padded: the operands are aligned copies that reach, filled with zeros, to the end of the last tile in every direction
+	const bool padded_in = padded && aligned_in && (K % kBK == 0) && (k_split % kBK == 0);
 	discard_stale_error();
 	if (full)
 		gemm_f32_kernel<A_LAYOUT, B_LAYOUT, kAccessFull, BM, BN, EPI><<<grid, dim3(256), 0, stream>>>(
+			A, B, B2, bias, C, M, N, K, lda, ldb, ldc, stride_a, stride_b, stride_c, ep_param, k_split);
+	else if (padded_in)
+		gemm_f32_kernel<A_LAYOUT, B_LAYOUT, kAccessPadded, BM, BN, EPI><<<grid, dim3(256), 0, stream>>>(
 			A, B, B2, bias, C, M, N, K, lda, ldb, ldc, stride_a, stride_b, stride_c, ep_param, k_split);
 	else if (aligned)
 		gemm_f32_kernel<A_LAYOUT, B_LAYOUT, kAccessAligned, BM, BN, EPI><<<grid, dim3(256), 0, stream>>>(
@@ -450,7 +457,7 @@ template <int A_LAYOUT, int B_LAYOUT, int BM, int BN, int EPI>
 static hipError_t launch_tiles(const float* A, const float* B, const float* B2, const float* bias, float* C,
                                 int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc,
                                 int64_t stride_a, int64_t stride_b, int64_t stride_c, int64_t batch,
-                                float ep_param, int64_t splits, hipStream_t stream)
+                                float ep_param, int64_t splits, hipStream_t stream, bool padded = false)
 {
 	if constexpr (EPI != kEpiGeluMul)
 	{
@@ -467,7 +474,7 @@ static hipError_t launch_tiles(const float* A, const float* B, const float* B2, 
 				const int64_t step_a = (A_LAYOUT == ANYGPU_A_ROW_MAJOR) ? k_split : k_split * lda;
 				const int64_t step_b = (B_LAYOUT == ANYGPU_B_COL_MAJOR) ? k_split : k_split * ldb;
 				const hipError_t err = launch_tiles_once<A_LAYOUT, B_LAYOUT, BM, BN, kEpiBias>(
-					A, B, nullptr, nullptr, partial, M, N, K, lda, ldb, N, step_a, step_b, M * N, splits, 0.0f, k_split, stream);
+					A, B, nullptr, nullptr, partial, M, N, K, lda, ldb, N, step_a, step_b, M * N, splits, 0.0f, k_split, stream, padded);
 				if (err != hipSuccess) return err;
 				const int64_t items = M * ((N + 3) / 4);
 				const dim3 grid((unsigned)((items + 255) / 256));
@@ -481,14 +488,14 @@ static hipError_t launch_tiles(const float* A, const float* B, const float* B2, 
 		}
 	}
 	return launch_tiles_once<A_LAYOUT, B_LAYOUT, BM, BN, EPI>(A, B, B2, bias, C, M, N, K, lda, ldb, ldc,
-	                                                          stride_a, stride_b, stride_c, batch, ep_param, 0, stream);
+	                                                          stride_a, stride_b, stride_c, batch, ep_param, 0, stream, padded);
 }
 
 template <int A_LAYOUT, int B_LAYOUT, int EPI>
 static hipError_t launch_layout(const float* A, const float* B, const float* B2, const float* bias, float* C,
                                 int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc,
                                 int64_t stride_a, int64_t stride_b, int64_t stride_c, int64_t batch,
-                                float ep_param, hipStream_t stream)
+                                float ep_param, hipStream_t stream, bool padded = false)
 {
 	const bool may_split = (EPI != kEpiGeluMul);
 	// (what the stream's workspace holds bounds the cuts along K: the caller's, or the library's own for eager launches;
@@ -515,23 +522,23 @@ static hipError_t launch_layout(const float* A, const float* B, const float* B2,
 			if (head.cost + tail.cost + 3.0 < 0.96 * best_whole)
 			{
 				const hipError_t err = launch_tiles<A_LAYOUT, B_LAYOUT, 128, 128, EPI>(
-					A, B, B2, bias, C, M, n_head, K, lda, ldb, ldc, 0, 0, 0, 1, ep_param, 1, stream);
+					A, B, B2, bias, C, M, n_head, K, lda, ldb, ldc, 0, 0, 0, 1, ep_param, 1, stream, padded);
 				if (err != hipSuccess) return err;
 				const float* b_tail = (B_LAYOUT == ANYGPU_B_COL_MAJOR) ? B + n_head * ldb : B + n_head;
 				const float* bias_tail = bias ? bias + n_head : nullptr;
 				if (tail.tile == 128)
 					return launch_tiles<A_LAYOUT, B_LAYOUT, 128, 128, EPI>(A, b_tail, nullptr, bias_tail, C + n_head, M, n_tail, K,
-					                                                       lda, ldb, ldc, 0, 0, 0, 1, ep_param, tail.splits, stream);
+					                                                       lda, ldb, ldc, 0, 0, 0, 1, ep_param, tail.splits, stream, padded);
 				return launch_tiles<A_LAYOUT, B_LAYOUT, 64, 64, EPI>(A, b_tail, nullptr, bias_tail, C + n_head, M, n_tail, K,
-				                                                     lda, ldb, ldc, 0, 0, 0, 1, ep_param, tail.splits, stream);
+				                                                     lda, ldb, ldc, 0, 0, 0, 1, ep_param, tail.splits, stream, padded);
 			}
 		}
 	}
 	if (big.cost <= small.cost)
 		return launch_tiles<A_LAYOUT, B_LAYOUT, 128, 128, EPI>(A, B, B2, bias, C, M, N, K, lda, ldb, ldc,
-		                                                       stride_a, stride_b, stride_c, batch, ep_param, big.splits, stream);
+		                                                       stride_a, stride_b, stride_c, batch, ep_param, big.splits, stream, padded);
 	return launch_tiles<A_LAYOUT, B_LAYOUT, 64, 64, EPI>(A, B, B2, bias, C, M, N, K, lda, ldb, ldc,
-	                                                     stride_a, stride_b, stride_c, batch, ep_param, small.splits, stream);
+	                                                     stride_a, stride_b, stride_c, batch, ep_param, small.splits, stream, padded);
 }
 
 hipError_t launch_gemm_f32(const float* A, const float* B, const float* bias, float* C,
@@ -541,6 +548,56 @@ hipError_t launch_gemm_f32(const float* A, const float* B, const float* bias, fl
                            int a_layout, int b_layout, hipStream_t stream)
 {
 	if (M == 0 || N == 0 || batch == 0) return hipSuccess;
+	// Operands that start at an odd address or have an odd row pitch would be fetched element by element, and operands
+	// that end inside a tile make the kernel test every vector it fetches (2047^3: 69 TFLOP/s, 2044^3: 70, against 119
+	// for 2048^3).  From 128 rows on (fewer rows stream the weights once, which a copy would triple), for products worth two more launches, such operands are copied into the stream's
+	// workspace in their own layout, aligned and filled with zeros up to whole tiles of 128 in every direction, and the
+	// tile kernels fetch the copies without tests; only the stores into C are guarded.
+	const bool a_odd = reinterpret_cast<uintptr_t>(A) % 16 != 0 || lda % 4 != 0;
+	const bool b_odd = reinterpret_cast<uintptr_t>(B) % 16 != 0 || ldb % 4 != 0;
+	const bool ragged = M % 128 != 0 || N % 128 != 0 || K % kBK != 0;
+	if ((a_odd || b_odd || ragged) && batch == 1 && M >= 128 && (double)M * (double)N * (double)K >= (double)(1 << 29))
+	{
+		const int64_t m_pad = (M + 127) / 128 * 128, n_pad = (N + 127) / 128 * 128, k_pad = (K + 127) / 128 * 128;
+		const bool copy_a = a_odd || M % 128 != 0 || K % kBK != 0, copy_b = b_odd || N % 128 != 0 || K % kBK != 0;
+		const bool a_rows_m = a_layout == ANYGPU_A_ROW_MAJOR, b_rows_n = b_layout == ANYGPU_B_COL_MAJOR;
+		const size_t bytes_a = copy_a ? (size_t)m_pad * k_pad * 4 : 0;
+		const size_t bytes_b = copy_b ? (size_t)n_pad * k_pad * 4 : 0;
+		if (bytes_a + bytes_b <= band::workspace_capacity(stream))
+		{
+			float* front = nullptr;
+			hipError_t err = band::workspace_acquire(stream, &front);
+			if (err != hipSuccess) return err;
+			float* a_copy = front;
+			float* b_copy = reinterpret_cast<float*>(reinterpret_cast<char*>(front) + bytes_a);
+			if (copy_a)
+			{
+				err = a_rows_m ? launch_repack_rows(A, lda, M, K, a_copy, k_pad, 4, stream, m_pad)
+				               : launch_repack_rows(A, lda, K, M, a_copy, m_pad, 4, stream, k_pad);
+				if (err != hipSuccess) return err;
+			}
+			if (copy_b)
+			{
+				err = b_rows_n ? launch_repack_rows(B, ldb, N, K, b_copy, k_pad, 4, stream, n_pad)
+				               : launch_repack_rows(B, ldb, K, N, b_copy, n_pad, 4, stream, k_pad);
+				if (err != hipSuccess) return err;
+			}
+			// (an operand that is used as it lies is whole and aligned already; K grows to the zeros only where both
+			// operands have them)
+			const int64_t k_used = K % kBK != 0 ? k_pad : K;
+			const float* a_use = copy_a ? a_copy : A;
+			const float* b_use = copy_b ? b_copy : B;
+			const int64_t lda_use = copy_a ? (a_rows_m ? k_pad : m_pad) : lda, ldb_use = copy_b ? (b_rows_n ? k_pad : n_pad) : ldb;
+			const band::WorkspaceReserve keep(bytes_a + bytes_b);
+#define ANYGPU_F32_PADDED(AL, BL) \
+			return launch_layout<AL, BL, kEpiBias>(a_use, b_use, nullptr, bias, C, M, N, k_used, lda_use, ldb_use, ldc, 0, 0, 0, 1, 0.0f, stream, true)
+			if (a_rows_m && b_rows_n) ANYGPU_F32_PADDED(ANYGPU_A_ROW_MAJOR, ANYGPU_B_COL_MAJOR);
+			if (a_rows_m) ANYGPU_F32_PADDED(ANYGPU_A_ROW_MAJOR, ANYGPU_B_ROW_MAJOR);
+			if (b_rows_n) ANYGPU_F32_PADDED(ANYGPU_A_COL_MAJOR, ANYGPU_B_COL_MAJOR);
+			ANYGPU_F32_PADDED(ANYGPU_A_COL_MAJOR, ANYGPU_B_ROW_MAJOR);
+#undef ANYGPU_F32_PADDED
+		}
+	}
 	if (batch == 1 && a_layout == ANYGPU_A_ROW_MAJOR && gemm_band_applies<float>(A, B, nullptr, C, M, N, K, lda, ldb, ldc, b_layout))
 		return launch_gemm_band<float>(A, B, nullptr, bias, C, M, N, K, lda, ldb, ldc, kEpiBias, 0.0f, stream);
 	if (batch == 1 && a_layout == ANYGPU_A_ROW_MAJOR && b_layout == ANYGPU_B_ROW_MAJOR &&

@@ -44,17 +44,17 @@ __device__ __forceinline__ uint4_t load_16_bytes_anywhere(const char* from, int 
 	return out;
 }
 
-// dst[row][c] = c < cols ? src[row][c] : 0 for c < ld_dst; one thread per 16 bytes of dst
+// dst[row][c] = (row < rows && c < cols) ? src[row][c] : 0 for row < rows_dst, c < ld_dst; one thread per 16 bytes of dst
 template <typename T>
 __global__ __launch_bounds__(256) void repack_rows_kernel(const T* __restrict__ src, int64_t ld_src, int64_t rows, int64_t cols,
-                                                          T* __restrict__ dst, int64_t ld_dst)
+                                                          T* __restrict__ dst, int64_t ld_dst, int64_t rows_dst)
 {
 	constexpr int kPer = 16 / sizeof(T);
 	const int64_t chunks = ld_dst / kPer;
 	const int64_t item = (int64_t)blockIdx.x * 256 + threadIdx.x;
-	if (item >= rows * chunks) return;
+	if (item >= rows_dst * chunks) return;
 	const int64_t row = item / chunks, c0 = (item % chunks) * kPer;
-	const int64_t left = cols - c0;
+	const int64_t left = row < rows ? cols - c0 : 0;
 	const int valid = left >= kPer ? 16 : left <= 0 ? 0 : (int)(left * sizeof(T));
 	*reinterpret_cast<uint4_t*>(dst + row * ld_dst + c0) =
 		load_16_bytes_anywhere(reinterpret_cast<const char*>(src + row * ld_src + c0), valid);
@@ -100,15 +100,16 @@ __global__ __launch_bounds__(256) void repack_transposed_kernel(const T* __restr
 }  // namespace
 
 hipError_t launch_repack_rows(const void* src, int64_t ld_src, int64_t rows, int64_t cols, void* dst, int64_t ld_dst,
-                              int elem_bytes, hipStream_t stream)
+                              int elem_bytes, hipStream_t stream, int64_t rows_dst)
 {
 	(void)hipGetLastError();
-	const int64_t items = rows * (ld_dst / (16 / elem_bytes));
+	if (rows_dst < rows) rows_dst = rows;
+	const int64_t items = rows_dst * (ld_dst / (16 / elem_bytes));
 	const dim3 grid((unsigned)((items + 255) / 256));
 	if (elem_bytes == 2)
-		repack_rows_kernel<uint16_t><<<grid, dim3(256), 0, stream>>>(static_cast<const uint16_t*>(src), ld_src, rows, cols, static_cast<uint16_t*>(dst), ld_dst);
+		repack_rows_kernel<uint16_t><<<grid, dim3(256), 0, stream>>>(static_cast<const uint16_t*>(src), ld_src, rows, cols, static_cast<uint16_t*>(dst), ld_dst, rows_dst);
 	else
-		repack_rows_kernel<uint32_t><<<grid, dim3(256), 0, stream>>>(static_cast<const uint32_t*>(src), ld_src, rows, cols, static_cast<uint32_t*>(dst), ld_dst);
+		repack_rows_kernel<uint32_t><<<grid, dim3(256), 0, stream>>>(static_cast<const uint32_t*>(src), ld_src, rows, cols, static_cast<uint32_t*>(dst), ld_dst, rows_dst);
 	return hipGetLastError();
 }
 

@@ -68,10 +68,11 @@ hipError_t launch_gemm_f16_probe(const void* A, const void* B, void* C, int64_t 
                                  int64_t lda, int64_t ldb, int64_t ldc, unsigned long long* probe, hipStream_t stream);
 
 // Aligned copies of operands the tile kernels cannot fetch as they lie (gemm_repack.hip): `rows` rows of `cols` elements
-// at any alignment into rows of pitch ld_dst (a multiple of 64 elements, 16-byte aligned), zeros behind `cols`; and the
-// same from a [k_rows, n_cols] matrix read down its columns, dst[n][k] = src[k][n].  elem_bytes 2 or 4.
+// at any alignment into rows of pitch ld_dst (a multiple of 64 elements, 16-byte aligned), zeros behind `cols` and in
+// the rows from `rows` up to rows_dst; and the same from a [k_rows, n_cols] matrix read down its columns,
+// dst[n][k] = src[k][n].  elem_bytes 2 or 4.
 hipError_t launch_repack_rows(const void* src, int64_t ld_src, int64_t rows, int64_t cols, void* dst, int64_t ld_dst,
-                              int elem_bytes, hipStream_t stream);
+                              int elem_bytes, hipStream_t stream, int64_t rows_dst = 0);
 hipError_t launch_repack_transposed(const void* src, int64_t ld_src, int64_t k_rows, int64_t n_cols, void* dst, int64_t ld_dst,
                                     int elem_bytes, hipStream_t stream);
 

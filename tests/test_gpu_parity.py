@@ -771,6 +771,33 @@ def test_mm_f16_operands_the_tile_kernels_cannot_fetch_are_copied(ops, layout, m
     assert np.all(got[m:, :] == -7) and np.all(got[:, n:] == -7)
 
 
+@pytest.mark.parametrize("layout,m,n,k,a_off,b_off,pad", [
+    ("row", 2047, 2047, 2047, 0, 0, 0), ("col", 1023, 1025, 1030, 0, 0, 0), ("row", 1024, 1024, 512, 1, 0, 0),
+    ("col", 1024, 1024, 512, 0, 3, 0), ("row", 700, 1096, 720, 2, 1, 1), ("col", 1024, 1024, 512, 0, 0, 3),
+    ("row", 1000, 1000, 1000, 0, 0, 0), ("col", 2044, 2044, 520, 0, 0, 0),
+])
+def test_mm_f32_operands_at_odd_addresses_are_copied(ops, layout, m, n, k, a_off, b_off, pad):
+    # fp32 operands with odd starts or row pitches, in products big enough to pay for it: aligned copies in the stream's
+    # workspace, then the ordinary kernels (C keeps its own alignment).  Integer operands: every sum exact in fp32.
+    import torch
+    from anygpu_amd import capi
+    a = synth.integers(m + k + 8, (m, k), -3, 3).astype(np.float32)
+    b = synth.integers(n + k + 9, (k, n), -3, 3).astype(np.float32)
+    a_flat = torch.full((a_off + m * (k + pad) + 8,), 9.0, dtype=torch.float32, device="cuda")
+    a_view = a_flat[a_off:a_off + m * (k + pad)].view(m, k + pad)[:, :k]
+    a_view.copy_(dev(a))
+    rows, cols = (k, n) if layout == "row" else (n, k)
+    b_flat = torch.full((b_off + rows * (cols + pad) + 8,), 9.0, dtype=torch.float32, device="cuda")
+    b_view = b_flat[b_off:b_off + rows * (cols + pad)].view(rows, cols + pad)[:, :cols]
+    b_view.copy_(dev(b if layout == "row" else np.ascontiguousarray(b.T)))
+    cbuf = torch.full((m + 2, n + 5), -7.0, device="cuda", dtype=torch.float32)
+    ops.tensor_mm(a_view, b_view, out=cbuf[:m, :n], b_layout=capi.B_ROW_MAJOR if layout == "row" else capi.B_COL_MAJOR)
+    got = host(cbuf).astype(np.int64)
+    want = a.astype(np.int64) @ b.astype(np.int64)
+    assert np.array_equal(got[:m, :n], want)
+    assert np.all(got[m:, :] == -7) and np.all(got[:, n:] == -7)
+
+
 def test_mm_f16_whole_256_tiles_batched(ops, oracle):
     # four products of 2048 x 2048 x 128 in one launch: 256 tiles of 256 x 256, the four-wave kernel over blockIdx.y
     from anygpu_amd import capi
