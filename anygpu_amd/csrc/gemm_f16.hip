@@ -222,13 +222,14 @@ struct FourWavePlan
 	double us = 1e30;
 };
 
-static FourWavePlan plan_four_wave(int64_t M, int64_t N, int64_t K, int64_t batch, int64_t cus, int64_t plane_room)
+// dual: two products side by side in a tile (GELU(gate) * up), which then covers half the output columns
+static FourWavePlan plan_four_wave(int64_t M, int64_t N, int64_t K, int64_t batch, int64_t cus, int64_t plane_room, bool dual = false)
 {
 	FourWavePlan best;
 	const int64_t slabs = K / 64;
 	for (int kind = 0; kind < 3; ++kind)
 	{
-		const int64_t bm = kind == 2 ? 128 : 256, bn = kind == 0 ? 256 : 128;
+		const int64_t bm = kind == 2 ? 128 : 256, bn = (kind == 0 ? 256 : 128) / (dual ? 2 : 1);
 		const int64_t blocks = ((M + bm - 1) / bm) * ((N + bn - 1) / bn) * batch;
 		if (blocks / batch > 0x7FFFFFFFLL) continue;
 		const int64_t max_splits = (kind == 0 || batch != 1) ? 1 : std::min<int64_t>({16, K / 512, plane_room});
@@ -659,9 +660,33 @@ hipError_t launch_gemm_f16_epilogue(const void* A, const void* B, const void* B2
 		else gemm_f16_finish_kernel<kEpiSoftcap><<<grid, dim3(256), 0, stream>>>(c, bs, M, N, ldc, ep_param);
 		return hipGetLastError();
 	}
+	const int64_t cus = device_cu_count();
+	// one product, k-contiguous weights, whole slabs: the four-wave kernels, priced like the unfused product, uncut
+	if (b_layout == ANYGPU_B_COL_MAJOR && gemm_f16_ring_applies(a, b, M, N, K, lda, ldb, 0, 0, 1, b_layout) &&
+	    (!dual || reinterpret_cast<uintptr_t>(B2) % 16 == 0))
+	{
+		const FourWavePlan four = plan_four_wave(M, N, K, 1, cus, 0, dual);
+		const auto small_blocks = [&](int64_t t) { return ((M + t - 1) / t) * ((N + (dual ? t / 2 : t) - 1) / (dual ? t / 2 : t)); };
+		const double small_us = (double)(K / 64) * slab_us(64, small_blocks(64), cus) + 6.0;
+		if (four.kind >= 0 && four.us < small_us)
+		{
+#define ANYGPU_F16_EPI_FOUR(EPI) \
+			do { \
+				if (four.kind == 0) return launch_gemm_f16_ring<EPI>(a, b, c, M, N, K, lda, ldb, ldc, 0, 0, 0, 1, stream, nullptr, b_layout, bs, ep_param); \
+				if (four.kind == 1) return launch_gemm_f16_ring3<8, 4, EPI>(a, b, c, M, N, K, lda, ldb, ldc, 0, 0, 0, 1, stream, nullptr, 0, bs, ep_param); \
+				return launch_gemm_f16_ring3<4, 4, EPI>(a, b, c, M, N, K, lda, ldb, ldc, 0, 0, 0, 1, stream, nullptr, 0, bs, ep_param); \
+			} while (0)
+			if (epilogue == kEpiSoftcap) ANYGPU_F16_EPI_FOUR(kEpiSoftcap);
+			if (epilogue == kEpiBias) ANYGPU_F16_EPI_FOUR(kEpiBias);
+			// (the second weight matrix travels in the bias argument)
+			if (four.kind == 0) return launch_gemm_f16_ring<kEpiGeluMul>(a, b, c, M, N, K, lda, ldb, ldc, 0, 0, 0, 1, stream, nullptr, b_layout, b2, 0.0f);
+			if (four.kind == 1) return launch_gemm_f16_ring3<8, 4, kEpiGeluMul>(a, b, c, M, N, K, lda, ldb, ldc, 0, 0, 0, 1, stream, nullptr, 0, b2, 0.0f);
+			return launch_gemm_f16_ring3<4, 4, kEpiGeluMul>(a, b, c, M, N, K, lda, ldb, ldc, 0, 0, 0, 1, stream, nullptr, 0, b2, 0.0f);
+#undef ANYGPU_F16_EPI_FOUR
+		}
+	}
 	// a tile of edge t covers t (t / 2 with two products) output columns
 	const auto blocks = [&](int64_t t) { return ((M + t - 1) / t) * ((N + (dual ? t / 2 : t) - 1) / (dual ? t / 2 : t)); };
-	const int64_t cus = device_cu_count();
 	const double cost256 = slab_us(256, blocks(256), cus), cost128 = slab_us(128, blocks(128), cus), cost64 = slab_us(64, blocks(64), cus);
 	const int64_t tile = (cost256 <= cost128 && cost256 <= cost64) ? 256 : cost128 <= cost64 ? 128 : 64;
 	if (blocks(tile) > 0x7FFFFFFFLL)

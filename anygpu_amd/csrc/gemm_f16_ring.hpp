@@ -34,11 +34,18 @@ struct GemmRingCfg
 // caller gets the clock the part sustained under this kernel and the share of those cycles the matrix cores were busy.
 // B_KN: B stored [K, N] (row k holds the n), staged as a [64 k][256 n] unit and read through transposing LDS reads; N is a
 // multiple of 8 then, and column chunks past N are read from the last whole chunk of the row.
-template <bool RAGGED, bool B_KN>
+// EPI: kEpiNone, kEpiBias (+ bias[n]) or kEpiSoftcap (ep_param * tanh(sum / ep_param)), applied to the fp32 sums; or
+// kEpiGeluMul (k-contiguous weights only): the tile is 128 output columns wide (N and tiles_n count those) and its B unit
+// is put together from two matrices: of every wave column's 128 unit rows the first 64 come from B (the gate weights) and
+// the second 64 from `bias`, which then is the second matrix B2 (the up weights, same pitch), both for the same 64 output
+// columns, so that gate and up sums of an output element meet in one lane, A is read once for both products and
+// gelu_tanh(gate) * up goes out.  The wave that loads a quarter of the unit loads it from one matrix.
+template <bool RAGGED, bool B_KN, int EPI = kEpiNone>
 __global__ __launch_bounds__(256) void gemm_f16_nt_ring_kernel(
 	const half_t* __restrict__ A, const half_t* __restrict__ B, half_t* __restrict__ C,
 	int K, int64_t lda, int64_t ldb, int64_t ldc, int tiles_m, int tiles_n,
-	int64_t stride_a, int64_t stride_b, int64_t stride_c, unsigned long long* __restrict__ probe, int64_t M, int64_t N)
+	int64_t stride_a, int64_t stride_b, int64_t stride_c, unsigned long long* __restrict__ probe, int64_t M, int64_t N,
+	const half_t* __restrict__ bias = nullptr, float ep_param = 0.0f)
 {
 	using Cfg = GemmRingCfg;
 	extern __shared__ __align__(1024) char lds[];
@@ -54,7 +61,12 @@ __global__ __launch_bounds__(256) void gemm_f16_nt_ring_kernel(
 	int tile_m, tile_n;
 	tile_of_block<4>(blockIdx.x, tiles_m, tiles_n, tile_m, tile_n);
 	const int64_t m0 = (int64_t)tile_m * 256;
-	const int64_t n0 = (int64_t)tile_n * 256;
+	constexpr bool DUAL = EPI == kEpiGeluMul;
+	static_assert(!DUAL || !B_KN, "two weight matrices: k-contiguous only");
+	const int64_t n0 = (int64_t)tile_n * (DUAL ? 128 : 256);
+	// DUAL: unit rows 64 w .. + 63 of wave w are output columns 64 (w / 2) .. + 63 of the tile, from B (w even) or B2
+	const half_t* const b_of_wave = DUAL && (wave & 1) ? bias : B;
+	const int b_unit_row = DUAL ? 64 * (wave >> 1) : 64 * wave;       // the wave's first row, as a column of the tile
 
 	// Direct loads.  A unit row is 64 halves = 128 bytes = eight 16-byte chunks; chunk c of row r sits at position
 	// c ^ ((r >> 1) & 7).  One instruction fills 8 rows: lane -> row lane / 8, position lane % 8.  Instruction q of this
@@ -68,7 +80,7 @@ __global__ __launch_bounds__(256) void gemm_f16_nt_ring_kernel(
 	// A [K, N] unit of B has rows of 256 n = 512 bytes = 32 chunks; one instruction fills 2 k rows: lane -> row lane / 32,
 	// position lane % 32, and the chunk at position p of row k is chunk p ^ kn_row_swizzle(k).  Instruction q of this wave
 	// covers rows 16 wave + 2 q, + 1 of the slab's 64.
-	int64_t a_first = m0 + 64 * wave, b_first = n0 + 64 * wave;
+	int64_t a_first = m0 + 64 * wave, b_first = n0 + b_unit_row;
 	if constexpr (RAGGED)
 	{
 		a_first = a_first < M - 1 ? a_first : M - 1;
@@ -79,7 +91,7 @@ __global__ __launch_bounds__(256) void gemm_f16_nt_ring_kernel(
 	{
 		const int row = 64 * wave + 8 * q + ld_row;
 		const unsigned chunk = ld_pos ^ ((row >> 1) & 7);
-		int64_t a_row = m0 + row, b_row = n0 + row;
+		int64_t a_row = m0 + row, b_row = n0 + b_unit_row + 8 * q + ld_row;
 		if constexpr (RAGGED)
 		{
 			a_row = a_row < M - 1 ? a_row : M - 1;
@@ -99,7 +111,7 @@ __global__ __launch_bounds__(256) void gemm_f16_nt_ring_kernel(
 	}
 	const unsigned table_addr = lds0 + 4 * Cfg::kUnitBytes + (wave * (16 * 64) + lane) * 4;
 	const uintptr_t a_wave = reinterpret_cast<uintptr_t>(A + a_first * lda);
-	const uintptr_t b_wave = reinterpret_cast<uintptr_t>(B_KN ? B + (int64_t)(16 * wave) * ldb + n0 : B + b_first * ldb);
+	const uintptr_t b_wave = reinterpret_cast<uintptr_t>(B_KN ? B + (int64_t)(16 * wave) * ldb + n0 : b_of_wave + b_first * ldb);
 	const unsigned wave_share = wave * 8192;               // the wave's 64 rows inside a unit
 	const unsigned lds_wave = lds0 + wave_share;
 	const int slabs = K / 64;
@@ -185,7 +197,7 @@ __global__ __launch_bounds__(256) void gemm_f16_nt_ring_kernel(
 #pragma unroll
 		for (int j = 0; j < 8; ++j)
 			acc[i][j] = float4_t{(*rows[i])[4 * j], (*rows[i])[4 * j + 1], (*rows[i])[4 * j + 2], (*rows[i])[4 * j + 3]};
-	store_patch_via_lds<Cfg, RAGGED, !RAGGED>(acc, lds, C, ldc, m0 + wm * 128, n0 + wn * 128, wave, lane, M, N);
+	store_patch_via_lds<Cfg, RAGGED, !RAGGED, EPI>(acc, lds, C, ldc, m0 + wm * 128, n0 + wn * (DUAL ? 64 : 128), wave, lane, M, N, bias, ep_param);
 }
 
 // What the kernel assumes, checked on the host before every launch: whole slabs, 16-byte aligned operand rows, and
@@ -201,17 +213,25 @@ inline bool gemm_f16_ring_applies(const half_t* A, const half_t* B, int64_t M, i
 	       ((M + 255) / 256) * ((N + 255) / 256) <= 0x7FFFFFFFLL && batch >= 1 && batch <= 65535;
 }
 
+template <int EPI = kEpiNone>
 inline hipError_t launch_gemm_f16_ring(const half_t* A, const half_t* B, half_t* C, int64_t M, int64_t N, int64_t K,
                                        int64_t lda, int64_t ldb, int64_t ldc,
                                        int64_t stride_a, int64_t stride_b, int64_t stride_c, int64_t batch, hipStream_t stream,
-                                       unsigned long long* probe = nullptr, int b_layout = ANYGPU_B_COL_MAJOR)
+                                       unsigned long long* probe = nullptr, int b_layout = ANYGPU_B_COL_MAJOR,
+                                       const half_t* bias = nullptr, float ep_param = 0.0f)
 {
 	const bool kn = b_layout == ANYGPU_B_ROW_MAJOR;
 	// (whole tiles of an aligned C are streamed out in 16-byte vectors; anything else takes the guarded stores)
 	const bool c_aligned = reinterpret_cast<uintptr_t>(C) % 16 == 0 && ldc % 8 == 0 && stride_c % 8 == 0;
-	const int ragged = (M % 256 != 0 || N % 256 != 0 || !c_aligned) + 2 * kn;       // which instantiation
-	auto kernel = ragged == 0 ? gemm_f16_nt_ring_kernel<false, false> : ragged == 1 ? gemm_f16_nt_ring_kernel<true, false>
-	            : ragged == 2 ? gemm_f16_nt_ring_kernel<false, true> : gemm_f16_nt_ring_kernel<true, true>;
+	constexpr int kOutN = EPI == kEpiGeluMul ? 128 : 256;             // output columns of a tile
+	const int ragged = (M % 256 != 0 || N % kOutN != 0 || !c_aligned) + 2 * kn;       // which instantiation
+	auto kernel = (ragged & 1) == 0 ? gemm_f16_nt_ring_kernel<false, false, EPI> : gemm_f16_nt_ring_kernel<true, false, EPI>;
+	if constexpr (EPI != kEpiGeluMul)
+	{
+		if (ragged == 2) kernel = gemm_f16_nt_ring_kernel<false, true, EPI>;
+		if (ragged == 3) kernel = gemm_f16_nt_ring_kernel<true, true, EPI>;
+	}
+	else if (kn) return hipErrorInvalidValue;
 	// More than 64 KB of dynamic LDS has to be granted per function and per device, once.
 	static std::atomic<uint64_t> configured_devices[4];
 	(void)hipGetLastError();
@@ -225,9 +245,9 @@ inline hipError_t launch_gemm_f16_ring(const half_t* A, const half_t* B, half_t*
 		if (e != hipSuccess) return e;
 		configured_devices[ragged].fetch_or(bit, std::memory_order_relaxed);
 	}
-	const int tiles_m = (int)((M + 255) / 256), tiles_n = (int)((N + 255) / 256);
+	const int tiles_m = (int)((M + 255) / 256), tiles_n = (int)((N + kOutN - 1) / kOutN);
 	kernel<<<dim3((unsigned)(tiles_m * tiles_n), (unsigned)batch), dim3(256), GemmRingCfg::kLdsBytes, stream>>>(
-		A, B, C, (int)K, lda, ldb, ldc, tiles_m, tiles_n, stride_a, stride_b, stride_c, probe, M, N);
+		A, B, C, (int)K, lda, ldb, ldc, tiles_m, tiles_n, stride_a, stride_b, stride_c, probe, M, N, bias, ep_param);
 	return hipGetLastError();
 }
 

@@ -30,12 +30,17 @@ struct GemmRing3Cfg
 // valid row and the stores are guarded.
 // SPLIT: blockIdx.y walks ranges of K (k_split deep, a multiple of 64; the strides step along K) of one product instead
 // of a batch, and the raw fp32 sums of range y go to planes[y][M][N]; C is not touched.
-template <int TM, int TN, bool RAGGED, bool SPLIT>
+// EPI: kEpiNone, kEpiBias (+ bias[n]) or kEpiSoftcap (ep_param * tanh(sum / ep_param)), applied to the fp32 sums (not SPLIT);
+// or kEpiGeluMul: the tile is BN / 2 output columns wide and its B unit holds, for every wave column, gate rows (from B) in
+// front of up rows (from `bias`, which then is the second weight matrix), as in gemm_f16_nt_ring_kernel.
+template <int TM, int TN, bool RAGGED, bool SPLIT, int EPI = kEpiNone>
 __global__ __launch_bounds__(256) void gemm_f16_nt_ring3_kernel(
 	const half_t* __restrict__ A, const half_t* __restrict__ B, half_t* __restrict__ C,
 	int K, int64_t lda, int64_t ldb, int64_t ldc, int tiles_m, int tiles_n,
-	int64_t stride_a, int64_t stride_b, int64_t stride_c, int64_t M, int64_t N, float* __restrict__ planes, int k_split)
+	int64_t stride_a, int64_t stride_b, int64_t stride_c, int64_t M, int64_t N, float* __restrict__ planes, int k_split,
+	const half_t* __restrict__ bias = nullptr, float ep_param = 0.0f)
 {
+	static_assert(!SPLIT || EPI == kEpiNone, "the planes hold raw sums");
 	using Cfg = GemmRing3Cfg<TM, TN>;
 	extern __shared__ __align__(1024) char lds[];
 	if constexpr (SPLIT)
@@ -55,7 +60,11 @@ __global__ __launch_bounds__(256) void gemm_f16_nt_ring3_kernel(
 	int tile_m, tile_n;
 	tile_of_block<4>(blockIdx.x, tiles_m, tiles_n, tile_m, tile_n);
 	const int64_t m0 = (int64_t)tile_m * Cfg::BM;
-	const int64_t n0 = (int64_t)tile_n * Cfg::BN;
+	constexpr bool DUAL = EPI == kEpiGeluMul;
+	const int64_t n0 = (int64_t)tile_n * (DUAL ? Cfg::BN / 2 : Cfg::BN);
+	// DUAL: the unit rows wave w loads are output columns (BN / 4) (w / 2) .. of the tile, from B (w even) or B2
+	const half_t* const b_of_wave = DUAL && (wave & 1) ? bias : B;
+	const int b_unit_row = DUAL ? 8 * Cfg::kLoadsB * (wave >> 1) : 8 * Cfg::kLoadsB * wave;
 
 	// Direct loads.  A unit row is 64 halves = eight 16-byte chunks; chunk c of row r sits at position c ^ ((r >> 1) & 7).
 	// One instruction fills 8 rows: lane -> row lane / 8, position lane % 8.  Instruction q of this wave covers rows
@@ -64,7 +73,7 @@ __global__ __launch_bounds__(256) void gemm_f16_nt_ring3_kernel(
 	const unsigned lds0 = (unsigned)(uintptr_t)(const __attribute__((address_space(3))) char*)lds;
 	const int ld_row = lane >> 3, ld_pos = lane & 7;
 	unsigned* const table = reinterpret_cast<unsigned*>(lds + 3 * Cfg::kStageBytes) + wave * (16 * 64) + lane;
-	int64_t a_first = m0 + 8 * Cfg::kLoadsA * wave, b_first = n0 + 8 * Cfg::kLoadsB * wave;
+	int64_t a_first = m0 + 8 * Cfg::kLoadsA * wave, b_first = n0 + b_unit_row;
 	if constexpr (RAGGED)
 	{
 		a_first = a_first < M - 1 ? a_first : M - 1;
@@ -81,14 +90,14 @@ __global__ __launch_bounds__(256) void gemm_f16_nt_ring3_kernel(
 #pragma unroll
 	for (int q = 0; q < Cfg::kLoadsB; ++q)
 	{
-		const int row = 8 * (Cfg::kLoadsB * wave + q) + ld_row;
-		int64_t b_row = n0 + row;
+		const int row = 8 * (Cfg::kLoadsB * wave + q) + ld_row;                  // in the unit
+		int64_t b_row = n0 + b_unit_row + 8 * q + ld_row;                        // in the matrix
 		if constexpr (RAGGED) b_row = b_row < N - 1 ? b_row : N - 1;
 		table[64 * (8 + q)] = (unsigned)(((b_row - b_first) * ldb + ((ld_pos ^ ((row >> 1) & 7)) << 3)) * 2);
 	}
 	const unsigned table_addr = lds0 + 3 * Cfg::kStageBytes + (wave * (16 * 64) + lane) * 4;
 	const uintptr_t a_wave = reinterpret_cast<uintptr_t>(A + a_first * lda);
-	const uintptr_t b_wave = reinterpret_cast<uintptr_t>(B + b_first * ldb);
+	const uintptr_t b_wave = reinterpret_cast<uintptr_t>(b_of_wave + b_first * ldb);
 	const unsigned share_a = wave * (Cfg::kLoadsA * 1024);                       // the wave's rows inside a stage
 	const unsigned share_b = Cfg::BM * 128 + wave * (Cfg::kLoadsB * 1024);
 	const int slabs = K / 64;
@@ -165,22 +174,28 @@ __global__ __launch_bounds__(256) void gemm_f16_nt_ring3_kernel(
 	if constexpr (SPLIT)
 		store_patch_f32<Cfg>(acc, planes + (int64_t)blockIdx.y * M * N, m0 + wm * Cfg::kWaveM, n0 + wn * Cfg::kWaveN, lane, M, N);
 	else
-		store_patch_via_lds<Cfg, RAGGED, !RAGGED>(acc, lds, C, ldc, m0 + wm * Cfg::kWaveM, n0 + wn * Cfg::kWaveN, wave, lane, M, N);
+		store_patch_via_lds<Cfg, RAGGED, !RAGGED, EPI>(acc, lds, C, ldc, m0 + wm * Cfg::kWaveM, n0 + wn * (DUAL ? Cfg::kWaveN / 2 : Cfg::kWaveN),
+		                                               wave, lane, M, N, bias, ep_param);
 }
 
 // planes != NULL: `batch` is the number of K ranges, k_split their depth, and the strides step along K.
-template <int TM, int TN>
+template <int TM, int TN, int EPI = kEpiNone>
 inline hipError_t launch_gemm_f16_ring3(const half_t* A, const half_t* B, half_t* C, int64_t M, int64_t N, int64_t K,
                                         int64_t lda, int64_t ldb, int64_t ldc,
                                         int64_t stride_a, int64_t stride_b, int64_t stride_c, int64_t batch, hipStream_t stream,
-                                        float* planes = nullptr, int64_t k_split = 0)
+                                        float* planes = nullptr, int64_t k_split = 0, const half_t* bias = nullptr, float ep_param = 0.0f)
 {
 	using Cfg = GemmRing3Cfg<TM, TN>;
 	const bool c_aligned = reinterpret_cast<uintptr_t>(C) % 16 == 0 && ldc % 8 == 0 && stride_c % 8 == 0;
-	const bool ragged = M % Cfg::BM != 0 || N % Cfg::BN != 0 || !c_aligned;
+	constexpr int kOutN = EPI == kEpiGeluMul ? Cfg::BN / 2 : Cfg::BN;       // output columns of a tile
+	const bool ragged = M % Cfg::BM != 0 || N % kOutN != 0 || !c_aligned;
 	const int which = planes != nullptr ? 2 : ragged ? 1 : 0;
-	auto kernel = which == 2 ? gemm_f16_nt_ring3_kernel<TM, TN, true, true>
-	            : which == 1 ? gemm_f16_nt_ring3_kernel<TM, TN, true, false> : gemm_f16_nt_ring3_kernel<TM, TN, false, false>;
+	auto kernel = which == 1 ? gemm_f16_nt_ring3_kernel<TM, TN, true, false, EPI> : gemm_f16_nt_ring3_kernel<TM, TN, false, false, EPI>;
+	if constexpr (EPI == kEpiNone)
+	{
+		if (which == 2) kernel = gemm_f16_nt_ring3_kernel<TM, TN, true, true, kEpiNone>;
+	}
+	else if (which == 2) return hipErrorInvalidValue;
 	// More than 64 KB of dynamic LDS has to be granted per function and per device, once.
 	static std::atomic<uint64_t> configured_devices[3];
 	(void)hipGetLastError();
@@ -194,9 +209,9 @@ inline hipError_t launch_gemm_f16_ring3(const half_t* A, const half_t* B, half_t
 		if (e != hipSuccess) return e;
 		configured_devices[which].fetch_or(bit, std::memory_order_relaxed);
 	}
-	const int tiles_m = (int)((M + Cfg::BM - 1) / Cfg::BM), tiles_n = (int)((N + Cfg::BN - 1) / Cfg::BN);
+	const int tiles_m = (int)((M + Cfg::BM - 1) / Cfg::BM), tiles_n = (int)((N + kOutN - 1) / kOutN);
 	kernel<<<dim3((unsigned)(tiles_m * tiles_n), (unsigned)batch), dim3(256), Cfg::kLdsBytes, stream>>>(
-		A, B, C, (int)K, lda, ldb, ldc, tiles_m, tiles_n, stride_a, stride_b, stride_c, M, N, planes, (int)k_split);
+		A, B, C, (int)K, lda, ldb, ldc, tiles_m, tiles_n, stride_a, stride_b, stride_c, M, N, planes, (int)k_split, bias, ep_param);
 	return hipGetLastError();
 }
 

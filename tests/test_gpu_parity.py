@@ -1044,6 +1044,8 @@ F16_EPILOGUE_SHAPES = [
     # m, k, n: few rows (band kernels), one tile, ragged tiles of every size, a K tail, whole 256 tiles, several rounds
     (1, 2304, 1000), (16, 512, 520), (64, 256, 264), (100, 320, 200), (130, 64, 72), (300, 1000, 392), (513, 2304, 1160),
     (1024, 512, 2048), (2048, 192, 4096), (2304, 136, 4104),
+    # k-contiguous weights in whole slabs: the four-wave kernels (128 x 128, 256 x 128 and 256 x 256 tiles, whole and ragged)
+    (2048, 256, 2048), (2048, 128, 4096), (4096, 128, 4096), (1000, 192, 3000), (3000, 64, 4104),
 ]
 
 
