@@ -40,12 +40,10 @@ constexpr int kNumXcd = 8;
 template <int kGroupM>
 __device__ __forceinline__ void tile_of_block(int bid, int tiles_m, int tiles_n, int& tm, int& tn)
 {
+	// XCD x runs the blocks x, x + 8, ...: they get a contiguous range of tile ids (the first total % 8 XCDs one more)
 	const int total = tiles_m * tiles_n;
-	int id = bid;
-	if (total % kNumXcd == 0)
-	{
-		id = (bid % kNumXcd) * (total / kNumXcd) + bid / kNumXcd;
-	}
+	const int xcd = bid % kNumXcd, share = total / kNumXcd, extra = total % kNumXcd;
+	const int id = xcd * share + (xcd < extra ? xcd : extra) + bid / kNumXcd;
 	const int per_group = kGroupM * tiles_n;
 	const int g = id / per_group;
 	const int first_m = g * kGroupM;
