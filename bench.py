@@ -155,6 +155,8 @@ def bench_gemm_f16(torch, ops, capi, synth, steps, warmup):
     # (the headline times exactly --steps launches; only the kernels below are floored)
     t = timed_region(torch, lambda: ops.tensor_mm(a, bt, out=c, b_layout=capi.B_COL_MAJOR), steps, warmup, floor=1)
     flops = 2.0 * n ** 3
+    # the vendor library on the same operands, timed the same way (torch.matmul = hipBLASLt): for scale, not the target
+    t_vendor = timed_region(torch, lambda: torch.matmul(a, bt.t(), out=c), steps, warmup, floor=1)
     # the clock the part sustains under this kernel and the matrix cores' share of those cycles, from the kernel's own
     # counters (anygpu_gemm_f16_f32acc_probe): launched for another settle period, the last launch read
     lib = capi.load()
@@ -177,6 +179,8 @@ def bench_gemm_f16(torch, ops, capi, synth, steps, warmup):
         "tflops_host": flops * t["steps"] / t["host_s"] / 1e12,
         "tflops_event": flops * t["steps"] / t["event_s"] / 1e12,
         "operands": (a, bt),
+        "vendor": {"what": "torch.matmul (hipBLASLt) on the same operands, timed the same way right after",
+                   "us_per_launch": t_vendor["us_per_launch"], "median_us": t_vendor["median_us"], "min_us": t_vendor["min_us"]},
         "clock": {"sustained_clock_ghz": clock_ghz, "mfma_busy_in_main_loop": busy,
                   "main_loop_us_mean": float(ns.mean() / 1e3), "main_loop_us_max": float(ns.max() / 1e3),
                   "main_loop_us_min": float(ns.min() / 1e3),
@@ -463,6 +467,37 @@ def sweep_gemm_shapes(torch, ops, capi):
           f"{sum(r > 1.05 for r in ratios)} above 1.05, {sum(r < 0.95 for r in ratios)} below 0.95")
 
 
+def sample_gemm_shapes(torch, ops, capi):
+    """A few products that do not fill the chip with 256 x 256 tiles, ragged ones and ones the chunk loads cannot fetch,
+    next to torch.matmul on the same operands: microseconds, the better of two runs of 40 launches each side."""
+    def timed(fn, iters=40, warm=10):
+        for _ in range(warm):
+            fn()
+        torch.cuda.synchronize()
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(iters):
+            fn()
+        stop.record()
+        torch.cuda.synchronize()
+        return start.elapsed_time(stop) / iters * 1e3
+
+    out = []
+    for m, n, k, layout in [(2048, 2048, 2048, "col"), (512, 6144, 4096, "col"), (1024, 4096, 4096, "col"), (2048, 4096, 4096, "col"),
+                            (4096, 4096, 4096, "row"), (4000, 4000, 4096, "col"), (4096, 4100, 4096, "row")]:
+        a = (torch.rand(m, k, device="cuda") * 2 - 1).half()
+        b = (torch.rand(n, k, device="cuda") * 2 - 1).half() if layout == "col" else (torch.rand(k, n, device="cuda") * 2 - 1).half()
+        c = torch.empty(m, n, device="cuda", dtype=torch.half)
+        flag = capi.B_COL_MAJOR if layout == "col" else capi.B_ROW_MAJOR
+        mine = lambda: ops.tensor_mm(a, b, out=c, b_layout=flag)
+        theirs = lambda: torch.matmul(a, b.t() if layout == "col" else b, out=c)
+        t_mine, t_theirs = timed(mine), timed(theirs)
+        t_mine, t_theirs = min(t_mine, timed(mine)), min(t_theirs, timed(theirs))
+        out.append({"m": m, "n": n, "k": k, "b_stored": "[N, K]" if layout == "col" else "[K, N]",
+                    "us": round(t_mine, 1), "torch_matmul_us": round(t_theirs, 1)})
+    return out
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -541,7 +576,9 @@ def main():
                             **traffic_fields("gemm_f16"), **timing_fields(t),
                             "algorithmic_flops": gemm["flops"], "min_bytes": 3 * 4096 * 4096 * 2,
                             **clock, "peak_at_sustained_clock": peak_at_clock,
-                            "frac_at_sustained_clock": gemm["tflops_event"] / peak_at_clock}
+                            "frac_at_sustained_clock": gemm["tflops_event"] / peak_at_clock,
+                            "vendor_library": gemm["vendor"]}
+        line["gemm_f16_other_shapes"] = sample_gemm_shapes(torch, ops, capi)
         if args.cpu_seconds > 0:
             import oracle
             a_dev, bt_dev = gemm["operands"]
