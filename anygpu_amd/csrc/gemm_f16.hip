@@ -488,13 +488,13 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
 		// The four-wave kernels where they apply and come out cheaper than the plan so far: their smaller tiles cost
 		// about half per slab of what the eight-wave tiles of the same size do (2048^3: 26 -> 16 us, vendor 22;
 		// 2048 x 4096 x 4096: 60 -> 44 us, vendor 55 - 60; 512 x 6144 x 4096: 43 -> 24 us, vendor 29 - 32).
-		if (whole_tiles && b_layout == ANYGPU_B_COL_MAJOR)
+		if (whole_tiles)
 		{
 			const FourWavePlan four = plan_four_wave(M, N, K, batch, cus, planes_ok ? plane_room : 0);
 			if (four.kind >= 0 && four.us < plan_us)
 			{
 				if (four.kind == 0)
-					return launch_gemm_f16_ring(a, b, c, M, N, K, lda, ldb, ldc, stride_a, stride_b, stride_c, batch, stream);
+					return launch_gemm_f16_ring(a, b, c, M, N, K, lda, ldb, ldc, stride_a, stride_b, stride_c, batch, stream, nullptr, b_layout);
 				float* planes = nullptr;
 				int64_t ranges = four.splits, k_split = 0;
 				if (ranges > 1)
@@ -507,11 +507,12 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
 					const hipError_t ws_err = band::workspace_acquire(stream, &planes);
 					if (ws_err != hipSuccess) return ws_err;
 				}
-				const int64_t sa = ranges > 1 ? k_split : stride_a, sb = ranges > 1 ? k_split : stride_b;
+				const int64_t sa = ranges > 1 ? k_split : stride_a;
+				const int64_t sb = ranges > 1 ? (b_layout == ANYGPU_B_COL_MAJOR ? k_split : k_split * ldb) : stride_b;
 				const int64_t count = ranges > 1 ? ranges : batch;
 				const hipError_t err = four.kind == 1
-					? launch_gemm_f16_ring3<8, 4>(a, b, c, M, N, K, lda, ldb, ldc, sa, sb, stride_c, count, stream, planes, k_split)
-					: launch_gemm_f16_ring3<4, 4>(a, b, c, M, N, K, lda, ldb, ldc, sa, sb, stride_c, count, stream, planes, k_split);
+					? launch_gemm_f16_ring3<8, 4>(a, b, c, M, N, K, lda, ldb, ldc, sa, sb, stride_c, count, stream, planes, k_split, nullptr, 0.0f, b_layout)
+					: launch_gemm_f16_ring3<4, 4>(a, b, c, M, N, K, lda, ldb, ldc, sa, sb, stride_c, count, stream, planes, k_split, nullptr, 0.0f, b_layout);
 				if (err != hipSuccess || ranges <= 1) return err;
 				const int64_t items = M * (N / 8);
 				gemm_f16_split_merge_kernel<<<dim3((unsigned)((items + 255) / 256)), dim3(256), 0, stream>>>(planes, c, M, N, ldc, (int)ranges);

@@ -33,7 +33,9 @@ struct GemmRing3Cfg
 // EPI: kEpiNone, kEpiBias (+ bias[n]) or kEpiSoftcap (ep_param * tanh(sum / ep_param)), applied to the fp32 sums (not SPLIT);
 // or kEpiGeluMul: the tile is BN / 2 output columns wide and its B unit holds, for every wave column, gate rows (from B) in
 // front of up rows (from `bias`, which then is the second weight matrix), as in gemm_f16_nt_ring_kernel.
-template <int TM, int TN, bool RAGGED, bool SPLIT, int EPI = kEpiNone>
+// B_KN: B stored [K, N] (N a multiple of 8): a B unit of 64 k rows x BN n, filled four rows per load, fragments by
+// transposing reads (gemm_f16_ring_loop_8x4kn.inc, _4x4kn.inc); not with kEpiGeluMul.
+template <int TM, int TN, bool RAGGED, bool SPLIT, int EPI = kEpiNone, bool B_KN = false>
 __global__ __launch_bounds__(256) void gemm_f16_nt_ring3_kernel(
 	const half_t* __restrict__ A, const half_t* __restrict__ B, half_t* __restrict__ C,
 	int K, int64_t lda, int64_t ldb, int64_t ldc, int tiles_m, int tiles_n,
@@ -41,6 +43,8 @@ __global__ __launch_bounds__(256) void gemm_f16_nt_ring3_kernel(
 	const half_t* __restrict__ bias = nullptr, float ep_param = 0.0f)
 {
 	static_assert(!SPLIT || EPI == kEpiNone, "the planes hold raw sums");
+	static_assert(!B_KN || EPI != kEpiGeluMul, "two weight matrices: k-contiguous only");
+	static_assert(TN == 4, "a [K, N] unit row of 256 bytes: 16 chunks, four k rows per load");
 	using Cfg = GemmRing3Cfg<TM, TN>;
 	extern __shared__ __align__(1024) char lds[];
 	if constexpr (SPLIT)
@@ -93,11 +97,22 @@ __global__ __launch_bounds__(256) void gemm_f16_nt_ring3_kernel(
 		const int row = 8 * (Cfg::kLoadsB * wave + q) + ld_row;                  // in the unit
 		int64_t b_row = n0 + b_unit_row + 8 * q + ld_row;                        // in the matrix
 		if constexpr (RAGGED) b_row = b_row < N - 1 ? b_row : N - 1;
-		table[64 * (8 + q)] = (unsigned)(((b_row - b_first) * ldb + ((ld_pos ^ ((row >> 1) & 7)) << 3)) * 2);
+		if constexpr (B_KN)
+		{
+			// one instruction fills 4 k rows of 256 bytes: lane -> row lane / 16, position lane % 16, and the chunk at
+			// position p of row k is chunk p ^ kn_row_swizzle(k); instruction q covers rows 16 wave + 4 q .. + 3
+			const int k_wave = 4 * q + (lane >> 4);
+			int64_t col = (int64_t)(((lane & 15) ^ kn_row_swizzle(16 * wave + k_wave)) << 3);
+			if constexpr (RAGGED)
+				if (n0 + col + 8 > N) col = N - 8 - n0;
+			table[64 * (8 + q)] = (unsigned)((k_wave * ldb + col) * 2);
+		}
+		else
+			table[64 * (8 + q)] = (unsigned)(((b_row - b_first) * ldb + ((ld_pos ^ ((row >> 1) & 7)) << 3)) * 2);
 	}
 	const unsigned table_addr = lds0 + 3 * Cfg::kStageBytes + (wave * (16 * 64) + lane) * 4;
 	const uintptr_t a_wave = reinterpret_cast<uintptr_t>(A + a_first * lda);
-	const uintptr_t b_wave = reinterpret_cast<uintptr_t>(b_of_wave + b_first * ldb);
+	const uintptr_t b_wave = reinterpret_cast<uintptr_t>(B_KN ? B + (int64_t)(16 * wave) * ldb + n0 : b_of_wave + b_first * ldb);
 	const unsigned share_a = wave * (Cfg::kLoadsA * 1024);                       // the wave's rows inside a stage
 	const unsigned share_b = Cfg::BM * 128 + wave * (Cfg::kLoadsB * 1024);
 	const int slabs = K / 64;
@@ -107,7 +122,14 @@ __global__ __launch_bounds__(256) void gemm_f16_nt_ring3_kernel(
 	const unsigned frag_row = lane & 15;
 	const unsigned frag_chunk = (lane >> 4) ^ ((frag_row >> 1) & 7);
 	const unsigned a_addr = (wm * Cfg::kWaveM + frag_row) * 128 + frag_chunk * 16;
-	const unsigned b_addr = Cfg::BM * 128 + (wn * Cfg::kWaveN + frag_row) * 128 + frag_chunk * 16;
+	// B stored [K, N]: lane r of a 16-lane group points a transposing read at k row 8 g + r / 4 (g: the lane's k group),
+	// columns 4 (r % 4) .. + 3 of the MFMA tile; column tile j of wave column wn lies at chunk pair (4 wn + j) ^ (row
+	// swizzle / 2), which the assembly block adds per tile from `b_swizzle`
+	const unsigned kn_k = 8 * (lane >> 4) + (frag_row >> 2);
+	const unsigned b_addr = B_KN ? Cfg::BM * 128 + kn_k * 256 + ((frag_row & 3) >> 1) * 16 + 8 * (frag_row & 1)
+	                             : Cfg::BM * 128 + (wn * Cfg::kWaveN + frag_row) * 128 + frag_chunk * 16;
+	[[maybe_unused]] const unsigned b_swizzle = (unsigned)((kn_row_swizzle((int)kn_k) >> 1) ^ (wn << 2)) << 5;
+	[[maybe_unused]] const unsigned b_step = (unsigned)(128 * ldb);      // bytes from one [K, N] slab to the next
 
 	// The accumulators leave the block as vectors of 32 registers pinned to a[0 : 4 TM TN): MFMA tile (i, j) in registers
 	// 4 (TN i + j) .. + 3.
@@ -119,6 +141,7 @@ __global__ __launch_bounds__(256) void gemm_f16_nt_ring3_kernel(
 	[bbaselo] "s"((unsigned)b_wave), [bbasehi] "s"((unsigned)(b_wave >> 32)), \
 	[lds0] "s"(lds0), [ldsa] "s"(share_a), [ldsb] "s"(share_b), [slabs] "s"(slabs)
 #define ANYGPU_RING3_CLOBBERS \
+	"v80", "v81", "v82", "v83", "v84", "v85", "v86", "v87", "v88", "v89", "v90", "v91", "v92", "v93", "v94", "v95", \
 	"v96", "v97", "v98", "v99", "v100", "v101", "v102", "v103", "v104", "v105", "v106", "v107", "v108", "v109", \
 	"v110", "v111", "v112", "v113", "v114", "v115", "v116", "v117", "v118", "v119", "v120", "v121", "v122", "v123", \
 	"v124", "v125", "v126", "v127", "v128", "v129", "v130", "v131", "v132", "v133", "v134", "v135", "v136", "v137", \
@@ -131,8 +154,20 @@ __global__ __launch_bounds__(256) void gemm_f16_nt_ring3_kernel(
 	"v222", "v223", "v224", "v225", "v226", "v227", "v228", "v229", "v230", "v231", "v232", "v233", "v234", "v235", \
 	"v236", "v237", "v238", "v239", "v240", "v241", "v242", "v243", "v244", "v245", "v246", "v247", "v248", "v249", \
 	"v250", "v251", "v252", "v253", "v254", "v255", "s60", "s61", "s62", "s63", "s64", "s65", "s66", "s67", "s68", \
-	"s69", "s70", "s71", "s72", "s73", "scc", "m0", "memory"
-	if constexpr (TM == 8)
+	"s69", "s70", "s71", "s72", "s73", "s74", "scc", "m0", "memory"
+	if constexpr (TM == 8 && B_KN)
+		asm volatile(
+#include "gemm_f16_ring_loop_8x4kn.inc"
+			: "={a[0:31]}"(r0), "={a[32:63]}"(r1), "={a[64:95]}"(r2), "={a[96:127]}"(r3)
+			: ANYGPU_RING3_INPUTS, [bsx] "v"(b_swizzle), [bstep] "s"(b_step)
+			: ANYGPU_RING3_CLOBBERS);
+	else if constexpr (B_KN)
+		asm volatile(
+#include "gemm_f16_ring_loop_4x4kn.inc"
+			: "={a[0:31]}"(r0), "={a[32:63]}"(r1)
+			: ANYGPU_RING3_INPUTS, [bsx] "v"(b_swizzle), [bstep] "s"(b_step)
+			: ANYGPU_RING3_CLOBBERS);
+	else if constexpr (TM == 8)
 		asm volatile(
 #include "gemm_f16_ring_loop_8x4.inc"
 			: "={a[0:31]}"(r0), "={a[32:63]}"(r1), "={a[64:95]}"(r2), "={a[96:127]}"(r3)
@@ -183,9 +218,11 @@ template <int TM, int TN, int EPI = kEpiNone>
 inline hipError_t launch_gemm_f16_ring3(const half_t* A, const half_t* B, half_t* C, int64_t M, int64_t N, int64_t K,
                                         int64_t lda, int64_t ldb, int64_t ldc,
                                         int64_t stride_a, int64_t stride_b, int64_t stride_c, int64_t batch, hipStream_t stream,
-                                        float* planes = nullptr, int64_t k_split = 0, const half_t* bias = nullptr, float ep_param = 0.0f)
+                                        float* planes = nullptr, int64_t k_split = 0, const half_t* bias = nullptr, float ep_param = 0.0f,
+                                        int b_layout = ANYGPU_B_COL_MAJOR)
 {
 	using Cfg = GemmRing3Cfg<TM, TN>;
+	const bool kn = b_layout == ANYGPU_B_ROW_MAJOR;
 	const bool c_aligned = reinterpret_cast<uintptr_t>(C) % 16 == 0 && ldc % 8 == 0 && stride_c % 8 == 0;
 	constexpr int kOutN = EPI == kEpiGeluMul ? Cfg::BN / 2 : Cfg::BN;       // output columns of a tile
 	const bool ragged = M % Cfg::BM != 0 || N % kOutN != 0 || !c_aligned;
@@ -194,20 +231,24 @@ inline hipError_t launch_gemm_f16_ring3(const half_t* A, const half_t* B, half_t
 	if constexpr (EPI == kEpiNone)
 	{
 		if (which == 2) kernel = gemm_f16_nt_ring3_kernel<TM, TN, true, true, kEpiNone>;
+		if (kn)
+			kernel = which == 2 ? gemm_f16_nt_ring3_kernel<TM, TN, true, true, kEpiNone, true>
+			       : which == 1 ? gemm_f16_nt_ring3_kernel<TM, TN, true, false, kEpiNone, true> : gemm_f16_nt_ring3_kernel<TM, TN, false, false, kEpiNone, true>;
 	}
-	else if (which == 2) return hipErrorInvalidValue;
+	else if (which == 2 || kn) return hipErrorInvalidValue;
 	// More than 64 KB of dynamic LDS has to be granted per function and per device, once.
-	static std::atomic<uint64_t> configured_devices[3];
+	static std::atomic<uint64_t> configured_devices[6];
 	(void)hipGetLastError();
 	int device = 0;
 	hipError_t e = hipGetDevice(&device);
 	if (e != hipSuccess) return e;
 	const uint64_t bit = 1ull << (device & 63);
-	if ((configured_devices[which].load(std::memory_order_relaxed) & bit) == 0)
+	const int slot = which + 3 * kn;
+	if ((configured_devices[slot].load(std::memory_order_relaxed) & bit) == 0)
 	{
 		e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::kLdsBytes);
 		if (e != hipSuccess) return e;
-		configured_devices[which].fetch_or(bit, std::memory_order_relaxed);
+		configured_devices[slot].fetch_or(bit, std::memory_order_relaxed);
 	}
 	const int tiles_m = (int)((M + Cfg::BM - 1) / Cfg::BM), tiles_n = (int)((N + kOutN - 1) / kOutN);
 	kernel<<<dim3((unsigned)(tiles_m * tiles_n), (unsigned)batch), dim3(256), Cfg::kLdsBytes, stream>>>(

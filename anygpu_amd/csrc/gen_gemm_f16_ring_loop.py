@@ -50,7 +50,7 @@ v112 / v113 and v114 / v115 the fragment addresses of the first and of the secon
 addresses inside a stage with bit 6 flipped.  Operands: vtab, aaddr, baddr (inside a stage), abaselo .. bbasehi, slabs as
 above, lds0 (SGPR: LDS address of stage 0), ldsa / ldsb (SGPR: offset of the wave's share of the A / B unit in a stage).
 
-Usage: gen_gemm_f16_ring_loop.py OUTPUT [kn | 8x4 | 4x4]
+Usage: gen_gemm_f16_ring_loop.py OUTPUT [kn | 8x4 | 4x4 | 8x4kn | 4x4kn]
 """
 import sys
 
@@ -223,8 +223,10 @@ def generate(kn):
     return lines
 
 
-def generate_three_stages(tm, tn):
-    """the block for a patch of tm x tn MFMA tiles per wave (tile 32 tm x 32 tn), three LDS stages"""
+def generate_three_stages(tm, tn, kn=False):
+    """the block for a patch of tm x tn MFMA tiles per wave (tile 32 tm x 32 tn), three LDS stages; kn: B stored [K, N]
+    (a B unit of 64 k rows x 32 tn n, fragments by transposing reads through one address register per column tile, as in
+    the kn form of the 256 x 256 tile; s64 and s74 hold the halves of the slab's byte offset)"""
     lines = []
     bm, bn = 32 * tm, 32 * tn
     stage = (bm + bn) * 128
@@ -249,10 +251,15 @@ def generate_three_stages(tm, tn):
 
     def load_set(stage_reg, add):
         """where the loads of slab min(t + add, last) go and come from: entries of one or two instructions"""
-        return [f"s_add_u32 {S_LDA}, {stage_reg}, %[ldsa]", f"s_add_u32 {S_LDB}, {stage_reg}, %[ldsb]",
-                f"s_add_u32 {S_TMP}, {S_T}, {add}", f"s_min_u32 {S_TMP}, {S_TMP}, {S_LAST}", f"s_lshl_b32 {S_TMP}, {S_TMP}, 7",
-                ("s_add_u32 s68, %[abaselo], " + S_TMP, "s_addc_u32 s69, %[abasehi], 0"),
-                ("s_add_u32 s70, %[bbaselo], " + S_TMP, "s_addc_u32 s71, %[bbasehi], 0")]
+        out = [f"s_add_u32 {S_LDA}, {stage_reg}, %[ldsa]", f"s_add_u32 {S_LDB}, {stage_reg}, %[ldsb]",
+               f"s_add_u32 {S_TMP}, {S_T}, {add}", f"s_min_u32 {S_TMP}, {S_TMP}, {S_LAST}"]
+        if kn:
+            out += ["s_mul_hi_u32 s64, " + S_TMP + ", %[bstep]", "s_mul_i32 s74, " + S_TMP + ", %[bstep]",
+                    ("s_add_u32 s70, %[bbaselo], s74", "s_addc_u32 s71, %[bbasehi], s64")]
+        out += [f"s_lshl_b32 {S_TMP}, {S_TMP}, 7", ("s_add_u32 s68, %[abaselo], " + S_TMP, "s_addc_u32 s69, %[abasehi], 0")]
+        if not kn:
+            out.append(("s_add_u32 s70, %[bbaselo], " + S_TMP, "s_addc_u32 s71, %[bbasehi], 0"))
+        return out
 
     def loads(which):
         out = []
@@ -262,10 +269,19 @@ def generate_three_stages(tm, tn):
                         f"global_load_lds_dwordx4 v{v}, {A_CUR if operand == 'a' else B_CUR}"))
         return out
 
-    def reads(buf, va, vb):
-        out = [f"ds_read_b128 {bfrag(buf, q)}, {vb} offset:{q * 2048}" for q in range(tn)]
+    row_kn = 64 * tn                            # bytes of a [k][n] unit row
+
+    def reads(buf, va, vb, second_half=False):
+        if kn:
+            off = 32 * row_kn if second_half else 0
+            out = [f"ds_read_b64_tr_b16 {bfrag(buf, q // 2, q % 2)}, v{V_BCUR + q // 2} offset:{off + 4 * row_kn * (q % 2)}" for q in range(2 * tn)]
+        else:
+            out = [f"ds_read_b128 {bfrag(buf, q)}, {vb} offset:{q * 2048}" for q in range(tn)]
         out += [f"ds_read_b128 {afrag(buf, q)}, {va} offset:{q * 2048}" for q in range(tm)]
         return out
+
+    def b_stage_addresses(stage_reg):
+        return [f"v_add_u32 v{V_BCUR + j}, {stage_reg}, v{V_BUNIT + j}" for j in range(tn)]
 
     # ---- prologue: slabs 0 and 1 and the first half of the loads of slab 2, fragments of the first step
     emit(f"s_mov_b32 {S_T}, 0", "prologue")
@@ -278,7 +294,12 @@ def generate_three_stages(tm, tn):
         emit(f"ds_read_b32 v{104 + q}, %[vtab] offset:{256 * (8 + q)}")
     emit("s_waitcnt lgkmcnt(0)")
     emit(f"v_xor_b32 {V_A64}, 64, %[aaddr]")
-    emit(f"v_xor_b32 {V_B64}, 64, %[baddr]")
+    if kn:
+        for j in range(tn):
+            emit(f"v_xor_b32 v{V_BUNIT + j}, {32 * j}, %[bsx]")
+            emit(f"v_add_u32 v{V_BUNIT + j}, %[baddr], v{V_BUNIT + j}")
+    else:
+        emit(f"v_xor_b32 {V_B64}, 64, %[baddr]")
     for slab in range(3):
         for ins in load_set(S[slab], slab):
             emit(ins)
@@ -291,11 +312,16 @@ def generate_three_stages(tm, tn):
     emit(f"s_waitcnt vmcnt({la + lb + half})", "slab 0 has landed")
     emit("s_barrier")
     emit(f"v_add_u32 {V_RA1}, {S[0]}, %[aaddr]")
-    emit(f"v_add_u32 {V_RB1}, {S[0]}, %[baddr]")
+    if kn:
+        for ins in b_stage_addresses(S[0]):
+            emit(ins)
+    else:
+        emit(f"v_add_u32 {V_RB1}, {S[0]}, %[baddr]")
     for ins in reads(0, V_RA1, V_RB1):
         emit(ins)
     emit(f"v_add_u32 {V_RA0}, {S[0]}, {V_A64}")
-    emit(f"v_add_u32 {V_RB0}, {S[0]}, {V_B64}")
+    if not kn:
+        emit(f"v_add_u32 {V_RB0}, {S[0]}, {V_B64}")
     emit("s_waitcnt lgkmcnt(0)")
 
     # ---- main loop: one slab per trip
@@ -304,9 +330,9 @@ def generate_three_stages(tm, tn):
         gaps = [[] for _ in range(mfmas)]
 
         def place(entry, earliest):
-            """behind the first MFMA from `earliest` on that has fewer than two instructions behind it (three if none has)"""
+            """behind the first MFMA from `earliest` on that has fewer than two instructions behind it (three, four if none has)"""
             n = len(entry) if isinstance(entry, tuple) else 1
-            for cap in (2, 3):
+            for cap in (2, 3, 4):
                 for g in range(earliest, mfmas):
                     if sum(len(x) if isinstance(x, tuple) else 1 for x in gaps[g]) + n <= cap:
                         gaps[g].append(entry)
@@ -315,8 +341,10 @@ def generate_three_stages(tm, tn):
 
         buf = step
         # fragments of the next step: step 0 reads the second half of slab t, step 1 the first half of slab t + 1
-        for q, ins in enumerate(reads(buf ^ 1, V_RA0 if step == 0 else V_RA1, V_RB0 if step == 0 else V_RB1)):
-            gaps[2 * q].append(ins)
+        step_reads = reads(buf ^ 1, V_RA0 if step == 0 else V_RA1, V_RB0 if step == 0 else V_RB1, step == 0)
+        spacing = 2 if 2 * (len(step_reads) - 1) < mfmas else 1
+        for q, ins in enumerate(step_reads):
+            gaps[spacing * q].append(ins)
         # step 0: the second half of the loads of slab t + 2; step 1: the first half of the loads of slab t + 3
         every = max(2, (mfmas - 10) // half)
         last_load = 0
@@ -328,15 +356,22 @@ def generate_three_stages(tm, tn):
             # fragment addresses of step 1; once this step's loads are out, where the loads of slab t + 3 go (the stage of
             # slab t) and come from
             g = place(f"v_add_u32 {V_RA1}, {S[1]}, %[aaddr]", 1)
-            g = place(f"v_add_u32 {V_RB1}, {S[1]}, %[baddr]", g)
+            if not kn:
+                g = place(f"v_add_u32 {V_RB1}, {S[1]}, %[baddr]", g)
             g = last_load + 1
             for ins in load_set(S[0], 3):
                 g = place(ins, g)
+            if kn:
+                # (the B addresses serve this step's reads first; the new ones stay for the first step of the next trip,
+                # which reads the second half of the same stage)
+                g = spacing * (2 * tn - 1) + 1
+                for ins in b_stage_addresses(S[1]):
+                    g = place(ins, g)
         else:
             # the stages move on by one slab, t advances; fragment addresses of the next trip's first step
             g = 1
             for ins in [f"s_mov_b32 {S_ROT}, {S[0]}", f"s_mov_b32 {S[0]}, {S[1]}", f"s_mov_b32 {S[1]}, {S[2]}", f"s_mov_b32 {S[2]}, {S_ROT}",
-                        f"s_add_u32 {S_T}, {S_T}, 1", f"v_add_u32 {V_RA0}, {S[0]}, {V_A64}", f"v_add_u32 {V_RB0}, {S[0]}, {V_B64}"]:
+                        f"s_add_u32 {S_T}, {S_T}, 1", f"v_add_u32 {V_RA0}, {S[0]}, {V_A64}"] + ([] if kn else [f"v_add_u32 {V_RB0}, {S[0]}, {V_B64}"]):
                 g = place(ins, g + 1)
         if step == 1:
             emit(f"s_waitcnt vmcnt({la + lb})", "mid-slab: slab t + 1 has landed (the loads of slab t + 2 may be in flight)")
@@ -363,7 +398,9 @@ if __name__ == "__main__":
     form = sys.argv[2] if len(sys.argv) > 2 else ""
     with open(sys.argv[1], "w") as f:
         f.write("// Written by gen_gemm_f16_ring_loop.py (the register plan and the schedule are explained there): do not edit.\n")
-        for s, c in (generate_three_stages(*(int(x) for x in form.split("x"))) if "x" in form else generate(form == "kn")):
+        kn = form.endswith("kn")
+        patch = form[:-2] if kn else form
+        for s, c in (generate_three_stages(*(int(x) for x in patch.split("x")), kn) if "x" in patch else generate(kn)):
             if c:
                 f.write(f"// {c}\n")
             f.write(f'"{s}\\n\\t"\n')

@@ -798,6 +798,24 @@ def test_mm_f32_operands_at_odd_addresses_are_copied(ops, layout, m, n, k, a_off
     assert np.all(got[m:, :] == -7) and np.all(got[:, n:] == -7)
 
 
+@pytest.mark.parametrize("m,n,k,pad,span", [(2048, 2048, 192, 0, 2), (1000, 2000, 128, 8, 2), (2048, 4096, 64, 0, 2), (1100, 4000, 320, 0, 2),
+                                            (520, 6152, 256, 16, 2), (128, 128, 64, 0, 2), (512, 2304, 9216, 0, 1), (300, 1000, 4096, 72, 1),
+                                            (2048, 1024, 2048, 0, 1)])
+def test_mm_f16_smaller_four_wave_tiles_reference_layout_exact(ops, m, n, k, pad, span):
+    # the same products with B stored [K, N]: units of 64 k rows x 128 n, transposing reads, a row pitch that is not the
+    # row length, last tiles of 8 columns, cuts along K that step down the rows of B
+    import torch
+    from anygpu_amd import capi
+    a = synth.integers(m + k + 10, (m, k), -span, span).astype(np.float16)
+    b = synth.integers(n + k + 11, (k, n), -span, span).astype(np.float16)
+    b_dev = torch.full((k, n + pad), 7.0, dtype=torch.float16, device="cuda")
+    b_dev[:, :n] = dev(b)
+    got = host(ops.tensor_mm(dev(a), b_dev[:, :n], b_layout=capi.B_ROW_MAJOR)).astype(np.int64)
+    want = a.astype(np.int64) @ b.astype(np.int64)
+    assert np.abs(want).max() < 2048
+    assert np.array_equal(got, want)
+
+
 def test_mm_f16_whole_256_tiles_batched(ops, oracle):
     # four products of 2048 x 2048 x 128 in one launch: 256 tiles of 256 x 256, the four-wave kernel over blockIdx.y
     from anygpu_amd import capi
