@@ -85,4 +85,14 @@ __device__ __forceinline__ float tanh_f32(float x)
 	return fabsf(x) < 0.0625f ? small : big;
 }
 
+// tanh for results that are rounded to fp16 (half an ulp: 5e-4 relative): the closed form, whose absolute error of about
+// 1.5e-7 is 4e-5 relative at |x| = 2^-8, and below that x itself (tanh(x) = x to 5e-6 relative there).  Two
+// transcendentals and five other instructions instead of eleven others.
+__device__ __forceinline__ float tanh_for_half(float x)
+{
+	const float e = fast_exp2(x * (2.0f * kLog2e));
+	const float big = fmaf(fast_rcp(1.0f + e), -2.0f, 1.0f);
+	return fabsf(x) < 0.00390625f ? x : big;
+}
+
 }  // namespace anygpu

@@ -264,9 +264,9 @@ __device__ __forceinline__ void store_patch_via_lds(
 				for (int e = 0; e < 4; ++e)
 				{
 					if constexpr (EPI == kEpiGeluMul)
-						out[e] = (half_t)finish_sum<EPI>(acc[i][j][4 * g + e], acc[i][j + TN][4 * g + e], 0.0f, ep_param);
+						out[e] = (half_t)finish_sum<EPI, true>(acc[i][j][4 * g + e], acc[i][j + TN][4 * g + e], 0.0f, ep_param);
 					else if constexpr (EPI == kEpiSoftcap)
-						out[e] = (half_t)finish_sum<EPI>(acc[i][j][4 * g + e], 0.0f, 0.0f, ep_param);
+						out[e] = (half_t)finish_sum<EPI, true>(acc[i][j][4 * g + e], 0.0f, 0.0f, ep_param);
 					else if constexpr (EPI == kEpiBias)
 						out[e] = (half_t)(acc[i][j][4 * g + e] + bias_of[j][g][e]);
 					else
