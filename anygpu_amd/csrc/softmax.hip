@@ -261,7 +261,7 @@ __global__ __launch_bounds__(256) void softmax_rows_f16_window_kernel(const Soft
 {
 	constexpr int EPV = 8;
 	const int lane = threadIdx.x & (kWaveSize - 1);
-	int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+	const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
 	if (row >= a.rows) return;  // uniform over the wave
 	const RowSpan span = row_span(a, row);
 	const half8_t* __restrict__ xr = reinterpret_cast<const half8_t*>(static_cast<const half_t*>(a.x) + row * a.xs);
