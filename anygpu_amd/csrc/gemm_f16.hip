@@ -1,11 +1,13 @@
-// fp16 x fp16 -> fp32-accumulate -> fp16 GEMM for gfx950 on the MFMA units.
+// fp16 x fp16 -> fp32-accumulate -> fp16 GEMM for gfx950 on the MFMA units: the launchers, their plans, the merge and
+// edge kernels.
 //
-// Tile kernel (gemm_f16_tile.hpp): 256 x 256 or 128 x 128 tiles of C, direct global -> LDS loads,
-// double-buffered LDS, software-pipelined MFMAs; B either [N, K] (k-contiguous like A) or [K, N]
-// (the reference layout, transposed on the way out of LDS).
-//
-// Edge kernel: 64 x 64 tiles, guarded scalar loads and stores, either B layout, any
-// shape, stride and alignment.
+// Four-wave kernels (gemm_f16_ring.hpp: 256 x 256 tiles; gemm_f16_ring3.hpp: 256 x 128 and 128 x 128): one wave per SIMD,
+// main loops in generated assembly, whole 64-deep slabs, any M and N, B either [N, K] (k-contiguous like A) or [K, N]
+// (the reference layout, transposed on the way out of LDS); the smaller two also cut along K.
+// Eight-wave and 64 x 64 tile kernels (gemm_f16_tile.hpp): everything the above do not take (a K tail, few rows).
+// Operands the 16-byte chunk loads cannot fetch are copied aligned into the stream's workspace first (gemm_repack.hip);
+// where that is not possible or not worth it, the edge kernel: 64 x 64 tiles, guarded scalar loads and stores, either
+// B layout, any shape, stride and alignment.
 #include <algorithm>
 
 #include "device_utils.hpp"

@@ -7,13 +7,16 @@
  *     outputs only written.  One kind of scratch exists: the GEMM entry points cut some products
  *     along K (few tiles and a deep K, few rows against a weight matrix) and pass the partial
  *     sums of such a launch through a workspace that belongs to the (device, stream) pair of the
- *     call.  Who owns it is the caller's choice, see anygpu_set_workspace: by default the library
+ *     call; the same workspace takes the aligned copy of a GEMM operand that cannot be fetched
+ *     in 16-byte pieces where it lies (an odd start or row pitch, a K or N that is no multiple
+ *     of 8) and the partial results of the key-split blocks of the fused attention.  Who owns
+ *     it is the caller's choice, see anygpu_set_workspace: by default the library
  *     allocates ANYGPU_WORKSPACE_BYTES (64 MiB) the first time an eager launch on a stream cuts a
  *     product and keeps them until anygpu_release_workspaces or the end of the process; a caller
  *     that hands in its own workspace for a stream makes the library allocate nothing there.
  *     While a stream is being captured into a graph only a caller's workspace is used, never the
- *     library's: without one every captured product runs uncut (a valid result, summed in
- *     another order than the cut one).  Nothing else allocates;
+ *     library's: without one every captured product runs uncut and uncopied (a valid result,
+ *     summed in another order than the cut one).  Nothing else allocates;
  *   - sizes, strides and leading dimensions are int64_t counts of ELEMENTS;
  *   - `stream` is a hipStream_t passed as void* (NULL = the null stream, which is what the
  *     reference uses for every launch); calls are asynchronous with respect to the host;
@@ -86,8 +89,8 @@ int anygpu_release_workspaces(void);
  * path of srcs/ops/mm_ops.hpp:62-65) and the cu_fast_mm_f16_* ladder
  * (srcs/kernels/cuda/fast_mm.cuh:70-98).  A is row-major with leading dimension lda >= K,
  * C row-major with ldc >= N, B as selected by b_layout (ldb >= N for row-major, >= K for
- * column-major).  Any M, N, K >= 0 are accepted; M, N multiples of 256 and K a multiple of 64
- * with 16-byte aligned rows take the fastest kernel.
+ * column-major).  Any M, N, K >= 0 are accepted; K a multiple of 64 with 16-byte aligned operand
+ * rows takes the fastest kernels (whatever M, N and the alignment of C).
  */
 int anygpu_gemm_f16_f32acc(const void* A, const void* B, void* C,
                            int64_t M, int64_t N, int64_t K,
