@@ -215,6 +215,7 @@ struct FourWavePrices
 	static constexpr double kSlabFull[3] = {1.41, 0.77, 0.465};
 	static constexpr double kSlabHalf[3] = {1.0, 0.575, 0.36};
 	static constexpr double kLaunch[3] = {8.5, 5.5, 3.0};
+	static constexpr double kOperandBytesPerUs = 5.5e6;      // what HBM gives a launch that reads its operands once
 };
 
 struct FourWavePlan
@@ -244,7 +245,11 @@ static FourWavePlan plan_four_wave(int64_t M, int64_t N, int64_t K, int64_t batc
 			const double t = fill <= 0.5 ? 0.0 : (fill - 0.5) / 0.5;
 			const double per_slab = FourWavePrices::kSlabHalf[kind] + t * (FourWavePrices::kSlabFull[kind] - FourWavePrices::kSlabHalf[kind]);
 			const int64_t depth = (slabs + sp - 1) / sp;
-			double us = (double)rounds * (double)depth * per_slab + FourWavePrices::kLaunch[kind];
+			double us = (double)rounds * (double)depth * per_slab;
+			// (few rows against a large weight matrix: the launch cannot end before the operands have come in once)
+			const double stream_us = 2.0 * ((double)M + (double)N) * (double)K * (double)batch / FourWavePrices::kOperandBytesPerUs;
+			if (us < stream_us) us = stream_us;
+			us += FourWavePrices::kLaunch[kind];
 			if (sp > 1) us += TilePrices::kMergeLaunchUs + 8.0 * (double)sp * (double)M * (double)N / TilePrices::kPlaneBytesPerUs;
 			if (us < best.us)
 			{
