@@ -17,6 +17,7 @@
 #include "gemm_epilogue.hpp"
 #include "launch.hpp"
 #include "gemm_band.hpp"
+#include "gemm_f32_ring.hpp"
 #include "anygpu_hip.h"
 
 #include <type_traits>
@@ -338,6 +339,13 @@ static hipError_t launch_tiles_once(const float* A, const float* B, const float*
                                     int64_t stride_a, int64_t stride_b, int64_t stride_c, int64_t batch,
                                     float ep_param, int64_t k_split, hipStream_t stream, bool padded = false)
 {
+	// k-contiguous operands in whole 32-deep slabs, one product per tile: the four-wave kernel (gemm_f32_ring.hpp), which
+	// keeps the matrix cores busier than this file's kernel does around its barriers (2048^3: 131 -> see the header)
+	if constexpr (A_LAYOUT == ANYGPU_A_ROW_MAJOR && B_LAYOUT == ANYGPU_B_COL_MAJOR && BM == BN && EPI != kEpiGeluMul)
+	{
+		if (gemm_f32_ring_applies(A, B, M, N, K, lda, ldb, stride_a, stride_b, batch, k_split, BM))
+			return launch_gemm_f32_ring<BM / 64, EPI>(A, B, bias, C, M, N, K, lda, ldb, ldc, stride_a, stride_b, stride_c, batch, ep_param, k_split, stream);
+	}
 	const dim3 grid((unsigned)((N + BN - 1) / BN), (unsigned)((M + BM - 1) / BM), (unsigned)batch);
 	const bool aligned_in = (reinterpret_cast<uintptr_t>(A) % 16 == 0) && (reinterpret_cast<uintptr_t>(B) % 16 == 0) &&
 	                        (reinterpret_cast<uintptr_t>(B2) % 16 == 0) && (lda % 4 == 0) && (ldb % 4 == 0) &&
@@ -431,13 +439,17 @@ constexpr int64_t kSplitMax = 16;
 // the number of CUs is the device's (256 on an MI355X)
 static inline int64_t chip_cus() { return device_cu_count(); }
 
-static TilePlan plan_tiles(int tile, int64_t M, int64_t N, int64_t K, int64_t batch, bool may_split, size_t workspace_bytes)
+// four_wave: the product takes the kernels of gemm_f32_ring.hpp, which run at the matrix cores' pace at either tile size
+// (per 16 of K and round: 128 x 128 0.9 us, 2048^3 in 123 us; 64 x 64 0.225 us)
+static TilePlan plan_tiles(int tile, int64_t M, int64_t N, int64_t K, int64_t batch, bool may_split, size_t workspace_bytes,
+                           bool four_wave = false)
 {
-	const double slab_us = tile == 128 ? 1.0 : 0.36;
+	const double slab_us = four_wave ? (tile == 128 ? 0.9 : 0.225) : (tile == 128 ? 1.0 : 0.36);
 	const int64_t tiles = ((M + tile - 1) / tile) * ((N + tile - 1) / tile) * batch;
 	const int64_t slabs = (K + kBK - 1) / kBK;
-	const auto rounds_of = [tile](int64_t blocks) {
-		if (tile == 64 && blocks > 2 * chip_cus()) return (double)blocks / (double)chip_cus();
+	// (the four-wave kernels hold two small tiles per CU at most, each then at half pace: whole rounds at either size)
+	const auto rounds_of = [tile, four_wave](int64_t blocks) {
+		if (tile == 64 && !four_wave && blocks > 2 * chip_cus()) return (double)blocks / (double)chip_cus();
 		return (double)((blocks + chip_cus() - 1) / chip_cus());
 	};
 	TilePlan best{tile, 1, rounds_of(tiles) * (double)slabs * slab_us};
@@ -464,7 +476,7 @@ static hipError_t launch_tiles(const float* A, const float* B, const float* B2, 
 		if (splits > 1)
 		{
 			int64_t k_split = (K + splits - 1) / splits;
-			k_split = (k_split + kBK - 1) / kBK * kBK;
+			k_split = (k_split + 31) / 32 * 32;             // whole slabs of either kernel family
 			splits = (K + k_split - 1) / k_split;
 			if (splits > 1)
 			{
@@ -501,8 +513,10 @@ static hipError_t launch_layout(const float* A, const float* B, const float* B2,
 	// (what the stream's workspace holds bounds the cuts along K: the caller's, or the library's own for eager launches;
 	// a stream under capture without a caller's workspace has none and runs uncut)
 	const size_t ws_bytes = (may_split && batch == 1) ? band::workspace_capacity(stream) : 0;
-	const TilePlan big = plan_tiles(128, M, N, K, batch, may_split, ws_bytes);
-	const TilePlan small = plan_tiles(64, M, N, K, batch, may_split, ws_bytes);
+	const bool four_wave = A_LAYOUT == ANYGPU_A_ROW_MAJOR && B_LAYOUT == ANYGPU_B_COL_MAJOR && EPI != kEpiGeluMul &&
+	                       gemm_f32_ring_applies(A, B, M, N, K, lda, ldb, stride_a, stride_b, batch, 0, 64);
+	const TilePlan big = plan_tiles(128, M, N, K, batch, may_split, ws_bytes, four_wave);
+	const TilePlan small = plan_tiles(64, M, N, K, batch, may_split, ws_bytes, four_wave);
 	if constexpr (EPI != kEpiGeluMul)
 	{
 		// A product of big tiles that fills whole rounds and a bit, e.g. 576 tiles = 2.25 rounds, pays three rounds.  It
@@ -514,9 +528,9 @@ static hipError_t launch_layout(const float* A, const float* B, const float* B2,
 		if (batch == 1 && whole > 0 && head_cols > 0 && head_cols < tiles_n)
 		{
 			const int64_t n_head = head_cols * 128, n_tail = N - n_head;
-			const TilePlan head = plan_tiles(128, M, n_head, K, 1, false, 0);
-			const TilePlan tail_big = plan_tiles(128, M, n_tail, K, 1, true, ws_bytes);
-			const TilePlan tail_small = plan_tiles(64, M, n_tail, K, 1, true, ws_bytes);
+			const TilePlan head = plan_tiles(128, M, n_head, K, 1, false, 0, four_wave);
+			const TilePlan tail_big = plan_tiles(128, M, n_tail, K, 1, true, ws_bytes, four_wave);
+			const TilePlan tail_small = plan_tiles(64, M, n_tail, K, 1, true, ws_bytes, four_wave);
 			const TilePlan& tail = tail_big.cost <= tail_small.cost ? tail_big : tail_small;
 			const double best_whole = big.cost <= small.cost ? big.cost : small.cost;
 			if (head.cost + tail.cost + 3.0 < 0.96 * best_whole)
@@ -598,7 +612,11 @@ hipError_t launch_gemm_f32(const float* A, const float* B, const float* bias, fl
 #undef ANYGPU_F32_PADDED
 		}
 	}
-	if (batch == 1 && a_layout == ANYGPU_A_ROW_MAJOR && gemm_band_applies<float>(A, B, nullptr, C, M, N, K, lda, ldb, ldc, b_layout))
+	// From 48 rows on, k-contiguous weights in whole slabs go to the four-wave 64 x 64 tiles cut along K rather than to
+	// the band kernels (64 x 4096 -> 6144: 45 us as a band, 37 us in tiles; 16 rows of the same: 24 us against 32 us).
+	const bool tiles_first = a_layout == ANYGPU_A_ROW_MAJOR && b_layout == ANYGPU_B_COL_MAJOR && M >= 48 &&
+	                         gemm_f32_ring_applies(A, B, M, N, K, lda, ldb, stride_a, stride_b, batch, 0, 64);
+	if (batch == 1 && !tiles_first && a_layout == ANYGPU_A_ROW_MAJOR && gemm_band_applies<float>(A, B, nullptr, C, M, N, K, lda, ldb, ldc, b_layout))
 		return launch_gemm_band<float>(A, B, nullptr, bias, C, M, N, K, lda, ldb, ldc, kEpiBias, 0.0f, stream);
 	if (batch == 1 && a_layout == ANYGPU_A_ROW_MAJOR && b_layout == ANYGPU_B_ROW_MAJOR &&
 	    gemm_band_ncontig_applies(A, B, nullptr, C, M, N, K, lda, ldb, ldc, false))

@@ -816,6 +816,28 @@ def test_mm_f16_smaller_four_wave_tiles_reference_layout_exact(ops, m, n, k, pad
     assert np.array_equal(got, want)
 
 
+@pytest.mark.parametrize("m,n,k,pad", [(128, 128, 32, 0), (2048, 2048, 64, 0), (2048, 2048, 96, 4), (1000, 2000, 160, 8), (130, 4100, 32, 0),
+                                       (2048, 1024, 2048, 0), (256, 2304, 9216, 0), (3000, 1031, 64, 1)])
+def test_mm_f32_four_wave_kernel_integer_inputs_exact(ops, m, n, k, pad):
+    # fp32 products of k-contiguous operands in whole 32-deep slabs take the four-wave kernel whose main loop is an
+    # assembly block: one slab, two, three, padded pitches, ragged M and N, a C with an odd pitch, deep K cut into planes.
+    # Integer operands: every sum is exact in fp32 whatever the order.
+    import torch
+    from anygpu_amd import capi
+    a = synth.integers(m + k + 12, (m, k), -3, 3).astype(np.float32)
+    bt = synth.integers(n + k + 13, (n, k), -3, 3).astype(np.float32)
+    a_dev = torch.full((m, k + pad), 7.0, dtype=torch.float32, device="cuda")
+    b_dev = torch.full((n, k + pad), 7.0, dtype=torch.float32, device="cuda")
+    a_dev[:, :k] = dev(a)
+    b_dev[:, :k] = dev(bt)
+    cbuf = torch.full((m + 1, n + 3), -7.0, device="cuda", dtype=torch.float32)
+    ops.tensor_mm(a_dev[:, :k], b_dev[:, :k], out=cbuf[:m, :n], b_layout=capi.B_COL_MAJOR)
+    got = host(cbuf).astype(np.int64)
+    want = a.astype(np.int64) @ bt.astype(np.int64).T
+    assert np.array_equal(got[:m, :n], want)
+    assert np.all(got[m:, :] == -7) and np.all(got[:, n:] == -7)
+
+
 def test_mm_f16_whole_256_tiles_batched(ops, oracle):
     # four products of 2048 x 2048 x 128 in one launch: 256 tiles of 256 x 256, the four-wave kernel over blockIdx.y
     from anygpu_amd import capi
