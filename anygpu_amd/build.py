@@ -68,6 +68,8 @@ def build_kernels(verbose: bool = False) -> Path:
     _run([sys.executable, str(CSRC_DIR / "gen_gemm_f16_ring_loop.py"), str(CSRC_DIR / "gemm_f16_ring_loop_4x4kn.inc"), "4x4kn"], quiet=not verbose)
     _run([sys.executable, str(CSRC_DIR / "gen_gemm_f32_ring_loop.py"), str(CSRC_DIR / "gemm_f32_ring_loop.inc")], quiet=not verbose)
     _run([sys.executable, str(CSRC_DIR / "gen_gemm_f32_ring_loop.py"), str(CSRC_DIR / "gemm_f32_ring_loop_64.inc"), "64"], quiet=not verbose)
+    _run([sys.executable, str(CSRC_DIR / "gen_gemm_f32_ring_loop.py"), str(CSRC_DIR / "gemm_f32_ring_loop_kn.inc"), "kn"], quiet=not verbose)
+    _run([sys.executable, str(CSRC_DIR / "gen_gemm_f32_ring_loop.py"), str(CSRC_DIR / "gemm_f32_ring_loop_64kn.inc"), "64", "kn"], quiet=not verbose)
 
     def compile_one(src: str) -> Path:
         obj = OBJ_DIR / (Path(src).stem + ".o")

@@ -341,10 +341,11 @@ static hipError_t launch_tiles_once(const float* A, const float* B, const float*
 {
 	// k-contiguous operands in whole 32-deep slabs, one product per tile: the four-wave kernel (gemm_f32_ring.hpp), which
 	// keeps the matrix cores busier than this file's kernel does around its barriers (2048^3: 131 -> see the header)
-	if constexpr (A_LAYOUT == ANYGPU_A_ROW_MAJOR && B_LAYOUT == ANYGPU_B_COL_MAJOR && BM == BN && EPI != kEpiGeluMul)
+	if constexpr (A_LAYOUT == ANYGPU_A_ROW_MAJOR && BM == BN && EPI != kEpiGeluMul)
 	{
-		if (gemm_f32_ring_applies(A, B, M, N, K, lda, ldb, stride_a, stride_b, batch, k_split, BM))
-			return launch_gemm_f32_ring<BM / 64, EPI>(A, B, bias, C, M, N, K, lda, ldb, ldc, stride_a, stride_b, stride_c, batch, ep_param, k_split, stream);
+		if (gemm_f32_ring_applies(A, B, M, N, K, lda, ldb, stride_a, stride_b, batch, k_split, BM, B_LAYOUT))
+			return launch_gemm_f32_ring<BM / 64, EPI, B_LAYOUT == ANYGPU_B_ROW_MAJOR>(A, B, bias, C, M, N, K, lda, ldb, ldc, stride_a, stride_b, stride_c,
+			                                                                        batch, ep_param, k_split, stream);
 	}
 	const dim3 grid((unsigned)((N + BN - 1) / BN), (unsigned)((M + BM - 1) / BM), (unsigned)batch);
 	const bool aligned_in = (reinterpret_cast<uintptr_t>(A) % 16 == 0) && (reinterpret_cast<uintptr_t>(B) % 16 == 0) &&
@@ -513,8 +514,8 @@ static hipError_t launch_layout(const float* A, const float* B, const float* B2,
 	// (what the stream's workspace holds bounds the cuts along K: the caller's, or the library's own for eager launches;
 	// a stream under capture without a caller's workspace has none and runs uncut)
 	const size_t ws_bytes = (may_split && batch == 1) ? band::workspace_capacity(stream) : 0;
-	const bool four_wave = A_LAYOUT == ANYGPU_A_ROW_MAJOR && B_LAYOUT == ANYGPU_B_COL_MAJOR && EPI != kEpiGeluMul &&
-	                       gemm_f32_ring_applies(A, B, M, N, K, lda, ldb, stride_a, stride_b, batch, 0, 64);
+	const bool four_wave = A_LAYOUT == ANYGPU_A_ROW_MAJOR && EPI != kEpiGeluMul &&
+	                       gemm_f32_ring_applies(A, B, M, N, K, lda, ldb, stride_a, stride_b, batch, 0, 64, B_LAYOUT);
 	const TilePlan big = plan_tiles(128, M, N, K, batch, may_split, ws_bytes, four_wave);
 	const TilePlan small = plan_tiles(64, M, N, K, batch, may_split, ws_bytes, four_wave);
 	if constexpr (EPI != kEpiGeluMul)

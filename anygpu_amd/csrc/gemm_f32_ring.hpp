@@ -34,7 +34,9 @@ struct GemmF32RingCfg
 // operand rows 16-byte aligned.  RAGGED: M and N need not be multiples of 128 and C may start and step at any element;
 // operand rows past the end are read from the last valid row (they only feed results that are not stored), the stores
 // are guarded.  EPI: kEpiBias (+ bias[n] when bias != NULL) or kEpiSoftcap, applied to the sums.
-template <int T, bool RAGGED, int EPI>
+// B_KN: B stored [K, N] (N a multiple of 4): a B unit of 32 k rows x BN n, the chunks of rows 16 .. 31 stored with bit 3
+// of their index flipped; a lane fetches its k one float at a time down its column.
+template <int T, bool RAGGED, int EPI, bool B_KN = false>
 __global__ __launch_bounds__(256) void gemm_f32_nt_ring_kernel(
 	const float* __restrict__ A, const float* __restrict__ B, const float* __restrict__ bias, float* __restrict__ C,
 	int64_t M, int64_t N, int K, int64_t lda, int64_t ldb, int64_t ldc,
@@ -84,11 +86,24 @@ __global__ __launch_bounds__(256) void gemm_f32_nt_ring_kernel(
 			b_row = b_row < N - 1 ? b_row : N - 1;
 		}
 		table[64 * q] = (unsigned)(((a_row - a_first) * lda + chunk * 4) * 4);
-		table[64 * (8 + q)] = (unsigned)(((b_row - b_first) * ldb + chunk * 4) * 4);
+		if constexpr (B_KN)
+		{
+			// one instruction fills 1024 / (4 BN) k rows: lane -> row lane / (BN / 4), position lane % (BN / 4); the wave's
+			// instructions cover rows 8 wave .. 8 wave + 7 of the slab's 32
+			constexpr int kLanesPerRow = Cfg::BN / 4, kRowsPerLoad = 64 / kLanesPerRow;
+			const int k_wave = kRowsPerLoad * q + lane / kLanesPerRow;
+			const int k = 8 * wave + k_wave;
+			int64_t col = (int64_t)(((lane % kLanesPerRow) ^ (((k >> 4) & 1) << 3)) << 2);
+			if constexpr (RAGGED)
+				if (n0 + col + 4 > N) col = N - 4 - n0;
+			table[64 * (8 + q)] = (unsigned)((k_wave * ldb + col) * 4);
+		}
+		else
+			table[64 * (8 + q)] = (unsigned)(((b_row - b_first) * ldb + chunk * 4) * 4);
 	}
 	const unsigned table_addr = lds0 + 3 * Cfg::kStageBytes + (wave * (16 * 64) + lane) * 4;
 	const uintptr_t a_wave = reinterpret_cast<uintptr_t>(A + a_first * lda);
-	const uintptr_t b_wave = reinterpret_cast<uintptr_t>(B + b_first * ldb);
+	const uintptr_t b_wave = reinterpret_cast<uintptr_t>(B_KN ? B + (int64_t)(8 * wave) * ldb + n0 : B + b_first * ldb);
 	const unsigned share_a = wave * (Cfg::kLoads * 1024);
 	const unsigned share_b = Cfg::BM * 128 + wave * (Cfg::kLoads * 1024);
 	const int slabs = K / 32;
@@ -98,7 +113,13 @@ __global__ __launch_bounds__(256) void gemm_f32_nt_ring_kernel(
 	const unsigned frag_row = lane & 31;
 	const unsigned first_pos = (4 * (lane >> 5)) ^ ((frag_row >> 1) & 7);
 	const unsigned a_addr = (wm * 32 * T + frag_row) * 128 + first_pos * 16;
-	const unsigned b_addr = Cfg::BM * 128 + (wn * 32 * T + frag_row) * 128 + first_pos * 16;
+	// B stored [K, N]: the lane's column n = wn 32 T + 32 j + frag_row of the tile, its first k row 16 half; chunk index
+	// bit 3 (byte bit 7) is j (T = 2) or wn (T = 1), flipped for the upper half of the lanes
+	const unsigned half = lane >> 5;
+	const unsigned b_addr = B_KN ? Cfg::BM * 128 + 16 * half * (Cfg::BN * 4) + (T == 2 ? wn * 256 : 0) + (frag_row >> 2) * 16 + (frag_row & 3) * 4
+	                             : Cfg::BM * 128 + (wn * 32 * T + frag_row) * 128 + first_pos * 16;
+	[[maybe_unused]] const unsigned b_flip = (T == 2 ? half : (half ^ (unsigned)wn)) << 7;
+	[[maybe_unused]] const unsigned b_step = (unsigned)(128 * ldb);        // bytes from one [K, N] slab (32 rows) to the next
 
 	// The accumulators leave the block as vectors pinned to a[0 : 16 T T): MFMA tile (i, j) in registers 16 (T i + j) .. + 15.
 	float32x_f32_t r0 = {}, r1 = {};
@@ -116,8 +137,20 @@ __global__ __launch_bounds__(256) void gemm_f32_nt_ring_kernel(
 		  "v152", "v153", "v154", "v155", "v156", "v157", "v158", "v159", "v160", "v161", "v162", "v163", "v164", "v165", \
 		  "v166", "v167", "v168", "v169", "v170", "v171", "v172", "v173", "v174", "v175", "v176", "v177", "v178", "v179", \
 		  "v180", "v181", "v182", "v183", "v184", "v185", "v186", "v187", "v188", "v189", "v190", "v191", \
-		  "s60", "s61", "s62", "s63", "s64", "s65", "s66", "s67", "s68", "s69", "s70", "s71", "s72", "s73", "scc", "m0", "memory"
-	if constexpr (T == 2)
+		  "s60", "s61", "s62", "s63", "s64", "s65", "s66", "s67", "s68", "s69", "s70", "s71", "s72", "s73", "s74", "scc", "m0", "memory"
+	if constexpr (T == 2 && B_KN)
+		asm volatile(
+#include "gemm_f32_ring_loop_kn.inc"
+			: "={a[0:31]}"(r0), "={a[32:63]}"(r1)
+			: ANYGPU_F32_RING_INPUTS, [bsx] "v"(b_flip), [bstep] "s"(b_step)
+			: ANYGPU_F32_RING_CLOBBERS);
+	else if constexpr (B_KN)
+		asm volatile(
+#include "gemm_f32_ring_loop_64kn.inc"
+			: "={a[0:15]}"(single)
+			: ANYGPU_F32_RING_INPUTS, [bsx] "v"(b_flip), [bstep] "s"(b_step)
+			: ANYGPU_F32_RING_CLOBBERS);
+	else if constexpr (T == 2)
 		asm volatile(
 #include "gemm_f32_ring_loop.inc"
 			: "={a[0:31]}"(r0), "={a[32:63]}"(r1)
@@ -172,15 +205,17 @@ __global__ __launch_bounds__(256) void gemm_f32_nt_ring_kernel(
 
 // What the kernel assumes, checked on the host before every launch.
 inline bool gemm_f32_ring_applies(const float* A, const float* B, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
-                                  int64_t stride_a, int64_t stride_b, int64_t batch, int64_t k_split, int64_t tile = 128)
+                                  int64_t stride_a, int64_t stride_b, int64_t batch, int64_t k_split, int64_t tile = 128,
+                                  int b_layout = ANYGPU_B_COL_MAJOR)
 {
+	if (b_layout == ANYGPU_B_ROW_MAJOR && N % 4 != 0) return false;
 	const bool aligned = reinterpret_cast<uintptr_t>(A) % 16 == 0 && reinterpret_cast<uintptr_t>(B) % 16 == 0 &&
 	                     lda % 4 == 0 && ldb % 4 == 0 && stride_a % 4 == 0 && stride_b % 4 == 0;
 	return aligned && M > 0 && N > 0 && K >= 32 && K % 32 == 0 && k_split % 32 == 0 && K <= 0x7FFFFFFFLL &&
 	       lda < (1 << 24) && ldb < (1 << 24) && ((M + tile - 1) / tile) * ((N + tile - 1) / tile) <= 0x7FFFFFFFLL && batch >= 1 && batch <= 65535;
 }
 
-template <int T, int EPI>
+template <int T, int EPI, bool B_KN = false>
 inline hipError_t launch_gemm_f32_ring(const float* A, const float* B, const float* bias, float* C, int64_t M, int64_t N, int64_t K,
                                        int64_t lda, int64_t ldb, int64_t ldc, int64_t stride_a, int64_t stride_b, int64_t stride_c,
                                        int64_t batch, float ep_param, int64_t k_split, hipStream_t stream)
@@ -188,7 +223,7 @@ inline hipError_t launch_gemm_f32_ring(const float* A, const float* B, const flo
 	const bool c_aligned = reinterpret_cast<uintptr_t>(C) % 16 == 0 && ldc % 4 == 0 && stride_c % 4 == 0;
 	using Cfg = GemmF32RingCfg<T>;
 	const bool ragged = M % Cfg::BM != 0 || N % Cfg::BN != 0 || !c_aligned;
-	auto kernel = ragged ? gemm_f32_nt_ring_kernel<T, true, EPI> : gemm_f32_nt_ring_kernel<T, false, EPI>;
+	auto kernel = ragged ? gemm_f32_nt_ring_kernel<T, true, EPI, B_KN> : gemm_f32_nt_ring_kernel<T, false, EPI, B_KN>;
 	// More than 64 KB of dynamic LDS has to be granted per function and per device, once.
 	static std::atomic<uint64_t> configured_devices[2];
 	(void)hipGetLastError();

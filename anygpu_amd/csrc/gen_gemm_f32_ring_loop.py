@@ -32,7 +32,15 @@ ldsa / ldsb (SGPR: offset of the wave's share of the A / B unit in a stage), sla
 
 The 64 x 64 tile (T = 1) has units of 64 rows: two loads per wave, operand and slab, a stage of 16 KB, 8 MFMAs per step.
 
-Usage: gen_gemm_f32_ring_loop.py OUTPUT [64]
+B stored [K, N] (the "kn" forms): a B unit is 32 k rows x 64 T n (rows of 256 T bytes, filled 2 or 4 rows per load); a
+lane (column n = lane % 32 of its tile, half h) fetches its eight k of a step one float at a time down a column,
+ds_read_b32 with the k row in the offset field.  Rows 16 apart (the two halves of the lanes) would fall on the same
+banks, so the 16-byte chunks of rows 16 .. 31 are stored with bit 3 of their index flipped; for the tile column j that
+bit is j, so each tile column has its address register (v112 + j inside a stage, v120 + j / v122 + j in the stages being
+read).  A slab of B is 32 rows further on in memory (s64 and s74 hold the halves of that product); bsx (VGPR) is the
+lane's flipped bit, bstep (SGPR) the bytes from one slab of B to the next.
+
+Usage: gen_gemm_f32_ring_loop.py OUTPUT [64] [kn]
 """
 import sys
 
@@ -51,9 +59,10 @@ def b_base(buf, j):
     return 144 + 32 * buf + 8 * j
 
 
-def generate(T):
-    """T: MFMA tiles per wave and direction (2: tile 128 x 128, 1: tile 64 x 64)"""
+def generate(T, kn=False):
+    """T: MFMA tiles per wave and direction (2: tile 128 x 128, 1: tile 64 x 64); kn: B stored [K, N]"""
     lines = []
+    ROWB = 256 * T                   # bytes of a [k][n] unit row
     STAGE = 2 * (64 * T) * 128       # bytes: A unit + B unit
     LOADS = 2 * T                    # per wave, operand and slab
     MFMAS = 8 * T * T                # per 16-deep step: 8 k pairs x T x T tiles
@@ -74,7 +83,7 @@ def generate(T):
         return f"v{108 + 2 * step + c}"
 
     def b_const(step, c):
-        return f"v{112 + 2 * step + c}"
+        return f"v{112 + c}" if kn else f"v{112 + 2 * step + c}"       # kn: c is the tile column
 
     def a_cur(step, c):
         return f"v{116 + 2 * step + c}"
@@ -84,10 +93,15 @@ def generate(T):
 
     def load_set(stage_reg, add):
         """where the loads of slab min(t + add, last) go and come from"""
-        return [f"s_add_u32 {S_LDA}, {stage_reg}, %[ldsa]", f"s_add_u32 {S_LDB}, {stage_reg}, %[ldsb]",
-                f"s_add_u32 {S_TMP}, {S_T}, {add}", f"s_min_u32 {S_TMP}, {S_TMP}, {S_LAST}", f"s_lshl_b32 {S_TMP}, {S_TMP}, 7",
-                ("s_add_u32 s68, %[abaselo], " + S_TMP, "s_addc_u32 s69, %[abasehi], 0"),
-                ("s_add_u32 s70, %[bbaselo], " + S_TMP, "s_addc_u32 s71, %[bbasehi], 0")]
+        out = [f"s_add_u32 {S_LDA}, {stage_reg}, %[ldsa]", f"s_add_u32 {S_LDB}, {stage_reg}, %[ldsb]",
+               f"s_add_u32 {S_TMP}, {S_T}, {add}", f"s_min_u32 {S_TMP}, {S_TMP}, {S_LAST}"]
+        if kn:
+            out += ["s_mul_hi_u32 s64, " + S_TMP + ", %[bstep]", "s_mul_i32 s74, " + S_TMP + ", %[bstep]",
+                    ("s_add_u32 s70, %[bbaselo], s74", "s_addc_u32 s71, %[bbasehi], s64")]
+        out += [f"s_lshl_b32 {S_TMP}, {S_TMP}, 7", ("s_add_u32 s68, %[abaselo], " + S_TMP, "s_addc_u32 s69, %[abasehi], 0")]
+        if not kn:
+            out.append(("s_add_u32 s70, %[bbaselo], " + S_TMP, "s_addc_u32 s71, %[bbasehi], 0"))
+        return out
 
     def loads(which):
         """half of the wave's eight loads of a slab as (M0 write, load) pairs: 0 the A loads, 1 the B loads"""
@@ -102,8 +116,12 @@ def generate(T):
         """the eight fragment reads of a step: tile row i of the patch lies 32 rows = 4096 bytes further on"""
         out = []
         for j in range(T):
-            for c in range(2):
-                out.append(f"ds_read_b128 {frag_quad(b_base(buf, j), c)}, {b_cur(step, c)} offset:{4096 * j}")
+            if kn:
+                for e in range(8):
+                    out.append(f"ds_read_b32 v{b_base(buf, j) + e}, {b_cur(step, j)} offset:{(8 * step + e) * ROWB}")
+            else:
+                for c in range(2):
+                    out.append(f"ds_read_b128 {frag_quad(b_base(buf, j), c)}, {b_cur(step, c)} offset:{4096 * j}")
         for i in range(T):
             for c in range(2):
                 out.append(f"ds_read_b128 {frag_quad(a_base(buf, i), c)}, {a_cur(step, c)} offset:{4096 * i}")
@@ -111,7 +129,7 @@ def generate(T):
 
     def stage_addresses(step, stage_reg):
         return [f"v_add_u32 {a_cur(step, c)}, {stage_reg}, {a_const(step, c)}" for c in range(2)] + \
-               [f"v_add_u32 {b_cur(step, c)}, {stage_reg}, {b_const(step, c)}" for c in range(2)]
+               [f"v_add_u32 {b_cur(step, c)}, {stage_reg}, {b_const(step, c)}" for c in range(T if kn else 2)]
 
     # ---- prologue: slabs 0 and 1 and the A loads of slab 2, fragments of the first step
     emit(f"s_mov_b32 {S_T}, 0", "prologue")
@@ -127,7 +145,12 @@ def generate(T):
         for c in range(2):
             x = 16 * (2 * step + c)
             emit(f"v_xor_b32 {a_const(step, c)}, {x}, %[aaddr]" if x else f"v_mov_b32 {a_const(step, c)}, %[aaddr]")
-            emit(f"v_xor_b32 {b_const(step, c)}, {x}, %[baddr]" if x else f"v_mov_b32 {b_const(step, c)}, %[baddr]")
+            if not kn:
+                emit(f"v_xor_b32 {b_const(step, c)}, {x}, %[baddr]" if x else f"v_mov_b32 {b_const(step, c)}, %[baddr]")
+    if kn:
+        for j in range(T):
+            emit(f"v_xor_b32 {b_const(0, j)}, {128 * j}, %[bsx]")
+            emit(f"v_add_u32 {b_const(0, j)}, %[baddr], {b_const(0, j)}")
     for slab in range(3):
         for ins in load_set(S[slab], slab):
             emit(ins)
@@ -157,7 +180,7 @@ def generate(T):
         def place(entry, earliest):
             n = len(entry) if isinstance(entry, tuple) else 1
             # (an fp32 MFMA covers 64 cycles, sixteen issue slots)
-            for cap in (1, 2, 3, 4, 6, 8):
+            for cap in (1, 2, 3, 4, 6, 8, 10, 12):
                 for g in range(earliest, MFMAS):
                     if sum(len(x) if isinstance(x, tuple) else 1 for x in gaps[g]) + n <= cap:
                         gaps[g].append(entry)
@@ -166,9 +189,10 @@ def generate(T):
 
         buf = step
         # the fragments of the next step: k step 1 of slab t in the stage of slab t, or k step 0 of slab t + 1
-        spacing = 2 if T == 2 else 1
-        for q, ins in enumerate(reads(buf ^ 1, 1 - step)):
-            gaps[spacing * q].append(ins)
+        step_reads = reads(buf ^ 1, 1 - step)
+        spacing = 2 if T == 2 and not kn else 1
+        for q, ins in enumerate(step_reads):
+            gaps[spacing * q if spacing * (len(step_reads) - 1) < MFMAS else q * MFMAS // len(step_reads)].append(ins)
         # step 0: the B loads of slab t + 2; step 1: the A loads of slab t + 3
         last_load = 0
         every = 3 if T == 2 else 1
@@ -214,7 +238,7 @@ def generate(T):
 if __name__ == "__main__":
     with open(sys.argv[1], "w") as f:
         f.write("// Written by gen_gemm_f32_ring_loop.py (the register plan and the schedule are explained there): do not edit.\n")
-        for s, c in generate(1 if len(sys.argv) > 2 and sys.argv[2] == "64" else 2):
+        for s, c in generate(1 if "64" in sys.argv[2:] else 2, "kn" in sys.argv[2:]):
             if c:
                 f.write(f"// {c}\n")
             f.write(f'"{s}\\n\\t"\n')

@@ -86,7 +86,8 @@ def test_generated_gemm_loop_is_current(tmp_path):
     # gemm_f16_ring_loop*.inc are generated texts that are committed: they have to be what the generator beside them writes
     import sys
     csrc = REPO / "anygpu_amd" / "csrc"
-    for name, form in (("gemm_f32_ring_loop.inc", []), ("gemm_f32_ring_loop_64.inc", ["64"])):
+    for name, form in (("gemm_f32_ring_loop.inc", []), ("gemm_f32_ring_loop_64.inc", ["64"]),
+                       ("gemm_f32_ring_loop_kn.inc", ["kn"]), ("gemm_f32_ring_loop_64kn.inc", ["64", "kn"])):
         out = tmp_path / name
         subprocess.run([sys.executable, str(csrc / "gen_gemm_f32_ring_loop.py"), str(out), *form], check=True)
         assert out.read_text() == (csrc / name).read_text()

@@ -838,6 +838,25 @@ def test_mm_f32_four_wave_kernel_integer_inputs_exact(ops, m, n, k, pad):
     assert np.all(got[m:, :] == -7) and np.all(got[:, n:] == -7)
 
 
+@pytest.mark.parametrize("m,n,k,pad", [(128, 128, 32, 0), (2048, 2048, 64, 0), (2048, 2048, 96, 4), (1000, 2000, 160, 8), (130, 4100, 32, 0),
+                                       (2048, 1024, 2048, 0), (256, 2304, 9216, 0), (3000, 1032, 64, 4), (64, 64, 32, 0), (500, 260, 128, 0)])
+def test_mm_f32_four_wave_kernel_reference_layout_exact(ops, m, n, k, pad):
+    # the same kernels with B stored [K, N] as the reference stores it: units of 32 k rows, a lane fetches its k down a
+    # column, the chunks of the upper sixteen rows stored with a flipped index bit; pitches that are not the row length,
+    # last tiles of 4 columns, deep K cut into planes that step down the rows of B
+    import torch
+    a = synth.integers(m + k + 14, (m, k), -3, 3).astype(np.float32)
+    b = synth.integers(n + k + 15, (k, n), -3, 3).astype(np.float32)
+    b_dev = torch.full((k, n + pad), 7.0, dtype=torch.float32, device="cuda")
+    b_dev[:, :n] = dev(b)
+    cbuf = torch.full((m + 1, n + 3), -7.0, device="cuda", dtype=torch.float32)
+    ops.tensor_mm(dev(a), b_dev[:, :n], out=cbuf[:m, :n])
+    got = host(cbuf).astype(np.int64)
+    want = a.astype(np.int64) @ b.astype(np.int64)
+    assert np.array_equal(got[:m, :n], want)
+    assert np.all(got[m:, :] == -7) and np.all(got[:, n:] == -7)
+
+
 def test_mm_f16_whole_256_tiles_batched(ops, oracle):
     # four products of 2048 x 2048 x 128 in one launch: 256 tiles of 256 x 256, the four-wave kernel over blockIdx.y
     from anygpu_amd import capi
