@@ -21,8 +21,8 @@ the parity tests).  Timing of every kernel:
 The memory-bound kernels rotate over several buffer sets so that the working set exceeds the
 256 MB Infinity Cache.
 
-`--gemm-shapes` prints, instead of the JSON line, a table of the fp16 GEMM over the projection shapes of the models
-the path serves (8 row counts x 14 weight shapes, weights k-contiguous) next to torch.matmul, i.e. the vendor library,
+`--gemm-shapes` (or `--gemm-shapes f32`) prints, instead of the JSON line, a table of the fp16 (fp32) GEMM over the
+projection shapes of the models the path serves (8 row counts x 14 weight shapes, weights k-contiguous) next to torch.matmul, i.e. the vendor library,
 on the same operands.
 """
 from __future__ import annotations
@@ -77,8 +77,8 @@ def parse_args():
                     help="target wall time of the CPU-oracle sample of the headline (0 disables every CPU baseline); "
                          "the other configurations get a quarter of it each")
     ap.add_argument("--only", default="", help="comma list of: gemm,gemm32,conv,softmax,attn,attn32,decode,norm (default: all)")
-    ap.add_argument("--gemm-shapes", action="store_true",
-                    help="print the table of fp16 GEMM layer shapes against torch.matmul and exit")
+    ap.add_argument("--gemm-shapes", nargs="?", const="f16", default=None, choices=("f16", "f32"),
+                    help="print the table of GEMM layer shapes (fp16, or fp32 with `--gemm-shapes f32`) against torch.matmul and exit")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain device copy of 256 MiB (read 256 MiB + write 256 MiB) a few times, "
                          "as the known-size reference for scaling FETCH_SIZE / WRITE_SIZE counter readings")
@@ -432,7 +432,7 @@ LAYER_WEIGHTS = [(9216, 2304), (18432, 2304), (2304, 9216), (2048, 2304), (1024,
 LAYER_ROWS = (16, 64, 128, 256, 512, 1024, 2048, 4096)
 
 
-def sweep_gemm_shapes(torch, ops, capi):
+def sweep_gemm_shapes(torch, ops, capi, dtype_name="f16"):
     """[rows, K] x [N, K]^T for the (N, K) of Gemma2-2B / Zamba2 / Llama-8B-sized projections: microseconds of this
     library and of torch.matmul (hipBLASLt) on the same uniform random operands, each the better of two runs of 40
     back-to-back launches taken alternately."""
@@ -448,14 +448,15 @@ def sweep_gemm_shapes(torch, ops, capi):
         torch.cuda.synchronize()
         return start.elapsed_time(stop) / iters * 1e3
 
+    dtype = torch.half if dtype_name == "f16" else torch.float
     print("| rows | K | N | this library us | torch.matmul us | ratio |")
     print("|---:|---:|---:|---:|---:|---:|")
     ratios = []
     for n, k in LAYER_WEIGHTS:
-        weight = (torch.rand(n, k, device="cuda") * 2 - 1).half()
+        weight = (torch.rand(n, k, device="cuda") * 2 - 1).to(dtype)
         for rows in LAYER_ROWS:
-            a = (torch.rand(rows, k, device="cuda") * 2 - 1).half()
-            c = torch.empty(rows, n, device="cuda", dtype=torch.half)
+            a = (torch.rand(rows, k, device="cuda") * 2 - 1).to(dtype)
+            c = torch.empty(rows, n, device="cuda", dtype=dtype)
             mine = lambda: ops.tensor_mm(a, weight, out=c, b_layout=capi.B_COL_MAJOR)
             theirs = lambda: torch.matmul(a, weight.t(), out=c)
             t_mine, t_theirs = timed(mine), timed(theirs)
@@ -514,7 +515,7 @@ def main():
     capi.load()
     torch.cuda.set_device(0)
     if args.gemm_shapes:
-        sweep_gemm_shapes(torch, ops, capi)
+        sweep_gemm_shapes(torch, ops, capi, args.gemm_shapes)
         return 0
     only = set(filter(None, args.only.split(",")))
     want = lambda name: not only or name in only
