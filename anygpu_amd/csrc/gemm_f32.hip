@@ -664,6 +664,11 @@ hipError_t launch_gemm_f32_gelu_mul(const float* A, const float* B_gate, const f
 		return launch_gemm_band_ncontig(A, B_gate, B_up, nullptr, C, M, N, K, lda, ldb, ldc, kEpiGeluMul, 0.0f, stream);
 	if (gemm_skinny_applies<float>(A, B_gate, B_up, M, N, K, lda, ldb, b_layout))
 		return launch_gemm_skinny<float>(A, B_gate, B_up, nullptr, C, M, N, K, lda, ldb, ldc, b_layout, kEpiGeluMul, 0.0f, stream);
+	// k-contiguous weights in whole slabs: the four-wave kernel with gate and up rows side by side in its B unit
+	// (2048 x 2304 -> 9216: 1.40 -> 1.27 ms)
+	if (b_layout == ANYGPU_B_COL_MAJOR && reinterpret_cast<uintptr_t>(B_up) % 16 == 0 &&
+	    gemm_f32_ring_applies(A, B_gate, M, N, K, lda, ldb, 0, 0, 1, 0, 64))
+		return launch_gemm_f32_ring<2, kEpiGeluMul>(A, B_gate, B_up, C, M, N, K, lda, ldb, ldc, 0, 0, 0, 1, 0.0f, 0, stream);
 	if (b_layout == ANYGPU_B_COL_MAJOR)
 		return launch_layout<ANYGPU_A_ROW_MAJOR, ANYGPU_B_COL_MAJOR, kEpiGeluMul>(A, B_gate, B_up, nullptr, C, M, N, K, lda, ldb, ldc,
 		                                                                         0, 0, 0, 1, 0.0f, stream);

@@ -33,7 +33,12 @@ struct GemmF32RingCfg
 // the strides then step along K and C is the range's [M, N] plane of partial sums.  K (and k_split) multiples of 32,
 // operand rows 16-byte aligned.  RAGGED: M and N need not be multiples of 128 and C may start and step at any element;
 // operand rows past the end are read from the last valid row (they only feed results that are not stored), the stores
-// are guarded.  EPI: kEpiBias (+ bias[n] when bias != NULL) or kEpiSoftcap, applied to the sums.
+// are guarded.  EPI: kEpiBias (+ bias[n] when bias != NULL) or kEpiSoftcap, applied to the sums; or kEpiGeluMul (big tile,
+// k-contiguous weights): the tile is 64 output columns wide (N counts those) and its B unit is put together from two
+// matrices, of every wave column's 64 unit rows the first 32 from B (the gate weights) and the second 32 from `bias`,
+// which then is the second matrix (the up weights, same pitch), both for the same 32 output columns: MFMA tile column 0
+// of a wave holds the gate sums and column 1 the up sums of the same outputs, gelu_tanh(gate) * up goes out.  The wave
+// that loads a quarter of the unit loads it from one matrix.
 // B_KN: B stored [K, N] (N a multiple of 4): a B unit of 32 k rows x BN n, the chunks of rows 16 .. 31 stored with bit 3
 // of their index flipped; a lane fetches its k one float at a time down its column.
 template <int T, bool RAGGED, int EPI, bool B_KN = false>
@@ -43,7 +48,8 @@ __global__ __launch_bounds__(256) void gemm_f32_nt_ring_kernel(
 	int64_t stride_a, int64_t stride_b, int64_t stride_c, float ep_param, int k_split)
 {
 	using Cfg = GemmF32RingCfg<T>;
-	static_assert(EPI == kEpiBias || EPI == kEpiSoftcap, "one product");
+	constexpr bool DUAL = EPI == kEpiGeluMul;
+	static_assert(!DUAL || (T == 2 && !B_KN), "two weight matrices: the big tile, k-contiguous");
 	extern __shared__ __align__(1024) char lds[];
 	if (k_split > 0)
 	{
@@ -58,8 +64,12 @@ __global__ __launch_bounds__(256) void gemm_f32_nt_ring_kernel(
 	const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 	const int wm = wave >> 1, wn = wave & 1;
 	int tile_m, tile_n;
-	tile_of_block<8>(blockIdx.x, (int)((M + Cfg::BM - 1) / Cfg::BM), (int)((N + Cfg::BN - 1) / Cfg::BN), tile_m, tile_n);
-	const int64_t m0 = (int64_t)tile_m * Cfg::BM, n0 = (int64_t)tile_n * Cfg::BN;
+	constexpr int kOutN = DUAL ? Cfg::BN / 2 : Cfg::BN;           // output columns of a tile
+	tile_of_block<8>(blockIdx.x, (int)((M + Cfg::BM - 1) / Cfg::BM), (int)((N + kOutN - 1) / kOutN), tile_m, tile_n);
+	const int64_t m0 = (int64_t)tile_m * Cfg::BM, n0 = (int64_t)tile_n * kOutN;
+	// DUAL: the unit rows wave w loads are output columns 32 (w / 2) .. of the tile, from B (w even) or the second matrix
+	const float* const b_of_wave = DUAL && (wave & 1) ? bias : B;
+	const int b_unit_row = DUAL ? 8 * Cfg::kLoads * (wave >> 1) : 8 * Cfg::kLoads * wave;
 
 	// Direct loads.  A unit row is 32 floats = eight 16-byte chunks; chunk c of row r sits at position c ^ ((r >> 1) & 7).
 	// One instruction fills 8 rows: lane -> row lane / 8, position lane % 8; instruction q of this wave covers rows
@@ -68,7 +78,7 @@ __global__ __launch_bounds__(256) void gemm_f32_nt_ring_kernel(
 	const unsigned lds0 = (unsigned)(uintptr_t)(const __attribute__((address_space(3))) char*)lds;
 	const int ld_row = lane >> 3, ld_pos = lane & 7;
 	unsigned* const table = reinterpret_cast<unsigned*>(lds + 3 * Cfg::kStageBytes) + wave * (16 * 64) + lane;
-	int64_t a_first = m0 + 8 * Cfg::kLoads * wave, b_first = n0 + 8 * Cfg::kLoads * wave;
+	int64_t a_first = m0 + 8 * Cfg::kLoads * wave, b_first = n0 + b_unit_row;
 	if constexpr (RAGGED)
 	{
 		a_first = a_first < M - 1 ? a_first : M - 1;
@@ -79,7 +89,7 @@ __global__ __launch_bounds__(256) void gemm_f32_nt_ring_kernel(
 	{
 		const int row = 8 * (Cfg::kLoads * wave + q) + ld_row;
 		const unsigned chunk = ld_pos ^ ((row >> 1) & 7);
-		int64_t a_row = m0 + row, b_row = n0 + row;
+		int64_t a_row = m0 + row, b_row = n0 + b_unit_row + 8 * q + ld_row;
 		if constexpr (RAGGED)
 		{
 			a_row = a_row < M - 1 ? a_row : M - 1;
@@ -103,7 +113,7 @@ __global__ __launch_bounds__(256) void gemm_f32_nt_ring_kernel(
 	}
 	const unsigned table_addr = lds0 + 3 * Cfg::kStageBytes + (wave * (16 * 64) + lane) * 4;
 	const uintptr_t a_wave = reinterpret_cast<uintptr_t>(A + a_first * lda);
-	const uintptr_t b_wave = reinterpret_cast<uintptr_t>(B_KN ? B + (int64_t)(8 * wave) * ldb + n0 : B + b_first * ldb);
+	const uintptr_t b_wave = reinterpret_cast<uintptr_t>(B_KN ? B + (int64_t)(8 * wave) * ldb + n0 : b_of_wave + b_first * ldb);
 	const unsigned share_a = wave * (Cfg::kLoads * 1024);
 	const unsigned share_b = Cfg::BM * 128 + wave * (Cfg::kLoads * 1024);
 	const int slabs = K / 32;
@@ -172,19 +182,23 @@ __global__ __launch_bounds__(256) void gemm_f32_nt_ring_kernel(
 	{
 		const int64_t m = m0 + wm * 32 * T + i * 32 + frag_row;
 #pragma unroll
-		for (int j = 0; j < T; ++j)
+		for (int j = 0; j < (DUAL ? 1 : T); ++j)
 		{
 			const float32x_f32_t& v = i == 0 ? r0 : r1;
 #pragma unroll
 			for (int g = 0; g < 4; ++g)
 			{
-				const int64_t n = n0 + wn * 32 * T + j * 32 + 8 * g + 4 * (lane >> 5);
+				const int64_t n = n0 + wn * (DUAL ? 32 : 32 * T) + j * 32 + 8 * g + 4 * (lane >> 5);
 				float4_t out;
 #pragma unroll
 				for (int e = 0; e < 4; ++e)
 				{
-					const float bias_n = (EPI == kEpiBias && bias != nullptr && (!RAGGED || n + e < N)) ? bias[n + e] : 0.0f;
-					out[e] = finish_sum<EPI>(T == 2 ? v[16 * j + 4 * g + e] : single[4 * g + e], 0.0f, bias_n, ep_param);
+					if constexpr (DUAL) out[e] = finish_sum<EPI>(v[4 * g + e], v[16 + 4 * g + e], 0.0f, ep_param);
+					else
+					{
+						const float bias_n = (EPI == kEpiBias && bias != nullptr && (!RAGGED || n + e < N)) ? bias[n + e] : 0.0f;
+						out[e] = finish_sum<EPI>(T == 2 ? v[16 * j + 4 * g + e] : single[4 * g + e], 0.0f, bias_n, ep_param);
+					}
 				}
 				if (!RAGGED || (m < M && n + 4 <= N))
 				{
@@ -222,7 +236,8 @@ inline hipError_t launch_gemm_f32_ring(const float* A, const float* B, const flo
 {
 	const bool c_aligned = reinterpret_cast<uintptr_t>(C) % 16 == 0 && ldc % 4 == 0 && stride_c % 4 == 0;
 	using Cfg = GemmF32RingCfg<T>;
-	const bool ragged = M % Cfg::BM != 0 || N % Cfg::BN != 0 || !c_aligned;
+	constexpr int kOutN = EPI == kEpiGeluMul ? Cfg::BN / 2 : Cfg::BN;
+	const bool ragged = M % Cfg::BM != 0 || N % kOutN != 0 || !c_aligned;
 	auto kernel = ragged ? gemm_f32_nt_ring_kernel<T, true, EPI, B_KN> : gemm_f32_nt_ring_kernel<T, false, EPI, B_KN>;
 	// More than 64 KB of dynamic LDS has to be granted per function and per device, once.
 	static std::atomic<uint64_t> configured_devices[2];
@@ -237,7 +252,7 @@ inline hipError_t launch_gemm_f32_ring(const float* A, const float* B, const flo
 		if (e != hipSuccess) return e;
 		configured_devices[ragged].fetch_or(bit, std::memory_order_relaxed);
 	}
-	const int64_t tiles = ((M + Cfg::BM - 1) / Cfg::BM) * ((N + Cfg::BN - 1) / Cfg::BN);
+	const int64_t tiles = ((M + Cfg::BM - 1) / Cfg::BM) * ((N + kOutN - 1) / kOutN);
 	kernel<<<dim3((unsigned)tiles, (unsigned)batch), dim3(256), Cfg::kLdsBytes, stream>>>(
 		A, B, bias, C, M, N, (int)K, lda, ldb, ldc, stride_a, stride_b, stride_c, ep_param, (int)k_split);
 	return hipGetLastError();
