@@ -5,10 +5,9 @@
 // reads q, k, v and writes y.
 //
 // A block of 8 waves owns 128 consecutive queries of one head, 16 per wave (256 and 32 at head
-// dimension 128), so that at least two waves share a SIMD and one wave's MFMAs run under the
-// other's softmax arithmetic.  It walks the visible key range in tiles of 64 keys.  Per tile:
-//   * K and V rows go global -> LDS directly into two stages (head dimension 256 with softcap: global -> registers
-//     -> LDS, one stage); the loads of the next tile are in flight while this one is being used;
+// dimension 128), so that two waves share a SIMD.  It walks the visible key range in tiles of 64 keys.  Per tile:
+//   * K and V rows go global -> LDS directly into two stages; the loads of the next tile are in flight while
+//     this one is being used;
 //   * S^T = K Q^T with v_mfma_f32_16x16x32_f16: the K fragment is the first operand, the Q
 //     fragment (kept in registers for the whole kernel) the second, so a lane ends up holding,
 //     for ONE query (lane % 16), the scores of keys 4 (lane / 16) + r of each 16-key block.
@@ -23,6 +22,10 @@
 // slot j <-> key 16 * (2 t + j / 4) + 4 * (lane / 16) + j % 4 of the tile, so no shuffle is needed
 // between the two products.
 //
+// At head dimension 256 with softcap a second kernel of the same layout (sdp_attention_fwd_f16_skew_kernel) computes
+// the scores of tile t + 1 beside the softmax of tile t, so that the matrix and the vector instructions of a wave
+// do not depend on each other.
+//
 // Masks are index rules (causal with the diagonal at n_k - n_q, sliding window); tiles without a
 // visible key are skipped.  A query without any visible key gets zeros.
 #include "device_utils.hpp"
@@ -33,6 +36,8 @@
 
 #include <algorithm>
 #include <atomic>
+#include <type_traits>
+#include <utility>
 
 namespace anygpu {
 
@@ -90,20 +95,17 @@ struct AttnLds
 };
 
 // QB: 16-query blocks per wave, WAVES: waves per block; a block owns 16 * QB * WAVES consecutive queries.
-template <int D, bool SOFTCAP, int QB, int WAVES, bool DIRECT>
+template <int D, bool SOFTCAP, int QB, int WAVES>
 __global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f16_kernel(const AttnArgs a, const AttnWalk walk)
 {
 	constexpr int kAttnQueriesPerBlock = 16 * QB * WAVES;
-	constexpr int THREADS = 64 * WAVES;
 	extern __shared__ __align__(16) char lds[];
 	using L = AttnLds<D>;
-	// (without DIRECT: the one stage; with it these follow the stage of the tile in use)
+	// (these follow the stage of the tile in use)
 	const char* k_lds = lds;
 	const char* v_lds = lds + kAttnKeysPerTile * L::kPitchK;
 	constexpr int KS = D / 32;                      // MFMA steps along the head dimension (q k^T)
 	constexpr int DC = D / 16;                      // 16-wide column blocks of the output
-	constexpr int VPT = kAttnKeysPerTile * D / 8 / THREADS;   // 16-byte vectors per thread per tile and matrix
-	constexpr int VPR = D / 8;                      // vectors per row
 
 	const int tid = threadIdx.x;
 	const int lane = tid & (kWaveSize - 1);
@@ -174,38 +176,7 @@ __global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f16_kernel(const
 	const int all_hi = a.causal ? (wq0 + a.diag < a.n_k - 1 ? wq0 + a.diag : a.n_k - 1) : a.n_k - 1;
 	const int all_lo = a.window > 0 ? wq1 + a.diag - a.window + 1 : 0;
 
-	float4_t kr[VPT], vr[VPT];
-	// vectors [i0, i1) of this thread's share of tile t
-	auto tile_load_part = [&](int t, int i0, int i1) {
-#pragma unroll
-		for (int i = i0; i < i1; ++i)
-		{
-			const int idx = tid + THREADS * i;
-			const int row = idx / VPR, col = idx % VPR;
-			const int key = t * kAttnKeysPerTile + row;
-			float4_t kv = {}, vv = {};
-			if (key < a.n_k)
-			{
-				kv = *reinterpret_cast<const float4_t*>(kp + (int64_t)key * D + col * 8);
-				vv = *reinterpret_cast<const float4_t*>(vp + (int64_t)key * D + col * 8);
-			}
-			kr[i] = kv;
-			vr[i] = vv;
-		}
-	};
-	auto tile_load = [&](int t) { tile_load_part(t, 0, VPT); };
-	auto tile_store = [&]() {
-#pragma unroll
-		for (int i = 0; i < VPT; ++i)
-		{
-			const int idx = tid + THREADS * i;
-			const int row = idx / VPR, col = idx % VPR;
-			*reinterpret_cast<float4_t*>(lds + row * L::kPitchK + col * 16) = kr[i];
-			*reinterpret_cast<float4_t*>(lds + kAttnKeysPerTile * L::kPitchK + row * L::kPitchV + col * 16) = vr[i];
-		}
-	};
-
-	// DIRECT: tiles go global -> LDS without staging registers, into two stages.  A load instruction fills 1 KB of
+	// Tiles go global -> LDS without staging registers, into two stages.  A load instruction fills 1 KB of
 	// consecutive LDS; with padded tile rows a few of its lanes land in the padding and fetch a valid chunk nobody
 	// reads.  Load i = wave + WAVES j of a tile: this lane's 16 bytes are the chunk at byte slot_src[j] from the
 	// tile's first key.  Rows past the last key are replaced by the last one (their scores are masked, their p is
@@ -214,26 +185,23 @@ __global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f16_kernel(const
 	constexpr int kStageBytes = L::kBytes;
 	constexpr int kLoadsPerTile = kAttnKeysPerTile * L::kPitchK / 1024;
 	constexpr int kSlots = (kLoadsPerTile + WAVES - 1) / WAVES;
-	static_assert(!DIRECT || (L::kPitchK == L::kPitchV && kAttnKeysPerTile * L::kPitchK % 1024 == 0), "whole load instructions");
-	int slot_src[DIRECT ? kSlots : 1];
+	static_assert(L::kPitchK == L::kPitchV && kAttnKeysPerTile * L::kPitchK % 1024 == 0, "whole load instructions");
+	int slot_src[kSlots];
 	const int wave_s = __builtin_amdgcn_readfirstlane(wave);
-	if constexpr (DIRECT)
-	{
 #pragma unroll
-		for (int j = 0; j < kSlots; ++j)
-		{
-			const int byte = (wave_s + WAVES * j) * 1024 + lane * 16;
-			const int row = (byte / L::kPitchK) % kAttnKeysPerTile;      // (an instruction past the tile is never issued)
-			const int off = byte % L::kPitchK;
-			slot_src[j] = row * (2 * D) + (off < 2 * D ? off : 0);
-		}
+	for (int j = 0; j < kSlots; ++j)
+	{
+		const int byte = (wave_s + WAVES * j) * 1024 + lane * 16;
+		const int row = (byte / L::kPitchK) % kAttnKeysPerTile;      // (an instruction past the tile is never issued)
+		const int off = byte % L::kPitchK;
+		slot_src[j] = row * (2 * D) + (off < 2 * D ? off : 0);
 	}
 	const unsigned lds_base = (unsigned)(uintptr_t)(__attribute__((address_space(3))) char*)lds;
 	auto issue_slot = [&](int t, int stage, int j) {
 		const int i = wave_s + WAVES * j;
 		if (WAVES * j + WAVES - 1 < kLoadsPerTile || i < kLoadsPerTile)
 		{
-			int rel = slot_src[DIRECT ? j : 0];
+			int rel = slot_src[j];
 			if ((t + 1) * kAttnKeysPerTile > a.n_k)                       // block-uniform: the ragged last tile
 			{
 				const int row = rel / (2 * D);
@@ -250,39 +218,20 @@ __global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f16_kernel(const
 		}
 	};
 
-	if constexpr (DIRECT)
+	if (t_first <= t_last)
 	{
-		if (t_first <= t_last)
-		{
 #pragma unroll
-			for (int j = 0; j < kSlots; ++j) issue_slot(t_first, 0, j);
-		}
+		for (int j = 0; j < kSlots; ++j) issue_slot(t_first, 0, j);
 	}
-	else if (t_first <= t_last) tile_load(t_first);
 	for (int t = t_first; t <= t_last; ++t)
 	{
-		if constexpr (DIRECT)
-		{
-			// own loads of tile t have landed; behind the barrier everybody's have, and everybody is done with the
-			// stage of tile t - 1, which the loads of tile t + 1 overwrite
-			__builtin_amdgcn_s_waitcnt(0x0F70);        // vmcnt(0)
-			__syncthreads();
-			k_lds = lds + ((t - t_first) & 1) * kStageBytes;
-			v_lds = k_lds + kAttnKeysPerTile * L::kPitchK;
-		}
-		else
-		{
-			__syncthreads();                           // the previous tile has been read by everybody
-			tile_store();
-			__syncthreads();
-		}
-		// At head dimension 256 the next tile's loads are issued two at a time behind the key blocks of the first
-		// product: a wave that issues its eight in one burst is held until the CU's vector memory path (64 bytes per
-		// clock) has taken them, and all eight waves are then held at once.  (With one or two vectors per thread and
-		// matrix the burst is as fast; spreading the V loads over the second product as well was slower.)
+		// own loads of tile t have landed; behind the barrier everybody's have, and everybody is done with the
+		// stage of tile t - 1, which the loads of tile t + 1 overwrite
+		__builtin_amdgcn_s_waitcnt(0x0F70);            // vmcnt(0)
+		__syncthreads();
+		k_lds = lds + ((t - t_first) & 1) * kStageBytes;
+		v_lds = k_lds + kAttnKeysPerTile * L::kPitchK;
 		const bool more = t < t_last;
-		constexpr int kLoadParts = DIRECT ? 0 : VPT >= 4 ? 4 : 0;
-		if (!DIRECT && kLoadParts == 0 && more) tile_load(t + 1);
 
 		// ---- S^T = K Q^T: s[b][kb] = scores of query block b against key block kb ----
 		float4_t s[QB][4];
@@ -299,18 +248,12 @@ __global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f16_kernel(const
 #pragma unroll
 				for (int b = 0; b < QB; ++b)
 					s[b][kb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf, qf[b][st], s[b][kb], 0, 0, 0);
-				if constexpr (kLoadParts > 0)
+				// the next tile's loads, spread behind the key blocks of this product: a wave that issues them in one
+				// burst is held until the CU's vector memory path (64 bytes per clock) has taken them
+				if (st == KS - 1 && more)
 				{
-					if (st == KS - 1 && more) tile_load_part(t + 1, kb * (VPT / kLoadParts), (kb + 1) * (VPT / kLoadParts));
-				}
-				if constexpr (DIRECT)
-				{
-					// the next tile's loads, spread behind the key blocks of this product
-					if (st == KS - 1 && more)
-					{
 #pragma unroll
-						for (int j = kb; j < kSlots; j += 4) issue_slot(t + 1, (t + 1 - t_first) & 1, j);
-					}
+					for (int j = kb; j < kSlots; j += 4) issue_slot(t + 1, (t + 1 - t_first) & 1, j);
 				}
 			}
 
@@ -431,12 +374,373 @@ __global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f16_kernel(const
 	}
 }
 
-template <int D, bool SOFTCAP, int QB, bool DIRECT = false>
+// The same product with the two halves of a tile's work taken from DIFFERENT tiles, so that matrix and vector
+// instructions of one wave have no dependence on each other and can issue side by side:
+//     step A of tile t:  S(t + 1) = K(t + 1) Q^T  (MFMA + LDS reads)   beside   max, exp2, sum, fp16 of z(t)  (VALU)
+//     step B of tile t:  O += V(t)^T P(t)^T        (MFMA + LDS reads)   beside   z(t + 1) = mask(softcap(S(t + 1)))  (VALU)
+// In the kernel above every wave of the block multiplies, then exponentiates, then multiplies (the barriers of a
+// tile keep the eight waves in step), so the matrix cores idle while the VALU works and the other way round.  The
+// LDS holds K of tile t + 1 next to V of tile t; tiles pass through registers, 16 queries per wave.
+template <int D, bool SOFTCAP, int QB, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f16_skew_kernel(const AttnArgs a, const AttnWalk walk)
+{
+	constexpr int kAttnQueriesPerBlock = 16 * QB * WAVES;
+	extern __shared__ __align__(16) char lds[];
+	using L = AttnLds<D>;
+	constexpr int KS = D / 32;
+	constexpr int DC = D / 16;
+
+	const int tid = threadIdx.x;
+	const int lane = tid & (kWaveSize - 1);
+	const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+	const int n = lane & 15;
+	const int g = lane >> 4;
+	int bh, q_block, part, parts, split_slot;
+	if (!attn_walk_locate_part(walk, blockIdx.x, bh, q_block, part, parts, split_slot)) return;
+	const int q0 = q_block * kAttnQueriesPerBlock;
+	const half_t* qp = a.q + (int64_t)bh * a.n_q * D;
+	const half_t* kp = a.k + (int64_t)(bh / a.q_per_kv) * a.n_k * D;
+	const half_t* vp = a.v + (int64_t)(bh / a.q_per_kv) * a.n_k * D;
+	half_t* yp = a.y + (int64_t)bh * a.n_q * D;
+
+	const int q_last = (q0 + kAttnQueriesPerBlock - 1 < a.n_q ? q0 + kAttnQueriesPerBlock - 1 : a.n_q - 1);
+	int key_hi = a.n_k - 1;
+	if (a.causal && q_last + a.diag < key_hi) key_hi = q_last + a.diag;
+	int key_lo = 0;
+	if (a.window > 0 && q0 + a.diag - a.window + 1 > 0) key_lo = q0 + a.diag - a.window + 1;
+	int t_first = key_lo / kAttnKeysPerTile;
+	int t_last = key_hi >= 0 ? key_hi / kAttnKeysPerTile : -1;
+	if (parts == 2)
+	{
+		const int mid = t_first + (t_last - t_first + 2) / 2;
+		if (part == 0) t_last = mid - 1;
+		else t_first = mid;
+	}
+
+	// this wave's queries as second operands: lane (n, g) holds q[row][32 s + 8 g .. + 7]
+	int q_row[QB], vis_lo[QB], vis_hi[QB];
+	half8_t qf[QB][KS];
+#pragma unroll
+	for (int b = 0; b < QB; ++b)
+	{
+		q_row[b] = q0 + 16 * QB * wave + 16 * b + n;
+#pragma unroll
+		for (int s = 0; s < KS; ++s)
+		{
+			half8_t val = {};
+			if (q_row[b] < a.n_q) val = *reinterpret_cast<const half8_t*>(qp + (int64_t)q_row[b] * D + 32 * s + 8 * g);
+			qf[b][s] = val;
+		}
+		vis_hi[b] = a.causal ? q_row[b] + a.diag : a.n_k - 1;
+		if (vis_hi[b] > a.n_k - 1) vis_hi[b] = a.n_k - 1;
+		vis_lo[b] = a.window > 0 ? q_row[b] + a.diag - a.window + 1 : 0;
+	}
+	// keys visible to every query of this wave need no per-element test: [all_lo, all_hi]
+	const int wq0 = q0 + 16 * QB * wave, wq1 = wq0 + 16 * QB - 1;
+	const int all_hi = a.causal ? (wq0 + a.diag < a.n_k - 1 ? wq0 + a.diag : a.n_k - 1) : a.n_k - 1;
+	const int all_lo = a.window > 0 ? wq1 + a.diag - a.window + 1 : 0;
+
+	float m_run[QB], m_new[QB], l_run[QB];         // l_run: this lane's share of the row sum
+	float4_t o[QB][DC];
+#pragma unroll
+	for (int b = 0; b < QB; ++b)
+	{
+		m_run[b] = -INFINITY;
+		l_run[b] = 0.0f;
+#pragma unroll
+		for (int c = 0; c < DC; ++c) o[b][c] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+	}
+
+	// Tiles go global -> LDS without staging registers, K and V in two stages each.  A load instruction fills 1 KB
+	// of consecutive LDS; with padded tile rows a few of its lanes land in the padding and fetch a valid chunk
+	// nobody reads.  Load i = wave + WAVES j of a tile: this lane's 16 bytes are the chunk at byte slot_src[j]
+	// from the tile's first key.  Rows past the last key are replaced by the last one (their scores are masked,
+	// their p is 0).  Written as assembly: the compiler would make every transposing LDS read wait for all
+	// outstanding direct loads of the wave; the waits they need are the explicit ones in front of the barrier.
+	constexpr int kStageBytes = L::kBytes;
+	constexpr int kLoadsPerTile = kAttnKeysPerTile * L::kPitchK / 1024;
+	constexpr int kSlots = (kLoadsPerTile + WAVES - 1) / WAVES;
+	static_assert(L::kPitchK == L::kPitchV && kAttnKeysPerTile * L::kPitchK % 1024 == 0, "whole load instructions");
+	// (slot_ragged: the same for the tile that holds the last key when it is not a whole tile)
+	int slot_src[kSlots], slot_ragged[kSlots];
+	const int t_ragged = a.n_k % kAttnKeysPerTile != 0 ? a.n_k / kAttnKeysPerTile : -1;
+#pragma unroll
+	for (int j = 0; j < kSlots; ++j)
+	{
+		const int byte = (wave + WAVES * j) * 1024 + lane * 16;
+		const int row = (byte / L::kPitchK) % kAttnKeysPerTile;      // (an instruction past the tile is never issued)
+		const int off = byte % L::kPitchK;
+		slot_src[j] = row * (2 * D) + (off < 2 * D ? off : 0);
+		const int last = a.n_k - 1 - t_ragged * kAttnKeysPerTile;
+		slot_ragged[j] = slot_src[j] - (row > last ? (row - last) * (2 * D) : 0);
+	}
+	const unsigned lds_base = (unsigned)(uintptr_t)(__attribute__((address_space(3))) char*)lds;
+	// slot j of tile t of matrix `src` into the K (which = 0) or V (which = 1) part of a stage.  The waves that have
+	// no load in the last slot skip it inside the statement, so that the code around it stays one scheduling region.
+	// The statements claim no memory effect (LDS reads may be scheduled across them: they fill the stage that is
+	// not being read); what keeps them between the barrier of their tile and the wait of the next is the token they
+	// hand from one to the next.
+	int token = 0;
+	auto issue_slot = [&](const half_t* src, int which, int t, int stage, int j) {
+		const int i = wave + WAVES * j;
+		const int rel = t == t_ragged ? slot_ragged[j] : slot_src[j];
+		const char* base = (const char*)src + (int64_t)t * (kAttnKeysPerTile * 2 * D);
+		const unsigned m0v = lds_base + stage * kStageBytes + which * (kAttnKeysPerTile * L::kPitchK) + i * 1024;
+		if (WAVES * j + WAVES - 1 < kLoadsPerTile)
+			asm("s_mov_b32 m0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : "+s"(token) : "v"(rel), "s"(base), "s"(m0v) : "m0");
+		else
+			asm("s_cmp_lt_u32 %4, %5\n\ts_cbranch_scc0 1f\n\ts_mov_b32 m0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2\n1:"
+			    : "+s"(token) : "v"(rel), "s"(base), "s"(m0v), "s"(i), "n"(kLoadsPerTile) : "m0", "scc");
+	};
+	// own loads have landed; behind the barrier everybody's have, and everybody is done with what the loads issued
+	// after it overwrite
+	auto tile_barrier = [&]() {
+		asm volatile("s_waitcnt vmcnt(0)" : : "s"(token) : "memory");
+		__syncthreads();
+		asm volatile("" : "=s"(token));
+	};
+	// z of score e = 4 kb + r of query block b against tile t: scale / softcap in the log2 domain, masked keys at -inf
+	auto logit_of_score = [&](auto interior_tag, float sv, int t, int b, int e) {
+		const float zz = logit2<SOFTCAP>(sv, a.k_in, a.k_cap);
+		if constexpr (decltype(interior_tag)::value) return zz;
+		else
+		{
+			// (a sum, so that the transform is not made conditional on the mask)
+			const int key = t * kAttnKeysPerTile + 16 * (e / 4) + 4 * g + e % 4;
+			return zz + ((key >= vis_lo[b] && key <= vis_hi[b]) ? 0.0f : -INFINITY);
+		}
+	};
+	auto is_interior = [&](int t) {
+		const int key0 = t * kAttnKeysPerTile;
+		return key0 >= all_lo && key0 + kAttnKeysPerTile - 1 <= all_hi;
+	};
+
+	float z[QB][16];
+	// running maximum including tile t (m_run: through tile t - 1); known one tile ahead, like z
+	auto row_max = [&](int b) {
+		float mt = -INFINITY;
+#pragma unroll
+		for (int e = 0; e < 16; ++e) mt = fmaxf(mt, z[b][e]);
+		return fmaxf(m_run[b], max_over_lane_rows(mt));
+	};
+	if (t_first <= t_last)
+	{
+#pragma unroll
+		for (int j = 0; j < kSlots; ++j)
+		{
+			issue_slot(kp, 0, t_first, 0, j);
+			issue_slot(vp, 1, t_first, 0, j);
+		}
+		tile_barrier();
+		if (t_first < t_last)
+		{
+#pragma unroll
+			for (int j = 0; j < kSlots; ++j) issue_slot(kp, 0, t_first + 1, 1, j);
+		}
+#pragma unroll
+		for (int kb = 0; kb < 4; ++kb)
+		{
+			float4_t acc[QB];
+#pragma unroll
+			for (int b = 0; b < QB; ++b) acc[b] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+			for (int st = 0; st < KS; ++st)
+			{
+				const half8_t kf = *reinterpret_cast<const half8_t*>(lds + (16 * kb + n) * L::kPitchK + (32 * st + 8 * g) * 2);
+#pragma unroll
+				for (int b = 0; b < QB; ++b) acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf, qf[b][st], acc[b], 0, 0, 0);
+			}
+#pragma unroll
+			for (int b = 0; b < QB; ++b)
+#pragma unroll
+				for (int r = 0; r < 4; ++r) z[b][4 * kb + r] = logit_of_score(std::false_type{}, acc[b][r], t_first, b, 4 * kb + r);
+		}
+	}
+#pragma unroll
+	for (int b = 0; b < QB; ++b) m_new[b] = t_first <= t_last ? row_max(b) : -INFINITY;
+
+	// One tile.  MORE: tile t + 1 exists (its K is on its way into the other stage); INTERIOR: every key of tile
+	// t + 1 is visible to every query of the wave.  Apart from the rescale at its top the tile is one stretch of
+	// code without branches.
+	auto tile = [&](auto more_tag, auto interior_tag, int t) {
+		constexpr bool MORE = decltype(more_tag)::value;
+		// the running maximum settles after a few tiles; when no query of the wave raised it, the rescale factor
+		// is 1 everywhere and the pass over the accumulators is skipped
+		float m_safe[QB];
+#pragma unroll
+		for (int b = 0; b < QB; ++b)
+		{
+			m_safe[b] = (m_new[b] == -INFINITY) ? 0.0f : m_new[b];   // nothing visible so far: every term is exp2(-inf) = 0
+			if (__builtin_amdgcn_ballot_w64(m_new[b] > m_run[b]) != 0)
+			{
+				const float corr = fast_exp2(m_run[b] - m_safe[b]);
+				l_run[b] *= corr;
+#pragma unroll
+				for (int c = 0; c < DC; ++c) o[b][c] *= corr;
+			}
+			m_run[b] = m_new[b];
+		}
+		// K(t + 1) and V(t) have landed; K(t) and V(t - 1) are free for the loads issued below
+		tile_barrier();
+		const int stage = (t - t_first) & 1;
+		const char* k_next = lds + (stage ^ 1) * kStageBytes;
+		const char* v_lds = lds + stage * kStageBytes + kAttnKeysPerTile * L::kPitchK;
+		const int t_k = t + 2 <= t_last ? t + 2 : t_last;       // (past the end: the last tile once more, into the free stage)
+
+		// The tile as 64 steps of one operand out of LDS and the QB MFMAs that use it, 32 of S(t + 1) = K(t + 1) Q^T (the
+		// four key blocks in turn, so that consecutive MFMAs do not wait for each other's result) and 32 of
+		// O^T += V(t)^T P(t)^T.  Behind its MFMAs a step issues the LDS reads of the operand kAhead steps later and
+		// does its share of the vector work: in the first half p(t) = exp2(z(t) - m), one score per query block every
+		// other step, in the second z(t + 1) likewise; the loads of the next tiles go out one slot every other step.
+		// The scheduler may reorder inside a step, not across steps.
+		constexpr int kAhead = 4;                                  // (6 and 8 measured slower: registers)
+		constexpr int kLoadSpacing = 6 < (4 * KS + 2 * DC) / (2 * kSlots) ? 6 : (4 * KS + 2 * DC) / (2 * kSlots);
+		constexpr int kStepsA = MORE ? 4 * KS : 0, kSteps = kStepsA + 2 * DC;
+		half8_t frag[kAhead];
+		auto read_operand = [&](int i) {
+			if (i < kStepsA)
+			{
+				const int st = i / 4, kb = i % 4;
+				return *reinterpret_cast<const half8_t*>(k_next + (16 * kb + n) * L::kPitchK + (32 * st + 8 * g) * 2);
+			}
+			const int tt = (i - kStepsA) / DC, c = (i - kStepsA) % DC;
+			const char* src = v_lds + (32 * tt + 4 * g + (n >> 2)) * L::kPitchV + (16 * c + 4 * (n & 3)) * 2;
+			const half4_t lo = lds_read_tr_b64(src);
+			const half4_t hi = lds_read_tr_b64(src + 16 * L::kPitchV);
+			return (half8_t)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+		};
+		float4_t s_next[QB][4];
+		float psum[QB];
+		half8_t pf[QB][2];
+#pragma unroll
+		for (int b = 0; b < QB; ++b)
+		{
+			psum[b] = 0.0f;
+#pragma unroll
+			for (int kb = 0; kb < 4; ++kb) s_next[b][kb] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+		}
+		auto p_of_score = [&](int b, int e) {
+			const float pv = fast_exp2(z[b][e] - m_safe[b]);
+			psum[b] += pv;
+			pf[b][e / 8][e % 8] = (half_t)pv;
+		};
+#pragma unroll
+		for (int i = 0; i < kAhead; ++i) frag[i] = read_operand(i);
+		if constexpr (!MORE)
+		{
+#pragma unroll
+			for (int b = 0; b < QB; ++b)
+#pragma unroll
+				for (int e = 0; e < 16; ++e) p_of_score(b, e);
+		}
+		__builtin_amdgcn_sched_barrier(0);
+		// (the step number as a type: every index below is a constant, whatever the optimiser makes of the loop)
+		auto step = [&](auto step_tag) {
+			constexpr int i = decltype(step_tag)::value;
+#pragma unroll
+			for (int b = 0; b < QB; ++b)
+			{
+				if (i < kStepsA) s_next[b][i % 4] = __builtin_amdgcn_mfma_f32_16x16x32_f16(frag[i % kAhead], qf[b][i / 4], s_next[b][i % 4], 0, 0, 0);
+				else o[b][(i - kStepsA) % DC] = __builtin_amdgcn_mfma_f32_16x16x32_f16(frag[i % kAhead], pf[b][(i - kStepsA) / DC], o[b][(i - kStepsA) % DC], 0, 0, 0);
+			}
+			if (i + kAhead < kSteps) frag[i % kAhead] = read_operand(i + kAhead);
+			if constexpr (MORE)
+			{
+				// the next tiles' loads, one every kLoadSpacing steps: a burst holds the wave at each load until the
+				// CU's vector memory path (64 bytes per clock) has taken the ones in front of it
+				if (i % kLoadSpacing == 1 && i / kLoadSpacing < 2 * kSlots)
+				{
+					const int m = i / kLoadSpacing;
+					if (m % 2 == 0) issue_slot(vp, 1, t + 1, stage ^ 1, m / 2);
+					else issue_slot(kp, 0, t_k, stage, m / 2);
+				}
+				// (the 16 scores of a query block spread evenly over the steps of each half)
+				if (i < kStepsA)
+				{
+#pragma unroll
+					for (int u = 0; u < (16 + kStepsA - 1) / kStepsA; ++u)
+#pragma unroll
+						for (int b = 0; b < QB; ++b)
+							if (i * 16 / kStepsA + u < (i + 1) * 16 / kStepsA) p_of_score(b, i * 16 / kStepsA + u);
+				}
+				else
+				{
+					constexpr int kStepsB = 2 * DC;
+#pragma unroll
+					for (int u = 0; u < (16 + kStepsB - 1) / kStepsB; ++u)
+#pragma unroll
+						for (int b = 0; b < QB; ++b)
+						{
+							const int e = (i - kStepsA) * 16 / kStepsB + u;
+							if (e < (i - kStepsA + 1) * 16 / kStepsB) z[b][e] = logit_of_score(interior_tag, s_next[b][e / 4][e % 4], t + 1, b, e);
+						}
+				}
+			}
+			__builtin_amdgcn_sched_barrier(0);
+		};
+		[&]<int... I>(std::integer_sequence<int, I...>) { (step(std::integral_constant<int, I>{}), ...); }(std::make_integer_sequence<int, kSteps>{});
+#pragma unroll
+		for (int b = 0; b < QB; ++b)
+		{
+			l_run[b] += psum[b];
+			if constexpr (MORE) m_new[b] = row_max(b);
+		}
+	};
+	for (int t = t_first; t < t_last; ++t)
+	{
+		if (is_interior(t + 1)) tile(std::true_type{}, std::true_type{}, t);
+		else tile(std::true_type{}, std::false_type{}, t);
+	}
+	if (t_first <= t_last) tile(std::false_type{}, std::true_type{}, t_last);
+
+	// ---- normalise and store: lane (n, g) holds y[row][16 c + 4 g .. + 3] ----
+#pragma unroll
+	for (int b = 0; b < QB; ++b)
+	{
+		float l = l_run[b];
+		l += __shfl_xor(l, 16);
+		l += __shfl_xor(l, 32);
+		if (parts == 2)
+		{
+			// unnormalised accumulators, running maximum and sum of this half of the keys
+			if (q_row[b] < a.n_q)
+			{
+				float* dst = a.partials + ((((int64_t)bh * walk.n_split + split_slot) * 2 + part) * kAttnQueriesPerBlock + (q_row[b] - q0)) * (D + 2);
+#pragma unroll
+				for (int c = 0; c < DC; ++c) *reinterpret_cast<WsFloat4*>(dst + 16 * c + 4 * g) = o[b][c];
+				if (g == 0)
+				{
+					dst[D] = m_run[b];
+					dst[D + 1] = l;
+				}
+			}
+			continue;
+		}
+		const float inv = l > 0.0f ? 1.0f / l : 0.0f;
+		if (q_row[b] < a.n_q)
+		{
+#pragma unroll
+			for (int c = 0; c < DC; ++c)
+			{
+				half4_t out;
+#pragma unroll
+				for (int r = 0; r < 4; ++r) out[r] = (half_t)(o[b][c][r] * inv);
+				*reinterpret_cast<half4_t*>(yp + (int64_t)q_row[b] * D + 16 * c + 4 * g) = out;
+			}
+		}
+	}
+}
+
+// SKEW: the kernel that takes the two halves of a tile's work from different tiles
+template <int D, bool SOFTCAP, int QB, bool SKEW = false>
 hipError_t launch_variant(const AttnArgs& args_in, int64_t batch_heads, hipStream_t stream)
 {
 	constexpr int WAVES = 8;
-	auto kernel = sdp_attention_fwd_f16_kernel<D, SOFTCAP, QB, WAVES, DIRECT>;
-	constexpr int kLdsBytes = AttnLds<D>::kBytes * (DIRECT ? 2 : 1);
+	auto kernel = [] {
+		if constexpr (SKEW) return sdp_attention_fwd_f16_skew_kernel<D, SOFTCAP, QB, WAVES>;
+		else return sdp_attention_fwd_f16_kernel<D, SOFTCAP, QB, WAVES>;
+	}();
+	constexpr int kLdsBytes = 2 * AttnLds<D>::kBytes;           // two stages
 	constexpr int kQueriesPerBlock = 16 * QB * WAVES;
 	(void)hipGetLastError();
 	if (kLdsBytes > 64 * 1024)
@@ -479,27 +783,24 @@ hipError_t launch_variant(const AttnArgs& args_in, int64_t batch_heads, hipStrea
 // register footprint lets more waves share a SIMD), except head_dim 128 with enough query blocks to fill the chip,
 // where 8 waves x 32 queries halve the LDS reads per flop and fit the register file (16 x 4096 x 128 causal: 148 us
 // against 172 us).  At head_dim 256 the 32-query form does not fit the registers.
+// The skewed kernel is used where the softmax arithmetic is a large share of a tile, head_dim 256 with softcap
+// (8 / 4 heads x 8192 x 256, softcap 50, window 4096: 321 -> 306 us in one process; full causal 438 -> 410 us).  Measured
+// against the kernel above on one GPU it loses elsewhere: head_dim 256 without softcap 390 -> 397 us, head_dim
+// 128 (16 x 4096 causal) 128 -> 141 us, head_dim 64 (32 x 2048 causal) 45 -> 61 us; with 32 queries per wave it
+// loses at every head dimension.
 template <int D>
 hipError_t launch_dim(const AttnArgs& args, bool softcap, int64_t batch_heads, hipStream_t stream)
 {
-	// Tiles go global -> LDS directly (two stages, no staging registers, one barrier per tile) at head_dim 64 and 128
-	// (16 x 4096 x 128 causal: 157 -> 141 us, with softcap 198 -> 182 us; 32 x 2048 x 64: 43 -> 41 us) and, at head_dim
-	// 256, without softcap (8 x 8192 x 256 causal: 384 -> 350 us); with it, where the softmax arithmetic weighs
-	// more, the same form measured 2 % slower than staging through registers.
 	if constexpr (D == 128)
 	{
 		if (batch_heads * ((args.n_q + 255) / 256) >= 256)
-			return softcap ? launch_variant<D, true, 2, true>(args, batch_heads, stream) : launch_variant<D, false, 2, true>(args, batch_heads, stream);
+			return softcap ? launch_variant<D, true, 2>(args, batch_heads, stream) : launch_variant<D, false, 2>(args, batch_heads, stream);
 	}
-	if constexpr (D != 256)
+	if constexpr (D == 256)
 	{
-		return softcap ? launch_variant<D, true, 1, true>(args, batch_heads, stream) : launch_variant<D, false, 1, true>(args, batch_heads, stream);
+		if (softcap) return launch_variant<D, true, 1, true>(args, batch_heads, stream);
 	}
-	else
-	{
-		if (!softcap) return launch_variant<D, false, 1, true>(args, batch_heads, stream);
-		return launch_variant<D, true, 1>(args, batch_heads, stream);
-	}
+	return softcap ? launch_variant<D, true, 1>(args, batch_heads, stream) : launch_variant<D, false, 1>(args, batch_heads, stream);
 }
 
 // ---------------------------------------------------------------------------------------------

@@ -1483,6 +1483,39 @@ def test_sdp_attention_fused_kernel_random_shapes(ops, oracle, dtype):
         assert scaled_rel_err(got[0], want, 1.0) <= tol, case
 
 
+# head_dim 256 with softcap runs the kernel that takes S of tile t + 1 beside the softmax of tile t: tile counts of
+# one and two (the pipelined loop body not entered / entered once), a last tile that is not whole, a key range longer
+# than the queries, windows below a tile and without the causal rule, queries without a visible key, grouped heads
+ATTN_D256_SOFTCAP_CASES = [
+    (2, 2, 17, 63, 256, 0.0625, 50.0, True, 0),
+    (2, 2, 17, 64, 256, 0.0625, 50.0, True, 0),
+    (2, 2, 20, 65, 256, 0.0625, 50.0, False, 0),
+    (2, 1, 128, 128, 256, 0.0625, 30.0, True, 0),
+    (2, 1, 129, 129, 256, 0.0625, 30.0, True, 0),
+    (4, 2, 200, 333, 256, 0.0625, 50.0, True, 0),
+    (2, 2, 300, 300, 256, -0.05, 50.0, True, 33),
+    (2, 2, 260, 260, 256, 0.0625, 50.0, False, 70),
+    (2, 2, 100, 40, 256, 0.0625, 50.0, True, 0),
+    (8, 2, 640, 700, 256, 0.0625, 50.0, True, 200),
+]
+
+
+@pytest.mark.parametrize("case", ATTN_D256_SOFTCAP_CASES)
+def test_sdp_attention_fused_kernel_head_dim_256_with_softcap(ops, oracle, case):
+    heads, kv_heads, n_q, n_k, d, alpha, cap, causal, window = case
+    q = synth.normal(1 + n_q, (1, heads, n_q, d)).astype(np.float16)
+    k = synth.normal(2 + n_k, (1, kv_heads, n_k, d)).astype(np.float16)
+    v = synth.normal(3 + d, (1, kv_heads, n_k, d)).astype(np.float16)
+    got = host(ops.sdp_attention_fwd(dev(q), dev(k), dev(v), alpha, softcap=cap, causal=causal, window=window)).astype(np.float32)
+    want = oracle.sdp_attention_rules(*(oracle.cvt_f16_to_f32(t)[0] for t in (q, k, v)), alpha=alpha, softcap=cap,
+                                      causal=causal, window=window, q_per_kv=heads // kv_heads, threads=8)
+    assert got.shape == (1, heads, n_q, d)
+    blind = ~np.isfinite(want).all(axis=-1)                      # queries without a visible key: zeros
+    assert not got[0][blind].any()
+    assert np.isfinite(got).all()
+    assert scaled_rel_err(got[0][~blind], want[~blind], 1.0) <= TOL_F16_ROWOPS * 2, case
+
+
 @pytest.mark.parametrize("case", ATTN_CASES)
 def test_sdp_attention_fused_kernel_f32(ops, oracle, case):
     # the float32 form of the same kernel: fp32 operands and the fp32 matrix instruction, fp32 tolerance
