@@ -500,14 +500,18 @@ __global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f16_skew_kernel(
 		asm volatile("" : "=s"(token));
 	};
 	// z of score e = 4 kb + r of query block b against tile t: scale / softcap in the log2 domain, masked keys at -inf
-	auto logit_of_score = [&](auto interior_tag, float sv, int t, int b, int e) {
+	auto logit_of_score = [&](auto interior_tag, float sv, int t, int b, int e, int g) {
 		const float zz = logit2<SOFTCAP>(sv, a.k_in, a.k_cap);
 		if constexpr (decltype(interior_tag)::value) return zz;
 		else
 		{
-			// (a sum, so that the transform is not made conditional on the mask)
+			// (a sum, so that the transform is not made conditional on the mask; the bounds pass through an empty
+			// statement, so that the compiler does not keep sixteen pre-combined pairs of them in registers over the
+			// whole kernel)
+			int lo = vis_lo[b], hi = vis_hi[b];
+			asm volatile("" : "+v"(lo), "+v"(hi));
 			const int key = t * kAttnKeysPerTile + 16 * (e / 4) + 4 * g + e % 4;
-			return zz + ((key >= vis_lo[b] && key <= vis_hi[b]) ? 0.0f : -INFINITY);
+			return zz + ((key >= lo && key <= hi) ? 0.0f : -INFINITY);
 		}
 	};
 	auto is_interior = [&](int t) {
@@ -553,7 +557,7 @@ __global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f16_skew_kernel(
 #pragma unroll
 			for (int b = 0; b < QB; ++b)
 #pragma unroll
-				for (int r = 0; r < 4; ++r) z[b][4 * kb + r] = logit_of_score(std::false_type{}, acc[b][r], t_first, b, 4 * kb + r);
+				for (int r = 0; r < 4; ++r) z[b][4 * kb + r] = logit_of_score(std::false_type{}, acc[b][r], t_first, b, 4 * kb + r, g);
 		}
 	}
 #pragma unroll
@@ -582,6 +586,12 @@ __global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f16_skew_kernel(
 		}
 		// K(t + 1) and V(t) have landed; K(t) and V(t - 1) are free for the loads issued below
 		tile_barrier();
+		// (the lane's coordinates derived again from a thread number the compiler takes for a new value: a handful of
+		// instructions per tile, and the registers they and the addresses made of them would occupy over the whole
+		// kernel are free)
+		int tid_again = threadIdx.x;
+		asm volatile("" : "+v"(tid_again));
+		const int n = tid_again & 15, g = (tid_again & (kWaveSize - 1)) >> 4;
 		const int stage = (t - t_first) & 1;
 		const char* k_next = lds + (stage ^ 1) * kStageBytes;
 		const char* v_lds = lds + stage * kStageBytes + kAttnKeysPerTile * L::kPitchK;
@@ -593,7 +603,8 @@ __global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f16_skew_kernel(
 		// does its share of the vector work: in the first half p(t) = exp2(z(t) - m), one score per query block every
 		// other step, in the second z(t + 1) likewise; the loads of the next tiles go out one slot every other step.
 		// The scheduler may reorder inside a step, not across steps.
-		constexpr int kAhead = 4;                                  // (6 and 8 measured slower: registers)
+		// (2 to 5 steps ahead measure alike, 6 and 8 slower; the boundary tiles, with their masks, have registers for 2)
+		constexpr int kAhead = decltype(interior_tag)::value ? 4 : 2;
 		constexpr int kLoadSpacing = 6 < (4 * KS + 2 * DC) / (2 * kSlots) ? 6 : (4 * KS + 2 * DC) / (2 * kSlots);
 		constexpr int kStepsA = MORE ? 4 * KS : 0, kSteps = kStepsA + 2 * DC;
 		half8_t frag[kAhead];
@@ -672,7 +683,7 @@ __global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f16_skew_kernel(
 						for (int b = 0; b < QB; ++b)
 						{
 							const int e = (i - kStepsA) * 16 / kStepsB + u;
-							if (e < (i - kStepsA + 1) * 16 / kStepsB) z[b][e] = logit_of_score(interior_tag, s_next[b][e / 4][e % 4], t + 1, b, e);
+							if (e < (i - kStepsA + 1) * 16 / kStepsB) z[b][e] = logit_of_score(interior_tag, s_next[b][e / 4][e % 4], t + 1, b, e, g);
 						}
 				}
 			}
@@ -694,21 +705,27 @@ __global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f16_skew_kernel(
 	if (t_first <= t_last) tile(std::false_type{}, std::true_type{}, t_last);
 
 	// ---- normalise and store: lane (n, g) holds y[row][16 c + 4 g .. + 3] ----
+	// (the lane's coordinates are derived again, from a thread number the compiler takes for a new value, so that
+	// nothing of them has to stay in registers over the tiles, where none is free)
+	int tid_again = threadIdx.x;
+	asm volatile("" : "+v"(tid_again));
+	const int n_out = tid_again & 15, g_out = (tid_again & (kWaveSize - 1)) >> 4;
 #pragma unroll
 	for (int b = 0; b < QB; ++b)
 	{
+		const int row_out = q0 + 16 * QB * wave + 16 * b + n_out;
 		float l = l_run[b];
 		l += __shfl_xor(l, 16);
 		l += __shfl_xor(l, 32);
 		if (parts == 2)
 		{
 			// unnormalised accumulators, running maximum and sum of this half of the keys
-			if (q_row[b] < a.n_q)
+			if (row_out < a.n_q)
 			{
-				float* dst = a.partials + ((((int64_t)bh * walk.n_split + split_slot) * 2 + part) * kAttnQueriesPerBlock + (q_row[b] - q0)) * (D + 2);
+				float* dst = a.partials + ((((int64_t)bh * walk.n_split + split_slot) * 2 + part) * kAttnQueriesPerBlock + (row_out - q0)) * (D + 2);
 #pragma unroll
-				for (int c = 0; c < DC; ++c) *reinterpret_cast<WsFloat4*>(dst + 16 * c + 4 * g) = o[b][c];
-				if (g == 0)
+				for (int c = 0; c < DC; ++c) *reinterpret_cast<WsFloat4*>(dst + 16 * c + 4 * g_out) = o[b][c];
+				if (g_out == 0)
 				{
 					dst[D] = m_run[b];
 					dst[D + 1] = l;
@@ -717,7 +734,7 @@ __global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f16_skew_kernel(
 			continue;
 		}
 		const float inv = l > 0.0f ? 1.0f / l : 0.0f;
-		if (q_row[b] < a.n_q)
+		if (row_out < a.n_q)
 		{
 #pragma unroll
 			for (int c = 0; c < DC; ++c)
@@ -725,7 +742,7 @@ __global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f16_skew_kernel(
 				half4_t out;
 #pragma unroll
 				for (int r = 0; r < 4; ++r) out[r] = (half_t)(o[b][c][r] * inv);
-				*reinterpret_cast<half4_t*>(yp + (int64_t)q_row[b] * D + 16 * c + 4 * g) = out;
+				*reinterpret_cast<half4_t*>(yp + (int64_t)row_out * D + 16 * c + 4 * g_out) = out;
 			}
 		}
 	}

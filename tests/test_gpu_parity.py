@@ -1798,6 +1798,8 @@ def _graph_problem(ops):
     cw, cb = dev(synth.normal(3, (16, 4)).astype(np.float16)), dev(synth.normal(4, (16,)).astype(np.float16))
     q = torch.empty((1, 4, 100, 128), device="cuda")
     kv = dev(synth.normal(5, (1, 2, 100, 128)))
+    q16 = torch.empty((1, 4, 150, 256), device="cuda", dtype=torch.float16)     # head_dim 256 with softcap: its own kernel
+    kv16 = dev(synth.normal(6, (1, 2, 150, 256)).astype(np.float16))
 
     def fill(seed):
         a32.copy_(dev(synth.uniform(seed, tuple(a32.shape))))
@@ -1805,13 +1807,15 @@ def _graph_problem(ops):
         sc.copy_(dev((synth.normal(seed + 2, tuple(sc.shape)) * np.float32(4.0)).astype(np.float16)))
         cx.copy_(dev(synth.normal(seed + 3, tuple(cx.shape)).astype(np.float16)))
         q.copy_(dev(synth.normal(seed + 4, tuple(q.shape))))
+        q16.copy_(dev(synth.normal(seed + 5, tuple(q16.shape)).astype(np.float16)))
 
     def work():
         return (ops.tensor_mm(a32, w32),
                 ops.tensor_mm(a16, w16, b_layout=capi.B_COL_MAJOR),
                 ops.tensor_softmax(sc, alpha=0.125, causal=True, q_len=64),
                 ops.tensor_causal_conv1d(cx, cw, cb),
-                ops.sdp_attention_fwd(q, kv, kv, 0.0884, softcap=30.0, causal=True, window=40))
+                ops.sdp_attention_fwd(q, kv, kv, 0.0884, softcap=30.0, causal=True, window=40),
+                ops.sdp_attention_fwd(q16, kv16, kv16, 0.0625, softcap=50.0, causal=True, window=70))
 
     return fill, work
 
