@@ -178,10 +178,15 @@ __global__ __launch_bounds__(256) void gemm_f16_nt_ring_kernel(
 #undef ANYGPU_RING_INPUTS
 #undef ANYGPU_RING_CLOBBERS
 
+	// (the lane number is derived again, from a thread number the compiler takes for a new value: the loop leaves it
+	// no register to carry one through, and a spilled value would make the kernel a user of scratch memory)
+	int tid_after = threadIdx.x;
+	asm volatile("" : "+v"(tid_after));
+	const int lane_after = tid_after & 63;
 	if (probe != nullptr)
 	{
 		const unsigned long long clock_out = __builtin_amdgcn_s_memtime(), ticks_out = __builtin_amdgcn_s_memrealtime();
-		if (tid == 0 && blockIdx.y == 0)
+		if (tid_after == 0 && blockIdx.y == 0)
 		{
 			unsigned long long* slot = probe + 4 * (size_t)blockIdx.x;
 			slot[0] = clock_in;
@@ -197,7 +202,7 @@ __global__ __launch_bounds__(256) void gemm_f16_nt_ring_kernel(
 #pragma unroll
 		for (int j = 0; j < 8; ++j)
 			acc[i][j] = float4_t{(*rows[i])[4 * j], (*rows[i])[4 * j + 1], (*rows[i])[4 * j + 2], (*rows[i])[4 * j + 3]};
-	store_patch_via_lds<Cfg, RAGGED, !RAGGED, EPI>(acc, lds, C, ldc, m0 + wm * 128, n0 + wn * (DUAL ? 64 : 128), wave, lane, M, N, bias, ep_param);
+	store_patch_via_lds<Cfg, RAGGED, !RAGGED, EPI>(acc, lds, C, ldc, m0 + wm * 128, n0 + wn * (DUAL ? 64 : 128), wave, lane_after, M, N, bias, ep_param);
 }
 
 // What the kernel assumes, checked on the host before every launch: whole slabs, 16-byte aligned operand rows, and
