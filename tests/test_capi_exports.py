@@ -97,3 +97,60 @@ def test_generated_gemm_loop_is_current(tmp_path):
         out = tmp_path / name
         subprocess.run([sys.executable, str(csrc / "gen_gemm_f16_ring_loop.py"), str(out), *form], check=True)
         assert out.read_text() == (csrc / name).read_text()
+
+
+def _gfx950_code_objects(library: Path):
+    """The gfx950 code objects inside the library's .hip_fatbin section (one clang offload bundle per source file)."""
+    import struct
+    import tempfile
+    objcopy = Path("/opt/rocm/llvm/bin/llvm-objcopy")
+    if not objcopy.exists():
+        pytest.skip("llvm-objcopy not found")
+    with tempfile.TemporaryDirectory() as tmp:
+        fat = Path(tmp) / "fat.bin"
+        subprocess.run([str(objcopy), "-O", "binary", "--only-section=.hip_fatbin", str(library), str(fat)], check=True)
+        data = fat.read_bytes()
+    magic = b"__CLANG_OFFLOAD_BUNDLE__"
+    pos = 0
+    while True:
+        start = data.find(magic, pos)
+        if start < 0:
+            return
+        (entries,) = struct.unpack_from("<Q", data, start + len(magic))
+        p = start + len(magic) + 8
+        for _ in range(entries):
+            offset, size, triple_len = struct.unpack_from("<QQQ", data, p)
+            p += 24
+            triple = data[p:p + triple_len].decode()
+            p += triple_len
+            if "gfx950" in triple:
+                yield data[start + offset:start + offset + size]
+        pos = start + len(magic)
+
+
+def test_kernels_use_no_scratch_memory(tmp_path):
+    # A kernel with a private segment (register spills, private arrays) makes the runtime allocate scratch memory for the
+    # queue at its first launch, tens of megabytes behind the caller's back.  Every kernel's metadata has to say 0 bytes,
+    # except the one instantiation listed (the eight-wave 256 x 256 tile with guarded rows, a K tail and partial planes,
+    # which products of that shape reach only when the four-wave kernels cannot take them).
+    readelf = Path("/opt/rocm/llvm/bin/llvm-readelf")
+    lib = REPO / "anygpu_amd" / "lib" / "libanygpu_hip.so"
+    if not readelf.exists() or not lib.exists():
+        pytest.skip("llvm-readelf or the built library not found")
+    allowed = re.compile(r"gemm_f16_nt_tile_kernelINS_11GemmTileCfgILi256ELi256E.*ELb1ELb1ELb1ELin1E")
+    seen, offenders = 0, []
+    for k, blob in enumerate(_gfx950_code_objects(lib)):
+        path = tmp_path / f"co{k}.elf"
+        path.write_bytes(blob)
+        notes = subprocess.run([str(readelf), "--notes", str(path)], check=True, capture_output=True, text=True).stdout
+        name = None
+        for line in notes.splitlines():
+            line = line.strip()
+            if line.startswith(".name:"):
+                name = line.split(":", 1)[1].strip()
+            elif line.startswith(".private_segment_fixed_size:"):
+                seen += 1
+                if int(line.split(":", 1)[1]) != 0 and not allowed.search(name or ""):
+                    offenders.append((name, line))
+    assert seen > 100, "kernel metadata not found"
+    assert not offenders, offenders
