@@ -459,9 +459,12 @@ static TilePlan plan_tiles(int tile, int64_t M, int64_t N, int64_t K, int64_t ba
 	for (int64_t s = 2; s <= kSplitMax && s <= K / kSplitMinDepth && s <= room; ++s)
 	{
 		const double rounds = rounds_of(tiles * s);
-		const double planes_us = 8.0 * (double)s * (double)M * (double)N / 3.0e6;    // written and read back at ~3 TB/s
+		// (the planes are written by the product's last waves and read back by a launch that only does that: priced at
+		// 6 TB/s, and a cut has to promise 3 % — with 3 TB/s and 10 % products of 48 to 128 rows against wide weight
+		// matrices stayed uncut that run 15 % faster in three or four ranges: 64 x 2304 -> 18432 75 -> 63 us)
+		const double planes_us = 8.0 * (double)s * (double)M * (double)N / 6.0e6;
 		const double cost = rounds * ((double)slabs / (double)s + 5.0) * slab_us + 3.0 + planes_us;
-		if (cost < best.cost * 0.9) best = TilePlan{tile, s, cost};
+		if (cost < best.cost * 0.97) best = TilePlan{tile, s, cost};
 	}
 	return best;
 }
