@@ -380,7 +380,8 @@ __global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f16_kernel(const
 //     step B of tile t:  O += V(t)^T P(t)^T        (MFMA + LDS reads)   beside   z(t + 1) = mask(softcap(S(t + 1)))  (VALU)
 // In the kernel above every wave of the block multiplies, then exponentiates, then multiplies (the barriers of a
 // tile keep the eight waves in step), so the matrix cores idle while the VALU works and the other way round.  The
-// LDS holds K of tile t + 1 next to V of tile t; tiles pass through registers, 16 queries per wave.
+// LDS holds K of tile t + 1 next to V of tile t (two stages of each, filled global -> LDS directly).  QB is 1 in
+// every launch: with two 16-query blocks per wave the kernel measured slower at every head dimension.
 template <int D, bool SOFTCAP, int QB, int WAVES>
 __global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f16_skew_kernel(const AttnArgs a, const AttnWalk walk)
 {
@@ -597,12 +598,12 @@ __global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f16_skew_kernel(
 		const char* v_lds = lds + stage * kStageBytes + kAttnKeysPerTile * L::kPitchK;
 		const int t_k = t + 2 <= t_last ? t + 2 : t_last;       // (past the end: the last tile once more, into the free stage)
 
-		// The tile as 64 steps of one operand out of LDS and the QB MFMAs that use it, 32 of S(t + 1) = K(t + 1) Q^T (the
-		// four key blocks in turn, so that consecutive MFMAs do not wait for each other's result) and 32 of
-		// O^T += V(t)^T P(t)^T.  Behind its MFMAs a step issues the LDS reads of the operand kAhead steps later and
-		// does its share of the vector work: in the first half p(t) = exp2(z(t) - m), one score per query block every
-		// other step, in the second z(t + 1) likewise; the loads of the next tiles go out one slot every other step.
-		// The scheduler may reorder inside a step, not across steps.
+		// The tile as steps of one operand out of LDS and the QB MFMAs that use it (64 at head dimension 256): those of
+		// S(t + 1) = K(t + 1) Q^T, the four key blocks in turn so that consecutive MFMAs do not wait for each other's
+		// result, then those of O^T += V(t)^T P(t)^T.  Behind its MFMAs a step issues the LDS reads of the operand
+		// kAhead steps later and does its share of the vector work: in the first half p(t) = exp2(z(t) - m), the 16
+		// scores of a query block spread evenly over the steps, in the second z(t + 1) likewise; one load of the next
+		// tiles goes out every kLoadSpacing steps.  The scheduler may reorder inside a step, not across steps.
 		// (2 to 5 steps ahead measure alike, 6 and 8 slower; the boundary tiles, with their masks, have registers for 2)
 		constexpr int kAhead = decltype(interior_tag)::value ? 4 : 2;
 		constexpr int kLoadSpacing = 6 < (4 * KS + 2 * DC) / (2 * kSlots) ? 6 : (4 * KS + 2 * DC) / (2 * kSlots);
