@@ -515,6 +515,28 @@ __global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f16_skew_kernel(
 			return zz + ((key >= lo && key <= hi) ? 0.0f : -INFINITY);
 		}
 	};
+	// the same in three pieces, for steps that must not contain an operation together with the one that needs its
+	// result: begin -> middle -> finish (without softcap the first is all there is)
+	auto logit_begin = [&](float sv) {
+		if constexpr (SOFTCAP) return fast_exp2(sv * a.k_in);
+		else return sv * a.k_in;
+	};
+	auto logit_middle = [&](float tv) {
+		if constexpr (SOFTCAP) return fast_rcp(1.0f + tv);
+		else return tv;
+	};
+	auto logit_finish = [&](auto interior_tag, float rv, int t, int b, int e, int g) {
+		float zz = rv;
+		if constexpr (SOFTCAP) zz = fmaf(rv, -2.0f * a.k_cap, a.k_cap);
+		if constexpr (decltype(interior_tag)::value) return zz;
+		else
+		{
+			int lo = vis_lo[b], hi = vis_hi[b];
+			asm volatile("" : "+v"(lo), "+v"(hi));
+			const int key = t * kAttnKeysPerTile + 16 * (e / 4) + 4 * g + e % 4;
+			return zz + ((key >= lo && key <= hi) ? 0.0f : -INFINITY);
+		}
+	};
 	auto is_interior = [&](int t) {
 		const int key0 = t * kAttnKeysPerTile;
 		return key0 >= all_lo && key0 + kAttnKeysPerTile - 1 <= all_hi;
@@ -622,7 +644,8 @@ __global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f16_skew_kernel(
 			return (half8_t)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
 		};
 		float4_t s_next[QB][4];
-		float psum[QB];
+		float psum[QB], carry[QB];               // carry: a score's intermediate result on its way to the next step
+		float z_max[QB];
 		half8_t pf[QB][2];
 #pragma unroll
 		for (int b = 0; b < QB; ++b)
@@ -675,8 +698,54 @@ __global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f16_skew_kernel(
 					if (m % 2 == 0) issue_slot(vp, 1, t + 1, stage ^ 1, m / 2);
 					else issue_slot(kp, 0, t_k, stage, m / 2);
 				}
-				// (the 16 scores of a query block spread evenly over the steps of each half)
-				if (i < kStepsA)
+				// The 16 scores of a query block spread evenly over the steps of each half.  With two steps per score
+				// (head dimension 256) an operation and the one that needs its result sit in different steps: a
+				// transcendental's result is not there for the next instruction, and a wave issues in order.
+				//   first half:   even step  x = exp2(z - m)                 odd step  sum += x, p = fp16(x)
+				//   second half:  even step  t = exp2(s k_in), z of the score before    odd step  r = 1 / (1 + t)
+				constexpr int kStepsB = 2 * DC;
+				constexpr bool kTwoSteps = kStepsA == 32 && kStepsB == 32;
+				if constexpr (kTwoSteps)
+				{
+					if (i < kStepsA)
+					{
+#pragma unroll
+						for (int b = 0; b < QB; ++b)
+						{
+							if (i % 2 == 0) carry[b] = fast_exp2(z[b][i / 2] - m_safe[b]);
+							else
+							{
+								psum[b] += carry[b];
+								pf[b][(i / 2) / 8][(i / 2) % 8] = (half_t)carry[b];
+							}
+						}
+					}
+					else
+					{
+						const int j = i - kStepsA, e = j / 2;
+#pragma unroll
+						for (int b = 0; b < QB; ++b)
+						{
+							if (j % 2 == 0)
+							{
+								if (e > 0) z[b][e - 1] = logit_finish(interior_tag, carry[b], t + 1, b, e - 1, g);
+								carry[b] = logit_begin(s_next[b][e / 4][e % 4]);
+							}
+							else
+							{
+								carry[b] = logit_middle(carry[b]);
+								// (the maximum of the tile's scores grows with them instead of in one chain behind the last)
+								if (e > 0) z_max[b] = e > 1 ? fmaxf(z_max[b], z[b][e - 1]) : z[b][0];
+							}
+							if (j == kStepsB - 1)
+							{
+								z[b][15] = logit_finish(interior_tag, carry[b], t + 1, b, 15, g);
+								z_max[b] = fmaxf(z_max[b], z[b][15]);
+							}
+						}
+					}
+				}
+				else if (i < kStepsA)
 				{
 #pragma unroll
 					for (int u = 0; u < (16 + kStepsA - 1) / kStepsA; ++u)
@@ -686,7 +755,6 @@ __global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f16_skew_kernel(
 				}
 				else
 				{
-					constexpr int kStepsB = 2 * DC;
 #pragma unroll
 					for (int u = 0; u < (16 + kStepsB - 1) / kStepsB; ++u)
 #pragma unroll
@@ -704,7 +772,11 @@ __global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f16_skew_kernel(
 		for (int b = 0; b < QB; ++b)
 		{
 			l_run[b] += psum[b];
-			if constexpr (MORE) m_new[b] = row_max(b);
+			if constexpr (MORE)
+			{
+				if constexpr (4 * KS == 32 && 2 * DC == 32) m_new[b] = fmaxf(m_run[b], max_over_lane_rows(z_max[b]));
+				else m_new[b] = row_max(b);
+			}
 		}
 	};
 	for (int t = t_first; t < t_last; ++t)
