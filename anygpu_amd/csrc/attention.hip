@@ -718,6 +718,9 @@ __global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f16_skew_kernel(
 								psum[b] += carry[b];
 								pf[b][(i / 2) / 8][(i / 2) % 8] = (half_t)carry[b];
 							}
+							// (p is first used behind the branch that follows this half: without a use here the compiler
+							// moves the whole half's vector work there)
+							if (i == kStepsA - 1) asm volatile("" : "+v"(pf[b][0]), "+v"(pf[b][1]), "+v"(psum[b]));
 						}
 					}
 					else
