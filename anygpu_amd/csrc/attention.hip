@@ -22,7 +22,7 @@
 // slot j <-> key 16 * (2 t + j / 4) + 4 * (lane / 16) + j % 4 of the tile, so no shuffle is needed
 // between the two products.
 //
-// At head dimension 256 with softcap a second kernel of the same layout (sdp_attention_fwd_f16_skew_kernel) computes
+// At head dimension 256 a second kernel of the same layout (sdp_attention_fwd_f16_skew_kernel) computes
 // the scores of tile t + 1 beside the softmax of tile t, so that the matrix and the vector instructions of a wave
 // do not depend on each other.
 //
@@ -886,11 +886,10 @@ hipError_t launch_variant(const AttnArgs& args_in, int64_t batch_heads, hipStrea
 // register footprint lets more waves share a SIMD), except head_dim 128 with enough query blocks to fill the chip,
 // where 8 waves x 32 queries halve the LDS reads per flop and fit the register file (16 x 4096 x 128 causal: 148 us
 // against 172 us).  At head_dim 256 the 32-query form does not fit the registers.
-// The skewed kernel is used where the softmax arithmetic is a large share of a tile, head_dim 256 with softcap
-// (8 / 4 heads x 8192 x 256, softcap 50, window 4096: 321 -> 306 us in one process; full causal 438 -> 410 us).  Measured
-// against the kernel above on one GPU it loses elsewhere: head_dim 256 without softcap 390 -> 397 us, head_dim
-// 128 (16 x 4096 causal) 128 -> 141 us, head_dim 64 (32 x 2048 causal) 45 -> 61 us; with 32 queries per wave it
-// loses at every head dimension.
+// The skewed kernel serves head_dim 256 (8 / 4 heads x 8192 x 256 with window 4096, one process: softcap 50
+// 321 -> 276 us, without softcap 277 -> 264 us; 8 heads causal without softcap 381 -> 355 us).  At head_dim 128 and 64 it
+// measured slower than the kernel above (16 x 4096 x 128 causal 128 -> 141 us, 32 x 2048 x 64 causal 45 -> 61 us, before
+// its last tenth), and with 32 queries per wave slower at every head dimension.
 template <int D>
 hipError_t launch_dim(const AttnArgs& args, bool softcap, int64_t batch_heads, hipStream_t stream)
 {
@@ -900,10 +899,9 @@ hipError_t launch_dim(const AttnArgs& args, bool softcap, int64_t batch_heads, h
 			return softcap ? launch_variant<D, true, 2>(args, batch_heads, stream) : launch_variant<D, false, 2>(args, batch_heads, stream);
 	}
 	if constexpr (D == 256)
-	{
-		if (softcap) return launch_variant<D, true, 1, true>(args, batch_heads, stream);
-	}
-	return softcap ? launch_variant<D, true, 1>(args, batch_heads, stream) : launch_variant<D, false, 1>(args, batch_heads, stream);
+		return softcap ? launch_variant<D, true, 1, true>(args, batch_heads, stream) : launch_variant<D, false, 1, true>(args, batch_heads, stream);
+	else
+		return softcap ? launch_variant<D, true, 1>(args, batch_heads, stream) : launch_variant<D, false, 1>(args, batch_heads, stream);
 }
 
 // ---------------------------------------------------------------------------------------------

@@ -1483,10 +1483,10 @@ def test_sdp_attention_fused_kernel_random_shapes(ops, oracle, dtype):
         assert scaled_rel_err(got[0], want, 1.0) <= tol, case
 
 
-# head_dim 256 with softcap runs the kernel that takes S of tile t + 1 beside the softmax of tile t: tile counts of
+# head_dim 256 runs the kernel that takes S of tile t + 1 beside the softmax of tile t: tile counts of
 # one and two (the pipelined loop body not entered / entered once), a last tile that is not whole, a key range longer
 # than the queries, windows below a tile and without the causal rule, queries without a visible key, grouped heads
-ATTN_D256_SOFTCAP_CASES = [
+ATTN_D256_CASES = [
     (2, 2, 17, 63, 256, 0.0625, 50.0, True, 0),
     (2, 2, 17, 64, 256, 0.0625, 50.0, True, 0),
     (2, 2, 20, 65, 256, 0.0625, 50.0, False, 0),
@@ -1497,11 +1497,17 @@ ATTN_D256_SOFTCAP_CASES = [
     (2, 2, 260, 260, 256, 0.0625, 50.0, False, 70),
     (2, 2, 100, 40, 256, 0.0625, 50.0, True, 0),
     (8, 2, 640, 700, 256, 0.0625, 50.0, True, 200),
+    # the same kernel without softcap
+    (2, 2, 17, 65, 256, 0.0625, 0.0, True, 0),
+    (2, 1, 129, 129, 256, 0.0625, 0.0, True, 0),
+    (4, 2, 200, 333, 256, -0.05, 0.0, True, 33),
+    (2, 2, 260, 260, 256, 0.0625, 0.0, False, 70),
+    (2, 2, 100, 40, 256, 0.0625, 0.0, True, 0),
 ]
 
 
-@pytest.mark.parametrize("case", ATTN_D256_SOFTCAP_CASES)
-def test_sdp_attention_fused_kernel_head_dim_256_with_softcap(ops, oracle, case):
+@pytest.mark.parametrize("case", ATTN_D256_CASES)
+def test_sdp_attention_fused_kernel_head_dim_256(ops, oracle, case):
     heads, kv_heads, n_q, n_k, d, alpha, cap, causal, window = case
     q = synth.normal(1 + n_q, (1, heads, n_q, d)).astype(np.float16)
     k = synth.normal(2 + n_k, (1, kv_heads, n_k, d)).astype(np.float16)
@@ -1798,7 +1804,7 @@ def _graph_problem(ops):
     cw, cb = dev(synth.normal(3, (16, 4)).astype(np.float16)), dev(synth.normal(4, (16,)).astype(np.float16))
     q = torch.empty((1, 4, 100, 128), device="cuda")
     kv = dev(synth.normal(5, (1, 2, 100, 128)))
-    q16 = torch.empty((1, 4, 150, 256), device="cuda", dtype=torch.float16)     # head_dim 256 with softcap: its own kernel
+    q16 = torch.empty((1, 4, 150, 256), device="cuda", dtype=torch.float16)     # head_dim 256: its own kernel
     kv16 = dev(synth.normal(6, (1, 2, 150, 256)).astype(np.float16))
 
     def fill(seed):
