@@ -65,7 +65,15 @@ MEASURED_TRAFFIC = {
 
 def traffic_fields(key):
     nbytes, source = MEASURED_TRAFFIC[key]
-    return {"traffic": nbytes, "traffic_source": f"{source} (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this command; copied, not measured in this run)"}
+    fields = {"traffic": nbytes, "traffic_source": f"{source} (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this command; copied, not measured in this run)"}
+    # which version of the summary the figure was copied from: the file's SHA-1 (the tree that runs here has no history)
+    try:
+        import hashlib
+        with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), source), "rb") as f:
+            fields["traffic_source_sha1"] = hashlib.sha1(f.read()).hexdigest()[:12]
+    except OSError:
+        fields["traffic_source_sha1"] = None
+    return fields
 
 
 def parse_args():
