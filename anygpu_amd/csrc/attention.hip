@@ -644,8 +644,7 @@ __global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f16_skew_kernel(
 			return (half8_t)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
 		};
 		float4_t s_next[QB][4];
-		float psum[QB], carry[QB];               // carry: a score's intermediate result on its way to the next step
-		float z_max[QB];
+		float psum[QB], z_max[QB];
 		half8_t pf[QB][2];
 #pragma unroll
 		for (int b = 0; b < QB; ++b)
@@ -658,6 +657,25 @@ __global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f16_skew_kernel(
 			const float pv = fast_exp2(z[b][e] - m_safe[b]);
 			psum[b] += pv;
 			pf[b][e / 8][e % 8] = (half_t)pv;
+		};
+		// stage of score e that belongs to step i, if any (see the table at its call)
+		float xa[QB][16], tb[QB][16];
+		auto vector_stage = [&](auto tag, int b, int e, int i) {
+			constexpr int kStepsB = 2 * DC;
+			const int a0 = e * kStepsA / 16, b0 = kStepsA + e * kStepsB / 16;
+			if (i == a0) xa[b][e] = fast_exp2(z[b][e] - m_safe[b]);
+			if (i == a0 + 1)
+			{
+				psum[b] += xa[b][e];
+				pf[b][e / 8][e % 8] = (half_t)xa[b][e];
+			}
+			if (i == b0) tb[b][e] = logit_begin(s_next[b][e / 4][e % 4]);
+			if (i == b0 + 1) tb[b][e] = logit_middle(tb[b][e]);
+			if (i == b0 + 2)
+			{
+				z[b][e] = logit_finish(tag, tb[b][e], t + 1, b, e, g);
+				z_max[b] = e == 0 ? z[b][0] : fmaxf(z_max[b], z[b][e]);
+			}
 		};
 #pragma unroll
 		for (int i = 0; i < kAhead; ++i) frag[i] = read_operand(i);
@@ -698,88 +716,44 @@ __global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f16_skew_kernel(
 					if (m % 2 == 0) issue_slot(vp, 1, t + 1, stage ^ 1, m / 2);
 					else issue_slot(kp, 0, t_k, stage, m / 2);
 				}
-				// The 16 scores of a query block spread evenly over the steps of each half.  With two steps per score
-				// (head dimension 256) an operation and the one that needs its result sit in different steps: a
-				// transcendental's result is not there for the next instruction, and a wave issues in order.
-				//   first half:   even step  x = exp2(z - m)                 odd step  sum += x, p = fp16(x)
-				//   second half:  even step  t = exp2(s k_in), z of the score before    odd step  r = 1 / (1 + t)
-				constexpr int kStepsB = 2 * DC;
-				constexpr bool kTwoSteps = kStepsA == 32 && kStepsB == 32;
-				if constexpr (kTwoSteps)
-				{
-					if (i < kStepsA)
-					{
+				// The 16 scores of a query block spread evenly over the steps of each half, every score's operations in
+				// stages one step apart, so that none sits in a step with the one that needs its result (a
+				// transcendental's result is not there for the next instruction, and a wave issues in order):
+				//   first half, score e from step e kStepsA / 16:   x = exp2(z - m)  |  sum += x, p = fp16(x)
+				//   second half, score e from step kStepsA + e kStepsB / 16:   t = exp2(s k_in)  |  r = 1 / (1 + t)  |
+				//                                                              z = k_cap - 2 k_cap r, masked; tile maximum
+				// (stages that fall behind the last step run behind it; p of the second half of the keys is needed from
+				// step kStepsA + DC on, so the last scores' second stage may sit in the second half)
 #pragma unroll
-						for (int b = 0; b < QB; ++b)
-						{
-							if (i % 2 == 0) carry[b] = fast_exp2(z[b][i / 2] - m_safe[b]);
-							else
-							{
-								psum[b] += carry[b];
-								pf[b][(i / 2) / 8][(i / 2) % 8] = (half_t)carry[b];
-							}
-							// (p is first used behind the branch that follows this half: without a use here the compiler
-							// moves the whole half's vector work there)
-							if (i == kStepsA - 1) asm volatile("" : "+v"(pf[b][0]), "+v"(pf[b][1]), "+v"(psum[b]));
-						}
-					}
-					else
-					{
-						const int j = i - kStepsA, e = j / 2;
+				for (int e = 0; e < 16; ++e)
 #pragma unroll
-						for (int b = 0; b < QB; ++b)
-						{
-							if (j % 2 == 0)
-							{
-								if (e > 0) z[b][e - 1] = logit_finish(interior_tag, carry[b], t + 1, b, e - 1, g);
-								carry[b] = logit_begin(s_next[b][e / 4][e % 4]);
-							}
-							else
-							{
-								carry[b] = logit_middle(carry[b]);
-								// (the maximum of the tile's scores grows with them instead of in one chain behind the last)
-								if (e > 0) z_max[b] = e > 1 ? fmaxf(z_max[b], z[b][e - 1]) : z[b][0];
-							}
-							if (j == kStepsB - 1)
-							{
-								z[b][15] = logit_finish(interior_tag, carry[b], t + 1, b, 15, g);
-								z_max[b] = fmaxf(z_max[b], z[b][15]);
-							}
-						}
-					}
-				}
-				else if (i < kStepsA)
+					for (int b = 0; b < QB; ++b) vector_stage(interior_tag, b, e, i);
+				// (p is first used behind the branch that follows the first half: without a use here the compiler moves
+				// the whole half's vector work there)
+				if constexpr (i == kStepsA - 1)
 				{
 #pragma unroll
-					for (int u = 0; u < (16 + kStepsA - 1) / kStepsA; ++u)
-#pragma unroll
-						for (int b = 0; b < QB; ++b)
-							if (i * 16 / kStepsA + u < (i + 1) * 16 / kStepsA) p_of_score(b, i * 16 / kStepsA + u);
-				}
-				else
-				{
-#pragma unroll
-					for (int u = 0; u < (16 + kStepsB - 1) / kStepsB; ++u)
-#pragma unroll
-						for (int b = 0; b < QB; ++b)
-						{
-							const int e = (i - kStepsA) * 16 / kStepsB + u;
-							if (e < (i - kStepsA + 1) * 16 / kStepsB) z[b][e] = logit_of_score(interior_tag, s_next[b][e / 4][e % 4], t + 1, b, e, g);
-						}
+					for (int b = 0; b < QB; ++b) asm volatile("" : "+v"(pf[b][0]), "+v"(psum[b]));
 				}
 			}
 			__builtin_amdgcn_sched_barrier(0);
 		};
 		[&]<int... I>(std::integer_sequence<int, I...>) { (step(std::integral_constant<int, I>{}), ...); }(std::make_integer_sequence<int, kSteps>{});
+		if constexpr (MORE)
+		{
+			// the stages behind the last step, in order
+#pragma unroll
+			for (int late = kSteps; late < kSteps + 2; ++late)
+#pragma unroll
+				for (int e = 0; e < 16; ++e)
+#pragma unroll
+					for (int b = 0; b < QB; ++b) vector_stage(interior_tag, b, e, late);
+		}
 #pragma unroll
 		for (int b = 0; b < QB; ++b)
 		{
 			l_run[b] += psum[b];
-			if constexpr (MORE)
-			{
-				if constexpr (4 * KS == 32 && 2 * DC == 32) m_new[b] = fmaxf(m_run[b], max_over_lane_rows(z_max[b]));
-				else m_new[b] = row_max(b);
-			}
+			if constexpr (MORE) m_new[b] = fmaxf(m_run[b], max_over_lane_rows(z_max[b]));
 		}
 	};
 	for (int t = t_first; t < t_last; ++t)
