@@ -51,15 +51,15 @@ MIN_TIMED_LAUNCHES = 20
 # command (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), scaled by what the same counters read for a plain 256 MiB
 # device copy (fetch x 2.000, write x 1.000); the summary each figure is copied from is named beside it.
 MEASURED_TRAFFIC = {
-    "gemm_f16": (235059557, "profiles/gemm_f16_4096_ring_kernel.md"),
-    "gemm_f32": (117654444, "profiles/gemm_f32_2048_kernel.md"),
-    "conv1d": (277191745, "profiles/causal_conv1d_silu_zamba2_tile_kernel.md"),
-    "softmax_causal": (406923951, "profiles/softmax_causal_32x2048x2048_window_kernel.md"),
-    "softmax_gemma2": (1483621609, "profiles/softmax_gemma2_8x8192x8192_window_kernel.md"),
-    "attention_gemma2": (531064542, "profiles/sdp_attention_fwd_f16_gemma2_kernel.md"),
-    "attention_gemma2_f32": (1332780135, "profiles/sdp_attention_fwd_f32_gemma2_kernel.md"),
-    "gated_rmsnorm": (805408668, "profiles/gated_rmsnorm_f16_row_kernel.md"),
-    "attention_decode": (144037176, "profiles/sdp_attention_decode_f16_partial_and_merge_kernels.md"),
+    "gemm_f16": (235046242, "profiles/gemm_f16_4096_ring_kernel.md"),
+    "gemm_f32": (117654803, "profiles/gemm_f32_2048_kernel.md"),
+    "conv1d": (277197415, "profiles/causal_conv1d_silu_zamba2_tile_kernel.md"),
+    "softmax_causal": (406922965, "profiles/softmax_causal_32x2048x2048_window_kernel.md"),
+    "softmax_gemma2": (1483615321, "profiles/softmax_gemma2_8x8192x8192_window_kernel.md"),
+    "attention_gemma2": (530927292, "profiles/sdp_attention_fwd_f16_gemma2_kernel.md"),
+    "attention_gemma2_f32": (1308870403, "profiles/sdp_attention_fwd_f32_gemma2_kernel.md"),
+    "gated_rmsnorm": (805405955, "profiles/gated_rmsnorm_f16_row_kernel.md"),
+    "attention_decode": (144037358, "profiles/sdp_attention_decode_f16_partial_and_merge_kernels.md"),
 }
 
 
