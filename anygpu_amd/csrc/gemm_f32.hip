@@ -343,9 +343,9 @@ static hipError_t launch_tiles_once(const float* A, const float* B, const float*
 	// keeps the matrix cores busier than this file's kernel does around its barriers (2048^3: 131 -> see the header)
 	if constexpr (A_LAYOUT == ANYGPU_A_ROW_MAJOR && BM == BN && EPI != kEpiGeluMul)
 	{
-		if (gemm_f32_ring_applies(A, B, M, N, K, lda, ldb, stride_a, stride_b, batch, k_split, BM, B_LAYOUT))
+		if (gemm_f32_ring_applies(A, B, M, N, K, lda, ldb, stride_a, stride_b, batch, k_split, BM, B_LAYOUT, padded))
 			return launch_gemm_f32_ring<BM / 64, EPI, B_LAYOUT == ANYGPU_B_ROW_MAJOR>(A, B, bias, C, M, N, K, lda, ldb, ldc, stride_a, stride_b, stride_c,
-			                                                                        batch, ep_param, k_split, stream);
+			                                                                        batch, ep_param, k_split, stream, padded);
 	}
 	const dim3 grid((unsigned)((N + BN - 1) / BN), (unsigned)((M + BM - 1) / BM), (unsigned)batch);
 	const bool aligned_in = (reinterpret_cast<uintptr_t>(A) % 16 == 0) && (reinterpret_cast<uintptr_t>(B) % 16 == 0) &&
@@ -518,7 +518,7 @@ static hipError_t launch_layout(const float* A, const float* B, const float* B2,
 	// a stream under capture without a caller's workspace has none and runs uncut)
 	const size_t ws_bytes = (may_split && batch == 1) ? band::workspace_capacity(stream) : 0;
 	const bool four_wave = A_LAYOUT == ANYGPU_A_ROW_MAJOR && EPI != kEpiGeluMul &&
-	                       gemm_f32_ring_applies(A, B, M, N, K, lda, ldb, stride_a, stride_b, batch, 0, 64, B_LAYOUT);
+	                       gemm_f32_ring_applies(A, B, M, N, K, lda, ldb, stride_a, stride_b, batch, 0, 64, B_LAYOUT, padded);
 	const TilePlan big = plan_tiles(128, M, N, K, batch, may_split, ws_bytes, four_wave);
 	const TilePlan small = plan_tiles(64, M, N, K, batch, may_split, ws_bytes, four_wave);
 	if constexpr (EPI != kEpiGeluMul)

@@ -45,7 +45,7 @@ template <int T, bool RAGGED, int EPI, bool B_KN = false>
 __global__ __launch_bounds__(256) void gemm_f32_nt_ring_kernel(
 	const float* __restrict__ A, const float* __restrict__ B, const float* __restrict__ bias, float* __restrict__ C,
 	int64_t M, int64_t N, int K, int64_t lda, int64_t ldb, int64_t ldc,
-	int64_t stride_a, int64_t stride_b, int64_t stride_c, float ep_param, int k_split)
+	int64_t stride_a, int64_t stride_b, int64_t stride_c, float ep_param, int k_split, int operands_padded)
 {
 	using Cfg = GemmF32RingCfg<T>;
 	constexpr bool DUAL = EPI == kEpiGeluMul;
@@ -79,7 +79,10 @@ __global__ __launch_bounds__(256) void gemm_f32_nt_ring_kernel(
 	const int ld_row = lane >> 3, ld_pos = lane & 7;
 	unsigned* const table = reinterpret_cast<unsigned*>(lds + 3 * Cfg::kStageBytes) + wave * (16 * 64) + lane;
 	int64_t a_first = m0 + 8 * Cfg::kLoads * wave, b_first = n0 + b_unit_row;
-	if constexpr (RAGGED)
+	// (operands_padded: the operands are copies that reach, filled with zeros, to the end of the last tile in every
+	// direction; nothing to clamp then, and N need not be a multiple of 4 for B stored [K, N])
+	const bool clamp = RAGGED && operands_padded == 0;
+	if (clamp)
 	{
 		a_first = a_first < M - 1 ? a_first : M - 1;
 		b_first = b_first < N - 1 ? b_first : N - 1;
@@ -90,7 +93,7 @@ __global__ __launch_bounds__(256) void gemm_f32_nt_ring_kernel(
 		const int row = 8 * (Cfg::kLoads * wave + q) + ld_row;
 		const unsigned chunk = ld_pos ^ ((row >> 1) & 7);
 		int64_t a_row = m0 + row, b_row = n0 + b_unit_row + 8 * q + ld_row;
-		if constexpr (RAGGED)
+		if (clamp)
 		{
 			a_row = a_row < M - 1 ? a_row : M - 1;
 			b_row = b_row < N - 1 ? b_row : N - 1;
@@ -104,8 +107,7 @@ __global__ __launch_bounds__(256) void gemm_f32_nt_ring_kernel(
 			const int k_wave = kRowsPerLoad * q + lane / kLanesPerRow;
 			const int k = 8 * wave + k_wave;
 			int64_t col = (int64_t)(((lane % kLanesPerRow) ^ (((k >> 4) & 1) << 3)) << 2);
-			if constexpr (RAGGED)
-				if (n0 + col + 4 > N) col = N - 4 - n0;
+			if (clamp && n0 + col + 4 > N) col = N - 4 - n0;
 			table[64 * (8 + q)] = (unsigned)((k_wave * ldb + col) * 4);
 		}
 		else
@@ -220,9 +222,9 @@ __global__ __launch_bounds__(256) void gemm_f32_nt_ring_kernel(
 // What the kernel assumes, checked on the host before every launch.
 inline bool gemm_f32_ring_applies(const float* A, const float* B, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
                                   int64_t stride_a, int64_t stride_b, int64_t batch, int64_t k_split, int64_t tile = 128,
-                                  int b_layout = ANYGPU_B_COL_MAJOR)
+                                  int b_layout = ANYGPU_B_COL_MAJOR, bool operands_padded = false)
 {
-	if (b_layout == ANYGPU_B_ROW_MAJOR && N % 4 != 0) return false;
+	if (b_layout == ANYGPU_B_ROW_MAJOR && N % 4 != 0 && !operands_padded) return false;
 	const bool aligned = reinterpret_cast<uintptr_t>(A) % 16 == 0 && reinterpret_cast<uintptr_t>(B) % 16 == 0 &&
 	                     lda % 4 == 0 && ldb % 4 == 0 && stride_a % 4 == 0 && stride_b % 4 == 0;
 	return aligned && M > 0 && N > 0 && K >= 32 && K % 32 == 0 && k_split % 32 == 0 && K <= 0x7FFFFFFFLL &&
@@ -232,7 +234,7 @@ inline bool gemm_f32_ring_applies(const float* A, const float* B, int64_t M, int
 template <int T, int EPI, bool B_KN = false>
 inline hipError_t launch_gemm_f32_ring(const float* A, const float* B, const float* bias, float* C, int64_t M, int64_t N, int64_t K,
                                        int64_t lda, int64_t ldb, int64_t ldc, int64_t stride_a, int64_t stride_b, int64_t stride_c,
-                                       int64_t batch, float ep_param, int64_t k_split, hipStream_t stream)
+                                       int64_t batch, float ep_param, int64_t k_split, hipStream_t stream, bool operands_padded = false)
 {
 	const bool c_aligned = reinterpret_cast<uintptr_t>(C) % 16 == 0 && ldc % 4 == 0 && stride_c % 4 == 0;
 	using Cfg = GemmF32RingCfg<T>;
@@ -254,7 +256,7 @@ inline hipError_t launch_gemm_f32_ring(const float* A, const float* B, const flo
 	}
 	const int64_t tiles = ((M + Cfg::BM - 1) / Cfg::BM) * ((N + kOutN - 1) / kOutN);
 	kernel<<<dim3((unsigned)tiles, (unsigned)batch), dim3(256), Cfg::kLdsBytes, stream>>>(
-		A, B, bias, C, M, N, (int)K, lda, ldb, ldc, stride_a, stride_b, stride_c, ep_param, (int)k_split);
+		A, B, bias, C, M, N, (int)K, lda, ldb, ldc, stride_a, stride_b, stride_c, ep_param, (int)k_split, operands_padded ? 1 : 0);
 	return hipGetLastError();
 }
 
