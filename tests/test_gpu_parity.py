@@ -1865,6 +1865,43 @@ def test_launches_replayed_from_a_graph_with_a_caller_workspace(ops, oracle):
         ops.set_workspace(None)
 
 
+def test_key_split_attention_replayed_from_a_graph(ops):
+    # The fused attention with its longest query blocks in two key halves (partial results in the caller's workspace, a
+    # merge launch behind) recorded into a graph: every replay equals the eager result bit for bit, new queries each time.
+    import torch
+    from anygpu_amd import capi
+    h, hkv, n, d, win, cap = 8, 4, 6144 - 40, 256, 2048, 50.0
+    k = dev(synth.normal(2, (hkv, n, d)).astype(np.float16))
+    v = dev(synth.normal(3, (hkv, n, d)).astype(np.float16))
+    q = torch.empty((h, n, d), device="cuda", dtype=torch.float16)
+    side = torch.cuda.Stream()
+    ws_side = torch.full((capi.WORKSPACE_BYTES // 4,), float("nan"), device="cuda")
+    ws_main = torch.empty((capi.WORKSPACE_BYTES // 4,), device="cuda")
+    ops.set_workspace(ws_side, side)
+    ops.set_workspace(ws_main)
+    try:
+        q.copy_(dev(synth.normal(10, (h, n, d)).astype(np.float16)))
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            out = ops.sdp_attention_fwd(q, k, v, 0.0625, softcap=cap, causal=True, window=win)
+        for rep in range(3):
+            q.copy_(dev(synth.normal(20 + rep, (h, n, d)).astype(np.float16)))
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            got = host(out).copy()
+            want = host(ops.sdp_attention_fwd(q, k, v, 0.0625, softcap=cap, causal=True, window=win))
+            torch.cuda.synchronize()
+            assert np.isfinite(got.astype(np.float32)).all()
+            assert np.array_equal(got, want)
+        assert not bool(torch.isnan(ws_side[:1024]).all()), "the replays were expected to leave partial results in the workspace"
+    finally:
+        torch.cuda.synchronize()
+        ops.set_workspace(None, side)
+        ops.set_workspace(None)
+
+
 def test_captured_launches_without_a_workspace_run_uncut(ops, oracle):
     # Under capture the library's own workspace is never used, warmed up or not: every product runs uncut, which is what
     # an eager launch does whose workspace is too small for a single plane.  Both agree bit for bit, and with the cut
