@@ -272,6 +272,80 @@ def test_sdp_attention_masked_scaled_vs_float64_formula(oracle):
     assert np.max(np.abs(y2 - want2)) < 1e-5
 
 
+def _attention_rules_float64(q, k, v, alpha, softcap, causal, window, q_per_kv):
+    """Independent float64 evaluation, one (head, query) at a time with explicit loops over the visible key set."""
+    heads, n_q, d = q.shape
+    n_k = k.shape[1]
+    out = np.zeros((heads, n_q, d))
+    for h in range(heads):
+        g = h // q_per_kv                                   # consecutive query heads share a key / value head
+        for i in range(n_q):
+            pos = i + (n_k - n_q)                           # the query's own key position
+            keys = [j for j in range(n_k)
+                    if (not causal or j <= pos) and (window <= 0 or j > pos - window)]
+            if not keys:
+                continue
+            s = np.array([alpha * float(np.dot(q[h, i].astype(np.float64), k[g, j].astype(np.float64))) for j in keys])
+            if softcap > 0:
+                s = softcap * np.tanh(s / softcap)
+            e = np.exp(s - s.max())
+            p = e / e.sum()
+            out[h, i] = sum(p[t] * v[g, j].astype(np.float64) for t, j in enumerate(keys))
+    return out
+
+
+@pytest.mark.parametrize("q_per_kv", [1, 2, 3])
+def test_sdp_attention_rules_vs_float64_brute_force(oracle, q_per_kv):
+    # more keys than queries (the diagonal sits at n_k - n_q), softcap, causal + window, grouped queries
+    kv_heads, n_q, n_k, d = 2, 7, 19, 16
+    heads = kv_heads * q_per_kv
+    q = synth.normal(40, (heads, n_q, d)) * np.float32(1.5)
+    k = synth.normal(41, (kv_heads, n_k, d)) * np.float32(1.5)
+    v = synth.normal(42, (kv_heads, n_k, d))
+    for kw in (dict(alpha=0.25, softcap=5.0, causal=True, window=6),
+               dict(alpha=0.25, softcap=0.0, causal=True, window=0),
+               dict(alpha=0.5, softcap=0.0, causal=False, window=0),
+               dict(alpha=0.25, softcap=3.0, causal=True, window=25)):
+        got = oracle.sdp_attention_rules(q, k, v, q_per_kv=q_per_kv, **kw)
+        want = _attention_rules_float64(q, k, v, q_per_kv=q_per_kv, **kw)
+        assert np.max(np.abs(got - want)) < 2e-6, kw
+    # the value heads really differ, so a wrong head mapping cannot pass: h % kv_heads instead of h // q_per_kv
+    if q_per_kv > 1:
+        kw = dict(alpha=0.25, softcap=5.0, causal=True, window=6)
+        got = oracle.sdp_attention_rules(q, k, v, q_per_kv=q_per_kv, **kw)
+        wrong = np.stack([_attention_rules_float64(q[h:h + 1], k[h % kv_heads:h % kv_heads + 1],
+                                                   v[h % kv_heads:h % kv_heads + 1], q_per_kv=1, **kw)[0]
+                          for h in range(heads)])
+        assert np.max(np.abs(got - wrong)) > 1e-2
+    # a diagonal at 0 instead of n_k - n_q (the queries taken for the FIRST positions) gives different rows
+    kw = dict(alpha=0.25, softcap=0.0, causal=True, window=0)
+    got = oracle.sdp_attention_rules(q, k, v, q_per_kv=q_per_kv, **kw)
+    first = _attention_rules_float64(q, k[:, :n_q], v[:, :n_q], q_per_kv=q_per_kv, **kw)
+    assert np.max(np.abs(got - first)) > 1e-2
+    # the last query sees every key when only the causal rule applies: plain softmax attention over all keys
+    full = _attention_rules_float64(q[:, -1:], k, v, alpha=0.25, softcap=0.0, causal=False, window=0, q_per_kv=q_per_kv)
+    assert np.max(np.abs(got[:, -1:] - full)) < 2e-6
+    # a subset of queries returns exactly those rows
+    idx = np.array([0, 3, 6])
+    sub = oracle.sdp_attention_rules(q, k, v, q_per_kv=q_per_kv, query_index=idx, **kw)
+    assert np.array_equal(sub, got[:, idx])
+
+
+def test_sdp_attention_rules_equal_the_mask_tensor_form(oracle):
+    # with one query head per key / value head the rule masks are the additive masks of the reference's chain:
+    # square scores with the slide mask (its rule carries no diagonal shift, gemma_slide_mask.cu:21) ...
+    heads, n, d = 3, 14, 8
+    q, k, v = synth.normal(43, (heads, n, d)), synth.normal(44, (heads, n, d)), synth.normal(45, (heads, n, d))
+    mask = oracle.slide_mask(oracle.causal_mask(n, n), 5)
+    a = oracle.sdp_attention_rules(q, k, v, alpha=0.3, causal=True, window=5)
+    assert np.array_equal(a, oracle.sdp_attention_masked_scaled_fwd(q, k, v, mask, 0.3))
+    # ... and more keys than queries with the causal mask shifted to the last queries
+    n_q = 9
+    mask = oracle.causal_mask(n_q, n, diag=n - n_q)
+    a = oracle.sdp_attention_rules(q[:, :n_q], k, v, alpha=0.3, causal=True)
+    assert np.array_equal(a, oracle.sdp_attention_masked_scaled_fwd(q[:, :n_q], k, v, mask, 0.3))
+
+
 # ---------------------------------------------------------------------------------------------
 # tensor_causal_conv1d
 # ---------------------------------------------------------------------------------------------
