@@ -43,6 +43,7 @@ SIGNATURES = {
                                                 c_int64, c_int64, c_int64, c_int, c_void_p]),
     "anygpu_gemm_f16_f32acc_probe": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64,
                                              c_int64, c_int64, c_int64, c_int, c_void_p, c_void_p]),
+    "anygpu_stream_probe": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_int, c_int, c_int, c_int64, c_void_p]),
     "anygpu_gemm_f32": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64,
                                 c_int64, c_int64, c_int64, c_int, c_int, c_void_p]),
     "anygpu_gemm_f32_softcap": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64,

@@ -286,6 +286,21 @@ ANYGPU_EXPORT int anygpu_gemm_f16_f32acc_probe(const void* A, const void* B, voi
 	return (int)anygpu::launch_gemm_f16_probe(A, B, C, M, N, K, lda, ldb, ldc, reinterpret_cast<unsigned long long*>(probe), as_stream(stream));
 }
 
+ANYGPU_EXPORT int anygpu_stream_probe(const void* src, void* dst, int64_t bytes, int block, int vectors_per_lane,
+                                      int nt_load, int nt_store, int64_t grid_limit, void* stream)
+{
+	if (bytes < 0 || bytes % 16 != 0 || grid_limit < 0) return ANYGPU_ERR_BAD_SHAPE;
+	if (block != 256 && block != 512 && block != 1024) return ANYGPU_ERR_UNSUPPORTED;
+	if (vectors_per_lane != 1 && vectors_per_lane != 2 && vectors_per_lane != 4 && vectors_per_lane != 8) return ANYGPU_ERR_UNSUPPORTED;
+	if (bytes == 0) return ANYGPU_OK;
+	if (src == nullptr || dst == nullptr) return ANYGPU_ERR_NULL_POINTER;
+	if ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 15) return ANYGPU_ERR_UNSUPPORTED;
+	const int64_t nvec = bytes / 16;
+	if (nvec / ((int64_t)block * vectors_per_lane) >= kMaxIndex32) return ANYGPU_ERR_TOO_LARGE;
+	return (int)anygpu::launch_stream_probe(src, dst, nvec, block, vectors_per_lane, nt_load != 0, nt_store != 0, grid_limit,
+	                                        as_stream(stream));
+}
+
 ANYGPU_EXPORT int anygpu_gemm_f16_f32acc_batched(const void* A, const void* B, void* C,
                                                  int64_t M, int64_t N, int64_t K,
                                                  int64_t lda, int64_t ldb, int64_t ldc,

@@ -67,6 +67,10 @@ bool gemm_f16_probe_applies(const void* A, const void* B, const void* C, int64_t
 hipError_t launch_gemm_f16_probe(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K,
                                  int64_t lda, int64_t ldb, int64_t ldc, unsigned long long* probe, hipStream_t stream);
 
+// dst[i] = src[i] over nvec 16-byte vectors in the stated launch geometry (stream_probe.hip)
+hipError_t launch_stream_probe(const void* src, void* dst, int64_t nvec, int block, int vectors_per_lane, int nt_load,
+                               int nt_store, int64_t grid_limit, hipStream_t stream);
+
 // Aligned copies of operands the tile kernels cannot fetch as they lie (gemm_repack.hip): `rows` rows of `cols` elements
 // at any alignment into rows of pitch ld_dst (a multiple of 64 elements, 16-byte aligned), zeros behind `cols` and in
 // the rows from `rows` up to rows_dst; and the same from a [k_rows, n_cols] matrix read down its columns,

@@ -15,8 +15,8 @@ the parity tests).  Timing of every kernel:
   * W untimed warm-up steps, then exactly K steps between two device synchronisations (host
     clock -> `value` of the headline) and between two HIP events recorded on the launch stream
     (-> `us_per_launch`, `roofline.achieved`); for the kernels under "kernels", whose K is a
-    fraction of --steps, K is never below 20;
-  * then the same number of launches (at least 20, at most 200) with an event pair around every
+    fraction of --steps, K is never below 100 and W never below 10;
+  * then the same number of launches (at least 100, at most 200) with an event pair around every
     single launch -> `median_us`, `min_us` (these leave out the gap between two launches).
 The memory-bound kernels rotate over several buffer sets so that the working set exceeds the
 256 MB Infinity Cache.
@@ -45,7 +45,8 @@ FP16_FLOP_PER_CLK_PER_CU = 4096
 PEAK_FP16_TFLOPS = 2516.6      # dense fp16 MFMA, 256 CU x 4096 flop/clk/CU x 2.4 GHz
 PEAK_FP32_TFLOPS = 157.3       # fp32 matrix path
 PEAK_HBM_GBS = 8000.0          # HBM3E
-MIN_TIMED_LAUNCHES = 20
+MIN_TIMED_LAUNCHES = 100       # every kernel under "kernels": at least this many back-to-back launches are timed ...
+MIN_WARMUP_LAUNCHES = 10       # ... after at least this many untimed ones (beyond the settle period), whatever --steps says
 
 # Bytes per launch moved behind the L2s: NOT measured by this run.  They come from two rocprofv3 --pmc runs of this
 # command (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), scaled by what the same counters read for a plain 256 MiB
@@ -105,6 +106,8 @@ def timed_region(torch, fn, steps, warmup, floor=MIN_TIMED_LAUNCHES):
     GEMM takes 124 us, then up to 160 us, then settles near 95 us after about 150 launches), and
     the number that matters for a long-running job is the settled one."""
     steps = max(int(steps), floor)
+    if floor > 1:
+        warmup = max(int(warmup), MIN_WARMUP_LAUNCHES)
     t_end = time.perf_counter() + SETTLE_SECONDS
     while time.perf_counter() < t_end:
         for _ in range(20):
@@ -129,14 +132,14 @@ def timed_region(torch, fn, steps, warmup, floor=MIN_TIMED_LAUNCHES):
         b.record()
     torch.cuda.synchronize()
     each = sorted(a.elapsed_time(b) * 1e3 for a, b in pairs)
-    return {"steps": steps, "host_s": t1 - t0, "event_s": start.elapsed_time(stop) * 1e-3,
+    return {"steps": steps, "warmup": warmup, "host_s": t1 - t0, "event_s": start.elapsed_time(stop) * 1e-3,
             "us_per_launch": start.elapsed_time(stop) * 1e3 / steps,
             "median_us": statistics.median(each), "min_us": each[0], "single_launches": singles}
 
 
 def timing_fields(t):
     return {"us_per_launch": t["us_per_launch"], "median_us": t["median_us"], "min_us": t["min_us"],
-            "timed_launches": t["steps"], "single_launches": t["single_launches"]}
+            "timed_launches": t["steps"], "warmup_launches": t["warmup"], "single_launches": t["single_launches"]}
 
 
 def sized_sample(run, unit_cost_probe, total_units, target_seconds):
@@ -155,18 +158,10 @@ def sized_sample(run, unit_cost_probe, total_units, target_seconds):
 # GEMM
 # ---------------------------------------------------------------------------------------------------------------
 
-def bench_gemm_f16(torch, ops, capi, synth, steps, warmup):
-    n = 4096
-    a = torch.from_numpy(synth.uniform(0, (n, n)).astype("float16")).cuda()
-    bt = torch.from_numpy(synth.uniform(1, (n, n)).astype("float16")).cuda()   # B stored [N, K]
-    c = torch.empty((n, n), dtype=torch.float16, device="cuda")
-    # (the headline times exactly --steps launches; only the kernels below are floored)
-    t = timed_region(torch, lambda: ops.tensor_mm(a, bt, out=c, b_layout=capi.B_COL_MAJOR), steps, warmup, floor=1)
-    flops = 2.0 * n ** 3
-    # the vendor library on the same operands, timed the same way (torch.matmul = hipBLASLt): for scale, not the target
-    t_vendor = timed_region(torch, lambda: torch.matmul(a, bt.t(), out=c), steps, warmup, floor=1)
-    # the clock the part sustains under this kernel and the matrix cores' share of those cycles, from the kernel's own
-    # counters (anygpu_gemm_f16_f32acc_probe): launched for another settle period, the last launch read
+def gemm_f16_clock_probe(torch, capi, a, bt, c, n):
+    """The clock the part sustains under the 256 x 256 tile kernel on these operands and the matrix cores' share of those
+    cycles, from the kernel's own counters (anygpu_gemm_f16_f32acc_probe): launched back to back for a settle period,
+    the last launch read."""
     lib = capi.load()
     tiles = (n // 256) ** 2
     probe = torch.zeros((tiles, 4), dtype=torch.int64, device="cuda")
@@ -180,8 +175,35 @@ def bench_gemm_f16(torch, ops, capi, synth, steps, warmup):
         torch.cuda.synchronize()
     p = probe.cpu().double()
     cycles, ns = p[:, 1] - p[:, 0], (p[:, 3] - p[:, 2]) * 10.0
-    clock_ghz = float((cycles / ns).mean())
-    busy = float(((n // 32) * 64 * 16 / cycles).mean())
+    per_xcd = [float(ns[x::8].mean() / 1e3) for x in range(8)]          # tile b runs on XCD b % 8
+    return {"sustained_clock_ghz": float((cycles / ns).mean()), "mfma_busy_in_main_loop": float(((n // 32) * 64 * 16 / cycles).mean()),
+            "main_loop_us_mean": float(ns.mean() / 1e3), "main_loop_us_max": float(ns.max() / 1e3),
+            "main_loop_us_min": float(ns.min() / 1e3), "main_loop_us_slowest_xcd": max(per_xcd), "main_loop_us_fastest_xcd": min(per_xcd)}
+
+
+def bench_gemm_f16(torch, ops, capi, synth, steps, warmup):
+    n = 4096
+    a = torch.from_numpy(synth.uniform(0, (n, n)).astype("float16")).cuda()
+    bt = torch.from_numpy(synth.uniform(1, (n, n)).astype("float16")).cuda()   # B stored [N, K]
+    c = torch.empty((n, n), dtype=torch.float16, device="cuda")
+    # (the headline times exactly --steps launches; only the kernels below are floored)
+    t = timed_region(torch, lambda: ops.tensor_mm(a, bt, out=c, b_layout=capi.B_COL_MAJOR), steps, warmup, floor=1)
+    flops = 2.0 * n ** 3
+    # the vendor library on the same operands, timed the same way (torch.matmul = hipBLASLt): for scale, not the target
+    t_vendor = timed_region(torch, lambda: torch.matmul(a, bt.t(), out=c), steps, warmup, floor=1)
+    clock = gemm_f16_clock_probe(torch, capi, a, bt, c, n)
+    clock["source"] = ("s_memtime / s_memrealtime around the main loop of every tile (anygpu_gemm_f16_f32acc_probe), "
+                       "last launch of a settle period of back-to-back launches after the timed region")
+    # The same launch on operands that toggle few bits (integers -2 .. 2, same shapes, layout, kernel and launch
+    # count): the matrix cores do the same number of operations, the data paths switch less, the part draws less
+    # power and holds a higher clock.  What this run gains over the U(-1, 1) run is what the power limit takes.
+    a_lo = torch.from_numpy(synth.integers(0, (n, n), -2, 2).astype("float16")).cuda()
+    bt_lo = torch.from_numpy(synth.integers(1, (n, n), -2, 2).astype("float16")).cuda()
+    floor_lo = 1 if steps >= MIN_TIMED_LAUNCHES else MIN_TIMED_LAUNCHES
+    t_lo = timed_region(torch, lambda: ops.tensor_mm(a_lo, bt_lo, out=c, b_layout=capi.B_COL_MAJOR), steps, warmup, floor=floor_lo)
+    t_vendor_lo = timed_region(torch, lambda: torch.matmul(a_lo, bt_lo.t(), out=c), steps, warmup, floor=floor_lo)
+    clock_lo = gemm_f16_clock_probe(torch, capi, a_lo, bt_lo, c, n)
+    del a_lo, bt_lo
     return {
         "timing": t, "flops": flops,
         "tflops_host": flops * t["steps"] / t["host_s"] / 1e12,
@@ -189,12 +211,15 @@ def bench_gemm_f16(torch, ops, capi, synth, steps, warmup):
         "operands": (a, bt),
         "vendor": {"what": "torch.matmul (hipBLASLt) on the same operands, timed the same way right after",
                    "us_per_launch": t_vendor["us_per_launch"], "median_us": t_vendor["median_us"], "min_us": t_vendor["min_us"]},
-        "clock": {"sustained_clock_ghz": clock_ghz, "mfma_busy_in_main_loop": busy,
-                  "main_loop_us_mean": float(ns.mean() / 1e3), "main_loop_us_max": float(ns.max() / 1e3),
-                  "main_loop_us_min": float(ns.min() / 1e3),
-                  "source": "s_memtime / s_memrealtime around the main loop of every tile (anygpu_gemm_f16_f32acc_probe), "
-                            "last launch of a settle period of back-to-back launches after the timed region"},
+        "clock": clock,
+        "low_toggle": {"us": t_lo["us_per_launch"], "median_us": t_lo["median_us"], "vendor_us": t_vendor_lo["us_per_launch"],
+                       "timed_launches": t_lo["steps"], "clock": clock_lo},
     }
+
+
+def host_cores(oracle):
+    """Threads for the all-cores leg of a CPU baseline: what the oracle's thread pool offers, at most the box's CPU share."""
+    return min(oracle.max_threads(), int(os.environ.get("OMP_NUM_THREADS", "16") or 16), 16)
 
 
 def cpu_baseline_gemm(oracle, a32, b_view, target_seconds, what):
@@ -208,7 +233,7 @@ def cpu_baseline_gemm(oracle, a32, b_view, target_seconds, what):
 
     rows, t1 = sized_sample(run, 2, m, target_seconds)
     flops = 2.0 * rows * n * k
-    cores = min(oracle.max_threads(), int(os.environ.get("OMP_NUM_THREADS", "16") or 16), 16)
+    cores = host_cores(oracle)
     rows_mt = min(m, rows * cores)
     t0 = time.perf_counter()
     run(rows_mt, cores)
@@ -252,7 +277,57 @@ def rotation(torch, first, nbuf):
     return [first] + [torch.roll(first, shifts=i, dims=0) for i in range(1, nbuf)]
 
 
-def bench_conv1d(torch, ops, synth, steps, warmup, cpu_seconds):
+def quick_us(torch, fn, launches=60, warm=10):
+    for _ in range(warm):
+        fn()
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(launches):
+        fn()
+    stop.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop) * 1e3 / launches
+
+
+def measure_hbm_ceiling(torch, capi, nbytes=138412032, nbuf=4):
+    """What read + write bandwidth this box gives a plain streaming kernel of this library (anygpu_stream_probe:
+    dst[i] = src[i], 16-byte accesses), on the working set of the conv1d configuration (138.4 MB read + 138.4 MB written
+    per launch, `nbuf` rotating buffer pairs): the best of block sizes {256, 512, 1024} x accesses per lane {1, 2, 4}
+    x non-temporal or plain stores, each timed over 60 back-to-back launches after 10 warm-ups; the three best are
+    timed again over 200."""
+    lib = capi.load()
+    stream = torch.cuda.current_stream().cuda_stream
+    srcs = [torch.empty(nbytes, dtype=torch.uint8, device="cuda").random_() for _ in range(nbuf)]
+    dsts = [torch.empty_like(x) for x in srcs]
+    it = [0]
+
+    def runner(block, vpl, nt_store):
+        def step():
+            i = it[0] % nbuf
+            it[0] += 1
+            capi.check("anygpu_stream_probe", lib.anygpu_stream_probe(srcs[i].data_ptr(), dsts[i].data_ptr(), nbytes, block, vpl,
+                                                                      1, nt_store, 0, stream))
+        return step
+
+    sweep = []
+    for block in (256, 512, 1024):
+        for vpl in (1, 2, 4):
+            for nt_store in (1, 0):
+                sweep.append((quick_us(torch, runner(block, vpl, nt_store)), block, vpl, nt_store))
+    sweep.sort()
+    finals = sorted((quick_us(torch, runner(b, v, nt), launches=200, warm=10), b, v, nt) for _, b, v, nt in sweep[:3])
+    us, block, vpl, nt_store = finals[0]
+    assert torch.equal(srcs[0], dsts[0])
+    return {"gbs": 2 * nbytes / us / 1e3, "us_per_launch": us, "frac_of_peak": 2 * nbytes / us / 1e3 / PEAK_HBM_GBS,
+            "bytes_read": nbytes, "bytes_written": nbytes, "rotating_buffer_pairs": nbuf,
+            "best": {"block": block, "vectors_per_lane": vpl, "nt_stores": bool(nt_store)},
+            "worst_gbs": 2 * nbytes / sweep[-1][0] / 1e3,
+            "what": "anygpu_stream_probe, dst[i] = src[i] in 16-byte accesses with non-temporal loads: best of block sizes "
+                    "{256, 512, 1024} x accesses per lane {1, 2, 4} x non-temporal / plain stores, measured in this run"}
+
+
+def bench_conv1d(torch, ops, capi, synth, steps, warmup, cpu_seconds):
     import numpy as np
     b, d, s, width = 4, 4224, 4096, 4
     nbuf = 4                                     # 4 x 277 MB of x + y: well past the Infinity Cache
@@ -272,29 +347,41 @@ def bench_conv1d(torch, ops, synth, steps, warmup, cpu_seconds):
     t = timed_region(torch, step, steps, warmup)
     nbytes = 2 * b * d * s * 2 + d * width * 2 + d * 2
     sec = t["us_per_launch"] * 1e-6
+    del xs[1:], ys[1:]
+    ceiling = measure_hbm_ceiling(torch, capi, nbytes=b * d * s * 2, nbuf=nbuf)
     out = {
         "name": "causal_conv1d_silu_f16",
         "workload": "Zamba2-1.2B conv1d + SiLU: x fp16 [4, 4224, 4096] N(0,1) seed 0, w [4224, 4] N(0,0.5) seed 1, bias [4224] "
                     "N(0,0.1) seed 2, left pad 3 (BASELINE.json configs[2]); 4 rotating buffer sets",
         **timing_fields(t), "value": nbytes / sec / 1e9, "unit": "GB/s", "dtype": "f16",
         "roofline": {"bound": "hbm", "achieved": nbytes / sec / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                     "frac": nbytes / sec / 1e9 / PEAK_HBM_GBS, **traffic_fields("conv1d"), "algorithmic_bytes": nbytes},
+                     "frac": nbytes / sec / 1e9 / PEAK_HBM_GBS, **traffic_fields("conv1d"), "algorithmic_bytes": nbytes,
+                     "frac_on_median": nbytes / (t["median_us"] * 1e-6) / 1e9 / PEAK_HBM_GBS,
+                     "hbm_ceiling_gbs": ceiling["gbs"], "frac_of_hbm_ceiling": nbytes / sec / 1e9 / ceiling["gbs"]},
+        "hbm_ceiling": ceiling,
     }
     if cpu_seconds > 0:
         import oracle
         x32 = oracle.cvt_f16_to_f32(x_host[0])[None]          # batch 0: [1, d, s]
         w32, b32 = oracle.cvt_f16_to_f32(w_host), oracle.cvt_f16_to_f32(b_host)
 
-        def run(chans):
-            oracle.tensor_causal_conv1d(x32[:, :chans], w32[:chans], b32[:chans])
+        def run(chans, threads=1):
+            oracle.tensor_causal_conv1d(x32[:, :chans], w32[:chans], b32[:chans], threads=threads)
 
         chans, sec_cpu = sized_sample(run, 8, d, cpu_seconds)
         sample_bytes = 2 * chans * s * 2 + chans * width * 2 + chans * 2
+        cores = host_cores(oracle)
+        chans_mt = min(d, chans * cores)
+        t0 = time.perf_counter()
+        run(chans_mt, cores)
+        sec_mt = time.perf_counter() - t0
         out["cpu_baseline"] = {
             "value": sample_bytes / sec_cpu / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
             "sample": f"channels 0..{chans - 1} of batch 0 ({chans} rows of 4096 samples; fp16 inputs up-cast to float32 as the "
                       f"reference's tests do) of the same inputs, {sec_cpu:.1f} s; algorithmic fp16 bytes of those rows over the "
-                      f"time, the whole tensor ({b * d} rows) extrapolates linearly"}
+                      f"time, the whole tensor ({b * d} rows) extrapolates linearly",
+            "all_cores": {"value": (2 * chans_mt * s * 2 + chans_mt * width * 2 + chans_mt * 2) / sec_mt / 1e9, "unit": "GB/s",
+                          "cores": cores, "sample": f"channels 0..{chans_mt - 1} of batch 0, rows split over {cores} threads, {sec_mt:.1f} s"}}
     return out
 
 
@@ -336,11 +423,22 @@ def bench_softmax(torch, ops, synth, steps, warmup, cpu_seconds, *, name, heads,
                 oracle.attention_softmax(x32[tt:tt + 1], alpha=alpha, softcap=cap, causal=True, window=window, q_len=0, diag=int(r % q))
 
         n, sec_cpu = sized_sample(run, 16, rows, cpu_seconds)
+        # all cores: a run of consecutive rows from the middle of head 0 (the query index travels as the diagonal
+        # shift), rows dealt to the threads; the oracle evaluates every column of a row whatever the mask hides
+        cores = host_cores(oracle)
+        n_mt = int(min(q // 2, max(n * cores, cores)))
+        first = q // 2 - n_mt // 2
+        x32_mt = oracle.cvt_f16_to_f32(x_host[first:first + n_mt])
+        t0 = time.perf_counter()
+        oracle.attention_softmax(x32_mt, alpha=alpha, softcap=cap, causal=True, window=window, q_len=0, diag=first, threads=cores)
+        sec_mt = time.perf_counter() - t0
         out["cpu_baseline"] = {
             "value": n * 2 * k * 2 / sec_cpu / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
             "sample": f"{n} rows spread evenly over the {rows} of the same inputs (fp16 up-cast to float32; scale, softcap, mask and "
                       f"softmax in the reference's arithmetic: exp in double, sum in float32), {sec_cpu:.1f} s; dense fp16 bytes "
-                      f"of those rows over the time, the whole matrix extrapolates linearly"}
+                      f"of those rows over the time, the whole matrix extrapolates linearly",
+            "all_cores": {"value": n_mt * 2 * k * 2 / sec_mt / 1e9, "unit": "GB/s", "cores": cores,
+                          "sample": f"rows {first}..{first + n_mt - 1} of head 0, rows dealt to {cores} threads, {sec_mt:.1f} s"}}
     return out
 
 
@@ -544,7 +642,7 @@ def main():
     if want("gemm32"):
         kernels.append(bench_gemm_f32(torch, ops, synth, args.steps // 2, args.warmup, cpu_side))
     if want("conv"):
-        kernels.append(bench_conv1d(torch, ops, synth, args.steps, args.warmup, cpu_side))
+        kernels.append(bench_conv1d(torch, ops, capi, synth, args.steps, args.warmup, cpu_side))
     if want("softmax"):
         kernels.append(bench_softmax(
             torch, ops, synth, args.steps, args.warmup, cpu_side, name="softmax_causal_f16", key="softmax_causal",
@@ -580,12 +678,25 @@ def main():
         line["ms_per_step"] = t["host_s"] / t["steps"] * 1e3
         clock = gemm["clock"]
         peak_at_clock = props.multi_processor_count * FP16_FLOP_PER_CLK_PER_CU * clock["sustained_clock_ghz"] * 1e9 / 1e12
+        lo = gemm["low_toggle"]
+        lo_tflops = gemm["flops"] / (lo["us"] * 1e-6) / 1e12
         line["roofline"] = {"bound": "mfma", "achieved": gemm["tflops_event"], "peak": PEAK_FP16_TFLOPS,
                             "unit": "TFLOP/s", "frac": gemm["tflops_event"] / PEAK_FP16_TFLOPS,
                             **traffic_fields("gemm_f16"), **timing_fields(t),
                             "algorithmic_flops": gemm["flops"], "min_bytes": 3 * 4096 * 4096 * 2,
                             **clock, "peak_at_sustained_clock": peak_at_clock,
                             "frac_at_sustained_clock": gemm["tflops_event"] / peak_at_clock,
+                            # scalars: the vendor library (torch.matmul = hipBLASLt) on the same operands in the same run, and
+                            # the same launch of this library and of the vendor's on integers -2 .. 2 (same shapes and layout)
+                            "vendor_us": gemm["vendor"]["us_per_launch"],
+                            "vendor_frac": gemm["flops"] / (gemm["vendor"]["us_per_launch"] * 1e-6) / 1e12 / PEAK_FP16_TFLOPS,
+                            "low_toggle_us": lo["us"], "low_toggle_median_us": lo["median_us"],
+                            "low_toggle_frac": lo_tflops / PEAK_FP16_TFLOPS,
+                            "low_toggle_clock_ghz": lo["clock"]["sustained_clock_ghz"],
+                            "low_toggle_mfma_busy_in_main_loop": lo["clock"]["mfma_busy_in_main_loop"],
+                            "vendor_low_toggle_us": lo["vendor_us"],
+                            "low_toggle_operands": "integers -2 .. 2 (seeds 0 / 1) in place of U(-1, 1); same kernel, shapes, layout; "
+                                                   f"{lo['timed_launches']} launches after the settle period and warm-up",
                             "vendor_library": gemm["vendor"]}
         line["gemm_f16_other_shapes"] = sample_gemm_shapes(torch, ops, capi)
         if args.cpu_seconds > 0:

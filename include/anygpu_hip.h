@@ -139,6 +139,17 @@ int anygpu_gemm_f16_f32acc_probe(const void* A, const void* B, void* C,
                                  int b_layout, uint64_t* probe, void* stream);
 
 /*
+ * Measurement hook: a plain streaming kernel, dst[i] = src[i] over `bytes` bytes (a multiple of 16, both pointers
+ * 16-byte aligned) in 16-byte accesses: blocks of `block` threads (256, 512 or 1024), `vectors_per_lane` (1, 2, 4 or 8)
+ * accesses per lane all loaded before the first store, non-temporal loads / stores when the flags are non-zero, and,
+ * with grid_limit > 0, at most that many blocks which walk the tiles in grid strides.  It states what read + write
+ * bandwidth the box gives a streaming kernel in the geometry chosen, the yardstick for the memory-bound kernels of
+ * this library (bytes read + bytes written = 2 * bytes).  No counterpart in the reference.
+ */
+int anygpu_stream_probe(const void* src, void* dst, int64_t bytes, int block, int vectors_per_lane,
+                        int nt_load, int nt_store, int64_t grid_limit, void* stream);
+
+/*
  * `batch` products of one shape in one launch: product i reads A + i * stride_a, B + i * stride_b and
  * writes C + i * stride_c (strides in elements, 0 shares an operand).  This is what the per-head host
  * loop of srcs/transformers/sdp.hpp:258-271 (one tensor_mm launch per head for Q K^T and again for P V)

@@ -10,6 +10,8 @@ from anygpu_amd import synth
 
 pytestmark = pytest.mark.gpu
 
+GRANULE = 2 << 20      # the runtime hands device memory out and takes it back in pieces of 2 MiB
+
 
 def _operands(heads, kv_heads, n_q, n_k, d, seed):
     import torch
@@ -41,11 +43,15 @@ def test_decode_static_scratch_matches_workspace_form_on_two_calls(ops, oracle):
         assert lib.anygpu_sdp_attention_decode_f16(q.data_ptr(), k.data_ptr(), v.data_ptr(), want.data_ptr(), ws.data_ptr(), need,
                                                    *shape, alpha, cap, causal, window, None) == capi.ANYGPU_OK
         torch.cuda.synchronize()
-        before = torch.cuda.memory_allocated()
+        # free device memory as the driver reports it: sees an allocation by the library or the runtime (queue scratch
+        # of a kernel with a private segment), which torch's own allocator statistics would not
+        free_before = torch.cuda.mem_get_info()[0]
+        allocated_before = torch.cuda.memory_allocated()
         assert lib.anygpu_sdp_attention_decode_f16_static(q.data_ptr(), k.data_ptr(), v.data_ptr(), got.data_ptr(),
                                                           *shape, alpha, cap, causal, window, None) == capi.ANYGPU_OK
         torch.cuda.synchronize()
-        assert torch.cuda.memory_allocated() == before
+        assert torch.cuda.memory_allocated() == allocated_before
+        assert free_before - torch.cuda.mem_get_info()[0] < GRANULE, "device memory was allocated during the call"
         assert torch.equal(got, want), f"case {i}: static-scratch form differs from the workspace form"
         # and the workspace form itself against the oracle (fp16 row-op tolerance, doubled for the two roundings of p)
         ref = oracle.sdp_attention_rules(*(oracle.cvt_f16_to_f32(t.cpu().numpy()) for t in (q, k, v)), alpha=alpha, softcap=cap,
@@ -69,3 +75,42 @@ def test_decode_static_scratch_rejects_what_does_not_fit(ops):
     assert f(q.data_ptr(), kv.data_ptr(), kv.data_ptr(), y.data_ptr(), 8, 2, 9, 100, 64, 0.125, 0.0, 1, 0, None) == capi.ANYGPU_ERR_UNSUPPORTED
     torch.cuda.synchronize()
     assert bool((y == 3.0).all())
+
+
+def test_decode_static_scratch_replayed_from_a_graph(ops):
+    # the use the entry point is for: captured into a graph (no allocation may happen under capture), replayed several
+    # times with eager work and synchronisations in between, every replay equal to the eager result bit for bit
+    import torch
+    from anygpu_amd import capi
+    lib = capi.load()
+    f = lib.anygpu_sdp_attention_decode_f16_static
+    assert f(None, None, None, None, 0, 1, 1, 100, 64, 0.125, 0.0, 1, 0, None) == capi.ANYGPU_OK      # set-up call, outside capture
+    heads, kv_heads, n_q, n_k, d = 8, 4, 1, 5000, 256
+    q, k, v = _operands(heads, kv_heads, n_q, n_k, d, 70)
+    shape = (heads, heads // kv_heads, n_q, n_k, d)
+    eager = torch.full_like(q, 5.0)
+    assert f(q.data_ptr(), k.data_ptr(), v.data_ptr(), eager.data_ptr(), *shape, 0.0625, 50.0, 1, 4096, None) == capi.ANYGPU_OK
+    torch.cuda.synchronize()
+    out = torch.full_like(q, 6.0)
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
+    with torch.cuda.graph(graph, stream=side):
+        rc = f(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), *shape, 0.0625, 50.0, 1, 4096,
+               torch.cuda.current_stream().cuda_stream)
+    assert rc == capi.ANYGPU_OK
+    assert bool((out == 6.0).all())                      # capture launches nothing
+    other_q, other_k, other_v = _operands(4, 2, 2, 900, 64, 80)
+    other = torch.empty_like(other_q)
+    for replay in range(3):
+        out.fill_(float(replay))
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager), f"replay {replay} differs from the eager call"
+        # the library's own eager work between the replays, through the same array
+        assert f(other_q.data_ptr(), other_k.data_ptr(), other_v.data_ptr(), other.data_ptr(), 4, 2, 2, 900, 64, 0.125, 0.0, 1, 0,
+                 None) == capi.ANYGPU_OK
+        torch.cuda.synchronize()
+    # (the graph object itself holds a little memory of the runtime's; the library's 64 MiB workspace would show)
+    assert free_before - torch.cuda.mem_get_info()[0] < 16 * GRANULE
