@@ -65,7 +65,7 @@ def main() -> None:
 
     # 1. the reference generator's case at a committed size: [1, heads, N, d], additive tril -inf mask, scale 0.125
     d = case_dir("torch_sdp_fwd_masked_scaled_f32")
-    heads, n, dh = 4, 16, 32
+    heads, n, dh = 4, 16, 128                                        # the generator's N = 16, d = 128 with 4 of its 32 heads
     q, k, v = (synth.normal(300 + i, (1, heads, n, dh)) for i in range(3))
     mask = torch.zeros(1, 1, n, n, dtype=torch.float64)
     mask.masked_fill_(torch.ones(1, 1, n, n, dtype=torch.bool).tril(diagonal=0).logical_not(), float("-inf"))
