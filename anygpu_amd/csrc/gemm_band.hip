@@ -379,10 +379,15 @@ struct WorkspaceEntry
 	float* base;
 	size_t bytes;
 	bool from_caller;
+	uint64_t last_use;                        // value of use_clock at the entry's last acquisition
 };
 
 std::mutex workspace_lock;
 std::map<std::pair<int, hipStream_t>, WorkspaceEntry> workspaces;
+uint64_t use_clock = 0;
+// The library keeps at most this many buffers of its own (ANYGPU_MAX_OWN_WORKSPACES in the header); a stream beyond that
+// takes over the place of the one used longest ago.
+constexpr size_t kMaxOwnWorkspaces = 8;
 
 bool stream_is_capturing(hipStream_t stream)
 {
@@ -442,8 +447,32 @@ hipError_t band::workspace_acquire(hipStream_t stream, float** base)
 	const auto found = workspaces.find(key);
 	if (found != workspaces.end())
 	{
+		found->second.last_use = ++use_clock;
 		*base = reinterpret_cast<float*>(reinterpret_cast<char*>(found->second.base) + reserved_front);
 		return hipSuccess;
+	}
+	// Streams come and go and the library does not see them go: when it already owns its limit of buffers, the one
+	// used longest ago makes way.  hipFree waits for the device, so work that may still use that buffer has finished.
+	size_t own = 0;
+	auto oldest = workspaces.end();
+	for (auto it = workspaces.begin(); it != workspaces.end(); ++it)
+	{
+		if (it->second.from_caller) continue;
+		++own;
+		if (oldest == workspaces.end() || it->second.last_use < oldest->second.last_use) oldest = it;
+	}
+	if (own >= kMaxOwnWorkspaces && oldest != workspaces.end())
+	{
+		int current = device;
+		if (oldest->first.first != device) (void)hipSetDevice(oldest->first.first);
+		const hipError_t freed = hipFree(oldest->second.base);
+		if (oldest->first.first != device) (void)hipSetDevice(current);
+		if (freed != hipSuccess)
+		{
+			(void)hipGetLastError();
+			return freed;
+		}
+		workspaces.erase(oldest);
 	}
 	// First cut on this stream.  Another thread may be capturing some other stream in the global mode, in which an
 	// allocation made anywhere invalidates its capture: this thread allocates in the relaxed mode.
@@ -457,7 +486,7 @@ hipError_t band::workspace_acquire(hipStream_t stream, float** base)
 		(void)hipGetLastError();
 		return err;
 	}
-	workspaces.emplace(key, WorkspaceEntry{static_cast<float*>(mem), kBandPartialBytes, false});
+	workspaces.emplace(key, WorkspaceEntry{static_cast<float*>(mem), kBandPartialBytes, false, ++use_clock});
 	*base = reinterpret_cast<float*>(static_cast<char*>(mem) + reserved_front);
 	return hipSuccess;
 }
@@ -481,7 +510,7 @@ int band::workspace_set(hipStream_t stream, void* base, size_t bytes)
 		}
 		workspaces.erase(found);
 	}
-	if (base != nullptr && bytes > 0) workspaces.emplace(key, WorkspaceEntry{static_cast<float*>(base), bytes, true});
+	if (base != nullptr && bytes > 0) workspaces.emplace(key, WorkspaceEntry{static_cast<float*>(base), bytes, true, ++use_clock});
 	return ANYGPU_OK;
 }
 

@@ -3,6 +3,7 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+#include <atomic>
 #include <cstdint>
 
 namespace anygpu {
@@ -15,16 +16,18 @@ inline void discard_stale_error() { (void)hipGetLastError(); }
 // Compute units of the current device (256 on an MI355X), asked once per device; 256 if the runtime cannot tell.
 inline int device_cu_count()
 {
-	static int cached[64] = {};
+	// (launchers on several host threads may ask at once: the cache is written and read atomically, and two threads
+	// that both find it empty store the same value)
+	static std::atomic<int> cached[64] = {};
 	int device = 0;
 	if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64) return 256;
-	if (cached[device] == 0)
+	int cus = cached[device].load(std::memory_order_relaxed);
+	if (cus == 0)
 	{
-		int cus = 0;
 		if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || cus <= 0) cus = 256;
-		cached[device] = cus;
+		cached[device].store(cus, std::memory_order_relaxed);
 	}
-	return cached[device];
+	return cus;
 }
 
 // mask (may be NULL): additive [q_len, cols] matrix of the element type, rows mask_stride apart

@@ -61,7 +61,10 @@ const char* anygpu_hip_target(void);            /* "gfx950" */
 const char* anygpu_hip_error_string(int code);  /* text for ANYGPU_ERR_* and for hipError_t values */
 
 /*
- * The K-split workspace of the GEMM entry points (all of anygpu_gemm_*), per (current device, stream).
+ * The workspace of a (current device, stream) pair.  Who uses it: every anygpu_gemm_* entry point (partial sums of
+ * products cut along K, aligned copies of operands that cannot be fetched where they lie) and the fused attention
+ * anygpu_sdp_attention_fwd_f16 / _f32 (partial results of query blocks whose keys are walked in two halves).  The decode
+ * attention takes its workspace as an argument instead.
  *
  * anygpu_set_workspace(stream, workspace, bytes) hands in `bytes` of device memory, 256-byte aligned, for the launches
  * made on `stream` from now on: the library then allocates nothing for that stream, plans its cuts along K within
@@ -74,11 +77,16 @@ const char* anygpu_hip_error_string(int code);  /* text for ANYGPU_ERR_* and for
  * scratch: its ops layer allocates every buffer and its kernels none (srcs/core/tensor.hpp:56-57).
  *
  * anygpu_release_workspaces() frees every buffer the library itself allocated (on all devices) and forgets all
- * registrations; call it when no GEMM of this library is in flight.  Every (device, stream) pair that cuts a product
- * without a caller's workspace holds ANYGPU_WORKSPACE_BYTES until then; the library does not notice a stream being
- * destroyed.
+ * registrations; call it when no launch of this library is in flight.  A (device, stream) pair that needs a workspace
+ * and has none from the caller takes ANYGPU_WORKSPACE_BYTES from the library at its first eager launch of that kind.
+ * The library does not notice a stream being destroyed, so it bounds what it holds itself: at most
+ * ANYGPU_MAX_OWN_WORKSPACES buffers; a further stream takes the place of the one used longest ago (whose buffer is
+ * freed, which waits for the device).  A caller's registration is the caller's to take back: call
+ * anygpu_set_workspace(stream, NULL, 0) before destroying a stream that has one, or a later stream that the runtime
+ * gives the same handle would write into that memory.
  */
 #define ANYGPU_WORKSPACE_BYTES (64 * 1024 * 1024)
+#define ANYGPU_MAX_OWN_WORKSPACES 8
 
 int anygpu_set_workspace(void* stream, void* workspace, int64_t bytes);
 int anygpu_release_workspaces(void);
@@ -108,7 +116,10 @@ int anygpu_gemm_f16_f32acc(const void* A, const void* B, void* C,
  *                                                       cu_mlp_gemma2_fused_upproj_f32_v1 / _v2); A is read once, B_gate and
  *                                                       B_up share b_layout and ldb
  * The reference runs these layers in float32 (anygpu_gemm_f32 and its _softcap / _gelu_mul forms); these are the same
- * operators for a model held in fp16.  K >= 1.  _gelu_mul needs 16-byte aligned operand rows, K >= 64 and K a multiple
+ * operators for a model held in fp16.  K >= 1.  One exception to "before the one rounding": operands no tile kernel can
+ * fetch and no copy is made of (K or N no multiple of 8 with fewer than 64 rows or without a workspace to copy into)
+ * run the plain product, rounded to fp16, and a pass over it that adds the bias or applies the softcap and rounds
+ * again; such results agree with the fused ones to the tolerance of the fp16 product (1e-2), not bit for bit.  _gelu_mul needs 16-byte aligned operand rows, K >= 64 and K a multiple
  * of 8 (with row-major B also N a multiple of 8) unless M <= 64; other shapes return ANYGPU_ERR_UNSUPPORTED.
  */
 int anygpu_gemm_f16_f32acc_bias(const void* A, const void* B, const void* bias, void* C,
@@ -265,6 +276,12 @@ int anygpu_softmax_rows_masked_f32(const float* x, const float* mask, float* y,
  * tensor_mm, tensor_mul, tensor_add, tensor_softmax, tensor_mm per head) for masks that are index rules, and
  * is the half-precision counterpart of cu_flash_sdpa_fwd_d256_v1 (srcs/kernels/cuda/flash_sdpa_fwd.cuh:6-15,
  * fp32, head_dim 256, no mask).
+ * Scratch: a launch with at least a block per compute unit whose longest query blocks would make the launch end
+ * unevenly (long key ranges under a sliding window) walks the keys of those blocks in two halves and passes their
+ * partial results through the stream's workspace (anygpu_set_workspace).  Without a caller's workspace the first such
+ * eager launch on a stream makes the library allocate ANYGPU_WORKSPACE_BYTES; a stream under capture without a
+ * caller's workspace runs whole blocks, whose sums are formed in another order (equal to the tolerance, not bit for
+ * bit).  The same holds for anygpu_sdp_attention_fwd_f32.
  */
 int anygpu_sdp_attention_fwd_f16(const void* q, const void* k, const void* v, void* y,
                                  int64_t batch_heads, int64_t q_per_kv, int64_t n_q, int64_t n_k, int64_t head_dim,

@@ -1963,6 +1963,36 @@ def test_release_workspaces_returns_the_memory(ops):
     ops.release_workspaces()
 
 
+def test_library_owned_workspaces_are_bounded(ops):
+    # streams come and go without the library seeing it: it keeps at most MAX_OWN_WORKSPACES buffers of its own, a
+    # further stream takes the place of the one used longest ago
+    import torch
+    from anygpu_amd import capi
+    ops.release_workspaces()
+    a = dev(synth.uniform(1, (24, 8192)))
+    w = dev(synth.uniform(2, (260, 8192)))
+    want = host(ops.tensor_mm(a, w, b_layout=capi.B_COL_MAJOR))
+    ops.release_workspaces()
+    torch.cuda.synchronize()
+    free0 = torch.cuda.mem_get_info()[0]
+    streams = [torch.cuda.Stream() for _ in range(capi.MAX_OWN_WORKSPACES + 3)]
+    outs = []
+    for st in streams:
+        with torch.cuda.stream(st):
+            outs.append(ops.tensor_mm(a, w, b_layout=capi.B_COL_MAJOR))     # few rows, deep K: cut, into the library's own buffer
+    torch.cuda.synchronize()
+    held = free0 - torch.cuda.mem_get_info()[0]
+    assert held <= capi.MAX_OWN_WORKSPACES * capi.WORKSPACE_BYTES + (32 << 20), held
+    assert held >= (capi.MAX_OWN_WORKSPACES - 1) * capi.WORKSPACE_BYTES
+    for out in outs:
+        assert np.array_equal(host(out), want)
+    # the first streams lost their buffers to the later ones and simply get new ones
+    with torch.cuda.stream(streams[0]):
+        again = ops.tensor_mm(a, w, b_layout=capi.B_COL_MAJOR)
+    assert np.array_equal(host(again), want)
+    ops.release_workspaces()
+
+
 def test_k_split_products_on_concurrent_streams(ops, oracle):
     # every stream owns its partial-sum workspace: products that are cut along K may overlap on different streams
     import torch
