@@ -88,6 +88,11 @@ def parse_args():
     ap.add_argument("--only", default="", help="comma list of: gemm,gemm32,conv,softmax,attn,attn32,decode,norm (default: all)")
     ap.add_argument("--gemm-shapes", nargs="?", const="f16", default=None, choices=("f16", "f32"),
                     help="print the table of GEMM layer shapes (fp16, or fp32 with `--gemm-shapes f32`) against torch.matmul and exit")
+    ap.add_argument("--gemm-operands", default="uniform", choices=("uniform", "low_toggle"),
+                    help="operands of the headline GEMM: U(-1, 1) as the metric names them (default), or integers -2 .. 2 "
+                         "(few bits toggle: for profiler runs of the power-limit comparison; the line then says so)")
+    ap.add_argument("--skip-low-toggle", action="store_true",
+                    help="leave out the headline's second leg on low-toggle operands (for profiler runs that must see one operand set only)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain device copy of 256 MiB (read 256 MiB + write 256 MiB) a few times, "
                          "as the known-size reference for scaling FETCH_SIZE / WRITE_SIZE counter readings")
@@ -181,10 +186,14 @@ def gemm_f16_clock_probe(torch, capi, a, bt, c, n):
             "main_loop_us_min": float(ns.min() / 1e3), "main_loop_us_slowest_xcd": max(per_xcd), "main_loop_us_fastest_xcd": min(per_xcd)}
 
 
-def bench_gemm_f16(torch, ops, capi, synth, steps, warmup):
+def bench_gemm_f16(torch, ops, capi, synth, steps, warmup, operands="uniform", low_toggle_leg=True):
     n = 4096
-    a = torch.from_numpy(synth.uniform(0, (n, n)).astype("float16")).cuda()
-    bt = torch.from_numpy(synth.uniform(1, (n, n)).astype("float16")).cuda()   # B stored [N, K]
+    if operands == "low_toggle":
+        a = torch.from_numpy(synth.integers(0, (n, n), -2, 2).astype("float16")).cuda()
+        bt = torch.from_numpy(synth.integers(1, (n, n), -2, 2).astype("float16")).cuda()
+    else:
+        a = torch.from_numpy(synth.uniform(0, (n, n)).astype("float16")).cuda()
+        bt = torch.from_numpy(synth.uniform(1, (n, n)).astype("float16")).cuda()   # B stored [N, K]
     c = torch.empty((n, n), dtype=torch.float16, device="cuda")
     # (the headline times exactly --steps launches; only the kernels below are floored)
     t = timed_region(torch, lambda: ops.tensor_mm(a, bt, out=c, b_layout=capi.B_COL_MAJOR), steps, warmup, floor=1)
@@ -197,13 +206,17 @@ def bench_gemm_f16(torch, ops, capi, synth, steps, warmup):
     # The same launch on operands that toggle few bits (integers -2 .. 2, same shapes, layout, kernel and launch
     # count): the matrix cores do the same number of operations, the data paths switch less, the part draws less
     # power and holds a higher clock.  What this run gains over the U(-1, 1) run is what the power limit takes.
-    a_lo = torch.from_numpy(synth.integers(0, (n, n), -2, 2).astype("float16")).cuda()
-    bt_lo = torch.from_numpy(synth.integers(1, (n, n), -2, 2).astype("float16")).cuda()
-    floor_lo = 1 if steps >= MIN_TIMED_LAUNCHES else MIN_TIMED_LAUNCHES
-    t_lo = timed_region(torch, lambda: ops.tensor_mm(a_lo, bt_lo, out=c, b_layout=capi.B_COL_MAJOR), steps, warmup, floor=floor_lo)
-    t_vendor_lo = timed_region(torch, lambda: torch.matmul(a_lo, bt_lo.t(), out=c), steps, warmup, floor=floor_lo)
-    clock_lo = gemm_f16_clock_probe(torch, capi, a_lo, bt_lo, c, n)
-    del a_lo, bt_lo
+    low_toggle = None
+    if low_toggle_leg:
+        a_lo = torch.from_numpy(synth.integers(0, (n, n), -2, 2).astype("float16")).cuda()
+        bt_lo = torch.from_numpy(synth.integers(1, (n, n), -2, 2).astype("float16")).cuda()
+        floor_lo = 1 if steps >= MIN_TIMED_LAUNCHES else MIN_TIMED_LAUNCHES
+        t_lo = timed_region(torch, lambda: ops.tensor_mm(a_lo, bt_lo, out=c, b_layout=capi.B_COL_MAJOR), steps, warmup, floor=floor_lo)
+        t_vendor_lo = timed_region(torch, lambda: torch.matmul(a_lo, bt_lo.t(), out=c), steps, warmup, floor=floor_lo)
+        clock_lo = gemm_f16_clock_probe(torch, capi, a_lo, bt_lo, c, n)
+        del a_lo, bt_lo
+        low_toggle = {"us": t_lo["us_per_launch"], "median_us": t_lo["median_us"], "vendor_us": t_vendor_lo["us_per_launch"],
+                      "timed_launches": t_lo["steps"], "clock": clock_lo}
     return {
         "timing": t, "flops": flops,
         "tflops_host": flops * t["steps"] / t["host_s"] / 1e12,
@@ -212,8 +225,7 @@ def bench_gemm_f16(torch, ops, capi, synth, steps, warmup):
         "vendor": {"what": "torch.matmul (hipBLASLt) on the same operands, timed the same way right after",
                    "us_per_launch": t_vendor["us_per_launch"], "median_us": t_vendor["median_us"], "min_us": t_vendor["min_us"]},
         "clock": clock,
-        "low_toggle": {"us": t_lo["us_per_launch"], "median_us": t_lo["median_us"], "vendor_us": t_vendor_lo["us_per_launch"],
-                       "timed_launches": t_lo["steps"], "clock": clock_lo},
+        "low_toggle": low_toggle,
     }
 
 
@@ -638,7 +650,7 @@ def main():
         torch.cuda.synchronize()
         del src, dst
     if want("gemm"):
-        gemm = bench_gemm_f16(torch, ops, capi, synth, args.steps, args.warmup)
+        gemm = bench_gemm_f16(torch, ops, capi, synth, args.steps, args.warmup, args.gemm_operands, not args.skip_low_toggle)
     if want("gemm32"):
         kernels.append(bench_gemm_f32(torch, ops, synth, args.steps // 2, args.warmup, cpu_side))
     if want("conv"):
@@ -672,32 +684,37 @@ def main():
                                "fp32 accumulate on MFMA, fp16 output (BASELINE.json configs[1])"},
         "device": {"name": props.name, "compute_units": props.multi_processor_count, "peak_clock_ghz": PEAK_CLOCK_GHZ},
     }
+    if args.gemm_operands != "uniform":
+        line["config"]["workload"] = ("NOT the metric's operands: fp16 GEMM M=N=K=4096 on integers -2 .. 2 (--gemm-operands low_toggle), "
+                                      "same shapes, layout and kernel; for the power-limit comparison only")
     if gemm is not None:
         t = gemm["timing"]
         line["value"] = gemm["tflops_host"]
         line["ms_per_step"] = t["host_s"] / t["steps"] * 1e3
         clock = gemm["clock"]
         peak_at_clock = props.multi_processor_count * FP16_FLOP_PER_CLK_PER_CU * clock["sustained_clock_ghz"] * 1e9 / 1e12
-        lo = gemm["low_toggle"]
-        lo_tflops = gemm["flops"] / (lo["us"] * 1e-6) / 1e12
         line["roofline"] = {"bound": "mfma", "achieved": gemm["tflops_event"], "peak": PEAK_FP16_TFLOPS,
                             "unit": "TFLOP/s", "frac": gemm["tflops_event"] / PEAK_FP16_TFLOPS,
                             **traffic_fields("gemm_f16"), **timing_fields(t),
                             "algorithmic_flops": gemm["flops"], "min_bytes": 3 * 4096 * 4096 * 2,
                             **clock, "peak_at_sustained_clock": peak_at_clock,
                             "frac_at_sustained_clock": gemm["tflops_event"] / peak_at_clock,
-                            # scalars: the vendor library (torch.matmul = hipBLASLt) on the same operands in the same run, and
-                            # the same launch of this library and of the vendor's on integers -2 .. 2 (same shapes and layout)
+                            # scalars: the vendor library (torch.matmul = hipBLASLt) on the same operands in the same run
                             "vendor_us": gemm["vendor"]["us_per_launch"],
                             "vendor_frac": gemm["flops"] / (gemm["vendor"]["us_per_launch"] * 1e-6) / 1e12 / PEAK_FP16_TFLOPS,
-                            "low_toggle_us": lo["us"], "low_toggle_median_us": lo["median_us"],
-                            "low_toggle_frac": lo_tflops / PEAK_FP16_TFLOPS,
-                            "low_toggle_clock_ghz": lo["clock"]["sustained_clock_ghz"],
-                            "low_toggle_mfma_busy_in_main_loop": lo["clock"]["mfma_busy_in_main_loop"],
-                            "vendor_low_toggle_us": lo["vendor_us"],
-                            "low_toggle_operands": "integers -2 .. 2 (seeds 0 / 1) in place of U(-1, 1); same kernel, shapes, layout; "
-                                                   f"{lo['timed_launches']} launches after the settle period and warm-up",
                             "vendor_library": gemm["vendor"]}
+        lo = gemm["low_toggle"]
+        if lo is not None:
+            # the same launch of this library and of the vendor's on integers -2 .. 2 (same shapes, layout and kernel)
+            lo_tflops = gemm["flops"] / (lo["us"] * 1e-6) / 1e12
+            line["roofline"].update({
+                "low_toggle_us": lo["us"], "low_toggle_median_us": lo["median_us"],
+                "low_toggle_frac": lo_tflops / PEAK_FP16_TFLOPS,
+                "low_toggle_clock_ghz": lo["clock"]["sustained_clock_ghz"],
+                "low_toggle_mfma_busy_in_main_loop": lo["clock"]["mfma_busy_in_main_loop"],
+                "vendor_low_toggle_us": lo["vendor_us"],
+                "low_toggle_operands": "integers -2 .. 2 (seeds 0 / 1) in place of U(-1, 1); same kernel, shapes, layout; "
+                                       f"{lo['timed_launches']} launches after the settle period and warm-up"})
         line["gemm_f16_other_shapes"] = sample_gemm_shapes(torch, ops, capi)
         if args.cpu_seconds > 0:
             import oracle
