@@ -396,6 +396,11 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
 			return hipSuccess;
 		}
 	}
+	// few rows against n-contiguous weights with so many columns that they alone fill the chip (the output head): the
+	// band kernel that transposes 8 x 8 blocks of the weights in its registers (2304 x 256000, 16 - 64 rows: the tile kernels
+	// take 234 - 282 us, the vendor library 215 - 230)
+	if (batch == 1 && b_layout == ANYGPU_B_ROW_MAJOR && gemm_band_kn_f16_applies(A, B, C, M, N, K, lda, ldb, ldc))
+		return launch_gemm_band_kn_f16(A, B, C, M, N, K, lda, ldb, ldc, kEpiBias, 0.0f, stream);
 	if (batch == 1 && !tiles_first && gemm_band_applies<half_t>(a, b, nullptr, c, M, N, K, lda, ldb, ldc, b_layout))
 		return launch_gemm_band<half_t>(a, b, nullptr, nullptr, c, M, N, K, lda, ldb, ldc, 0, 0.0f, stream);
 	if (batch == 1 && !tiles_first && gemm_skinny_applies<half_t>(a, b, nullptr, M, N, K, lda, ldb, b_layout))
@@ -654,6 +659,8 @@ hipError_t launch_gemm_f16_epilogue(const void* A, const void* B, const void* B2
 	const bool tiles_ok = aligned && K >= 64 && K % 8 == 0 && (b_layout == ANYGPU_B_COL_MAJOR || N % 8 == 0);
 	if (epilogue != kEpiBias && gemm_band_applies<half_t>(a, b, b2, c, M, N, K, lda, ldb, ldc, b_layout))
 		return launch_gemm_band<half_t>(a, b, b2, nullptr, c, M, N, K, lda, ldb, ldc, epilogue, ep_param, stream);
+	if (epilogue == kEpiSoftcap && b_layout == ANYGPU_B_ROW_MAJOR && gemm_band_kn_f16_applies(A, B, C, M, N, K, lda, ldb, ldc))
+		return launch_gemm_band_kn_f16(A, B, C, M, N, K, lda, ldb, ldc, kEpiSoftcap, ep_param, stream);
 	if (!tiles_ok)
 	{
 		if (dual)

@@ -70,6 +70,13 @@ bool gemm_f16_probe_applies(const void* A, const void* B, const void* C, int64_t
 hipError_t launch_gemm_f16_probe(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K,
                                  int64_t lda, int64_t ldb, int64_t ldc, unsigned long long* probe, hipStream_t stream);
 
+// Few rows (M <= 64) against n-contiguous fp16 weights with very many columns (gemm_band_kn_f16.hip); epilogue kEpiBias
+// (nothing added) or kEpiSoftcap.
+bool gemm_band_kn_f16_applies(const void* A, const void* B, const void* C, int64_t M, int64_t N, int64_t K,
+                              int64_t lda, int64_t ldb, int64_t ldc);
+hipError_t launch_gemm_band_kn_f16(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K,
+                                   int64_t lda, int64_t ldb, int64_t ldc, int epilogue, float ep_param, hipStream_t stream);
+
 // dst[i] = src[i] over nvec 16-byte vectors in the stated launch geometry (stream_probe.hip)
 hipError_t launch_stream_probe(const void* src, void* dst, int64_t nvec, int block, int vectors_per_lane, int nt_load,
                                int nt_store, int64_t grid_limit, hipStream_t stream);

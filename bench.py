@@ -587,8 +587,8 @@ def sweep_gemm_shapes(torch, ops, capi, dtype_name="f16"):
 
 
 def sample_gemm_shapes(torch, ops, capi):
-    """A few products that do not fill the chip with 256 x 256 tiles, ragged ones and ones the chunk loads cannot fetch,
-    next to torch.matmul on the same operands: microseconds, the better of two runs of 40 launches each side."""
+    """A few products that do not fill the chip with 256 x 256 tiles, ragged ones, ones the chunk loads cannot fetch and two
+    output heads with [K, N] weights and few rows, next to torch.matmul on the same operands: microseconds, the better of two runs of 40 launches each side."""
     def timed(fn, iters=40, warm=10):
         for _ in range(warm):
             fn()
@@ -603,7 +603,8 @@ def sample_gemm_shapes(torch, ops, capi):
 
     out = []
     for m, n, k, layout in [(2048, 2048, 2048, "col"), (512, 6144, 4096, "col"), (1024, 4096, 4096, "col"), (2048, 4096, 4096, "col"),
-                            (4096, 4096, 4096, "row"), (4000, 4000, 4096, "col"), (4096, 4100, 4096, "row")]:
+                            (4096, 4096, 4096, "row"), (4000, 4000, 4096, "col"), (4096, 4100, 4096, "row"),
+                            (16, 256000, 2304, "row"), (64, 128256, 4096, "row")]:
         a = (torch.rand(m, k, device="cuda") * 2 - 1).half()
         b = (torch.rand(n, k, device="cuda") * 2 - 1).half() if layout == "col" else (torch.rand(k, n, device="cuda") * 2 - 1).half()
         c = torch.empty(m, n, device="cuda", dtype=torch.half)

@@ -1002,6 +1002,46 @@ def test_mm_row_bands_rows_of_any_length(ops, oracle, m, k, n):
     assert bool((cbuf[:, n:] == -1.0).all())
 
 
+@pytest.mark.parametrize("m,k,n", [(1, 64, 131072), (8, 96, 131080), (16, 32, 200000), (17, 160, 140000), (33, 128, 131592),
+                                   (48, 64, 131072), (64, 224, 132096), (8, 96, 32000), (40, 160, 65544), (64, 64, 24576),
+                                   (3, 32, 100000), (20, 288, 50264), (24, 64, 65536), (32, 96, 65544)])
+def test_mm_f16_row_bands_n_contiguous_weights_many_columns(ops, oracle, m, k, n):
+    # few rows against [K, N] fp16 weights with the columns of an output head: the band kernel that transposes 8 x 8
+    # blocks of the weights in registers, waves side by side (from about 123000 columns) or sharing their columns and
+    # dividing K; small integers, so every sum is exact in fp16
+    import torch
+    from anygpu_amd import capi
+    a = synth.integers(m + 11, (m, k), -2, 2)
+    b = synth.integers(n + 12, (k, n), -2, 2)
+    want = oracle.tensor_mm(a, b, threads=8)
+    assert np.abs(want).max() <= 2048
+    da, db = dev(a.astype(np.float16)), dev(b.astype(np.float16))
+    got = host(ops.tensor_mm(da, db)).astype(np.float32)
+    assert np.array_equal(got, want)
+    # operands and result inside wider buffers: nothing beyond column n is touched
+    abuf = torch.zeros((m, k + 8), device="cuda", dtype=torch.float16)
+    bbuf = torch.zeros((k, n + 16), device="cuda", dtype=torch.float16)
+    abuf[:, :k], bbuf[:, :n] = da, db
+    cbuf = torch.full((m, n + 8), -1.0, device="cuda", dtype=torch.float16)
+    ops.tensor_mm(abuf[:, :k], bbuf[:, :n], out=cbuf[:, :n])
+    assert np.array_equal(host(cbuf[:, :n]).astype(np.float32), want)
+    assert bool((cbuf[:, n:] == -1.0).all())
+    # uniform operands against the oracle at the fp16 GEMM tolerance, and the softcap epilogue on the same sums
+    au = synth.uniform(m + 13, (m, k)).astype(np.float16)
+    bu = synth.uniform(n + 14, (k, n)).astype(np.float16)
+    ref = oracle.tensor_mm(oracle.cvt_f16_to_f32(au), oracle.cvt_f16_to_f32(bu), threads=8)
+    dau, dbu = dev(au), dev(bu)
+    got = host(ops.tensor_mm(dau, dbu)).astype(np.float32)
+    assert scaled_rel_err(got, ref, math.sqrt(k) / 3.0) <= TOL_F16_GEMM
+    out = torch.empty((m, n), device="cuda", dtype=torch.float16)
+    lib = capi.load()
+    capi.check("anygpu_gemm_f16_f32acc_softcap",
+               lib.anygpu_gemm_f16_f32acc_softcap(dau.data_ptr(), dbu.data_ptr(), out.data_ptr(), m, n, k, k, n, n, capi.B_ROW_MAJOR,
+                                                  2.0, torch.cuda.current_stream().cuda_stream))
+    capped = oracle.softcap(ref, 2.0).reshape(m, n)
+    assert scaled_rel_err(host(out).astype(np.float32), capped, 2.0 / 3.0) <= TOL_F16_GEMM
+
+
 @pytest.mark.parametrize("m,k,n", [(512, 256, 1003), (300, 512, 259), (128, 64, 65), (1000, 128, 4097), (65, 192, 7), (257, 320, 511)])
 def test_mm_f16_k_contiguous_weights_result_rows_of_any_length(ops, oracle, m, k, n):
     # the tile kernels with [N, K] weights: N, the row length of C and its first element are free; integers, exact
