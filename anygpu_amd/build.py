@@ -27,7 +27,7 @@ ORACLE_DIR = REPO_DIR / "oracle"
 
 ROCM_DIR = Path(os.environ.get("ROCM_PATH", "/opt/rocm"))
 GPU_ARCH = "gfx950"
-KERNEL_SOURCES = ["softmax.hip", "conv1d.hip", "gemm_f16.hip", "gemm_f32.hip", "gemm_skinny.hip", "gemm_band.hip", "gemm_band_ncontig.hip", "gemm_band_kn_f16.hip", "gemm_repack.hip", "rmsnorm.hip", "attention.hip", "attention_f32.hip", "stream_probe.hip", "capi.hip"]
+KERNEL_SOURCES = ["softmax.hip", "conv1d.hip", "gemm_f16.hip", "gemm_f32.hip", "gemm_skinny.hip", "gemm_band.hip", "gemm_band_ncontig.hip", "gemm_band_kn_f16.hip", "gemm_band_kc_wide.hip", "gemm_repack.hip", "rmsnorm.hip", "attention.hip", "attention_f32.hip", "stream_probe.hip", "capi.hip"]
 
 # -packed-fp32-ops is switched off on purpose: packed fp32 VALU forms are not to be generated.
 DEVICE_FLAGS = [

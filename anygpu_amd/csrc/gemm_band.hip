@@ -181,7 +181,7 @@ __global__ __launch_bounds__(kBandThreads) void gemm_band_kernel(
 			ar[i] = *reinterpret_cast<const Vec*>(A + (int64_t)(row < M ? row : M - 1) * lda + (k < ke ? k : kb));
 		}
 	};
-	auto stage_band = [&](int chunk) {
+	auto stage_band = [&](int slot, int chunk) {
 		const int64_t kc = kb + (int64_t)chunk * S::kChunk;
 #pragma unroll
 		for (int i = 0; i < 4; ++i)
@@ -189,7 +189,7 @@ __global__ __launch_bounds__(kBandThreads) void gemm_band_kernel(
 			const int q = tid + kBandThreads * i;
 			const int row = q / S::kChunkVecs;
 			const bool valid = row < M && kc + (q % S::kChunkVecs) * S::kEV < ke;
-			band[chunk & 1][row * S::kPitchVecs + (q % S::kChunkVecs)] = valid ? ar[i] : zero;
+			band[slot & 1][row * S::kPitchVecs + (q % S::kChunkVecs)] = valid ? ar[i] : zero;
 		}
 	};
 
@@ -222,26 +222,36 @@ __global__ __launch_bounds__(kBandThreads) void gemm_band_kernel(
 	using Guarded = std::true_type;
 	const int full_chunks = (int)((ke - kb) / S::kChunk);          // chunks whose every vector lies inside the range
 	const bool tail = (ke - kb) % S::kChunk != 0;
-	const int64_t last_full_step = (int64_t)full_chunks * S::kStepsPerChunk - 1;
 
-	issue_band(0);
-	if (full_chunks > 0) issue_w(wr[0], 0, Plain{});
-	stage_band(0);
+	// Blocks walk the full chunks of their k range from different starting chunks and wrap around (the chunk with
+	// the ragged end, if any, comes last for all): blocks that run side by side then read different parts of their
+	// weight rows at any one time.  With weight rows a power of two apart, equal offsets in all rows are addresses
+	// that share their low bits, and with them the memory channel.
+	const int first = full_chunks > 1 ? (int)(((blockIdx.x + 977u * blockIdx.y) * 2654435761u >> 8) % (unsigned)full_chunks) : 0;
+	auto chunk_at = [&](int i) {                            // i <= full_chunks; i == full_chunks: the chunk after them
+		if (i >= full_chunks) return i;
+		const int c = i + first;
+		return c >= full_chunks ? c - full_chunks : c;
+	};
+	issue_band(chunk_at(0));
+	if (full_chunks > 0) issue_w(wr[0], (int64_t)chunk_at(0) * S::kStepsPerChunk, Plain{});
+	stage_band(0, chunk_at(0));
 	__syncthreads();
 	for (int c = 0; c < full_chunks; ++c)
 	{
-		issue_band(c + 1);                       // past the end: zeros, staged into a buffer nobody reads
+		const int64_t here = (int64_t)chunk_at(c) * S::kStepsPerChunk;       // first step of this chunk
+		// after the last full step the same step is fetched again and dropped
+		const int64_t after = c + 1 < full_chunks ? (int64_t)chunk_at(c + 1) * S::kStepsPerChunk : here + S::kStepsPerChunk - 1;
+		issue_band(chunk_at(c + 1));             // past the end: zeros, staged into a buffer nobody reads
 #pragma unroll
 		for (int s = 0; s < S::kStepsPerChunk; ++s)
 		{
-			// the loads of the next step are issued before this step's MFMAs; after the last full step the same
-			// step is fetched again and dropped
-			const int64_t next = (int64_t)c * S::kStepsPerChunk + s + 1;
-			issue_w(wr[(s + 1) & 1], next < last_full_step ? next : last_full_step, Plain{});
+			// the loads of the next step are issued before this step's MFMAs
+			issue_w(wr[(s + 1) & 1], s + 1 < S::kStepsPerChunk ? here + s + 1 : after, Plain{});
 			__builtin_amdgcn_sched_barrier(0);
 			multiply(wr[s & 1], c & 1, s);
 		}
-		stage_band(c + 1);
+		stage_band(c + 1, chunk_at(c + 1));
 		__syncthreads();
 	}
 	if (tail)
@@ -538,7 +548,7 @@ bool gemm_band_applies(const T* A, const T* B, const T* B2, const T* C, int64_t 
 {
 	constexpr int EV = 16 / (int)sizeof(T);
 	if (b_layout != ANYGPU_B_COL_MAJOR) return false;
-	if (M < kBandMinRows || M > kBandMaxRows || N < 1 || K < 1) return false;
+	if (M < (sizeof(T) == 4 ? kBandMinRowsF32 : kBandMinRows) || M > kBandMaxRows || N < 1 || K < 1) return false;
 	if ((N + kBandCols - 1) / kBandCols > 0x7FFFFFFFLL) return false;
 	// 33 .. 64 rows: two row blocks per weight register.  Worth it where the weights dominate and the columns or a
 	// deep K give the chip enough blocks (256000 x 2304 fp32, 64 rows: 711 us against 1238 us through the tiles;

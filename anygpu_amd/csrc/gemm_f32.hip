@@ -559,6 +559,11 @@ static hipError_t launch_layout(const float* A, const float* B, const float* B2,
 	                                                     stride_a, stride_b, stride_c, batch, ep_param, small.splits, stream, padded);
 }
 
+// rows from which (below: the skinny kernels, as for the other band kernel) and up to which (above: the fp32 matrix cores, not the memory, are what
+// the product waits for, and the band kernel with the cut along K is as fast) the wide band kernel takes fp32 output heads
+constexpr int64_t kWideMinRowsF32 = 3;
+constexpr int64_t kWideMaxRowsF32 = 16;
+
 hipError_t launch_gemm_f32(const float* A, const float* B, const float* bias, float* C,
                            int64_t M, int64_t N, int64_t K,
                            int64_t lda, int64_t ldb, int64_t ldc,
@@ -620,6 +625,10 @@ hipError_t launch_gemm_f32(const float* A, const float* B, const float* bias, fl
 	// the band kernels (64 x 4096 -> 6144: 45 us as a band, 37 us in tiles; 16 rows of the same: 24 us against 32 us).
 	const bool tiles_first = a_layout == ANYGPU_A_ROW_MAJOR && b_layout == ANYGPU_B_COL_MAJOR && M >= 48 &&
 	                         gemm_f32_ring_applies(A, B, M, N, K, lda, ldb, stride_a, stride_b, batch, 0, 64);
+	// few rows against k-contiguous weights with the columns of an output head: whole lines per row and load instruction
+	if (batch == 1 && a_layout == ANYGPU_A_ROW_MAJOR && b_layout == ANYGPU_B_COL_MAJOR && M >= kWideMinRowsF32 &&
+	    gemm_band_kc_wide_applies<float>(A, B, C, M, N, K, lda, ldb, ldc, kWideMaxRowsF32))
+		return launch_gemm_band_kc_wide<float>(A, B, bias, C, M, N, K, lda, ldb, ldc, kEpiBias, 0.0f, stream);
 	if (batch == 1 && !tiles_first && a_layout == ANYGPU_A_ROW_MAJOR && gemm_band_applies<float>(A, B, nullptr, C, M, N, K, lda, ldb, ldc, b_layout))
 		return launch_gemm_band<float>(A, B, nullptr, bias, C, M, N, K, lda, ldb, ldc, kEpiBias, 0.0f, stream);
 	if (batch == 1 && a_layout == ANYGPU_A_ROW_MAJOR && b_layout == ANYGPU_B_ROW_MAJOR &&
@@ -643,6 +652,8 @@ hipError_t launch_gemm_f32_softcap(const float* A, const float* B, float* C, int
                                    int64_t lda, int64_t ldb, int64_t ldc, int b_layout, float softcap, hipStream_t stream)
 {
 	if (M == 0 || N == 0) return hipSuccess;
+	if (b_layout == ANYGPU_B_COL_MAJOR && M >= kWideMinRowsF32 && gemm_band_kc_wide_applies<float>(A, B, C, M, N, K, lda, ldb, ldc, kWideMaxRowsF32))
+		return launch_gemm_band_kc_wide<float>(A, B, nullptr, C, M, N, K, lda, ldb, ldc, kEpiSoftcap, softcap, stream);
 	if (gemm_band_applies<float>(A, B, nullptr, C, M, N, K, lda, ldb, ldc, b_layout))
 		return launch_gemm_band<float>(A, B, nullptr, nullptr, C, M, N, K, lda, ldb, ldc, kEpiSoftcap, softcap, stream);
 	if (b_layout == ANYGPU_B_ROW_MAJOR && gemm_band_ncontig_applies(A, B, nullptr, C, M, N, K, lda, ldb, ldc, false))

@@ -77,6 +77,15 @@ bool gemm_band_kn_f16_applies(const void* A, const void* B, const void* C, int64
 hipError_t launch_gemm_band_kn_f16(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K,
                                    int64_t lda, int64_t ldb, int64_t ldc, int epilogue, float ep_param, hipStream_t stream);
 
+// Few rows (M <= max_rows <= 64) against k-contiguous weights ([N, K]) with the many columns of an output head, fp32 or
+// fp16 (gemm_band_kc_wide.hip); epilogue kEpiBias (bias may be NULL) or kEpiSoftcap.
+template <typename T>
+bool gemm_band_kc_wide_applies(const T* A, const T* B, const T* C, int64_t M, int64_t N, int64_t K,
+                               int64_t lda, int64_t ldb, int64_t ldc, int64_t max_rows);
+template <typename T>
+hipError_t launch_gemm_band_kc_wide(const T* A, const T* B, const float* bias, T* C, int64_t M, int64_t N, int64_t K,
+                                    int64_t lda, int64_t ldb, int64_t ldc, int epilogue, float ep_param, hipStream_t stream);
+
 // dst[i] = src[i] over nvec 16-byte vectors in the stated launch geometry (stream_probe.hip)
 hipError_t launch_stream_probe(const void* src, void* dst, int64_t nvec, int block, int vectors_per_lane, int nt_load,
                                int nt_store, int64_t grid_limit, hipStream_t stream);
@@ -154,8 +163,10 @@ hipError_t launch_gemm_skinny(const T* A, const T* B, const T* B2, const float* 
 // weights stream through the MFMA operand registers once, K is split over blocks when the columns alone do
 // not fill the chip.  Same arguments as the skinny launchers, which the launchers ask after these: from 5
 // rows on the FMA loops of the skinny kernels fall behind (256000 x 2304 fp32 weights, 8 rows: 511 us
-// against 398 us).
+// against 398 us); in fp32 already from 3 rows (4 rows x 14336 -> 4096: 86 us with FMAs, 41 us as a band;
+// 4096 -> 32768: 113 against 93; the fp16 skinny kernel with its packed dot products holds up to 4 rows).
 constexpr int64_t kBandMinRows = 5;
+constexpr int64_t kBandMinRowsF32 = 3;
 constexpr int64_t kBandMaxRows = 64;
 
 template <typename T>

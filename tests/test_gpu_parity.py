@@ -1042,6 +1042,58 @@ def test_mm_f16_row_bands_n_contiguous_weights_many_columns(ops, oracle, m, k, n
     assert scaled_rel_err(host(out).astype(np.float32), capped, 2.0 / 3.0) <= TOL_F16_GEMM
 
 
+@pytest.mark.parametrize("dtype", ["f16", "f32"])
+@pytest.mark.parametrize("m,steps,n", [(3, 1, 131072), (5, 2, 125000), (8, 3, 131068), (16, 4, 196608), (13, 5, 124672),
+                                       (17, 6, 131072), (32, 2, 125000), (9, 8, 262144)])
+def test_mm_row_bands_k_contiguous_weights_many_columns(ops, oracle, dtype, m, steps, n):
+    # few rows against [N, K] weights with the columns of an output head: the band kernel that loads whole 128-byte
+    # lines per weight row and lets lane pairs exchange halves, blocks starting at different chunks of K (an odd number
+    # of 128-byte steps: all at chunk 0); the column counts give (nearly) two or more blocks of 256 columns per CU
+    # of a 256-CU device, some with a ragged last block.  Row counts outside the kernel's range (fp32: 5 to 16 rows,
+    # fp16: 3 to 32) check the kernels that take those.  Small integers: every sum is exact.
+    import torch
+    from anygpu_amd import capi
+    half = dtype == "f16"
+    tdt, ndt = (torch.float16, np.float16) if half else (torch.float32, np.float32)
+    k = steps * (64 if half else 32)
+    a = synth.integers(m + 21, (m, k), -2, 2)
+    w = synth.integers(n + 22, (n, k), -2, 2)
+    want = oracle.tensor_mm(a, np.ascontiguousarray(w.T), threads=8)
+    assert np.abs(want).max() <= 2048
+    da, dw = dev(a.astype(ndt)), dev(w.astype(ndt))
+    got = host(ops.tensor_mm(da, dw, b_layout=capi.B_COL_MAJOR)).astype(np.float32)
+    assert np.array_equal(got, want)
+    # operands and result inside wider buffers: nothing beyond column n is touched
+    pad = 8 if half else 4
+    abuf = torch.zeros((m, k + pad), device="cuda", dtype=tdt)
+    wbuf = torch.zeros((n, k + 2 * pad), device="cuda", dtype=tdt)
+    abuf[:, :k], wbuf[:, :k] = da, dw
+    cbuf = torch.full((m, n + 4), -1.0, device="cuda", dtype=tdt)
+    ops.tensor_mm(abuf[:, :k], wbuf[:, :k], out=cbuf[:, :n], b_layout=capi.B_COL_MAJOR)
+    assert np.array_equal(host(cbuf[:, :n]).astype(np.float32), want)
+    assert bool((cbuf[:, n:] == -1.0).all())
+    # uniform operands against the oracle at the GEMM tolerance, the softcap epilogue on the same sums, and (fp32) a bias
+    au, wu = synth.uniform(m + 23, (m, k)).astype(ndt), synth.uniform(n + 24, (n, k)).astype(ndt)
+    ref = oracle.tensor_mm(au.astype(np.float32), np.ascontiguousarray(wu.astype(np.float32).T), threads=8)
+    dau, dwu = dev(au), dev(wu)
+    tol = TOL_F16_GEMM if half else TOL_F32
+    got = host(ops.tensor_mm(dau, dwu, b_layout=capi.B_COL_MAJOR)).astype(np.float32)
+    assert scaled_rel_err(got, ref, math.sqrt(k) / 3.0) <= tol
+    out = torch.empty((m, n), device="cuda", dtype=tdt)
+    lib = capi.load()
+    stream = torch.cuda.current_stream().cuda_stream
+    name = "anygpu_gemm_f16_f32acc_softcap" if half else "anygpu_gemm_f32_softcap"
+    capi.check(name, getattr(lib, name)(dau.data_ptr(), dwu.data_ptr(), out.data_ptr(), m, n, k, k, k, n, capi.B_COL_MAJOR, 2.0, stream))
+    capped = oracle.softcap(ref, 2.0).reshape(m, n)
+    assert scaled_rel_err(host(out).astype(np.float32), capped, 2.0 / 3.0) <= tol
+    if not half:
+        bias = synth.uniform(n + 25, (n,))
+        dbias = dev(bias)
+        capi.check("anygpu_gemm_f32", lib.anygpu_gemm_f32(dau.data_ptr(), dwu.data_ptr(), dbias.data_ptr(), out.data_ptr(), m, n, k,
+                                                          k, k, n, capi.A_ROW_MAJOR, capi.B_COL_MAJOR, stream))
+        assert scaled_rel_err(host(out), ref + bias[None, :], math.sqrt(k) / 3.0 + 1.0) <= tol
+
+
 @pytest.mark.parametrize("m,k,n", [(512, 256, 1003), (300, 512, 259), (128, 64, 65), (1000, 128, 4097), (65, 192, 7), (257, 320, 511)])
 def test_mm_f16_k_contiguous_weights_result_rows_of_any_length(ops, oracle, m, k, n):
     # the tile kernels with [N, K] weights: N, the row length of C and its first element are free; integers, exact
