@@ -34,7 +34,8 @@ constexpr int kWidePitchBytes = kWideChunkBytes + 16;   // band rows 272 bytes a
 constexpr int kWideTiles = 4;                      // MFMA column tiles of 16 per wave
 constexpr int kWideWaveCols = 16 * kWideTiles;
 constexpr int kWideBlockCols = 4 * kWideWaveCols;
-constexpr int kWideSets = 3;                       // weight register sets: loads run two steps ahead
+constexpr int kWideSets = 2;                       // weight register sets: loads run a step ahead (three sets: 3 % slower,
+                                                   // the registers cost a wave per SIMD)
 
 typedef int int4v __attribute__((ext_vector_type(4)));
 
@@ -273,6 +274,7 @@ hipError_t launch_gemm_band_kc_wide(const T* A, const T* B, const float* bias, T
 {
 	if (M <= 16) return launch_rows<T, 1>(A, B, bias, C, (int)M, N, K, lda, ldb, ldc, epilogue, ep_param, stream);
 	if (M <= 32) return launch_rows<T, 2>(A, B, bias, C, (int)M, N, K, lda, ldb, ldc, epilogue, ep_param, stream);
+	if (M <= 48) return launch_rows<T, 3>(A, B, bias, C, (int)M, N, K, lda, ldb, ldc, epilogue, ep_param, stream);
 	return launch_rows<T, 4>(A, B, bias, C, (int)M, N, K, lda, ldb, ldc, epilogue, ep_param, stream);
 }
 

@@ -322,7 +322,7 @@ hipError_t launch_gemm_f16_probe(const void* A, const void* B, void* C, int64_t 
 }
 
 // rows up to which the wide band kernel takes fp16 output heads with k-contiguous weights
-constexpr int64_t kWideMaxRowsF16 = 32;
+constexpr int64_t kWideMaxRowsF16 = 64;
 
 hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K,
                            int64_t lda, int64_t ldb, int64_t ldc,
@@ -404,9 +404,8 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
 	// take 234 - 282 us, the vendor library 215 - 230)
 	if (batch == 1 && b_layout == ANYGPU_B_ROW_MAJOR && gemm_band_kn_f16_applies(A, B, C, M, N, K, lda, ldb, ldc))
 		return launch_gemm_band_kn_f16(A, B, C, M, N, K, lda, ldb, ldc, kEpiBias, 0.0f, stream);
-	// the same for k-contiguous weights, from three rows on (one and two rows: the skinny kernels) to 32 (at 64 the band
-	// kernel with the cut along K is as fast or faster): whole 128-byte lines per weight row and load instruction, an
-	// exchange between lane pairs in front of the MFMAs
+	// the same for k-contiguous weights, from three rows on (one and two rows: the skinny kernels): whole 128-byte lines
+	// per weight row and load instruction, an exchange between lane pairs in front of the MFMAs
 	if (batch == 1 && b_layout == ANYGPU_B_COL_MAJOR && M >= 3 && gemm_band_kc_wide_applies<half_t>(a, b, c, M, N, K, lda, ldb, ldc, kWideMaxRowsF16))
 		return launch_gemm_band_kc_wide<half_t>(a, b, nullptr, c, M, N, K, lda, ldb, ldc, kEpiBias, 0.0f, stream);
 	if (batch == 1 && !tiles_first && gemm_band_applies<half_t>(a, b, nullptr, c, M, N, K, lda, ldb, ldc, b_layout))

@@ -559,10 +559,11 @@ static hipError_t launch_layout(const float* A, const float* B, const float* B2,
 	                                                     stride_a, stride_b, stride_c, batch, ep_param, small.splits, stream, padded);
 }
 
-// rows from which (below: the skinny kernels, as for the other band kernel) and up to which (above: the fp32 matrix cores, not the memory, are what
-// the product waits for, and the band kernel with the cut along K is as fast) the wide band kernel takes fp32 output heads
+// rows from which (below: the skinny kernels, as for the other band kernel) and up to which (three row blocks of 16;
+// with four the fp32 matrix cores, not the memory, are what the product waits for, and the band kernel with the cut
+// along K is as fast) the wide band kernel takes fp32 output heads
 constexpr int64_t kWideMinRowsF32 = 3;
-constexpr int64_t kWideMaxRowsF32 = 16;
+constexpr int64_t kWideMaxRowsF32 = 48;
 
 hipError_t launch_gemm_f32(const float* A, const float* B, const float* bias, float* C,
                            int64_t M, int64_t N, int64_t K,

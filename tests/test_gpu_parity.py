@@ -1044,13 +1044,14 @@ def test_mm_f16_row_bands_n_contiguous_weights_many_columns(ops, oracle, m, k, n
 
 @pytest.mark.parametrize("dtype", ["f16", "f32"])
 @pytest.mark.parametrize("m,steps,n", [(3, 1, 131072), (5, 2, 125000), (8, 3, 131068), (16, 4, 196608), (13, 5, 124672),
-                                       (17, 6, 131072), (32, 2, 125000), (9, 8, 262144)])
+                                       (17, 6, 131072), (32, 2, 125000), (9, 8, 262144), (40, 2, 131072), (48, 3, 125000),
+                                       (64, 2, 131072)])
 def test_mm_row_bands_k_contiguous_weights_many_columns(ops, oracle, dtype, m, steps, n):
     # few rows against [N, K] weights with the columns of an output head: the band kernel that loads whole 128-byte
     # lines per weight row and lets lane pairs exchange halves, blocks starting at different chunks of K (an odd number
     # of 128-byte steps: all at chunk 0); the column counts give (nearly) two or more blocks of 256 columns per CU
-    # of a 256-CU device, some with a ragged last block.  Row counts outside the kernel's range (fp32: 5 to 16 rows,
-    # fp16: 3 to 32) check the kernels that take those.  Small integers: every sum is exact.
+    # of a 256-CU device, some with a ragged last block.  Row counts outside the kernel's range (fp32: 3 to 48 rows,
+    # fp16: 3 to 64) check the kernels that take those.  Small integers: every sum is exact.
     import torch
     from anygpu_amd import capi
     half = dtype == "f16"
