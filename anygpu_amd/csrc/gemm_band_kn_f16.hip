@@ -30,7 +30,7 @@ constexpr int kKnStep = 32;                        // k per MFMA step
 constexpr int kKnPitch = kKnChunk + 8;             // halves per band row in LDS: rows 272 bytes apart, no bank conflicts
 constexpr int kKnWaveCols = 128;
 constexpr int kKnBlockCols = 4 * kKnWaveCols;
-constexpr int kKnSets = 3;                         // weight register sets: loads run two steps ahead
+constexpr int kKnSets = 2;                         // weight register sets: loads run a step ahead (two steps: no faster)
 
 // MB: row blocks of 16 (M <= 16 MB).  EPI: kEpiBias (nothing added: the fp16 bias form goes elsewhere) or kEpiSoftcap.
 // KW: the waves of a block share their columns and divide K.

@@ -45,12 +45,14 @@
  *                            the steps holds the last width-1 samples.
  *   oracle_cvt_f16_to_f32    all 65536 bit patterns vs numpy.float16.
  *   oracle_compare_*         hand-computed three-element cases.
+ * On top of those: tests/test_torch_fixtures.py holds tensor_mm, sdp_attention_masked_scaled_fwd, the rule form of the
+ * attention (grouped queries, softcap, window), oracle_attention_softmax_f32 (scale -> softcap -> mask -> softmax),
+ * tensor_causal_conv1d and its decode step, zamba_gated_rmsnorm, gemma_linear_softcap and gemma_mlp_upproj to fixtures
+ * whose expected values PyTorch's library routines computed in float64 (tests/golden/torch_*, written by
+ * tests/golden/make_torch_fixtures.py from the one-line formulas of the reference's generators).
  * The reference repository holds no golden vectors for this path (its .dat fixtures are
  * git-ignored and were drawn from an unseeded generator), so nothing here is pinned against
- * reference-held data.  PARITY UNPINNED: the composition "scale -> softcap -> mask -> softmax"
- * (oracle_attention_softmax_f32 with softcap != 0) has no counterpart call site in the
- * reference; it is the composition of the pinned primitives in the stated order and is
- * pinned only by the checks listed for those primitives plus a float64 brute force.
+ * reference-held data.  No function of this file is left "parity unpinned".
  */
 #include <math.h>
 #include <stdint.h>

@@ -9,6 +9,8 @@ the one-line torch formula the reference's own generator uses for that operator:
                                    scripts/gemma2/slide_mask_test.py:17-22 (tril(diagonal=-W) is masked)
     causal conv1d + SiLU           F.silu(F.conv1d(x, w.unsqueeze(1), b, padding=width-1, groups=dims))[..., :seq_len]
                                    scripts/fused_test_cases.py:41
+    conv1d decode step             the same F.conv1d without padding over [state | new sample]: one output per row; the new
+                                   state is the old one shifted by a sample (the step the Mamba2 mixer takes per token)
     gated RMS norm                 rms_norm(x * silu(z)) * w, srcs/models/zamba2/zamba_gated_rmsnorm.hpp:9-23
     matmul                         torch.matmul, scripts/mm_test_cases.py:18,42
 
@@ -129,6 +131,17 @@ def main() -> None:
         y = F.silu(F.conv1d(t64(x), t64(w).unsqueeze(1), t64(bias), stride=1, padding=width - 1, groups=dims))[:, :, :s]
         save_tensor(x, d / "x.dat"); save_tensor(w, d / "w.dat"); save_tensor(bias, d / "b.dat")
         save_tensor(f32(y), d / "y.dat")
+
+    # 5b. the decode step: a state of width - 1 earlier samples (oldest first), one new sample per row
+    for name, (b, dims, width), seed in (("torch_causal_conv1d_update_f32", (3, 11, 4), 347),
+                                         ("torch_causal_conv1d_update_w2_f32", (2, 6, 2), 348)):
+        d = case_dir(name)
+        state, x = synth.normal(seed, (b, dims, width - 1)), synth.normal(seed + 10, (b, dims))
+        w, bias = synth.normal(seed + 20, (dims, width)), synth.normal(seed + 30, (dims,))
+        seq = torch.cat([t64(state), t64(x).unsqueeze(-1)], dim=-1)                       # [b, dims, width]
+        y = F.silu(F.conv1d(seq, t64(w).unsqueeze(1), t64(bias), stride=1, padding=0, groups=dims))[:, :, 0]
+        save_tensor(state, d / "state.dat"); save_tensor(x, d / "x.dat"); save_tensor(w, d / "w.dat"); save_tensor(bias, d / "b.dat")
+        save_tensor(f32(y), d / "y.dat"); save_tensor(f32(seq[:, :, 1:]), d / "new_state.dat")
 
     # 6. gated RMS norm of the Mamba2 mixer: rms_norm(x * silu(z), eps) * w over the last dimension
     d = case_dir("torch_gated_rmsnorm_f32")

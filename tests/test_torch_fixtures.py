@@ -75,6 +75,14 @@ def test_oracle_conv1d_vs_torch(oracle):
         assert np.max(np.abs(oracle.tensor_causal_conv1d(x, w, b) - y)) <= 2e-6
 
 
+def test_oracle_conv1d_update_vs_torch(oracle):
+    for name in ("torch_causal_conv1d_update_f32", "torch_causal_conv1d_update_w2_f32"):
+        state, x, w, b, y, new_state = case(name, "state", "x", "w", "b", "y", "new_state")
+        got, got_state = oracle.causal_conv1d_update(x, state, w, b)
+        assert np.max(np.abs(got - y)) <= 2e-6
+        assert np.array_equal(got_state, new_state)
+
+
 def test_oracle_gated_rmsnorm_vs_torch(oracle):
     x, z, w, y = case("torch_gated_rmsnorm_f32", "in_0", "in_1", "weight", "out_0")
     assert np.max(np.abs(oracle.zamba_gated_rmsnorm(x, z, w, 1e-5) - y)) <= 1e-5
@@ -167,6 +175,16 @@ def test_hip_conv1d_vs_torch(ops):
     tx, tw, tb = (torch.from_numpy(t).double() for t in (xh, wh, bh))
     yh = F.silu(F.conv1d(tx, tw.unsqueeze(1), tb, padding=w.shape[1] - 1, groups=w.shape[0]))[..., :x.shape[2]].numpy()
     assert scaled_rel_err(up(host(ops.tensor_causal_conv1d(dev(xh), dev(wh), dev(bh)))), yh, 1.0) <= TOL_F16_ROWOPS
+
+
+@pytest.mark.gpu
+def test_hip_conv1d_update_vs_torch(ops):
+    for name in ("torch_causal_conv1d_update_f32", "torch_causal_conv1d_update_w2_f32"):
+        state, x, w, b, y, new_state = case(name, "state", "x", "w", "b", "y", "new_state")
+        dstate = dev(state)
+        got = host(ops.tensor_causal_conv1d_update(dev(x), dstate, dev(w), dev(b)))
+        assert scaled_rel_err(got, y, 1.0) <= TOL_F32
+        assert np.array_equal(host(dstate), new_state)
 
 
 @pytest.mark.gpu
