@@ -5,13 +5,13 @@ Headline (one JSON line on stdout): fp16 GEMM M = N = K = 4096, A row-major, B c
 fp32 accumulate, fp16 output -- TFLOP/s, with the roofline of that kernel and the CPU oracle
 timed next to it.  The other kernels of the path (fp32 GEMM 2048^3, Zamba2-shaped causal conv1d +
 SiLU, causal softmax 32 x 2048 x 2048, Gemma2 softmax 8 x 8192 x 8192 with softcap and sliding
-window, and the callers either side: fused attention, decode attention, gated RMS norm) are
-measured in the same run and reported under "kernels", each with its own roofline object and,
+window, and the callers either side: fused attention, decode attention, gated RMS norm, the Gemma2
+output head at 8 rows) are measured in the same run and reported under "kernels", each with its own roofline object and,
 for the configurations the metric names, the CPU oracle timed on a bounded sample.
 
 A step is one launch of the kernel over one batch of synthetic input that is already resident
 in HBM.  Inputs are drawn on the host by anygpu_amd.synth with the stated seeds (the generator of
-the parity tests).  Timing of every kernel:
+the parity tests; the 2.4 GB of output-head weights by torch's generator on the device).  Timing of every kernel:
   * W untimed warm-up steps, then exactly K steps between two device synchronisations (host
     clock -> `value` of the headline) and between two HIP events recorded on the launch stream
     (-> `us_per_launch`, `roofline.achieved`); for the kernels under "kernels", whose K is a
@@ -61,6 +61,8 @@ MEASURED_TRAFFIC = {
     "attention_gemma2_f32": (1308870403, "profiles/sdp_attention_fwd_f32_gemma2_kernel.md"),
     "gated_rmsnorm": (805405955, "profiles/gated_rmsnorm_f16_row_kernel.md"),
     "attention_decode": (144037358, "profiles/sdp_attention_decode_f16_partial_and_merge_kernels.md"),
+    "lm_head_f32": (2391557676, "profiles/gemma_linear_softcap_head_band_kernels.md"),
+    "lm_head_f16": (1203714309, "profiles/gemma_linear_softcap_head_band_kernels.md"),
 }
 
 
@@ -85,7 +87,7 @@ def parse_args():
     ap.add_argument("--cpu-seconds", type=float, default=12.0,
                     help="target wall time of the CPU-oracle sample of the headline (0 disables every CPU baseline); "
                          "the other configurations get a quarter of it each")
-    ap.add_argument("--only", default="", help="comma list of: gemm,gemm32,conv,softmax,attn,attn32,decode,norm (default: all)")
+    ap.add_argument("--only", default="", help="comma list of: gemm,gemm32,conv,softmax,attn,attn32,decode,norm,head (default: all)")
     ap.add_argument("--gemm-shapes", nargs="?", const="f16", default=None, choices=("f16", "f32"),
                     help="print the table of GEMM layer shapes (fp16, or fp32 with `--gemm-shapes f32`) against torch.matmul and exit")
     ap.add_argument("--gemm-operands", default="uniform", choices=("uniform", "low_toggle"),
@@ -545,6 +547,33 @@ def bench_gated_rmsnorm(torch, ops, synth, steps, warmup):
     }
 
 
+def bench_lm_head(torch, ops, steps, warmup, dtype):
+    # The Gemma2 output head: softcap(x W^T, 30) with W [vocab, hidden] = [256000, 2304] as the reference stores it
+    # (srcs/models/gemma2/gemma_linsoftcap.cu:11-33), 8 rows of x (a decode step of batch 8, or a prompt's last positions).
+    # The weights (2.36 GB in float32, 1.18 GB in half) are streamed once per call: the bound is the memory.
+    rows, vocab, hidden = 8, 256000, 2304
+    tdt = torch.float32 if dtype == "f32" else torch.float16
+    gen = torch.Generator(device="cuda").manual_seed(0)
+    w = ((torch.rand((vocab, hidden), device="cuda", generator=gen) * 2 - 1) * 0.05).to(tdt)
+    x = (torch.rand((1, rows, hidden), device="cuda", generator=gen) * 2 - 1).to(tdt)
+
+    def step():
+        ops.tensor_gemma_linear_softcap(x, w, 30.0)
+
+    t = timed_region(torch, step, steps, warmup)
+    esize = 4 if dtype == "f32" else 2
+    nbytes = (vocab * hidden + rows * hidden + rows * vocab) * esize
+    sec = t["us_per_launch"] * 1e-6
+    return {
+        "name": f"gemma_linear_softcap_{dtype}",
+        "workload": f"Gemma2 output head {dtype}: x [1, 8, 2304] U(-1,1), W [256000, 2304] U(-0.05,0.05) (torch generator on the "
+                    "device, seed 0), softcap 30",
+        **timing_fields(t), "value": nbytes / sec / 1e9, "unit": "GB/s", "dtype": dtype,
+        "roofline": {"bound": "hbm", "achieved": nbytes / sec / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": nbytes / sec / 1e9 / PEAK_HBM_GBS, **traffic_fields(f"lm_head_{dtype}"), "algorithmic_bytes": nbytes},
+    }
+
+
 LAYER_WEIGHTS = [(9216, 2304), (18432, 2304), (2304, 9216), (2048, 2304), (1024, 2304), (4096, 2304), (2304, 2048),
                  (2048, 2048), (8192, 2048), (2048, 8192), (4096, 4096), (14336, 4096), (4096, 14336), (6144, 4096)]
 LAYER_ROWS = (16, 64, 128, 256, 512, 1024, 2048, 4096)
@@ -675,6 +704,9 @@ def main():
         kernels.append(bench_attention_decode(torch, capi, synth, args.steps, args.warmup))
     if want("norm"):
         kernels.append(bench_gated_rmsnorm(torch, ops, synth, args.steps // 4, max(args.warmup // 4, 1)))
+    if want("head"):
+        kernels.append(bench_lm_head(torch, ops, args.steps // 4, max(args.warmup // 4, 1), "f32"))
+        kernels.append(bench_lm_head(torch, ops, args.steps // 4, max(args.warmup // 4, 1), "f16"))
 
     line = {
         "metric": "fp16 GEMM TFLOP/s; conv1d & softmax HBM GB/s (% roofline) on 1 MI355X",
