@@ -20,6 +20,7 @@ ANYGPU_ERR_TOO_LARGE = -5
 ANYGPU_ERR_SCRATCH_TOO_SMALL = -6
 DECODE_STATIC_SCRATCH_BYTES = 8 * 1024 * 1024
 WORKSPACE_BYTES = 64 * 1024 * 1024
+WORKSPACE_MAX_BYTES = 1024 * 1024 * 1024
 MAX_OWN_WORKSPACES = 8
 
 A_ROW_MAJOR = 0

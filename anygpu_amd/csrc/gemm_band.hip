@@ -426,7 +426,9 @@ band::WorkspaceReserve::~WorkspaceReserve()
 	reserved_front = previous_;
 }
 
-size_t band::workspace_capacity(hipStream_t stream)
+namespace {
+// bytes the stream's workspace offers: a caller's buffer as it is; the library's own `own_bytes`, to eager launches only
+size_t capacity_of(hipStream_t stream, size_t own_bytes)
 {
 	int device = 0;
 	if (hipGetDevice(&device) != hipSuccess) return 0;
@@ -441,12 +443,15 @@ size_t band::workspace_capacity(hipStream_t stream)
 			from_caller = true;
 		}
 	}
-	// the library's own buffer: eager launches only
-	if (!from_caller) bytes = stream_is_capturing(stream) ? 0 : kBandPartialBytes;
+	if (!from_caller) bytes = stream_is_capturing(stream) ? 0 : own_bytes;
 	return bytes > reserved_front ? bytes - reserved_front : 0;
 }
+}  // namespace
 
-hipError_t band::workspace_acquire(hipStream_t stream, float** base)
+size_t band::workspace_capacity(hipStream_t stream) { return capacity_of(stream, kBandPartialBytes); }
+size_t band::workspace_copy_capacity(hipStream_t stream) { return capacity_of(stream, kBandCopyBytes); }
+
+hipError_t band::workspace_acquire(hipStream_t stream, float** base, size_t at_least)
 {
 	*base = nullptr;
 	int device = 0;
@@ -454,12 +459,26 @@ hipError_t band::workspace_acquire(hipStream_t stream, float** base)
 	if (err != hipSuccess) return err;
 	std::lock_guard<std::mutex> guard(workspace_lock);
 	const auto key = std::make_pair(device, stream);
+	// what the library's own buffer has to hold: the reserved front and `at_least` behind it, in whole steps
+	size_t want = reserved_front + at_least;
+	want = want <= kBandPartialBytes ? kBandPartialBytes : (want + kBandPartialBytes - 1) / kBandPartialBytes * kBandPartialBytes;
 	const auto found = workspaces.find(key);
 	if (found != workspaces.end())
 	{
-		found->second.last_use = ++use_clock;
-		*base = reinterpret_cast<float*>(reinterpret_cast<char*>(found->second.base) + reserved_front);
-		return hipSuccess;
+		if (found->second.from_caller || found->second.bytes >= want)
+		{
+			found->second.last_use = ++use_clock;
+			*base = reinterpret_cast<float*>(reinterpret_cast<char*>(found->second.base) + reserved_front);
+			return hipSuccess;
+		}
+		// the library's own buffer is too small for this copy: a larger one takes its place
+		const hipError_t freed = hipFree(found->second.base);
+		if (freed != hipSuccess)
+		{
+			(void)hipGetLastError();
+			return freed;
+		}
+		workspaces.erase(found);
 	}
 	// Streams come and go and the library does not see them go: when it already owns its limit of buffers, the one
 	// used longest ago makes way.  hipFree waits for the device, so work that may still use that buffer has finished.
@@ -489,14 +508,14 @@ hipError_t band::workspace_acquire(hipStream_t stream, float** base)
 	hipStreamCaptureMode mode = hipStreamCaptureModeRelaxed;
 	(void)hipThreadExchangeStreamCaptureMode(&mode);
 	void* mem = nullptr;
-	err = hipMalloc(&mem, kBandPartialBytes);
+	err = hipMalloc(&mem, want);
 	(void)hipThreadExchangeStreamCaptureMode(&mode);
 	if (err != hipSuccess)
 	{
 		(void)hipGetLastError();
 		return err;
 	}
-	workspaces.emplace(key, WorkspaceEntry{static_cast<float*>(mem), kBandPartialBytes, false, ++use_clock});
+	workspaces.emplace(key, WorkspaceEntry{static_cast<float*>(mem), want, false, ++use_clock});
 	*base = reinterpret_cast<float*>(static_cast<char*>(mem) + reserved_front);
 	return hipSuccess;
 }

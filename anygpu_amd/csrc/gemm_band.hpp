@@ -18,6 +18,9 @@ constexpr int64_t kBandWantedBlocks = 512;
 // partial sums within the first kBandPlanBytes: their plan does not price that traffic, and more splits than fit
 // there lost (64 x 4096 . 4096 x 14336 fp32: 83 us with 2 splits, 95 us with 5).
 constexpr size_t kBandPartialBytes = (size_t)64 << 20;
+// Aligned copies of GEMM operands that the tile kernels cannot fetch as they lie may need more (4095^3 fp32: two copies
+// of 64 MiB): for those the library's own buffer of a stream grows on demand, in steps of kBandPartialBytes, up to this.
+constexpr size_t kBandCopyBytes = (size_t)1 << 30;
 constexpr size_t kBandPlanBytes = (size_t)16 << 20;
 
 typedef float4_t Vec;      // 16 raw bytes of either element type
@@ -75,8 +78,12 @@ template <> struct BandMma<half_t, 32>
 // workspace_capacity: bytes a launch on `stream` may plan partial sums for right now (0: run uncut), without allocating.
 // workspace_acquire: the buffer of at least that size; allocates the library's own on first use and returns the error if
 // that fails.
+// workspace_copy_capacity: the same for operand copies, which may make the library's own buffer grow (up to
+// kBandCopyBytes); workspace_acquire with `at_least` > 0 returns a buffer of at least that many bytes, reallocating the
+// library's own if it is smaller (hipFree waits for the device, so nothing still uses the old one).
 size_t workspace_capacity(hipStream_t stream);
-hipError_t workspace_acquire(hipStream_t stream, float** base);
+size_t workspace_copy_capacity(hipStream_t stream);
+hipError_t workspace_acquire(hipStream_t stream, float** base, size_t at_least = 0);
 // While one of these lives, the calling thread's view of every workspace starts `bytes` (rounded up to 256) further on:
 // a launcher that has parked operand copies at the front of the stream's workspace calls the ordinary launchers
 // underneath it, whose partial sums then go behind the copies.

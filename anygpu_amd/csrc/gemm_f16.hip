@@ -362,7 +362,7 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
 		const bool copy_b = k_odd || reinterpret_cast<uintptr_t>(B) % 16 != 0 || ldb % 8 != 0 || (b_layout == ANYGPU_B_ROW_MAJOR && N % 8 != 0);
 		const int64_t k_pad = (K + 63) / 64 * 64;
 		const size_t bytes_b = copy_b ? ((size_t)N * k_pad * 2 + 255) / 256 * 256 : 0;
-		const size_t room = band::workspace_capacity(stream);
+		const size_t room = band::workspace_copy_capacity(stream);
 		// (a copy of A that does not fit beside the one of B is made and used in bands of rows, one after the other)
 		int64_t band_rows = M;
 		if (copy_a && bytes_b < room && (size_t)M * k_pad * 2 > room - bytes_b)
@@ -371,7 +371,7 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
 		if ((copy_a || copy_b) && (band_rows == M || band_rows >= 256) && bytes_a + bytes_b <= room)
 		{
 			float* front = nullptr;
-			hipError_t err = band::workspace_acquire(stream, &front);
+			hipError_t err = band::workspace_acquire(stream, &front, bytes_a + bytes_b);
 			if (err != hipSuccess) return err;
 			half_t* b_copy = reinterpret_cast<half_t*>(front);
 			half_t* a_copy = reinterpret_cast<half_t*>(reinterpret_cast<char*>(front) + bytes_b);

@@ -587,10 +587,10 @@ hipError_t launch_gemm_f32(const float* A, const float* B, const float* bias, fl
 		const bool a_rows_m = a_layout == ANYGPU_A_ROW_MAJOR, b_rows_n = b_layout == ANYGPU_B_COL_MAJOR;
 		const size_t bytes_a = copy_a ? (size_t)m_pad * k_pad * 4 : 0;
 		const size_t bytes_b = copy_b ? (size_t)n_pad * k_pad * 4 : 0;
-		if (bytes_a + bytes_b <= band::workspace_capacity(stream))
+		if (bytes_a + bytes_b <= band::workspace_copy_capacity(stream))
 		{
 			float* front = nullptr;
-			hipError_t err = band::workspace_acquire(stream, &front);
+			hipError_t err = band::workspace_acquire(stream, &front, bytes_a + bytes_b);
 			if (err != hipSuccess) return err;
 			float* a_copy = front;
 			float* b_copy = reinterpret_cast<float*>(reinterpret_cast<char*>(front) + bytes_a);

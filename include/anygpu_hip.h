@@ -12,7 +12,9 @@
  *     of 8) and the partial results of the key-split blocks of the fused attention.  Who owns
  *     it is the caller's choice, see anygpu_set_workspace: by default the library
  *     allocates ANYGPU_WORKSPACE_BYTES (64 MiB) the first time an eager launch on a stream cuts a
- *     product and keeps them until anygpu_release_workspaces or the end of the process; a caller
+ *     product and keeps them until anygpu_release_workspaces or the end of the process (operand
+ *     copies that need more make that buffer grow, in steps of the same size, up to
+ *     ANYGPU_WORKSPACE_MAX_BYTES: the old buffer is freed, which waits for the device); a caller
  *     that hands in its own workspace for a stream makes the library allocate nothing there.
  *     While a stream is being captured into a graph only a caller's workspace is used, never the
  *     library's: without one every captured product runs uncut and uncopied (a valid result,
@@ -86,6 +88,7 @@ const char* anygpu_hip_error_string(int code);  /* text for ANYGPU_ERR_* and for
  * gives the same handle would write into that memory.
  */
 #define ANYGPU_WORKSPACE_BYTES (64 * 1024 * 1024)
+#define ANYGPU_WORKSPACE_MAX_BYTES (1024 * 1024 * 1024)
 #define ANYGPU_MAX_OWN_WORKSPACES 8
 
 int anygpu_set_workspace(void* stream, void* workspace, int64_t bytes);

@@ -2086,6 +2086,38 @@ def test_library_owned_workspaces_are_bounded(ops):
     ops.release_workspaces()
 
 
+def test_mm_f32_operand_copies_larger_than_the_first_workspace(ops, oracle):
+    # odd row pitches and a K that is no multiple of 32: both operands are copied, aligned and padded, into the stream's
+    # workspace; the two copies (52 + 69 MB) exceed the 64 MiB the library allocates first, so its buffer grows.
+    # Small integers: every sum is exact, whatever the order; torch.matmul on the same operands must agree bit for bit,
+    # and a few rows are held against the oracle.
+    import torch
+    from anygpu_amd import capi
+    ops.release_workspaces()
+    m, k, n = 3000, 4099, 4095
+    a = synth.integers(71, (m, k), -2, 2)
+    w = synth.integers(72, (n, k), -2, 2)
+    da, dw = dev(a), dev(w)
+    torch.cuda.synchronize()
+    free0 = torch.cuda.mem_get_info()[0]
+    got = ops.tensor_mm(da, dw, b_layout=capi.B_COL_MAJOR)
+    torch.cuda.synchronize()
+    held = free0 - torch.cuda.mem_get_info()[0] - got.numel() * 4
+    assert capi.WORKSPACE_BYTES < held <= 3 * capi.WORKSPACE_BYTES, held       # 121 MB of copies in steps of 64 MiB
+    assert torch.equal(got, torch.matmul(da, dw.t()))
+    rows = [0, 1, 1499, 2999]
+    want = oracle.tensor_mm(a[rows], np.ascontiguousarray(w.T), threads=8)
+    assert np.array_equal(host(got)[rows], want)
+    # the grown buffer serves later calls, large and small
+    free1 = torch.cuda.mem_get_info()[0]
+    again = ops.tensor_mm(da, dw, b_layout=capi.B_COL_MAJOR)
+    small = ops.tensor_mm(da[:24], dw[:260], b_layout=capi.B_COL_MAJOR)
+    torch.cuda.synchronize()
+    assert free1 - torch.cuda.mem_get_info()[0] <= again.numel() * 4 + (8 << 20)
+    assert torch.equal(again, got) and torch.equal(small, got[:24, :260])
+    ops.release_workspaces()
+
+
 def test_k_split_products_on_concurrent_streams(ops, oracle):
     # every stream owns its partial-sum workspace: products that are cut along K may overlap on different streams
     import torch
