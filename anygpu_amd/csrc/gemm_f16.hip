@@ -603,6 +603,11 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
 		{
 			// whole 256 x 256 tiles of k-contiguous operands: the four-wave kernel with 128 x 128 patches (4096^3: 93 us
 			// against 99 us for the eight-wave tile on the same box, vendor library 93 us)
+			// (up to 128 rows half of a 256 x 256 tile is empty and the product waits for its weights: the 128 x 128
+			// four-wave tiles, of which a CU holds more loads in flight, stream them faster once they fill the chip,
+			// 128 x 8192 -> 131072: 449 -> 383 us, 65 x 2304 -> 256000: 308 -> 253, vendor 391 / 236)
+			if (tile == 256 && whole_tiles && M <= 128 && batch == 1 && blocks(128) >= cus)
+				return launch_gemm_f16_ring3<4, 4>(a, b, c, M, N, K, lda, ldb, ldc, stride_a, stride_b, stride_c, batch, stream, nullptr, 0, nullptr, 0.0f, b_layout);
 			if (tile == 256 && whole_tiles)
 				return launch_gemm_f16_ring(a, b, c, M, N, K, lda, ldb, ldc, stride_a, stride_b, stride_c, batch, stream);
 			if (tile == 256) ANYGPU_F16_TILE(256, 2, 4, false, 2, 1);
@@ -612,6 +617,8 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
 		}
 		if (fits && b_layout == ANYGPU_B_ROW_MAJOR)
 		{
+			if (tile == 256 && whole_tiles && M <= 128 && batch == 1 && blocks(128) >= cus)        // (as above; [K, N]: 451 -> 395 us)
+				return launch_gemm_f16_ring3<4, 4>(a, b, c, M, N, K, lda, ldb, ldc, stride_a, stride_b, stride_c, batch, stream, nullptr, 0, nullptr, 0.0f, b_layout);
 			if (tile == 256 && whole_tiles)
 				return launch_gemm_f16_ring(a, b, c, M, N, K, lda, ldb, ldc, stride_a, stride_b, stride_c, batch, stream, nullptr, b_layout);
 			if (tile == 256) ANYGPU_F16_TILE(256, 2, 4, true, 2, 1);

@@ -1095,6 +1095,25 @@ def test_mm_row_bands_k_contiguous_weights_many_columns(ops, oracle, dtype, m, s
         assert scaled_rel_err(host(out), ref + bias[None, :], math.sqrt(k) / 3.0 + 1.0) <= tol
 
 
+@pytest.mark.parametrize("layout", ["nk", "kn"])
+@pytest.mark.parametrize("m,k,n", [(65, 128, 40000), (96, 192, 32768), (128, 64, 65536), (100, 256, 33000)])
+def test_mm_f16_up_to_128_rows_against_many_columns(ops, oracle, layout, m, k, n):
+    # 65 to 128 rows against weights with enough columns for 128 x 128 tiles to fill the chip: the four-wave kernel with
+    # those tiles instead of half-empty 256 x 256 ones, both weight layouts; small integers, every sum exact
+    import torch
+    from anygpu_amd import capi
+    a = synth.integers(m + 31, (m, k), -2, 2)
+    b = synth.integers(n + 32, (k, n), -2, 2)
+    want = oracle.tensor_mm(a, b, threads=8)
+    assert np.abs(want).max() <= 2048
+    da = dev(a.astype(np.float16))
+    if layout == "kn":
+        got = ops.tensor_mm(da, dev(b.astype(np.float16)))
+    else:
+        got = ops.tensor_mm(da, dev(np.ascontiguousarray(b.T).astype(np.float16)), b_layout=capi.B_COL_MAJOR)
+    assert np.array_equal(host(got).astype(np.float32), want)
+
+
 @pytest.mark.parametrize("m,k,n", [(512, 256, 1003), (300, 512, 259), (128, 64, 65), (1000, 128, 4097), (65, 192, 7), (257, 320, 511)])
 def test_mm_f16_k_contiguous_weights_result_rows_of_any_length(ops, oracle, m, k, n):
     # the tile kernels with [N, K] weights: N, the row length of C and its first element are free; integers, exact
