@@ -622,9 +622,11 @@ hipError_t launch_gemm_f32(const float* A, const float* B, const float* bias, fl
 #undef ANYGPU_F32_PADDED
 		}
 	}
-	// From 48 rows on, k-contiguous weights in whole slabs go to the four-wave 64 x 64 tiles cut along K rather than to
-	// the band kernels (64 x 4096 -> 6144: 45 us as a band, 37 us in tiles; 16 rows of the same: 24 us against 32 us).
-	const bool tiles_first = a_layout == ANYGPU_A_ROW_MAJOR && b_layout == ANYGPU_B_COL_MAJOR && M >= 48 &&
+	// From 33 rows on (where the band kernels go from two row blocks of 16 to two of 32), k-contiguous weights in whole
+	// slabs go to the four-wave 64 x 64 tiles cut along K rather than to the band kernels (64 x 4096 -> 6144: 45 us as a
+	// band, 37 us in tiles; 40 x 9216 -> 2304: 44 against 28.5, 40 x 4096 -> 14336: 80 against 65; 17 - 32 rows of the
+	// same: 48 us as a band, 64 in tiles).
+	const bool tiles_first = a_layout == ANYGPU_A_ROW_MAJOR && b_layout == ANYGPU_B_COL_MAJOR && M >= 33 &&
 	                         gemm_f32_ring_applies(A, B, M, N, K, lda, ldb, stride_a, stride_b, batch, 0, 64);
 	// few rows against k-contiguous weights with the columns of an output head: whole lines per row and load instruction
 	if (batch == 1 && a_layout == ANYGPU_A_ROW_MAJOR && b_layout == ANYGPU_B_COL_MAJOR && M >= kWideMinRowsF32 &&
