@@ -262,6 +262,22 @@ static FourWavePlan plan_four_wave(int64_t M, int64_t N, int64_t K, int64_t batc
 	return best;
 }
 
+// What the launcher expects one uncut product to take with the best of its tile kernels, from the prices above (for
+// comparing a product with the same product divided by rows; microseconds).
+static double estimate_tiles_us(int64_t M, int64_t N, int64_t K, int64_t cus, bool whole_tiles)
+{
+	const double slabs = (double)((K + 63) / 64);
+	const auto blocks = [&](int64_t t) { return ((M + t - 1) / t) * ((N + t - 1) / t); };
+	double per_slab = std::min({slab_us(256, blocks(256), cus, whole_tiles), slab_us(128, blocks(128), cus), slab_us(64, blocks(64), cus)});
+	const int64_t blocks_rect = ((M + 255) / 256) * ((N + 127) / 128);
+	per_slab = std::min(per_slab, TilePrices::kRect * (double)((blocks_rect + cus - 1) / cus));
+	double us = per_slab * slabs + 6.0;
+	if (whole_tiles) us = std::min(us, plan_four_wave(M, N, K, 1, cus, 0).us);
+	// no launch ends before its operands have come in once (few rows: at what the bandwidth-shaped kernels reach)
+	const double stream_us = 2.0 * ((double)M + (double)N) * (double)K / 6.2e6 + 3.0;
+	return std::max(us, stream_us);
+}
+
 // C[m, n] = half(sum over splits of planes[split][m][n]), one thread per eight columns (N a multiple of 8), the
 // planes added in order
 __global__ __launch_bounds__(256) void gemm_f16_split_merge_kernel(
@@ -429,6 +445,23 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
 		// 256 x 256 tiles of whole 64-deep slabs take the four-wave kernel, which is cheaper per slab
 		const bool whole_tiles = gemm_f16_ring_applies(a, b, M, N, K, lda, ldb, stride_a, stride_b, batch, b_layout);
 		const auto slab_us = [cus, whole_tiles](int64_t t, int64_t nblocks) { return anygpu::slab_us(t, nblocks, cus, whole_tiles); };
+		// Rows that end a little past a multiple of 256 make a whole further row of tiles (520 rows: three of 256, the
+		// last one with 8 rows) and often a worse choice of tile for all of them: where the prices say so, the product
+		// is divided into the whole multiples and the rest, which is launched as a product of its own with its own
+		// kernel (520 x 4096 -> 14336: 84 us whole, 50 + 19 divided; vendor 66).
+		// (a rest of more than 128 rows fills half of its tiles and more: 900 x 3584 -> 18944 got slower divided)
+		if (batch == 1 && M > 256 && M % 256 != 0 && M % 256 <= 128)
+		{
+			const int64_t m_body = M / 256 * 256, m_tail = M - m_body;
+			const double whole_us = estimate_tiles_us(M, N, K, cus, whole_tiles);
+			const double divided_us = estimate_tiles_us(m_body, N, K, cus, whole_tiles) + estimate_tiles_us(m_tail, N, K, cus, whole_tiles);
+			if (divided_us < 0.97 * whole_us)
+			{
+				const hipError_t err = launch_gemm_f16(A, B, C, m_body, N, K, lda, ldb, ldc, 0, 0, 0, 1, b_layout, stream);
+				if (err != hipSuccess) return err;
+				return launch_gemm_f16(a + m_body * lda, B, c + m_body * ldc, m_tail, N, K, lda, ldb, ldc, 0, 0, 0, 1, b_layout, stream);
+			}
+		}
 		const double cost256 = slab_us(256, blocks(256)), cost128 = slab_us(128, blocks(128)), cost64 = slab_us(64, blocks(64));
 		int64_t tile = (cost256 <= cost128 && cost256 <= cost64) ? 256 : cost128 <= cost64 ? 128 : 64;
 

@@ -1096,6 +1096,24 @@ def test_mm_row_bands_k_contiguous_weights_many_columns(ops, oracle, dtype, m, s
 
 
 @pytest.mark.parametrize("layout", ["nk", "kn"])
+@pytest.mark.parametrize("m,k,n", [(520, 4096, 14336), (264, 1024, 8192), (1100, 512, 9216), (640, 2048, 14336)])
+def test_mm_f16_rows_just_past_a_multiple_of_256(ops, oracle, layout, m, k, n):
+    # products the launcher may divide by rows into the whole multiples of 256 and the rest; small integers, every sum
+    # exact, so the result does not depend on whether or where it was divided
+    from anygpu_amd import capi
+    a = synth.integers(m + 41, (m, k), -1, 1)
+    b = synth.integers(n + 42, (k, n), -1, 1)
+    want = oracle.tensor_mm(a, b, threads=8)
+    assert np.abs(want).max() <= 2048
+    da = dev(a.astype(np.float16))
+    if layout == "kn":
+        got = ops.tensor_mm(da, dev(b.astype(np.float16)))
+    else:
+        got = ops.tensor_mm(da, dev(np.ascontiguousarray(b.T).astype(np.float16)), b_layout=capi.B_COL_MAJOR)
+    assert np.array_equal(host(got).astype(np.float32), want)
+
+
+@pytest.mark.parametrize("layout", ["nk", "kn"])
 @pytest.mark.parametrize("m,k,n", [(65, 128, 40000), (96, 192, 32768), (128, 64, 65536), (100, 256, 33000)])
 def test_mm_f16_up_to_128_rows_against_many_columns(ops, oracle, layout, m, k, n):
     # 65 to 128 rows against weights with enough columns for 128 x 128 tiles to fill the chip: the four-wave kernel with
