@@ -1095,6 +1095,40 @@ def test_mm_row_bands_k_contiguous_weights_many_columns(ops, oracle, dtype, m, s
         assert scaled_rel_err(host(out), ref + bias[None, :], math.sqrt(k) / 3.0 + 1.0) <= tol
 
 
+ROUTING_EDGES = [
+    # (rows, K in 128-byte steps of the dtype, columns): either side of what the launchers decide by
+    (2, 2, 131072), (3, 2, 131072),                 # skinny kernels / band kernels
+    (16, 3, 124672), (16, 3, 124416),               # 487 / 486 blocks of 256 columns: the wide band kernel or not
+    (17, 2, 131072), (32, 1, 131072), (33, 2, 131072), (48, 2, 131072), (49, 2, 131072), (64, 3, 131072), (65, 2, 131072),
+    (8, 2, 131328),                                 # 513 blocks: a third round with one block
+    (8, 2, 131074), (8, 2, 131076),                 # columns no multiple of four / of eight
+    (12, 5, 98304), (12, 4, 196608),                # 1.5 and 3 blocks per CU
+    (128, 2, 32768), (129, 2, 32768), (128, 2, 32640),   # 128 x 128 tiles that fill the chip, or not quite
+    (33, 4, 4096), (47, 4, 9216), (48, 4, 9216),    # fp32: band kernel / tiles first
+    (257, 2, 14336), (384, 2, 14336), (385, 2, 14336), (300, 8, 8192),   # rows past a multiple of 256
+]
+
+
+@pytest.mark.parametrize("dtype", ["f16", "f32"])
+@pytest.mark.parametrize("m,steps,n", ROUTING_EDGES)
+def test_mm_k_contiguous_weights_either_side_of_the_routing_rules(ops, oracle, dtype, m, steps, n):
+    # small integers: every sum is exact, so whichever kernel a shape is routed to must return the oracle's result bit
+    # for bit; the result sits inside a wider buffer whose other columns must stay untouched
+    import torch
+    from anygpu_amd import capi
+    half = dtype == "f16"
+    tdt, ndt = (torch.float16, np.float16) if half else (torch.float32, np.float32)
+    k = steps * (64 if half else 32)
+    a = synth.integers(m + 51, (m, k), -2, 2)
+    w = synth.integers(n + 52, (n, k), -2, 2)
+    want = oracle.tensor_mm(a, np.ascontiguousarray(w.T), threads=8)
+    assert np.abs(want).max() <= 2048
+    cbuf = torch.full((m, n + 8), -3.0, device="cuda", dtype=tdt)
+    ops.tensor_mm(dev(a.astype(ndt)), dev(w.astype(ndt)), out=cbuf[:, :n], b_layout=capi.B_COL_MAJOR)
+    assert np.array_equal(host(cbuf[:, :n]).astype(np.float32), want)
+    assert bool((cbuf[:, n:] == -3.0).all())
+
+
 @pytest.mark.parametrize("layout", ["nk", "kn"])
 @pytest.mark.parametrize("m,k,n", [(520, 4096, 14336), (264, 1024, 8192), (1100, 512, 9216), (640, 2048, 14336)])
 def test_mm_f16_rows_just_past_a_multiple_of_256(ops, oracle, layout, m, k, n):
