@@ -622,6 +622,29 @@ hipError_t launch_gemm_f32(const float* A, const float* B, const float* bias, fl
 #undef ANYGPU_F32_PADDED
 		}
 	}
+	// Rows that end a little past a multiple of 64 make a whole further row of tiles, which in fp32 costs matrix-core
+	// time, where the few rows past the multiple would only cost another pass over the weights through the few-row
+	// kernels: where the plans' prices say so, the product is divided into the multiples of 64 and the rest
+	// (65 x 4096 -> 14336: 123 us whole, 67 + 37 divided; 80 x 2304 -> 9216: 57 -> 47; vendor 95 / 39).
+	// (a rest of 17 - 32 rows only behind the first 64: 160 x 4096 -> 14336 as 128 + 32 got 3 % slower)
+	if (batch == 1 && a_layout == ANYGPU_A_ROW_MAJOR && M > 64 && M % 64 != 0 && M % 64 <= (M < 128 ? 32 : 16))
+	{
+		const int64_t m_body = M / 64 * 64, m_tail = M - m_body;
+		const bool ring = gemm_f32_ring_applies(A, B, M, N, K, lda, ldb, stride_a, stride_b, batch, 0, 64, b_layout, false);
+		const size_t ws_bytes = band::workspace_capacity(stream);
+		const auto tiles_us = [&](int64_t rows) {
+			return std::min(plan_tiles(128, rows, N, K, 1, true, ws_bytes, ring).cost, plan_tiles(64, rows, N, K, 1, true, ws_bytes, ring).cost) + 6.0;
+		};
+		// the rest: one pass over the weights at what the few-row kernels reach, or its products where those take longer
+		const double rest_us = std::max(4.0 * ((double)N + (double)m_tail) * (double)K / 6.0e6,
+		                                2.0 * (double)((m_tail + 15) / 16 * 16) * (double)N * (double)K / 1.0e8) + 4.0;
+		if (tiles_us(m_body) + rest_us < 0.95 * tiles_us(M))
+		{
+			const hipError_t err = launch_gemm_f32(A, B, bias, C, m_body, N, K, lda, ldb, ldc, 0, 0, 0, 1, a_layout, b_layout, stream);
+			if (err != hipSuccess) return err;
+			return launch_gemm_f32(A + m_body * lda, B, bias, C + m_body * ldc, m_tail, N, K, lda, ldb, ldc, 0, 0, 0, 1, a_layout, b_layout, stream);
+		}
+	}
 	// From 33 rows on (where the band kernels go from two row blocks of 16 to two of 32), k-contiguous weights in whole
 	// slabs go to the four-wave 64 x 64 tiles cut along K rather than to the band kernels (64 x 4096 -> 6144: 45 us as a
 	// band, 37 us in tiles; 40 x 9216 -> 2304: 44 against 28.5, 40 x 4096 -> 14336: 80 against 65; 17 - 32 rows of the

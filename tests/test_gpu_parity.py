@@ -1095,6 +1095,27 @@ def test_mm_row_bands_k_contiguous_weights_many_columns(ops, oracle, dtype, m, s
         assert scaled_rel_err(host(out), ref + bias[None, :], math.sqrt(k) / 3.0 + 1.0) <= tol
 
 
+@pytest.mark.parametrize("layout", ["nk", "kn"])
+@pytest.mark.parametrize("m,k,n", [(65, 2048, 14336), (80, 4096, 14336), (96, 2304, 9216), (130, 4096, 14336), (200, 2048, 8192)])
+def test_mm_f32_rows_just_past_a_multiple_of_64(ops, oracle, layout, m, k, n):
+    # products the launcher may divide by rows into the multiples of 64 and the rest (few-row kernels); entries -1 .. 1,
+    # every sum exact in float32, so the result does not depend on whether it was divided; with a bias
+    import torch
+    from anygpu_amd import capi
+    a = synth.integers(m + 61, (m, k), -1, 1)
+    b = synth.integers(n + 62, (k, n), -1, 1)
+    bias = synth.integers(n + 63, (n,), -3, 3)
+    want = oracle.tensor_mm(a, b, threads=8) + bias[None, :].astype(np.float32)
+    da, dbias = dev(a.astype(np.float32)), dev(bias.astype(np.float32))
+    dw = dev(b.astype(np.float32)) if layout == "kn" else dev(np.ascontiguousarray(b.T).astype(np.float32))
+    out = torch.empty((m, n), device="cuda")
+    ldb = n if layout == "kn" else k
+    capi.check("anygpu_gemm_f32", capi.load().anygpu_gemm_f32(
+        da.data_ptr(), dw.data_ptr(), dbias.data_ptr(), out.data_ptr(), m, n, k, k, ldb, n, capi.A_ROW_MAJOR,
+        capi.B_ROW_MAJOR if layout == "kn" else capi.B_COL_MAJOR, torch.cuda.current_stream().cuda_stream))
+    assert np.array_equal(host(out), want)
+
+
 ROUTING_EDGES = [
     # (rows, K in 128-byte steps of the dtype, columns): either side of what the launchers decide by
     (2, 2, 131072), (3, 2, 131072),                 # skinny kernels / band kernels
