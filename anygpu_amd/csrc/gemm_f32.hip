@@ -638,7 +638,8 @@ hipError_t launch_gemm_f32(const float* A, const float* B, const float* bias, fl
 		// the rest: one pass over the weights at what the few-row kernels reach, or its products where those take longer
 		const double rest_us = std::max(4.0 * ((double)N + (double)m_tail) * (double)K / 6.0e6,
 		                                2.0 * (double)((m_tail + 15) / 16 * 16) * (double)N * (double)K / 1.0e8) + 4.0;
-		if (tiles_us(m_body) + rest_us < 0.95 * tiles_us(M))
+		// (up to 16 rows the few-row kernels reliably run at the pace of the weights: taken at par; beyond, a margin)
+		if (tiles_us(m_body) + rest_us < (m_tail <= 16 ? 1.0 : 0.95) * tiles_us(M))
 		{
 			const hipError_t err = launch_gemm_f32(A, B, bias, C, m_body, N, K, lda, ldb, ldc, 0, 0, 0, 1, a_layout, b_layout, stream);
 			if (err != hipSuccess) return err;
