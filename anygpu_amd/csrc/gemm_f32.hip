@@ -572,6 +572,30 @@ hipError_t launch_gemm_f32(const float* A, const float* B, const float* bias, fl
                            int a_layout, int b_layout, hipStream_t stream)
 {
 	if (M == 0 || N == 0 || batch == 0) return hipSuccess;
+	// Rows that end a little past a multiple of 64 make a whole further row of tiles, which in fp32 costs matrix-core
+	// time, where the few rows past the multiple would only cost another pass over the weights through the few-row
+	// kernels: where the plans' prices say so, the product is divided into the multiples of 64 and the rest
+	// (65 x 4096 -> 14336: 123 us whole, 67 + 37 divided; 80 x 2304 -> 9216: 57 -> 47; vendor 95 / 39).
+	// (a rest of 17 - 32 rows only behind the first 64: 160 x 4096 -> 14336 as 128 + 32 got 3 % slower)
+	if (batch == 1 && a_layout == ANYGPU_A_ROW_MAJOR && M > 64 && M % 64 != 0 && M % 64 <= (M < 128 ? 32 : 16))
+	{
+		const int64_t m_body = M / 64 * 64, m_tail = M - m_body;
+		const bool ring = gemm_f32_ring_applies(A, B, M, N, K, lda, ldb, stride_a, stride_b, batch, 0, 64, b_layout, false);
+		const size_t ws_bytes = band::workspace_capacity(stream);
+		const auto tiles_us = [&](int64_t rows) {
+			return std::min(plan_tiles(128, rows, N, K, 1, true, ws_bytes, ring).cost, plan_tiles(64, rows, N, K, 1, true, ws_bytes, ring).cost) + 6.0;
+		};
+		// the rest: one pass over the weights at what the few-row kernels reach, or its products where those take longer
+		const double rest_us = std::max(4.0 * ((double)N + (double)m_tail) * (double)K / 6.0e6,
+		                                2.0 * (double)((m_tail + 15) / 16 * 16) * (double)N * (double)K / 1.0e8) + 4.0;
+		// (up to 16 rows the few-row kernels reliably run at the pace of the weights: taken at par; beyond, a margin)
+		if (tiles_us(m_body) + rest_us < (m_tail <= 16 ? 1.0 : 0.95) * tiles_us(M))
+		{
+			const hipError_t err = launch_gemm_f32(A, B, bias, C, m_body, N, K, lda, ldb, ldc, 0, 0, 0, 1, a_layout, b_layout, stream);
+			if (err != hipSuccess) return err;
+			return launch_gemm_f32(A + m_body * lda, B, bias, C + m_body * ldc, m_tail, N, K, lda, ldb, ldc, 0, 0, 0, 1, a_layout, b_layout, stream);
+		}
+	}
 	// Operands that start at an odd address or have an odd row pitch would be fetched element by element, and operands
 	// that end inside a tile make the kernel test every vector it fetches (2047^3: 69 TFLOP/s, 2044^3: 70, against 119
 	// for 2048^3).  From 128 rows on (fewer rows stream the weights once, which a copy would triple), for products worth two more launches, such operands are copied into the stream's
@@ -579,7 +603,10 @@ hipError_t launch_gemm_f32(const float* A, const float* B, const float* bias, fl
 	// tile kernels fetch the copies without tests; only the stores into C are guarded.
 	const bool a_odd = reinterpret_cast<uintptr_t>(A) % 16 != 0 || lda % 4 != 0;
 	const bool b_odd = reinterpret_cast<uintptr_t>(B) % 16 != 0 || ldb % 4 != 0;
-	const bool ragged = M % 128 != 0 || N % 128 != 0 || K % kBK != 0;
+	// (the four-wave kernels fetch ragged M and N through their offset tables: no copies where they take the operands as
+	// they lie; 270 x 4096 -> 4100: 149 us with copies, 93 without)
+	const bool ring_takes = a_layout == ANYGPU_A_ROW_MAJOR && gemm_f32_ring_applies(A, B, M, N, K, lda, ldb, stride_a, stride_b, batch, 0, 64, b_layout, false);
+	const bool ragged = !ring_takes && (M % 128 != 0 || N % 128 != 0 || K % kBK != 0);
 	if ((a_odd || b_odd || ragged) && batch == 1 && M >= 128 && (double)M * (double)N * (double)K >= (double)(1 << 29))
 	{
 		const int64_t m_pad = (M + 127) / 128 * 128, n_pad = (N + 127) / 128 * 128, k_pad = (K + 127) / 128 * 128;
@@ -620,30 +647,6 @@ hipError_t launch_gemm_f32(const float* A, const float* B, const float* bias, fl
 			if (b_rows_n) ANYGPU_F32_PADDED(ANYGPU_A_COL_MAJOR, ANYGPU_B_COL_MAJOR);
 			ANYGPU_F32_PADDED(ANYGPU_A_COL_MAJOR, ANYGPU_B_ROW_MAJOR);
 #undef ANYGPU_F32_PADDED
-		}
-	}
-	// Rows that end a little past a multiple of 64 make a whole further row of tiles, which in fp32 costs matrix-core
-	// time, where the few rows past the multiple would only cost another pass over the weights through the few-row
-	// kernels: where the plans' prices say so, the product is divided into the multiples of 64 and the rest
-	// (65 x 4096 -> 14336: 123 us whole, 67 + 37 divided; 80 x 2304 -> 9216: 57 -> 47; vendor 95 / 39).
-	// (a rest of 17 - 32 rows only behind the first 64: 160 x 4096 -> 14336 as 128 + 32 got 3 % slower)
-	if (batch == 1 && a_layout == ANYGPU_A_ROW_MAJOR && M > 64 && M % 64 != 0 && M % 64 <= (M < 128 ? 32 : 16))
-	{
-		const int64_t m_body = M / 64 * 64, m_tail = M - m_body;
-		const bool ring = gemm_f32_ring_applies(A, B, M, N, K, lda, ldb, stride_a, stride_b, batch, 0, 64, b_layout, false);
-		const size_t ws_bytes = band::workspace_capacity(stream);
-		const auto tiles_us = [&](int64_t rows) {
-			return std::min(plan_tiles(128, rows, N, K, 1, true, ws_bytes, ring).cost, plan_tiles(64, rows, N, K, 1, true, ws_bytes, ring).cost) + 6.0;
-		};
-		// the rest: one pass over the weights at what the few-row kernels reach, or its products where those take longer
-		const double rest_us = std::max(4.0 * ((double)N + (double)m_tail) * (double)K / 6.0e6,
-		                                2.0 * (double)((m_tail + 15) / 16 * 16) * (double)N * (double)K / 1.0e8) + 4.0;
-		// (up to 16 rows the few-row kernels reliably run at the pace of the weights: taken at par; beyond, a margin)
-		if (tiles_us(m_body) + rest_us < (m_tail <= 16 ? 1.0 : 0.95) * tiles_us(M))
-		{
-			const hipError_t err = launch_gemm_f32(A, B, bias, C, m_body, N, K, lda, ldb, ldc, 0, 0, 0, 1, a_layout, b_layout, stream);
-			if (err != hipSuccess) return err;
-			return launch_gemm_f32(A + m_body * lda, B, bias, C + m_body * ldc, m_tail, N, K, lda, ldb, ldc, 0, 0, 0, 1, a_layout, b_layout, stream);
 		}
 	}
 	// From 33 rows on (where the band kernels go from two row blocks of 16 to two of 32), k-contiguous weights in whole
