@@ -653,15 +653,17 @@ hipError_t launch_gemm_f32(const float* A, const float* B, const float* bias, fl
 	// slabs go to the four-wave 64 x 64 tiles cut along K rather than to the band kernels (64 x 4096 -> 6144: 45 us as a
 	// band, 37 us in tiles; 40 x 9216 -> 2304: 44 against 28.5, 40 x 4096 -> 14336: 80 against 65; 17 - 32 rows of the
 	// same: 48 us as a band, 64 in tiles).
-	const bool tiles_first = a_layout == ANYGPU_A_ROW_MAJOR && b_layout == ANYGPU_B_COL_MAJOR && M >= 33 &&
-	                         gemm_f32_ring_applies(A, B, M, N, K, lda, ldb, stride_a, stride_b, batch, 0, 64);
+	// ([K, N] weights alike, up to 65536 columns: 48 x 4096 -> 14336 94 us through the band kernel for that layout, 66 in
+	// tiles; 9216 -> 2304 59 against 29; with the 256000 columns of an output head the band kernel stays 5 % ahead)
+	const bool tiles_first = a_layout == ANYGPU_A_ROW_MAJOR && M >= 33 && (b_layout == ANYGPU_B_COL_MAJOR || N <= 65536) &&
+	                         gemm_f32_ring_applies(A, B, M, N, K, lda, ldb, stride_a, stride_b, batch, 0, 64, b_layout);
 	// few rows against k-contiguous weights with the columns of an output head: whole lines per row and load instruction
 	if (batch == 1 && a_layout == ANYGPU_A_ROW_MAJOR && b_layout == ANYGPU_B_COL_MAJOR && M >= kWideMinRowsF32 &&
 	    gemm_band_kc_wide_applies<float>(A, B, C, M, N, K, lda, ldb, ldc, kWideMaxRowsF32))
 		return launch_gemm_band_kc_wide<float>(A, B, bias, C, M, N, K, lda, ldb, ldc, kEpiBias, 0.0f, stream);
 	if (batch == 1 && !tiles_first && a_layout == ANYGPU_A_ROW_MAJOR && gemm_band_applies<float>(A, B, nullptr, C, M, N, K, lda, ldb, ldc, b_layout))
 		return launch_gemm_band<float>(A, B, nullptr, bias, C, M, N, K, lda, ldb, ldc, kEpiBias, 0.0f, stream);
-	if (batch == 1 && a_layout == ANYGPU_A_ROW_MAJOR && b_layout == ANYGPU_B_ROW_MAJOR &&
+	if (batch == 1 && !tiles_first && a_layout == ANYGPU_A_ROW_MAJOR && b_layout == ANYGPU_B_ROW_MAJOR &&
 	    gemm_band_ncontig_applies(A, B, nullptr, C, M, N, K, lda, ldb, ldc, false))
 		return launch_gemm_band_ncontig(A, B, nullptr, bias, C, M, N, K, lda, ldb, ldc, kEpiBias, 0.0f, stream);
 	if (batch == 1 && a_layout == ANYGPU_A_ROW_MAJOR && gemm_skinny_applies<float>(A, B, nullptr, M, N, K, lda, ldb, b_layout))

@@ -1150,6 +1150,17 @@ def test_mm_k_contiguous_weights_either_side_of_the_routing_rules(ops, oracle, d
     assert bool((cbuf[:, n:] == -3.0).all())
 
 
+@pytest.mark.parametrize("m,k,n", [(32, 128, 4096), (33, 128, 4096), (40, 256, 65536), (40, 256, 65540), (64, 96, 9216), (48, 64, 70000)])
+def test_mm_f32_n_contiguous_weights_either_side_of_the_routing_rules(ops, oracle, m, k, n):
+    # [K, N] float32 weights: the band kernel for that layout up to 32 rows and for output heads, the tile kernels from 33
+    # rows on up to 65536 columns; small integers, every sum exact
+    a = synth.integers(m + 71, (m, k), -2, 2)
+    b = synth.integers(n + 72, (k, n), -2, 2)
+    want = oracle.tensor_mm(a, b, threads=8)
+    got = host(ops.tensor_mm(dev(a.astype(np.float32)), dev(b.astype(np.float32))))
+    assert np.array_equal(got, want)
+
+
 @pytest.mark.parametrize("layout", ["nk", "kn"])
 @pytest.mark.parametrize("m,k,n", [(520, 4096, 14336), (264, 1024, 8192), (1100, 512, 9216), (640, 2048, 14336)])
 def test_mm_f16_rows_just_past_a_multiple_of_256(ops, oracle, layout, m, k, n):
