@@ -23,7 +23,8 @@ The memory-bound kernels rotate over several buffer sets so that the working set
 
 `--gemm-shapes` (or `--gemm-shapes f32`) prints, instead of the JSON line, a table of the fp16 (fp32) GEMM over the
 projection shapes of the models the path serves (8 row counts x 14 weight shapes, weights k-contiguous) next to torch.matmul, i.e. the vendor library,
-on the same operands.
+on the same operands; with `--gemm-rows between` 22 row counts between the tile heights (3 .. 2060) over 8 of the
+shapes, with `--gemm-layout kn` the weights stored [K, N].
 """
 from __future__ import annotations
 
@@ -90,6 +91,11 @@ def parse_args():
     ap.add_argument("--only", default="", help="comma list of: gemm,gemm32,conv,softmax,attn,attn32,decode,norm,head (default: all)")
     ap.add_argument("--gemm-shapes", nargs="?", const="f16", default=None, choices=("f16", "f32"),
                     help="print the table of GEMM layer shapes (fp16, or fp32 with `--gemm-shapes f32`) against torch.matmul and exit")
+    ap.add_argument("--gemm-rows", default="layer", choices=("layer", "between"),
+                    help="with --gemm-shapes: the row counts of the layer table (powers of two, default) or 22 row counts between "
+                         "the tile heights over 8 of the shapes")
+    ap.add_argument("--gemm-layout", default="nk", choices=("nk", "kn"),
+                    help="with --gemm-shapes: weights stored [N, K] (default) or [K, N]")
     ap.add_argument("--gemm-operands", default="uniform", choices=("uniform", "low_toggle"),
                     help="operands of the headline GEMM: U(-1, 1) as the metric names them (default), or integers -2 .. 2 "
                          "(few bits toggle: for profiler runs of the power-limit comparison; the line then says so)")
@@ -577,12 +583,16 @@ def bench_lm_head(torch, ops, steps, warmup, dtype):
 LAYER_WEIGHTS = [(9216, 2304), (18432, 2304), (2304, 9216), (2048, 2304), (1024, 2304), (4096, 2304), (2304, 2048),
                  (2048, 2048), (8192, 2048), (2048, 8192), (4096, 4096), (14336, 4096), (4096, 14336), (6144, 4096)]
 LAYER_ROWS = (16, 64, 128, 256, 512, 1024, 2048, 4096)
+# row counts between the heights of the tiles and of the few-row kernels' row blocks
+BETWEEN_WEIGHTS = [(9216, 2304), (2304, 9216), (4096, 4096), (14336, 4096), (4096, 14336), (8192, 2048), (6144, 4096), (18944, 3584)]
+BETWEEN_ROWS = (3, 8, 16, 24, 32, 40, 48, 64, 65, 80, 96, 128, 130, 160, 200, 256, 270, 384, 520, 768, 1100, 2060)
 
 
-def sweep_gemm_shapes(torch, ops, capi, dtype_name="f16"):
+def sweep_gemm_shapes(torch, ops, capi, dtype_name="f16", row_set="layer", layout="nk"):
     """[rows, K] x [N, K]^T for the (N, K) of Gemma2-2B / Zamba2 / Llama-8B-sized projections: microseconds of this
     library and of torch.matmul (hipBLASLt) on the same uniform random operands, each the better of two runs of 40
-    back-to-back launches taken alternately."""
+    back-to-back launches taken alternately.  row_set "between": row counts between the tile heights (3 .. 2060) over 8 of
+    the shapes; layout "kn": the weights stored [K, N]."""
     def timed(fn, iters=40, warm=8):
         for _ in range(warm):
             fn()
@@ -599,20 +609,25 @@ def sweep_gemm_shapes(torch, ops, capi, dtype_name="f16"):
     print("| rows | K | N | this library us | torch.matmul us | ratio |")
     print("|---:|---:|---:|---:|---:|---:|")
     ratios = []
-    for n, k in LAYER_WEIGHTS:
-        weight = (torch.rand(n, k, device="cuda") * 2 - 1).to(dtype)
-        for rows in LAYER_ROWS:
+    weights, row_counts = (LAYER_WEIGHTS, LAYER_ROWS) if row_set == "layer" else (BETWEEN_WEIGHTS, BETWEEN_ROWS)
+    for n, k in weights:
+        weight = (torch.rand(n, k, device="cuda") * 2 - 1).to(dtype) if layout == "nk" else (torch.rand(k, n, device="cuda") * 2 - 1).to(dtype)
+        for rows in row_counts:
             a = (torch.rand(rows, k, device="cuda") * 2 - 1).to(dtype)
             c = torch.empty(rows, n, device="cuda", dtype=dtype)
-            mine = lambda: ops.tensor_mm(a, weight, out=c, b_layout=capi.B_COL_MAJOR)
-            theirs = lambda: torch.matmul(a, weight.t(), out=c)
+            if layout == "nk":
+                mine = lambda: ops.tensor_mm(a, weight, out=c, b_layout=capi.B_COL_MAJOR)
+                theirs = lambda: torch.matmul(a, weight.t(), out=c)
+            else:
+                mine = lambda: ops.tensor_mm(a, weight, out=c)
+                theirs = lambda: torch.matmul(a, weight, out=c)
             t_mine, t_theirs = timed(mine), timed(theirs)
             t_mine, t_theirs = min(t_mine, timed(mine)), min(t_theirs, timed(theirs))
             ratios.append(t_mine / t_theirs)
             print(f"| {rows} | {k} | {n} | {t_mine:.1f} | {t_theirs:.1f} | {t_mine / t_theirs:.2f} |", flush=True)
     ratios.sort()
     print(f"\n{len(ratios)} shapes: median ratio {statistics.median(ratios):.2f}, worst {ratios[-1]:.2f}, "
-          f"{sum(r > 1.05 for r in ratios)} above 1.05, {sum(r < 0.95 for r in ratios)} below 0.95")
+          f"{sum(r > 1.10 for r in ratios)} above 1.10, {sum(r > 1.05 for r in ratios)} above 1.05, {sum(r < 0.95 for r in ratios)} below 0.95")
 
 
 def sample_gemm_shapes(torch, ops, capi):
@@ -663,7 +678,7 @@ def main():
     capi.load()
     torch.cuda.set_device(0)
     if args.gemm_shapes:
-        sweep_gemm_shapes(torch, ops, capi, args.gemm_shapes)
+        sweep_gemm_shapes(torch, ops, capi, args.gemm_shapes, args.gemm_rows, args.gemm_layout)
         return 0
     only = set(filter(None, args.only.split(",")))
     want = lambda name: not only or name in only
