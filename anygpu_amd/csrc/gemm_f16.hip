@@ -264,7 +264,8 @@ static FourWavePlan plan_four_wave(int64_t M, int64_t N, int64_t K, int64_t batc
 
 // What the launcher expects one uncut product to take with the best of its tile kernels, from the prices above (for
 // comparing a product with the same product divided by rows; microseconds).
-static double estimate_tiles_us(int64_t M, int64_t N, int64_t K, int64_t cus, bool whole_tiles)
+// `plane_bytes`: what the stream's workspace offers the planes of a cut along K (0: none).
+static double estimate_tiles_us(int64_t M, int64_t N, int64_t K, int64_t cus, bool whole_tiles, size_t plane_bytes)
 {
 	const double slabs = (double)((K + 63) / 64);
 	const auto blocks = [&](int64_t t) { return ((M + t - 1) / t) * ((N + t - 1) / t); };
@@ -272,7 +273,8 @@ static double estimate_tiles_us(int64_t M, int64_t N, int64_t K, int64_t cus, bo
 	const int64_t blocks_rect = ((M + 255) / 256) * ((N + 127) / 128);
 	per_slab = std::min(per_slab, TilePrices::kRect * (double)((blocks_rect + cus - 1) / cus));
 	double us = per_slab * slabs + 6.0;
-	if (whole_tiles) us = std::min(us, plan_four_wave(M, N, K, 1, cus, 0).us);
+	const int64_t plane_room = (K >= 1024 && N % 8 == 0) ? (int64_t)(plane_bytes / ((size_t)M * N * sizeof(float))) : 0;
+	if (whole_tiles) us = std::min(us, plan_four_wave(M, N, K, 1, cus, plane_room).us);
 	// no launch ends before its operands have come in once (few rows: at what the bandwidth-shaped kernels reach)
 	const double stream_us = 2.0 * ((double)M + (double)N) * (double)K / 6.2e6 + 3.0;
 	return std::max(us, stream_us);
@@ -453,8 +455,9 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
 		if (batch == 1 && M > 256 && M % 256 != 0 && M % 256 <= 128)
 		{
 			const int64_t m_body = M / 256 * 256, m_tail = M - m_body;
-			const double whole_us = estimate_tiles_us(M, N, K, cus, whole_tiles);
-			const double divided_us = estimate_tiles_us(m_body, N, K, cus, whole_tiles) + estimate_tiles_us(m_tail, N, K, cus, whole_tiles);
+			const size_t plane_bytes = band::workspace_capacity(stream);
+			const double whole_us = estimate_tiles_us(M, N, K, cus, whole_tiles, plane_bytes);
+			const double divided_us = estimate_tiles_us(m_body, N, K, cus, whole_tiles, plane_bytes) + estimate_tiles_us(m_tail, N, K, cus, whole_tiles, plane_bytes);
 			if (divided_us < 0.97 * whole_us)
 			{
 				const hipError_t err = launch_gemm_f16(A, B, C, m_body, N, K, lda, ldb, ldc, 0, 0, 0, 1, b_layout, stream);
