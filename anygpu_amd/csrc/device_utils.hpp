@@ -53,6 +53,18 @@ __device__ __forceinline__ float wave_allreduce(float v, Op op)
 	return op(op(r0, r1), op(r2, r3));
 }
 
+// All-reduce over each row of 16 lanes of a wave (the first four steps of the above): every lane ends up with the
+// result of its own row.
+template <typename Op>
+__device__ __forceinline__ float row_allreduce(float v, Op op)
+{
+	v = op(v, dpp_move<0xB1>(v));    // quad_perm [1,0,3,2]
+	v = op(v, dpp_move<0x4E>(v));    // quad_perm [2,3,0,1]
+	v = op(v, dpp_move<0x124>(v));   // row_ror:4
+	v = op(v, dpp_move<0x128>(v));   // row_ror:8
+	return v;
+}
+
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
 

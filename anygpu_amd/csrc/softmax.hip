@@ -7,8 +7,10 @@
 // states with DPP reductions, then normalises from registers.  Vectors that lie wholly
 // outside the visible key interval [lo, hi] of the row are never loaded; their outputs are
 // stored as zeros.
-// General kernel: one 256-thread block per row with scalar accesses for any width, stride
-// or alignment; it reads the visible part of the row twice.
+// Short rows (up to 64 vectors) share a wave four at a time; rows longer than a block's registers hold are walked
+// twice by a block of 1024 threads with 16-byte accesses.
+// General kernel (such rows with a mask tensor): one 256-thread block per row with scalar accesses for any width,
+// stride or alignment; it reads the visible part of the row twice.
 #include "device_utils.hpp"
 #include "launch.hpp"
 
@@ -86,12 +88,13 @@ __device__ __forceinline__ float exp2_shift(float a, float b)
 // LOOSE: rows may start at any element (not only at 16-byte boundaries) and cols need not be a multiple of
 // the vector length.  Vector accesses then go out at element alignment (global memory takes them; the
 // compiler is told through the type) and the last, partial vector of a row is moved element by element.
-// GROUP: threads that share a row: 64 (a wave per row, four rows per block) or 256 (the block per row, for rows
-// longer than a wave's registers hold).
+// GROUP: threads that share a row: 16 (a row of lanes per row, four rows per wave and sixteen per block, for rows of up
+// to 64 vectors: a wave per row would leave most of its lanes without a vector and few bytes in flight), 64 (a wave per
+// row, four rows per block) or 256 (the block per row, for rows longer than a wave's registers hold).
 template <typename T, int VPL, bool LOOSE, int GROUP>
 __global__ __launch_bounds__(256) void softmax_rows_wave_kernel(const SoftmaxArgs a)
 {
-	static_assert(GROUP == 64 || GROUP == 256, "a wave or the block per row");
+	static_assert(GROUP == 16 || GROUP == 64 || GROUP == 256, "a row of lanes, a wave or the block per row");
 	constexpr int EPV = 16 / (int)sizeof(T);
 	using Vec = typename Vec16<T>::type;
 	typedef Vec LooseVec __attribute__((aligned(sizeof(T))));
@@ -99,7 +102,8 @@ __global__ __launch_bounds__(256) void softmax_rows_wave_kernel(const SoftmaxArg
 	__shared__ float red_m[4], red_s[4];
 
 	const int lane = threadIdx.x & (GROUP - 1);
-	const int64_t row = GROUP == 64 ? (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6) : (int64_t)blockIdx.x;
+	const int64_t row = GROUP == 16 ? (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4)
+	                  : GROUP == 64 ? (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6) : (int64_t)blockIdx.x;
 	if (row >= a.rows) return;  // uniform over the group
 
 	const RowSpan span = row_span(a, row);
@@ -186,8 +190,8 @@ __global__ __launch_bounds__(256) void softmax_rows_wave_kernel(const SoftmaxArg
 		}
 	}
 
-	float M = wave_allreduce(st.m, MaxOp());
-	float S = wave_allreduce(st.s * exp2_shift(st.m, M), SumOp());
+	float M = GROUP == 16 ? row_allreduce(st.m, MaxOp()) : wave_allreduce(st.m, MaxOp());
+	float S = GROUP == 16 ? row_allreduce(st.s * exp2_shift(st.m, M), SumOp()) : wave_allreduce(st.s * exp2_shift(st.m, M), SumOp());
 	if constexpr (GROUP == 256)
 	{
 		const int wave = threadIdx.x >> 6;
@@ -421,10 +425,142 @@ __global__ __launch_bounds__(256) void softmax_rows_block_kernel(const SoftmaxAr
 	}
 }
 
+// Rows longer than a block's registers hold (more than 32768 elements: the logits of an output head), without a mask
+// tensor: a block of 1024 threads per row walks the row twice with 16-byte accesses, four per thread in flight: first
+// the online maximum and sum, then, the row coming out of the L2 this time, the probabilities.  The vectors are
+// aligned to the row's own start (rows of any length and pitch); where the result row is not aligned alike its vectors
+// go out at element alignment.
+template <typename T>
+__global__ __launch_bounds__(1024) void softmax_rows_long_kernel(const SoftmaxArgs a)
+{
+	constexpr int EPV = 16 / (int)sizeof(T);
+	constexpr int kThreads = 1024, kAhead = 4;
+	using Vec = typename Vec16<T>::type;
+	typedef Vec LooseVec __attribute__((aligned(sizeof(T))));
+	__shared__ float red_m[16], red_s[16];
+
+	const int64_t row = blockIdx.x;
+	const RowSpan span = row_span(a, row);
+	const T* __restrict__ xr = static_cast<const T*>(a.x) + row * a.xs;
+	T* __restrict__ yr = static_cast<T*>(a.y) + row * a.ys;
+	// elements [0, head): one by one; then nvec whole vectors at 16-byte boundaries of x; then the rest one by one
+	const int64_t to_boundary = (int64_t)(((16 - reinterpret_cast<uintptr_t>(xr) % 16) % 16) / sizeof(T));
+	const int64_t head = to_boundary < a.cols ? to_boundary : a.cols;
+	const int64_t nvec = (a.cols - head) / EPV;
+	const int64_t rest = head + nvec * EPV;
+	const Vec* __restrict__ xv = reinterpret_cast<const Vec*>(xr + head);
+	const bool y_aligned = reinterpret_cast<uintptr_t>(yr + head) % 16 == 0;
+	const int64_t lo = span.lo, hi = span.hi;
+	const int tid = threadIdx.x;
+
+	OnlineState st;
+	auto take_one = [&](int64_t j) {
+		if (j < lo || j > hi) return;
+		const float z = logit2(a, (float)xr[j]);
+		const float mn = fmaxf(st.m, z);
+		st.s = st.s * exp2_shift(st.m, mn) + exp2_shift(z, mn);
+		st.m = mn;
+	};
+	auto take_vec = [&](int64_t v, const Vec& val) {
+		const int64_t e0 = head + v * EPV;
+		if (e0 > hi || e0 + EPV - 1 < lo) return;
+		float z[EPV];
+		float vmax = -INFINITY;
+#pragma unroll
+		for (int e = 0; e < EPV; ++e)
+		{
+			const int64_t j = e0 + e;
+			z[e] = (j >= lo && j <= hi) ? logit2(a, (float)val[e]) : -INFINITY;
+			vmax = fmaxf(vmax, z[e]);
+		}
+		const float mn = fmaxf(st.m, vmax);
+		float acc = st.s * exp2_shift(st.m, mn);
+#pragma unroll
+		for (int e = 0; e < EPV; ++e) acc += exp2_shift(z[e], mn);
+		st.s = acc;
+		st.m = mn;
+	};
+	if (tid < head) take_one(tid);
+	for (int64_t j = rest + tid; j < a.cols; j += kThreads) take_one(j);
+	for (int64_t v0 = tid; v0 < nvec; v0 += (int64_t)kThreads * kAhead)
+	{
+		Vec val[kAhead];
+#pragma unroll
+		for (int u = 0; u < kAhead; ++u)
+		{
+			const int64_t v = v0 + (int64_t)u * kThreads;
+			const int64_t e0 = head + v * EPV;
+			val[u] = Vec{};
+			if (v < nvec && e0 <= hi && e0 + EPV - 1 >= lo) val[u] = xv[v];
+		}
+#pragma unroll
+		for (int u = 0; u < kAhead; ++u)
+		{
+			const int64_t v = v0 + (int64_t)u * kThreads;
+			if (v < nvec) take_vec(v, val[u]);
+		}
+	}
+
+	const int wave = tid >> 6;
+	const float wm = wave_allreduce(st.m, MaxOp());
+	const float ws = wave_allreduce(st.s * exp2_shift(st.m, wm), SumOp());
+	if ((tid & 63) == 0)
+	{
+		red_m[wave] = wm;
+		red_s[wave] = ws;
+	}
+	__syncthreads();
+	float M = -INFINITY;
+#pragma unroll
+	for (int w = 0; w < 16; ++w) M = fmaxf(M, red_m[w]);
+	float S = 0.0f;
+#pragma unroll
+	for (int w = 0; w < 16; ++w) S += red_s[w] * exp2_shift(red_m[w], M);
+	const float inv = S > 0.0f ? 1.0f / S : 0.0f;
+
+	auto put_one = [&](int64_t j) {
+		const float p = (j >= lo && j <= hi) ? exp2_shift(logit2(a, (float)xr[j]), M) * inv : 0.0f;
+		yr[j] = (T)p;
+	};
+	if (tid < head) put_one(tid);
+	for (int64_t j = rest + tid; j < a.cols; j += kThreads) put_one(j);
+	for (int64_t v0 = tid; v0 < nvec; v0 += (int64_t)kThreads * kAhead)
+	{
+		Vec val[kAhead];
+#pragma unroll
+		for (int u = 0; u < kAhead; ++u)
+		{
+			const int64_t v = v0 + (int64_t)u * kThreads;
+			const int64_t e0 = head + v * EPV;
+			val[u] = Vec{};
+			if (v < nvec && e0 <= hi && e0 + EPV - 1 >= lo) val[u] = xv[v];
+		}
+#pragma unroll
+		for (int u = 0; u < kAhead; ++u)
+		{
+			const int64_t v = v0 + (int64_t)u * kThreads;
+			if (v >= nvec) continue;
+			const int64_t e0 = head + v * EPV;
+			Vec out = {};
+			if (e0 <= hi && e0 + EPV - 1 >= lo)
+			{
+#pragma unroll
+				for (int e = 0; e < EPV; ++e)
+				{
+					const int64_t j = e0 + e;
+					out[e] = (T)((j >= lo && j <= hi) ? exp2_shift(logit2(a, (float)val[u][e]), M) * inv : 0.0f);
+				}
+			}
+			if (y_aligned) __builtin_nontemporal_store(out, reinterpret_cast<Vec*>(yr + e0));
+			else *reinterpret_cast<LooseVec*>(yr + e0) = out;
+		}
+	}
+}
+
 template <typename T, int VPL, bool LOOSE = false, int GROUP = 64>
 static hipError_t launch_wave(const SoftmaxArgs& a, hipStream_t stream)
 {
-	const unsigned blocks = GROUP == 64 ? (unsigned)((a.rows + 3) / 4) : (unsigned)a.rows;
+	const unsigned blocks = GROUP == 16 ? (unsigned)((a.rows + 15) / 16) : GROUP == 64 ? (unsigned)((a.rows + 3) / 4) : (unsigned)a.rows;
 	discard_stale_error();
 	softmax_rows_wave_kernel<T, VPL, LOOSE, GROUP><<<dim3(blocks), dim3(256), 0, stream>>>(a);
 	return hipGetLastError();
@@ -434,11 +570,8 @@ static hipError_t launch_wave(const SoftmaxArgs& a, hipStream_t stream)
 template <typename T, bool LOOSE>
 static hipError_t launch_long_rows(const SoftmaxArgs& a, int64_t nvec, hipStream_t stream)
 {
-	constexpr int kMaxVpl = sizeof(T) == 2 ? 16 : 32;
 	if (nvec <= 256 * 8) return launch_wave<T, 8, LOOSE, 256>(a, stream);
-	if (nvec <= 256 * 16) return launch_wave<T, 16, LOOSE, 256>(a, stream);
-	if constexpr (kMaxVpl >= 32) return launch_wave<T, 32, LOOSE, 256>(a, stream);
-	return hipErrorInvalidValue;       // not reached: the caller checks the capacity
+	return launch_wave<T, 16, LOOSE, 256>(a, stream);       // (the caller checks the capacity: 256 x 16 vectors)
 }
 
 template <typename T>
@@ -462,6 +595,20 @@ hipError_t launch_softmax_rows(const void* x, void* y, int64_t rows, int64_t col
 	                    (reinterpret_cast<uintptr_t>(x) % 16 == 0) && (reinterpret_cast<uintptr_t>(y) % 16 == 0) &&
 	                    (mask == nullptr || (mask_stride % EPV == 0 && reinterpret_cast<uintptr_t>(mask) % 16 == 0));
 	const int64_t nvec = cols / EPV;
+	// short rows (up to 64 vectors: 512 halves, 256 floats): sixteen lanes per row, four rows per wave
+	if (vec_ok && nvec <= 64 && rows >= 64)
+	{
+		if (nvec <= 16) return launch_wave<T, 1, false, 16>(a, stream);
+		if (nvec <= 32) return launch_wave<T, 2, false, 16>(a, stream);
+		return launch_wave<T, 4, false, 16>(a, stream);       // (twice as many vectors per lane: slower than a wave per row)
+	}
+	if (!vec_ok && (cols + EPV - 1) / EPV <= 64 && rows >= 64)
+	{
+		const int64_t loose = (cols + EPV - 1) / EPV;
+		if (loose <= 16) return launch_wave<T, 1, true, 16>(a, stream);
+		if (loose <= 32) return launch_wave<T, 2, true, 16>(a, stream);
+		return launch_wave<T, 4, true, 16>(a, stream);
+	}
 	if constexpr (sizeof(T) == 2)
 	{
 		// vectors a row can touch: its visible keys (the window when causal + window, else the
@@ -482,15 +629,25 @@ hipError_t launch_softmax_rows(const void* x, void* y, int64_t rows, int64_t col
 			if (span_vecs <= kWaveSize * 16) return launch_f16_window<16>(a, stream);
 		}
 	}
-	constexpr int kMaxVpl = sizeof(T) == 2 ? 16 : 32;
+	// A wave holds up to 16 vectors per lane of its row (32 of float32 fit the registers, but leave a SIMD with too few
+	// waves: 16384 x 8192 float32 353 us that way, 185 us with the block per row); the block per row up to 16 as well
+	// (32768 halves, 16384 floats); longer rows, and long rows too few to give every CU a block, are walked twice by
+	// 1024 threads (8192 x 32768 float32: 751 us in registers, 426 us walked twice; 128 x 32768 halves: 18 -> 10 us).
+	constexpr int kMaxVpl = 16;
+	const bool walk_twice = mask == nullptr && (nvec > (int64_t)256 * kMaxVpl || (nvec > 2048 && rows < 256));
+	if (vec_ok && walk_twice)
+	{
+		discard_stale_error();
+		softmax_rows_long_kernel<T><<<dim3((unsigned)rows), dim3(1024), 0, stream>>>(a);
+		return hipGetLastError();
+	}
 	if (vec_ok && nvec <= (int64_t)kWaveSize * kMaxVpl)
 	{
 		if (nvec <= kWaveSize * 1) return launch_wave<T, 1>(a, stream);
 		if (nvec <= kWaveSize * 2) return launch_wave<T, 2>(a, stream);
 		if (nvec <= kWaveSize * 4) return launch_wave<T, 4>(a, stream);
 		if (nvec <= kWaveSize * 8) return launch_wave<T, 8>(a, stream);
-		if (nvec <= kWaveSize * 16) return launch_wave<T, 16>(a, stream);
-		if constexpr (kMaxVpl >= 32) return launch_wave<T, 32>(a, stream);
+		return launch_wave<T, 16>(a, stream);
 	}
 	if (vec_ok && nvec <= (int64_t)256 * kMaxVpl) return launch_long_rows<T, false>(a, nvec, stream);
 	// rows at element alignment, any width: the same wave kernel with element-aligned vector accesses
@@ -501,12 +658,13 @@ hipError_t launch_softmax_rows(const void* x, void* y, int64_t rows, int64_t col
 		if (nvec_loose <= kWaveSize * 2) return launch_wave<T, 2, true>(a, stream);
 		if (nvec_loose <= kWaveSize * 4) return launch_wave<T, 4, true>(a, stream);
 		if (nvec_loose <= kWaveSize * 8) return launch_wave<T, 8, true>(a, stream);
-		if (nvec_loose <= kWaveSize * 16) return launch_wave<T, 16, true>(a, stream);
-		if constexpr (kMaxVpl >= 32) return launch_wave<T, 32, true>(a, stream);
+		return launch_wave<T, 16, true>(a, stream);
 	}
-	if (!vec_ok && nvec_loose <= (int64_t)256 * kMaxVpl) return launch_long_rows<T, true>(a, nvec_loose, stream);
+	if (!vec_ok && nvec_loose <= (int64_t)256 * kMaxVpl && !(mask == nullptr && nvec_loose > 2048 && rows < 256))
+		return launch_long_rows<T, true>(a, nvec_loose, stream);
 	discard_stale_error();
-	softmax_rows_block_kernel<T><<<dim3((unsigned)rows), dim3(256), 0, stream>>>(a);
+	if (mask == nullptr) softmax_rows_long_kernel<T><<<dim3((unsigned)rows), dim3(1024), 0, stream>>>(a);
+	else softmax_rows_block_kernel<T><<<dim3((unsigned)rows), dim3(256), 0, stream>>>(a);
 	return hipGetLastError();
 }
 

@@ -47,7 +47,10 @@ def test_softmax_f32_reference_case_6x45(ops, oracle):
 @pytest.mark.parametrize("dtype", ["f16", "f32"])
 @pytest.mark.parametrize("rows,cols", [(1, 1), (3, 7), (5, 8), (64, 512), (33, 520), (17, 1024), (9, 2048),
                                        (6, 4096), (5, 8192), (3, 8200), (2, 16384), (4, 100), (7, 2047),
-                                       (2, 20000), (3, 20001), (2, 32768), (1, 40000), (2, 33001)])
+                                       (2, 20000), (3, 20001), (2, 32768), (1, 40000), (2, 33001),
+                                       # many short rows (a row of 16 lanes each) and rows a block walks twice
+                                       (200, 64), (77, 128), (100, 256), (65, 8), (130, 100), (300, 333), (1000, 500),
+                                       (70, 50257), (3, 131072), (2, 262147), (300, 16400)])
 def test_softmax_plain_shapes(ops, oracle, dtype, rows, cols):
     np_dt = np.float16 if dtype == "f16" else np.float32
     x = synth.normal(rows * 131 + cols, (rows, cols), std=2.0).astype(np_dt)
@@ -118,6 +121,10 @@ FUSED_CASES = [
     (50, 37, 25, 0, 0.3, 5.0, True, 7),
     (16, 8192, 16, 8176, 0.0625, 50.0, True, 4096),
     (8, 64, 8, -3, 0.125, 0.0, True, 0),            # first rows see nothing at all
+    (128, 96, 64, 32, 0.25, 10.0, True, 20),        # many short rows, sixteen lanes per row
+    (80, 200, 80, 120, 0.5, 0.0, True, 0),
+    (4, 40000, 4, 39996, 0.1, 30.0, True, 1000),    # rows longer than a block's registers
+    (3, 70001, 3, 69000, 0.05, 0.0, True, 0),
 ]
 
 
