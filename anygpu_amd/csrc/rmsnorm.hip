@@ -3,9 +3,10 @@
 //   y = g / sqrt(mean(g^2) + eps) * (w + delta),   delta = 1 for zero-centred weights, else 0
 // The step between the SSD scan and the output projection of a Mamba2 mixer.  HBM-bound: x and z are
 // read once, y is written once, the row lives in registers between the sum of squares and the
-// scaling.  One 256-thread block per row, 16-byte accesses; the row length picks how many vectors a
-// thread keeps (1, 2, 4 or 8: up to 8192 floats or 16384 halves).  Longer rows, and rows whose
-// length or pointers do not allow 16-byte access, take a two-pass kernel that reads x and z twice.
+// scaling.  16-byte accesses; the row length picks how many threads share a row (a row of 16 lanes, a wave or the
+// 256-thread block: short rows would leave most of a block without a vector) and how many vectors a thread keeps (1, 2,
+// 4 or 8: up to 8192 floats or 16384 halves).  Longer rows are walked twice by a block of 1024 threads, the second time
+// out of the L2; rows whose length or pointers do not allow 16-byte access take a scalar two-pass kernel.
 #include "device_utils.hpp"
 #include "launch.hpp"
 
@@ -28,15 +29,19 @@ __device__ __forceinline__ float block_sum(float v, float* slots)
 	return (slots[0] + slots[1]) + (slots[2] + slots[3]);
 }
 
-template <typename T, int VPT, bool GATED>
+// GROUP threads share a row (16, 64 or 256), 256 / GROUP rows share a block.
+template <typename T, int VPT, bool GATED, int GROUP>
 __global__ __launch_bounds__(256) void gated_rmsnorm_row_kernel(
 	const T* __restrict__ x, const T* __restrict__ z, const T* __restrict__ w, T* __restrict__ y,
-	int cols, float eps, float delta)
+	int64_t rows, int cols, float eps, float delta)
 {
+	static_assert(GROUP == 16 || GROUP == 64 || GROUP == 256, "a row of lanes, a wave or the block per row");
 	typedef typename NormVec<T>::type vec_t;
 	constexpr int VEC = NormVec<T>::kLen;
 	__shared__ float slots[4];
-	const int64_t row = blockIdx.x;
+	const int64_t row = (int64_t)blockIdx.x * (256 / GROUP) + threadIdx.x / GROUP;
+	const int lane = threadIdx.x % GROUP;
+	if (row >= rows) return;                    // uniform over the group (GROUP == 256: never taken)
 	const vec_t* xr = reinterpret_cast<const vec_t*>(x + row * cols);
 	const vec_t* zr = reinterpret_cast<const vec_t*>(z + row * cols);
 	const vec_t* wr = reinterpret_cast<const vec_t*>(w);
@@ -48,7 +53,7 @@ __global__ __launch_bounds__(256) void gated_rmsnorm_row_kernel(
 #pragma unroll
 	for (int i = 0; i < VPT; ++i)
 	{
-		const int v = threadIdx.x + 256 * i;
+		const int v = lane + GROUP * i;
 		vec_t xv = {}, zv = {};
 		if (v < nvec)
 		{
@@ -63,18 +68,100 @@ __global__ __launch_bounds__(256) void gated_rmsnorm_row_kernel(
 			ss += val * val;
 		}
 	}
-	ss = block_sum(ss, slots);
+	ss = GROUP == 16 ? row_allreduce(ss, SumOp()) : GROUP == 64 ? wave_allreduce(ss, SumOp()) : block_sum(ss, slots);
 	const float scale = 1.0f / sqrtf(ss / (float)cols + eps);
 #pragma unroll
 	for (int i = 0; i < VPT; ++i)
 	{
-		const int v = threadIdx.x + 256 * i;
+		const int v = lane + GROUP * i;
 		if (v < nvec)
 		{
 			const vec_t wv = wr[v];
 			vec_t out;
 #pragma unroll
 			for (int e = 0; e < VEC; ++e) out[e] = (T)(g[i][e] * scale * ((float)wv[e] + delta));
+			__builtin_nontemporal_store(out, yr + v);
+		}
+	}
+}
+
+// Rows longer than a block keeps in registers: 1024 threads walk the row twice with 16-byte accesses, four per thread
+// in flight (the second time the row comes out of the L2).
+template <typename T, bool GATED>
+__global__ __launch_bounds__(1024) void gated_rmsnorm_long_kernel(
+	const T* __restrict__ x, const T* __restrict__ z, const T* __restrict__ w, T* __restrict__ y,
+	int64_t cols, float eps, float delta)
+{
+	typedef typename NormVec<T>::type vec_t;
+	constexpr int VEC = NormVec<T>::kLen, kThreads = 1024, kAhead = 4;
+	__shared__ float slots[16];
+	const int64_t row = blockIdx.x;
+	const vec_t* xr = reinterpret_cast<const vec_t*>(x + row * cols);
+	const vec_t* zr = reinterpret_cast<const vec_t*>(z + row * cols);
+	const vec_t* wr = reinterpret_cast<const vec_t*>(w);
+	vec_t* yr = reinterpret_cast<vec_t*>(y + row * cols);
+	const int64_t nvec = cols / VEC;
+	float ss = 0.0f;
+	for (int64_t v0 = threadIdx.x; v0 < nvec; v0 += (int64_t)kThreads * kAhead)
+	{
+		vec_t xv[kAhead], zv[kAhead];
+#pragma unroll
+		for (int u = 0; u < kAhead; ++u)
+		{
+			const int64_t v = v0 + (int64_t)u * kThreads;
+			xv[u] = vec_t{};
+			zv[u] = vec_t{};
+			if (v < nvec)
+			{
+				xv[u] = xr[v];
+				if (GATED) zv[u] = zr[v];
+			}
+		}
+#pragma unroll
+		for (int u = 0; u < kAhead; ++u)
+#pragma unroll
+			for (int e = 0; e < VEC; ++e)
+			{
+				const float val = GATED ? (float)xv[u][e] * silu_gate((float)zv[u][e]) : (float)xv[u][e];
+				ss += val * val;
+			}
+	}
+	ss = wave_allreduce(ss, SumOp());
+	if ((threadIdx.x & (kWaveSize - 1)) == 0) slots[threadIdx.x >> 6] = ss;
+	__syncthreads();
+	ss = 0.0f;
+#pragma unroll
+	for (int i = 0; i < 16; ++i) ss += slots[i];
+	const float scale = 1.0f / sqrtf(ss / (float)cols + eps);
+	for (int64_t v0 = threadIdx.x; v0 < nvec; v0 += (int64_t)kThreads * kAhead)
+	{
+		vec_t xv[kAhead], zv[kAhead], wv[kAhead];
+#pragma unroll
+		for (int u = 0; u < kAhead; ++u)
+		{
+			const int64_t v = v0 + (int64_t)u * kThreads;
+			xv[u] = vec_t{};
+			zv[u] = vec_t{};
+			wv[u] = vec_t{};
+			if (v < nvec)
+			{
+				xv[u] = xr[v];
+				if (GATED) zv[u] = zr[v];
+				wv[u] = wr[v];
+			}
+		}
+#pragma unroll
+		for (int u = 0; u < kAhead; ++u)
+		{
+			const int64_t v = v0 + (int64_t)u * kThreads;
+			if (v >= nvec) continue;
+			vec_t out;
+#pragma unroll
+			for (int e = 0; e < VEC; ++e)
+			{
+				const float val = GATED ? (float)xv[u][e] * silu_gate((float)zv[u][e]) : (float)xv[u][e];
+				out[e] = (T)(val * scale * ((float)wv[u][e] + delta));
+			}
 			__builtin_nontemporal_store(out, yr + v);
 		}
 	}
@@ -115,16 +202,22 @@ hipError_t launch_gated(const T* x, const T* z, const T* w, T* y, int64_t rows, 
 	                    reinterpret_cast<uintptr_t>(w) % 16 == 0 && (!GATED || reinterpret_cast<uintptr_t>(z) % 16 == 0);
 	const int64_t nvec = cols / VEC;
 	discard_stale_error();
-	if (vec_ok && nvec <= 256)
-		gated_rmsnorm_row_kernel<T, 1, GATED><<<grid, block, 0, stream>>>(x, z, w, y, (int)cols, eps, delta);
-	else if (vec_ok && nvec <= 512)
-		gated_rmsnorm_row_kernel<T, 2, GATED><<<grid, block, 0, stream>>>(x, z, w, y, (int)cols, eps, delta);
-	else if (vec_ok && nvec <= 1024)
-		gated_rmsnorm_row_kernel<T, 4, GATED><<<grid, block, 0, stream>>>(x, z, w, y, (int)cols, eps, delta);
-	else if (vec_ok && nvec <= 2048)
-		gated_rmsnorm_row_kernel<T, 8, GATED><<<grid, block, 0, stream>>>(x, z, w, y, (int)cols, eps, delta);
+#define ANYGPU_NORM_ROWS(VPT, GROUP) \
+	gated_rmsnorm_row_kernel<T, VPT, GATED, GROUP><<<dim3((unsigned)((rows + 256 / GROUP - 1) / (256 / GROUP))), block, 0, stream>>>( \
+		x, z, w, y, rows, (int)cols, eps, delta)
+	if (vec_ok && nvec <= 16) ANYGPU_NORM_ROWS(1, 16);
+	else if (vec_ok && nvec <= 32) ANYGPU_NORM_ROWS(2, 16);
+	else if (vec_ok && nvec <= 64) ANYGPU_NORM_ROWS(1, 64);
+	else if (vec_ok && nvec <= 128) ANYGPU_NORM_ROWS(2, 64);
+	else if (vec_ok && nvec <= 256) ANYGPU_NORM_ROWS(1, 256);
+	else if (vec_ok && nvec <= 512) ANYGPU_NORM_ROWS(2, 256);
+	else if (vec_ok && nvec <= 1024) ANYGPU_NORM_ROWS(4, 256);
+	else if (vec_ok && nvec <= 2048) ANYGPU_NORM_ROWS(8, 256);
+	else if (vec_ok)
+		gated_rmsnorm_long_kernel<T, GATED><<<grid, dim3(1024), 0, stream>>>(x, z, w, y, cols, eps, delta);
 	else
 		gated_rmsnorm_two_pass_kernel<T, GATED><<<grid, block, 0, stream>>>(x, z, w, y, cols, eps, delta);
+#undef ANYGPU_NORM_ROWS
 	return hipGetLastError();
 }
 

@@ -364,7 +364,10 @@ def test_conv1d_update_steps_match_whole_sequence(ops, oracle, dtype, b, d, widt
 
 @pytest.mark.parametrize("dtype", ["f16", "f32"])
 @pytest.mark.parametrize("rows,cols", [(1, 1), (3, 7), (5, 64), (4, 1000), (6, 1024), (3, 2048), (2, 4096), (2, 8192),
-                                       (2, 8200), (1, 16384), (2, 20000), (9, 4104)])
+                                       (2, 8200), (1, 16384), (2, 20000), (9, 4104),
+                                       # short rows sharing a block (16 lanes or a wave per row), rows walked twice
+                                       (1000, 64), (300, 128), (77, 256), (501, 32), (130, 512), (45, 1000), (19, 96),
+                                       (3, 50000), (2, 131072), (2, 16392)])
 def test_gated_rmsnorm_shapes(ops, oracle, dtype, rows, cols):
     np_dt = np.float16 if dtype == "f16" else np.float32
     eps = 1e-5
