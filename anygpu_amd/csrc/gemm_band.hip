@@ -64,7 +64,7 @@ __device__ __forceinline__ void store4(half_t* dst, const float4_t& v)
 // Epilogue and store of one thread's sums.  Register 4 q + e of a lane: column 4 * grp + e (16-row form) or
 // 8 q + 4 * grp + e (32-row form) of the MFMA column group, band row idx.
 template <typename T, int MR, int MB, int EPI, typename Acc>
-__device__ __forceinline__ void band_store(const Acc (*acc)[MB], const float* __restrict__ bias, T* __restrict__ C,
+__device__ __forceinline__ void band_store(const Acc (*acc)[MB], const T* __restrict__ bias, T* __restrict__ C,
                                            int M, int64_t N, int64_t ldc, int64_t n0, int idx, int grp, float ep_param)
 {
 	using S = BandShape<T, MR, MB>;
@@ -86,7 +86,7 @@ __device__ __forceinline__ void band_store(const Acc (*acc)[MB], const float* __
 				for (int e = 0; e < 4; ++e)
 				{
 					const float sum2 = DUAL ? acc[DUAL ? S::kNG + j : 0][b][4 * q + e] : 0.0f;
-					const float bias_n = (EPI == kEpiBias && bias && n + e < N) ? bias[n + e] : 0.0f;
+					const float bias_n = (EPI == kEpiBias && bias && n + e < N) ? (float)bias[n + e] : 0.0f;
 					out[e] = finish_sum<EPI>(acc[j][b][4 * q + e], sum2, bias_n, ep_param);
 				}
 				T* dst = C + (int64_t)m * ldc + n;
@@ -106,7 +106,7 @@ __device__ __forceinline__ void band_store(const Acc (*acc)[MB], const float* __
 // partial[tile][y][thread][register] and gemm_band_merge_kernel finishes.
 template <typename T, int MR, int MB, int EPI>
 __global__ __launch_bounds__(kBandThreads) void gemm_band_kernel(
-	const T* __restrict__ A, const T* __restrict__ B, const T* __restrict__ B2, const float* __restrict__ bias,
+	const T* __restrict__ A, const T* __restrict__ B, const T* __restrict__ B2, const T* __restrict__ bias,
 	T* __restrict__ C, float* __restrict__ partial,
 	int M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc, int chunks_per_split, float ep_param)
 {
@@ -291,7 +291,7 @@ __global__ __launch_bounds__(kBandThreads) void gemm_band_kernel(
 // latency-bound job is spread over many waves; the loads of four splits are in flight together and added in order.
 template <typename T, int MR, int MB, int EPI>
 __global__ __launch_bounds__(kBandThreads) void gemm_band_merge_kernel(
-	const float* __restrict__ partial, const float* __restrict__ bias, T* __restrict__ C,
+	const float* __restrict__ partial, const T* __restrict__ bias, T* __restrict__ C,
 	int M, int64_t N, int64_t ldc, int splits, int64_t tiles, float ep_param)
 {
 	using S = BandShape<T, MR, MB>;
@@ -340,7 +340,7 @@ __global__ __launch_bounds__(kBandThreads) void gemm_band_merge_kernel(
 #pragma unroll
 	for (int e = 0; e < 4; ++e)
 	{
-		const float bias_n = (EPI == kEpiBias && bias && n + e < N) ? bias[n + e] : 0.0f;
+		const float bias_n = (EPI == kEpiBias && bias && n + e < N) ? (float)bias[n + e] : 0.0f;
 		out[e] = finish_sum<EPI>(sum[0][e], sum[kMats - 1][e], bias_n, ep_param);
 	}
 	T* dst = C + (int64_t)m * ldc + n;
@@ -354,7 +354,7 @@ __global__ __launch_bounds__(kBandThreads) void gemm_band_merge_kernel(
 }
 
 template <typename T, int MR, int MB, int EPI>
-hipError_t launch_band(const T* A, const T* B, const T* B2, const float* bias, T* C, int M, int64_t N, int64_t K,
+hipError_t launch_band(const T* A, const T* B, const T* B2, const T* bias, T* C, int M, int64_t N, int64_t K,
                        int64_t lda, int64_t ldb, int64_t ldc, float ep_param, hipStream_t stream)
 {
 	using S = BandShape<T, MR, MB>;
@@ -580,7 +580,7 @@ bool gemm_band_applies(const T* A, const T* B, const T* B2, const T* C, int64_t 
 }
 
 template <typename T>
-hipError_t launch_gemm_band(const T* A, const T* B, const T* B2, const float* bias, T* C,
+hipError_t launch_gemm_band(const T* A, const T* B, const T* B2, const T* bias, T* C,
                             int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc,
                             int epilogue, float ep_param, hipStream_t stream)
 {
@@ -603,7 +603,7 @@ template bool gemm_band_applies<half_t>(const half_t*, const half_t*, const half
                                         int64_t, int64_t, int64_t, int);
 template hipError_t launch_gemm_band<float>(const float*, const float*, const float*, const float*, float*, int64_t, int64_t, int64_t,
                                             int64_t, int64_t, int64_t, int, float, hipStream_t);
-template hipError_t launch_gemm_band<half_t>(const half_t*, const half_t*, const half_t*, const float*, half_t*, int64_t, int64_t, int64_t,
+template hipError_t launch_gemm_band<half_t>(const half_t*, const half_t*, const half_t*, const half_t*, half_t*, int64_t, int64_t, int64_t,
                                              int64_t, int64_t, int64_t, int, float, hipStream_t);
 
 }  // namespace anygpu

@@ -51,7 +51,7 @@ __device__ __forceinline__ int4v from_partner(const int4v& v)
 // MB: row blocks of 16 (M <= 16 MB).  EPI: kEpiBias (+ bias[n] when bias != NULL) or kEpiSoftcap.
 template <typename T, int MB, int EPI>
 __global__ __launch_bounds__(kBandThreads) void gemm_band_kc_wide_kernel(
-	const T* __restrict__ A, const T* __restrict__ B, const float* __restrict__ bias, T* __restrict__ C,
+	const T* __restrict__ A, const T* __restrict__ B, const T* __restrict__ bias, T* __restrict__ C,
 	int M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc, float ep_param)
 {
 	constexpr int EPC = 16 / (int)sizeof(T);                       // elements per 16-byte chunk
@@ -226,7 +226,7 @@ __global__ __launch_bounds__(kBandThreads) void gemm_band_kc_wide_kernel(
 #pragma unroll
 			for (int r = 0; r < 4; ++r)
 			{
-				const float bias_n = (EPI == kEpiBias && bias) ? bias[n + r] : 0.0f;
+				const float bias_n = (EPI == kEpiBias && bias) ? (float)bias[n + r] : 0.0f;
 				out[r] = (T)finish_sum<EPI, sizeof(T) == 2>(acc[t][b][r], 0.0f, bias_n, ep_param);
 			}
 			*reinterpret_cast<OutVec*>(C + (int64_t)m * ldc + n) = out;
@@ -235,7 +235,7 @@ __global__ __launch_bounds__(kBandThreads) void gemm_band_kc_wide_kernel(
 }
 
 template <typename T, int MB>
-hipError_t launch_rows(const T* A, const T* B, const float* bias, T* C, int M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
+hipError_t launch_rows(const T* A, const T* B, const T* bias, T* C, int M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
                        int64_t ldc, int epilogue, float ep_param, hipStream_t stream)
 {
 	const dim3 grid((unsigned)((N + kWideBlockCols - 1) / kWideBlockCols));
@@ -269,7 +269,7 @@ bool gemm_band_kc_wide_applies(const T* A, const T* B, const T* C, int64_t M, in
 }
 
 template <typename T>
-hipError_t launch_gemm_band_kc_wide(const T* A, const T* B, const float* bias, T* C, int64_t M, int64_t N, int64_t K,
+hipError_t launch_gemm_band_kc_wide(const T* A, const T* B, const T* bias, T* C, int64_t M, int64_t N, int64_t K,
                                     int64_t lda, int64_t ldb, int64_t ldc, int epilogue, float ep_param, hipStream_t stream)
 {
 	if (M <= 16) return launch_rows<T, 1>(A, B, bias, C, (int)M, N, K, lda, ldb, ldc, epilogue, ep_param, stream);
@@ -282,7 +282,7 @@ template bool gemm_band_kc_wide_applies<float>(const float*, const float*, const
 template bool gemm_band_kc_wide_applies<half_t>(const half_t*, const half_t*, const half_t*, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t);
 template hipError_t launch_gemm_band_kc_wide<float>(const float*, const float*, const float*, float*, int64_t, int64_t, int64_t,
                                                     int64_t, int64_t, int64_t, int, float, hipStream_t);
-template hipError_t launch_gemm_band_kc_wide<half_t>(const half_t*, const half_t*, const float*, half_t*, int64_t, int64_t, int64_t,
+template hipError_t launch_gemm_band_kc_wide<half_t>(const half_t*, const half_t*, const half_t*, half_t*, int64_t, int64_t, int64_t,
                                                      int64_t, int64_t, int64_t, int, float, hipStream_t);
 
 }  // namespace anygpu

@@ -280,10 +280,12 @@ static double estimate_tiles_us(int64_t M, int64_t N, int64_t K, int64_t cus, bo
 	return std::max(us, stream_us);
 }
 
-// C[m, n] = half(sum over splits of planes[split][m][n]), one thread per eight columns (N a multiple of 8), the
-// planes added in order
+// C[m, n] = half(finish(sum over splits of planes[split][m][n])), one thread per eight columns (N a multiple of 8), the
+// planes added in order.  EPI: kEpiBias (+ bias[n] when bias != NULL) or kEpiSoftcap.
+template <int EPI>
 __global__ __launch_bounds__(256) void gemm_f16_split_merge_kernel(
-	const float* __restrict__ planes, half_t* __restrict__ C, int64_t M, int64_t N, int64_t ldc, int splits)
+	const float* __restrict__ planes, half_t* __restrict__ C, int64_t M, int64_t N, int64_t ldc, int splits,
+	const half_t* __restrict__ bias, float ep_param)
 {
 	const int64_t chunks = N / 8;
 	const int64_t item = (int64_t)blockIdx.x * 256 + threadIdx.x;
@@ -319,10 +321,25 @@ __global__ __launch_bounds__(256) void gemm_f16_split_merge_kernel(
 #pragma unroll
 	for (int e = 0; e < 4; ++e)
 	{
-		out[e] = (half_t)lo[e];
-		out[4 + e] = (half_t)hi[e];
+		const float bias_lo = (EPI == kEpiBias && bias) ? (float)bias[n + e] : 0.0f;
+		const float bias_hi = (EPI == kEpiBias && bias) ? (float)bias[n + 4 + e] : 0.0f;
+		out[e] = (half_t)finish_sum<EPI, true>(lo[e], 0.0f, bias_lo, ep_param);
+		out[4 + e] = (half_t)finish_sum<EPI, true>(hi[e], 0.0f, bias_hi, ep_param);
 	}
 	*reinterpret_cast<LooseHalf8*>(C + m * ldc + n) = out;      // rows of C may start at any element
+}
+
+static hipError_t launch_split_merge(const float* planes, half_t* c, int64_t M, int64_t N, int64_t ldc, int splits,
+                                     const GemmF16Finish* finish, hipStream_t stream)
+{
+	const int64_t items = M * (N / 8);
+	const dim3 grid((unsigned)((items + 255) / 256));
+	if (finish && finish->epilogue == kEpiSoftcap)
+		gemm_f16_split_merge_kernel<kEpiSoftcap><<<grid, dim3(256), 0, stream>>>(planes, c, M, N, ldc, splits, nullptr, finish->ep_param);
+	else
+		gemm_f16_split_merge_kernel<kEpiBias><<<grid, dim3(256), 0, stream>>>(
+			planes, c, M, N, ldc, splits, finish ? static_cast<const half_t*>(finish->bias) : nullptr, 0.0f);
+	return hipGetLastError();
 }
 
 bool gemm_f16_probe_applies(const void* A, const void* B, const void* C, int64_t M, int64_t N, int64_t K,
@@ -345,9 +362,24 @@ constexpr int64_t kWideMaxRowsF16 = 64;
 hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K,
                            int64_t lda, int64_t ldb, int64_t ldc,
                            int64_t stride_a, int64_t stride_b, int64_t stride_c, int64_t batch,
-                           int b_layout, hipStream_t stream)
+                           int b_layout, hipStream_t stream, GemmF16Finish* finish)
 {
+	if (finish) finish->handled = false;
 	if (M == 0 || N == 0 || batch == 0) return hipSuccess;
+	if (finish && batch != 1) return hipErrorInvalidValue;
+	// (with `finish`: a part of a divided product, with whichever kernel takes it and the epilogue)
+	const auto launch_part = [&](const half_t* a_part, const half_t* b_part, half_t* c_part, int64_t m, int64_t n, int64_t n_first) -> hipError_t
+	{
+		if (!finish) return launch_gemm_f16(a_part, b_part, c_part, m, n, K, lda, ldb, ldc, 0, 0, 0, 1, b_layout, stream);
+		const half_t* bias_part = finish->bias ? static_cast<const half_t*>(finish->bias) + n_first : nullptr;
+		bool supported = false;
+		const hipError_t err = launch_gemm_f16_epilogue(a_part, b_part, nullptr, bias_part, c_part, m, n, K, lda, ldb, ldc, b_layout,
+		                                                finish->epilogue, finish->ep_param, stream, &supported);
+		return err != hipSuccess ? err : supported ? hipSuccess : hipErrorInvalidValue;
+	};
+	const int fin_epi = finish ? finish->epilogue : (int)kEpiBias;
+	const half_t* fin_bias = finish ? static_cast<const half_t*>(finish->bias) : nullptr;
+	const float fin_param = finish ? finish->ep_param : 0.0f;
 	const half_t* a = static_cast<const half_t*>(A);
 	const half_t* b = static_cast<const half_t*>(B);
 	half_t* c = static_cast<half_t*>(C);
@@ -373,7 +405,7 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
 	// K, and the product runs on the copies: 4096 x 4100 . [4096, 4100] weights 270 -> 117 us (vendor 105 - 110).  From
 	// 64 rows on (below that the weights are streamed once anyway and a copy would triple that), for products worth
 	// two more launches, where the workspace holds the copies; otherwise the element-wise kernel at the bottom.
-	if (!tiles_ok && batch == 1 && M >= 64 && (double)M * (double)N * (double)K >= (double)(1 << 27))
+	if (!tiles_ok && !finish && batch == 1 && M >= 64 && (double)M * (double)N * (double)K >= (double)(1 << 27))
 	{
 		const bool k_odd = K % 8 != 0;
 		const bool copy_a = k_odd || reinterpret_cast<uintptr_t>(A) % 16 != 0 || lda % 8 != 0;
@@ -420,16 +452,18 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
 	// few rows against n-contiguous weights with so many columns that they alone fill the chip (the output head): the
 	// band kernel that transposes 8 x 8 blocks of the weights in its registers (2304 x 256000, 16 - 64 rows: the tile kernels
 	// take 234 - 282 us, the vendor library 215 - 230)
-	if (batch == 1 && b_layout == ANYGPU_B_ROW_MAJOR && gemm_band_kn_f16_applies(A, B, C, M, N, K, lda, ldb, ldc))
-		return launch_gemm_band_kn_f16(A, B, C, M, N, K, lda, ldb, ldc, kEpiBias, 0.0f, stream);
+	// (the kernels for few rows and the merges below take the caller's epilogue; that band kernel has no bias form)
+	const auto done = [&](hipError_t err) { if (finish) finish->handled = true; return err; };
+	if (batch == 1 && b_layout == ANYGPU_B_ROW_MAJOR && !(fin_epi == kEpiBias && fin_bias) && gemm_band_kn_f16_applies(A, B, C, M, N, K, lda, ldb, ldc))
+		return done(launch_gemm_band_kn_f16(A, B, C, M, N, K, lda, ldb, ldc, fin_epi, fin_param, stream));
 	// the same for k-contiguous weights, from three rows on (one and two rows: the skinny kernels): whole 128-byte lines
 	// per weight row and load instruction, an exchange between lane pairs in front of the MFMAs
 	if (batch == 1 && b_layout == ANYGPU_B_COL_MAJOR && M >= 3 && gemm_band_kc_wide_applies<half_t>(a, b, c, M, N, K, lda, ldb, ldc, kWideMaxRowsF16))
-		return launch_gemm_band_kc_wide<half_t>(a, b, nullptr, c, M, N, K, lda, ldb, ldc, kEpiBias, 0.0f, stream);
+		return done(launch_gemm_band_kc_wide<half_t>(a, b, fin_bias, c, M, N, K, lda, ldb, ldc, fin_epi, fin_param, stream));
 	if (batch == 1 && !tiles_first && gemm_band_applies<half_t>(a, b, nullptr, c, M, N, K, lda, ldb, ldc, b_layout))
-		return launch_gemm_band<half_t>(a, b, nullptr, nullptr, c, M, N, K, lda, ldb, ldc, 0, 0.0f, stream);
+		return done(launch_gemm_band<half_t>(a, b, nullptr, fin_bias, c, M, N, K, lda, ldb, ldc, fin_epi, fin_param, stream));
 	if (batch == 1 && !tiles_first && gemm_skinny_applies<half_t>(a, b, nullptr, M, N, K, lda, ldb, b_layout))
-		return launch_gemm_skinny<half_t>(a, b, nullptr, nullptr, c, M, N, K, lda, ldb, ldc, b_layout, 0, 0.0f, stream);
+		return done(launch_gemm_skinny<half_t>(a, b, nullptr, fin_bias, c, M, N, K, lda, ldb, ldc, b_layout, fin_epi, fin_param, stream));
 
 	if (tiles_ok)
 	{
@@ -460,9 +494,9 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
 			const double divided_us = estimate_tiles_us(m_body, N, K, cus, whole_tiles, plane_bytes) + estimate_tiles_us(m_tail, N, K, cus, whole_tiles, plane_bytes);
 			if (divided_us < 0.97 * whole_us)
 			{
-				const hipError_t err = launch_gemm_f16(A, B, C, m_body, N, K, lda, ldb, ldc, 0, 0, 0, 1, b_layout, stream);
+				const hipError_t err = launch_part(a, b, c, m_body, N, 0);
 				if (err != hipSuccess) return err;
-				return launch_gemm_f16(a + m_body * lda, B, c + m_body * ldc, m_tail, N, K, lda, ldb, ldc, 0, 0, 0, 1, b_layout, stream);
+				return done(launch_part(a + m_body * lda, b, c + m_body * ldc, m_tail, N, 0));
 			}
 		}
 		const double cost256 = slab_us(256, blocks(256)), cost128 = slab_us(128, blocks(128)), cost64 = slab_us(64, blocks(64));
@@ -486,10 +520,10 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
 				const double divided = (slab_us(256, head_cols * tiles_m) + tail_cost) * slabs + TilePrices::kSplitSetupSlabs;
 				if (divided < 0.93 * cost256 * slabs)
 				{
-					const hipError_t err = launch_gemm_f16(A, B, C, M, n_head, K, lda, ldb, ldc, 0, 0, 0, 1, b_layout, stream);
+					const hipError_t err = launch_part(a, b, c, M, n_head, 0);
 					if (err != hipSuccess) return err;
 					const half_t* b_tail = (b_layout == ANYGPU_B_COL_MAJOR) ? b + n_head * ldb : b + n_head;
-					return launch_gemm_f16(A, b_tail, c + n_head, M, n_tail, K, lda, ldb, ldc, 0, 0, 0, 1, b_layout, stream);
+					return done(launch_part(a, b_tail, c + n_head, M, n_tail, n_head));
 				}
 			}
 		}
@@ -549,7 +583,10 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
 			if (four.kind >= 0 && four.us < plan_us)
 			{
 				if (four.kind == 0)
+				{
+					if (finish) return hipSuccess;
 					return launch_gemm_f16_ring(a, b, c, M, N, K, lda, ldb, ldc, stride_a, stride_b, stride_c, batch, stream, nullptr, b_layout);
+				}
 				float* planes = nullptr;
 				int64_t ranges = four.splits, k_split = 0;
 				if (ranges > 1)
@@ -557,6 +594,7 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
 					k_split = ((K / 64 + ranges - 1) / ranges) * 64;
 					ranges = (K + k_split - 1) / k_split;
 				}
+				if (finish && ranges <= 1) return hipSuccess;
 				if (ranges > 1)
 				{
 					const hipError_t ws_err = band::workspace_acquire(stream, &planes);
@@ -569,9 +607,7 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
 					? launch_gemm_f16_ring3<8, 4>(a, b, c, M, N, K, lda, ldb, ldc, sa, sb, stride_c, count, stream, planes, k_split, nullptr, 0.0f, b_layout)
 					: launch_gemm_f16_ring3<4, 4>(a, b, c, M, N, K, lda, ldb, ldc, sa, sb, stride_c, count, stream, planes, k_split, nullptr, 0.0f, b_layout);
 				if (err != hipSuccess || ranges <= 1) return err;
-				const int64_t items = M * (N / 8);
-				gemm_f16_split_merge_kernel<<<dim3((unsigned)((items + 255) / 256)), dim3(256), 0, stream>>>(planes, c, M, N, ldc, (int)ranges);
-				return hipGetLastError();
+				return done(launch_split_merge(planes, c, M, N, ldc, (int)ranges, finish, stream));
 			}
 		}
 		if (splits > 1)
@@ -611,13 +647,12 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
 				}
 #undef ANYGPU_F16_SPLIT
 				if (err != hipSuccess) return err;
-				const int64_t items = M * (N / 8);
-				gemm_f16_split_merge_kernel<<<dim3((unsigned)((items + 255) / 256)), dim3(256), 0, stream>>>(planes, c, M, N, ldc, (int)splits);
-				return hipGetLastError();
+				return done(launch_split_merge(planes, c, M, N, ldc, (int)splits, finish, stream));
 			}
 		}
 		// unsplit (also where the stream has no workspace to cut into, as under capture): the tile priced for that.
 		// One "general" instantiation serves ragged M / N and a K tail alike.
+		if (finish) return hipSuccess;
 		tile = tile_unsplit;
 		if (rect && blocks_rect / batch <= 0x7FFFFFFFLL)
 		{
@@ -664,6 +699,7 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
 		}
 #undef ANYGPU_F16_TILE
 	}
+	if (finish) return hipSuccess;
 
 	const dim3 grid((unsigned)((N + kEdgeTile - 1) / kEdgeTile), (unsigned)((M + kEdgeTile - 1) / kEdgeTile), (unsigned)batch);
 	discard_stale_error();
@@ -707,12 +743,16 @@ hipError_t launch_gemm_f16_epilogue(const void* A, const void* B, const void* B2
 	const bool aligned = (reinterpret_cast<uintptr_t>(A) % 16 == 0) && (reinterpret_cast<uintptr_t>(B) % 16 == 0) &&
 	                     (!dual || reinterpret_cast<uintptr_t>(B2) % 16 == 0) && (lda % 8 == 0) && (ldb % 8 == 0);
 	const bool tiles_ok = aligned && K >= 64 && K % 8 == 0 && (b_layout == ANYGPU_B_COL_MAJOR || N % 8 == 0);
-	if (epilogue == kEpiSoftcap && b_layout == ANYGPU_B_COL_MAJOR && M >= 3 && gemm_band_kc_wide_applies<half_t>(a, b, c, M, N, K, lda, ldb, ldc, kWideMaxRowsF16))
-		return launch_gemm_band_kc_wide<half_t>(a, b, nullptr, c, M, N, K, lda, ldb, ldc, kEpiSoftcap, ep_param, stream);
-	if (epilogue != kEpiBias && gemm_band_applies<half_t>(a, b, b2, c, M, N, K, lda, ldb, ldc, b_layout))
+	// one product: the few-row kernels and the plans cut along K of the plain product, which take the epilogue along
+	// (8 x 9216 -> 2304 with a bias: 64 us through an uncut tile kernel, the plain product takes 14)
+	if (!dual)
+	{
+		GemmF16Finish finish = {epilogue, bias, ep_param, false};
+		const hipError_t err = launch_gemm_f16(A, B, C, M, N, K, lda, ldb, ldc, 0, 0, 0, 1, b_layout, stream, &finish);
+		if (err != hipSuccess || finish.handled) return err;
+	}
+	if (dual && gemm_band_applies<half_t>(a, b, b2, c, M, N, K, lda, ldb, ldc, b_layout))
 		return launch_gemm_band<half_t>(a, b, b2, nullptr, c, M, N, K, lda, ldb, ldc, epilogue, ep_param, stream);
-	if (epilogue == kEpiSoftcap && b_layout == ANYGPU_B_ROW_MAJOR && gemm_band_kn_f16_applies(A, B, C, M, N, K, lda, ldb, ldc))
-		return launch_gemm_band_kn_f16(A, B, C, M, N, K, lda, ldb, ldc, kEpiSoftcap, ep_param, stream);
 	if (!tiles_ok)
 	{
 		if (dual)

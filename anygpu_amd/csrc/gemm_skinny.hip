@@ -57,7 +57,7 @@ __device__ __forceinline__ float dot_acc(half8_t a, half8_t b, float acc)
 // C[m, n] = finish(sum_k A[m, k] * B[n, k])
 template <typename T, int MROWS, int EPI>
 __global__ __launch_bounds__(256) void gemm_skinny_kcontig_kernel(
-	const T* __restrict__ A, const T* __restrict__ B, const T* __restrict__ B2, const float* __restrict__ bias,
+	const T* __restrict__ A, const T* __restrict__ B, const T* __restrict__ B2, const T* __restrict__ bias,
 	T* __restrict__ C, int M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc, float ep_param)
 {
 	typedef typename Vec16<T>::type vec_t;
@@ -121,7 +121,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_kcontig_kernel(
 			const int64_t n = n0 + c;
 			if (lane == 0 && m < M && n < N)
 			{
-				const float bias_n = (EPI == kEpiBias && bias) ? bias[n] : 0.0f;
+				const float bias_n = (EPI == kEpiBias && bias) ? (float)bias[n] : 0.0f;
 				C[(int64_t)m * ldc + n] = (T)finish_sum<EPI>(sum, sum2, bias_n, ep_param);
 			}
 		}
@@ -133,7 +133,7 @@ constexpr int kSkinnyDepth = 16;           // weight loads in flight per lane
 // C[m, n] = finish(sum_k A[m, k] * B[k, n])
 template <typename T, int MROWS, int EPI>
 __global__ __launch_bounds__(1024) void gemm_skinny_ncontig_kernel(
-	const T* __restrict__ A, const T* __restrict__ B, const T* __restrict__ B2, const float* __restrict__ bias,
+	const T* __restrict__ A, const T* __restrict__ B, const T* __restrict__ B2, const T* __restrict__ bias,
 	T* __restrict__ C, int M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc, float ep_param)
 {
 	typedef typename Vec4B<T>::type vec_t;
@@ -244,14 +244,14 @@ __global__ __launch_bounds__(1024) void gemm_skinny_ncontig_kernel(
 		const int64_t n = n_vec + v;
 		if (m < M && n < N)
 		{
-			const float bias_n = (EPI == kEpiBias && bias) ? bias[n] : 0.0f;
+			const float bias_n = (EPI == kEpiBias && bias) ? (float)bias[n] : 0.0f;
 			C[(int64_t)m * ldc + n] = (T)finish_sum<EPI>(sum, sum2, bias_n, ep_param);
 		}
 	}
 }
 
 template <typename T, int MROWS, int EPI>
-hipError_t launch_rows(const T* A, const T* B, const T* B2, const float* bias, T* C, int M, int64_t N, int64_t K,
+hipError_t launch_rows(const T* A, const T* B, const T* B2, const T* bias, T* C, int M, int64_t N, int64_t K,
                        int64_t lda, int64_t ldb, int64_t ldc, int b_layout, float ep_param, hipStream_t stream)
 {
 	discard_stale_error();
@@ -294,7 +294,7 @@ bool gemm_skinny_applies(const T* A, const T* B, const T* B2, int64_t M, int64_t
 }
 
 template <typename T>
-hipError_t launch_gemm_skinny(const T* A, const T* B, const T* B2, const float* bias, T* C,
+hipError_t launch_gemm_skinny(const T* A, const T* B, const T* B2, const T* bias, T* C,
                               int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc,
                               int b_layout, int epilogue, float ep_param, hipStream_t stream)
 {
@@ -320,7 +320,7 @@ template bool gemm_skinny_applies<float>(const float*, const float*, const float
 template bool gemm_skinny_applies<half_t>(const half_t*, const half_t*, const half_t*, int64_t, int64_t, int64_t, int64_t, int64_t, int);
 template hipError_t launch_gemm_skinny<float>(const float*, const float*, const float*, const float*, float*, int64_t, int64_t, int64_t,
                                               int64_t, int64_t, int64_t, int, int, float, hipStream_t);
-template hipError_t launch_gemm_skinny<half_t>(const half_t*, const half_t*, const half_t*, const float*, half_t*, int64_t, int64_t, int64_t,
+template hipError_t launch_gemm_skinny<half_t>(const half_t*, const half_t*, const half_t*, const half_t*, half_t*, int64_t, int64_t, int64_t,
                                                int64_t, int64_t, int64_t, int, int, float, hipStream_t);
 
 }  // namespace anygpu

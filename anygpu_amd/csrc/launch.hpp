@@ -51,11 +51,23 @@ template <typename T>
 hipError_t launch_gated_rmsnorm(const void* x, const void* z, const void* w, void* y, int64_t rows, int64_t cols,
                                 float eps, int zero_centered, hipStream_t stream);
 
-// `batch` independent products of one shape, operand b of product i at base + i * stride_b (elements)
+// What launch_gemm_f16 does to the sums where its plan has a place for it besides a tile kernel's own epilogue: the
+// few-row kernels and the merge behind a cut along K.  epilogue: kEpiBias (fp16 bias) or kEpiSoftcap.  On return
+// `handled` says whether the product was launched that way; if not, nothing was launched.
+struct GemmF16Finish
+{
+	int epilogue;
+	const void* bias;
+	float ep_param;
+	bool handled;
+};
+
+// `batch` independent products of one shape, operand b of product i at base + i * stride_b (elements).  `finish`
+// (batch 1 only): see GemmF16Finish.
 hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K,
                            int64_t lda, int64_t ldb, int64_t ldc,
                            int64_t stride_a, int64_t stride_b, int64_t stride_c, int64_t batch,
-                           int b_layout, hipStream_t stream);
+                           int b_layout, hipStream_t stream, GemmF16Finish* finish = nullptr);
 
 // The fp16 product with an epilogue (gemm_epilogue.hpp: kEpiBias with an fp16 bias, kEpiSoftcap, kEpiGeluMul with B2);
 // *supported = false and nothing launched for the few shapes no kernel with that epilogue takes.
@@ -83,7 +95,7 @@ template <typename T>
 bool gemm_band_kc_wide_applies(const T* A, const T* B, const T* C, int64_t M, int64_t N, int64_t K,
                                int64_t lda, int64_t ldb, int64_t ldc, int64_t max_rows);
 template <typename T>
-hipError_t launch_gemm_band_kc_wide(const T* A, const T* B, const float* bias, T* C, int64_t M, int64_t N, int64_t K,
+hipError_t launch_gemm_band_kc_wide(const T* A, const T* B, const T* bias, T* C, int64_t M, int64_t N, int64_t K,
                                     int64_t lda, int64_t ldb, int64_t ldc, int epilogue, float ep_param, hipStream_t stream);
 
 // dst[i] = src[i] over nvec 16-byte vectors in the stated launch geometry (stream_probe.hip)
@@ -155,7 +167,7 @@ bool gemm_skinny_applies(const T* A, const T* B, const T* B2, int64_t M, int64_t
                          int64_t lda, int64_t ldb, int b_layout);
 
 template <typename T>
-hipError_t launch_gemm_skinny(const T* A, const T* B, const T* B2, const float* bias, T* C,
+hipError_t launch_gemm_skinny(const T* A, const T* B, const T* B2, const T* bias, T* C,
                               int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc,
                               int b_layout, int epilogue, float ep_param, hipStream_t stream);
 
@@ -174,7 +186,7 @@ bool gemm_band_applies(const T* A, const T* B, const T* B2, const T* C, int64_t 
                        int64_t lda, int64_t ldb, int64_t ldc, int b_layout);
 
 template <typename T>
-hipError_t launch_gemm_band(const T* A, const T* B, const T* B2, const float* bias, T* C,
+hipError_t launch_gemm_band(const T* A, const T* B, const T* B2, const T* bias, T* C,
                             int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc,
                             int epilogue, float ep_param, hipStream_t stream);
 

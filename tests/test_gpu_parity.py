@@ -1311,6 +1311,9 @@ F16_EPILOGUE_SHAPES = [
     (1024, 512, 2048), (2048, 192, 4096), (2304, 136, 4104),
     # k-contiguous weights in whole slabs: the four-wave kernels (128 x 128, 256 x 128 and 256 x 256 tiles, whole and ragged)
     (2048, 256, 2048), (2048, 128, 4096), (4096, 128, 4096), (1000, 192, 3000), (3000, 64, 4104),
+    # few rows against a deep K (the plans cut along K, whose merge applies the epilogue), two rows (skinny kernels), so many
+    # columns that the wide band kernel takes them, rows and columns a little past whole tiles (divided products)
+    (8, 9216, 2304), (2, 4096, 2304), (5, 512, 131072), (48, 4096, 4096), (130, 4096, 2304), (300, 2048, 8192), (2048, 256, 10240),
 ]
 
 
