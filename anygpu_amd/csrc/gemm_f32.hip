@@ -699,11 +699,85 @@ hipError_t launch_gemm_f32_softcap(const float* A, const float* B, float* C, int
 	                                                                         0, 0, 0, 1, softcap, stream);
 }
 
+// C[m, n] = gelu_tanh(gate[m, n]) * up[m, n] from two [M, N] planes of sums; VEC: four columns per thread (N a multiple
+// of 4, rows of C 16-byte aligned)
+template <bool VEC>
+__global__ __launch_bounds__(256) void gelu_mul_planes_kernel(const float* __restrict__ gate, const float* __restrict__ up,
+                                                              float* __restrict__ C, int64_t M, int64_t N, int64_t ldc)
+{
+	constexpr int kPer = VEC ? 4 : 1;
+	const int64_t per_row = N / kPer;
+	const int64_t item = (int64_t)blockIdx.x * 256 + threadIdx.x;
+	if (item >= M * per_row) return;
+	const int64_t m = item / per_row, n = (item % per_row) * kPer;
+	if constexpr (VEC)
+	{
+		const float4_t g = *reinterpret_cast<const float4_t*>(gate + m * N + n);
+		const float4_t u = *reinterpret_cast<const float4_t*>(up + m * N + n);
+		float4_t out;
+#pragma unroll
+		for (int e = 0; e < 4; ++e) out[e] = finish_sum<kEpiGeluMul>(g[e], u[e], 0.0f, 0.0f);
+		*reinterpret_cast<float4_t*>(C + m * ldc + n) = out;
+	}
+	else
+		C[m * ldc + n] = finish_sum<kEpiGeluMul>(gate[m * N + n], up[m * N + n], 0.0f, 0.0f);
+}
+
+// rows from which the fused up-projection may run as two plain products and a pass that combines them (below, the band
+// kernels stream both weight matrices in one launch)
+constexpr int64_t kTwoProductsMinRows = 33;
+
 hipError_t launch_gemm_f32_gelu_mul(const float* A, const float* B_gate, const float* B_up, float* C,
                                     int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc,
                                     int b_layout, hipStream_t stream)
 {
 	if (M == 0 || N == 0) return hipSuccess;
+	// The plain product has more kernels to choose from (64-row tiles, cuts along K, divided products) than there are
+	// forms with this epilogue, whose one four-wave kernel has 128-row tiles of 64 output columns: 40 rows of
+	// 2304 -> 9216 took 133 us fused (144 blocks) and take 65 as two products into planes of the stream's workspace and a
+	// pass over the planes that combines them; 300 rows 264 -> 217; 512 rows 393 -> 330 (2.25 rounds of blocks fused).
+	// Where the fused kernel's blocks come out in whole rounds it stays ahead (384 rows: 261 against 278).  Priced with
+	// the plans of the plain product.  Weights stored [K, N] have no four-wave form with this epilogue and run as two
+	// products from the same row count on once they are large (1000 x 2304 -> 9216: 991 -> 695 us; 1024 -> 4096 stays).
+	bool two_products = false;
+	if (M >= kTwoProductsMinRows && K >= 256)
+	{
+		const bool fused_ring = b_layout == ANYGPU_B_COL_MAJOR && reinterpret_cast<uintptr_t>(B_up) % 16 == 0 &&
+		                        gemm_f32_ring_applies(A, B_gate, M, N, K, lda, ldb, 0, 0, 1, 0, 64);
+		if (M <= 200 || (!fused_ring && (double)K * (double)N >= 8.0e6)) two_products = true;
+		else if (fused_ring)
+		{
+			const int64_t cus = chip_cus();
+			const double slabs = (double)((K + kBK - 1) / kBK);
+			const double fused_us = (double)((((M + 127) / 128) * ((N + 63) / 64) + cus - 1) / cus) * slabs * 0.9 + 6.0;
+			const size_t ws_bytes = band::workspace_capacity(stream);
+			const double plain_us = std::min(plan_tiles(128, M, N, K, 1, true, ws_bytes, true).cost, plan_tiles(64, M, N, K, 1, true, ws_bytes, true).cost) + 6.0;
+			const double combine_us = 4.5 + 12.0 * (double)M * (double)N / 5.0e6;
+			two_products = 2.0 * plain_us + combine_us < 0.97 * fused_us;
+		}
+	}
+	if (two_products)
+	{
+		const size_t bytes = ((size_t)2 * M * N * sizeof(float) + 255) / 256 * 256;
+		if (bytes <= band::workspace_copy_capacity(stream))
+		{
+			float* planes = nullptr;
+			hipError_t err = band::workspace_acquire(stream, &planes, bytes);
+			if (err != hipSuccess) return err;
+			const band::WorkspaceReserve keep(bytes);
+			float* up = planes + M * N;
+			err = launch_gemm_f32(A, B_gate, nullptr, planes, M, N, K, lda, ldb, N, 0, 0, 0, 1, ANYGPU_A_ROW_MAJOR, b_layout, stream);
+			if (err != hipSuccess) return err;
+			err = launch_gemm_f32(A, B_up, nullptr, up, M, N, K, lda, ldb, N, 0, 0, 0, 1, ANYGPU_A_ROW_MAJOR, b_layout, stream);
+			if (err != hipSuccess) return err;
+			const bool vec = N % 4 == 0 && ldc % 4 == 0 && reinterpret_cast<uintptr_t>(C) % 16 == 0;
+			const int64_t items = vec ? M * (N / 4) : M * N;
+			const dim3 grid((unsigned)((items + 255) / 256));
+			if (vec) gelu_mul_planes_kernel<true><<<grid, dim3(256), 0, stream>>>(planes, up, C, M, N, ldc);
+			else gelu_mul_planes_kernel<false><<<grid, dim3(256), 0, stream>>>(planes, up, C, M, N, ldc);
+			return hipGetLastError();
+		}
+	}
 	if (gemm_band_applies<float>(A, B_gate, B_up, C, M, N, K, lda, ldb, ldc, b_layout))
 		return launch_gemm_band<float>(A, B_gate, B_up, nullptr, C, M, N, K, lda, ldb, ldc, kEpiGeluMul, 0.0f, stream);
 	if (b_layout == ANYGPU_B_ROW_MAJOR && gemm_band_ncontig_applies(A, B_gate, B_up, C, M, N, K, lda, ldb, ldc, true))

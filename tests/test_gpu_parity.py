@@ -1488,7 +1488,9 @@ def test_gemma_linear_softcap_gemma2_hidden_2304_vocab_slice(ops, oracle):
 
 
 @pytest.mark.parametrize("b,s,hsize,isize", [(1, 1, 1, 1), (1, 37, 288, 1152), (1, 9, 2304, 1156), (2, 16, 520, 9216), (2, 5, 64, 37), (1, 128, 256, 512),
-                                             (3, 50, 130, 259), (1, 256, 512, 2048), (3, 50, 132, 260)])
+                                             (3, 50, 130, 259), (1, 256, 512, 2048), (3, 50, 132, 260),
+                                             # 33 rows and more: two plain products and a combining pass (odd columns; large weights)
+                                             (1, 70, 256, 259), (1, 33, 260, 512), (1, 300, 1024, 8192)])
 def test_gemma_mlp_fused_upproj_shapes(ops, oracle, b, s, hsize, isize):
     x = synth.normal(b * s + hsize, (b, s, hsize))
     wg = synth.normal(isize + 1, (hsize, isize)) * np.float32(1.5 / math.sqrt(hsize))
@@ -1522,7 +1524,9 @@ def test_gemma_mlp_fused_upproj_gemma2_2304_9216(ops, oracle):
     assert scaled_rel_err(got.reshape(s, isize), chain, 1.0) <= TOL_F32
 
 
-@pytest.mark.parametrize("m,hsize,isize", [(3, 288, 1152), (12, 288, 1152), (32, 2304, 516), (17, 64, 40), (64, 4608, 300), (37, 2304, 9216)])
+@pytest.mark.parametrize("m,hsize,isize", [(3, 288, 1152), (12, 288, 1152), (32, 2304, 516), (17, 64, 40), (64, 4608, 300), (37, 2304, 9216),
+                                           # two products (priced) / the fused four-wave kernel in whole rounds / ragged columns
+                                           (100, 512, 1030), (300, 2304, 9216), (384, 2304, 9216)])
 def test_gemm_gelu_mul_k_contiguous_weights(ops, oracle, m, hsize, isize):
     # the fused up-projection with the weights stored [intermediate, hidden], through the C entry point
     import torch
