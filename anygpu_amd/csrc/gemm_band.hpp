@@ -11,7 +11,7 @@ namespace band {
 
 constexpr int kBandThreads = 256;
 constexpr int kBandMaxSplits = 32;
-constexpr int64_t kBandEnoughBlocks = 256;        // tiles from which K is not split
+constexpr int64_t kBandEnoughBlocks = 256;        // tiles from which K is not split (but see plan_band_splits)
 constexpr int64_t kBandWantedBlocks = 512;
 // Workspace of a (device, stream) pair.  The cut along K of the tile kernels prices the traffic of its fp32 planes and
 // uses all of it (2048 x 14336 . 14336 x 4096 fp16: two planes of 32 MB, 244 -> 184 us); the band kernels keep their
@@ -119,8 +119,13 @@ inline hipError_t plan_band_splits(int64_t tiles, int64_t K, int64_t chunk, int6
 {
 	const int64_t kchunks = (K + chunk - 1) / chunk;
 	int64_t splits = 1;
-	const size_t capacity = tiles < kBandEnoughBlocks ? workspace_capacity(stream) : 0;
-	if (tiles < kBandEnoughBlocks && capacity > 0)
+	// (a few more tiles than CUs, up to 1.4 per CU: most CUs would idle while the rest work on their second tile, and two
+	// ranges of K fill the chip better, 16 x 4608 -> 36864 fp32, 288 tiles: 167 -> 141 us; from there on the merge launch
+	// costs what the balance gains, 16 x 1024 -> 50272, 393 tiles: 37 -> 42)
+	const int64_t cus = device_cu_count();
+	const bool cut = tiles < kBandEnoughBlocks || (tiles < 2 * kBandEnoughBlocks && tiles * 10 < ((tiles + cus - 1) / cus) * cus * 7);
+	const size_t capacity = cut ? workspace_capacity(stream) : 0;
+	if (cut && capacity > 0)
 	{
 		splits = (kBandWantedBlocks + tiles - 1) / tiles;
 		if (splits > kBandMaxSplits) splits = kBandMaxSplits;

@@ -49,11 +49,21 @@ __device__ __forceinline__ int4v from_partner(const int4v& v)
 }
 
 // MB: row blocks of 16 (M <= 16 MB).  EPI: kEpiBias (+ bias[n] when bias != NULL) or kEpiSoftcap.
-template <typename T, int MB, int EPI>
+// PARTIAL: blockIdx.y walks ranges of k_split elements of K (whole LDS chunks) and the raw fp32 sums of range y go to
+// plane y ([M, N] floats) of `partial`; the merge kernel below adds the planes and applies the epilogue.
+template <typename T, int MB, int EPI, bool PARTIAL>
 __global__ __launch_bounds__(kBandThreads) void gemm_band_kc_wide_kernel(
 	const T* __restrict__ A, const T* __restrict__ B, const T* __restrict__ bias, T* __restrict__ C,
-	int M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc, float ep_param)
+	int M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc, float ep_param,
+	float* __restrict__ partial, int64_t k_split)
 {
+	if constexpr (PARTIAL)
+	{
+		const int64_t k_begin = (int64_t)blockIdx.y * k_split;
+		A += k_begin;
+		B += k_begin;
+		K = K - k_begin < k_split ? K - k_begin : k_split;
+	}
 	constexpr int EPC = 16 / (int)sizeof(T);                       // elements per 16-byte chunk
 	constexpr int kStep = kWideStepBytes / (int)sizeof(T);         // k per step
 	constexpr int kChunk = kStep * kWideStepsPerChunk;             // k per LDS chunk of the band
@@ -169,7 +179,7 @@ __global__ __launch_bounds__(kBandThreads) void gemm_band_kc_wide_kernel(
 	// their weight rows at any one time (with rows a power of two apart, equal offsets in all rows are addresses that
 	// share their low bits, and with them the memory channel).  Whole chunks only: with a half chunk at the end of K the
 	// order stays 0, 1, 2, ...
-	const int64_t first = steps % kWideStepsPerChunk == 0 ? (int64_t)((blockIdx.x * 2654435761u) >> 8) % chunks : 0;
+	const int64_t first = steps % kWideStepsPerChunk == 0 ? (int64_t)(((blockIdx.x + 977u * blockIdx.y) * 2654435761u) >> 8) % chunks : 0;
 	auto chunk_at = [&](int64_t i) { const int64_t c = i + first; return c >= chunks ? c - chunks : c; };   // i <= chunks
 	auto step_at = [&](int64_t i) { const int64_t t = i + first * kWideStepsPerChunk; return t >= steps ? t - steps : t; };
 	issue_band(chunk_at(0));
@@ -222,6 +232,11 @@ __global__ __launch_bounds__(kBandThreads) void gemm_band_kc_wide_kernel(
 		{
 			const int64_t n = n0 + 16 * t + 4 * grp;
 			if (n + 4 > N) continue;
+			if constexpr (PARTIAL)
+			{
+				*reinterpret_cast<float4_t*>(partial + ((int64_t)blockIdx.y * M + m) * N + n) = acc[t][b];
+				continue;
+			}
 			OutVec out;
 #pragma unroll
 			for (int r = 0; r < 4; ++r)
@@ -234,17 +249,107 @@ __global__ __launch_bounds__(kBandThreads) void gemm_band_kc_wide_kernel(
 	}
 }
 
+// C[m, n .. n + 3] = finish(sum over the planes, in order), one thread per four columns
+template <typename T, int EPI>
+__global__ __launch_bounds__(256) void gemm_band_kc_wide_merge_kernel(
+	const float* __restrict__ partial, const T* __restrict__ bias, T* __restrict__ C, int M, int64_t N, int64_t ldc,
+	int splits, float ep_param)
+{
+	const int64_t per_row = N / 4;
+	const int64_t item = (int64_t)blockIdx.x * 256 + threadIdx.x;
+	if (item >= (int64_t)M * per_row) return;
+	const int64_t m = item / per_row, n = (item % per_row) * 4;
+	const float* src = partial + m * N + n;
+	const int64_t plane = (int64_t)M * N;
+	float4_t sum = {0.0f, 0.0f, 0.0f, 0.0f};
+	int sp = 0;
+	for (; sp + 4 <= splits; sp += 4)
+	{
+		float4_t v[4];
+#pragma unroll
+		for (int i = 0; i < 4; ++i) v[i] = *reinterpret_cast<const float4_t*>(src + (sp + i) * plane);
+#pragma unroll
+		for (int i = 0; i < 4; ++i) sum += v[i];
+	}
+	for (; sp < splits; ++sp) sum += *reinterpret_cast<const float4_t*>(src + sp * plane);
+	typedef T OutVec __attribute__((ext_vector_type(4)));
+	OutVec out;
+#pragma unroll
+	for (int r = 0; r < 4; ++r)
+	{
+		const float bias_n = (EPI == kEpiBias && bias) ? (float)bias[n + r] : 0.0f;
+		out[r] = (T)finish_sum<EPI, sizeof(T) == 2>(sum[r], 0.0f, bias_n, ep_param);
+	}
+	*reinterpret_cast<OutVec*>(C + m * ldc + n) = out;
+}
+
+// How a product whose columns alone do not fill the chip is cut along K: ranges of whole LDS chunks, as few as give
+// every CU (nearly) two blocks with no more than 15 % of the CUs idle in the last round, every range at least
+// kWideMinChunks chunks deep (16 x 3584 -> 18944 fp32 in ten ranges of six chunks: 58 us, the other band kernel 51),
+// the planes within `room` bytes.  0: no such cut.  17 - 32 rows (where the matrix cores' time comes close to the
+// memory's in fp32 and the other band kernel is as fast on most shapes) only in three ranges or more.
+constexpr int64_t kWideMinChunks = 12;
+template <typename T>
+int64_t wide_split_chunks(int64_t M, int64_t N, int64_t K, size_t room)
+{
+	constexpr int kChunk = kWideChunkBytes / (int)sizeof(T);
+	const int64_t chunks = (K + kChunk - 1) / kChunk;
+	const int64_t blocks = (N + kWideBlockCols - 1) / kWideBlockCols;
+	const int64_t cus = device_cu_count();
+	for (int64_t s = 2; s <= 16; ++s)
+	{
+		const int64_t per = (chunks + s - 1) / s;
+		if (per < kWideMinChunks) break;
+		const int64_t ranges = (chunks + per - 1) / per;
+		if ((size_t)ranges * (size_t)M * (size_t)N * sizeof(float) > room) break;
+		const int64_t total = blocks * ranges, rounds = (total + cus - 1) / cus;
+		if (total * 20 < cus * 38 || total * 100 < rounds * cus * 85) continue;
+		if (M > 16 && M <= 32 && ranges < 3) return 0;
+		return per;
+	}
+	return 0;
+}
+
 template <typename T, int MB>
 hipError_t launch_rows(const T* A, const T* B, const T* bias, T* C, int M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
-                       int64_t ldc, int epilogue, float ep_param, hipStream_t stream)
+                       int64_t ldc, int epilogue, float ep_param, hipStream_t stream, int64_t split_chunks)
 {
-	const dim3 grid((unsigned)((N + kWideBlockCols - 1) / kWideBlockCols));
+	const unsigned blocks = (unsigned)((N + kWideBlockCols - 1) / kWideBlockCols);
 	discard_stale_error();
+	if (split_chunks > 0)
+	{
+		constexpr int kChunk = kWideChunkBytes / (int)sizeof(T);
+		const int64_t k_split = split_chunks * kChunk;
+		const int ranges = (int)((K + k_split - 1) / k_split);
+		float* partial = nullptr;
+		const hipError_t err = workspace_acquire(stream, &partial);
+		if (err != hipSuccess) return err;
+		gemm_band_kc_wide_kernel<T, MB, kEpiBias, true><<<dim3(blocks, (unsigned)ranges), dim3(kBandThreads), 0, stream>>>(
+			A, B, nullptr, C, M, N, K, lda, ldb, ldc, 0.0f, partial, k_split);
+		const dim3 grid((unsigned)(((int64_t)M * (N / 4) + 255) / 256));
+		if (epilogue == kEpiSoftcap)
+			gemm_band_kc_wide_merge_kernel<T, kEpiSoftcap><<<grid, dim3(256), 0, stream>>>(partial, bias, C, M, N, ldc, ranges, ep_param);
+		else
+			gemm_band_kc_wide_merge_kernel<T, kEpiBias><<<grid, dim3(256), 0, stream>>>(partial, bias, C, M, N, ldc, ranges, ep_param);
+		return hipGetLastError();
+	}
 	if (epilogue == kEpiSoftcap)
-		gemm_band_kc_wide_kernel<T, MB, kEpiSoftcap><<<grid, dim3(kBandThreads), 0, stream>>>(A, B, bias, C, M, N, K, lda, ldb, ldc, ep_param);
+		gemm_band_kc_wide_kernel<T, MB, kEpiSoftcap, false><<<dim3(blocks), dim3(kBandThreads), 0, stream>>>(A, B, bias, C, M, N, K, lda, ldb, ldc, ep_param, nullptr, 0);
 	else
-		gemm_band_kc_wide_kernel<T, MB, kEpiBias><<<grid, dim3(kBandThreads), 0, stream>>>(A, B, bias, C, M, N, K, lda, ldb, ldc, ep_param);
+		gemm_band_kc_wide_kernel<T, MB, kEpiBias, false><<<dim3(blocks), dim3(kBandThreads), 0, stream>>>(A, B, bias, C, M, N, K, lda, ldb, ldc, ep_param, nullptr, 0);
 	return hipGetLastError();
+}
+
+// what both forms assume of the operands
+template <typename T>
+bool wide_operands_ok(const T* A, const T* B, const T* C, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc, int64_t max_rows)
+{
+	constexpr int EPC = 16 / (int)sizeof(T);
+	constexpr int kStep = kWideStepBytes / (int)sizeof(T);
+	if (M < 1 || M > max_rows || M > 64 || K < kStep || K % kStep != 0 || N % 4 != 0) return false;
+	if ((N + kWideBlockCols - 1) / kWideBlockCols > 0x7FFFFFFFLL) return false;
+	return lda % EPC == 0 && ldb % EPC == 0 && ldc % 4 == 0 && aligned16(A) && aligned16(B) &&
+	       reinterpret_cast<uintptr_t>(C) % (4 * sizeof(T)) == 0;
 }
 
 }  // namespace
@@ -257,29 +362,38 @@ template <typename T>
 bool gemm_band_kc_wide_applies(const T* A, const T* B, const T* C, int64_t M, int64_t N, int64_t K,
                                int64_t lda, int64_t ldb, int64_t ldc, int64_t max_rows)
 {
-	constexpr int EPC = 16 / (int)sizeof(T);
-	constexpr int kStep = kWideStepBytes / (int)sizeof(T);
-	if (M < 1 || M > max_rows || M > 64 || K < kStep || K % kStep != 0 || N % 4 != 0) return false;
+	if (!wide_operands_ok(A, B, C, M, N, K, lda, ldb, ldc, max_rows)) return false;
 	const int64_t blocks = (N + kWideBlockCols - 1) / kWideBlockCols;
 	const int64_t cus = device_cu_count();
 	const int64_t rounds = (blocks + cus - 1) / cus;
-	if (cus <= 0 || blocks * 20 < cus * 38 || blocks * 100 < rounds * cus * 85 || blocks > 0x7FFFFFFFLL) return false;
-	return lda % EPC == 0 && ldb % EPC == 0 && ldc % 4 == 0 && aligned16(A) && aligned16(B) &&
-	       reinterpret_cast<uintptr_t>(C) % (4 * sizeof(T)) == 0;
+	return cus > 0 && blocks * 20 >= cus * 38 && blocks * 100 >= rounds * cus * 85;
+}
+
+// The same with fewer columns, where a cut along K brings the block count there (see wide_split_chunks)
+template <typename T>
+bool gemm_band_kc_wide_split_applies(const T* A, const T* B, const T* C, int64_t M, int64_t N, int64_t K,
+                                     int64_t lda, int64_t ldb, int64_t ldc, int64_t max_rows, hipStream_t stream)
+{
+	if (!wide_operands_ok(A, B, C, M, N, K, lda, ldb, ldc, max_rows)) return false;
+	if (gemm_band_kc_wide_applies(A, B, C, M, N, K, lda, ldb, ldc, max_rows)) return false;
+	return wide_split_chunks<T>(M, N, K, workspace_capacity(stream)) > 0;
 }
 
 template <typename T>
 hipError_t launch_gemm_band_kc_wide(const T* A, const T* B, const T* bias, T* C, int64_t M, int64_t N, int64_t K,
                                     int64_t lda, int64_t ldb, int64_t ldc, int epilogue, float ep_param, hipStream_t stream)
 {
-	if (M <= 16) return launch_rows<T, 1>(A, B, bias, C, (int)M, N, K, lda, ldb, ldc, epilogue, ep_param, stream);
-	if (M <= 32) return launch_rows<T, 2>(A, B, bias, C, (int)M, N, K, lda, ldb, ldc, epilogue, ep_param, stream);
-	if (M <= 48) return launch_rows<T, 3>(A, B, bias, C, (int)M, N, K, lda, ldb, ldc, epilogue, ep_param, stream);
-	return launch_rows<T, 4>(A, B, bias, C, (int)M, N, K, lda, ldb, ldc, epilogue, ep_param, stream);
+	const int64_t split_chunks = gemm_band_kc_wide_applies(A, B, C, M, N, K, lda, ldb, ldc, 64) ? 0 : wide_split_chunks<T>(M, N, K, workspace_capacity(stream));
+	if (M <= 16) return launch_rows<T, 1>(A, B, bias, C, (int)M, N, K, lda, ldb, ldc, epilogue, ep_param, stream, split_chunks);
+	if (M <= 32) return launch_rows<T, 2>(A, B, bias, C, (int)M, N, K, lda, ldb, ldc, epilogue, ep_param, stream, split_chunks);
+	if (M <= 48) return launch_rows<T, 3>(A, B, bias, C, (int)M, N, K, lda, ldb, ldc, epilogue, ep_param, stream, split_chunks);
+	return launch_rows<T, 4>(A, B, bias, C, (int)M, N, K, lda, ldb, ldc, epilogue, ep_param, stream, split_chunks);
 }
 
 template bool gemm_band_kc_wide_applies<float>(const float*, const float*, const float*, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t);
 template bool gemm_band_kc_wide_applies<half_t>(const half_t*, const half_t*, const half_t*, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t);
+template bool gemm_band_kc_wide_split_applies<float>(const float*, const float*, const float*, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, hipStream_t);
+template bool gemm_band_kc_wide_split_applies<half_t>(const half_t*, const half_t*, const half_t*, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, hipStream_t);
 template hipError_t launch_gemm_band_kc_wide<float>(const float*, const float*, const float*, float*, int64_t, int64_t, int64_t,
                                                     int64_t, int64_t, int64_t, int, float, hipStream_t);
 template hipError_t launch_gemm_band_kc_wide<half_t>(const half_t*, const half_t*, const half_t*, half_t*, int64_t, int64_t, int64_t,

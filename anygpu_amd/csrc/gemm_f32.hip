@@ -564,6 +564,9 @@ static hipError_t launch_layout(const float* A, const float* B, const float* B2,
 // along K is as fast) the wide band kernel takes fp32 output heads
 constexpr int64_t kWideMinRowsF32 = 3;
 constexpr int64_t kWideMaxRowsF32 = 48;
+// (and with fewer columns where a cut along K fills the chip: 16 x 4096 -> 32000 106 -> 85 us, 16 x 4608 -> 36864 167 -> 120,
+// 48 x 5120 -> 65536 367 -> 330)
+constexpr int64_t kWideSplitMaxRowsF32 = 48;
 
 hipError_t launch_gemm_f32(const float* A, const float* B, const float* bias, float* C,
                            int64_t M, int64_t N, int64_t K,
@@ -661,6 +664,9 @@ hipError_t launch_gemm_f32(const float* A, const float* B, const float* bias, fl
 	if (batch == 1 && a_layout == ANYGPU_A_ROW_MAJOR && b_layout == ANYGPU_B_COL_MAJOR && M >= kWideMinRowsF32 &&
 	    gemm_band_kc_wide_applies<float>(A, B, C, M, N, K, lda, ldb, ldc, kWideMaxRowsF32))
 		return launch_gemm_band_kc_wide<float>(A, B, bias, C, M, N, K, lda, ldb, ldc, kEpiBias, 0.0f, stream);
+	if (batch == 1 && a_layout == ANYGPU_A_ROW_MAJOR && b_layout == ANYGPU_B_COL_MAJOR && M >= kWideMinRowsF32 &&
+	    gemm_band_kc_wide_split_applies<float>(A, B, C, M, N, K, lda, ldb, ldc, kWideSplitMaxRowsF32, stream))
+		return launch_gemm_band_kc_wide<float>(A, B, bias, C, M, N, K, lda, ldb, ldc, kEpiBias, 0.0f, stream);
 	if (batch == 1 && !tiles_first && a_layout == ANYGPU_A_ROW_MAJOR && gemm_band_applies<float>(A, B, nullptr, C, M, N, K, lda, ldb, ldc, b_layout))
 		return launch_gemm_band<float>(A, B, nullptr, bias, C, M, N, K, lda, ldb, ldc, kEpiBias, 0.0f, stream);
 	if (batch == 1 && !tiles_first && a_layout == ANYGPU_A_ROW_MAJOR && b_layout == ANYGPU_B_ROW_MAJOR &&
@@ -685,6 +691,8 @@ hipError_t launch_gemm_f32_softcap(const float* A, const float* B, float* C, int
 {
 	if (M == 0 || N == 0) return hipSuccess;
 	if (b_layout == ANYGPU_B_COL_MAJOR && M >= kWideMinRowsF32 && gemm_band_kc_wide_applies<float>(A, B, C, M, N, K, lda, ldb, ldc, kWideMaxRowsF32))
+		return launch_gemm_band_kc_wide<float>(A, B, nullptr, C, M, N, K, lda, ldb, ldc, kEpiSoftcap, softcap, stream);
+	if (b_layout == ANYGPU_B_COL_MAJOR && M >= kWideMinRowsF32 && gemm_band_kc_wide_split_applies<float>(A, B, C, M, N, K, lda, ldb, ldc, kWideSplitMaxRowsF32, stream))
 		return launch_gemm_band_kc_wide<float>(A, B, nullptr, C, M, N, K, lda, ldb, ldc, kEpiSoftcap, softcap, stream);
 	if (gemm_band_applies<float>(A, B, nullptr, C, M, N, K, lda, ldb, ldc, b_layout))
 		return launch_gemm_band<float>(A, B, nullptr, nullptr, C, M, N, K, lda, ldb, ldc, kEpiSoftcap, softcap, stream);

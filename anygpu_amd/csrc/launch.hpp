@@ -94,6 +94,10 @@ hipError_t launch_gemm_band_kn_f16(const void* A, const void* B, void* C, int64_
 template <typename T>
 bool gemm_band_kc_wide_applies(const T* A, const T* B, const T* C, int64_t M, int64_t N, int64_t K,
                                int64_t lda, int64_t ldb, int64_t ldc, int64_t max_rows);
+// (fewer columns, with the cut along K that then fills the chip; planes in the stream's workspace)
+template <typename T>
+bool gemm_band_kc_wide_split_applies(const T* A, const T* B, const T* C, int64_t M, int64_t N, int64_t K,
+                                     int64_t lda, int64_t ldb, int64_t ldc, int64_t max_rows, hipStream_t stream);
 template <typename T>
 hipError_t launch_gemm_band_kc_wide(const T* A, const T* B, const T* bias, T* C, int64_t M, int64_t N, int64_t K,
                                     int64_t lda, int64_t ldb, int64_t ldc, int epilogue, float ep_param, hipStream_t stream);

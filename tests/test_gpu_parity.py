@@ -1055,7 +1055,9 @@ def test_mm_f16_row_bands_n_contiguous_weights_many_columns(ops, oracle, m, k, n
 @pytest.mark.parametrize("dtype", ["f16", "f32"])
 @pytest.mark.parametrize("m,steps,n", [(3, 1, 131072), (5, 2, 125000), (8, 3, 131068), (16, 4, 196608), (13, 5, 124672),
                                        (17, 6, 131072), (32, 2, 125000), (9, 8, 262144), (40, 2, 131072), (48, 3, 125000),
-                                       (64, 2, 131072)])
+                                       (64, 2, 131072),
+                                       # fewer columns and a deep K: the same kernel over ranges of K, planes and a merge (fp32)
+                                       (16, 128, 32000), (24, 128, 32000), (5, 96, 32004), (40, 144, 36864)])
 def test_mm_row_bands_k_contiguous_weights_many_columns(ops, oracle, dtype, m, steps, n):
     # few rows against [N, K] weights with the columns of an output head: the band kernel that loads whole 128-byte
     # lines per weight row and lets lane pairs exchange halves, blocks starting at different chunks of K (an odd number
@@ -1096,7 +1098,9 @@ def test_mm_row_bands_k_contiguous_weights_many_columns(ops, oracle, dtype, m, s
     name = "anygpu_gemm_f16_f32acc_softcap" if half else "anygpu_gemm_f32_softcap"
     capi.check(name, getattr(lib, name)(dau.data_ptr(), dwu.data_ptr(), out.data_ptr(), m, n, k, k, k, n, capi.B_COL_MAJOR, 2.0, stream))
     capped = oracle.softcap(ref, 2.0).reshape(m, n)
-    assert scaled_rel_err(host(out).astype(np.float32), capped, 2.0 / 3.0) <= tol
+    # (the cap's slope is at most 1: a capped sum is off by no more than the sum, whose error grows with sqrt(k); the
+    # outputs themselves stay within the cap)
+    assert scaled_rel_err(host(out).astype(np.float32), capped, 2.0 / 3.0 if k <= 512 else 2.0) <= tol
     if not half:
         bias = synth.uniform(n + 25, (n,))
         dbias = dev(bias)
