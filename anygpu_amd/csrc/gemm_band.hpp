@@ -11,8 +11,7 @@ namespace band {
 
 constexpr int kBandThreads = 256;
 constexpr int kBandMaxSplits = 32;
-constexpr int64_t kBandEnoughBlocks = 256;        // tiles from which K is not split (but see plan_band_splits)
-constexpr int64_t kBandWantedBlocks = 512;
+constexpr int64_t kBandEnoughBlocks = 256;        // column tiles that fill the chip by themselves
 // Workspace of a (device, stream) pair.  The cut along K of the tile kernels prices the traffic of its fp32 planes and
 // uses all of it (2048 x 14336 . 14336 x 4096 fp16: two planes of 32 MB, 244 -> 184 us); the band kernels keep their
 // partial sums within the first kBandPlanBytes: their plan does not price that traffic, and more splits than fit
@@ -119,25 +118,40 @@ inline hipError_t plan_band_splits(int64_t tiles, int64_t K, int64_t chunk, int6
 {
 	const int64_t kchunks = (K + chunk - 1) / chunk;
 	int64_t splits = 1;
-	// (a few more tiles than CUs, up to 1.4 per CU: most CUs would idle while the rest work on their second tile, and two
-	// ranges of K fill the chip better, 16 x 4608 -> 36864 fp32, 288 tiles: 167 -> 141 us; from there on the merge launch
-	// costs what the balance gains, 16 x 1024 -> 50272, 393 tiles: 37 -> 42)
 	const int64_t cus = device_cu_count();
-	const bool cut = tiles < kBandEnoughBlocks || (tiles < 2 * kBandEnoughBlocks && tiles * 10 < ((tiles + cus - 1) / cus) * cus * 7);
-	const size_t capacity = cut ? workspace_capacity(stream) : 0;
-	if (cut && capacity > 0)
+	// Every count of ranges is priced: the blocks of a launch run side by side, a CU's share of the memory bandwidth is
+	// what its blocks divide, so the launch lasts as long as the CU with the most blocks needs for them (one block alone
+	// does not keep enough loads in flight: priced like two); a cut adds the merge launch and the planes' traffic.
+	// (Before: as many ranges as bring the blocks to 512.  32 x 36864 -> 4608 fp32: 141 -> 130 us, [K, N] 139 -> 123; 24 x 5120 ->
+	// 65536 [K, N]: 233 -> 221; 16 x 4608 -> 36864, 288 tiles, now in two ranges: 167 -> 141; a few small products lose a
+	// microsecond.)
+	const size_t capacity = tiles < 2 * kBandEnoughBlocks ? workspace_capacity(stream) : 0;
+	if (capacity > 0 && cus > 0)
 	{
-		splits = (kBandWantedBlocks + tiles - 1) / tiles;
-		if (splits > kBandMaxSplits) splits = kBandMaxSplits;
-		// a split writes and reads back 8 bytes per sum where it streams depth * elem_bytes bytes of weights per
-		// column: splits stay deep enough for the partial sums to be at most a quarter of the traffic
 		const int64_t min_depth = 32 * rows / elem_bytes;
 		const int64_t min_chunks = (min_depth + chunk - 1) / chunk;
-		if (splits > kchunks / min_chunks) splits = kchunks / min_chunks;
 		const size_t plan_bytes = capacity < kBandPlanBytes ? capacity : kBandPlanBytes;
-		const int64_t room = (int64_t)(plan_bytes / ((size_t)tiles * kBandThreads * acc_floats * sizeof(float)));
-		if (splits > room) splits = room;
-		if (splits < 1) splits = 1;
+		const double tile_sums = (double)kBandThreads * (double)acc_floats;
+		const int64_t room = (int64_t)((double)plan_bytes / ((double)tiles * tile_sums * sizeof(float)));
+		int64_t most = kchunks / min_chunks;
+		if (most > kBandMaxSplits) most = kBandMaxSplits;
+		if (most > room) most = room;
+		const double chunk_us = (double)chunk * tile_sums / (double)rows * (double)elem_bytes * (double)cus / 6.4e6;
+		double best = 0.0;
+		for (int64_t s = 1; s <= most || s == 1; ++s)
+		{
+			const int64_t per = (kchunks + s - 1) / s;
+			const int64_t ranges = (kchunks + per - 1) / per;
+			if (ranges != s) continue;
+			const int64_t most_per_cu = (tiles * ranges + cus - 1) / cus;
+			double us = (double)(most_per_cu < 2 ? 2 : most_per_cu) * (double)per * chunk_us;
+			if (ranges > 1) us += 4.6 + 8.0 * tile_sums * (double)tiles * (double)ranges / 5.0e6;
+			if (s == 1 || us < 0.97 * best)
+			{
+				best = us;
+				splits = ranges;
+			}
+		}
 	}
 	SplitPlan plan;
 	plan.chunks_per_split = (kchunks + splits - 1) / splits;

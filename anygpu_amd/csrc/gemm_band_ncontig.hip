@@ -27,7 +27,7 @@ using namespace band;
 
 namespace {
 
-template <int MR, int MB, int EPI, bool KW>
+template <int MR, int MB, int EPI, bool KW, int SETS = 4>
 struct RowBandShape
 {
 	static constexpr bool kDual = (EPI == kEpiGeluMul);
@@ -39,7 +39,7 @@ struct RowBandShape
 	static constexpr int kChunk = 4 * kChunkVecs;             // in elements of K
 	static constexpr int kStepsPerChunk = kChunk / kStep;
 	static constexpr int kWaveSteps = KW ? kStepsPerChunk / 4 : kStepsPerChunk;   // steps of a chunk one wave takes
-	static constexpr int kSets = kWaveSteps >= 4 ? 4 : 2;     // register sets: the loads run kSets - 1 steps ahead
+	static constexpr int kSets = kWaveSteps < 4 ? 2 : SETS;   // register sets: the loads run kSets - 1 steps ahead
 	static constexpr int kPitchVecs = kChunkVecs + 1;
 	static constexpr int kWaveCols = 4 * MR;
 	static constexpr int kBlockCols = KW ? kWaveCols : 4 * kWaveCols;
@@ -94,13 +94,13 @@ __device__ __forceinline__ void row_band_store(const Acc (*acc)[4][MB], const fl
 // C[m, n] = finish(sum_k A[m, k] * B[k, n]), M <= MR * MB, N >= 4.  grid (column tiles, splits of K).
 // KW: the waves of a block share their columns and divide K.  With gridDim.y > 1 the sums go to
 // partial[wave tile][split][lane][register].
-template <int MR, int MB, int EPI, bool KW>
+template <int MR, int MB, int EPI, bool KW, int SETS>
 __global__ __launch_bounds__(kBandThreads) void gemm_band_ncontig_kernel(
 	const float* __restrict__ A, const float* __restrict__ B, const float* __restrict__ B2, const float* __restrict__ bias,
 	float* __restrict__ C, float* __restrict__ partial,
 	int M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc, int chunks_per_split, float ep_param)
 {
-	using S = RowBandShape<MR, MB, EPI, KW>;
+	using S = RowBandShape<MR, MB, EPI, KW, SETS>;
 	using Acc = typename BandMma<float, MR>::Acc;
 
 	__shared__ Vec band_lds[2][S::kRows * S::kPitchVecs];
@@ -363,11 +363,11 @@ __global__ __launch_bounds__(kBandThreads) void gemm_band_ncontig_merge_kernel(
 	*reinterpret_cast<LooseVec*>(C + (int64_t)m * ldc + n) = out;
 }
 
-template <int MR, int MB, int EPI, bool KW>
+template <int MR, int MB, int EPI, bool KW, int SETS>
 hipError_t launch_row_band_waves(const float* A, const float* B, const float* B2, const float* bias, float* C, int M, int64_t N,
                                  int64_t K, int64_t lda, int64_t ldb, int64_t ldc, float ep_param, hipStream_t stream)
 {
-	using S = RowBandShape<MR, MB, EPI, KW>;
+	using S = RowBandShape<MR, MB, EPI, KW, SETS>;
 	const int64_t tiles = (N + S::kBlockCols - 1) / S::kBlockCols;
 	const int64_t wave_tiles = (N + S::kWaveCols - 1) / S::kWaveCols;
 	// one wave's worth of sums per wave tile and split: a quarter of a 256-thread block's
@@ -375,7 +375,7 @@ hipError_t launch_row_band_waves(const float* A, const float* B, const float* B2
 	const hipError_t plan_err = plan_band_splits(tiles, K, S::kChunk, S::kRows, (int)sizeof(float), S::kAccFloats / (KW ? 4 : 1), stream, &plan);
 	if (plan_err != hipSuccess) return plan_err;
 	discard_stale_error();
-	gemm_band_ncontig_kernel<MR, MB, EPI, KW><<<dim3((unsigned)tiles, (unsigned)plan.splits), dim3(kBandThreads), 0, stream>>>(
+	gemm_band_ncontig_kernel<MR, MB, EPI, KW, SETS><<<dim3((unsigned)tiles, (unsigned)plan.splits), dim3(kBandThreads), 0, stream>>>(
 		A, B, B2, bias, C, plan.partial, M, N, K, lda, ldb, ldc, (int)plan.chunks_per_split, ep_param);
 	if (plan.splits > 1)
 	{
@@ -392,8 +392,17 @@ hipError_t launch_row_band(const float* A, const float* B, const float* B2, cons
 {
 	// waves side by side when that alone gives the chip enough blocks, else the waves of a block divide K
 	if ((N + 16 * MR - 1) / (16 * MR) >= kBandEnoughBlocks)
-		return launch_row_band_waves<MR, MB, EPI, false>(A, B, B2, bias, C, M, N, K, lda, ldb, ldc, ep_param, stream);
-	return launch_row_band_waves<MR, MB, EPI, true>(A, B, B2, bias, C, M, N, K, lda, ldb, ldc, ep_param, stream);
+		return launch_row_band_waves<MR, MB, EPI, false, 4>(A, B, B2, bias, C, M, N, K, lda, ldb, ldc, ep_param, stream);
+	// 32 rows of one product, waves dividing K: with two register sets for the weights instead of four (loads one step
+	// ahead instead of three) three waves fit a SIMD instead of two, which hides more of the matrix cores' time than the
+	// deeper queue does (32 x 4096 -> 6144: 37 -> 32 us, 4096 -> 11008: 48 -> 45.7); with 200 tiles and more, or a K of 16384 and
+	// more, the deeper queue stays ahead (24 x 5120 -> 65536: 224 against 234, 32 x 36864 -> 4608: 123 against 139)
+	if constexpr (MR == 32 && MB == 1 && EPI != kEpiGeluMul)
+	{
+		if ((N + 4 * MR - 1) / (4 * MR) < 200 && K < 16384)
+			return launch_row_band_waves<MR, MB, EPI, true, 2>(A, B, B2, bias, C, M, N, K, lda, ldb, ldc, ep_param, stream);
+	}
+	return launch_row_band_waves<MR, MB, EPI, true, 4>(A, B, B2, bias, C, M, N, K, lda, ldb, ldc, ep_param, stream);
 }
 
 }  // namespace
