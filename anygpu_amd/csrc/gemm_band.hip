@@ -433,17 +433,19 @@ size_t capacity_of(hipStream_t stream, size_t own_bytes)
 	int device = 0;
 	if (hipGetDevice(&device) != hipSuccess) return 0;
 	size_t bytes = 0;
-	bool from_caller = false;
+	bool fixed = false;
 	{
 		std::lock_guard<std::mutex> guard(workspace_lock);
 		const auto found = workspaces.find(std::make_pair(device, stream));
-		if (found != workspaces.end() && found->second.from_caller)
+		// a caller's buffer is what it is; so is the library's own while a launcher above holds pointers into it (a
+		// reserved front): growing it would free what they point at
+		if (found != workspaces.end() && (found->second.from_caller || reserved_front > 0))
 		{
 			bytes = found->second.bytes;
-			from_caller = true;
+			fixed = true;
 		}
 	}
-	if (!from_caller) bytes = stream_is_capturing(stream) ? 0 : own_bytes;
+	if (!fixed) bytes = (stream_is_capturing(stream) || reserved_front > 0) ? 0 : own_bytes;
 	return bytes > reserved_front ? bytes - reserved_front : 0;
 }
 }  // namespace
@@ -471,7 +473,9 @@ hipError_t band::workspace_acquire(hipStream_t stream, float** base, size_t at_l
 			*base = reinterpret_cast<float*>(reinterpret_cast<char*>(found->second.base) + reserved_front);
 			return hipSuccess;
 		}
-		// the library's own buffer is too small for this copy: a larger one takes its place
+		// the library's own buffer is too small for this copy: a larger one takes its place (never under a launcher
+		// that holds pointers into it; the capacities above say so beforehand)
+		if (reserved_front > 0) return hipErrorInvalidValue;
 		const hipError_t freed = hipFree(found->second.base);
 		if (freed != hipSuccess)
 		{

@@ -85,7 +85,8 @@ size_t workspace_copy_capacity(hipStream_t stream);
 hipError_t workspace_acquire(hipStream_t stream, float** base, size_t at_least = 0);
 // While one of these lives, the calling thread's view of every workspace starts `bytes` (rounded up to 256) further on:
 // a launcher that has parked operand copies at the front of the stream's workspace calls the ordinary launchers
-// underneath it, whose partial sums then go behind the copies.
+// underneath it, whose partial sums then go behind the copies.  The launcher holds pointers into the buffer, so while a
+// reservation lives the library's own buffer does not grow: both capacities report what is left of it as it is.
 class WorkspaceReserve
 {
 public:

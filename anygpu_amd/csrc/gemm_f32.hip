@@ -453,7 +453,11 @@ static TilePlan plan_tiles(int tile, int64_t M, int64_t N, int64_t K, int64_t ba
 		if (tile == 64 && !four_wave && blocks > 2 * chip_cus()) return (double)blocks / (double)chip_cus();
 		return (double)((blocks + chip_cus() - 1) / chip_cus());
 	};
-	TilePlan best{tile, 1, rounds_of(tiles) * (double)slabs * slab_us};
+	// (with a short K the time a block takes to start and to store its tile counts: a CU holds one big tile, whose loads
+	// and stores nothing overlaps, or several small ones; 32 x 1024 x 128 . 128 x 1024 batched: 119 -> 111 us, 8192 x 64 -> 8192:
+	// 143 -> 133.  From K = 512 on the slab prices alone choose better.)
+	const double store_us = (four_wave && K <= 256) ? (tile == 128 ? 3.0 : 0.4) : 0.0;
+	TilePlan best{tile, 1, rounds_of(tiles) * ((double)slabs * slab_us + store_us)};
 	if (!may_split || batch != 1) return best;
 	const int64_t room = (int64_t)(workspace_bytes / ((size_t)M * N * sizeof(float)));
 	for (int64_t s = 2; s <= kSplitMax && s <= K / kSplitMinDepth && s <= room; ++s)

@@ -1547,6 +1547,30 @@ def test_gemm_gelu_mul_k_contiguous_weights(ops, oracle, m, hsize, isize):
     assert scaled_rel_err(host(out), want, 1.0) <= TOL_F32
 
 
+def test_gemm_gelu_mul_as_two_products_whose_operands_want_copies(ops, oracle):
+    # 200 rows: the fused up-projection runs as two plain products into planes of the stream's workspace.  K is no
+    # multiple of 32, so each product would like aligned zero-padded copies of its operands, 80 MB for these weights:
+    # more than the library's buffer holds behind the planes, and the buffer must not grow (be freed and allocated
+    # anew) while the planes live in it.  Twice, so that a buffer that did change hands shows.
+    import torch
+    from anygpu_amd import capi
+    m, hsize, isize = 200, 2052, 9216
+    x = synth.normal(m, (m, hsize))
+    wg = synth.normal(5, (hsize, isize)) * np.float32(1.0 / math.sqrt(hsize))
+    wu = synth.normal(6, (hsize, isize)) * np.float32(1.0 / math.sqrt(hsize))
+    want = oracle.gemma_mlp_upproj(x, wg, wu, threads=8)
+    dx, dg, du = dev(x), dev(np.ascontiguousarray(wg.T)), dev(np.ascontiguousarray(wu.T))
+    for _ in range(2):
+        out = torch.empty((m, isize), device="cuda")
+        rc = capi.load().anygpu_gemm_f32_gelu_mul(dx.data_ptr(), dg.data_ptr(), du.data_ptr(), out.data_ptr(), m, isize, hsize,
+                                                  hsize, hsize, isize, capi.B_COL_MAJOR, None)
+        assert rc == capi.ANYGPU_OK
+        assert scaled_rel_err(host(out), want, 1.0) <= TOL_F32
+    # and the plain product of the same operands afterwards (which may now grow the buffer for its copies)
+    got = host(ops.tensor_mm(dx, dg, b_layout=capi.B_COL_MAJOR))
+    assert scaled_rel_err(got, oracle.tensor_mm(x, wg, threads=8), 1.0) <= TOL_F32
+
+
 def test_gemm_epilogues_rejected_arguments(ops):
     import torch
     from anygpu_amd import capi
