@@ -8,9 +8,9 @@
 // outside the visible key interval [lo, hi] of the row are never loaded; their outputs are
 // stored as zeros.
 // Short rows (up to 64 vectors) share a wave four at a time; rows longer than a block's registers hold are walked
-// twice by a block of 1024 threads with 16-byte accesses.
-// General kernel (such rows with a mask tensor): one 256-thread block per row with scalar accesses for any width,
-// stride or alignment; it reads the visible part of the row twice.
+// twice by a block of 1024 threads with 16-byte accesses, at any width, stride or alignment.
+// An additive mask tensor [q_len, cols] shared by the heads of a batch is read with ordinary (cached) loads, and the
+// blocks are dealt so that the heads of a mask row run side by side on one XCD (block_rows).
 #include "device_utils.hpp"
 #include "launch.hpp"
 
@@ -33,6 +33,7 @@ struct SoftmaxArgs
 	int64_t window;
 	const void* mask;      // optional additive mask [q_len, cols] of the element type (NULL: none)
 	int64_t mask_stride;   // elements between mask rows
+	int heads;             // > 1: rows = heads x q_len share the mask rows and the blocks are dealt as block_rows() says
 };
 
 template <typename T> struct Vec16;
@@ -43,6 +44,34 @@ template <> struct Vec16<float> { using type = float4_t; };
 __device__ __forceinline__ int64_t query_of_row(const SoftmaxArgs& a, int64_t row)
 {
 	return a.q_len > 0 ? (int64_t)((uint32_t)row % (uint32_t)a.q_len) : row;
+}
+
+// First row of a block that works on `per_block` consecutive rows, or -1 for a block without rows.  Plain: block b
+// takes rows b * per_block on.  With a mask tensor shared by `heads` heads (rows = heads x q_len, row = head * q_len +
+// query) the blocks that read one mask row should run at the same time on the same XCD, so that the row comes out of
+// that XCD's L2 for all heads but one: consecutive blocks go to the eight XCDs in turn, so block b = 8 s + x takes head
+// s % heads of query group 8 (s / heads) + x, and the launch has ceil(groups / 8) * 8 * heads blocks.
+__device__ __forceinline__ int64_t block_rows(const SoftmaxArgs& a, int per_block, int64_t* rows_end)
+{
+	if (a.heads <= 1)
+	{
+		*rows_end = a.rows;
+		return (int64_t)blockIdx.x * per_block;
+	}
+	const uint32_t x = blockIdx.x % 8u, slot = blockIdx.x / 8u;
+	const uint32_t head = slot % (uint32_t)a.heads;
+	const int64_t group = (int64_t)(slot / (uint32_t)a.heads) * 8 + x;
+	const int64_t q0 = group * per_block;
+	*rows_end = (int64_t)(head + 1) * a.q_len;
+	return q0 < a.q_len ? (int64_t)head * a.q_len + q0 : -1;
+}
+
+// blocks of such a launch
+static inline unsigned blocks_for_rows(const SoftmaxArgs& a, int per_block)
+{
+	if (a.heads <= 1) return (unsigned)((a.rows + per_block - 1) / per_block);
+	const int64_t groups = (a.q_len + per_block - 1) / per_block;
+	return (unsigned)((groups + 7) / 8 * 8 * a.heads);
 }
 
 // Visible key interval of a row, inclusive on both ends; empty when hi < lo.
@@ -91,7 +120,8 @@ __device__ __forceinline__ float exp2_shift(float a, float b)
 // GROUP: threads that share a row: 16 (a row of lanes per row, four rows per wave and sixteen per block, for rows of up
 // to 64 vectors: a wave per row would leave most of its lanes without a vector and few bytes in flight), 64 (a wave per
 // row, four rows per block) or 256 (the block per row, for rows longer than a wave's registers hold).
-template <typename T, int VPL, bool LOOSE, int GROUP>
+// MASK: the launch has a mask tensor; its vectors are loaded beside the row's and kept in registers like them.
+template <typename T, int VPL, bool LOOSE, int GROUP, bool MASK>
 __global__ __launch_bounds__(256) void softmax_rows_wave_kernel(const SoftmaxArgs a)
 {
 	static_assert(GROUP == 16 || GROUP == 64 || GROUP == 256, "a row of lanes, a wave or the block per row");
@@ -102,9 +132,10 @@ __global__ __launch_bounds__(256) void softmax_rows_wave_kernel(const SoftmaxArg
 	__shared__ float red_m[4], red_s[4];
 
 	const int lane = threadIdx.x & (GROUP - 1);
-	const int64_t row = GROUP == 16 ? (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4)
-	                  : GROUP == 64 ? (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6) : (int64_t)blockIdx.x;
-	if (row >= a.rows) return;  // uniform over the group
+	int64_t rows_end;
+	const int64_t first_row = block_rows(a, 256 / GROUP, &rows_end);
+	const int64_t row = first_row + (GROUP == 16 ? (threadIdx.x >> 4) : GROUP == 64 ? (threadIdx.x >> 6) : 0);
+	if (first_row < 0 || row >= rows_end) return;  // uniform over the group
 
 	const RowSpan span = row_span(a, row);
 	const T* __restrict__ xr = static_cast<const T*>(a.x) + row * a.xs;
@@ -135,21 +166,23 @@ __global__ __launch_bounds__(256) void softmax_rows_wave_kernel(const SoftmaxArg
 		else if (LOOSE) __builtin_nontemporal_store(val, reinterpret_cast<LooseVec*>(base) + v);
 		else __builtin_nontemporal_store(val, reinterpret_cast<Vec*>(base) + v);
 	};
-	// additive mask row of this query (shared by all heads, so it is served from L2); it is
-	// fetched again in each register pass instead of being held in registers
-	const T* __restrict__ mrow = a.mask ? static_cast<const T*>(a.mask) + query_of_row(a, row) * a.mask_stride : nullptr;
-	auto mask_of = [&](int v, float (&mk)[EPV]) {
-#pragma unroll
-		for (int e = 0; e < EPV; ++e) mk[e] = 0.0f;
-		if (mrow != nullptr)
+	// additive mask row of this query, shared by all heads: ordinary loads, so that it stays in the caches for them
+	const T* __restrict__ mrow = MASK ? static_cast<const T*>(a.mask) + query_of_row(a, row) * a.mask_stride : nullptr;
+	auto fetch_mask = [&](int v) {
+		Vec mv = {};
+		if (LOOSE && tail && v == nvec - 1)
 		{
-			const Vec mv = fetch(mrow, v);
 #pragma unroll
-			for (int e = 0; e < EPV; ++e) mk[e] = (float)mv[e] * kLog2e;   // -inf and float lowest both end at -inf
+			for (int e = 0; e < EPV; ++e)
+				if (e < tail) mv[e] = mrow[(int64_t)v * EPV + e];
 		}
+		else if (LOOSE) mv = *(reinterpret_cast<const LooseVec*>(mrow) + v);
+		else mv = *(reinterpret_cast<const Vec*>(mrow) + v);
+		return mv;
 	};
 
 	Vec raw[VPL];
+	Vec mraw[MASK ? VPL : 1];
 #pragma unroll
 	for (int t = 0; t < VPL; ++t)
 	{
@@ -159,7 +192,17 @@ __global__ __launch_bounds__(256) void softmax_rows_wave_kernel(const SoftmaxArg
 		Vec val = {};
 		if (need) val = fetch(xr, v);
 		raw[t] = val;
+		if constexpr (MASK)
+		{
+			Vec mv = {};
+			if (need) mv = fetch_mask(v);
+			mraw[t] = mv;
+		}
 	}
+	auto mask_of = [&](int t, float (&mk)[EPV]) {
+#pragma unroll
+		for (int e = 0; e < EPV; ++e) mk[e] = MASK ? (float)mraw[MASK ? t : 0][e] * kLog2e : 0.0f;   // -inf and float lowest both end at -inf
+	};
 
 	OnlineState st;
 #pragma unroll
@@ -171,7 +214,7 @@ __global__ __launch_bounds__(256) void softmax_rows_wave_kernel(const SoftmaxArg
 		if (need)
 		{
 			float z[EPV], mk[EPV];
-			mask_of(v, mk);
+			mask_of(t, mk);
 			float vmax = -INFINITY;
 #pragma unroll
 			for (int e = 0; e < EPV; ++e)
@@ -220,7 +263,7 @@ __global__ __launch_bounds__(256) void softmax_rows_wave_kernel(const SoftmaxArg
 			if (need)
 			{
 				float mk[EPV];
-				mask_of(v, mk);
+				mask_of(t, mk);
 #pragma unroll
 				for (int e = 0; e < EPV; ++e)
 				{
@@ -380,56 +423,11 @@ static hipError_t launch_f16_window(const SoftmaxArgs& a, hipStream_t stream)
 	return hipGetLastError();
 }
 
-template <typename T>
-__global__ __launch_bounds__(256) void softmax_rows_block_kernel(const SoftmaxArgs a)
-{
-	__shared__ float red_m[4];
-	__shared__ float red_s[4];
-
-	const int64_t row = blockIdx.x;
-	const RowSpan span = row_span(a, row);
-	const T* __restrict__ xr = static_cast<const T*>(a.x) + row * a.xs;
-	T* __restrict__ yr = static_cast<T*>(a.y) + row * a.ys;
-	const T* __restrict__ mrow = a.mask ? static_cast<const T*>(a.mask) + query_of_row(a, row) * a.mask_stride : nullptr;
-	auto mask_at = [&](int64_t j) { return mrow ? (float)mrow[j] * kLog2e : 0.0f; };
-
-	OnlineState st;
-	for (int64_t j = span.lo + threadIdx.x; j <= span.hi; j += blockDim.x)
-	{
-		const float z = logit2(a, (float)xr[j]) + mask_at(j);
-		const float mn = fmaxf(st.m, z);
-		st.s = st.s * exp2_shift(st.m, mn) + exp2_shift(z, mn);
-		st.m = mn;
-	}
-
-	const int wave = threadIdx.x >> 6;
-	const float wm = wave_allreduce(st.m, MaxOp());
-	const float ws = wave_allreduce(st.s * exp2_shift(st.m, wm), SumOp());
-	if ((threadIdx.x & (kWaveSize - 1)) == 0)
-	{
-		red_m[wave] = wm;
-		red_s[wave] = ws;
-	}
-	__syncthreads();
-	float M = fmaxf(fmaxf(red_m[0], red_m[1]), fmaxf(red_m[2], red_m[3]));
-	float S = 0.0f;
-#pragma unroll
-	for (int w = 0; w < 4; ++w) S += red_s[w] * exp2_shift(red_m[w], M);
-	const float inv = S > 0.0f ? 1.0f / S : 0.0f;
-
-	for (int64_t j = threadIdx.x; j < a.cols; j += blockDim.x)
-	{
-		float p = 0.0f;
-		if (j >= span.lo && j <= span.hi) p = exp2_shift(logit2(a, (float)xr[j]) + mask_at(j), M) * inv;
-		yr[j] = (T)p;
-	}
-}
-
-// Rows longer than a block's registers hold (more than 32768 elements: the logits of an output head), without a mask
-// tensor: a block of 1024 threads per row walks the row twice with 16-byte accesses, four per thread in flight: first
-// the online maximum and sum, then, the row coming out of the L2 this time, the probabilities.  The vectors are
-// aligned to the row's own start (rows of any length and pitch); where the result row is not aligned alike its vectors
-// go out at element alignment.
+// Rows longer than a block's registers hold (more than 32768 elements: the logits of an output head): a block of 1024
+// threads per row walks the row twice with 16-byte accesses, four per thread in flight: first the online maximum and
+// sum, then, the row coming out of the L2 this time, the probabilities.  The vectors are aligned to the row's own start
+// (rows of any length and pitch); where the result row, or the row of a mask tensor, is not aligned alike its vectors
+// move at element alignment.
 template <typename T>
 __global__ __launch_bounds__(1024) void softmax_rows_long_kernel(const SoftmaxArgs a)
 {
@@ -439,10 +437,15 @@ __global__ __launch_bounds__(1024) void softmax_rows_long_kernel(const SoftmaxAr
 	typedef Vec LooseVec __attribute__((aligned(sizeof(T))));
 	__shared__ float red_m[16], red_s[16];
 
-	const int64_t row = blockIdx.x;
+	int64_t rows_end;
+	const int64_t row = block_rows(a, 1, &rows_end);
+	if (row < 0) return;
 	const RowSpan span = row_span(a, row);
 	const T* __restrict__ xr = static_cast<const T*>(a.x) + row * a.xs;
 	T* __restrict__ yr = static_cast<T*>(a.y) + row * a.ys;
+	const T* __restrict__ mrow = a.mask ? static_cast<const T*>(a.mask) + query_of_row(a, row) * a.mask_stride : nullptr;
+	auto mask_at = [&](int64_t j) { return mrow ? (float)mrow[j] * kLog2e : 0.0f; };
+	auto mask_vec = [&](int64_t e0) { return mrow ? *reinterpret_cast<const LooseVec*>(mrow + e0) : Vec{}; };
 	// elements [0, head): one by one; then nvec whole vectors at 16-byte boundaries of x; then the rest one by one
 	const int64_t to_boundary = (int64_t)(((16 - reinterpret_cast<uintptr_t>(xr) % 16) % 16) / sizeof(T));
 	const int64_t head = to_boundary < a.cols ? to_boundary : a.cols;
@@ -456,12 +459,12 @@ __global__ __launch_bounds__(1024) void softmax_rows_long_kernel(const SoftmaxAr
 	OnlineState st;
 	auto take_one = [&](int64_t j) {
 		if (j < lo || j > hi) return;
-		const float z = logit2(a, (float)xr[j]);
+		const float z = logit2(a, (float)xr[j]) + mask_at(j);
 		const float mn = fmaxf(st.m, z);
 		st.s = st.s * exp2_shift(st.m, mn) + exp2_shift(z, mn);
 		st.m = mn;
 	};
-	auto take_vec = [&](int64_t v, const Vec& val) {
+	auto take_vec = [&](int64_t v, const Vec& val, const Vec& mval) {
 		const int64_t e0 = head + v * EPV;
 		if (e0 > hi || e0 + EPV - 1 < lo) return;
 		float z[EPV];
@@ -470,7 +473,7 @@ __global__ __launch_bounds__(1024) void softmax_rows_long_kernel(const SoftmaxAr
 		for (int e = 0; e < EPV; ++e)
 		{
 			const int64_t j = e0 + e;
-			z[e] = (j >= lo && j <= hi) ? logit2(a, (float)val[e]) : -INFINITY;
+			z[e] = (j >= lo && j <= hi) ? logit2(a, (float)val[e]) + (float)mval[e] * kLog2e : -INFINITY;
 			vmax = fmaxf(vmax, z[e]);
 		}
 		const float mn = fmaxf(st.m, vmax);
@@ -484,20 +487,25 @@ __global__ __launch_bounds__(1024) void softmax_rows_long_kernel(const SoftmaxAr
 	for (int64_t j = rest + tid; j < a.cols; j += kThreads) take_one(j);
 	for (int64_t v0 = tid; v0 < nvec; v0 += (int64_t)kThreads * kAhead)
 	{
-		Vec val[kAhead];
+		Vec val[kAhead], mval[kAhead];
 #pragma unroll
 		for (int u = 0; u < kAhead; ++u)
 		{
 			const int64_t v = v0 + (int64_t)u * kThreads;
 			const int64_t e0 = head + v * EPV;
 			val[u] = Vec{};
-			if (v < nvec && e0 <= hi && e0 + EPV - 1 >= lo) val[u] = xv[v];
+			mval[u] = Vec{};
+			if (v < nvec && e0 <= hi && e0 + EPV - 1 >= lo)
+			{
+				val[u] = xv[v];
+				mval[u] = mask_vec(e0);
+			}
 		}
 #pragma unroll
 		for (int u = 0; u < kAhead; ++u)
 		{
 			const int64_t v = v0 + (int64_t)u * kThreads;
-			if (v < nvec) take_vec(v, val[u]);
+			if (v < nvec) take_vec(v, val[u], mval[u]);
 		}
 	}
 
@@ -519,21 +527,26 @@ __global__ __launch_bounds__(1024) void softmax_rows_long_kernel(const SoftmaxAr
 	const float inv = S > 0.0f ? 1.0f / S : 0.0f;
 
 	auto put_one = [&](int64_t j) {
-		const float p = (j >= lo && j <= hi) ? exp2_shift(logit2(a, (float)xr[j]), M) * inv : 0.0f;
+		const float p = (j >= lo && j <= hi) ? exp2_shift(logit2(a, (float)xr[j]) + mask_at(j), M) * inv : 0.0f;
 		yr[j] = (T)p;
 	};
 	if (tid < head) put_one(tid);
 	for (int64_t j = rest + tid; j < a.cols; j += kThreads) put_one(j);
 	for (int64_t v0 = tid; v0 < nvec; v0 += (int64_t)kThreads * kAhead)
 	{
-		Vec val[kAhead];
+		Vec val[kAhead], mval[kAhead];
 #pragma unroll
 		for (int u = 0; u < kAhead; ++u)
 		{
 			const int64_t v = v0 + (int64_t)u * kThreads;
 			const int64_t e0 = head + v * EPV;
 			val[u] = Vec{};
-			if (v < nvec && e0 <= hi && e0 + EPV - 1 >= lo) val[u] = xv[v];
+			mval[u] = Vec{};
+			if (v < nvec && e0 <= hi && e0 + EPV - 1 >= lo)
+			{
+				val[u] = xv[v];
+				mval[u] = mask_vec(e0);
+			}
 		}
 #pragma unroll
 		for (int u = 0; u < kAhead; ++u)
@@ -548,7 +561,7 @@ __global__ __launch_bounds__(1024) void softmax_rows_long_kernel(const SoftmaxAr
 				for (int e = 0; e < EPV; ++e)
 				{
 					const int64_t j = e0 + e;
-					out[e] = (T)((j >= lo && j <= hi) ? exp2_shift(logit2(a, (float)val[u][e]), M) * inv : 0.0f);
+					out[e] = (T)((j >= lo && j <= hi) ? exp2_shift(logit2(a, (float)val[u][e]) + (float)mval[u][e] * kLog2e, M) * inv : 0.0f);
 				}
 			}
 			if (y_aligned) __builtin_nontemporal_store(out, reinterpret_cast<Vec*>(yr + e0));
@@ -560,9 +573,10 @@ __global__ __launch_bounds__(1024) void softmax_rows_long_kernel(const SoftmaxAr
 template <typename T, int VPL, bool LOOSE = false, int GROUP = 64>
 static hipError_t launch_wave(const SoftmaxArgs& a, hipStream_t stream)
 {
-	const unsigned blocks = GROUP == 16 ? (unsigned)((a.rows + 15) / 16) : GROUP == 64 ? (unsigned)((a.rows + 3) / 4) : (unsigned)a.rows;
+	const unsigned blocks = blocks_for_rows(a, 256 / GROUP);
 	discard_stale_error();
-	softmax_rows_wave_kernel<T, VPL, LOOSE, GROUP><<<dim3(blocks), dim3(256), 0, stream>>>(a);
+	if (a.mask != nullptr) softmax_rows_wave_kernel<T, VPL, LOOSE, GROUP, true><<<dim3(blocks), dim3(256), 0, stream>>>(a);
+	else softmax_rows_wave_kernel<T, VPL, LOOSE, GROUP, false><<<dim3(blocks), dim3(256), 0, stream>>>(a);
 	return hipGetLastError();
 }
 
@@ -570,6 +584,7 @@ static hipError_t launch_wave(const SoftmaxArgs& a, hipStream_t stream)
 template <typename T, bool LOOSE>
 static hipError_t launch_long_rows(const SoftmaxArgs& a, int64_t nvec, hipStream_t stream)
 {
+	if (nvec <= 256 * 4) return launch_wave<T, 4, LOOSE, 256>(a, stream);       // (rows with a mask tensor: a wave takes fewer)
 	if (nvec <= 256 * 8) return launch_wave<T, 8, LOOSE, 256>(a, stream);
 	return launch_wave<T, 16, LOOSE, 256>(a, stream);       // (the caller checks the capacity: 256 x 16 vectors)
 }
@@ -589,6 +604,8 @@ hipError_t launch_softmax_rows(const void* x, void* y, int64_t rows, int64_t col
 	a.alpha_log2e = alpha * kLog2e;
 	a.causal = causal; a.window = window;
 	a.mask = mask; a.mask_stride = mask_stride;
+	// (several heads over one mask: the blocks are dealt so that the heads of a mask row meet in one L2)
+	a.heads = (mask != nullptr && q_len > 0 && rows > q_len && rows % q_len == 0 && rows / q_len <= 65536) ? (int)(rows / q_len) : 1;
 
 	constexpr int EPV = 16 / (int)sizeof(T);
 	const bool vec_ok = (cols % EPV == 0) && (xs % EPV == 0) && (ys % EPV == 0) &&
@@ -634,14 +651,15 @@ hipError_t launch_softmax_rows(const void* x, void* y, int64_t rows, int64_t col
 	// (32768 halves, 16384 floats); longer rows, and long rows too few to give every CU a block, are walked twice by
 	// 1024 threads (8192 x 32768 float32: 751 us in registers, 426 us walked twice; 128 x 32768 halves: 18 -> 10 us).
 	constexpr int kMaxVpl = 16;
-	const bool walk_twice = mask == nullptr && (nvec > (int64_t)256 * kMaxVpl || (nvec > 2048 && rows < 256));
+	const bool walk_twice = nvec > (int64_t)256 * kMaxVpl || (nvec > 2048 && rows < 256);
 	if (vec_ok && walk_twice)
 	{
 		discard_stale_error();
-		softmax_rows_long_kernel<T><<<dim3((unsigned)rows), dim3(1024), 0, stream>>>(a);
+		softmax_rows_long_kernel<T><<<dim3(blocks_for_rows(a, 1)), dim3(1024), 0, stream>>>(a);
 		return hipGetLastError();
 	}
-	if (vec_ok && nvec <= (int64_t)kWaveSize * kMaxVpl)
+	// (with a mask tensor, whose vectors sit in registers beside the row's, a wave takes up to 8 vectors per lane)
+	if (vec_ok && nvec <= (int64_t)kWaveSize * (mask ? 8 : kMaxVpl))
 	{
 		if (nvec <= kWaveSize * 1) return launch_wave<T, 1>(a, stream);
 		if (nvec <= kWaveSize * 2) return launch_wave<T, 2>(a, stream);
@@ -652,7 +670,7 @@ hipError_t launch_softmax_rows(const void* x, void* y, int64_t rows, int64_t col
 	if (vec_ok && nvec <= (int64_t)256 * kMaxVpl) return launch_long_rows<T, false>(a, nvec, stream);
 	// rows at element alignment, any width: the same wave kernel with element-aligned vector accesses
 	const int64_t nvec_loose = (cols + EPV - 1) / EPV;
-	if (!vec_ok && nvec_loose <= (int64_t)kWaveSize * kMaxVpl)
+	if (!vec_ok && nvec_loose <= (int64_t)kWaveSize * (mask ? 8 : kMaxVpl))
 	{
 		if (nvec_loose <= kWaveSize * 1) return launch_wave<T, 1, true>(a, stream);
 		if (nvec_loose <= kWaveSize * 2) return launch_wave<T, 2, true>(a, stream);
@@ -660,11 +678,10 @@ hipError_t launch_softmax_rows(const void* x, void* y, int64_t rows, int64_t col
 		if (nvec_loose <= kWaveSize * 8) return launch_wave<T, 8, true>(a, stream);
 		return launch_wave<T, 16, true>(a, stream);
 	}
-	if (!vec_ok && nvec_loose <= (int64_t)256 * kMaxVpl && !(mask == nullptr && nvec_loose > 2048 && rows < 256))
+	if (!vec_ok && nvec_loose <= (int64_t)256 * kMaxVpl && !(nvec_loose > 2048 && rows < 256))
 		return launch_long_rows<T, true>(a, nvec_loose, stream);
 	discard_stale_error();
-	if (mask == nullptr) softmax_rows_long_kernel<T><<<dim3((unsigned)rows), dim3(1024), 0, stream>>>(a);
-	else softmax_rows_block_kernel<T><<<dim3((unsigned)rows), dim3(256), 0, stream>>>(a);
+	softmax_rows_long_kernel<T><<<dim3(blocks_for_rows(a, 1)), dim3(1024), 0, stream>>>(a);
 	return hipGetLastError();
 }
 

@@ -1616,7 +1616,12 @@ def test_mm_batched(ops, oracle, dtype, batch, m, k, n):
 
 @pytest.mark.parametrize("dtype", ["f16", "f32"])
 @pytest.mark.parametrize("rows,cols,q_len,cap", [(64, 64, 64, 0.0), (96, 48, 48, 0.0), (40, 72, 40, 30.0), (33, 100, 33, 0.0),
-                                                 (256, 2048, 128, 0.0), (12, 8192, 4, 50.0)])
+                                                 (256, 2048, 128, 0.0), (12, 8192, 4, 50.0),
+                                                 # several heads over one mask, query counts that do not fill the blocks' row
+                                                 # groups (sixteen rows, four rows, one row per block); rows walked twice,
+                                                 # whole and at odd widths
+                                                 (3 * 37, 40, 37, 0.0), (5 * 9, 600, 9, 0.0), (20 * 70, 1024, 70, 30.0), (6 * 7, 20000, 7, 0.0),
+                                                 (4 * 16, 40000, 16, 0.0), (2 * 3, 70001, 3, 50.0), (10, 33000, 10, 0.0)])
 def test_softmax_with_mask_tensor(ops, oracle, dtype, rows, cols, q_len, cap):
     # the mask arrives as data (the reference's attention interface); it must agree with the index-rule form
     np_dt = np.float16 if dtype == "f16" else np.float32
