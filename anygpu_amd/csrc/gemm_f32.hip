@@ -662,7 +662,9 @@ hipError_t launch_gemm_f32(const float* A, const float* B, const float* bias, fl
 	// same: 48 us as a band, 64 in tiles).
 	// ([K, N] weights alike, up to 65536 columns: 48 x 4096 -> 14336 94 us through the band kernel for that layout, 66 in
 	// tiles; 9216 -> 2304 59 against 29; with the 256000 columns of an output head the band kernel stays 5 % ahead)
-	const bool tiles_first = a_layout == ANYGPU_A_ROW_MAJOR && M >= 33 && (b_layout == ANYGPU_B_COL_MAJOR || N <= 65536) &&
+		// (small [K, N] weights, up to 6 M elements, from 17 rows on: 32 x 2048 -> 2048 14.2 -> 11.5 us, 4096 -> 1024 14.5 -> 12)
+	const int64_t tiles_first_rows = (b_layout == ANYGPU_B_ROW_MAJOR && (double)K * (double)N <= 6.0e6) ? 17 : 33;
+	const bool tiles_first = a_layout == ANYGPU_A_ROW_MAJOR && M >= tiles_first_rows && (b_layout == ANYGPU_B_COL_MAJOR || N <= 65536) &&
 	                         gemm_f32_ring_applies(A, B, M, N, K, lda, ldb, stride_a, stride_b, batch, 0, 64, b_layout);
 	// few rows against k-contiguous weights with the columns of an output head: whole lines per row and load instruction
 	if (batch == 1 && a_layout == ANYGPU_A_ROW_MAJOR && b_layout == ANYGPU_B_COL_MAJOR && M >= kWideMinRowsF32 &&

@@ -1164,10 +1164,11 @@ def test_mm_k_contiguous_weights_either_side_of_the_routing_rules(ops, oracle, d
     assert bool((cbuf[:, n:] == -3.0).all())
 
 
-@pytest.mark.parametrize("m,k,n", [(32, 128, 4096), (33, 128, 4096), (40, 256, 65536), (40, 256, 65540), (64, 96, 9216), (48, 64, 70000)])
+@pytest.mark.parametrize("m,k,n", [(32, 128, 4096), (33, 128, 4096), (40, 256, 65536), (40, 256, 65540), (64, 96, 9216), (48, 64, 70000),
+                                   (16, 2048, 2048), (17, 2048, 2048), (32, 2400, 2500), (24, 2464, 2500), (24, 4096, 1024)])
 def test_mm_f32_n_contiguous_weights_either_side_of_the_routing_rules(ops, oracle, m, k, n):
     # [K, N] float32 weights: the band kernel for that layout up to 32 rows and for output heads, the tile kernels from 33
-    # rows on up to 65536 columns; small integers, every sum exact
+    # rows on up to 65536 columns (weights of up to 6 M elements: from 17 rows on); small integers, every sum exact
     a = synth.integers(m + 71, (m, k), -2, 2)
     b = synth.integers(n + 72, (k, n), -2, 2)
     want = oracle.tensor_mm(a, b, threads=8)
