@@ -897,6 +897,7 @@ struct DecodeArgs
 	AttnArgs a;
 	float* ws;              // [kv_heads][splits][rows][D + 2]
 	int rows;               // q_per_kv * n_q
+	int groups;             // of 16 rows: a wave each
 	int splits;
 	int tiles_per_split;
 	int t_first, t_last;    // visible key tiles of the group
@@ -913,20 +914,22 @@ __global__ __launch_bounds__(64) void sdp_decode_partial_kernel(const DecodeArgs
 
 	const int lane = threadIdx.x;
 	const int n = lane & 15, g = lane >> 4;
-	const int split = blockIdx.x;
+	int split, group;
+	if (!decode_locate(da.groups, da.splits, split, group)) return;
 	const int kvh = blockIdx.y;
-	const half_t* qp = a.q + (int64_t)kvh * da.rows * D;  // the rows of a group are contiguous: [q_per_kv][n_q][D]
+	const half_t* qp = a.q + (int64_t)kvh * da.rows * D;  // the rows of a key / value head are contiguous: [q_per_kv][n_q][D]
+	const int row = kDecodeRowsPerWave * group + n;        // this lane's row among them
 	const half_t* kp = a.k + (int64_t)kvh * a.n_k * D;
 	const half_t* vp = a.v + (int64_t)kvh * a.n_k * D;
 
-	const bool row_ok = n < da.rows;
-	const int q_idx = row_ok ? n % a.n_q : 0;             // position of this lane's row among the n_q queries
+	const bool row_ok = row < da.rows;
+	const int q_idx = row_ok ? row % a.n_q : 0;             // position of this lane's row among the n_q queries
 	half8_t qf[KS];
 #pragma unroll
 	for (int s = 0; s < KS; ++s)
 	{
 		half8_t val = {};
-		if (row_ok) val = *reinterpret_cast<const half8_t*>(qp + (int64_t)n * D + 32 * s + 8 * g);
+		if (row_ok) val = *reinterpret_cast<const half8_t*>(qp + (int64_t)row * D + 32 * s + 8 * g);
 		qf[s] = val;
 	}
 	int vis_hi = a.causal ? q_idx + a.diag : a.n_k - 1;
@@ -1056,7 +1059,7 @@ __global__ __launch_bounds__(64) void sdp_decode_partial_kernel(const DecodeArgs
 	l += __shfl_xor(l, 32);
 	if (row_ok)
 	{
-		float* dst = da.ws + (((int64_t)kvh * da.splits + split) * da.rows + n) * (D + 2);
+		float* dst = da.ws + (((int64_t)kvh * da.splits + split) * da.rows + row) * (D + 2);
 #pragma unroll
 		for (int c = 0; c < DC; ++c) *reinterpret_cast<WsFloat4*>(dst + 16 * c + 4 * g) = o[c];
 		if (g == 0)
@@ -1072,7 +1075,7 @@ hipError_t launch_decode_variant(const DecodeArgs& da, int64_t kv_heads, hipStre
 {
 	constexpr int kLdsBytes = kAttnKeysPerTile * AttnLds<D>::kPitchV;
 	(void)hipGetLastError();
-	sdp_decode_partial_kernel<D, SOFTCAP><<<dim3((unsigned)da.splits, (unsigned)kv_heads), dim3(64), kLdsBytes, stream>>>(da);
+	sdp_decode_partial_kernel<D, SOFTCAP><<<dim3(decode_blocks(da.groups, da.splits), (unsigned)kv_heads), dim3(64), kLdsBytes, stream>>>(da);
 	hipError_t e = hipGetLastError();
 	if (e != hipSuccess) return e;
 	sdp_decode_merge_kernel<D, half_t><<<dim3((unsigned)da.rows, (unsigned)kv_heads), dim3(256), 0, stream>>>(da.ws, da.a.y, da.rows, da.splits);
@@ -1124,7 +1127,7 @@ int64_t sdp_attention_decode_workspace_bytes(int64_t batch_heads, int64_t q_per_
 {
 	if (batch_heads == 0 || n_q == 0) return 0;
 	const int64_t kv_heads = batch_heads / q_per_kv;
-	const DecodePlan p = plan_decode(kv_heads, n_q, n_k, causal, window, kAttnKeysPerTile);
+	const DecodePlan p = plan_decode(kv_heads * ((q_per_kv * n_q + kDecodeRowsPerWave - 1) / kDecodeRowsPerWave), n_q, n_k, causal, window, kAttnKeysPerTile);
 	return kv_heads * p.splits * (q_per_kv * n_q) * (head_dim + 2) * (int64_t)sizeof(float);
 }
 
@@ -1134,7 +1137,7 @@ hipError_t launch_sdp_attention_decode_f16(const void* q, const void* k, const v
 {
 	if (batch_heads == 0 || n_q == 0) return hipSuccess;
 	const int64_t kv_heads = batch_heads / q_per_kv;
-	const DecodePlan p = plan_decode(kv_heads, n_q, n_k, causal, window, kAttnKeysPerTile);
+	const DecodePlan p = plan_decode(kv_heads * ((q_per_kv * n_q + kDecodeRowsPerWave - 1) / kDecodeRowsPerWave), n_q, n_k, causal, window, kAttnKeysPerTile);
 	DecodeArgs da;
 	da.a.q = static_cast<const half_t*>(q);
 	da.a.k = static_cast<const half_t*>(k);
@@ -1152,6 +1155,7 @@ hipError_t launch_sdp_attention_decode_f16(const void* q, const void* k, const v
 	da.a.partials = nullptr;
 	da.ws = static_cast<float*>(workspace);
 	da.rows = (int)(q_per_kv * n_q);
+	da.groups = (da.rows + kDecodeRowsPerWave - 1) / kDecodeRowsPerWave;
 	da.splits = p.splits;
 	da.tiles_per_split = p.tiles_per_split;
 	da.t_first = p.t_first;

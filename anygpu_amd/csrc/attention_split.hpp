@@ -1,7 +1,8 @@
 // Split-key plan and merge kernel of the decode forms of the attention (fp16 and fp32).
 //
-// With at most 16 query rows per key / value head there are too few (head, query block) pairs to fill the chip, so
-// the visible keys of a head are cut into SPLITS, one wave each.  A wave leaves, per row, its unnormalised
+// With few query rows per key / value head there are too few (head, query block) pairs to fill the chip, so
+// the visible keys of a head are cut into SPLITS, one wave each per group of 16 rows (the rows of a head beyond 16 go to
+// further waves, which read the same keys out of the caches).  A wave leaves, per row, its unnormalised
 // accumulators o_i (head_dim floats), its running maximum m_i (in the exponent's base-2 units) and its sum l_i in
 // the workspace, [kv_heads][splits][rows][head_dim + 2] floats, and the merge kernel combines the splits of a row:
 // M = max m_i,  y = sum o_i 2^(m_i - M) / sum l_i 2^(m_i - M).
@@ -17,7 +18,8 @@
 
 namespace anygpu {
 
-constexpr int kDecodeMaxRows = 16;
+constexpr int kDecodeRowsPerWave = 16;
+constexpr int kDecodeMaxRows = 128;               // eight groups of sixteen
 // One split per thread of the merge block.  64 splits of 8 tiles left 64 q heads / 8 kv heads x 32768 keys x 128
 // at 33.8 us for the two launches, 128 splits of 4 tiles take 28.0 us; the old merge (one thread per column walking
 // all splits) would have eaten that gain, since its time grew with the number of splits.
@@ -32,8 +34,10 @@ struct DecodePlan
 	int t_first, t_last, splits, tiles_per_split;
 };
 
-inline DecodePlan plan_decode(int64_t kv_heads, int64_t n_q, int64_t n_k, int causal, int64_t window, int keys_per_tile)
+// `units`: (key / value head, group of 16 rows) pairs, each of which walks the keys
+inline DecodePlan plan_decode(int64_t units, int64_t n_q, int64_t n_k, int causal, int64_t window, int keys_per_tile)
 {
+	const int64_t kv_heads = units;
 	// visible key tiles of a group: its first query decides the low end, its last the high end
 	const int64_t diag = n_k - n_q;
 	int64_t key_hi = n_k - 1;
@@ -58,6 +62,18 @@ inline DecodePlan plan_decode(int64_t kv_heads, int64_t n_q, int64_t n_k, int ca
 	p.splits = (int)((tiles + p.tiles_per_split - 1) / p.tiles_per_split);
 	return p;
 }
+
+// Which split and which group of 16 rows a block of the partial kernels works on.  The groups of one split read the
+// same keys, so they should run at the same time on the same XCD: consecutive blocks go to the eight XCDs in turn, so
+// block 8 t + x takes split 8 (t / groups) + x of group t % groups.  False: a block past the last split.
+__device__ __forceinline__ bool decode_locate(int groups, int splits, int& split, int& group)
+{
+	const unsigned x = blockIdx.x % 8u, t = blockIdx.x / 8u;
+	group = (int)(t % (unsigned)groups);
+	split = (int)(t / (unsigned)groups) * 8 + (int)x;
+	return split < splits;
+}
+inline unsigned decode_blocks(int groups, int splits) { return (unsigned)((splits + 7) / 8 * 8 * groups); }
 
 __device__ __forceinline__ void store_merged(float* dst, const float4_t& v) { *reinterpret_cast<float4_t*>(dst) = v; }
 __device__ __forceinline__ void store_merged(half_t* dst, const float4_t& v)

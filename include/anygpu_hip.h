@@ -303,9 +303,10 @@ int anygpu_sdp_attention_fwd_f32(const float* q, const float* k, const float* v,
 
 /*
  * Decode form of anygpu_sdp_attention_fwd_f16 for generation steps: few queries per head, long key range.  Same
- * arguments, meaning and result; additionally q_per_kv * n_q <= 16 (the queries of the heads that share a key /
- * value head are processed together, so k and v are read once per key / value head) and a workspace: the visible
- * key range is split over up to 64 waves per key / value head, whose partial results (running maximum, sum and
+ * arguments, meaning and result; additionally q_per_kv * n_q <= 128 (the queries of the heads that share a key /
+ * value head are processed together, sixteen rows to a wave, so k and v come from memory once per key / value head
+ * and from the caches for the further groups of sixteen) and a workspace: the visible
+ * key range is split over up to 256 waves per key / value head and group, whose partial results (running maximum, sum and
  * unnormalised accumulators, fp32) pass through `workspace` and are merged by a second kernel on the same stream.
  * anygpu_sdp_attention_decode_workspace_bytes returns the bytes needed for a shape (a negative error code for
  * arguments the decode form rejects); workspace must be 16-byte aligned device memory of at least that size and

@@ -1878,6 +1878,11 @@ DECODE_CASES = [
     (2, 1, 1, 63, 128, 0.0884, 0.0, True, 0),             # less than one tile of keys
     (4, 2, 5, 3, 64, 0.125, 0.0, True, 0),                # more queries than keys: the first two see nothing
     (4, 2, 1, 12000, 64, 0.125, 0.0, True, 0),            # 188 key tiles of 64: more splits than one wave of the merge holds
+    # more than 16 rows per key / value head: groups of 16 rows, a wave each (the last group partly filled)
+    (8, 1, 4, 3000, 64, 0.125, 0.0, True, 0),             # 32 rows: two groups
+    (16, 2, 5, 2049, 128, 0.0884, 0.0, True, 0),          # 40 rows: 16 + 16 + 8
+    (8, 1, 16, 1500, 256, 0.0625, 50.0, True, 700),       # 128 rows: eight groups, softcap and window
+    (6, 2, 7, 900, 64, 0.125, 0.0, False, 0),             # 21 rows
 ]
 
 
@@ -1928,7 +1933,8 @@ def test_sdp_attention_decode_f32_workspace_and_rejected_arguments(ops):
     assert ws_bytes(8, 2, 1, 8192, 256, 1, 4096) == 4 * 256 * 2 * 258 * 4
     assert ws_bytes(8, 2, 1, 40, 256, 1, 0) == 4 * 3 * 2 * 258 * 4           # 3 tiles -> 3 splits
     assert ws_bytes(0, 1, 1, 100, 64, 1, 0) == 0
-    assert ws_bytes(8, 2, 9, 100, 64, 1, 0) == capi.ANYGPU_ERR_UNSUPPORTED   # 18 rows per key / value head
+    assert ws_bytes(8, 2, 9, 100, 64, 1, 0) == 4 * 7 * 18 * 66 * 4           # 18 rows per key / value head: two groups; 7 tiles
+    assert ws_bytes(8, 2, 65, 100, 64, 1, 0) == capi.ANYGPU_ERR_UNSUPPORTED  # 130 rows per key / value head
     q = torch.zeros((4, 1, 64), device="cuda")
     kv = torch.zeros((2, 500, 64), device="cuda")
     y = torch.full_like(q, 3.0)
@@ -1951,7 +1957,8 @@ def test_sdp_attention_decode_workspace_and_rejected_arguments(ops):
     assert ws_bytes(8, 2, 1, 8192, 256, 1, 4096) == 4 * 64 * 2 * 258 * 4
     assert ws_bytes(8, 2, 1, 100, 256, 1, 0) == 4 * 2 * 2 * 258 * 4          # 2 tiles -> 2 splits
     assert ws_bytes(0, 1, 1, 100, 64, 1, 0) == 0
-    assert ws_bytes(8, 2, 9, 100, 64, 1, 0) == capi.ANYGPU_ERR_UNSUPPORTED   # 18 rows per key / value head
+    assert ws_bytes(8, 2, 9, 100, 64, 1, 0) == 4 * 2 * 18 * 66 * 4           # 18 rows per key / value head: two groups; 2 tiles
+    assert ws_bytes(8, 2, 65, 100, 64, 1, 0) == capi.ANYGPU_ERR_UNSUPPORTED  # 130 rows per key / value head
     assert ws_bytes(8, 3, 1, 100, 64, 1, 0) == capi.ANYGPU_ERR_BAD_SHAPE
     q = torch.zeros((4, 1, 64), device="cuda", dtype=torch.float16)
     kv = torch.zeros((2, 500, 64), device="cuda", dtype=torch.float16)

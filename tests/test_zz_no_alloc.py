@@ -72,7 +72,7 @@ def test_decode_static_scratch_rejects_what_does_not_fit(ops):
     f = lib.anygpu_sdp_attention_decode_f16_static
     assert f(q.data_ptr(), kv.data_ptr(), kv.data_ptr(), y.data_ptr(), *shape, 0.0625, 0.0, 1, 0, None) == capi.ANYGPU_ERR_SCRATCH_TOO_SMALL
     assert f(q.data_ptr(), kv.data_ptr(), kv.data_ptr(), None, 4, 2, 1, 500, 256, 0.0625, 0.0, 1, 0, None) == capi.ANYGPU_ERR_NULL_POINTER
-    assert f(q.data_ptr(), kv.data_ptr(), kv.data_ptr(), y.data_ptr(), 8, 2, 9, 100, 64, 0.125, 0.0, 1, 0, None) == capi.ANYGPU_ERR_UNSUPPORTED
+    assert f(q.data_ptr(), kv.data_ptr(), kv.data_ptr(), y.data_ptr(), 8, 2, 65, 100, 64, 0.125, 0.0, 1, 0, None) == capi.ANYGPU_ERR_UNSUPPORTED   # 130 rows
     torch.cuda.synchronize()
     assert bool((y == 3.0).all())
 
