@@ -125,12 +125,12 @@ __global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f32_kernel(const
 	if (a.window > 0 && q0 + a.diag - a.window + 1 > 0) key_lo = q0 + a.diag - a.window + 1;
 	int t_first = key_lo / kKeysPerTile;
 	int t_last = key_hi >= 0 ? key_hi / kKeysPerTile : -1;
-	if (parts == 2)
+	if (parts > 1)
 	{
-		// one half of the block's key tiles; the other half is another block's, a merge kernel combines the two
-		const int mid = t_first + (t_last - t_first + 2) / 2;
-		if (part == 0) t_last = mid - 1;
-		else t_first = mid;
+		// one part of the block's key tiles; the other parts are other blocks', a merge kernel combines them
+		const int per = (t_last - t_first + parts) / parts;
+		t_first += part * per;
+		if (t_first + per - 1 < t_last) t_last = t_first + per - 1;
 	}
 
 	// this lane's query as second operand: q[row][16 s + 4 g .. + 3]
@@ -348,12 +348,12 @@ __global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f32_kernel(const
 	float l = l_run;
 	l += __shfl_xor(l, 16);
 	l += __shfl_xor(l, 32);
-	if (parts == 2)
+	if (parts > 1)
 	{
 		// unnormalised accumulators, running maximum and sum of this half of the keys
 		if (q_row < a.n_q)
 		{
-			float* dst = a.partials + ((((int64_t)bh * walk.n_split + split_slot) * 2 + part) * kQueriesPerBlock + (q_row - q0)) * (D + 2);
+			float* dst = a.partials + ((((int64_t)bh * walk.n_split + split_slot) * parts + part) * kQueriesPerBlock + (q_row - q0)) * (D + 2);
 #pragma unroll
 			for (int c = 0; c < DC; ++c)
 #pragma unroll
@@ -413,20 +413,23 @@ hipError_t launch_variant_f32(const AttnArgsF32& args_in, int64_t batch_heads, h
 	const int64_t q_blocks = (args.n_q + kQueriesPerBlock - 1) / kQueriesPerBlock;
 	const AttnSplitPlan plan = plan_attention_split(args.n_q, args.n_k, args.causal, args.diag, args.window, batch_heads,
 	                                                kQueriesPerBlock, KT, D, band::workspace_capacity(stream));
+	// (or, with too few query blocks for the chip, every block in several parts of its key range)
+	const int64_t parts_all = plan.n_split > 0 ? 1 : plan_attention_parts(args.n_q, args.n_k, args.causal, args.diag, batch_heads, kQueriesPerBlock,
+	                                                                    KT, D, band::workspace_capacity(stream));
 	args.partials = nullptr;
-	if (plan.n_split > 0)
+	if (plan.n_split > 0 || parts_all > 1)
 	{
 		const hipError_t ws_err = band::workspace_acquire(stream, &args.partials);
 		if (ws_err != hipSuccess) return ws_err;
 	}
-	const AttnWalk walk = make_attn_walk(q_blocks, batch_heads, args.q_per_kv, plan.n_split, plan.n_big);
+	const AttnWalk walk = make_attn_walk(q_blocks, batch_heads, args.q_per_kv, plan.n_split, plan.n_big, parts_all);
 	if (attn_walk_blocks(walk) > 0x7FFFFFFFLL) return hipErrorInvalidValue;
 	kernel<<<dim3((unsigned)attn_walk_blocks(walk)), dim3(64 * WAVES), kLdsBytes, stream>>>(args, walk);
 	const hipError_t err = hipGetLastError();
-	if (err != hipSuccess || plan.n_split == 0) return err;
-	const int64_t items = batch_heads * plan.n_split * kQueriesPerBlock * (D / 4);
+	if (err != hipSuccess || walk.n_split == 0) return err;
+	const int64_t items = batch_heads * walk.n_split * kQueriesPerBlock * (D / 4);
 	sdp_attention_merge_halves_kernel<D, float><<<dim3((unsigned)((items + 255) / 256)), dim3(256), 0, stream>>>(
-		args.partials, args.y, args.n_q, (int)q_blocks, (int)plan.n_split, kQueriesPerBlock);
+		args.partials, args.y, args.n_q, (int)q_blocks, walk.n_split, kQueriesPerBlock, parts_all > 1 ? (int)parts_all : 2);
 	return hipGetLastError();
 }
 

@@ -138,10 +138,11 @@ __global__ __launch_bounds__(256) void sdp_decode_merge_kernel(const float* __re
 // and leave [query][head_dim accumulators, maximum, sum] in the workspace, [head][split slot][half][query][head_dim + 2].
 // ---------------------------------------------------------------------------------------------
 
-// y rows of the key-split blocks from the two partial results of each: one thread per four columns of a row.
+// y rows of the key-split blocks from the `parts` partial results of each: one thread per four columns of a row.
 template <int D, typename OutT>
 __global__ __launch_bounds__(256) void sdp_attention_merge_halves_kernel(const float* __restrict__ partials, OutT* __restrict__ y,
-                                                                         int n_q, int q_blocks, int n_split, int queries_per_block)
+                                                                         int n_q, int q_blocks, int n_split, int queries_per_block,
+                                                                         int parts)
 {
 	constexpr int kQuads = D / 4;
 	const int64_t item = (int64_t)blockIdx.x * 256 + threadIdx.x;
@@ -153,16 +154,21 @@ __global__ __launch_bounds__(256) void sdp_attention_merge_halves_kernel(const f
 	const int64_t bh = slot_item / n_split;
 	const int q_row = (q_blocks - 1 - split_slot) * queries_per_block + r;
 	if (q_row >= n_q) return;
-	const float* p0 = partials + ((slot_item * 2) * queries_per_block + r) * (D + 2);
-	const float* p1 = p0 + (int64_t)queries_per_block * (D + 2);
-	const float m0 = p0[D], l0 = p0[D + 1], m1 = p1[D], l1 = p1[D + 1];
-	const float big = fmaxf(m0, m1);
+	const float* p0 = partials + ((slot_item * parts) * queries_per_block + r) * (D + 2);
+	const int64_t step = (int64_t)queries_per_block * (D + 2);
+	float big = -INFINITY;
+	for (int i = 0; i < parts; ++i) big = fmaxf(big, p0[i * step + D]);
 	const float safe = big == -INFINITY ? 0.0f : big;
-	const float w0 = fast_exp2(m0 - safe), w1 = fast_exp2(m1 - safe);
-	const float sum = l0 * w0 + l1 * w1;
+	float sum = 0.0f;
+	float4_t acc = {0.0f, 0.0f, 0.0f, 0.0f};
+	for (int i = 0; i < parts; ++i)
+	{
+		const float w = fast_exp2(p0[i * step + D] - safe);
+		sum += p0[i * step + D + 1] * w;
+		acc += *reinterpret_cast<const WsFloat4*>(p0 + i * step + 4 * quad) * w;
+	}
 	const float inv = sum > 0.0f ? 1.0f / sum : 0.0f;
-	const float4_t a0 = *reinterpret_cast<const WsFloat4*>(p0 + 4 * quad), a1 = *reinterpret_cast<const WsFloat4*>(p1 + 4 * quad);
-	store_merged(y + (bh * n_q + q_row) * D + 4 * quad, (a0 * w0 + a1 * w1) * inv);
+	store_merged(y + (bh * n_q + q_row) * D + 4 * quad, acc * inv);
 }
 
 // How many of a head's latest query blocks to dispatch in two key halves (and how many unsplit ones go out before the
@@ -206,6 +212,29 @@ inline AttnSplitPlan plan_attention_split(int n_q, int n_k, int causal, int diag
 	plan.n_split = n_split;
 	plan.n_big = n_big;
 	return plan;
+}
+
+// Launches with so few query blocks that most CUs would idle while each block walks a long key range alone (a chunk of a
+// long prompt against its cache): every query block goes out as `parts` blocks, one per part of its key tiles.  Twice
+// as many blocks as CUs are aimed at, every part at least 4 tiles, the partial results within `capacity` bytes.
+// 1: no split.
+inline int64_t plan_attention_parts(int n_q, int n_k, int causal, int diag, int64_t batch_heads, int queries_per_block,
+                                    int keys_per_tile, int head_dim, size_t capacity)
+{
+	const int64_t q_blocks = (n_q + queries_per_block - 1) / queries_per_block;
+	const int64_t blocks = q_blocks * batch_heads;
+	const int cus = device_cu_count();
+	if (blocks <= 0 || blocks * 2 > cus || capacity == 0) return 1;
+	// the key tiles of the last (longest) query block, from key 0 on or from the window's start: the window only shortens it
+	int64_t key_hi = n_k - 1;
+	if (causal && (int64_t)(n_q - 1) + diag < key_hi) key_hi = (int64_t)(n_q - 1) + diag;
+	const int64_t tiles = key_hi >= 0 ? key_hi / keys_per_tile + 1 : 0;
+	int64_t parts = (2 * cus + blocks - 1) / blocks;
+	if (parts > tiles / 4) parts = tiles / 4;
+	if (parts > 64) parts = 64;
+	const int64_t room = (int64_t)(capacity / ((size_t)blocks * queries_per_block * (head_dim + 2) * sizeof(float)));
+	if (parts > room) parts = room;
+	return parts >= 2 ? parts : 1;
 }
 
 }  // namespace anygpu

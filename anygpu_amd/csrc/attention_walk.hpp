@@ -41,15 +41,25 @@ struct AttnWalk
 	int real_q_blocks;   // query blocks per head
 	int n_split;         // the latest n_split query blocks of a head are dispatched in two halves of their key range
 	int n_big;           // unsplit blocks dispatched before the halves
+	int parts_all;       // > 1: every query block is dispatched as that many blocks, one per part of its key range
 };
 
-inline AttnWalk make_attn_walk(int64_t q_blocks, int64_t batch_heads, int64_t q_per_kv, int64_t n_split = 0, int64_t n_big = 0)
+// parts_all > 1 (launches with too few query blocks for the chip, long key ranges): n_split and n_big do not apply, the
+// partial results are laid out as if every query block were a split one (slot = blocks from the last).
+inline AttnWalk make_attn_walk(int64_t q_blocks, int64_t batch_heads, int64_t q_per_kv, int64_t n_split = 0, int64_t n_big = 0,
+                               int64_t parts_all = 1)
 {
 	AttnWalk w;
 	w.real_q_blocks = (int)q_blocks;
+	w.parts_all = (int)parts_all;
+	if (parts_all > 1)
+	{
+		n_split = q_blocks;
+		n_big = 0;
+	}
 	w.n_split = (int)n_split;
 	w.n_big = (int)n_big;
-	w.q_blocks = (int)(q_blocks + n_split);
+	w.q_blocks = parts_all > 1 ? (int)(q_blocks * parts_all) : (int)(q_blocks + n_split);
 	w.q_per_kv = (int)q_per_kv;
 	w.groups = (int)(batch_heads / q_per_kv);
 	w.chunk = q_per_kv >= kAttnUnitBlocks ? 1 : (int)(kAttnUnitBlocks / q_per_kv);
@@ -94,6 +104,14 @@ __device__ __forceinline__ bool attn_walk_locate_part(const AttnWalk& w, unsigne
 	split_slot = 0;
 	q_block = v_block;
 	if (v_block >= w.q_blocks) return false;
+	if (w.parts_all > 1)
+	{
+		q_block = v_block / w.parts_all;
+		part = v_block % w.parts_all;
+		parts = w.parts_all;
+		split_slot = w.real_q_blocks - 1 - q_block;
+		return true;
+	}
 	if (w.n_split > 0)
 	{
 		const int rank = w.q_blocks - 1 - v_block;               // 0: dispatched first

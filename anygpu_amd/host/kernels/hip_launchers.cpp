@@ -394,11 +394,11 @@ AttentionShape attention_shape(const Tensor<T, CUDA>& qt, const Tensor<T, CUDA>&
 bool hip_flash_sdpa_decode_applies(const Tensor<float16, CUDA>& qt, const Tensor<float16, CUDA>& kt)
 {
 	const AttentionShape s = attention_shape(qt, kt);
-	// few rows per key / value head and enough keys for the split to pay; up to 128 rows where the fused form (a block
-	// per head and 128 queries) would leave half of the chip idle
+	// few rows per key / value head and enough keys for the split to pay; up to 128 rows of up to 16 queries per head
+	// where the fused form (a block per head and 128 queries) would leave half of the chip idle
 	const int64 rows = s.q_per_kv * s.n_q;
 	if (rows < 1 || s.n_k < 256) return false;
-	return rows <= 16 || (rows <= 128 && s.batch_heads * ((s.n_q + 127) / 128) <= 128);
+	return rows <= 16 || (rows <= 128 && s.n_q <= 16 && s.batch_heads <= 128);
 }
 
 int64 hip_flash_sdpa_decode_workspace_floats(const SoftmaxPrologue& prologue, const Tensor<float16, CUDA>& qt,
@@ -426,7 +426,7 @@ bool hip_flash_sdpa_decode_applies(const Tensor<float32, CUDA>& qt, const Tensor
 	const AttentionShape s = attention_shape(qt, kt);
 	const int64 rows = s.q_per_kv * s.n_q;
 	if (rows < 1 || s.n_k < 256) return false;
-	return rows <= 16 || (rows <= 128 && s.batch_heads * ((s.n_q + 127) / 128) <= 128);
+	return rows <= 16 || (rows <= 128 && s.n_q <= 16 && s.batch_heads <= 128);
 }
 
 int64 hip_flash_sdpa_decode_workspace_floats(const SoftmaxPrologue& prologue, const Tensor<float32, CUDA>& qt,

@@ -345,10 +345,10 @@ def sdp_attention_fwd(qw: torch.Tensor, kw: torch.Tensor, vw: torch.Tensor, alph
     out = torch.empty_like(qw)
     lib = capi.load()
     if decode is None:
-        # generation steps: few rows per key / value head and enough keys for the split to pay; up to 128 rows where
-        # the fused form (a block per head and 128 queries) would leave half of the chip idle
+        # generation steps: few rows per key / value head and enough keys for the split to pay; up to 128 rows of up to
+        # 16 queries per head where the fused form (a block per head and 128 queries) would leave half of the chip idle
         rows = q_per_kv * n_q
-        decode = n_k >= 256 and d in (64, 128, 256) and (0 < rows <= 16 or (rows <= 128 and batch_heads * ((n_q + 127) // 128) <= 128))
+        decode = n_k >= 256 and d in (64, 128, 256) and (0 < rows <= 16 or (rows <= 128 and n_q <= 16 and batch_heads <= 128))
     if qw.dtype == torch.float32:
         if decode:
             need = lib.anygpu_sdp_attention_decode_f32_workspace_bytes(batch_heads, q_per_kv, n_q, n_k, d, int(causal), int(window))

@@ -1677,6 +1677,10 @@ ATTN_CASES = [
     (2, 2, 1, 300, 128, 0.0884, 30.0, True, 128),        # decode step
     (1, 1, 200, 77, 64, 0.125, 0.0, False, 0),
     (2, 2, 192, 192, 64, 0.125, 0.0, False, 40),         # window without the causal rule
+    # a chunk of a long prompt against its cache: few query blocks, long key ranges, every block in several parts
+    (8, 1, 200, 5000, 64, 0.125, 0.0, True, 0),
+    (4, 2, 130, 3000, 128, 0.0884, 30.0, True, 1000),
+    (2, 2, 300, 2500, 128, 0.0884, 0.0, False, 0),
 ]
 
 
@@ -1750,6 +1754,9 @@ ATTN_D256_CASES = [
     (4, 2, 200, 333, 256, -0.05, 0.0, True, 33),
     (2, 2, 260, 260, 256, 0.0625, 0.0, False, 70),
     (2, 2, 100, 40, 256, 0.0625, 0.0, True, 0),
+    # few query blocks against a long cache: every block in several parts of its key range
+    (4, 1, 150, 4100, 256, 0.0625, 50.0, True, 0),
+    (2, 2, 129, 2000, 256, 0.0625, 0.0, True, 700),
 ]
 
 
