@@ -215,8 +215,9 @@ inline AttnSplitPlan plan_attention_split(int n_q, int n_k, int causal, int diag
 }
 
 // Launches with so few query blocks that most CUs would idle while each block walks a long key range alone (a chunk of a
-// long prompt against its cache): every query block goes out as `parts` blocks, one per part of its key tiles.  Twice
-// as many blocks as CUs are aimed at, every part at least 4 tiles, the partial results within `capacity` bytes.
+// long prompt against its cache; fewer blocks than CUs): every query block goes out as `parts` blocks, one per part of
+// its key tiles.  Twice as many blocks as CUs are aimed at, every part at least 4 tiles, the partial results within
+// `capacity` bytes.
 // 1: no split.
 inline int64_t plan_attention_parts(int n_q, int n_k, int causal, int diag, int64_t batch_heads, int queries_per_block,
                                     int keys_per_tile, int head_dim, size_t capacity)
@@ -224,13 +225,16 @@ inline int64_t plan_attention_parts(int n_q, int n_k, int causal, int diag, int6
 	const int64_t q_blocks = (n_q + queries_per_block - 1) / queries_per_block;
 	const int64_t blocks = q_blocks * batch_heads;
 	const int cus = device_cu_count();
-	if (blocks <= 0 || blocks * 2 > cus || capacity == 0) return 1;
+	if (blocks <= 0 || blocks >= cus || capacity == 0) return 1;
 	// the key tiles of the last (longest) query block, from key 0 on or from the window's start: the window only shortens it
 	int64_t key_hi = n_k - 1;
 	if (causal && (int64_t)(n_q - 1) + diag < key_hi) key_hi = (int64_t)(n_q - 1) + diag;
 	const int64_t tiles = key_hi >= 0 ? key_hi / keys_per_tile + 1 : 0;
 	int64_t parts = (2 * cus + blocks - 1) / blocks;
-	if (parts > tiles / 4) parts = tiles / 4;
+	// (with more blocks than half the CUs only long ranges, 16 tiles a part: 8 heads x 3000 x 3000 x 128 causal 63 -> 46 us, but
+	// 32 heads x 640 x 640 20 -> 27 in parts of 3 tiles)
+	const int64_t part_tiles = blocks * 2 > cus ? 16 : 4;
+	if (parts > tiles / part_tiles) parts = tiles / part_tiles;
 	if (parts > 64) parts = 64;
 	const int64_t room = (int64_t)(capacity / ((size_t)blocks * queries_per_block * (head_dim + 2) * sizeof(float)));
 	if (parts > room) parts = room;
