@@ -405,7 +405,18 @@ hipError_t launch_gemm_f16(const void* A, const void* B, void* C, int64_t M, int
 	// K, and the product runs on the copies: 4096 x 4100 . [4096, 4100] weights 270 -> 117 us (vendor 105 - 110).  From
 	// 64 rows on (below that the weights are streamed once anyway and a copy would triple that), for products worth
 	// two more launches, where the workspace holds the copies; otherwise the element-wise kernel at the bottom.
-	if (!tiles_ok && !finish && batch == 1 && M >= 64 && (double)M * (double)N * (double)K >= (double)(1 << 27))
+	// (fewer rows as well where none of the kernels for few rows takes the operands as they lie and the element-wise
+	// kernel would be left: 16 x 4095 -> 4096 87 us that way, [K, N] weights with 4095 columns 287; the vendor 20 - 22)
+	bool few_rows_copy = false;
+	if (!tiles_ok && !finish && batch == 1 && M < 64 && (double)N * (double)K >= (double)(1 << 20))
+	{
+		const bool taken = (b_layout == ANYGPU_B_ROW_MAJOR && gemm_band_kn_f16_applies(A, B, C, M, N, K, lda, ldb, ldc)) ||
+		                   (b_layout == ANYGPU_B_COL_MAJOR && M >= 3 && gemm_band_kc_wide_applies<half_t>(a, b, c, M, N, K, lda, ldb, ldc, kWideMaxRowsF16)) ||
+		                   gemm_band_applies<half_t>(a, b, nullptr, c, M, N, K, lda, ldb, ldc, b_layout) ||
+		                   gemm_skinny_applies<half_t>(a, b, nullptr, M, N, K, lda, ldb, b_layout);
+		few_rows_copy = !taken;
+	}
+	if (!tiles_ok && !finish && batch == 1 && ((M >= 64 && (double)M * (double)N * (double)K >= (double)(1 << 27)) || few_rows_copy))
 	{
 		const bool k_odd = K % 8 != 0;
 		const bool copy_a = k_odd || reinterpret_cast<uintptr_t>(A) % 16 != 0 || lda % 8 != 0;

@@ -1177,6 +1177,46 @@ def test_mm_f32_n_contiguous_weights_either_side_of_the_routing_rules(ops, oracl
 
 
 @pytest.mark.parametrize("layout", ["nk", "kn"])
+@pytest.mark.parametrize("m,k,n", [(16, 1023, 2048), (33, 1024, 2047), (5, 1028, 2052), (63, 2050, 1030), (1, 1025, 4100)])
+def test_mm_f16_few_rows_of_operands_no_kernel_fetches_as_they_lie(ops, oracle, layout, m, k, n):
+    # few rows, a K or an N that leaves the rows of an operand off 16-byte boundaries: where none of the kernels for few
+    # rows takes the operands, aligned zero-padded copies are made and the product runs on those; small integers, exact
+    from anygpu_amd import capi
+    a = synth.integers(m + 61, (m, k), -2, 2)
+    b = synth.integers(n + 62, (k, n), -2, 2)
+    want = oracle.tensor_mm(a, b, threads=8)
+    assert np.abs(want).max() <= 2048
+    da = dev(a.astype(np.float16))
+    if layout == "kn":
+        got = ops.tensor_mm(da, dev(b.astype(np.float16)))
+    else:
+        got = ops.tensor_mm(da, dev(np.ascontiguousarray(b.T).astype(np.float16)), b_layout=capi.B_COL_MAJOR)
+    assert np.array_equal(host(got).astype(np.float32), want)
+
+
+@pytest.mark.parametrize("layout", ["nk", "kn"])
+@pytest.mark.parametrize("m,k,n", [(16, 1023, 2048), (33, 1026, 2050), (100, 2050, 1030), (1, 1025, 4100), (127, 1031, 1100)])
+def test_mm_f32_few_rows_of_operands_no_kernel_fetches_as_they_lie(ops, oracle, layout, m, k, n):
+    # the same shapes in float32: a K that is no multiple of 4 (rows of A, and of [N, K] weights, off 16-byte boundaries)
+    # goes to the general tile kernels (copies of 4-byte operands cost more than they save: 16 x 4098 -> 14338 110 -> 131 us)
+    from anygpu_amd import capi
+    a = synth.integers(m + 63, (m, k), -2, 2)
+    b = synth.integers(n + 64, (k, n), -2, 2)
+    want = oracle.tensor_mm(a, b, threads=8)
+    da = dev(a.astype(np.float32))
+    if layout == "kn":
+        got = ops.tensor_mm(da, dev(b.astype(np.float32)))
+    else:
+        got = ops.tensor_mm(da, dev(np.ascontiguousarray(b.T).astype(np.float32)), b_layout=capi.B_COL_MAJOR)
+    assert np.array_equal(host(got), want)
+    # and with a bias, through the entry point that adds it
+    bias = synth.integers(n + 65, (n,), -5, 5).astype(np.float32)
+    w = dev(b.astype(np.float32)) if layout == "kn" else dev(np.ascontiguousarray(b.T).astype(np.float32))
+    got = ops.tensor_gemm(da, w, dev(bias), b_layout=capi.B_ROW_MAJOR if layout == "kn" else capi.B_COL_MAJOR)
+    assert np.array_equal(host(got), want + bias[None, :])
+
+
+@pytest.mark.parametrize("layout", ["nk", "kn"])
 @pytest.mark.parametrize("m,k,n", [(520, 4096, 14336), (264, 1024, 8192), (1100, 512, 9216), (640, 2048, 14336)])
 def test_mm_f16_rows_just_past_a_multiple_of_256(ops, oracle, layout, m, k, n):
     # products the launcher may divide by rows into the whole multiples of 256 and the rest; small integers, every sum
