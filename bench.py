@@ -25,6 +25,11 @@ The memory-bound kernels rotate over several buffer sets so that the working set
 projection shapes of the models the path serves (8 row counts x 14 weight shapes, weights k-contiguous) next to torch.matmul, i.e. the vendor library,
 on the same operands; with `--gemm-rows between` 22 row counts between the tile heights (3 .. 2060) over 8 of the
 shapes, with `--gemm-layout kn` the weights stored [K, N].
+
+`--attention-shapes` prints a table of the attention forms away from the benchmark's block (generation steps with 1 - 16
+queries per head, chunks of 32 - 1024 queries against a cache of 4096 and 32768 keys, causal prompts of a few thousand
+tokens; fp16 and fp32, head dimensions 64 / 128 / 256, grouped heads) next to torch's scaled_dot_product_attention on the
+same operands, and of the softmax with a mask tensor next to torch.softmax(x * alpha + mask).
 """
 from __future__ import annotations
 
@@ -91,6 +96,9 @@ def parse_args():
     ap.add_argument("--only", default="", help="comma list of: gemm,gemm32,conv,softmax,attn,attn32,decode,norm,head (default: all)")
     ap.add_argument("--gemm-shapes", nargs="?", const="f16", default=None, choices=("f16", "f32"),
                     help="print the table of GEMM layer shapes (fp16, or fp32 with `--gemm-shapes f32`) against torch.matmul and exit")
+    ap.add_argument("--attention-shapes", action="store_true",
+                    help="print the table of attention shapes (generation steps, chunks of a prompt against a cache, masked "
+                         "softmax) against torch and exit")
     ap.add_argument("--gemm-rows", default="layer", choices=("layer", "between"),
                     help="with --gemm-shapes: the row counts of the layer table (powers of two, default) or 22 row counts between "
                          "the tile heights over 8 of the shapes")
@@ -630,6 +638,68 @@ def sweep_gemm_shapes(torch, ops, capi, dtype_name="f16", row_set="layer", layou
           f"{sum(r > 1.10 for r in ratios)} above 1.10, {sum(r > 1.05 for r in ratios)} above 1.05, {sum(r < 0.95 for r in ratios)} below 0.95")
 
 
+def sweep_attention_shapes(torch, ops):
+    """Generation steps, chunks of a prompt against a cache and whole causal prompts through sdp_attention_fwd (which picks
+    the decode form, the fused form, and the split of the key range) next to torch's scaled_dot_product_attention with the
+    same causal rule as a boolean mask (grouped heads by enable_gqa); then the softmax with a mask tensor shared by the
+    heads next to torch.softmax(x * alpha + mask).  Microseconds, the better of two runs of 5 launches each side."""
+    import torch.nn.functional as F
+
+    def timed(fn, iters=5, warm=2):
+        for _ in range(warm):
+            fn()
+        torch.cuda.synchronize()
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(iters):
+            fn()
+        stop.record()
+        torch.cuda.synchronize()
+        return start.elapsed_time(stop) / iters * 1e3
+
+    print("| dtype | batch | heads / kv heads | head dim | queries | keys | this library us | torch SDPA us | ratio |")
+    print("|---|---:|---:|---:|---:|---:|---:|---:|---:|")
+    ratios = []
+    for dtype in (torch.half, torch.float):
+        for batch, heads, kv_heads in ((1, 32, 8), (1, 8, 1), (1, 64, 8), (4, 32, 8)):
+            for d in (64, 128, 256):
+                for n_q in (1, 4, 16, 64, 256, 1024):
+                    for n_k in (4096, 32768):
+                        q = torch.randn(batch, heads, n_q, d, device="cuda").to(dtype)
+                        k = torch.randn(batch, kv_heads, n_k, d, device="cuda").to(dtype)
+                        v = torch.randn(batch, kv_heads, n_k, d, device="cuda").to(dtype)
+                        alpha = d ** -0.5
+                        visible = torch.ones(n_q, n_k, dtype=torch.bool, device="cuda").tril(diagonal=n_k - n_q)
+                        mine = lambda: ops.sdp_attention_fwd(q, k, v, alpha, causal=True)
+                        theirs = lambda: F.scaled_dot_product_attention(q, k, v, attn_mask=visible, scale=alpha, enable_gqa=True)
+                        t_mine, t_theirs = min(timed(mine), timed(mine)), min(timed(theirs), timed(theirs))
+                        ratios.append(t_mine / t_theirs)
+                        print(f"| {str(dtype)[6:]} | {batch} | {heads} / {kv_heads} | {d} | {n_q} | {n_k} | {t_mine:.1f} | {t_theirs:.1f} | {t_mine / t_theirs:.2f} |", flush=True)
+        for heads, n, d in ((32, 1024, 128), (8, 3000, 128), (16, 2048, 64), (8, 5000, 256), (32, 640, 128)):
+            q, k, v = (torch.randn(1, heads, n, d, device="cuda").to(dtype) for _ in range(3))
+            alpha = d ** -0.5
+            mine = lambda: ops.sdp_attention_fwd(q, k, v, alpha, causal=True)
+            theirs = lambda: F.scaled_dot_product_attention(q, k, v, is_causal=True, scale=alpha)
+            t_mine, t_theirs = min(timed(mine), timed(mine)), min(timed(theirs), timed(theirs))
+            ratios.append(t_mine / t_theirs)
+            print(f"| {str(dtype)[6:]} | 1 | {heads} / {heads} | {d} | {n} | {n} | {t_mine:.1f} | {t_theirs:.1f} | {t_mine / t_theirs:.2f} |", flush=True)
+    ratios.sort()
+    print(f"\n{len(ratios)} shapes: median ratio {statistics.median(ratios):.2f}, worst {ratios[-1]:.2f}, {sum(r > 1.0 for r in ratios)} above 1.00")
+    print("\n| dtype | heads | queries | keys | softmax with mask tensor us | GB/s | without mask us | torch.softmax(x * alpha + mask) us |")
+    print("|---|---:|---:|---:|---:|---:|---:|---:|")
+    for dtype in (torch.half, torch.float):
+        for heads, n_q, n_k in ((32, 1024, 1024), (8, 4096, 4096), (8, 8192, 8192), (16, 2000, 2000), (2, 16384, 16384), (8, 1024, 20000), (4, 64, 100000), (8, 16, 32768)):
+            x = torch.randn(heads * n_q, n_k, device="cuda").to(dtype)
+            mask = torch.zeros(n_q, n_k, device="cuda").to(dtype)
+            mask.masked_fill_(torch.ones(n_q, n_k, device="cuda").triu(n_k - n_q + 1).bool(), float("-inf"))
+            masked = lambda: ops.tensor_softmax_masked(x, mask, alpha=0.125, q_len=n_q)
+            plain = lambda: ops.tensor_softmax(x, alpha=0.125)
+            theirs = lambda: torch.softmax(x.view(heads, n_q, n_k) * 0.125 + mask, dim=-1)
+            t_masked, t_plain, t_theirs = min(timed(masked), timed(masked)), min(timed(plain), timed(plain)), min(timed(theirs), timed(theirs))
+            gbs = (2 * x.numel() + mask.numel()) * x.element_size() / t_masked / 1e3
+            print(f"| {str(dtype)[6:]} | {heads} | {n_q} | {n_k} | {t_masked:.1f} | {gbs:.0f} | {t_plain:.1f} | {t_theirs:.1f} |", flush=True)
+
+
 def sample_gemm_shapes(torch, ops, capi):
     """A few products that do not fill the chip with 256 x 256 tiles, ragged ones, ones the chunk loads cannot fetch and two
     output heads with [K, N] weights and few rows, next to torch.matmul on the same operands: microseconds, the better of two runs of 40 launches each side."""
@@ -679,6 +749,9 @@ def main():
     torch.cuda.set_device(0)
     if args.gemm_shapes:
         sweep_gemm_shapes(torch, ops, capi, args.gemm_shapes, args.gemm_rows, args.gemm_layout)
+        return 0
+    if args.attention_shapes:
+        sweep_attention_shapes(torch, ops)
         return 0
     only = set(filter(None, args.only.split(",")))
     want = lambda name: not only or name in only
