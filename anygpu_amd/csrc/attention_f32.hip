@@ -48,6 +48,8 @@ struct AttnArgsF32
 	int window;            // 0: off; else key j is visible iff j > i + diag - window
 	float k_in, k_cap;     // logit transform constants (see logit2)
 	float* partials;       // key-split blocks leave their partial results here: [head][split slot][part][query][D + 2]
+	const float* mask;     // MASK kernels: additive mask [n_q, n_k] shared by all heads (added behind scale and softcap)
+	int64_t mask_stride;   // floats between its rows
 };
 
 // log2(e) * softcap(alpha * s); without softcap k_in = alpha log2(e); with it
@@ -85,7 +87,10 @@ __device__ __forceinline__ void wait_vmem_all()
 // tiles go from memory straight into LDS, into one of two stages, so no staging registers are held and a block of
 // 8 waves (two per SIMD: one multiplies while the other does its softmax arithmetic) fits the register file.
 // Otherwise the tiles pass through registers into a single stage.
-template <int D, bool SOFTCAP, int WAVES, int KT, bool DIRECT>
+// MASK: an additive mask tensor instead of (or on top of) the index rules: the four mask values of a lane's four scores
+// of a key block are consecutive in memory; they are requested in front of the tile's first product and added behind
+// scale and softcap.  No tile is skipped on account of the mask.
+template <int D, bool SOFTCAP, int WAVES, int KT, bool DIRECT, bool MASK>
 __global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f32_kernel(const AttnArgsF32 a, const AttnWalk walk)
 {
 	constexpr int kKeysPerTile = KT;
@@ -206,8 +211,33 @@ __global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f32_kernel(const
 		}
 	};
 
+	// MASK: the mask values of this lane's scores of tile t, times log2(e): four consecutive floats per key block, at any
+	// alignment; keys past the end and rows past the last query read nothing (their scores are masked by the rules)
+	float4_t mk_next[MASK ? KB : 1];
+	auto load_mask = [&](float4_t (&dst)[MASK ? KB : 1], int t) {
+		typedef float4_t LooseF4 __attribute__((aligned(4)));
+#pragma unroll
+		for (int kb = 0; kb < (MASK ? KB : 0); ++kb)
+		{
+			const int key = t * kKeysPerTile + 16 * kb + 4 * g;
+			float4_t val = {-INFINITY, -INFINITY, -INFINITY, -INFINITY};
+			if (q_row < a.n_q)
+			{
+				const float* src = a.mask + (int64_t)q_row * a.mask_stride + key;
+				if (key + 3 < a.n_k) val = *reinterpret_cast<const LooseF4*>(src) * kLog2e;
+				else
+				{
+#pragma unroll
+					for (int r = 0; r < 4; ++r)
+						if (key + r < a.n_k) val[r] = src[r] * kLog2e;
+				}
+			}
+			dst[kb] = val;
+		}
+	};
 	if (t_first <= t_last)
 	{
+		if constexpr (MASK) load_mask(mk_next, t_first);
 		if constexpr (DIRECT) tile_direct(t_first, 0);
 		else tile_load(t_first);
 	}
@@ -231,6 +261,24 @@ __global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f32_kernel(const
 			if (t < t_last) tile_load(t + 1);      // in flight while this tile is used
 		}
 		const float* v_lds = k_lds + kKeysPerTile * L::kPitch;
+
+		// the mask values of this lane's scores of the tile (log2 domain) were requested a tile ahead; those of the next
+		// tile go out now.  A tile in which the mask hides every key from every query of the wave costs the wave nothing
+		// further (under a causal mask tensor that is half of the tiles).
+		float4_t mk[MASK ? KB : 1];
+		if constexpr (MASK)
+		{
+			bool any_visible = false;
+#pragma unroll
+			for (int kb = 0; kb < KB; ++kb)
+			{
+				mk[kb] = mk_next[kb];
+#pragma unroll
+				for (int r = 0; r < 4; ++r) any_visible |= mk[kb][r] > -INFINITY;
+			}
+			if (t < t_last) load_mask(mk_next, t + 1);
+			if (__builtin_amdgcn_ballot_w64(any_visible) == 0) continue;
+		}
 
 		// ---- S^T = K Q^T: s[kb][r] = score of key 16 kb + 4 g + r against this lane's query ----
 		// The K vectors of step st + 1 are read from LDS before the MFMAs of step st are issued (the scheduling
@@ -268,7 +316,7 @@ __global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f32_kernel(const
 		const bool interior = tile_key0 >= all_lo && tile_key0 + kKeysPerTile - 1 <= all_hi;   // wave-uniform
 		float z[KB][4];
 		float mt = -INFINITY;
-		if (interior)
+		if (interior && !MASK)
 		{
 #pragma unroll
 			for (int kb = 0; kb < KB; ++kb)
@@ -287,7 +335,7 @@ __global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f32_kernel(const
 				for (int r = 0; r < 4; ++r)
 				{
 					const int key = tile_key0 + 16 * kb + 4 * g + r;
-					const float zz = logit2<SOFTCAP>(s[kb][r], a.k_in, a.k_cap);
+					const float zz = logit2<SOFTCAP>(s[kb][r], a.k_in, a.k_cap) + (MASK ? mk[MASK ? kb : 0][r] : 0.0f);
 					z[kb][r] = (key >= vis_lo && key <= vis_hi) ? zz : -INFINITY;
 					mt = fmaxf(mt, z[kb][r]);
 				}
@@ -381,7 +429,7 @@ __global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f32_kernel(const
 	}
 }
 
-template <int D, bool SOFTCAP>
+template <int D, bool SOFTCAP, bool MASK>
 hipError_t launch_variant_f32(const AttnArgsF32& args_in, int64_t batch_heads, hipStream_t stream)
 {
 	// head dimension 256: 8 waves (two per SIMD) on tiles of 32 keys in two stages, 130 KB, one block per CU.  Two
@@ -390,7 +438,7 @@ hipError_t launch_variant_f32(const AttnArgsF32& args_in, int64_t batch_heads, h
 	constexpr bool DIRECT = (D == 256);
 	constexpr int WAVES = DIRECT ? 8 : 4;
 	constexpr int KT = DIRECT ? 32 : 64;
-	auto kernel = sdp_attention_fwd_f32_kernel<D, SOFTCAP, WAVES, KT, DIRECT>;
+	auto kernel = sdp_attention_fwd_f32_kernel<D, SOFTCAP, WAVES, KT, DIRECT, MASK>;
 	constexpr int kLdsBytes = AttnLdsF32<D, KT>::kStageFloats * 4 * (DIRECT ? 2 : 1);
 	constexpr int kQueriesPerBlock = 16 * WAVES;
 	(void)hipGetLastError();
@@ -629,7 +677,8 @@ bool sdp_attention_fwd_f32_supports(int64_t head_dim)
 
 hipError_t launch_sdp_attention_fwd_f32(const float* q, const float* k, const float* v, float* y,
                                         int64_t batch_heads, int64_t q_per_kv, int64_t n_q, int64_t n_k, int64_t head_dim,
-                                        float alpha, float softcap, int causal, int64_t window, hipStream_t stream)
+                                        float alpha, float softcap, int causal, int64_t window, hipStream_t stream,
+                                        const float* mask, int64_t mask_stride)
 {
 	if (batch_heads == 0 || n_q == 0) return hipSuccess;
 	AttnArgsF32 args;
@@ -647,8 +696,12 @@ hipError_t launch_sdp_attention_fwd_f32(const float* q, const float* k, const fl
 	args.k_in = capped ? 2.0f * kLog2e * alpha / softcap : alpha * kLog2e;
 	args.k_cap = capped ? softcap * kLog2e : 0.0f;
 	args.partials = nullptr;
+	args.mask = mask;
+	args.mask_stride = mask_stride;
 #define ANYGPU_ATTN_F32_DIM(DIM) \
-	return capped ? launch_variant_f32<DIM, true>(args, batch_heads, stream) : launch_variant_f32<DIM, false>(args, batch_heads, stream)
+	if (mask != nullptr) \
+		return capped ? launch_variant_f32<DIM, true, true>(args, batch_heads, stream) : launch_variant_f32<DIM, false, true>(args, batch_heads, stream); \
+	return capped ? launch_variant_f32<DIM, true, false>(args, batch_heads, stream) : launch_variant_f32<DIM, false, false>(args, batch_heads, stream)
 	switch (head_dim)
 	{
 	case 64: ANYGPU_ATTN_F32_DIM(64);

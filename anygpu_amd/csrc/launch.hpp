@@ -137,11 +137,13 @@ hipError_t launch_sdp_attention_fwd_f16(const void* q, const void* k, const void
                                         int64_t batch_heads, int64_t q_per_kv, int64_t n_q, int64_t n_k, int64_t head_dim,
                                         float alpha, float softcap, int causal, int64_t window, hipStream_t stream);
 
-// The same in float32 with the fp32 matrix instruction.
+// The same in float32 with the fp32 matrix instruction.  mask: optional additive mask [n_q, n_k] (rows mask_stride floats
+// apart) shared by all heads, added behind scale and softcap, on top of the index rules.
 bool sdp_attention_fwd_f32_supports(int64_t head_dim);
 hipError_t launch_sdp_attention_fwd_f32(const float* q, const float* k, const float* v, float* y,
                                         int64_t batch_heads, int64_t q_per_kv, int64_t n_q, int64_t n_k, int64_t head_dim,
-                                        float alpha, float softcap, int causal, int64_t window, hipStream_t stream);
+                                        float alpha, float softcap, int causal, int64_t window, hipStream_t stream,
+                                        const float* mask = nullptr, int64_t mask_stride = 0);
 
 // Decode form of the fused attention (q_per_kv * n_q <= 16 rows per key / value head): the key range is split over
 // waves, partial results go through `workspace` (sdp_attention_decode_workspace_bytes of fp32 scratch, 16-byte aligned).

@@ -302,6 +302,19 @@ int anygpu_sdp_attention_fwd_f32(const float* q, const float* k, const float* v,
                                  float alpha, float softcap, int causal, int64_t window, void* stream);
 
 /*
+ * anygpu_sdp_attention_fwd_f32 with the mask as data: y = softmax(softcap(alpha q k^T) + mask) v, mask an additive
+ * [n_q, n_k] float32 matrix (rows mask_stride >= n_k floats apart, any alignment) shared by all heads, -inf (or the
+ * float lowest the reference's mask builders write) where a key is hidden; a query without a visible key gives zeros.
+ * One kernel, no score matrix in memory: the fused counterpart of sdp_attention_masked_scaled_fwd
+ * (srcs/transformers/sdp.hpp:207-274), whose mask argument is a tensor, in the precision the reference runs it in.
+ * No key tile is skipped on account of the mask; callers whose mask is an index rule are better served by
+ * anygpu_sdp_attention_fwd_f32.  Same key splits through the stream's workspace as that entry point.
+ */
+int anygpu_sdp_attention_fwd_masked_f32(const float* q, const float* k, const float* v, const float* mask, float* y,
+                                        int64_t batch_heads, int64_t q_per_kv, int64_t n_q, int64_t n_k, int64_t head_dim,
+                                        int64_t mask_stride, float alpha, float softcap, void* stream);
+
+/*
  * Decode form of anygpu_sdp_attention_fwd_f16 for generation steps: few queries per head, long key range.  Same
  * arguments, meaning and result; additionally q_per_kv * n_q <= 128 (the queries of the heads that share a key /
  * value head are processed together, sixteen rows to a wave, so k and v come from memory once per key / value head

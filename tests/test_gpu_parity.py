@@ -1707,6 +1707,60 @@ def test_sdp_attention_masked_scaled_fwd(ops, oracle):
     assert scaled_rel_err(got, want, 1.0) <= TOL_F16_GEMM
 
 
+@pytest.mark.parametrize("heads,n_q,n_k,d,kind", [
+    (4, 100, 100, 64, "causal"), (2, 130, 131, 128, "slide"), (3, 257, 257, 256, "slide"), (2, 64, 203, 128, "random"),
+    (2, 33, 1001, 256, "random"), (8, 200, 5000, 64, "causal"),          # (the last: few query blocks, the key range in parts)
+    (2, 70, 70, 128, "blind_rows"), (1, 17, 3, 64, "random"),
+])
+def test_sdp_attention_fused_kernel_f32_with_mask_tensor(ops, oracle, heads, n_q, n_k, d, kind):
+    # the reference's own attention interface (srcs/transformers/sdp.hpp:207-274): the mask arrives as a tensor.  In
+    # float32 one kernel reads it as data; against the oracle's operator chain and against the three-launch form
+    # (batched product, softmax with the mask tensor, batched product) on the device.
+    import torch
+    q = synth.normal(1 + n_q, (1, heads, n_q, d))
+    k = synth.normal(2 + n_k, (1, heads, n_k, d))
+    v = synth.normal(3 + d, (1, heads, n_k, d))
+    alpha = float(d) ** -0.5
+    diag = n_k - n_q
+    if kind == "causal":
+        mask = oracle.causal_mask(n_q, n_k, diag=diag)
+    elif kind == "slide":
+        mask = oracle.slide_mask(oracle.causal_mask(n_q, n_k, diag=diag), max(n_k // 3, 1))
+    else:
+        # finite biases everywhere, a third of the keys hidden at random (every query keeps key 0)
+        rng = np.random.default_rng(n_q * 1000 + n_k)
+        mask = rng.normal(0.0, 2.0, (n_q, n_k)).astype(np.float32)
+        mask[rng.random((n_q, n_k)) < 0.33] = -np.inf
+        mask[:, 0] = 0.5
+        if kind == "blind_rows":
+            mask[5] = -np.inf                     # queries without a visible key: zeros, where the operator chain has NaN
+            mask[n_q // 2] = -np.inf
+            mask[n_q - 1, 1:] = np.finfo(np.float32).min      # the float lowest of the reference's mask builders hides as well
+    mask4 = np.ascontiguousarray(mask, dtype=np.float32).reshape(1, 1, n_q, n_k)
+    with np.errstate(invalid="ignore", over="ignore"):
+        want = oracle.sdp_attention_masked_scaled_fwd(q, k, v, mask4, alpha, threads=8)
+    got = host(ops.sdp_attention_masked_scaled_fwd(dev(q), dev(k), dev(v), dev(mask4), alpha))
+    assert got.shape == q.shape and got.dtype == np.float32 and np.isfinite(got).all()
+    blind = ~np.isfinite(want).all(axis=-1)
+    assert blind.sum() == (2 * heads if kind == "blind_rows" else 0)
+    assert not got[blind].any()
+    assert scaled_rel_err(got[~blind], want[~blind], 1.0) <= TOL_F32
+    # the three launches on the device
+    scores = ops.tensor_mm_batched(dev(q[0]), dev(k[0]), b_layout=__import__("anygpu_amd").capi.B_COL_MAJOR)
+    probs = ops.tensor_softmax_masked(scores.reshape(-1, n_k), dev(mask4.reshape(n_q, n_k)), alpha=alpha, q_len=n_q)
+    three = host(ops.tensor_mm_batched(probs.reshape(heads, n_q, n_k), dev(v[0])))
+    assert scaled_rel_err(got[0][~blind[0]], three[~blind[0]], 1.0) <= TOL_F32 * 2
+    # the C entry point's own checks
+    from anygpu_amd import capi
+    f = capi.load().anygpu_sdp_attention_fwd_masked_f32
+    dq, dk, dv, dm = dev(q), dev(k), dev(v), dev(mask4)
+    y = torch.full(q.shape, 3.0, device="cuda")
+    assert f(dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), None, y.data_ptr(), heads, 1, n_q, n_k, d, n_k, alpha, 0.0, None) == capi.ANYGPU_ERR_NULL_POINTER
+    assert f(dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), dm.data_ptr(), y.data_ptr(), heads, 1, n_q, n_k, d, n_k - 1, alpha, 0.0, None) == capi.ANYGPU_ERR_BAD_STRIDE
+    torch.cuda.synchronize()
+    assert bool((y == 3.0).all())
+
+
 ATTN_CASES = [
     # heads, kv_heads, n_q, n_k, d, alpha, softcap, causal, window
     (2, 2, 16, 16, 64, 0.125, 0.0, False, 0),
