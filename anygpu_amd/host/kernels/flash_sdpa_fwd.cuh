@@ -30,6 +30,18 @@ void hip_flash_sdpa_fwd_f32(
 	Tensor<float32, CUDA>& yt);
 
 /*
+  The float32 kernel with the mask as a tensor: y = softmax(alpha q k^T + mask) v, mask [.., n_q, n_k] with leading 1s,
+  shared by all matrices of q (the interface of sdp_attention_masked_scaled_fwd, srcs/transformers/sdp.hpp:207-274).
+*/
+void hip_flash_sdpa_fwd_masked_f32(
+	const float32 alpha,
+	const Tensor<float32, CUDA>& qt,
+	const Tensor<float32, CUDA>& kt,
+	const Tensor<float32, CUDA>& vt,
+	const Tensor<float32, CUDA>& mask,
+	Tensor<float32, CUDA>& yt);
+
+/*
   The reference's fused kernel by its own name and contract (srcs/kernels/cuda/flash_sdpa_fwd.cuh:6-15): one
   matrix, hidden dim 256, no mask; any sequence length here.
 */

@@ -87,6 +87,15 @@ inline Tensor<dtype, device> sdp_attention_masked_scaled_fwd(
 	else
 	{
 		static_assert(std::is_same_v<dtype, float32> || std::is_same_v<dtype, float16>, "Unsupported data type");
+		if constexpr (std::is_same_v<dtype, float32>)
+		{
+			// float32, a head dimension the fused kernel has: one kernel that reads the mask as data, no score matrix
+			if (d == d_v && (d == 64 || d == 128 || d == 256) && num_mtcs > 0 && n_q > 0 && n_k > 0)
+			{
+				hip_flash_sdpa_fwd_masked_f32(static_cast<float32>(alpha), qw, kw, vw, mask, y);
+				return y;
+			}
+		}
 		Tensor<dtype, CUDA> scores(std::vector<int64>({ num_mtcs * n_q, n_k }));
 		Tensor<dtype, CUDA> probs(std::vector<int64>({ num_mtcs * n_q, n_k }));
 		hip_tensor_mm_batched(qw, kw, scores, num_mtcs, n_q, n_k, d, /*rhs stored [n, k]*/ true);
