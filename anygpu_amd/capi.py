@@ -80,6 +80,8 @@ SIGNATURES = {
                                              c_float, c_float, c_int, c_int64, c_void_p]),
     "anygpu_sdp_attention_fwd_masked_f32": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64,
                                                     c_int64, c_int64, c_float, c_float, c_void_p]),
+    "anygpu_sdp_attention_fwd_masked_f16": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64,
+                                                    c_int64, c_int64, c_float, c_float, c_void_p]),
     "anygpu_sdp_attention_decode_workspace_bytes": (c_int64, [c_int64, c_int64, c_int64, c_int64, c_int64, c_int, c_int64]),
     "anygpu_sdp_attention_decode_f32_workspace_bytes": (c_int64, [c_int64, c_int64, c_int64, c_int64, c_int64, c_int, c_int64]),
     "anygpu_sdp_attention_decode_f16": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64,

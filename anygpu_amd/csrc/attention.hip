@@ -69,6 +69,8 @@ struct AttnArgs
 	int window;            // 0: off; else key j is visible iff j > i + diag - window
 	float k_in, k_cap;     // logit transform constants (see logit2)
 	float* partials;       // key-split blocks leave their partial results here: [head][split slot][part][query][D + 2]
+	const half_t* mask;    // MASK kernels: additive mask [n_q, n_k] shared by all heads (added behind scale and softcap)
+	int64_t mask_stride;   // halves between its rows
 };
 
 // log2(e) * softcap(alpha * s); without softcap k_in = alpha log2(e); with it
@@ -95,7 +97,11 @@ struct AttnLds
 };
 
 // QB: 16-query blocks per wave, WAVES: waves per block; a block owns 16 * QB * WAVES consecutive queries.
-template <int D, bool SOFTCAP, int QB, int WAVES>
+// MASK: an additive mask tensor instead of the index rules (the launcher passes none): the four mask values of a lane's four scores
+// of a key block are consecutive in memory; they are requested a tile ahead and added behind scale and softcap; a tile
+// that the mask hides from every query of a wave costs the wave no products (it still issues its share of the next
+// tile's loads).  No tile is skipped for the whole block on account of the mask.
+template <int D, bool SOFTCAP, int QB, int WAVES, bool MASK = false>
 __global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f16_kernel(const AttnArgs a, const AttnWalk walk)
 {
 	constexpr int kAttnQueriesPerBlock = 16 * QB * WAVES;
@@ -218,8 +224,36 @@ __global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f16_kernel(const
 		}
 	};
 
+	// MASK: the mask values of this lane's scores of tile t: four consecutive halves per query block and key block, at any
+	// alignment; keys past the end and rows past the last query count as hidden
+	half4_t mk_next[MASK ? QB : 1][4];
+	auto load_mask = [&](int t) {
+		typedef half4_t LooseHalf4 __attribute__((aligned(2)));
+#pragma unroll
+		for (int b = 0; b < (MASK ? QB : 0); ++b)
+#pragma unroll
+			for (int kb = 0; kb < 4; ++kb)
+			{
+				const int key = t * kAttnKeysPerTile + 16 * kb + 4 * g;
+				const half_t hidden = (half_t)(-INFINITY);
+				half4_t val = {hidden, hidden, hidden, hidden};
+				if (q_row[b] < a.n_q)
+				{
+					const half_t* src = a.mask + (int64_t)q_row[b] * a.mask_stride + key;
+					if (key + 3 < a.n_k) val = *reinterpret_cast<const LooseHalf4*>(src);
+					else
+					{
+#pragma unroll
+						for (int r = 0; r < 4; ++r)
+							if (key + r < a.n_k) val[r] = src[r];
+					}
+				}
+				mk_next[b][kb] = val;
+			}
+	};
 	if (t_first <= t_last)
 	{
+		if constexpr (MASK) load_mask(t_first);
 #pragma unroll
 		for (int j = 0; j < kSlots; ++j) issue_slot(t_first, 0, j);
 	}
@@ -232,6 +266,32 @@ __global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f16_kernel(const
 		k_lds = lds + ((t - t_first) & 1) * kStageBytes;
 		v_lds = k_lds + kAttnKeysPerTile * L::kPitchK;
 		const bool more = t < t_last;
+		// the mask values of this tile move out of the way of the next tile's, which go out now; they stay halves until
+		// the scores meet them (the float form would not fit the registers at head_dim 256)
+		half4_t mk[MASK ? QB : 1][4];
+		if constexpr (MASK)
+		{
+			bool any_visible = false;
+#pragma unroll
+			for (int b = 0; b < QB; ++b)
+#pragma unroll
+				for (int kb = 0; kb < 4; ++kb)
+				{
+					mk[b][kb] = mk_next[b][kb];
+#pragma unroll
+					for (int r = 0; r < 4; ++r) any_visible |= mk[b][kb][r] > (half_t)(-INFINITY);
+				}
+			if (more) load_mask(t + 1);
+			if (__builtin_amdgcn_ballot_w64(any_visible) == 0)
+			{
+				if (more)
+				{
+#pragma unroll
+					for (int j = 0; j < kSlots; ++j) issue_slot(t + 1, (t + 1 - t_first) & 1, j);
+				}
+				continue;
+			}
+		}
 
 		// ---- S^T = K Q^T: s[b][kb] = scores of query block b against key block kb ----
 		float4_t s[QB][4];
@@ -266,7 +326,7 @@ __global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f16_kernel(const
 		{
 			float z[4][4];
 			float mt = -INFINITY;
-			if (interior)
+			if (interior && !MASK)
 			{
 #pragma unroll
 				for (int kb = 0; kb < 4; ++kb)
@@ -285,8 +345,8 @@ __global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f16_kernel(const
 					for (int r = 0; r < 4; ++r)
 					{
 						const int key = tile_key0 + 16 * kb + 4 * g + r;
-						const float zz = logit2<SOFTCAP>(s[b][kb][r], a.k_in, a.k_cap);
-						z[kb][r] = (key >= vis_lo[b] && key <= vis_hi[b]) ? zz : -INFINITY;
+						const float zz = logit2<SOFTCAP>(s[b][kb][r], a.k_in, a.k_cap) + (MASK ? (float)mk[MASK ? b : 0][kb][r] * kLog2e : 0.0f);
+						z[kb][r] = (MASK || (key >= vis_lo[b] && key <= vis_hi[b])) ? zz : -INFINITY;
 						mt = fmaxf(mt, z[kb][r]);
 					}
 			}
@@ -810,13 +870,14 @@ __global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f16_skew_kernel(
 }
 
 // SKEW: the kernel that takes the two halves of a tile's work from different tiles
-template <int D, bool SOFTCAP, int QB, bool SKEW = false>
+template <int D, bool SOFTCAP, int QB, bool SKEW = false, bool MASK = false>
 hipError_t launch_variant(const AttnArgs& args_in, int64_t batch_heads, hipStream_t stream)
 {
 	constexpr int WAVES = 8;
+	static_assert(!(SKEW && MASK), "the mask tensor goes through the plain kernel");
 	auto kernel = [] {
 		if constexpr (SKEW) return sdp_attention_fwd_f16_skew_kernel<D, SOFTCAP, QB, WAVES>;
-		else return sdp_attention_fwd_f16_kernel<D, SOFTCAP, QB, WAVES>;
+		else return sdp_attention_fwd_f16_kernel<D, SOFTCAP, QB, WAVES, MASK>;
 	}();
 	constexpr int kLdsBytes = 2 * AttnLds<D>::kBytes;           // two stages
 	constexpr int kQueriesPerBlock = 16 * QB * WAVES;
@@ -1095,7 +1156,8 @@ bool sdp_attention_fwd_f16_supports(int64_t head_dim)
 
 hipError_t launch_sdp_attention_fwd_f16(const void* q, const void* k, const void* v, void* y,
                                         int64_t batch_heads, int64_t q_per_kv, int64_t n_q, int64_t n_k, int64_t head_dim,
-                                        float alpha, float softcap, int causal, int64_t window, hipStream_t stream)
+                                        float alpha, float softcap, int causal, int64_t window, hipStream_t stream,
+                                        const void* mask, int64_t mask_stride)
 {
 	if (batch_heads == 0 || n_q == 0) return hipSuccess;
 	AttnArgs args;
@@ -1113,6 +1175,23 @@ hipError_t launch_sdp_attention_fwd_f16(const void* q, const void* k, const void
 	args.k_in = capped ? 2.0f * kLog2e * alpha / softcap : alpha * kLog2e;
 	args.k_cap = capped ? softcap * kLog2e : 0.0f;
 	args.partials = nullptr;
+	args.mask = static_cast<const half_t*>(mask);
+	args.mask_stride = mask_stride;
+	if (mask != nullptr)
+	{
+		args.causal = 0;
+		args.window = 0;
+		// sixteen queries per wave at every head dimension: the mask values of a tile take the registers of a second block
+#define ANYGPU_ATTN_F16_MASK_DIM(DIM) \
+		return capped ? launch_variant<DIM, true, 1, false, true>(args, batch_heads, stream) : launch_variant<DIM, false, 1, false, true>(args, batch_heads, stream)
+		switch (head_dim)
+		{
+		case 64: ANYGPU_ATTN_F16_MASK_DIM(64);
+		case 128: ANYGPU_ATTN_F16_MASK_DIM(128);
+		default: ANYGPU_ATTN_F16_MASK_DIM(256);
+		}
+#undef ANYGPU_ATTN_F16_MASK_DIM
+	}
 	switch (head_dim)
 	{
 	case 64: return launch_dim<64>(args, capped, batch_heads, stream);

@@ -405,6 +405,20 @@ ANYGPU_EXPORT int anygpu_sdp_attention_fwd_f16(const void* q, const void* k, con
 	                                                 causal, window, as_stream(stream));
 }
 
+ANYGPU_EXPORT int anygpu_sdp_attention_fwd_masked_f16(const void* q, const void* k, const void* v, const void* mask, void* y,
+                                                      int64_t batch_heads, int64_t q_per_kv, int64_t n_q, int64_t n_k, int64_t head_dim,
+                                                      int64_t mask_stride, float alpha, float softcap, void* stream)
+{
+	const int rc = check_attention(q, k, v, y, batch_heads, q_per_kv, n_q, n_k, head_dim, alpha, softcap, 0);
+	if (rc != ANYGPU_OK) return rc;
+	if (batch_heads == 0 || n_q == 0) return ANYGPU_OK;
+	if (mask == nullptr) return ANYGPU_ERR_NULL_POINTER;
+	if (mask_stride < n_k) return ANYGPU_ERR_BAD_STRIDE;
+	if (reinterpret_cast<uintptr_t>(mask) % 2 != 0) return ANYGPU_ERR_UNSUPPORTED;
+	return (int)anygpu::launch_sdp_attention_fwd_f16(q, k, v, y, batch_heads, q_per_kv, n_q, n_k, head_dim, alpha, softcap,
+	                                                 0, 0, as_stream(stream), mask, mask_stride);
+}
+
 ANYGPU_EXPORT int anygpu_sdp_attention_fwd_f32(const float* q, const float* k, const float* v, float* y,
                                                int64_t batch_heads, int64_t q_per_kv, int64_t n_q, int64_t n_k, int64_t head_dim,
                                                float alpha, float softcap, int causal, int64_t window, void* stream)

@@ -131,11 +131,14 @@ hipError_t launch_gemm_f32_gelu_mul(const float* A, const float* B_gate, const f
                                     int b_layout, hipStream_t stream);
 
 // Fused attention forward, fp16: q [batch_heads, n_q, head_dim], k and v [batch_heads / q_per_kv, n_k, head_dim],
-// y like q; mask rules as in launch_softmax_rows with the diagonal at n_k - n_q.
+// y like q; mask rules as in launch_softmax_rows with the diagonal at n_k - n_q.  mask: optional additive mask of halves
+// [n_q, n_k] (rows mask_stride halves apart) shared by all heads, added behind scale and softcap; it replaces the index rules
+// (causal and window are ignored with it).
 bool sdp_attention_fwd_f16_supports(int64_t head_dim);
 hipError_t launch_sdp_attention_fwd_f16(const void* q, const void* k, const void* v, void* y,
                                         int64_t batch_heads, int64_t q_per_kv, int64_t n_q, int64_t n_k, int64_t head_dim,
-                                        float alpha, float softcap, int causal, int64_t window, hipStream_t stream);
+                                        float alpha, float softcap, int causal, int64_t window, hipStream_t stream,
+                                        const void* mask = nullptr, int64_t mask_stride = 0);
 
 // The same in float32 with the fp32 matrix instruction.  mask: optional additive mask [n_q, n_k] (rows mask_stride floats
 // apart) shared by all heads, added behind scale and softcap, on top of the index rules.

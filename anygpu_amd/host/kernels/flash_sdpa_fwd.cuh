@@ -41,6 +41,15 @@ void hip_flash_sdpa_fwd_masked_f32(
 	const Tensor<float32, CUDA>& mask,
 	Tensor<float32, CUDA>& yt);
 
+/* The same in half precision (mask of halves, fp32 sums on the matrix cores). */
+void hip_flash_sdpa_fwd_masked_f16(
+	const float32 alpha,
+	const Tensor<float16, CUDA>& qt,
+	const Tensor<float16, CUDA>& kt,
+	const Tensor<float16, CUDA>& vt,
+	const Tensor<float16, CUDA>& mask,
+	Tensor<float16, CUDA>& yt);
+
 /*
   The reference's fused kernel by its own name and contract (srcs/kernels/cuda/flash_sdpa_fwd.cuh:6-15): one
   matrix, hidden dim 256, no mask; any sequence length here.

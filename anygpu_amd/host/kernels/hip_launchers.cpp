@@ -370,6 +370,16 @@ void hip_flash_sdpa_fwd_masked_f32(const float32 alpha, const Tensor<float32, CU
 	                                              n_q, n_k, d, n_k, alpha, 0.0f, kNullStream));
 }
 
+void hip_flash_sdpa_fwd_masked_f16(const float32 alpha, const Tensor<float16, CUDA>& qt, const Tensor<float16, CUDA>& kt,
+                                   const Tensor<float16, CUDA>& vt, const Tensor<float16, CUDA>& mask, Tensor<float16, CUDA>& yt)
+{
+	const int64 dim = qt.dim;
+	const int64 n_q = qt.shape[dim - 2], d = qt.shape[dim - 1], n_k = kt.shape[dim - 2];
+	const int64 batch_heads = (n_q * d) > 0 ? qt.numel() / (n_q * d) : 0;
+	ABI_CHECK(anygpu_sdp_attention_fwd_masked_f16(qt.buffer(), kt.buffer(), vt.buffer(), mask.buffer(), yt.buffer(), batch_heads, 1,
+	                                              n_q, n_k, d, n_k, alpha, 0.0f, kNullStream));
+}
+
 void cu_flash_sdpa_fwd_d256_v1(const float32 alpha, const Tensor<float32, CUDA>& qt, const Tensor<float32, CUDA>& kt,
                                const Tensor<float32, CUDA>& vt, Tensor<float32, CUDA>& yt)
 {

@@ -87,14 +87,14 @@ inline Tensor<dtype, device> sdp_attention_masked_scaled_fwd(
 	else
 	{
 		static_assert(std::is_same_v<dtype, float32> || std::is_same_v<dtype, float16>, "Unsupported data type");
-		if constexpr (std::is_same_v<dtype, float32>)
+		// a head dimension the fused kernels have: one kernel that reads the mask as data, no score matrix
+		if (d == d_v && (d == 64 || d == 128 || d == 256) && num_mtcs > 0 && n_q > 0 && n_k > 0)
 		{
-			// float32, a head dimension the fused kernel has: one kernel that reads the mask as data, no score matrix
-			if (d == d_v && (d == 64 || d == 128 || d == 256) && num_mtcs > 0 && n_q > 0 && n_k > 0)
-			{
+			if constexpr (std::is_same_v<dtype, float32>)
 				hip_flash_sdpa_fwd_masked_f32(static_cast<float32>(alpha), qw, kw, vw, mask, y);
-				return y;
-			}
+			else
+				hip_flash_sdpa_fwd_masked_f16(static_cast<float32>(alpha), qw, kw, vw, mask, y);
+			return y;
 		}
 		Tensor<dtype, CUDA> scores(std::vector<int64>({ num_mtcs * n_q, n_k }));
 		Tensor<dtype, CUDA> probs(std::vector<int64>({ num_mtcs * n_q, n_k }));

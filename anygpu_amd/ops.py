@@ -319,15 +319,16 @@ def sdp_attention_masked_scaled_fwd(qw: torch.Tensor, kw: torch.Tensor, vw: torc
     n_k, d_v = kw.shape[-2], vw.shape[-1]
     lead = qw.shape[:-2]
     _require(all(s == 1 for s in mask.shape[:-2]), "mask needs to have 1s in the first dims except the last two")
-    if (qw.dtype == torch.float32 and kw.dtype == vw.dtype == mask.dtype == torch.float32 and d == d_v and d in (64, 128, 256)
+    if (qw.dtype in (torch.float32, torch.float16) and kw.dtype == vw.dtype == mask.dtype == qw.dtype and d == d_v and d in (64, 128, 256)
             and kw.shape[:-2] == qw.shape[:-2] and n_q > 0 and qw.numel() > 0 and n_k > 0):
-        # float32: one kernel that reads the mask as data, no score matrix in memory
+        # one kernel that reads the mask as data, no score matrix in memory
         _check_device(qw, kw, vw, mask)
         q4, k4, v4, m2 = qw.contiguous(), kw.contiguous(), vw.contiguous(), mask.reshape(n_q, n_k).contiguous()
         out = torch.empty_like(q4)
-        rc = capi.load().anygpu_sdp_attention_fwd_masked_f32(q4.data_ptr(), k4.data_ptr(), v4.data_ptr(), m2.data_ptr(), out.data_ptr(),
-                                                             q4.numel() // (n_q * d), 1, n_q, n_k, d, n_k, float(alpha), 0.0, _stream_ptr())
-        capi.check("anygpu_sdp_attention_fwd_masked_f32", rc)
+        name = "anygpu_sdp_attention_fwd_masked_f32" if qw.dtype == torch.float32 else "anygpu_sdp_attention_fwd_masked_f16"
+        rc = getattr(capi.load(), name)(q4.data_ptr(), k4.data_ptr(), v4.data_ptr(), m2.data_ptr(), out.data_ptr(),
+                                        q4.numel() // (n_q * d), 1, n_q, n_k, d, n_k, float(alpha), 0.0, _stream_ptr())
+        capi.check(name, rc)
         return out
     q3, k3, v3 = qw.reshape(-1, n_q, d), kw.reshape(-1, n_k, d), vw.reshape(-1, n_k, d_v)
     scores = tensor_mm_batched(q3.contiguous(), k3.contiguous(), b_layout=capi.B_COL_MAJOR)

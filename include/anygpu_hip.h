@@ -315,6 +315,16 @@ int anygpu_sdp_attention_fwd_masked_f32(const float* q, const float* k, const fl
                                         int64_t mask_stride, float alpha, float softcap, void* stream);
 
 /*
+ * The same in half precision: q, k, v, y and the mask are halves (the mask 2-byte aligned, rows mask_stride >= n_k
+ * halves apart), sums in fp32 on the matrix cores as in anygpu_sdp_attention_fwd_f16.  -inf hides a key; the half
+ * lowest (-65504) is an ordinary, very negative bias, which hides a key wherever the row has a less negative one.
+ * A key tile in which the mask hides every key from all sixteen queries of a wave costs that wave no products.
+ */
+int anygpu_sdp_attention_fwd_masked_f16(const void* q, const void* k, const void* v, const void* mask, void* y,
+                                        int64_t batch_heads, int64_t q_per_kv, int64_t n_q, int64_t n_k, int64_t head_dim,
+                                        int64_t mask_stride, float alpha, float softcap, void* stream);
+
+/*
  * Decode form of anygpu_sdp_attention_fwd_f16 for generation steps: few queries per head, long key range.  Same
  * arguments, meaning and result; additionally q_per_kv * n_q <= 128 (the queries of the heads that share a key /
  * value head are processed together, sixteen rows to a wave, so k and v come from memory once per key / value head

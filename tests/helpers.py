@@ -28,3 +28,11 @@ def sample_rows(n_rows: int, count: int, seed: int = 0) -> np.ndarray:
     edge = [r for r in (0, 1, 2, 3, n_rows - 2, n_rows - 1) if 0 <= r < n_rows]
     mid = rng.integers(0, n_rows, size=max(count - len(edge), 0)).tolist()
     return np.unique(np.array(edge + mid, dtype=np.int64))
+
+
+def exact_int_product(a: np.ndarray, b: np.ndarray) -> np.ndarray:
+    """a @ b for integer-valued operands as int64.  Computed in float64 (the BLAS path, which numpy's own int64
+    product is not): every partial sum of integer products stays far below 2^53, so any order of summation is exact."""
+    a64, b64 = np.asarray(a, dtype=np.float64), np.asarray(b, dtype=np.float64)
+    assert float(np.abs(a64).max(initial=0.0)) * float(np.abs(b64).max(initial=0.0)) * a64.shape[-1] < 2.0 ** 52
+    return (a64 @ b64).astype(np.int64)

@@ -10,13 +10,69 @@ import numpy as np
 import pytest
 
 from anygpu_amd import synth
-from helpers import rel_l2, sample_rows, scaled_rel_err
+from helpers import exact_int_product, rel_l2, sample_rows, scaled_rel_err
 
 pytestmark = pytest.mark.gpu
 
 TOL_F16_GEMM = 1e-2
 TOL_F32 = 1e-4
 TOL_F16_ROWOPS = 2e-3
+
+
+
+def mm_want(oracle, a, b, macs=1.0e8):
+    """a @ b as the parity checks of the larger products take it.  Up to `macs` multiply-adds the oracle computes the
+    whole product the reference's way.  Beyond that (the reference's loop order takes minutes there) the whole product
+    comes from float64 BLAS, exact for the integer-valued operands of the bit-exact tests and closer to the true sums
+    than any float32 summation otherwise, and the oracle's own values are written over a sample of rows (first, last
+    and a seeded spread) and, where the rows are few, of columns; for integer-valued operands the two have to agree
+    bit for bit on the sample."""
+    m, k = a.shape
+    n = b.shape[1]
+    if float(m) * k * n <= macs:
+        return oracle.tensor_mm(a, b, threads=8)
+    full = (a.astype(np.float64) @ b.astype(np.float64)).astype(a.dtype)
+    rows = sample_rows(m, int(max(8, min(m, macs / (float(k) * n)))))
+    cols = np.arange(n) if float(len(rows)) * k * n <= macs else sample_rows(n, int(max(64, macs / (float(len(rows)) * k))), seed=1)
+    sub = oracle.tensor_mm(np.ascontiguousarray(a[rows]), np.ascontiguousarray(b[:, cols]), threads=8)
+    if np.array_equal(a, np.rint(a)) and np.array_equal(b, np.rint(b)):
+        assert np.array_equal(sub, full[np.ix_(rows, cols)])
+    full[np.ix_(rows, cols)] = sub
+    return full
+
+
+def _rows_want(oracle_fn, blas_fn, x, macs_per_row, macs=1.0e8):
+    """A row-wise operator over x [..., rows, k] for the parity checks of the larger shapes: the oracle computes all rows
+    where that is up to `macs` multiply-adds; beyond, the whole result comes from blas_fn (products in float64 BLAS, the
+    element-wise steps by the oracle's own functions) and the oracle's values the reference's way are written over a sample
+    of rows (first, last and a seeded spread, at least 8)."""
+    m = x.shape[-2]
+    if float(m) * macs_per_row <= macs:
+        return oracle_fn(x)
+    full = blas_fn(x)
+    rows = sample_rows(m, int(max(8, macs / macs_per_row)))
+    full[..., rows, :] = oracle_fn(np.ascontiguousarray(x[..., rows, :]))
+    return full
+
+
+def _blas_mm(x, w):
+    return (x.astype(np.float64) @ w.astype(np.float64)).astype(np.float32)
+
+
+def gemm_want(oracle, a, b, bias):
+    return _rows_want(lambda r: oracle.tensor_gemm(r, b, bias, threads=8), lambda r: oracle.tensor_add(_blas_mm(r, b), np.broadcast_to(bias, (r.shape[0], b.shape[1])).copy()),
+                      a, float(b.shape[0]) * b.shape[1])
+
+
+def softcap_head_want(oracle, x, w, cap):
+    return _rows_want(lambda r: oracle.gemma_linear_softcap(r, w, cap, threads=8), lambda r: oracle.softcap(_blas_mm(r, w.T), cap).reshape(r.shape[:-1] + (w.shape[0],)),
+                      x, float(w.shape[0]) * w.shape[1])
+
+
+def upproj_want(oracle, x, wg, wu):
+    return _rows_want(lambda r: oracle.gemma_mlp_upproj(r, wg, wu, threads=8),
+                      lambda r: oracle.tensor_mul(oracle.tensor_gelu_tanh(_blas_mm(r, wg)), _blas_mm(r, wu)).reshape(r.shape[:-1] + (wg.shape[1],)),
+                      x, 2.0 * wg.shape[0] * wg.shape[1])
 
 
 def dev(a):
@@ -428,9 +484,9 @@ def test_mm_f32_reference_cases_integer_inputs_exact(ops, oracle):
         a = synth.integers(11, (m, k), 0, 10)
         b = synth.integers(18, (k, n), 0, 10)
         got = host(ops.tensor_mm(dev(a), dev(b)))
-        want = oracle.tensor_mm(a, b, threads=8)
+        want = mm_want(oracle, a, b)
         assert np.array_equal(got, want)
-        assert np.array_equal(got.astype(np.int64), a.astype(np.int64) @ b.astype(np.int64))
+        assert np.array_equal(got.astype(np.int64), exact_int_product(a, b))
 
 
 @pytest.mark.parametrize("layout", ["row", "col"])
@@ -444,11 +500,11 @@ def test_mm_f32_shapes_and_layouts(ops, oracle, layout, m, k, n):
     if layout == "row":
         b = synth.uniform(k + n, (k, n))
         got = host(ops.tensor_mm(dev(a), dev(b)))
-        want = oracle.tensor_mm(a, b, threads=8)
+        want = mm_want(oracle, a, b)
     else:
         bt = synth.uniform(k + n, (n, k))
         got = host(ops.tensor_mm(dev(a), dev(bt), b_layout=capi.B_COL_MAJOR))
-        want = oracle.tensor_mm(a, bt.T, threads=8)
+        want = mm_want(oracle, a, bt.T)
     floor = math.sqrt(k) / 3.0          # sigma_a * sigma_b * sqrt(K) for U(-1, 1): sigma^2 = 1/3
     assert scaled_rel_err(got, want, floor) <= TOL_F32
 
@@ -461,7 +517,7 @@ def test_mm_f32_few_tiles_split_along_k(ops, oracle, layout, m, k, n):
     from anygpu_amd import capi
     a = synth.uniform(m + k, (m, k))
     b = synth.uniform(k + n, (k, n))
-    want = oracle.tensor_mm(a, b, threads=8)
+    want = mm_want(oracle, a, b)
     da = dev(a)
     db = dev(b) if layout == "row" else dev(np.ascontiguousarray(b.T))
     lay = capi.B_ROW_MAJOR if layout == "row" else capi.B_COL_MAJOR
@@ -473,7 +529,7 @@ def test_mm_f32_few_tiles_split_along_k(ops, oracle, layout, m, k, n):
     assert scaled_rel_err(got, want + bias, math.sqrt(k) / 3.0) <= TOL_F32
     ai, bi = synth.integers(1, (m, k), -4, 4), synth.integers(2, (k, n), -4, 4)
     dbi = dev(bi) if layout == "row" else dev(np.ascontiguousarray(bi.T))
-    assert np.array_equal(host(ops.tensor_mm(dev(ai), dbi, b_layout=lay)), oracle.tensor_mm(ai, bi, threads=8))
+    assert np.array_equal(host(ops.tensor_mm(dev(ai), dbi, b_layout=lay)), mm_want(oracle, ai, bi))
     if layout == "row":
         got = host(ops.tensor_mm(dev(np.ascontiguousarray(a.T)), db, a_layout=capi.A_COL_MAJOR))
         assert scaled_rel_err(got, want, math.sqrt(k) / 3.0) <= TOL_F32
@@ -488,7 +544,7 @@ def test_mm_f32_whole_rounds_and_a_rest(ops, oracle, layout, m, k, n):
     a = synth.uniform(m + k, (m, k))
     b = synth.uniform(k + n, (k, n))
     bias = synth.uniform(5, (n,))
-    want = oracle.tensor_mm(a, b, threads=8)
+    want = mm_want(oracle, a, b)
     da = dev(a)
     db = dev(b) if layout == "row" else dev(np.ascontiguousarray(b.T))
     lay = capi.B_ROW_MAJOR if layout == "row" else capi.B_COL_MAJOR
@@ -498,7 +554,7 @@ def test_mm_f32_whole_rounds_and_a_rest(ops, oracle, layout, m, k, n):
     assert scaled_rel_err(got, want + bias, math.sqrt(k) / 3.0) <= TOL_F32
     if layout == "col":
         got = host(ops.tensor_gemma_linear_softcap(da.reshape(1, m, k), db, 30.0))[0]
-        ref = oracle.gemma_linear_softcap(a.reshape(1, m, k), np.ascontiguousarray(b.T), 30.0, threads=8)[0]
+        ref = softcap_head_want(oracle, a.reshape(1, m, k), np.ascontiguousarray(b.T), 30.0)[0]
         assert scaled_rel_err(got, ref, math.sqrt(k) / 3.0) <= TOL_F32
 
 
@@ -510,7 +566,7 @@ def test_mm_f32_transposed_left_operand(ops, oracle):
         b = synth.uniform(k * 5 + n, (k, n))
         at = np.ascontiguousarray(a.T)
         got = host(ops.tensor_mm(dev(at), dev(b), a_layout=capi.A_COL_MAJOR))
-        want = oracle.tensor_mm(a, b, threads=8)
+        want = mm_want(oracle, a, b)
         assert scaled_rel_err(got, want, math.sqrt(k) / 3.0) <= TOL_F32
         bt = np.ascontiguousarray(b.T)
         got2 = host(ops.tensor_mm(dev(at), dev(bt), a_layout=capi.A_COL_MAJOR, b_layout=capi.B_COL_MAJOR))
@@ -568,7 +624,7 @@ def test_mm_f16_reference_case_640x1280_1280x320(ops, oracle):
     a = synth.normal(11, (640, 1280)).astype(np.float16)
     b = synth.normal(18, (1280, 320)).astype(np.float16)
     got = host(ops.tensor_mm(dev(a), dev(b))).astype(np.float32)
-    want = oracle.tensor_mm(oracle.cvt_f16_to_f32(a), oracle.cvt_f16_to_f32(b), threads=8)
+    want = mm_want(oracle, oracle.cvt_f16_to_f32(a), oracle.cvt_f16_to_f32(b))
     ok, val = oracle.compare_data_buffers_l2(got, want, 0.01)
     assert ok, val
     assert scaled_rel_err(got, want, math.sqrt(1280)) <= TOL_F16_GEMM
@@ -581,7 +637,7 @@ def test_mm_f16_tile_kernel_shapes(ops, oracle, m, k, n):
     from anygpu_amd import capi
     a = synth.uniform(m + 1, (m, k)).astype(np.float16)
     bt = synth.uniform(n + 2, (n, k)).astype(np.float16)
-    want = oracle.tensor_mm(oracle.cvt_f16_to_f32(a), oracle.cvt_f16_to_f32(bt).T, threads=8)
+    want = mm_want(oracle, oracle.cvt_f16_to_f32(a), oracle.cvt_f16_to_f32(bt).T)
     got = host(ops.tensor_mm(dev(a), dev(bt), b_layout=capi.B_COL_MAJOR)).astype(np.float32)
     assert scaled_rel_err(got, want, math.sqrt(k) / 3.0) <= TOL_F16_GEMM
     assert rel_l2(got, want) <= 1e-2
@@ -603,7 +659,7 @@ def test_mm_f16_ragged_shapes_through_tile_kernels(ops, oracle, layout, m, k, n)
     from anygpu_amd import capi
     a = synth.uniform(m + k, (m, k)).astype(np.float16)
     b = synth.uniform(k + n, (k, n)).astype(np.float16)
-    want = oracle.tensor_mm(oracle.cvt_f16_to_f32(a), oracle.cvt_f16_to_f32(b), threads=8)
+    want = mm_want(oracle, oracle.cvt_f16_to_f32(a), oracle.cvt_f16_to_f32(b))
     # the result sits inside a larger buffer: nothing outside [m, n] may be touched
     cbuf = torch.full((m + 3, n + 16), -7.0, device="cuda", dtype=torch.float16)
     if layout == "row":
@@ -623,7 +679,7 @@ def test_mm_f16_few_tiles_split_along_k(ops, oracle, layout, m, k, n):
     from anygpu_amd import capi
     a = synth.uniform(m + k, (m, k)).astype(np.float16)
     b = synth.uniform(k + n, (k, n)).astype(np.float16)
-    want = oracle.tensor_mm(oracle.cvt_f16_to_f32(a), oracle.cvt_f16_to_f32(b), threads=8)
+    want = mm_want(oracle, oracle.cvt_f16_to_f32(a), oracle.cvt_f16_to_f32(b))
     da = dev(a)
     db = dev(b) if layout == "row" else dev(np.ascontiguousarray(b.T))
     lay = capi.B_ROW_MAJOR if layout == "row" else capi.B_COL_MAJOR
@@ -632,7 +688,7 @@ def test_mm_f16_few_tiles_split_along_k(ops, oracle, layout, m, k, n):
     assert np.array_equal(got, host(ops.tensor_mm(da, db, b_layout=lay)))
     ai, bi = synth.integers(1, (m, k), -2, 2).astype(np.float16), synth.integers(2, (k, n), -2, 2).astype(np.float16)
     dbi = dev(bi) if layout == "row" else dev(np.ascontiguousarray(bi.T))
-    want_i = oracle.tensor_mm(ai.astype(np.float32), bi.astype(np.float32), threads=8)
+    want_i = mm_want(oracle, ai.astype(np.float32), bi.astype(np.float32))
     assert np.array_equal(host(ops.tensor_mm(dev(ai), dbi, b_layout=lay)).astype(np.float32), want_i.astype(np.float16).astype(np.float32))
 
 
@@ -643,7 +699,7 @@ def test_mm_f16_whole_rounds_and_a_rest(ops, oracle, layout, m, k, n):
     from anygpu_amd import capi
     a = synth.integers(m + k, (m, k), -2, 2).astype(np.float16)
     b = synth.integers(k + n, (k, n), -2, 2).astype(np.float16)
-    want = oracle.tensor_mm(a.astype(np.float32), b.astype(np.float32), threads=8)
+    want = mm_want(oracle, a.astype(np.float32), b.astype(np.float32))
     db = dev(b) if layout == "row" else dev(np.ascontiguousarray(b.T))
     lay = capi.B_ROW_MAJOR if layout == "row" else capi.B_COL_MAJOR
     got = host(ops.tensor_mm(dev(a), db, b_layout=lay)).astype(np.float32)
@@ -705,7 +761,7 @@ def test_mm_f16_whole_256_tiles_integer_inputs_exact(ops, m, n, k, pad):
     a_dev[:, :k] = dev(a)
     b_dev[:, :k] = dev(bt)
     got = host(ops.tensor_mm(a_dev[:, :k], b_dev[:, :k], b_layout=capi.B_COL_MAJOR)).astype(np.int64)
-    want = a.astype(np.int64) @ bt.astype(np.int64).T
+    want = exact_int_product(a, bt.T)
     assert np.array_equal(got, want)
 
 
@@ -721,7 +777,7 @@ def test_mm_f16_256_tiles_reference_layout_integer_inputs_exact(ops, m, n, k, pa
     b_dev = torch.full((k, n + pad), 7.0, dtype=torch.float16, device="cuda")
     b_dev[:, :n] = dev(b)
     got = host(ops.tensor_mm(dev(a), b_dev[:, :n], b_layout=capi.B_ROW_MAJOR)).astype(np.int64)
-    want = a.astype(np.int64) @ b.astype(np.int64)
+    want = exact_int_product(a, b)
     assert np.array_equal(got, want)
 
 
@@ -741,7 +797,7 @@ def test_mm_f16_smaller_four_wave_tiles_integer_inputs_exact(ops, m, n, k, pad, 
     a_dev[:, :k] = dev(a)
     b_dev[:, :k] = dev(bt)
     got = host(ops.tensor_mm(a_dev[:, :k], b_dev[:, :k], b_layout=capi.B_COL_MAJOR)).astype(np.int64)
-    want = a.astype(np.int64) @ bt.astype(np.int64).T
+    want = exact_int_product(a, bt.T)
     assert np.abs(want).max() < 2048
     assert np.array_equal(got, want)
 
@@ -775,7 +831,7 @@ def test_mm_f16_operands_the_tile_kernels_cannot_fetch_are_copied(ops, layout, m
     cbuf = torch.full((m + 2, n + 9), -7.0, device="cuda", dtype=torch.float16)
     ops.tensor_mm(a_view, b_view, out=cbuf[:m, :n], b_layout=capi.B_ROW_MAJOR if layout == "row" else capi.B_COL_MAJOR)
     got = host(cbuf).astype(np.int64)
-    want = a.astype(np.int64) @ b.astype(np.int64)
+    want = exact_int_product(a, b)
     assert np.abs(want).max() < 2048
     assert np.array_equal(got[:m, :n], want)
     assert np.all(got[m:, :] == -7) and np.all(got[:, n:] == -7)
@@ -803,7 +859,7 @@ def test_mm_f32_operands_at_odd_addresses_are_copied(ops, layout, m, n, k, a_off
     cbuf = torch.full((m + 2, n + 5), -7.0, device="cuda", dtype=torch.float32)
     ops.tensor_mm(a_view, b_view, out=cbuf[:m, :n], b_layout=capi.B_ROW_MAJOR if layout == "row" else capi.B_COL_MAJOR)
     got = host(cbuf).astype(np.int64)
-    want = a.astype(np.int64) @ b.astype(np.int64)
+    want = exact_int_product(a, b)
     assert np.array_equal(got[:m, :n], want)
     assert np.all(got[m:, :] == -7) and np.all(got[:, n:] == -7)
 
@@ -821,7 +877,7 @@ def test_mm_f16_smaller_four_wave_tiles_reference_layout_exact(ops, m, n, k, pad
     b_dev = torch.full((k, n + pad), 7.0, dtype=torch.float16, device="cuda")
     b_dev[:, :n] = dev(b)
     got = host(ops.tensor_mm(dev(a), b_dev[:, :n], b_layout=capi.B_ROW_MAJOR)).astype(np.int64)
-    want = a.astype(np.int64) @ b.astype(np.int64)
+    want = exact_int_product(a, b)
     assert np.abs(want).max() < 2048
     assert np.array_equal(got, want)
 
@@ -843,7 +899,7 @@ def test_mm_f32_four_wave_kernel_integer_inputs_exact(ops, m, n, k, pad):
     cbuf = torch.full((m + 1, n + 3), -7.0, device="cuda", dtype=torch.float32)
     ops.tensor_mm(a_dev[:, :k], b_dev[:, :k], out=cbuf[:m, :n], b_layout=capi.B_COL_MAJOR)
     got = host(cbuf).astype(np.int64)
-    want = a.astype(np.int64) @ bt.astype(np.int64).T
+    want = exact_int_product(a, bt.T)
     assert np.array_equal(got[:m, :n], want)
     assert np.all(got[m:, :] == -7) and np.all(got[:, n:] == -7)
 
@@ -862,7 +918,7 @@ def test_mm_f32_four_wave_kernel_reference_layout_exact(ops, m, n, k, pad):
     cbuf = torch.full((m + 1, n + 3), -7.0, device="cuda", dtype=torch.float32)
     ops.tensor_mm(dev(a), b_dev[:, :n], out=cbuf[:m, :n])
     got = host(cbuf).astype(np.int64)
-    want = a.astype(np.int64) @ b.astype(np.int64)
+    want = exact_int_product(a, b)
     assert np.array_equal(got[:m, :n], want)
     assert np.all(got[m:, :] == -7) and np.all(got[:, n:] == -7)
 
@@ -896,7 +952,7 @@ def test_mm_few_rows(ops, oracle, dtype, layout, m, k, n):
     b = synth.uniform(k * 5 + n, (k, n)).astype(np_dt)
     a32 = oracle.cvt_f16_to_f32(a) if dtype == "f16" else a
     b32 = oracle.cvt_f16_to_f32(b) if dtype == "f16" else b
-    want = oracle.tensor_mm(a32, b32, threads=8)
+    want = mm_want(oracle, a32, b32)
     if layout == "row":
         got = host(ops.tensor_mm(dev(a), dev(b)))
     else:
@@ -941,7 +997,7 @@ def test_mm_row_bands(ops, oracle, dtype, m, k, n):
     bt = synth.uniform(k * 5 + n, (n, k)).astype(np_dt)
     a32 = oracle.cvt_f16_to_f32(a) if dtype == "f16" else a
     b32 = np.ascontiguousarray((oracle.cvt_f16_to_f32(bt) if dtype == "f16" else bt).T)
-    want = oracle.tensor_mm(a32, b32, threads=8)
+    want = mm_want(oracle, a32, b32)
     da, db = dev(a), dev(bt)
     got = host(ops.tensor_mm(da, db, b_layout=capi.B_COL_MAJOR))
     tol = TOL_F16_GEMM if dtype == "f16" else TOL_F32
@@ -960,7 +1016,7 @@ def test_mm_f32_row_bands_n_contiguous_weights(ops, oracle, m, k, n):
     import torch
     a = synth.uniform(m * 3 + k, (m, k))
     b = synth.uniform(k * 5 + n, (k, n))
-    want = oracle.tensor_mm(a, b, threads=8)
+    want = mm_want(oracle, a, b)
     da, db = dev(a), dev(b)
     got = host(ops.tensor_mm(da, db))
     assert scaled_rel_err(got, want, math.sqrt(k) / 3.0) <= TOL_F32
@@ -970,7 +1026,7 @@ def test_mm_f32_row_bands_n_contiguous_weights(ops, oracle, m, k, n):
     assert scaled_rel_err(got, want + bias, math.sqrt(k) / 3.0) <= TOL_F32
     if m <= 40 and n <= 9216:
         ai, bi = synth.integers(1, (m, k), -4, 4), synth.integers(2, (k, n), -4, 4)
-        assert np.array_equal(host(ops.tensor_mm(dev(ai), dev(bi))), oracle.tensor_mm(ai, bi, threads=8))
+        assert np.array_equal(host(ops.tensor_mm(dev(ai), dev(bi))), mm_want(oracle, ai, bi))
         # operands and result inside wider buffers
         abuf, bbuf = torch.zeros((m, k + 8), device="cuda"), torch.zeros((k, n + 12), device="cuda")
         abuf[:, :k], bbuf[:, :n] = da, db
@@ -989,7 +1045,7 @@ def test_mm_row_bands_rows_of_any_length(ops, oracle, m, k, n):
     from anygpu_amd import capi
     a = synth.integers(m + 1, (m, k), -4, 4)
     b = synth.integers(n + 2, (k, n), -4, 4)
-    want = oracle.tensor_mm(a, b, threads=8)
+    want = mm_want(oracle, a, b)
     da, db = dev(a), dev(b)
     assert np.array_equal(host(ops.tensor_mm(da, db)), want)
     bias = synth.integers(3, (n,), -9, 9)
@@ -1023,7 +1079,7 @@ def test_mm_f16_row_bands_n_contiguous_weights_many_columns(ops, oracle, m, k, n
     from anygpu_amd import capi
     a = synth.integers(m + 11, (m, k), -2, 2)
     b = synth.integers(n + 12, (k, n), -2, 2)
-    want = oracle.tensor_mm(a, b, threads=8)
+    want = mm_want(oracle, a, b)
     assert np.abs(want).max() <= 2048
     da, db = dev(a.astype(np.float16)), dev(b.astype(np.float16))
     got = host(ops.tensor_mm(da, db)).astype(np.float32)
@@ -1039,7 +1095,7 @@ def test_mm_f16_row_bands_n_contiguous_weights_many_columns(ops, oracle, m, k, n
     # uniform operands against the oracle at the fp16 GEMM tolerance, and the softcap epilogue on the same sums
     au = synth.uniform(m + 13, (m, k)).astype(np.float16)
     bu = synth.uniform(n + 14, (k, n)).astype(np.float16)
-    ref = oracle.tensor_mm(oracle.cvt_f16_to_f32(au), oracle.cvt_f16_to_f32(bu), threads=8)
+    ref = mm_want(oracle, oracle.cvt_f16_to_f32(au), oracle.cvt_f16_to_f32(bu))
     dau, dbu = dev(au), dev(bu)
     got = host(ops.tensor_mm(dau, dbu)).astype(np.float32)
     assert scaled_rel_err(got, ref, math.sqrt(k) / 3.0) <= TOL_F16_GEMM
@@ -1071,7 +1127,7 @@ def test_mm_row_bands_k_contiguous_weights_many_columns(ops, oracle, dtype, m, s
     k = steps * (64 if half else 32)
     a = synth.integers(m + 21, (m, k), -2, 2)
     w = synth.integers(n + 22, (n, k), -2, 2)
-    want = oracle.tensor_mm(a, np.ascontiguousarray(w.T), threads=8)
+    want = mm_want(oracle, a, w.T)
     assert np.abs(want).max() <= 2048
     da, dw = dev(a.astype(ndt)), dev(w.astype(ndt))
     got = host(ops.tensor_mm(da, dw, b_layout=capi.B_COL_MAJOR)).astype(np.float32)
@@ -1087,7 +1143,7 @@ def test_mm_row_bands_k_contiguous_weights_many_columns(ops, oracle, dtype, m, s
     assert bool((cbuf[:, n:] == -1.0).all())
     # uniform operands against the oracle at the GEMM tolerance, the softcap epilogue on the same sums, and (fp32) a bias
     au, wu = synth.uniform(m + 23, (m, k)).astype(ndt), synth.uniform(n + 24, (n, k)).astype(ndt)
-    ref = oracle.tensor_mm(au.astype(np.float32), np.ascontiguousarray(wu.astype(np.float32).T), threads=8)
+    ref = mm_want(oracle, au.astype(np.float32), wu.astype(np.float32).T)      # (the oracle and BLAS take the transposed view as it is)
     dau, dwu = dev(au), dev(wu)
     tol = TOL_F16_GEMM if half else TOL_F32
     got = host(ops.tensor_mm(dau, dwu, b_layout=capi.B_COL_MAJOR)).astype(np.float32)
@@ -1119,7 +1175,7 @@ def test_mm_f32_rows_just_past_a_multiple_of_64(ops, oracle, layout, m, k, n):
     a = synth.integers(m + 61, (m, k), -1, 1)
     b = synth.integers(n + 62, (k, n), -1, 1)
     bias = synth.integers(n + 63, (n,), -3, 3)
-    want = oracle.tensor_mm(a, b, threads=8) + bias[None, :].astype(np.float32)
+    want = mm_want(oracle, a, b) + bias[None, :].astype(np.float32)
     da, dbias = dev(a.astype(np.float32)), dev(bias.astype(np.float32))
     dw = dev(b.astype(np.float32)) if layout == "kn" else dev(np.ascontiguousarray(b.T).astype(np.float32))
     out = torch.empty((m, n), device="cuda")
@@ -1156,7 +1212,7 @@ def test_mm_k_contiguous_weights_either_side_of_the_routing_rules(ops, oracle, d
     k = steps * (64 if half else 32)
     a = synth.integers(m + 51, (m, k), -2, 2)
     w = synth.integers(n + 52, (n, k), -2, 2)
-    want = oracle.tensor_mm(a, np.ascontiguousarray(w.T), threads=8)
+    want = mm_want(oracle, a, np.ascontiguousarray(w.T))
     assert np.abs(want).max() <= 2048
     cbuf = torch.full((m, n + 8), -3.0, device="cuda", dtype=tdt)
     ops.tensor_mm(dev(a.astype(ndt)), dev(w.astype(ndt)), out=cbuf[:, :n], b_layout=capi.B_COL_MAJOR)
@@ -1171,7 +1227,7 @@ def test_mm_f32_n_contiguous_weights_either_side_of_the_routing_rules(ops, oracl
     # rows on up to 65536 columns (weights of up to 6 M elements: from 17 rows on); small integers, every sum exact
     a = synth.integers(m + 71, (m, k), -2, 2)
     b = synth.integers(n + 72, (k, n), -2, 2)
-    want = oracle.tensor_mm(a, b, threads=8)
+    want = mm_want(oracle, a, b)
     got = host(ops.tensor_mm(dev(a.astype(np.float32)), dev(b.astype(np.float32))))
     assert np.array_equal(got, want)
 
@@ -1184,7 +1240,7 @@ def test_mm_f16_few_rows_of_operands_no_kernel_fetches_as_they_lie(ops, oracle, 
     from anygpu_amd import capi
     a = synth.integers(m + 61, (m, k), -2, 2)
     b = synth.integers(n + 62, (k, n), -2, 2)
-    want = oracle.tensor_mm(a, b, threads=8)
+    want = mm_want(oracle, a, b)
     assert np.abs(want).max() <= 2048
     da = dev(a.astype(np.float16))
     if layout == "kn":
@@ -1202,7 +1258,7 @@ def test_mm_f32_few_rows_of_operands_no_kernel_fetches_as_they_lie(ops, oracle, 
     from anygpu_amd import capi
     a = synth.integers(m + 63, (m, k), -2, 2)
     b = synth.integers(n + 64, (k, n), -2, 2)
-    want = oracle.tensor_mm(a, b, threads=8)
+    want = mm_want(oracle, a, b)
     da = dev(a.astype(np.float32))
     if layout == "kn":
         got = ops.tensor_mm(da, dev(b.astype(np.float32)))
@@ -1224,7 +1280,7 @@ def test_mm_f16_rows_just_past_a_multiple_of_256(ops, oracle, layout, m, k, n):
     from anygpu_amd import capi
     a = synth.integers(m + 41, (m, k), -1, 1)
     b = synth.integers(n + 42, (k, n), -1, 1)
-    want = oracle.tensor_mm(a, b, threads=8)
+    want = mm_want(oracle, a, b)
     assert np.abs(want).max() <= 2048
     da = dev(a.astype(np.float16))
     if layout == "kn":
@@ -1243,7 +1299,7 @@ def test_mm_f16_up_to_128_rows_against_many_columns(ops, oracle, layout, m, k, n
     from anygpu_amd import capi
     a = synth.integers(m + 31, (m, k), -2, 2)
     b = synth.integers(n + 32, (k, n), -2, 2)
-    want = oracle.tensor_mm(a, b, threads=8)
+    want = mm_want(oracle, a, b)
     assert np.abs(want).max() <= 2048
     da = dev(a.astype(np.float16))
     if layout == "kn":
@@ -1260,7 +1316,7 @@ def test_mm_f16_k_contiguous_weights_result_rows_of_any_length(ops, oracle, m, k
     from anygpu_amd import capi
     a = synth.integers(m + 5, (m, k), -2, 2)
     b = synth.integers(n + 6, (k, n), -2, 2)
-    want = oracle.tensor_mm(a, b, threads=8)
+    want = mm_want(oracle, a, b)
     assert np.abs(want).max() <= 2048
     da, dbt = dev(a.astype(np.float16)), dev(np.ascontiguousarray(b.T).astype(np.float16))
     assert np.array_equal(host(ops.tensor_mm(da, dbt, b_layout=capi.B_COL_MAJOR)).astype(np.float32), want)
@@ -1279,7 +1335,7 @@ def test_mm_f16_sparse_launches_of_small_tiles(ops, oracle, m, k, n):
     from anygpu_amd import capi
     a = synth.integers(m + 11, (m, k), -1, 1)
     b = synth.integers(n + 12, (k, n), -1, 1)
-    want = oracle.tensor_mm(a, b, threads=8)
+    want = mm_want(oracle, a, b)
     assert np.abs(want).max() <= 2048
     da = dev(a.astype(np.float16))
     dbt = dev(np.ascontiguousarray(b.T).astype(np.float16))
@@ -1294,7 +1350,7 @@ def test_mm_f16_tiles_of_two_k_groups(ops, oracle, m, k, n):
     from anygpu_amd import capi
     a = synth.integers(m + 21, (m, k), -1, 1)
     b = synth.integers(n + 22, (k, n), -1, 1)
-    want = oracle.tensor_mm(a, b, threads=8)
+    want = mm_want(oracle, a, b)
     assert np.abs(want).max() <= 2048
     da = dev(a.astype(np.float16))
     dbt = dev(np.ascontiguousarray(b.T).astype(np.float16))
@@ -1340,12 +1396,12 @@ def test_gemm_epilogues_decode_step(ops, oracle, s):
     x = synth.normal(s, (1, s, hsize))
     w = synth.normal(2, (vsize, hsize)) * np.float32(0.3)
     got = host(ops.tensor_gemma_linear_softcap(dev(x), dev(w), cap))
-    want = oracle.gemma_linear_softcap(x, w, cap, threads=8)
+    want = softcap_head_want(oracle, x, w, cap)
     assert scaled_rel_err(got, want, 0.3 * math.sqrt(hsize)) <= TOL_F32
     wg = synth.normal(3, (hsize, isize)) * np.float32(1.0 / math.sqrt(hsize))
     wu = synth.normal(4, (hsize, isize)) * np.float32(1.0 / math.sqrt(hsize))
     got = host(ops.mlp_gemma2_fused_upproj(dev(x), dev(wg), dev(wu)))
-    want = oracle.gemma_mlp_upproj(x, wg, wu, threads=8)
+    want = upproj_want(oracle, x, wg, wu)
     assert scaled_rel_err(got, want, 1.0) <= TOL_F32
 
 
@@ -1369,7 +1425,7 @@ def test_gemm_f16_bias(ops, oracle, layout, m, k, n):
     a = synth.uniform(m + k, (m, k)).astype(np.float16)
     b = synth.uniform(k + n, (k, n)).astype(np.float16)
     bias = (synth.normal(n, (n,)) * np.float32(3.0)).astype(np.float16)
-    want = oracle.tensor_gemm(oracle.cvt_f16_to_f32(a), oracle.cvt_f16_to_f32(b), oracle.cvt_f16_to_f32(bias), threads=8)
+    want = gemm_want(oracle, oracle.cvt_f16_to_f32(a), oracle.cvt_f16_to_f32(b), oracle.cvt_f16_to_f32(bias))
     if layout == "row":
         got = host(ops.tensor_gemm(dev(a), dev(b), dev(bias)))
     else:
@@ -1377,7 +1433,7 @@ def test_gemm_f16_bias(ops, oracle, layout, m, k, n):
     assert got.dtype == np.float16 and got.shape == (m, n)
     assert scaled_rel_err(got.astype(np.float32), want, math.sqrt(k) / 3.0 + 3.0) <= TOL_F16_GEMM
     # the bias is part of the result: without it the columns are off by it
-    assert rel_l2(got.astype(np.float32) - oracle.cvt_f16_to_f32(bias)[None, :], oracle.tensor_mm(oracle.cvt_f16_to_f32(a), oracle.cvt_f16_to_f32(b), threads=8)) <= 2e-2
+    assert rel_l2(got.astype(np.float32) - oracle.cvt_f16_to_f32(bias)[None, :], mm_want(oracle, oracle.cvt_f16_to_f32(a), oracle.cvt_f16_to_f32(b))) <= 2e-2
 
 
 @pytest.mark.parametrize("m,k,n", F16_EPILOGUE_SHAPES)
@@ -1387,7 +1443,7 @@ def test_gemm_f16_softcap(ops, oracle, m, k, n):
     x = synth.normal(m + k, (1, m, k)).astype(np.float16)
     w = (synth.normal(k + n, (n, k)) * np.float32(2.0)).astype(np.float16)
     got = host(ops.tensor_gemma_linear_softcap(dev(x), dev(w), cap)).astype(np.float32)
-    want = oracle.gemma_linear_softcap(oracle.cvt_f16_to_f32(x), oracle.cvt_f16_to_f32(w), cap, threads=8)
+    want = softcap_head_want(oracle, oracle.cvt_f16_to_f32(x), oracle.cvt_f16_to_f32(w), cap)
     assert got.shape == (1, m, n)
     assert scaled_rel_err(got, want, min(cap, 2.0 * math.sqrt(k))) <= TOL_F16_GEMM
     assert np.all(np.abs(got) <= cap)
@@ -1401,7 +1457,7 @@ def test_gemm_f16_gelu_mul(ops, oracle, layout, m, k, n):
     x = synth.normal(m + k, (1, m, k)).astype(np.float16)
     wg = (synth.normal(n + 1, (k, n)) * np.float32(1.5 / math.sqrt(k))).astype(np.float16)
     wu = (synth.normal(n + 2, (k, n)) * np.float32(1.5 / math.sqrt(k))).astype(np.float16)
-    want = oracle.gemma_mlp_upproj(oracle.cvt_f16_to_f32(x), oracle.cvt_f16_to_f32(wg), oracle.cvt_f16_to_f32(wu), threads=8)
+    want = upproj_want(oracle, oracle.cvt_f16_to_f32(x), oracle.cvt_f16_to_f32(wg), oracle.cvt_f16_to_f32(wu))
     if layout == "row":
         got = host(ops.mlp_gemma2_fused_upproj(dev(x), dev(wg), dev(wu))).astype(np.float32)
         swapped = host(ops.mlp_gemma2_fused_upproj(dev(x), dev(wu), dev(wg))).astype(np.float32)
@@ -1469,7 +1525,7 @@ def test_mm_random_shapes_integer_inputs_exact(ops, oracle, dtype):
     for i, (m, k, n) in enumerate(_random_mm_shapes(7 if dtype == "f32" else 8, 40, k_max)):
         a = synth.integers(100 + i, (m, k), lo, hi)
         b = synth.integers(200 + i, (k, n), lo, hi)
-        want = oracle.tensor_mm(a, b, threads=8)
+        want = mm_want(oracle, a, b)
         da = dev(a.astype(np_dt))
         got_row = host(ops.tensor_mm(da, dev(b.astype(np_dt)))).astype(np.float32)
         got_col = host(ops.tensor_mm(da, dev(np.ascontiguousarray(b.T).astype(np_dt)), b_layout=capi.B_COL_MAJOR)).astype(np.float32)
@@ -1510,7 +1566,7 @@ def test_gemma_linear_softcap_shapes(ops, oracle, b, s, hsize, vsize):
     x = synth.normal(b * s + hsize, (b, s, hsize))
     w = synth.normal(vsize + hsize, (vsize, hsize)) * np.float32(4.0)      # logits reach well past the cap
     got = host(ops.tensor_gemma_linear_softcap(dev(x), dev(w), cap))
-    want = oracle.gemma_linear_softcap(x, w, cap, threads=8)
+    want = softcap_head_want(oracle, x, w, cap)
     assert got.shape == (b, s, vsize)
     # |d softcap / d logit| <= 1: the GEMM's tolerance carries over, floored by the logit scale (at most the cap)
     assert scaled_rel_err(got, want, min(cap, 4.0 * math.sqrt(hsize))) <= TOL_F32
@@ -1524,7 +1580,7 @@ def test_gemma_linear_softcap_gemma2_hidden_2304_vocab_slice(ops, oracle):
     w = synth.normal(2, (vsize, hsize)) * np.float32(0.3)
     got = host(ops.tensor_gemma_linear_softcap(dev(x), dev(w), cap))
     idx = sample_rows(s, 12, seed=3)
-    want = oracle.gemma_linear_softcap(x[:, idx], w, cap, threads=8)
+    want = softcap_head_want(oracle, x[:, idx], w, cap)
     assert scaled_rel_err(got[:, idx], want, 0.3 * math.sqrt(hsize)) <= TOL_F32
     # all rows: tanh is odd and monotone, so atanh(y / cap) * cap recovers the logits; check their row sums
     logits = np.arctanh(np.clip(got.astype(np.float64) / cap, -1 + 1e-12, 1 - 1e-12)) * cap
@@ -1541,7 +1597,7 @@ def test_gemma_mlp_fused_upproj_shapes(ops, oracle, b, s, hsize, isize):
     wg = synth.normal(isize + 1, (hsize, isize)) * np.float32(1.5 / math.sqrt(hsize))
     wu = synth.normal(isize + 2, (hsize, isize)) * np.float32(1.5 / math.sqrt(hsize))
     got = host(ops.mlp_gemma2_fused_upproj(dev(x), dev(wg), dev(wu)))
-    want = oracle.gemma_mlp_upproj(x, wg, wu, threads=8)
+    want = upproj_want(oracle, x, wg, wu)
     assert got.shape == (b, s, isize)
     # gate and up are O(1.5) each; |gelu'| <= 1.13, so the product's error scale is that of the two sums
     assert scaled_rel_err(got, want, 1.5 * 1.5) <= TOL_F32
@@ -1559,7 +1615,7 @@ def test_gemma_mlp_fused_upproj_gemma2_2304_9216(ops, oracle):
     wu = synth.normal(3, (hsize, isize)) * np.float32(1.0 / math.sqrt(hsize))
     got = host(ops.mlp_gemma2_fused_upproj(dev(x), dev(wg), dev(wu)))
     idx = sample_rows(s, 10, seed=4)
-    want = oracle.gemma_mlp_upproj(x[:, idx], wg, wu, threads=8)
+    want = upproj_want(oracle, x[:, idx], wg, wu)
     assert scaled_rel_err(got[:, idx], want, 1.0) <= TOL_F32
     # against the three-kernel chain on the device: same sums, so only the activation's rounding differs
     import torch
@@ -1579,7 +1635,7 @@ def test_gemm_gelu_mul_k_contiguous_weights(ops, oracle, m, hsize, isize):
     x = synth.normal(m, (m, hsize))
     wg = synth.normal(3, (hsize, isize)) * np.float32(1.0 / math.sqrt(hsize))
     wu = synth.normal(4, (hsize, isize)) * np.float32(1.0 / math.sqrt(hsize))
-    want = oracle.gemma_mlp_upproj(x, wg, wu, threads=8)
+    want = upproj_want(oracle, x, wg, wu)
     dx, dg, du = dev(x), dev(np.ascontiguousarray(wg.T)), dev(np.ascontiguousarray(wu.T))
     out = torch.empty((m, isize), device="cuda")
     rc = capi.load().anygpu_gemm_f32_gelu_mul(dx.data_ptr(), dg.data_ptr(), du.data_ptr(), out.data_ptr(), m, isize, hsize,
@@ -1599,7 +1655,7 @@ def test_gemm_gelu_mul_as_two_products_whose_operands_want_copies(ops, oracle):
     x = synth.normal(m, (m, hsize))
     wg = synth.normal(5, (hsize, isize)) * np.float32(1.0 / math.sqrt(hsize))
     wu = synth.normal(6, (hsize, isize)) * np.float32(1.0 / math.sqrt(hsize))
-    want = oracle.gemma_mlp_upproj(x, wg, wu, threads=8)
+    want = upproj_want(oracle, x, wg, wu)
     dx, dg, du = dev(x), dev(np.ascontiguousarray(wg.T)), dev(np.ascontiguousarray(wu.T))
     for _ in range(2):
         out = torch.empty((m, isize), device="cuda")
@@ -1609,7 +1665,7 @@ def test_gemm_gelu_mul_as_two_products_whose_operands_want_copies(ops, oracle):
         assert scaled_rel_err(host(out), want, 1.0) <= TOL_F32
     # and the plain product of the same operands afterwards (which may now grow the buffer for its copies)
     got = host(ops.tensor_mm(dx, dg, b_layout=capi.B_COL_MAJOR))
-    assert scaled_rel_err(got, oracle.tensor_mm(x, wg, threads=8), 1.0) <= TOL_F32
+    assert scaled_rel_err(got, mm_want(oracle, x, wg), 1.0) <= TOL_F32
 
 
 def test_gemm_epilogues_rejected_arguments(ops):
@@ -1757,6 +1813,72 @@ def test_sdp_attention_fused_kernel_f32_with_mask_tensor(ops, oracle, heads, n_q
     y = torch.full(q.shape, 3.0, device="cuda")
     assert f(dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), None, y.data_ptr(), heads, 1, n_q, n_k, d, n_k, alpha, 0.0, None) == capi.ANYGPU_ERR_NULL_POINTER
     assert f(dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), dm.data_ptr(), y.data_ptr(), heads, 1, n_q, n_k, d, n_k - 1, alpha, 0.0, None) == capi.ANYGPU_ERR_BAD_STRIDE
+    torch.cuda.synchronize()
+    assert bool((y == 3.0).all())
+
+
+@pytest.mark.parametrize("heads,n_q,n_k,d,kind", [
+    (4, 100, 100, 64, "causal"), (2, 130, 131, 128, "slide"), (3, 257, 257, 256, "slide"), (2, 64, 203, 128, "random"),
+    (2, 33, 1001, 256, "random"), (8, 200, 5000, 64, "causal"),          # (the last: few query blocks, the key range in parts)
+    (2, 70, 70, 128, "blind_rows"), (1, 17, 3, 64, "random"), (2, 300, 300, 256, "odd_stride"),
+])
+def test_sdp_attention_fused_kernel_f16_with_mask_tensor(ops, oracle, heads, n_q, n_k, d, kind):
+    # the same interface in half precision: one kernel reads the mask (halves, -inf where a key is hidden) as data;
+    # against the oracle's operator chain on the up-cast operands and against the three launches on the device
+    import torch
+    from anygpu_amd import capi
+    q = synth.normal(1 + n_q, (1, heads, n_q, d)).astype(np.float16)
+    k = synth.normal(2 + n_k, (1, heads, n_k, d)).astype(np.float16)
+    v = synth.normal(3 + d, (1, heads, n_k, d)).astype(np.float16)
+    alpha = float(d) ** -0.5
+    diag = n_k - n_q
+    if kind == "causal":
+        mask = oracle.causal_mask(n_q, n_k, diag=diag)
+    elif kind in ("slide", "odd_stride"):
+        mask = oracle.slide_mask(oracle.causal_mask(n_q, n_k, diag=diag), max(n_k // 3, 1))
+    else:
+        rng = np.random.default_rng(n_q * 1000 + n_k)
+        mask = rng.normal(0.0, 2.0, (n_q, n_k)).astype(np.float32)
+        mask[rng.random((n_q, n_k)) < 0.33] = -np.inf
+        mask[:, 0] = 0.5
+        if kind == "blind_rows":
+            mask[5] = -np.inf                     # queries without a visible key: zeros, where the operator chain has NaN
+            mask[n_q // 2] = -np.inf
+    with np.errstate(over="ignore"):
+        mask16 = np.ascontiguousarray(mask, dtype=np.float32).astype(np.float16).reshape(1, 1, n_q, n_k)
+    with np.errstate(invalid="ignore", over="ignore"):
+        want = oracle.sdp_attention_masked_scaled_fwd(*(oracle.cvt_f16_to_f32(t) for t in (q, k, v)), mask16.astype(np.float32), alpha, threads=8)
+    dq, dk, dv, dm = dev(q), dev(k), dev(v), dev(mask16)
+    if kind == "odd_stride":
+        # mask rows an odd number of halves apart, starting off a 4-byte boundary, through the C entry point itself
+        pitch = n_k + 3
+        store = torch.full((n_q * pitch + 1,), float("nan"), dtype=torch.float16, device="cuda")
+        rows = store[1:].reshape(n_q, pitch)
+        rows[:, :n_k] = dm.reshape(n_q, n_k)
+        y = torch.empty_like(dq)
+        rc = capi.load().anygpu_sdp_attention_fwd_masked_f16(dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), rows.data_ptr(), y.data_ptr(),
+                                                             heads, 1, n_q, n_k, d, pitch, alpha, 0.0, None)
+        assert rc == capi.ANYGPU_OK
+        got = host(y).astype(np.float32)
+    else:
+        got = host(ops.sdp_attention_masked_scaled_fwd(dq, dk, dv, dm, alpha)).astype(np.float32)
+    assert got.shape == q.shape and np.isfinite(got).all()
+    blind = ~np.isfinite(want).all(axis=-1)
+    assert blind.sum() == (2 * heads if kind == "blind_rows" else 0)
+    assert not got[blind].any()
+    assert rel_l2(got[~blind], want[~blind]) <= 1e-2
+    assert scaled_rel_err(got[~blind], want[~blind], 1.0) <= TOL_F16_GEMM
+    # the three launches on the device
+    scores = ops.tensor_mm_batched(dq[0], dk[0], b_layout=capi.B_COL_MAJOR)
+    probs = ops.tensor_softmax_masked(scores.reshape(-1, n_k), dm.reshape(n_q, n_k), alpha=alpha, q_len=n_q)
+    three = host(ops.tensor_mm_batched(probs.reshape(heads, n_q, n_k), dv[0])).astype(np.float32)
+    assert scaled_rel_err(got[0][~blind[0]], three[~blind[0]], 1.0) <= TOL_F16_GEMM
+    # the C entry point's own checks
+    f = capi.load().anygpu_sdp_attention_fwd_masked_f16
+    y = torch.full(q.shape, 3.0, device="cuda", dtype=torch.float16)
+    assert f(dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), None, y.data_ptr(), heads, 1, n_q, n_k, d, n_k, alpha, 0.0, None) == capi.ANYGPU_ERR_NULL_POINTER
+    assert f(dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), dm.data_ptr(), y.data_ptr(), heads, 1, n_q, n_k, d, n_k - 1, alpha, 0.0, None) == capi.ANYGPU_ERR_BAD_STRIDE
+    assert f(dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), dm.data_ptr() + 1, y.data_ptr(), heads, 1, n_q, n_k, d, n_k, alpha, 0.0, None) == capi.ANYGPU_ERR_UNSUPPORTED
     torch.cuda.synchronize()
     assert bool((y == 3.0).all())
 
@@ -2368,7 +2490,7 @@ def test_mm_f32_operand_copies_larger_than_the_first_workspace(ops, oracle):
     assert capi.WORKSPACE_BYTES < held <= 3 * capi.WORKSPACE_BYTES, held       # 121 MB of copies in steps of 64 MiB
     assert torch.equal(got, torch.matmul(da, dw.t()))
     rows = [0, 1, 1499, 2999]
-    want = oracle.tensor_mm(a[rows], np.ascontiguousarray(w.T), threads=8)
+    want = mm_want(oracle, a[rows], np.ascontiguousarray(w.T))
     assert np.array_equal(host(got)[rows], want)
     # the grown buffer serves later calls, large and small
     free1 = torch.cuda.mem_get_info()[0]
