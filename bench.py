@@ -96,9 +96,10 @@ def parse_args():
     ap.add_argument("--only", default="", help="comma list of: gemm,gemm32,conv,softmax,attn,attn32,decode,norm,head (default: all)")
     ap.add_argument("--gemm-shapes", nargs="?", const="f16", default=None, choices=("f16", "f32"),
                     help="print the table of GEMM layer shapes (fp16, or fp32 with `--gemm-shapes f32`) against torch.matmul and exit")
-    ap.add_argument("--attention-shapes", action="store_true",
+    ap.add_argument("--attention-shapes", nargs="?", const="all", default=None, choices=("all", "mask_tensor"),
                     help="print the table of attention shapes (generation steps, chunks of a prompt against a cache, masked "
-                         "softmax) against torch and exit")
+                         "softmax) against torch and exit; `--attention-shapes mask_tensor`: only the attention with the mask "
+                         "as a tensor (fused kernel, three launches, torch)")
     ap.add_argument("--gemm-rows", default="layer", choices=("layer", "between"),
                     help="with --gemm-shapes: the row counts of the layer table (powers of two, default) or 22 row counts between "
                          "the tile heights over 8 of the shapes")
@@ -700,6 +701,55 @@ def sweep_attention_shapes(torch, ops):
             print(f"| {str(dtype)[6:]} | {heads} | {n_q} | {n_k} | {t_masked:.1f} | {gbs:.0f} | {t_plain:.1f} | {t_theirs:.1f} |", flush=True)
 
 
+def sweep_attention_mask_tensor(torch, ops, capi):
+    """sdp_attention_masked_scaled_fwd, the reference's attention interface with the mask as a tensor (a causal -inf mask, or
+    a dense bias), through the fused kernel that reads the mask as data, next to the three launches it replaces (batched
+    q k^T, softmax with the mask tensor, batched p v), the rule form of the same causal mask and torch's
+    scaled_dot_product_attention with the same mask tensor.  Microseconds, the better of two runs of 10 launches."""
+    import torch.nn.functional as F
+
+    def timed(fn, iters=10, warm=3):
+        for _ in range(warm):
+            fn()
+        torch.cuda.synchronize()
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(iters):
+            fn()
+        stop.record()
+        torch.cuda.synchronize()
+        return start.elapsed_time(stop) / iters * 1e3
+
+    print("\n| dtype | heads | queries | keys | head dim | mask | fused with mask tensor us | three launches us | rule form us | torch SDPA with the mask us |")
+    print("|---|---:|---:|---:|---:|---|---:|---:|---:|---:|")
+    for dtype in (torch.half, torch.float):
+        for heads, n_q, n_k, d, kind in ((8, 8192, 8192, 256, "causal"), (32, 1024, 1024, 128, "causal"), (32, 2048, 2048, 64, "causal"),
+                                         (8, 16, 8192, 256, "causal"), (16, 512, 8192, 128, "causal"), (8, 4096, 4096, 128, "dense bias")):
+            q = torch.randn(1, heads, n_q, d, device="cuda").to(dtype)
+            k, v = (torch.randn(1, heads, n_k, d, device="cuda").to(dtype) for _ in range(2))
+            if kind == "causal":
+                mask = torch.zeros(n_q, n_k, device="cuda").to(dtype)
+                mask.masked_fill_(torch.ones(n_q, n_k, device="cuda").triu(n_k - n_q + 1).bool(), float("-inf"))
+            else:
+                mask = torch.randn(n_q, n_k, device="cuda").to(dtype)
+            m4 = mask.reshape(1, 1, n_q, n_k)
+            alpha = d ** -0.5
+
+            def three():
+                scores = ops.tensor_mm_batched(q[0], k[0], b_layout=capi.B_COL_MAJOR)
+                probs = ops.tensor_softmax_masked(scores.reshape(-1, n_k), mask, alpha=alpha, q_len=n_q)
+                return ops.tensor_mm_batched(probs.reshape(heads, n_q, n_k), v[0])
+
+            fused = lambda: ops.sdp_attention_masked_scaled_fwd(q, k, v, m4, alpha)
+            theirs = lambda: F.scaled_dot_product_attention(q, k, v, attn_mask=m4, scale=alpha)
+            t_fused, t_three, t_theirs = min(timed(fused), timed(fused)), min(timed(three), timed(three)), min(timed(theirs), timed(theirs))
+            rule = "-"
+            if kind == "causal":
+                by_rule = lambda: ops.sdp_attention_fwd(q, k, v, alpha, causal=True, decode=False)
+                rule = f"{min(timed(by_rule), timed(by_rule)):.1f}"
+            print(f"| {str(dtype)[6:]} | {heads} | {n_q} | {n_k} | {d} | {kind} | {t_fused:.1f} | {t_three:.1f} | {rule} | {t_theirs:.1f} |", flush=True)
+
+
 def sample_gemm_shapes(torch, ops, capi):
     """A few products that do not fill the chip with 256 x 256 tiles, ragged ones, ones the chunk loads cannot fetch and two
     output heads with [K, N] weights and few rows, next to torch.matmul on the same operands: microseconds, the better of two runs of 40 launches each side."""
@@ -751,7 +801,9 @@ def main():
         sweep_gemm_shapes(torch, ops, capi, args.gemm_shapes, args.gemm_rows, args.gemm_layout)
         return 0
     if args.attention_shapes:
-        sweep_attention_shapes(torch, ops)
+        if args.attention_shapes == "all":
+            sweep_attention_shapes(torch, ops)
+        sweep_attention_mask_tensor(torch, ops, capi)
         return 0
     only = set(filter(None, args.only.split(",")))
     want = lambda name: not only or name in only
