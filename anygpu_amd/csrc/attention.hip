@@ -31,11 +31,13 @@
 #include "device_utils.hpp"
 #include "attention_walk.hpp"
 #include "attention_split.hpp"
+#include "attention_tile_map.hpp"
 #include "gemm_band.hpp"
 #include "launch.hpp"
 
 #include <algorithm>
 #include <atomic>
+#include <optional>
 #include <type_traits>
 #include <utility>
 
@@ -71,6 +73,8 @@ struct AttnArgs
 	float* partials;       // key-split blocks leave their partial results here: [head][split slot][part][query][D + 2]
 	const half_t* mask;    // MASK kernels: additive mask [n_q, n_k] shared by all heads (added behind scale and softcap)
 	int64_t mask_stride;   // halves between its rows
+	const unsigned long long* tile_map;   // MASK kernels: visible-tile words [query block][map_words] (attention_tile_map.hpp), or nullptr
+	int map_words;
 };
 
 // log2(e) * softcap(alpha * s); without softcap k_in = alpha log2(e); with it
@@ -100,7 +104,8 @@ struct AttnLds
 // MASK: an additive mask tensor instead of the index rules (the launcher passes none): the four mask values of a lane's four scores
 // of a key block are consecutive in memory; they are requested a tile ahead and added behind scale and softcap; a tile
 // that the mask hides from every query of a wave costs the wave no products (it still issues its share of the next
-// tile's loads).  No tile is skipped for the whole block on account of the mask.
+// tile's loads); a tile that the visible-tile map of the mask (attention_tile_map.hpp) has not set for the block is
+// neither loaded nor waited for.
 template <int D, bool SOFTCAP, int QB, int WAVES, bool MASK = false>
 __global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f16_kernel(const AttnArgs a, const AttnWalk walk)
 {
@@ -251,21 +256,33 @@ __global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f16_kernel(const
 				mk_next[b][kb] = val;
 			}
 	};
+	// MASK: the walk visits the tiles that the visible-tile map of the mask has set for this query block (all of them
+	// without a map); t_next is the tile after t on that walk, the stages alternate along it
+	const unsigned long long* map_row = nullptr;
+	if constexpr (MASK)
+	{
+		if (a.tile_map != nullptr) map_row = a.tile_map + (int64_t)q_block * a.map_words;
+		t_first = attention_next_visible_tile(map_row, t_first, t_last);
+	}
 	if (t_first <= t_last)
 	{
 		if constexpr (MASK) load_mask(t_first);
 #pragma unroll
 		for (int j = 0; j < kSlots; ++j) issue_slot(t_first, 0, j);
 	}
-	for (int t = t_first; t <= t_last; ++t)
+	int t_next = 0, stage_m = 0;
+	for (int t = t_first; t <= t_last; t = MASK ? t_next : t + 1, stage_m ^= 1)
 	{
 		// own loads of tile t have landed; behind the barrier everybody's have, and everybody is done with the
-		// stage of tile t - 1, which the loads of tile t + 1 overwrite
+		// stage of the tile before, which the loads of the next tile overwrite
 		__builtin_amdgcn_s_waitcnt(0x0F70);            // vmcnt(0)
 		__syncthreads();
-		k_lds = lds + ((t - t_first) & 1) * kStageBytes;
+		const int stage = MASK ? stage_m : (t - t_first) & 1;
+		if constexpr (MASK) t_next = attention_next_visible_tile(map_row, t + 1, t_last);
+		else t_next = t + 1;
+		k_lds = lds + stage * kStageBytes;
 		v_lds = k_lds + kAttnKeysPerTile * L::kPitchK;
-		const bool more = t < t_last;
+		const bool more = t_next <= t_last;
 		// the mask values of this tile move out of the way of the next tile's, which go out now; they stay halves until
 		// the scores meet them (the float form would not fit the registers at head_dim 256)
 		half4_t mk[MASK ? QB : 1][4];
@@ -281,13 +298,13 @@ __global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f16_kernel(const
 #pragma unroll
 					for (int r = 0; r < 4; ++r) any_visible |= mk[b][kb][r] > (half_t)(-INFINITY);
 				}
-			if (more) load_mask(t + 1);
+			if (more) load_mask(t_next);
 			if (__builtin_amdgcn_ballot_w64(any_visible) == 0)
 			{
 				if (more)
 				{
 #pragma unroll
-					for (int j = 0; j < kSlots; ++j) issue_slot(t + 1, (t + 1 - t_first) & 1, j);
+					for (int j = 0; j < kSlots; ++j) issue_slot(t_next, stage ^ 1, j);
 				}
 				continue;
 			}
@@ -313,7 +330,7 @@ __global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f16_kernel(const
 				if (st == KS - 1 && more)
 				{
 #pragma unroll
-					for (int j = kb; j < kSlots; j += 4) issue_slot(t + 1, (t + 1 - t_first) & 1, j);
+					for (int j = kb; j < kSlots; j += 4) issue_slot(t_next, stage ^ 1, j);
 				}
 			}
 
@@ -1177,10 +1194,32 @@ hipError_t launch_sdp_attention_fwd_f16(const void* q, const void* k, const void
 	args.partials = nullptr;
 	args.mask = static_cast<const half_t*>(mask);
 	args.mask_stride = mask_stride;
+	args.tile_map = nullptr;
+	args.map_words = 0;
 	if (mask != nullptr)
 	{
 		args.causal = 0;
 		args.window = 0;
+		// The visible-tile map of the mask, at the front of the stream's workspace (the partial results of a split key
+		// range go behind it): worth its pass over the mask from 4 M mask values on, and left out where the stream has no
+		// workspace to offer (a capture without a caller's workspace); the results are the same bit for bit, the map
+		// only saves the loads and barriers of tiles that every wave of a block would skip.
+		constexpr int kMaskQueriesPerBlock = 16 * 8;
+		const int64_t words = attention_tile_map_words(n_k, kAttnKeysPerTile);
+		const size_t map_bytes = (size_t)((n_q + kMaskQueriesPerBlock - 1) / kMaskQueriesPerBlock * words) * sizeof(unsigned long long);
+		std::optional<band::WorkspaceReserve> map_hold;
+		if (n_q * n_k >= attention_mask_map_from() && band::workspace_capacity(stream) >= map_bytes + (1u << 16))
+		{
+			float* front = nullptr;
+			hipError_t e = band::workspace_acquire(stream, &front);
+			if (e != hipSuccess) return e;
+			unsigned long long* map = reinterpret_cast<unsigned long long*>(front);
+			e = launch_attention_mask_tile_map(args.mask, mask_stride, n_q, n_k, kMaskQueriesPerBlock, kAttnKeysPerTile, map, stream);
+			if (e != hipSuccess) return e;
+			args.tile_map = map;
+			args.map_words = (int)words;
+			map_hold.emplace(map_bytes);
+		}
 		// sixteen queries per wave at every head dimension: the mask values of a tile take the registers of a second block
 #define ANYGPU_ATTN_F16_MASK_DIM(DIM) \
 		return capped ? launch_variant<DIM, true, 1, false, true>(args, batch_heads, stream) : launch_variant<DIM, false, 1, false, true>(args, batch_heads, stream)

@@ -25,10 +25,12 @@
 #include "device_utils.hpp"
 #include "attention_walk.hpp"
 #include "attention_split.hpp"
+#include "attention_tile_map.hpp"
 #include "gemm_band.hpp"
 #include "launch.hpp"
 
 #include <atomic>
+#include <optional>
 
 namespace anygpu {
 
@@ -50,6 +52,8 @@ struct AttnArgsF32
 	float* partials;       // key-split blocks leave their partial results here: [head][split slot][part][query][D + 2]
 	const float* mask;     // MASK kernels: additive mask [n_q, n_k] shared by all heads (added behind scale and softcap)
 	int64_t mask_stride;   // floats between its rows
+	const unsigned long long* tile_map;   // MASK kernels: visible-tile words [query block][map_words] (attention_tile_map.hpp), or nullptr
+	int map_words;
 };
 
 // log2(e) * softcap(alpha * s); without softcap k_in = alpha log2(e); with it
@@ -89,7 +93,8 @@ __device__ __forceinline__ void wait_vmem_all()
 // Otherwise the tiles pass through registers into a single stage.
 // MASK: an additive mask tensor instead of (or on top of) the index rules: the four mask values of a lane's four scores
 // of a key block are consecutive in memory; they are requested in front of the tile's first product and added behind
-// scale and softcap.  No tile is skipped on account of the mask.
+// scale and softcap.  A tile that the mask hides from every query of a wave costs the wave no products; a tile that the
+// visible-tile map of the mask (attention_tile_map.hpp) has not set for the block is neither loaded nor waited for.
 template <int D, bool SOFTCAP, int WAVES, int KT, bool DIRECT, bool MASK>
 __global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f32_kernel(const AttnArgsF32 a, const AttnWalk walk)
 {
@@ -235,30 +240,42 @@ __global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f32_kernel(const
 			dst[kb] = val;
 		}
 	};
+	// MASK: the walk visits the tiles that the visible-tile map of the mask has set for this query block (all of them
+	// without a map); t_next is the tile after t on that walk, the stages alternate along it
+	const unsigned long long* map_row = nullptr;
+	if constexpr (MASK)
+	{
+		if (a.tile_map != nullptr) map_row = a.tile_map + (int64_t)q_block * a.map_words;
+		t_first = attention_next_visible_tile(map_row, t_first, t_last);
+	}
 	if (t_first <= t_last)
 	{
 		if constexpr (MASK) load_mask(mk_next, t_first);
 		if constexpr (DIRECT) tile_direct(t_first, 0);
 		else tile_load(t_first);
 	}
-	for (int t = t_first; t <= t_last; ++t)
+	int t_next = 0, stage_m = 0;
+	for (int t = t_first; t <= t_last; t = MASK ? t_next : t + 1, stage_m ^= 1)
 	{
 		const float* k_lds = lds_base;
+		const int stage = MASK ? stage_m : (t - t_first) & 1;
+		if constexpr (MASK) t_next = attention_next_visible_tile(map_row, t + 1, t_last);
+		else t_next = t + 1;
 		if constexpr (DIRECT)
 		{
 			// own loads of tile t have landed; behind the barrier everybody's have, and everybody is done with the
-			// stage of tile t - 1, which the loads of tile t + 1 overwrite
+			// stage of the tile before, which the loads of the next tile overwrite
 			wait_vmem_all();
 			__syncthreads();
-			if (t < t_last) tile_direct(t + 1, (t - t_first + 1) & 1);
-			k_lds = lds_base + ((t - t_first) & 1) * L::kStageFloats;
+			if (t_next <= t_last) tile_direct(t_next, stage ^ 1);
+			k_lds = lds_base + stage * L::kStageFloats;
 		}
 		else
 		{
 			__syncthreads();                       // the previous tile has been read by everybody
 			tile_store();
 			__syncthreads();
-			if (t < t_last) tile_load(t + 1);      // in flight while this tile is used
+			if (t_next <= t_last) tile_load(t_next);      // in flight while this tile is used
 		}
 		const float* v_lds = k_lds + kKeysPerTile * L::kPitch;
 
@@ -276,7 +293,7 @@ __global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f32_kernel(const
 #pragma unroll
 				for (int r = 0; r < 4; ++r) any_visible |= mk[kb][r] > -INFINITY;
 			}
-			if (t < t_last) load_mask(mk_next, t + 1);
+			if (t_next <= t_last) load_mask(mk_next, t_next);
 			if (__builtin_amdgcn_ballot_w64(any_visible) == 0) continue;
 		}
 
@@ -459,6 +476,30 @@ hipError_t launch_variant_f32(const AttnArgsF32& args_in, int64_t batch_heads, h
 	}
 	AttnArgsF32 args = args_in;
 	const int64_t q_blocks = (args.n_q + kQueriesPerBlock - 1) / kQueriesPerBlock;
+	args.tile_map = nullptr;
+	args.map_words = 0;
+	std::optional<band::WorkspaceReserve> map_hold;
+	if constexpr (MASK)
+	{
+		// The visible-tile map of the mask, at the front of the stream's workspace (the partial results of a split key
+		// range go behind it): worth its pass over the mask from 4 M mask values on, and left out where the stream has no
+		// workspace to offer (a capture without a caller's workspace); the results are the same bit for bit, the map
+		// only saves the loads and barriers of tiles that every wave of a block would skip.
+		const int64_t words = attention_tile_map_words(args.n_k, KT);
+		const size_t map_bytes = (size_t)(q_blocks * words) * sizeof(unsigned long long);
+		if ((int64_t)args.n_q * args.n_k >= attention_mask_map_from() && band::workspace_capacity(stream) >= map_bytes + (1u << 16))
+		{
+			float* front = nullptr;
+			hipError_t e = band::workspace_acquire(stream, &front);
+			if (e != hipSuccess) return e;
+			unsigned long long* map = reinterpret_cast<unsigned long long*>(front);
+			e = launch_attention_mask_tile_map(args.mask, args.mask_stride, args.n_q, args.n_k, kQueriesPerBlock, KT, map, stream);
+			if (e != hipSuccess) return e;
+			args.tile_map = map;
+			args.map_words = (int)words;
+			map_hold.emplace(map_bytes);
+		}
+	}
 	const AttnSplitPlan plan = plan_attention_split(args.n_q, args.n_k, args.causal, args.diag, args.window, batch_heads,
 	                                                kQueriesPerBlock, KT, D, band::workspace_capacity(stream));
 	// (or, with too few query blocks for the chip, every block in several parts of its key range)

@@ -307,7 +307,11 @@ int anygpu_sdp_attention_fwd_f32(const float* q, const float* k, const float* v,
  * float lowest the reference's mask builders write) where a key is hidden; a query without a visible key gives zeros.
  * One kernel, no score matrix in memory: the fused counterpart of sdp_attention_masked_scaled_fwd
  * (srcs/transformers/sdp.hpp:207-274), whose mask argument is a tensor, in the precision the reference runs it in.
- * No key tile is skipped on account of the mask; callers whose mask is an index rule are better served by
+ * For masks of 4 M values and more (the environment variable ANYGPU_ATTN_MASK_MAP_FROM, read at every call, replaces that
+ * number) a pass over the mask ahead of the kernel (once, not per head) notes which key tiles it hides from which
+ * blocks of queries; those are neither loaded nor multiplied.  The note lives at the front of the stream's workspace;
+ * under a capture without a caller's workspace there is none, every tile is loaded and the hidden ones cost no products.
+ * The results are the same bit for bit either way.  Callers whose mask is an index rule are still better served by
  * anygpu_sdp_attention_fwd_f32.  Same key splits through the stream's workspace as that entry point.
  */
 int anygpu_sdp_attention_fwd_masked_f32(const float* q, const float* k, const float* v, const float* mask, float* y,
@@ -318,7 +322,7 @@ int anygpu_sdp_attention_fwd_masked_f32(const float* q, const float* k, const fl
  * The same in half precision: q, k, v, y and the mask are halves (the mask 2-byte aligned, rows mask_stride >= n_k
  * halves apart), sums in fp32 on the matrix cores as in anygpu_sdp_attention_fwd_f16.  -inf hides a key; the half
  * lowest (-65504) is an ordinary, very negative bias, which hides a key wherever the row has a less negative one.
- * A key tile in which the mask hides every key from all sixteen queries of a wave costs that wave no products.
+ * Hidden key tiles are left out as in the float32 form.
  */
 int anygpu_sdp_attention_fwd_masked_f16(const void* q, const void* k, const void* v, const void* mask, void* y,
                                         int64_t batch_heads, int64_t q_per_kv, int64_t n_q, int64_t n_k, int64_t head_dim,

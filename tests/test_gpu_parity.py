@@ -75,6 +75,19 @@ def upproj_want(oracle, x, wg, wu):
                       x, 2.0 * wg.shape[0] * wg.shape[1])
 
 
+def hide_key_stripes(mask, rng):
+    """Hides long key ranges from long query ranges of an additive mask [n_q, n_k] in place (whole key tiles hidden from
+    whole blocks of queries, their edges anywhere), the first keys among them; every query keeps one visible key, each
+    somewhere else."""
+    n_q, n_k = mask.shape
+    for _ in range(6):
+        r0, c0 = int(rng.integers(0, n_q)), int(rng.integers(0, n_k))
+        mask[r0:r0 + int(rng.integers(40, 400)), c0:c0 + int(rng.integers(100, 1200))] = -np.inf
+    mask[: n_q // 2, :200] = -np.inf
+    mask[n_q // 3:, n_k - 300:] = -np.inf
+    mask[np.arange(n_q), rng.integers(0, n_k, n_q)] = 0.25
+
+
 def dev(a):
     import torch
     return torch.from_numpy(np.ascontiguousarray(a)).cuda()
@@ -1767,8 +1780,10 @@ def test_sdp_attention_masked_scaled_fwd(ops, oracle):
     (4, 100, 100, 64, "causal"), (2, 130, 131, 128, "slide"), (3, 257, 257, 256, "slide"), (2, 64, 203, 128, "random"),
     (2, 33, 1001, 256, "random"), (8, 200, 5000, 64, "causal"),          # (the last: few query blocks, the key range in parts)
     (2, 70, 70, 128, "blind_rows"), (1, 17, 3, 64, "random"),
+    # key ranges hidden from whole blocks of queries (key tiles the visible-tile map of the mask leaves out), ragged last tiles and blocks
+    (2, 300, 1500, 128, "slide"), (3, 200, 2100, 64, "stripes"), (2, 150, 4200, 256, "stripes"), (1, 520, 1030, 128, "stripes"),
 ])
-def test_sdp_attention_fused_kernel_f32_with_mask_tensor(ops, oracle, heads, n_q, n_k, d, kind):
+def test_sdp_attention_fused_kernel_f32_with_mask_tensor(ops, oracle, monkeypatch, heads, n_q, n_k, d, kind):
     # the reference's own attention interface (srcs/transformers/sdp.hpp:207-274): the mask arrives as a tensor.  In
     # float32 one kernel reads it as data; against the oracle's operator chain and against the three-launch form
     # (batched product, softmax with the mask tensor, batched product) on the device.
@@ -1788,6 +1803,8 @@ def test_sdp_attention_fused_kernel_f32_with_mask_tensor(ops, oracle, heads, n_q
         mask = rng.normal(0.0, 2.0, (n_q, n_k)).astype(np.float32)
         mask[rng.random((n_q, n_k)) < 0.33] = -np.inf
         mask[:, 0] = 0.5
+        if kind == "stripes":
+            hide_key_stripes(mask, rng)
         if kind == "blind_rows":
             mask[5] = -np.inf                     # queries without a visible key: zeros, where the operator chain has NaN
             mask[n_q // 2] = -np.inf
@@ -1795,7 +1812,12 @@ def test_sdp_attention_fused_kernel_f32_with_mask_tensor(ops, oracle, heads, n_q
     mask4 = np.ascontiguousarray(mask, dtype=np.float32).reshape(1, 1, n_q, n_k)
     with np.errstate(invalid="ignore", over="ignore"):
         want = oracle.sdp_attention_masked_scaled_fwd(q, k, v, mask4, alpha, threads=8)
+    # with the visible-tile map of the mask (a pass over the mask ahead of the kernel; by default only for large masks)
+    # and without: the same bit for bit
+    monkeypatch.setenv("ANYGPU_ATTN_MASK_MAP_FROM", "0")
     got = host(ops.sdp_attention_masked_scaled_fwd(dev(q), dev(k), dev(v), dev(mask4), alpha))
+    monkeypatch.setenv("ANYGPU_ATTN_MASK_MAP_FROM", str(1 << 60))
+    assert np.array_equal(got, host(ops.sdp_attention_masked_scaled_fwd(dev(q), dev(k), dev(v), dev(mask4), alpha)), equal_nan=True)
     assert got.shape == q.shape and got.dtype == np.float32 and np.isfinite(got).all()
     blind = ~np.isfinite(want).all(axis=-1)
     assert blind.sum() == (2 * heads if kind == "blind_rows" else 0)
@@ -1821,8 +1843,11 @@ def test_sdp_attention_fused_kernel_f32_with_mask_tensor(ops, oracle, heads, n_q
     (4, 100, 100, 64, "causal"), (2, 130, 131, 128, "slide"), (3, 257, 257, 256, "slide"), (2, 64, 203, 128, "random"),
     (2, 33, 1001, 256, "random"), (8, 200, 5000, 64, "causal"),          # (the last: few query blocks, the key range in parts)
     (2, 70, 70, 128, "blind_rows"), (1, 17, 3, 64, "random"), (2, 300, 300, 256, "odd_stride"),
+    # key ranges hidden from whole blocks of queries (key tiles the visible-tile map of the mask leaves out), ragged last tiles and blocks
+    (2, 300, 1500, 128, "slide"), (3, 200, 2100, 64, "stripes"), (2, 150, 4200, 256, "stripes"), (1, 520, 1030, 128, "stripes"),
+    (2, 260, 1500, 64, "odd_stride"),
 ])
-def test_sdp_attention_fused_kernel_f16_with_mask_tensor(ops, oracle, heads, n_q, n_k, d, kind):
+def test_sdp_attention_fused_kernel_f16_with_mask_tensor(ops, oracle, monkeypatch, heads, n_q, n_k, d, kind):
     # the same interface in half precision: one kernel reads the mask (halves, -inf where a key is hidden) as data;
     # against the oracle's operator chain on the up-cast operands and against the three launches on the device
     import torch
@@ -1841,6 +1866,8 @@ def test_sdp_attention_fused_kernel_f16_with_mask_tensor(ops, oracle, heads, n_q
         mask = rng.normal(0.0, 2.0, (n_q, n_k)).astype(np.float32)
         mask[rng.random((n_q, n_k)) < 0.33] = -np.inf
         mask[:, 0] = 0.5
+        if kind == "stripes":
+            hide_key_stripes(mask, rng)
         if kind == "blind_rows":
             mask[5] = -np.inf                     # queries without a visible key: zeros, where the operator chain has NaN
             mask[n_q // 2] = -np.inf
@@ -1855,13 +1882,22 @@ def test_sdp_attention_fused_kernel_f16_with_mask_tensor(ops, oracle, heads, n_q
         store = torch.full((n_q * pitch + 1,), float("nan"), dtype=torch.float16, device="cuda")
         rows = store[1:].reshape(n_q, pitch)
         rows[:, :n_k] = dm.reshape(n_q, n_k)
-        y = torch.empty_like(dq)
-        rc = capi.load().anygpu_sdp_attention_fwd_masked_f16(dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), rows.data_ptr(), y.data_ptr(),
-                                                             heads, 1, n_q, n_k, d, pitch, alpha, 0.0, None)
-        assert rc == capi.ANYGPU_OK
-        got = host(y).astype(np.float32)
+
+        def run():
+            y = torch.empty_like(dq)
+            rc = capi.load().anygpu_sdp_attention_fwd_masked_f16(dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), rows.data_ptr(), y.data_ptr(),
+                                                                 heads, 1, n_q, n_k, d, pitch, alpha, 0.0, None)
+            assert rc == capi.ANYGPU_OK
+            return host(y).astype(np.float32)
     else:
-        got = host(ops.sdp_attention_masked_scaled_fwd(dq, dk, dv, dm, alpha)).astype(np.float32)
+        def run():
+            return host(ops.sdp_attention_masked_scaled_fwd(dq, dk, dv, dm, alpha)).astype(np.float32)
+    # with the visible-tile map of the mask (a pass over the mask ahead of the kernel; by default only for large masks)
+    # and without: the same bit for bit
+    monkeypatch.setenv("ANYGPU_ATTN_MASK_MAP_FROM", "0")
+    got = run()
+    monkeypatch.setenv("ANYGPU_ATTN_MASK_MAP_FROM", str(1 << 60))
+    assert np.array_equal(got, run(), equal_nan=True)
     assert got.shape == q.shape and np.isfinite(got).all()
     blind = ~np.isfinite(want).all(axis=-1)
     assert blind.sum() == (2 * heads if kind == "blind_rows" else 0)
