@@ -229,32 +229,68 @@ __global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f16_kernel(const
 		}
 	};
 
-	// MASK: the mask values of this lane's scores of tile t: four consecutive halves per query block and key block, at any
-	// alignment; keys past the end and rows past the last query count as hidden
+	// MASK: the mask values of tile t.  A lane's four scores of key block kb belong to keys 16 kb + 4 g .. + 3: fetched as
+	// they are needed, the four lanes of a query would take 32 bytes of its mask row per instruction, sixteen quarter
+	// lines.  Instead lane (n, g) fetches the sixteen values of key block g of its query (32 consecutive bytes at any
+	// alignment: a whole 128-byte line per query and pair of instructions), and when the tile's turn comes the lane
+	// groups exchange 8-byte pieces by row swaps in the VALU (a 4 x 4 transposition over g).  Keys past the end and
+	// rows past the last query count as hidden.
 	half4_t mk_next[MASK ? QB : 1][4];
 	auto load_mask = [&](int t) {
-		typedef half4_t LooseHalf4 __attribute__((aligned(2)));
+		typedef half8_t LooseHalf8 __attribute__((aligned(2)));
 #pragma unroll
 		for (int b = 0; b < (MASK ? QB : 0); ++b)
-#pragma unroll
-			for (int kb = 0; kb < 4; ++kb)
+		{
+			const int key = t * kAttnKeysPerTile + 16 * g;
+			const half_t hidden = (half_t)(-INFINITY);
+			half8_t lo = {hidden, hidden, hidden, hidden, hidden, hidden, hidden, hidden}, hi = lo;
+			if (q_row[b] < a.n_q)
 			{
-				const int key = t * kAttnKeysPerTile + 16 * kb + 4 * g;
-				const half_t hidden = (half_t)(-INFINITY);
-				half4_t val = {hidden, hidden, hidden, hidden};
-				if (q_row[b] < a.n_q)
+				const half_t* src = a.mask + (int64_t)q_row[b] * a.mask_stride + key;
+				if (key + 15 < a.n_k)
 				{
-					const half_t* src = a.mask + (int64_t)q_row[b] * a.mask_stride + key;
-					if (key + 3 < a.n_k) val = *reinterpret_cast<const LooseHalf4*>(src);
-					else
-					{
+					lo = *reinterpret_cast<const LooseHalf8*>(src);
+					hi = *reinterpret_cast<const LooseHalf8*>(src + 8);
+				}
+				else
+				{
 #pragma unroll
-						for (int r = 0; r < 4; ++r)
-							if (key + r < a.n_k) val[r] = src[r];
+					for (int r = 0; r < 8; ++r)
+					{
+						if (key + r < a.n_k) lo[r] = src[r];
+						if (key + 8 + r < a.n_k) hi[r] = src[8 + r];
 					}
 				}
-				mk_next[b][kb] = val;
 			}
+			mk_next[b][0] = __builtin_shufflevector(lo, lo, 0, 1, 2, 3);
+			mk_next[b][1] = __builtin_shufflevector(lo, lo, 4, 5, 6, 7);
+			mk_next[b][2] = __builtin_shufflevector(hi, hi, 0, 1, 2, 3);
+			mk_next[b][3] = __builtin_shufflevector(hi, hi, 4, 5, 6, 7);
+		}
+	};
+	// piece j of lane group g <-> piece g of lane group j, for every lane % 16: v_permlane32_swap exchanges the upper half
+	// of its first operand with the lower half of its second, v_permlane16_swap the odd rows of the first with the even
+	// rows of the second (all lanes of the wave are active here)
+	auto exchange_mask_pieces = [&](half4_t (&piece)[4]) {
+		typedef unsigned int uint2_t __attribute__((ext_vector_type(2)));
+		uint2_t w[4];
+#pragma unroll
+		for (int j = 0; j < 4; ++j) w[j] = __builtin_bit_cast(uint2_t, piece[j]);
+#pragma unroll
+		for (int d = 0; d < 2; ++d)
+		{
+			unsigned int r0 = w[0][d], r1 = w[1][d], r2 = w[2][d], r3 = w[3][d];
+			asm("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(r0), "+v"(r2));
+			asm("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(r1), "+v"(r3));
+			asm("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(r0), "+v"(r1));
+			asm("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(r2), "+v"(r3));
+			w[0][d] = r0;
+			w[1][d] = r1;
+			w[2][d] = r2;
+			w[3][d] = r3;
+		}
+#pragma unroll
+		for (int j = 0; j < 4; ++j) piece[j] = __builtin_bit_cast(half4_t, w[j]);
 	};
 	// MASK: the walk visits the tiles that the visible-tile map of the mask has set for this query block (all of them
 	// without a map); t_next is the tile after t on that walk, the stages alternate along it
@@ -291,13 +327,15 @@ __global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f16_kernel(const
 			bool any_visible = false;
 #pragma unroll
 			for (int b = 0; b < QB; ++b)
+			{
+#pragma unroll
+				for (int kb = 0; kb < 4; ++kb) mk[b][kb] = mk_next[b][kb];
+				exchange_mask_pieces(mk[b]);
 #pragma unroll
 				for (int kb = 0; kb < 4; ++kb)
-				{
-					mk[b][kb] = mk_next[b][kb];
 #pragma unroll
 					for (int r = 0; r < 4; ++r) any_visible |= mk[b][kb][r] > (half_t)(-INFINITY);
-				}
+			}
 			if (more) load_mask(t_next);
 			if (__builtin_amdgcn_ballot_w64(any_visible) == 0)
 			{
