@@ -93,7 +93,7 @@ def parse_args():
     ap.add_argument("--cpu-seconds", type=float, default=12.0,
                     help="target wall time of the CPU-oracle sample of the headline (0 disables every CPU baseline); "
                          "the other configurations get a quarter of it each")
-    ap.add_argument("--only", default="", help="comma list of: gemm,gemm32,conv,softmax,attn,attn32,decode,norm,head (default: all)")
+    ap.add_argument("--only", default="", help="comma list of: gemm,gemm32,conv,softmax,attn,attn32,attnmask,decode,norm,head (default: all)")
     ap.add_argument("--gemm-shapes", nargs="?", const="f16", default=None, choices=("f16", "f32"),
                     help="print the table of GEMM layer shapes (fp16, or fp32 with `--gemm-shapes f32`) against torch.matmul and exit")
     ap.add_argument("--attention-shapes", nargs="?", const="all", default=None, choices=("all", "mask_tensor"),
@@ -505,6 +505,35 @@ def bench_attention(torch, ops, synth, steps, warmup, dtype):
     }
 
 
+def bench_attention_mask_tensor(torch, ops, synth, steps, warmup, dtype):
+    # The reference's own attention interface (sdp_attention_masked_scaled_fwd, srcs/transformers/sdp.hpp:207-274): the
+    # mask arrives as a tensor [1, 1, queries, keys], here the causal + sliding-window mask of a Gemma2 local layer
+    # (-inf where hidden), shared by 8 heads of 8192 positions, head_dim 256, scale 1 / 16.  One pass over the mask (which
+    # key tiles are hidden from which blocks of queries) and one fused kernel that reads the mask as data; timed together.
+    h, n, d, win = 8, 8192, 256, 4096
+    tdt = torch.float16 if dtype == "f16" else torch.float32
+    q, k, v = attention_inputs(torch, synth, h, h, n, d, "float16" if dtype == "f16" else "float32")
+    rows = torch.arange(n, device="cuda").reshape(n, 1)
+    cols = torch.arange(n, device="cuda").reshape(1, n)
+    mask = torch.zeros(n, n, device="cuda", dtype=tdt)
+    mask.masked_fill_((cols > rows) | (cols <= rows - win), float("-inf"))
+    m4 = mask.reshape(1, 1, n, n)
+    t = timed_region(torch, lambda: ops.sdp_attention_masked_scaled_fwd(q, k, v, m4, 1.0 / 16.0), steps, warmup)
+    pairs = win * (win + 1) // 2 + (n - win) * win          # visible (query, key) pairs per head
+    flops = 4.0 * d * pairs * h
+    sec = t["us_per_launch"] * 1e-6
+    peak = PEAK_FP16_TFLOPS if dtype == "f16" else PEAK_FP32_TFLOPS
+    return {
+        "name": f"sdp_attention_mask_tensor_{dtype}",
+        "workload": f"attention with the mask as a tensor, {'fp16' if dtype == 'f16' else 'fp32'}: q, k, v [1, 8, 8192, 256] N(0,1) seeds 1 / 2 / 3, x 1/16, "
+                    "mask [1, 1, 8192, 8192] causal + window 4096 as 0 / -inf; pass over the mask + fused kernel",
+        **timing_fields(t), "value": flops / sec / 1e12, "unit": "TFLOP/s", "dtype": dtype,
+        "roofline": {"bound": "mfma", "achieved": flops / sec / 1e12, "peak": peak, "unit": "TFLOP/s",
+                     "frac": flops / sec / 1e12 / peak, "traffic": None,
+                     "algorithmic_flops": flops, "visible_pairs_per_head": pairs, "mask_bytes": mask.numel() * mask.element_size()},
+    }
+
+
 def bench_attention_decode(torch, capi, synth, steps, warmup):
     # One generation step against a long cache: 64 query heads over 8 key / value heads, 32768 cached positions,
     # head_dim 128, causal.  The split-key decode form through the C ABI with the caller's workspace: two launches
@@ -840,6 +869,9 @@ def main():
         kernels.append(bench_attention(torch, ops, synth, args.steps // 8, max(args.warmup // 4, 1), "f16"))
     if want("attn32"):
         kernels.append(bench_attention(torch, ops, synth, args.steps // 16, max(args.warmup // 8, 1), "f32"))
+    if want("attnmask"):
+        kernels.append(bench_attention_mask_tensor(torch, ops, synth, args.steps // 8, max(args.warmup // 4, 1), "f16"))
+        kernels.append(bench_attention_mask_tensor(torch, ops, synth, args.steps // 16, max(args.warmup // 8, 1), "f32"))
     if want("decode"):
         kernels.append(bench_attention_decode(torch, capi, synth, args.steps, args.warmup))
     if want("norm"):
