@@ -135,12 +135,23 @@ __global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f32_kernel(const
 	if (a.window > 0 && q0 + a.diag - a.window + 1 > 0) key_lo = q0 + a.diag - a.window + 1;
 	int t_first = key_lo / kKeysPerTile;
 	int t_last = key_hi >= 0 ? key_hi / kKeysPerTile : -1;
+	// MASK: the visible-tile map of the mask, where the launcher has made one: the words of this query block
+	const unsigned long long* map_row = nullptr;
+	if constexpr (MASK)
+	{
+		if (a.tile_map != nullptr) map_row = a.tile_map + (int64_t)q_block * a.map_words;
+	}
 	if (parts > 1)
 	{
-		// one part of the block's key tiles; the other parts are other blocks', a merge kernel combines them
-		const int per = (t_last - t_first + parts) / parts;
-		t_first += part * per;
-		if (t_first + per - 1 < t_last) t_last = t_first + per - 1;
+		// one part of the block's key tiles; the other parts are other blocks', a merge kernel combines them.  With a
+		// map the parts divide the VISIBLE tiles among them, else the range
+		if (MASK && map_row != nullptr) attention_visible_share(map_row, part, parts, t_first, t_last);
+		else
+		{
+			const int per = (t_last - t_first + parts) / parts;
+			t_first += part * per;
+			if (t_first + per - 1 < t_last) t_last = t_first + per - 1;
+		}
 	}
 
 	// this lane's query as second operand: q[row][16 s + 4 g .. + 3]
@@ -240,14 +251,9 @@ __global__ __launch_bounds__(64 * WAVES) void sdp_attention_fwd_f32_kernel(const
 			dst[kb] = val;
 		}
 	};
-	// MASK: the walk visits the tiles that the visible-tile map of the mask has set for this query block (all of them
-	// without a map); t_next is the tile after t on that walk, the stages alternate along it
-	const unsigned long long* map_row = nullptr;
-	if constexpr (MASK)
-	{
-		if (a.tile_map != nullptr) map_row = a.tile_map + (int64_t)q_block * a.map_words;
-		t_first = attention_next_visible_tile(map_row, t_first, t_last);
-	}
+	// MASK: the walk visits the tiles that the map has set (all of them without a map); t_next is the tile after t on
+	// that walk, the stages alternate along it
+	if constexpr (MASK) t_first = attention_next_visible_tile(map_row, t_first, t_last);
 	if (t_first <= t_last)
 	{
 		if constexpr (MASK) load_mask(mk_next, t_first);
@@ -482,12 +488,12 @@ hipError_t launch_variant_f32(const AttnArgsF32& args_in, int64_t batch_heads, h
 	if constexpr (MASK)
 	{
 		// The visible-tile map of the mask, at the front of the stream's workspace (the partial results of a split key
-		// range go behind it): worth its pass over the mask from 4 M mask values on, and left out where the stream has no
+		// range go behind it): worth its pass over the mask for large masks and long key ranges (attention_mask_map_wanted), and left out where the stream has no
 		// workspace to offer (a capture without a caller's workspace); the results are the same bit for bit, the map
 		// only saves the loads and barriers of tiles that every wave of a block would skip.
 		const int64_t words = attention_tile_map_words(args.n_k, KT);
 		const size_t map_bytes = (size_t)(q_blocks * words) * sizeof(unsigned long long);
-		if ((int64_t)args.n_q * args.n_k >= attention_mask_map_from() && band::workspace_capacity(stream) >= map_bytes + (1u << 16))
+		if (attention_mask_map_wanted(args.n_q, args.n_k) && band::workspace_capacity(stream) >= map_bytes + (1u << 16))
 		{
 			float* front = nullptr;
 			hipError_t e = band::workspace_acquire(stream, &front);

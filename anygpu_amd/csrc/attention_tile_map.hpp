@@ -67,14 +67,16 @@ __global__ __launch_bounds__(1024) void attention_mask_tile_map_kernel(const T* 
 	if (threadIdx.x == 0) map[(int64_t)q_block * groups + group] = (unsigned short)bits;
 }
 
-// Masks of fewer values than this go without the map: its pass costs a launch and a few memory latencies, which a short
-// key range does not earn back.  The environment variable ANYGPU_ATTN_MASK_MAP_FROM, read at every launch, replaces the
-// number (0: always, a huge value: never); the results do not depend on it.
-inline int64_t attention_mask_map_from()
+// Whether the map is made for a mask of n_q x n_k values.  Its pass costs a launch and a few memory latencies (8 - 12 us for
+// small masks, 5.6 TB/s for large ones), which short key ranges do not earn back: from 4 M mask values on, or from 16384 keys
+// on whatever the queries (a sliding window over a long cache hides most of them from a few queries as well).  The
+// environment variable ANYGPU_ATTN_MASK_MAP_FROM, read at every launch, replaces the rule by "from that many mask values
+// on" (0: always, a huge value: never).
+inline bool attention_mask_map_wanted(int64_t n_q, int64_t n_k)
 {
 	const char* text = std::getenv("ANYGPU_ATTN_MASK_MAP_FROM");
-	if (text != nullptr && *text != 0) return std::atoll(text);
-	return 4ll << 20;
+	if (text != nullptr && *text != 0) return n_q * n_k >= std::atoll(text);
+	return n_q * n_k >= (4ll << 20) || n_k >= 16384;
 }
 
 // 64-bit words of the map per query block
@@ -112,6 +114,52 @@ __device__ __forceinline__ int attention_next_visible_tile(const unsigned long l
 		t = (t | 63) + 1;
 	}
 	return t_last + 1;
+}
+
+// The share of part `part` of `parts` among the set tiles of [t_first, t_last]: narrows the range to the set tiles number
+// part * per .. (part + 1) * per - 1, per = ceil(set tiles / parts), so that the parts of a query block's key range carry
+// equal numbers of visible tiles wherever the mask hides the others (a sliding window over a long cache leaves most
+// equal parts of the RANGE empty).  An empty share comes back as t_first > t_last.  Block-uniform, scalar work.
+__device__ __forceinline__ void attention_visible_share(const unsigned long long* __restrict__ map_row, int part, int parts,
+                                                        int& t_first, int& t_last)
+{
+	if (t_first > t_last) return;
+	const int w_first = t_first >> 6, w_last = t_last >> 6;
+	auto word_in_range = [&](int w) {
+		unsigned long long bits = map_row[w];
+		if (w == w_first) bits &= ~0ull << (t_first & 63);
+		if (w == w_last && (t_last & 63) != 63) bits &= (1ull << ((t_last & 63) + 1)) - 1;
+		return bits;
+	};
+	int total = 0;
+	for (int w = w_first; w <= w_last; ++w) total += __builtin_popcountll(word_in_range(w));
+	const int per = (total + parts - 1) / parts;
+	const int lo = part * per;
+	const int hi = lo + per < total ? lo + per : total;           // set tiles lo .. hi - 1
+	if (per == 0 || lo >= hi)
+	{
+		t_first = t_last + 1;
+		return;
+	}
+	// tile index of the set bit number `nth` (counted from 0) of the range
+	auto locate = [&](int nth) {
+		for (int w = w_first; w <= w_last; ++w)
+		{
+			unsigned long long bits = word_in_range(w);
+			const int here = __builtin_popcountll(bits);
+			if (nth >= here)
+			{
+				nth -= here;
+				continue;
+			}
+			for (; nth > 0; --nth) bits &= bits - 1;
+			return 64 * w + __builtin_ctzll(bits);
+		}
+		return t_last;                                            // (not reached: nth < total)
+	};
+	const int first = locate(lo), last = locate(hi - 1);
+	t_first = first;
+	t_last = last;
 }
 
 }  // namespace anygpu

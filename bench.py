@@ -768,14 +768,19 @@ def sweep_attention_mask_tensor(torch, ops, capi):
     print("|---|---:|---:|---:|---:|---|---:|---:|---:|---:|")
     for dtype in (torch.half, torch.float):
         for heads, n_q, n_k, d, kind in ((8, 8192, 8192, 256, "causal"), (32, 1024, 1024, 128, "causal"), (32, 2048, 2048, 64, "causal"),
-                                         (8, 16, 8192, 256, "causal"), (16, 512, 8192, 128, "causal"), (8, 4096, 4096, 128, "dense bias")):
+                                         (8, 16, 8192, 256, "causal"), (16, 512, 8192, 128, "causal"), (8, 4096, 4096, 128, "dense bias"),
+                                         (8, 256, 32768, 128, "window 4096"), (8, 1024, 32768, 256, "window 4096")):
             q = torch.randn(1, heads, n_q, d, device="cuda").to(dtype)
             k, v = (torch.randn(1, heads, n_k, d, device="cuda").to(dtype) for _ in range(2))
-            if kind == "causal":
-                mask = torch.zeros(n_q, n_k, device="cuda").to(dtype)
-                mask.masked_fill_(torch.ones(n_q, n_k, device="cuda").triu(n_k - n_q + 1).bool(), float("-inf"))
-            else:
+            window = 4096 if kind.startswith("window") else 0
+            if kind == "dense bias":
                 mask = torch.randn(n_q, n_k, device="cuda").to(dtype)
+            else:
+                hidden = torch.ones(n_q, n_k, device="cuda").triu(n_k - n_q + 1).bool()
+                if window:
+                    hidden |= torch.ones(n_q, n_k, device="cuda").tril(n_k - n_q - window).bool()
+                mask = torch.zeros(n_q, n_k, device="cuda").to(dtype)
+                mask.masked_fill_(hidden, float("-inf"))
             m4 = mask.reshape(1, 1, n_q, n_k)
             alpha = d ** -0.5
 
@@ -788,8 +793,8 @@ def sweep_attention_mask_tensor(torch, ops, capi):
             theirs = lambda: F.scaled_dot_product_attention(q, k, v, attn_mask=m4, scale=alpha)
             t_fused, t_three, t_theirs = min(timed(fused), timed(fused)), min(timed(three), timed(three)), min(timed(theirs), timed(theirs))
             rule = "-"
-            if kind == "causal":
-                by_rule = lambda: ops.sdp_attention_fwd(q, k, v, alpha, causal=True, decode=False)
+            if kind != "dense bias":
+                by_rule = lambda: ops.sdp_attention_fwd(q, k, v, alpha, causal=True, window=window, decode=False)
                 rule = f"{min(timed(by_rule), timed(by_rule)):.1f}"
             print(f"| {str(dtype)[6:]} | {heads} | {n_q} | {n_k} | {d} | {kind} | {t_fused:.1f} | {t_three:.1f} | {rule} | {t_theirs:.1f} |", flush=True)
 

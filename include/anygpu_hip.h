@@ -307,11 +307,13 @@ int anygpu_sdp_attention_fwd_f32(const float* q, const float* k, const float* v,
  * float lowest the reference's mask builders write) where a key is hidden; a query without a visible key gives zeros.
  * One kernel, no score matrix in memory: the fused counterpart of sdp_attention_masked_scaled_fwd
  * (srcs/transformers/sdp.hpp:207-274), whose mask argument is a tensor, in the precision the reference runs it in.
- * For masks of 4 M values and more (the environment variable ANYGPU_ATTN_MASK_MAP_FROM, read at every call, replaces that
- * number) a pass over the mask ahead of the kernel (once, not per head) notes which key tiles it hides from which
+ * For masks of 4 M values and more, and for key ranges of 16384 keys and more whatever the queries (the environment variable
+ * ANYGPU_ATTN_MASK_MAP_FROM, read at every call, replaces both by a number of mask values) a pass over the mask ahead of the kernel (once, not per head) notes which key tiles it hides from which
  * blocks of queries; those are neither loaded nor multiplied.  The note lives at the front of the stream's workspace;
  * under a capture without a caller's workspace there is none, every tile is loaded and the hidden ones cost no products.
- * The results are the same bit for bit either way.  Callers whose mask is an index rule are still better served by
+ * The results are the same bit for bit either way, except where few query blocks go out in parts of their key range:
+ * with the note the parts divide the visible tiles among them (a sliding window over a long cache leaves most equal
+ * parts of the range empty), without it the range, and the sums are taken in another order.  Callers whose mask is an index rule are still better served by
  * anygpu_sdp_attention_fwd_f32.  Same key splits through the stream's workspace as that entry point.
  */
 int anygpu_sdp_attention_fwd_masked_f32(const float* q, const float* k, const float* v, const float* mask, float* y,

@@ -1813,11 +1813,14 @@ def test_sdp_attention_fused_kernel_f32_with_mask_tensor(ops, oracle, monkeypatc
     with np.errstate(invalid="ignore", over="ignore"):
         want = oracle.sdp_attention_masked_scaled_fwd(q, k, v, mask4, alpha, threads=8)
     # with the visible-tile map of the mask (a pass over the mask ahead of the kernel; by default only for large masks)
-    # and without: the same bit for bit
+    # and without
     monkeypatch.setenv("ANYGPU_ATTN_MASK_MAP_FROM", "0")
     got = host(ops.sdp_attention_masked_scaled_fwd(dev(q), dev(k), dev(v), dev(mask4), alpha))
     monkeypatch.setenv("ANYGPU_ATTN_MASK_MAP_FROM", str(1 << 60))
-    assert np.array_equal(got, host(ops.sdp_attention_masked_scaled_fwd(dev(q), dev(k), dev(v), dev(mask4), alpha)), equal_nan=True)
+    without_map = host(ops.sdp_attention_masked_scaled_fwd(dev(q), dev(k), dev(v), dev(mask4), alpha))
+    # (few query blocks go out in parts of their key range, cut by visible tiles with the map and by range without:
+    # another order of summation)
+    assert scaled_rel_err(got, without_map, 1.0) <= 1e-5
     assert got.shape == q.shape and got.dtype == np.float32 and np.isfinite(got).all()
     blind = ~np.isfinite(want).all(axis=-1)
     assert blind.sum() == (2 * heads if kind == "blind_rows" else 0)
@@ -1893,11 +1896,12 @@ def test_sdp_attention_fused_kernel_f16_with_mask_tensor(ops, oracle, monkeypatc
         def run():
             return host(ops.sdp_attention_masked_scaled_fwd(dq, dk, dv, dm, alpha)).astype(np.float32)
     # with the visible-tile map of the mask (a pass over the mask ahead of the kernel; by default only for large masks)
-    # and without: the same bit for bit
+    # and without (few query blocks go out in parts of their key range, cut by visible tiles with the map and by range
+    # without: another order of summation, a last place of the half result)
     monkeypatch.setenv("ANYGPU_ATTN_MASK_MAP_FROM", "0")
     got = run()
     monkeypatch.setenv("ANYGPU_ATTN_MASK_MAP_FROM", str(1 << 60))
-    assert np.array_equal(got, run(), equal_nan=True)
+    assert scaled_rel_err(got, run(), 1.0) <= TOL_F16_ROWOPS
     assert got.shape == q.shape and np.isfinite(got).all()
     blind = ~np.isfinite(want).all(axis=-1)
     assert blind.sum() == (2 * heads if kind == "blind_rows" else 0)
