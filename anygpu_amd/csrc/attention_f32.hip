@@ -485,6 +485,7 @@ hipError_t launch_variant_f32(const AttnArgsF32& args_in, int64_t batch_heads, h
 	args.tile_map = nullptr;
 	args.map_words = 0;
 	std::optional<band::WorkspaceReserve> map_hold;
+	bool mask_two_parts = false;
 	if constexpr (MASK)
 	{
 		// The visible-tile map of the mask, at the front of the stream's workspace (the partial results of a split key
@@ -493,11 +494,24 @@ hipError_t launch_variant_f32(const AttnArgsF32& args_in, int64_t batch_heads, h
 		// only saves the loads and barriers of tiles that every wave of a block would skip.
 		const int64_t words = attention_tile_map_words(args.n_k, KT);
 		const size_t map_bytes = (size_t)(q_blocks * words) * sizeof(unsigned long long);
-		if (attention_mask_map_wanted(args.n_q, args.n_k) && band::workspace_capacity(stream) >= map_bytes + (1u << 16))
+		// With as many blocks as one to four rounds of the chip the rounds do not even out where the mask leaves the
+		// blocks unequal shares of their key range (a sliding window: the late query blocks carry the full window, the
+		// early ones little): every block then goes out in two parts, each with half of its VISIBLE tiles.  Their
+		// partial results may take more than the library's own workspace holds to begin with; it grows for them as
+		// it does for operand copies (eager launches only), before anything points into it.
+		const int64_t blocks = q_blocks * batch_heads;
+		const int cus = device_cu_count();
+		size_t two_parts_bytes = 0;
+		if (blocks >= cus && blocks < 4 * (int64_t)cus && (args.n_k + KT - 1) / KT >= 32)
+			two_parts_bytes = (size_t)2 * blocks * kQueriesPerBlock * (D + 2) * sizeof(float);
+		const size_t map_room = (map_bytes + 255) / 256 * 256 + (1u << 16);
+		if (two_parts_bytes > 0 && band::workspace_copy_capacity(stream) < map_room + two_parts_bytes) two_parts_bytes = 0;
+		if (attention_mask_map_wanted(args.n_q, args.n_k) && (two_parts_bytes > 0 || band::workspace_capacity(stream) >= map_room))
 		{
 			float* front = nullptr;
-			hipError_t e = band::workspace_acquire(stream, &front);
+			hipError_t e = band::workspace_acquire(stream, &front, two_parts_bytes > 0 ? map_room + two_parts_bytes : 0);
 			if (e != hipSuccess) return e;
+			mask_two_parts = two_parts_bytes > 0;
 			unsigned long long* map = reinterpret_cast<unsigned long long*>(front);
 			e = launch_attention_mask_tile_map(args.mask, args.mask_stride, args.n_q, args.n_k, kQueriesPerBlock, KT, map, stream);
 			if (e != hipSuccess) return e;
@@ -509,8 +523,9 @@ hipError_t launch_variant_f32(const AttnArgsF32& args_in, int64_t batch_heads, h
 	const AttnSplitPlan plan = plan_attention_split(args.n_q, args.n_k, args.causal, args.diag, args.window, batch_heads,
 	                                                kQueriesPerBlock, KT, D, band::workspace_capacity(stream));
 	// (or, with too few query blocks for the chip, every block in several parts of its key range)
-	const int64_t parts_all = plan.n_split > 0 ? 1 : plan_attention_parts(args.n_q, args.n_k, args.causal, args.diag, batch_heads, kQueriesPerBlock,
-	                                                                    KT, D, band::workspace_capacity(stream));
+	int64_t parts_all = plan.n_split > 0 ? 1 : plan_attention_parts(args.n_q, args.n_k, args.causal, args.diag, batch_heads, kQueriesPerBlock,
+	                                                                  KT, D, band::workspace_capacity(stream));
+	if (mask_two_parts && plan.n_split == 0 && parts_all == 1) parts_all = 2;
 	args.partials = nullptr;
 	if (plan.n_split > 0 || parts_all > 1)
 	{

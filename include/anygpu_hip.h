@@ -313,7 +313,10 @@ int anygpu_sdp_attention_fwd_f32(const float* q, const float* k, const float* v,
  * under a capture without a caller's workspace there is none, every tile is loaded and the hidden ones cost no products.
  * The results are the same bit for bit either way, except where few query blocks go out in parts of their key range:
  * with the note the parts divide the visible tiles among them (a sliding window over a long cache leaves most equal
- * parts of the range empty), without it the range, and the sums are taken in another order.  Callers whose mask is an index rule are still better served by
+ * parts of the range empty), without it the range, and the sums are taken in another order.  With as many query blocks as
+ * one to four rounds of the device's compute units the float32 form sends every block out in two such parts; for their
+ * partial results an eager launch without a caller's workspace lets the library's own grow (as operand copies do, up to
+ * 1 GiB; 192 MiB for 8 heads x 8192 queries x 256).  Callers whose mask is an index rule are still better served by
  * anygpu_sdp_attention_fwd_f32.  Same key splits through the stream's workspace as that entry point.
  */
 int anygpu_sdp_attention_fwd_masked_f32(const float* q, const float* k, const float* v, const float* mask, float* y,

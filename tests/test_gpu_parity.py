@@ -1923,6 +1923,38 @@ def test_sdp_attention_fused_kernel_f16_with_mask_tensor(ops, oracle, monkeypatc
     assert bool((y == 3.0).all())
 
 
+def test_sdp_attention_f32_mask_tensor_blocks_in_two_parts_of_their_visible_tiles(ops, oracle, monkeypatch):
+    # as many query blocks as one to four rounds of the chip (16 heads x 18 blocks of 64 queries): with the map of the mask
+    # every block goes out in two parts, each with half of its visible tiles, and a merge launch; against the run without
+    # the map (whole blocks), against the three launches on the device, and two of the heads against the oracle
+    import torch
+    from anygpu_amd import capi
+    heads, n_q, n_k, d = 16, 1100, 2100, 64
+    q = synth.normal(71, (1, heads, n_q, d))
+    k = synth.normal(72, (1, heads, n_k, d))
+    v = synth.normal(73, (1, heads, n_k, d))
+    alpha = float(d) ** -0.5
+    rng = np.random.default_rng(74)
+    mask = rng.normal(0.0, 1.0, (n_q, n_k)).astype(np.float32)
+    hide_key_stripes(mask, rng)
+    mask4 = mask.reshape(1, 1, n_q, n_k)
+    dq, dk, dv, dm = dev(q), dev(k), dev(v), dev(mask4)
+    monkeypatch.setenv("ANYGPU_ATTN_MASK_MAP_FROM", "0")
+    got = host(ops.sdp_attention_masked_scaled_fwd(dq, dk, dv, dm, alpha))
+    monkeypatch.setenv("ANYGPU_ATTN_MASK_MAP_FROM", str(1 << 60))
+    whole = host(ops.sdp_attention_masked_scaled_fwd(dq, dk, dv, dm, alpha))
+    assert np.isfinite(got).all()
+    assert scaled_rel_err(got, whole, 1.0) <= 1e-5
+    assert not np.array_equal(got, whole), "the two runs were expected to sum in different orders"
+    scores = ops.tensor_mm_batched(dq[0], dk[0], b_layout=capi.B_COL_MAJOR)
+    probs = ops.tensor_softmax_masked(scores.reshape(-1, n_k), dm.reshape(n_q, n_k), alpha=alpha, q_len=n_q)
+    three = host(ops.tensor_mm_batched(probs.reshape(heads, n_q, n_k), dv[0]))
+    assert scaled_rel_err(got[0], three, 1.0) <= TOL_F32 * 2
+    for h in (0, heads - 1):
+        want = oracle.sdp_attention_masked_scaled_fwd(q[:, h:h + 1], k[:, h:h + 1], v[:, h:h + 1], mask4, alpha, threads=8)
+        assert scaled_rel_err(got[:, h:h + 1], want, 1.0) <= TOL_F32
+
+
 ATTN_CASES = [
     # heads, kv_heads, n_q, n_k, d, alpha, softcap, causal, window
     (2, 2, 16, 16, 64, 0.125, 0.0, False, 0),
