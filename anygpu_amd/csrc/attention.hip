@@ -1245,9 +1245,10 @@ hipError_t launch_sdp_attention_fwd_f16(const void* q, const void* k, const void
 		args.causal = 0;
 		args.window = 0;
 		// The visible-tile map of the mask, at the front of the stream's workspace (the partial results of a split key
-		// range go behind it): worth its pass over the mask for large masks and long key ranges (attention_mask_map_wanted), and left out where the stream has no
-		// workspace to offer (a capture without a caller's workspace); the results are the same bit for bit, the map
-		// only saves the loads and barriers of tiles that every wave of a block would skip.
+		// range go behind it): worth its pass over the mask for large masks and long key ranges
+		// (attention_mask_map_wanted), and left out where the stream has no workspace to offer (a capture without a
+		// caller's workspace).  For whole query blocks the results are the same bit for bit: the map only saves the loads
+		// and barriers of tiles that every wave of a block would skip.
 		constexpr int kMaskQueriesPerBlock = 16 * 8;
 		const int64_t words = attention_tile_map_words(n_k, kAttnKeysPerTile);
 		const size_t map_bytes = (size_t)((n_q + kMaskQueriesPerBlock - 1) / kMaskQueriesPerBlock * words) * sizeof(unsigned long long);

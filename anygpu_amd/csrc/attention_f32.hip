@@ -489,9 +489,10 @@ hipError_t launch_variant_f32(const AttnArgsF32& args_in, int64_t batch_heads, h
 	if constexpr (MASK)
 	{
 		// The visible-tile map of the mask, at the front of the stream's workspace (the partial results of a split key
-		// range go behind it): worth its pass over the mask for large masks and long key ranges (attention_mask_map_wanted), and left out where the stream has no
-		// workspace to offer (a capture without a caller's workspace); the results are the same bit for bit, the map
-		// only saves the loads and barriers of tiles that every wave of a block would skip.
+		// range go behind it): worth its pass over the mask for large masks and long key ranges
+		// (attention_mask_map_wanted), and left out where the stream has no workspace to offer (a capture without a
+		// caller's workspace).  For whole query blocks the results are the same bit for bit: the map only saves the loads
+		// and barriers of tiles that every wave of a block would skip.
 		const int64_t words = attention_tile_map_words(args.n_k, KT);
 		const size_t map_bytes = (size_t)(q_blocks * words) * sizeof(unsigned long long);
 		// With as many blocks as one to four rounds of the chip the rounds do not even out where the mask leaves the
